@@ -1,0 +1,397 @@
+// FakeQuantize / requantize kernels (HBM-bound) and their load-time object.
+// Reference semantics: ngraph/core/reference/.../fake_quantize.hpp:175-265.
+//
+// Traffic per element: 4 B read + 1 B written (q8 forms) or + 4 B written (f32 op form).
+// One wave reads 64 x 16 B = 1 KiB contiguous per load instruction; the per-channel table
+// (32 B per channel) stays in L1/L2.
+#include "fq.h"
+
+#include <algorithm>
+#include <atomic>
+#include <cmath>
+
+namespace hipie {
+
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ uint32_t pack_levels(float k0, float k1, float k2, float k3, float off) {
+    // levels are small integers held exactly in floats; off shifts them into the output type
+    const uint32_t b0 = static_cast<uint32_t>(static_cast<int>(k0 + off)) & 0xffu;
+    const uint32_t b1 = static_cast<uint32_t>(static_cast<int>(k1 + off)) & 0xffu;
+    const uint32_t b2 = static_cast<uint32_t>(static_cast<int>(k2 + off)) & 0xffu;
+    const uint32_t b3 = static_cast<uint32_t>(static_cast<int>(k3 + off)) & 0xffu;
+    return b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+}
+
+// [N, C, HW] f32 -> same layout, one byte per element.  hw4 = HW / 4 (HW % 4 == 0).
+template <bool RCP>
+__global__ __launch_bounds__(kThreads) void fq_nchw_q8_vec4(const float4* __restrict__ x,
+                                                             uint32_t* __restrict__ y,
+                                                             const FqChannel* __restrict__ tab,
+                                                             float lm1, float off, int64_t n4,
+                                                             uint32_t hw4, uint32_t C) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n4; i += stride) {
+        const uint32_t plane = static_cast<uint32_t>(i / hw4);
+        const FqChannel p = tab[plane % C];
+        const float4 v = x[i];
+        y[i] = pack_levels(fq_level_clamped<RCP>(p, lm1, v.x), fq_level_clamped<RCP>(p, lm1, v.y),
+                           fq_level_clamped<RCP>(p, lm1, v.z), fq_level_clamped<RCP>(p, lm1, v.w),
+                           off);
+    }
+}
+
+// any HW: one element per thread-iteration
+template <bool RCP>
+__global__ __launch_bounds__(kThreads) void fq_nchw_q8_scalar(const float* __restrict__ x,
+                                                               uint8_t* __restrict__ y,
+                                                               const FqChannel* __restrict__ tab,
+                                                               float lm1, float off, int64_t n,
+                                                               uint32_t hw, uint32_t C) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) {
+        const FqChannel p = tab[static_cast<uint32_t>(i / hw) % C];
+        y[i] = static_cast<uint8_t>(static_cast<int>(fq_level_clamped<RCP>(p, lm1, x[i]) + off));
+    }
+}
+
+// f32 op form, same layout
+template <bool RCP>
+__global__ __launch_bounds__(kThreads) void fq_nchw_f32(const float* __restrict__ x,
+                                                         float* __restrict__ y,
+                                                         const FqChannel* __restrict__ tab,
+                                                         float lm1, int64_t n, uint32_t hw,
+                                                         uint32_t C) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) {
+        const FqChannel p = tab[static_cast<uint32_t>(i / hw) % C];
+        y[i] = fq_value<RCP>(p, lm1, x[i]);
+    }
+}
+
+template <bool RCP>
+__global__ __launch_bounds__(kThreads) void fq_nchw_f32_vec4(const float4* __restrict__ x,
+                                                              float4* __restrict__ y,
+                                                              const FqChannel* __restrict__ tab,
+                                                              float lm1, int64_t n4, uint32_t hw4,
+                                                              uint32_t C) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n4; i += stride) {
+        const FqChannel p = tab[static_cast<uint32_t>(i / hw4) % C];
+        const float4 v = x[i];
+        float4 o;
+        o.x = fq_value<RCP>(p, lm1, v.x);
+        o.y = fq_value<RCP>(p, lm1, v.y);
+        o.z = fq_value<RCP>(p, lm1, v.z);
+        o.w = fq_value<RCP>(p, lm1, v.w);
+        y[i] = o;
+    }
+}
+
+// [N, C, HW] f32 -> [N, HW, c_stride] bytes.  A block transposes 64 pixels x 64 channels
+// through LDS so that both the f32 reads (256 B per channel row) and the byte writes (16 B per
+// thread, whole pixels contiguous) are coalesced.  grid = (N * ceil(HW/64), ceil(c_stride/64)).
+template <bool RCP>
+__global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc_q8(const float* __restrict__ x,
+                                                                uint8_t* __restrict__ y,
+                                                                const FqChannel* __restrict__ tab,
+                                                                float lm1, float off, uint32_t hw,
+                                                                uint32_t C, uint32_t c_stride,
+                                                                uint32_t tiles_per_image) {
+    __shared__ uint32_t tile[64][17];  // [pixel][16 dwords = 64 channel bytes] + 1 pad
+    const uint32_t n = blockIdx.x / tiles_per_image;
+    const uint32_t p0 = (blockIdx.x % tiles_per_image) * 64;
+    const uint32_t c0 = blockIdx.y * 64;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t pix = p0 + lane;
+    // each wave quantises 16 channels of the 64; a lane owns one pixel and packs 4 channels/dword
+    for (uint32_t cc = 0; cc < 16; cc += 4) {
+        float k[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t c = c0 + wave * 16 + cc + j;
+            if (c < C && pix < hw) {
+                const FqChannel p = tab[c];
+                k[j] = fq_level_clamped<RCP>(p, lm1, x[(static_cast<int64_t>(n) * C + c) * hw + pix]);
+            } else {
+                k[j] = 0.0f;
+            }
+        }
+        tile[lane][wave * 4 + cc / 4] = pack_levels(k[0], k[1], k[2], k[3], off);
+    }
+    __syncthreads();
+    // 256 threads x 16 B: thread t writes channels [16*(t%4), +16) of pixel t/4
+    const uint32_t op = threadIdx.x >> 2, oq = threadIdx.x & 3;
+    const uint32_t cbyte = c0 + oq * 16;
+    if (p0 + op < hw && cbyte < c_stride) {
+        uint4 v;
+        v.x = tile[op][oq * 4 + 0];
+        v.y = tile[op][oq * 4 + 1];
+        v.z = tile[op][oq * 4 + 2];
+        v.w = tile[op][oq * 4 + 3];
+        uint8_t* dst = y + (static_cast<int64_t>(n) * hw + p0 + op) * c_stride + cbyte;
+        if (cbyte + 16 <= c_stride && c_stride % 16 == 0) {
+            *reinterpret_cast<uint4*>(dst) = v;
+        } else {  // c_stride is a multiple of 4
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+            for (uint32_t j = 0; j < 4 && cbyte + 4 * j < c_stride; ++j)
+                reinterpret_cast<uint32_t*>(dst)[j] = w[j];
+        }
+    }
+}
+
+int grid_for(int64_t work_items) {
+    // enough blocks to fill 256 CUs several times over, capped so the grid-stride loop amortises
+    const int64_t blocks = ceil_div(work_items, kThreads);
+    return static_cast<int>(std::min<int64_t>(blocks, 256 * 16));
+}
+
+// r = correctly rounded 1/d: pick among the neighbours of (float)(1.0/d) the one whose exact
+// residual |1 - d*r| (a product of two floats is exact in double) is smallest.
+float rounded_reciprocal(float d) {
+    float r = static_cast<float>(1.0 / static_cast<double>(d));
+    float best = r;
+    double best_err = std::fabs(1.0 - static_cast<double>(d) * r);
+    for (float cand : {std::nextafterf(r, INFINITY), std::nextafterf(r, -INFINITY)}) {
+        const double err = std::fabs(1.0 - static_cast<double>(d) * cand);
+        if (err < best_err) { best = cand; best_err = err; }
+    }
+    return best;
+}
+
+// monotone map float <-> ordered int, for bisection over floats
+int32_t ordered(float f) {
+    int32_t i;
+    std::memcpy(&i, &f, 4);
+    return i < 0 ? static_cast<int32_t>(0x80000000u - static_cast<uint32_t>(i)) : i;
+}
+float unordered(int32_t o) {
+    int32_t i = o < 0 ? static_cast<int32_t>(0x80000000u - static_cast<uint32_t>(o)) : o;
+    float f;
+    std::memcpy(&f, &i, 4);
+    return f;
+}
+
+}  // namespace
+
+bool fq_reciprocal_exact_on_boundaries(const FqChannel& p, float lm1) {
+    if (!(p.il < p.ih)) return false;
+    if (!(std::fabs(p.d) > 0x1p-60f && std::fabs(p.d) < 0x1p60f)) return false;
+    uint32_t bits;
+    std::memcpy(&bits, &p.d, 4);
+    if ((bits & 0x7fffffu) == 0x7fffffu) return false;  // all-ones significand: excluded by the theorem
+    const int levels = static_cast<int>(lm1) + 1;
+    const int32_t o_lo = ordered(p.il), o_hi = ordered(p.ih);
+    for (int k = 1; k < levels; ++k) {
+        // smallest x in (il, ih] whose reference level is >= k (the level is monotone in x)
+        int32_t a = o_lo, b = o_hi;  // level(a) < k <= level(b)
+        if (fq_level_div(p, lm1, p.ih) < k) break;
+        while (b - a > 1) {
+            const int32_t m = a + (b - a) / 2;
+            if (fq_level_div(p, lm1, unordered(m)) >= k) b = m; else a = m;
+        }
+        for (int32_t o : {a, b, b + 1 <= o_hi ? b + 1 : b, a - 1 >= o_lo ? a - 1 : a}) {
+            const float x = unordered(o);
+            if (fq_level_rcp(p, lm1, x) != fq_level_div(p, lm1, x)) return false;
+        }
+    }
+    return true;
+}
+
+}  // namespace hipie
+
+using namespace hipie;
+
+struct hipie_fq {
+    int device = 0;
+    int64_t C = 0;
+    int64_t levels = 0;
+    float lm1 = 0;
+    bool rcp = false;           // reciprocal path proven on every boundary of every channel
+    bool clamp_ok = false;      // il < ih everywhere (q8 kernels fold the saturating branches)
+    bool q8_ok = false;         // op results are the integers out_low + k
+    float q8_base = 0;          // out_low (integer valued) when q8_ok
+    std::vector<FqChannel> host;
+    DeviceBuffer table;
+};
+
+extern "C" {
+
+int hipie_fq_create(int device, int64_t channels, int64_t levels, const float* in_low,
+                    int64_t n_in_low, const float* in_high, int64_t n_in_high,
+                    const float* out_low, int64_t n_out_low, const float* out_high,
+                    int64_t n_out_high, hipie_fq** out) {
+    return guarded([&] {
+        HIPIE_REQUIRE(out && in_low && in_high && out_low && out_high, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_fq_create: null argument");
+        HIPIE_REQUIRE(channels > 0 && levels >= 2 && levels <= 65536, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_fq_create: channels=%lld levels=%lld", (long long)channels,
+                      (long long)levels);
+        for (int64_t n : {n_in_low, n_in_high, n_out_low, n_out_high})
+            HIPIE_REQUIRE(n == 1 || n == channels, HIPIE_PARAMETER_MISMATCH,
+                          "hipie_fq_create: a bound has %lld values, expected 1 or %lld",
+                          (long long)n, (long long)channels);
+        auto fq = std::make_unique<hipie_fq>();
+        fq->device = device;
+        fq->C = channels;
+        fq->levels = levels;
+        fq->lm1 = static_cast<float>(static_cast<size_t>(levels - 1));
+        fq->host.resize(channels);
+        fq->rcp = true;
+        fq->clamp_ok = true;
+        for (int64_t c = 0; c < channels; ++c) {
+            FqChannel& p = fq->host[c];
+            p.il = in_low[n_in_low == 1 ? 0 : c];
+            p.ih = in_high[n_in_high == 1 ? 0 : c];
+            p.ol = out_low[n_out_low == 1 ? 0 : c];
+            p.oh = out_high[n_out_high == 1 ? 0 : c];
+            p.lo = std::min(p.il, p.ih);
+            p.hi = std::max(p.il, p.ih);
+            p.d = p.ih - p.il;
+            p.r = (p.d != 0.0f && std::isfinite(p.d)) ? rounded_reciprocal(p.d) : 0.0f;
+            if (!(p.il < p.ih)) fq->clamp_ok = false;
+        }
+        std::atomic<bool> all_exact{true};
+        parallel_for(channels, [&](int64_t c) {
+            if (!fq_reciprocal_exact_on_boundaries(fq->host[c], fq->lm1)) all_exact = false;
+        });
+        fq->rcp = all_exact;
+        // integer output forms: scalar out range whose op results are out_low + k exactly
+        if (n_out_low == 1 && n_out_high == 1 && levels <= 256) {
+            const float ol = out_low[0], oh = out_high[0];
+            bool ok = ol == std::nearbyintf(ol) && ol >= -128.0f && ol + fq->lm1 <= 255.0f;
+            for (int k = 0; ok && k < levels; ++k)
+                ok = (static_cast<float>(k) / fq->lm1 * (oh - ol) + ol) == ol + static_cast<float>(k);
+            // x > max(il, ih) returns out_high itself, which must be the last level
+            ok = ok && oh == ol + fq->lm1;
+            fq->q8_ok = ok;
+            fq->q8_base = ol;
+        }
+        // device < 0: host-only object for load-time checks without a GPU; it cannot run
+        if (device >= 0) fq->table.upload(device, fq->host.data(), sizeof(FqChannel) * channels);
+        *out = fq.release();
+    });
+}
+
+void hipie_fq_destroy(hipie_fq* fq) { delete fq; }
+
+int hipie_fq_uses_reciprocal(const hipie_fq* fq) { return fq && fq->rcp ? 1 : 0; }
+
+float hipie_fq_host_eval(const hipie_fq* fq, int64_t channel, float x) {
+    if (!fq || channel < 0 || channel >= fq->C) return NAN;
+    return fq->rcp ? fq_value<true>(fq->host[channel], fq->lm1, x)
+                   : fq_value<false>(fq->host[channel], fq->lm1, x);
+}
+
+int hipie_fq_run_f32(const hipie_fq* fq, const float* x, float* y, int64_t n, int64_t hw,
+                     void* stream) {
+    return guarded([&] {
+        HIPIE_REQUIRE(fq, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_f32: null handle");
+        if (n == 0 || hw == 0) return;  // empty tensor: nothing to do, pointers may be null
+        HIPIE_REQUIRE(x && y, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_f32: null argument");
+        HIPIE_REQUIRE(fq->table.ptr, HIPIE_NOT_ALLOCATED, "hipie_fq_run_f32: host-only object");
+        HIPIE_REQUIRE(n >= 0 && hw >= 0 && hw < (1ll << 31), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_fq_run_f32: n=%lld hw=%lld", (long long)n, (long long)hw);
+        const int64_t total = n * fq->C * hw;
+        if (total == 0) return;
+        DeviceGuard g(fq->device);
+        const FqChannel* tab = fq->table.as<FqChannel>();
+        const uint32_t C = static_cast<uint32_t>(fq->C);
+        const bool vec = hw % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) &&
+                         (reinterpret_cast<uintptr_t>(y) % 16 == 0);
+        hipStream_t s = as_stream(stream);
+        if (vec) {
+            const int64_t n4 = total / 4;
+            auto k = fq->rcp ? fq_nchw_f32_vec4<true> : fq_nchw_f32_vec4<false>;
+            hipLaunchKernelGGL(k, dim3(grid_for(n4)), dim3(kThreads), 0, s,
+                               reinterpret_cast<const float4*>(x), reinterpret_cast<float4*>(y),
+                               tab, fq->lm1, n4, static_cast<uint32_t>(hw / 4), C);
+        } else {
+            auto k = fq->rcp ? fq_nchw_f32<true> : fq_nchw_f32<false>;
+            hipLaunchKernelGGL(k, dim3(grid_for(total)), dim3(kThreads), 0, s, x, y, tab, fq->lm1,
+                               total, static_cast<uint32_t>(hw), C);
+        }
+        HIPIE_CHECK_HIP(hipGetLastError());
+    });
+}
+
+int hipie_fq_run_q8(const hipie_fq* fq, const float* x, void* y, int64_t n, int64_t hw,
+                    hipie_dtype out_dtype, hipie_layout out_layout, int64_t c_stride,
+                    void* stream) {
+    return guarded([&] {
+        HIPIE_REQUIRE(fq, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8: null handle");
+        if (n == 0 || hw == 0) return;  // empty tensor: nothing to do, pointers may be null
+        HIPIE_REQUIRE(x && y, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8: null argument");
+        HIPIE_REQUIRE(fq->table.ptr, HIPIE_NOT_ALLOCATED, "hipie_fq_run_q8: host-only object");
+        HIPIE_REQUIRE(n >= 0 && hw >= 0 && hw < (1ll << 31), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_fq_run_q8: n=%lld hw=%lld", (long long)n, (long long)hw);
+        HIPIE_REQUIRE(fq->q8_ok && fq->clamp_ok, HIPIE_NOT_IMPLEMENTED,
+                      "hipie_fq_run_q8: needs input_low < input_high and a scalar output range "
+                      "whose %lld values are consecutive integers in [-128, 255]",
+                      (long long)fq->levels);
+        float off;
+        switch (out_dtype) {
+        case HIPIE_U8:
+            HIPIE_REQUIRE(fq->q8_base >= 0, HIPIE_PARAMETER_MISMATCH,
+                          "hipie_fq_run_q8: negative levels do not fit u8");
+            off = fq->q8_base;
+            break;
+        case HIPIE_U8B:
+            HIPIE_REQUIRE(fq->q8_base >= 0, HIPIE_PARAMETER_MISMATCH,
+                          "hipie_fq_run_q8: negative levels do not fit u8");
+            off = fq->q8_base - 128.0f;
+            break;
+        case HIPIE_I8:
+            HIPIE_REQUIRE(fq->q8_base + fq->lm1 <= 127.0f, HIPIE_PARAMETER_MISMATCH,
+                          "hipie_fq_run_q8: levels do not fit i8");
+            off = fq->q8_base;
+            break;
+        default:
+            fail(HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8: out_dtype %d", (int)out_dtype);
+        }
+        const int64_t total = n * fq->C * hw;
+        if (total == 0) return;
+        DeviceGuard g(fq->device);
+        const FqChannel* tab = fq->table.as<FqChannel>();
+        const uint32_t C = static_cast<uint32_t>(fq->C);
+        hipStream_t s = as_stream(stream);
+        if (out_layout == HIPIE_NCHW) {
+            const bool vec = hw % 4 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 == 0) &&
+                             (reinterpret_cast<uintptr_t>(y) % 4 == 0);
+            if (vec) {
+                const int64_t n4 = total / 4;
+                auto k = fq->rcp ? fq_nchw_q8_vec4<true> : fq_nchw_q8_vec4<false>;
+                hipLaunchKernelGGL(k, dim3(grid_for(n4)), dim3(kThreads), 0, s,
+                                   reinterpret_cast<const float4*>(x),
+                                   static_cast<uint32_t*>(y), tab, fq->lm1, off, n4,
+                                   static_cast<uint32_t>(hw / 4), C);
+            } else {
+                auto k = fq->rcp ? fq_nchw_q8_scalar<true> : fq_nchw_q8_scalar<false>;
+                hipLaunchKernelGGL(k, dim3(grid_for(total)), dim3(kThreads), 0, s, x,
+                                   static_cast<uint8_t*>(y), tab, fq->lm1, off, total,
+                                   static_cast<uint32_t>(hw), C);
+            }
+        } else if (out_layout == HIPIE_NHWC) {
+            HIPIE_REQUIRE(c_stride >= fq->C && c_stride % 4 == 0, HIPIE_PARAMETER_MISMATCH,
+                          "hipie_fq_run_q8: c_stride=%lld must be a multiple of 4 >= C=%lld",
+                          (long long)c_stride, (long long)fq->C);
+            HIPIE_REQUIRE(reinterpret_cast<uintptr_t>(y) % 16 == 0 || c_stride % 16 != 0,
+                          HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8: output must be 16 B aligned");
+            const uint32_t tiles = static_cast<uint32_t>(ceil_div(hw, 64));
+            const int64_t gx = n * tiles;
+            HIPIE_REQUIRE(gx < (1ll << 31), HIPIE_OUT_OF_BOUNDS, "hipie_fq_run_q8: grid too large");
+            auto k = fq->rcp ? fq_nchw_to_nhwc_q8<true> : fq_nchw_to_nhwc_q8<false>;
+            hipLaunchKernelGGL(k, dim3(static_cast<uint32_t>(gx),
+                                       static_cast<uint32_t>(ceil_div(c_stride, 64))),
+                               dim3(kThreads), 0, s, x, static_cast<uint8_t*>(y), tab, fq->lm1, off,
+                               static_cast<uint32_t>(hw), C, static_cast<uint32_t>(c_stride), tiles);
+        } else {
+            fail(HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8: out_layout %d", (int)out_layout);
+        }
+        HIPIE_CHECK_HIP(hipGetLastError());
+    });
+}
+
+}  // extern "C"

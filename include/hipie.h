@@ -1,0 +1,114 @@
+/*
+ * hipie — C ABI of the MI355X (gfx950) INT8 execution engine.
+ *
+ * This is the boundary an OpenVINO 2021.4 device plugin binds: plain pointers, sizes and opaque
+ * handles, no C++ types, no exceptions.  Every call returns a hipie_status (0 = OK) that mirrors
+ * InferenceEngine::StatusCode (inference-engine/include/ie_common.h:231-249); the message of the
+ * last failure on the calling thread is available from hipie_last_error().
+ *
+ * Two levels are exported:
+ *   1. operator level  — one "create" (load time: validates, packs constants, uploads them) and
+ *      one "run" (enqueue on a HIP stream; allocates nothing, never synchronises) per reference
+ *      kernel of the INT8 path.  Each declaration cites the reference function it replaces.
+ *   2. graph level     — the post-LPT nGraph Function described node by node, compiled into a
+ *      plan over one static HBM arena, and executed by infer requests; this is what
+ *      IInferencePlugin::LoadExeNetworkImpl / IInferRequestInternal::InferImpl bind
+ *      (inference-engine/src/plugin_api/cpp_interfaces/interface/ie_iplugin_internal.hpp:270,
+ *       ie_iinfer_request_internal.hpp:57).
+ *
+ * Device pointers are raw HIP device addresses; `stream` is a hipStream_t passed as void*
+ * (NULL = the null stream).  Unless stated otherwise tensors are dense, row-major.
+ *
+ * Activation storage inside the engine ("U8B"): a u8 quantisation level q is stored as the
+ * signed byte q - 128 (bit pattern q ^ 0x80), NHWC, channels padded to a multiple of 16 with
+ * level 0.  CDNA4 int8 MFMA multiplies signed bytes only; the constant 128 * sum(w) is folded
+ * into the per-channel bias at load time, which keeps the integer sum exactly the u8 x i8 one.
+ */
+#ifndef HIPIE_H
+#define HIPIE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ie_common.h:231-249 (StatusCode) */
+typedef enum hipie_status {
+    HIPIE_OK = 0,
+    HIPIE_GENERAL_ERROR = -1,
+    HIPIE_NOT_IMPLEMENTED = -2,
+    HIPIE_NETWORK_NOT_LOADED = -3,
+    HIPIE_PARAMETER_MISMATCH = -4,
+    HIPIE_NOT_FOUND = -5,
+    HIPIE_OUT_OF_BOUNDS = -6,
+    HIPIE_UNEXPECTED = -7,
+    HIPIE_REQUEST_BUSY = -8,
+    HIPIE_RESULT_NOT_READY = -9,
+    HIPIE_NOT_ALLOCATED = -10,
+    HIPIE_INFER_NOT_STARTED = -11,
+    HIPIE_NETWORK_NOT_READ = -12,
+    HIPIE_INFER_CANCELLED = -13
+} hipie_status;
+
+/* element types (numbering of InferenceEngine::Precision::ePrecision, ie_precision.hpp:27-48,
+ * plus the engine's internal biased-u8 storage) */
+typedef enum hipie_dtype {
+    HIPIE_F32 = 10,
+    HIPIE_U8 = 40,
+    HIPIE_I8 = 50,
+    HIPIE_I32 = 70,
+    HIPIE_U8B = 41 /* u8 level stored as (level - 128); engine-internal */
+} hipie_dtype;
+
+typedef enum hipie_layout { HIPIE_NCHW = 1, HIPIE_NHWC = 2 } hipie_layout; /* ie_common.h:70-100 */
+
+const char* hipie_last_error(void);
+/* "major.minor gfx950" build string */
+const char* hipie_version(void);
+/* number of visible HIP devices, their names (AVAILABLE_DEVICES / FULL_DEVICE_NAME metrics) */
+int hipie_device_count(void);
+int hipie_device_name(int device, char* buf, size_t buf_len);
+
+/* ======================================================================================
+ * 1a. FakeQuantize — ngraph/core/reference/.../fake_quantize.hpp:175-194 (quantize),
+ *     :199-265 (broadcast driver).  Data is [N, C, HW] (NCHW with the spatial dims flattened);
+ *     each bound is a host array of length 1 (scalar) or C (per channel, shape [1,C,1,1] or
+ *     [C,1,1] in the reference).  Bit-exact with the reference expression
+ *         x <= min(il,ih) ? ol : x > max(il,ih) ? oh
+ *           : nearbyint((x-il)/(ih-il)*(L-1))/(L-1)*(oh-ol)+ol        (float, ties-to-even).
+ * ==================================================================================== */
+typedef struct hipie_fq hipie_fq;
+
+/* device < 0 builds a host-only object (load-time checks without a GPU); its run calls return
+ * HIPIE_NOT_ALLOCATED. */
+int hipie_fq_create(int device, int64_t channels, int64_t levels,
+                    const float* in_low, int64_t n_in_low, const float* in_high, int64_t n_in_high,
+                    const float* out_low, int64_t n_out_low, const float* out_high,
+                    int64_t n_out_high, hipie_fq** fq);
+void hipie_fq_destroy(hipie_fq* fq);
+
+/* op form: f32 in, f32 out, same layout (what reference::fake_quantize<float> returns) */
+int hipie_fq_run_f32(const hipie_fq* fq, const float* x, float* y, int64_t n, int64_t hw,
+                     void* stream);
+/* post-LPT form (network_helper.cpp:943-1087: FQ with out range [0, L-1] and u8 output):
+ * writes static_cast<uint8_t>(op result).  Requires scalar out_low/out_high whose op results are
+ * the integers out_low + k; HIPIE_NOT_IMPLEMENTED otherwise. out_layout NCHW keeps the layout;
+ * NHWC writes [N, HW, c_stride] (c_stride >= C, multiple of 16, padding = level 0).
+ * out_dtype: HIPIE_U8 (plain level), HIPIE_U8B (level - 128), HIPIE_I8 (signed levels). */
+int hipie_fq_run_q8(const hipie_fq* fq, const float* x, void* y, int64_t n, int64_t hw,
+                    hipie_dtype out_dtype, hipie_layout out_layout, int64_t c_stride,
+                    void* stream);
+
+/* host evaluation of exactly the arithmetic the device kernel uses (reciprocal multiply with
+ * two FMA corrections); the planner checks it against IEEE division at every level boundary of
+ * every channel and falls back to the dividing kernel if any differs. */
+float hipie_fq_host_eval(const hipie_fq* fq, int64_t channel, float x);
+/* 1 when the reciprocal path was proven equal to division on all boundaries of all channels */
+int hipie_fq_uses_reciprocal(const hipie_fq* fq);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPIE_H */
