@@ -1,0 +1,23 @@
+// Host-side pieces of the MFMA convolution shared with MatMul and the graph planner.
+#pragma once
+#include <atomic>
+
+#include "common.h"
+#include "conv_kernel.h"
+#include "fq.h"
+
+namespace hipie {
+
+// Per-channel epilogue tables on the device (padded to the packed channel count) + flags.
+struct Epilogue {
+    int device = 0;
+    uint32_t flags = 0;
+    int out_dtype = HIPIE_F32;
+    float lm1 = 0, out_off = 0, clamp_lo = 0, clamp_hi = 0;
+    DeviceBuffer bias, scale, res_sub, res_mul, post_scale, fq_il, fq_ih, fq_d, fq_r;
+    std::vector<float> host_bias;
+    void build(int device, const hipie_epilogue& e, int64_t oc, int64_t ocp);
+    void fill(ConvArgs& a) const;
+};
+
+}  // namespace hipie

@@ -1,0 +1,74 @@
+// u8/i8 x i8 -> i32 implicit-GEMM convolution on CDNA4 int8 MFMA with a fused f32 epilogue.
+//
+// Reference semantics: reference::convolution<int32_t> on widened inputs
+// (ngraph/core/reference/.../convolution.hpp:63-146) followed by the post-LPT elementwise chain
+// (Add bias, Multiply, residual Add, ReLU/Clamp, FakeQuantize) evaluated one IEEE f32 operation
+// at a time in graph order, so the u8 levels are the reference's bit for bit.
+//
+// GEMM view: rows = output channels (MFMA A operand, packed weights [OCp][Kp]), columns = output
+// pixels (MFMA B operand, NHWC activations gathered through a per-16-byte offset table),
+// K = (kh, kw, ic).  v_mfma_i32_32x32x32_i8: lane l feeds row/col l%32 with the 16 K-bytes
+// starting at 16*(l/32); it receives rows 8*(r/4) + 4*(l/32) + r%4 of column l%32.
+// Weight rows are read through a permutation so that each lane ends up with 32 CONSECUTIVE
+// output channels of one pixel: results leave as 16-byte stores into NHWC.
+//
+// A workgroup owns (WOC*64) channels x (WPIX*64) pixels; each wave a 64x64 tile (2x2 MFMA
+// tiles, 64 accumulator registers).  K advances 64 bytes per step; global loads for step k+1
+// are issued before the MFMAs of step k and land in the other LDS buffer (one barrier per step).
+// LDS rows are 64 data bytes + 16 pad (stride 80 B = 20 banks): ds_read_b128 of 16 consecutive
+// rows touches distinct banks.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hipie {
+
+enum ConvFlags : uint32_t {
+    CF_BIAS = 1u << 0,        // v += bias[c]
+    CF_SCALE = 1u << 1,       // v *= scale[c]
+    CF_RES = 1u << 2,         // residual operand present
+    CF_RES_F32 = 1u << 3,     // residual is f32 (else U8B / I8 bytes converted to float)
+    CF_RES_SUB = 1u << 4,     // r -= res_sub[c]
+    CF_RES_MUL = 1u << 5,     // r *= res_mul[c]
+    CF_POST_SCALE = 1u << 6,  // v *= post_scale[c]   (after the residual add)
+    CF_RELU = 1u << 7,        // v = v > 0 ? v : 0
+    CF_CLAMP = 1u << 8,       // v = clamp(v, clamp_lo, clamp_hi)
+    CF_OUT_FQ = 1u << 9,      // FakeQuantize -> one byte per element
+    CF_OUT_I32 = 1u << 10,    // raw accumulators (integer parity tests, MatMul without epilogue)
+    CF_FQ_RCP = 1u << 11,     // reciprocal evaluation of the FQ division (proven at load time)
+    CF_RES_U8B = 1u << 12,    // residual bytes are level-128 (add 128 after conversion)
+};
+
+struct ConvArgs {
+    const int8_t* in;     // element (n=0, h=0, w=0, c=0) of the input tensor
+    const int8_t* wgt;    // packed [OCp][Kp]
+    void* out;            // element (0,0,0,0) of the output tensor
+    const void* res;      // residual tensor or nullptr
+    const int32_t* koff;  // [Kp/16] byte offset of every 16-byte K piece relative to the window origin
+    // per-channel tables, each [OCp]
+    const int32_t* corr;  // 128 * sum_k w[oc][k] for U8B inputs (0 for I8)
+    const float* bias;
+    const float* scale;
+    const float* res_sub;
+    const float* res_mul;
+    const float* post_scale;
+    const float* fq_il;
+    const float* fq_ih;
+    const float* fq_d;
+    const float* fq_r;
+    int32_t M;            // N * OH * OW
+    int32_t OW, OHOW;
+    int32_t in_sn, in_sh, in_sw;     // input strides in bytes
+    int32_t conv_sh, conv_sw;        // convolution strides
+    int32_t in_origin;               // -(pad_top * in_sh + pad_left * in_sw)
+    int32_t out_sn, out_sh, out_sw;  // output strides in elements
+    int32_t res_sn, res_sh, res_sw;  // residual strides in elements
+    int32_t OC, OCp;
+    int32_t nk;                      // Kp / 64
+    int32_t Kp;
+    int32_t p_tiles, t_tiles, p_per_xcd;
+    uint32_t flags;
+    float lm1, out_off, clamp_lo, clamp_hi;
+};
+
+}  // namespace hipie

@@ -12,4 +12,7 @@ namespace hipie {
 // around every step of the reference means agreement everywhere between il and ih).
 bool fq_reciprocal_exact_on_boundaries(const FqChannel& p, float lm1);
 
+// r = correctly rounded 1/d
+float fq_rounded_reciprocal(float d);
+
 }  // namespace hipie

@@ -150,7 +150,9 @@ int grid_for(int64_t work_items) {
 
 // r = correctly rounded 1/d: pick among the neighbours of (float)(1.0/d) the one whose exact
 // residual |1 - d*r| (a product of two floats is exact in double) is smallest.
-float rounded_reciprocal(float d) {
+}  // namespace
+
+float fq_rounded_reciprocal(float d) {
     float r = static_cast<float>(1.0 / static_cast<double>(d));
     float best = r;
     double best_err = std::fabs(1.0 - static_cast<double>(d) * r);
@@ -160,6 +162,8 @@ float rounded_reciprocal(float d) {
     }
     return best;
 }
+
+namespace {
 
 // monotone map float <-> ordered int, for bisection over floats
 int32_t ordered(float f) {
@@ -250,7 +254,7 @@ int hipie_fq_create(int device, int64_t channels, int64_t levels, const float* i
             p.lo = std::min(p.il, p.ih);
             p.hi = std::max(p.il, p.ih);
             p.d = p.ih - p.il;
-            p.r = (p.d != 0.0f && std::isfinite(p.d)) ? rounded_reciprocal(p.d) : 0.0f;
+            p.r = (p.d != 0.0f && std::isfinite(p.d)) ? fq_rounded_reciprocal(p.d) : 0.0f;
             if (!(p.il < p.ih)) fq->clamp_ok = false;
         }
         std::atomic<bool> all_exact{true};

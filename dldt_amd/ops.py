@@ -88,3 +88,96 @@ class FakeQuantize:
                                     ctypes.c_int(NCHW if layout == "nchw" else NHWC),
                                     ctypes.c_int64(cs), _stream()))
         return y
+
+
+class hipie_epilogue(ctypes.Structure):
+    _fp = ctypes.POINTER(ctypes.c_float)
+    _fields_ = [("bias", _fp), ("n_bias", ctypes.c_int64), ("scale", _fp), ("n_scale", ctypes.c_int64),
+                ("residual_dtype", ctypes.c_int32),
+                ("res_sub", _fp), ("n_res_sub", ctypes.c_int64), ("res_mul", _fp), ("n_res_mul", ctypes.c_int64),
+                ("post_scale", _fp), ("n_post_scale", ctypes.c_int64),
+                ("activation", ctypes.c_int32), ("clamp_lo", ctypes.c_float), ("clamp_hi", ctypes.c_float),
+                ("out_dtype", ctypes.c_int32), ("fq_levels", ctypes.c_int64),
+                ("fq_in_low", _fp), ("n_fq_in_low", ctypes.c_int64),
+                ("fq_in_high", _fp), ("n_fq_in_high", ctypes.c_int64),
+                ("fq_out_low", ctypes.c_float), ("fq_out_high", ctypes.c_float)]
+
+
+class hipie_conv_desc(ctypes.Structure):
+    _fields_ = [(k, ctypes.c_int32) for k in (
+        "in_dtype", "ic", "oc", "kh", "kw", "stride_h", "stride_w", "dil_h", "dil_w",
+        "pad_top", "pad_left", "pad_bottom", "pad_right", "groups", "in_c_stride",
+        "in_stride_h", "in_stride_w")]
+
+
+def make_epilogue(bias=None, scale=None, residual_dtype=0, res_sub=None, res_mul=None,
+                  post_scale=None, activation=None, clamp=(0.0, 0.0), out_dtype=F32,
+                  fq=None):
+    """fq = (levels, in_low, in_high, out_low, out_high) for 8-bit outputs."""
+    e = hipie_epilogue()
+    keep = []
+
+    def put(name, v):
+        if v is None:
+            return
+        a = np.ascontiguousarray(np.asarray(v, np.float32).reshape(-1))
+        keep.append(a)
+        setattr(e, name, _fptr(a))
+        setattr(e, "n_" + name, a.size)
+
+    put("bias", bias)
+    put("scale", scale)
+    e.residual_dtype = residual_dtype
+    put("res_sub", res_sub)
+    put("res_mul", res_mul)
+    put("post_scale", post_scale)
+    e.activation = {None: 0, "relu": 1, "clamp": 2}[activation]
+    e.clamp_lo, e.clamp_hi = float(clamp[0]), float(clamp[1])
+    e.out_dtype = out_dtype
+    if fq is not None:
+        e.fq_levels = int(fq[0])
+        put("fq_in_low", fq[1])
+        put("fq_in_high", fq[2])
+        e.fq_out_low, e.fq_out_high = float(fq[3]), float(fq[4])
+    e._keep = keep
+    return e
+
+
+class Convolution:
+    """u8/i8 x i8 convolution with fused epilogue (ngraph Convolution-1 after LPT).
+
+    ``weights`` is int8 OIHW; ``in_tensor`` fixes the input geometry the weights are packed for.
+    """
+
+    def __init__(self, weights, in_tensor, strides=(1, 1), dilations=(1, 1), pads_begin=(0, 0),
+                 pads_end=(0, 0), epilogue=None, device=0):
+        w = np.ascontiguousarray(weights, np.int8)
+        self.oc, self.ic, self.kh, self.kw = w.shape
+        d = hipie_conv_desc(in_tensor.dtype, self.ic, self.oc, self.kh, self.kw, strides[0], strides[1],
+                            dilations[0], dilations[1], pads_begin[0], pads_begin[1], pads_end[0],
+                            pads_end[1], 1, in_tensor.cs, in_tensor.stride_h, in_tensor.stride_w)
+        self.epilogue = epilogue or make_epilogue(out_dtype=I32)
+        self._h = ctypes.c_void_p()
+        check(lib().hipie_conv_create(ctypes.c_int(device), ctypes.byref(d),
+                                      w.ctypes.data_as(ctypes.c_void_p), ctypes.byref(self.epilogue),
+                                      ctypes.byref(self._h)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().hipie_conv_destroy(self._h)
+            self._h = None
+
+    def out_dims(self, h, w):
+        oh, ow = ctypes.c_int32(), ctypes.c_int32()
+        check(lib().hipie_conv_out_dims(self._h, h, w, ctypes.byref(oh), ctypes.byref(ow)))
+        return oh.value, ow.value
+
+    def set_tile(self, tile):
+        check(lib().hipie_conv_set_tile(self._h, tile))
+
+    def run(self, x, out, residual=None):
+        xd, od = x.desc(), out.desc()
+        rd = residual.desc() if residual is not None else None
+        check(lib().hipie_conv_run(self._h, ctypes.byref(xd), ctypes.byref(rd) if rd else None,
+                                   ctypes.byref(od), _stream()))
+        return out

@@ -108,6 +108,80 @@ float hipie_fq_host_eval(const hipie_fq* fq, int64_t channel, float x);
 /* 1 when the reciprocal path was proven equal to division on all boundaries of all channels */
 int hipie_fq_uses_reciprocal(const hipie_fq* fq);
 
+/* ======================================================================================
+ * Activation tensors handed to the engine's kernels: NHWC, channel stride 1, with a readable
+ * border ("halo") of `halo` pixels around every image plane that holds quantisation level 0.
+ * Convolution and pooling padding is read from that border instead of being bounds-checked, so
+ * a consumer with padding p needs halo >= p.  `data` addresses element (n=0,h=0,w=0,c=0).
+ * ==================================================================================== */
+typedef struct hipie_tensor {
+    void* data;
+    int32_t dtype;                        /* hipie_dtype */
+    int32_t n, h, w, c;                   /* logical dims */
+    int64_t stride_n, stride_h, stride_w; /* in elements; stride_w is the (padded) channel count */
+    int32_t halo;
+} hipie_tensor;
+
+/* ======================================================================================
+ * 1b. Fused f32 epilogue applied to i32 accumulators, in this fixed order (each step one IEEE
+ *     f32 operation, as the post-LPT graph evaluates them with reference::add / multiply /
+ *     subtract / relu / clamp / fake_quantize):
+ *        v = float(acc)                     convert.hpp
+ *        v = v + bias[c]                    Add after swapMultiplyAndAdd (network_helper.cpp:216-292)
+ *        v = v * scale[c]                   dequantization Multiply (convolution.cpp:249-258)
+ *        r = float(residual); r -= res_sub[c]; r *= res_mul[c]; v = v + r     (add.cpp:154-218)
+ *        v = v * post_scale[c]
+ *        relu | clamp(lo, hi)               relu.hpp, clamp.hpp
+ *        FakeQuantize(in_low[c], in_high[c], out_low, out_high, levels) -> 8-bit     or f32 store
+ *     Arrays are host pointers with 1 (broadcast) or OC values; NULL skips the step.
+ * ==================================================================================== */
+typedef struct hipie_epilogue {
+    const float* bias;        int64_t n_bias;
+    const float* scale;       int64_t n_scale;
+    int32_t residual_dtype;   /* 0 = none, HIPIE_F32, HIPIE_U8B (value = level), HIPIE_I8 */
+    const float* res_sub;     int64_t n_res_sub;
+    const float* res_mul;     int64_t n_res_mul;
+    const float* post_scale;  int64_t n_post_scale;
+    int32_t activation;       /* 0 none, 1 relu, 2 clamp */
+    float clamp_lo, clamp_hi;
+    int32_t out_dtype;        /* HIPIE_F32, HIPIE_U8B, HIPIE_I8, or HIPIE_I32 (raw accumulators) */
+    int64_t fq_levels;
+    const float* fq_in_low;   int64_t n_fq_in_low;
+    const float* fq_in_high;  int64_t n_fq_in_high;
+    float fq_out_low, fq_out_high;
+} hipie_epilogue;
+
+/* ======================================================================================
+ * 1c. Convolution — reference::convolution<int32_t> on widened u8/i8 inputs
+ *     (ngraph/core/reference/.../convolution.hpp:63-146, 245-293; dispatched by
+ *     ngraph/test/runtime/interpreter/evaluates_map.cpp:193-216), i.e. the TypeRelaxed
+ *     Convolution LPT emits (low_precision_transformations/src/convolution.cpp:201-259), plus
+ *     the fused epilogue above.  Weights are i8 OIHW (host); they are packed for the input
+ *     tensor's strides at creation.  i32 accumulators are exact.
+ * ==================================================================================== */
+typedef struct hipie_conv_desc {
+    int32_t in_dtype;                     /* HIPIE_U8B or HIPIE_I8 */
+    int32_t ic, oc, kh, kw;
+    int32_t stride_h, stride_w, dil_h, dil_w;
+    int32_t pad_top, pad_left, pad_bottom, pad_right;
+    int32_t groups;                       /* 1 */
+    int32_t in_c_stride;                  /* channel stride of the input tensor (>= ic) */
+    int32_t in_stride_h, in_stride_w;     /* element strides of the input tensor */
+} hipie_conv_desc;
+
+typedef struct hipie_conv hipie_conv;
+
+int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* weights_oihw,
+                      const hipie_epilogue* epilogue, hipie_conv** conv);
+void hipie_conv_destroy(hipie_conv* conv);
+/* output spatial dims for an input of h x w (convolution.hpp:168-183) */
+int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* oh, int32_t* ow);
+/* workgroup tile: 0 = 128 channels x 128 pixels, 1 = 64 x 256, 2 = 64 x 64 (chosen automatically
+ * at creation; exposed for tuning and tests) */
+int hipie_conv_set_tile(hipie_conv* conv, int tile);
+int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,
+                   const hipie_tensor* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,224 @@
+"""Convolution on int8 MFMA through the C ABI vs the oracle: exact i32 accumulators and
+bit-exact fused epilogues (bias, dequant scale, residual add, ReLU/Clamp, per-channel FQ)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+F32, I8, I32, U8B = 10, 50, 70, 41
+
+# name: (N, C, H, W, OC, KH, KW, strides, dilations, pads_begin, pads_end)
+GEOMS = {
+    "3x3_s1_p1_c64": (2, 64, 14, 14, 64, 3, 3, (1, 1), (1, 1), (1, 1), (1, 1)),
+    "1x1_c256_oc64": (2, 256, 7, 9, 64, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0)),
+    "1x1_c64_oc256": (1, 64, 15, 15, 256, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0)),
+    "1x1_s2_c128_oc512": (2, 128, 14, 14, 512, 1, 1, (2, 2), (1, 1), (0, 0), (0, 0)),
+    "3x3_s2_p1_c128": (2, 128, 13, 13, 128, 3, 3, (2, 2), (1, 1), (1, 1), (1, 1)),
+    "7x7_s2_p3_c3": (2, 3, 32, 32, 64, 7, 7, (2, 2), (1, 1), (3, 3), (3, 3)),
+    "3x3_d2_p2_c16_oc40": (1, 16, 11, 10, 40, 3, 3, (1, 1), (2, 2), (2, 2), (2, 2)),
+    "3x2_asym_c32_oc200": (3, 32, 9, 8, 200, 3, 2, (1, 2), (1, 1), (0, 1), (2, 0)),
+    "5x5_p2_c20_oc24": (1, 20, 8, 8, 24, 5, 5, (1, 1), (1, 1), (2, 2), (2, 2)),
+}
+
+
+def _inputs(rng, g, signed=False):
+    N, C, H, W, OC, KH, KW = g[:7]
+    if signed:
+        x = rng.integers(-128, 128, (N, C, H, W)).astype(np.int32)
+    else:
+        x = rng.integers(0, 256, (N, C, H, W)).astype(np.int32)
+    w = rng.integers(-127, 128, (OC, C, KH, KW)).astype(np.int32)
+    return x, w
+
+
+def _device_in(x, g, signed=False):
+    from dldt_amd import DeviceTensor
+    pb, pe = g[9], g[10]
+    halo = max(max(pb), max(pe))
+    cs = 4 if x.shape[1] <= 4 else None
+    return DeviceTensor.from_nchw(x, I8 if signed else U8B, halo=halo, c_stride=cs)
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("name", sorted(GEOMS))
+def test_conv_i32_accumulators_exact(orc, name, tile):
+    import torch
+    from dldt_amd import Convolution, DeviceTensor
+    g = GEOMS[name]
+    rng = np.random.default_rng(abs(hash(name)) % 1000)
+    x, w = _inputs(rng, g)
+    want = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    xin = _device_in(x, g)
+    conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10])
+    conv.set_tile(tile)
+    out = DeviceTensor(want.shape[0], want.shape[2], want.shape[3], want.shape[1], I32)
+    conv.run(xin, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.to_nchw(), want)
+
+
+def test_conv_i8_activations_exact(orc):
+    from dldt_amd import Convolution, DeviceTensor
+    g = GEOMS["3x3_s1_p1_c64"]
+    rng = np.random.default_rng(77)
+    x, w = _inputs(rng, g, signed=True)
+    want = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    xin = _device_in(x, g, signed=True)
+    out = DeviceTensor(want.shape[0], want.shape[2], want.shape[3], want.shape[1], I32)
+    Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10]).run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw(), want)
+
+
+def test_conv_extreme_values_do_not_overflow(orc):
+    """All-255 activations against all -127 / +127 weights at K = 4608 (the largest ResNet-50
+    reduction): |acc| = 1.49e8 < 2^31 and must come back exactly."""
+    from dldt_amd import Convolution, DeviceTensor
+    x = np.full((1, 512, 5, 5), 255, np.int32)
+    w = np.full((64, 512, 3, 3), -127, np.int32)
+    w[::2] = 127
+    want = orc.convolution(x, w, (1, 1), (1, 1), (1, 1), (1, 1))
+    assert abs(int(want.min())) > 1.4e8
+    xin = DeviceTensor.from_nchw(x, U8B, halo=1)
+    out = DeviceTensor(1, 5, 5, 64, I32)
+    Convolution(w.astype(np.int8), xin, pads_begin=(1, 1), pads_end=(1, 1)).run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw(), want)
+
+
+def _chain(orc, acc, bias=None, scale=None, res=None, res_scale=None, act=None, clamp=None, fq=None):
+    """The post-LPT elementwise chain evaluated with the oracle's reference ops, NCHW."""
+    OC = acc.shape[1]
+    bc = (1, OC, 1, 1)
+    v = acc.astype(np.float32)                       # Convert i32 -> f32
+    if bias is not None:
+        v = orc.add(v, np.asarray(bias, np.float32).reshape(bc))
+    if scale is not None:
+        v = orc.multiply(v, np.asarray(scale, np.float32).reshape(bc))
+    if res is not None:
+        r = res.astype(np.float32)
+        if res_scale is not None:
+            r = orc.multiply(r, np.asarray(res_scale, np.float32).reshape(-1, 1, 1) if np.size(res_scale) > 1
+                             else np.float32(res_scale))
+        v = orc.add(v, r)
+    if act == "relu":
+        v = orc.relu(v)
+    elif act == "clamp":
+        v = orc.clamp(v, clamp[0], clamp[1])
+    if fq is not None:
+        levels, il, ih, ol, oh = fq
+        v = orc.fake_quantize(v, np.asarray(il, np.float32).reshape(bc if np.size(il) > 1 else ()),
+                              np.asarray(ih, np.float32).reshape(bc if np.size(ih) > 1 else ()),
+                              np.float32(ol), np.float32(oh), levels)
+    return v
+
+
+@pytest.mark.parametrize("name", ["3x3_s1_p1_c64", "1x1_c64_oc256", "7x7_s2_p3_c3", "3x2_asym_c32_oc200"])
+def test_conv_bias_requantize_u8(orc, name):
+    """Steady-state ResNet layer: u8 -> Conv'(i8 W) -> +b'[c] -> FQ(0, ih'[c] -> 0..255) -> u8."""
+    from dldt_amd import Convolution, DeviceTensor, make_epilogue
+    g = GEOMS[name]
+    rng = np.random.default_rng(5)
+    x, w = _inputs(rng, g)
+    w = (w // 4)
+    OC = g[4]
+    acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    amax = np.abs(acc).max()
+    bias = rng.normal(0, amax / 20, OC).astype(np.float32)
+    ih = rng.uniform(0.3, 1.0, OC).astype(np.float32) * np.float32(amax)
+    il = np.zeros(OC, np.float32)
+    fq = (256, il, ih, 0.0, 255.0)
+    want = _chain(orc, acc, bias=bias, fq=fq).astype(np.uint8)
+    xin = _device_in(x, g)
+    out = DeviceTensor(acc.shape[0], acc.shape[2], acc.shape[3], OC, U8B)
+    Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10],
+                make_epilogue(bias=bias, out_dtype=U8B, fq=fq)).run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw(), want)
+    assert np.all(out.padded_channels() == 0)
+
+
+def test_conv_nonzero_input_low_and_ties(orc):
+    """FQ with il != 0 and bias chosen so that many outputs sit exactly on level boundaries."""
+    from dldt_amd import Convolution, DeviceTensor, make_epilogue
+    g = GEOMS["1x1_c256_oc64"]
+    rng = np.random.default_rng(6)
+    x, w = _inputs(rng, g)
+    w = np.sign(w)
+    OC = g[4]
+    acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    # integer accumulators + half-integer bias against a range of width 255*2: x/2 lands on k+0.5
+    bias = np.full(OC, 0.0, np.float32)
+    il = np.full(OC, -255.0, np.float32)
+    ih = np.full(OC, 255.0, np.float32)
+    fq = (256, il, ih, 0.0, 255.0)
+    want = _chain(orc, acc, bias=bias, fq=fq).astype(np.uint8)
+    xin = _device_in(x, g)
+    out = DeviceTensor(acc.shape[0], acc.shape[2], acc.shape[3], OC, U8B)
+    Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10],
+                make_epilogue(bias=bias, out_dtype=U8B, fq=fq)).run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw(), want)
+
+
+@pytest.mark.parametrize("res_kind", ["u8", "f32"])
+def test_conv_residual_add_relu_requantize(orc, res_kind):
+    """Bottleneck tail: (acc + b') * s[c] + residual -> ReLU -> FQ, residual either the u8 block
+    input dequantised by a scalar (Convert, Multiply) or an f32 tensor (downsample branch)."""
+    from dldt_amd import Convolution, DeviceTensor, make_epilogue
+    g = GEOMS["1x1_c64_oc256"]
+    rng = np.random.default_rng(8)
+    x, w = _inputs(rng, g)
+    OC = g[4]
+    acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    scale = (rng.uniform(0.5, 2.0, OC) * 1e-4).astype(np.float32)
+    bias = rng.normal(0, 2000, OC).astype(np.float32)
+    N, _, OH, OW = acc.shape
+    fq = (256, 0.0, np.float32(6.0), 0.0, 255.0)
+    xin = _device_in(x, g)
+    out = DeviceTensor(N, OH, OW, OC, U8B)
+    if res_kind == "u8":
+        res = rng.integers(0, 256, acc.shape).astype(np.int32)
+        s_x = np.float32(0.0173)
+        want = _chain(orc, acc, bias=bias, scale=scale, res=res, res_scale=s_x, act="relu", fq=fq)
+        rt = DeviceTensor.from_nchw(res, U8B)
+        epi = make_epilogue(bias=bias, scale=scale, residual_dtype=U8B, res_mul=[s_x],
+                            activation="relu", out_dtype=U8B, fq=fq)
+    else:
+        res = rng.normal(0, 3, acc.shape).astype(np.float32)
+        want = _chain(orc, acc, bias=bias, scale=scale, res=res, act="relu", fq=fq)
+        rt = DeviceTensor.from_nchw(res, F32)
+        epi = make_epilogue(bias=bias, scale=scale, residual_dtype=F32, activation="relu",
+                            out_dtype=U8B, fq=fq)
+    Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10], epi).run(xin, out, rt)
+    np.testing.assert_array_equal(out.to_nchw(), want.astype(np.uint8))
+
+
+@pytest.mark.parametrize("act", [None, "relu", "clamp"])
+def test_conv_dequantised_f32_output(orc, act):
+    """Graph tail (BASELINE config 1): Conv' -> +b' -> *s[c] -> ReLU, f32 out; bit-exact floats."""
+    from dldt_amd import Convolution, DeviceTensor, make_epilogue
+    g = GEOMS["3x3_s1_p1_c64"]
+    rng = np.random.default_rng(10)
+    x, w = _inputs(rng, g)
+    OC = g[4]
+    acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    scale = (rng.uniform(0.5, 2.0, OC) * 1e-4).astype(np.float32)
+    bias = rng.normal(0, 3000, OC).astype(np.float32)
+    want = _chain(orc, acc, bias=bias, scale=scale, act=act, clamp=(0.0, 6.0))
+    xin = _device_in(x, g)
+    out = DeviceTensor(acc.shape[0], acc.shape[2], acc.shape[3], OC, F32)
+    Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10],
+                make_epilogue(bias=bias, scale=scale, activation=act, clamp=(0.0, 6.0),
+                              out_dtype=F32)).run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw().view(np.uint32), want.view(np.uint32))
+
+
+def test_conv_rejects_missing_halo_and_shape_mismatch():
+    from dldt_amd import Convolution, DeviceTensor, HipieError
+    w = np.ones((64, 64, 3, 3), np.int8)
+    xin = DeviceTensor(1, 8, 8, 64, U8B, halo=0)
+    conv = Convolution(w, xin, pads_begin=(1, 1), pads_end=(1, 1))
+    with pytest.raises(HipieError) as e:
+        conv.run(xin, DeviceTensor(1, 8, 8, 64, I32))
+    assert e.value.status == -4 and "halo" in str(e.value)
+    xin = DeviceTensor(1, 8, 8, 64, U8B, halo=1)
+    conv = Convolution(w, xin, pads_begin=(1, 1), pads_end=(1, 1))
+    with pytest.raises(HipieError):
+        conv.run(xin, DeviceTensor(1, 7, 8, 64, I32))
