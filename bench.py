@@ -1,0 +1,129 @@
+#!/usr/bin/env python3
+"""ResNet-50 v1.5 INT8 inference throughput on one MI355X (BASELINE.json metric).
+
+One step = one batch-64 inference of the post-LPT graph (entry FakeQuantize, 53 fused int8 MFMA
+convolutions + FC, pools, exit), kernels only, inputs resident in HBM.  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
+HBM_PEAK_GBS = 8000.0
+
+
+def cpu_baseline(batch_images, budget_s=20.0):
+    """The oracle (C restatement of the reference kernels, OpenMP over host cores) evaluating the
+    same post-LPT ResNet-50 graph on a bounded sample of images."""
+    import numpy as np
+    import oracle
+    from interp import evaluate
+    from dldt_amd import builders
+    orc = oracle.require_ops()
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    g, _ = builders.resnet50(batch=1, res=224)
+    x = np.random.default_rng(5).uniform(0, 1, (1, 3, 224, 224)).astype(np.float32)
+    t0 = time.perf_counter()
+    evaluate(orc, g.nodes, {"data": x}, keep=[])
+    one = time.perf_counter() - t0
+    n = 1
+    total = one
+    while total + one < budget_s and n < batch_images:
+        t0 = time.perf_counter()
+        evaluate(orc, g.nodes, {"data": x}, keep=[])
+        total += time.perf_counter() - t0
+        n += 1
+    return {"value": n / total, "unit": "images/sec", "cores": cores, "kind": "port",
+            "sample": "%d image(s) of ResNet-50 v1.5 INT8 224x224 through oracle/ngraph_ops.c "
+                      "(scalar int32 reference loops, OpenMP over batch x output channels), %.1f s" % (n, total)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU (requests are independent; see DESIGN.md for "
+                 "how the path shards); --gpus %d is not supported" % args.gpus)
+    import numpy as np
+    import torch
+    from dldt_amd import builders
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+
+    g, meta = builders.resnet50(batch=args.batch, res=224)
+    plan = g.compile(0)
+    req = plan.create_request(perf_count=False)
+    ins, outs = req.device_buffers()
+    gen = torch.Generator(device="cuda").manual_seed(20211)
+    ins[0].copy_(torch.rand(ins[0].shape, generator=gen, device="cuda"))
+    stream = torch.cuda.ExternalStream(req.stream)
+    torch.cuda.synchronize()
+
+    for _ in range(args.warmup):
+        req.enqueue(ins, outs)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(args.steps):
+        req.enqueue(ins, outs)
+    e1.record(stream)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    images_per_s = args.batch / (ms_per_step * 1e-3)
+
+    # per-step HIP events on the same stream: time spent in the int8 MFMA kernel
+    preq = plan.create_request(perf_count=True)
+    acc = {}
+    reps = max(3, min(10, args.steps))
+    for _ in range(2):
+        preq.infer_device(ins, outs)
+    for _ in range(reps):
+        preq.infer_device(ins, outs)
+        for i, st in enumerate(preq.perf()):
+            acc[i] = acc.get(i, 0.0) + st["ms"]
+    steps = [dict(st, ms=acc[i] / reps) for i, st in enumerate(plan.steps)]
+    mfma = [s for s in steps if s["type"] in ("Convolution", "MatMul")]
+    mfma_ms = sum(s["ms"] for s in mfma)
+    mfma_ops = 2.0 * sum(s["macs"] for s in mfma)
+    achieved_tops = mfma_ops / (mfma_ms * 1e-3) / 1e12
+    total_ops = 2.0 * meta["macs_per_image"] * args.batch
+
+    line = {
+        "metric": "ResNet-50 INT8 images/sec @b%d on 1 MI355X" % args.batch,
+        "value": images_per_s, "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8 x i8 -> i32 (f32 epilogue)", "data": "synthetic",
+        "config": {"workload": "ResNet-50 v1.5 INT8 (post-LPT graph), batch %d, 224x224, He-normal weights, "
+                               "seeded calibration" % args.batch,
+                   "batch": args.batch, "kernels_per_step": len(steps), "wall_ms_per_step": wall_ms / args.steps},
+        "tops": total_ops / (ms_per_step * 1e-3) / 1e12,
+        "frac_int8_peak_whole_net": total_ops / (ms_per_step * 1e-3) / 1e12 / INT8_PEAK_TOPS,
+        "roofline": {"bound": "mfma", "achieved": achieved_tops, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
+                     "frac": achieved_tops / INT8_PEAK_TOPS, "traffic": None,
+                     "kernel": "conv_mfma_kernel (all %d convolution/FC launches of one step)" % len(mfma),
+                     "ops_per_step": mfma_ops, "kernel_ms_per_step": mfma_ms,
+                     "avg_launch_us": mfma_ms * 1e3 / len(mfma), "note": "int8 TOP/s, dense peak 5.0 POP/s"},
+        "other_kernels_ms_per_step": {t: sum(s["ms"] for s in steps if s["type"] == t)
+                                      for t in sorted({s["type"] for s in steps} - {"Convolution", "MatMul"})},
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(args.batch)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

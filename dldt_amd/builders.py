@@ -1,0 +1,245 @@
+"""Seeded builders of the benchmark configurations as post-LPT graphs.
+
+The reference ships no whole-model builders or weights, so the networks are defined here:
+architecture, He-normal weights (BatchNorm folded into conv + bias), a seeded calibration batch
+run in fp32 on the host to fix every activation FakeQuantize range, and then the graph that the
+stock low-precision transformations leave for a plugin (derivation in ``QuantizedNet``).
+"""
+import numpy as np
+
+from . import lpt
+from .graph import Graph
+from .tensor import F32, I8, U8
+
+
+class QuantizedNet:
+    """Emits post-LPT layers.  An *activation* is a dict(node=<u8 value id>, scale=<f32 scalar>):
+    the u8 FakeQuantize output and the scale of its pending dequantization Multiply
+    (decomposeFakeQuantize: scale = (out_high - out_low) / 255 for [0, ih] ranges).
+
+    Per layer, with s[c] = s_act * s_w[c] (ConvolutionTransformation, optimizeMultipliesAfter):
+        Conv'(u8 x, i8 W) -> Add(b[c] / s[c])  (AddTransformation / swapMultiplyAndAdd)
+        followed either by the next activation FakeQuantize with the Multiply folded into its
+        input range (FakeQuantizeTransformation::fuseElementwise: il / s[c], ih / s[c]), or by
+        Multiply(s[c]) when the value is used in f32 (residual Add, graph output).
+    ReLU in front of a FakeQuantize with input_low >= 0 is already gone before LPT
+    (ReluFakeQuantizeFusion), so it only survives in f32 tails.
+    """
+
+    def __init__(self):
+        self.g = Graph()
+
+    # -- graph input ---------------------------------------------------------------------------
+    def input(self, name, shape, in_high):
+        g = self.g
+        x = g.parameter(name, shape)
+        d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(in_high))
+        q = g.fake_quantize(x, np.float32(0), np.float32(in_high), d["new_low"], d["new_high"], 256, U8)
+        return dict(node=q, scale=np.float32(d["scale"]))
+
+    def _channel(self, v, rank):
+        v = np.asarray(v, np.float32)
+        return v.reshape((1, -1) + (1,) * (rank - 2))
+
+    def _accumulate(self, act, w, bias, conv_attrs, matmul=False):
+        """Conv'/MatMul' -> Add(b / s): returns (node, s[c])."""
+        g = self.g
+        wq, s_w = lpt.quantize_weights(w, 255)
+        s = (np.float32(act["scale"]) * s_w).astype(np.float32)            # fold<Multiply>(s_a, s_w)
+        wc = g.constant(wq, I8)
+        if matmul:
+            y = g.matmul(act["node"], wc, False, True)
+            rank = 2
+        else:
+            y = g.convolution(act["node"], wc, **conv_attrs)
+            rank = 4
+        if bias is not None:
+            b = np.asarray(bias, np.float32)
+            with np.errstate(divide="ignore", invalid="ignore"):
+                bdiv = np.where((b != 0) | (s != 0), b / s, np.float32(0)).astype(np.float32)  # bi / ai
+            y = g.add(y, g.constant(self._channel(bdiv, rank)))
+        return y, s, rank
+
+    def conv(self, act, w, bias, out_high, strides=(1, 1), pads=(0, 0), dilations=(1, 1)):
+        """Quantized conv whose ReLU output feeds the next FakeQuantize [0, out_high]."""
+        g = self.g
+        attrs = dict(strides=strides, dilations=dilations, pads_begin=pads, pads_end=pads)
+        y, s, rank = self._accumulate(act, w, bias, attrs)
+        d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(out_high))
+        il = (np.float32(0) / s).astype(np.float32)                          # fold<Divide>(il, s)
+        ih = (np.float32(out_high) / s).astype(np.float32)
+        q = g.fake_quantize(y, self._channel(il, rank), self._channel(ih, rank), d["new_low"], d["new_high"],
+                            256, U8)
+        return dict(node=q, scale=np.float32(d["scale"]))
+
+    def conv_f32(self, act, w, bias, strides=(1, 1), pads=(0, 0), relu=False, matmul=False):
+        """Quantized conv / FC whose result is consumed in f32: ... -> Multiply(s[c]) [-> ReLU]."""
+        g = self.g
+        attrs = dict(strides=strides, dilations=(1, 1), pads_begin=pads, pads_end=pads)
+        y, s, rank = self._accumulate(act, w, bias, attrs, matmul)
+        y = g.multiply(y, g.constant(self._channel(s, rank)))
+        return g.relu(y) if relu else y
+
+    def dequantize(self, act):
+        """Convert + Multiply left on a u8 value that is consumed in f32."""
+        g = self.g
+        return g.multiply(g.convert(act["node"], F32), g.constant(np.float32(act["scale"]).reshape(())))
+
+    def requantize(self, y, out_high):
+        """Activation FakeQuantize [0, out_high] on an f32 value (no pending Multiply to fold)."""
+        d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(out_high))
+        q = self.g.fake_quantize(y, np.float32(0), np.float32(out_high), d["new_low"], d["new_high"], 256, U8)
+        return dict(node=q, scale=np.float32(d["scale"]))
+
+    def max_pool(self, act, kernel, strides, pads):
+        # MaxPoolTransformation: the Multiply moves behind the pool, which then runs on u8
+        return dict(node=self.g.max_pool(act["node"], kernel, strides, pads, pads), scale=act["scale"])
+
+
+# ---------------------------------------------------------------------------------------------
+def he_normal(rng, shape):
+    fan_in = int(np.prod(shape[1:]))
+    return (rng.standard_normal(shape, dtype=np.float32) * np.float32(np.sqrt(2.0 / fan_in))).astype(np.float32)
+
+
+def conv_block(seed=20211, n=1, c=64, hw=56, oc=64):
+    """BASELINE config 1: FQ(u8) -> Conv 3x3 s1 p1 (per-channel i8 weights) -> bias -> ReLU, f32 out."""
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(0, 2.55, (n, c, hw, hw)).astype(np.float32)
+    w = (rng.standard_normal((oc, c, 3, 3), dtype=np.float32) * np.float32(0.05)).astype(np.float32)
+    b = (rng.standard_normal(oc, dtype=np.float32) * np.float32(0.1)).astype(np.float32)
+    net = QuantizedNet()
+    a = net.input("data", x.shape, 2.55)
+    y = net.conv_f32(a, w, b, pads=(1, 1), relu=True)
+    net.g.result(y, "out")
+    return net.g, dict(data=x), dict(w=w, b=b)
+
+
+RESNET50_STAGES = [(64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)]
+
+
+def resnet50_weights(seed=20211, classes=1000, width=64, stages=RESNET50_STAGES):
+    """ResNet-50 v1.5 parameters: He-normal convs with a folded-BN bias ~ N(0, 0.1)."""
+    rng = np.random.default_rng(seed)
+    P = {}
+
+    def conv(name, oc, ic, k):
+        P[name + ".w"] = he_normal(rng, (oc, ic, k, k))
+        P[name + ".b"] = (rng.standard_normal(oc, dtype=np.float32) * np.float32(0.1)).astype(np.float32)
+
+    conv("conv1", width, 3, 7)
+    ic = width
+    for si, (mid, blocks, _) in enumerate(stages):
+        mid = mid * width // 64
+        for bi in range(blocks):
+            p = "layer%d.%d" % (si + 1, bi)
+            conv(p + ".a", mid, ic, 1)
+            conv(p + ".b", mid, mid, 3)
+            conv(p + ".c", mid * 4, mid, 1)
+            if bi == 0:
+                conv(p + ".ds", mid * 4, ic, 1)
+            ic = mid * 4
+    P["fc.w"] = he_normal(rng, (classes, ic))
+    P["fc.b"] = (rng.standard_normal(classes, dtype=np.float32) * np.float32(0.1)).astype(np.float32)
+    return P
+
+
+def resnet50_fp32(P, x, stages=RESNET50_STAGES, record=None):
+    """fp32 forward on the host (torch CPU) — used only to calibrate activation ranges."""
+    import torch
+    import torch.nn.functional as F
+
+    def t(a):
+        return torch.from_numpy(np.ascontiguousarray(a))
+
+    def conv(name, v, stride=1, pad=0):
+        return F.conv2d(v, t(P[name + ".w"]), t(P[name + ".b"]), stride=stride, padding=pad)
+
+    def rec(name, v):
+        if record is not None:
+            record[name] = max(record.get(name, 0.0), float(v.max()))
+        return v
+
+    with torch.no_grad():
+        v = rec("input", t(x))
+        v = rec("conv1", F.relu(conv("conv1", v, 2, 3)))
+        v = F.max_pool2d(v, 3, 2, 1)
+        for si, (_, blocks, stride) in enumerate(stages):
+            for bi in range(blocks):
+                p = "layer%d.%d" % (si + 1, bi)
+                s = stride if bi == 0 else 1
+                y = rec(p + ".a", F.relu(conv(p + ".a", v)))
+                y = rec(p + ".b", F.relu(conv(p + ".b", y, s, 1)))      # v1.5: stride on the 3x3
+                y = conv(p + ".c", y)
+                sc = conv(p + ".ds", v, s) if bi == 0 else v
+                v = rec(p + ".out", F.relu(y + sc))
+        v = rec("pool", v.mean(dim=(2, 3)))
+        v = F.linear(v, t(P["fc.w"]), t(P["fc.b"]))
+    return v.numpy()
+
+
+def resnet50(batch=1, res=224, seed=20211, classes=1000, width=64, stages=RESNET50_STAGES, calib_batch=2):
+    """BASELINE config 3 as a post-LPT graph.  Returns (graph, meta) where meta holds the
+    parameters, the calibrated ranges and the ids of every quantized activation."""
+    P = resnet50_weights(seed, classes, width, stages)
+    rng = np.random.default_rng(seed + 1)
+    calib = rng.uniform(0, 1, (calib_batch, 3, res, res)).astype(np.float32)
+    R = {}
+    resnet50_fp32(P, calib, stages, R)
+    net = QuantizedNet()
+    g = net.g
+    acts = {}
+    a = net.input("data", (batch, 3, res, res), R["input"])
+    acts["input"] = a
+    a = net.conv(a, P["conv1.w"], P["conv1.b"], R["conv1"], strides=(2, 2), pads=(3, 3))
+    acts["conv1"] = a
+    a = net.max_pool(a, (3, 3), (2, 2), (1, 1))
+    acts["maxpool"] = a
+    for si, (_, blocks, stride) in enumerate(stages):
+        for bi in range(blocks):
+            p = "layer%d.%d" % (si + 1, bi)
+            s = stride if bi == 0 else 1
+            ya = net.conv(a, P[p + ".a.w"], P[p + ".a.b"], R[p + ".a"])
+            yb = net.conv(ya, P[p + ".b.w"], P[p + ".b.b"], R[p + ".b"], strides=(s, s), pads=(1, 1))
+            yc = net.conv_f32(yb, P[p + ".c.w"], P[p + ".c.b"])
+            if bi == 0:
+                sc = net.conv_f32(a, P[p + ".ds.w"], P[p + ".ds.b"], strides=(s, s))
+            else:
+                sc = net.dequantize(a)
+            # the residual Add stays f32 (AddTransformation leaves it: the conv branch is not low
+            # precision); the ReLU behind it was fused into the next FakeQuantize before LPT
+            a = net.requantize(g.add(yc, sc), R[p + ".out"])
+            acts[p + ".a"], acts[p + ".b"], acts[p + ".out"] = ya, yb, a
+    final_hw = res // 32
+    y = g.avg_pool(a["node"], (final_hw, final_hw), (1, 1), (0, 0), (0, 0), exclude_pad=True, out_dtype=F32)
+    y = g.reshape(y, (batch, P["fc.w"].shape[1]))
+    d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(R["pool"]))
+    s_x = np.float32(a["scale"])
+    q = g.fake_quantize(y, (np.float32(0) / s_x).astype(np.float32), (np.float32(R["pool"]) / s_x).astype(np.float32),
+                        d["new_low"], d["new_high"], 256, U8)
+    pooled = dict(node=q, scale=np.float32(d["scale"]))
+    acts["pool"] = pooled
+    logits = net.conv_f32(pooled, P["fc.w"], P["fc.b"], matmul=True)
+    g.result(logits, "logits")
+    macs = resnet50_macs(res, classes, width, stages)
+    return g, dict(params=P, ranges=R, acts=acts, macs_per_image=macs, calib=calib)
+
+
+def resnet50_macs(res=224, classes=1000, width=64, stages=RESNET50_STAGES):
+    h = res // 2
+    macs = h * h * width * 3 * 49
+    h = h // 2
+    ic = width
+    for mid, blocks, stride in stages:
+        mid = mid * width // 64
+        for bi in range(blocks):
+            s = stride if bi == 0 else 1
+            macs += h * h * mid * ic
+            h2 = h // s
+            macs += h2 * h2 * mid * mid * 9
+            macs += h2 * h2 * mid * 4 * mid
+            if bi == 0:
+                macs += h2 * h2 * mid * 4 * ic
+            ic = mid * 4
+            h = h2
+    return macs + classes * ic

@@ -30,4 +30,12 @@ int hipie_device_name(int device, char* buf, size_t buf_len) {
     });
 }
 
+int hipie_memcpy(void* dst, const void* src, size_t bytes, int to_device) {
+    return guarded([&] {
+        HIPIE_REQUIRE((dst && src) || bytes == 0, HIPIE_PARAMETER_MISMATCH, "hipie_memcpy: null argument");
+        if (bytes)
+            HIPIE_CHECK_HIP(hipMemcpy(dst, src, bytes, to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost));
+    });
+}
+
 }  // extern "C"

@@ -99,7 +99,8 @@ __global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc_q8(const float* __re
                                                                 const FqChannel* __restrict__ tab,
                                                                 float lm1, float off, uint32_t hw,
                                                                 uint32_t C, uint32_t c_stride,
-                                                                uint32_t tiles_per_image) {
+                                                                uint32_t tiles_per_image, uint32_t W,
+                                                                int64_t out_sn, int64_t out_sh) {
     __shared__ uint32_t tile[64][17];  // [pixel][16 dwords = 64 channel bytes] + 1 pad
     const uint32_t n = blockIdx.x / tiles_per_image;
     const uint32_t p0 = (blockIdx.x % tiles_per_image) * 64;
@@ -131,7 +132,8 @@ __global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc_q8(const float* __re
         v.y = tile[op][oq * 4 + 1];
         v.z = tile[op][oq * 4 + 2];
         v.w = tile[op][oq * 4 + 3];
-        uint8_t* dst = y + (static_cast<int64_t>(n) * hw + p0 + op) * c_stride + cbyte;
+        const uint32_t ph = (p0 + op) / W, pw = (p0 + op) - ph * W;
+        uint8_t* dst = y + static_cast<int64_t>(n) * out_sn + ph * out_sh + static_cast<int64_t>(pw) * c_stride + cbyte;
         if (cbyte + 16 <= c_stride && c_stride % 16 == 0) {
             *reinterpret_cast<uint4*>(dst) = v;
         } else {  // c_stride is a multiple of 4
@@ -390,10 +392,44 @@ int hipie_fq_run_q8(const hipie_fq* fq, const float* x, void* y, int64_t n, int6
             hipLaunchKernelGGL(k, dim3(static_cast<uint32_t>(gx),
                                        static_cast<uint32_t>(ceil_div(c_stride, 64))),
                                dim3(kThreads), 0, s, x, static_cast<uint8_t*>(y), tab, fq->lm1, off,
-                               static_cast<uint32_t>(hw), C, static_cast<uint32_t>(c_stride), tiles);
+                               static_cast<uint32_t>(hw), C, static_cast<uint32_t>(c_stride), tiles,
+                               static_cast<uint32_t>(hw), hw * c_stride, hw * c_stride);
         } else {
             fail(HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8: out_layout %d", (int)out_layout);
         }
+        HIPIE_CHECK_HIP(hipGetLastError());
+    });
+}
+
+int hipie_fq_run_q8_tensor(const hipie_fq* fq, const float* x, const hipie_tensor* out, void* stream) {
+    return guarded([&] {
+        HIPIE_REQUIRE(fq && out, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: null argument");
+        HIPIE_REQUIRE(fq->table.ptr, HIPIE_NOT_ALLOCATED, "hipie_fq_run_q8_tensor: host-only object");
+        const int64_t hw = static_cast<int64_t>(out->h) * out->w;
+        if (out->n == 0 || hw == 0) return;
+        HIPIE_REQUIRE(x && out->data, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: null data");
+        HIPIE_REQUIRE(out->c == fq->C, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: %d channels, expected %lld",
+                      out->c, (long long)fq->C);
+        HIPIE_REQUIRE(fq->q8_ok && fq->clamp_ok, HIPIE_NOT_IMPLEMENTED,
+                      "hipie_fq_run_q8_tensor: needs input_low < input_high and consecutive integer output levels");
+        float off;
+        if (out->dtype == HIPIE_U8B) off = fq->q8_base - 128.0f;
+        else if (out->dtype == HIPIE_I8) off = fq->q8_base;
+        else fail(HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: output dtype %d", out->dtype);
+        HIPIE_REQUIRE(out->dtype == HIPIE_U8B ? fq->q8_base >= 0 : fq->q8_base + fq->lm1 <= 127.0f,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: levels do not fit the output type");
+        const int64_t cs = out->stride_w;
+        HIPIE_REQUIRE(cs >= fq->C && cs % 4 == 0 && reinterpret_cast<uintptr_t>(out->data) % 4 == 0 &&
+                          (cs % 16 != 0 || reinterpret_cast<uintptr_t>(out->data) % 16 == 0),
+                      HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: channel stride / alignment");
+        const uint32_t tiles = static_cast<uint32_t>(ceil_div(hw, 64));
+        DeviceGuard g(fq->device);
+        auto k = fq->rcp ? fq_nchw_to_nhwc_q8<true> : fq_nchw_to_nhwc_q8<false>;
+        hipLaunchKernelGGL(k, dim3(static_cast<uint32_t>(out->n * tiles), static_cast<uint32_t>(ceil_div(cs, 64))),
+                           dim3(kThreads), 0, as_stream(stream), x, static_cast<uint8_t*>(out->data),
+                           fq->table.as<FqChannel>(), fq->lm1, off, static_cast<uint32_t>(hw),
+                           static_cast<uint32_t>(fq->C), static_cast<uint32_t>(cs), tiles,
+                           static_cast<uint32_t>(out->w), out->stride_n, out->stride_h);
         HIPIE_CHECK_HIP(hipGetLastError());
     });
 }

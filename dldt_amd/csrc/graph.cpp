@@ -1,0 +1,347 @@
+// Graph description entry points: one call per nGraph node of the post-LPT Function, with the
+// shape/type inference the planner relies on (ngraph/core/src/op/{convolution,group_conv,matmul,
+// max_pool,avg_pool,fake_quantize}.cpp validate_and_infer_types).
+#include "graph.h"
+
+namespace hipie {
+
+const char* op_name(int op) {
+    static const char* names[] = {"Parameter", "Constant", "FakeQuantize", "Convolution",
+                                  "GroupConvolution", "MatMul", "Add", "Multiply", "Subtract", "Relu",
+                                  "Clamp", "Convert", "MaxPool", "AvgPool", "Reshape", "Result"};
+    return op >= 0 && op <= OP_RESULT ? names[op] : "?";
+}
+
+namespace {
+
+size_t dtype_size(int dt) {
+    switch (dt) {
+    case HIPIE_F32: case HIPIE_I32: return 4;
+    case HIPIE_U8: case HIPIE_I8: case HIPIE_U8B: return 1;
+    default: fail(HIPIE_PARAMETER_MISMATCH, "unknown element type %d", dt);
+    }
+}
+
+GNode& node(hipie_graph* g, int id, const char* what) {
+    HIPIE_REQUIRE(g, HIPIE_PARAMETER_MISMATCH, "%s: null graph", what);
+    HIPIE_REQUIRE(id >= 0 && id < static_cast<int>(g->nodes.size()), HIPIE_NOT_FOUND,
+                  "%s: no value with id %d", what, id);
+    HIPIE_REQUIRE(g->nodes[id].op != OP_RESULT, HIPIE_PARAMETER_MISMATCH, "%s: id %d is a Result", what, id);
+    return g->nodes[id];
+}
+
+int add_node(hipie_graph* g, GNode&& n) {
+    const int id = static_cast<int>(g->nodes.size());
+    if (n.name.empty()) n.name = std::string(op_name(n.op)) + "_" + std::to_string(id);
+    for (int i : n.in) g->nodes[i].users.push_back(id);
+    g->nodes.push_back(std::move(n));
+    return id;
+}
+
+std::vector<int64_t> broadcast_shape(const std::vector<int64_t>& a, const std::vector<int64_t>& b,
+                                     const char* what) {
+    const size_t r = std::max(a.size(), b.size());
+    std::vector<int64_t> o(r);
+    for (size_t i = 0; i < r; ++i) {
+        const int64_t da = i + a.size() >= r ? a[i + a.size() - r] : 1;
+        const int64_t db = i + b.size() >= r ? b[i + b.size() - r] : 1;
+        HIPIE_REQUIRE(da == db || da == 1 || db == 1, HIPIE_PARAMETER_MISMATCH,
+                      "%s: shapes do not broadcast", what);
+        o[i] = std::max(da, db);
+    }
+    return o;
+}
+
+int64_t pooled(int64_t in, int64_t pb, int64_t pe, int64_t window, int64_t stride, bool ceil_mode) {
+    const int64_t span = in + pb + pe - window;
+    HIPIE_REQUIRE(span >= 0, HIPIE_PARAMETER_MISMATCH, "window larger than the padded input");
+    return (ceil_mode ? ceil_div(span, stride) : span / stride) + 1;
+}
+
+}  // namespace
+}  // namespace hipie
+
+using namespace hipie;
+
+extern "C" {
+
+int hipie_graph_create(hipie_graph** g) {
+    return guarded([&] {
+        HIPIE_REQUIRE(g, HIPIE_PARAMETER_MISMATCH, "hipie_graph_create: null argument");
+        *g = new hipie_graph();
+    });
+}
+
+void hipie_graph_destroy(hipie_graph* g) { delete g; }
+
+int hipie_graph_parameter(hipie_graph* g, const char* name, int dtype, const int64_t* dims, int rank, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(g && dims && id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_parameter: null argument");
+        HIPIE_REQUIRE(rank >= 2 && rank <= 4, HIPIE_NOT_IMPLEMENTED, "hipie_graph_parameter: rank %d", rank);
+        HIPIE_REQUIRE(dtype == HIPIE_F32 || dtype == HIPIE_U8, HIPIE_NOT_IMPLEMENTED,
+                      "hipie_graph_parameter: element type %d", dtype);
+        GNode n;
+        n.op = OP_PARAMETER;
+        n.name = name ? name : "";
+        n.dtype = dtype;
+        n.shape.assign(dims, dims + rank);
+        *id = add_node(g, std::move(n));
+        g->params.push_back(*id);
+    });
+}
+
+int hipie_graph_constant(hipie_graph* g, int dtype, const int64_t* dims, int rank, const void* data, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(g && id && data && (dims || rank == 0), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_graph_constant: null argument");
+        GNode n;
+        n.op = OP_CONSTANT;
+        n.dtype = dtype;
+        n.shape.assign(dims, dims + rank);
+        const size_t bytes = static_cast<size_t>(n.numel()) * dtype_size(dtype);
+        n.data.assign(static_cast<const uint8_t*>(data), static_cast<const uint8_t*>(data) + bytes);
+        *id = add_node(g, std::move(n));
+    });
+}
+
+int hipie_graph_fake_quantize(hipie_graph* g, int x, int il, int ih, int ol, int oh, int64_t levels,
+                              int out_dtype, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_fake_quantize: null argument");
+        GNode& X = node(g, x, "hipie_graph_fake_quantize");
+        HIPIE_REQUIRE(X.dtype == HIPIE_F32, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_graph_fake_quantize: data must be f32");
+        for (int b : {il, ih, ol, oh}) {
+            GNode& B = node(g, b, "hipie_graph_fake_quantize");
+            HIPIE_REQUIRE(B.op == OP_CONSTANT && B.dtype == HIPIE_F32, HIPIE_NOT_IMPLEMENTED,
+                          "hipie_graph_fake_quantize: bounds must be f32 constants");
+            broadcast_shape(X.shape, B.shape, "hipie_graph_fake_quantize");
+        }
+        HIPIE_REQUIRE(levels >= 2, HIPIE_PARAMETER_MISMATCH, "hipie_graph_fake_quantize: levels");
+        HIPIE_REQUIRE(out_dtype == HIPIE_F32 || out_dtype == HIPIE_U8 || out_dtype == HIPIE_I8,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_graph_fake_quantize: output type %d", out_dtype);
+        GNode n;
+        n.op = OP_FAKE_QUANTIZE;
+        n.in = {x, il, ih, ol, oh};
+        n.levels = levels;
+        n.dtype = out_dtype;
+        n.shape = X.shape;
+        *id = add_node(g, std::move(n));
+    });
+}
+
+static int add_conv(hipie_graph* g, int x, int w, const int64_t* strides, const int64_t* dilations,
+                    const int64_t* pads_begin, const int64_t* pads_end, bool grouped, int* id) {
+    return guarded([&] {
+        const char* what = grouped ? "hipie_graph_group_convolution" : "hipie_graph_convolution";
+        HIPIE_REQUIRE(id && strides && dilations && pads_begin && pads_end, HIPIE_PARAMETER_MISMATCH,
+                      "%s: null argument", what);
+        GNode& X = node(g, x, what);
+        GNode& W = node(g, w, what);
+        HIPIE_REQUIRE(X.shape.size() == 4, HIPIE_NOT_IMPLEMENTED, "%s: only 2-D spatial", what);
+        HIPIE_REQUIRE(W.shape.size() == (grouped ? 5u : 4u), HIPIE_PARAMETER_MISMATCH, "%s: filter rank", what);
+        const int o = grouped ? 1 : 0;
+        const int64_t G = grouped ? W.shape[0] : 1;
+        HIPIE_REQUIRE(X.shape[1] == W.shape[o + 1] * G, HIPIE_PARAMETER_MISMATCH,
+                      "%s: input channels %lld vs filter %lld x %lld groups", what, (long long)X.shape[1],
+                      (long long)W.shape[o + 1], (long long)G);
+        GNode n;
+        n.op = grouped ? OP_GROUP_CONVOLUTION : OP_CONVOLUTION;
+        n.in = {x, w};
+        n.strides.assign(strides, strides + 2);
+        n.dilations.assign(dilations, dilations + 2);
+        n.pads_begin.assign(pads_begin, pads_begin + 2);
+        n.pads_end.assign(pads_end, pads_end + 2);
+        n.dtype = HIPIE_F32;  // TypeRelaxed<Convolution>: f32 holding the integer sum
+        n.shape = {X.shape[0], W.shape[o] * G};
+        for (int i = 0; i < 2; ++i) {
+            HIPIE_REQUIRE(n.strides[i] > 0 && n.dilations[i] > 0 && n.pads_begin[i] >= 0 && n.pads_end[i] >= 0,
+                          HIPIE_PARAMETER_MISMATCH, "%s: attributes", what);
+            const int64_t dk = n.dilations[i] * (W.shape[o + 2 + i] - 1) + 1;
+            const int64_t span = X.shape[2 + i] + n.pads_begin[i] + n.pads_end[i] - dk;
+            HIPIE_REQUIRE(span >= 0, HIPIE_PARAMETER_MISMATCH, "%s: filter larger than padded input", what);
+            n.shape.push_back(span / n.strides[i] + 1);
+        }
+        *id = add_node(g, std::move(n));
+    });
+}
+
+int hipie_graph_convolution(hipie_graph* g, int x, int w, const int64_t* strides, const int64_t* dilations,
+                            const int64_t* pads_begin, const int64_t* pads_end, int* id) {
+    return add_conv(g, x, w, strides, dilations, pads_begin, pads_end, false, id);
+}
+
+int hipie_graph_group_convolution(hipie_graph* g, int x, int w, const int64_t* strides,
+                                  const int64_t* dilations, const int64_t* pads_begin,
+                                  const int64_t* pads_end, int* id) {
+    return add_conv(g, x, w, strides, dilations, pads_begin, pads_end, true, id);
+}
+
+int hipie_graph_matmul(hipie_graph* g, int a, int b, int transpose_a, int transpose_b, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_matmul: null argument");
+        GNode& A = node(g, a, "hipie_graph_matmul");
+        GNode& B = node(g, b, "hipie_graph_matmul");
+        HIPIE_REQUIRE(A.shape.size() >= 2 && B.shape.size() >= 2, HIPIE_NOT_IMPLEMENTED,
+                      "hipie_graph_matmul: 1-D operands");
+        std::vector<int64_t> sa = A.shape, sb = B.shape;
+        if (transpose_a) std::swap(sa[sa.size() - 1], sa[sa.size() - 2]);
+        if (transpose_b) std::swap(sb[sb.size() - 1], sb[sb.size() - 2]);
+        HIPIE_REQUIRE(sa.back() == sb[sb.size() - 2], HIPIE_PARAMETER_MISMATCH,
+                      "hipie_graph_matmul: inner dimensions %lld vs %lld", (long long)sa.back(),
+                      (long long)sb[sb.size() - 2]);
+        std::vector<int64_t> ba(sa.begin(), sa.end() - 2), bb(sb.begin(), sb.end() - 2);
+        GNode n;
+        n.op = OP_MATMUL;
+        n.in = {a, b};
+        n.ta = transpose_a != 0;
+        n.tb = transpose_b != 0;
+        n.dtype = HIPIE_F32;
+        n.shape = broadcast_shape(ba, bb, "hipie_graph_matmul");
+        n.shape.push_back(sa[sa.size() - 2]);
+        n.shape.push_back(sb.back());
+        *id = add_node(g, std::move(n));
+    });
+}
+
+int hipie_graph_eltwise(hipie_graph* g, int kind, int a, int b, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_eltwise: null argument");
+        HIPIE_REQUIRE(kind == OP_ADD || kind == OP_MULTIPLY || kind == OP_SUBTRACT, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_graph_eltwise: kind %d", kind);
+        GNode& A = node(g, a, "hipie_graph_eltwise");
+        GNode& B = node(g, b, "hipie_graph_eltwise");
+        HIPIE_REQUIRE(A.dtype == HIPIE_F32 && B.dtype == HIPIE_F32, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_graph_eltwise: operands must be f32 (insert Convert)");
+        GNode n;
+        n.op = kind;
+        n.in = {a, b};
+        n.dtype = HIPIE_F32;
+        n.shape = broadcast_shape(A.shape, B.shape, "hipie_graph_eltwise");
+        *id = add_node(g, std::move(n));
+    });
+}
+
+int hipie_graph_relu(hipie_graph* g, int x, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_relu: null argument");
+        GNode& X = node(g, x, "hipie_graph_relu");
+        GNode n;
+        n.op = OP_RELU;
+        n.in = {x};
+        n.dtype = X.dtype;
+        n.shape = X.shape;
+        *id = add_node(g, std::move(n));
+    });
+}
+
+int hipie_graph_clamp(hipie_graph* g, int x, float lo, float hi, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_clamp: null argument");
+        HIPIE_REQUIRE(lo <= hi, HIPIE_PARAMETER_MISMATCH, "hipie_graph_clamp: min > max");
+        GNode& X = node(g, x, "hipie_graph_clamp");
+        GNode n;
+        n.op = OP_CLAMP;
+        n.in = {x};
+        n.lo = lo;
+        n.hi = hi;
+        n.dtype = X.dtype;
+        n.shape = X.shape;
+        *id = add_node(g, std::move(n));
+    });
+}
+
+int hipie_graph_convert(hipie_graph* g, int x, int dtype, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_convert: null argument");
+        GNode& X = node(g, x, "hipie_graph_convert");
+        dtype_size(dtype);
+        GNode n;
+        n.op = OP_CONVERT;
+        n.in = {x};
+        n.dtype = dtype;
+        n.shape = X.shape;
+        *id = add_node(g, std::move(n));
+    });
+}
+
+static int add_pool(hipie_graph* g, int op, int x, const int64_t* kernel, const int64_t* strides,
+                    const int64_t* pads_begin, const int64_t* pads_end, int exclude_pad, int ceil_mode,
+                    int out_dtype, int* id) {
+    return guarded([&] {
+        const char* what = op == OP_MAX_POOL ? "hipie_graph_max_pool" : "hipie_graph_avg_pool";
+        HIPIE_REQUIRE(id && kernel && strides && pads_begin && pads_end, HIPIE_PARAMETER_MISMATCH,
+                      "%s: null argument", what);
+        GNode& X = node(g, x, what);
+        HIPIE_REQUIRE(X.shape.size() == 4, HIPIE_NOT_IMPLEMENTED, "%s: only 2-D spatial", what);
+        GNode n;
+        n.op = op;
+        n.in = {x};
+        n.kernel.assign(kernel, kernel + 2);
+        n.strides.assign(strides, strides + 2);
+        n.pads_begin.assign(pads_begin, pads_begin + 2);
+        n.pads_end.assign(pads_end, pads_end + 2);
+        n.exclude_pad = exclude_pad != 0;
+        n.ceil_mode = ceil_mode != 0;
+        n.dtype = out_dtype;
+        n.shape = {X.shape[0], X.shape[1]};
+        for (int i = 0; i < 2; ++i) {
+            HIPIE_REQUIRE(kernel[i] > 0 && strides[i] > 0 && pads_begin[i] >= 0 && pads_end[i] >= 0,
+                          HIPIE_PARAMETER_MISMATCH, "%s: attributes", what);
+            n.shape.push_back(pooled(X.shape[2 + i], pads_begin[i], pads_end[i], kernel[i], strides[i], n.ceil_mode));
+        }
+        *id = add_node(g, std::move(n));
+    });
+}
+
+int hipie_graph_max_pool(hipie_graph* g, int x, const int64_t* kernel, const int64_t* strides,
+                         const int64_t* pads_begin, const int64_t* pads_end, int ceil_mode, int* id) {
+    if (!g || x < 0 || x >= static_cast<int>(g->nodes.size()))
+        return guarded([&] { fail(HIPIE_NOT_FOUND, "hipie_graph_max_pool: no value with id %d", x); });
+    return add_pool(g, OP_MAX_POOL, x, kernel, strides, pads_begin, pads_end, 0, ceil_mode,
+                    g->nodes[x].dtype, id);
+}
+
+int hipie_graph_avg_pool(hipie_graph* g, int x, const int64_t* kernel, const int64_t* strides,
+                         const int64_t* pads_begin, const int64_t* pads_end, int exclude_pad, int ceil_mode,
+                         int out_dtype, int* id) {
+    return add_pool(g, OP_AVG_POOL, x, kernel, strides, pads_begin, pads_end, exclude_pad, ceil_mode,
+                    out_dtype, id);
+}
+
+int hipie_graph_reshape(hipie_graph* g, int x, const int64_t* dims, int rank, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id && dims, HIPIE_PARAMETER_MISMATCH, "hipie_graph_reshape: null argument");
+        GNode& X = node(g, x, "hipie_graph_reshape");
+        GNode n;
+        n.op = OP_RESHAPE;
+        n.in = {x};
+        n.dtype = X.dtype;
+        n.shape.assign(dims, dims + rank);
+        HIPIE_REQUIRE(n.numel() == X.numel(), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_graph_reshape: element count changes");
+        *id = add_node(g, std::move(n));
+    });
+}
+
+int hipie_graph_result(hipie_graph* g, int x, const char* name) {
+    return guarded([&] {
+        GNode& X = node(g, x, "hipie_graph_result");
+        GNode n;
+        n.op = OP_RESULT;
+        n.in = {x};
+        n.name = name ? name : X.name;
+        n.dtype = X.dtype;
+        n.shape = X.shape;
+        g->results.push_back(add_node(g, std::move(n)));
+    });
+}
+
+int hipie_graph_set_name(hipie_graph* g, int id, const char* name) {
+    return guarded([&] {
+        HIPIE_REQUIRE(name, HIPIE_PARAMETER_MISMATCH, "hipie_graph_set_name: null name");
+        node(g, id, "hipie_graph_set_name").name = name;
+    });
+}
+
+}  // extern "C"

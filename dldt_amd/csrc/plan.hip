@@ -1,0 +1,859 @@
+// Planner: post-LPT graph -> fused steps over one static HBM arena -> infer requests.
+//
+// The matcher walks the graph demand-driven from the Results.  A Convolution / MatMul head
+// absorbs the elementwise chain LPT leaves behind it (Add bias, dequantization Multiply, residual
+// Add, ReLU/Clamp, FakeQuantize) into one kernel epilogue; Convert/Subtract/Multiply chains over
+// byte tensors stay symbolic ("dequantization views") until a consumer fuses or materialises
+// them.  Every materialised tensor gets its own arena region (NHWC, padded channels, a halo as
+// wide as the largest padding among its consumers, pre-filled with level 0 once); nothing is
+// allocated or freed after compilation.
+#include <chrono>
+#include <condition_variable>
+#include <mutex>
+
+#include "graph.h"
+
+namespace hipie {
+namespace {
+
+struct TensorInfo {
+    int dtype = HIPIE_U8B;   // storage type
+    int n = 1, h = 1, w = 1, c = 1, cs = 16, halo = 0;
+    int64_t offset = 0, bytes = 0;
+    int producer = -1;       // graph node whose value it holds
+    int64_t esize() const { return dtype == HIPIE_F32 || dtype == HIPIE_I32 ? 4 : 1; }
+    int wp() const { return w + 2 * halo; }
+    int hp() const { return h + 2 * halo; }
+    hipie_tensor desc(uint8_t* arena) const {
+        hipie_tensor t;
+        t.dtype = dtype; t.n = n; t.h = h; t.w = w; t.c = c;
+        t.stride_w = cs;
+        t.stride_h = static_cast<int64_t>(wp()) * cs;
+        t.stride_n = static_cast<int64_t>(hp()) * wp() * cs;
+        t.halo = halo;
+        t.data = arena + offset + (static_cast<int64_t>(halo) * wp() + halo) * cs * esize();
+        return t;
+    }
+};
+
+enum ValueKind { VK_NONE = 0, VK_PARAM, VK_CONST, VK_TENSOR, VK_DEQ, VK_FUSED };
+
+struct Value {
+    int kind = VK_NONE;
+    int tensor = -1;
+    std::vector<float> sub, mul;   // VK_DEQ: (float(q) - sub) * mul, each empty / 1 / C values
+};
+
+struct EpilogueSpec {
+    std::vector<float> bias, scale, res_sub, res_mul, post_scale, fq_il, fq_ih;
+    int residual_dtype = 0, activation = 0, out_dtype = HIPIE_F32;
+    float clamp_lo = 0, clamp_hi = 0, fq_ol = 0, fq_oh = 0;
+    int64_t levels = 0;
+    hipie_epilogue c_struct() const {
+        hipie_epilogue e{};
+        auto set = [](const std::vector<float>& v, const float*& p, int64_t& n) {
+            if (!v.empty()) { p = v.data(); n = static_cast<int64_t>(v.size()); }
+        };
+        set(bias, e.bias, e.n_bias);
+        set(scale, e.scale, e.n_scale);
+        e.residual_dtype = residual_dtype;
+        set(res_sub, e.res_sub, e.n_res_sub);
+        set(res_mul, e.res_mul, e.n_res_mul);
+        set(post_scale, e.post_scale, e.n_post_scale);
+        e.activation = activation;
+        e.clamp_lo = clamp_lo;
+        e.clamp_hi = clamp_hi;
+        e.out_dtype = out_dtype;
+        e.fq_levels = levels;
+        set(fq_il, e.fq_in_low, e.n_fq_in_low);
+        set(fq_ih, e.fq_in_high, e.n_fq_in_high);
+        e.fq_out_low = fq_ol;
+        e.fq_out_high = fq_oh;
+        return e;
+    }
+};
+
+struct Step {
+    std::string name, type;
+    int64_t macs = 0, bytes = 0;
+    int out_node = -1;
+    virtual ~Step() = default;
+    virtual void create(int device, const std::vector<TensorInfo>& tensors) = 0;
+    virtual void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs,
+                     void* const* outputs, hipStream_t s) const = 0;
+};
+
+void check_status(int st, const char* what) {
+    if (st != HIPIE_OK) fail(static_cast<hipie_status>(st), "%s: %s", what, hipie_last_error());
+}
+
+// FakeQuantize on a graph input: f32 NCHW in the request's input buffer -> byte NHWC tensor
+struct EntryStep : Step {
+    int param_index = 0, out = -1;
+    int64_t channels = 0, levels = 0;
+    std::vector<float> il, ih, ol, oh;
+    hipie_fq* fq = nullptr;
+    ~EntryStep() override { hipie_fq_destroy(fq); }
+    void create(int device, const std::vector<TensorInfo>&) override {
+        check_status(hipie_fq_create(device, channels, levels, il.data(), il.size(), ih.data(), ih.size(),
+                                     ol.data(), ol.size(), oh.data(), oh.size(), &fq), name.c_str());
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
+             hipStream_t s) const override {
+        const hipie_tensor d = tensors[out].desc(arena);
+        check_status(hipie_fq_run_q8_tensor(fq, static_cast<const float*>(inputs[param_index]), &d, s),
+                     name.c_str());
+    }
+};
+
+struct ConvStep : Step {
+    int in = -1, res = -1, out = -1;
+    hipie_conv_desc desc{};
+    std::vector<int8_t> weights;   // OIHW
+    EpilogueSpec epi;
+    hipie_conv* conv = nullptr;
+    ~ConvStep() override { hipie_conv_destroy(conv); }
+    void create(int device, const std::vector<TensorInfo>& tensors) override {
+        const TensorInfo& t = tensors[in];
+        desc.in_dtype = t.dtype;
+        desc.in_c_stride = t.cs;
+        desc.in_stride_w = t.cs;
+        desc.in_stride_h = t.wp() * t.cs;
+        const hipie_epilogue e = epi.c_struct();
+        check_status(hipie_conv_create(device, &desc, weights.data(), &e, &conv), name.c_str());
+        weights.clear();
+        weights.shrink_to_fit();
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const*, void* const*,
+             hipStream_t s) const override {
+        const hipie_tensor i = tensors[in].desc(arena), o = tensors[out].desc(arena);
+        hipie_tensor r{};
+        if (res >= 0) r = tensors[res].desc(arena);
+        check_status(hipie_conv_run(conv, &i, res >= 0 ? &r : nullptr, &o, s), name.c_str());
+    }
+};
+
+struct PoolStep : Step {
+    int in = -1, out = -1;
+    bool avg = false, rcp = false;
+    PoolArgs a{};
+    std::vector<float> mul, fq_il, fq_ih;
+    float fq_ol = 0, fq_oh = 0;
+    int64_t levels = 0;
+    DeviceBuffer d_mul, d_il, d_ih, d_d, d_r;
+    void create(int device, const std::vector<TensorInfo>& tensors) override {
+        const TensorInfo& ti = tensors[in];
+        const TensorInfo& to = tensors[out];
+        a.M = to.n * to.h * to.w;
+        a.OW = to.w;
+        a.OHOW = to.h * to.w;
+        a.H = ti.h;
+        a.W = ti.w;
+        a.cs = to.cs;
+        a.in_bias = ti.dtype == HIPIE_U8B ? 128 : 0;
+        auto expand = [&](const std::vector<float>& v, float pad) {
+            std::vector<float> o(to.cs, pad);
+            for (int c = 0; c < to.c; ++c) o[c] = v[v.size() == 1 ? 0 : c];
+            return o;
+        };
+        if (!mul.empty()) {
+            const auto m = expand(mul, 1.f);
+            d_mul.upload(device, m.data(), m.size() * 4);
+            a.mul = d_mul.as<float>();
+        }
+        if (!fq_il.empty()) {
+            const auto il = expand(fq_il, 0.f), ih = expand(fq_ih, 1.f);
+            std::vector<float> d(to.cs), r(to.cs);
+            a.lm1 = static_cast<float>(static_cast<size_t>(levels - 1));
+            rcp = true;
+            for (int c = 0; c < to.cs; ++c) {
+                HIPIE_REQUIRE(il[c] < ih[c], HIPIE_NOT_IMPLEMENTED, "%s: FakeQuantize needs low < high", name.c_str());
+                FqChannel p{};
+                p.il = il[c]; p.ih = ih[c]; p.lo = il[c]; p.hi = ih[c]; p.d = ih[c] - il[c];
+                p.r = fq_rounded_reciprocal(p.d);
+                d[c] = p.d;
+                r[c] = p.r;
+                if (!fq_reciprocal_exact_on_boundaries(p, a.lm1)) rcp = false;
+            }
+            HIPIE_REQUIRE(fq_ol == std::nearbyintf(fq_ol) && fq_oh == fq_ol + a.lm1, HIPIE_NOT_IMPLEMENTED,
+                          "%s: output range is not consecutive integers", name.c_str());
+            for (int k = 0; k < levels; ++k)
+                HIPIE_REQUIRE((static_cast<float>(k) / a.lm1 * (fq_oh - fq_ol) + fq_ol) == fq_ol + k,
+                              HIPIE_NOT_IMPLEMENTED, "%s: output levels are not integers", name.c_str());
+            a.out_off = to.dtype == HIPIE_U8B ? fq_ol - 128.f : fq_ol;
+            d_il.upload(device, il.data(), il.size() * 4);
+            d_ih.upload(device, ih.data(), ih.size() * 4);
+            d_d.upload(device, d.data(), d.size() * 4);
+            d_r.upload(device, r.data(), r.size() * 4);
+            a.fq_il = d_il.as<float>(); a.fq_ih = d_ih.as<float>();
+            a.fq_d = d_d.as<float>(); a.fq_r = d_r.as<float>();
+        }
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const*, void* const*,
+             hipStream_t s) const override {
+        const hipie_tensor i = tensors[in].desc(arena), o = tensors[out].desc(arena);
+        PoolArgs b = a;
+        b.in = i.data;
+        b.out = o.data;
+        b.in_sn = static_cast<int32_t>(i.stride_n); b.in_sh = static_cast<int32_t>(i.stride_h);
+        b.in_sw = static_cast<int32_t>(i.stride_w);
+        b.out_sn = static_cast<int32_t>(o.stride_n); b.out_sh = static_cast<int32_t>(o.stride_h);
+        b.out_sw = static_cast<int32_t>(o.stride_w);
+        if (avg) launch_avg_pool(b, rcp, s);
+        else launch_max_pool(b, s);
+        HIPIE_CHECK_HIP(hipGetLastError());
+    }
+};
+
+// Result: engine tensor -> dense NCHW output buffer of the request (f32, or u8 levels)
+struct ExitStep : Step {
+    int in = -1, result_index = 0, C = 0;
+    bool out_u8 = false;
+    std::vector<float> sub, mul;
+    DeviceBuffer d_sub, d_mul;
+    void create(int device, const std::vector<TensorInfo>&) override {
+        auto expand = [&](const std::vector<float>& v) {
+            std::vector<float> o(C);
+            for (int c = 0; c < C; ++c) o[c] = v[v.size() == 1 ? 0 : c];
+            return o;
+        };
+        if (!sub.empty()) { const auto v = expand(sub); d_sub.upload(device, v.data(), v.size() * 4); }
+        if (!mul.empty()) { const auto v = expand(mul); d_mul.upload(device, v.data(), v.size() * 4); }
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const*, void* const* outputs,
+             hipStream_t s) const override {
+        const TensorInfo& t = tensors[in];
+        const hipie_tensor i = t.desc(arena);
+        ExitArgs a{};
+        a.in = i.data;
+        a.out = outputs[result_index];
+        a.N = t.n; a.C = t.c; a.HW = t.h * t.w; a.W = t.w;
+        a.in_sn = static_cast<int32_t>(i.stride_n); a.in_sh = static_cast<int32_t>(i.stride_h);
+        a.in_sw = static_cast<int32_t>(i.stride_w);
+        a.in_bias = t.dtype == HIPIE_U8B ? 128.f : 0.f;
+        a.sub = sub.empty() ? nullptr : d_sub.as<float>();
+        a.mul = mul.empty() ? nullptr : d_mul.as<float>();
+        a.out_u8 = out_u8;
+        launch_exit(a, t.dtype, s);
+        HIPIE_CHECK_HIP(hipGetLastError());
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
+struct Planner {
+    const hipie_graph& g;
+    std::vector<Value> values;
+    std::vector<TensorInfo> tensors;
+    std::vector<std::unique_ptr<Step>> steps;
+    std::vector<char> visiting;
+
+    explicit Planner(const hipie_graph& graph) : g(graph), values(graph.nodes.size()), visiting(graph.nodes.size(), 0) {}
+
+    const GNode& N(int id) const { return g.nodes[id]; }
+
+    [[noreturn]] void unsupported(int id, const char* why) const {
+        fail(HIPIE_NOT_IMPLEMENTED, "node %d '%s' (%s): %s", id, N(id).name.c_str(), op_name(N(id).op), why);
+    }
+
+    // constant broadcastable along the channel axis of an [N, C, ...] value: 1 or C numbers
+    bool channel_constant(int id, int64_t C, size_t out_rank, std::vector<float>& v) const {
+        const GNode& c = N(id);
+        if (c.op != OP_CONSTANT || c.dtype != HIPIE_F32) return false;
+        const int64_t n = c.numel();
+        if (n == 1) { v.assign(1, c.f32()[0]); return true; }
+        if (n != C) return false;
+        // the single non-unit axis must align with axis 1 of the output
+        const size_t r = c.shape.size();
+        for (size_t i = 0; i < r; ++i)
+            if (c.shape[i] != 1 && i + out_rank - r != 1) return false;
+        v.assign(c.f32(), c.f32() + C);
+        return true;
+    }
+
+    int new_tensor(int node, int dtype, int n, int h, int w, int c, int cs = 0) {
+        TensorInfo t;
+        t.dtype = dtype; t.n = n; t.h = h; t.w = w; t.c = c;
+        const int gran = (dtype == HIPIE_F32 || dtype == HIPIE_I32) ? 4 : 16;
+        t.cs = cs ? cs : static_cast<int>(round_up(c, gran));
+        t.producer = node;
+        tensors.push_back(t);
+        return static_cast<int>(tensors.size()) - 1;
+    }
+
+    static void nhwc_dims(const std::vector<int64_t>& s, int& n, int& c, int& h, int& w) {
+        n = static_cast<int>(s[0]);
+        c = static_cast<int>(s.size() > 1 ? s[1] : 1);
+        h = static_cast<int>(s.size() > 2 ? s[2] : 1);
+        w = static_cast<int>(s.size() > 3 ? s[3] : 1);
+    }
+
+    int storage_type(int graph_dtype) const { return graph_dtype == HIPIE_U8 ? HIPIE_U8B : graph_dtype; }
+
+    const Value& value(int id) {
+        if (!visit(id)) unsupported(id, "value depends on a node that is still being planned");
+        return values[id];
+    }
+
+    bool single_user(int id) const { return N(id).users.size() == 1; }
+
+    // Post-order: producers first, so a Convolution / pooling head is planned before the
+    // elementwise nodes behind it and can absorb them.  Returns false when the node (or one of
+    // its inputs) is already on the visiting stack, i.e. it cannot be scheduled yet.
+    bool visit(int id) {
+        if (values[id].kind != VK_NONE) return true;
+        if (visiting[id]) return false;
+        visiting[id] = 1;
+        bool ok = true;
+        for (int i : N(id).in) ok = visit(i) && ok;
+        if (ok && values[id].kind == VK_NONE) plan_node(id);
+        visiting[id] = 0;
+        return ok;
+    }
+
+    void plan_node(int id) {
+        const GNode& n = N(id);
+        switch (n.op) {
+        case OP_PARAMETER: values[id].kind = VK_PARAM; break;
+        case OP_CONSTANT: values[id].kind = VK_CONST; break;
+        case OP_FAKE_QUANTIZE: plan_fake_quantize(id); break;
+        case OP_CONVOLUTION: case OP_MATMUL: plan_conv(id); break;
+        case OP_GROUP_CONVOLUTION: unsupported(id, "grouped convolution is not planned yet");
+        case OP_CONVERT: case OP_SUBTRACT: case OP_MULTIPLY: plan_dequant(id); break;
+        case OP_MAX_POOL: case OP_AVG_POOL: plan_pool(id); break;
+        case OP_RESHAPE: plan_reshape(id); break;
+        case OP_RESULT: plan_result(id); values[id].kind = VK_FUSED; break;
+        default: unsupported(id, "only planned as part of a fused convolution / pooling chain");
+        }
+        if (values[id].kind == VK_NONE) unsupported(id, "planner produced no value");
+    }
+
+    void plan_fake_quantize(int id) {
+        const GNode& n = N(id);
+        const Value& x = value(n.in[0]);
+        if (x.kind != VK_PARAM) unsupported(id, "stand-alone FakeQuantize is only planned on graph inputs");
+        if (n.dtype == HIPIE_F32) unsupported(id, "FakeQuantize with f32 output (graph was not run through LPT)");
+        const GNode& p = N(n.in[0]);
+        HIPIE_REQUIRE(p.dtype == HIPIE_F32, HIPIE_NOT_IMPLEMENTED, "u8 graph inputs are not planned yet");
+        auto st = std::make_unique<EntryStep>();
+        int nn, c, h, w;
+        nhwc_dims(n.shape, nn, c, h, w);
+        st->channels = c;
+        st->levels = n.levels;
+        std::vector<float>* dst[4] = {&st->il, &st->ih, &st->ol, &st->oh};
+        for (int i = 0; i < 4; ++i)
+            if (!channel_constant(n.in[1 + i], c, n.shape.size(), *dst[i]))
+                unsupported(id, "FakeQuantize bounds must be scalars or per-channel constants");
+        for (size_t i = 0; i < g.params.size(); ++i)
+            if (g.params[i] == n.in[0]) st->param_index = static_cast<int>(i);
+        // small-channel images keep a 4-byte pixel so the first convolution reads filter rows contiguously
+        st->out = new_tensor(id, storage_type(n.dtype), nn, h, w, c, c <= 4 ? 4 : 0);
+        st->name = n.name;
+        st->type = "FakeQuantize";
+        st->bytes = n.numel() * 5;
+        st->out_node = id;
+        values[id].kind = VK_TENSOR;
+        values[id].tensor = st->out;
+        steps.push_back(std::move(st));
+    }
+
+    void plan_dequant(int id) {
+        const GNode& n = N(id);
+        const Value& x = value(n.in[0]);
+        Value v;
+        if (n.op == OP_CONVERT) {
+            if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1 || n.dtype != HIPIE_F32)
+                unsupported(id, "Convert is planned only as the start of a dequantization (u8/i8 -> f32)");
+            v.kind = VK_DEQ;
+            v.tensor = x.tensor;
+        } else {
+            if (x.kind != VK_DEQ) unsupported(id, "stand-alone elementwise op outside a fused chain");
+            std::vector<float> c;
+            if (!channel_constant(n.in[1], tensors[x.tensor].c, n.shape.size(), c))
+                unsupported(id, "dequantization constant must be scalar or per-channel");
+            v = x;
+            if (n.op == OP_SUBTRACT) {
+                if (!v.mul.empty() || !v.sub.empty()) unsupported(id, "Subtract after Multiply in a dequantization");
+                v.sub = c;
+            } else {
+                if (!v.mul.empty()) unsupported(id, "two Multiplies in a dequantization");
+                v.mul = c;
+            }
+        }
+        values[id] = v;
+    }
+
+    void plan_reshape(int id) {
+        const GNode& n = N(id);
+        const Value& x = value(n.in[0]);
+        const GNode& src = N(n.in[0]);
+        // [N, C, 1, 1] <-> [N, C]: same bytes in NHWC
+        const bool flatten = src.shape.size() == 4 && n.shape.size() == 2 && src.shape[2] == 1 &&
+                             src.shape[3] == 1 && n.shape[0] == src.shape[0] && n.shape[1] == src.shape[1];
+        if (!flatten || (x.kind != VK_TENSOR && x.kind != VK_DEQ))
+            unsupported(id, "only [N,C,1,1] -> [N,C] reshapes are planned");
+        values[id] = x;
+    }
+
+    void plan_conv(int id) {
+        const GNode& n = N(id);
+        const bool is_mm = n.op == OP_MATMUL;
+        const Value x = value(n.in[0]);
+        if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1)
+            unsupported(id, x.kind == VK_DEQ ? "activation zero points / unquantized inputs are not planned yet"
+                                             : "input must be a quantized (u8/i8) tensor");
+        const GNode& W = N(n.in[1]);
+        if (W.op != OP_CONSTANT || W.dtype != HIPIE_I8) unsupported(id, "weights must be an i8 constant");
+        auto st = std::make_unique<ConvStep>();
+        const TensorInfo& tin = tensors[x.tensor];
+        hipie_conv_desc& d = st->desc;
+        d.groups = 1;
+        int64_t OC, IC;
+        if (is_mm) {
+            if (n.ta || W.shape.size() != 2 || N(n.in[0]).shape.size() != 2)
+                unsupported(id, "MatMul is planned for [N,K] x constant [K,OC] / [OC,K]^T");
+            IC = n.tb ? W.shape[1] : W.shape[0];
+            OC = n.tb ? W.shape[0] : W.shape[1];
+            d.kh = d.kw = d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1;
+            st->weights.resize(OC * IC);
+            const int8_t* w = reinterpret_cast<const int8_t*>(W.data.data());
+            for (int64_t o = 0; o < OC; ++o)
+                for (int64_t k = 0; k < IC; ++k) st->weights[o * IC + k] = n.tb ? w[o * IC + k] : w[k * OC + o];
+        } else {
+            OC = W.shape[0];
+            IC = W.shape[1];
+            d.kh = static_cast<int>(W.shape[2]); d.kw = static_cast<int>(W.shape[3]);
+            d.stride_h = static_cast<int>(n.strides[0]); d.stride_w = static_cast<int>(n.strides[1]);
+            d.dil_h = static_cast<int>(n.dilations[0]); d.dil_w = static_cast<int>(n.dilations[1]);
+            d.pad_top = static_cast<int>(n.pads_begin[0]); d.pad_left = static_cast<int>(n.pads_begin[1]);
+            d.pad_bottom = static_cast<int>(n.pads_end[0]); d.pad_right = static_cast<int>(n.pads_end[1]);
+            st->weights.assign(reinterpret_cast<const int8_t*>(W.data.data()),
+                               reinterpret_cast<const int8_t*>(W.data.data()) + W.data.size());
+        }
+        d.ic = static_cast<int>(IC);
+        d.oc = static_cast<int>(OC);
+        HIPIE_REQUIRE(tin.c == IC, HIPIE_PARAMETER_MISMATCH, "node %d: input has %d channels, weights %lld", id,
+                      tin.c, (long long)IC);
+        const int halo = std::max(std::max(d.pad_top, d.pad_bottom), std::max(d.pad_left, d.pad_right));
+        tensors[x.tensor].halo = std::max(tensors[x.tensor].halo, halo);
+        st->in = x.tensor;
+
+        // ---- absorb the elementwise chain behind the accumulator --------------------------------
+        EpilogueSpec& e = st->epi;
+        int cur = id, stage = 0;
+        const size_t rank = n.shape.size();
+        while (single_user(cur)) {
+            const int nx = N(cur).users[0];
+            const GNode& u = N(nx);
+            if (u.op == OP_ADD || u.op == OP_MULTIPLY) {
+                const int other = u.in[0] == cur ? u.in[1] : u.in[0];
+                std::vector<float> c;
+                if (channel_constant(other, OC, rank, c)) {
+                    if (u.op == OP_ADD && stage < 1) { e.bias = c; stage = 1; }
+                    else if (u.op == OP_MULTIPLY && stage < 2) { e.scale = c; stage = 2; }
+                    else if (u.op == OP_MULTIPLY && stage == 3) { e.post_scale = c; stage = 4; }
+                    else break;
+                } else if (u.op == OP_ADD && stage < 3 && N(other).op != OP_CONSTANT) {
+                    // schedules the other branch first; if that branch is the one being planned
+                    // right now (it reached this Add from the other side) leave the Add to it
+                    if (!visit(other)) break;
+                    const Value r = values[other];
+                    if (r.kind == VK_DEQ) {
+                        const TensorInfo& tr = tensors[r.tensor];
+                        e.residual_dtype = tr.dtype;
+                        e.res_sub = r.sub;
+                        e.res_mul = r.mul;
+                    } else if (r.kind == VK_TENSOR && tensors[r.tensor].dtype == HIPIE_F32) {
+                        e.residual_dtype = HIPIE_F32;
+                    } else {
+                        break;
+                    }
+                    if (N(other).shape != u.shape) break;
+                    st->res = r.tensor;
+                    stage = 3;
+                } else {
+                    break;
+                }
+            } else if (u.op == OP_RELU && stage < 5) {
+                e.activation = 1;
+                stage = 5;
+            } else if (u.op == OP_CLAMP && stage < 5) {
+                e.activation = 2;
+                e.clamp_lo = u.lo;
+                e.clamp_hi = u.hi;
+                stage = 5;
+            } else if (u.op == OP_FAKE_QUANTIZE && u.in[0] == cur && u.dtype != HIPIE_F32) {
+                std::vector<float> ol, oh;
+                if (!channel_constant(u.in[1], OC, rank, e.fq_il) || !channel_constant(u.in[2], OC, rank, e.fq_ih) ||
+                    !channel_constant(u.in[3], OC, rank, ol) || !channel_constant(u.in[4], OC, rank, oh) ||
+                    ol.size() != 1 || oh.size() != 1)
+                    break;
+                e.fq_ol = ol[0];
+                e.fq_oh = oh[0];
+                e.levels = u.levels;
+                e.out_dtype = storage_type(u.dtype);
+                cur = nx;
+                stage = 6;
+                break;
+            } else {
+                break;
+            }
+            cur = nx;
+        }
+        if (e.residual_dtype == 0) { e.res_sub.clear(); e.res_mul.clear(); }
+        // mark the absorbed nodes
+        for (int k = id; k != cur;) {
+            const int nx = N(k).users[0];
+            if (nx != cur) values[nx].kind = VK_FUSED;  // never read: its only user is in the chain
+            k = nx;
+        }
+        int nn, c, h, w;
+        nhwc_dims(N(cur).shape, nn, c, h, w);
+        st->out = new_tensor(cur, e.out_dtype, nn, h, w, c);
+        st->name = N(cur).name;
+        st->type = is_mm ? "MatMul" : "Convolution";
+        st->macs = N(id).numel() * IC * d.kh * d.kw;
+        st->bytes = 0;
+        st->out_node = cur;
+        values[cur].kind = VK_TENSOR;
+        values[cur].tensor = st->out;
+        if (cur != id) values[id].kind = VK_FUSED;
+        steps.push_back(std::move(st));
+    }
+
+    void plan_pool(int id) {
+        const GNode& n = N(id);
+        const Value x = value(n.in[0]);
+        if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1)
+            unsupported(id, "pooling is planned on quantized (u8/i8) tensors");
+        auto st = std::make_unique<PoolStep>();
+        st->avg = n.op == OP_AVG_POOL;
+        PoolArgs& a = st->a;
+        a.kh = static_cast<int>(n.kernel[0]); a.kw = static_cast<int>(n.kernel[1]);
+        a.sh = static_cast<int>(n.strides[0]); a.sw = static_cast<int>(n.strides[1]);
+        a.pt = static_cast<int>(n.pads_begin[0]); a.pl = static_cast<int>(n.pads_begin[1]);
+        a.pb = static_cast<int>(n.pads_end[0]); a.pr = static_cast<int>(n.pads_end[1]);
+        a.include_pad = st->avg && !n.exclude_pad;
+        const int halo = std::max(std::max(a.pt, a.pb), std::max(a.pl, a.pr));
+        tensors[x.tensor].halo = std::max(tensors[x.tensor].halo, halo);
+        st->in = x.tensor;
+        int cur = id;
+        int out_dtype = tensors[x.tensor].dtype;
+        if (st->avg) {
+            if (n.dtype != HIPIE_F32) unsupported(id, "AvgPool is planned with f32 output (not precision preserved)");
+            out_dtype = HIPIE_F32;
+            const int64_t C = n.shape[1];
+            bool scaled = false;
+            while (single_user(cur)) {
+                const int nx = N(cur).users[0];
+                const GNode& u = N(nx);
+                std::vector<float> c;
+                if (u.op == OP_MULTIPLY && !scaled &&
+                    channel_constant(u.in[0] == cur ? u.in[1] : u.in[0], C, u.shape.size(), c)) {
+                    st->mul = c;
+                    scaled = true;
+                } else if (u.op == OP_RESHAPE && N(cur).shape.size() == 4 && N(cur).shape[2] == 1 &&
+                           N(cur).shape[3] == 1 && u.shape.size() == 2 && u.shape[1] == C) {
+                    // metadata only
+                } else if (u.op == OP_FAKE_QUANTIZE && u.in[0] == cur && u.dtype != HIPIE_F32) {
+                    std::vector<float> ol, oh;
+                    if (!channel_constant(u.in[1], C, u.shape.size(), st->fq_il) ||
+                        !channel_constant(u.in[2], C, u.shape.size(), st->fq_ih) ||
+                        !channel_constant(u.in[3], C, u.shape.size(), ol) ||
+                        !channel_constant(u.in[4], C, u.shape.size(), oh) || ol.size() != 1 || oh.size() != 1)
+                        break;
+                    st->fq_ol = ol[0];
+                    st->fq_oh = oh[0];
+                    st->levels = u.levels;
+                    out_dtype = storage_type(u.dtype);
+                    cur = nx;
+                    break;
+                } else {
+                    break;
+                }
+                cur = nx;
+            }
+            for (int k = id; k != cur;) {
+                const int nx = N(k).users[0];
+                if (nx != cur) values[nx].kind = VK_FUSED;
+                k = nx;
+            }
+        }
+        int nn, c, h, w;
+        nhwc_dims(n.shape, nn, c, h, w);
+        st->out = new_tensor(cur, out_dtype, nn, h, w, c, out_dtype == tensors[x.tensor].dtype ? tensors[x.tensor].cs : 0);
+        st->name = N(cur).name;
+        st->type = st->avg ? "AvgPool" : "MaxPool";
+        st->bytes = N(n.in[0]).numel() + n.numel() * (out_dtype == HIPIE_F32 ? 4 : 1);
+        st->out_node = cur;
+        values[cur].kind = VK_TENSOR;
+        values[cur].tensor = st->out;
+        if (cur != id) values[id].kind = VK_FUSED;
+        steps.push_back(std::move(st));
+    }
+
+    void plan_result(int id) {
+        const GNode& n = N(id);
+        const Value x = value(n.in[0]);
+        if (x.kind != VK_TENSOR && x.kind != VK_DEQ) unsupported(id, "result of a constant or parameter");
+        auto st = std::make_unique<ExitStep>();
+        st->in = x.tensor;
+        st->C = tensors[x.tensor].c;
+        st->sub = x.sub;
+        st->mul = x.mul;
+        st->out_u8 = x.kind == VK_TENSOR && tensors[x.tensor].esize() == 1;
+        for (size_t i = 0; i < g.results.size(); ++i)
+            if (g.results[i] == id) st->result_index = static_cast<int>(i);
+        st->name = n.name;
+        st->type = "Result";
+        st->bytes = n.numel() * 5;
+        st->out_node = id;
+        steps.push_back(std::move(st));
+    }
+};
+
+}  // namespace
+}  // namespace hipie
+
+using namespace hipie;
+
+struct hipie_plan {
+    int device = 0;
+    hipie_graph graph;                       // private copy (constants are dropped after packing)
+    std::vector<TensorInfo> tensors;
+    std::vector<std::unique_ptr<Step>> steps;
+    std::map<int, int> node_tensor;          // graph node -> tensor holding its value
+    int64_t arena_bytes = 0;
+    struct Io { std::string name; int dtype; std::vector<int64_t> shape; int64_t bytes; };
+    std::vector<Io> inputs, outputs;
+};
+
+struct hipie_request {
+    const hipie_plan* plan = nullptr;
+    DeviceBuffer arena;
+    std::vector<DeviceBuffer> in_dev, out_dev;
+    hipStream_t stream = nullptr;
+    bool perf = false;
+    std::vector<hipEvent_t> events;
+    bool started = false;
+    std::vector<void*> pending_out;          // host destinations of the running async infer
+    ~hipie_request() {
+        for (auto e : events) (void)hipEventDestroy(e);
+        if (stream) (void)hipStreamDestroy(stream);
+    }
+};
+
+namespace {
+
+__global__ void fill_bytes(uint8_t* p, int64_t n, uint8_t v) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+
+void enqueue(hipie_request* r, void* const* in, void* const* out) {
+    const hipie_plan& p = *r->plan;
+    uint8_t* arena = r->arena.as<uint8_t>();
+    for (size_t i = 0; i < p.steps.size(); ++i) {
+        if (r->perf) HIPIE_CHECK_HIP(hipEventRecord(r->events[i], r->stream));
+        p.steps[i]->run(arena, p.tensors, in, out, r->stream);
+    }
+    if (r->perf) HIPIE_CHECK_HIP(hipEventRecord(r->events[p.steps.size()], r->stream));
+}
+
+}  // namespace
+
+extern "C" {
+
+int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
+    return guarded([&] {
+        HIPIE_REQUIRE(g && out, HIPIE_PARAMETER_MISMATCH, "hipie_compile: null argument");
+        HIPIE_REQUIRE(!g->results.empty(), HIPIE_PARAMETER_MISMATCH, "hipie_compile: graph has no Result");
+        auto plan = std::make_unique<hipie_plan>();
+        plan->device = device;
+        Planner pl(*g);
+        for (int r : g->results) pl.visit(r);
+        // arena layout: one region per tensor, 256-byte aligned, with slack on both sides so that
+        // K-padding reads of a first-layer filter row stay inside the arena
+        int64_t off = 256;
+        for (auto& t : pl.tensors) {
+            t.bytes = static_cast<int64_t>(t.n) * t.hp() * t.wp() * t.cs * t.esize();
+            t.offset = off;
+            off = round_up(off + t.bytes + 256, 256);
+        }
+        plan->arena_bytes = off;
+        plan->tensors = pl.tensors;
+        for (auto& s : pl.steps) s->create(device, plan->tensors);
+        plan->steps = std::move(pl.steps);
+        for (size_t i = 0; i < pl.values.size(); ++i)
+            if (pl.values[i].kind == VK_TENSOR) plan->node_tensor[static_cast<int>(i)] = pl.values[i].tensor;
+        for (int p : g->params) {
+            const GNode& n = g->nodes[p];
+            plan->inputs.push_back({n.name, n.dtype, n.shape, n.numel() * (n.dtype == HIPIE_F32 ? 4 : 1)});
+        }
+        for (int r : g->results) {
+            const GNode& n = g->nodes[r];
+            const int dt = n.dtype == HIPIE_F32 ? HIPIE_F32 : HIPIE_U8;
+            plan->outputs.push_back({n.name, dt, n.shape, n.numel() * (dt == HIPIE_F32 ? 4 : 1)});
+        }
+        *out = plan.release();
+    });
+}
+
+void hipie_plan_destroy(hipie_plan* p) { delete p; }
+
+int hipie_plan_num_inputs(const hipie_plan* p) { return p ? static_cast<int>(p->inputs.size()) : 0; }
+int hipie_plan_num_outputs(const hipie_plan* p) { return p ? static_cast<int>(p->outputs.size()) : 0; }
+int hipie_plan_num_steps(const hipie_plan* p) { return p ? static_cast<int>(p->steps.size()) : 0; }
+int64_t hipie_plan_arena_bytes(const hipie_plan* p) { return p ? p->arena_bytes : 0; }
+
+int hipie_plan_io_desc(const hipie_plan* p, int is_output, int index, char* name, size_t name_len, int* dtype,
+                       int64_t* dims, int* rank) {
+    return guarded([&] {
+        HIPIE_REQUIRE(p && dtype && dims && rank, HIPIE_PARAMETER_MISMATCH, "hipie_plan_io_desc: null argument");
+        const auto& v = is_output ? p->outputs : p->inputs;
+        HIPIE_REQUIRE(index >= 0 && index < static_cast<int>(v.size()), HIPIE_OUT_OF_BOUNDS,
+                      "hipie_plan_io_desc: index %d", index);
+        if (name && name_len) snprintf(name, name_len, "%s", v[index].name.c_str());
+        *dtype = v[index].dtype;
+        *rank = static_cast<int>(v[index].shape.size());
+        for (int i = 0; i < *rank; ++i) dims[i] = v[index].shape[i];
+    });
+}
+
+int hipie_plan_step_info(const hipie_plan* p, int index, char* name, size_t name_len, char* type,
+                         size_t type_len, int64_t* macs, int64_t* bytes) {
+    return guarded([&] {
+        HIPIE_REQUIRE(p && index >= 0 && index < static_cast<int>(p->steps.size()), HIPIE_OUT_OF_BOUNDS,
+                      "hipie_plan_step_info: index %d", index);
+        const Step& s = *p->steps[index];
+        if (name && name_len) snprintf(name, name_len, "%s", s.name.c_str());
+        if (type && type_len) snprintf(type, type_len, "%s", s.type.c_str());
+        if (macs) *macs = s.macs;
+        if (bytes) *bytes = s.bytes;
+    });
+}
+
+int hipie_request_create(const hipie_plan* p, int perf_count, hipie_request** out) {
+    return guarded([&] {
+        HIPIE_REQUIRE(p && out, HIPIE_PARAMETER_MISMATCH, "hipie_request_create: null argument");
+        auto r = std::make_unique<hipie_request>();
+        r->plan = p;
+        r->perf = perf_count != 0;
+        DeviceGuard g(p->device);
+        HIPIE_CHECK_HIP(hipStreamCreateWithFlags(&r->stream, hipStreamNonBlocking));
+        r->arena.alloc(p->device, static_cast<size_t>(p->arena_bytes));
+        // level 0 everywhere: halos and channel padding are never written again
+        uint8_t* a = r->arena.as<uint8_t>();
+        HIPIE_CHECK_HIP(hipMemsetAsync(a, 0, static_cast<size_t>(p->arena_bytes), r->stream));
+        for (const auto& t : p->tensors)
+            if (t.dtype == HIPIE_U8B)
+                hipLaunchKernelGGL(fill_bytes, dim3(1024), dim3(256), 0, r->stream, a + t.offset, t.bytes,
+                                   static_cast<uint8_t>(0x80));
+        HIPIE_CHECK_HIP(hipGetLastError());
+        for (const auto& io : p->inputs) {
+            r->in_dev.emplace_back();
+            r->in_dev.back().alloc(p->device, static_cast<size_t>(io.bytes));
+        }
+        for (const auto& io : p->outputs) {
+            r->out_dev.emplace_back();
+            r->out_dev.back().alloc(p->device, static_cast<size_t>(io.bytes));
+        }
+        if (r->perf) {
+            r->events.resize(p->steps.size() + 1);
+            for (auto& e : r->events) HIPIE_CHECK_HIP(hipEventCreate(&e));
+        }
+        HIPIE_CHECK_HIP(hipStreamSynchronize(r->stream));
+        *out = r.release();
+    });
+}
+
+void hipie_request_destroy(hipie_request* r) {
+    if (r && r->stream) (void)hipStreamSynchronize(r->stream);
+    delete r;
+}
+
+int hipie_request_stream(hipie_request* r, void** stream) {
+    return guarded([&] {
+        HIPIE_REQUIRE(r && stream, HIPIE_PARAMETER_MISMATCH, "hipie_request_stream: null argument");
+        *stream = r->stream;
+    });
+}
+
+int hipie_request_start(hipie_request* r, const void* const* inputs, void* const* outputs, int device_memory) {
+    return guarded([&] {
+        HIPIE_REQUIRE(r && inputs && outputs, HIPIE_PARAMETER_MISMATCH, "hipie_request_start: null argument");
+        HIPIE_REQUIRE(!r->started, HIPIE_REQUEST_BUSY, "hipie_request_start: request is busy");
+        const hipie_plan& p = *r->plan;
+        DeviceGuard g(p.device);
+        std::vector<void*> in(p.inputs.size()), out(p.outputs.size());
+        for (size_t i = 0; i < in.size(); ++i) {
+            HIPIE_REQUIRE(inputs[i], HIPIE_PARAMETER_MISMATCH, "hipie_request_start: input %zu is null", i);
+            if (device_memory) {
+                in[i] = const_cast<void*>(inputs[i]);
+            } else {
+                in[i] = r->in_dev[i].ptr;
+                HIPIE_CHECK_HIP(hipMemcpyAsync(in[i], inputs[i], static_cast<size_t>(p.inputs[i].bytes),
+                                               hipMemcpyHostToDevice, r->stream));
+            }
+        }
+        for (size_t i = 0; i < out.size(); ++i) {
+            HIPIE_REQUIRE(outputs[i], HIPIE_PARAMETER_MISMATCH, "hipie_request_start: output %zu is null", i);
+            out[i] = device_memory ? outputs[i] : r->out_dev[i].ptr;
+        }
+        enqueue(r, in.data(), out.data());
+        if (!device_memory)
+            for (size_t i = 0; i < out.size(); ++i)
+                HIPIE_CHECK_HIP(hipMemcpyAsync(outputs[i], out[i], static_cast<size_t>(p.outputs[i].bytes),
+                                               hipMemcpyDeviceToHost, r->stream));
+        r->started = true;
+    });
+}
+
+int hipie_request_wait(hipie_request* r) {
+    return guarded([&] {
+        HIPIE_REQUIRE(r, HIPIE_PARAMETER_MISMATCH, "hipie_request_wait: null argument");
+        HIPIE_REQUIRE(r->started, HIPIE_INFER_NOT_STARTED, "hipie_request_wait: nothing was started");
+        DeviceGuard g(r->plan->device);
+        r->started = false;
+        HIPIE_CHECK_HIP(hipStreamSynchronize(r->stream));
+    });
+}
+
+int hipie_request_infer(hipie_request* r, const void* const* inputs, void* const* outputs, int device_memory) {
+    const int st = hipie_request_start(r, inputs, outputs, device_memory);
+    return st != HIPIE_OK ? st : hipie_request_wait(r);
+}
+
+/* enqueue only (no copies, no synchronisation): inputs/outputs are device buffers and the caller
+ * owns ordering on the request's stream; used for back-to-back throughput runs */
+int hipie_request_enqueue(hipie_request* r, const void* const* inputs, void* const* outputs) {
+    return guarded([&] {
+        HIPIE_REQUIRE(r && inputs && outputs, HIPIE_PARAMETER_MISMATCH, "hipie_request_enqueue: null argument");
+        DeviceGuard g(r->plan->device);
+        std::vector<void*> in(r->plan->inputs.size());
+        for (size_t i = 0; i < in.size(); ++i) in[i] = const_cast<void*>(inputs[i]);
+        enqueue(r, in.data(), outputs);
+    });
+}
+
+int hipie_request_perf(hipie_request* r, int step, float* ms) {
+    return guarded([&] {
+        HIPIE_REQUIRE(r && ms, HIPIE_PARAMETER_MISMATCH, "hipie_request_perf: null argument");
+        HIPIE_REQUIRE(r->perf, HIPIE_NOT_FOUND, "hipie_request_perf: request was created without PERF_COUNT");
+        HIPIE_REQUIRE(step >= 0 && step < static_cast<int>(r->plan->steps.size()), HIPIE_OUT_OF_BOUNDS,
+                      "hipie_request_perf: step %d", step);
+        HIPIE_CHECK_HIP(hipEventElapsedTime(ms, r->events[step], r->events[step + 1]));
+    });
+}
+
+/* the arena tensor that holds the value of graph node `node_id` (for inspection and tests) */
+int hipie_request_tensor(const hipie_request* r, int node_id, hipie_tensor* t) {
+    return guarded([&] {
+        HIPIE_REQUIRE(r && t, HIPIE_PARAMETER_MISMATCH, "hipie_request_tensor: null argument");
+        auto it = r->plan->node_tensor.find(node_id);
+        HIPIE_REQUIRE(it != r->plan->node_tensor.end(), HIPIE_NOT_FOUND,
+                      "hipie_request_tensor: node %d was fused away or is not a tensor", node_id);
+        *t = r->plan->tensors[it->second].desc(r->arena.as<uint8_t>());
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,154 @@
+// Precision-preserved ops on the engine's NHWC byte tensors (HBM-bound): MaxPool, AvgPool with an
+// optional fused requantize, and the exit conversion back to the reference's NCHW layout.
+// Reference semantics: ngraph/core/reference/.../max_pool.hpp, avg_pool.hpp:114-265.
+#include "pool.h"
+
+namespace hipie {
+namespace {
+
+constexpr int kThreads = 256;
+
+// bytewise signed max of two dwords
+__device__ __forceinline__ uint32_t max_i8x4(uint32_t a, uint32_t b) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int x = static_cast<int8_t>(a >> (8 * j)), y = static_cast<int8_t>(b >> (8 * j));
+        r |= (static_cast<uint32_t>(x > y ? x : y) & 0xffu) << (8 * j);
+    }
+    return r;
+}
+
+// One thread = 16 channels of one output pixel.  Padding cells hold the lowest value (level 0
+// for U8B, -128 for I8) in the tensor's halo, which is the identity of max; the window is
+// trimmed at the padded upper bound as in max_pool.hpp.
+__global__ __launch_bounds__(kThreads) void max_pool_nhwc_i8(PoolArgs a) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const int cg = a.cs / 16;
+    if (t >= static_cast<int64_t>(a.M) * cg) return;
+    const int m = static_cast<int>(t / cg), c = static_cast<int>(t % cg) * 16;
+    const int n = m / a.OHOW, rem = m - n * a.OHOW, oh = rem / a.OW, ow = rem - oh * a.OW;
+    const int y0 = oh * a.sh - a.pt, x0 = ow * a.sw - a.pl;
+    const int y1 = min(y0 + a.kh, a.H + a.pb), x1 = min(x0 + a.kw, a.W + a.pr);
+    uint4 r = make_uint4(0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u);
+    const int8_t* base = static_cast<const int8_t*>(a.in) + static_cast<int64_t>(n) * a.in_sn + c;
+    for (int y = y0; y < y1; ++y)
+        for (int x = x0; x < x1; ++x) {
+            const uint4 v = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(y) * a.in_sh + x * a.in_sw);
+            r.x = max_i8x4(r.x, v.x);
+            r.y = max_i8x4(r.y, v.y);
+            r.z = max_i8x4(r.z, v.z);
+            r.w = max_i8x4(r.w, v.w);
+        }
+    *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + static_cast<int64_t>(n) * a.out_sn +
+                              oh * a.out_sh + ow * a.out_sw + c) = r;
+}
+
+// One thread = 4 channels of one output pixel.  Integer window sum (exact; equals the
+// reference's float accumulation of integer levels below 2^24), float(sum) / n as in
+// avg_pool.hpp:236-262, then optional Multiply and FakeQuantize.
+template <bool RCP>
+__global__ __launch_bounds__(kThreads) void avg_pool_nhwc_i8(PoolArgs a) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const int cg = a.cs / 4;
+    if (t >= static_cast<int64_t>(a.M) * cg) return;
+    const int m = static_cast<int>(t / cg), c = static_cast<int>(t % cg) * 4;
+    const int n = m / a.OHOW, rem = m - n * a.OHOW, oh = rem / a.OW, ow = rem - oh * a.OW;
+    const int y0 = oh * a.sh - a.pt, x0 = ow * a.sw - a.pl;
+    const int y1 = min(y0 + a.kh, a.H + a.pb), x1 = min(x0 + a.kw, a.W + a.pr);
+    const bool padding_present = a.pt || a.pl || a.pb || a.pr;
+    int sum[4] = {0, 0, 0, 0};
+    int count = 0, cells = 0;
+    const int8_t* base = static_cast<const int8_t*>(a.in) + static_cast<int64_t>(n) * a.in_sn + c;
+    for (int y = y0; y < y1; ++y)
+        for (int x = x0; x < x1; ++x) {
+            const bool in_bounds = y >= 0 && y < a.H && x >= 0 && x < a.W;
+            if (in_bounds || a.include_pad) {
+                if (in_bounds) {
+                    const uint32_t v = *reinterpret_cast<const uint32_t*>(base + static_cast<int64_t>(y) * a.in_sh + x * a.in_sw);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) sum[j] += static_cast<int8_t>(v >> (8 * j));
+                    ++cells;
+                }
+                if (!padding_present || (in_bounds && !a.include_pad)) ++count;
+            }
+        }
+    if (a.include_pad && padding_present) count = a.kh * a.kw;
+    const float nf = static_cast<float>(count);
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float x = static_cast<float>(sum[j] + a.in_bias * cells) / nf;
+        if (a.mul) x = x * a.mul[c + j];
+        v[j] = x;
+    }
+    const int64_t o = static_cast<int64_t>(n) * a.out_sn + oh * a.out_sh + ow * a.out_sw + c;
+    if (a.fq_il) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            FqChannel p;
+            p.il = a.fq_il[c + j]; p.ih = a.fq_ih[c + j]; p.d = a.fq_d[c + j]; p.r = a.fq_r[c + j];
+            const float k = fq_level_clamped<RCP>(p, a.lm1, v[j]);
+            packed |= (static_cast<uint32_t>(static_cast<int>(k + a.out_off)) & 0xffu) << (8 * j);
+        }
+        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(a.out) + o) = packed;
+    } else {
+        *reinterpret_cast<float4*>(static_cast<float*>(a.out) + o) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+}
+
+// NHWC engine tensor -> dense NCHW f32 (optionally (x - sub[c]) * mul[c]) or NCHW u8 levels.
+// A block transposes 64 pixels x 64 channels through LDS: channel-contiguous reads, pixel-
+// contiguous writes.
+template <typename TIn>
+__global__ __launch_bounds__(kThreads) void exit_nhwc_to_nchw(ExitArgs a) {
+    __shared__ float tile[64][65];
+    const int n = blockIdx.z, p0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int i = ty; i < 64; i += 4) {   // pixel p0 + i, channel c0 + tx
+        const int p = p0 + i, c = c0 + tx;
+        float v = 0.f;
+        if (p < a.HW && c < a.C) {
+            const int h = p / a.W, w = p - h * a.W;
+            const TIn raw = static_cast<const TIn*>(a.in)[static_cast<int64_t>(n) * a.in_sn + h * a.in_sh + w * a.in_sw + c];
+            v = static_cast<float>(raw) + a.in_bias;
+            if (a.sub) v = v - a.sub[c];
+            if (a.mul) v = v * a.mul[c];
+        }
+        tile[i][tx] = v;
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {   // channel c0 + i, pixel p0 + tx
+        const int p = p0 + tx, c = c0 + i;
+        if (p < a.HW && c < a.C) {
+            const int64_t o = (static_cast<int64_t>(n) * a.C + c) * a.HW + p;
+            if (a.out_u8) static_cast<uint8_t*>(a.out)[o] = static_cast<uint8_t>(static_cast<int>(tile[tx][i]));
+            else static_cast<float*>(a.out)[o] = tile[tx][i];
+        }
+    }
+}
+
+}  // namespace
+
+void launch_max_pool(const PoolArgs& a, hipStream_t s) {
+    const int64_t threads = static_cast<int64_t>(a.M) * (a.cs / 16);
+    hipLaunchKernelGGL(max_pool_nhwc_i8, dim3(static_cast<uint32_t>(ceil_div(threads, kThreads))),
+                       dim3(kThreads), 0, s, a);
+}
+
+void launch_avg_pool(const PoolArgs& a, bool rcp, hipStream_t s) {
+    const int64_t threads = static_cast<int64_t>(a.M) * (a.cs / 4);
+    auto k = rcp ? avg_pool_nhwc_i8<true> : avg_pool_nhwc_i8<false>;
+    hipLaunchKernelGGL(k, dim3(static_cast<uint32_t>(ceil_div(threads, kThreads))), dim3(kThreads), 0, s, a);
+}
+
+void launch_exit(const ExitArgs& a, int in_dtype, hipStream_t s) {
+    dim3 grid(static_cast<uint32_t>(ceil_div(a.HW, 64)), static_cast<uint32_t>(ceil_div(a.C, 64)),
+              static_cast<uint32_t>(a.N));
+    if (in_dtype == HIPIE_F32) hipLaunchKernelGGL(exit_nhwc_to_nchw<float>, grid, dim3(kThreads), 0, s, a);
+    else if (in_dtype == HIPIE_I32) hipLaunchKernelGGL(exit_nhwc_to_nchw<int32_t>, grid, dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL(exit_nhwc_to_nchw<int8_t>, grid, dim3(kThreads), 0, s, a);
+}
+
+}  // namespace hipie

@@ -1,0 +1,249 @@
+"""Graph-level binding: describes a post-LPT function node by node through the C ABI
+(include/hipie.h section 2), compiles it and runs infer requests.
+
+Every node is also recorded in ``Graph.nodes`` (plain dicts with numpy constants) so that a
+checker can evaluate the very same graph with reference kernels.
+"""
+import ctypes
+
+import numpy as np
+
+from ._lib import check, lib
+from .tensor import F32, I8, I32, U8, U8B, hipie_tensor
+
+OP_ADD, OP_MULTIPLY, OP_SUBTRACT = 6, 7, 8
+_NP = {F32: np.float32, U8: np.uint8, I8: np.int8, I32: np.int32}
+
+
+def _i64(v):
+    return (ctypes.c_int64 * max(len(v), 1))(*[int(x) for x in v])
+
+
+class Graph:
+    def __init__(self):
+        self._h = ctypes.c_void_p()
+        check(lib().hipie_graph_create(ctypes.byref(self._h)))
+        self.nodes = []
+        self.params, self.results = [], []
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().hipie_graph_destroy(self._h)
+            self._h = None
+
+    def _rec(self, id_, op, inputs, dtype, **attrs):
+        assert id_ == len(self.nodes), (id_, len(self.nodes))
+        self.nodes.append(dict(op=op, inputs=list(inputs), dtype=dtype, **attrs))
+        return id_
+
+    def parameter(self, name, shape, dtype=F32):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_parameter(self._h, name.encode(), dtype, _i64(shape), len(shape), ctypes.byref(i)))
+        self.params.append(i.value)
+        return self._rec(i.value, "Parameter", [], dtype, name=name, shape=tuple(shape))
+
+    def constant(self, value, dtype=F32):
+        a = np.ascontiguousarray(value, _NP[dtype])
+        i = ctypes.c_int()
+        check(lib().hipie_graph_constant(self._h, dtype, _i64(a.shape), a.ndim, a.ctypes.data_as(ctypes.c_void_p),
+                                         ctypes.byref(i)))
+        return self._rec(i.value, "Constant", [], dtype, value=a)
+
+    def _const_if_needed(self, v):
+        return v if isinstance(v, int) and not isinstance(v, bool) else self.constant(np.asarray(v, np.float32))
+
+    def fake_quantize(self, x, in_low, in_high, out_low, out_high, levels, out_dtype=F32):
+        b = [self.constant(np.asarray(v, np.float32)) for v in (in_low, in_high, out_low, out_high)]
+        i = ctypes.c_int()
+        check(lib().hipie_graph_fake_quantize(self._h, x, *b, ctypes.c_int64(levels), out_dtype, ctypes.byref(i)))
+        return self._rec(i.value, "FakeQuantize", [x] + b, out_dtype, levels=levels)
+
+    def convolution(self, x, w, strides=(1, 1), dilations=(1, 1), pads_begin=(0, 0), pads_end=(0, 0), grouped=False):
+        i = ctypes.c_int()
+        fn = lib().hipie_graph_group_convolution if grouped else lib().hipie_graph_convolution
+        check(fn(self._h, x, w, _i64(strides), _i64(dilations), _i64(pads_begin), _i64(pads_end), ctypes.byref(i)))
+        return self._rec(i.value, "GroupConvolution" if grouped else "Convolution", [x, w], F32,
+                         strides=tuple(strides), dilations=tuple(dilations), pads_begin=tuple(pads_begin),
+                         pads_end=tuple(pads_end))
+
+    def matmul(self, a, b, transpose_a=False, transpose_b=False):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_matmul(self._h, a, b, int(transpose_a), int(transpose_b), ctypes.byref(i)))
+        return self._rec(i.value, "MatMul", [a, b], F32, ta=transpose_a, tb=transpose_b)
+
+    def _eltwise(self, kind, name, a, b):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_eltwise(self._h, kind, a, b, ctypes.byref(i)))
+        return self._rec(i.value, name, [a, b], F32)
+
+    def add(self, a, b):
+        return self._eltwise(OP_ADD, "Add", a, b)
+
+    def multiply(self, a, b):
+        return self._eltwise(OP_MULTIPLY, "Multiply", a, b)
+
+    def subtract(self, a, b):
+        return self._eltwise(OP_SUBTRACT, "Subtract", a, b)
+
+    def relu(self, x):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_relu(self._h, x, ctypes.byref(i)))
+        return self._rec(i.value, "Relu", [x], self.nodes[x]["dtype"])
+
+    def clamp(self, x, lo, hi):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_clamp(self._h, x, ctypes.c_float(lo), ctypes.c_float(hi), ctypes.byref(i)))
+        return self._rec(i.value, "Clamp", [x], self.nodes[x]["dtype"], lo=float(lo), hi=float(hi))
+
+    def convert(self, x, dtype):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_convert(self._h, x, dtype, ctypes.byref(i)))
+        return self._rec(i.value, "Convert", [x], dtype)
+
+    def max_pool(self, x, kernel, strides, pads_begin=(0, 0), pads_end=(0, 0), ceil_mode=False):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_max_pool(self._h, x, _i64(kernel), _i64(strides), _i64(pads_begin), _i64(pads_end),
+                                         int(ceil_mode), ctypes.byref(i)))
+        return self._rec(i.value, "MaxPool", [x], self.nodes[x]["dtype"], kernel=tuple(kernel),
+                         strides=tuple(strides), pads_begin=tuple(pads_begin), pads_end=tuple(pads_end),
+                         ceil_mode=ceil_mode)
+
+    def avg_pool(self, x, kernel, strides, pads_begin=(0, 0), pads_end=(0, 0), exclude_pad=True, ceil_mode=False,
+                 out_dtype=F32):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_avg_pool(self._h, x, _i64(kernel), _i64(strides), _i64(pads_begin), _i64(pads_end),
+                                         int(exclude_pad), int(ceil_mode), out_dtype, ctypes.byref(i)))
+        return self._rec(i.value, "AvgPool", [x], out_dtype, kernel=tuple(kernel), strides=tuple(strides),
+                         pads_begin=tuple(pads_begin), pads_end=tuple(pads_end), exclude_pad=exclude_pad,
+                         ceil_mode=ceil_mode)
+
+    def reshape(self, x, shape):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_reshape(self._h, x, _i64(shape), len(shape), ctypes.byref(i)))
+        return self._rec(i.value, "Reshape", [x], self.nodes[x]["dtype"], shape=tuple(shape))
+
+    def result(self, x, name):
+        check(lib().hipie_graph_result(self._h, x, name.encode()))
+        self.results.append(len(self.nodes))
+        return self._rec(len(self.nodes), "Result", [x], self.nodes[x]["dtype"], name=name)
+
+    def set_name(self, id_, name):
+        check(lib().hipie_graph_set_name(self._h, id_, name.encode()))
+        self.nodes[id_]["name"] = name
+
+    def compile(self, device=0):
+        return Plan(self, device)
+
+
+class Plan:
+    """ExecutableNetwork analogue: fused steps + arena layout + uploaded constants."""
+
+    def __init__(self, graph, device=0):
+        self._h = ctypes.c_void_p()
+        check(lib().hipie_compile(graph._h, device, ctypes.byref(self._h)))
+        self.device = device
+        L = lib()
+        L.hipie_plan_arena_bytes.restype = ctypes.c_int64
+        self.inputs = [self._io(0, i) for i in range(L.hipie_plan_num_inputs(self._h))]
+        self.outputs = [self._io(1, i) for i in range(L.hipie_plan_num_outputs(self._h))]
+        self.arena_bytes = L.hipie_plan_arena_bytes(self._h)
+        self.steps = []
+        for i in range(L.hipie_plan_num_steps(self._h)):
+            name, typ = ctypes.create_string_buffer(256), ctypes.create_string_buffer(64)
+            macs, byts = ctypes.c_int64(), ctypes.c_int64()
+            check(L.hipie_plan_step_info(self._h, i, name, 256, typ, 64, ctypes.byref(macs), ctypes.byref(byts)))
+            self.steps.append(dict(name=name.value.decode(), type=typ.value.decode(), macs=macs.value,
+                                   bytes=byts.value))
+
+    def _io(self, is_out, idx):
+        name = ctypes.create_string_buffer(256)
+        dt, rank = ctypes.c_int(), ctypes.c_int()
+        dims = (ctypes.c_int64 * 4)()
+        check(lib().hipie_plan_io_desc(self._h, is_out, idx, name, 256, ctypes.byref(dt), dims, ctypes.byref(rank)))
+        return dict(name=name.value.decode(), dtype=dt.value, shape=tuple(dims[:rank.value]))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().hipie_plan_destroy(self._h)
+            self._h = None
+
+    def create_request(self, perf_count=False):
+        return Request(self, perf_count)
+
+
+class Request:
+    """InferRequest analogue: own stream and activation arena."""
+
+    def __init__(self, plan, perf_count=False):
+        self.plan = plan
+        self._h = ctypes.c_void_p()
+        check(lib().hipie_request_create(plan._h, int(perf_count), ctypes.byref(self._h)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().hipie_request_destroy(self._h)
+            self._h = None
+
+    def infer(self, *inputs):
+        """Host path: numpy NCHW in, numpy out (H2D, kernels, D2H)."""
+        ins = [np.ascontiguousarray(a, _NP[d["dtype"]]) for a, d in zip(inputs, self.plan.inputs)]
+        for a, d in zip(ins, self.plan.inputs):
+            assert a.shape == d["shape"], (a.shape, d["shape"])
+        outs = [np.empty(d["shape"], _NP[d["dtype"]]) for d in self.plan.outputs]
+        ip = (ctypes.c_void_p * len(ins))(*[a.ctypes.data for a in ins])
+        op = (ctypes.c_void_p * len(outs))(*[a.ctypes.data for a in outs])
+        check(lib().hipie_request_infer(self._h, ip, op, 0))
+        return outs
+
+    def device_buffers(self):
+        """torch tensors shaped like the plan's inputs and outputs (for resident-in-HBM runs)."""
+        import torch
+        tdt = {F32: torch.float32, U8: torch.uint8}
+        dev = "cuda:%d" % self.plan.device
+        ins = [torch.empty(d["shape"], dtype=tdt[d["dtype"]], device=dev) for d in self.plan.inputs]
+        outs = [torch.empty(d["shape"], dtype=tdt[d["dtype"]], device=dev) for d in self.plan.outputs]
+        return ins, outs
+
+    def _ptrs(self, ins, outs):
+        ip = (ctypes.c_void_p * len(ins))(*[t.data_ptr() for t in ins])
+        op = (ctypes.c_void_p * len(outs))(*[t.data_ptr() for t in outs])
+        return ip, op
+
+    def infer_device(self, ins, outs):
+        ip, op = self._ptrs(ins, outs)
+        check(lib().hipie_request_infer(self._h, ip, op, 1))
+
+    def enqueue(self, ins, outs):
+        ip, op = self._ptrs(ins, outs)
+        check(lib().hipie_request_enqueue(self._h, ip, op))
+
+    @property
+    def stream(self):
+        s = ctypes.c_void_p()
+        check(lib().hipie_request_stream(self._h, ctypes.byref(s)))
+        return s.value
+
+    def perf(self):
+        out = []
+        for i, st in enumerate(self.plan.steps):
+            ms = ctypes.c_float()
+            check(lib().hipie_request_perf(self._h, i, ctypes.byref(ms)))
+            out.append(dict(st, ms=ms.value))
+        return out
+
+    def tensor(self, node_id):
+        """numpy NCHW copy of the arena tensor holding graph node `node_id` (u8 levels / f32)."""
+        import torch
+        t = hipie_tensor()
+        check(lib().hipie_request_tensor(self._h, node_id, ctypes.byref(t)))
+        esz = 4 if t.dtype in (F32, I32) else 1
+        tdt = {F32: torch.float32, I32: torch.int32}.get(t.dtype, torch.int8)
+        # view [n, h, w, c] through the strides
+        span = (t.n - 1) * t.stride_n + (t.h - 1) * t.stride_h + (t.w - 1) * t.stride_w + t.c
+        flat = torch.empty(span, dtype=tdt)
+        check(lib().hipie_memcpy(ctypes.c_void_p(flat.data_ptr()), ctypes.c_void_p(t.data),
+                                 ctypes.c_size_t(span * esz), 0))
+        v = torch.as_strided(flat, (t.n, t.h, t.w, t.c), (t.stride_n, t.stride_h, t.stride_w, 1)).numpy()
+        if t.dtype == U8B:
+            v = (v.astype(np.int16) + 128).astype(np.uint8)
+        return np.ascontiguousarray(np.transpose(v, (0, 3, 1, 2)))

@@ -1,0 +1,83 @@
+"""Bindings to the load-time LPT arithmetic (include/hipie.h section 3) and the few compositions
+a model builder needs to write down the post-LPT constants of a quantized layer.
+
+Every float operation is a single IEEE f32 step in the order the reference's constant folding
+performs it (numpy float32 elementwise ops == reference::multiply / divide on constants).
+"""
+import ctypes
+
+import numpy as np
+
+from ._lib import check, lib
+
+U8, I8 = 40, 50
+_f32p = ctypes.POINTER(ctypes.c_float)
+
+
+def _p(a):
+    return a.ctypes.data_as(_f32p)
+
+
+def precision_details(levels, out_low, out_high):
+    """LayerTransformation::getPrecisionDetails -> (precision or None, has_negative, has_zero_point)."""
+    ol = np.ascontiguousarray(np.asarray(out_low, np.float32).reshape(-1))
+    oh = np.ascontiguousarray(np.asarray(out_high, np.float32).reshape(-1))
+    prec, neg, zp = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    check(lib().hipie_lpt_precision_details(ctypes.c_int64(levels), _p(ol), _p(oh), ctypes.c_int64(ol.size),
+                                            ctypes.byref(prec), ctypes.byref(neg), ctypes.byref(zp)))
+    return (prec.value or None), bool(neg.value), bool(zp.value)
+
+
+def data_precision_range(precision, levels):
+    mn, mx = ctypes.c_float(), ctypes.c_float()
+    check(lib().hipie_lpt_data_precision_range(precision, ctypes.c_int64(levels), ctypes.byref(mn),
+                                               ctypes.byref(mx)))
+    return mn.value, mx.value
+
+
+def decompose_fake_quantize(levels, out_low, out_high):
+    """NetworkHelper::decomposeFakeQuantize for an FQ whose precision getPrecisionDetails resolves.
+
+    Returns dict(precision, new_low, new_high, scale, shift) with arrays shaped like out_low.
+    """
+    ol = np.ascontiguousarray(np.asarray(out_low, np.float32))
+    oh = np.ascontiguousarray(np.asarray(out_high, np.float32))
+    prec, _, zp = precision_details(levels, ol, oh)
+    if prec is None:
+        raise NotImplementedError("FakeQuantize needs a zero point (asymmetric range): next tier")
+    mn, mx = data_precision_range(prec, levels)
+    sc, sh, nl, nh = (np.empty(ol.size, np.float32) for _ in range(4))
+    check(lib().hipie_lpt_decompose_fake_quantize(_p(ol.reshape(-1)), _p(oh.reshape(-1)), ctypes.c_int64(ol.size),
+                                                  ctypes.c_float(mn), ctypes.c_float(mx), _p(sc), _p(sh),
+                                                  _p(nl), _p(nh)))
+    return dict(precision=prec, new_low=np.float32(mn), new_high=np.float32(mx),
+                scale=sc.reshape(ol.shape), shift=sh.reshape(ol.shape), has_zero_point=zp)
+
+
+def fold_fake_quantize(values, in_low, in_high, out_low, out_high, levels, round_values=True):
+    """NetworkHelper::foldFakeQuantize on a constant whose axis 0 is the output-channel axis."""
+    v = np.ascontiguousarray(values, np.float32)
+    oc = v.shape[0]
+    inner = v.size // oc
+    b = [np.ascontiguousarray(np.asarray(x, np.float32).reshape(-1)) for x in (in_low, in_high, out_low, out_high)]
+    out = np.empty_like(v)
+    args = []
+    for x in b:
+        args += [_p(x), ctypes.c_int64(x.size)]
+    check(lib().hipie_lpt_fold_fake_quantize(_p(v), ctypes.c_int64(oc), ctypes.c_int64(inner), *args,
+                                             ctypes.c_int64(levels), int(round_values), _p(out)))
+    return out
+
+
+def quantize_weights(w, levels=255):
+    """Per-output-channel symmetric weight FakeQuantize (range +-max|w_c|) taken through
+    decomposeFakeQuantize + foldFakeQuantize: returns (i8 weights, scale[OC])."""
+    w = np.ascontiguousarray(w, np.float32)
+    oc = w.shape[0]
+    m = np.abs(w.reshape(oc, -1)).max(axis=1).astype(np.float32)
+    m = np.where(m == 0, np.float32(1.0), m)
+    d = decompose_fake_quantize(levels, -m, m)
+    assert d["precision"] == I8 and not d["has_zero_point"]
+    q = fold_fake_quantize(w, -m, m, d["new_low"], d["new_high"], levels, round_values=True)
+    assert np.abs(q).max() <= 127
+    return q.astype(np.int8), d["scale"].astype(np.float32)

@@ -70,6 +70,22 @@ const char* hipie_version(void);
 /* number of visible HIP devices, their names (AVAILABLE_DEVICES / FULL_DEVICE_NAME metrics) */
 int hipie_device_count(void);
 int hipie_device_name(int device, char* buf, size_t buf_len);
+/* synchronous copy between host and device memory (to_device = 1: host -> device) */
+int hipie_memcpy(void* dst, const void* src, size_t bytes, int to_device);
+
+/* ======================================================================================
+ * Activation tensors handed to the engine's kernels: NHWC, channel stride 1, with a readable
+ * border ("halo") of `halo` pixels around every image plane that holds quantisation level 0.
+ * Convolution and pooling padding is read from that border instead of being bounds-checked, so
+ * a consumer with padding p needs halo >= p.  `data` addresses element (n=0,h=0,w=0,c=0).
+ * ==================================================================================== */
+typedef struct hipie_tensor {
+    void* data;
+    int32_t dtype;                        /* hipie_dtype */
+    int32_t n, h, w, c;                   /* logical dims */
+    int64_t stride_n, stride_h, stride_w; /* in elements; stride_w is the (padded) channel count */
+    int32_t halo;
+} hipie_tensor;
 
 /* ======================================================================================
  * 1a. FakeQuantize — ngraph/core/reference/.../fake_quantize.hpp:175-194 (quantize),
@@ -101,26 +117,16 @@ int hipie_fq_run_q8(const hipie_fq* fq, const float* x, void* y, int64_t n, int6
                     hipie_dtype out_dtype, hipie_layout out_layout, int64_t c_stride,
                     void* stream);
 
+/* same as hipie_fq_run_q8 with NHWC output, but into an engine tensor (any strides / halo);
+ * this is how a graph input enters the arena */
+int hipie_fq_run_q8_tensor(const hipie_fq* fq, const float* x, const hipie_tensor* out, void* stream);
+
 /* host evaluation of exactly the arithmetic the device kernel uses (reciprocal multiply with
  * two FMA corrections); the planner checks it against IEEE division at every level boundary of
  * every channel and falls back to the dividing kernel if any differs. */
 float hipie_fq_host_eval(const hipie_fq* fq, int64_t channel, float x);
 /* 1 when the reciprocal path was proven equal to division on all boundaries of all channels */
 int hipie_fq_uses_reciprocal(const hipie_fq* fq);
-
-/* ======================================================================================
- * Activation tensors handed to the engine's kernels: NHWC, channel stride 1, with a readable
- * border ("halo") of `halo` pixels around every image plane that holds quantisation level 0.
- * Convolution and pooling padding is read from that border instead of being bounds-checked, so
- * a consumer with padding p needs halo >= p.  `data` addresses element (n=0,h=0,w=0,c=0).
- * ==================================================================================== */
-typedef struct hipie_tensor {
-    void* data;
-    int32_t dtype;                        /* hipie_dtype */
-    int32_t n, h, w, c;                   /* logical dims */
-    int64_t stride_n, stride_h, stride_w; /* in elements; stride_w is the (padded) channel count */
-    int32_t halo;
-} hipie_tensor;
 
 /* ======================================================================================
  * 1b. Fused f32 epilogue applied to i32 accumulators, in this fixed order (each step one IEEE
@@ -181,6 +187,104 @@ int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* o
 int hipie_conv_set_tile(hipie_conv* conv, int tile);
 int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,
                    const hipie_tensor* out, void* stream);
+
+/* ======================================================================================
+ * 2. Graph level.  The plugin's LoadExeNetworkImpl walks Function::get_ordered_ops()
+ *    (ngraph/core/include/ngraph/function.hpp:126) of the post-LPT function and issues one call
+ *    per node; value ids are returned in creation order.  Shapes are the reference's (NCHW,
+ *    OIHW, [N, C]); element types are the node's output types (TypeRelaxed ops included).
+ *    Supported nodes: Parameter(f32), Constant, FakeQuantize, Convolution, GroupConvolution,
+ *    MatMul, Add, Multiply, Subtract, Relu, Clamp, Convert, MaxPool, AvgPool, Reshape, Result.
+ * ==================================================================================== */
+typedef struct hipie_graph hipie_graph;
+typedef struct hipie_plan hipie_plan;
+typedef struct hipie_request hipie_request;
+
+enum { HIPIE_OP_ADD = 6, HIPIE_OP_MULTIPLY = 7, HIPIE_OP_SUBTRACT = 8 }; /* hipie_graph_eltwise kinds */
+
+int hipie_graph_create(hipie_graph** graph);
+void hipie_graph_destroy(hipie_graph* graph);
+int hipie_graph_parameter(hipie_graph* g, const char* name, int dtype, const int64_t* dims, int rank, int* id);
+int hipie_graph_constant(hipie_graph* g, int dtype, const int64_t* dims, int rank, const void* data, int* id);
+/* op::v0::FakeQuantize (TypeRelaxed when out_dtype is HIPIE_U8 / HIPIE_I8) */
+int hipie_graph_fake_quantize(hipie_graph* g, int x, int in_low, int in_high, int out_low, int out_high,
+                              int64_t levels, int out_dtype, int* id);
+/* op::v1::Convolution / GroupConvolution: 2 spatial dims, attributes are arrays of 2 */
+int hipie_graph_convolution(hipie_graph* g, int x, int weights, const int64_t* strides,
+                            const int64_t* dilations, const int64_t* pads_begin, const int64_t* pads_end,
+                            int* id);
+int hipie_graph_group_convolution(hipie_graph* g, int x, int weights, const int64_t* strides,
+                                  const int64_t* dilations, const int64_t* pads_begin,
+                                  const int64_t* pads_end, int* id);
+int hipie_graph_matmul(hipie_graph* g, int a, int b, int transpose_a, int transpose_b, int* id);
+int hipie_graph_eltwise(hipie_graph* g, int kind, int a, int b, int* id);
+int hipie_graph_relu(hipie_graph* g, int x, int* id);
+int hipie_graph_clamp(hipie_graph* g, int x, float min, float max, int* id);
+int hipie_graph_convert(hipie_graph* g, int x, int dtype, int* id);
+int hipie_graph_max_pool(hipie_graph* g, int x, const int64_t* kernel, const int64_t* strides,
+                         const int64_t* pads_begin, const int64_t* pads_end, int ceil_mode, int* id);
+int hipie_graph_avg_pool(hipie_graph* g, int x, const int64_t* kernel, const int64_t* strides,
+                         const int64_t* pads_begin, const int64_t* pads_end, int exclude_pad, int ceil_mode,
+                         int out_dtype, int* id);
+int hipie_graph_reshape(hipie_graph* g, int x, const int64_t* dims, int rank, int* id);
+int hipie_graph_result(hipie_graph* g, int x, const char* name);
+int hipie_graph_set_name(hipie_graph* g, int id, const char* friendly_name);
+
+/* IInferencePlugin::LoadExeNetworkImpl (ie_iplugin_internal.hpp:270-271): fuse, lay out the static
+ * HBM arena, pack and upload constants.  The graph may be destroyed afterwards. */
+int hipie_compile(const hipie_graph* graph, int device, hipie_plan** plan);
+void hipie_plan_destroy(hipie_plan* plan);
+int hipie_plan_num_inputs(const hipie_plan* plan);
+int hipie_plan_num_outputs(const hipie_plan* plan);
+int hipie_plan_io_desc(const hipie_plan* plan, int is_output, int index, char* name, size_t name_len,
+                       int* dtype, int64_t* dims /* [4] */, int* rank);
+int64_t hipie_plan_arena_bytes(const hipie_plan* plan);
+/* executed (fused) steps, in order: the exec-graph / perf-counter view
+ * (exec_graph_info.hpp:34-76, ie_common.h InferenceEngineProfileInfo) */
+int hipie_plan_num_steps(const hipie_plan* plan);
+int hipie_plan_step_info(const hipie_plan* plan, int index, char* name, size_t name_len, char* type,
+                         size_t type_len, int64_t* macs, int64_t* bytes);
+
+/* IExecutableNetworkInternal::CreateInferRequestImpl: own stream + own activation arena; weights
+ * stay shared in the plan.  perf_count mirrors the PERF_COUNT config key (ie_plugin_config.hpp:277). */
+int hipie_request_create(const hipie_plan* plan, int perf_count, hipie_request** request);
+void hipie_request_destroy(hipie_request* request);
+/* IInferRequestInternal::InferImpl (ie_iinfer_request_internal.hpp:57).  inputs / outputs are dense
+ * NCHW buffers in plan order: host memory (device_memory = 0: H2D, kernels, D2H on the request's
+ * stream) or device memory (device_memory = 1: kernels only). */
+int hipie_request_infer(hipie_request* request, const void* const* inputs, void* const* outputs,
+                        int device_memory);
+/* StartAsync / Wait(RESULT_READY) (ie_infer_async_request_thread_safe_default.hpp:167-214) */
+int hipie_request_start(hipie_request* request, const void* const* inputs, void* const* outputs,
+                        int device_memory);
+int hipie_request_wait(hipie_request* request);
+/* enqueue the kernels only, on the request's stream, without copies or synchronisation */
+int hipie_request_enqueue(hipie_request* request, const void* const* inputs, void* const* outputs);
+int hipie_request_stream(hipie_request* request, void** stream);
+/* milliseconds of step `index` in the last inference (GetPerformanceCounts) */
+int hipie_request_perf(hipie_request* request, int index, float* ms);
+/* the arena tensor holding the value of graph node `node_id` (inspection, parity tests) */
+int hipie_request_tensor(const hipie_request* request, int node_id, hipie_tensor* tensor);
+
+/* ======================================================================================
+ * 3. Load-time arithmetic of the low-precision transformations (host only), for harnesses that
+ *    build post-LPT graphs without OpenVINO.  Reference, all under
+ *    inference-engine/src/low_precision_transformations/:
+ *      src/layer_transformation.cpp:194-273          getPrecisionDetails
+ *      include/low_precision/layer_transformation.hpp:63-107   DataPrecision::getMin/MaxValue
+ *      src/network_helper.cpp:943-1087               decomposeFakeQuantize (scale, shift, clamp)
+ *      src/network_helper.cpp:700-827                foldFakeQuantize (i8 weights)
+ * ==================================================================================== */
+int hipie_lpt_precision_details(int64_t levels, const float* out_low, const float* out_high, int64_t n,
+                                int* precision, int* has_negative, int* has_zero_point);
+int hipie_lpt_data_precision_range(int precision, int64_t levels, float* min, float* max);
+int hipie_lpt_decompose_fake_quantize(const float* out_low, const float* out_high, int64_t n, float min,
+                                      float max, float* scales, float* shifts, float* new_low,
+                                      float* new_high);
+int hipie_lpt_fold_fake_quantize(const float* values, int64_t oc, int64_t inner, const float* in_low,
+                                 int64_t n_in_low, const float* in_high, int64_t n_in_high,
+                                 const float* out_low, int64_t n_out_low, const float* out_high,
+                                 int64_t n_out_high, int64_t levels, int round_values, float* out);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,67 @@
+"""Evaluates a recorded post-LPT graph (dldt_amd.graph.Graph.nodes) with the oracle's reference
+kernels, the way the reference's INTERPRETER backend walks a Function
+(ngraph/test/runtime/interpreter/int_executable.cpp:33-154), except that TypeRelaxed integer ops
+are evaluated in int32 on widened inputs (the interpreter has no mixed-type evaluator)."""
+import numpy as np
+
+F32, U8, I8, I32 = 10, 40, 50, 70
+_NP = {F32: np.float32, U8: np.uint8, I8: np.int8, I32: np.int32}
+
+
+def evaluate(orc, nodes, feeds, keep=None):
+    """feeds: {parameter name: array}.  Returns ({result name: array}, {node id: array} for `keep`)."""
+    val = {}
+    results = {}
+    for i, n in enumerate(nodes):
+        op = n["op"]
+        x = [val[j] for j in n["inputs"]]
+        if op == "Parameter":
+            v = np.ascontiguousarray(feeds[n["name"]], _NP[n["dtype"]])
+        elif op == "Constant":
+            v = n["value"]
+        elif op == "FakeQuantize":
+            v = orc.fake_quantize(x[0], x[1], x[2], x[3], x[4], n["levels"])
+            if n["dtype"] != F32:
+                v = v.astype(_NP[n["dtype"]])            # TypeRelaxed output: Convert of the f32 result
+        elif op in ("Convolution", "GroupConvolution"):
+            v = orc.convolution(x[0].astype(np.int32), x[1].astype(np.int32), n["strides"], n["dilations"],
+                                n["pads_begin"], n["pads_end"], grouped=op == "GroupConvolution")
+            v = v.astype(np.float32)                      # declared f32 holding the integer sum
+        elif op == "MatMul":
+            v = orc.matmul(x[0].astype(np.int32), x[1].astype(np.int32), n["ta"], n["tb"]).astype(np.float32)
+        elif op == "Add":
+            v = orc.add(x[0], x[1])
+        elif op == "Multiply":
+            v = orc.multiply(x[0], x[1])
+        elif op == "Subtract":
+            v = orc.subtract(x[0], x[1])
+        elif op == "Relu":
+            v = orc.relu(x[0])
+        elif op == "Clamp":
+            v = orc.clamp(x[0], n["lo"], n["hi"])
+        elif op == "Convert":
+            v = x[0].astype(_NP[n["dtype"]])
+        elif op == "MaxPool":
+            oshape = orc.pool_out_shape(x[0].shape, n["kernel"], n["strides"], n["pads_begin"], n["pads_end"],
+                                        n["ceil_mode"])
+            v = orc.max_pool(x[0], n["kernel"], n["strides"], n["pads_begin"], n["pads_end"], out_shape=oshape)
+        elif op == "AvgPool":
+            oshape = orc.pool_out_shape(x[0].shape, n["kernel"], n["strides"], n["pads_begin"], n["pads_end"],
+                                        n["ceil_mode"])
+            v = orc.avg_pool(x[0].astype(np.float32), n["kernel"], n["strides"], n["pads_begin"], n["pads_end"],
+                             not n["exclude_pad"], out_shape=oshape)
+        elif op == "Reshape":
+            v = x[0].reshape(n["shape"])
+        elif op == "Result":
+            v = x[0]
+            results[n["name"]] = v
+        else:
+            raise NotImplementedError(op)
+        val[i] = v
+        # free what is no longer needed (full-size ResNet keeps ~1 GB otherwise)
+        if keep is not None:
+            for j in n["inputs"]:
+                if j not in keep and nodes[j]["op"] != "Constant" and all(j not in m["inputs"] for m in nodes[i + 1:]):
+                    val.pop(j, None)
+    kept = {k: val[k] for k in (keep or []) if k in val}
+    return results, kept

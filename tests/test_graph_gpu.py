@@ -1,0 +1,60 @@
+"""Whole graphs through the planner (graph-level C ABI) vs the oracle interpreter."""
+import numpy as np
+import pytest
+
+from interp import evaluate
+
+pytestmark = pytest.mark.gpu
+
+
+def test_conv_block_config1(orc):
+    """BASELINE config 1: [1,64,56,56] -> FQ u8 -> 3x3 conv (i8 per-channel W) -> bias -> ReLU."""
+    from dldt_amd import builders
+    g, feeds, _ = builders.conv_block()
+    want, _ = evaluate(orc, g.nodes, feeds)
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps] == ["FakeQuantize", "Convolution", "Result"]
+    req = plan.create_request()
+    (got,) = req.infer(feeds["data"])
+    np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))
+    # the quantized input levels held in the arena are the reference's
+    q_node = next(i for i, n in enumerate(g.nodes) if n["op"] == "FakeQuantize")
+    _, kept = evaluate(orc, g.nodes, feeds, keep=[q_node])
+    np.testing.assert_array_equal(req.tensor(q_node), kept[q_node])
+
+
+@pytest.mark.parametrize("batch", [1, 3])
+def test_small_resnet_bit_exact(orc, batch):
+    """ResNet-50 v1.5 topology at reduced width/resolution: every quantized activation and the
+    f32 logits must equal the oracle's."""
+    from dldt_amd import builders
+    g, meta = builders.resnet50(batch=batch, res=64, width=16, classes=10, seed=7)
+    rng = np.random.default_rng(99)
+    x = rng.uniform(0, 1, (batch, 3, 64, 64)).astype(np.float32)
+    keep = [a["node"] for a in meta["acts"].values()]
+    want, kept = evaluate(orc, g.nodes, {"data": x}, keep=keep)
+    plan = g.compile()
+    req = plan.create_request()
+    (got,) = req.infer(x)
+    for name, a in meta["acts"].items():
+        w = kept[a["node"]]
+        np.testing.assert_array_equal(req.tensor(a["node"]).reshape(w.shape), w, err_msg=name)
+    np.testing.assert_array_equal(got.view(np.uint32), want["logits"].view(np.uint32))
+    # device-resident path gives the same bytes
+    import torch
+    ins, outs = req.device_buffers()
+    ins[0].copy_(torch.from_numpy(x))
+    req.infer_device(ins, outs)
+    np.testing.assert_array_equal(outs[0].cpu().numpy(), got)
+
+
+def test_planner_reports_unsupported_nodes():
+    from dldt_amd import HipieError
+    from dldt_amd.graph import Graph
+    g = Graph()
+    x = g.parameter("x", (1, 8, 4, 4))
+    y = g.relu(x)
+    g.result(y, "y")
+    with pytest.raises(HipieError) as e:
+        g.compile()
+    assert e.value.status == -2 and "Relu" in str(e.value)
