@@ -11,63 +11,315 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 namespace {
 
-constexpr int kRow = 80;  // LDS row stride: 64 K-bytes + 16 pad
+constexpr int kRow = 80;  // LDS row stride of the tiled kernel: 64 K-bytes + 16 pad
+
+// m -> (m / d, m % d) for m < 2^24 through a float reciprocal (exact after one correction step)
+__device__ __forceinline__ void fast_divmod(int m, int d, float inv_d, int& q, int& r) {
+    q = static_cast<int>(static_cast<float>(m) * inv_d);
+    r = m - q * d;
+    if (r < 0) { --q; r += d; }
+    else if (r >= d) { ++q; r -= d; }
+}
+
+struct PixelCoord { int n, oh, ow; };
+
+__device__ __forceinline__ PixelCoord decode_pixel(const ConvArgs& a, int m) {
+    PixelCoord p;
+    int rem;
+    fast_divmod(m, a.OHOW, a.inv_OHOW, p.n, rem);
+    fast_divmod(rem, a.OW, a.inv_OW, p.oh, p.ow);
+    return p;
+}
+
+__device__ __forceinline__ float4 ld4f(const float* p) { return *reinterpret_cast<const float4*>(p); }
+
+// Accumulators start from the per-channel integer correction, so the epilogue begins with the
+// exact u8 x i8 sum.  acc[ob][pb][r] = channel oc_lane + 16*ob + r of pixel pb.
+__device__ __forceinline__ void init_acc(const ConvArgs& a, int oc_lane, v16i (&acc)[2][2]) {
+#pragma unroll
+    for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int4 c = *reinterpret_cast<const int4*>(a.corr + oc_lane + 16 * ob + 4 * q);
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) {
+                acc[ob][pb][4 * q + 0] = c.x;
+                acc[ob][pb][4 * q + 1] = c.y;
+                acc[ob][pb][4 * q + 2] = c.z;
+                acc[ob][pb][4 * q + 3] = c.w;
+            }
+        }
+}
+
+// level index of one value; the clamp folds both saturating branches of the reference
+template <bool RCP, bool IL0>
+__device__ __forceinline__ float fq_level_fast(float x, float il, float ih, float d, float r, float lm1) {
+    const float xc = __builtin_amdgcn_fmed3f(x, il, ih);
+    const float n = IL0 ? xc : xc - il;
+    float q;
+    if (RCP) {
+        const float q0 = n * r;
+        const float e0 = fmaf(-d, q0, n);
+        const float q1 = fmaf(e0, r, q0);
+        const float e1 = fmaf(-d, q1, n);
+        q = fmaf(e1, r, q1);
+    } else {
+        q = n / d;
+    }
+    return q * lm1;   // rounded to nearest-even by the packing conversion
+}
+
+// bytewise (a + b) mod 256 on four packed bytes
+__device__ __forceinline__ uint32_t add_bytes(uint32_t a, uint32_t b) {
+    return ((a & 0x7f7f7f7fu) + (b & 0x7f7f7f7fu)) ^ ((a ^ b) & 0x80808080u);
+}
+
+// The steady-state epilogue (float(acc) + bias -> FakeQuantize -> byte) for one lane: 32
+// consecutive channels starting at oc_lane, two pixels.  Per-channel constants are fetched one
+// group of four channels ahead of their use; the scheduling barriers keep the compiler from
+// hoisting all of them to the top (which costs an occupancy step).
+template <bool IL0>
+struct PlainParams {
+    float4 bias, ih, r, il, d;
+    __device__ __forceinline__ void load(const ConvArgs& a, int oc) {
+        bias = ld4f(a.bias + oc);
+        ih = ld4f(a.fq_ih + oc);
+        r = ld4f(a.fq_r + oc);
+        if (!IL0) {
+            il = ld4f(a.fq_il + oc);
+            d = ld4f(a.fq_d + oc);
+        }
+    }
+};
+
+template <bool IL0>
+__device__ __forceinline__ void epilogue_fq_plain(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
+                                                  const bool (&valid)[2], const int64_t (&out_off)[2]) {
+    const int out_cs = a.out_sw;
+    uint32_t out_dw[2][8];
+    PlainParams<IL0> cur, nxt;
+    cur.load(a, oc_lane);
+#pragma unroll
+    for (int e4 = 0; e4 < 8; ++e4) {
+        if (e4 + 1 < 8) nxt.load(a, oc_lane + 4 * (e4 + 1));
+        const int ob = e4 >> 2, r0 = (e4 & 3) * 4;
+        const float bias_[4] = {cur.bias.x, cur.bias.y, cur.bias.z, cur.bias.w};
+        const float ih_[4] = {cur.ih.x, cur.ih.y, cur.ih.z, cur.ih.w};
+        const float rr_[4] = {cur.r.x, cur.r.y, cur.r.z, cur.r.w};
+        // input_low == +0: x - il == x and d == ih
+        const float il_[4] = {IL0 ? 0.f : cur.il.x, IL0 ? 0.f : cur.il.y, IL0 ? 0.f : cur.il.z, IL0 ? 0.f : cur.il.w};
+        const float d_[4] = {IL0 ? cur.ih.x : cur.d.x, IL0 ? cur.ih.y : cur.d.y, IL0 ? cur.ih.z : cur.d.z,
+                             IL0 ? cur.ih.w : cur.d.w};
+        uint32_t packed[2] = {0, 0};
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float x = static_cast<float>(acc[ob][pb][r0 + j]) + bias_[j];
+                const float t = fq_level_fast<true, IL0>(x, il_[j], ih_[j], d_[j], rr_[j], a.lm1);
+                packed[pb] = __builtin_amdgcn_cvt_pk_u8_f32(t, j, packed[pb]);
+            }
+        // pin the results here: without this the compiler sinks the arithmetic into the
+        // store predicates and hoists every table load of the epilogue to its top
+        asm volatile("" : "+v"(packed[0]), "+v"(packed[1]) : : "memory");
+        out_dw[0][e4] = packed[0];
+        out_dw[1][e4] = packed[1];
+        cur = nxt;
+    }
+    const uint32_t x80 = (a.flags & CF_OUT_XOR) ? 0x80808080u : 0u;
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            if (valid[pb] && oc_lane + 16 * j < out_cs)
+                *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + out_off[pb] + 16 * j) =
+                    make_uint4(out_dw[pb][4 * j] ^ x80, out_dw[pb][4 * j + 1] ^ x80, out_dw[pb][4 * j + 2] ^ x80,
+                               out_dw[pb][4 * j + 3] ^ x80);
+}
 
 __device__ __forceinline__ float res_byte_to_float(uint32_t dw, int j, float add) {
     const int b = static_cast<int>(static_cast<int8_t>((dw >> (8 * j)) & 0xffu));
     return static_cast<float>(b) + add;
 }
 
-template <int WOC, int WPIX>
-__global__ __launch_bounds__(WOC* WPIX * 64) void conv_mfma_kernel(const ConvArgs a) {
+// every other combination of epilogue steps (uniform branches on the flag word)
+__device__ __forceinline__ void epilogue_general(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
+                                              const bool (&valid)[2], const int64_t (&out_off)[2],
+                                              const int64_t (&res_off)[2]) {
+    const uint32_t fl = a.flags;
+    const int out_cs = a.out_sw;
+    uint32_t res_dw[2][8];
+    if ((fl & CF_RES) && !(fl & CF_RES_F32)) {
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (valid[pb] && oc_lane + 16 * j < a.res_sw)
+                    v = *reinterpret_cast<const uint4*>(static_cast<const int8_t*>(a.res) + res_off[pb] + 16 * j);
+                res_dw[pb][4 * j + 0] = v.x;
+                res_dw[pb][4 * j + 1] = v.y;
+                res_dw[pb][4 * j + 2] = v.z;
+                res_dw[pb][4 * j + 3] = v.w;
+            }
+    }
+    const float res_add = (fl & CF_RES_U8B) ? 128.0f : 0.0f;
+    // stored byte = level + out_off (mod 256): added bytewise after the saturating u8 packing
+    const uint32_t off_b = static_cast<uint32_t>(static_cast<int>(a.out_off)) & 0xffu;
+    const uint32_t off4 = off_b * 0x01010101u;
+
+    uint32_t out_dw[2][8];
+#pragma unroll
+    for (int e4 = 0; e4 < 8; ++e4) {
+        const int oc = oc_lane + 4 * e4;
+        const int ob = e4 >> 2, r0 = (e4 & 3) * 4;
+        float bias_[4], scale_[4], rsub_[4], rmul_[4], post_[4], il_[4], ih_[4], d_[4], rr_[4];
+        auto ld4 = [&](const float* p, float* dst) {
+            const float4 v = ld4f(p + oc);
+            dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+        };
+        if (fl & CF_BIAS) ld4(a.bias, bias_);
+        if (fl & CF_SCALE) ld4(a.scale, scale_);
+        if (fl & CF_RES_SUB) ld4(a.res_sub, rsub_);
+        if (fl & CF_RES_MUL) ld4(a.res_mul, rmul_);
+        if (fl & CF_POST_SCALE) ld4(a.post_scale, post_);
+        if (fl & CF_OUT_FQ) {
+            ld4(a.fq_il, il_);
+            ld4(a.fq_ih, ih_);
+            ld4(a.fq_d, d_);
+            ld4(a.fq_r, rr_);
+        }
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb) {
+            if (fl & CF_OUT_I32) {
+                if (valid[pb] && oc + 4 <= out_cs)
+                    *reinterpret_cast<int4*>(static_cast<int32_t*>(a.out) + out_off[pb] + 4 * e4) =
+                        make_int4(acc[ob][pb][r0], acc[ob][pb][r0 + 1], acc[ob][pb][r0 + 2], acc[ob][pb][r0 + 3]);
+                continue;
+            }
+            float rv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (fl & CF_RES) {
+                if (fl & CF_RES_F32) {
+                    float4 r4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (valid[pb] && oc + 4 <= a.res_sw)
+                        r4 = ld4f(static_cast<const float*>(a.res) + res_off[pb] + 4 * e4);
+                    rv[0] = r4.x; rv[1] = r4.y; rv[2] = r4.z; rv[3] = r4.w;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) rv[j] = res_byte_to_float(res_dw[pb][e4], j, res_add);
+                }
+            }
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float x = static_cast<float>(acc[ob][pb][r0 + j]);
+                if (fl & CF_BIAS) x = x + bias_[j];
+                if (fl & CF_SCALE) x = x * scale_[j];
+                if (fl & CF_RES) {
+                    float r = rv[j];
+                    if (fl & CF_RES_SUB) r = r - rsub_[j];
+                    if (fl & CF_RES_MUL) r = r * rmul_[j];
+                    x = x + r;
+                }
+                if (fl & CF_POST_SCALE) x = x * post_[j];
+                if (fl & CF_RELU) x = x > 0.0f ? x : 0.0f;
+                if (fl & CF_CLAMP) x = x < a.clamp_lo ? a.clamp_lo : (x > a.clamp_hi ? a.clamp_hi : x);
+                v[j] = x;
+            }
+            // pin: keeps the arithmetic of this channel group here instead of inside the store predicates
+            asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
+            if (fl & CF_OUT_FQ) {
+                uint32_t packed = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float t = (fl & CF_FQ_RCP)
+                                        ? fq_level_fast<true, false>(v[j], il_[j], ih_[j], d_[j], rr_[j], a.lm1)
+                                        : fq_level_fast<false, false>(v[j], il_[j], ih_[j], d_[j], rr_[j], a.lm1);
+                    packed = __builtin_amdgcn_cvt_pk_u8_f32(t, j, packed);
+                }
+                out_dw[pb][e4] = add_bytes(packed, off4);
+            } else {
+                if (valid[pb] && oc + 4 <= out_cs)
+                    *reinterpret_cast<float4*>(static_cast<float*>(a.out) + out_off[pb] + 4 * e4) =
+                        make_float4(v[0], v[1], v[2], v[3]);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (fl & CF_OUT_FQ) {
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if (valid[pb] && oc_lane + 16 * j < out_cs)
+                    *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + out_off[pb] + 16 * j) =
+                        make_uint4(out_dw[pb][4 * j], out_dw[pb][4 * j + 1], out_dw[pb][4 * j + 2],
+                                   out_dw[pb][4 * j + 3]);
+    }
+}
+
+// mode 0: general; 1: bias + FQ (reciprocal, il == 0); 2: bias + FQ (reciprocal)
+template <int MODE>
+__device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
+                                             int m0, int m1) {
+    bool valid[2];
+    int64_t out_off[2], res_off[2];
+    const int m[2] = {m0, m1};
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+        valid[pb] = m[pb] < a.M;
+        const PixelCoord p = decode_pixel(a, valid[pb] ? m[pb] : a.M - 1);
+        out_off[pb] = static_cast<int64_t>(p.n) * a.out_sn + p.oh * a.out_sh + p.ow * a.out_sw + oc_lane;
+        res_off[pb] = static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh + p.ow * a.res_sw + oc_lane;
+    }
+    if (MODE == 1) epilogue_fq_plain<true>(a, acc, oc_lane, valid, out_off);
+    else if (MODE == 2) epilogue_fq_plain<false>(a, acc, oc_lane, valid, out_off);
+    else epilogue_general(a, acc, oc_lane, valid, out_off, res_off);
+}
+
+// ------------------------------------------------------------------------------------------------
+// LDS-tiled kernel
+template <int WOC, int WPIX, int MODE>
+__global__ __launch_bounds__(WOC* WPIX * 64, WOC* WPIX >= 4 ? 3 : 2) void conv_tiled_kernel(const ConvArgs a) {
     constexpr int NT = WOC * WPIX * 64;
     constexpr int BOC = WOC * 64, BPIX = WPIX * 64;
     constexpr int A_PIECES = BOC * 4 / NT, B_PIECES = BPIX * 4 / NT;
     __shared__ __attribute__((aligned(16))) int8_t sA[2][BOC * kRow];
     __shared__ __attribute__((aligned(16))) int8_t sB[2][BPIX * kRow];
-    extern __shared__ int32_t s_koff[];  // [Kp / 16]
 
-    // ---- block -> (pixel tile, channel tile): consecutive pixel tiles stay on one XCD ----------
+    // block -> (pixel tile, channel tile): consecutive pixel tiles stay on one XCD
     const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
     const int t_tile = y % a.t_tiles, p_local = y / a.t_tiles;
     const int p_tile = xcd * a.p_per_xcd + p_local;
-    if (p_tile >= a.p_tiles) return;  // whole block leaves before any barrier
+    if (p_local >= a.p_per_xcd || p_tile >= a.p_tiles) return;  // whole block leaves before any barrier
     const int pix0 = p_tile * BPIX, oc0 = t_tile * BOC;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int woc = wave % WOC, wpix = wave / WOC;
     const int l32 = lane & 31, h = lane >> 5;
+    const int chunk = tid & 3;
 
-    for (int i = tid; i < a.nk * 4; i += NT) s_koff[i] = a.koff[i];
-
-    // ---- this thread's global->LDS pieces ------------------------------------------------------
     int32_t b_base[B_PIECES];
     const int8_t* a_ptr[A_PIECES];
-    const int chunk = tid & 3;
 #pragma unroll
     for (int i = 0; i < B_PIECES; ++i) {
-        const int row = (tid + i * NT) >> 2;
-        int m = pix0 + row;
+        int m = pix0 + ((tid + i * NT) >> 2);
         m = m < a.M ? m : a.M - 1;
-        const int n = m / a.OHOW, rem = m - n * a.OHOW;
-        const int oh = rem / a.OW, ow = rem - oh * a.OW;
-        b_base[i] = n * a.in_sn + oh * a.conv_sh * a.in_sh + ow * a.conv_sw * a.in_sw + a.in_origin;
+        const PixelCoord p = decode_pixel(a, m);
+        b_base[i] = p.n * a.in_sn + p.oh * a.conv_sh * a.in_sh + p.ow * a.conv_sw * a.in_sw + a.in_origin;
     }
 #pragma unroll
-    for (int i = 0; i < A_PIECES; ++i) {
-        const int row = (tid + i * NT) >> 2;
-        a_ptr[i] = a.wgt + static_cast<int64_t>(oc0 + row) * a.Kp + chunk * 16;
-    }
-    __syncthreads();  // s_koff visible
+    for (int i = 0; i < A_PIECES; ++i)
+        a_ptr[i] = a.wgt + static_cast<int64_t>(oc0 + ((tid + i * NT) >> 2)) * a.Kp + chunk * 16;
 
     v4i ga[A_PIECES], gb[B_PIECES];
     auto load_global = [&](int k) {
-        const int32_t off = s_koff[k * 4 + chunk];
+        const int4 ko = *reinterpret_cast<const int4*>(a.koff + 4 * k);   // uniform: scalar load
+        const int32_t off = chunk == 0 ? ko.x : (chunk == 1 ? ko.y : (chunk == 2 ? ko.z : ko.w));
 #pragma unroll
         for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(a_ptr[i] + k * 64);
 #pragma unroll
-        for (int i = 0; i < B_PIECES; ++i)
-            gb[i] = *reinterpret_cast<const v4i*>(a.in + (b_base[i] + off));
+        for (int i = 0; i < B_PIECES; ++i) gb[i] = *reinterpret_cast<const v4i*>(a.in + (b_base[i] + off));
     };
     auto store_lds = [&](int buf) {
 #pragma unroll
@@ -78,20 +330,13 @@ __global__ __launch_bounds__(WOC* WPIX * 64) void conv_mfma_kernel(const ConvArg
             *reinterpret_cast<v4i*>(&sB[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = gb[i];
     };
 
-    // weight rows are read permuted so that the lane's results are 32 consecutive channels
-    const int perm0 = 32 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3);
-    const int a_row[2] = {woc * 64 + perm0, woc * 64 + perm0 + 16};
+    const int a_row[2] = {woc * 64 + l32, woc * 64 + 32 + l32};
     const int b_row[2] = {wpix * 64 + l32, wpix * 64 + 32 + l32};
-
-    v16i acc[2][2];
-#pragma unroll
-    for (int ob = 0; ob < 2; ++ob)
-#pragma unroll
-        for (int pb = 0; pb < 2; ++pb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[ob][pb][r] = 0;
+    const int oc_lane = oc0 + woc * 64 + 32 * h;
 
     load_global(0);
+    v16i acc[2][2];
+    init_acc(a, oc_lane, acc);
     store_lds(0);
     __syncthreads();
     for (int k = 0; k < a.nk; ++k) {
@@ -115,140 +360,125 @@ __global__ __launch_bounds__(WOC* WPIX * 64) void conv_mfma_kernel(const ConvArg
         if (k + 1 < a.nk) store_lds(buf ^ 1);
         __syncthreads();
     }
+    const int m0 = pix0 + wpix * 64 + l32;
+    run_epilogue<MODE>(a, acc, oc_lane, m0, m0 + 32);
+}
 
-    // ---- fused epilogue -----------------------------------------------------------------------
-    // acc[ob][pb][r] = channel oc_lane + 16*ob + r of pixel pix0 + wpix*64 + pb*32 + l32
-    const int oc_lane = oc0 + woc * 64 + 32 * h;
-    const uint32_t fl = a.flags;
-    bool valid[2];
-    int64_t out_off[2], res_off[2];
-#pragma unroll
-    for (int pb = 0; pb < 2; ++pb) {
-        const int m = pix0 + wpix * 64 + pb * 32 + l32;
-        valid[pb] = m < a.M;
-        const int mm = valid[pb] ? m : a.M - 1;
-        const int n = mm / a.OHOW, rem = mm - n * a.OHOW;
-        const int oh = rem / a.OW, ow = rem - oh * a.OW;
-        out_off[pb] = static_cast<int64_t>(n) * a.out_sn + oh * a.out_sh + ow * a.out_sw + oc_lane;
-        res_off[pb] = static_cast<int64_t>(n) * a.res_sn + oh * a.res_sh + ow * a.res_sw + oc_lane;
-    }
-    const int out_cs = a.out_sw;  // NHWC: pixel stride == channel stride of the output tensor
+// ------------------------------------------------------------------------------------------------
+// Streaming kernel: grid (x, channel tiles of 64); a workgroup of 4 waves walks pixel tiles of 256
+// (64 per wave) with stride gridDim.x.  Dynamic LDS: 64 rows of (Kp + 16) weight bytes.
+template <int MODE>
+__global__ __launch_bounds__(256, 3) void conv_stream_kernel(const ConvArgs a) {
+    extern __shared__ __attribute__((aligned(16))) int8_t sW[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int oc0 = blockIdx.y * 64;
+    const int wrow = a.Kp + 16;   // 16 * odd: 16 consecutive rows hit distinct bank groups
 
-    uint32_t res_dw[2][8];
-    if ((fl & CF_RES) && !(fl & CF_RES_F32)) {
-#pragma unroll
-        for (int pb = 0; pb < 2; ++pb)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                uint4 v = make_uint4(0, 0, 0, 0);
-                if (valid[pb] && oc_lane + 16 * j < a.res_sw)
-                    v = *reinterpret_cast<const uint4*>(static_cast<const int8_t*>(a.res) + res_off[pb] + 16 * j);
-                res_dw[pb][4 * j + 0] = v.x;
-                res_dw[pb][4 * j + 1] = v.y;
-                res_dw[pb][4 * j + 2] = v.z;
-                res_dw[pb][4 * j + 3] = v.w;
-            }
-    }
-    const float res_add = (fl & CF_RES_U8B) ? 128.0f : 0.0f;
-
-    uint32_t out_dw[2][8];
-#pragma unroll
-    for (int e4 = 0; e4 < 8; ++e4) {
-        const int oc = oc_lane + 4 * e4;
-        const int ob = e4 >> 2, r0 = (e4 & 3) * 4;
-        const int4 corr = *reinterpret_cast<const int4*>(a.corr + oc);
-        const int corr_[4] = {corr.x, corr.y, corr.z, corr.w};
-        float bias_[4], scale_[4], rsub_[4], rmul_[4], post_[4], il_[4], ih_[4], d_[4], rr_[4];
-        auto ld4 = [&](const float* p, float* dst) {
-            const float4 v = *reinterpret_cast<const float4*>(p + oc);
-            dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
-        };
-        if (fl & CF_BIAS) ld4(a.bias, bias_);
-        if (fl & CF_SCALE) ld4(a.scale, scale_);
-        if (fl & CF_RES_SUB) ld4(a.res_sub, rsub_);
-        if (fl & CF_RES_MUL) ld4(a.res_mul, rmul_);
-        if (fl & CF_POST_SCALE) ld4(a.post_scale, post_);
-        if (fl & CF_OUT_FQ) {
-            ld4(a.fq_il, il_);
-            ld4(a.fq_ih, ih_);
-            ld4(a.fq_d, d_);
-            ld4(a.fq_r, rr_);
+    {   // the channel tile's whole weight slab -> LDS, once
+        const int pieces_per_row = a.Kp >> 4, total = 64 * pieces_per_row;
+        const int8_t* src = a.wgt + static_cast<int64_t>(oc0) * a.Kp;
+        for (int i = tid; i < total; i += 256) {
+            const int row = i / pieces_per_row, pc = i - row * pieces_per_row;
+            *reinterpret_cast<v4i*>(&sW[row * wrow + pc * 16]) =
+                *reinterpret_cast<const v4i*>(src + static_cast<int64_t>(row) * a.Kp + pc * 16);
         }
+    }
+    const int oc_lane = oc0 + 32 * h;
+    const int a_row[2] = {l32 * wrow + h * 16, (32 + l32) * wrow + h * 16};
+
+    int tile = blockIdx.x;
+    const int n_tiles = a.p_tiles;
+    int32_t base[2];
+    auto pixel_base = [&](int t, int32_t (&b)[2]) {
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb) {
-            int ai[4];
+            int m = t * 256 + wave * 64 + pb * 32 + l32;
+            m = m < a.M ? m : a.M - 1;
+            const PixelCoord p = decode_pixel(a, m);
+            b[pb] = p.n * a.in_sn + p.oh * a.conv_sh * a.in_sh + p.ow * a.conv_sw * a.in_sw + a.in_origin;
+        }
+    };
+    auto load_b = [&](const int32_t (&b)[2], int k, v4i (&f)[2][2]) {
+        const int4 ko = *reinterpret_cast<const int4*>(a.koff + 4 * k);   // uniform: scalar load
+        const int32_t o0 = h ? ko.y : ko.x, o1 = h ? ko.w : ko.z;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) ai[j] = acc[ob][pb][r0 + j] + corr_[j];
-            if (fl & CF_OUT_I32) {
-                if (valid[pb] && oc + 4 <= out_cs)
-                    *reinterpret_cast<int4*>(static_cast<int32_t*>(a.out) + out_off[pb] + 4 * e4) =
-                        make_int4(ai[0], ai[1], ai[2], ai[3]);
-                continue;
-            }
-            float rv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (fl & CF_RES) {
-                if (fl & CF_RES_F32) {
-                    float4 r4 = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (valid[pb] && oc + 4 <= a.res_sw)
-                        r4 = *reinterpret_cast<const float4*>(static_cast<const float*>(a.res) + res_off[pb] + 4 * e4);
-                    rv[0] = r4.x; rv[1] = r4.y; rv[2] = r4.z; rv[3] = r4.w;
-                } else {
+        for (int pb = 0; pb < 2; ++pb) {
+            f[0][pb] = *reinterpret_cast<const v4i*>(a.in + (b[pb] + o0));
+            f[1][pb] = *reinterpret_cast<const v4i*>(a.in + (b[pb] + o1));
+        }
+    };
+    // Work items are (tile, k) pairs in order; item i+1 is loaded while item i is multiplied.
+    // Two register sets alternate (no copies: a copy would wait for the load it copies).
+    v4i bset[2][2][2];
+    int k = 0;
+    bool have = tile < n_tiles;
+    if (have) {
+        pixel_base(tile, base);
+        load_b(base, 0, bset[0]);
+    }
+    __syncthreads();   // weights resident; no barrier after this point
+    v16i acc[2][2];
+    init_acc(a, oc_lane, acc);
+    auto compute = [&](const v4i (&b)[2][2], int kk) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) rv[j] = res_byte_to_float(res_dw[pb][e4], j, res_add);
-                }
-            }
-            float v[4];
+        for (int ks = 0; ks < 2; ++ks) {
+            v4i af[2];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float x = static_cast<float>(ai[j]);
-                if (fl & CF_BIAS) x = x + bias_[j];
-                if (fl & CF_SCALE) x = x * scale_[j];
-                if (fl & CF_RES) {
-                    float r = rv[j];
-                    if (fl & CF_RES_SUB) r = r - rsub_[j];
-                    if (fl & CF_RES_MUL) r = r * rmul_[j];
-                    x = x + r;
-                }
-                if (fl & CF_POST_SCALE) x = x * post_[j];
-                if (fl & CF_RELU) x = x > 0.0f ? x : 0.0f;
-                if (fl & CF_CLAMP) x = x < a.clamp_lo ? a.clamp_lo : (x > a.clamp_hi ? a.clamp_hi : x);
-                v[j] = x;
-            }
-            if (fl & CF_OUT_FQ) {
-                uint32_t packed = 0;
+            for (int ob = 0; ob < 2; ++ob)
+                af[ob] = *reinterpret_cast<const v4i*>(&sW[a_row[ob] + kk * 64 + ks * 32]);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    FqChannel p;
-                    p.il = il_[j]; p.ih = ih_[j]; p.d = d_[j]; p.r = rr_[j];
-                    const float kf = (fl & CF_FQ_RCP) ? fq_level_clamped<true>(p, a.lm1, v[j])
-                                                     : fq_level_clamped<false>(p, a.lm1, v[j]);
-                    packed |= (static_cast<uint32_t>(static_cast<int>(kf + a.out_off)) & 0xffu) << (8 * j);
-                }
-                out_dw[pb][e4] = packed;
-            } else {
-                if (valid[pb] && oc + 4 <= out_cs)
-                    *reinterpret_cast<float4*>(static_cast<float*>(a.out) + out_off[pb] + 4 * e4) =
-                        make_float4(v[0], v[1], v[2], v[3]);
+            for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+                    acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], b[ks][pb], acc[ob][pb], 0, 0, 0);
+        }
+    };
+    // one pipeline stage: prefetch the next item into `nxt`, multiply `cur`, finish the tile if
+    // this was its last K step.  Returns false when there is no next item.
+    auto stage = [&](const v4i (&cur)[2][2], v4i (&nxt)[2][2]) -> bool {
+        const int cur_tile = tile, cur_k = k;
+        bool more = true;
+        if (k + 1 < a.nk) {
+            ++k;
+            load_b(base, k, nxt);
+        } else {
+            k = 0;
+            tile += gridDim.x;
+            more = tile < n_tiles;
+            if (more) {
+                pixel_base(tile, base);
+                load_b(base, 0, nxt);
             }
         }
-    }
-    if (fl & CF_OUT_FQ) {
-#pragma unroll
-        for (int pb = 0; pb < 2; ++pb)
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-                if (valid[pb] && oc_lane + 16 * j < out_cs)
-                    *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + out_off[pb] + 16 * j) =
-                        make_uint4(out_dw[pb][4 * j], out_dw[pb][4 * j + 1], out_dw[pb][4 * j + 2],
-                                   out_dw[pb][4 * j + 3]);
+        compute(cur, cur_k);
+        if (cur_k + 1 == a.nk) {
+            const int m0 = cur_tile * 256 + wave * 64 + l32;
+            run_epilogue<MODE>(a, acc, oc_lane, m0, m0 + 32);
+            init_acc(a, oc_lane, acc);
+        }
+        return more;
+    };
+    while (have) {
+        if (!stage(bset[0], bset[1])) break;
+        if (!stage(bset[1], bset[0])) break;
     }
 }
 
 template <int WOC, int WPIX>
-void launch(const ConvArgs& a, hipStream_t s) {
-    const int grid = 8 * a.p_per_xcd * a.t_tiles;
-    const size_t dyn = static_cast<size_t>(a.nk) * 4 * sizeof(int32_t);
-    hipLaunchKernelGGL((conv_mfma_kernel<WOC, WPIX>), dim3(grid), dim3(WOC * WPIX * 64), dyn, s, a);
+void launch_tiled(const ConvArgs& a, int mode, hipStream_t s) {
+    const dim3 grid(8 * a.p_per_xcd * a.t_tiles), block(WOC * WPIX * 64);
+    if (mode == 1) hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, 1>), grid, block, 0, s, a);
+    else if (mode == 2) hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, 2>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, 0>), grid, block, 0, s, a);
+}
+
+void launch_stream(const ConvArgs& a, int mode, int grid_x, hipStream_t s) {
+    const dim3 grid(grid_x, a.t_tiles), block(256);
+    const size_t lds = static_cast<size_t>(64) * (a.Kp + 16);
+    if (mode == 1) hipLaunchKernelGGL((conv_stream_kernel<1>), grid, block, lds, s, a);
+    else if (mode == 2) hipLaunchKernelGGL((conv_stream_kernel<2>), grid, block, lds, s, a);
+    else hipLaunchKernelGGL((conv_stream_kernel<0>), grid, block, lds, s, a);
 }
 
 }  // namespace
@@ -331,6 +561,10 @@ void Epilogue::build(int device_, const hipie_epilogue& e, int64_t oc, int64_t o
         up(fq_il, il); up(fq_ih, ih); up(fq_d, d); up(fq_r, r);
         flags |= CF_OUT_FQ;
         if (exact) flags |= CF_FQ_RCP;
+        bool il0 = true;
+        for (int64_t c = 0; c < ocp; ++c) il0 = il0 && il[c] == 0.0f && !std::signbit(il[c]);
+        if (il0) flags |= CF_FQ_IL0;
+        if (out_off == -128.0f) flags |= CF_OUT_XOR;
         break;
     }
     default: fail(HIPIE_PARAMETER_MISMATCH, "epilogue: out dtype %d", e.out_dtype);
@@ -350,11 +584,19 @@ void Epilogue::fill(ConvArgs& a) const {
 
 using namespace hipie;
 
+// row of the packed weight matrix that holds logical channel oc: inside every group of 64 the rows
+// are in MFMA order so that a lane's 16 results per tile are consecutive channels
+static int64_t packed_row(int64_t oc) {
+    const int64_t e = oc & 63;
+    const int64_t hh = e >> 5, ob = (e >> 4) & 1, q = (e >> 2) & 3, t = e & 3;
+    return (oc & ~int64_t(63)) + 32 * ob + 8 * q + 4 * hh + t;
+}
+
 struct hipie_conv {
     int device = 0;
     hipie_conv_desc d{};
     int64_t K = 0, Kp = 0, OCp = 0;
-    int tile = 0;  // 0: 128 ch x 128 px (2x2 waves), 1: 64 ch x 256 px (1x4), 2: 64 ch x 64 px (1 wave)
+    int tile = 0;  // 0: tiled 128 ch x 128 px, 1: tiled 64 x 256, 2: tiled 64 x 64, 3: streaming (64 ch, weights in LDS)
     DeviceBuffer wgt, koff, corr;
     Epilogue epi;
 };
@@ -415,14 +657,15 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
                         const int8_t v = weights[((oc * d.ic + ic) * d.kh + kh) * d.kw + kw];
                         const int64_t k = per_row ? kh * row_kp + kw * cs + ic
                                                   : (static_cast<int64_t>(kh) * d.kw + kw) * cs + ic;
-                        w[oc * c->Kp + k] = v;
+                        w[packed_row(oc) * c->Kp + k] = v;
                         sum += v;
                     }
             corr[oc] = d.in_dtype == HIPIE_U8B ? static_cast<int32_t>(128 * sum) : 0;
         });
         c->epi.build(device, *epilogue, d.oc, c->OCp);
         // tile choice: wide channel tiles when there are enough channels, else all waves on pixels
-        c->tile = d.oc > 64 ? 0 : 1;
+        // weights of one 64-channel tile resident in LDS when they fit twice per CU; else LDS tiling
+        c->tile = 64 * (c->Kp + 16) <= 80 * 1024 ? 3 : (d.oc > 64 ? 0 : 1);
         if (device >= 0) {
             c->wgt.upload(device, w.data(), w.size());
             c->koff.upload(device, koff.data(), koff.size() * sizeof(int32_t));
@@ -436,7 +679,9 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 2, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 3, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_set_tile: K=%lld does not fit the streaming kernel's LDS", (long long)c->Kp);
         c->tile = tile;
     });
 }
@@ -485,8 +730,8 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         const int64_t M = static_cast<int64_t>(in->n) * oh * ow;
         if (M == 0) return;
         const int64_t in_span = static_cast<int64_t>(in->n) * in->stride_n;
-        HIPIE_REQUIRE(in_span < (1ll << 31) && M < (1ll << 31), HIPIE_OUT_OF_BOUNDS,
-                      "hipie_conv_run: tensor too large for 32-bit offsets");
+        HIPIE_REQUIRE(in_span < (1ll << 31) && M < (1ll << 24), HIPIE_OUT_OF_BOUNDS,
+                      "hipie_conv_run: tensor too large (32-bit byte offsets, < 2^24 output pixels)");
         ConvArgs a{};
         a.in = static_cast<const int8_t*>(in->data);
         a.wgt = c->wgt.as<int8_t>();
@@ -511,6 +756,8 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         a.M = static_cast<int32_t>(M);
         a.OW = ow;
         a.OHOW = oh * ow;
+        a.inv_OW = 1.0f / static_cast<float>(ow);
+        a.inv_OHOW = 1.0f / static_cast<float>(oh * ow);
         a.in_sn = static_cast<int32_t>(in->stride_n);
         a.in_sh = static_cast<int32_t>(in->stride_h);
         a.in_sw = static_cast<int32_t>(in->stride_w);
@@ -525,16 +772,31 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         a.Kp = static_cast<int32_t>(c->Kp);
         a.nk = static_cast<int32_t>(c->Kp / 64);
         const int boc = c->tile == 0 ? 128 : 64;
-        const int bpix = c->tile == 0 ? 128 : (c->tile == 1 ? 256 : 64);
+        const int bpix = c->tile == 0 ? 128 : (c->tile == 2 ? 64 : 256);
         a.p_tiles = static_cast<int32_t>(ceil_div(M, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.oc, boc));
         a.p_per_xcd = static_cast<int32_t>(ceil_div(a.p_tiles, 8));
+        // epilogue specialisation: bias + reciprocal FakeQuantize only (the steady-state layer)
+        const uint32_t core = a.flags & ~(CF_FQ_IL0 | CF_OUT_XOR);
+        int mode = 0;
+        if (core == (CF_BIAS | CF_OUT_FQ | CF_FQ_RCP) && ((a.flags & CF_OUT_XOR) || a.out_off == 0.0f))
+            mode = (a.flags & CF_FQ_IL0) ? 1 : 2;
         DeviceGuard g(c->device);
         hipStream_t s = as_stream(stream);
         switch (c->tile) {
-        case 0: launch<2, 2>(a, s); break;
-        case 1: launch<1, 4>(a, s); break;
-        default: launch<1, 1>(a, s); break;
+        case 0: launch_tiled<2, 2>(a, mode, s); break;
+        case 1: launch_tiled<1, 4>(a, mode, s); break;
+        case 2: launch_tiled<1, 1>(a, mode, s); break;
+        default: {
+            // persistent workgroups: as many as fit per CU by LDS (at most 4), spread over the
+            // channel tiles; a multiple of 8 so that sibling channel tiles share an XCD
+            const int64_t lds = 64 * (c->Kp + 16);
+            const int per_cu = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(4, (160 * 1024) / lds)));
+            int64_t gx = std::max<int64_t>(8, (256 * per_cu) / a.t_tiles);
+            gx = std::min<int64_t>(round_up(gx, 8), round_up(a.p_tiles, 8));
+            launch_stream(a, mode, static_cast<int>(gx), s);
+            break;
+        }
         }
         HIPIE_CHECK_HIP(hipGetLastError());
     });

@@ -9,14 +9,19 @@
 // pixels (MFMA B operand, NHWC activations gathered through a per-16-byte offset table),
 // K = (kh, kw, ic).  v_mfma_i32_32x32x32_i8: lane l feeds row/col l%32 with the 16 K-bytes
 // starting at 16*(l/32); it receives rows 8*(r/4) + 4*(l/32) + r%4 of column l%32.
-// Weight rows are read through a permutation so that each lane ends up with 32 CONSECUTIVE
-// output channels of one pixel: results leave as 16-byte stores into NHWC.
+// Weight rows are stored permuted inside every group of 64 channels (packed row 32*ob + i holds
+// channel 32*((i>>2)&1) + 16*ob + 4*(i>>3) + (i&3)), so each lane ends up with 32 CONSECUTIVE
+// output channels of one pixel and results leave as 16-byte stores into NHWC.
 //
-// A workgroup owns (WOC*64) channels x (WPIX*64) pixels; each wave a 64x64 tile (2x2 MFMA
-// tiles, 64 accumulator registers).  K advances 64 bytes per step; global loads for step k+1
-// are issued before the MFMAs of step k and land in the other LDS buffer (one barrier per step).
-// LDS rows are 64 data bytes + 16 pad (stride 80 B = 20 banks): ds_read_b128 of 16 consecutive
-// rows touches distinct banks.
+// Two kernels share the epilogue:
+//   conv_stream_kernel  channel tile 64, the whole [64][K] weight slab resident in LDS for the
+//                       life of a persistent workgroup, activations loaded from global memory
+//                       straight into MFMA operand registers (no barrier in the loop, loads of
+//                       the next K step / next pixel tile in flight during MFMAs and epilogue).
+//                       For the HBM-bound layers (small K * OC).
+//   conv_tiled_kernel   (WOC*64) channels x (WPIX*64) pixels per workgroup, both operands staged
+//                       through double-buffered LDS (rows 64 B + 16 B pad: conflict-free
+//                       ds_read_b128), one barrier per 64-byte K step.  For the MFMA-bound layers.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -37,6 +42,8 @@ enum ConvFlags : uint32_t {
     CF_OUT_I32 = 1u << 10,    // raw accumulators (integer parity tests, MatMul without epilogue)
     CF_FQ_RCP = 1u << 11,     // reciprocal evaluation of the FQ division (proven at load time)
     CF_RES_U8B = 1u << 12,    // residual bytes are level-128 (add 128 after conversion)
+    CF_FQ_IL0 = 1u << 13,     // every input_low is +0: x - il == x
+    CF_OUT_XOR = 1u << 14,    // packed levels ^ 0x80808080 is the stored byte (offset -128)
 };
 
 struct ConvArgs {
@@ -58,6 +65,7 @@ struct ConvArgs {
     const float* fq_r;
     int32_t M;            // N * OH * OW
     int32_t OW, OHOW;
+    float inv_OW, inv_OHOW;          // for the reciprocal pixel decode (M < 2^24)
     int32_t in_sn, in_sh, in_sw;     // input strides in bytes
     int32_t conv_sh, conv_sw;        // convolution strides
     int32_t in_origin;               // -(pad_top * in_sh + pad_left * in_sw)
