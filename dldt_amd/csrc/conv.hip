@@ -74,80 +74,55 @@ __device__ __forceinline__ uint32_t add_bytes(uint32_t a, uint32_t b) {
     return ((a & 0x7f7f7f7fu) + (b & 0x7f7f7f7fu)) ^ ((a ^ b) & 0x80808080u);
 }
 
-// The steady-state epilogue (float(acc) + bias -> FakeQuantize -> byte) for one lane: 32
-// consecutive channels starting at oc_lane, two pixels.  Per-channel constants are fetched one
-// group of four channels ahead of their use; the scheduling barriers keep the compiler from
-// hoisting all of them to the top (which costs an occupancy step).
-template <bool IL0>
-struct PlainParams {
-    float4 bias, ih, r, il, d;
-    __device__ __forceinline__ void load(const ConvArgs& a, int oc) {
-        bias = ld4f(a.bias + oc);
-        ih = ld4f(a.fq_ih + oc);
-        r = ld4f(a.fq_r + oc);
-        if (!IL0) {
-            il = ld4f(a.fq_il + oc);
-            d = ld4f(a.fq_d + oc);
-        }
-    }
-};
+// ---- fused epilogue ---------------------------------------------------------------------------
+// One lane owns 32 consecutive channels (oc_lane ...) of two pixels.  The step list is a flag
+// word; the hot combinations are instantiated with the flags as a template constant so that
+// unused steps vanish, kDyn reads them from the kernel arguments.  Per-channel constants are
+// fetched one group of four channels ahead of their use, and each group's results are pinned
+// with an empty asm: otherwise the compiler sinks the arithmetic into the store predicates and
+// hoists every table load of the epilogue to its top, which costs an occupancy step.
+constexpr uint32_t kDyn = 0xffffffffu;
+constexpr uint32_t E_PLAIN0 = CF_BIAS | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
+constexpr uint32_t E_PLAIN = CF_BIAS | CF_OUT_FQ | CF_FQ_RCP;
+constexpr uint32_t E_RESU8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_U8B | CF_RES_MUL | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
+constexpr uint32_t E_RESF32 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32 | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
+constexpr uint32_t E_F32 = CF_BIAS | CF_SCALE;
+constexpr uint32_t E_F32RELU = CF_BIAS | CF_SCALE | CF_RELU;
 
-template <bool IL0>
-__device__ __forceinline__ void epilogue_fq_plain(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
-                                                  const bool (&valid)[2], const int64_t (&out_off)[2]) {
-    const int out_cs = a.out_sw;
-    uint32_t out_dw[2][8];
-    PlainParams<IL0> cur, nxt;
-    cur.load(a, oc_lane);
-#pragma unroll
-    for (int e4 = 0; e4 < 8; ++e4) {
-        if (e4 + 1 < 8) nxt.load(a, oc_lane + 4 * (e4 + 1));
-        const int ob = e4 >> 2, r0 = (e4 & 3) * 4;
-        const float bias_[4] = {cur.bias.x, cur.bias.y, cur.bias.z, cur.bias.w};
-        const float ih_[4] = {cur.ih.x, cur.ih.y, cur.ih.z, cur.ih.w};
-        const float rr_[4] = {cur.r.x, cur.r.y, cur.r.z, cur.r.w};
-        // input_low == +0: x - il == x and d == ih
-        const float il_[4] = {IL0 ? 0.f : cur.il.x, IL0 ? 0.f : cur.il.y, IL0 ? 0.f : cur.il.z, IL0 ? 0.f : cur.il.w};
-        const float d_[4] = {IL0 ? cur.ih.x : cur.d.x, IL0 ? cur.ih.y : cur.d.y, IL0 ? cur.ih.z : cur.d.z,
-                             IL0 ? cur.ih.w : cur.d.w};
-        uint32_t packed[2] = {0, 0};
-#pragma unroll
-        for (int pb = 0; pb < 2; ++pb)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float x = static_cast<float>(acc[ob][pb][r0 + j]) + bias_[j];
-                const float t = fq_level_fast<true, IL0>(x, il_[j], ih_[j], d_[j], rr_[j], a.lm1);
-                packed[pb] = __builtin_amdgcn_cvt_pk_u8_f32(t, j, packed[pb]);
-            }
-        // pin the results here: without this the compiler sinks the arithmetic into the
-        // store predicates and hoists every table load of the epilogue to its top
-        asm volatile("" : "+v"(packed[0]), "+v"(packed[1]) : : "memory");
-        out_dw[0][e4] = packed[0];
-        out_dw[1][e4] = packed[1];
-        cur = nxt;
-    }
-    const uint32_t x80 = (a.flags & CF_OUT_XOR) ? 0x80808080u : 0u;
-#pragma unroll
-    for (int pb = 0; pb < 2; ++pb)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-            if (valid[pb] && oc_lane + 16 * j < out_cs)
-                *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + out_off[pb] + 16 * j) =
-                    make_uint4(out_dw[pb][4 * j] ^ x80, out_dw[pb][4 * j + 1] ^ x80, out_dw[pb][4 * j + 2] ^ x80,
-                               out_dw[pb][4 * j + 3] ^ x80);
-}
+struct EpiParams {
+    float4 bias, scale, rsub, rmul, post, il, ih, d, r;
+    float4 res[2];   // f32 residual of the two pixels
+};
 
 __device__ __forceinline__ float res_byte_to_float(uint32_t dw, int j, float add) {
     const int b = static_cast<int>(static_cast<int8_t>((dw >> (8 * j)) & 0xffu));
     return static_cast<float>(b) + add;
 }
 
-// every other combination of epilogue steps (uniform branches on the flag word)
-__device__ __forceinline__ void epilogue_general(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
-                                              const bool (&valid)[2], const int64_t (&out_off)[2],
-                                              const int64_t (&res_off)[2]) {
-    const uint32_t fl = a.flags;
+__device__ __forceinline__ void f4_to_array(const float4& v, float (&o)[4]) {
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+
+template <uint32_t F>
+__device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
+                                         const bool (&valid)[2], const int64_t (&out_off)[2],
+                                         const int64_t (&res_off)[2]) {
+    const uint32_t fl = F == kDyn ? a.flags : F;
     const int out_cs = a.out_sw;
+
+    if (fl & CF_OUT_I32) {   // raw accumulators
+#pragma unroll
+        for (int e4 = 0; e4 < 8; ++e4)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+                if (valid[pb] && oc_lane + 4 * e4 + 4 <= out_cs) {
+                    const int ob = e4 >> 2, r0 = (e4 & 3) * 4;
+                    *reinterpret_cast<int4*>(static_cast<int32_t*>(a.out) + out_off[pb] + 4 * e4) =
+                        make_int4(acc[ob][pb][r0], acc[ob][pb][r0 + 1], acc[ob][pb][r0 + 2], acc[ob][pb][r0 + 3]);
+                }
+        return;
+    }
+
     uint32_t res_dw[2][8];
     if ((fl & CF_RES) && !(fl & CF_RES_F32)) {
 #pragma unroll
@@ -164,52 +139,65 @@ __device__ __forceinline__ void epilogue_general(const ConvArgs& a, const v16i (
             }
     }
     const float res_add = (fl & CF_RES_U8B) ? 128.0f : 0.0f;
-    // stored byte = level + out_off (mod 256): added bytewise after the saturating u8 packing
-    const uint32_t off_b = static_cast<uint32_t>(static_cast<int>(a.out_off)) & 0xffu;
-    const uint32_t off4 = off_b * 0x01010101u;
+
+    auto load = [&](int e4, EpiParams& p) {
+        const int oc = oc_lane + 4 * e4;
+        if (fl & CF_BIAS) p.bias = ld4f(a.bias + oc);
+        if (fl & CF_SCALE) p.scale = ld4f(a.scale + oc);
+        if (fl & CF_RES_SUB) p.rsub = ld4f(a.res_sub + oc);
+        if (fl & CF_RES_MUL) p.rmul = ld4f(a.res_mul + oc);
+        if (fl & CF_POST_SCALE) p.post = ld4f(a.post_scale + oc);
+        if (fl & CF_OUT_FQ) {
+            p.ih = ld4f(a.fq_ih + oc);
+            if (fl & CF_FQ_RCP) p.r = ld4f(a.fq_r + oc);
+            if (!(fl & CF_FQ_IL0)) {
+                p.il = ld4f(a.fq_il + oc);
+                p.d = ld4f(a.fq_d + oc);
+            }
+        }
+        if ((fl & CF_RES) && (fl & CF_RES_F32)) {
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) {
+                p.res[pb] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (valid[pb] && oc + 4 <= a.res_sw)
+                    p.res[pb] = ld4f(static_cast<const float*>(a.res) + res_off[pb] + 4 * e4);
+            }
+        }
+    };
 
     uint32_t out_dw[2][8];
+    EpiParams cur, nxt;
+    load(0, cur);
 #pragma unroll
     for (int e4 = 0; e4 < 8; ++e4) {
-        const int oc = oc_lane + 4 * e4;
+        if (e4 + 1 < 8) load(e4 + 1, nxt);
         const int ob = e4 >> 2, r0 = (e4 & 3) * 4;
         float bias_[4], scale_[4], rsub_[4], rmul_[4], post_[4], il_[4], ih_[4], d_[4], rr_[4];
-        auto ld4 = [&](const float* p, float* dst) {
-            const float4 v = ld4f(p + oc);
-            dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
-        };
-        if (fl & CF_BIAS) ld4(a.bias, bias_);
-        if (fl & CF_SCALE) ld4(a.scale, scale_);
-        if (fl & CF_RES_SUB) ld4(a.res_sub, rsub_);
-        if (fl & CF_RES_MUL) ld4(a.res_mul, rmul_);
-        if (fl & CF_POST_SCALE) ld4(a.post_scale, post_);
-        if (fl & CF_OUT_FQ) {
-            ld4(a.fq_il, il_);
-            ld4(a.fq_ih, ih_);
-            ld4(a.fq_d, d_);
-            ld4(a.fq_r, rr_);
+        f4_to_array(cur.bias, bias_);
+        f4_to_array(cur.scale, scale_);
+        f4_to_array(cur.rsub, rsub_);
+        f4_to_array(cur.rmul, rmul_);
+        f4_to_array(cur.post, post_);
+        f4_to_array(cur.ih, ih_);
+        f4_to_array(cur.r, rr_);
+        if (fl & CF_FQ_IL0) {   // input_low == +0: x - il == x and d == ih
+            il_[0] = il_[1] = il_[2] = il_[3] = 0.f;
+            f4_to_array(cur.ih, d_);
+        } else {
+            f4_to_array(cur.il, il_);
+            f4_to_array(cur.d, d_);
         }
+        float v[2][4];
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb) {
-            if (fl & CF_OUT_I32) {
-                if (valid[pb] && oc + 4 <= out_cs)
-                    *reinterpret_cast<int4*>(static_cast<int32_t*>(a.out) + out_off[pb] + 4 * e4) =
-                        make_int4(acc[ob][pb][r0], acc[ob][pb][r0 + 1], acc[ob][pb][r0 + 2], acc[ob][pb][r0 + 3]);
-                continue;
-            }
-            float rv[4] = {0.f, 0.f, 0.f, 0.f};
+            float rv[4];
             if (fl & CF_RES) {
-                if (fl & CF_RES_F32) {
-                    float4 r4 = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (valid[pb] && oc + 4 <= a.res_sw)
-                        r4 = ld4f(static_cast<const float*>(a.res) + res_off[pb] + 4 * e4);
-                    rv[0] = r4.x; rv[1] = r4.y; rv[2] = r4.z; rv[3] = r4.w;
-                } else {
+                if (fl & CF_RES_F32) f4_to_array(cur.res[pb], rv);
+                else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) rv[j] = res_byte_to_float(res_dw[pb][e4], j, res_add);
                 }
             }
-            float v[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 float x = static_cast<float>(acc[ob][pb][r0 + j]);
@@ -224,42 +212,58 @@ __device__ __forceinline__ void epilogue_general(const ConvArgs& a, const v16i (
                 if (fl & CF_POST_SCALE) x = x * post_[j];
                 if (fl & CF_RELU) x = x > 0.0f ? x : 0.0f;
                 if (fl & CF_CLAMP) x = x < a.clamp_lo ? a.clamp_lo : (x > a.clamp_hi ? a.clamp_hi : x);
-                v[j] = x;
-            }
-            // pin: keeps the arithmetic of this channel group here instead of inside the store predicates
-            asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
-            if (fl & CF_OUT_FQ) {
-                uint32_t packed = 0;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float t = (fl & CF_FQ_RCP)
-                                        ? fq_level_fast<true, false>(v[j], il_[j], ih_[j], d_[j], rr_[j], a.lm1)
-                                        : fq_level_fast<false, false>(v[j], il_[j], ih_[j], d_[j], rr_[j], a.lm1);
-                    packed = __builtin_amdgcn_cvt_pk_u8_f32(t, j, packed);
-                }
-                out_dw[pb][e4] = add_bytes(packed, off4);
-            } else {
-                if (valid[pb] && oc + 4 <= out_cs)
-                    *reinterpret_cast<float4*>(static_cast<float*>(a.out) + out_off[pb] + 4 * e4) =
-                        make_float4(v[0], v[1], v[2], v[3]);
+                v[pb][j] = x;
             }
         }
-        __builtin_amdgcn_sched_barrier(0);
+        if (fl & CF_OUT_FQ) {
+            uint32_t packed[2] = {0, 0};
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float t;
+                    if (fl & CF_FQ_RCP) {
+                        t = (fl & CF_FQ_IL0) ? fq_level_fast<true, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], a.lm1)
+                                             : fq_level_fast<true, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], a.lm1);
+                    } else {
+                        t = fq_level_fast<false, false>(v[pb][j], il_[j], ih_[j], d_[j], 0.f, a.lm1);
+                    }
+                    packed[pb] = __builtin_amdgcn_cvt_pk_u8_f32(t, j, packed[pb]);
+                }
+            asm volatile("" : "+v"(packed[0]), "+v"(packed[1]) : : "memory");
+            out_dw[0][e4] = packed[0];
+            out_dw[1][e4] = packed[1];
+        } else {
+            asm volatile("" : "+v"(v[0][0]), "+v"(v[0][1]), "+v"(v[0][2]), "+v"(v[0][3]), "+v"(v[1][0]),
+                         "+v"(v[1][1]), "+v"(v[1][2]), "+v"(v[1][3]) : : "memory");
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+                if (valid[pb] && oc_lane + 4 * e4 + 4 <= out_cs)
+                    *reinterpret_cast<float4*>(static_cast<float*>(a.out) + out_off[pb] + 4 * e4) =
+                        make_float4(v[pb][0], v[pb][1], v[pb][2], v[pb][3]);
+        }
+        cur = nxt;
     }
     if (fl & CF_OUT_FQ) {
+        // stored byte = level + out_off (mod 256); -128 is a sign-bit flip
+        const bool flip = a.flags & CF_OUT_XOR;
+        const uint32_t off4 = (static_cast<uint32_t>(static_cast<int>(a.out_off)) & 0xffu) * 0x01010101u;
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb)
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                if (valid[pb] && oc_lane + 16 * j < out_cs)
+                if (valid[pb] && oc_lane + 16 * j < out_cs) {
+                    uint32_t w[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        w[q] = flip ? out_dw[pb][4 * j + q] ^ 0x80808080u : add_bytes(out_dw[pb][4 * j + q], off4);
                     *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + out_off[pb] + 16 * j) =
-                        make_uint4(out_dw[pb][4 * j], out_dw[pb][4 * j + 1], out_dw[pb][4 * j + 2],
-                                   out_dw[pb][4 * j + 3]);
+                        make_uint4(w[0], w[1], w[2], w[3]);
+                }
     }
 }
 
-// mode 0: general; 1: bias + FQ (reciprocal, il == 0); 2: bias + FQ (reciprocal)
-template <int MODE>
+template <uint32_t F>
 __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                              int m0, int m1) {
     bool valid[2];
@@ -272,14 +276,12 @@ __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc
         out_off[pb] = static_cast<int64_t>(p.n) * a.out_sn + p.oh * a.out_sh + p.ow * a.out_sw + oc_lane;
         res_off[pb] = static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh + p.ow * a.res_sw + oc_lane;
     }
-    if (MODE == 1) epilogue_fq_plain<true>(a, acc, oc_lane, valid, out_off);
-    else if (MODE == 2) epilogue_fq_plain<false>(a, acc, oc_lane, valid, out_off);
-    else epilogue_general(a, acc, oc_lane, valid, out_off, res_off);
+    epilogue<F>(a, acc, oc_lane, valid, out_off, res_off);
 }
 
 // ------------------------------------------------------------------------------------------------
 // LDS-tiled kernel
-template <int WOC, int WPIX, int MODE>
+template <int WOC, int WPIX, uint32_t F>
 __global__ __launch_bounds__(WOC* WPIX * 64, WOC* WPIX >= 4 ? 3 : 2) void conv_tiled_kernel(const ConvArgs a) {
     constexpr int NT = WOC * WPIX * 64;
     constexpr int BOC = WOC * 64, BPIX = WPIX * 64;
@@ -361,13 +363,13 @@ __global__ __launch_bounds__(WOC* WPIX * 64, WOC* WPIX >= 4 ? 3 : 2) void conv_t
         __syncthreads();
     }
     const int m0 = pix0 + wpix * 64 + l32;
-    run_epilogue<MODE>(a, acc, oc_lane, m0, m0 + 32);
+    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32);
 }
 
 // ------------------------------------------------------------------------------------------------
 // Streaming kernel: grid (x, channel tiles of 64); a workgroup of 4 waves walks pixel tiles of 256
 // (64 per wave) with stride gridDim.x.  Dynamic LDS: 64 rows of (Kp + 16) weight bytes.
-template <int MODE>
+template <uint32_t F>
 __global__ __launch_bounds__(256, 3) void conv_stream_kernel(const ConvArgs a) {
     extern __shared__ __attribute__((aligned(16))) int8_t sW[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -454,7 +456,7 @@ __global__ __launch_bounds__(256, 3) void conv_stream_kernel(const ConvArgs a) {
         compute(cur, cur_k);
         if (cur_k + 1 == a.nk) {
             const int m0 = cur_tile * 256 + wave * 64 + l32;
-            run_epilogue<MODE>(a, acc, oc_lane, m0, m0 + 32);
+            run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32);
             init_acc(a, oc_lane, acc);
         }
         return more;
@@ -465,20 +467,40 @@ __global__ __launch_bounds__(256, 3) void conv_stream_kernel(const ConvArgs a) {
     }
 }
 
+// flag word -> kernel instance
+#define HIPIE_FOR_EACH_EPILOGUE(X, ...)                                                      \
+    switch (core) {                                                                          \
+    case E_PLAIN0: X(E_PLAIN0, __VA_ARGS__); break;                                          \
+    case E_PLAIN: X(E_PLAIN, __VA_ARGS__); break;                                            \
+    case E_RESU8: X(E_RESU8, __VA_ARGS__); break;                                            \
+    case E_RESF32: X(E_RESF32, __VA_ARGS__); break;                                          \
+    case E_F32: X(E_F32, __VA_ARGS__); break;                                                \
+    case E_F32RELU: X(E_F32RELU, __VA_ARGS__); break;                                        \
+    default: X(kDyn, __VA_ARGS__); break;                                                    \
+    }
+
 template <int WOC, int WPIX>
-void launch_tiled(const ConvArgs& a, int mode, hipStream_t s) {
+void launch_tiled(const ConvArgs& a, hipStream_t s) {
     const dim3 grid(8 * a.p_per_xcd * a.t_tiles), block(WOC * WPIX * 64);
-    if (mode == 1) hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, 1>), grid, block, 0, s, a);
-    else if (mode == 2) hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, 2>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, 0>), grid, block, 0, s, a);
+    const uint32_t core = a.flags & ~CF_OUT_XOR;
+#define HIPIE_LAUNCH_TILED(FLAGS, ...) \
+    hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, FLAGS>), grid, block, 0, s, a)
+    HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_TILED, 0)
+#undef HIPIE_LAUNCH_TILED
 }
 
-void launch_stream(const ConvArgs& a, int mode, int grid_x, hipStream_t s) {
+void launch_tiled_small(const ConvArgs& a, hipStream_t s) {   // 64 x 64 tile, one wave: generic epilogue only
+    hipLaunchKernelGGL((conv_tiled_kernel<1, 1, kDyn>), dim3(8 * a.p_per_xcd * a.t_tiles), dim3(64), 0, s, a);
+}
+
+void launch_stream(const ConvArgs& a, int grid_x, hipStream_t s) {
     const dim3 grid(grid_x, a.t_tiles), block(256);
     const size_t lds = static_cast<size_t>(64) * (a.Kp + 16);
-    if (mode == 1) hipLaunchKernelGGL((conv_stream_kernel<1>), grid, block, lds, s, a);
-    else if (mode == 2) hipLaunchKernelGGL((conv_stream_kernel<2>), grid, block, lds, s, a);
-    else hipLaunchKernelGGL((conv_stream_kernel<0>), grid, block, lds, s, a);
+    const uint32_t core = a.flags & ~CF_OUT_XOR;
+#define HIPIE_LAUNCH_STREAM(FLAGS, ...) \
+    hipLaunchKernelGGL((conv_stream_kernel<FLAGS>), grid, block, lds, s, a)
+    HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_STREAM, 0)
+#undef HIPIE_LAUNCH_STREAM
 }
 
 }  // namespace
@@ -664,8 +686,9 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
         });
         c->epi.build(device, *epilogue, d.oc, c->OCp);
         // tile choice: wide channel tiles when there are enough channels, else all waves on pixels
-        // weights of one 64-channel tile resident in LDS when they fit twice per CU; else LDS tiling
-        c->tile = 64 * (c->Kp + 16) <= 80 * 1024 ? 3 : (d.oc > 64 ? 0 : 1);
+        // default: wide channel tiles when there are enough channels, else all waves on pixels
+        // (the planner may override this after timing the candidates)
+        c->tile = d.oc > 64 ? 0 : 1;
         if (device >= 0) {
             c->wgt.upload(device, w.data(), w.size());
             c->koff.upload(device, koff.data(), koff.size() * sizeof(int32_t));
@@ -776,17 +799,12 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         a.p_tiles = static_cast<int32_t>(ceil_div(M, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.oc, boc));
         a.p_per_xcd = static_cast<int32_t>(ceil_div(a.p_tiles, 8));
-        // epilogue specialisation: bias + reciprocal FakeQuantize only (the steady-state layer)
-        const uint32_t core = a.flags & ~(CF_FQ_IL0 | CF_OUT_XOR);
-        int mode = 0;
-        if (core == (CF_BIAS | CF_OUT_FQ | CF_FQ_RCP) && ((a.flags & CF_OUT_XOR) || a.out_off == 0.0f))
-            mode = (a.flags & CF_FQ_IL0) ? 1 : 2;
         DeviceGuard g(c->device);
         hipStream_t s = as_stream(stream);
         switch (c->tile) {
-        case 0: launch_tiled<2, 2>(a, mode, s); break;
-        case 1: launch_tiled<1, 4>(a, mode, s); break;
-        case 2: launch_tiled<1, 1>(a, mode, s); break;
+        case 0: launch_tiled<2, 2>(a, s); break;
+        case 1: launch_tiled<1, 4>(a, s); break;
+        case 2: launch_tiled_small(a, s); break;
         default: {
             // persistent workgroups: as many as fit per CU by LDS (at most 4), spread over the
             // channel tiles; a multiple of 8 so that sibling channel tiles share an XCD
@@ -794,7 +812,7 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
             const int per_cu = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(4, (160 * 1024) / lds)));
             int64_t gx = std::max<int64_t>(8, (256 * per_cu) / a.t_tiles);
             gx = std::min<int64_t>(round_up(gx, 8), round_up(a.p_tiles, 8));
-            launch_stream(a, mode, static_cast<int>(gx), s);
+            launch_stream(a, static_cast<int>(gx), s);
             break;
         }
         }
