@@ -20,4 +20,6 @@ struct Epilogue {
     void fill(ConvArgs& a) const;
 };
 
+void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipStream_t s);
+
 }  // namespace hipie

@@ -1,0 +1,281 @@
+// Device-side pieces shared by the MFMA convolution kernels and the depthwise kernel: pixel
+// decode, accumulator initialisation and the fused f32 epilogue.  A lane always owns 32
+// consecutive output channels (oc_lane ...) of two pixels, held as acc[ob][pb][r] = channel
+// oc_lane + 16*ob + r of pixel pb.
+#pragma once
+#include "conv_kernel.h"
+#include "fq_math.h"
+
+namespace hipie {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// m -> (m / d, m % d) for m < 2^24 through a float reciprocal (exact after one correction step)
+__device__ __forceinline__ void fast_divmod(int m, int d, float inv_d, int& q, int& r) {
+    q = static_cast<int>(static_cast<float>(m) * inv_d);
+    r = m - q * d;
+    if (r < 0) { --q; r += d; }
+    else if (r >= d) { ++q; r -= d; }
+}
+
+struct PixelCoord { int n, oh, ow; };
+
+__device__ __forceinline__ PixelCoord decode_pixel(const ConvArgs& a, int m) {
+    PixelCoord p;
+    int rem;
+    fast_divmod(m, a.OHOW, a.inv_OHOW, p.n, rem);
+    fast_divmod(rem, a.OW, a.inv_OW, p.oh, p.ow);
+    return p;
+}
+
+__device__ __forceinline__ float4 ld4f(const float* p) { return *reinterpret_cast<const float4*>(p); }
+
+// Accumulators start from the per-channel integer correction, so the epilogue begins with the
+// exact u8 x i8 sum.  acc[ob][pb][r] = channel oc_lane + 16*ob + r of pixel pb.
+__device__ __forceinline__ void init_acc(const ConvArgs& a, int oc_lane, v16i (&acc)[2][2]) {
+#pragma unroll
+    for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int4 c = *reinterpret_cast<const int4*>(a.corr + oc_lane + 16 * ob + 4 * q);
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) {
+                acc[ob][pb][4 * q + 0] = c.x;
+                acc[ob][pb][4 * q + 1] = c.y;
+                acc[ob][pb][4 * q + 2] = c.z;
+                acc[ob][pb][4 * q + 3] = c.w;
+            }
+        }
+}
+
+// level index of one value; the clamp folds both saturating branches of the reference
+template <bool RCP, bool IL0>
+__device__ __forceinline__ float fq_level_fast(float x, float il, float ih, float d, float r, float lm1) {
+    const float xc = __builtin_amdgcn_fmed3f(x, il, ih);
+    const float n = IL0 ? xc : xc - il;
+    float q;
+    if (RCP) {
+        const float q0 = n * r;
+        const float e0 = fmaf(-d, q0, n);
+        const float q1 = fmaf(e0, r, q0);
+        const float e1 = fmaf(-d, q1, n);
+        q = fmaf(e1, r, q1);
+    } else {
+        q = n / d;
+    }
+    return q * lm1;   // rounded to nearest-even by the packing conversion
+}
+
+// bytewise (a + b) mod 256 on four packed bytes
+__device__ __forceinline__ uint32_t add_bytes(uint32_t a, uint32_t b) {
+    return ((a & 0x7f7f7f7fu) + (b & 0x7f7f7f7fu)) ^ ((a ^ b) & 0x80808080u);
+}
+
+// ---- fused epilogue ---------------------------------------------------------------------------
+// One lane owns 32 consecutive channels (oc_lane ...) of two pixels.  The step list is a flag
+// word; the hot combinations are instantiated with the flags as a template constant so that
+// unused steps vanish, kDyn reads them from the kernel arguments.  Per-channel constants are
+// fetched one group of four channels ahead of their use, and each group's results are pinned
+// with an empty asm: otherwise the compiler sinks the arithmetic into the store predicates and
+// hoists every table load of the epilogue to its top, which costs an occupancy step.
+constexpr uint32_t kDyn = 0xffffffffu;
+constexpr uint32_t E_PLAIN0 = CF_BIAS | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
+constexpr uint32_t E_PLAIN = CF_BIAS | CF_OUT_FQ | CF_FQ_RCP;
+constexpr uint32_t E_RESU8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_U8B | CF_RES_MUL | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
+constexpr uint32_t E_RESF32 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32 | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
+constexpr uint32_t E_F32 = CF_BIAS | CF_SCALE;
+constexpr uint32_t E_F32RELU = CF_BIAS | CF_SCALE | CF_RELU;
+constexpr uint32_t E_CLAMPFQ = CF_BIAS | CF_SCALE | CF_CLAMP | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
+
+struct EpiParams {
+    float4 bias, scale, rsub, rmul, post, il, ih, d, r;
+    float4 res[2];   // f32 residual of the two pixels
+};
+
+__device__ __forceinline__ float res_byte_to_float(uint32_t dw, int j, float add) {
+    const int b = static_cast<int>(static_cast<int8_t>((dw >> (8 * j)) & 0xffu));
+    return static_cast<float>(b) + add;
+}
+
+__device__ __forceinline__ void f4_to_array(const float4& v, float (&o)[4]) {
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+
+template <uint32_t F>
+__device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
+                                         const bool (&valid)[2], const int64_t (&out_off)[2],
+                                         const int64_t (&res_off)[2]) {
+    const uint32_t fl = F == kDyn ? a.flags : F;
+    const int out_cs = a.out_sw;
+
+    if (fl & CF_OUT_I32) {   // raw accumulators
+#pragma unroll
+        for (int e4 = 0; e4 < 8; ++e4)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+                if (valid[pb] && oc_lane + 4 * e4 + 4 <= out_cs) {
+                    const int ob = e4 >> 2, r0 = (e4 & 3) * 4;
+                    *reinterpret_cast<int4*>(static_cast<int32_t*>(a.out) + out_off[pb] + 4 * e4) =
+                        make_int4(acc[ob][pb][r0], acc[ob][pb][r0 + 1], acc[ob][pb][r0 + 2], acc[ob][pb][r0 + 3]);
+                }
+        return;
+    }
+
+    uint32_t res_dw[2][8];
+    if ((fl & CF_RES) && !(fl & CF_RES_F32)) {
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (valid[pb] && oc_lane + 16 * j < a.res_sw)
+                    v = *reinterpret_cast<const uint4*>(static_cast<const int8_t*>(a.res) + res_off[pb] + 16 * j);
+                res_dw[pb][4 * j + 0] = v.x;
+                res_dw[pb][4 * j + 1] = v.y;
+                res_dw[pb][4 * j + 2] = v.z;
+                res_dw[pb][4 * j + 3] = v.w;
+            }
+    }
+    const float res_add = (fl & CF_RES_U8B) ? 128.0f : 0.0f;
+
+    auto load = [&](int e4, EpiParams& p) {
+        const int oc = oc_lane + 4 * e4;
+        if (fl & CF_BIAS) p.bias = ld4f(a.bias + oc);
+        if (fl & CF_SCALE) p.scale = ld4f(a.scale + oc);
+        if (fl & CF_RES_SUB) p.rsub = ld4f(a.res_sub + oc);
+        if (fl & CF_RES_MUL) p.rmul = ld4f(a.res_mul + oc);
+        if (fl & CF_POST_SCALE) p.post = ld4f(a.post_scale + oc);
+        if (fl & CF_OUT_FQ) {
+            p.ih = ld4f(a.fq_ih + oc);
+            if (fl & CF_FQ_RCP) p.r = ld4f(a.fq_r + oc);
+            if (!(fl & CF_FQ_IL0)) {
+                p.il = ld4f(a.fq_il + oc);
+                p.d = ld4f(a.fq_d + oc);
+            }
+        }
+        if ((fl & CF_RES) && (fl & CF_RES_F32)) {
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) {
+                p.res[pb] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (valid[pb] && oc + 4 <= a.res_sw)
+                    p.res[pb] = ld4f(static_cast<const float*>(a.res) + res_off[pb] + 4 * e4);
+            }
+        }
+    };
+
+    uint32_t out_dw[2][8];
+    EpiParams cur, nxt;
+    load(0, cur);
+#pragma unroll
+    for (int e4 = 0; e4 < 8; ++e4) {
+        if (e4 + 1 < 8) load(e4 + 1, nxt);
+        const int ob = e4 >> 2, r0 = (e4 & 3) * 4;
+        float bias_[4], scale_[4], rsub_[4], rmul_[4], post_[4], il_[4], ih_[4], d_[4], rr_[4];
+        f4_to_array(cur.bias, bias_);
+        f4_to_array(cur.scale, scale_);
+        f4_to_array(cur.rsub, rsub_);
+        f4_to_array(cur.rmul, rmul_);
+        f4_to_array(cur.post, post_);
+        f4_to_array(cur.ih, ih_);
+        f4_to_array(cur.r, rr_);
+        if (fl & CF_FQ_IL0) {   // input_low == +0: x - il == x and d == ih
+            il_[0] = il_[1] = il_[2] = il_[3] = 0.f;
+            f4_to_array(cur.ih, d_);
+        } else {
+            f4_to_array(cur.il, il_);
+            f4_to_array(cur.d, d_);
+        }
+        float v[2][4];
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb) {
+            float rv[4];
+            if (fl & CF_RES) {
+                if (fl & CF_RES_F32) f4_to_array(cur.res[pb], rv);
+                else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) rv[j] = res_byte_to_float(res_dw[pb][e4], j, res_add);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float x = static_cast<float>(acc[ob][pb][r0 + j]);
+                if (fl & CF_BIAS) x = x + bias_[j];
+                if (fl & CF_SCALE) x = x * scale_[j];
+                if (fl & CF_RES) {
+                    float r = rv[j];
+                    if (fl & CF_RES_SUB) r = r - rsub_[j];
+                    if (fl & CF_RES_MUL) r = r * rmul_[j];
+                    x = x + r;
+                }
+                if (fl & CF_POST_SCALE) x = x * post_[j];
+                if (fl & CF_RELU) x = x > 0.0f ? x : 0.0f;
+                if (fl & CF_CLAMP) x = x < a.clamp_lo ? a.clamp_lo : (x > a.clamp_hi ? a.clamp_hi : x);
+                v[pb][j] = x;
+            }
+        }
+        if (fl & CF_OUT_FQ) {
+            uint32_t packed[2] = {0, 0};
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float t;
+                    if (fl & CF_FQ_RCP) {
+                        t = (fl & CF_FQ_IL0) ? fq_level_fast<true, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], a.lm1)
+                                             : fq_level_fast<true, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], a.lm1);
+                    } else {
+                        t = fq_level_fast<false, false>(v[pb][j], il_[j], ih_[j], d_[j], 0.f, a.lm1);
+                    }
+                    packed[pb] = __builtin_amdgcn_cvt_pk_u8_f32(t, j, packed[pb]);
+                }
+            asm volatile("" : "+v"(packed[0]), "+v"(packed[1]) : : "memory");
+            out_dw[0][e4] = packed[0];
+            out_dw[1][e4] = packed[1];
+        } else {
+            asm volatile("" : "+v"(v[0][0]), "+v"(v[0][1]), "+v"(v[0][2]), "+v"(v[0][3]), "+v"(v[1][0]),
+                         "+v"(v[1][1]), "+v"(v[1][2]), "+v"(v[1][3]) : : "memory");
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+                if (valid[pb] && oc_lane + 4 * e4 + 4 <= out_cs)
+                    *reinterpret_cast<float4*>(static_cast<float*>(a.out) + out_off[pb] + 4 * e4) =
+                        make_float4(v[pb][0], v[pb][1], v[pb][2], v[pb][3]);
+        }
+        cur = nxt;
+    }
+    if (fl & CF_OUT_FQ) {
+        // stored byte = level + out_off (mod 256); -128 is a sign-bit flip
+        const bool flip = a.flags & CF_OUT_XOR;
+        const uint32_t off4 = (static_cast<uint32_t>(static_cast<int>(a.out_off)) & 0xffu) * 0x01010101u;
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if (valid[pb] && oc_lane + 16 * j < out_cs) {
+                    uint32_t w[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        w[q] = flip ? out_dw[pb][4 * j + q] ^ 0x80808080u : add_bytes(out_dw[pb][4 * j + q], off4);
+                    *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + out_off[pb] + 16 * j) =
+                        make_uint4(w[0], w[1], w[2], w[3]);
+                }
+    }
+}
+
+template <uint32_t F>
+__device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
+                                             int m0, int m1) {
+    bool valid[2];
+    int64_t out_off[2], res_off[2];
+    const int m[2] = {m0, m1};
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+        valid[pb] = m[pb] < a.M;
+        const PixelCoord p = decode_pixel(a, valid[pb] ? m[pb] : a.M - 1);
+        out_off[pb] = static_cast<int64_t>(p.n) * a.out_sn + p.oh * a.out_sh + p.ow * a.out_sw + oc_lane;
+        res_off[pb] = static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh + p.ow * a.res_sw + oc_lane;
+    }
+    epilogue<F>(a, acc, oc_lane, valid, out_off, res_off);
+}
+
+}  // namespace hipie

@@ -144,6 +144,44 @@ __global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc_q8(const float* __re
     }
 }
 
+// Image-like inputs (C <= 4) -> pixels of 4 bytes: a thread quantises 4 consecutive pixels of one
+// row from C coalesced float4 reads and writes 16 contiguous bytes.  W % 4 == 0.
+template <bool RCP>
+__global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc4_q8(const float* __restrict__ x,
+                                                                 uint8_t* __restrict__ y,
+                                                                 const FqChannel* __restrict__ tab,
+                                                                 float lm1, float off, uint32_t N, uint32_t C,
+                                                                 uint32_t H, uint32_t W, int64_t out_sn,
+                                                                 int64_t out_sh) {
+    const uint32_t w4 = W / 4;
+    const int64_t total = static_cast<int64_t>(N) * H * w4;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < total; i += stride) {
+        const uint32_t wq = static_cast<uint32_t>(i % w4);
+        const uint32_t row = static_cast<uint32_t>(i / w4);
+        const uint32_t h = row % H, n = row / H;
+        float k[4][4];   // [pixel][channel]
+#pragma unroll
+        for (uint32_t c = 0; c < 4; ++c) {
+            if (c < C) {
+                const FqChannel p = tab[c];
+                const float4 v = *reinterpret_cast<const float4*>(
+                    x + ((static_cast<int64_t>(n) * C + c) * H + h) * W + wq * 4);
+                k[0][c] = fq_level_clamped<RCP>(p, lm1, v.x);
+                k[1][c] = fq_level_clamped<RCP>(p, lm1, v.y);
+                k[2][c] = fq_level_clamped<RCP>(p, lm1, v.z);
+                k[3][c] = fq_level_clamped<RCP>(p, lm1, v.w);
+            } else {
+                k[0][c] = k[1][c] = k[2][c] = k[3][c] = 0.0f;
+            }
+        }
+        uint32_t* dst = reinterpret_cast<uint32_t*>(y + static_cast<int64_t>(n) * out_sn + h * out_sh +
+                                                    static_cast<int64_t>(wq) * 16);
+#pragma unroll
+        for (uint32_t p = 0; p < 4; ++p) dst[p] = pack_levels(k[p][0], k[p][1], k[p][2], k[p][3], off);
+    }
+}
+
 int grid_for(int64_t work_items) {
     // enough blocks to fill 256 CUs several times over, capped so the grid-stride loop amortises
     const int64_t blocks = ceil_div(work_items, kThreads);
@@ -422,8 +460,19 @@ int hipie_fq_run_q8_tensor(const hipie_fq* fq, const float* x, const hipie_tenso
         HIPIE_REQUIRE(cs >= fq->C && cs % 4 == 0 && reinterpret_cast<uintptr_t>(out->data) % 4 == 0 &&
                           (cs % 16 != 0 || reinterpret_cast<uintptr_t>(out->data) % 16 == 0),
                       HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: channel stride / alignment");
-        const uint32_t tiles = static_cast<uint32_t>(ceil_div(hw, 64));
         DeviceGuard g(fq->device);
+        if (fq->C <= 4 && cs == 4 && out->w % 4 == 0) {
+            auto k4 = fq->rcp ? fq_nchw_to_nhwc4_q8<true> : fq_nchw_to_nhwc4_q8<false>;
+            const int64_t work = static_cast<int64_t>(out->n) * out->h * (out->w / 4);
+            hipLaunchKernelGGL(k4, dim3(grid_for(work)), dim3(kThreads), 0, as_stream(stream), x,
+                               static_cast<uint8_t*>(out->data), fq->table.as<FqChannel>(), fq->lm1, off,
+                               static_cast<uint32_t>(out->n), static_cast<uint32_t>(fq->C),
+                               static_cast<uint32_t>(out->h), static_cast<uint32_t>(out->w), out->stride_n,
+                               out->stride_h);
+            HIPIE_CHECK_HIP(hipGetLastError());
+            return;
+        }
+        const uint32_t tiles = static_cast<uint32_t>(ceil_div(hw, 64));
         auto k = fq->rcp ? fq_nchw_to_nhwc_q8<true> : fq_nchw_to_nhwc_q8<false>;
         hipLaunchKernelGGL(k, dim3(static_cast<uint32_t>(out->n * tiles), static_cast<uint32_t>(ceil_div(cs, 64))),
                            dim3(kThreads), 0, as_stream(stream), x, static_cast<uint8_t*>(out->data),

@@ -316,8 +316,7 @@ struct Planner {
         case OP_PARAMETER: values[id].kind = VK_PARAM; break;
         case OP_CONSTANT: values[id].kind = VK_CONST; break;
         case OP_FAKE_QUANTIZE: plan_fake_quantize(id); break;
-        case OP_CONVOLUTION: case OP_MATMUL: plan_conv(id); break;
-        case OP_GROUP_CONVOLUTION: unsupported(id, "grouped convolution is not planned yet");
+        case OP_CONVOLUTION: case OP_MATMUL: case OP_GROUP_CONVOLUTION: plan_conv(id); break;
         case OP_CONVERT: case OP_SUBTRACT: case OP_MULTIPLY: plan_dequant(id); break;
         case OP_MAX_POOL: case OP_AVG_POOL: plan_pool(id); break;
         case OP_RESHAPE: plan_reshape(id); break;
@@ -419,9 +418,15 @@ struct Planner {
             for (int64_t o = 0; o < OC; ++o)
                 for (int64_t k = 0; k < IC; ++k) st->weights[o * IC + k] = n.tb ? w[o * IC + k] : w[k * OC + o];
         } else {
-            OC = W.shape[0];
-            IC = W.shape[1];
-            d.kh = static_cast<int>(W.shape[2]); d.kw = static_cast<int>(W.shape[3]);
+            const bool grouped = n.op == OP_GROUP_CONVOLUTION;
+            if (grouped) {   // [G, OC/G, IC/G, kh, kw]: only depthwise (one filter per channel) is built
+                if (W.shape[1] != 1 || W.shape[2] != 1)
+                    unsupported(id, "grouped convolution other than depthwise");
+                d.groups = static_cast<int>(W.shape[0]);
+            }
+            OC = grouped ? W.shape[0] : W.shape[0];
+            IC = grouped ? W.shape[0] : W.shape[1];
+            d.kh = static_cast<int>(W.shape[grouped ? 3 : 2]); d.kw = static_cast<int>(W.shape[grouped ? 4 : 3]);
             d.stride_h = static_cast<int>(n.strides[0]); d.stride_w = static_cast<int>(n.strides[1]);
             d.dil_h = static_cast<int>(n.dilations[0]); d.dil_w = static_cast<int>(n.dilations[1]);
             d.pad_top = static_cast<int>(n.pads_begin[0]); d.pad_left = static_cast<int>(n.pads_begin[1]);
@@ -510,8 +515,8 @@ struct Planner {
         nhwc_dims(N(cur).shape, nn, c, h, w);
         st->out = new_tensor(cur, e.out_dtype, nn, h, w, c);
         st->name = N(cur).name;
-        st->type = is_mm ? "MatMul" : "Convolution";
-        st->macs = N(id).numel() * IC * d.kh * d.kw;
+        st->type = is_mm ? "MatMul" : (d.groups > 1 ? "GroupConvolution" : "Convolution");
+        st->macs = N(id).numel() * (d.groups > 1 ? 1 : IC) * d.kh * d.kw;
         st->bytes = 0;
         st->out_node = cur;
         values[cur].kind = VK_TENSOR;

@@ -152,10 +152,17 @@ class Convolution:
     def __init__(self, weights, in_tensor, strides=(1, 1), dilations=(1, 1), pads_begin=(0, 0),
                  pads_end=(0, 0), epilogue=None, device=0):
         w = np.ascontiguousarray(weights, np.int8)
-        self.oc, self.ic, self.kh, self.kw = w.shape
+        if w.ndim == 5:   # GroupConvolution filters [G, OC/G, IC/G, kh, kw]; depthwise only
+            groups = w.shape[0]
+            assert w.shape[1] == 1 and w.shape[2] == 1, "only depthwise group convolution"
+            self.oc = self.ic = groups
+            self.kh, self.kw = w.shape[3:]
+        else:
+            groups = 1
+            self.oc, self.ic, self.kh, self.kw = w.shape
         d = hipie_conv_desc(in_tensor.dtype, self.ic, self.oc, self.kh, self.kw, strides[0], strides[1],
                             dilations[0], dilations[1], pads_begin[0], pads_begin[1], pads_end[0],
-                            pads_end[1], 1, in_tensor.cs, in_tensor.stride_h, in_tensor.stride_w)
+                            pads_end[1], groups, in_tensor.cs, in_tensor.stride_h, in_tensor.stride_w)
         self.epilogue = epilogue or make_epilogue(out_dtype=I32)
         self._h = ctypes.c_void_p()
         check(lib().hipie_conv_create(ctypes.c_int(device), ctypes.byref(d),

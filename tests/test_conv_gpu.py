@@ -222,3 +222,29 @@ def test_conv_rejects_missing_halo_and_shape_mismatch():
     conv = Convolution(w, xin, pads_begin=(1, 1), pads_end=(1, 1))
     with pytest.raises(HipieError):
         conv.run(xin, DeviceTensor(1, 7, 8, 64, I32))
+
+
+@pytest.mark.parametrize("C,H,stride", [(32, 14, 1), (96, 15, 2), (144, 9, 1), (960, 7, 1)])
+def test_depthwise_conv_exact_and_relu6_requantize(orc, C, H, stride):
+    """MobileNetV2 depthwise 3x3 (GroupConvolution, G = C): i32 sums exact, then the post-LPT tail
+    Add(b') -> Multiply(s[c]) -> Clamp(0, 6) -> FQ(0, 6 -> u8) bit-exact."""
+    from dldt_amd import Convolution, DeviceTensor, make_epilogue
+    rng = np.random.default_rng(C)
+    x = rng.integers(0, 256, (2, C, H, H)).astype(np.int32)
+    w = rng.integers(-127, 128, (C, 1, 1, 3, 3)).astype(np.int32)
+    st = (stride, stride)
+    acc = orc.convolution(x, w, st, (1, 1), (1, 1), (1, 1), grouped=True)
+    xin = DeviceTensor.from_nchw(x, U8B, halo=1)
+    N, _, OH, OW = acc.shape
+    out = DeviceTensor(N, OH, OW, C, I32)
+    Convolution(w.astype(np.int8), xin, st, (1, 1), (1, 1), (1, 1)).run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw(), acc)
+    scale = (rng.uniform(0.5, 2.0, C) * 2e-4).astype(np.float32)
+    bias = rng.normal(0, 3000, C).astype(np.float32)
+    fq = (256, 0.0, np.float32(6.0), 0.0, 255.0)
+    want = _chain(orc, acc, bias=bias, scale=scale, act="clamp", clamp=(0.0, 6.0), fq=fq).astype(np.uint8)
+    out8 = DeviceTensor(N, OH, OW, C, U8B)
+    Convolution(w.astype(np.int8), xin, st, (1, 1), (1, 1), (1, 1),
+                make_epilogue(bias=bias, scale=scale, activation="clamp", clamp=(0.0, 6.0), out_dtype=U8B,
+                              fq=fq)).run(xin, out8)
+    np.testing.assert_array_equal(out8.to_nchw(), want)
