@@ -21,6 +21,13 @@ def lib():
             raise ImportError(
                 "%s is missing: build it with `python -m dldt_amd.build` "
                 "(there is no CPU fallback)" % LIB_PATH)
+        # One HIP runtime per process: PyTorch bundles its own libamdhip64.so.7; importing torch first
+        # makes the dynamic loader bind libhipie.so to that copy (same SONAME) instead of mapping a
+        # second runtime from /opt/rocm, which leaves whichever initialises second without a GPU.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         _lib = ctypes.CDLL(LIB_PATH)
         _lib.hipie_last_error.restype = ctypes.c_char_p
         _lib.hipie_version.restype = ctypes.c_char_p

@@ -46,6 +46,10 @@ class QuantizedNet:
         g = self.g
         wq, s_w = lpt.quantize_weights(w, 255)
         s = (np.float32(act["scale"]) * s_w).astype(np.float32)            # fold<Multiply>(s_a, s_w)
+        if conv_attrs.get("grouped"):
+            # GroupConvolution weights: FQ on [C, 1, kh, kw] then Reshape to [G, 1, 1, kh, kw]
+            # (the pattern LPT recognises, group_convolution.cpp:50-52); both fold into one constant
+            wq = wq.reshape(wq.shape[0], 1, 1, wq.shape[2], wq.shape[3])
         wc = g.constant(wq, I8)
         if matmul:
             y = g.matmul(act["node"], wc, False, True)
@@ -60,17 +64,36 @@ class QuantizedNet:
             y = g.add(y, g.constant(self._channel(bdiv, rank)))
         return y, s, rank
 
-    def conv(self, act, w, bias, out_high, strides=(1, 1), pads=(0, 0), dilations=(1, 1)):
-        """Quantized conv whose ReLU output feeds the next FakeQuantize [0, out_high]."""
+    @staticmethod
+    def signed_range(m):
+        """FakeQuantize range that getPrecisionDetails resolves to i8 without a zero point."""
+        hi = np.float32(m)
+        return np.float32(-hi * np.float32(128.0) / np.float32(127.0)), hi
+
+    def conv(self, act, w, bias, out_high, strides=(1, 1), pads=(0, 0), dilations=(1, 1), signed=False,
+             grouped=False):
+        """Quantized conv feeding the next activation FakeQuantize: [0, out_high] -> u8 (ReLU fused
+        away) or, for linear outputs, the symmetric range of signed_range(out_high) -> i8."""
         g = self.g
-        attrs = dict(strides=strides, dilations=dilations, pads_begin=pads, pads_end=pads)
+        attrs = dict(strides=strides, dilations=dilations, pads_begin=pads, pads_end=pads, grouped=grouped)
         y, s, rank = self._accumulate(act, w, bias, attrs)
-        d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(out_high))
-        il = (np.float32(0) / s).astype(np.float32)                          # fold<Divide>(il, s)
-        ih = (np.float32(out_high) / s).astype(np.float32)
+        lo, hi = self.signed_range(out_high) if signed else (np.float32(0), np.float32(out_high))
+        d = lpt.decompose_fake_quantize(256, lo, hi)
+        il = (lo / s).astype(np.float32)                                     # fold<Divide>(il, s)
+        ih = (hi / s).astype(np.float32)
         q = g.fake_quantize(y, self._channel(il, rank), self._channel(ih, rank), d["new_low"], d["new_high"],
-                            256, U8)
+                            256, d["precision"])
         return dict(node=q, scale=np.float32(d["scale"]))
+
+    def conv_relu6(self, act, w, bias, out_high, strides=(1, 1), pads=(0, 0), grouped=False):
+        """Conv -> bias -> ReLU6 -> FakeQuantize [0, out_high].  The dequantization Multiply is per
+        channel, so ClampTransformation leaves the Clamp in f32 (clamp.cpp:100-112) and the
+        FakeQuantize keeps its per-tensor range."""
+        g = self.g
+        attrs = dict(strides=strides, dilations=(1, 1), pads_begin=pads, pads_end=pads, grouped=grouped)
+        y, s, rank = self._accumulate(act, w, bias, attrs)
+        y = g.clamp(g.multiply(y, g.constant(self._channel(s, rank))), 0.0, 6.0)
+        return self.requantize(y, out_high)
 
     def conv_f32(self, act, w, bias, strides=(1, 1), pads=(0, 0), relu=False, matmul=False):
         """Quantized conv / FC whose result is consumed in f32: ... -> Multiply(s[c]) [-> ReLU]."""
@@ -85,10 +108,11 @@ class QuantizedNet:
         g = self.g
         return g.multiply(g.convert(act["node"], F32), g.constant(np.float32(act["scale"]).reshape(())))
 
-    def requantize(self, y, out_high):
-        """Activation FakeQuantize [0, out_high] on an f32 value (no pending Multiply to fold)."""
-        d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(out_high))
-        q = self.g.fake_quantize(y, np.float32(0), np.float32(out_high), d["new_low"], d["new_high"], 256, U8)
+    def requantize(self, y, out_high, signed=False):
+        """Activation FakeQuantize on an f32 value (no pending Multiply to fold)."""
+        lo, hi = self.signed_range(out_high) if signed else (np.float32(0), np.float32(out_high))
+        d = lpt.decompose_fake_quantize(256, lo, hi)
+        q = self.g.fake_quantize(y, lo, hi, d["new_low"], d["new_high"], 256, d["precision"])
         return dict(node=q, scale=np.float32(d["scale"]))
 
     def max_pool(self, act, kernel, strides, pads):
@@ -243,3 +267,134 @@ def resnet50_macs(res=224, classes=1000, width=64, stages=RESNET50_STAGES):
             ic = mid * 4
             h = h2
     return macs + classes * ic
+
+
+# ---------------------------------------------------------------------------------------------
+MOBILENETV2_BLOCKS = [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2),
+                      (6, 320, 1, 1)]
+
+
+def _mbv2_layers(width=1.0, blocks=MOBILENETV2_BLOCKS, last=1280):
+    """(name, kind, ic, oc, stride, residual) in execution order; channels rounded to multiples of 8."""
+    def ch(c):
+        return max(8, int(round(c * width / 8.0)) * 8)
+    layers = [("stem", "conv3", 3, ch(32), 2, False)]
+    ic = ch(32)
+    for bi, (t, c, n, s) in enumerate(blocks):
+        oc = ch(c)
+        for i in range(n):
+            p = "b%d.%d" % (bi, i)
+            mid = ic * t
+            stride = s if i == 0 else 1
+            if t != 1:
+                layers.append((p + ".expand", "pw_relu6", ic, mid, 1, False))
+            layers.append((p + ".dw", "dw", mid, mid, stride, False))
+            layers.append((p + ".project", "pw_linear", mid, oc, 1, stride == 1 and ic == oc))
+            ic = oc
+    layers.append(("head", "pw_relu6", ic, ch(last), 1, False))
+    return layers
+
+
+def mobilenet_v2_weights(seed=20211, classes=1000, width=1.0, blocks=MOBILENETV2_BLOCKS, last=1280):
+    rng = np.random.default_rng(seed)
+    P = {}
+    for name, kind, ic, oc, _, _ in _mbv2_layers(width, blocks, last):
+        shape = (oc, 1, 3, 3) if kind == "dw" else (oc, ic, 3, 3) if kind == "conv3" else (oc, ic, 1, 1)
+        P[name + ".w"] = he_normal(rng, shape)
+        P[name + ".b"] = (rng.standard_normal(oc, dtype=np.float32) * np.float32(0.1)).astype(np.float32)
+    feat = _mbv2_layers(width, blocks, last)[-1][3]
+    P["fc.w"] = he_normal(rng, (classes, feat))
+    P["fc.b"] = (rng.standard_normal(classes, dtype=np.float32) * np.float32(0.1)).astype(np.float32)
+    return P
+
+
+def mobilenet_v2_fp32(P, x, width=1.0, blocks=MOBILENETV2_BLOCKS, last=1280, record=None):
+    """fp32 forward on the host (torch CPU) for calibration."""
+    import torch
+    import torch.nn.functional as F
+
+    def t(a):
+        return torch.from_numpy(np.ascontiguousarray(a))
+
+    def rec(name, v, signed=False):
+        if record is not None:
+            record[name] = max(record.get(name, 0.0), float(v.abs().max() if signed else v.max()))
+        return v
+
+    names = {n for n, *_ in _mbv2_layers(width, blocks, last)}
+    with torch.no_grad():
+        v = rec("input", t(x))
+        block_in = None
+        for name, kind, ic, oc, stride, residual in _mbv2_layers(width, blocks, last):
+            w, b = t(P[name + ".w"]), t(P[name + ".b"])
+            if name.endswith(".expand") or (kind == "dw" and name[:-3] + ".expand" not in names):
+                block_in = v
+            if kind == "conv3":
+                v = rec(name, F.relu6(F.conv2d(v, w, b, stride=stride, padding=1)))
+            elif kind == "pw_relu6":
+                v = rec(name, F.relu6(F.conv2d(v, w, b)))
+            elif kind == "dw":
+                v = rec(name, F.relu6(F.conv2d(v, w, b, stride=stride, padding=1, groups=oc)))
+            else:
+                v = F.conv2d(v, w, b)
+                if residual:
+                    v = v + block_in
+                v = rec(name, v, signed=True)
+        v = rec("pool", v.mean(dim=(2, 3)))
+        v = F.linear(v, t(P["fc.w"]), t(P["fc.b"]))
+    return v.numpy()
+
+
+def mobilenet_v2(batch=1, res=224, seed=20211, classes=1000, width=1.0, blocks=MOBILENETV2_BLOCKS, last=1280,
+                 calib_batch=2):
+    """BASELINE config 4 as a post-LPT graph: ReLU6 outputs are u8 [0, max], linear bottleneck
+    outputs symmetric i8; depthwise layers are GroupConvolutions with [G,1,1,3,3] i8 filters."""
+    P = mobilenet_v2_weights(seed, classes, width, blocks, last)
+    rng = np.random.default_rng(seed + 1)
+    calib = rng.uniform(0, 1, (calib_batch, 3, res, res)).astype(np.float32)
+    R = {}
+    mobilenet_v2_fp32(P, calib, width, blocks, last, R)
+    net = QuantizedNet()
+    g = net.g
+    acts = {}
+    a = net.input("data", (batch, 3, res, res), R["input"])
+    layers = _mbv2_layers(width, blocks, last)
+    names = {n for n, *_ in layers}
+    block_in = None
+    macs = 0
+    hw = res
+    for name, kind, ic, oc, stride, residual in layers:
+        w, b = P[name + ".w"], P[name + ".b"]
+        if name.endswith(".expand") or (kind == "dw" and name[:-3] + ".expand" not in names):
+            block_in = a
+        if kind == "conv3":
+            a = net.conv_relu6(a, w, b, R[name], strides=(stride, stride), pads=(1, 1))
+            hw //= stride
+            macs += hw * hw * oc * ic * 9
+        elif kind == "pw_relu6":
+            a = net.conv_relu6(a, w, b, R[name])
+            macs += hw * hw * oc * ic
+        elif kind == "dw":
+            a = net.conv_relu6(a, w, b, R[name], strides=(stride, stride), pads=(1, 1), grouped=True)
+            hw //= stride
+            macs += hw * hw * oc * 9
+        else:
+            macs += hw * hw * oc * ic
+            if residual:
+                y = net.conv_f32(a, w, b)
+                a = net.requantize(g.add(y, net.dequantize(block_in)), R[name], signed=True)
+            else:
+                a = net.conv(a, w, b, R[name], signed=True)
+        acts[name] = a
+    y = g.avg_pool(a["node"], (hw, hw), (1, 1), (0, 0), (0, 0), exclude_pad=True, out_dtype=F32)
+    y = g.reshape(y, (batch, P["fc.w"].shape[1]))
+    d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(R["pool"]))
+    s_x = np.float32(a["scale"])
+    q = g.fake_quantize(y, (np.float32(0) / s_x).astype(np.float32), (np.float32(R["pool"]) / s_x).astype(np.float32),
+                        d["new_low"], d["new_high"], 256, U8)
+    pooled = dict(node=q, scale=np.float32(d["scale"]))
+    acts["pool"] = pooled
+    logits = net.conv_f32(pooled, P["fc.w"], P["fc.b"], matmul=True)
+    g.result(logits, "logits")
+    macs += P["fc.w"].size
+    return g, dict(params=P, ranges=R, acts=acts, macs_per_image=macs, calib=calib)

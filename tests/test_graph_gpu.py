@@ -58,3 +58,24 @@ def test_planner_reports_unsupported_nodes():
     with pytest.raises(HipieError) as e:
         g.compile()
     assert e.value.status == -2 and "Relu" in str(e.value)
+
+
+def test_small_mobilenet_v2_bit_exact(orc):
+    """MobileNetV2 topology (config 4) at reduced width/resolution: pointwise MFMA convs, depthwise
+    GroupConvolutions, ReLU6 (Clamp), signed i8 bottleneck outputs, residual adds."""
+    from dldt_amd import builders
+    g, meta = builders.mobilenet_v2(batch=2, res=64, width=0.5, classes=10, last=128, seed=3)
+    x = np.random.default_rng(4).uniform(0, 1, (2, 3, 64, 64)).astype(np.float32)
+    keep = [a["node"] for a in meta["acts"].values()]
+    want, kept = evaluate(orc, g.nodes, {"data": x}, keep=keep)
+    plan = g.compile()
+    assert any(s["type"] == "GroupConvolution" for s in plan.steps)
+    req = plan.create_request()
+    (got,) = req.infer(x)
+    for name, a in meta["acts"].items():
+        w = kept[a["node"]]
+        have = req.tensor(a["node"]).reshape(w.shape)
+        if w.dtype == np.int8:      # signed levels are stored as they are
+            have = have.view(np.int8)
+        np.testing.assert_array_equal(have, w, err_msg=name)
+    np.testing.assert_array_equal(got.view(np.uint32), want["logits"].view(np.uint32))
