@@ -42,9 +42,18 @@ __global__ __launch_bounds__(WOC* WPIX * 64, WOC* WPIX >= 4 ? 3 : 2) void conv_t
         const PixelCoord p = decode_pixel(a, m);
         b_base[i] = p.n * a.in_sn + p.oh * a.conv_sh * a.in_sh + p.ow * a.conv_sw * a.in_sw + a.in_origin;
     }
+    const int batch = blockIdx.y;
+    const int8_t* in_base = a.in + batch * a.batch_in;
 #pragma unroll
-    for (int i = 0; i < A_PIECES; ++i)
-        a_ptr[i] = a.wgt + static_cast<int64_t>(oc0 + ((tid + i * NT) >> 2)) * a.Kp + chunk * 16;
+    for (int i = 0; i < A_PIECES; ++i) {
+        int row = (tid + i * NT) >> 2;                 // row of the LDS tile
+        if (a.wgt_plain) {                             // natural row order in memory: LDS row 32*ob + j
+            const int j = row & 31;                    // must hold channel 32*((j>>2)&1) + 16*ob + 4*(j>>3) + (j&3)
+            row = (row & ~63) + 32 * ((j >> 2) & 1) + 16 * ((row >> 5) & 1) + 4 * (j >> 3) + (j & 3);
+        }
+        row = min(oc0 + row, a.wgt_rows - 1);
+        a_ptr[i] = a.wgt + batch * a.batch_wgt + static_cast<int64_t>(row) * a.wgt_ld + chunk * 16;
+    }
 
     v4i ga[A_PIECES], gb[B_PIECES];
     auto load_global = [&](int k) {
@@ -53,7 +62,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, WOC* WPIX >= 4 ? 3 : 2) void conv_t
 #pragma unroll
         for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(a_ptr[i] + k * 64);
 #pragma unroll
-        for (int i = 0; i < B_PIECES; ++i) gb[i] = *reinterpret_cast<const v4i*>(a.in + (b_base[i] + off));
+        for (int i = 0; i < B_PIECES; ++i) gb[i] = *reinterpret_cast<const v4i*>(in_base + (b_base[i] + off));
     };
     auto store_lds = [&](int buf) {
 #pragma unroll
@@ -95,7 +104,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, WOC* WPIX >= 4 ? 3 : 2) void conv_t
         __syncthreads();
     }
     const int m0 = pix0 + wpix * 64 + l32;
-    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32);
+    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -213,8 +222,8 @@ __global__ __launch_bounds__(256, 3) void conv_stream_kernel(const ConvArgs a) {
     }
 
 template <int WOC, int WPIX>
-void launch_tiled(const ConvArgs& a, hipStream_t s) {
-    const dim3 grid(8 * a.p_per_xcd * a.t_tiles), block(WOC * WPIX * 64);
+void launch_tiled(const ConvArgs& a, hipStream_t s, int batches = 1) {
+    const dim3 grid(8 * a.p_per_xcd * a.t_tiles, batches), block(WOC * WPIX * 64);
     const uint32_t core = a.flags & ~CF_OUT_XOR;
 #define HIPIE_LAUNCH_TILED(FLAGS, ...) \
     hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, FLAGS>), grid, block, 0, s, a)
@@ -357,7 +366,103 @@ struct hipie_conv {
     Epilogue epi;
 };
 
+struct hipie_matmul {
+    int device = 0;
+    hipie_matmul_desc d{};
+    int64_t Np = 0;
+    DeviceBuffer koff, corr;
+    Epilogue epi;
+};
+
 extern "C" {
+
+int hipie_matmul_create(int device, const hipie_matmul_desc* desc, const hipie_epilogue* epilogue,
+                        hipie_matmul** out) {
+    return guarded([&] {
+        HIPIE_REQUIRE(desc && epilogue && out, HIPIE_PARAMETER_MISMATCH, "hipie_matmul_create: null argument");
+        const hipie_matmul_desc& d = *desc;
+        HIPIE_REQUIRE(d.a_dtype == HIPIE_I8 && d.b_dtype == HIPIE_I8, HIPIE_NOT_IMPLEMENTED,
+                      "hipie_matmul_create: both operands must be i8 (a u8 left operand against a non-constant "
+                      "right operand would need its column sums at run time)");
+        HIPIE_REQUIRE(d.k > 0 && d.n > 0 && d.k % 64 == 0, HIPIE_NOT_IMPLEMENTED,
+                      "hipie_matmul_create: K=%d must be a positive multiple of 64", d.k);
+        auto m = std::make_unique<hipie_matmul>();
+        m->device = device;
+        m->d = d;
+        m->Np = round_up(d.n, 128);
+        std::vector<int32_t> koff(d.k / 16), corr(m->Np, 0);
+        for (size_t p = 0; p < koff.size(); ++p) koff[p] = static_cast<int32_t>(16 * p);
+        m->epi.build(device, *epilogue, d.n, m->Np);
+        if (device >= 0) {
+            m->koff.upload(device, koff.data(), koff.size() * sizeof(int32_t));
+            m->corr.upload(device, corr.data(), corr.size() * sizeof(int32_t));
+        }
+        *out = m.release();
+    });
+}
+
+void hipie_matmul_destroy(hipie_matmul* m) { delete m; }
+
+int hipie_matmul_run(const hipie_matmul* mm, const void* a_ptr, int64_t lda, int64_t stride_a, const void* bt_ptr,
+                     int64_t ldb, int64_t stride_b, void* out, int64_t ldo, int64_t stride_o, int32_t m,
+                     int32_t batch, void* stream) {
+    return guarded([&] {
+        HIPIE_REQUIRE(mm, HIPIE_PARAMETER_MISMATCH, "hipie_matmul_run: null handle");
+        HIPIE_REQUIRE(mm->koff.ptr, HIPIE_NOT_ALLOCATED, "hipie_matmul_run: host-only object");
+        if (m == 0 || batch == 0) return;
+        HIPIE_REQUIRE(a_ptr && bt_ptr && out && m > 0 && batch > 0, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_matmul_run: null operand or negative size");
+        const hipie_matmul_desc& d = mm->d;
+        const bool byte_out = mm->epi.out_dtype == HIPIE_U8B || mm->epi.out_dtype == HIPIE_I8;
+        const int gran = byte_out ? 16 : 4;
+        const int64_t n_pad = round_up(d.n, gran);
+        HIPIE_REQUIRE(lda >= d.k && ldb >= d.k && lda % 16 == 0 && ldb % 16 == 0 && ldo >= n_pad && ldo % gran == 0,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_matmul_run: leading dimensions (lda %lld, ldb %lld, ldo %lld)",
+                      (long long)lda, (long long)ldb, (long long)ldo);
+        HIPIE_REQUIRE(reinterpret_cast<uintptr_t>(a_ptr) % 16 == 0 && reinterpret_cast<uintptr_t>(bt_ptr) % 16 == 0 &&
+                          reinterpret_cast<uintptr_t>(out) % 16 == 0 && stride_a % 16 == 0 && stride_b % 16 == 0 &&
+                          stride_o % gran == 0,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_matmul_run: operands must be 16-byte aligned");
+        HIPIE_REQUIRE(static_cast<int64_t>(m) * lda < (1ll << 31) && m < (1 << 24), HIPIE_OUT_OF_BOUNDS,
+                      "hipie_matmul_run: matrix too large for 32-bit offsets");
+        HIPIE_REQUIRE(!(mm->epi.flags & CF_RES), HIPIE_NOT_IMPLEMENTED, "hipie_matmul_run: residual operand");
+        ConvArgs a{};
+        a.in = static_cast<const int8_t*>(a_ptr);
+        a.wgt = static_cast<const int8_t*>(bt_ptr);
+        a.out = out;
+        a.koff = mm->koff.as<int32_t>();
+        a.corr = mm->corr.as<int32_t>();
+        mm->epi.fill(a);
+        a.M = m;
+        a.OW = 1;
+        a.OHOW = m;
+        a.inv_OW = 1.0f;
+        a.inv_OHOW = 1.0f / static_cast<float>(m);
+        a.in_sh = static_cast<int32_t>(lda);
+        a.conv_sh = a.conv_sw = 1;
+        a.out_sh = static_cast<int32_t>(ldo);
+        a.out_sw = static_cast<int32_t>(n_pad);
+        a.OC = d.n;
+        a.OCp = static_cast<int32_t>(mm->Np);
+        a.Kp = d.k;
+        a.nk = d.k / 64;
+        a.wgt_ld = static_cast<int32_t>(ldb);
+        a.wgt_rows = d.n;
+        a.wgt_plain = 1;
+        a.batch_in = stride_a;
+        a.batch_wgt = stride_b;
+        a.batch_out = stride_o;
+        const bool wide = d.n > 64;
+        const int boc = wide ? 128 : 64, bpix = wide ? 128 : 256;
+        a.p_tiles = static_cast<int32_t>(ceil_div(m, bpix));
+        a.t_tiles = static_cast<int32_t>(ceil_div(d.n, boc));
+        a.p_per_xcd = static_cast<int32_t>(ceil_div(a.p_tiles, 8));
+        DeviceGuard g(mm->device);
+        if (wide) launch_tiled<2, 2>(a, as_stream(stream), batch);
+        else launch_tiled<1, 4>(a, as_stream(stream), batch);
+        HIPIE_CHECK_HIP(hipGetLastError());
+    });
+}
 
 int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* weights,
                       const hipie_epilogue* epilogue, hipie_conv** out) {
@@ -555,6 +660,9 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         a.OCp = static_cast<int32_t>(c->OCp);
         a.Kp = static_cast<int32_t>(c->Kp);
         a.nk = static_cast<int32_t>(c->Kp / 64);
+        a.wgt_ld = a.Kp;
+        a.wgt_rows = static_cast<int32_t>(c->OCp);
+        a.wgt_plain = 0;
         if (c->depthwise) {
             HIPIE_REQUIRE(in->stride_w >= d.ic && in->stride_w % 16 == 0, HIPIE_PARAMETER_MISMATCH,
                           "hipie_conv_run: depthwise input channel stride");

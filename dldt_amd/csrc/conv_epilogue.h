@@ -264,7 +264,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
 
 template <uint32_t F>
 __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
-                                             int m0, int m1) {
+                                             int m0, int m1, int batch = 0) {
     bool valid[2];
     int64_t out_off[2], res_off[2];
     const int m[2] = {m0, m1};
@@ -272,8 +272,10 @@ __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc
     for (int pb = 0; pb < 2; ++pb) {
         valid[pb] = m[pb] < a.M;
         const PixelCoord p = decode_pixel(a, valid[pb] ? m[pb] : a.M - 1);
-        out_off[pb] = static_cast<int64_t>(p.n) * a.out_sn + p.oh * a.out_sh + p.ow * a.out_sw + oc_lane;
-        res_off[pb] = static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh + p.ow * a.res_sw + oc_lane;
+        out_off[pb] = batch * a.batch_out + static_cast<int64_t>(p.n) * a.out_sn + p.oh * a.out_sh +
+                      p.ow * a.out_sw + oc_lane;
+        res_off[pb] = batch * a.batch_res + static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh +
+                      p.ow * a.res_sw + oc_lane;
     }
     epilogue<F>(a, acc, oc_lane, valid, out_off, res_off);
 }

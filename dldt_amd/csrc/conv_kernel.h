@@ -77,6 +77,12 @@ struct ConvArgs {
     int32_t p_tiles, t_tiles, p_per_xcd;
     uint32_t flags;
     float lm1, out_off, clamp_lo, clamp_hi;
+    // batched MatMul (grid.y = batch): per-batch strides in bytes (operands) / elements (out, res);
+    // wgt_ld = row stride of the weight-side operand, wgt_rows = rows that exist (others clamped),
+    // wgt_plain = rows are in natural order (activation operand): the loader applies the MFMA
+    // row permutation that constant weights carry from packing
+    int64_t batch_in, batch_wgt, batch_out, batch_res;
+    int32_t wgt_ld, wgt_rows, wgt_plain;
 };
 
 }  // namespace hipie

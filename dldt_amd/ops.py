@@ -188,3 +188,71 @@ class Convolution:
         check(lib().hipie_conv_run(self._h, ctypes.byref(xd), ctypes.byref(rd) if rd else None,
                                    ctypes.byref(od), _stream()))
         return out
+
+
+class hipie_matmul_desc(ctypes.Structure):
+    _fields_ = [(k, ctypes.c_int32) for k in ("a_dtype", "b_dtype", "k", "n")]
+
+
+class BatchedMatMul:
+    """i8 x i8 MatMul between two activation tensors: out[b] = A[b] @ Bt[b]^T (+ fused epilogue).
+
+    ``a`` is a torch int8 tensor [batch, M, K], ``bt`` is [batch, N, K] (the transpose_b = true
+    form); the result is [batch, M, ldo] with ldo = N padded to the store granularity.
+    """
+
+    def __init__(self, k, n, epilogue=None, device=0):
+        self.k, self.n = k, n
+        self.epilogue = epilogue or make_epilogue(out_dtype=I32)
+        d = hipie_matmul_desc(I8, I8, k, n)
+        self._h = ctypes.c_void_p()
+        check(lib().hipie_matmul_create(ctypes.c_int(device), ctypes.byref(d), ctypes.byref(self.epilogue),
+                                        ctypes.byref(self._h)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().hipie_matmul_destroy(self._h)
+            self._h = None
+
+    def run(self, a, bt):
+        import torch
+        batch, m, k = a.shape
+        assert bt.shape[0] == batch and bt.shape[2] == k and bt.shape[1] == self.n and k == self.k
+        assert a.is_contiguous() and bt.is_contiguous()
+        od = self.epilogue.out_dtype
+        tdt, gran = {I32: (torch.int32, 4), F32: (torch.float32, 4)}.get(od, (torch.int8, 16))
+        ldo = -(-self.n // gran) * gran
+        out = torch.zeros((batch, m, ldo), dtype=tdt, device=a.device)
+        i64 = ctypes.c_int64
+        check(lib().hipie_matmul_run(self._h, _dptr(a), i64(k), i64(m * k), _dptr(bt), i64(k), i64(self.n * k),
+                                     _dptr(out), i64(ldo), i64(m * ldo), ctypes.c_int32(m), ctypes.c_int32(batch),
+                                     _stream()))
+        return out[..., :self.n]
+
+
+def softmax(x):
+    import torch
+    assert x.is_contiguous() and x.dtype == torch.float32
+    y = torch.empty_like(x)
+    check(lib().hipie_softmax_f32(_dptr(x), _dptr(y), ctypes.c_int64(x.numel() // x.shape[-1]),
+                                  ctypes.c_int64(x.shape[-1]), _stream()))
+    return y
+
+
+def mvn(x, normalize_variance=True, eps=1e-5, eps_inside=True, gamma=None, beta=None):
+    import torch
+    assert x.is_contiguous() and x.dtype == torch.float32
+    y = torch.empty_like(x)
+    check(lib().hipie_mvn_f32(_dptr(x), _dptr(y), ctypes.c_int64(x.numel() // x.shape[-1]),
+                              ctypes.c_int64(x.shape[-1]), int(normalize_variance), ctypes.c_float(eps),
+                              int(eps_inside), _dptr(gamma) if gamma is not None else None,
+                              _dptr(beta) if beta is not None else None, _stream()))
+    return y
+
+
+def gelu(x):
+    import torch
+    assert x.is_contiguous() and x.dtype == torch.float32
+    y = torch.empty_like(x)
+    check(lib().hipie_gelu_f32(_dptr(x), _dptr(y), ctypes.c_int64(x.numel()), _stream()))
+    return y

@@ -189,6 +189,41 @@ int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_t
                    const hipie_tensor* out, void* stream);
 
 /* ======================================================================================
+ * 1d. MatMul between two activations (attention scores and context) — reference::matmul<int32_t>
+ *     on widened inputs (ngraph/core/reference/.../matmul.hpp:24-57 dot, :75-247 batching), as the
+ *     TypeRelaxed MatMul LPT emits (low_precision_transformations/src/mat_mul.cpp:81-171), plus the
+ *     fused epilogue.  out[b][i][j] = sum_k A[b][i][k] * Bt[b][j][k]: the right operand is passed
+ *     in its transpose_b = true form ([N][K], K contiguous).  MatMul against constant weights is a
+ *     1x1 convolution (hipie_conv_*).  Leading dimensions and batch strides are in elements.
+ * ==================================================================================== */
+typedef struct hipie_matmul_desc {
+    int32_t a_dtype, b_dtype;   /* HIPIE_I8 (symmetric activations on both sides) */
+    int32_t k, n;               /* reduction length (multiple of 64), output columns */
+} hipie_matmul_desc;
+
+typedef struct hipie_matmul hipie_matmul;
+
+int hipie_matmul_create(int device, const hipie_matmul_desc* desc, const hipie_epilogue* epilogue,
+                        hipie_matmul** matmul);
+void hipie_matmul_destroy(hipie_matmul* matmul);
+int hipie_matmul_run(const hipie_matmul* matmul, const void* a, int64_t lda, int64_t stride_a,
+                     const void* b_transposed, int64_t ldb, int64_t stride_b, void* out, int64_t ldo,
+                     int64_t stride_o, int32_t m, int32_t batch, void* stream);
+
+/* ======================================================================================
+ * 1e. fp32 glue of the transformer path, over the last axis of a dense [rows, axis] f32 matrix
+ *     (device pointers).  Tolerance parity only (GPU exp / erf differ from libm in the last ulp).
+ *       hipie_softmax_f32  reference::softmax      (.../reference/softmax.hpp:20-50)
+ *       hipie_mvn_f32      reference::mvn_6        (.../reference/mvn.hpp:64-117), optionally followed
+ *                          by the LayerNorm Multiply(gamma[axis]) and Add(beta[axis]) (device arrays or NULL)
+ *       hipie_gelu_f32     reference::gelu, ERF    (.../reference/gelu.hpp:18-28)
+ * ==================================================================================== */
+int hipie_softmax_f32(const float* x, float* y, int64_t rows, int64_t axis, void* stream);
+int hipie_mvn_f32(const float* x, float* y, int64_t rows, int64_t axis, int normalize_variance, float eps,
+                  int eps_inside_sqrt, const float* gamma, const float* beta, void* stream);
+int hipie_gelu_f32(const float* x, float* y, int64_t n, void* stream);
+
+/* ======================================================================================
  * 2. Graph level.  The plugin's LoadExeNetworkImpl walks Function::get_ordered_ops()
  *    (ngraph/core/include/ngraph/function.hpp:126) of the post-LPT function and issues one call
  *    per node; value ids are returned in creation order.  Shapes are the reference's (NCHW,

@@ -1,0 +1,76 @@
+"""MatMul on int8 MFMA (constant weights and activation x activation, BASELINE config 5 shapes) and
+the fp32 glue (softmax, MVN/LayerNorm, GELU) through the C ABI vs the oracle."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+F32, I8, I32, U8B = 10, 50, 70, 41
+
+
+@pytest.mark.parametrize("batch,m,k,n", [(6, 384, 64, 384), (6, 384, 384, 64), (3, 100, 128, 200), (2, 7, 64, 40)])
+def test_batched_matmul_i8_exact(orc, batch, m, k, n):
+    """Attention scores [S,64]x[64,S] and context [S,S]x[S,64]: exact i32 = reference matmul<int32_t>."""
+    import torch
+    from dldt_amd import BatchedMatMul
+    rng = np.random.default_rng(m + n)
+    a = rng.integers(-128, 128, (batch, m, k)).astype(np.int8)
+    bt = rng.integers(-128, 128, (batch, n, k)).astype(np.int8)
+    want = orc.matmul(a.astype(np.int32), bt.astype(np.int32), False, True)
+    got = BatchedMatMul(k, n).run(torch.from_numpy(a).cuda(), torch.from_numpy(bt).cuda()).cpu().numpy()
+    np.testing.assert_array_equal(got, want)
+
+
+def test_batched_matmul_scaled_and_requantized(orc):
+    """MatMul' -> Multiply(s_a * s_b) -> f32, and -> FakeQuantize (symmetric i8) as the next MatMul wants it."""
+    import torch
+    from dldt_amd import BatchedMatMul, make_epilogue
+    rng = np.random.default_rng(3)
+    batch, m, k, n = 4, 96, 64, 128
+    a = rng.integers(-128, 128, (batch, m, k)).astype(np.int8)
+    bt = rng.integers(-128, 128, (batch, n, k)).astype(np.int8)
+    acc = orc.matmul(a.astype(np.int32), bt.astype(np.int32), False, True).astype(np.float32)
+    s = np.float32(0.02) * np.float32(0.03)                 # mat_mul_transformation.cpp:156-174 golden: 0.0006
+    want = orc.multiply(acc, s)
+    ad, bd = torch.from_numpy(a).cuda(), torch.from_numpy(bt).cuda()
+    got = BatchedMatMul(k, n, make_epilogue(scale=[s], out_dtype=F32)).run(ad, bd).cpu().numpy()
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    hi = np.float32(np.abs(want).max())
+    lo = np.float32(-hi * np.float32(128) / np.float32(127))
+    lv = orc.fake_quantize(want, lo, hi, np.float32(-128), np.float32(127), 256).astype(np.int8)
+    got8 = BatchedMatMul(k, n, make_epilogue(scale=[s], out_dtype=I8, fq=(256, lo, hi, -128.0, 127.0))).run(ad, bd)
+    np.testing.assert_array_equal(got8.cpu().numpy(), lv)
+
+
+def test_fc_matmul_constant_weights(orc):
+    """FC [N,2048] x [2048,1000]^T as the 1x1 convolution path: u8 rows, i8 constant weights."""
+    from dldt_amd import Convolution, DeviceTensor
+    rng = np.random.default_rng(11)
+    x = rng.integers(0, 256, (5, 2048, 1, 1)).astype(np.int32)
+    w = rng.integers(-127, 128, (1000, 2048, 1, 1)).astype(np.int32)
+    want = orc.matmul(x[:, :, 0, 0], w[:, :, 0, 0], False, True)
+    xin = DeviceTensor.from_nchw(x, U8B)
+    out = DeviceTensor(5, 1, 1, 1000, I32)
+    Convolution(w.astype(np.int8), xin).run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw()[:, :, 0, 0], want)
+
+
+def test_softmax_mvn_gelu_tolerance(orc):
+    import torch
+    from dldt_amd import gelu, mvn, softmax
+    rng = np.random.default_rng(13)
+    x = (rng.standard_normal((2, 12, 48, 384)) * 3).astype(np.float32)
+    xd = torch.from_numpy(x).cuda()
+    np.testing.assert_allclose(softmax(xd).cpu().numpy(), orc.softmax(x, -1), rtol=2e-6, atol=1e-8)
+    h = (rng.standard_normal((96, 768)) * 2 + 0.3).astype(np.float32)
+    hd = torch.from_numpy(h).cuda()
+    for inside in (True, False):
+        np.testing.assert_allclose(mvn(hd, True, 1e-5, inside).cpu().numpy(),
+                                   orc.mvn_last_axis(h, True, 1e-5, inside), rtol=1e-5, atol=2e-6)
+    gamma = rng.uniform(0.5, 1.5, 768).astype(np.float32)
+    beta = rng.normal(0, 0.1, 768).astype(np.float32)
+    want = orc.add(orc.multiply(orc.mvn_last_axis(h, True, 1e-5, True), gamma), beta)
+    got = mvn(hd, True, 1e-5, True, torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()).cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=2e-6)
+    f = (rng.standard_normal((64, 3072)) * 2).astype(np.float32)
+    np.testing.assert_allclose(gelu(torch.from_numpy(f).cuda()).cpu().numpy(), orc.gelu_erf(f), rtol=1e-6, atol=1e-8)
