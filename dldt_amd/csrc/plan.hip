@@ -158,7 +158,7 @@ struct PoolStep : Step {
         };
         if (!mul.empty()) {
             const auto m = expand(mul, 1.f);
-            d_mul.upload(device, m.data(), m.size() * 4);
+            if (device >= 0) d_mul.upload(device, m.data(), m.size() * 4);
             a.mul = d_mul.as<float>();
         }
         if (!fq_il.empty()) {
@@ -181,10 +181,12 @@ struct PoolStep : Step {
                 HIPIE_REQUIRE((static_cast<float>(k) / a.lm1 * (fq_oh - fq_ol) + fq_ol) == fq_ol + k,
                               HIPIE_NOT_IMPLEMENTED, "%s: output levels are not integers", name.c_str());
             a.out_off = to.dtype == HIPIE_U8B ? fq_ol - 128.f : fq_ol;
-            d_il.upload(device, il.data(), il.size() * 4);
-            d_ih.upload(device, ih.data(), ih.size() * 4);
-            d_d.upload(device, d.data(), d.size() * 4);
-            d_r.upload(device, r.data(), r.size() * 4);
+            if (device >= 0) {
+                d_il.upload(device, il.data(), il.size() * 4);
+                d_ih.upload(device, ih.data(), ih.size() * 4);
+                d_d.upload(device, d.data(), d.size() * 4);
+                d_r.upload(device, r.data(), r.size() * 4);
+            }
             a.fq_il = d_il.as<float>(); a.fq_ih = d_ih.as<float>();
             a.fq_d = d_d.as<float>(); a.fq_r = d_r.as<float>();
         }
@@ -217,6 +219,7 @@ struct ExitStep : Step {
             for (int c = 0; c < C; ++c) o[c] = v[v.size() == 1 ? 0 : c];
             return o;
         };
+        if (device < 0) return;
         if (!sub.empty()) { const auto v = expand(sub); d_sub.upload(device, v.data(), v.size() * 4); }
         if (!mul.empty()) { const auto v = expand(mul); d_mul.upload(device, v.data(), v.size() * 4); }
     }
@@ -740,6 +743,8 @@ int hipie_plan_step_info(const hipie_plan* p, int index, char* name, size_t name
 int hipie_request_create(const hipie_plan* p, int perf_count, hipie_request** out) {
     return guarded([&] {
         HIPIE_REQUIRE(p && out, HIPIE_PARAMETER_MISMATCH, "hipie_request_create: null argument");
+        HIPIE_REQUIRE(p->device >= 0, HIPIE_NOT_ALLOCATED,
+                      "hipie_request_create: the plan was compiled without a device (dry run)");
         auto r = std::make_unique<hipie_request>();
         r->plan = p;
         r->perf = perf_count != 0;

@@ -1,0 +1,109 @@
+"""The restated LPT load-time arithmetic (include/hipie.h section 3) against the constants the
+reference's own LPT unit tests expect (tests/golden/lpt.json), and the planner's fusion decisions in
+a dry run without a device."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from dldt_amd import lpt
+
+G = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "lpt.json")))
+PREC = {"u8": 40, "i8": 50, None: None}
+
+
+@pytest.mark.parametrize("case", G["precision_details"]["cases"])
+def test_precision_details(case):
+    prec, neg, zp = lpt.precision_details(case["levels"], np.float32(case["out_low"]), np.float32(case["out_high"]))
+    assert prec == PREC[case["precision"]] and neg == case["has_negative"] and zp == case["has_zero_point"]
+
+
+@pytest.mark.parametrize("case", G["decompose"]["cases"])
+def test_decompose_scale_shift(case):
+    import ctypes
+    from dldt_amd._lib import check, lib
+    ol, oh = np.array([case["out_low"]], np.float32), np.array([case["out_high"]], np.float32)
+    sc, sh, nl, nh = (np.empty(1, np.float32) for _ in range(4))
+    p = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))  # noqa: E731
+    check(lib().hipie_lpt_decompose_fake_quantize(p(ol), p(oh), ctypes.c_int64(1), ctypes.c_float(case["min"]),
+                                                  ctypes.c_float(case["max"]), p(sc), p(sh), p(nl), p(nh)))
+    np.testing.assert_allclose(sc[0], case["scale"], rtol=1e-6)
+    np.testing.assert_allclose(sh[0], case["shift"], rtol=1e-6, atol=1e-6)
+    assert nl[0] == case["min"] and nh[0] == case["max"]
+
+
+def test_decompose_picks_precision_and_range():
+    d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(2.55))
+    assert d["precision"] == 40 and d["new_low"] == 0 and d["new_high"] == 255
+    np.testing.assert_allclose(d["scale"], 0.01, rtol=1e-6)
+    d = lpt.decompose_fake_quantize(256, np.float32(-1.28), np.float32(1.27))
+    assert d["precision"] == 50 and d["new_low"] == -128 and d["new_high"] == 127
+    with pytest.raises(NotImplementedError):
+        lpt.decompose_fake_quantize(256, np.float32(0.12), np.float32(1.23))   # needs a zero point
+
+
+@pytest.mark.parametrize("case", G["fold"]["cases"])
+def test_fold_fake_quantize(case):
+    v = np.array(case["values"], np.float32).reshape(2, 8)
+    got = lpt.fold_fake_quantize(v, case["il"], case["ih"], case["ol"], case["oh"], case["levels"], case["round"])
+    np.testing.assert_allclose(got.ravel(), np.array(case["expected"], np.float32), rtol=1e-5, atol=1e-5)
+
+
+def test_convolution_weight_and_scale_golden():
+    c = G["convolution"]
+    d = lpt.decompose_fake_quantize(c["levels"], np.float32(c["ol"]), np.float32(c["oh"]))
+    assert d["precision"] == 50 and (d["new_low"], d["new_high"]) == (-127, 127)
+    q = lpt.fold_fake_quantize(np.array([[c["weight"]]], np.float32), c["il"], c["ih"], d["new_low"], d["new_high"],
+                               c["levels"], True)
+    assert q[0, 0] == c["expected_i8"]
+    np.testing.assert_allclose(np.float32(c["act_scale"]) * d["scale"], c["expected_scale"], rtol=1e-6)
+    m = G["matmul"]
+    np.testing.assert_allclose(np.float32(m["scale_a"]) * np.float32(m["scale_b"]), m["expected"], rtol=1e-6)
+
+
+def test_quantize_weights_roundtrip():
+    rng = np.random.default_rng(0)
+    w = rng.normal(0, 0.05, (8, 4, 3, 3)).astype(np.float32)
+    q, s = lpt.quantize_weights(w)
+    assert q.dtype == np.int8 and np.abs(q).max() == 127
+    assert np.abs(q.astype(np.float32) * s.reshape(-1, 1, 1, 1) - w).max() <= s.max() / 2 + 1e-7
+
+
+# ------------------------------------------------------------------ planner dry run (no device)
+def _steps(g):
+    from dldt_amd.graph import Plan
+    return [(s["type"], s["name"]) for s in Plan(g, device=-1).steps]
+
+
+def test_planner_fuses_resnet_block_chains():
+    from dldt_amd import builders
+    g, meta = builders.resnet50(batch=1, res=64, width=16, classes=10, seed=7)
+    from dldt_amd.graph import Plan
+    plan = Plan(g, device=-1)
+    types = [s["type"] for s in plan.steps]
+    # entry FQ, 53 convolutions, max-pool, avg-pool(+FQ), FC, exit; every elementwise node is fused away
+    assert types.count("Convolution") == 53 and types.count("MatMul") == 1
+    assert types.count("MaxPool") == 1 and types.count("AvgPool") == 1
+    assert types[0] == "FakeQuantize" and types[-1] == "Result" and len(types) == 58
+    assert sum(s["macs"] for s in plan.steps) == meta["macs_per_image"]
+    assert plan.arena_bytes > 0
+    with pytest.raises(Exception) as e:
+        plan.create_request()
+    assert "dry run" in str(e.value)
+
+
+def test_planner_mobilenet_has_depthwise_steps():
+    from dldt_amd import builders
+    from dldt_amd.graph import Plan
+    g, meta = builders.mobilenet_v2(batch=1, res=64, width=0.5, classes=10, last=128, seed=3)
+    plan = Plan(g, device=-1)
+    types = [s["type"] for s in plan.steps]
+    assert types.count("GroupConvolution") == 17
+    assert sum(s["macs"] for s in plan.steps) == meta["macs_per_image"]
+
+
+def test_full_size_mac_counts_match_the_published_architecture():
+    from dldt_amd import builders
+    assert builders.resnet50_macs() == 4089184256          # 4.089 GMAC per image
+    assert 0.29e9 < builders.mobilenet_v2(batch=1, res=224)[1]["macs_per_image"] < 0.32e9
