@@ -96,7 +96,7 @@ def main():
         for i, st in enumerate(preq.perf()):
             acc[i] = acc.get(i, 0.0) + st["ms"]
     steps = [dict(st, ms=acc[i] / reps) for i, st in enumerate(plan.steps)]
-    mfma = [s for s in steps if s["type"] in ("Convolution", "MatMul")]
+    mfma = [s for s in steps if s["type"] in ("Convolution", "Convolution+Shortcut", "MatMul")]
     mfma_ms = sum(s["ms"] for s in mfma)
     mfma_ops = 2.0 * sum(s["macs"] for s in mfma)
     achieved_tops = mfma_ops / (mfma_ms * 1e-3) / 1e12
@@ -118,7 +118,7 @@ def main():
                      "ops_per_step": mfma_ops, "kernel_ms_per_step": mfma_ms,
                      "avg_launch_us": mfma_ms * 1e3 / len(mfma), "note": "int8 TOP/s, dense peak 5.0 POP/s"},
         "other_kernels_ms_per_step": {t: sum(s["ms"] for s in steps if s["type"] == t)
-                                      for t in sorted({s["type"] for s in steps} - {"Convolution", "MatMul"})},
+                                      for t in sorted({s["type"] for s in steps} - {"Convolution", "Convolution+Shortcut", "MatMul"})},
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.batch)

@@ -14,7 +14,7 @@ constexpr int kRow = 80;  // LDS row stride of the tiled kernel: 64 K-bytes + 16
 // ------------------------------------------------------------------------------------------------
 // LDS-tiled kernel
 template <int WOC, int WPIX, uint32_t F>
-__global__ __launch_bounds__(WOC* WPIX * 64, WOC* WPIX >= 4 ? 3 : 2) void conv_tiled_kernel(const ConvArgs a) {
+__global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && (F & CF_RES_GEMM))) ? 3 : 2) void conv_tiled_kernel(const ConvArgs a) {
     constexpr int NT = WOC * WPIX * 64;
     constexpr int BOC = WOC * 64, BPIX = WPIX * 64;
     constexpr int A_PIECES = BOC * 4 / NT, B_PIECES = BPIX * 4 / NT;
@@ -33,78 +33,108 @@ __global__ __launch_bounds__(WOC* WPIX * 64, WOC* WPIX >= 4 ? 3 : 2) void conv_t
     const int l32 = lane & 31, h = lane >> 5;
     const int chunk = tid & 3;
 
-    int32_t b_base[B_PIECES];
-    const int8_t* a_ptr[A_PIECES];
-#pragma unroll
-    for (int i = 0; i < B_PIECES; ++i) {
-        int m = pix0 + ((tid + i * NT) >> 2);
-        m = m < a.M ? m : a.M - 1;
-        const PixelCoord p = decode_pixel(a, m);
-        b_base[i] = p.n * a.in_sn + p.oh * a.conv_sh * a.in_sh + p.ow * a.conv_sw * a.in_sw + a.in_origin;
-    }
     const int batch = blockIdx.y;
-    const int8_t* in_base = a.in + batch * a.batch_in;
-#pragma unroll
-    for (int i = 0; i < A_PIECES; ++i) {
-        int row = (tid + i * NT) >> 2;                 // row of the LDS tile
-        if (a.wgt_plain) {                             // natural row order in memory: LDS row 32*ob + j
-            const int j = row & 31;                    // must hold channel 32*((j>>2)&1) + 16*ob + 4*(j>>3) + (j&3)
-            row = (row & ~63) + 32 * ((j >> 2) & 1) + 16 * ((row >> 5) & 1) + 4 * (j >> 3) + (j & 3);
-        }
-        row = min(oc0 + row, a.wgt_rows - 1);
-        a_ptr[i] = a.wgt + batch * a.batch_wgt + static_cast<int64_t>(row) * a.wgt_ld + chunk * 16;
-    }
-
-    v4i ga[A_PIECES], gb[B_PIECES];
-    auto load_global = [&](int k) {
-        const int4 ko = *reinterpret_cast<const int4*>(a.koff + 4 * k);   // uniform: scalar load
-        const int32_t off = chunk == 0 ? ko.x : (chunk == 1 ? ko.y : (chunk == 2 ? ko.z : ko.w));
-#pragma unroll
-        for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(a_ptr[i] + k * 64);
-#pragma unroll
-        for (int i = 0; i < B_PIECES; ++i) gb[i] = *reinterpret_cast<const v4i*>(in_base + (b_base[i] + off));
-    };
-    auto store_lds = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < A_PIECES; ++i)
-            *reinterpret_cast<v4i*>(&sA[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = ga[i];
-#pragma unroll
-        for (int i = 0; i < B_PIECES; ++i)
-            *reinterpret_cast<v4i*>(&sB[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = gb[i];
-    };
-
     const int a_row[2] = {woc * 64 + l32, woc * 64 + 32 + l32};
     const int b_row[2] = {wpix * 64 + l32, wpix * 64 + 32 + l32};
     const int oc_lane = oc0 + woc * 64 + 32 * h;
 
-    load_global(0);
-    v16i acc[2][2];
-    init_acc(a, oc_lane, acc);
-    store_lds(0);
-    __syncthreads();
-    for (int k = 0; k < a.nk; ++k) {
-        const int buf = k & 1;
-        if (k + 1 < a.nk) load_global(k + 1);
+    // one implicit GEMM over an operand set (activation tensor, packed weights, K-offset table)
+    auto gemm = [&](const int8_t* in_base, int in_sn, int in_sh, int in_sw, int csh, int csw, int origin,
+                    const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk,
+                    v16i (&acc)[2][2]) {
+        int32_t b_base[B_PIECES];
+        const int8_t* a_ptr[A_PIECES];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            v4i af[2], bf[2];
+        for (int i = 0; i < B_PIECES; ++i) {
+            int m = pix0 + ((tid + i * NT) >> 2);
+            m = m < a.M ? m : a.M - 1;
+            const PixelCoord p = decode_pixel(a, m);
+            b_base[i] = p.n * in_sn + p.oh * csh * in_sh + p.ow * csw * in_sw + origin;
+        }
 #pragma unroll
-            for (int ob = 0; ob < 2; ++ob)
-                af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][a_row[ob] * kRow + ks * 32 + h * 16]);
+        for (int i = 0; i < A_PIECES; ++i) {
+            int row = (tid + i * NT) >> 2;                 // row of the LDS tile
+            if (wgt_plain) {                               // natural row order in memory: LDS row 32*ob + j
+                const int j = row & 31;                    // must hold channel 32*((j>>2)&1) + 16*ob + 4*(j>>3) + (j&3)
+                row = (row & ~63) + 32 * ((j >> 2) & 1) + 16 * ((row >> 5) & 1) + 4 * (j >> 3) + (j & 3);
+            }
+            row = min(oc0 + row, wgt_rows - 1);
+            a_ptr[i] = wgt_base + static_cast<int64_t>(row) * wgt_ld + chunk * 16;
+        }
+        v4i ga[A_PIECES], gb[B_PIECES];
+        auto load_global = [&](int k) {
+            const int4 ko = *reinterpret_cast<const int4*>(koff + 4 * k);   // uniform: scalar load
+            const int32_t off = chunk == 0 ? ko.x : (chunk == 1 ? ko.y : (chunk == 2 ? ko.z : ko.w));
 #pragma unroll
-            for (int pb = 0; pb < 2; ++pb)
-                bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][b_row[pb] * kRow + ks * 32 + h * 16]);
+            for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(a_ptr[i] + k * 64);
 #pragma unroll
-            for (int ob = 0; ob < 2; ++ob)
+            for (int i = 0; i < B_PIECES; ++i) gb[i] = *reinterpret_cast<const v4i*>(in_base + (b_base[i] + off));
+        };
+        auto store_lds = [&](int buf) {
+#pragma unroll
+            for (int i = 0; i < A_PIECES; ++i)
+                *reinterpret_cast<v4i*>(&sA[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = ga[i];
+#pragma unroll
+            for (int i = 0; i < B_PIECES; ++i)
+                *reinterpret_cast<v4i*>(&sB[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = gb[i];
+        };
+        load_global(0);
+        store_lds(0);
+        __syncthreads();
+        for (int k = 0; k < nk; ++k) {
+            const int buf = k & 1;
+            if (k + 1 < nk) load_global(k + 1);
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                v4i af[2], bf[2];
+#pragma unroll
+                for (int ob = 0; ob < 2; ++ob)
+                    af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][a_row[ob] * kRow + ks * 32 + h * 16]);
 #pragma unroll
                 for (int pb = 0; pb < 2; ++pb)
-                    acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
+                    bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][b_row[pb] * kRow + ks * 32 + h * 16]);
+#pragma unroll
+                for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                    for (int pb = 0; pb < 2; ++pb)
+                        acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
+            }
+            if (k + 1 < nk) store_lds(buf ^ 1);
+            __syncthreads();
         }
-        if (k + 1 < a.nk) store_lds(buf ^ 1);
-        __syncthreads();
+    };
+
+    v16i acc[2][2];
+    v16f rres[2][2];
+    constexpr bool kFused = F != kDyn && (F & CF_RES_GEMM);
+    if (kFused) {
+        // shortcut convolution first: (float(acc2) + bias2[c]) * scale2[c] stays in registers
+        ConvArgs a2 = a;
+        a2.corr = a.corr2;
+        init_acc(a2, oc_lane, acc);
+        gemm(a.in2, a.in2_sn, a.in2_sh, a.in2_sw, a.conv2_sh, a.conv2_sw, a.in2_origin, a.wgt2, a.Kp2, a.OCp, false,
+             a.koff2, a.nk2, acc);
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float4 b4 = ld4f(a.bias2 + oc_lane + 16 * ob + 4 * q);
+                const float4 s4 = ld4f(a.scale2 + oc_lane + 16 * ob + 4 * q);
+                const float bb[4] = {b4.x, b4.y, b4.z, b4.w}, ss[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float x = static_cast<float>(acc[ob][pb][4 * q + j]) + bb[j];
+                        rres[ob][pb][4 * q + j] = x * ss[j];
+                    }
+            }
     }
+    init_acc(a, oc_lane, acc);
+    gemm(a.in + batch * a.batch_in, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
+         a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc);
     const int m0 = pix0 + wpix * 64 + l32;
-    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch);
+    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -215,6 +245,7 @@ __global__ __launch_bounds__(256, 3) void conv_stream_kernel(const ConvArgs a) {
     case E_PLAIN: X(E_PLAIN, __VA_ARGS__); break;                                            \
     case E_RESU8: X(E_RESU8, __VA_ARGS__); break;                                            \
     case E_RESF32: X(E_RESF32, __VA_ARGS__); break;                                          \
+    case E_RESGEMM: X(E_RESGEMM, __VA_ARGS__); break;                                        \
     case E_F32: X(E_F32, __VA_ARGS__); break;                                                \
     case E_F32RELU: X(E_F32RELU, __VA_ARGS__); break;                                        \
     case E_CLAMPFQ: X(E_CLAMPFQ, __VA_ARGS__); break;                                        \
@@ -268,6 +299,7 @@ void Epilogue::build(int device_, const hipie_epilogue& e, int64_t oc, int64_t o
     case HIPIE_F32: flags |= CF_RES | CF_RES_F32; break;
     case HIPIE_U8B: flags |= CF_RES | CF_RES_U8B; break;
     case HIPIE_I8: flags |= CF_RES; break;
+    case HIPIE_RESIDUAL_SHORTCUT_CONV: flags |= CF_RES | CF_RES_GEMM; break;
     default: fail(HIPIE_PARAMETER_MISMATCH, "epilogue: residual dtype %d", e.residual_dtype);
     }
     if (flags & CF_RES) {
@@ -356,10 +388,23 @@ static int64_t packed_row(int64_t oc) {
     return (oc & ~int64_t(63)) + 32 * ob + 8 * q + 4 * hh + t;
 }
 
+// Dense convolution operand set packed for the MFMA kernels: weights [OCp][Kp] (rows in MFMA
+// order), byte offset of every 16-byte K piece, per-channel integer correction.
+struct PackedGemm {
+    int64_t K = 0, Kp = 0, OCp = 0;
+    DeviceBuffer wgt, koff, corr;
+    void pack(int device, const hipie_conv_desc& d, const int8_t* weights);
+};
+
 struct hipie_conv {
     int device = 0;
     hipie_conv_desc d{};
     int64_t K = 0, Kp = 0, OCp = 0;
+    // fused shortcut convolution (second operand set + its bias / scale tables)
+    bool fused = false;
+    hipie_conv_desc sd{};
+    PackedGemm sg;
+    DeviceBuffer s_bias, s_scale;
     bool depthwise = false;
     int tile = 0;  // 0: tiled 128 ch x 128 px, 1: tiled 64 x 256, 2: tiled 64 x 64, 3: streaming (64 ch, weights in LDS)
     DeviceBuffer wgt, koff, corr;
@@ -373,6 +418,67 @@ struct hipie_matmul {
     DeviceBuffer koff, corr;
     Epilogue epi;
 };
+
+void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weights) {
+    // K order (kh, kw, ic) over the padded channel stride.  A 16-byte piece must not straddle
+    // two filter taps unless consecutive taps are contiguous in memory (in_stride_w == c stride).
+    const bool row_contig = d.in_stride_w == d.in_c_stride && d.dil_w == 1;
+    HIPIE_REQUIRE(d.in_c_stride % 16 == 0 || row_contig, HIPIE_NOT_IMPLEMENTED,
+                  "convolution: channel stride %d needs a multiple of 16", d.in_c_stride);
+    const int64_t cs = d.in_c_stride;
+    const int64_t row_kp = round_up(d.kw * cs, 16);   // bytes of one filter row when taps are contiguous
+    const bool per_row = cs % 16 != 0;                // small-channel first layer: pad every filter row
+    K = per_row ? d.kh * row_kp : static_cast<int64_t>(d.kh) * d.kw * cs;
+    Kp = round_up(K, 64);
+    OCp = round_up(d.oc, 128);
+    std::vector<int32_t> off(Kp / 16, 0);
+    for (int64_t p = 0; p < K / 16; ++p) {
+        const int64_t k = p * 16;
+        if (per_row) {
+            const int64_t kh = k / row_kp, within = k % row_kp;
+            off[p] = static_cast<int32_t>(kh * d.dil_h * d.in_stride_h + within);
+        } else {
+            const int64_t tap = k / cs, ic0 = k % cs;
+            const int64_t kh = tap / d.kw, kw = tap % d.kw;
+            off[p] = static_cast<int32_t>(kh * d.dil_h * d.in_stride_h + kw * d.dil_w * d.in_stride_w + ic0);
+        }
+    }
+    std::vector<int8_t> w(static_cast<size_t>(OCp) * Kp, 0);
+    std::vector<int32_t> cr(OCp, 0);
+    parallel_for(d.oc, [&](int64_t oc) {
+        int64_t sum = 0;
+        for (int kh = 0; kh < d.kh; ++kh)
+            for (int kw = 0; kw < d.kw; ++kw)
+                for (int ic = 0; ic < d.ic; ++ic) {
+                    const int8_t v = weights[((oc * d.ic + ic) * d.kh + kh) * d.kw + kw];
+                    const int64_t k = per_row ? kh * row_kp + kw * cs + ic
+                                              : (static_cast<int64_t>(kh) * d.kw + kw) * cs + ic;
+                    w[packed_row(oc) * Kp + k] = v;
+                    sum += v;
+                }
+        cr[oc] = d.in_dtype == HIPIE_U8B ? static_cast<int32_t>(128 * sum) : 0;
+    });
+    if (device >= 0) {
+        wgt.upload(device, w.data(), w.size());
+        koff.upload(device, off.data(), off.size() * sizeof(int32_t));
+        corr.upload(device, cr.data(), cr.size() * sizeof(int32_t));
+    }
+}
+
+static void check_conv_desc(const hipie_conv_desc& d, const char* what) {
+    HIPIE_REQUIRE(d.in_dtype == HIPIE_U8B || d.in_dtype == HIPIE_I8, HIPIE_PARAMETER_MISMATCH,
+                  "%s: input dtype %d (U8B or I8 expected)", what, d.in_dtype);
+    HIPIE_REQUIRE(d.ic > 0 && d.oc > 0 && d.kh > 0 && d.kw > 0 && d.stride_h > 0 && d.stride_w > 0 && d.dil_h > 0 &&
+                      d.dil_w > 0 && d.pad_top >= 0 && d.pad_left >= 0 && d.pad_bottom >= 0 && d.pad_right >= 0,
+                  HIPIE_PARAMETER_MISMATCH, "%s: bad geometry", what);
+    HIPIE_REQUIRE(d.in_c_stride >= d.ic && d.in_c_stride % 4 == 0, HIPIE_PARAMETER_MISMATCH,
+                  "%s: in_c_stride=%d must be a multiple of 4 >= ic=%d", what, d.in_c_stride, d.ic);
+}
+
+static void conv_out_hw(const hipie_conv_desc& d, int h, int w, int& oh, int& ow) {
+    oh = (h + d.pad_top + d.pad_bottom - (d.dil_h * (d.kh - 1) + 1)) / d.stride_h + 1;
+    ow = (w + d.pad_left + d.pad_right - (d.dil_w * (d.kw - 1) + 1)) / d.stride_w + 1;
+}
 
 extern "C" {
 
@@ -509,58 +615,54 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
             *out = c.release();
             return;
         }
-        // K order (kh, kw, ic) over the padded channel stride.  A 16-byte piece must not straddle
-        // two filter taps unless consecutive taps are contiguous in memory (in_stride_w == c stride).
-        const bool row_contig = d.in_stride_w == d.in_c_stride && d.dil_w == 1;
-        HIPIE_REQUIRE(d.in_c_stride % 16 == 0 || row_contig, HIPIE_NOT_IMPLEMENTED,
-                      "hipie_conv_create: channel stride %d needs a multiple of 16", d.in_c_stride);
-        const int64_t cs = d.in_c_stride;
-        int64_t row_k = d.kw * cs;             // bytes of one filter row when taps are contiguous
-        int64_t row_kp = round_up(row_k, 16);
-        const bool per_row = cs % 16 != 0;      // small-channel first layer: pad every filter row
-        c->K = per_row ? d.kh * row_kp : static_cast<int64_t>(d.kh) * d.kw * cs;
-        c->Kp = round_up(c->K, 64);
-        c->OCp = round_up(d.oc, 128);
-        // offsets of every 16-byte K piece
-        std::vector<int32_t> koff(c->Kp / 16, 0);
-        for (int64_t p = 0; p < c->K / 16; ++p) {
-            const int64_t k = p * 16;
-            if (per_row) {
-                const int64_t kh = k / row_kp, within = k % row_kp;
-                koff[p] = static_cast<int32_t>(kh * d.dil_h * d.in_stride_h + within);
-            } else {
-                const int64_t tap = k / cs, ic0 = k % cs;
-                const int64_t kh = tap / d.kw, kw = tap % d.kw;
-                koff[p] = static_cast<int32_t>(kh * d.dil_h * d.in_stride_h + kw * d.dil_w * d.in_stride_w + ic0);
-            }
-        }
-        // pack weights OIHW -> [OCp][Kp]
-        std::vector<int8_t> w(static_cast<size_t>(c->OCp) * c->Kp, 0);
-        std::vector<int32_t> corr(c->OCp, 0);
-        parallel_for(d.oc, [&](int64_t oc) {
-            int64_t sum = 0;
-            for (int kh = 0; kh < d.kh; ++kh)
-                for (int kw = 0; kw < d.kw; ++kw)
-                    for (int ic = 0; ic < d.ic; ++ic) {
-                        const int8_t v = weights[((oc * d.ic + ic) * d.kh + kh) * d.kw + kw];
-                        const int64_t k = per_row ? kh * row_kp + kw * cs + ic
-                                                  : (static_cast<int64_t>(kh) * d.kw + kw) * cs + ic;
-                        w[packed_row(oc) * c->Kp + k] = v;
-                        sum += v;
-                    }
-            corr[oc] = d.in_dtype == HIPIE_U8B ? static_cast<int32_t>(128 * sum) : 0;
-        });
+        PackedGemm g;
+        g.pack(device, d, weights);
+        c->K = g.K; c->Kp = g.Kp; c->OCp = g.OCp;
+        c->wgt = std::move(g.wgt); c->koff = std::move(g.koff); c->corr = std::move(g.corr);
         c->epi.build(device, *epilogue, d.oc, c->OCp);
-        // tile choice: wide channel tiles when there are enough channels, else all waves on pixels
         // default: wide channel tiles when there are enough channels, else all waves on pixels
         // (the planner may override this after timing the candidates)
         c->tile = d.oc > 64 ? 0 : 1;
-        if (device >= 0) {
-            c->wgt.upload(device, w.data(), w.size());
-            c->koff.upload(device, koff.data(), koff.size() * sizeof(int32_t));
-            c->corr.upload(device, corr.data(), corr.size() * sizeof(int32_t));
-        }
         *out = c.release();
+    });
+}
+
+int hipie_conv_create_fused(int device, const hipie_conv_desc* desc, const int8_t* weights,
+                            const hipie_epilogue* epilogue, const hipie_conv_desc* shortcut_desc,
+                            const int8_t* shortcut_weights, const float* shortcut_bias, int64_t n_bias,
+                            const float* shortcut_scale, int64_t n_scale, hipie_conv** out) {
+    return guarded([&] {
+        HIPIE_REQUIRE(desc && weights && epilogue && shortcut_desc && shortcut_weights && shortcut_bias &&
+                          shortcut_scale && out,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_conv_create_fused: null argument");
+        HIPIE_REQUIRE(epilogue->residual_dtype == HIPIE_RESIDUAL_SHORTCUT_CONV, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_create_fused: the epilogue's residual must be HIPIE_RESIDUAL_SHORTCUT_CONV");
+        const hipie_conv_desc& sd = *shortcut_desc;
+        check_conv_desc(sd, "hipie_conv_create_fused (shortcut)");
+        HIPIE_REQUIRE(sd.groups == 1 && desc->groups == 1 && sd.oc == desc->oc, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_create_fused: both convolutions must be dense with the same output channels");
+        for (int64_t n : {n_bias, n_scale})
+            HIPIE_REQUIRE(n == 1 || n == sd.oc, HIPIE_PARAMETER_MISMATCH, "hipie_conv_create_fused: table length");
+        hipie_conv* c = nullptr;
+        const int st = hipie_conv_create(device, desc, weights, epilogue, &c);
+        if (st != HIPIE_OK) fail(static_cast<hipie_status>(st), "%s", hipie_last_error());
+        std::unique_ptr<hipie_conv> guard(c);
+        HIPIE_REQUIRE((c->epi.flags & ~CF_OUT_XOR) == E_RESGEMM, HIPIE_NOT_IMPLEMENTED,
+                      "hipie_conv_create_fused: the fused form needs bias, scale, FakeQuantize with input_low 0");
+        c->fused = true;
+        c->sd = sd;
+        c->sg.pack(device, sd, shortcut_weights);
+        std::vector<float> b(c->OCp, 0.f), s(c->OCp, 1.f);
+        for (int oc = 0; oc < sd.oc; ++oc) {
+            b[oc] = shortcut_bias[n_bias == 1 ? 0 : oc];
+            s[oc] = shortcut_scale[n_scale == 1 ? 0 : oc];
+        }
+        if (device >= 0) {
+            c->s_bias.upload(device, b.data(), b.size() * sizeof(float));
+            c->s_scale.upload(device, s.data(), s.size() * sizeof(float));
+        }
+        c->tile = 0;
+        *out = guard.release();
     });
 }
 
@@ -569,6 +671,7 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
         HIPIE_REQUIRE(c && tile >= 0 && tile <= 3, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        if (c->fused || c->depthwise) return;   // one kernel only
         HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: K=%lld does not fit the streaming kernel's LDS", (long long)c->Kp);
         c->tile = tile;
@@ -628,7 +731,37 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         a.koff = c->koff.as<int32_t>();
         a.corr = c->corr.as<int32_t>();
         c->epi.fill(a);
-        if (a.flags & CF_RES) {
+        if (a.flags & CF_RES_GEMM) {
+            // `residual` is the INPUT of the fused shortcut convolution
+            HIPIE_REQUIRE(c->fused && residual && residual->data, HIPIE_PARAMETER_MISMATCH,
+                          "hipie_conv_run: shortcut input missing");
+            const hipie_conv_desc& sd = c->sd;
+            HIPIE_REQUIRE(residual->dtype == sd.in_dtype && residual->c == sd.ic && residual->n == in->n &&
+                              residual->stride_w == sd.in_stride_w && residual->stride_h == sd.in_stride_h,
+                          HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: shortcut input does not match its packing");
+            int soh, sow;
+            conv_out_hw(sd, residual->h, residual->w, soh, sow);
+            HIPIE_REQUIRE(soh == oh && sow == ow, HIPIE_PARAMETER_MISMATCH,
+                          "hipie_conv_run: shortcut convolution yields %dx%d, main %dx%d", soh, sow, oh, ow);
+            HIPIE_REQUIRE(residual->halo >= std::max(std::max(sd.pad_top, sd.pad_bottom), std::max(sd.pad_left, sd.pad_right)),
+                          HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: shortcut input halo");
+            HIPIE_REQUIRE(static_cast<int64_t>(residual->n) * residual->stride_n < (1ll << 31), HIPIE_OUT_OF_BOUNDS,
+                          "hipie_conv_run: shortcut tensor too large");
+            a.in2 = static_cast<const int8_t*>(residual->data);
+            a.wgt2 = c->sg.wgt.as<int8_t>();
+            a.koff2 = c->sg.koff.as<int32_t>();
+            a.corr2 = c->sg.corr.as<int32_t>();
+            a.bias2 = c->s_bias.as<float>();
+            a.scale2 = c->s_scale.as<float>();
+            a.in2_sn = static_cast<int32_t>(residual->stride_n);
+            a.in2_sh = static_cast<int32_t>(residual->stride_h);
+            a.in2_sw = static_cast<int32_t>(residual->stride_w);
+            a.conv2_sh = sd.stride_h;
+            a.conv2_sw = sd.stride_w;
+            a.in2_origin = -(sd.pad_top * a.in2_sh + sd.pad_left * a.in2_sw);
+            a.Kp2 = static_cast<int32_t>(c->sg.Kp);
+            a.nk2 = static_cast<int32_t>(c->sg.Kp / 64);
+        } else if (a.flags & CF_RES) {
             HIPIE_REQUIRE(residual && residual->data, HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: residual missing");
             const int want = (a.flags & CF_RES_F32) ? HIPIE_F32 : ((a.flags & CF_RES_U8B) ? HIPIE_U8B : HIPIE_I8);
             HIPIE_REQUIRE(residual->dtype == want && residual->n == out->n && residual->h == oh &&
@@ -678,7 +811,7 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         a.p_per_xcd = static_cast<int32_t>(ceil_div(a.p_tiles, 8));
         DeviceGuard g(c->device);
         hipStream_t s = as_stream(stream);
-        switch (c->tile) {
+        switch (c->fused ? 0 : c->tile) {
         case 0: launch_tiled<2, 2>(a, s); break;
         case 1: launch_tiled<1, 4>(a, s); break;
         case 2: launch_tiled_small(a, s); break;

@@ -10,6 +10,7 @@ namespace hipie {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 
 // m -> (m / d, m % d) for m < 2^24 through a float reciprocal (exact after one correction step)
 __device__ __forceinline__ void fast_divmod(int m, int d, float inv_d, int& q, int& r) {
@@ -84,6 +85,7 @@ constexpr uint32_t E_PLAIN0 = CF_BIAS | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
 constexpr uint32_t E_PLAIN = CF_BIAS | CF_OUT_FQ | CF_FQ_RCP;
 constexpr uint32_t E_RESU8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_U8B | CF_RES_MUL | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
 constexpr uint32_t E_RESF32 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32 | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
+constexpr uint32_t E_RESGEMM = CF_BIAS | CF_SCALE | CF_RES | CF_RES_GEMM | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
 constexpr uint32_t E_F32 = CF_BIAS | CF_SCALE;
 constexpr uint32_t E_F32RELU = CF_BIAS | CF_SCALE | CF_RELU;
 constexpr uint32_t E_CLAMPFQ = CF_BIAS | CF_SCALE | CF_CLAMP | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
@@ -105,7 +107,7 @@ __device__ __forceinline__ void f4_to_array(const float4& v, float (&o)[4]) {
 template <uint32_t F>
 __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                          const bool (&valid)[2], const int64_t (&out_off)[2],
-                                         const int64_t (&res_off)[2]) {
+                                         const int64_t (&res_off)[2], const v16f (&rres)[2][2]) {
     const uint32_t fl = F == kDyn ? a.flags : F;
     const int out_cs = a.out_sw;
 
@@ -123,7 +125,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
     }
 
     uint32_t res_dw[2][8];
-    if ((fl & CF_RES) && !(fl & CF_RES_F32)) {
+    if ((fl & CF_RES) && !(fl & (CF_RES_F32 | CF_RES_GEMM))) {
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb)
 #pragma unroll
@@ -191,7 +193,10 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
         for (int pb = 0; pb < 2; ++pb) {
             float rv[4];
             if (fl & CF_RES) {
-                if (fl & CF_RES_F32) f4_to_array(cur.res[pb], rv);
+                if (fl & CF_RES_GEMM) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) rv[j] = rres[ob][pb][r0 + j];
+                } else if (fl & CF_RES_F32) f4_to_array(cur.res[pb], rv);
                 else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) rv[j] = res_byte_to_float(res_dw[pb][e4], j, res_add);
@@ -264,7 +269,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
 
 template <uint32_t F>
 __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
-                                             int m0, int m1, int batch = 0) {
+                                             int m0, int m1, int batch, const v16f (&rres)[2][2]) {
     bool valid[2];
     int64_t out_off[2], res_off[2];
     const int m[2] = {m0, m1};
@@ -277,7 +282,14 @@ __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc
         res_off[pb] = batch * a.batch_res + static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh +
                       p.ow * a.res_sw + oc_lane;
     }
-    epilogue<F>(a, acc, oc_lane, valid, out_off, res_off);
+    epilogue<F>(a, acc, oc_lane, valid, out_off, res_off, rres);
+}
+
+template <uint32_t F>
+__device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
+                                             int m0, int m1, int batch = 0) {
+    v16f none[2][2];
+    run_epilogue<F>(a, acc, oc_lane, m0, m1, batch, none);
 }
 
 }  // namespace hipie

@@ -44,6 +44,7 @@ enum ConvFlags : uint32_t {
     CF_RES_U8B = 1u << 12,    // residual bytes are level-128 (add 128 after conversion)
     CF_FQ_IL0 = 1u << 13,     // every input_low is +0: x - il == x
     CF_OUT_XOR = 1u << 14,    // packed levels ^ 0x80808080 is the stored byte (offset -128)
+    CF_RES_GEMM = 1u << 15,   // residual = (float(acc2) + bias2[c]) * scale2[c] of a second GEMM run in the same kernel
 };
 
 struct ConvArgs {
@@ -83,6 +84,15 @@ struct ConvArgs {
     // row permutation that constant weights carry from packing
     int64_t batch_in, batch_wgt, batch_out, batch_res;
     int32_t wgt_ld, wgt_rows, wgt_plain;
+    // fused shortcut convolution (CF_RES_GEMM): a second operand set accumulated first; its
+    // dequantised result stays in registers as the residual of the main convolution
+    const int8_t* in2;
+    const int8_t* wgt2;
+    const int32_t* koff2;
+    const int32_t* corr2;
+    const float* bias2;
+    const float* scale2;
+    int32_t in2_sn, in2_sh, in2_sw, conv2_sh, conv2_sw, in2_origin, nk2, Kp2;
 };
 
 }  // namespace hipie

@@ -112,24 +112,56 @@ struct ConvStep : Step {
     std::vector<int8_t> weights;   // OIHW
     EpilogueSpec epi;
     hipie_conv* conv = nullptr;
+    // projection shortcut (Conv' -> Add -> Multiply, f32, used only by this step's residual Add):
+    // run inside this step's kernel when the fused form applies, else right before it
+    std::unique_ptr<ConvStep> shortcut;
+    bool fused = false;
     ~ConvStep() override { hipie_conv_destroy(conv); }
-    void create(int device, const std::vector<TensorInfo>& tensors) override {
+    void fill_desc(const std::vector<TensorInfo>& tensors) {
         const TensorInfo& t = tensors[in];
         desc.in_dtype = t.dtype;
         desc.in_c_stride = t.cs;
         desc.in_stride_w = t.cs;
         desc.in_stride_h = t.wp() * t.cs;
-        const hipie_epilogue e = epi.c_struct();
-        check_status(hipie_conv_create(device, &desc, weights.data(), &e, &conv), name.c_str());
+    }
+    void create(int device, const std::vector<TensorInfo>& tensors) override {
+        fill_desc(tensors);
+        if (shortcut) {
+            shortcut->fill_desc(tensors);
+            EpilogueSpec fe = epi;
+            fe.residual_dtype = HIPIE_RESIDUAL_SHORTCUT_CONV;
+            const hipie_epilogue e = fe.c_struct();
+            const EpilogueSpec& se = shortcut->epi;
+            const int st = hipie_conv_create_fused(device, &desc, weights.data(), &e, &shortcut->desc,
+                                                   shortcut->weights.data(), se.bias.data(), se.bias.size(),
+                                                   se.scale.data(), se.scale.size(), &conv);
+            if (st == HIPIE_OK) {
+                fused = true;
+                type = "Convolution+Shortcut";
+            } else if (st == HIPIE_NOT_IMPLEMENTED) {
+                shortcut->create(device, tensors);   // run it as its own kernel, f32 through the arena
+            } else {
+                check_status(st, name.c_str());
+            }
+        }
+        if (!fused) {
+            const hipie_epilogue e = epi.c_struct();
+            check_status(hipie_conv_create(device, &desc, weights.data(), &e, &conv), name.c_str());
+        }
         weights.clear();
         weights.shrink_to_fit();
     }
-    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const*, void* const*,
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const* outputs,
              hipStream_t s) const override {
         const hipie_tensor i = tensors[in].desc(arena), o = tensors[out].desc(arena);
         hipie_tensor r{};
-        if (res >= 0) r = tensors[res].desc(arena);
-        check_status(hipie_conv_run(conv, &i, res >= 0 ? &r : nullptr, &o, s), name.c_str());
+        if (fused) {
+            r = tensors[shortcut->in].desc(arena);
+        } else {
+            if (shortcut) shortcut->run(arena, tensors, inputs, outputs, s);
+            if (res >= 0) r = tensors[res].desc(arena);
+        }
+        check_status(hipie_conv_run(conv, &i, (fused || res >= 0) ? &r : nullptr, &o, s), name.c_str());
     }
 };
 
@@ -447,7 +479,7 @@ struct Planner {
 
         // ---- absorb the elementwise chain behind the accumulator --------------------------------
         EpilogueSpec& e = st->epi;
-        int cur = id, stage = 0;
+        int cur = id, stage = 0, shortcut_step = -1;
         const size_t rank = n.shape.size();
         while (single_user(cur)) {
             const int nx = N(cur).users[0];
@@ -472,6 +504,7 @@ struct Planner {
                         e.res_mul = r.mul;
                     } else if (r.kind == VK_TENSOR && tensors[r.tensor].dtype == HIPIE_F32) {
                         e.residual_dtype = HIPIE_F32;
+                        shortcut_step = find_shortcut(r.tensor, other);
                     } else {
                         break;
                     }
@@ -508,6 +541,11 @@ struct Planner {
             cur = nx;
         }
         if (e.residual_dtype == 0) { e.res_sub.clear(); e.res_mul.clear(); }
+        if (shortcut_step >= 0 && st->res >= 0 && !is_mm && d.groups == 1) {
+            // take the projection shortcut out of the step list: it runs inside this step
+            st->shortcut.reset(static_cast<ConvStep*>(steps[shortcut_step].release()));
+            steps.erase(steps.begin() + shortcut_step);
+        }
         // mark the absorbed nodes
         for (int k = id; k != cur;) {
             const int nx = N(k).users[0];
@@ -519,13 +557,28 @@ struct Planner {
         st->out = new_tensor(cur, e.out_dtype, nn, h, w, c);
         st->name = N(cur).name;
         st->type = is_mm ? "MatMul" : (d.groups > 1 ? "GroupConvolution" : "Convolution");
-        st->macs = N(id).numel() * (d.groups > 1 ? 1 : IC) * d.kh * d.kw;
+        st->macs = N(id).numel() * (d.groups > 1 ? 1 : IC) * d.kh * d.kw + (st->shortcut ? st->shortcut->macs : 0);
         st->bytes = 0;
         st->out_node = cur;
         values[cur].kind = VK_TENSOR;
         values[cur].tensor = st->out;
         if (cur != id) values[id].kind = VK_FUSED;
         steps.push_back(std::move(st));
+    }
+
+    // A dense convolution step that produces f32 tensor `t` with nothing but bias and scale, consumed
+    // only by the residual Add: candidate for running inside the consumer's kernel.
+    int find_shortcut(int t, int value_node) const {
+        if (N(value_node).users.size() != 1) return -1;
+        for (size_t i = 0; i < steps.size(); ++i) {
+            auto* cs = dynamic_cast<ConvStep*>(steps[i].get());
+            if (!cs || cs->out != t) continue;
+            const EpilogueSpec& e = cs->epi;
+            const bool plain = !e.bias.empty() && !e.scale.empty() && e.residual_dtype == 0 && e.post_scale.empty() &&
+                               e.activation == 0 && e.out_dtype == HIPIE_F32 && cs->desc.groups == 1 && !cs->shortcut;
+            return plain && cs->type == "Convolution" ? static_cast<int>(i) : -1;
+        }
+        return -1;
     }
 
     void plan_pool(int id) {

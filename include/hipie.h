@@ -141,10 +141,13 @@ int hipie_fq_uses_reciprocal(const hipie_fq* fq);
  *        FakeQuantize(in_low[c], in_high[c], out_low, out_high, levels) -> 8-bit     or f32 store
  *     Arrays are host pointers with 1 (broadcast) or OC values; NULL skips the step.
  * ==================================================================================== */
+#define HIPIE_RESIDUAL_SHORTCUT_CONV 1
+
 typedef struct hipie_epilogue {
     const float* bias;        int64_t n_bias;
     const float* scale;       int64_t n_scale;
-    int32_t residual_dtype;   /* 0 = none, HIPIE_F32, HIPIE_U8B (value = level), HIPIE_I8 */
+    int32_t residual_dtype;   /* 0 = none, HIPIE_F32, HIPIE_U8B (value = level), HIPIE_I8, or
+                                 HIPIE_RESIDUAL_SHORTCUT_CONV (hipie_conv_create_fused) */
     const float* res_sub;     int64_t n_res_sub;
     const float* res_mul;     int64_t n_res_mul;
     const float* post_scale;  int64_t n_post_scale;
@@ -179,6 +182,17 @@ typedef struct hipie_conv hipie_conv;
 
 int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* weights_oihw,
                       const hipie_epilogue* epilogue, hipie_conv** conv);
+/* Residual block tail with a projection shortcut in ONE kernel: the shortcut convolution
+ * (Conv' -> Add(bias) -> Multiply(scale), f32, consumed only by the residual Add) is accumulated
+ * first and its dequantised value stays in registers as the residual operand of the main
+ * convolution's epilogue, instead of an f32 round trip through HBM.  Same arithmetic, same order,
+ * same bits as running the two convolutions separately.  The epilogue must be bias, scale,
+ * residual = HIPIE_RESIDUAL_SHORTCUT_CONV, FakeQuantize with input_low 0.  hipie_conv_run takes the
+ * shortcut convolution's INPUT tensor in its `residual` argument. */
+int hipie_conv_create_fused(int device, const hipie_conv_desc* desc, const int8_t* weights_oihw,
+                            const hipie_epilogue* epilogue, const hipie_conv_desc* shortcut_desc,
+                            const int8_t* shortcut_weights_oihw, const float* shortcut_bias, int64_t n_bias,
+                            const float* shortcut_scale, int64_t n_scale, hipie_conv** conv);
 void hipie_conv_destroy(hipie_conv* conv);
 /* output spatial dims for an input of h x w (convolution.hpp:168-183) */
 int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* oh, int32_t* ow);

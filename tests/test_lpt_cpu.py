@@ -82,10 +82,11 @@ def test_planner_fuses_resnet_block_chains():
     from dldt_amd.graph import Plan
     plan = Plan(g, device=-1)
     types = [s["type"] for s in plan.steps]
-    # entry FQ, 53 convolutions, max-pool, avg-pool(+FQ), FC, exit; every elementwise node is fused away
-    assert types.count("Convolution") == 53 and types.count("MatMul") == 1
-    assert types.count("MaxPool") == 1 and types.count("AvgPool") == 1
-    assert types[0] == "FakeQuantize" and types[-1] == "Result" and len(types) == 58
+    # entry FQ, 53 convolutions (the 4 projection shortcuts run inside their residual convolution),
+    # max-pool, avg-pool(+FQ), FC, exit; every elementwise node is fused away
+    assert types.count("Convolution") == 45 and types.count("Convolution+Shortcut") == 4
+    assert types.count("MatMul") == 1 and types.count("MaxPool") == 1 and types.count("AvgPool") == 1
+    assert types[0] == "FakeQuantize" and types[-1] == "Result" and len(types) == 54
     assert sum(s["macs"] for s in plan.steps) == meta["macs_per_image"]
     assert plan.arena_bytes > 0
     with pytest.raises(Exception) as e:
