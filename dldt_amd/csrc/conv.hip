@@ -138,6 +138,164 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
 }
 
 // ------------------------------------------------------------------------------------------------
+// Pipelined LDS-tiled kernel: a ring of `stages` K steps in LDS filled by direct global->LDS loads
+// (global_load_lds_dwordx4: no staging registers, so many K steps can be in flight), one raw
+// s_barrier per step.  Rows are 64 bytes without padding; the 16-byte chunk c of row r sits in
+// slot c ^ ((r >> 2) & 3), which makes both the DMA writes (lane t -> byte 16 t of a 1 KiB group)
+// and the ds_read_b128 fragment reads (16 consecutive rows, one logical chunk) conflict-free.
+// Hazards are ordered by hand: a wave waits for its own loads of the step it is about to read
+// (s_waitcnt vmcnt(n) with the younger stages still in flight), then the barrier makes every
+// wave's part of that step visible and proves that the stage about to be refilled is no longer read.
+constexpr int waitcnt_vm(int n) {
+    // s_waitcnt immediate: vmcnt in bits [3:0] and [15:14]; expcnt / lgkmcnt left at "no wait"
+    return 0x0F70 | (n & 15) | ((n >> 4) << 14);
+}
+
+// wait until at most LPS * younger of this wave's loads are outstanding (younger = 0..6 stages)
+template <int LPS>
+__device__ __forceinline__ void wait_vmcnt_stages(int younger) {
+    switch (younger) {
+    case 0: __builtin_amdgcn_s_waitcnt(waitcnt_vm(0)); break;
+    case 1: __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPS)); break;
+    case 2: __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * LPS)); break;
+    case 3: __builtin_amdgcn_s_waitcnt(waitcnt_vm(3 * LPS)); break;
+    case 4: __builtin_amdgcn_s_waitcnt(waitcnt_vm(4 * LPS)); break;
+    case 5: __builtin_amdgcn_s_waitcnt(waitcnt_vm(5 * LPS)); break;
+    default: __builtin_amdgcn_s_waitcnt(waitcnt_vm(6 * LPS)); break;
+    }
+}
+
+template <int WOC, int WPIX, uint32_t F>
+__global__ __launch_bounds__(WOC* WPIX * 64, (F != kDyn && (F & CF_RES_GEMM)) ? 2 : 3)
+void conv_pipe_kernel(const ConvArgs a, const int stages) {
+    constexpr int NT = WOC * WPIX * 64;
+    constexpr int BOC = WOC * 64, BPIX = WPIX * 64;
+    constexpr int A_GROUPS = BOC / 16 / (NT / 64), B_GROUPS = BPIX / 16 / (NT / 64);   // 1 KiB groups per wave
+    constexpr int LPS = A_GROUPS + B_GROUPS;   // loads per wave per stage
+    static_assert(6 * LPS < 64, "vmcnt is a 6-bit counter");
+    constexpr int STAGE = (BOC + BPIX) * 64;
+    extern __shared__ __attribute__((aligned(16))) int8_t ring[];
+
+    const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
+    const int t_tile = y % a.t_tiles, p_local = y / a.t_tiles;
+    const int p_tile = xcd * a.p_per_xcd + p_local;
+    if (p_local >= a.p_per_xcd || p_tile >= a.p_tiles) return;
+    const int pix0 = p_tile * BPIX, oc0 = t_tile * BOC;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int woc = wave % WOC, wpix = wave / WOC;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int batch = blockIdx.y;
+    const int oc_lane = oc0 + woc * 64 + 32 * h;
+    // DMA role of this lane inside a 16-row group: row lane>>2, logical chunk (lane&3) ^ ((lane>>4)&3)
+    const int dma_row = lane >> 2, dma_chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    // fragment reads: row l32 (+32 ob / pb), logical chunk 2*ks + h -> slot
+    const int swz = (l32 >> 2) & 3;
+    const int frag_off[2] = {l32 * 64 + ((0 + h) ^ swz) * 16, l32 * 64 + ((2 + h) ^ swz) * 16};
+
+    auto gemm = [&](const int8_t* in_base, int in_sn, int in_sh, int in_sw, int csh, int csw, int origin,
+                    const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk,
+                    v16i (&acc)[2][2]) {
+        const int8_t* a_ptr[A_GROUPS];
+        int32_t b_base[B_GROUPS];
+#pragma unroll
+        for (int i = 0; i < A_GROUPS; ++i) {
+            int row = (wave * A_GROUPS + i) * 16 + dma_row;
+            if (wgt_plain) {
+                const int j = row & 31;
+                row = (row & ~63) + 32 * ((j >> 2) & 1) + 16 * ((row >> 5) & 1) + 4 * (j >> 3) + (j & 3);
+            }
+            row = min(oc0 + row, wgt_rows - 1);
+            a_ptr[i] = wgt_base + static_cast<int64_t>(row) * wgt_ld + dma_chunk * 16;
+        }
+#pragma unroll
+        for (int i = 0; i < B_GROUPS; ++i) {
+            int m = pix0 + (wave * B_GROUPS + i) * 16 + dma_row;
+            m = m < a.M ? m : a.M - 1;
+            const PixelCoord p = decode_pixel(a, m);
+            b_base[i] = p.n * in_sn + p.oh * csh * in_sh + p.ow * csw * in_sw + origin;
+        }
+        auto issue = [&](int stage, int k) {
+            int8_t* sa = ring + stage * STAGE;
+            int8_t* sb = sa + BOC * 64;
+            const int4 ko = *reinterpret_cast<const int4*>(koff + 4 * k);   // uniform: scalar load
+            const int32_t off = dma_chunk == 0 ? ko.x : (dma_chunk == 1 ? ko.y : (dma_chunk == 2 ? ko.z : ko.w));
+#pragma unroll
+            for (int i = 0; i < A_GROUPS; ++i)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_ptr[i] + k * 64),
+                                                 (__attribute__((address_space(3))) void*)(sa + (wave * A_GROUPS + i) * 1024),
+                                                 16, 0, 0);
+#pragma unroll
+            for (int i = 0; i < B_GROUPS; ++i)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(in_base + (b_base[i] + off)),
+                                                 (__attribute__((address_space(3))) void*)(sb + (wave * B_GROUPS + i) * 1024),
+                                                 16, 0, 0);
+        };
+        const int ahead = min(stages - 1, nk);
+        for (int s0 = 0; s0 < ahead; ++s0) issue(s0, s0);
+        int rd = 0, wr = ahead % stages;
+        for (int k = 0; k < nk; ++k) {
+            // loads of steps k .. min(k + stages - 2, nk - 1) are outstanding; step k must have landed
+            const int younger = min(min(stages - 2, nk - 1 - k), 6);
+            wait_vmcnt_stages<LPS>(younger);
+            __builtin_amdgcn_s_barrier();
+            if (k + stages - 1 < nk) {
+                issue(wr, k + stages - 1);
+                wr = wr + 1 == stages ? 0 : wr + 1;
+            }
+            const int8_t* sa = ring + rd * STAGE + (woc * 64) * 64;
+            const int8_t* sb = ring + rd * STAGE + BOC * 64 + (wpix * 64) * 64;
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                v4i af[2], bf[2];
+#pragma unroll
+                for (int ob = 0; ob < 2; ++ob) af[ob] = *reinterpret_cast<const v4i*>(sa + ob * 32 * 64 + frag_off[ks]);
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb) bf[pb] = *reinterpret_cast<const v4i*>(sb + pb * 32 * 64 + frag_off[ks]);
+#pragma unroll
+                for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                    for (int pb = 0; pb < 2; ++pb)
+                        acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
+            }
+            rd = rd + 1 == stages ? 0 : rd + 1;
+        }
+        __builtin_amdgcn_s_barrier();   // every wave is done reading before the ring is refilled
+    };
+
+    v16i acc[2][2];
+    v16f rres[2][2];
+    constexpr bool kFused = F != kDyn && (F & CF_RES_GEMM);
+    if (kFused) {
+        ConvArgs a2 = a;
+        a2.corr = a.corr2;
+        init_acc(a2, oc_lane, acc);
+        gemm(a.in2, a.in2_sn, a.in2_sh, a.in2_sw, a.conv2_sh, a.conv2_sw, a.in2_origin, a.wgt2, a.Kp2, a.OCp, false,
+             a.koff2, a.nk2, acc);
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float4 b4 = ld4f(a.bias2 + oc_lane + 16 * ob + 4 * q);
+                const float4 s4 = ld4f(a.scale2 + oc_lane + 16 * ob + 4 * q);
+                const float bb[4] = {b4.x, b4.y, b4.z, b4.w}, ss[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float x = static_cast<float>(acc[ob][pb][4 * q + j]) + bb[j];
+                        rres[ob][pb][4 * q + j] = x * ss[j];
+                    }
+            }
+    }
+    init_acc(a, oc_lane, acc);
+    gemm(a.in + batch * a.batch_in, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
+         a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc);
+    const int m0 = pix0 + wpix * 64 + l32;
+    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres);
+}
+
+// ------------------------------------------------------------------------------------------------
 // Streaming kernel: grid (x, channel tiles of 64); a workgroup of 4 waves walks pixel tiles of 256
 // (64 per wave) with stride gridDim.x.  Dynamic LDS: 64 rows of (Kp + 16) weight bytes.
 template <uint32_t F>
@@ -260,6 +418,25 @@ void launch_tiled(const ConvArgs& a, hipStream_t s, int batches = 1) {
     hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, FLAGS>), grid, block, 0, s, a)
     HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_TILED, 0)
 #undef HIPIE_LAUNCH_TILED
+}
+
+template <int WOC, int WPIX>
+void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) {
+    const dim3 grid(8 * a.p_per_xcd * a.t_tiles, batches), block(WOC * WPIX * 64);
+    const size_t lds = static_cast<size_t>(stages) * (WOC + WPIX) * 64 * 64;
+    const uint32_t core = a.flags & ~CF_OUT_XOR;
+#define HIPIE_LAUNCH_PIPE(FLAGS, ...)                                                                       \
+    do {                                                                                                    \
+        static bool attr_set = false;                                                                       \
+        if (!attr_set) {                                                                                    \
+            HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_pipe_kernel<WOC, WPIX, FLAGS>), \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));   \
+            attr_set = true;                                                                                \
+        }                                                                                                   \
+        hipLaunchKernelGGL((conv_pipe_kernel<WOC, WPIX, FLAGS>), grid, block, lds, s, a, stages);           \
+    } while (0)
+    HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_PIPE, 0)
+#undef HIPIE_LAUNCH_PIPE
 }
 
 void launch_tiled_small(const ConvArgs& a, hipStream_t s) {   // 64 x 64 tile, one wave: generic epilogue only
@@ -406,7 +583,9 @@ struct hipie_conv {
     PackedGemm sg;
     DeviceBuffer s_bias, s_scale;
     bool depthwise = false;
-    int tile = 0;  // 0: tiled 128 ch x 128 px, 1: tiled 64 x 256, 2: tiled 64 x 64, 3: streaming (64 ch, weights in LDS)
+    int tile = 0;  // 0: tiled 128 ch x 128 px, 1: tiled 64 x 256, 2: tiled 64 x 64, 3: streaming (64 ch, weights
+                   // in LDS), 4: pipelined 128 x 128, 5: pipelined 64 x 256
+    int stages = 0;  // ring depth of the pipelined kernels (0 = choose from K)
     DeviceBuffer wgt, koff, corr;
     Epilogue epi;
 };
@@ -670,11 +849,19 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 3, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
-        if (c->fused || c->depthwise) return;   // one kernel only
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 5, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        if (c->depthwise) return;               // one kernel only
+        if (c->fused && tile != 0 && tile != 4) return;   // the second GEMM exists in the 128 x 128 kernels
         HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: K=%lld does not fit the streaming kernel's LDS", (long long)c->Kp);
         c->tile = tile;
+    });
+}
+
+int hipie_conv_set_stages(hipie_conv* c, int stages) {
+    return guarded([&] {
+        HIPIE_REQUIRE(c && stages >= 0 && stages <= 8, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_stages: %d", stages);
+        c->stages = stages;
     });
 }
 
@@ -804,14 +991,22 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
             HIPIE_CHECK_HIP(hipGetLastError());
             return;
         }
-        const int boc = c->tile == 0 ? 128 : 64;
-        const int bpix = c->tile == 0 ? 128 : (c->tile == 2 ? 64 : 256);
+        const int tile = c->tile;
+        const int boc = (tile == 0 || tile == 4) ? 128 : 64;
+        const int bpix = (tile == 0 || tile == 4) ? 128 : (tile == 2 ? 64 : 256);
         a.p_tiles = static_cast<int32_t>(ceil_div(M, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.oc, boc));
         a.p_per_xcd = static_cast<int32_t>(ceil_div(a.p_tiles, 8));
         DeviceGuard g(c->device);
         hipStream_t s = as_stream(stream);
-        switch (c->fused ? 0 : c->tile) {
+        // ring depth: enough K steps in flight to cover the load latency, within 160 KB of LDS
+        const int stage_bytes = (tile == 4 ? 256 : 320) * 64;
+        const int max_stages = std::min(8, (150 * 1024) / stage_bytes);   // at most 6 younger stages + current + refill
+        const int stages = c->stages > 0 ? std::min(c->stages, max_stages)
+                                         : std::max(2, std::min<int>(max_stages, std::min<int>(a.nk, a.nk2 > 0 ? std::max(a.nk, a.nk2) : a.nk) + 1));
+        switch (tile) {
+        case 4: launch_pipe<2, 2>(a, stages, s); break;
+        case 5: launch_pipe<1, 4>(a, stages, s); break;
         case 0: launch_tiled<2, 2>(a, s); break;
         case 1: launch_tiled<1, 4>(a, s); break;
         case 2: launch_tiled_small(a, s); break;

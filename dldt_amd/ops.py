@@ -179,8 +179,9 @@ class Convolution:
         check(lib().hipie_conv_out_dims(self._h, h, w, ctypes.byref(oh), ctypes.byref(ow)))
         return oh.value, ow.value
 
-    def set_tile(self, tile):
+    def set_tile(self, tile, stages=0):
         check(lib().hipie_conv_set_tile(self._h, tile))
+        check(lib().hipie_conv_set_stages(self._h, stages))
 
     def run(self, x, out, residual=None):
         xd, od = x.desc(), out.desc()

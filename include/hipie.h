@@ -196,9 +196,12 @@ int hipie_conv_create_fused(int device, const hipie_conv_desc* desc, const int8_
 void hipie_conv_destroy(hipie_conv* conv);
 /* output spatial dims for an input of h x w (convolution.hpp:168-183) */
 int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* oh, int32_t* ow);
-/* workgroup tile: 0 = 128 channels x 128 pixels, 1 = 64 x 256, 2 = 64 x 64 (chosen automatically
- * at creation; exposed for tuning and tests) */
+/* kernel variant: 0 = LDS-tiled 128 channels x 128 pixels, 1 = 64 x 256, 2 = 64 x 64, 3 = streaming
+ * (weights resident in LDS), 4 / 5 = 128 x 128 / 64 x 256 with a multi-stage direct-to-LDS K pipeline
+ * (chosen automatically; exposed for tuning and tests) */
 int hipie_conv_set_tile(hipie_conv* conv, int tile);
+/* ring depth (2..8 K steps in LDS) of the pipelined variants; 0 = choose from K */
+int hipie_conv_set_stages(hipie_conv* conv, int stages);
 int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,
                    const hipie_tensor* out, void* stream);
 

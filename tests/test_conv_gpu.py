@@ -39,7 +39,7 @@ def _device_in(x, g, signed=False):
     return DeviceTensor.from_nchw(x, I8 if signed else U8B, halo=halo, c_stride=cs)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("name", sorted(GEOMS))
 def test_conv_i32_accumulators_exact(orc, name, tile):
     import torch
