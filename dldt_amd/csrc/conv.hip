@@ -165,10 +165,14 @@ __device__ __forceinline__ void wait_vmcnt_stages(int younger) {
     }
 }
 
-template <int WOC, int WPIX, uint32_t F>
-__global__ __launch_bounds__(WOC* WPIX * 64, (F != kDyn && (F & CF_RES_GEMM)) ? 2 : 3)
+// KS = 2: eight waves; wave group g (four waves, own ring) multiplies the K steps k = g mod 2 and
+// group 1 hands its partial sums to group 0 through LDS.  Twice the waves per compute unit keep
+// twice the loads in flight, which is what bounds the layers with fewer tiles than compute units.
+template <int WOC, int WPIX, uint32_t F, int KS>
+__global__ __launch_bounds__(WOC* WPIX * 64 * KS, KS == 2 ? 1 : ((F != kDyn && (F & CF_RES_GEMM)) ? 2 : 3))
 void conv_pipe_kernel(const ConvArgs a, const int stages) {
-    constexpr int NT = WOC * WPIX * 64;
+    constexpr int NT = WOC * WPIX * 64;          // threads of one wave group
+    constexpr int NT_ALL = NT * KS;
     constexpr int BOC = WOC * 64, BPIX = WPIX * 64;
     constexpr int A_GROUPS = BOC / 16 / (NT / 64), B_GROUPS = BPIX / 16 / (NT / 64);   // 1 KiB groups per wave
     constexpr int LPS = A_GROUPS + B_GROUPS;   // loads per wave per stage
@@ -182,8 +186,10 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
     if (p_local >= a.p_per_xcd || p_tile >= a.p_tiles) return;
     const int pix0 = p_tile * BPIX, oc0 = t_tile * BOC;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int grp = KS == 1 ? 0 : (tid / NT), wave = (tid >> 6) % (NT / 64);
     const int woc = wave % WOC, wpix = wave / WOC;
+    int8_t* const gring = ring + grp * stages * STAGE;
     const int l32 = lane & 31, h = lane >> 5;
     const int batch = blockIdx.y;
     const int oc_lane = oc0 + woc * 64 + 32 * h;
@@ -194,8 +200,9 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
     const int frag_off[2] = {l32 * 64 + ((0 + h) ^ swz) * 16, l32 * 64 + ((2 + h) ^ swz) * 16};
 
     auto gemm = [&](const int8_t* in_base, int in_sn, int in_sh, int in_sw, int csh, int csw, int origin,
-                    const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk,
+                    const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk_all,
                     v16i (&acc)[2][2]) {
+        const int nk = nk_all / KS;   // steps of this wave group: local step j is global step j * KS + grp
         const int8_t* a_ptr[A_GROUPS];
         int32_t b_base[B_GROUPS];
 #pragma unroll
@@ -215,11 +222,18 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
             const PixelCoord p = decode_pixel(a, m);
             b_base[i] = p.n * in_sn + p.oh * csh * in_sh + p.ow * csw * in_sw + origin;
         }
-        auto issue = [&](int stage, int k) {
-            int8_t* sa = ring + stage * STAGE;
+        // The K-offset table lives in LDS behind the ring: a vector-memory load of it would have to
+        // be awaited with vmcnt(0), which drains every DMA load in flight and serialises the ring.
+        int32_t* kt = reinterpret_cast<int32_t*>(ring + KS * stages * STAGE);
+        for (int i = tid; i < 4 * nk_all; i += NT_ALL) kt[i] = koff[i];
+        __syncthreads();
+        int32_t off_next = kt[4 * grp + dma_chunk];
+        auto issue = [&](int stage, int j) {
+            int8_t* sa = gring + stage * STAGE;
             int8_t* sb = sa + BOC * 64;
-            const int4 ko = *reinterpret_cast<const int4*>(koff + 4 * k);   // uniform: scalar load
-            const int32_t off = dma_chunk == 0 ? ko.x : (dma_chunk == 1 ? ko.y : (dma_chunk == 2 ? ko.z : ko.w));
+            const int k = j * KS + grp;
+            const int32_t off = off_next;
+            off_next = kt[4 * (min(j + 1, nk - 1) * KS + grp) + dma_chunk];   // steps are issued in order
 #pragma unroll
             for (int i = 0; i < A_GROUPS; ++i)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_ptr[i] + k * 64),
@@ -231,34 +245,51 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
                                                  (__attribute__((address_space(3))) void*)(sb + (wave * B_GROUPS + i) * 1024),
                                                  16, 0, 0);
         };
+        // Software pipeline (stages >= 3).  Iteration k multiplies step k in two halves of 32 K
+        // bytes; the fragments of each half are read from LDS while the other half is in the matrix
+        // pipe, and the barrier sits between the halves:
+        //   read (k, half 1) | mfma (k, half 0) | wait own loads of step k+1, barrier |
+        //   refill the slot of step k-1 with step k+stages-1 | read (k+1, half 0) | mfma (k, half 1)
+        // After barrier k every wave's part of step k+1 has landed and every wave has consumed
+        // step k-1, whose slot is the one refilled.
         const int ahead = min(stages - 1, nk);
         for (int s0 = 0; s0 < ahead; ++s0) issue(s0, s0);
+        wait_vmcnt_stages<LPS>(min(ahead - 1, 6));
+        __builtin_amdgcn_s_barrier();
         int rd = 0, wr = ahead % stages;
+        v4i fa[2][2], fb[2][2];
+        auto read_frags = [&](int slot, int ks, v4i (&af)[2], v4i (&bf)[2]) {
+            const int8_t* sa = gring + slot * STAGE + (woc * 64) * 64;
+            const int8_t* sb = gring + slot * STAGE + BOC * 64 + (wpix * 64) * 64;
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob) af[ob] = *reinterpret_cast<const v4i*>(sa + ob * 32 * 64 + frag_off[ks]);
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) bf[pb] = *reinterpret_cast<const v4i*>(sb + pb * 32 * 64 + frag_off[ks]);
+        };
+        auto mfma4 = [&](const v4i (&af)[2], const v4i (&bf)[2]) {
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+                    acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
+        };
+        read_frags(0, 0, fa[0], fb[0]);
         for (int k = 0; k < nk; ++k) {
-            // loads of steps k .. min(k + stages - 2, nk - 1) are outstanding; step k must have landed
-            const int younger = min(min(stages - 2, nk - 1 - k), 6);
-            wait_vmcnt_stages<LPS>(younger);
-            __builtin_amdgcn_s_barrier();
-            if (k + stages - 1 < nk) {
-                issue(wr, k + stages - 1);
-                wr = wr + 1 == stages ? 0 : wr + 1;
+            read_frags(rd, 1, fa[1], fb[1]);
+            mfma4(fa[0], fb[0]);
+            const int nrd = rd + 1 == stages ? 0 : rd + 1;
+            if (k + 1 < nk) {
+                // outstanding: steps k+1 .. min(k + stages - 2, nk - 1)
+                wait_vmcnt_stages<LPS>(min(min(stages - 3, nk - 2 - k), 6));
+                __builtin_amdgcn_s_barrier();
+                if (k + stages - 1 < nk) {
+                    issue(wr, k + stages - 1);
+                    wr = wr + 1 == stages ? 0 : wr + 1;
+                }
+                read_frags(nrd, 0, fa[0], fb[0]);
             }
-            const int8_t* sa = ring + rd * STAGE + (woc * 64) * 64;
-            const int8_t* sb = ring + rd * STAGE + BOC * 64 + (wpix * 64) * 64;
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                v4i af[2], bf[2];
-#pragma unroll
-                for (int ob = 0; ob < 2; ++ob) af[ob] = *reinterpret_cast<const v4i*>(sa + ob * 32 * 64 + frag_off[ks]);
-#pragma unroll
-                for (int pb = 0; pb < 2; ++pb) bf[pb] = *reinterpret_cast<const v4i*>(sb + pb * 32 * 64 + frag_off[ks]);
-#pragma unroll
-                for (int ob = 0; ob < 2; ++ob)
-#pragma unroll
-                    for (int pb = 0; pb < 2; ++pb)
-                        acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
-            }
-            rd = rd + 1 == stages ? 0 : rd + 1;
+            mfma4(fa[1], fb[1]);
+            rd = nrd;
         }
         __builtin_amdgcn_s_barrier();   // every wave is done reading before the ring is refilled
     };
@@ -288,9 +319,39 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
                     }
             }
     }
-    init_acc(a, oc_lane, acc);
+    if (grp == 0) {
+        init_acc(a, oc_lane, acc);
+    } else {
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[ob][pb][r] = 0;
+    }
     gemm(a.in + batch * a.batch_in, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
          a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc);
+    if (KS == 2) {
+        // partial sums of group 1 -> LDS (register r of thread t at dword r * NT + t), added by group 0
+        int32_t* red = reinterpret_cast<int32_t*>(ring);
+        const int t = tid % NT;
+        if (grp == 1) {
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) red[((ob * 2 + pb) * 16 + r) * NT + t] = acc[ob][pb][r];
+        }
+        __syncthreads();
+        if (grp == 1) return;
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[ob][pb][r] += red[((ob * 2 + pb) * 16 + r) * NT + t];
+    }
     const int m0 = pix0 + wpix * 64 + l32;
     run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres);
 }
@@ -420,20 +481,20 @@ void launch_tiled(const ConvArgs& a, hipStream_t s, int batches = 1) {
 #undef HIPIE_LAUNCH_TILED
 }
 
-template <int WOC, int WPIX>
+template <int WOC, int WPIX, int KS>
 void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) {
-    const dim3 grid(8 * a.p_per_xcd * a.t_tiles, batches), block(WOC * WPIX * 64);
-    const size_t lds = static_cast<size_t>(stages) * (WOC + WPIX) * 64 * 64;
+    const dim3 grid(8 * a.p_per_xcd * a.t_tiles, batches), block(WOC * WPIX * 64 * KS);
+    const size_t lds = static_cast<size_t>(KS) * stages * (WOC + WPIX) * 64 * 64 + 16 * static_cast<size_t>(std::max(a.nk, a.nk2));
     const uint32_t core = a.flags & ~CF_OUT_XOR;
 #define HIPIE_LAUNCH_PIPE(FLAGS, ...)                                                                       \
     do {                                                                                                    \
         static bool attr_set = false;                                                                       \
         if (!attr_set) {                                                                                    \
-            HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_pipe_kernel<WOC, WPIX, FLAGS>), \
+            HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_pipe_kernel<WOC, WPIX, FLAGS, KS>), \
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));   \
             attr_set = true;                                                                                \
         }                                                                                                   \
-        hipLaunchKernelGGL((conv_pipe_kernel<WOC, WPIX, FLAGS>), grid, block, lds, s, a, stages);           \
+        hipLaunchKernelGGL((conv_pipe_kernel<WOC, WPIX, FLAGS, KS>), grid, block, lds, s, a, stages);       \
     } while (0)
     HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_PIPE, 0)
 #undef HIPIE_LAUNCH_PIPE
@@ -849,12 +910,21 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 5, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 7, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
         if (c->depthwise) return;               // one kernel only
         if (c->fused && tile != 0 && tile != 4) return;   // the second GEMM exists in the 128 x 128 kernels
+        HIPIE_REQUIRE(tile < 6 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_set_tile: the split-K kernels need an even number of 64-byte K steps (K=%lld)", (long long)c->Kp);
         HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: K=%lld does not fit the streaming kernel's LDS", (long long)c->Kp);
         c->tile = tile;
+    });
+}
+
+int hipie_conv_get_tile(const hipie_conv* c, int* tile) {
+    return guarded([&] {
+        HIPIE_REQUIRE(c && tile, HIPIE_PARAMETER_MISMATCH, "hipie_conv_get_tile: null argument");
+        *tile = c->depthwise ? -1 : c->tile;
     });
 }
 
@@ -992,21 +1062,23 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
             return;
         }
         const int tile = c->tile;
-        const int boc = (tile == 0 || tile == 4) ? 128 : 64;
-        const int bpix = (tile == 0 || tile == 4) ? 128 : (tile == 2 ? 64 : 256);
+        const bool square = tile == 0 || tile == 4 || tile == 6;
+        const int boc = square ? 128 : 64;
+        const int bpix = square ? 128 : (tile == 2 ? 64 : 256);
         a.p_tiles = static_cast<int32_t>(ceil_div(M, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.oc, boc));
         a.p_per_xcd = static_cast<int32_t>(ceil_div(a.p_tiles, 8));
         DeviceGuard g(c->device);
         hipStream_t s = as_stream(stream);
         // ring depth: enough K steps in flight to cover the load latency, within 160 KB of LDS
-        const int stage_bytes = (tile == 4 ? 256 : 320) * 64;
-        const int max_stages = std::min(8, (150 * 1024) / stage_bytes);   // at most 6 younger stages + current + refill
-        const int stages = c->stages > 0 ? std::min(c->stages, max_stages)
-                                         : std::max(2, std::min<int>(max_stages, std::min<int>(a.nk, a.nk2 > 0 ? std::max(a.nk, a.nk2) : a.nk) + 1));
+        const int stage_bytes = (square ? 256 : 320) * 64 * (tile >= 6 ? 2 : 1);
+        const int max_stages = std::min(8, (144 * 1024) / stage_bytes);   // at most 6 younger stages + current + refill
+        const int stages = c->stages > 0 ? std::max(3, std::min(c->stages, max_stages)) : (tile == 4 ? 4 : 3);
         switch (tile) {
-        case 4: launch_pipe<2, 2>(a, stages, s); break;
-        case 5: launch_pipe<1, 4>(a, stages, s); break;
+        case 4: launch_pipe<2, 2, 1>(a, stages, s); break;
+        case 5: launch_pipe<1, 4, 1>(a, stages, s); break;
+        case 6: launch_pipe<2, 2, 2>(a, stages, s); break;
+        case 7: launch_pipe<1, 4, 2>(a, stages, s); break;
         case 0: launch_tiled<2, 2>(a, s); break;
         case 1: launch_tiled<1, 4>(a, s); break;
         case 2: launch_tiled_small(a, s); break;

@@ -81,6 +81,8 @@ struct Step {
     virtual void create(int device, const std::vector<TensorInfo>& tensors) = 0;
     virtual void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs,
                      void* const* outputs, hipStream_t s) const = 0;
+    // pick the fastest kernel variant by timing it on a scratch arena (load time, optional)
+    virtual void tune(uint8_t*, const std::vector<TensorInfo>&, hipStream_t) {}
 };
 
 void check_status(int st, const char* what) {
@@ -162,6 +164,50 @@ struct ConvStep : Step {
             if (res >= 0) r = tensors[res].desc(arena);
         }
         check_status(hipie_conv_run(conv, &i, (fused || res >= 0) ? &r : nullptr, &o, s), name.c_str());
+    }
+    // Every variant computes the same integers, so the choice changes time only.  Variants a layer
+    // cannot use are refused by hipie_conv_set_tile and skipped.
+    void tune(uint8_t* arena, const std::vector<TensorInfo>& tensors, hipStream_t s) override {
+        if (shortcut && !fused) shortcut->tune(arena, tensors, s);
+        int current = -1;
+        check_status(hipie_conv_get_tile(conv, &current), name.c_str());
+        if (current < 0) return;   // depthwise: one kernel
+        const hipie_tensor i = tensors[in].desc(arena), o = tensors[out].desc(arena);
+        hipie_tensor r{};
+        if (fused) r = tensors[shortcut->in].desc(arena);
+        else if (res >= 0) r = tensors[res].desc(arena);
+        const hipie_tensor* rp = (fused || res >= 0) ? &r : nullptr;
+        hipEvent_t e0, e1;
+        HIPIE_CHECK_HIP(hipEventCreate(&e0));
+        HIPIE_CHECK_HIP(hipEventCreate(&e1));
+        int best = current;
+        float best_ms = 0.f;
+        const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7};
+        for (size_t c = 0; c < sizeof(candidates) / sizeof(candidates[0]); ++c) {
+            const int tile = candidates[c];
+            if (c > 0 && tile == current) continue;
+            if (hipie_conv_set_tile(conv, tile) != HIPIE_OK) continue;
+            int applied = -1;
+            check_status(hipie_conv_get_tile(conv, &applied), name.c_str());
+            if (applied != tile) continue;   // not available for this layer (kept its previous variant)
+            for (int w = 0; w < 2; ++w) check_status(hipie_conv_run(conv, &i, rp, &o, s), name.c_str());
+            HIPIE_CHECK_HIP(hipEventRecord(e0, s));
+            for (int w = 0; w < 5; ++w) check_status(hipie_conv_run(conv, &i, rp, &o, s), name.c_str());
+            HIPIE_CHECK_HIP(hipEventRecord(e1, s));
+            HIPIE_CHECK_HIP(hipEventSynchronize(e1));
+            float ms = 0.f;
+            HIPIE_CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+            if (c == 0 || ms < best_ms) {
+                best_ms = ms;
+                best = tile;
+            }
+        }
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        check_status(hipie_conv_set_tile(conv, best), name.c_str());
+        if (std::getenv("HIPIE_TUNE_LOG"))
+            std::fprintf(stderr, "hipie tune: %-28s variant %d (%.1f us; default %d)\n", name.c_str(), best,
+                         best_ms * 200.f, current);
     }
 };
 
@@ -754,6 +800,18 @@ int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
             const GNode& n = g->nodes[r];
             const int dt = n.dtype == HIPIE_F32 ? HIPIE_F32 : HIPIE_U8;
             plan->outputs.push_back({n.name, dt, n.shape, n.numel() * (dt == HIPIE_F32 ? 4 : 1)});
+        }
+        // kernel selection by measurement on a scratch request (HIPIE_TUNE=0 keeps the shape-based defaults)
+        const char* tune_env = std::getenv("HIPIE_TUNE");
+        if (device >= 0 && !(tune_env && tune_env[0] == '0')) {
+            hipie_request* scratch = nullptr;
+            check_status(hipie_request_create(plan.get(), 0, &scratch), "hipie_compile: tuning request");
+            struct Release {
+                hipie_request* r;
+                ~Release() { hipie_request_destroy(r); }
+            } release{scratch};
+            DeviceGuard dg(device);
+            for (auto& s : plan->steps) s->tune(scratch->arena.as<uint8_t>(), plan->tensors, scratch->stream);
         }
         *out = plan.release();
     });

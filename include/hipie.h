@@ -197,9 +197,13 @@ void hipie_conv_destroy(hipie_conv* conv);
 /* output spatial dims for an input of h x w (convolution.hpp:168-183) */
 int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* oh, int32_t* ow);
 /* kernel variant: 0 = LDS-tiled 128 channels x 128 pixels, 1 = 64 x 256, 2 = 64 x 64, 3 = streaming
- * (weights resident in LDS), 4 / 5 = 128 x 128 / 64 x 256 with a multi-stage direct-to-LDS K pipeline
- * (chosen automatically; exposed for tuning and tests) */
+ * (weights resident in LDS), 4 / 5 = 128 x 128 / 64 x 256 with a multi-stage direct-to-LDS K pipeline,
+ * 6 / 7 = the same two with eight waves that split the K steps between two wave groups (for layers
+ * with fewer tiles than compute units; needs an even number of 64-byte K steps).  A default is chosen
+ * from the shape; hipie_compile times the variants on the device and keeps the fastest.  Every
+ * variant produces the same bits. */
 int hipie_conv_set_tile(hipie_conv* conv, int tile);
+int hipie_conv_get_tile(const hipie_conv* conv, int* tile);
 /* ring depth (2..8 K steps in LDS) of the pipelined variants; 0 = choose from K */
 int hipie_conv_set_stages(hipie_conv* conv, int stages);
 int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,

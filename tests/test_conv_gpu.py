@@ -1,5 +1,7 @@
 """Convolution on int8 MFMA through the C ABI vs the oracle: exact i32 accumulators and
 bit-exact fused epilogues (bias, dequant scale, residual add, ReLU/Clamp, per-channel FQ)."""
+import zlib
+
 import numpy as np
 import pytest
 
@@ -39,18 +41,22 @@ def _device_in(x, g, signed=False):
     return DeviceTensor.from_nchw(x, I8 if signed else U8B, halo=halo, c_stride=cs)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("name", sorted(GEOMS))
 def test_conv_i32_accumulators_exact(orc, name, tile):
     import torch
-    from dldt_amd import Convolution, DeviceTensor
+    from dldt_amd import Convolution, DeviceTensor, HipieError
     g = GEOMS[name]
-    rng = np.random.default_rng(abs(hash(name)) % 1000)
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
     x, w = _inputs(rng, g)
     want = orc.convolution(x, w, g[7], g[8], g[9], g[10])
     xin = _device_in(x, g)
     conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10])
-    conv.set_tile(tile)
+    try:
+        conv.set_tile(tile)
+    except HipieError as e:       # the split-K variants need an even number of K steps
+        assert tile >= 6 and e.status == -4
+        pytest.skip(str(e))
     out = DeviceTensor(want.shape[0], want.shape[2], want.shape[3], want.shape[1], I32)
     conv.run(xin, out)
     torch.cuda.synchronize()
