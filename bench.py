@@ -16,6 +16,10 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 INT8_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per convolution/FC launch at batch 64, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script (profiles/conv_kernels_resnet50_b64.md: 2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE, factors
+# calibrated on copies of known size in the same runs)
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH_B64 = 33.9e6
 
 
 def cpu_baseline(batch_images, budget_s=20.0):
@@ -113,8 +117,10 @@ def main():
         "tops": total_ops / (ms_per_step * 1e-3) / 1e12,
         "frac_int8_peak_whole_net": total_ops / (ms_per_step * 1e-3) / 1e12 / INT8_PEAK_TOPS,
         "roofline": {"bound": "mfma", "achieved": achieved_tops, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
-                     "frac": achieved_tops / INT8_PEAK_TOPS, "traffic": None,
-                     "kernel": "conv_mfma_kernel (all %d convolution/FC launches of one step)" % len(mfma),
+                     "frac": achieved_tops / INT8_PEAK_TOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH_B64 if args.batch == 64 else None,
+                     "algorithmic_bytes_per_launch": sum(s["bytes"] for s in mfma) / len(mfma),
+                     "kernel": "conv_tiled_kernel / conv_pipe_kernel / conv_stream_kernel (all %d convolution/FC launches of one step)" % len(mfma),
                      "ops_per_step": mfma_ops, "kernel_ms_per_step": mfma_ms,
                      "avg_launch_us": mfma_ms * 1e3 / len(mfma), "note": "int8 TOP/s, dense peak 5.0 POP/s"},
         "other_kernels_ms_per_step": {t: sum(s["ms"] for s in steps if s["type"] == t)

@@ -83,6 +83,9 @@ struct Step {
                      void* const* outputs, hipStream_t s) const = 0;
     // pick the fastest kernel variant by timing it on a scratch arena (load time, optional)
     virtual void tune(uint8_t*, const std::vector<TensorInfo>&, hipStream_t) {}
+    // the chosen variant as an integer (-1: the step has no variants), and its inverse
+    virtual int variant() const { return -1; }
+    virtual void set_variant(int) {}
 };
 
 void check_status(int st, const char* what) {
@@ -114,6 +117,7 @@ struct ConvStep : Step {
     std::vector<int8_t> weights;   // OIHW
     EpilogueSpec epi;
     hipie_conv* conv = nullptr;
+    int64_t in_w_bytes = 0;        // input + weight bytes (what a fused consumer still has to read)
     // projection shortcut (Conv' -> Add -> Multiply, f32, used only by this step's residual Add):
     // run inside this step's kernel when the fused form applies, else right before it
     std::unique_ptr<ConvStep> shortcut;
@@ -164,6 +168,14 @@ struct ConvStep : Step {
             if (res >= 0) r = tensors[res].desc(arena);
         }
         check_status(hipie_conv_run(conv, &i, (fused || res >= 0) ? &r : nullptr, &o, s), name.c_str());
+    }
+    int variant() const override {
+        int t = -1;
+        if (conv) (void)hipie_conv_get_tile(conv, &t);
+        return t;
+    }
+    void set_variant(int v) override {
+        if (conv && v >= 0) check_status(hipie_conv_set_tile(conv, v), name.c_str());
     }
     // Every variant computes the same integers, so the choice changes time only.  Variants a layer
     // cannot use are refused by hipie_conv_set_tile and skipped.
@@ -604,7 +616,16 @@ struct Planner {
         st->name = N(cur).name;
         st->type = is_mm ? "MatMul" : (d.groups > 1 ? "GroupConvolution" : "Convolution");
         st->macs = N(id).numel() * (d.groups > 1 ? 1 : IC) * d.kh * d.kw + (st->shortcut ? st->shortcut->macs : 0);
-        st->bytes = 0;
+        // algorithmic HBM bytes: every operand once (input, weights, output, residual); a fused
+        // projection shortcut adds its input and weights and removes the f32 residual round trip
+        auto elems = [&](int t) {
+            const TensorInfo& ti = tensors[t];
+            return static_cast<int64_t>(ti.n) * ti.h * ti.w * ti.c * ti.esize();
+        };
+        st->in_w_bytes = elems(st->in) + static_cast<int64_t>(OC) * (d.groups > 1 ? 1 : IC) * d.kh * d.kw;
+        st->bytes = st->in_w_bytes + elems(st->out);
+        if (st->shortcut) st->bytes += st->shortcut->in_w_bytes;
+        else if (st->res >= 0) st->bytes += elems(st->res);
         st->out_node = cur;
         values[cur].kind = VK_TENSOR;
         values[cur].tensor = st->out;
@@ -801,17 +822,51 @@ int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
             const int dt = n.dtype == HIPIE_F32 ? HIPIE_F32 : HIPIE_U8;
             plan->outputs.push_back({n.name, dt, n.shape, n.numel() * (dt == HIPIE_F32 ? 4 : 1)});
         }
-        // kernel selection by measurement on a scratch request (HIPIE_TUNE=0 keeps the shape-based defaults)
+        // Kernel selection by measurement on a scratch request (HIPIE_TUNE=0 keeps the shape-based
+        // defaults).  HIPIE_TUNE_FILE names a cache of the choices, one "step variant" pair a line:
+        // read when it matches this plan, written after tuning otherwise (the reference's GPU plugin
+        // keeps its tuning results in a file the same way, inference-engine/include/cldnn/cldnn_config.hpp:125 KEY_TUNING_FILE).
         const char* tune_env = std::getenv("HIPIE_TUNE");
         if (device >= 0 && !(tune_env && tune_env[0] == '0')) {
-            hipie_request* scratch = nullptr;
-            check_status(hipie_request_create(plan.get(), 0, &scratch), "hipie_compile: tuning request");
-            struct Release {
-                hipie_request* r;
-                ~Release() { hipie_request_destroy(r); }
-            } release{scratch};
-            DeviceGuard dg(device);
-            for (auto& s : plan->steps) s->tune(scratch->arena.as<uint8_t>(), plan->tensors, scratch->stream);
+            const char* cache = std::getenv("HIPIE_TUNE_FILE");
+            bool loaded = false;
+            if (cache) {
+                if (FILE* f = std::fopen(cache, "r")) {
+                    std::vector<int> v(plan->steps.size(), -2);
+                    size_t n = 0;
+                    int idx = 0, var = 0;
+                    while (std::fscanf(f, "%d %d", &idx, &var) == 2)
+                        if (idx >= 0 && static_cast<size_t>(idx) < v.size() && v[idx] == -2) {
+                            v[idx] = var;
+                            ++n;
+                        }
+                    std::fclose(f);
+                    bool match = n == v.size();
+                    for (size_t i = 0; match && i < v.size(); ++i)
+                        match = (v[i] < 0) == (plan->steps[i]->variant() < 0);
+                    if (match) {
+                        for (size_t i = 0; i < v.size(); ++i) plan->steps[i]->set_variant(v[i]);
+                        loaded = true;
+                    }
+                }
+            }
+            if (!loaded) {
+                hipie_request* scratch = nullptr;
+                check_status(hipie_request_create(plan.get(), 0, &scratch), "hipie_compile: tuning request");
+                struct Release {
+                    hipie_request* r;
+                    ~Release() { hipie_request_destroy(r); }
+                } release{scratch};
+                DeviceGuard dg(device);
+                for (auto& s : plan->steps) s->tune(scratch->arena.as<uint8_t>(), plan->tensors, scratch->stream);
+                if (cache) {
+                    if (FILE* f = std::fopen(cache, "w")) {
+                        for (size_t i = 0; i < plan->steps.size(); ++i)
+                            std::fprintf(f, "%zu %d\n", i, plan->steps[i]->variant());
+                        std::fclose(f);
+                    }
+                }
+            }
         }
         *out = plan.release();
     });
