@@ -14,7 +14,7 @@ struct Epilogue {
     uint32_t flags = 0;
     int out_dtype = HIPIE_F32;
     float lm1 = 0, out_off = 0, clamp_lo = 0, clamp_hi = 0;
-    DeviceBuffer bias, scale, res_sub, res_mul, post_scale, fq_il, fq_ih, fq_d, fq_r;
+    DeviceBuffer bias, scale, res_sub, res_mul, post_scale, fq_il, fq_ih, fq_d, fq_r, fq_r2;
     std::vector<float> host_bias;
     void build(int device, const hipie_epilogue& e, int64_t oc, int64_t ocp);
     void fill(ConvArgs& a) const;

@@ -1,5 +1,6 @@
 // Convolution / MatMul on int8 MFMA: kernel instantiations, load-time packing, launcher.
 #include "conv.h"
+#include "div2.h"
 #include "conv_epilogue.h"
 
 #include <cmath>
@@ -20,6 +21,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     constexpr int A_PIECES = BOC * 4 / NT, B_PIECES = BPIX * 4 / NT;
     __shared__ __attribute__((aligned(16))) int8_t sA[2][BOC * kRow];
     __shared__ __attribute__((aligned(16))) int8_t sB[2][BPIX * kRow];
+    __shared__ __attribute__((aligned(16))) float sP[PT_COUNT * BOC];
 
     // block -> (pixel tile, channel tile): consecutive pixel tiles stay on one XCD
     const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
@@ -34,6 +36,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     const int chunk = tid & 3;
 
     const int batch = blockIdx.y;
+    stage_params<F>(a, oc0, sP, BOC, tid, NT);   // visible after the first barrier of the K loop
     const int a_row[2] = {woc * 64 + l32, woc * 64 + 32 + l32};
     const int b_row[2] = {wpix * 64 + l32, wpix * 64 + 32 + l32};
     const int oc_lane = oc0 + woc * 64 + 32 * h;
@@ -134,7 +137,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     gemm(a.in + batch * a.batch_in, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
          a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc);
     const int m0 = pix0 + wpix * 64 + l32;
-    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres);
+    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, sP, BOC, oc0);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -198,6 +201,9 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
     // fragment reads: row l32 (+32 ob / pb), logical chunk 2*ks + h -> slot
     const int swz = (l32 >> 2) & 3;
     const int frag_off[2] = {l32 * 64 + ((0 + h) ^ swz) * 16, l32 * 64 + ((2 + h) ^ swz) * 16};
+    // epilogue tables behind the rings; visible after the barrier that follows the K-offset table fill
+    float* const sP = reinterpret_cast<float*>(ring + KS * stages * STAGE);
+    stage_params<F>(a, oc0, sP, BOC, tid, NT_ALL);
 
     auto gemm = [&](const int8_t* in_base, int in_sn, int in_sh, int in_sw, int csh, int csw, int origin,
                     const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk_all,
@@ -224,7 +230,7 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
         }
         // The K-offset table lives in LDS behind the ring: a vector-memory load of it would have to
         // be awaited with vmcnt(0), which drains every DMA load in flight and serialises the ring.
-        int32_t* kt = reinterpret_cast<int32_t*>(ring + KS * stages * STAGE);
+        int32_t* kt = reinterpret_cast<int32_t*>(ring + KS * stages * STAGE + PT_COUNT * BOC * 4);
         for (int i = tid; i < 4 * nk_all; i += NT_ALL) kt[i] = koff[i];
         __syncthreads();
         int32_t off_next = kt[4 * grp + dma_chunk];
@@ -353,14 +359,14 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
                 for (int r = 0; r < 16; ++r) acc[ob][pb][r] += red[((ob * 2 + pb) * 16 + r) * NT + t];
     }
     const int m0 = pix0 + wpix * 64 + l32;
-    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres);
+    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, sP, BOC, oc0);
 }
 
 // ------------------------------------------------------------------------------------------------
 // Streaming kernel: grid (x, channel tiles of 64); a workgroup of 4 waves walks pixel tiles of 256
 // (64 per wave) with stride gridDim.x.  Dynamic LDS: 64 rows of (Kp + 16) weight bytes.
 template <uint32_t F>
-__global__ __launch_bounds__(256, 3) void conv_stream_kernel(const ConvArgs a) {
+__global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
     extern __shared__ __attribute__((aligned(16))) int8_t sW[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, h = lane >> 5;
@@ -376,6 +382,8 @@ __global__ __launch_bounds__(256, 3) void conv_stream_kernel(const ConvArgs a) {
                 *reinterpret_cast<const v4i*>(src + static_cast<int64_t>(row) * a.Kp + pc * 16);
         }
     }
+    float* const sP = reinterpret_cast<float*>(sW + 64 * wrow);
+    stage_params<F>(a, oc0, sP, 64, tid, 256);
     const int oc_lane = oc0 + 32 * h;
     const int a_row[2] = {l32 * wrow + h * 16, (32 + l32) * wrow + h * 16};
 
@@ -446,7 +454,7 @@ __global__ __launch_bounds__(256, 3) void conv_stream_kernel(const ConvArgs a) {
         compute(cur, cur_k);
         if (cur_k + 1 == a.nk) {
             const int m0 = cur_tile * 256 + wave * 64 + l32;
-            run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32);
+            run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, 0, sP, 64, oc0);
             init_acc(a, oc_lane, acc);
         }
         return more;
@@ -468,6 +476,10 @@ __global__ __launch_bounds__(256, 3) void conv_stream_kernel(const ConvArgs a) {
     case E_F32: X(E_F32, __VA_ARGS__); break;                                                \
     case E_F32RELU: X(E_F32RELU, __VA_ARGS__); break;                                        \
     case E_CLAMPFQ: X(E_CLAMPFQ, __VA_ARGS__); break;                                        \
+    case E_PLAIN0 & ~CF_FQ_DIV2: X((E_PLAIN0 & ~CF_FQ_DIV2), __VA_ARGS__); break;            \
+    case E_RESU8 & ~CF_FQ_DIV2: X((E_RESU8 & ~CF_FQ_DIV2), __VA_ARGS__); break;              \
+    case E_RESGEMM & ~CF_FQ_DIV2: X((E_RESGEMM & ~CF_FQ_DIV2), __VA_ARGS__); break;          \
+    case E_CLAMPFQ & ~CF_FQ_DIV2: X((E_CLAMPFQ & ~CF_FQ_DIV2), __VA_ARGS__); break;          \
     default: X(kDyn, __VA_ARGS__); break;                                                    \
     }
 
@@ -484,7 +496,8 @@ void launch_tiled(const ConvArgs& a, hipStream_t s, int batches = 1) {
 template <int WOC, int WPIX, int KS>
 void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) {
     const dim3 grid(8 * a.p_per_xcd * a.t_tiles, batches), block(WOC * WPIX * 64 * KS);
-    const size_t lds = static_cast<size_t>(KS) * stages * (WOC + WPIX) * 64 * 64 + 16 * static_cast<size_t>(std::max(a.nk, a.nk2));
+    const size_t lds = static_cast<size_t>(KS) * stages * (WOC + WPIX) * 64 * 64 + PT_COUNT * WOC * 64 * 4 +
+                       16 * static_cast<size_t>(std::max(a.nk, a.nk2));
     const uint32_t core = a.flags & ~CF_OUT_XOR;
 #define HIPIE_LAUNCH_PIPE(FLAGS, ...)                                                                       \
     do {                                                                                                    \
@@ -506,7 +519,7 @@ void launch_tiled_small(const ConvArgs& a, hipStream_t s) {   // 64 x 64 tile, o
 
 void launch_stream(const ConvArgs& a, int grid_x, hipStream_t s) {
     const dim3 grid(grid_x, a.t_tiles), block(256);
-    const size_t lds = static_cast<size_t>(64) * (a.Kp + 16);
+    const size_t lds = static_cast<size_t>(64) * (a.Kp + 16) + PT_COUNT * 64 * 4;
     const uint32_t core = a.flags & ~CF_OUT_XOR;
 #define HIPIE_LAUNCH_STREAM(FLAGS, ...) \
     hipLaunchKernelGGL((conv_stream_kernel<FLAGS>), grid, block, lds, s, a)
@@ -595,6 +608,14 @@ void Epilogue::build(int device_, const hipie_epilogue& e, int64_t oc, int64_t o
         up(fq_il, il); up(fq_ih, ih); up(fq_d, d); up(fq_r, r);
         flags |= CF_OUT_FQ;
         if (exact) flags |= CF_FQ_RCP;
+        std::vector<float> zh, zl;
+        if (exact && device < 0) {
+            flags |= CF_FQ_DIV2;   // dry run: nothing executes, plan as if the constants verify
+        } else if (exact && fq_div2_constants(device, d, zh, zl)) {
+            up(fq_r, zh);
+            up(fq_r2, zl);
+            flags |= CF_FQ_DIV2;
+        }
         bool il0 = true;
         for (int64_t c = 0; c < ocp; ++c) il0 = il0 && il[c] == 0.0f && !std::signbit(il[c]);
         if (il0) flags |= CF_FQ_IL0;
@@ -610,7 +631,7 @@ void Epilogue::fill(ConvArgs& a) const {
     a.res_sub = res_sub.as<float>(); a.res_mul = res_mul.as<float>();
     a.post_scale = post_scale.as<float>();
     a.fq_il = fq_il.as<float>(); a.fq_ih = fq_ih.as<float>();
-    a.fq_d = fq_d.as<float>(); a.fq_r = fq_r.as<float>();
+    a.fq_d = fq_d.as<float>(); a.fq_r = fq_r.as<float>(); a.fq_r2 = fq_r2.as<float>();
     a.flags = flags; a.lm1 = lm1; a.out_off = out_off; a.clamp_lo = clamp_lo; a.clamp_hi = clamp_hi;
 }
 
@@ -887,7 +908,7 @@ int hipie_conv_create_fused(int device, const hipie_conv_desc* desc, const int8_
         const int st = hipie_conv_create(device, desc, weights, epilogue, &c);
         if (st != HIPIE_OK) fail(static_cast<hipie_status>(st), "%s", hipie_last_error());
         std::unique_ptr<hipie_conv> guard(c);
-        HIPIE_REQUIRE((c->epi.flags & ~CF_OUT_XOR) == E_RESGEMM, HIPIE_NOT_IMPLEMENTED,
+        HIPIE_REQUIRE((c->epi.flags & ~(CF_OUT_XOR | CF_FQ_DIV2)) == (E_RESGEMM & ~CF_FQ_DIV2), HIPIE_NOT_IMPLEMENTED,
                       "hipie_conv_create_fused: the fused form needs bias, scale, FakeQuantize with input_low 0");
         c->fused = true;
         c->sd = sd;
@@ -915,7 +936,7 @@ int hipie_conv_set_tile(hipie_conv* c, int tile) {
         if (c->fused && tile != 0 && tile != 4) return;   // the second GEMM exists in the 128 x 128 kernels
         HIPIE_REQUIRE(tile < 6 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the split-K kernels need an even number of 64-byte K steps (K=%lld)", (long long)c->Kp);
-        HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
+        HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) + PT_COUNT * 64 * 4 <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: K=%lld does not fit the streaming kernel's LDS", (long long)c->Kp);
         c->tile = tile;
     });
@@ -1085,7 +1106,7 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         default: {
             // persistent workgroups: as many as fit per CU by LDS (at most 4), spread over the
             // channel tiles; a multiple of 8 so that sibling channel tiles share an XCD
-            const int64_t lds = 64 * (c->Kp + 16);
+            const int64_t lds = 64 * (c->Kp + 16) + PT_COUNT * 64 * 4;
             const int per_cu = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(4, (160 * 1024) / lds)));
             int64_t gx = std::max<int64_t>(8, (256 * per_cu) / a.t_tiles);
             gx = std::min<int64_t>(round_up(gx, 8), round_up(a.p_tiles, 8));

@@ -51,12 +51,16 @@ __device__ __forceinline__ void init_acc(const ConvArgs& a, int oc_lane, v16i (&
 }
 
 // level index of one value; the clamp folds both saturating branches of the reference
-template <bool RCP, bool IL0>
-__device__ __forceinline__ float fq_level_fast(float x, float il, float ih, float d, float r, float lm1) {
+// MODE 0: IEEE division, 1: reciprocal with two correction rounds, 2: fma(n, r, n * r2)
+template <int MODE, bool IL0>
+__device__ __forceinline__ float fq_level_fast(float x, float il, float ih, float d, float r, float r2, float lm1) {
     const float xc = __builtin_amdgcn_fmed3f(x, il, ih);
     const float n = IL0 ? xc : xc - il;
     float q;
-    if (RCP) {
+    if (MODE == 2) {
+        const float lo = n * r2;
+        q = fmaf(n, r, lo);
+    } else if (MODE == 1) {
         const float q0 = n * r;
         const float e0 = fmaf(-d, q0, n);
         const float q1 = fmaf(e0, r, q0);
@@ -81,17 +85,46 @@ __device__ __forceinline__ uint32_t add_bytes(uint32_t a, uint32_t b) {
 // with an empty asm: otherwise the compiler sinks the arithmetic into the store predicates and
 // hoists every table load of the epilogue to its top, which costs an occupancy step.
 constexpr uint32_t kDyn = 0xffffffffu;
-constexpr uint32_t E_PLAIN0 = CF_BIAS | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
-constexpr uint32_t E_PLAIN = CF_BIAS | CF_OUT_FQ | CF_FQ_RCP;
-constexpr uint32_t E_RESU8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_U8B | CF_RES_MUL | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
-constexpr uint32_t E_RESF32 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32 | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
-constexpr uint32_t E_RESGEMM = CF_BIAS | CF_SCALE | CF_RES | CF_RES_GEMM | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
+constexpr uint32_t E_FQ = CF_OUT_FQ | CF_FQ_RCP | CF_FQ_DIV2;   // the division every verified layer uses
+constexpr uint32_t E_PLAIN0 = CF_BIAS | E_FQ | CF_FQ_IL0;
+constexpr uint32_t E_PLAIN = CF_BIAS | E_FQ;
+constexpr uint32_t E_RESU8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_U8B | CF_RES_MUL | E_FQ | CF_FQ_IL0;
+constexpr uint32_t E_RESF32 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32 | E_FQ | CF_FQ_IL0;
+constexpr uint32_t E_RESGEMM = CF_BIAS | CF_SCALE | CF_RES | CF_RES_GEMM | E_FQ | CF_FQ_IL0;
 constexpr uint32_t E_F32 = CF_BIAS | CF_SCALE;
 constexpr uint32_t E_F32RELU = CF_BIAS | CF_SCALE | CF_RELU;
-constexpr uint32_t E_CLAMPFQ = CF_BIAS | CF_SCALE | CF_CLAMP | CF_OUT_FQ | CF_FQ_RCP | CF_FQ_IL0;
+constexpr uint32_t E_CLAMPFQ = CF_BIAS | CF_SCALE | CF_CLAMP | E_FQ | CF_FQ_IL0;
+
+// Per-channel tables of the epilogue staged in LDS, one row of `stride` floats per table.  Every
+// lane of a half-wave needs the same four channels at a time: read from global memory that is a
+// 64-lane vector load whose address processing costs as much as a real gather (the convolution
+// kernels spent most of their texture-addresser cycles there); read from LDS it is a broadcast.
+enum ParamTable { PT_BIAS, PT_SCALE, PT_RSUB, PT_RMUL, PT_POST, PT_IL, PT_IH, PT_D, PT_R, PT_R2, PT_COUNT };
+
+template <uint32_t F>
+__device__ __forceinline__ void stage_params(const ConvArgs& a, int oc0, float* sp, int stride, int tid, int nt) {
+    const uint32_t fl = F == kDyn ? a.flags : F;
+    auto put = [&](int t, const float* src) {
+        for (int c = tid; c < stride; c += nt) sp[t * stride + c] = src[oc0 + c];
+    };
+    if (fl & CF_BIAS) put(PT_BIAS, a.bias);
+    if (fl & CF_SCALE) put(PT_SCALE, a.scale);
+    if (fl & CF_RES_SUB) put(PT_RSUB, a.res_sub);
+    if (fl & CF_RES_MUL) put(PT_RMUL, a.res_mul);
+    if (fl & CF_POST_SCALE) put(PT_POST, a.post_scale);
+    if (fl & CF_OUT_FQ) {
+        put(PT_IH, a.fq_ih);
+        if (fl & CF_FQ_RCP) put(PT_R, a.fq_r);
+        if (fl & CF_FQ_DIV2) put(PT_R2, a.fq_r2);
+        if (!(fl & CF_FQ_IL0)) {
+            put(PT_IL, a.fq_il);
+            put(PT_D, a.fq_d);
+        }
+    }
+}
 
 struct EpiParams {
-    float4 bias, scale, rsub, rmul, post, il, ih, d, r;
+    float4 bias, scale, rsub, rmul, post, il, ih, d, r, r2;
     float4 res[2];   // f32 residual of the two pixels
 };
 
@@ -104,11 +137,17 @@ __device__ __forceinline__ void f4_to_array(const float4& v, float (&o)[4]) {
     o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
 }
 
+// sp: the tile's staged tables (stage_params) with local channel 0 = channel oc0, or nullptr to
+// read the tables from global memory
 template <uint32_t F>
 __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                          const bool (&valid)[2], const int64_t (&out_off)[2],
-                                         const int64_t (&res_off)[2], const v16f (&rres)[2][2]) {
+                                         const int64_t (&res_off)[2], const v16f (&rres)[2][2],
+                                         const float* sp, int sp_stride, int oc0) {
     const uint32_t fl = F == kDyn ? a.flags : F;
+    auto tab = [&](int t, const float* g, int oc) {
+        return sp ? *reinterpret_cast<const float4*>(sp + t * sp_stride + (oc - oc0)) : ld4f(g + oc);
+    };
     const int out_cs = a.out_sw;
 
     if (fl & CF_OUT_I32) {   // raw accumulators
@@ -143,17 +182,18 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
 
     auto load = [&](int e4, EpiParams& p) {
         const int oc = oc_lane + 4 * e4;
-        if (fl & CF_BIAS) p.bias = ld4f(a.bias + oc);
-        if (fl & CF_SCALE) p.scale = ld4f(a.scale + oc);
-        if (fl & CF_RES_SUB) p.rsub = ld4f(a.res_sub + oc);
-        if (fl & CF_RES_MUL) p.rmul = ld4f(a.res_mul + oc);
-        if (fl & CF_POST_SCALE) p.post = ld4f(a.post_scale + oc);
+        if (fl & CF_BIAS) p.bias = tab(PT_BIAS, a.bias, oc);
+        if (fl & CF_SCALE) p.scale = tab(PT_SCALE, a.scale, oc);
+        if (fl & CF_RES_SUB) p.rsub = tab(PT_RSUB, a.res_sub, oc);
+        if (fl & CF_RES_MUL) p.rmul = tab(PT_RMUL, a.res_mul, oc);
+        if (fl & CF_POST_SCALE) p.post = tab(PT_POST, a.post_scale, oc);
         if (fl & CF_OUT_FQ) {
-            p.ih = ld4f(a.fq_ih + oc);
-            if (fl & CF_FQ_RCP) p.r = ld4f(a.fq_r + oc);
+            p.ih = tab(PT_IH, a.fq_ih, oc);
+            if (fl & CF_FQ_RCP) p.r = tab(PT_R, a.fq_r, oc);
+            if (fl & CF_FQ_DIV2) p.r2 = tab(PT_R2, a.fq_r2, oc);
             if (!(fl & CF_FQ_IL0)) {
-                p.il = ld4f(a.fq_il + oc);
-                p.d = ld4f(a.fq_d + oc);
+                p.il = tab(PT_IL, a.fq_il, oc);
+                p.d = tab(PT_D, a.fq_d, oc);
             }
         }
         if ((fl & CF_RES) && (fl & CF_RES_F32)) {
@@ -173,7 +213,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
     for (int e4 = 0; e4 < 8; ++e4) {
         if (e4 + 1 < 8) load(e4 + 1, nxt);
         const int ob = e4 >> 2, r0 = (e4 & 3) * 4;
-        float bias_[4], scale_[4], rsub_[4], rmul_[4], post_[4], il_[4], ih_[4], d_[4], rr_[4];
+        float bias_[4], scale_[4], rsub_[4], rmul_[4], post_[4], il_[4], ih_[4], d_[4], rr_[4], r2_[4];
         f4_to_array(cur.bias, bias_);
         f4_to_array(cur.scale, scale_);
         f4_to_array(cur.rsub, rsub_);
@@ -181,6 +221,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
         f4_to_array(cur.post, post_);
         f4_to_array(cur.ih, ih_);
         f4_to_array(cur.r, rr_);
+        f4_to_array(cur.r2, r2_);
         if (fl & CF_FQ_IL0) {   // input_low == +0: x - il == x and d == ih
             il_[0] = il_[1] = il_[2] = il_[3] = 0.f;
             f4_to_array(cur.ih, d_);
@@ -226,11 +267,14 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     float t;
-                    if (fl & CF_FQ_RCP) {
-                        t = (fl & CF_FQ_IL0) ? fq_level_fast<true, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], a.lm1)
-                                             : fq_level_fast<true, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], a.lm1);
+                    if (fl & CF_FQ_DIV2) {
+                        t = (fl & CF_FQ_IL0) ? fq_level_fast<2, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], r2_[j], a.lm1)
+                                             : fq_level_fast<2, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], r2_[j], a.lm1);
+                    } else if (fl & CF_FQ_RCP) {
+                        t = (fl & CF_FQ_IL0) ? fq_level_fast<1, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], 0.f, a.lm1)
+                                             : fq_level_fast<1, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], 0.f, a.lm1);
                     } else {
-                        t = fq_level_fast<false, false>(v[pb][j], il_[j], ih_[j], d_[j], 0.f, a.lm1);
+                        t = fq_level_fast<0, false>(v[pb][j], il_[j], ih_[j], d_[j], 0.f, 0.f, a.lm1);
                     }
                     packed[pb] = __builtin_amdgcn_cvt_pk_u8_f32(t, j, packed[pb]);
                 }
@@ -269,7 +313,8 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
 
 template <uint32_t F>
 __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
-                                             int m0, int m1, int batch, const v16f (&rres)[2][2]) {
+                                             int m0, int m1, int batch, const v16f (&rres)[2][2],
+                                             const float* sp = nullptr, int sp_stride = 0, int oc0 = 0) {
     bool valid[2];
     int64_t out_off[2], res_off[2];
     const int m[2] = {m0, m1};
@@ -282,14 +327,15 @@ __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc
         res_off[pb] = batch * a.batch_res + static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh +
                       p.ow * a.res_sw + oc_lane;
     }
-    epilogue<F>(a, acc, oc_lane, valid, out_off, res_off, rres);
+    epilogue<F>(a, acc, oc_lane, valid, out_off, res_off, rres, sp, sp_stride, oc0);
 }
 
 template <uint32_t F>
 __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
-                                             int m0, int m1, int batch = 0) {
+                                             int m0, int m1, int batch = 0, const float* sp = nullptr,
+                                             int sp_stride = 0, int oc0 = 0) {
     v16f none[2][2];
-    run_epilogue<F>(a, acc, oc_lane, m0, m1, batch, none);
+    run_epilogue<F>(a, acc, oc_lane, m0, m1, batch, none, sp, sp_stride, oc0);
 }
 
 }  // namespace hipie

@@ -44,6 +44,7 @@ enum ConvFlags : uint32_t {
     CF_RES_U8B = 1u << 12,    // residual bytes are level-128 (add 128 after conversion)
     CF_FQ_IL0 = 1u << 13,     // every input_low is +0: x - il == x
     CF_OUT_XOR = 1u << 14,    // packed levels ^ 0x80808080 is the stored byte (offset -128)
+    CF_FQ_DIV2 = 1u << 16,    // two-operation division by the channel constant: fma(n, fq_r, n * fq_r2), verified at load time
     CF_RES_GEMM = 1u << 15,   // residual = (float(acc2) + bias2[c]) * scale2[c] of a second GEMM run in the same kernel
 };
 
@@ -64,6 +65,7 @@ struct ConvArgs {
     const float* fq_ih;
     const float* fq_d;
     const float* fq_r;
+    const float* fq_r2;
     int32_t M;            // N * OH * OW
     int32_t OW, OHOW;
     float inv_OW, inv_OHOW;          // for the reciprocal pixel decode (M < 2^24)

@@ -1,0 +1,127 @@
+#include "div2.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+
+#include "common.h"
+
+namespace hipie {
+namespace {
+
+constexpr int kBlocksPerDivisor = 32, kThreads = 256;
+
+// fail[i] != 0 when fma(n, zh[i], n * zl[i]) != n / d[i] for some significand of n
+__global__ __launch_bounds__(kThreads) void div2_check(const float* d, const float* zh, const float* zl, int* fail) {
+    const int i = blockIdx.y;
+    const float dd = d[i], h = zh[i], l = zl[i];
+    bool bad = false;
+    const uint32_t stride = kBlocksPerDivisor * kThreads;
+    for (uint32_t m = blockIdx.x * kThreads + threadIdx.x; m < (1u << 23); m += stride) {
+        const float n = __uint_as_float(0x3f800000u | m);
+        const float lo = n * l;
+        const float fast = fmaf(n, h, lo);
+        const float ref = n / dd;
+        bad = bad || !(fast == ref);
+    }
+    if (bad) atomicOr(&fail[i], 1);
+}
+
+float next_float(float x, int k) {
+    // k units in the last place away from x (x finite, non-zero, result keeps the sign)
+    int32_t b;
+    std::memcpy(&b, &x, 4);
+    b += (b >= 0) ? k : -k;
+    float y;
+    std::memcpy(&y, &b, 4);
+    return y;
+}
+
+}  // namespace
+
+bool fq_div2_constants(int device, const std::vector<float>& d, std::vector<float>& zh, std::vector<float>& zl) {
+    zh.assign(d.size(), 0.f);
+    zl.assign(d.size(), 0.f);
+    if (device < 0 || d.empty()) return false;
+    // distinct divisors only (a per-tensor range repeats one value for every channel)
+    std::map<uint32_t, int> index;
+    std::vector<float> ud;
+    for (float v : d) {
+        if (!(v > 0.f) || !std::isfinite(v)) return false;
+        uint32_t b;
+        std::memcpy(&b, &v, 4);
+        if (index.emplace(b, static_cast<int>(ud.size())).second) ud.push_back(v);
+    }
+    const size_t n = ud.size();
+    std::vector<float> uh(n), ul(n);
+    std::vector<double> inv(n);
+    for (size_t i = 0; i < n; ++i) {
+        inv[i] = 1.0 / static_cast<double>(ud[i]);
+        const float h = static_cast<float>(inv[i]);
+        if (!std::isnormal(h) || !std::isnormal(static_cast<float>(inv[i] - static_cast<double>(h)))) return false;
+    }
+    DeviceGuard g(device);
+    std::vector<int> todo(n);
+    for (size_t i = 0; i < n; ++i) todo[i] = static_cast<int>(i);
+    // candidates: zh = RN(1/d) moved by hs units in the last place, zl = RN(1/d - zh) moved by ls
+    static const int kShift[] = {0, 1, -1, 2, -2, 3, -3, 4, -4};
+    DeviceBuffer bd, bh, bl, bf;
+    for (int hs : {0, 1, -1}) {
+        for (int ls : kShift) {
+            if (todo.empty()) break;
+            const size_t m = todo.size();
+            std::vector<float> cd(m), ch(m), cl(m);
+            for (size_t j = 0; j < m; ++j) {
+                const int i = todo[j];
+                cd[j] = ud[i];
+                ch[j] = next_float(static_cast<float>(inv[i]), hs);
+                cl[j] = next_float(static_cast<float>(inv[i] - static_cast<double>(ch[j])), ls);
+            }
+            std::vector<int> fail(m, 0);
+            bd.upload(device, cd.data(), m * sizeof(float));
+            bh.upload(device, ch.data(), m * sizeof(float));
+            bl.upload(device, cl.data(), m * sizeof(float));
+            bf.upload(device, fail.data(), m * sizeof(int));
+            for (size_t off = 0; off < m; off += 32768) {   // grid.y limit
+                const size_t cnt = std::min<size_t>(32768, m - off);
+                hipLaunchKernelGGL(div2_check, dim3(kBlocksPerDivisor, static_cast<unsigned>(cnt)), dim3(kThreads), 0,
+                                   nullptr, bd.as<float>() + off, bh.as<float>() + off, bl.as<float>() + off,
+                                   bf.as<int>() + off);
+            }
+            HIPIE_CHECK_HIP(hipGetLastError());
+            HIPIE_CHECK_HIP(hipMemcpy(fail.data(), bf.as<int>(), m * sizeof(int), hipMemcpyDeviceToHost));
+            std::vector<int> still;
+            for (size_t j = 0; j < m; ++j) {
+                if (fail[j]) {
+                    still.push_back(todo[j]);
+                } else {
+                    uh[todo[j]] = ch[j];
+                    ul[todo[j]] = cl[j];
+                }
+            }
+            todo.swap(still);
+            if (std::getenv("HIPIE_TUNE_LOG"))
+                std::fprintf(stderr, "hipie div2: %zu divisors, zh%+d zl%+d ulp: %zu unmatched\n", n, hs, ls, todo.size());
+        }
+    }
+    if (!todo.empty()) {
+        if (std::getenv("HIPIE_TUNE_LOG"))
+            for (int i : todo) std::fprintf(stderr, "hipie div2: no constants for d = %a (%.9g)\n", ud[i], ud[i]);
+        return false;
+    }
+    for (size_t c = 0; c < d.size(); ++c) {
+        uint32_t b;
+        std::memcpy(&b, &d[c], 4);
+        const int i = index[b];
+        zh[c] = uh[i];
+        zl[c] = ul[i];
+    }
+    return true;
+}
+
+}  // namespace hipie
