@@ -33,7 +33,8 @@ __global__ __launch_bounds__(kThreads) void div2_check(const float* d, const flo
 }
 
 float next_float(float x, int k) {
-    // k units in the last place away from x (x finite, non-zero, result keeps the sign)
+    // k units in the last place away from x (x finite; zero stays zero)
+    if (x == 0.f) return x;
     int32_t b;
     std::memcpy(&b, &x, 4);
     b += (b >= 0) ? k : -k;
@@ -63,7 +64,8 @@ bool fq_div2_constants(int device, const std::vector<float>& d, std::vector<floa
     for (size_t i = 0; i < n; ++i) {
         inv[i] = 1.0 / static_cast<double>(ud[i]);
         const float h = static_cast<float>(inv[i]);
-        if (!std::isnormal(h) || !std::isnormal(static_cast<float>(inv[i] - static_cast<double>(h)))) return false;
+        const float l = static_cast<float>(inv[i] - static_cast<double>(h));
+        if (!std::isnormal(h) || !(l == 0.f || std::isnormal(l))) return false;   // l == 0: d is a power of two
     }
     DeviceGuard g(device);
     std::vector<int> todo(n);
@@ -125,3 +127,14 @@ bool fq_div2_constants(int device, const std::vector<float>& d, std::vector<floa
 }
 
 }  // namespace hipie
+
+extern "C" int hipie_fq_div2_constants(int device, const float* d, int64_t n, float* zh, float* zl, int* verified) {
+    return hipie::guarded([&] {
+        HIPIE_REQUIRE(d && zh && zl && verified && n > 0, HIPIE_PARAMETER_MISMATCH, "hipie_fq_div2_constants: null argument");
+        HIPIE_REQUIRE(device >= 0, HIPIE_PARAMETER_MISMATCH, "hipie_fq_div2_constants: needs a device");
+        std::vector<float> dv(d, d + n), h, l;
+        *verified = hipie::fq_div2_constants(device, dv, h, l) ? 1 : 0;
+        std::copy(h.begin(), h.end(), zh);
+        std::copy(l.begin(), l.end(), zl);
+    });
+}

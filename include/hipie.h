@@ -127,6 +127,11 @@ int hipie_fq_run_q8_tensor(const hipie_fq* fq, const float* x, const hipie_tenso
 float hipie_fq_host_eval(const hipie_fq* fq, int64_t channel, float x);
 /* 1 when the reciprocal path was proven equal to division on all boundaries of all channels */
 int hipie_fq_uses_reciprocal(const hipie_fq* fq);
+/* Constants of the convolution epilogue's two-operation division: for each divisor d[i] a pair with
+ * fma(x, zh[i], x * zl[i]) == x / d[i] for every float x, checked on the device against IEEE division
+ * over all 2^23 significands.  *verified = 1 when every divisor has a pair (otherwise the epilogue
+ * keeps the reciprocal-with-corrections sequence and zh, zl are unspecified). */
+int hipie_fq_div2_constants(int device, const float* d, int64_t n, float* zh, float* zl, int* verified);
 
 /* ======================================================================================
  * 1b. Fused f32 epilogue applied to i32 accumulators, in this fixed order (each step one IEEE

@@ -112,3 +112,40 @@ def test_fq_full_size_properties(orc):
         want = orc.fake_quantize(x[n, c].cpu().numpy().reshape(1, 1, H, W), il[c], ih[c],
                                  np.float32(0), np.float32(255), 256)
         np.testing.assert_array_equal(q[n, c].cpu().numpy(), want[0, 0].astype(np.uint8))
+
+
+def test_two_operation_division_constants_match_ieee_division():
+    """fma(x, zh, x * zl) == x / d for the verified constants: spot-check 2 * 10^5 random x per divisor
+    against IEEE f32 division on the host (the library itself checks all 2^23 significands)."""
+    import ctypes
+    from dldt_amd._lib import lib, check
+    rng = np.random.default_rng(11)
+    d = np.concatenate([rng.uniform(0.01, 3e5, 61).astype(np.float32),
+                        np.array([1.0, 255.0, 2.55], np.float32)])
+    zh, zl = np.zeros_like(d), np.zeros_like(d)
+    ok = ctypes.c_int(0)
+    fp = ctypes.POINTER(ctypes.c_float)
+    check(lib().hipie_fq_div2_constants(0, d.ctypes.data_as(fp), ctypes.c_int64(d.size), zh.ctypes.data_as(fp),
+                                        zl.ctypes.data_as(fp), ctypes.byref(ok)))
+    assert ok.value == 1
+    assert np.finfo(np.longdouble).nmant >= 63
+    x = np.concatenate([rng.uniform(0, 1, 100000), rng.uniform(0, 4e5, 100000)]).astype(np.float32)
+    for i in range(d.size):
+        lo = x * zl[i]                                                   # one f32 rounding
+        # the fma: exact product and a sum rounded once (64-bit significands make a double rounding negligible)
+        fast = (x.astype(np.longdouble) * np.longdouble(zh[i]) + lo.astype(np.longdouble)).astype(np.float32)
+        np.testing.assert_array_equal(fast, x / d[i])
+
+
+def test_two_operation_division_reports_unmatched_divisor():
+    """A divisor for which no constant pair within the searched neighbourhood reproduces division for
+    every significand: the library must say so (the epilogue then keeps the slower exact sequence)."""
+    import ctypes
+    from dldt_amd._lib import lib, check
+    d = np.array([float.fromhex("0x1.e447fep+17")], np.float32)
+    zh, zl = np.zeros_like(d), np.zeros_like(d)
+    ok = ctypes.c_int(1)
+    fp = ctypes.POINTER(ctypes.c_float)
+    check(lib().hipie_fq_div2_constants(0, d.ctypes.data_as(fp), ctypes.c_int64(1), zh.ctypes.data_as(fp),
+                                        zl.ctypes.data_as(fp), ctypes.byref(ok)))
+    assert ok.value == 0
