@@ -474,6 +474,7 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
     case E_RESF32: X(E_RESF32, __VA_ARGS__); break;                                          \
     case E_RESGEMM: X(E_RESGEMM, __VA_ARGS__); break;                                        \
     case E_F32: X(E_F32, __VA_ARGS__); break;                                                \
+    case E_SCALE: X(E_SCALE, __VA_ARGS__); break;                                            \
     case E_F32RELU: X(E_F32RELU, __VA_ARGS__); break;                                        \
     case E_CLAMPFQ: X(E_CLAMPFQ, __VA_ARGS__); break;                                        \
     case E_PLAIN0 & ~CF_FQ_DIV2: X((E_PLAIN0 & ~CF_FQ_DIV2), __VA_ARGS__); break;            \

@@ -92,6 +92,7 @@ constexpr uint32_t E_RESU8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_U8B | CF_RES_M
 constexpr uint32_t E_RESF32 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32 | E_FQ | CF_FQ_IL0;
 constexpr uint32_t E_RESGEMM = CF_BIAS | CF_SCALE | CF_RES | CF_RES_GEMM | E_FQ | CF_FQ_IL0;
 constexpr uint32_t E_F32 = CF_BIAS | CF_SCALE;
+constexpr uint32_t E_SCALE = CF_SCALE;                      // MatMul' -> Multiply(s_a * s_b)
 constexpr uint32_t E_F32RELU = CF_BIAS | CF_SCALE | CF_RELU;
 constexpr uint32_t E_CLAMPFQ = CF_BIAS | CF_SCALE | CF_CLAMP | E_FQ | CF_FQ_IL0;
 

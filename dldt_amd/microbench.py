@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Kernel timings at the shapes of the five benchmark configurations, against each kernel's roofline.
+
+    python -m dldt_amd.microbench            # all rows, markdown table on stdout
+
+Rows: config 1 (one quantized 3x3 convolution block, batch 1), config 2 (per-channel FakeQuantize of
+[32,256,56,56]), config 3 (ResNet-50 v1.5 INT8, batch 1 and 64), config 4 (MobileNetV2 INT8, batch 64:
+whole graph, its depthwise and pointwise kernels), config 5 (one BERT-base encoder layer at batch 16,
+sequence 384: the int8 GEMMs and the fp32 softmax / LayerNorm / GELU kernels, each on its own).
+Inputs are resident in HBM, times are HIP-event averages over back-to-back launches.
+"""
+import sys
+
+import numpy as np
+
+INT8_PEAK_TOPS = 5000.0
+HBM_PEAK_GBS = 8000.0
+F32, U8, I8, I32, U8B = 10, 40, 50, 70, 41
+
+
+def _time(fn, reps=30, warm=5):
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps * 1e3   # us
+
+
+def _graph_time(g, reps=20, warm=5):
+    """(us per inference, plan) of a compiled graph, kernels only, on the request's stream."""
+    import torch
+    plan = g.compile(0)
+    req = plan.create_request()
+    ins, outs = req.device_buffers()
+    for t in ins:
+        t.copy_(torch.rand(t.shape, device="cuda"))
+    stream = torch.cuda.ExternalStream(req.stream)
+    torch.cuda.synchronize()
+    for _ in range(warm):
+        req.enqueue(ins, outs)
+    stream.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record(stream)
+    for _ in range(reps):
+        req.enqueue(ins, outs)
+    b.record(stream)
+    stream.synchronize()
+    return a.elapsed_time(b) / reps * 1e3, plan
+
+
+def _row(name, us, macs=0, bytes_=0, bound=None):
+    tops = 2.0 * macs / us / 1e6 if macs else 0.0
+    gbs = bytes_ / us / 1e3 if bytes_ else 0.0
+    if bound is None:
+        bound = "mfma" if macs and (tops / INT8_PEAK_TOPS >= gbs / HBM_PEAK_GBS) else "hbm"
+    frac = tops / INT8_PEAK_TOPS if bound == "mfma" else gbs / HBM_PEAK_GBS
+    return {"row": name, "us": us, "TOP/s": tops, "GB/s": gbs, "bound": bound, "frac": frac}
+
+
+def config1():
+    from . import builders
+    g, _, _ = builders.conv_block()
+    us, plan = _graph_time(g)
+    macs = sum(s["macs"] for s in plan.steps)
+    return [_row("cfg1 FQ + 3x3 conv 64->64 @56x56 + bias + ReLU, batch 1 (3 launches)", us, macs=macs,
+                 bytes_=200704 * 4 + 200704 + 36864 + 802816)]
+
+
+def config2():
+    import torch
+    from . import FakeQuantize
+    n, c, h, w = 32, 256, 56, 56
+    rng = np.random.default_rng(2)
+    mu = rng.uniform(-0.5, 0.5, c).astype(np.float32)
+    x = torch.randn((n, c, h, w), device="cuda") + torch.from_numpy(mu).cuda().view(1, c, 1, 1)
+    fq = FakeQuantize(c, 256, mu - 3, mu + 3, 0.0, 255.0)
+    y8 = torch.empty(x.shape, dtype=torch.uint8, device="cuda")
+    yf = torch.empty_like(x)
+    yn = torch.empty((n, h, w, c), dtype=torch.int8, device="cuda")
+    e = x.numel()
+    return [
+        _row("cfg2 FakeQuantize [32,256,56,56] per-channel, f32 -> u8 levels (NCHW)",
+             _time(lambda: fq.run_q8(x, "u8", "nchw", out=y8)), bytes_=5 * e),
+        _row("cfg2 same, f32 -> u8 levels NHWC (graph entry form)",
+             _time(lambda: fq.run_q8(x, "u8b", "nhwc", c, out=yn)), bytes_=5 * e),
+        _row("cfg2 same, f32 -> f32 (the operator as specified)", _time(lambda: fq.run_f32(x, out=yf)), bytes_=8 * e),
+    ]
+
+
+def config3():
+    from . import builders
+    rows = []
+    for batch in (1, 64):
+        g, meta = builders.resnet50(batch=batch, res=224)
+        us, plan = _graph_time(g)
+        r = _row("cfg3 ResNet-50 v1.5 INT8 batch %d, whole graph (%d launches)" % (batch, len(plan.steps)), us,
+                 macs=meta["macs_per_image"] * batch, bytes_=sum(s["bytes"] for s in plan.steps), bound="mfma")
+        r["images/s"] = batch / us * 1e6
+        rows.append(r)
+    return rows
+
+
+def config4():
+    import torch
+    from . import builders, Convolution, DeviceTensor, make_epilogue
+    g, meta = builders.mobilenet_v2(batch=64, res=224)
+    us, plan = _graph_time(g)
+    r = _row("cfg4 MobileNetV2-1.0 INT8 batch 64, whole graph (%d launches)" % len(plan.steps), us,
+             macs=meta["macs_per_image"] * 64, bytes_=sum(s["bytes"] for s in plan.steps))
+    r["images/s"] = 64 / us * 1e6
+    rows = [r]
+    rng = np.random.default_rng(4)
+    for c, hw, stride in ((96, 112, 2), (384, 14, 1), (960, 7, 1)):
+        cs = -(-c // 16) * 16
+        xin = DeviceTensor(64, hw, hw, c, U8B, halo=1)
+        xin.interior().copy_(torch.randint(-128, 127, xin.interior().shape, dtype=torch.int8, device="cuda"))
+        w = rng.integers(-127, 128, (c, 1, 1, 3, 3)).astype(np.int8)
+        fq = (256, 0.0, np.full(c, 3000.0, np.float32), 0.0, 255.0)
+        conv = Convolution(w, xin, (stride, stride), (1, 1), (1, 1), (1, 1),
+                           make_epilogue(bias=np.zeros(c, np.float32), out_dtype=U8B, fq=fq))
+        oh = (hw + 2 - 3) // stride + 1
+        out = DeviceTensor(64, oh, oh, c, U8B)
+        rows.append(_row("cfg4 depthwise 3x3 s%d C=%d @%dx%d batch 64" % (stride, c, hw, hw),
+                         _time(lambda: conv.run(xin, out)), macs=64 * oh * oh * c * 9,
+                         bytes_=64 * (hw * hw + oh * oh) * cs + 9 * c, bound="hbm"))
+    return rows
+
+
+def config5():
+    import torch
+    from . import BatchedMatMul, Convolution, DeviceTensor, make_epilogue, softmax, mvn, gelu
+    B, S, H, NH, FF = 16, 384, 768, 12, 3072
+    T = B * S
+    rng = np.random.default_rng(5)
+    rows = []
+    layer_us = 0.0
+
+    def linear(name, k, n, out_dtype, count=1):
+        nonlocal layer_us
+        xin = DeviceTensor(1, 1, T, k, I8)
+        xin.interior().copy_(torch.randint(-128, 127, xin.interior().shape, dtype=torch.int8, device="cuda"))
+        w = rng.integers(-127, 128, (n, k, 1, 1)).astype(np.int8)
+        if out_dtype == F32:
+            ep = make_epilogue(bias=np.zeros(n, np.float32), scale=np.full(n, 1e-4, np.float32), out_dtype=F32)
+        else:
+            ep = make_epilogue(bias=np.zeros(n, np.float32), out_dtype=I8,
+                               fq=(256, np.full(n, -128e3, np.float32), np.full(n, 127e3, np.float32), -128.0, 127.0))
+        conv = Convolution(w, xin, epilogue=ep)
+        out = DeviceTensor(1, 1, T, n, out_dtype)
+        us = _time(lambda: conv.run(xin, out))
+        layer_us += us * count
+        rows.append(_row("cfg5 %s [%d,%d]x[%d,%d] -> %s" % (name, T, k, k, n, "f32" if out_dtype == F32 else "i8"), us,
+                         macs=T * k * n, bytes_=T * k + k * n + T * n * (4 if out_dtype == F32 else 1), bound="mfma"))
+
+    linear("QKV projection", H, 3 * H, I8)
+    linear("attention output projection", H, H, F32)
+    linear("FFN up", H, FF, F32)
+    linear("FFN down", FF, H, F32)
+
+    def attention(name, m, k, n):
+        nonlocal layer_us
+        a = torch.randint(-128, 127, (B * NH, m, k), dtype=torch.int8, device="cuda")
+        bt = torch.randint(-128, 127, (B * NH, n, k), dtype=torch.int8, device="cuda")
+        mm = BatchedMatMul(k, n, make_epilogue(scale=[1e-3], out_dtype=F32))
+        out = torch.empty((B * NH, m, n), dtype=torch.float32, device="cuda")
+        us = _time(lambda: mm.run(a, bt, out), reps=10, warm=3)
+        layer_us += us
+        rows.append(_row("cfg5 %s %dx[%d,%d]x[%d,%d] -> f32" % (name, B * NH, m, k, k, n), us,
+                         macs=B * NH * m * k * n, bytes_=B * NH * (m * k + n * k + 4 * m * n)))
+
+    attention("attention scores", S, 64, S)
+    attention("attention context", S, S, 64)
+
+    def glue(name, fn, x, passes):
+        nonlocal layer_us
+        us = _time(lambda: fn(x), reps=10, warm=3)
+        layer_us += us * (2 if name.startswith("LayerNorm") else 1)
+        rows.append(_row("cfg5 %s %s f32" % (name, list(x.shape)), us, bytes_=passes * 4 * x.numel(), bound="hbm"))
+
+    glue("softmax", softmax, torch.randn((B * NH * S, S), device="cuda"), 2)
+    gamma, beta = torch.ones(H, device="cuda"), torch.zeros(H, device="cuda")
+    glue("LayerNorm (MVN, gamma, beta)", lambda t: mvn(t, gamma=gamma, beta=beta), torch.randn((T, H), device="cuda"), 2)
+    glue("GELU (erf)", gelu, torch.randn((T, FF), device="cuda"), 2)
+    r = _row("cfg5 one encoder layer, sum of the kernels above (LayerNorm twice)", layer_us,
+             macs=T * (4 * H * H + 2 * H * FF) + 2 * B * NH * S * S * 64, bound="mfma")
+    r["sequences/s (12 layers, these kernels only)"] = B / (12 * layer_us) * 1e6
+    rows.append(r)
+    return rows
+
+
+def main():
+    import torch
+    assert torch.cuda.is_available(), "microbench needs a GPU"
+    which = sys.argv[1:] or ["1", "2", "3", "4", "5"]
+    table = {"1": config1, "2": config2, "3": config3, "4": config4, "5": config5}
+    print("| kernel / graph | us | TOP/s | GB/s | bound | fraction of peak | notes |")
+    print("|---|---|---|---|---|---|---|")
+    for k in which:
+        for r in table[k]():
+            extra = ", ".join("%s %.0f" % (n, v) for n, v in r.items()
+                              if n not in ("row", "us", "TOP/s", "GB/s", "bound", "frac"))
+            print("| %s | %.1f | %.1f | %.0f | %s | %.3f | %s |" % (r["row"], r["us"], r["TOP/s"], r["GB/s"], r["bound"],
+                                                                  r["frac"], extra))
+            sys.stdout.flush()
+
+
+if __name__ == "__main__":
+    main()

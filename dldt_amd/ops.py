@@ -215,7 +215,7 @@ class BatchedMatMul:
             lib().hipie_matmul_destroy(self._h)
             self._h = None
 
-    def run(self, a, bt):
+    def run(self, a, bt, out=None):
         import torch
         batch, m, k = a.shape
         assert bt.shape[0] == batch and bt.shape[2] == k and bt.shape[1] == self.n and k == self.k
@@ -223,7 +223,9 @@ class BatchedMatMul:
         od = self.epilogue.out_dtype
         tdt, gran = {I32: (torch.int32, 4), F32: (torch.float32, 4)}.get(od, (torch.int8, 16))
         ldo = -(-self.n // gran) * gran
-        out = torch.zeros((batch, m, ldo), dtype=tdt, device=a.device)
+        if out is None:
+            out = torch.zeros((batch, m, ldo), dtype=tdt, device=a.device)
+        assert out.shape == (batch, m, ldo) and out.dtype == tdt and out.is_contiguous()
         i64 = ctypes.c_int64
         check(lib().hipie_matmul_run(self._h, _dptr(a), i64(k), i64(m * k), _dptr(bt), i64(k), i64(self.n * k),
                                      _dptr(out), i64(ldo), i64(m * ldo), ctypes.c_int32(m), ctypes.c_int32(batch),
