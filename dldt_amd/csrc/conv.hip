@@ -36,7 +36,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     const int chunk = tid & 3;
 
     const int batch = blockIdx.y;
-    stage_params<F>(a, oc0, sP, BOC, tid, NT);   // visible after the first barrier of the K loop
+    stage_params<F>(a, oc0, (lds_float_ptr)sP, BOC, tid, NT);   // visible after the first barrier of the K loop
     const int a_row[2] = {woc * 64 + l32, woc * 64 + 32 + l32};
     const int b_row[2] = {wpix * 64 + l32, wpix * 64 + 32 + l32};
     const int oc_lane = oc0 + woc * 64 + 32 * h;
@@ -137,7 +137,140 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     gemm(a.in + batch * a.batch_in, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
          a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc);
     const int m0 = pix0 + wpix * 64 + l32;
-    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, sP, BOC, oc0);
+    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, (lds_cfloat_ptr)sP, BOC, oc0);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Persistent LDS-tiled kernel for the layers whose time is the epilogue and the memory latency
+// around it (small K): a workgroup keeps its channel tile and walks pixel tiles.  The operands of
+// the next tile's first K step and the next tile's residual bytes are requested before the
+// epilogue of the current tile, so memory latency, the matrix pipe and the epilogue's VALU work of
+// one wave overlap by construction instead of by occupancy.  Grid: 8 XCDs x channel tiles x n_per
+// workgroups, workgroup (xcd, t_tile, i) takes the XCD's pixel tiles i, i + n_per, ...
+template <int WOC, int WPIX, uint32_t F>
+__global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const ConvArgs a, const int n_per) {
+    constexpr int NT = WOC * WPIX * 64;
+    constexpr int BOC = WOC * 64, BPIX = WPIX * 64;
+    constexpr int A_PIECES = BOC * 4 / NT, B_PIECES = BPIX * 4 / NT;
+    constexpr bool kByteRes = (F & CF_RES) && !(F & (CF_RES_F32 | CF_RES_GEMM));
+    __shared__ __attribute__((aligned(16))) int8_t sA[2][BOC * kRow];
+    __shared__ __attribute__((aligned(16))) int8_t sB[2][BPIX * kRow];
+    __shared__ __attribute__((aligned(16))) float sP[PT_COUNT * BOC];
+
+    const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
+    const int t_tile = y % a.t_tiles;
+    int p_local = y / a.t_tiles;   // < n_per
+    auto tile_exists = [&](int pl) { return pl < a.p_per_xcd && xcd * a.p_per_xcd + pl < a.p_tiles; };
+    if (!tile_exists(p_local)) return;   // uniform over the workgroup
+    const int oc0 = t_tile * BOC;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int woc = wave % WOC, wpix = wave / WOC;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int chunk = tid & 3;
+    stage_params<F>(a, oc0, (lds_float_ptr)sP, BOC, tid, NT);   // visible after the first barrier
+    const int a_row[2] = {woc * 64 + l32, woc * 64 + 32 + l32};
+    const int b_row[2] = {wpix * 64 + l32, wpix * 64 + 32 + l32};
+    const int oc_lane = oc0 + woc * 64 + 32 * h;
+    const int nk = a.nk;
+
+    const int8_t* a_ptr[A_PIECES];
+#pragma unroll
+    for (int i = 0; i < A_PIECES; ++i) {
+        const int row = min(oc0 + ((tid + i * NT) >> 2), a.wgt_rows - 1);
+        a_ptr[i] = a.wgt + static_cast<int64_t>(row) * a.wgt_ld + chunk * 16;
+    }
+    int32_t b_base[B_PIECES];
+    auto pixel_bases = [&](int pl) {
+        const int pix0 = (xcd * a.p_per_xcd + pl) * BPIX;
+#pragma unroll
+        for (int i = 0; i < B_PIECES; ++i) {
+            int m = pix0 + ((tid + i * NT) >> 2);
+            m = m < a.M ? m : a.M - 1;
+            const PixelCoord p = decode_pixel(a, m);
+            b_base[i] = p.n * a.in_sn + p.oh * a.conv_sh * a.in_sh + p.ow * a.conv_sw * a.in_sw + a.in_origin;
+        }
+    };
+    v4i ga[A_PIECES], gb[B_PIECES];
+    auto load_global = [&](int k) {
+        const int4 ko = *reinterpret_cast<const int4*>(a.koff + 4 * k);
+        const int32_t off = chunk == 0 ? ko.x : (chunk == 1 ? ko.y : (chunk == 2 ? ko.z : ko.w));
+#pragma unroll
+        for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(a_ptr[i] + k * 64);
+#pragma unroll
+        for (int i = 0; i < B_PIECES; ++i) gb[i] = *reinterpret_cast<const v4i*>(a.in + (b_base[i] + off));
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < A_PIECES; ++i)
+            *reinterpret_cast<v4i*>(&sA[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = ga[i];
+#pragma unroll
+        for (int i = 0; i < B_PIECES; ++i)
+            *reinterpret_cast<v4i*>(&sB[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = gb[i];
+    };
+    auto addresses = [&](int pl, EpiAddr& e) {
+        const int m0 = (xcd * a.p_per_xcd + pl) * BPIX + wpix * 64 + l32;
+        epilogue_addresses(a, oc_lane, m0, m0 + 32, 0, e);
+    };
+
+    EpiAddr cur, nxt;
+    uint32_t res_cur[2][8], res_nxt[2][8];
+    pixel_bases(p_local);
+    load_global(0);
+    addresses(p_local, cur);
+    if (kByteRes) load_residual_bytes(a, oc_lane, cur.valid, cur.res_off, res_cur);
+    v16f none[2][2];
+    while (true) {
+        v16i acc[2][2];
+        init_acc(a, oc_lane, acc);
+        store_lds(0);
+        __syncthreads();
+        const int next_p = p_local + n_per;
+        const bool has_next = tile_exists(next_p);
+        for (int k = 0; k < nk; ++k) {
+            const int buf = k & 1;
+            if (k + 1 < nk) {
+                load_global(k + 1);
+            } else if (has_next) {   // first K step of the next tile, in flight during the epilogue
+                pixel_bases(next_p);
+                load_global(0);
+            }
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                v4i af[2], bf[2];
+#pragma unroll
+                for (int ob = 0; ob < 2; ++ob)
+                    af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][a_row[ob] * kRow + ks * 32 + h * 16]);
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+                    bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][b_row[pb] * kRow + ks * 32 + h * 16]);
+#pragma unroll
+                for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                    for (int pb = 0; pb < 2; ++pb)
+                        acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
+            }
+            if (k + 1 < nk) {
+                store_lds(buf ^ 1);
+                __syncthreads();
+            }
+        }
+        if (has_next) {
+            addresses(next_p, nxt);
+            if (kByteRes) load_residual_bytes(a, oc_lane, nxt.valid, nxt.res_off, res_nxt);
+        }
+        epilogue<F>(a, acc, oc_lane, cur.valid, cur.out_off, cur.res_off, none, (lds_cfloat_ptr)sP, BOC, oc0, kByteRes ? res_cur : nullptr);
+        if (!has_next) break;
+        cur = nxt;
+        if (kByteRes) {
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) res_cur[pb][q] = res_nxt[pb][q];
+        }
+        p_local = next_p;
+        __syncthreads();   // every wave has read the last K step before the buffers are refilled
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -203,7 +336,7 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
     const int frag_off[2] = {l32 * 64 + ((0 + h) ^ swz) * 16, l32 * 64 + ((2 + h) ^ swz) * 16};
     // epilogue tables behind the rings; visible after the barrier that follows the K-offset table fill
     float* const sP = reinterpret_cast<float*>(ring + KS * stages * STAGE);
-    stage_params<F>(a, oc0, sP, BOC, tid, NT_ALL);
+    stage_params<F>(a, oc0, (lds_float_ptr)sP, BOC, tid, NT_ALL);
 
     auto gemm = [&](const int8_t* in_base, int in_sn, int in_sh, int in_sw, int csh, int csw, int origin,
                     const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk_all,
@@ -359,7 +492,7 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
                 for (int r = 0; r < 16; ++r) acc[ob][pb][r] += red[((ob * 2 + pb) * 16 + r) * NT + t];
     }
     const int m0 = pix0 + wpix * 64 + l32;
-    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, sP, BOC, oc0);
+    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, (lds_cfloat_ptr)sP, BOC, oc0);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -383,7 +516,7 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
         }
     }
     float* const sP = reinterpret_cast<float*>(sW + 64 * wrow);
-    stage_params<F>(a, oc0, sP, 64, tid, 256);
+    stage_params<F>(a, oc0, (lds_float_ptr)sP, 64, tid, 256);
     const int oc_lane = oc0 + 32 * h;
     const int a_row[2] = {l32 * wrow + h * 16, (32 + l32) * wrow + h * 16};
 
@@ -454,7 +587,7 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
         compute(cur, cur_k);
         if (cur_k + 1 == a.nk) {
             const int m0 = cur_tile * 256 + wave * 64 + l32;
-            run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, 0, sP, 64, oc0);
+            run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, 0, (lds_cfloat_ptr)sP, 64, oc0);
             init_acc(a, oc_lane, acc);
         }
         return more;
@@ -514,8 +647,35 @@ void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) 
 #undef HIPIE_LAUNCH_PIPE
 }
 
-void launch_tiled_small(const ConvArgs& a, hipStream_t s) {   // 64 x 64 tile, one wave: generic epilogue only
-    hipLaunchKernelGGL((conv_tiled_kernel<1, 1, kDyn>), dim3(8 * a.p_per_xcd * a.t_tiles), dim3(64), 0, s, a);
+// the template instances of the persistent kernel: byte outputs and byte / no residual
+bool persist_available(uint32_t flags) {
+    switch (flags & ~CF_OUT_XOR) {
+    case E_PLAIN0: case E_PLAIN: case E_RESU8: case E_CLAMPFQ: return true;
+    default: return false;
+    }
+}
+
+template <int WOC, int WPIX>
+void launch_persist(const ConvArgs& a, hipStream_t s) {
+    // two workgroups per compute unit, a whole number of them per (XCD, channel tile)
+    const int n_per = std::max(1, std::min<int>(a.p_per_xcd, 512 / (8 * a.t_tiles)));
+    const dim3 grid(8 * a.t_tiles * n_per), block(WOC * WPIX * 64);
+    switch (a.flags & ~CF_OUT_XOR) {
+    case E_PLAIN0: hipLaunchKernelGGL((conv_persist_kernel<WOC, WPIX, E_PLAIN0>), grid, block, 0, s, a, n_per); break;
+    case E_PLAIN: hipLaunchKernelGGL((conv_persist_kernel<WOC, WPIX, E_PLAIN>), grid, block, 0, s, a, n_per); break;
+    case E_RESU8: hipLaunchKernelGGL((conv_persist_kernel<WOC, WPIX, E_RESU8>), grid, block, 0, s, a, n_per); break;
+    case E_CLAMPFQ: hipLaunchKernelGGL((conv_persist_kernel<WOC, WPIX, E_CLAMPFQ>), grid, block, 0, s, a, n_per); break;
+    default: fail(HIPIE_GENERAL_ERROR, "persistent convolution kernel: no instance for epilogue %#x", a.flags);
+    }
+}
+
+void launch_tiled_small(const ConvArgs& a, hipStream_t s) {   // 64 x 64 tile, one wave per workgroup
+    const dim3 grid(8 * a.p_per_xcd * a.t_tiles), block(64);
+    const uint32_t core = a.flags & ~CF_OUT_XOR;
+#define HIPIE_LAUNCH_SMALL(FLAGS, ...) \
+    hipLaunchKernelGGL((conv_tiled_kernel<1, 1, FLAGS>), grid, block, 0, s, a)
+    HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_SMALL, 0)
+#undef HIPIE_LAUNCH_SMALL
 }
 
 void launch_stream(const ConvArgs& a, int grid_x, hipStream_t s) {
@@ -932,10 +1092,12 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 7, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 9, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
         if (c->depthwise) return;               // one kernel only
         if (c->fused && tile != 0 && tile != 4) return;   // the second GEMM exists in the 128 x 128 kernels
-        HIPIE_REQUIRE(tile < 6 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
+        HIPIE_REQUIRE(tile < 8 || (!c->fused && persist_available(c->epi.flags)), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_set_tile: the persistent kernels exist for byte outputs with a byte residual or none");
+        HIPIE_REQUIRE(tile < 6 || tile > 7 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the split-K kernels need an even number of 64-byte K steps (K=%lld)", (long long)c->Kp);
         HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) + PT_COUNT * 64 * 4 <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: K=%lld does not fit the streaming kernel's LDS", (long long)c->Kp);
@@ -1084,7 +1246,7 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
             return;
         }
         const int tile = c->tile;
-        const bool square = tile == 0 || tile == 4 || tile == 6;
+        const bool square = tile == 0 || tile == 4 || tile == 6 || tile == 8;
         const int boc = square ? 128 : 64;
         const int bpix = square ? 128 : (tile == 2 ? 64 : 256);
         a.p_tiles = static_cast<int32_t>(ceil_div(M, bpix));
@@ -1099,6 +1261,8 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         switch (tile) {
         case 4: launch_pipe<2, 2, 1>(a, stages, s); break;
         case 5: launch_pipe<1, 4, 1>(a, stages, s); break;
+        case 8: launch_persist<2, 2>(a, s); break;
+        case 9: launch_persist<1, 4>(a, s); break;
         case 6: launch_pipe<2, 2, 2>(a, stages, s); break;
         case 7: launch_pipe<1, 4, 2>(a, stages, s); break;
         case 0: launch_tiled<2, 2>(a, s); break;

@@ -100,10 +100,13 @@ constexpr uint32_t E_CLAMPFQ = CF_BIAS | CF_SCALE | CF_CLAMP | E_FQ | CF_FQ_IL0;
 // lane of a half-wave needs the same four channels at a time: read from global memory that is a
 // 64-lane vector load whose address processing costs as much as a real gather (the convolution
 // kernels spent most of their texture-addresser cycles there); read from LDS it is a broadcast.
+typedef const __attribute__((address_space(3))) float* lds_cfloat_ptr;   // keeps ds_read (a generic pointer makes them FLAT loads)
+typedef __attribute__((address_space(3))) float* lds_float_ptr;
+
 enum ParamTable { PT_BIAS, PT_SCALE, PT_RSUB, PT_RMUL, PT_POST, PT_IL, PT_IH, PT_D, PT_R, PT_R2, PT_COUNT };
 
 template <uint32_t F>
-__device__ __forceinline__ void stage_params(const ConvArgs& a, int oc0, float* sp, int stride, int tid, int nt) {
+__device__ __forceinline__ void stage_params(const ConvArgs& a, int oc0, lds_float_ptr sp, int stride, int tid, int nt) {
     const uint32_t fl = F == kDyn ? a.flags : F;
     auto put = [&](int t, const float* src) {
         for (int c = tid; c < stride; c += nt) sp[t * stride + c] = src[oc0 + c];
@@ -129,13 +132,43 @@ struct EpiParams {
     float4 res[2];   // f32 residual of the two pixels
 };
 
-__device__ __forceinline__ float res_byte_to_float(uint32_t dw, int j, float add) {
-    const int b = static_cast<int>(static_cast<int8_t>((dw >> (8 * j)) & 0xffu));
-    return static_cast<float>(b) + add;
+// residual level as float: signed bytes as they are; level-128 bytes through a sign-bit flip of the
+// whole dword and the unsigned byte conversion (v_cvt_f32_ubyteN), the same exact integer value
+template <bool U8B>
+__device__ __forceinline__ float res_byte_to_float(uint32_t dw, int j) {
+    if (U8B) return static_cast<float>(((dw ^ 0x80808080u) >> (8 * j)) & 0xffu);
+    return static_cast<float>(static_cast<int>(static_cast<int8_t>((dw >> (8 * j)) & 0xffu)));
 }
 
 __device__ __forceinline__ void f4_to_array(const float4& v, float (&o)[4]) {
     o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+
+// The 32 residual bytes of each of a lane's two pixels (zero where the pixel or channel does not
+// exist).  The loads are unconditional - a lane without a valid element reads the first 16 bytes
+// of its (clamped, existing) pixel and discards them - so that all four are in flight together;
+// a load inside a divergent branch is awaited at the end of its branch.
+__device__ __forceinline__ void load_residual_bytes(const ConvArgs& a, int oc_lane, const bool (&valid)[2],
+                                                    const int64_t (&res_off)[2], uint32_t (&res_dw)[2][8]) {
+    uint4 v[2][2];
+    bool ok[2][2];
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            ok[pb][j] = valid[pb] && oc_lane + 16 * j < a.res_sw;
+            const int64_t off = ok[pb][j] ? res_off[pb] + 16 * j : res_off[pb] - oc_lane;
+            v[pb][j] = *reinterpret_cast<const uint4*>(static_cast<const int8_t*>(a.res) + off);
+        }
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            res_dw[pb][4 * j + 0] = ok[pb][j] ? v[pb][j].x : 0u;
+            res_dw[pb][4 * j + 1] = ok[pb][j] ? v[pb][j].y : 0u;
+            res_dw[pb][4 * j + 2] = ok[pb][j] ? v[pb][j].z : 0u;
+            res_dw[pb][4 * j + 3] = ok[pb][j] ? v[pb][j].w : 0u;
+        }
 }
 
 // sp: the tile's staged tables (stage_params) with local channel 0 = channel oc0, or nullptr to
@@ -144,10 +177,16 @@ template <uint32_t F>
 __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                          const bool (&valid)[2], const int64_t (&out_off)[2],
                                          const int64_t (&res_off)[2], const v16f (&rres)[2][2],
-                                         const float* sp, int sp_stride, int oc0) {
+                                         lds_cfloat_ptr sp, int sp_stride, int oc0,
+                                         const uint32_t (*pre_res)[8] = nullptr) {
     const uint32_t fl = F == kDyn ? a.flags : F;
     auto tab = [&](int t, const float* g, int oc) {
-        return sp ? *reinterpret_cast<const float4*>(sp + t * sp_stride + (oc - oc0)) : ld4f(g + oc);
+        if (sp) {
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            const v4f v = *(const __attribute__((address_space(3))) v4f*)(sp + t * sp_stride + (oc - oc0));
+            return make_float4(v.x, v.y, v.z, v.w);
+        }
+        return ld4f(g + oc);
     };
     const int out_cs = a.out_sw;
 
@@ -166,20 +205,15 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
 
     uint32_t res_dw[2][8];
     if ((fl & CF_RES) && !(fl & (CF_RES_F32 | CF_RES_GEMM))) {
+        if (pre_res) {
 #pragma unroll
-        for (int pb = 0; pb < 2; ++pb)
+            for (int pb = 0; pb < 2; ++pb)
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                uint4 v = make_uint4(0, 0, 0, 0);
-                if (valid[pb] && oc_lane + 16 * j < a.res_sw)
-                    v = *reinterpret_cast<const uint4*>(static_cast<const int8_t*>(a.res) + res_off[pb] + 16 * j);
-                res_dw[pb][4 * j + 0] = v.x;
-                res_dw[pb][4 * j + 1] = v.y;
-                res_dw[pb][4 * j + 2] = v.z;
-                res_dw[pb][4 * j + 3] = v.w;
-            }
+                for (int q = 0; q < 8; ++q) res_dw[pb][q] = pre_res[pb][q];
+        } else {
+            load_residual_bytes(a, oc_lane, valid, res_off, res_dw);
+        }
     }
-    const float res_add = (fl & CF_RES_U8B) ? 128.0f : 0.0f;
 
     auto load = [&](int e4, EpiParams& p) {
         const int oc = oc_lane + 4 * e4;
@@ -241,7 +275,8 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
                 } else if (fl & CF_RES_F32) f4_to_array(cur.res[pb], rv);
                 else {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) rv[j] = res_byte_to_float(res_dw[pb][e4], j, res_add);
+                    for (int j = 0; j < 4; ++j)
+                        rv[j] = (fl & CF_RES_U8B) ? res_byte_to_float<true>(res_dw[pb][e4], j) : res_byte_to_float<false>(res_dw[pb][e4], j);
                 }
             }
 #pragma unroll
@@ -312,28 +347,37 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
     }
 }
 
-template <uint32_t F>
-__device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
-                                             int m0, int m1, int batch, const v16f (&rres)[2][2],
-                                             const float* sp = nullptr, int sp_stride = 0, int oc0 = 0) {
+// where a lane's two pixels live in the output and residual tensors
+struct EpiAddr {
     bool valid[2];
     int64_t out_off[2], res_off[2];
+};
+
+__device__ __forceinline__ void epilogue_addresses(const ConvArgs& a, int oc_lane, int m0, int m1, int batch, EpiAddr& e) {
     const int m[2] = {m0, m1};
 #pragma unroll
     for (int pb = 0; pb < 2; ++pb) {
-        valid[pb] = m[pb] < a.M;
-        const PixelCoord p = decode_pixel(a, valid[pb] ? m[pb] : a.M - 1);
-        out_off[pb] = batch * a.batch_out + static_cast<int64_t>(p.n) * a.out_sn + p.oh * a.out_sh +
-                      p.ow * a.out_sw + oc_lane;
-        res_off[pb] = batch * a.batch_res + static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh +
-                      p.ow * a.res_sw + oc_lane;
+        e.valid[pb] = m[pb] < a.M;
+        const PixelCoord p = decode_pixel(a, e.valid[pb] ? m[pb] : a.M - 1);
+        e.out_off[pb] = batch * a.batch_out + static_cast<int64_t>(p.n) * a.out_sn + p.oh * a.out_sh +
+                        p.ow * a.out_sw + oc_lane;
+        e.res_off[pb] = batch * a.batch_res + static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh +
+                        p.ow * a.res_sw + oc_lane;
     }
-    epilogue<F>(a, acc, oc_lane, valid, out_off, res_off, rres, sp, sp_stride, oc0);
 }
 
 template <uint32_t F>
 __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
-                                             int m0, int m1, int batch = 0, const float* sp = nullptr,
+                                             int m0, int m1, int batch, const v16f (&rres)[2][2],
+                                             lds_cfloat_ptr sp = nullptr, int sp_stride = 0, int oc0 = 0) {
+    EpiAddr e;
+    epilogue_addresses(a, oc_lane, m0, m1, batch, e);
+    epilogue<F>(a, acc, oc_lane, e.valid, e.out_off, e.res_off, rres, sp, sp_stride, oc0);
+}
+
+template <uint32_t F>
+__device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
+                                             int m0, int m1, int batch = 0, lds_cfloat_ptr sp = nullptr,
                                              int sp_stride = 0, int oc0 = 0) {
     v16f none[2][2];
     run_epilogue<F>(a, acc, oc_lane, m0, m1, batch, none, sp, sp_stride, oc0);

@@ -163,6 +163,67 @@ def test_conv_nonzero_input_low_and_ties(orc):
     np.testing.assert_array_equal(out.to_nchw(), want)
 
 
+_VARIANT_CASES = {}
+
+
+def _variant_case(orc, kind):
+    """One large layer per epilogue kind (enough pixel tiles that a persistent workgroup walks several),
+    evaluated once by the oracle."""
+    if kind in _VARIANT_CASES:
+        return _VARIANT_CASES[kind]
+    from dldt_amd import make_epilogue
+    rng = np.random.default_rng(zlib.crc32(kind.encode()))
+    if kind == "plain_3x3":
+        g = (4, 16, 184, 184, 64, 3, 3, (1, 1), (1, 1), (1, 1), (1, 1))
+    else:
+        g = (4, 64, 184, 184, 64, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0))
+    x, w = _inputs(rng, g)
+    OC = g[4]
+    acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    amax = np.float32(np.abs(acc).max())
+    bias = rng.normal(0, amax / 20, OC).astype(np.float32)
+    ih = rng.uniform(0.3, 1.0, OC).astype(np.float32) * amax
+    res = None
+    if kind in ("plain", "plain_3x3"):
+        fq = (256, np.zeros(OC, np.float32), ih, 0.0, 255.0)
+        want = _chain(orc, acc, bias=bias, fq=fq)
+        epi = dict(bias=bias, out_dtype=U8B, fq=fq)
+    elif kind == "plain_il":
+        fq = (256, -ih / 3, ih, 0.0, 255.0)
+        want = _chain(orc, acc, bias=bias, fq=fq)
+        epi = dict(bias=bias, out_dtype=U8B, fq=fq)
+    elif kind == "res_u8":
+        scale = (rng.uniform(0.5, 2.0, OC) / amax).astype(np.float32)
+        res = rng.integers(0, 256, acc.shape).astype(np.int32)
+        s_x = rng.uniform(0.002, 0.004, OC).astype(np.float32)
+        fq = (256, 0.0, np.float32(1.7), 0.0, 255.0)
+        want = _chain(orc, acc, bias=bias, scale=scale, res=res, res_scale=s_x, fq=fq)
+        epi = dict(bias=bias, scale=scale, residual_dtype=U8B, res_mul=s_x, out_dtype=U8B, fq=fq)
+    else:   # "clamp": MobileNetV2 pointwise + ReLU6
+        scale = (rng.uniform(2.0, 6.0, OC) / amax).astype(np.float32)
+        fq = (256, 0.0, np.float32(6.0), 0.0, 255.0)
+        want = _chain(orc, acc, bias=bias, scale=scale, act="clamp", clamp=(0.0, 6.0), fq=fq)
+        epi = dict(bias=bias, scale=scale, activation="clamp", clamp=(0.0, 6.0), out_dtype=U8B, fq=fq)
+    _VARIANT_CASES[kind] = (g, x, w, res, epi, want.astype(np.uint8))
+    return _VARIANT_CASES[kind]
+
+
+@pytest.mark.parametrize("tile", [0, 1, 4, 5, 8, 9])
+@pytest.mark.parametrize("kind", ["plain", "plain_3x3", "plain_il", "res_u8", "clamp"])
+def test_conv_kernel_variants_give_the_reference_bytes(orc, kind, tile):
+    """Every kernel variant the tuner may pick, on layers of 135 424 pixels (529 or 1058 pixel tiles:
+    the persistent variants walk several tiles per workgroup), against the oracle's fused chain."""
+    from dldt_amd import Convolution, DeviceTensor, make_epilogue
+    g, x, w, res, epi, want = _variant_case(orc, kind)
+    xin = _device_in(x, g)
+    conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10], make_epilogue(**epi))
+    conv.set_tile(tile)
+    out = DeviceTensor(want.shape[0], want.shape[2], want.shape[3], want.shape[1], U8B)
+    rt = DeviceTensor.from_nchw(res, U8B) if res is not None else None
+    conv.run(xin, out, rt)
+    np.testing.assert_array_equal(out.to_nchw(), want)
+
+
 @pytest.mark.parametrize("res_kind", ["u8", "f32"])
 def test_conv_residual_add_relu_requantize(orc, res_kind):
     """Bottleneck tail: (acc + b') * s[c] + residual -> ReLU -> FQ, residual either the u8 block
