@@ -21,7 +21,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     constexpr int A_PIECES = BOC * 4 / NT, B_PIECES = BPIX * 4 / NT;
     __shared__ __attribute__((aligned(16))) int8_t sA[2][BOC * kRow];
     __shared__ __attribute__((aligned(16))) int8_t sB[2][BPIX * kRow];
-    __shared__ __attribute__((aligned(16))) float sP[PT_COUNT * BOC];
+    __shared__ __attribute__((aligned(16))) float sP[PT_ROWS * BOC];
 
     // block -> (pixel tile, channel tile): consecutive pixel tiles stay on one XCD
     const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
@@ -36,7 +36,9 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     const int chunk = tid & 3;
 
     const int batch = blockIdx.y;
-    stage_params<F>(a, oc0, (lds_float_ptr)sP, BOC, tid, NT);   // visible after the first barrier of the K loop
+    static_assert(BOC <= NT, "one table element per thread");
+    StagedParams staged;
+    stage_params_load<F>(a, oc0, BOC, tid, staged);   // awaited only after the first K step has been requested
     const int a_row[2] = {woc * 64 + l32, woc * 64 + 32 + l32};
     const int b_row[2] = {wpix * 64 + l32, wpix * 64 + 32 + l32};
     const int oc_lane = oc0 + woc * 64 + 32 * h;
@@ -44,7 +46,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     // one implicit GEMM over an operand set (activation tensor, packed weights, K-offset table)
     auto gemm = [&](const int8_t* in_base, int in_sn, int in_sh, int in_sw, int csh, int csw, int origin,
                     const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk,
-                    v16i (&acc)[2][2]) {
+                    v16i (&acc)[2][2], bool first, bool acc_from_lds) {
         int32_t b_base[B_PIECES];
         const int8_t* a_ptr[A_PIECES];
 #pragma unroll
@@ -83,7 +85,9 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
         };
         load_global(0);
         store_lds(0);
+        if (first) stage_params_store<F>(a, (lds_float_ptr)sP, BOC, tid, staged);
         __syncthreads();
+        if (acc_from_lds) init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);
         for (int k = 0; k < nk; ++k) {
             const int buf = k & 1;
             if (k + 1 < nk) load_global(k + 1);
@@ -116,7 +120,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
         a2.corr = a.corr2;
         init_acc(a2, oc_lane, acc);
         gemm(a.in2, a.in2_sn, a.in2_sh, a.in2_sw, a.conv2_sh, a.conv2_sw, a.in2_origin, a.wgt2, a.Kp2, a.OCp, false,
-             a.koff2, a.nk2, acc);
+             a.koff2, a.nk2, acc, true, false);
 #pragma unroll
         for (int ob = 0; ob < 2; ++ob)
 #pragma unroll
@@ -133,14 +137,13 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
                     }
             }
     }
-    init_acc(a, oc_lane, acc);
+    if (kFused) init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);   // published by the shortcut GEMM's first barrier
     gemm(a.in + batch * a.batch_in, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
-         a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc);
+         a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused);
     const int m0 = pix0 + wpix * 64 + l32;
     run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, (lds_cfloat_ptr)sP, BOC, oc0);
 }
 
-// ------------------------------------------------------------------------------------------------
 // Persistent LDS-tiled kernel for the layers whose time is the epilogue and the memory latency
 // around it (small K): a workgroup keeps its channel tile and walks pixel tiles.  The operands of
 // the next tile's first K step and the next tile's residual bytes are requested before the
@@ -155,7 +158,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const C
     constexpr bool kByteRes = (F & CF_RES) && !(F & (CF_RES_F32 | CF_RES_GEMM));
     __shared__ __attribute__((aligned(16))) int8_t sA[2][BOC * kRow];
     __shared__ __attribute__((aligned(16))) int8_t sB[2][BPIX * kRow];
-    __shared__ __attribute__((aligned(16))) float sP[PT_COUNT * BOC];
+    __shared__ __attribute__((aligned(16))) float sP[PT_ROWS * BOC];
 
     const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
     const int t_tile = y % a.t_tiles;
@@ -168,7 +171,10 @@ __global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const C
     const int woc = wave % WOC, wpix = wave / WOC;
     const int l32 = lane & 31, h = lane >> 5;
     const int chunk = tid & 3;
-    stage_params<F>(a, oc0, (lds_float_ptr)sP, BOC, tid, NT);   // visible after the first barrier
+    static_assert(BOC <= NT, "one table element per thread");
+    StagedParams staged;
+    stage_params_load<F>(a, oc0, BOC, tid, staged);
+    bool first = true;
     const int a_row[2] = {woc * 64 + l32, woc * 64 + 32 + l32};
     const int b_row[2] = {wpix * 64 + l32, wpix * 64 + 32 + l32};
     const int oc_lane = oc0 + woc * 64 + 32 * h;
@@ -222,9 +228,11 @@ __global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const C
     v16f none[2][2];
     while (true) {
         v16i acc[2][2];
-        init_acc(a, oc_lane, acc);
         store_lds(0);
+        if (first) stage_params_store<F>(a, (lds_float_ptr)sP, BOC, tid, staged);
+        first = false;
         __syncthreads();
+        init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);
         const int next_p = p_local + n_per;
         const bool has_next = tile_exists(next_p);
         for (int k = 0; k < nk; ++k) {
@@ -363,7 +371,7 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
         }
         // The K-offset table lives in LDS behind the ring: a vector-memory load of it would have to
         // be awaited with vmcnt(0), which drains every DMA load in flight and serialises the ring.
-        int32_t* kt = reinterpret_cast<int32_t*>(ring + KS * stages * STAGE + PT_COUNT * BOC * 4);
+        int32_t* kt = reinterpret_cast<int32_t*>(ring + KS * stages * STAGE + PT_ROWS * BOC * 4);
         for (int i = tid; i < 4 * nk_all; i += NT_ALL) kt[i] = koff[i];
         __syncthreads();
         int32_t off_next = kt[4 * grp + dma_chunk];
@@ -630,7 +638,7 @@ void launch_tiled(const ConvArgs& a, hipStream_t s, int batches = 1) {
 template <int WOC, int WPIX, int KS>
 void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) {
     const dim3 grid(8 * a.p_per_xcd * a.t_tiles, batches), block(WOC * WPIX * 64 * KS);
-    const size_t lds = static_cast<size_t>(KS) * stages * (WOC + WPIX) * 64 * 64 + PT_COUNT * WOC * 64 * 4 +
+    const size_t lds = static_cast<size_t>(KS) * stages * (WOC + WPIX) * 64 * 64 + PT_ROWS * WOC * 64 * 4 +
                        16 * static_cast<size_t>(std::max(a.nk, a.nk2));
     const uint32_t core = a.flags & ~CF_OUT_XOR;
 #define HIPIE_LAUNCH_PIPE(FLAGS, ...)                                                                       \
@@ -680,7 +688,7 @@ void launch_tiled_small(const ConvArgs& a, hipStream_t s) {   // 64 x 64 tile, o
 
 void launch_stream(const ConvArgs& a, int grid_x, hipStream_t s) {
     const dim3 grid(grid_x, a.t_tiles), block(256);
-    const size_t lds = static_cast<size_t>(64) * (a.Kp + 16) + PT_COUNT * 64 * 4;
+    const size_t lds = static_cast<size_t>(64) * (a.Kp + 16) + PT_ROWS * 64 * 4;
     const uint32_t core = a.flags & ~CF_OUT_XOR;
 #define HIPIE_LAUNCH_STREAM(FLAGS, ...) \
     hipLaunchKernelGGL((conv_stream_kernel<FLAGS>), grid, block, lds, s, a)
@@ -1099,7 +1107,7 @@ int hipie_conv_set_tile(hipie_conv* c, int tile) {
                       "hipie_conv_set_tile: the persistent kernels exist for byte outputs with a byte residual or none");
         HIPIE_REQUIRE(tile < 6 || tile > 7 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the split-K kernels need an even number of 64-byte K steps (K=%lld)", (long long)c->Kp);
-        HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) + PT_COUNT * 64 * 4 <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
+        HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) + PT_ROWS * 64 * 4 <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: K=%lld does not fit the streaming kernel's LDS", (long long)c->Kp);
         c->tile = tile;
     });
@@ -1271,7 +1279,7 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         default: {
             // persistent workgroups: as many as fit per CU by LDS (at most 4), spread over the
             // channel tiles; a multiple of 8 so that sibling channel tiles share an XCD
-            const int64_t lds = 64 * (c->Kp + 16) + PT_COUNT * 64 * 4;
+            const int64_t lds = 64 * (c->Kp + 16) + PT_ROWS * 64 * 4;
             const int per_cu = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(4, (160 * 1024) / lds)));
             int64_t gx = std::max<int64_t>(8, (256 * per_cu) / a.t_tiles);
             gx = std::min<int64_t>(round_up(gx, 8), round_up(a.p_tiles, 8));

@@ -104,27 +104,109 @@ typedef const __attribute__((address_space(3))) float* lds_cfloat_ptr;   // keep
 typedef __attribute__((address_space(3))) float* lds_float_ptr;
 
 enum ParamTable { PT_BIAS, PT_SCALE, PT_RSUB, PT_RMUL, PT_POST, PT_IL, PT_IH, PT_D, PT_R, PT_R2, PT_COUNT };
+constexpr int PT_ROWS = PT_COUNT + 1;   // plus the row of integer accumulator corrections
+
+// Two phases so that the caller can put its operand loads between them: the table loads must not
+// be awaited (for the LDS writes) before the first K step has been requested.
+struct StagedParams {
+    float v[PT_COUNT];
+    int32_t corr;
+};
 
 template <uint32_t F>
-__device__ __forceinline__ void stage_params(const ConvArgs& a, int oc0, lds_float_ptr sp, int stride, int tid, int nt) {
+__device__ __forceinline__ void stage_params_load(const ConvArgs& a, int oc0, int stride, int tid, StagedParams& r) {
     const uint32_t fl = F == kDyn ? a.flags : F;
-    auto put = [&](int t, const float* src) {
-        for (int c = tid; c < stride; c += nt) sp[t * stride + c] = src[oc0 + c];
-    };
-    if (fl & CF_BIAS) put(PT_BIAS, a.bias);
-    if (fl & CF_SCALE) put(PT_SCALE, a.scale);
-    if (fl & CF_RES_SUB) put(PT_RSUB, a.res_sub);
-    if (fl & CF_RES_MUL) put(PT_RMUL, a.res_mul);
-    if (fl & CF_POST_SCALE) put(PT_POST, a.post_scale);
+    const int c = oc0 + (tid < stride ? tid : 0);
+    auto get = [&](int t, const float* src) { r.v[t] = src[c]; };
+    r.corr = a.corr[c];
+    if (fl & CF_BIAS) get(PT_BIAS, a.bias);
+    if (fl & CF_SCALE) get(PT_SCALE, a.scale);
+    if (fl & CF_RES_SUB) get(PT_RSUB, a.res_sub);
+    if (fl & CF_RES_MUL) get(PT_RMUL, a.res_mul);
+    if (fl & CF_POST_SCALE) get(PT_POST, a.post_scale);
     if (fl & CF_OUT_FQ) {
-        put(PT_IH, a.fq_ih);
-        if (fl & CF_FQ_RCP) put(PT_R, a.fq_r);
-        if (fl & CF_FQ_DIV2) put(PT_R2, a.fq_r2);
+        get(PT_IH, a.fq_ih);
+        if (fl & CF_FQ_RCP) get(PT_R, a.fq_r);
+        if (fl & CF_FQ_DIV2) get(PT_R2, a.fq_r2);
         if (!(fl & CF_FQ_IL0)) {
-            put(PT_IL, a.fq_il);
-            put(PT_D, a.fq_d);
+            get(PT_IL, a.fq_il);
+            get(PT_D, a.fq_d);
         }
     }
+}
+
+// rows PT_BIAS .. PT_R2 of `stride` floats, then one row of the integer accumulator corrections
+template <uint32_t F>
+__device__ __forceinline__ void stage_params_store(const ConvArgs& a, lds_float_ptr sp, int stride, int tid,
+                                                   const StagedParams& r) {
+    const uint32_t fl = F == kDyn ? a.flags : F;
+    if (tid >= stride) return;
+    auto put = [&](int t) { sp[t * stride + tid] = r.v[t]; };
+    ((__attribute__((address_space(3))) int32_t*)sp)[PT_COUNT * stride + tid] = r.corr;
+    if (fl & CF_BIAS) put(PT_BIAS);
+    if (fl & CF_SCALE) put(PT_SCALE);
+    if (fl & CF_RES_SUB) put(PT_RSUB);
+    if (fl & CF_RES_MUL) put(PT_RMUL);
+    if (fl & CF_POST_SCALE) put(PT_POST);
+    if (fl & CF_OUT_FQ) {
+        put(PT_IH);
+        if (fl & CF_FQ_RCP) put(PT_R);
+        if (fl & CF_FQ_DIV2) put(PT_R2);
+        if (!(fl & CF_FQ_IL0)) {
+            put(PT_IL);
+            put(PT_D);
+        }
+    }
+}
+
+// single-phase form (threads tid, tid + nt, ... of a workgroup of nt threads)
+template <uint32_t F>
+__device__ __forceinline__ void stage_params(const ConvArgs& a, int oc0, lds_float_ptr sp, int stride, int tid, int nt) {
+    for (int t0 = 0; t0 < stride; t0 += nt) {
+        StagedParams r;
+        const int t = t0 + tid;
+        if (t < stride) {   // uniform for all but the last round
+            stage_params_load<F>(a, oc0 + t0, stride - t0, tid, r);
+            // rows are indexed by the channel inside the tile
+            lds_float_ptr base = sp + t0;
+            const uint32_t fl = F == kDyn ? a.flags : F;
+            auto put = [&](int tb) { base[tb * stride + tid] = r.v[tb]; };
+            ((__attribute__((address_space(3))) int32_t*)sp)[PT_COUNT * stride + t] = r.corr;
+            if (fl & CF_BIAS) put(PT_BIAS);
+            if (fl & CF_SCALE) put(PT_SCALE);
+            if (fl & CF_RES_SUB) put(PT_RSUB);
+            if (fl & CF_RES_MUL) put(PT_RMUL);
+            if (fl & CF_POST_SCALE) put(PT_POST);
+            if (fl & CF_OUT_FQ) {
+                put(PT_IH);
+                if (fl & CF_FQ_RCP) put(PT_R);
+                if (fl & CF_FQ_DIV2) put(PT_R2);
+                if (!(fl & CF_FQ_IL0)) {
+                    put(PT_IL);
+                    put(PT_D);
+                }
+            }
+        }
+    }
+}
+
+// accumulators from the staged corrections (after the barrier that publishes them)
+__device__ __forceinline__ void init_acc_lds(lds_cfloat_ptr sp, int stride, int oc_local, v16i (&acc)[2][2]) {
+    const __attribute__((address_space(3))) int32_t* corr =
+        (const __attribute__((address_space(3))) int32_t*)sp + PT_COUNT * stride + oc_local;
+#pragma unroll
+    for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const v4i c = *(const __attribute__((address_space(3))) v4i*)(corr + 16 * ob + 4 * q);
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) {
+                acc[ob][pb][4 * q + 0] = c.x;
+                acc[ob][pb][4 * q + 1] = c.y;
+                acc[ob][pb][4 * q + 2] = c.z;
+                acc[ob][pb][4 * q + 3] = c.w;
+            }
+        }
 }
 
 struct EpiParams {
