@@ -81,6 +81,31 @@ __global__ __launch_bounds__(kThreads) void gelu_erf(const float* __restrict__ x
     }
 }
 
+// Batched 2-D transpose of bytes through a 64 x 64 LDS tile (row stride 65 words would not help
+// bytes: rows are read as 16-byte pieces and written back byte-wise from a 64 x 65 tile).
+// dst[b][c][r] = src[b][r][c]; the two inner dimensions of a Transpose node on an i8 tensor
+// (reference::transpose, transpose.hpp:20-25, moves elements only).
+__global__ __launch_bounds__(256) void transpose_bytes_kernel(const int8_t* __restrict__ src, int64_t ld_src,
+                                                              int64_t bs_src, int8_t* __restrict__ dst, int64_t ld_dst,
+                                                              int64_t bs_dst, int rows, int cols) {
+    __shared__ int8_t tile[64][65];
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int8_t* s = src + static_cast<int64_t>(blockIdx.z) * bs_src;
+    int8_t* d = dst + static_cast<int64_t>(blockIdx.z) * bs_dst;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int r = r0 + ty * 16 + i, c = c0 + tx;
+        tile[ty * 16 + i][tx] = (r < rows && c < cols) ? s[static_cast<int64_t>(r) * ld_src + c] : int8_t(0);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int c = c0 + ty * 16 + i, r = r0 + tx;
+        if (c < cols && r < rows) d[static_cast<int64_t>(c) * ld_dst + r] = tile[tx][ty * 16 + i];
+    }
+}
+
 }  // namespace
 }  // namespace hipie
 
@@ -118,6 +143,20 @@ int hipie_gelu_f32(const float* x, float* y, int64_t n, void* stream) {
         HIPIE_REQUIRE(x && y && n > 0, HIPIE_PARAMETER_MISMATCH, "hipie_gelu_f32: bad argument");
         const int64_t blocks = std::min<int64_t>(ceil_div(n, kThreads), 256 * 16);
         hipLaunchKernelGGL(gelu_erf, dim3(static_cast<uint32_t>(blocks)), dim3(kThreads), 0, as_stream(stream), x, y, n);
+        HIPIE_CHECK_HIP(hipGetLastError());
+    });
+}
+
+int hipie_transpose_bytes(const void* src, int64_t ld_src, int64_t batch_stride_src, void* dst, int64_t ld_dst,
+                          int64_t batch_stride_dst, int32_t rows, int32_t cols, int32_t batch, void* stream) {
+    return guarded([&] {
+        if (rows == 0 || cols == 0 || batch == 0) return;
+        HIPIE_REQUIRE(src && dst && rows > 0 && cols > 0 && batch > 0 && batch < 65536 && ld_src >= cols && ld_dst >= rows,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_transpose_bytes: bad argument");
+        const dim3 grid(static_cast<uint32_t>(ceil_div(cols, 64)), static_cast<uint32_t>(ceil_div(rows, 64)),
+                        static_cast<uint32_t>(batch));
+        hipLaunchKernelGGL(transpose_bytes_kernel, grid, dim3(256), 0, as_stream(stream), static_cast<const int8_t*>(src),
+                           ld_src, batch_stride_src, static_cast<int8_t*>(dst), ld_dst, batch_stride_dst, rows, cols);
         HIPIE_CHECK_HIP(hipGetLastError());
     });
 }

@@ -250,6 +250,12 @@ int hipie_softmax_f32(const float* x, float* y, int64_t rows, int64_t axis, void
 int hipie_mvn_f32(const float* x, float* y, int64_t rows, int64_t axis, int normalize_variance, float eps,
                   int eps_inside_sqrt, const float* gamma, const float* beta, void* stream);
 int hipie_gelu_f32(const float* x, float* y, int64_t n, void* stream);
+/* Transpose of the two inner dimensions of a byte tensor (opset1 Transpose on quantized activations,
+ * e.g. V [S, d] -> [d, S] so that the context MatMul finds its reduction axis contiguous;
+ * reference::transpose, .../reference/transpose.hpp:20-25): dst[b][c][r] = src[b][r][c], leading
+ * dimensions and batch strides in bytes. */
+int hipie_transpose_bytes(const void* src, int64_t ld_src, int64_t batch_stride_src, void* dst, int64_t ld_dst,
+                          int64_t batch_stride_dst, int32_t rows, int32_t cols, int32_t batch, void* stream);
 
 /* ======================================================================================
  * 2. Graph level.  The plugin's LoadExeNetworkImpl walks Function::get_ordered_ops()
