@@ -126,16 +126,16 @@ class EncoderLayer:
         self.lin["qkv"].run(d["xq"], d["qkv"])
         qkv = flat(d["qkv"])
         base = qkv.data_ptr()
-        for b in range(B):   # heads of one sequence are a strided batch inside [T, 3H]
-            row = base + b * S * 3 * H
-            matmul_strided(self.mm_scores, row, 3 * H, 64, row + H, 3 * H, 64,
-                           self.scores[b].data_ptr(), S, S * S, S, NH)
-            transpose_bytes(row + 2 * H, 3 * H, 64, self.vt[b].data_ptr(), S, 64 * S, S, 64, NH)
+        # (sequence, head) is a two-level batch inside [T, 3H]: heads 64 columns apart, sequences S rows apart
+        matmul_strided(self.mm_scores, base, 3 * H, 64, base + H, 3 * H, 64, self.scores.data_ptr(), S, S * S, S, NH,
+                       batch_outer=B, outer_a=S * 3 * H, outer_b=S * 3 * H, outer_o=NH * S * S)
+        transpose_bytes(base + 2 * H, 3 * H, 64, self.vt.data_ptr(), S, 64 * S, S, 64, NH,
+                        batch_outer=B, outer_src=S * 3 * H, outer_dst=NH * 64 * S)
         p = softmax(self.scores.view(B * NH * S, S))
         self.fq["p"].run_q8(p.view(1, 1, B * NH * S, S), "i8", "nchw", out=self.pq.view(1, 1, B * NH * S, S))
-        for b in range(B):   # context written straight into [T, H] at its head's columns
-            matmul_strided(self.mm_ctx, self.pq[b].data_ptr(), S, S * S, self.vt[b].data_ptr(), S, 64 * S,
-                           self.ctx.data_ptr() + b * S * H * 4, H, 64, S, NH)
+        # context written straight into [T, H] at its head's columns
+        matmul_strided(self.mm_ctx, self.pq.data_ptr(), S, S * S, self.vt.data_ptr(), S, 64 * S, self.ctx.data_ptr(), H, 64,
+                       S, NH, batch_outer=B, outer_a=NH * S * S, outer_b=NH * 64 * S, outer_o=S * H)
         self.fq["ctx"].run_q8(q4(self.ctx, H), "i8", "nchw", out=q4(flat(d["ctxq"]), H))
         self.lin["o"].run(d["ctxq"], d["attn"], d["x"])
         h1 = mvn(flat(d["attn"]), gamma=self.g[0][0], beta=self.g[0][1])

@@ -138,8 +138,8 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
             }
     }
     if (kFused) init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);   // published by the shortcut GEMM's first barrier
-    gemm(a.in + batch * a.batch_in, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
-         a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused);
+    gemm(a.in + batch_offset(a, batch, a.batch_in, a.batch_in_o), a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
+         a.wgt + batch_offset(a, batch, a.batch_wgt, a.batch_wgt_o), a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused);
     const int m0 = pix0 + wpix * 64 + l32;
     run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, (lds_cfloat_ptr)sP, BOC, oc0);
 }
@@ -616,6 +616,8 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
     case E_RESGEMM: X(E_RESGEMM, __VA_ARGS__); break;                                        \
     case E_F32: X(E_F32, __VA_ARGS__); break;                                                \
     case E_SCALE: X(E_SCALE, __VA_ARGS__); break;                                            \
+    case E_SCALEFQ: X(E_SCALEFQ, __VA_ARGS__); break;                                        \
+    case E_F32RES: X(E_F32RES, __VA_ARGS__); break;                                          \
     case E_F32RELU: X(E_F32RELU, __VA_ARGS__); break;                                        \
     case E_CLAMPFQ: X(E_CLAMPFQ, __VA_ARGS__); break;                                        \
     case E_PLAIN0 & ~CF_FQ_DIV2: X((E_PLAIN0 & ~CF_FQ_DIV2), __VA_ARGS__); break;            \
@@ -942,11 +944,21 @@ void hipie_matmul_destroy(hipie_matmul* m) { delete m; }
 int hipie_matmul_run(const hipie_matmul* mm, const void* a_ptr, int64_t lda, int64_t stride_a, const void* bt_ptr,
                      int64_t ldb, int64_t stride_b, void* out, int64_t ldo, int64_t stride_o, int32_t m,
                      int32_t batch, void* stream) {
+    return hipie_matmul_run_nested(mm, a_ptr, lda, stride_a, 0, bt_ptr, ldb, stride_b, 0, out, ldo, stride_o, 0, m, batch,
+                                   1, stream);
+}
+
+int hipie_matmul_run_nested(const hipie_matmul* mm, const void* a_ptr, int64_t lda, int64_t stride_a, int64_t outer_a,
+                            const void* bt_ptr, int64_t ldb, int64_t stride_b, int64_t outer_b, void* out, int64_t ldo,
+                            int64_t stride_o, int64_t outer_o, int32_t m, int32_t batch, int32_t batch_outer,
+                            void* stream) {
     return guarded([&] {
         HIPIE_REQUIRE(mm, HIPIE_PARAMETER_MISMATCH, "hipie_matmul_run: null handle");
         HIPIE_REQUIRE(mm->koff.ptr, HIPIE_NOT_ALLOCATED, "hipie_matmul_run: host-only object");
-        if (m == 0 || batch == 0) return;
-        HIPIE_REQUIRE(a_ptr && bt_ptr && out && m > 0 && batch > 0, HIPIE_PARAMETER_MISMATCH,
+        if (m == 0 || batch == 0 || batch_outer == 0) return;
+        HIPIE_REQUIRE(a_ptr && bt_ptr && out && m > 0 && batch > 0 && batch_outer > 0 &&
+                          static_cast<int64_t>(batch) * batch_outer < 65536 && outer_a % 16 == 0 && outer_b % 16 == 0,
+                      HIPIE_PARAMETER_MISMATCH,
                       "hipie_matmul_run: null operand or negative size");
         const hipie_matmul_desc& d = mm->d;
         const bool byte_out = mm->epi.out_dtype == HIPIE_U8B || mm->epi.out_dtype == HIPIE_I8;
@@ -988,14 +1000,18 @@ int hipie_matmul_run(const hipie_matmul* mm, const void* a_ptr, int64_t lda, int
         a.batch_in = stride_a;
         a.batch_wgt = stride_b;
         a.batch_out = stride_o;
+        a.batch_inner = batch_outer > 1 ? batch : 0;
+        a.batch_in_o = outer_a;
+        a.batch_wgt_o = outer_b;
+        a.batch_out_o = outer_o;
         const bool wide = d.n > 64;
         const int boc = wide ? 128 : 64, bpix = wide ? 128 : 256;
         a.p_tiles = static_cast<int32_t>(ceil_div(m, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.n, boc));
         a.p_per_xcd = static_cast<int32_t>(ceil_div(a.p_tiles, 8));
         DeviceGuard g(mm->device);
-        if (wide) launch_tiled<2, 2>(a, as_stream(stream), batch);
-        else launch_tiled<1, 4>(a, as_stream(stream), batch);
+        if (wide) launch_tiled<2, 2>(a, as_stream(stream), batch * batch_outer);
+        else launch_tiled<1, 4>(a, as_stream(stream), batch * batch_outer);
         HIPIE_CHECK_HIP(hipGetLastError());
     });
 }

@@ -22,6 +22,13 @@ __device__ __forceinline__ void fast_divmod(int m, int d, float inv_d, int& q, i
 
 struct PixelCoord { int n, oh, ow; };
 
+// offset of batch element `batch` for an operand with inner stride `stride` and outer stride `outer`
+__device__ __forceinline__ int64_t batch_offset(const ConvArgs& a, int batch, int64_t stride, int64_t outer) {
+    if (a.batch_inner <= 0) return batch * stride;
+    const int o = batch / a.batch_inner;
+    return o * outer + (batch - o * a.batch_inner) * stride;
+}
+
 __device__ __forceinline__ PixelCoord decode_pixel(const ConvArgs& a, int m) {
     PixelCoord p;
     int rem;
@@ -92,7 +99,9 @@ constexpr uint32_t E_RESU8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_U8B | CF_RES_M
 constexpr uint32_t E_RESF32 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32 | E_FQ | CF_FQ_IL0;
 constexpr uint32_t E_RESGEMM = CF_BIAS | CF_SCALE | CF_RES | CF_RES_GEMM | E_FQ | CF_FQ_IL0;
 constexpr uint32_t E_F32 = CF_BIAS | CF_SCALE;
-constexpr uint32_t E_SCALE = CF_SCALE;                      // MatMul' -> Multiply(s_a * s_b)
+constexpr uint32_t E_SCALE = CF_SCALE;
+constexpr uint32_t E_SCALEFQ = CF_BIAS | CF_SCALE | E_FQ;              // linear layer requantised to symmetric i8
+constexpr uint32_t E_F32RES = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32;   // linear layer + f32 residual, f32 out                      // MatMul' -> Multiply(s_a * s_b)
 constexpr uint32_t E_F32RELU = CF_BIAS | CF_SCALE | CF_RELU;
 constexpr uint32_t E_CLAMPFQ = CF_BIAS | CF_SCALE | CF_CLAMP | E_FQ | CF_FQ_IL0;
 
@@ -441,7 +450,7 @@ __device__ __forceinline__ void epilogue_addresses(const ConvArgs& a, int oc_lan
     for (int pb = 0; pb < 2; ++pb) {
         e.valid[pb] = m[pb] < a.M;
         const PixelCoord p = decode_pixel(a, e.valid[pb] ? m[pb] : a.M - 1);
-        e.out_off[pb] = batch * a.batch_out + static_cast<int64_t>(p.n) * a.out_sn + p.oh * a.out_sh +
+        e.out_off[pb] = batch_offset(a, batch, a.batch_out, a.batch_out_o) + static_cast<int64_t>(p.n) * a.out_sn + p.oh * a.out_sh +
                         p.ow * a.out_sw + oc_lane;
         e.res_off[pb] = batch * a.batch_res + static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh +
                         p.ow * a.res_sw + oc_lane;

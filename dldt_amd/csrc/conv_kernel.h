@@ -85,6 +85,10 @@ struct ConvArgs {
     // wgt_plain = rows are in natural order (activation operand): the loader applies the MFMA
     // row permutation that constant weights carry from packing
     int64_t batch_in, batch_wgt, batch_out, batch_res;
+    // two-level batches (sequence, head): batch index y -> (y / batch_inner) * outer stride + (y % batch_inner) * stride;
+    // batch_inner = 0 means one level
+    int32_t batch_inner;
+    int64_t batch_in_o, batch_wgt_o, batch_out_o;
     int32_t wgt_ld, wgt_rows, wgt_plain;
     // fused shortcut convolution (CF_RES_GEMM): a second operand set accumulated first; its
     // dequantised result stays in registers as the residual of the main convolution

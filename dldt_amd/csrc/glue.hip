@@ -86,12 +86,14 @@ __global__ __launch_bounds__(kThreads) void gelu_erf(const float* __restrict__ x
 // dst[b][c][r] = src[b][r][c]; the two inner dimensions of a Transpose node on an i8 tensor
 // (reference::transpose, transpose.hpp:20-25, moves elements only).
 __global__ __launch_bounds__(256) void transpose_bytes_kernel(const int8_t* __restrict__ src, int64_t ld_src,
-                                                              int64_t bs_src, int8_t* __restrict__ dst, int64_t ld_dst,
-                                                              int64_t bs_dst, int rows, int cols) {
+                                                              int64_t bs_src, int64_t os_src, int8_t* __restrict__ dst,
+                                                              int64_t ld_dst, int64_t bs_dst, int64_t os_dst, int rows,
+                                                              int cols, int batch_inner) {
     __shared__ int8_t tile[64][65];
     const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-    const int8_t* s = src + static_cast<int64_t>(blockIdx.z) * bs_src;
-    int8_t* d = dst + static_cast<int64_t>(blockIdx.z) * bs_dst;
+    const int bo = blockIdx.z / batch_inner, bi = blockIdx.z - bo * batch_inner;
+    const int8_t* s = src + bo * os_src + bi * bs_src;
+    int8_t* d = dst + bo * os_dst + bi * bs_dst;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -149,14 +151,23 @@ int hipie_gelu_f32(const float* x, float* y, int64_t n, void* stream) {
 
 int hipie_transpose_bytes(const void* src, int64_t ld_src, int64_t batch_stride_src, void* dst, int64_t ld_dst,
                           int64_t batch_stride_dst, int32_t rows, int32_t cols, int32_t batch, void* stream) {
+    return hipie_transpose_bytes_nested(src, ld_src, batch_stride_src, 0, dst, ld_dst, batch_stride_dst, 0, rows, cols,
+                                        batch, 1, stream);
+}
+
+int hipie_transpose_bytes_nested(const void* src, int64_t ld_src, int64_t stride_src, int64_t outer_src, void* dst,
+                                 int64_t ld_dst, int64_t stride_dst, int64_t outer_dst, int32_t rows, int32_t cols,
+                                 int32_t batch, int32_t batch_outer, void* stream) {
     return guarded([&] {
-        if (rows == 0 || cols == 0 || batch == 0) return;
-        HIPIE_REQUIRE(src && dst && rows > 0 && cols > 0 && batch > 0 && batch < 65536 && ld_src >= cols && ld_dst >= rows,
+        if (rows == 0 || cols == 0 || batch == 0 || batch_outer == 0) return;
+        HIPIE_REQUIRE(src && dst && rows > 0 && cols > 0 && batch > 0 && batch_outer > 0 &&
+                          static_cast<int64_t>(batch) * batch_outer < 65536 && ld_src >= cols && ld_dst >= rows,
                       HIPIE_PARAMETER_MISMATCH, "hipie_transpose_bytes: bad argument");
         const dim3 grid(static_cast<uint32_t>(ceil_div(cols, 64)), static_cast<uint32_t>(ceil_div(rows, 64)),
-                        static_cast<uint32_t>(batch));
+                        static_cast<uint32_t>(batch * batch_outer));
         hipLaunchKernelGGL(transpose_bytes_kernel, grid, dim3(256), 0, as_stream(stream), static_cast<const int8_t*>(src),
-                           ld_src, batch_stride_src, static_cast<int8_t*>(dst), ld_dst, batch_stride_dst, rows, cols);
+                           ld_src, stride_src, outer_src, static_cast<int8_t*>(dst), ld_dst, stride_dst, outer_dst, rows,
+                           cols, batch);
         HIPIE_CHECK_HIP(hipGetLastError());
     });
 }

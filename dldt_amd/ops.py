@@ -233,21 +233,25 @@ class BatchedMatMul:
         return out[..., :self.n]
 
 
-def matmul_strided(mm, a, lda, stride_a, bt, ldb, stride_b, out, ldo, stride_o, m, batch):
-    """hipie_matmul_run on raw device pointers (ints) with explicit leading dimensions and batch
-    strides, for operands that are slices of larger tensors (attention heads inside [T, 3H])."""
+def matmul_strided(mm, a, lda, stride_a, bt, ldb, stride_b, out, ldo, stride_o, m, batch,
+                   batch_outer=1, outer_a=0, outer_b=0, outer_o=0):
+    """hipie_matmul_run_nested on raw device pointers (ints) with explicit leading dimensions and
+    batch strides, for operands that are slices of larger tensors (attention heads inside [T, 3H]:
+    batch = heads with stride 64, batch_outer = sequences)."""
     i64 = ctypes.c_int64
-    check(lib().hipie_matmul_run(mm._h, ctypes.c_void_p(a), i64(lda), i64(stride_a), ctypes.c_void_p(bt), i64(ldb),
-                                 i64(stride_b), ctypes.c_void_p(out), i64(ldo), i64(stride_o), ctypes.c_int32(m),
-                                 ctypes.c_int32(batch), _stream()))
+    check(lib().hipie_matmul_run_nested(mm._h, ctypes.c_void_p(a), i64(lda), i64(stride_a), i64(outer_a),
+                                        ctypes.c_void_p(bt), i64(ldb), i64(stride_b), i64(outer_b), ctypes.c_void_p(out),
+                                        i64(ldo), i64(stride_o), i64(outer_o), ctypes.c_int32(m), ctypes.c_int32(batch),
+                                        ctypes.c_int32(batch_outer), _stream()))
 
 
-def transpose_bytes(src, ld_src, bs_src, dst, ld_dst, bs_dst, rows, cols, batch):
-    """dst[b][c][r] = src[b][r][c] on raw device pointers (ints), sizes in bytes."""
+def transpose_bytes(src, ld_src, bs_src, dst, ld_dst, bs_dst, rows, cols, batch, batch_outer=1, outer_src=0, outer_dst=0):
+    """dst[o][b][c][r] = src[o][b][r][c] on raw device pointers (ints), sizes in bytes."""
     i64 = ctypes.c_int64
-    check(lib().hipie_transpose_bytes(ctypes.c_void_p(src), i64(ld_src), i64(bs_src), ctypes.c_void_p(dst), i64(ld_dst),
-                                      i64(bs_dst), ctypes.c_int32(rows), ctypes.c_int32(cols), ctypes.c_int32(batch),
-                                      _stream()))
+    check(lib().hipie_transpose_bytes_nested(ctypes.c_void_p(src), i64(ld_src), i64(bs_src), i64(outer_src),
+                                             ctypes.c_void_p(dst), i64(ld_dst), i64(bs_dst), i64(outer_dst),
+                                             ctypes.c_int32(rows), ctypes.c_int32(cols), ctypes.c_int32(batch),
+                                             ctypes.c_int32(batch_outer), _stream()))
 
 
 def softmax(x):

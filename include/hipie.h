@@ -237,6 +237,12 @@ void hipie_matmul_destroy(hipie_matmul* matmul);
 int hipie_matmul_run(const hipie_matmul* matmul, const void* a, int64_t lda, int64_t stride_a,
                      const void* b_transposed, int64_t ldb, int64_t stride_b, void* out, int64_t ldo,
                      int64_t stride_o, int32_t m, int32_t batch, void* stream);
+/* Two-level batch, e.g. (sequence, head) with the heads of one sequence interleaved in a [T, 3H]
+ * tensor: element (o, i), o < batch_outer, i < batch, starts at o * outer + i * stride of each operand. */
+int hipie_matmul_run_nested(const hipie_matmul* matmul, const void* a, int64_t lda, int64_t stride_a, int64_t outer_a,
+                            const void* b_transposed, int64_t ldb, int64_t stride_b, int64_t outer_b, void* out,
+                            int64_t ldo, int64_t stride_o, int64_t outer_o, int32_t m, int32_t batch,
+                            int32_t batch_outer, void* stream);
 
 /* ======================================================================================
  * 1e. fp32 glue of the transformer path, over the last axis of a dense [rows, axis] f32 matrix
@@ -256,6 +262,10 @@ int hipie_gelu_f32(const float* x, float* y, int64_t n, void* stream);
  * dimensions and batch strides in bytes. */
 int hipie_transpose_bytes(const void* src, int64_t ld_src, int64_t batch_stride_src, void* dst, int64_t ld_dst,
                           int64_t batch_stride_dst, int32_t rows, int32_t cols, int32_t batch, void* stream);
+/* two-level batch as in hipie_matmul_run_nested */
+int hipie_transpose_bytes_nested(const void* src, int64_t ld_src, int64_t stride_src, int64_t outer_src, void* dst,
+                                 int64_t ld_dst, int64_t stride_dst, int64_t outer_dst, int32_t rows, int32_t cols,
+                                 int32_t batch, int32_t batch_outer, void* stream);
 
 /* ======================================================================================
  * 2. Graph level.  The plugin's LoadExeNetworkImpl walks Function::get_ordered_ops()
