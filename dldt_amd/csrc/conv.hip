@@ -24,10 +24,17 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     __shared__ __attribute__((aligned(16))) float sP[PT_ROWS * BOC];
 
     // block -> (pixel tile, channel tile): consecutive pixel tiles stay on one XCD
-    const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
-    const int t_tile = y % a.t_tiles, p_local = y / a.t_tiles;
-    const int p_tile = xcd * a.p_per_xcd + p_local;
-    if (p_local >= a.p_per_xcd || p_tile >= a.p_tiles) return;  // whole block leaves before any barrier
+    int t_tile, p_tile;
+    if (a.p_per_xcd > 0) {
+        const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
+        const int p_local = y / a.t_tiles;
+        t_tile = y % a.t_tiles;
+        p_tile = xcd * a.p_per_xcd + p_local;
+        if (p_local >= a.p_per_xcd || p_tile >= a.p_tiles) return;  // whole block leaves before any barrier
+    } else {   // few pixel tiles: plain order, consecutive workgroups land on consecutive XCDs
+        t_tile = blockIdx.x % a.t_tiles;
+        p_tile = blockIdx.x / a.t_tiles;
+    }
     const int pix0 = p_tile * BPIX, oc0 = t_tile * BOC;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -324,10 +331,17 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
     constexpr int STAGE = (BOC + BPIX) * 64;
     extern __shared__ __attribute__((aligned(16))) int8_t ring[];
 
-    const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
-    const int t_tile = y % a.t_tiles, p_local = y / a.t_tiles;
-    const int p_tile = xcd * a.p_per_xcd + p_local;
-    if (p_local >= a.p_per_xcd || p_tile >= a.p_tiles) return;
+    int t_tile, p_tile;
+    if (a.p_per_xcd > 0) {
+        const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
+        const int p_local = y / a.t_tiles;
+        t_tile = y % a.t_tiles;
+        p_tile = xcd * a.p_per_xcd + p_local;
+        if (p_local >= a.p_per_xcd || p_tile >= a.p_tiles) return;
+    } else {   // few pixel tiles: plain order, consecutive workgroups land on consecutive XCDs
+        t_tile = blockIdx.x % a.t_tiles;
+        p_tile = blockIdx.x / a.t_tiles;
+    }
     const int pix0 = p_tile * BPIX, oc0 = t_tile * BOC;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -629,7 +643,7 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
 
 template <int WOC, int WPIX>
 void launch_tiled(const ConvArgs& a, hipStream_t s, int batches = 1) {
-    const dim3 grid(8 * a.p_per_xcd * a.t_tiles, batches), block(WOC * WPIX * 64);
+    const dim3 grid(a.p_per_xcd > 0 ? 8 * a.p_per_xcd * a.t_tiles : a.p_tiles * a.t_tiles, batches), block(WOC * WPIX * 64);
     const uint32_t core = a.flags & ~CF_OUT_XOR;
 #define HIPIE_LAUNCH_TILED(FLAGS, ...) \
     hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, FLAGS>), grid, block, 0, s, a)
@@ -639,7 +653,7 @@ void launch_tiled(const ConvArgs& a, hipStream_t s, int batches = 1) {
 
 template <int WOC, int WPIX, int KS>
 void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) {
-    const dim3 grid(8 * a.p_per_xcd * a.t_tiles, batches), block(WOC * WPIX * 64 * KS);
+    const dim3 grid(a.p_per_xcd > 0 ? 8 * a.p_per_xcd * a.t_tiles : a.p_tiles * a.t_tiles, batches), block(WOC * WPIX * 64 * KS);
     const size_t lds = static_cast<size_t>(KS) * stages * (WOC + WPIX) * 64 * 64 + PT_ROWS * WOC * 64 * 4 +
                        16 * static_cast<size_t>(std::max(a.nk, a.nk2));
     const uint32_t core = a.flags & ~CF_OUT_XOR;
@@ -680,7 +694,7 @@ void launch_persist(const ConvArgs& a, hipStream_t s) {
 }
 
 void launch_tiled_small(const ConvArgs& a, hipStream_t s) {   // 64 x 64 tile, one wave per workgroup
-    const dim3 grid(8 * a.p_per_xcd * a.t_tiles), block(64);
+    const dim3 grid(a.p_per_xcd > 0 ? 8 * a.p_per_xcd * a.t_tiles : a.p_tiles * a.t_tiles), block(64);
     const uint32_t core = a.flags & ~CF_OUT_XOR;
 #define HIPIE_LAUNCH_SMALL(FLAGS, ...) \
     hipLaunchKernelGGL((conv_tiled_kernel<1, 1, FLAGS>), grid, block, 0, s, a)
@@ -1008,7 +1022,7 @@ int hipie_matmul_run_nested(const hipie_matmul* mm, const void* a_ptr, int64_t l
         const int boc = wide ? 128 : 64, bpix = wide ? 128 : 256;
         a.p_tiles = static_cast<int32_t>(ceil_div(m, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.n, boc));
-        a.p_per_xcd = static_cast<int32_t>(ceil_div(a.p_tiles, 8));
+        a.p_per_xcd = 0;   // plain order: batches are spread over the XCDs by their launch order
         DeviceGuard g(mm->device);
         if (wide) launch_tiled<2, 2>(a, as_stream(stream), batch * batch_outer);
         else launch_tiled<1, 4>(a, as_stream(stream), batch * batch_outer);
@@ -1275,7 +1289,10 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         const int bpix = square ? 128 : (tile == 2 ? 64 : 256);
         a.p_tiles = static_cast<int32_t>(ceil_div(M, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.oc, boc));
-        a.p_per_xcd = static_cast<int32_t>(ceil_div(a.p_tiles, 8));
+        // XCD-aware tile order (neighbouring pixel tiles share an L2) once every XCD gets at least 8
+        // pixel tiles; below that the plain order, which spreads what few tiles there are over all XCDs
+        const bool xcd_order = a.p_tiles >= 64 || tile == 3 || tile == 8 || tile == 9;
+        a.p_per_xcd = xcd_order ? static_cast<int32_t>(ceil_div(a.p_tiles, 8)) : 0;
         DeviceGuard g(c->device);
         hipStream_t s = as_stream(stream);
         // ring depth: enough K steps in flight to cover the load latency, within 160 KB of LDS
