@@ -1289,9 +1289,9 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         const int bpix = square ? 128 : (tile == 2 ? 64 : 256);
         a.p_tiles = static_cast<int32_t>(ceil_div(M, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.oc, boc));
-        // XCD-aware tile order (neighbouring pixel tiles share an L2) once every XCD gets at least 8
+        // XCD-aware tile order (neighbouring pixel tiles share an L2) once every XCD gets at least two
         // pixel tiles; below that the plain order, which spreads what few tiles there are over all XCDs
-        const bool xcd_order = a.p_tiles >= 64 || tile == 3 || tile == 8 || tile == 9;
+        const bool xcd_order = a.p_tiles >= 16 || tile == 3 || tile == 8 || tile == 9;
         a.p_per_xcd = xcd_order ? static_cast<int32_t>(ceil_div(a.p_tiles, 8)) : 0;
         DeviceGuard g(c->device);
         hipStream_t s = as_stream(stream);
