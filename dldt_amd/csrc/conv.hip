@@ -27,13 +27,12 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     int t_tile, p_tile;
     if (a.p_per_xcd > 0) {
         const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
-        const int p_local = y / a.t_tiles;
-        t_tile = y % a.t_tiles;
+        int p_local;
+        split_tile_index(a, y, p_local, t_tile);
         p_tile = xcd * a.p_per_xcd + p_local;
         if (p_local >= a.p_per_xcd || p_tile >= a.p_tiles) return;  // whole block leaves before any barrier
     } else {   // few pixel tiles: plain order, consecutive workgroups land on consecutive XCDs
-        t_tile = blockIdx.x % a.t_tiles;
-        p_tile = blockIdx.x / a.t_tiles;
+        split_tile_index(a, blockIdx.x, p_tile, t_tile);
     }
     const int pix0 = p_tile * BPIX, oc0 = t_tile * BOC;
 
@@ -168,8 +167,8 @@ __global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const C
     __shared__ __attribute__((aligned(16))) float sP[PT_ROWS * BOC];
 
     const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
-    const int t_tile = y % a.t_tiles;
-    int p_local = y / a.t_tiles;   // < n_per
+    int t_tile, p_local;           // p_local < n_per
+    split_tile_index(a, y, p_local, t_tile);
     auto tile_exists = [&](int pl) { return pl < a.p_per_xcd && xcd * a.p_per_xcd + pl < a.p_tiles; };
     if (!tile_exists(p_local)) return;   // uniform over the workgroup
     const int oc0 = t_tile * BOC;
@@ -334,13 +333,12 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
     int t_tile, p_tile;
     if (a.p_per_xcd > 0) {
         const int xcd = blockIdx.x & 7, y = blockIdx.x >> 3;
-        const int p_local = y / a.t_tiles;
-        t_tile = y % a.t_tiles;
+        int p_local;
+        split_tile_index(a, y, p_local, t_tile);
         p_tile = xcd * a.p_per_xcd + p_local;
         if (p_local >= a.p_per_xcd || p_tile >= a.p_tiles) return;
     } else {   // few pixel tiles: plain order, consecutive workgroups land on consecutive XCDs
-        t_tile = blockIdx.x % a.t_tiles;
-        p_tile = blockIdx.x / a.t_tiles;
+        split_tile_index(a, blockIdx.x, p_tile, t_tile);
     }
     const int pix0 = p_tile * BPIX, oc0 = t_tile * BOC;
 
@@ -1022,6 +1020,7 @@ int hipie_matmul_run_nested(const hipie_matmul* mm, const void* a_ptr, int64_t l
         const int boc = wide ? 128 : 64, bpix = wide ? 128 : 256;
         a.p_tiles = static_cast<int32_t>(ceil_div(m, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.n, boc));
+        a.t_shift = (a.t_tiles & (a.t_tiles - 1)) == 0 ? __builtin_ctz(a.t_tiles) : -1;
         a.p_per_xcd = 0;   // plain order: batches are spread over the XCDs by their launch order
         DeviceGuard g(mm->device);
         if (wide) launch_tiled<2, 2>(a, as_stream(stream), batch * batch_outer);
@@ -1289,6 +1288,7 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         const int bpix = square ? 128 : (tile == 2 ? 64 : 256);
         a.p_tiles = static_cast<int32_t>(ceil_div(M, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.oc, boc));
+        a.t_shift = (a.t_tiles & (a.t_tiles - 1)) == 0 ? __builtin_ctz(a.t_tiles) : -1;
         // XCD-aware tile order (neighbouring pixel tiles share an L2) once every XCD gets at least two
         // pixel tiles; below that the plain order, which spreads what few tiles there are over all XCDs
         const bool xcd_order = a.p_tiles >= 16 || tile == 3 || tile == 8 || tile == 9;

@@ -16,8 +16,21 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 __device__ __forceinline__ void fast_divmod(int m, int d, float inv_d, int& q, int& r) {
     q = static_cast<int>(static_cast<float>(m) * inv_d);
     r = m - q * d;
-    if (r < 0) { --q; r += d; }
-    else if (r >= d) { ++q; r -= d; }
+    // branch-free correction by one in either direction (selects, no divergent flow)
+    const int lo = r < 0 ? 1 : 0, hi = r >= d ? 1 : 0;
+    q += hi - lo;
+    r += (lo - hi) * d;
+}
+
+// y -> (y / t_tiles, y % t_tiles) of a workgroup index: shifts when the channel tile count is a power of two
+__device__ __forceinline__ void split_tile_index(const ConvArgs& a, int y, int& p_local, int& t_tile) {
+    if (a.t_shift >= 0) {
+        p_local = y >> a.t_shift;
+        t_tile = y & (a.t_tiles - 1);
+    } else {
+        p_local = y / a.t_tiles;
+        t_tile = y - p_local * a.t_tiles;
+    }
 }
 
 struct PixelCoord { int n, oh, ow; };
@@ -420,21 +433,25 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
         cur = nxt;
     }
     if (fl & CF_OUT_FQ) {
-        // stored byte = level + out_off (mod 256); -128 is a sign-bit flip
+        // stored byte = level + out_off (mod 256); -128 is a sign-bit flip, 0 nothing: one XOR mask
+        // covers both, anything else goes through the bytewise add (one uniform branch for all stores)
         const bool flip = a.flags & CF_OUT_XOR;
         const uint32_t off4 = (static_cast<uint32_t>(static_cast<int>(a.out_off)) & 0xffu) * 0x01010101u;
+        if (!flip && off4 != 0) {
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) out_dw[pb][q] = add_bytes(out_dw[pb][q], off4);
+        }
+        const uint32_t xmask = flip ? 0x80808080u : 0u;
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb)
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                if (valid[pb] && oc_lane + 16 * j < out_cs) {
-                    uint32_t w[4];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        w[q] = flip ? out_dw[pb][4 * j + q] ^ 0x80808080u : add_bytes(out_dw[pb][4 * j + q], off4);
+                if (valid[pb] && oc_lane + 16 * j < out_cs)
                     *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + out_off[pb] + 16 * j) =
-                        make_uint4(w[0], w[1], w[2], w[3]);
-                }
+                        make_uint4(out_dw[pb][4 * j] ^ xmask, out_dw[pb][4 * j + 1] ^ xmask,
+                                   out_dw[pb][4 * j + 2] ^ xmask, out_dw[pb][4 * j + 3] ^ xmask);
     }
 }
 

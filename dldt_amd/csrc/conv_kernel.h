@@ -78,6 +78,7 @@ struct ConvArgs {
     int32_t nk;                      // Kp / 64
     int32_t Kp;
     int32_t p_tiles, t_tiles, p_per_xcd;
+    int32_t t_shift;                 // log2(t_tiles) when it is a power of two, else -1 (tile decode by shifts)
     uint32_t flags;
     float lm1, out_off, clamp_lo, clamp_hi;
     // batched MatMul (grid.y = batch): per-batch strides in bytes (operands) / elements (out, res);
