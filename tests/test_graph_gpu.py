@@ -79,3 +79,23 @@ def test_small_mobilenet_v2_bit_exact(orc):
             have = have.view(np.int8)
         np.testing.assert_array_equal(have, w, err_msg=name)
     np.testing.assert_array_equal(got.view(np.uint32), want["logits"].view(np.uint32))
+
+
+@pytest.mark.parametrize("net", ["resnet50", "mobilenet_v2"])
+def test_full_size_batch_consistency(net):
+    """Full-size networks (224x224, width 1.0), where the oracle would take minutes: every image's
+    logits in a batch-16 inference must equal, bit for bit, the logits of the same image inferred
+    alone.  The two plans differ in tile counts, in the kernel variants the tuner picks and in which
+    tiles are partial, so this pins the full-size indexing that the reduced networks cannot reach."""
+    from dldt_amd import builders
+    build = getattr(builders, net)
+    rng = np.random.default_rng(2024)
+    x = rng.uniform(0, 1, (16, 3, 224, 224)).astype(np.float32)
+    g16, _ = build(batch=16, res=224)
+    (y16,) = g16.compile().create_request().infer(x)
+    assert np.isfinite(y16).all() and not np.array_equal(y16[0], y16[7])   # the images do differ
+    g1, _ = build(batch=1, res=224)
+    req1 = g1.compile().create_request()
+    for i in (0, 7, 15):
+        (y1,) = req1.infer(x[i:i + 1])
+        np.testing.assert_array_equal(y1.view(np.uint32), y16[i:i + 1].view(np.uint32), err_msg="image %d" % i)
