@@ -629,6 +629,7 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
     case E_F32: X(E_F32, __VA_ARGS__); break;                                                \
     case E_SCALE: X(E_SCALE, __VA_ARGS__); break;                                            \
     case E_SCALEFQ: X(E_SCALEFQ, __VA_ARGS__); break;                                        \
+    case E_RESI8: X(E_RESI8, __VA_ARGS__); break;                                            \
     case E_F32RES: X(E_F32RES, __VA_ARGS__); break;                                          \
     case E_F32RELU: X(E_F32RELU, __VA_ARGS__); break;                                        \
     case E_CLAMPFQ: X(E_CLAMPFQ, __VA_ARGS__); break;                                        \
@@ -1146,6 +1147,19 @@ int hipie_conv_get_tile(const hipie_conv* c, int* tile) {
     return guarded([&] {
         HIPIE_REQUIRE(c && tile, HIPIE_PARAMETER_MISMATCH, "hipie_conv_get_tile: null argument");
         *tile = c->depthwise ? -1 : c->tile;
+    });
+}
+
+int hipie_conv_epilogue_flags(const hipie_conv* c, uint32_t* flags, int* specialised) {
+    return guarded([&] {
+        HIPIE_REQUIRE(c && flags && specialised, HIPIE_PARAMETER_MISMATCH, "hipie_conv_epilogue_flags: null argument");
+        *flags = c->epi.flags;
+        const uint32_t core = c->epi.flags & ~CF_OUT_XOR;
+        bool generic = false;
+#define HIPIE_IS_GENERIC(FLAGS, ...) generic = (FLAGS) == kDyn
+        HIPIE_FOR_EACH_EPILOGUE(HIPIE_IS_GENERIC, 0)
+#undef HIPIE_IS_GENERIC
+        *specialised = generic ? 0 : 1;
     });
 }
 

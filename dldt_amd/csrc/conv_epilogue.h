@@ -113,6 +113,7 @@ constexpr uint32_t E_RESF32 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32 | E_FQ | 
 constexpr uint32_t E_RESGEMM = CF_BIAS | CF_SCALE | CF_RES | CF_RES_GEMM | E_FQ | CF_FQ_IL0;
 constexpr uint32_t E_F32 = CF_BIAS | CF_SCALE;
 constexpr uint32_t E_SCALE = CF_SCALE;
+constexpr uint32_t E_RESI8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_MUL | E_FQ;   // linear bottleneck + i8 residual (MobileNetV2)
 constexpr uint32_t E_SCALEFQ = CF_BIAS | CF_SCALE | E_FQ;              // linear layer requantised to symmetric i8
 constexpr uint32_t E_F32RES = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32;   // linear layer + f32 residual, f32 out                      // MatMul' -> Multiply(s_a * s_b)
 constexpr uint32_t E_F32RELU = CF_BIAS | CF_SCALE | CF_RELU;
@@ -277,7 +278,8 @@ __device__ __forceinline__ void load_residual_bytes(const ConvArgs& a, int oc_la
 
 // sp: the tile's staged tables (stage_params) with local channel 0 = channel oc0, or nullptr to
 // read the tables from global memory
-template <uint32_t F>
+// NOB = 2: a lane owns 32 channels (acc[0..1]); NOB = 1: 16 channels (acc[0] only)
+template <uint32_t F, int NOB = 2>
 __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                          const bool (&valid)[2], const int64_t (&out_off)[2],
                                          const int64_t (&res_off)[2], const v16f (&rres)[2][2],
@@ -296,7 +298,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
 
     if (fl & CF_OUT_I32) {   // raw accumulators
 #pragma unroll
-        for (int e4 = 0; e4 < 8; ++e4)
+        for (int e4 = 0; e4 < 4 * NOB; ++e4)
 #pragma unroll
             for (int pb = 0; pb < 2; ++pb)
                 if (valid[pb] && oc_lane + 4 * e4 + 4 <= out_cs) {
@@ -349,8 +351,8 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
     EpiParams cur, nxt;
     load(0, cur);
 #pragma unroll
-    for (int e4 = 0; e4 < 8; ++e4) {
-        if (e4 + 1 < 8) load(e4 + 1, nxt);
+    for (int e4 = 0; e4 < 4 * NOB; ++e4) {
+        if (e4 + 1 < 4 * NOB) load(e4 + 1, nxt);
         const int ob = e4 >> 2, r0 = (e4 & 3) * 4;
         float bias_[4], scale_[4], rsub_[4], rmul_[4], post_[4], il_[4], ih_[4], d_[4], rr_[4], r2_[4];
         f4_to_array(cur.bias, bias_);
@@ -441,13 +443,13 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
 #pragma unroll
             for (int pb = 0; pb < 2; ++pb)
 #pragma unroll
-                for (int q = 0; q < 8; ++q) out_dw[pb][q] = add_bytes(out_dw[pb][q], off4);
+                for (int q = 0; q < 4 * NOB; ++q) out_dw[pb][q] = add_bytes(out_dw[pb][q], off4);
         }
         const uint32_t xmask = flip ? 0x80808080u : 0u;
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < NOB; ++j)
                 if (valid[pb] && oc_lane + 16 * j < out_cs)
                     *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + out_off[pb] + 16 * j) =
                         make_uint4(out_dw[pb][4 * j] ^ xmask, out_dw[pb][4 * j + 1] ^ xmask,

@@ -60,13 +60,105 @@ __global__ __launch_bounds__(256) void dwconv_kernel(const ConvArgs a, int KH, i
     run_epilogue<F>(a, acc, oc_lane, m0, m0 + 1);
 }
 
+
+// 3x3, dilation 1, stride 1 or 2: a lane owns 16 channels of two horizontally adjacent output
+// pixels.  All 9 weight pieces and the 12 (stride 1) or 15 (stride 2) input pieces the two windows
+// cover are requested before the first multiply, so a wave waits for memory once instead of once
+// per tap, and the two windows share their overlapping input columns in registers.
+template <uint32_t F, int STRIDE>
+__global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cgroups, int pairs_per_row, int64_t items) {
+    const int64_t item = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (item >= items) return;
+    const int cgi = static_cast<int>(item % cgroups);
+    const int pair = static_cast<int>(item / cgroups);
+    const int oc_lane = cgi * 16;
+    // pair -> (n, oh, ow0): pairs never straddle a row
+    const int OH = a.OHOW / a.OW;
+    const int rowi = pair / pairs_per_row, ow0 = (pair - rowi * pairs_per_row) * 2;
+    const int n = rowi / OH, oh = rowi - n * OH;
+    constexpr int COLS = 3 + STRIDE;   // input columns under the two windows
+    const int8_t* xp = a.in + (static_cast<int64_t>(n) * a.in_sn + oh * STRIDE * a.in_sh + ow0 * STRIDE * a.in_sw +
+                               a.in_origin + oc_lane);
+    uint4 x[3][COLS], w[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) w[t] = *reinterpret_cast<const uint4*>(a.wgt + static_cast<int64_t>(t) * a.OCp + oc_lane);
+    // the last pair of an odd row has one pixel: its second window's extra columns are clamped onto
+    // existing ones (the results are discarded)
+    const bool two = ow0 + 1 < a.OW;
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            const int cc = (c < 3 || two) ? c : 2;
+            x[r][c] = *reinterpret_cast<const uint4*>(xp + r * a.in_sh + cc * a.in_sw);
+        }
+    v16i acc[2][2];
+    {
+        const int4 c0 = *reinterpret_cast<const int4*>(a.corr + oc_lane), c1 = *reinterpret_cast<const int4*>(a.corr + oc_lane + 4);
+        const int4 c2 = *reinterpret_cast<const int4*>(a.corr + oc_lane + 8), c3 = *reinterpret_cast<const int4*>(a.corr + oc_lane + 12);
+        const int cv[16] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w, c2.x, c2.y, c2.z, c2.w, c3.x, c3.y, c3.z, c3.w};
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                acc[0][pb][r] = cv[r];
+                acc[1][pb][r] = 0;
+            }
+    }
+#pragma unroll
+    for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw) {
+            const uint4 wv = w[kh * 3 + kw];
+            const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) {
+                const uint4 xv = x[kh][kw + pb * STRIDE];
+                const uint32_t xd[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    int c0 = acc[0][pb][4 * q], c1 = acc[0][pb][4 * q + 1], c2 = acc[0][pb][4 * q + 2], c3 = acc[0][pb][4 * q + 3];
+                    mac_bytes(xd[q], wd[q], c0, c1, c2, c3);
+                    acc[0][pb][4 * q] = c0; acc[0][pb][4 * q + 1] = c1; acc[0][pb][4 * q + 2] = c2; acc[0][pb][4 * q + 3] = c3;
+                }
+            }
+        }
+    bool valid[2] = {true, two};
+    int64_t out_off[2], res_off[2];
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+        const int ow = two || pb == 0 ? ow0 + pb : ow0;
+        out_off[pb] = static_cast<int64_t>(n) * a.out_sn + oh * a.out_sh + ow * a.out_sw + oc_lane;
+        res_off[pb] = static_cast<int64_t>(n) * a.res_sn + oh * a.res_sh + ow * a.res_sw + oc_lane;
+    }
+    v16f none[2][2];
+    epilogue<F, 1>(a, acc, oc_lane, valid, out_off, res_off, none, nullptr, 0, 0);
+}
+
 }  // namespace
 
 void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipStream_t s) {
+    const uint32_t core = a.flags & ~CF_OUT_XOR;
+    const bool known = core == E_PLAIN0 || core == E_CLAMPFQ;
+    if (KH == 3 && KW == 3 && dil_h == 1 && dil_w == 1 && a.conv_sh == a.conv_sw && (a.conv_sh == 1 || a.conv_sh == 2) &&
+        known && !(a.flags & CF_RES)) {
+        const int cgroups = std::min(a.OCp, a.in_sw) / 16;   // groups of 16 channels that exist in the tensors
+        const int pairs_per_row = (a.OW + 1) / 2;
+        const int64_t items = static_cast<int64_t>(a.M / a.OW) * pairs_per_row * cgroups;
+        const dim3 grid(static_cast<uint32_t>(ceil_div(items, 256))), block(256);
+#define HIPIE_LAUNCH_DW3(FLAGS, STRIDE) \
+    hipLaunchKernelGGL((dwconv3x3_kernel<FLAGS, STRIDE>), grid, block, 0, s, a, cgroups, pairs_per_row, items)
+        if (core == E_PLAIN0) {
+            if (a.conv_sh == 1) HIPIE_LAUNCH_DW3(E_PLAIN0, 1); else HIPIE_LAUNCH_DW3(E_PLAIN0, 2);
+        } else {
+            if (a.conv_sh == 1) HIPIE_LAUNCH_DW3(E_CLAMPFQ, 1); else HIPIE_LAUNCH_DW3(E_CLAMPFQ, 2);
+        }
+#undef HIPIE_LAUNCH_DW3
+        return;
+    }
     const int cgroups = a.OCp / 32;
     const int64_t items = ceil_div(a.M, 2) * cgroups;
     const dim3 grid(static_cast<uint32_t>(ceil_div(items, 256))), block(256);
-    const uint32_t core = a.flags & ~CF_OUT_XOR;
     switch (core) {
     case E_PLAIN0: hipLaunchKernelGGL((dwconv_kernel<E_PLAIN0>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items); break;
     case E_CLAMPFQ: hipLaunchKernelGGL((dwconv_kernel<E_CLAMPFQ>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items); break;

@@ -217,9 +217,13 @@ struct ConvStep : Step {
         (void)hipEventDestroy(e0);
         (void)hipEventDestroy(e1);
         check_status(hipie_conv_set_tile(conv, best), name.c_str());
-        if (std::getenv("HIPIE_TUNE_LOG"))
-            std::fprintf(stderr, "hipie tune: %-28s variant %d (%.1f us; default %d)\n", name.c_str(), best,
-                         best_ms * 200.f, current);
+        if (std::getenv("HIPIE_TUNE_LOG")) {
+            uint32_t fl = 0;
+            int spec = 0;
+            (void)hipie_conv_epilogue_flags(conv, &fl, &spec);
+            std::fprintf(stderr, "hipie tune: %-28s variant %d (%.1f us; default %d) epilogue %#x%s\n", name.c_str(), best,
+                         best_ms * 200.f, current, fl, spec ? "" : " GENERIC");
+        }
     }
 };
 

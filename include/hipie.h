@@ -211,6 +211,9 @@ int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* o
  * variant produces the same bits. */
 int hipie_conv_set_tile(hipie_conv* conv, int tile);
 int hipie_conv_get_tile(const hipie_conv* conv, int* tile);
+/* diagnostics: the epilogue's step flags (conv_kernel.h ConvFlags) and whether a kernel instance with
+ * these steps compiled in exists (otherwise the generic, slower instance runs) */
+int hipie_conv_epilogue_flags(const hipie_conv* conv, uint32_t* flags, int* specialised);
 /* ring depth (2..8 K steps in LDS) of the pipelined variants; 0 = choose from K */
 int hipie_conv_set_stages(hipie_conv* conv, int stages);
 int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,
