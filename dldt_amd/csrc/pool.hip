@@ -8,20 +8,26 @@ namespace {
 
 constexpr int kThreads = 256;
 
-// bytewise signed max of two dwords
-__device__ __forceinline__ uint32_t max_i8x4(uint32_t a, uint32_t b) {
-    uint32_t r = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int x = static_cast<int8_t>(a >> (8 * j)), y = static_cast<int8_t>(b >> (8 * j));
-        r |= (static_cast<uint32_t>(x > y ? x : y) & 0xffu) << (8 * j);
+// Bytewise max on four packed bytes in the order-preserving unsigned domain (byte ^ 0x80 for signed
+// storage): even and odd bytes are compared as the low / high byte of 16-bit lanes (v_pk_max_u16).
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+struct ByteMax {
+    uint32_t even = 0, odd = 0;   // running maxima, unsigned domain; 0 is the identity
+    __device__ __forceinline__ void take(uint32_t stored) {
+        const uint32_t x = stored ^ 0x80808080u;
+        const uint32_t e = x & 0x00ff00ffu, o = x & 0xff00ff00u;
+        even = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, even), __builtin_bit_cast(u16x2, e)));
+        odd = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, odd), __builtin_bit_cast(u16x2, o)));
     }
-    return r;
-}
+    __device__ __forceinline__ uint32_t stored() const { return (even | odd) ^ 0x80808080u; }
+};
 
 // One thread = 16 channels of one output pixel.  Padding cells hold the lowest value (level 0
 // for U8B, -128 for I8) in the tensor's halo, which is the identity of max; the window is
-// trimmed at the padded upper bound as in max_pool.hpp.
+// trimmed at the padded upper bound as in max_pool.hpp.  K3 = true: a 3 x 3 window that the upper
+// bounds do not trim, all nine loads requested up front.
+template <bool K3>
 __global__ __launch_bounds__(kThreads) void max_pool_nhwc_i8(PoolArgs a) {
     const int64_t t = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
     const int cg = a.cs / 16;
@@ -29,19 +35,38 @@ __global__ __launch_bounds__(kThreads) void max_pool_nhwc_i8(PoolArgs a) {
     const int m = static_cast<int>(t / cg), c = static_cast<int>(t % cg) * 16;
     const int n = m / a.OHOW, rem = m - n * a.OHOW, oh = rem / a.OW, ow = rem - oh * a.OW;
     const int y0 = oh * a.sh - a.pt, x0 = ow * a.sw - a.pl;
-    const int y1 = min(y0 + a.kh, a.H + a.pb), x1 = min(x0 + a.kw, a.W + a.pr);
-    uint4 r = make_uint4(0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u);
     const int8_t* base = static_cast<const int8_t*>(a.in) + static_cast<int64_t>(n) * a.in_sn + c;
-    for (int y = y0; y < y1; ++y)
-        for (int x = x0; x < x1; ++x) {
-            const uint4 v = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(y) * a.in_sh + x * a.in_sw);
-            r.x = max_i8x4(r.x, v.x);
-            r.y = max_i8x4(r.y, v.y);
-            r.z = max_i8x4(r.z, v.z);
-            r.w = max_i8x4(r.w, v.w);
-        }
+    ByteMax r[4];
+    if (K3) {
+        uint4 v[3][3];
+#pragma unroll
+        for (int y = 0; y < 3; ++y)
+#pragma unroll
+            for (int x = 0; x < 3; ++x)
+                v[y][x] = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(y0 + y) * a.in_sh + (x0 + x) * a.in_sw);
+#pragma unroll
+        for (int y = 0; y < 3; ++y)
+#pragma unroll
+            for (int x = 0; x < 3; ++x) {
+                r[0].take(v[y][x].x);
+                r[1].take(v[y][x].y);
+                r[2].take(v[y][x].z);
+                r[3].take(v[y][x].w);
+            }
+    } else {
+        const int y1 = min(y0 + a.kh, a.H + a.pb), x1 = min(x0 + a.kw, a.W + a.pr);
+        for (int y = y0; y < y1; ++y)
+            for (int x = x0; x < x1; ++x) {
+                const uint4 v = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(y) * a.in_sh + x * a.in_sw);
+                r[0].take(v.x);
+                r[1].take(v.y);
+                r[2].take(v.z);
+                r[3].take(v.w);
+            }
+    }
     *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + static_cast<int64_t>(n) * a.out_sn +
-                              oh * a.out_sh + ow * a.out_sw + c) = r;
+                              oh * a.out_sh + ow * a.out_sw + c) =
+        make_uint4(r[0].stored(), r[1].stored(), r[2].stored(), r[3].stored());
 }
 
 // One thread = 4 channels of one output pixel.  Integer window sum (exact; equals the
@@ -58,20 +83,30 @@ __global__ __launch_bounds__(kThreads) void avg_pool_nhwc_i8(PoolArgs a) {
     const int y1 = min(y0 + a.kh, a.H + a.pb), x1 = min(x0 + a.kw, a.W + a.pr);
     const bool padding_present = a.pt || a.pl || a.pb || a.pr;
     int sum[4] = {0, 0, 0, 0};
-    int count = 0, cells = 0;
+    // the in-bounds part of the window, walked two rows x eight columns at a time with all sixteen
+    // loads requested before the first add (a global 7x7 pool is 49 dependent round trips otherwise)
+    const int ya = max(y0, 0), yb = min(y1, a.H), xa = max(x0, 0), xb = min(x1, a.W);
+    const int cells = max(yb - ya, 0) * max(xb - xa, 0);
+    int count = padding_present ? cells : (y1 - y0) * (x1 - x0);
     const int8_t* base = static_cast<const int8_t*>(a.in) + static_cast<int64_t>(n) * a.in_sn + c;
-    for (int y = y0; y < y1; ++y)
-        for (int x = x0; x < x1; ++x) {
-            const bool in_bounds = y >= 0 && y < a.H && x >= 0 && x < a.W;
-            if (in_bounds || a.include_pad) {
-                if (in_bounds) {
-                    const uint32_t v = *reinterpret_cast<const uint32_t*>(base + static_cast<int64_t>(y) * a.in_sh + x * a.in_sw);
+    for (int y = ya; y < yb; y += 2)
+        for (int x = xa; x < xb; x += 8) {
+            uint32_t v[2][8];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) sum[j] += static_cast<int8_t>(v >> (8 * j));
-                    ++cells;
+            for (int r = 0; r < 2; ++r)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const bool ok = y + r < yb && x + i < xb;
+                    const int yy = ok ? y + r : ya, xx = ok ? x + i : xa;   // clamped onto an existing cell
+                    const uint32_t t = *reinterpret_cast<const uint32_t*>(base + static_cast<int64_t>(yy) * a.in_sh + xx * a.in_sw);
+                    v[r][i] = ok ? t : 0u;
                 }
-                if (!padding_present || (in_bounds && !a.include_pad)) ++count;
-            }
+#pragma unroll
+            for (int r = 0; r < 2; ++r)
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) sum[j] += static_cast<int8_t>(v[r][i] >> (8 * j));
         }
     if (a.include_pad && padding_present) count = a.kh * a.kw;
     const float nf = static_cast<float>(count);
@@ -133,8 +168,13 @@ __global__ __launch_bounds__(kThreads) void exit_nhwc_to_nchw(ExitArgs a) {
 
 void launch_max_pool(const PoolArgs& a, hipStream_t s) {
     const int64_t threads = static_cast<int64_t>(a.M) * (a.cs / 16);
-    hipLaunchKernelGGL(max_pool_nhwc_i8, dim3(static_cast<uint32_t>(ceil_div(threads, kThreads))),
-                       dim3(kThreads), 0, s, a);
+    // every 3 x 3 window lies inside the padded tensor: the last one ends at (OH-1)*s - pad + 3 <= H + pad_end
+    const int OH = a.OHOW / a.OW;
+    const bool k3 = a.kh == 3 && a.kw == 3 && (OH - 1) * a.sh - a.pt + 3 <= a.H + a.pb &&
+                    (a.OW - 1) * a.sw - a.pl + 3 <= a.W + a.pr;
+    const dim3 grid(static_cast<uint32_t>(ceil_div(threads, kThreads)));
+    if (k3) hipLaunchKernelGGL(max_pool_nhwc_i8<true>, grid, dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL(max_pool_nhwc_i8<false>, grid, dim3(kThreads), 0, s, a);
 }
 
 void launch_avg_pool(const PoolArgs& a, bool rcp, hipStream_t s) {
