@@ -853,6 +853,7 @@ struct hipie_conv {
                    // in LDS), 4: pipelined 128 x 128, 5: pipelined 64 x 256
     int stages = 0;  // ring depth of the pipelined kernels (0 = choose from K)
     DeviceBuffer wgt, koff, corr;
+    DeviceBuffer wgt_rows;   // depthwise 3 x 3: [kh][OCp] dwords, bytes (w[kh][0], w[kh][1], w[kh][2], 0) of a channel
     Epilogue epi;
 };
 
@@ -1068,9 +1069,21 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
                 corr[ch] = d.in_dtype == HIPIE_U8B ? 128 * sum : 0;
             }
             c->epi.build(device, *epilogue, d.oc, c->OCp);
+            std::vector<uint32_t> rows;
+            if (d.kh == 3 && d.kw == 3) {
+                rows.assign(static_cast<size_t>(3) * c->OCp, 0u);
+                for (int ch = 0; ch < d.oc; ++ch)
+                    for (int kh = 0; kh < 3; ++kh) {
+                        uint32_t v = 0;
+                        for (int kw = 0; kw < 3; ++kw)
+                            v |= static_cast<uint32_t>(static_cast<uint8_t>(weights[ch * 9 + kh * 3 + kw])) << (8 * kw);
+                        rows[static_cast<size_t>(kh) * c->OCp + ch] = v;
+                    }
+            }
             if (device >= 0) {
                 c->wgt.upload(device, w.data(), w.size());
                 c->corr.upload(device, corr.data(), corr.size() * sizeof(int32_t));
+                if (!rows.empty()) c->wgt_rows.upload(device, rows.data(), rows.size() * sizeof(uint32_t));
             }
             *out = c.release();
             return;
@@ -1219,6 +1232,7 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         ConvArgs a{};
         a.in = static_cast<const int8_t*>(in->data);
         a.wgt = c->wgt.as<int8_t>();
+        a.wgt2 = c->wgt_rows.as<int8_t>();   // depthwise only; a fused shortcut overwrites it below
         a.out = out->data;
         a.koff = c->koff.as<int32_t>();
         a.corr = c->corr.as<int32_t>();

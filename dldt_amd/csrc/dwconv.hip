@@ -79,9 +79,13 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cg
     constexpr int COLS = 3 + STRIDE;   // input columns under the two windows
     const int8_t* xp = a.in + (static_cast<int64_t>(n) * a.in_sn + oh * STRIDE * a.in_sh + ow0 * STRIDE * a.in_sw +
                                a.in_origin + oc_lane);
-    uint4 x[3][COLS], w[9];
+    // a.wgt2: [kh][OCp] dwords, the three taps of a filter row of one channel in bytes 0..2
+    uint4 x[3][COLS], wr[3][4];
 #pragma unroll
-    for (int t = 0; t < 9; ++t) w[t] = *reinterpret_cast<const uint4*>(a.wgt + static_cast<int64_t>(t) * a.OCp + oc_lane);
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            wr[r][q] = *reinterpret_cast<const uint4*>(a.wgt2 + (static_cast<int64_t>(r) * a.OCp + oc_lane + 4 * q) * 4);
     // the last pair of an odd row has one pixel: its second window's extra columns are clamped onto
     // existing ones (the results are discarded)
     const bool two = ow0 + 1 < a.OW;
@@ -105,21 +109,39 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cg
                 acc[1][pb][r] = 0;
             }
     }
+    // Four pixels x four channels of bytes are transposed with 8 v_perm_b32 into one dword per
+    // channel holding that channel's byte of four consecutive pixels; a filter row is then one
+    // v_dot4_i32_i8 per channel and output pixel against (w0, w1, w2, 0) - shifted by one byte for the
+    // second pixel of a stride-1 pair, whose window starts one column later.
 #pragma unroll
     for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
-        for (int kw = 0; kw < 3; ++kw) {
-            const uint4 wv = w[kh * 3 + kw];
-            const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
+        for (int q = 0; q < 4; ++q) {
+            auto dw = [&](const uint4& v) { return q == 0 ? v.x : (q == 1 ? v.y : (q == 2 ? v.z : v.w)); };
+            auto transpose4 = [&](uint32_t p0, uint32_t p1, uint32_t p2, uint32_t p3, uint32_t (&t)[4]) {
+                const uint32_t lo01 = __builtin_amdgcn_perm(p1, p0, 0x05010400u), hi01 = __builtin_amdgcn_perm(p1, p0, 0x07030602u);
+                const uint32_t lo23 = __builtin_amdgcn_perm(p3, p2, 0x05010400u), hi23 = __builtin_amdgcn_perm(p3, p2, 0x07030602u);
+                t[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+                t[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+                t[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+                t[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+            };
+            const uint32_t wq[4] = {wr[kh][q].x, wr[kh][q].y, wr[kh][q].z, wr[kh][q].w};
+            uint32_t t0[4];
+            transpose4(dw(x[kh][0]), dw(x[kh][1]), dw(x[kh][2]), dw(x[kh][3]), t0);
+            if (STRIDE == 1) {
 #pragma unroll
-            for (int pb = 0; pb < 2; ++pb) {
-                const uint4 xv = x[kh][kw + pb * STRIDE];
-                const uint32_t xd[4] = {xv.x, xv.y, xv.z, xv.w};
+                for (int c = 0; c < 4; ++c) {
+                    acc[0][0][4 * q + c] = __builtin_amdgcn_sdot4(static_cast<int>(t0[c]), static_cast<int>(wq[c]), acc[0][0][4 * q + c], false);
+                    acc[0][1][4 * q + c] = __builtin_amdgcn_sdot4(static_cast<int>(t0[c]), static_cast<int>(wq[c] << 8), acc[0][1][4 * q + c], false);
+                }
+            } else {   // second window: columns 2, 3, 4
+                uint32_t t1[4];
+                transpose4(dw(x[kh][2]), dw(x[kh][3]), dw(x[kh][4]), dw(x[kh][4]), t1);
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    int c0 = acc[0][pb][4 * q], c1 = acc[0][pb][4 * q + 1], c2 = acc[0][pb][4 * q + 2], c3 = acc[0][pb][4 * q + 3];
-                    mac_bytes(xd[q], wd[q], c0, c1, c2, c3);
-                    acc[0][pb][4 * q] = c0; acc[0][pb][4 * q + 1] = c1; acc[0][pb][4 * q + 2] = c2; acc[0][pb][4 * q + 3] = c3;
+                for (int c = 0; c < 4; ++c) {
+                    acc[0][0][4 * q + c] = __builtin_amdgcn_sdot4(static_cast<int>(t0[c]), static_cast<int>(wq[c]), acc[0][0][4 * q + c], false);
+                    acc[0][1][4 * q + c] = __builtin_amdgcn_sdot4(static_cast<int>(t1[c]), static_cast<int>(wq[c]), acc[0][1][4 * q + c], false);
                 }
             }
         }
