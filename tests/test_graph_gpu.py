@@ -99,3 +99,29 @@ def test_full_size_batch_consistency(net):
     for i in (0, 7, 15):
         (y1,) = req1.infer(x[i:i + 1])
         np.testing.assert_array_equal(y1.view(np.uint32), y16[i:i + 1].view(np.uint32), err_msg="image %d" % i)
+
+
+def test_requests_in_flight_do_not_disturb_each_other():
+    """Three requests of one plan on their own streams and arenas, fed different images and kept in
+    flight together (the throughput mode bench.py measures): every result equals the same image's
+    result from a request that ran alone."""
+    import torch
+    from dldt_amd import builders
+    g, _ = builders.resnet50(batch=4, res=96, width=32, classes=16, seed=5)
+    plan = g.compile()
+    rng = np.random.default_rng(6)
+    xs = [rng.uniform(0, 1, (4, 3, 96, 96)).astype(np.float32) for _ in range(3)]
+    alone = plan.create_request()
+    want = [alone.infer(x)[0].copy() for x in xs]
+    reqs = [plan.create_request() for _ in xs]
+    bufs = [r.device_buffers() for r in reqs]
+    for (ins, _), x in zip(bufs, xs):
+        ins[0].copy_(torch.from_numpy(x))
+    torch.cuda.synchronize()
+    for _ in range(5):                      # several rounds back to back, nothing waits in between
+        for r, (ins, outs) in zip(reqs, bufs):
+            r.enqueue(ins, outs)
+    for r in reqs:
+        torch.cuda.ExternalStream(r.stream).synchronize()
+    for (_, outs), w in zip(bufs, want):
+        np.testing.assert_array_equal(outs[0].cpu().numpy().view(np.uint32), w.view(np.uint32))
