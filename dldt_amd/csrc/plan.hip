@@ -73,6 +73,11 @@ struct EpilogueSpec {
     }
 };
 
+struct TuneLane {
+    uint8_t* arena;
+    hipStream_t stream;
+};
+
 struct Step {
     std::string name, type;
     int64_t macs = 0, bytes = 0;
@@ -82,7 +87,9 @@ struct Step {
     virtual void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs,
                      void* const* outputs, hipStream_t s) const = 0;
     // pick the fastest kernel variant by timing it on a scratch arena (load time, optional)
-    virtual void tune(uint8_t*, const std::vector<TensorInfo>&, hipStream_t) {}
+    // `lanes`: scratch arenas and streams of as many requests as are expected in flight together; a
+    // variant is timed with one copy of the layer running on every lane at once
+    virtual void tune(const std::vector<TuneLane>&, const std::vector<TensorInfo>&) {}
     // the chosen variant as an integer (-1: the step has no variants), and its inverse
     virtual int variant() const { return -1; }
     virtual void set_variant(int) {}
@@ -179,19 +186,30 @@ struct ConvStep : Step {
     }
     // Every variant computes the same integers, so the choice changes time only.  Variants a layer
     // cannot use are refused by hipie_conv_set_tile and skipped.
-    void tune(uint8_t* arena, const std::vector<TensorInfo>& tensors, hipStream_t s) override {
-        if (shortcut && !fused) shortcut->tune(arena, tensors, s);
+    void tune(const std::vector<TuneLane>& lanes, const std::vector<TensorInfo>& tensors) override {
+        if (shortcut && !fused) shortcut->tune(lanes, tensors);
         int current = -1;
         check_status(hipie_conv_get_tile(conv, &current), name.c_str());
         if (current < 0) return;   // depthwise: one kernel
-        const hipie_tensor i = tensors[in].desc(arena), o = tensors[out].desc(arena);
-        hipie_tensor r{};
-        if (fused) r = tensors[shortcut->in].desc(arena);
-        else if (res >= 0) r = tensors[res].desc(arena);
-        const hipie_tensor* rp = (fused || res >= 0) ? &r : nullptr;
-        hipEvent_t e0, e1;
-        HIPIE_CHECK_HIP(hipEventCreate(&e0));
-        HIPIE_CHECK_HIP(hipEventCreate(&e1));
+        const size_t nl = lanes.size();
+        std::vector<hipie_tensor> ti(nl), to(nl), tr(nl);
+        for (size_t l = 0; l < nl; ++l) {
+            ti[l] = tensors[in].desc(lanes[l].arena);
+            to[l] = tensors[out].desc(lanes[l].arena);
+            if (fused) tr[l] = tensors[shortcut->in].desc(lanes[l].arena);
+            else if (res >= 0) tr[l] = tensors[res].desc(lanes[l].arena);
+        }
+        const bool has_res = fused || res >= 0;
+        auto launch_all = [&](int times) {
+            for (int w = 0; w < times; ++w)
+                for (size_t l = 0; l < nl; ++l)
+                    check_status(hipie_conv_run(conv, &ti[l], has_res ? &tr[l] : nullptr, &to[l], lanes[l].stream), name.c_str());
+        };
+        std::vector<hipEvent_t> e0(nl), e1(nl);
+        for (size_t l = 0; l < nl; ++l) {
+            HIPIE_CHECK_HIP(hipEventCreate(&e0[l]));
+            HIPIE_CHECK_HIP(hipEventCreate(&e1[l]));
+        }
         int best = current;
         float best_ms = 0.f;
         const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7, 8, 9};
@@ -202,27 +220,35 @@ struct ConvStep : Step {
             int applied = -1;
             check_status(hipie_conv_get_tile(conv, &applied), name.c_str());
             if (applied != tile) continue;   // not available for this layer (kept its previous variant)
-            for (int w = 0; w < 2; ++w) check_status(hipie_conv_run(conv, &i, rp, &o, s), name.c_str());
-            HIPIE_CHECK_HIP(hipEventRecord(e0, s));
-            for (int w = 0; w < 5; ++w) check_status(hipie_conv_run(conv, &i, rp, &o, s), name.c_str());
-            HIPIE_CHECK_HIP(hipEventRecord(e1, s));
-            HIPIE_CHECK_HIP(hipEventSynchronize(e1));
-            float ms = 0.f;
-            HIPIE_CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+            launch_all(2);
+            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipStreamSynchronize(lanes[l].stream));
+            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventRecord(e0[l], lanes[l].stream));
+            launch_all(5);
+            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventRecord(e1[l], lanes[l].stream));
+            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventSynchronize(e1[l]));
+            float ms = 0.f;   // earliest start to latest end
+            for (size_t a = 0; a < nl; ++a)
+                for (size_t b = 0; b < nl; ++b) {
+                    float t = 0.f;
+                    HIPIE_CHECK_HIP(hipEventElapsedTime(&t, e0[a], e1[b]));
+                    ms = std::max(ms, t);
+                }
             if (c == 0 || ms < best_ms) {
                 best_ms = ms;
                 best = tile;
             }
         }
-        (void)hipEventDestroy(e0);
-        (void)hipEventDestroy(e1);
+        for (size_t l = 0; l < nl; ++l) {
+            (void)hipEventDestroy(e0[l]);
+            (void)hipEventDestroy(e1[l]);
+        }
         check_status(hipie_conv_set_tile(conv, best), name.c_str());
         if (std::getenv("HIPIE_TUNE_LOG")) {
             uint32_t fl = 0;
             int spec = 0;
             (void)hipie_conv_epilogue_flags(conv, &fl, &spec);
-            std::fprintf(stderr, "hipie tune: %-28s variant %d (%.1f us; default %d) epilogue %#x%s\n", name.c_str(), best,
-                         best_ms * 200.f, current, fl, spec ? "" : " GENERIC");
+            std::fprintf(stderr, "hipie tune: %-28s variant %d (%.1f us per launch with %zu in flight; default %d) epilogue %#x%s\n",
+                         name.c_str(), best, best_ms * 200.f / static_cast<float>(nl), nl, current, fl, spec ? "" : " GENERIC");
         }
     }
 };
@@ -855,14 +881,23 @@ int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
                 }
             }
             if (!loaded) {
-                hipie_request* scratch = nullptr;
-                check_status(hipie_request_create(plan.get(), 0, &scratch), "hipie_compile: tuning request");
-                struct Release {
-                    hipie_request* r;
-                    ~Release() { hipie_request_destroy(r); }
-                } release{scratch};
+                // HIPIE_TUNE_STREAMS requests are assumed in flight together (default 3, the throughput
+                // mode of a plugin with three streams; 1 tunes for the latency of a lone request)
+                const char* ts = std::getenv("HIPIE_TUNE_STREAMS");
+                const int n_lanes = std::max(1, std::min(8, ts ? std::atoi(ts) : 3));
+                struct Scratch {
+                    std::vector<hipie_request*> r;
+                    ~Scratch() { for (auto* q : r) hipie_request_destroy(q); }
+                } scratch;
+                std::vector<TuneLane> lanes;
+                for (int l = 0; l < n_lanes; ++l) {
+                    hipie_request* q = nullptr;
+                    check_status(hipie_request_create(plan.get(), 0, &q), "hipie_compile: tuning request");
+                    scratch.r.push_back(q);
+                    lanes.push_back({q->arena.as<uint8_t>(), q->stream});
+                }
                 DeviceGuard dg(device);
-                for (auto& s : plan->steps) s->tune(scratch->arena.as<uint8_t>(), plan->tensors, scratch->stream);
+                for (auto& s : plan->steps) s->tune(lanes, plan->tensors);
                 if (cache) {
                     if (FILE* f = std::fopen(cache, "w")) {
                         for (size_t i = 0; i < plan->steps.size(); ++i)
