@@ -10,7 +10,7 @@ namespace hipie {
 
 namespace {
 
-constexpr int kRow = 80;  // LDS row stride of the tiled kernel: 64 K-bytes + 16 pad
+constexpr int kRow = 64;  // LDS rows of the tiled kernels: 64 K-bytes, chunk c of row r in slot c ^ ((r >> 2) & 3)
 
 // ------------------------------------------------------------------------------------------------
 // LDS-tiled kernel
@@ -40,6 +40,11 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     const int woc = wave % WOC, wpix = wave / WOC;
     const int l32 = lane & 31, h = lane >> 5;
     const int chunk = tid & 3;
+    // XOR swizzle instead of row padding: the thread that stages (row, chunk) and the lanes that read
+    // fragments (rows l32 + 32 i, chunk 2 ks + h) agree on slot = chunk ^ ((row >> 2) & 3); rows that
+    // differ by a multiple of 16 share the swizzle, so (tid + i NT) >> 2 and l32 + 32 i need one value each
+    const int lds_slot = (chunk ^ ((tid >> 4) & 3)) * 16;
+    const int frag_slot[2] = {((0 + h) ^ ((l32 >> 2) & 3)) * 16, ((2 + h) ^ ((l32 >> 2) & 3)) * 16};
 
     const int batch = blockIdx.y;
     static_assert(BOC <= NT, "one table element per thread");
@@ -84,10 +89,10 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
         auto store_lds = [&](int buf) {
 #pragma unroll
             for (int i = 0; i < A_PIECES; ++i)
-                *reinterpret_cast<v4i*>(&sA[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = ga[i];
+                *reinterpret_cast<v4i*>(&sA[buf][((tid + i * NT) >> 2) * kRow + lds_slot]) = ga[i];
 #pragma unroll
             for (int i = 0; i < B_PIECES; ++i)
-                *reinterpret_cast<v4i*>(&sB[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = gb[i];
+                *reinterpret_cast<v4i*>(&sB[buf][((tid + i * NT) >> 2) * kRow + lds_slot]) = gb[i];
         };
         load_global(0);
         store_lds(0);
@@ -102,10 +107,10 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
                 v4i af[2], bf[2];
 #pragma unroll
                 for (int ob = 0; ob < 2; ++ob)
-                    af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][a_row[ob] * kRow + ks * 32 + h * 16]);
+                    af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][a_row[ob] * kRow + frag_slot[ks]]);
 #pragma unroll
                 for (int pb = 0; pb < 2; ++pb)
-                    bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][b_row[pb] * kRow + ks * 32 + h * 16]);
+                    bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][b_row[pb] * kRow + frag_slot[ks]]);
 #pragma unroll
                 for (int ob = 0; ob < 2; ++ob)
 #pragma unroll
@@ -177,6 +182,11 @@ __global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const C
     const int woc = wave % WOC, wpix = wave / WOC;
     const int l32 = lane & 31, h = lane >> 5;
     const int chunk = tid & 3;
+    // XOR swizzle instead of row padding: the thread that stages (row, chunk) and the lanes that read
+    // fragments (rows l32 + 32 i, chunk 2 ks + h) agree on slot = chunk ^ ((row >> 2) & 3); rows that
+    // differ by a multiple of 16 share the swizzle, so (tid + i NT) >> 2 and l32 + 32 i need one value each
+    const int lds_slot = (chunk ^ ((tid >> 4) & 3)) * 16;
+    const int frag_slot[2] = {((0 + h) ^ ((l32 >> 2) & 3)) * 16, ((2 + h) ^ ((l32 >> 2) & 3)) * 16};
     static_assert(BOC <= NT, "one table element per thread");
     StagedParams staged;
     stage_params_load<F>(a, oc0, BOC, tid, staged);
@@ -215,10 +225,10 @@ __global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const C
     auto store_lds = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < A_PIECES; ++i)
-            *reinterpret_cast<v4i*>(&sA[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = ga[i];
+            *reinterpret_cast<v4i*>(&sA[buf][((tid + i * NT) >> 2) * kRow + lds_slot]) = ga[i];
 #pragma unroll
         for (int i = 0; i < B_PIECES; ++i)
-            *reinterpret_cast<v4i*>(&sB[buf][((tid + i * NT) >> 2) * kRow + chunk * 16]) = gb[i];
+            *reinterpret_cast<v4i*>(&sB[buf][((tid + i * NT) >> 2) * kRow + lds_slot]) = gb[i];
     };
     auto addresses = [&](int pl, EpiAddr& e) {
         const int m0 = (xcd * a.p_per_xcd + pl) * BPIX + wpix * 64 + l32;
@@ -254,10 +264,10 @@ __global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const C
                 v4i af[2], bf[2];
 #pragma unroll
                 for (int ob = 0; ob < 2; ++ob)
-                    af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][a_row[ob] * kRow + ks * 32 + h * 16]);
+                    af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][a_row[ob] * kRow + frag_slot[ks]]);
 #pragma unroll
                 for (int pb = 0; pb < 2; ++pb)
-                    bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][b_row[pb] * kRow + ks * 32 + h * 16]);
+                    bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][b_row[pb] * kRow + frag_slot[ks]]);
 #pragma unroll
                 for (int ob = 0; ob < 2; ++ob)
 #pragma unroll
