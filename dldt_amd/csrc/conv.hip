@@ -15,7 +15,7 @@ constexpr int kRow = 64;  // LDS rows of the tiled kernels: 64 K-bytes, chunk c 
 // ------------------------------------------------------------------------------------------------
 // LDS-tiled kernel
 template <int WOC, int WPIX, uint32_t F>
-__global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && (F & CF_RES_GEMM))) ? 3 : 2) void conv_tiled_kernel(const ConvArgs a) {
+__global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && (F & CF_RES_GEMM))) ? (F == kDyn ? 3 : 4) : 2) void conv_tiled_kernel(const ConvArgs a) {
     constexpr int NT = WOC * WPIX * 64;
     constexpr int BOC = WOC * 64, BPIX = WPIX * 64;
     constexpr int A_PIECES = BOC * 4 / NT, B_PIECES = BPIX * 4 / NT;
