@@ -18,7 +18,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-ffp-contract=off",                       # float op order is part of the bit-exact contract
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes", "-Wno-pass-failed",
     "-I", os.path.join(os.path.dirname(HERE), "include"),
 ]
 

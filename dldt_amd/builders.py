@@ -398,3 +398,105 @@ def mobilenet_v2(batch=1, res=224, seed=20211, classes=1000, width=1.0, blocks=M
     g.result(logits, "logits")
     macs += P["fc.w"].size
     return g, dict(params=P, ranges=R, acts=acts, macs_per_image=macs, calib=calib)
+
+
+# ---------------------------------------------------------------------------------------------
+BERT_RANGES = dict(x=4.0, q=1.2, k=3.0, v=3.0, p=1.0, ctx=1.0, h1=4.0, g=3.0)
+
+
+def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, seed=20211, ranges=None):
+    """BASELINE config 5: BERT-base style encoder stack in its post-LPT form.  Activations are
+    per-tensor symmetric i8 (FakeQuantize ranges of signed_range), weights per-channel i8, Softmax /
+    LayerNorm (MVN, Multiply, Add) / Gelu stay f32.
+
+    Per layer, with x the f32 hidden states [batch, seq, hidden]:
+        xq = FQ(x);  q, k, v = FQ(MatMul'(xq, W^T) + b')        dequantization folded into the FQ range
+        s = MatMul'(heads(q), heads(k)^T) * (s_q s_k);  p = Softmax(s)   1/sqrt(d) folded into W_q
+        c = merge(MatMul'(FQ(p), heads(v)) * (s_p s_v))
+        a = (MatMul'(FQ(c), W_o^T) + b') * s + x;  h1 = LayerNorm(a)
+        f = Gelu((MatMul'(FQ(h1), W_1^T) + b') * s)
+        o = (MatMul'(FQ(f), W_2^T) + b') * s + h1;  y = LayerNorm(o)
+    (MatMulTransformation, mat_mul.cpp:81-171; AddTransformation moves the bias in front of the
+    Multiply, add.cpp:125-153; FakeQuantizeTransformation::fuseElementwise, fake_quantize.cpp:127-157.)
+
+    Returns (graph, meta); meta["layers"][l] maps tensor names to node ids, meta["glue"] lists the
+    nodes that only have tolerance parity (Softmax, LayerNorm tails, Gelu)."""
+    assert hidden % heads == 0
+    D = hidden // heads
+    r = dict(BERT_RANGES)
+    r.update(ranges or {})
+    rng = np.random.default_rng(seed)
+    net = QuantizedNet()
+    g = net.g
+    nrm = lambda *shape: (rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02)).astype(np.float32)
+    x = g.parameter("hidden_states", (batch, seq, hidden))
+    meta = dict(layers=[], glue=[], macs=0)
+
+    def fq(v, absmax):
+        lo, hi = net.signed_range(absmax)
+        d = lpt.decompose_fake_quantize(256, lo, hi)
+        assert d["precision"] == I8
+        return dict(node=g.fake_quantize(v, lo, hi, d["new_low"], d["new_high"], 256, I8), scale=np.float32(d["scale"]))
+
+    def linear(act, w, b):
+        """MatMul' -> Add(b / s): returns (node, s[c])"""
+        wq, s_w = lpt.quantize_weights(w, 255)
+        s = (np.float32(act["scale"]) * s_w).astype(np.float32)
+        y = g.matmul(act["node"], g.constant(wq, I8), False, True)
+        return g.add(y, g.constant((b / s).astype(np.float32))), s
+
+    def linear_fq(act, w, b, absmax):
+        y, s = linear(act, w, b)
+        lo, hi = net.signed_range(absmax)
+        d = lpt.decompose_fake_quantize(256, lo, hi)
+        q = g.fake_quantize(y, (lo / s).astype(np.float32), (hi / s).astype(np.float32), d["new_low"], d["new_high"],
+                            256, I8)
+        return dict(node=q, scale=np.float32(d["scale"]))
+
+    def linear_f32(act, w, b):
+        y, s = linear(act, w, b)
+        return g.multiply(y, g.constant(s))
+
+    def layer_norm(v):
+        n = g.mvn(v, (-1,), True, 1e-5, True)
+        out = g.add(g.multiply(n, g.constant(np.float32(1) + nrm(hidden))), g.constant(nrm(hidden)))
+        meta["glue"].append(out)
+        return out
+
+    def split_heads(node):
+        return g.transpose(g.reshape(node, (batch, seq, heads, D)), (0, 2, 1, 3))
+
+    for _ in range(layers):
+        L = {}
+        wq_ = nrm(hidden, hidden) * np.float32(1.0 / np.sqrt(D))
+        xq = fq(x, r["x"])
+        q = linear_fq(xq, wq_, nrm(hidden), r["q"])
+        k = linear_fq(xq, nrm(hidden, hidden), nrm(hidden), r["k"])
+        v = linear_fq(xq, nrm(hidden, hidden), nrm(hidden), r["v"])
+        s = g.multiply(g.matmul(split_heads(q["node"]), split_heads(k["node"]), False, True),
+                       g.constant(np.float32(q["scale"] * k["scale"]).reshape(())))
+        p = g.softmax(s, -1)
+        meta["glue"].append(p)
+        pq = fq(p, r["p"])
+        c = g.multiply(g.matmul(pq["node"], split_heads(v["node"])),
+                       g.constant(np.float32(pq["scale"] * v["scale"]).reshape(())))
+        c_t = g.transpose(c, (0, 2, 1, 3))
+        c_m = g.reshape(c_t, (batch, seq, hidden))
+        cq = fq(c_m, r["ctx"])
+        a = g.add(linear_f32(cq, nrm(hidden, hidden), nrm(hidden)), x)
+        h1 = layer_norm(a)
+        h1q = fq(h1, r["h1"])
+        f = linear_f32(h1q, nrm(ffn, hidden), nrm(ffn))
+        gl = g.gelu(f)
+        meta["glue"].append(gl)
+        gq = fq(gl, r["g"])
+        o = g.add(linear_f32(gq, nrm(hidden, ffn), nrm(hidden)), h1)
+        y = layer_norm(o)
+        L.update(xq=xq["node"], q=q["node"], k=k["node"], v=v["node"], scores=s, p=p, pq=pq["node"], ctx=c_t,
+                 ctxq=cq["node"], attn=a, h1=h1, h1q=h1q["node"], up=f, gelu=gl, gq=gq["node"], down=o, y=y)
+        meta["layers"].append(L)
+        x = y
+    g.result(x, "out")
+    T = batch * seq
+    meta["macs"] = layers * (T * (4 * hidden * hidden + 2 * hidden * ffn) + 2 * batch * heads * seq * seq * D)
+    return g, meta

@@ -8,8 +8,9 @@ namespace hipie {
 const char* op_name(int op) {
     static const char* names[] = {"Parameter", "Constant", "FakeQuantize", "Convolution",
                                   "GroupConvolution", "MatMul", "Add", "Multiply", "Subtract", "Relu",
-                                  "Clamp", "Convert", "MaxPool", "AvgPool", "Reshape", "Result"};
-    return op >= 0 && op <= OP_RESULT ? names[op] : "?";
+                                  "Clamp", "Convert", "MaxPool", "AvgPool", "Reshape", "Result", "Softmax", "MVN",
+                                  "Gelu", "Transpose"};
+    return op >= 0 && op <= OP_TRANSPOSE ? names[op] : "?";
 }
 
 namespace {
@@ -320,6 +321,88 @@ int hipie_graph_reshape(hipie_graph* g, int x, const int64_t* dims, int rank, in
         n.shape.assign(dims, dims + rank);
         HIPIE_REQUIRE(n.numel() == X.numel(), HIPIE_PARAMETER_MISMATCH,
                       "hipie_graph_reshape: element count changes");
+        *id = add_node(g, std::move(n));
+    });
+}
+
+/* op::v1::Softmax (ngraph/core/src/op/softmax.cpp): same shape and type; the axis may be negative */
+int hipie_graph_softmax(hipie_graph* g, int x, int64_t axis, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_softmax: null argument");
+        GNode& X = node(g, x, "hipie_graph_softmax");
+        const int64_t r = static_cast<int64_t>(X.shape.size());
+        HIPIE_REQUIRE(X.dtype == HIPIE_F32, HIPIE_PARAMETER_MISMATCH, "hipie_graph_softmax: data must be f32");
+        HIPIE_REQUIRE(axis >= -r && axis < r, HIPIE_PARAMETER_MISMATCH, "hipie_graph_softmax: axis %lld of rank %lld",
+                      (long long)axis, (long long)r);
+        GNode n;
+        n.op = OP_SOFTMAX;
+        n.in = {x};
+        n.axes = {axis < 0 ? axis + r : axis};
+        n.dtype = HIPIE_F32;
+        n.shape = X.shape;
+        *id = add_node(g, std::move(n));
+    });
+}
+
+/* op::v6::MVN (ngraph/core/src/op/mvn.cpp:93-140): the axes input is passed as an array */
+int hipie_graph_mvn(hipie_graph* g, int x, const int64_t* axes, int n_axes, int normalize_variance, float eps,
+                    int eps_inside_sqrt, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id && axes && n_axes > 0, HIPIE_PARAMETER_MISMATCH, "hipie_graph_mvn: null argument");
+        GNode& X = node(g, x, "hipie_graph_mvn");
+        const int64_t r = static_cast<int64_t>(X.shape.size());
+        HIPIE_REQUIRE(X.dtype == HIPIE_F32, HIPIE_PARAMETER_MISMATCH, "hipie_graph_mvn: data must be f32");
+        GNode n;
+        n.op = OP_MVN;
+        n.in = {x};
+        for (int i = 0; i < n_axes; ++i) {
+            HIPIE_REQUIRE(axes[i] >= -r && axes[i] < r, HIPIE_PARAMETER_MISMATCH, "hipie_graph_mvn: axis %lld of rank %lld",
+                          (long long)axes[i], (long long)r);
+            n.axes.push_back(axes[i] < 0 ? axes[i] + r : axes[i]);
+        }
+        n.normalize_variance = normalize_variance != 0;
+        n.eps = eps;
+        n.eps_inside_sqrt = eps_inside_sqrt != 0;
+        n.dtype = HIPIE_F32;
+        n.shape = X.shape;
+        *id = add_node(g, std::move(n));
+    });
+}
+
+/* op::v0::Gelu / op::v7::Gelu in ERF mode (ngraph/core/src/op/gelu.cpp) */
+int hipie_graph_gelu(hipie_graph* g, int x, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_gelu: null argument");
+        GNode& X = node(g, x, "hipie_graph_gelu");
+        HIPIE_REQUIRE(X.dtype == HIPIE_F32, HIPIE_PARAMETER_MISMATCH, "hipie_graph_gelu: data must be f32");
+        GNode n;
+        n.op = OP_GELU;
+        n.in = {x};
+        n.dtype = HIPIE_F32;
+        n.shape = X.shape;
+        *id = add_node(g, std::move(n));
+    });
+}
+
+/* op::v1::Transpose (ngraph/core/src/op/transpose.cpp:40-80): out.shape[i] = in.shape[order[i]] */
+int hipie_graph_transpose(hipie_graph* g, int x, const int64_t* order, int rank, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id && order, HIPIE_PARAMETER_MISMATCH, "hipie_graph_transpose: null argument");
+        GNode& X = node(g, x, "hipie_graph_transpose");
+        HIPIE_REQUIRE(rank == static_cast<int>(X.shape.size()), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_graph_transpose: order has %d entries for a rank-%zu value", rank, X.shape.size());
+        GNode n;
+        n.op = OP_TRANSPOSE;
+        n.in = {x};
+        std::vector<char> seen(rank, 0);
+        for (int i = 0; i < rank; ++i) {
+            HIPIE_REQUIRE(order[i] >= 0 && order[i] < rank && !seen[order[i]], HIPIE_PARAMETER_MISMATCH,
+                          "hipie_graph_transpose: order is not a permutation");
+            seen[order[i]] = 1;
+            n.axes.push_back(order[i]);
+            n.shape.push_back(X.shape[order[i]]);
+        }
+        n.dtype = X.dtype;
         *id = add_node(g, std::move(n));
     });
 }

@@ -21,6 +21,7 @@ struct TensorInfo {
     int n = 1, h = 1, w = 1, c = 1, cs = 16, halo = 0;
     int64_t offset = 0, bytes = 0;
     int producer = -1;       // graph node whose value it holds
+    int alias = -1;          // shares the bytes of this earlier tensor (same element count, other row split)
     int64_t esize() const { return dtype == HIPIE_F32 || dtype == HIPIE_I32 ? 4 : 1; }
     int wp() const { return w + 2 * halo; }
     int hp() const { return h + 2 * halo; }
@@ -36,12 +37,52 @@ struct TensorInfo {
     }
 };
 
-enum ValueKind { VK_NONE = 0, VK_PARAM, VK_CONST, VK_TENSOR, VK_DEQ, VK_FUSED };
+enum ValueKind { VK_NONE = 0, VK_PARAM, VK_CONST, VK_TENSOR, VK_DEQ, VK_FUSED, VK_MAT };
+
+// Row-major strided view of an arena tensor or of a request input buffer: how the values of a
+// transformer encoder (rank-3 Parameter [batch, sequence, hidden] and everything computed from it)
+// are held.  Memory order is the graph's own dimension order, so Reshape and Transpose are
+// arithmetic on shape / stride and move no bytes.
+struct View {
+    int tensor = -1, param = -1;
+    int dtype = HIPIE_F32;
+    std::vector<int64_t> shape, stride;   // stride in elements
+    int64_t offset = 0;                   // elements
+    int64_t esize() const { return dtype == HIPIE_F32 || dtype == HIPIE_I32 ? 4 : 1; }
+    int64_t numel() const {
+        int64_t n = 1;
+        for (auto d : shape) n *= d;
+        return n;
+    }
+    size_t rank() const { return shape.size(); }
+    static std::vector<int64_t> dense_strides(const std::vector<int64_t>& shape) {
+        std::vector<int64_t> st(shape.size());
+        int64_t s = 1;
+        for (size_t i = shape.size(); i-- > 0;) {
+            st[i] = s;
+            s *= shape[i];
+        }
+        return st;
+    }
+    bool dense() const {
+        int64_t s = 1;
+        for (size_t i = shape.size(); i-- > 0;) {
+            if (shape[i] != 1 && stride[i] != s) return false;
+            s *= shape[i];
+        }
+        return true;
+    }
+    uint8_t* ptr(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs) const {
+        uint8_t* base = tensor >= 0 ? arena + tensors[tensor].offset : static_cast<uint8_t*>(inputs[param]);
+        return base + offset * esize();
+    }
+};
 
 struct Value {
     int kind = VK_NONE;
     int tensor = -1;
     std::vector<float> sub, mul;   // VK_DEQ: (float(q) - sub) * mul, each empty / 1 / C values
+    View view;                     // VK_MAT
 };
 
 struct EpilogueSpec {
@@ -76,6 +117,7 @@ struct EpilogueSpec {
 struct TuneLane {
     uint8_t* arena;
     hipStream_t stream;
+    std::vector<void*> inputs;   // the scratch request's input buffers
 };
 
 struct Step {
@@ -120,6 +162,7 @@ struct EntryStep : Step {
 
 struct ConvStep : Step {
     int in = -1, res = -1, out = -1;
+    int res_param = -1;            // f32 residual read from this request input instead of the arena
     hipie_conv_desc desc{};
     std::vector<int8_t> weights;   // OIHW
     EpilogueSpec epi;
@@ -173,8 +216,20 @@ struct ConvStep : Step {
         } else {
             if (shortcut) shortcut->run(arena, tensors, inputs, outputs, s);
             if (res >= 0) r = tensors[res].desc(arena);
+            else if (res_param >= 0) r = input_residual(o, inputs[res_param]);
         }
-        check_status(hipie_conv_run(conv, &i, (fused || res >= 0) ? &r : nullptr, &o, s), name.c_str());
+        check_status(hipie_conv_run(conv, &i, (fused || res >= 0 || res_param >= 0) ? &r : nullptr, &o, s), name.c_str());
+    }
+    // a dense f32 [rows, channels] request input as the residual operand of output tensor `o`
+    static hipie_tensor input_residual(const hipie_tensor& o, void* data) {
+        hipie_tensor r = o;
+        r.data = data;
+        r.dtype = HIPIE_F32;
+        r.stride_w = o.c;
+        r.stride_h = static_cast<int64_t>(o.w) * o.c;
+        r.stride_n = static_cast<int64_t>(o.h) * r.stride_h;
+        r.halo = 0;
+        return r;
     }
     int variant() const override {
         int t = -1;
@@ -198,8 +253,9 @@ struct ConvStep : Step {
             to[l] = tensors[out].desc(lanes[l].arena);
             if (fused) tr[l] = tensors[shortcut->in].desc(lanes[l].arena);
             else if (res >= 0) tr[l] = tensors[res].desc(lanes[l].arena);
+            else if (res_param >= 0) tr[l] = input_residual(to[l], lanes[l].inputs[res_param]);
         }
-        const bool has_res = fused || res >= 0;
+        const bool has_res = fused || res >= 0 || res_param >= 0;
         auto launch_all = [&](int times) {
             for (int w = 0; w < times; ++w)
                 for (size_t l = 0; l < nl; ++l)
@@ -362,6 +418,109 @@ struct ExitStep : Step {
     }
 };
 
+// ---- steps over row-major views (transformer encoders) ------------------------------------------
+
+// FakeQuantize of a dense f32 value with per-tensor bounds -> i8 levels
+struct MatFqStep : Step {
+    View in;
+    int out = -1;
+    int64_t n = 0, levels = 0;
+    float il = 0, ih = 0, ol = 0, oh = 0;
+    hipie_fq* fq = nullptr;
+    ~MatFqStep() override { hipie_fq_destroy(fq); }
+    void create(int device, const std::vector<TensorInfo>&) override {
+        check_status(hipie_fq_create(device, 1, levels, &il, 1, &ih, 1, &ol, 1, &oh, 1, &fq), name.c_str());
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
+             hipStream_t s) const override {
+        check_status(hipie_fq_run_q8(fq, reinterpret_cast<const float*>(in.ptr(arena, tensors, inputs)),
+                                     arena + tensors[out].offset, 1, n, HIPIE_I8, HIPIE_NCHW, 0, s), name.c_str());
+    }
+};
+
+// Softmax / MVN (+ LayerNorm gamma, beta) / Gelu over the last axis of a dense f32 value
+struct GlueStep : Step {
+    int kind = OP_SOFTMAX;
+    View in;
+    int out = -1;
+    int64_t rows = 0, axis = 0;
+    bool normalize_variance = true, eps_inside_sqrt = true;
+    float eps = 0;
+    std::vector<float> gamma, beta;
+    DeviceBuffer d_gamma, d_beta;
+    void create(int device, const std::vector<TensorInfo>&) override {
+        if (device < 0) return;
+        if (!gamma.empty()) d_gamma.upload(device, gamma.data(), gamma.size() * 4);
+        if (!beta.empty()) d_beta.upload(device, beta.data(), beta.size() * 4);
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
+             hipStream_t s) const override {
+        const float* x = reinterpret_cast<const float*>(in.ptr(arena, tensors, inputs));
+        float* y = reinterpret_cast<float*>(arena + tensors[out].offset);
+        int st = HIPIE_OK;
+        if (kind == OP_SOFTMAX) st = hipie_softmax_f32(x, y, rows, axis, s);
+        else if (kind == OP_GELU) st = hipie_gelu_f32(x, y, rows * axis, s);
+        else st = hipie_mvn_f32(x, y, rows, axis, normalize_variance, eps, eps_inside_sqrt,
+                                gamma.empty() ? nullptr : d_gamma.as<float>(), beta.empty() ? nullptr : d_beta.as<float>(), s);
+        check_status(st, name.c_str());
+    }
+};
+
+// MatMul between two i8 activations, batched over one or two leading dimensions
+struct BatchMatMulStep : Step {
+    View a, b;                     // b as [.., N, K] with K contiguous
+    int out = -1;
+    int64_t lda = 0, sa = 0, oa = 0, ldb = 0, sb = 0, ob = 0, ldo = 0, so = 0, oo = 0;
+    int32_t m = 0, k = 0, n = 0, batch = 1, outer = 1;
+    EpilogueSpec epi;
+    hipie_matmul* mm = nullptr;
+    ~BatchMatMulStep() override { hipie_matmul_destroy(mm); }
+    void create(int device, const std::vector<TensorInfo>&) override {
+        hipie_matmul_desc d{};
+        d.a_dtype = a.dtype;
+        d.b_dtype = b.dtype;
+        d.k = k;
+        d.n = n;
+        const hipie_epilogue e = epi.c_struct();
+        check_status(hipie_matmul_create(device, &d, &e, &mm), name.c_str());
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
+             hipStream_t s) const override {
+        check_status(hipie_matmul_run_nested(mm, a.ptr(arena, tensors, inputs), lda, sa, oa, b.ptr(arena, tensors, inputs), ldb,
+                                             sb, ob, arena + tensors[out].offset, ldo, so, oo, m, batch, outer, s),
+                     name.c_str());
+    }
+};
+
+// physical transpose of the two inner dimensions of a byte view (the right operand of a MatMul whose
+// reduction axis is not contiguous)
+struct MatTransposeStep : Step {
+    View in;                       // [.., rows, cols], cols contiguous
+    int out = -1;                  // dense [.., cols, rows]
+    int64_t ld_src = 0, s_src = 0, o_src = 0, ld_dst = 0, s_dst = 0, o_dst = 0;
+    int32_t rows = 0, cols = 0, batch = 1, outer = 1;
+    void create(int, const std::vector<TensorInfo>&) override {}
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
+             hipStream_t s) const override {
+        check_status(hipie_transpose_bytes_nested(in.ptr(arena, tensors, inputs), ld_src, s_src, o_src,
+                                                  arena + tensors[out].offset, ld_dst, s_dst, o_dst, rows, cols, batch,
+                                                  outer, s), name.c_str());
+    }
+};
+
+// Result of a dense row-major value: its bytes are the output buffer's
+struct MatExitStep : Step {
+    View in;
+    int result_index = 0;
+    int64_t nbytes = 0;
+    void create(int, const std::vector<TensorInfo>&) override {}
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const* outputs,
+             hipStream_t s) const override {
+        HIPIE_CHECK_HIP(hipMemcpyAsync(outputs[result_index], in.ptr(arena, tensors, inputs), static_cast<size_t>(nbytes),
+                                       hipMemcpyDeviceToDevice, s));
+    }
+};
+
 // ------------------------------------------------------------------------------------------------
 struct Planner {
     const hipie_graph& g;
@@ -435,18 +594,416 @@ struct Planner {
 
     void plan_node(int id) {
         const GNode& n = N(id);
+        const bool mat = !n.in.empty() && n.op != OP_CONSTANT && value(n.in[0]).kind == VK_MAT;
         switch (n.op) {
-        case OP_PARAMETER: values[id].kind = VK_PARAM; break;
+        case OP_PARAMETER: plan_parameter(id); break;
         case OP_CONSTANT: values[id].kind = VK_CONST; break;
-        case OP_FAKE_QUANTIZE: plan_fake_quantize(id); break;
-        case OP_CONVOLUTION: case OP_MATMUL: case OP_GROUP_CONVOLUTION: plan_conv(id); break;
+        case OP_FAKE_QUANTIZE: mat ? plan_mat_fq(id) : plan_fake_quantize(id); break;
+        case OP_MATMUL: mat ? plan_mat_matmul(id) : plan_conv(id); break;
+        case OP_CONVOLUTION: case OP_GROUP_CONVOLUTION: plan_conv(id); break;
         case OP_CONVERT: case OP_SUBTRACT: case OP_MULTIPLY: plan_dequant(id); break;
         case OP_MAX_POOL: case OP_AVG_POOL: plan_pool(id); break;
-        case OP_RESHAPE: plan_reshape(id); break;
-        case OP_RESULT: plan_result(id); values[id].kind = VK_FUSED; break;
+        case OP_RESHAPE: mat ? plan_mat_reshape(id) : plan_reshape(id); break;
+        case OP_TRANSPOSE: plan_mat_transpose(id); break;
+        case OP_SOFTMAX: case OP_MVN: case OP_GELU: plan_glue(id); break;
+        case OP_RESULT: mat ? plan_mat_result(id) : plan_result(id); values[id].kind = VK_FUSED; break;
         default: unsupported(id, "only planned as part of a fused convolution / pooling chain");
         }
         if (values[id].kind == VK_NONE) unsupported(id, "planner produced no value");
+    }
+
+
+    // ---- row-major world: values of a transformer encoder ---------------------------------------
+    // A rank-3 Parameter [batch, sequence, hidden] is read where the request keeps it.
+    void plan_parameter(int id) {
+        const GNode& n = N(id);
+        if (n.shape.size() != 3) {
+            values[id].kind = VK_PARAM;
+            return;
+        }
+        HIPIE_REQUIRE(n.dtype == HIPIE_F32, HIPIE_NOT_IMPLEMENTED, "node %d: rank-3 inputs must be f32", id);
+        View v;
+        for (size_t i = 0; i < g.params.size(); ++i)
+            if (g.params[i] == id) v.param = static_cast<int>(i);
+        v.dtype = HIPIE_F32;
+        v.shape = n.shape;
+        v.stride = View::dense_strides(n.shape);
+        values[id].kind = VK_MAT;
+        values[id].view = v;
+    }
+
+    // constant broadcastable along the last axis: 1 or C numbers
+    bool last_axis_constant(int id, int64_t C, std::vector<float>& v) const {
+        const GNode& c = N(id);
+        if (c.op != OP_CONSTANT || c.dtype != HIPIE_F32) return false;
+        const int64_t n = c.numel();
+        if (n == 1) { v.assign(1, c.f32()[0]); return true; }
+        if (n != C || c.shape.empty() || c.shape.back() != C) return false;
+        v.assign(c.f32(), c.f32() + C);
+        return true;
+    }
+
+    // dense [rows, cols] arena tensor for a value of `shape` (cols = last dimension)
+    int new_matrix(int node, int dtype, const std::vector<int64_t>& shape) {
+        int64_t numel = 1;
+        for (auto d : shape) numel *= d;
+        const int64_t cols = shape.back();
+        const int gran = dtype == HIPIE_F32 ? 4 : 16;
+        if (cols % gran != 0) unsupported(node, "last dimension must be a multiple of 16 (bytes) / 4 (f32)");
+        return new_tensor(node, dtype, 1, 1, static_cast<int>(numel / cols), static_cast<int>(cols), static_cast<int>(cols));
+    }
+
+    void set_matrix_value(int id, int tensor, int dtype) {
+        View v;
+        v.tensor = tensor;
+        v.dtype = dtype;
+        v.shape = N(id).shape;
+        v.stride = View::dense_strides(v.shape);
+        values[id].kind = VK_MAT;
+        values[id].view = v;
+    }
+
+    // marks the nodes strictly between a chain's head and its last node as fused away
+    void mark_chain(int head, int last) {
+        for (int k = head; k != last;) {
+            const int nx = N(k).users[0];
+            if (nx != last) values[nx].kind = VK_FUSED;
+            k = nx;
+        }
+        if (last != head) values[head].kind = VK_FUSED;
+    }
+
+    const View& dense_f32_input(int id, const char* what) {
+        const Value& x = value(N(id).in[0]);
+        if (x.kind != VK_MAT || x.view.dtype != HIPIE_F32 || !x.view.dense()) unsupported(id, what);
+        return x.view;
+    }
+
+    void plan_mat_fq(int id) {
+        const GNode& n = N(id);
+        const View x = dense_f32_input(id, "FakeQuantize input must be a dense f32 value");
+        if (n.dtype != HIPIE_I8) unsupported(id, "activations of the row-major path are symmetric i8");
+        auto st = std::make_unique<MatFqStep>();
+        float* dst[4] = {&st->il, &st->ih, &st->ol, &st->oh};
+        for (int i = 0; i < 4; ++i) {
+            std::vector<float> c;
+            if (!last_axis_constant(n.in[1 + i], -1, c)) unsupported(id, "FakeQuantize bounds must be per tensor");
+            *dst[i] = c[0];
+        }
+        st->in = x;
+        st->n = n.numel();
+        st->levels = n.levels;
+        st->out = new_matrix(id, HIPIE_I8, n.shape);
+        st->name = n.name;
+        st->type = "FakeQuantize";
+        st->bytes = n.numel() * 5;
+        st->out_node = id;
+        set_matrix_value(id, st->out, HIPIE_I8);
+        steps.push_back(std::move(st));
+    }
+
+    void plan_glue(int id) {
+        const GNode& n = N(id);
+        const View x = dense_f32_input(id, "Softmax / MVN / Gelu are planned on dense f32 values of the row-major path");
+        const int64_t r = static_cast<int64_t>(n.shape.size()), C = n.shape.back();
+        auto st = std::make_unique<GlueStep>();
+        st->kind = n.op;
+        if (n.op == OP_SOFTMAX && n.axes[0] != r - 1) unsupported(id, "Softmax over an axis other than the last");
+        if (n.op == OP_MVN && (n.axes.size() != 1 || n.axes[0] != r - 1)) unsupported(id, "MVN over axes other than the last");
+        int cur = id;
+        if (n.op == OP_MVN) {
+            st->normalize_variance = n.normalize_variance;
+            st->eps = n.eps;
+            st->eps_inside_sqrt = n.eps_inside_sqrt;
+            // LayerNorm: Multiply(gamma[C]) then Add(beta[C])
+            while (single_user(cur)) {
+                const int nx = N(cur).users[0];
+                const GNode& u = N(nx);
+                if (u.op != OP_MULTIPLY && u.op != OP_ADD) break;
+                std::vector<float> c;
+                if (!last_axis_constant(u.in[0] == cur ? u.in[1] : u.in[0], C, c)) break;
+                if (c.size() == 1) c.assign(static_cast<size_t>(C), c[0]);
+                if (u.op == OP_MULTIPLY && st->gamma.empty() && st->beta.empty()) st->gamma = c;
+                else if (u.op == OP_ADD && st->beta.empty()) st->beta = c;
+                else break;
+                cur = nx;
+            }
+            mark_chain(id, cur);
+        }
+        st->in = x;
+        st->axis = C;
+        st->rows = n.numel() / C;
+        st->out = new_matrix(cur, HIPIE_F32, n.shape);
+        st->name = N(cur).name;
+        st->type = op_name(n.op);
+        st->bytes = n.numel() * 8;
+        st->out_node = cur;
+        set_matrix_value(cur, st->out, HIPIE_F32);
+        steps.push_back(std::move(st));
+    }
+
+    // numpy's no-copy reshape: succeeds when every group of merged dimensions is contiguous in itself
+    static bool reshape_view(const View& v, const std::vector<int64_t>& ns, View& out) {
+        std::vector<int64_t> od, os;
+        for (size_t i = 0; i < v.shape.size(); ++i)
+            if (v.shape[i] != 1) { od.push_back(v.shape[i]); os.push_back(v.stride[i]); }
+        std::vector<int64_t> nstr(ns.size(), 1);
+        size_t oi = 0, oj = 1, ni = 0, nj = 1;
+        while (ni < ns.size() && oi < od.size()) {
+            int64_t np = ns[ni], op = od[oi];
+            while (np != op) {
+                if (np < op) { if (nj >= ns.size()) return false; np *= ns[nj++]; }
+                else { if (oj >= od.size()) return false; op *= od[oj++]; }
+            }
+            for (size_t k = oi; k + 1 < oj; ++k)
+                if (os[k] != od[k + 1] * os[k + 1]) return false;
+            nstr[nj - 1] = os[oj - 1];
+            for (size_t k = nj - 1; k > ni; --k) nstr[k - 1] = nstr[k] * ns[k];
+            ni = nj++;
+            oi = oj++;
+        }
+        for (size_t k = ni; k < ns.size(); ++k) {
+            if (ns[k] != 1) return false;
+            nstr[k] = 1;
+        }
+        if (oi < od.size()) return false;
+        out = v;
+        out.shape = ns;
+        out.stride = nstr;
+        return true;
+    }
+
+    void plan_mat_reshape(int id) {
+        const Value& x = value(N(id).in[0]);
+        View v;
+        if (!reshape_view(x.view, N(id).shape, v)) unsupported(id, "Reshape that would have to move bytes");
+        values[id].kind = VK_MAT;
+        values[id].view = v;
+    }
+
+    void plan_mat_transpose(int id) {
+        const GNode& n = N(id);
+        const Value& x = value(n.in[0]);
+        if (x.kind != VK_MAT) unsupported(id, "Transpose is planned on values of the row-major path");
+        View v = x.view;
+        for (size_t i = 0; i < n.axes.size(); ++i) {
+            v.shape[i] = x.view.shape[n.axes[i]];
+            v.stride[i] = x.view.stride[n.axes[i]];
+        }
+        values[id].kind = VK_MAT;
+        values[id].view = v;
+    }
+
+    void plan_mat_result(int id) {
+        const GNode& n = N(id);
+        const Value& x = value(n.in[0]);
+        if (!x.view.dense()) unsupported(id, "Result of a transposed view");
+        auto st = std::make_unique<MatExitStep>();
+        st->in = x.view;
+        st->nbytes = x.view.numel() * x.view.esize();
+        for (size_t i = 0; i < g.results.size(); ++i)
+            if (g.results[i] == id) st->result_index = static_cast<int>(i);
+        st->name = n.name;
+        st->type = "Result";
+        st->bytes = st->nbytes * 2;
+        st->out_node = id;
+        steps.push_back(std::move(st));
+    }
+
+    void plan_mat_matmul(int id) {
+        const GNode& n = N(id);
+        const Value a = value(n.in[0]);
+        if (a.view.dtype != HIPIE_I8) unsupported(id, "left operand must be quantized to i8");
+        if (n.ta) unsupported(id, "transpose_a");
+        if (N(n.in[1]).op == OP_CONSTANT) plan_linear(id, a.view);
+        else plan_batch_matmul(id, a.view);
+    }
+
+    // MatMul against constant i8 weights: a 1x1 convolution over [rows, K]
+    void plan_linear(int id, const View& av) {
+        const GNode& n = N(id);
+        const GNode& W = N(n.in[1]);
+        if (W.dtype != HIPIE_I8 || W.shape.size() != 2) unsupported(id, "weights must be a rank-2 i8 constant");
+        if (!av.dense() || av.tensor < 0 || av.offset != 0) unsupported(id, "left operand must be a whole dense tensor");
+        const int64_t IC = n.tb ? W.shape[1] : W.shape[0], OC = n.tb ? W.shape[0] : W.shape[1];
+        HIPIE_REQUIRE(av.shape.back() == IC, HIPIE_PARAMETER_MISMATCH, "node %d: inner dimensions %lld vs %lld", id,
+                      (long long)av.shape.back(), (long long)IC);
+        const int64_t T = av.numel() / IC;
+        auto st = std::make_unique<ConvStep>();
+        st->in = av.tensor;
+        if (tensors[av.tensor].w != T || tensors[av.tensor].c != IC) {   // same bytes, other row split
+            if (IC % 16 != 0) unsupported(id, "reduction length must be a multiple of 16");
+            st->in = new_tensor(tensors[av.tensor].producer, HIPIE_I8, 1, 1, static_cast<int>(T), static_cast<int>(IC),
+                                static_cast<int>(IC));
+            tensors[st->in].alias = av.tensor;
+        }
+        hipie_conv_desc& d = st->desc;
+        d.groups = 1;
+        d.kh = d.kw = d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1;
+        d.ic = static_cast<int>(IC);
+        d.oc = static_cast<int>(OC);
+        st->weights.resize(OC * IC);
+        const int8_t* w = reinterpret_cast<const int8_t*>(W.data.data());
+        for (int64_t o = 0; o < OC; ++o)
+            for (int64_t k = 0; k < IC; ++k) st->weights[o * IC + k] = n.tb ? w[o * IC + k] : w[k * OC + o];
+
+        EpilogueSpec& e = st->epi;
+        int cur = id, stage = 0;
+        while (single_user(cur)) {
+            const int nx = N(cur).users[0];
+            const GNode& u = N(nx);
+            if (u.op == OP_ADD || u.op == OP_MULTIPLY) {
+                const int other = u.in[0] == cur ? u.in[1] : u.in[0];
+                std::vector<float> c;
+                if (last_axis_constant(other, OC, c)) {
+                    if (u.op == OP_ADD && stage < 1) { e.bias = c; stage = 1; }
+                    else if (u.op == OP_MULTIPLY && stage < 2) { e.scale = c; stage = 2; }
+                    else break;
+                } else if (u.op == OP_ADD && stage < 3 && N(other).op != OP_CONSTANT) {
+                    if (!visit(other)) break;
+                    const Value& r = values[other];
+                    if (r.kind != VK_MAT || r.view.dtype != HIPIE_F32 || !r.view.dense() || r.view.offset != 0 ||
+                        N(other).shape != u.shape)
+                        break;
+                    if (r.view.tensor >= 0 && (tensors[r.view.tensor].w != T || tensors[r.view.tensor].c != OC)) break;
+                    e.residual_dtype = HIPIE_F32;
+                    st->res = r.view.tensor;
+                    st->res_param = r.view.param;
+                    stage = 3;
+                } else {
+                    break;
+                }
+            } else if (u.op == OP_FAKE_QUANTIZE && u.in[0] == cur && u.dtype == HIPIE_I8) {
+                std::vector<float> ol, oh;
+                if (!last_axis_constant(u.in[1], OC, e.fq_il) || !last_axis_constant(u.in[2], OC, e.fq_ih) ||
+                    !last_axis_constant(u.in[3], -1, ol) || !last_axis_constant(u.in[4], -1, oh))
+                    break;
+                e.fq_ol = ol[0];
+                e.fq_oh = oh[0];
+                e.levels = u.levels;
+                e.out_dtype = HIPIE_I8;
+                cur = nx;
+                break;
+            } else {
+                break;
+            }
+            cur = nx;
+        }
+        mark_chain(id, cur);
+        st->out = new_matrix(cur, e.out_dtype, N(cur).shape);
+        st->name = N(cur).name;
+        st->type = "MatMul";
+        st->macs = T * OC * IC;
+        st->in_w_bytes = T * IC + OC * IC;
+        st->bytes = st->in_w_bytes + T * OC * (e.out_dtype == HIPIE_F32 ? 4 : 1) + (stage == 3 ? T * OC * 4 : 0);
+        st->out_node = cur;
+        set_matrix_value(cur, st->out, e.out_dtype);
+        steps.push_back(std::move(st));
+    }
+
+    // byte strides of the one or two batch dimensions in front of a [.., rows, cols] view
+    static void batch_strides(const View& v, int64_t& inner, int64_t& outer) {
+        const size_t r = v.rank();
+        inner = r >= 3 ? v.stride[r - 3] : 0;
+        outer = r >= 4 ? v.stride[r - 4] : 0;
+    }
+
+    void plan_batch_matmul(int id, const View& av) {
+        const GNode& n = N(id);
+        const Value bval = value(n.in[1]);
+        if (bval.kind != VK_MAT || bval.view.dtype != HIPIE_I8) unsupported(id, "right operand must be quantized to i8");
+        View bv = bval.view;
+        const size_t r = av.rank();
+        if (r < 3 || r > 4 || bv.rank() != r) unsupported(id, "MatMul between activations needs equal ranks of 3 or 4");
+        if (!n.tb) {   // bring the right operand to its [.., N, K] form
+            std::swap(bv.shape[r - 1], bv.shape[r - 2]);
+            std::swap(bv.stride[r - 1], bv.stride[r - 2]);
+        }
+        const int64_t M = av.shape[r - 2], K = av.shape[r - 1], Nn = bv.shape[r - 2];
+        HIPIE_REQUIRE(bv.shape[r - 1] == K, HIPIE_PARAMETER_MISMATCH, "node %d: inner dimensions %lld vs %lld", id,
+                      (long long)K, (long long)bv.shape[r - 1]);
+        for (size_t i = 0; i + 2 < r; ++i)
+            if (av.shape[i] != bv.shape[i]) unsupported(id, "broadcast batch dimensions");
+        if (av.stride[r - 1] != 1) unsupported(id, "left operand with a strided reduction axis");
+        if (K % 64 != 0) unsupported(id, "reduction length must be a multiple of 64");
+        const int32_t inner = static_cast<int32_t>(av.shape[r - 3]), outer = r == 4 ? static_cast<int32_t>(av.shape[0]) : 1;
+        if (bv.stride[r - 1] != 1) {
+            // reduction axis not contiguous: transpose the operand's inner dimensions into a new tensor
+            if (bv.stride[r - 2] != 1) unsupported(id, "right operand with both inner dimensions strided");
+            auto tp = std::make_unique<MatTransposeStep>();
+            tp->in = bv;             // as [.., N, K]: in memory K rows of N contiguous bytes
+            tp->rows = static_cast<int32_t>(K);
+            tp->cols = static_cast<int32_t>(Nn);
+            tp->ld_src = bv.stride[r - 1];
+            batch_strides(bv, tp->s_src, tp->o_src);
+            std::vector<int64_t> tshape(bv.shape);
+            tp->out = new_matrix(n.in[1], HIPIE_I8, tshape);
+            const auto ds = View::dense_strides(tshape);
+            tp->ld_dst = K;
+            tp->s_dst = ds[r - 3];
+            tp->o_dst = r == 4 ? ds[0] : 0;
+            tp->batch = inner;
+            tp->outer = outer;
+            tp->name = N(n.in[1]).name + "/transposed";
+            tp->type = "Transpose";
+            tp->bytes = 2 * bv.numel();
+            View nb;
+            nb.tensor = tp->out;
+            nb.dtype = HIPIE_I8;
+            nb.shape = tshape;
+            nb.stride = ds;
+            bv = nb;
+            steps.push_back(std::move(tp));
+        }
+        auto st = std::make_unique<BatchMatMulStep>();
+        st->a = av;
+        st->b = bv;
+        st->m = static_cast<int32_t>(M);
+        st->k = static_cast<int32_t>(K);
+        st->n = static_cast<int32_t>(Nn);
+        st->batch = inner;
+        st->outer = outer;
+        st->lda = av.stride[r - 2];
+        batch_strides(av, st->sa, st->oa);
+        st->ldb = bv.stride[r - 2];
+        batch_strides(bv, st->sb, st->ob);
+        // epilogue: the dequantization Multiply(s_a * s_b), then optionally a Transpose that keeps the
+        // last axis last (the head merge of attention), written through the output strides
+        EpilogueSpec& e = st->epi;
+        e.out_dtype = HIPIE_F32;
+        int cur = id;
+        std::vector<int64_t> oshape = n.shape;
+        std::vector<int64_t> ostride = View::dense_strides(oshape);   // of the MatMul's own dimensions
+        while (single_user(cur)) {
+            const int nx = N(cur).users[0];
+            const GNode& u = N(nx);
+            std::vector<float> c;
+            if (u.op == OP_MULTIPLY && e.scale.empty() &&
+                last_axis_constant(u.in[0] == cur ? u.in[1] : u.in[0], -1, c)) {
+                e.scale = c;
+            } else if (u.op == OP_TRANSPOSE && u.axes.back() == static_cast<int64_t>(r) - 1 && oshape == n.shape) {
+                oshape = u.shape;
+                const auto ts = View::dense_strides(oshape);
+                for (size_t p = 0; p < r; ++p) ostride[u.axes[p]] = ts[p];
+                cur = nx;
+                break;
+            } else {
+                break;
+            }
+            cur = nx;
+        }
+        mark_chain(id, cur);
+        st->out = new_matrix(cur, HIPIE_F32, oshape);
+        st->ldo = ostride[r - 2];
+        st->so = ostride[r - 3];
+        st->oo = r == 4 ? ostride[0] : 0;
+        st->name = N(cur).name;
+        st->type = "MatMul";
+        st->macs = n.numel() * K;
+        st->bytes = av.numel() + bv.numel() + n.numel() * 4;
+        st->out_node = cur;
+        set_matrix_value(cur, st->out, HIPIE_F32);
+        steps.push_back(std::move(st));
     }
 
     void plan_fake_quantize(int id) {
@@ -834,6 +1391,10 @@ int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
         int64_t off = 256;
         for (auto& t : pl.tensors) {
             t.bytes = static_cast<int64_t>(t.n) * t.hp() * t.wp() * t.cs * t.esize();
+            if (t.alias >= 0) {
+                t.offset = pl.tensors[t.alias].offset;
+                continue;
+            }
             t.offset = off;
             off = round_up(off + t.bytes + 256, 256);
         }
@@ -842,7 +1403,14 @@ int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
         for (auto& s : pl.steps) s->create(device, plan->tensors);
         plan->steps = std::move(pl.steps);
         for (size_t i = 0; i < pl.values.size(); ++i)
-            if (pl.values[i].kind == VK_TENSOR) plan->node_tensor[static_cast<int>(i)] = pl.values[i].tensor;
+            if (pl.values[i].kind == VK_TENSOR) {
+                plan->node_tensor[static_cast<int>(i)] = pl.values[i].tensor;
+            } else if (pl.values[i].kind == VK_MAT) {   // a dense view that is its whole tensor
+                const View& v = pl.values[i].view;
+                if (v.tensor >= 0 && v.offset == 0 && v.dense() &&
+                    v.numel() == static_cast<int64_t>(pl.tensors[v.tensor].w) * pl.tensors[v.tensor].c)
+                    plan->node_tensor[static_cast<int>(i)] = v.tensor;
+            }
         for (int p : g->params) {
             const GNode& n = g->nodes[p];
             plan->inputs.push_back({n.name, n.dtype, n.shape, n.numel() * (n.dtype == HIPIE_F32 ? 4 : 1)});
@@ -894,7 +1462,9 @@ int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
                     hipie_request* q = nullptr;
                     check_status(hipie_request_create(plan.get(), 0, &q), "hipie_compile: tuning request");
                     scratch.r.push_back(q);
-                    lanes.push_back({q->arena.as<uint8_t>(), q->stream});
+                    TuneLane lane{q->arena.as<uint8_t>(), q->stream, {}};
+                    for (auto& b : q->in_dev) lane.inputs.push_back(b.ptr);
+                    lanes.push_back(std::move(lane));
                 }
                 DeviceGuard dg(device);
                 for (auto& s : plan->steps) s->tune(lanes, plan->tensors);

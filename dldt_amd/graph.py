@@ -122,6 +122,28 @@ class Graph:
         check(lib().hipie_graph_reshape(self._h, x, _i64(shape), len(shape), ctypes.byref(i)))
         return self._rec(i.value, "Reshape", [x], self.nodes[x]["dtype"], shape=tuple(shape))
 
+    def softmax(self, x, axis=-1):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_softmax(self._h, x, ctypes.c_int64(axis), ctypes.byref(i)))
+        return self._rec(i.value, "Softmax", [x], F32, axis=axis)
+
+    def mvn(self, x, axes=(-1,), normalize_variance=True, eps=1e-5, eps_inside_sqrt=True):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_mvn(self._h, x, _i64(axes), len(axes), int(normalize_variance), ctypes.c_float(eps),
+                                    int(eps_inside_sqrt), ctypes.byref(i)))
+        return self._rec(i.value, "MVN", [x], F32, axes=tuple(axes), normalize_variance=normalize_variance,
+                         eps=float(eps), eps_inside_sqrt=eps_inside_sqrt)
+
+    def gelu(self, x):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_gelu(self._h, x, ctypes.byref(i)))
+        return self._rec(i.value, "Gelu", [x], F32)
+
+    def transpose(self, x, order):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_transpose(self._h, x, _i64(order), len(order), ctypes.byref(i)))
+        return self._rec(i.value, "Transpose", [x], self.nodes[x]["dtype"], order=tuple(order))
+
     def result(self, x, name):
         check(lib().hipie_graph_result(self._h, x, name.encode()))
         self.results.append(len(self.nodes))
@@ -230,6 +252,11 @@ class Request:
             check(lib().hipie_request_perf(self._h, i, ctypes.byref(ms)))
             out.append(dict(st, ms=ms.value))
         return out
+
+    def matrix(self, node_id):
+        """numpy [rows, last dimension] copy of a value of the row-major (transformer) path."""
+        v = self.tensor(node_id)              # stored as n = h = 1, w = rows, c = columns
+        return np.ascontiguousarray(v[0, :, 0, :].T)
 
     def tensor(self, node_id):
         """numpy NCHW copy of the arena tensor holding graph node `node_id` (u8 levels / f32)."""

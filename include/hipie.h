@@ -276,7 +276,9 @@ int hipie_transpose_bytes_nested(const void* src, int64_t ld_src, int64_t stride
  *    per node; value ids are returned in creation order.  Shapes are the reference's (NCHW,
  *    OIHW, [N, C]); element types are the node's output types (TypeRelaxed ops included).
  *    Supported nodes: Parameter(f32), Constant, FakeQuantize, Convolution, GroupConvolution,
- *    MatMul, Add, Multiply, Subtract, Relu, Clamp, Convert, MaxPool, AvgPool, Reshape, Result.
+ *    MatMul, Add, Multiply, Subtract, Relu, Clamp, Convert, MaxPool, AvgPool, Reshape, Result, and
+ *    for transformer encoders (rank-3 Parameter [batch, sequence, hidden]): MatMul between two
+ *    activations, Softmax, MVN, Gelu, Transpose.
  * ==================================================================================== */
 typedef struct hipie_graph hipie_graph;
 typedef struct hipie_plan hipie_plan;
@@ -309,6 +311,12 @@ int hipie_graph_avg_pool(hipie_graph* g, int x, const int64_t* kernel, const int
                          const int64_t* pads_begin, const int64_t* pads_end, int exclude_pad, int ceil_mode,
                          int out_dtype, int* id);
 int hipie_graph_reshape(hipie_graph* g, int x, const int64_t* dims, int rank, int* id);
+/* op::v1::Softmax, op::v6::MVN (axes as an array), Gelu (ERF), op::v1::Transpose */
+int hipie_graph_softmax(hipie_graph* g, int x, int64_t axis, int* id);
+int hipie_graph_mvn(hipie_graph* g, int x, const int64_t* axes, int n_axes, int normalize_variance, float eps,
+                    int eps_inside_sqrt, int* id);
+int hipie_graph_gelu(hipie_graph* g, int x, int* id);
+int hipie_graph_transpose(hipie_graph* g, int x, const int64_t* order, int rank, int* id);
 int hipie_graph_result(hipie_graph* g, int x, const char* name);
 int hipie_graph_set_name(hipie_graph* g, int id, const char* friendly_name);
 

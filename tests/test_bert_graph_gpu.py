@@ -1,0 +1,76 @@
+"""BERT-style encoder stack (BASELINE config 5 at reduced width) as a post-LPT graph through the
+planner: MatMul against constant weights and between activations, Reshape / Transpose as views,
+Softmax, LayerNorm, Gelu, per-tensor FakeQuantize.
+
+The fp32 glue has tolerance parity only and a FakeQuantize behind it can turn a last-ulp difference
+into another level, so the oracle interpreter continues from the DEVICE's value behind every glue op:
+all integer GEMMs, dequantisations, requantisations, residual adds and data movement must then be
+bit-exact, and each glue op is compared with what the oracle makes of the same inputs."""
+import numpy as np
+import pytest
+
+from interp import evaluate
+
+pytestmark = pytest.mark.gpu
+
+EXACT = ("xq", "q", "k", "v", "scores", "pq", "ctx", "ctxq", "attn", "h1q", "up", "gq", "down")
+GLUE_TOL = dict(p=dict(rtol=2e-6, atol=1e-8), h1=dict(rtol=1e-5, atol=4e-6), gelu=dict(rtol=1e-6, atol=1e-8),
+                y=dict(rtol=1e-5, atol=4e-6))
+
+
+def _check_stack(orc, layers, hidden, heads, ffn, batch, seq):
+    from dldt_amd import builders
+    # ranges for the reduced width: about 30 levels per standard deviation, so the tails saturate
+    g, meta = builders.bert_encoder(layers=layers, hidden=hidden, heads=heads, ffn=ffn, batch=batch, seq=seq, seed=7,
+                                    ranges=dict(q=0.12, k=0.9, v=0.9, ctx=0.6))
+    x = np.random.default_rng(70).normal(0, 1, (batch, seq, hidden)).astype(np.float32)
+    plan = g.compile()
+    types = [s["type"] for s in plan.steps]
+    assert types.count("MatMul") == 8 * layers and types.count("Softmax") == layers
+    assert types.count("MVN") == 2 * layers and types.count("Gelu") == layers and types.count("Transpose") == layers
+    req = plan.create_request()
+    (y,) = req.infer(x)
+    device = {n: req.matrix(n) for n in meta["glue"]}
+    keep = [n for L in meta["layers"] for n in L.values()]
+    want, kept = evaluate(orc, g.nodes, {"hidden_states": x}, keep=keep, override=device)
+    for li, L in enumerate(meta["layers"]):
+        for name in EXACT:
+            w = kept[L[name]]
+            have = req.matrix(L[name]).reshape(w.shape)
+            if w.dtype == np.float32:
+                np.testing.assert_array_equal(have.view(np.uint32), w.view(np.uint32), err_msg="layer %d %s" % (li, name))
+            else:
+                np.testing.assert_array_equal(have.view(np.int8), w.astype(np.int8), err_msg="layer %d %s" % (li, name))
+        for name, tol in GLUE_TOL.items():
+            w = kept[("oracle", L[name])]
+            np.testing.assert_allclose(device[L[name]].reshape(w.shape), w, err_msg="layer %d %s" % (li, name), **tol)
+        q = kept[L["q"]]
+        assert len(np.unique(q)) > 60                      # the ranges are exercised, not saturated
+    np.testing.assert_array_equal(y.view(np.uint32), want["out"].view(np.uint32))
+    return plan, req, x, y
+
+
+def test_encoder_stack_matches_the_oracle(orc):
+    plan, req, x, y = _check_stack(orc, layers=2, hidden=128, heads=2, ffn=256, batch=2, seq=128)
+    # device-resident path gives the same bytes
+    import torch
+    ins, outs = req.device_buffers()
+    ins[0].copy_(torch.from_numpy(x))
+    req.infer_device(ins, outs)
+    np.testing.assert_array_equal(outs[0].cpu().numpy(), y)
+
+
+def test_encoder_stack_other_head_count_and_ragged_rows(orc):
+    """three heads, a sequence length that is not a multiple of the 128-row tiles"""
+    _check_stack(orc, layers=1, hidden=192, heads=3, ffn=320, batch=3, seq=64)
+
+
+def test_unsupported_transformer_nodes_are_reported():
+    from dldt_amd import HipieError
+    from dldt_amd.graph import Graph
+    g = Graph()
+    x = g.parameter("x", (2, 64, 64))
+    g.result(g.softmax(x, 1), "y")                         # not over the last axis
+    with pytest.raises(HipieError) as e:
+        g.compile()
+    assert e.value.status == -2 and "Softmax" in str(e.value)

@@ -108,3 +108,32 @@ def test_full_size_mac_counts_match_the_published_architecture():
     from dldt_amd import builders
     assert builders.resnet50_macs() == 4089184256          # 4.089 GMAC per image
     assert 0.29e9 < builders.mobilenet_v2(batch=1, res=224)[1]["macs_per_image"] < 0.32e9
+
+
+def test_planner_encoder_stack_steps_and_views():
+    """BERT-style encoder: head split / merge are views (no step), the V operand gets one physical
+    transpose, LayerNorm's Multiply and Add ride in the MVN step, and the published operation count of
+    config 5 comes out: 565.3 GMAC for 12 layers at batch 16 x 384 tokens."""
+    from dldt_amd import builders
+    from dldt_amd.graph import Plan
+    g, meta = builders.bert_encoder(layers=2, hidden=128, heads=2, ffn=256, batch=2, seq=128, seed=7)
+    plan = Plan(g, device=-1)
+    types = [s["type"] for s in plan.steps]
+    per_layer = ["FakeQuantize", "MatMul", "MatMul", "MatMul", "Softmax", "FakeQuantize", "MatMul", "Transpose", "MatMul",
+                 "FakeQuantize", "MatMul", "MVN", "FakeQuantize", "MatMul", "Gelu", "FakeQuantize", "MatMul", "MVN"]
+    assert types == per_layer * 2 + ["Result"]
+    assert sum(s["macs"] for s in plan.steps) == meta["macs"]
+    T, H, FF = 16 * 384, 768, 3072
+    assert 12 * (T * (4 * H * H + 2 * H * FF) + 2 * 16 * 12 * 384 * 384 * 64) == 565_325_070_336
+
+
+def test_planner_refuses_a_reshape_that_moves_bytes():
+    from dldt_amd import HipieError
+    from dldt_amd.graph import Graph
+    g = Graph()
+    x = g.parameter("x", (2, 64, 128))
+    t = g.transpose(x, (0, 2, 1))
+    g.result(g.reshape(t, (2, 128 * 64)), "y")
+    with pytest.raises(HipieError) as e:
+        g.compile(device=-1)
+    assert e.value.status == -2 and "Reshape" in str(e.value)
