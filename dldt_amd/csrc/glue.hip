@@ -3,7 +3,9 @@
 //   softmax.hpp (subtract the row maximum, exp, sum, divide),
 //   mvn.hpp mvn_6 (mean, centre, mean of squares, sqrt(var + eps) | sqrt(var) + eps, divide),
 //   gelu.hpp ERF mode (0.5 * x * (1 + erf(x / sqrt(2))) evaluated in double).
-// One wavefront owns one row: coalesced 256-byte row segments, reductions by cross-lane shuffles.
+// One wavefront owns one row and holds it in registers: the row is read once and written once,
+// reductions by cross-lane shuffles.  The per-tensor FakeQuantize that follows each of them in a
+// post-LPT encoder can be fused in (i8 levels written beside or instead of the f32 result).
 #include "common.h"
 
 namespace hipie {
@@ -22,6 +24,111 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// Per-tensor FakeQuantize of a glue result, fused into the kernel that produces it: the level index
+// in the reference's own operation order (fake_quantize.hpp:175-194, IEEE division), stored as
+// out_low + k.  levels == 0: no quantized output.
+struct Requant {
+    float il, ih, d, lm1, ol;
+    int levels;
+};
+
+__device__ __forceinline__ int requant_level(const Requant& f, float x) {
+    const float xc = fminf(fmaxf(x, f.il), f.ih);   // x <= il -> level 0, x > ih -> level L - 1
+    return static_cast<int>(rintf((xc - f.il) / f.d * f.lm1) + f.ol);
+}
+
+__device__ __forceinline__ uint32_t requant4(const Requant& f, const float4& v) {
+    return (static_cast<uint32_t>(requant_level(f, v.x)) & 0xffu) | ((static_cast<uint32_t>(requant_level(f, v.y)) & 0xffu) << 8) |
+           ((static_cast<uint32_t>(requant_level(f, v.z)) & 0xffu) << 16) | (static_cast<uint32_t>(requant_level(f, v.w)) << 24);
+}
+
+// Row kernels: one wavefront owns one row and keeps it in registers (NCH float4 per lane, lane l holds
+// elements 4 l .. 4 l + 3 of every 256-element chunk), so a row is read once in 1 KB wave loads and
+// written once; y and/or q may be null.
+template <int NCH>
+__global__ __launch_bounds__(kThreads) void softmax_rows_reg(const float* __restrict__ x, float* __restrict__ y,
+                                                             int8_t* __restrict__ q, int64_t rows, int axis, Requant fq) {
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * (kThreads / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const float* p = x + row * axis;
+    float4 v[NCH];
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        const int i = 256 * j + 4 * lane;
+        v[j] = i < axis ? *reinterpret_cast<const float4*>(p + i) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        m = fmaxf(fmaxf(m, fmaxf(v[j].x, v[j].y)), fmaxf(v[j].z, v[j].w));
+    }
+    m = wave_max(m);
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        v[j].x = expf(v[j].x - m); v[j].y = expf(v[j].y - m); v[j].z = expf(v[j].z - m); v[j].w = expf(v[j].w - m);
+        s += (v[j].x + v[j].y) + (v[j].z + v[j].w);    // exp(-inf) = 0 in the padding
+    }
+    s = wave_sum(s);
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        const int i = 256 * j + 4 * lane;
+        if (i >= axis) continue;
+        const float4 o = make_float4(v[j].x / s, v[j].y / s, v[j].z / s, v[j].w / s);
+        if (y) *reinterpret_cast<float4*>(y + row * axis + i) = o;
+        if (q) *reinterpret_cast<uint32_t*>(q + row * axis + i) = requant4(fq, o);
+    }
+}
+
+template <int NCH>
+__global__ __launch_bounds__(kThreads) void mvn_rows_reg(const float* __restrict__ x, float* __restrict__ y,
+                                                         int8_t* __restrict__ q, int64_t rows, int axis,
+                                                         int normalize_variance, float eps, int eps_inside,
+                                                         const float* __restrict__ gamma, const float* __restrict__ beta,
+                                                         Requant fq) {
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * (kThreads / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const float* p = x + row * axis;
+    float4 v[NCH];
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        const int i = 256 * j + 4 * lane;
+        v[j] = i < axis ? *reinterpret_cast<const float4*>(p + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+        s += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+    }
+    const float mean = wave_sum(s) / static_cast<float>(axis);
+    float sq = 0.f;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        const int i = 256 * j + 4 * lane;
+        v[j].x -= mean; v[j].y -= mean; v[j].z -= mean; v[j].w -= mean;
+        if (i < axis) sq += (v[j].x * v[j].x + v[j].y * v[j].y) + (v[j].z * v[j].z + v[j].w * v[j].w);
+    }
+    float denom = 1.f;
+    if (normalize_variance) {
+        const float var = wave_sum(sq) / static_cast<float>(axis);
+        denom = eps_inside ? sqrtf(var + eps) : sqrtf(var) + eps;
+    }
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        const int i = 256 * j + 4 * lane;
+        if (i >= axis) continue;
+        float4 o = v[j];
+        if (normalize_variance) { o.x = o.x / denom; o.y = o.y / denom; o.z = o.z / denom; o.w = o.w / denom; }
+        if (gamma) {
+            const float4 gm = *reinterpret_cast<const float4*>(gamma + i);
+            o.x = o.x * gm.x; o.y = o.y * gm.y; o.z = o.z * gm.z; o.w = o.w * gm.w;
+        }
+        if (beta) {
+            const float4 bt = *reinterpret_cast<const float4*>(beta + i);
+            o.x = o.x + bt.x; o.y = o.y + bt.y; o.z = o.z + bt.z; o.w = o.w + bt.w;
+        }
+        if (y) *reinterpret_cast<float4*>(y + row * axis + i) = o;
+        if (q) *reinterpret_cast<uint32_t*>(q + row * axis + i) = requant4(fq, o);
+    }
+}
+
+// rows of any length (not a multiple of 4, or longer than 4096): three passes over the row
 __global__ __launch_bounds__(kThreads) void softmax_rows(const float* __restrict__ x, float* __restrict__ y,
                                                          int64_t rows, int axis) {
     const int64_t row = static_cast<int64_t>(blockIdx.x) * (kThreads / 64) + (threadIdx.x >> 6);
@@ -73,12 +180,145 @@ __global__ __launch_bounds__(kThreads) void mvn_rows(const float* __restrict__ x
     }
 }
 
-__global__ __launch_bounds__(kThreads) void gelu_erf(const float* __restrict__ x, float* __restrict__ y, int64_t n) {
+__device__ __forceinline__ float gelu_one(float x) {
+    const double v = static_cast<double>(x);
+    return static_cast<float>(0.5 * v * (1.0 + erf(v / 1.4142135623730951)));
+}
+
+// four elements per lane and step (n4 = n / 4 full groups), then the tail one by one
+__global__ __launch_bounds__(kThreads) void gelu_erf(const float* __restrict__ x, float* __restrict__ y,
+                                                     int8_t* __restrict__ q, int64_t n, Requant fq) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) {
-        const double v = static_cast<double>(x[i]);
-        y[i] = static_cast<float>(0.5 * v * (1.0 + erf(v / 1.4142135623730951)));
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const int64_t n4 = n >> 2;
+    for (int64_t i = t; i < n4; i += stride) {
+        const float4 v = reinterpret_cast<const float4*>(x)[i];
+        const float4 o = make_float4(gelu_one(v.x), gelu_one(v.y), gelu_one(v.z), gelu_one(v.w));
+        if (y) reinterpret_cast<float4*>(y)[i] = o;
+        if (q) reinterpret_cast<uint32_t*>(q)[i] = requant4(fq, o);
     }
+    for (int64_t i = 4 * n4 + t; i < n; i += stride) {
+        const float o = gelu_one(x[i]);
+        if (y) y[i] = o;
+        if (q) q[i] = static_cast<int8_t>(requant_level(fq, o));
+    }
+}
+
+// plain per-tensor requantisation of a dense f32 array (behind the long-row fallbacks)
+__global__ __launch_bounds__(kThreads) void requant_flat(const float* __restrict__ x, int8_t* __restrict__ q, int64_t n,
+                                                         Requant fq) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride)
+        q[i] = static_cast<int8_t>(requant_level(fq, x[i]));
+}
+
+Requant make_requant(const hipie_requant* r, const char* what) {
+    Requant f{};
+    if (!r) return f;
+    HIPIE_REQUIRE(r->levels >= 2 && r->levels <= 256 && r->in_low < r->in_high, HIPIE_PARAMETER_MISMATCH,
+                  "%s: requantisation needs 2..256 levels and in_low < in_high", what);
+    f.il = r->in_low;
+    f.ih = r->in_high;
+    f.d = r->in_high - r->in_low;
+    f.lm1 = static_cast<float>(r->levels - 1);
+    f.ol = r->out_low;
+    f.levels = static_cast<int>(r->levels);
+    const float oh = r->out_low + f.lm1;
+    HIPIE_REQUIRE(f.ol == std::nearbyintf(f.ol) && f.ol >= -128.f && oh <= 127.f, HIPIE_NOT_IMPLEMENTED,
+                  "%s: output levels must be the i8 integers out_low .. out_low + levels - 1", what);
+    for (int k = 0; k < f.levels; ++k)   // the reference's own output expression yields these integers
+        HIPIE_REQUIRE(static_cast<float>(k) / f.lm1 * (oh - f.ol) + f.ol == f.ol + static_cast<float>(k),
+                      HIPIE_NOT_IMPLEMENTED, "%s: output level %d is not an integer", what, k);
+    return f;
+}
+
+template <template <int> class Launch, typename... A>
+bool dispatch_chunks(int axis, A&&... a) {
+    if (axis % 4 != 0 || axis > 4096) return false;
+    const int nch = static_cast<int>(ceil_div(axis, 256));
+    switch (nch) {
+    case 1: Launch<1>::go(a...); break;
+    case 2: Launch<2>::go(a...); break;
+    case 3: Launch<3>::go(a...); break;
+    case 4: Launch<4>::go(a...); break;
+    case 5: case 6: Launch<6>::go(a...); break;
+    case 7: case 8: Launch<8>::go(a...); break;
+    case 9: case 10: case 11: case 12: Launch<12>::go(a...); break;
+    default: Launch<16>::go(a...); break;
+    }
+    return true;
+}
+
+template <int NCH>
+struct LaunchSoftmax {
+    static void go(const float* x, float* y, int8_t* q, int64_t rows, int axis, const Requant& fq, hipStream_t s) {
+        hipLaunchKernelGGL(softmax_rows_reg<NCH>, dim3(static_cast<uint32_t>(ceil_div(rows, kThreads / 64))), dim3(kThreads), 0,
+                           s, x, y, q, rows, axis, fq);
+    }
+};
+template <int NCH>
+struct LaunchMvn {
+    static void go(const float* x, float* y, int8_t* q, int64_t rows, int axis, int nv, float eps, int inside,
+                   const float* gamma, const float* beta, const Requant& fq, hipStream_t s) {
+        hipLaunchKernelGGL(mvn_rows_reg<NCH>, dim3(static_cast<uint32_t>(ceil_div(rows, kThreads / 64))), dim3(kThreads), 0, s,
+                           x, y, q, rows, axis, nv, eps, inside, gamma, beta, fq);
+    }
+};
+
+void launch_requant_flat(const float* x, int8_t* q, int64_t n, const Requant& fq, hipStream_t s) {
+    const int64_t blocks = std::min<int64_t>(ceil_div(n, kThreads), 256 * 16);
+    hipLaunchKernelGGL(requant_flat, dim3(static_cast<uint32_t>(blocks)), dim3(kThreads), 0, s, x, q, n, fq);
+}
+
+void run_softmax(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis, const hipie_requant* r, void* stream,
+                 const char* what) {
+    if (rows == 0 || axis == 0) return;
+    HIPIE_REQUIRE(x && (y || q) && rows > 0 && axis > 0 && axis < (1ll << 31), HIPIE_PARAMETER_MISMATCH, "%s: bad argument", what);
+    HIPIE_REQUIRE(!q || r, HIPIE_PARAMETER_MISMATCH, "%s: quantized output without a requantisation", what);
+    const Requant fq = q ? make_requant(r, what) : Requant{};
+    hipStream_t s = as_stream(stream);
+    const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(q) % 4 == 0;
+    if (!(aligned && dispatch_chunks<LaunchSoftmax>(static_cast<int>(axis), x, y, q, rows, static_cast<int>(axis), fq, s))) {
+        HIPIE_REQUIRE(y, HIPIE_NOT_IMPLEMENTED, "%s: rows of %lld elements need the f32 output as well", what, (long long)axis);
+        hipLaunchKernelGGL(softmax_rows, dim3(static_cast<uint32_t>(ceil_div(rows, kThreads / 64))), dim3(kThreads), 0, s, x, y,
+                           rows, static_cast<int>(axis));
+        if (q) launch_requant_flat(y, q, rows * axis, fq, s);
+    }
+    HIPIE_CHECK_HIP(hipGetLastError());
+}
+
+void run_mvn(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis, int normalize_variance, float eps,
+             int eps_inside_sqrt, const float* gamma, const float* beta, const hipie_requant* r, void* stream,
+             const char* what) {
+    if (rows == 0 || axis == 0) return;
+    HIPIE_REQUIRE(x && (y || q) && rows > 0 && axis > 0 && axis < (1ll << 31), HIPIE_PARAMETER_MISMATCH, "%s: bad argument", what);
+    HIPIE_REQUIRE(!q || r, HIPIE_PARAMETER_MISMATCH, "%s: quantized output without a requantisation", what);
+    const Requant fq = q ? make_requant(r, what) : Requant{};
+    hipStream_t s = as_stream(stream);
+    const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(q) % 4 == 0 && reinterpret_cast<uintptr_t>(gamma) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(beta) % 16 == 0;
+    if (!(aligned && dispatch_chunks<LaunchMvn>(static_cast<int>(axis), x, y, q, rows, static_cast<int>(axis),
+                                                normalize_variance, eps, eps_inside_sqrt, gamma, beta, fq, s))) {
+        HIPIE_REQUIRE(y, HIPIE_NOT_IMPLEMENTED, "%s: rows of %lld elements need the f32 output as well", what, (long long)axis);
+        hipLaunchKernelGGL(mvn_rows, dim3(static_cast<uint32_t>(ceil_div(rows, kThreads / 64))), dim3(kThreads), 0, s, x, y, rows,
+                           static_cast<int>(axis), normalize_variance, eps, eps_inside_sqrt, gamma, beta);
+        if (q) launch_requant_flat(y, q, rows * axis, fq, s);
+    }
+    HIPIE_CHECK_HIP(hipGetLastError());
+}
+
+void run_gelu(const float* x, float* y, int8_t* q, int64_t n, const hipie_requant* r, void* stream, const char* what) {
+    if (n == 0) return;
+    HIPIE_REQUIRE(x && (y || q) && n > 0, HIPIE_PARAMETER_MISMATCH, "%s: bad argument", what);
+    HIPIE_REQUIRE(!q || r, HIPIE_PARAMETER_MISMATCH, "%s: quantized output without a requantisation", what);
+    HIPIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(q) % 4 == 0, HIPIE_PARAMETER_MISMATCH, "%s: buffers must be 16-byte aligned", what);
+    const Requant fq = q ? make_requant(r, what) : Requant{};
+    const int64_t blocks = std::min<int64_t>(ceil_div(ceil_div(n, 4), kThreads), 256 * 32);
+    hipLaunchKernelGGL(gelu_erf, dim3(static_cast<uint32_t>(blocks)), dim3(kThreads), 0, as_stream(stream), x, y, q, n, fq);
+    HIPIE_CHECK_HIP(hipGetLastError());
 }
 
 // Batched 2-D transpose of bytes through a 64 x 64 LDS tile (row stride 65 words would not help
@@ -116,37 +356,34 @@ using namespace hipie;
 extern "C" {
 
 int hipie_softmax_f32(const float* x, float* y, int64_t rows, int64_t axis, void* stream) {
-    return guarded([&] {
-        if (rows == 0 || axis == 0) return;
-        HIPIE_REQUIRE(x && y && rows > 0 && axis > 0 && axis < (1ll << 31), HIPIE_PARAMETER_MISMATCH,
-                      "hipie_softmax_f32: bad argument");
-        hipLaunchKernelGGL(softmax_rows, dim3(static_cast<uint32_t>(ceil_div(rows, kThreads / 64))), dim3(kThreads), 0,
-                           as_stream(stream), x, y, rows, static_cast<int>(axis));
-        HIPIE_CHECK_HIP(hipGetLastError());
-    });
+    return guarded([&] { run_softmax(x, y, nullptr, rows, axis, nullptr, stream, "hipie_softmax_f32"); });
 }
 
 int hipie_mvn_f32(const float* x, float* y, int64_t rows, int64_t axis, int normalize_variance, float eps,
                   int eps_inside_sqrt, const float* gamma, const float* beta, void* stream) {
     return guarded([&] {
-        if (rows == 0 || axis == 0) return;
-        HIPIE_REQUIRE(x && y && rows > 0 && axis > 0 && axis < (1ll << 31), HIPIE_PARAMETER_MISMATCH,
-                      "hipie_mvn_f32: bad argument");
-        hipLaunchKernelGGL(mvn_rows, dim3(static_cast<uint32_t>(ceil_div(rows, kThreads / 64))), dim3(kThreads), 0,
-                           as_stream(stream), x, y, rows, static_cast<int>(axis), normalize_variance, eps,
-                           eps_inside_sqrt, gamma, beta);
-        HIPIE_CHECK_HIP(hipGetLastError());
+        run_mvn(x, y, nullptr, rows, axis, normalize_variance, eps, eps_inside_sqrt, gamma, beta, nullptr, stream, "hipie_mvn_f32");
     });
 }
 
 int hipie_gelu_f32(const float* x, float* y, int64_t n, void* stream) {
+    return guarded([&] { run_gelu(x, y, nullptr, n, nullptr, stream, "hipie_gelu_f32"); });
+}
+
+int hipie_softmax_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis, const hipie_requant* requant,
+                     void* stream) {
+    return guarded([&] { run_softmax(x, y, q, rows, axis, requant, stream, "hipie_softmax_q8"); });
+}
+
+int hipie_mvn_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis, int normalize_variance, float eps,
+                 int eps_inside_sqrt, const float* gamma, const float* beta, const hipie_requant* requant, void* stream) {
     return guarded([&] {
-        if (n == 0) return;
-        HIPIE_REQUIRE(x && y && n > 0, HIPIE_PARAMETER_MISMATCH, "hipie_gelu_f32: bad argument");
-        const int64_t blocks = std::min<int64_t>(ceil_div(n, kThreads), 256 * 16);
-        hipLaunchKernelGGL(gelu_erf, dim3(static_cast<uint32_t>(blocks)), dim3(kThreads), 0, as_stream(stream), x, y, n);
-        HIPIE_CHECK_HIP(hipGetLastError());
+        run_mvn(x, y, q, rows, axis, normalize_variance, eps, eps_inside_sqrt, gamma, beta, requant, stream, "hipie_mvn_q8");
     });
+}
+
+int hipie_gelu_q8(const float* x, float* y, int8_t* q, int64_t n, const hipie_requant* requant, void* stream) {
+    return guarded([&] { run_gelu(x, y, q, n, requant, stream, "hipie_gelu_q8"); });
 }
 
 int hipie_transpose_bytes(const void* src, int64_t ld_src, int64_t batch_stride_src, void* dst, int64_t ld_dst,

@@ -442,7 +442,9 @@ struct MatFqStep : Step {
 struct GlueStep : Step {
     int kind = OP_SOFTMAX;
     View in;
-    int out = -1;
+    int out = -1;                  // f32 result (-1: only the quantized one is kept)
+    int outq = -1;                 // i8 levels of the FakeQuantize fused behind it (-1: none)
+    hipie_requant rq{};
     int64_t rows = 0, axis = 0;
     bool normalize_variance = true, eps_inside_sqrt = true;
     float eps = 0;
@@ -456,12 +458,16 @@ struct GlueStep : Step {
     void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
              hipStream_t s) const override {
         const float* x = reinterpret_cast<const float*>(in.ptr(arena, tensors, inputs));
-        float* y = reinterpret_cast<float*>(arena + tensors[out].offset);
+        float* y = out >= 0 ? reinterpret_cast<float*>(arena + tensors[out].offset) : nullptr;
+        int8_t* q = outq >= 0 ? reinterpret_cast<int8_t*>(arena + tensors[outq].offset) : nullptr;
+        const hipie_requant* r = outq >= 0 ? &rq : nullptr;
+        const float* gm = gamma.empty() ? nullptr : d_gamma.as<float>();
+        const float* bt = beta.empty() ? nullptr : d_beta.as<float>();
         int st = HIPIE_OK;
-        if (kind == OP_SOFTMAX) st = hipie_softmax_f32(x, y, rows, axis, s);
-        else if (kind == OP_GELU) st = hipie_gelu_f32(x, y, rows * axis, s);
-        else st = hipie_mvn_f32(x, y, rows, axis, normalize_variance, eps, eps_inside_sqrt,
-                                gamma.empty() ? nullptr : d_gamma.as<float>(), beta.empty() ? nullptr : d_beta.as<float>(), s);
+        if (kind == OP_SOFTMAX) st = q ? hipie_softmax_q8(x, y, q, rows, axis, r, s) : hipie_softmax_f32(x, y, rows, axis, s);
+        else if (kind == OP_GELU) st = q ? hipie_gelu_q8(x, y, q, rows * axis, r, s) : hipie_gelu_f32(x, y, rows * axis, s);
+        else st = q ? hipie_mvn_q8(x, y, q, rows, axis, normalize_variance, eps, eps_inside_sqrt, gm, bt, r, s)
+                    : hipie_mvn_f32(x, y, rows, axis, normalize_variance, eps, eps_inside_sqrt, gm, bt, s);
         check_status(st, name.c_str());
     }
 };
@@ -528,8 +534,14 @@ struct Planner {
     std::vector<TensorInfo> tensors;
     std::vector<std::unique_ptr<Step>> steps;
     std::vector<char> visiting;
+    // HIPIE_KEEP_F32=1: store the f32 result of Softmax / MVN / Gelu even when only a fused
+    // FakeQuantize reads it (inspection of the values behind the tolerance-only operations)
+    bool keep_f32 = false;
 
-    explicit Planner(const hipie_graph& graph) : g(graph), values(graph.nodes.size()), visiting(graph.nodes.size(), 0) {}
+    explicit Planner(const hipie_graph& graph) : g(graph), values(graph.nodes.size()), visiting(graph.nodes.size(), 0) {
+        const char* k = std::getenv("HIPIE_KEEP_F32");
+        keep_f32 = k && k[0] == '1';
+    }
 
     const GNode& N(int id) const { return g.nodes[id]; }
 
@@ -702,6 +714,28 @@ struct Planner {
         steps.push_back(std::move(st));
     }
 
+    // FakeQuantize node `u` on value `x` with per-tensor bounds whose outputs are the i8 integers
+    // out_low + k: can be evaluated inside the kernel that produces x
+    bool fusable_requant(int u, int x, hipie_requant& rq) const {
+        const GNode& f = N(u);
+        if (f.op != OP_FAKE_QUANTIZE || f.in[0] != x || f.dtype != HIPIE_I8 || f.levels < 2 || f.levels > 256) return false;
+        float b[4];
+        for (int i = 0; i < 4; ++i) {
+            std::vector<float> c;
+            if (!last_axis_constant(f.in[1 + i], -1, c)) return false;
+            b[i] = c[0];
+        }
+        const float lm1 = static_cast<float>(f.levels - 1);
+        if (!(b[0] < b[1]) || b[2] != std::nearbyintf(b[2]) || b[2] < -128.f || b[3] != b[2] + lm1 || b[3] > 127.f) return false;
+        for (int k = 0; k < f.levels; ++k)
+            if (static_cast<float>(k) / lm1 * (b[3] - b[2]) + b[2] != b[2] + static_cast<float>(k)) return false;
+        rq.in_low = b[0];
+        rq.in_high = b[1];
+        rq.out_low = b[2];
+        rq.levels = f.levels;
+        return true;
+    }
+
     void plan_glue(int id) {
         const GNode& n = N(id);
         const View x = dense_f32_input(id, "Softmax / MVN / Gelu are planned on dense f32 values of the row-major path");
@@ -733,12 +767,27 @@ struct Planner {
         st->in = x;
         st->axis = C;
         st->rows = n.numel() / C;
-        st->out = new_matrix(cur, HIPIE_F32, n.shape);
-        st->name = N(cur).name;
-        st->type = op_name(n.op);
-        st->bytes = n.numel() * 8;
-        st->out_node = cur;
-        set_matrix_value(cur, st->out, HIPIE_F32);
+        // A per-tensor FakeQuantize to i8 among the users rides in the same kernel; the f32 result is
+        // then only stored when something else reads it too (rows the kernel cannot keep in registers
+        // need it as well).
+        int fq_node = -1;
+        for (int u : N(cur).users)
+            if (fq_node < 0 && fusable_requant(u, cur, st->rq)) fq_node = u;
+        const bool keep = fq_node < 0 || N(cur).users.size() > 1 || keep_f32 || C % 4 != 0 || C > 4096;
+        if (keep) {
+            st->out = new_matrix(cur, HIPIE_F32, n.shape);
+            set_matrix_value(cur, st->out, HIPIE_F32);
+        } else {
+            values[cur].kind = VK_FUSED;
+        }
+        if (fq_node >= 0) {
+            st->outq = new_matrix(fq_node, HIPIE_I8, n.shape);
+            set_matrix_value(fq_node, st->outq, HIPIE_I8);
+        }
+        st->name = N(fq_node >= 0 ? fq_node : cur).name;
+        st->type = std::string(op_name(n.op)) + (fq_node >= 0 ? "+FakeQuantize" : "");
+        st->bytes = n.numel() * (4 + (keep ? 4 : 0) + (fq_node >= 0 ? 1 : 0));
+        st->out_node = fq_node >= 0 ? fq_node : cur;
         steps.push_back(std::move(st));
     }
 
@@ -974,6 +1023,7 @@ struct Planner {
         int cur = id;
         std::vector<int64_t> oshape = n.shape;
         std::vector<int64_t> ostride = View::dense_strides(oshape);   // of the MatMul's own dimensions
+        hipie_requant rq{};
         while (single_user(cur)) {
             const int nx = N(cur).users[0];
             const GNode& u = N(nx);
@@ -985,6 +1035,19 @@ struct Planner {
                 oshape = u.shape;
                 const auto ts = View::dense_strides(oshape);
                 for (size_t p = 0; p < r; ++p) ostride[u.axes[p]] = ts[p];
+            } else if (u.op == OP_RESHAPE && !keep_f32 && single_user(nx) && u.shape.back() % oshape.back() == 0 &&
+                       fusable_requant(N(nx).users[0], nx, rq)) {
+                // head merge in front of the FakeQuantize: the output tensor is dense, so the Reshape
+                // only renames its dimensions (the last one must stay a multiple of this MatMul's columns)
+                oshape = u.shape;
+            } else if (!keep_f32 && fusable_requant(nx, cur, rq)) {
+                e.levels = rq.levels;
+                e.fq_il.assign(1, rq.in_low);
+                e.fq_ih.assign(1, rq.in_high);
+                e.fq_ol = rq.out_low;
+                e.fq_oh = rq.out_low + static_cast<float>(rq.levels - 1);
+                e.out_dtype = HIPIE_I8;
+                oshape = u.shape;
                 cur = nx;
                 break;
             } else {
@@ -993,16 +1056,16 @@ struct Planner {
             cur = nx;
         }
         mark_chain(id, cur);
-        st->out = new_matrix(cur, HIPIE_F32, oshape);
+        st->out = new_matrix(cur, e.out_dtype, oshape);
         st->ldo = ostride[r - 2];
         st->so = ostride[r - 3];
         st->oo = r == 4 ? ostride[0] : 0;
         st->name = N(cur).name;
         st->type = "MatMul";
         st->macs = n.numel() * K;
-        st->bytes = av.numel() + bv.numel() + n.numel() * 4;
+        st->bytes = av.numel() + bv.numel() + n.numel() * (e.out_dtype == HIPIE_F32 ? 4 : 1);
         st->out_node = cur;
-        set_matrix_value(cur, st->out, HIPIE_F32);
+        set_matrix_value(cur, st->out, e.out_dtype);
         steps.push_back(std::move(st));
     }
 

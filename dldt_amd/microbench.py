@@ -6,7 +6,8 @@
 Rows: config 1 (one quantized 3x3 convolution block, batch 1), config 2 (per-channel FakeQuantize of
 [32,256,56,56]), config 3 (ResNet-50 v1.5 INT8, batch 1 and 64), config 4 (MobileNetV2 INT8, batch 64:
 whole graph, its depthwise and pointwise kernels), config 5 (one BERT-base encoder layer at batch 16,
-sequence 384: the int8 GEMMs and the fp32 softmax / LayerNorm / GELU kernels, each on its own).
+sequence 384: the int8 GEMMs and the fp32 softmax / LayerNorm / GELU kernels, each on its own; then the
+12-layer encoder as one graph through the planner).
 Inputs are resident in HBM, times are HIP-event averages over back-to-back launches.
 """
 import sys
@@ -232,6 +233,20 @@ def config5():
     us = _time(lambda: layer.run(x), reps=5, warm=2)
     r = _row("cfg5 one encoder layer end to end (dldt_amd.bert, %d launches)" % (15 + 3 * B), us, macs=layer.macs(), bound="mfma")
     r["sequences/s (12 layers)"] = B / (12 * us) * 1e6
+    rows.append(r)
+    del layer
+    # the 12-layer encoder as a post-LPT graph through the planner (graph-level C ABI)
+    from . import builders
+    g, meta = builders.bert_encoder(layers=12, hidden=H, heads=NH, ffn=FF, batch=B, seq=S)
+    us, plan = _graph_time(g, reps=5, warm=2)
+    r = _row("cfg5 BERT-base encoder, 12 layers, batch %d x %d tokens, one request (%d launches)" % (B, S, len(plan.steps)),
+             us, macs=meta["macs"], bytes_=sum(s["bytes"] for s in plan.steps), bound="mfma")
+    r["sequences/s"] = B / us * 1e6
+    rows.append(r)
+    us3 = _throughput_time(plan, reps=12, warm=3)
+    r = _row("cfg5 BERT-base encoder, 12 layers, three requests in flight", us3, macs=meta["macs"],
+             bytes_=sum(s["bytes"] for s in plan.steps), bound="mfma")
+    r["sequences/s"] = B / us3 * 1e6
     rows.append(r)
     return rows
 

@@ -254,29 +254,57 @@ def transpose_bytes(src, ld_src, bs_src, dst, ld_dst, bs_dst, rows, cols, batch,
                                              ctypes.c_int32(batch_outer), _stream()))
 
 
-def softmax(x):
+class hipie_requant(ctypes.Structure):
+    _fields_ = [("in_low", ctypes.c_float), ("in_high", ctypes.c_float), ("out_low", ctypes.c_float),
+                ("levels", ctypes.c_int64)]
+
+
+def _glue_outputs(x, requant, keep_f32):
+    """(y, q, requant struct pointer): f32 result and / or i8 levels of the fused per-tensor FakeQuantize
+    requant = (in_low, in_high, out_low, levels)."""
     import torch
     assert x.is_contiguous() and x.dtype == torch.float32
-    y = torch.empty_like(x)
-    check(lib().hipie_softmax_f32(_dptr(x), _dptr(y), ctypes.c_int64(x.numel() // x.shape[-1]),
-                                  ctypes.c_int64(x.shape[-1]), _stream()))
-    return y
+    y = torch.empty_like(x) if (requant is None or keep_f32) else None
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device) if requant is not None else None
+    r = hipie_requant(*[float(v) for v in requant[:3]], int(requant[3])) if requant is not None else None
+    return y, q, r
 
 
-def mvn(x, normalize_variance=True, eps=1e-5, eps_inside=True, gamma=None, beta=None):
-    import torch
-    assert x.is_contiguous() and x.dtype == torch.float32
-    y = torch.empty_like(x)
-    check(lib().hipie_mvn_f32(_dptr(x), _dptr(y), ctypes.c_int64(x.numel() // x.shape[-1]),
-                              ctypes.c_int64(x.shape[-1]), int(normalize_variance), ctypes.c_float(eps),
-                              int(eps_inside), _dptr(gamma) if gamma is not None else None,
-                              _dptr(beta) if beta is not None else None, _stream()))
-    return y
+def _ret(y, q):
+    return y if q is None else (q if y is None else (y, q))
 
 
-def gelu(x):
-    import torch
-    assert x.is_contiguous() and x.dtype == torch.float32
-    y = torch.empty_like(x)
-    check(lib().hipie_gelu_f32(_dptr(x), _dptr(y), ctypes.c_int64(x.numel()), _stream()))
-    return y
+def softmax(x, requant=None, keep_f32=True):
+    """Softmax over the last axis; with requant also (or only, keep_f32=False) the i8 levels of the
+    FakeQuantize behind it."""
+    y, q, r = _glue_outputs(x, requant, keep_f32)
+    rows, axis = ctypes.c_int64(x.numel() // x.shape[-1]), ctypes.c_int64(x.shape[-1])
+    if q is None:
+        check(lib().hipie_softmax_f32(_dptr(x), _dptr(y), rows, axis, _stream()))
+    else:
+        check(lib().hipie_softmax_q8(_dptr(x), _dptr(y) if y is not None else None, _dptr(q), rows, axis,
+                                     ctypes.byref(r), _stream()))
+    return _ret(y, q)
+
+
+def mvn(x, normalize_variance=True, eps=1e-5, eps_inside=True, gamma=None, beta=None, requant=None, keep_f32=True):
+    y, q, r = _glue_outputs(x, requant, keep_f32)
+    args = [ctypes.c_int64(x.numel() // x.shape[-1]), ctypes.c_int64(x.shape[-1]), int(normalize_variance),
+            ctypes.c_float(eps), int(eps_inside), _dptr(gamma) if gamma is not None else None,
+            _dptr(beta) if beta is not None else None]
+    if q is None:
+        check(lib().hipie_mvn_f32(_dptr(x), _dptr(y), *args, _stream()))
+    else:
+        check(lib().hipie_mvn_q8(_dptr(x), _dptr(y) if y is not None else None, _dptr(q), *args, ctypes.byref(r),
+                                 _stream()))
+    return _ret(y, q)
+
+
+def gelu(x, requant=None, keep_f32=True):
+    y, q, r = _glue_outputs(x, requant, keep_f32)
+    if q is None:
+        check(lib().hipie_gelu_f32(_dptr(x), _dptr(y), ctypes.c_int64(x.numel()), _stream()))
+    else:
+        check(lib().hipie_gelu_q8(_dptr(x), _dptr(y) if y is not None else None, _dptr(q), ctypes.c_int64(x.numel()),
+                                  ctypes.byref(r), _stream()))
+    return _ret(y, q)

@@ -259,6 +259,20 @@ int hipie_softmax_f32(const float* x, float* y, int64_t rows, int64_t axis, void
 int hipie_mvn_f32(const float* x, float* y, int64_t rows, int64_t axis, int normalize_variance, float eps,
                   int eps_inside_sqrt, const float* gamma, const float* beta, void* stream);
 int hipie_gelu_f32(const float* x, float* y, int64_t n, void* stream);
+/* The same three with the per-tensor FakeQuantize that consumes their result in a post-LPT encoder
+ * fused in: q receives the i8 levels of FakeQuantize(result, in_low, in_high, out_low,
+ * out_low + levels - 1, levels), bit-exact with hipie_fq_run_q8 applied to the f32 result (the
+ * level index is evaluated in the reference's operation order, fake_quantize.hpp:175-194); y still
+ * receives the f32 result unless it is NULL. */
+typedef struct hipie_requant {
+    float in_low, in_high, out_low;
+    int64_t levels;
+} hipie_requant;
+int hipie_softmax_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis, const hipie_requant* requant,
+                     void* stream);
+int hipie_mvn_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis, int normalize_variance, float eps,
+                 int eps_inside_sqrt, const float* gamma, const float* beta, const hipie_requant* requant, void* stream);
+int hipie_gelu_q8(const float* x, float* y, int8_t* q, int64_t n, const hipie_requant* requant, void* stream);
 /* Transpose of the two inner dimensions of a byte tensor (opset1 Transpose on quantized activations,
  * e.g. V [S, d] -> [d, S] so that the context MatMul finds its reduction axis contiguous;
  * reference::transpose, .../reference/transpose.hpp:20-25): dst[b][c][r] = src[b][r][c], leading

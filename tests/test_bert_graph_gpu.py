@@ -18,16 +18,18 @@ GLUE_TOL = dict(p=dict(rtol=2e-6, atol=1e-8), h1=dict(rtol=1e-5, atol=4e-6), gel
                 y=dict(rtol=1e-5, atol=4e-6))
 
 
-def _check_stack(orc, layers, hidden, heads, ffn, batch, seq):
+def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq):
     from dldt_amd import builders
+    # first with every f32 value behind a tolerance-only op kept in the arena (segment-wise check) ...
+    monkeypatch.setenv("HIPIE_KEEP_F32", "1")
     # ranges for the reduced width: about 30 levels per standard deviation, so the tails saturate
     g, meta = builders.bert_encoder(layers=layers, hidden=hidden, heads=heads, ffn=ffn, batch=batch, seq=seq, seed=7,
                                     ranges=dict(q=0.12, k=0.9, v=0.9, ctx=0.6))
     x = np.random.default_rng(70).normal(0, 1, (batch, seq, hidden)).astype(np.float32)
     plan = g.compile()
     types = [s["type"] for s in plan.steps]
-    assert types.count("MatMul") == 8 * layers and types.count("Softmax") == layers
-    assert types.count("MVN") == 2 * layers and types.count("Gelu") == layers and types.count("Transpose") == layers
+    assert types.count("MatMul") == 8 * layers and types.count("Transpose") == layers
+    assert types.count("Softmax+FakeQuantize") == layers and types.count("Gelu+FakeQuantize") == layers
     req = plan.create_request()
     (y,) = req.infer(x)
     device = {n: req.matrix(n) for n in meta["glue"]}
@@ -47,11 +49,25 @@ def _check_stack(orc, layers, hidden, heads, ffn, batch, seq):
         q = kept[L["q"]]
         assert len(np.unique(q)) > 60                      # the ranges are exercised, not saturated
     np.testing.assert_array_equal(y.view(np.uint32), want["out"].view(np.uint32))
-    return plan, req, x, y
+    # ... then as it runs by default: results that only a fused FakeQuantize reads are not stored, the
+    # same kernels compute the same bits
+    monkeypatch.delenv("HIPIE_KEEP_F32")
+    plan2 = g.compile()
+    assert len(plan2.steps) < len(plan.steps)
+    req2 = plan2.create_request()
+    (y2,) = req2.infer(x)
+    np.testing.assert_array_equal(y2.view(np.uint32), y.view(np.uint32))
+    for li, L in enumerate(meta["layers"]):
+        for name in ("q", "k", "v", "scores", "pq", "ctxq", "attn", "h1q", "up", "gq", "down"):
+            np.testing.assert_array_equal(req2.matrix(L[name]), req.matrix(L[name]), err_msg="layer %d %s" % (li, name))
+        for name in ("p", "ctx", "gelu"):
+            with pytest.raises(Exception):
+                req2.matrix(L[name])
+    return plan2, req2, x, y
 
 
-def test_encoder_stack_matches_the_oracle(orc):
-    plan, req, x, y = _check_stack(orc, layers=2, hidden=128, heads=2, ffn=256, batch=2, seq=128)
+def test_encoder_stack_matches_the_oracle(orc, monkeypatch):
+    plan, req, x, y = _check_stack(orc, monkeypatch, layers=2, hidden=128, heads=2, ffn=256, batch=2, seq=128)
     # device-resident path gives the same bytes
     import torch
     ins, outs = req.device_buffers()
@@ -60,9 +76,9 @@ def test_encoder_stack_matches_the_oracle(orc):
     np.testing.assert_array_equal(outs[0].cpu().numpy(), y)
 
 
-def test_encoder_stack_other_head_count_and_ragged_rows(orc):
+def test_encoder_stack_other_head_count_and_ragged_rows(orc, monkeypatch):
     """three heads, a sequence length that is not a multiple of the 128-row tiles"""
-    _check_stack(orc, layers=1, hidden=192, heads=3, ffn=320, batch=3, seq=64)
+    _check_stack(orc, monkeypatch, layers=1, hidden=192, heads=3, ffn=320, batch=3, seq=64)
 
 
 def test_unsupported_transformer_nodes_are_reported():

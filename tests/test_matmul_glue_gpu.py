@@ -74,3 +74,60 @@ def test_softmax_mvn_gelu_tolerance(orc):
     np.testing.assert_allclose(got, want, rtol=1e-5, atol=2e-6)
     f = (rng.standard_normal((64, 3072)) * 2).astype(np.float32)
     np.testing.assert_allclose(gelu(torch.from_numpy(f).cuda()).cpu().numpy(), orc.gelu_erf(f), rtol=1e-6, atol=1e-8)
+
+
+@pytest.mark.parametrize("axis", [4, 64, 100, 252, 384, 390, 768, 1500, 3072, 4100])
+def test_glue_row_lengths(orc, axis):
+    """rows held in registers (multiples of 4 up to 4096, partial last chunk) and the three-pass fallback"""
+    import torch
+    from dldt_amd import mvn, softmax
+    rng = np.random.default_rng(axis)
+    x = (rng.standard_normal((37, axis)) * 3).astype(np.float32)
+    xd = torch.from_numpy(x).cuda()
+    np.testing.assert_allclose(softmax(xd).cpu().numpy(), orc.softmax(x, -1), rtol=3e-6, atol=1e-8)
+    tol = dict(rtol=2e-5, atol=4e-6)
+    np.testing.assert_allclose(mvn(xd).cpu().numpy(), orc.mvn_last_axis(x, True, 1e-5, True), **tol)
+    np.testing.assert_allclose(mvn(xd, False).cpu().numpy(), orc.mvn_last_axis(x, False, 1e-5, True), **tol)
+
+
+def _fq_i8(orc, v, il, ih):
+    return orc.fake_quantize(v, np.float32(il), np.float32(ih), np.float32(-128), np.float32(127), 256).astype(np.int8)
+
+
+@pytest.mark.parametrize("axis", [384, 100, 390])
+def test_glue_with_fused_requantisation(orc, axis):
+    """The fused i8 output equals the reference FakeQuantize of the kernel's own f32 result bit for bit,
+    and the f32 result does not depend on whether the quantized output is asked for."""
+    import torch
+    from dldt_amd import gelu, mvn, softmax
+    rng = np.random.default_rng(5 + axis)
+    x = (rng.standard_normal((61, axis)) * 2).astype(np.float32)
+    xd = torch.from_numpy(x).cuda()
+    gamma = torch.from_numpy(rng.uniform(0.5, 1.5, axis).astype(np.float32)).cuda()
+    beta = torch.from_numpy(rng.normal(0, 0.1, axis).astype(np.float32)).cuda()
+    il, ih = np.float32(-128) * np.float32(1.0 / 127), np.float32(1.0)
+    cases = [
+        ("softmax", lambda **k: softmax(xd, **k), (il * np.float32(0.2), ih * np.float32(0.2))),
+        ("mvn", lambda **k: mvn(xd, True, 1e-5, True, gamma, beta, **k), (il * 2, ih * 2)),
+        ("gelu", lambda **k: gelu(xd, **k), (il * 3, ih * 3)),
+    ]
+    for name, fn, (lo, hi) in cases:
+        plain = fn().cpu().numpy()
+        y, q = fn(requant=(lo, hi, -128, 256))
+        np.testing.assert_array_equal(y.cpu().numpy().view(np.uint32), plain.view(np.uint32), err_msg=name)
+        want = _fq_i8(orc, plain, lo, hi)
+        np.testing.assert_array_equal(q.cpu().numpy(), want, err_msg=name)
+        assert len(np.unique(want)) > 40, name
+        if axis % 4 == 0:                                   # f32 output left out: register-resident rows only
+            q_only = fn(requant=(lo, hi, -128, 256), keep_f32=False)
+            np.testing.assert_array_equal(q_only.cpu().numpy(), want, err_msg=name)
+
+
+def test_glue_requantisation_rejects_non_integer_levels():
+    import torch
+    from dldt_amd import HipieError, gelu
+    x = torch.zeros((4, 64), device="cuda")
+    with pytest.raises(HipieError):
+        gelu(x, requant=(-1.0, 1.0, -0.5, 256))
+    with pytest.raises(HipieError):
+        gelu(x, requant=(1.0, -1.0, -128, 256))
