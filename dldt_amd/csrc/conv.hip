@@ -152,7 +152,13 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     gemm(a.in + batch_offset(a, batch, a.batch_in, a.batch_in_o), a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
          a.wgt + batch_offset(a, batch, a.batch_wgt, a.batch_wgt_o), a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused);
     const int m0 = pix0 + wpix * 64 + l32;
-    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, (lds_cfloat_ptr)sP, BOC, oc0);
+    // the K loop ends with a barrier, so the operand tiles are free: every wave takes 8 KB of them as
+    // the staging buffer of its f32 stores (2 (BOC + BPIX) 64 bytes cover 8 KB per wave for all shapes)
+    constexpr int kStageWavesA = 2 * BOC * kRow / 8192;
+    static_assert(2 * (BOC + BPIX) * kRow >= (NT / 64) * 8192 && 2 * BOC * kRow % 8192 == 0, "staging space");
+    lds_float_ptr stage = wave < kStageWavesA ? (lds_float_ptr)&sA[0][0] + wave * 2048
+                                              : (lds_float_ptr)&sB[0][0] + (wave - kStageWavesA) * 2048;
+    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, (lds_cfloat_ptr)sP, BOC, oc0, stage);
 }
 
 // Persistent LDS-tiled kernel for the layers whose time is the epilogue and the memory latency

@@ -284,8 +284,16 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
                                          const bool (&valid)[2], const int64_t (&out_off)[2],
                                          const int64_t (&res_off)[2], const v16f (&rres)[2][2],
                                          lds_cfloat_ptr sp, int sp_stride, int oc0,
-                                         const uint32_t (*pre_res)[8] = nullptr) {
+                                         const uint32_t (*pre_res)[8] = nullptr, lds_float_ptr stage = nullptr) {
     const uint32_t fl = F == kDyn ? a.flags : F;
+    // f32 results leave through a wave-private 8 KB LDS buffer (`stage`, when the kernel has one): a
+    // lane owns 32 channels of two pixels, so direct stores put 16-byte pieces of 32 different rows in
+    // one instruction; staged, 16 lanes store the 256 contiguous bytes of one pixel's 64 channels.
+    // One pixel block (32 pixels) at a time, rows of 16 chunks with chunk c of row r kept in slot
+    // c ^ (r & 15): conflict-free for the writes (rows r .. r + 7, one chunk) and the reads (one row).
+    constexpr bool kCanStage = F != kDyn && !(F & (CF_OUT_FQ | CF_OUT_I32)) && NOB == 2;
+    const bool staged_out = kCanStage && stage != nullptr;
+    const int lane_id = static_cast<int>(threadIdx.x) & 63;
     auto tab = [&](int t, const float* g, int oc) {
         if (sp) {
             typedef float v4f __attribute__((ext_vector_type(4)));
@@ -321,6 +329,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
         }
     }
 
+    int pass_now = 0;   // pixel block of the current pass over the channels (staged f32 output only)
     auto load = [&](int e4, EpiParams& p) {
         const int oc = oc_lane + 4 * e4;
         if (fl & CF_BIAS) p.bias = tab(PT_BIAS, a.bias, oc);
@@ -340,6 +349,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
         if ((fl & CF_RES) && (fl & CF_RES_F32)) {
 #pragma unroll
             for (int pb = 0; pb < 2; ++pb) {
+                if (staged_out && pb != pass_now) continue;
                 p.res[pb] = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (valid[pb] && oc + 4 <= a.res_sw)
                     p.res[pb] = ld4f(static_cast<const float*>(a.res) + res_off[pb] + 4 * e4);
@@ -348,6 +358,10 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
     };
 
     uint32_t out_dw[2][8];
+#pragma unroll
+    for (int pass = 0; pass < (kCanStage ? 2 : 1); ++pass) {
+    if (pass == 1 && !staged_out) break;
+    pass_now = pass;
     EpiParams cur, nxt;
     load(0, cur);
 #pragma unroll
@@ -373,6 +387,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
         float v[2][4];
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb) {
+            if (staged_out && pb != pass) continue;   // staged: pixel block `pass` only
             float rv[4];
             if (fl & CF_RES) {
                 if (fl & CF_RES_GEMM) {
@@ -423,6 +438,12 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
             asm volatile("" : "+v"(packed[0]), "+v"(packed[1]) : : "memory");
             out_dw[0][e4] = packed[0];
             out_dw[1][e4] = packed[1];
+        } else if (staged_out) {
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            const int row = lane_id & 31, c = ((lane_id >> 5) * 8 + e4) ^ (row & 15);
+            v4f o;
+            o.x = v[pass][0]; o.y = v[pass][1]; o.z = v[pass][2]; o.w = v[pass][3];
+            *(__attribute__((address_space(3))) v4f*)(stage + row * 64 + c * 4) = o;
         } else {
             asm volatile("" : "+v"(v[0][0]), "+v"(v[0][1]), "+v"(v[0][2]), "+v"(v[0][3]), "+v"(v[1][0]),
                          "+v"(v[1][1]), "+v"(v[1][2]), "+v"(v[1][3]) : : "memory");
@@ -433,6 +454,28 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
                         make_float4(v[pb][0], v[pb][1], v[pb][2], v[pb][3]);
         }
         cur = nxt;
+    }
+    if (staged_out) {
+        // LDS operations of one wave complete in order; the waits only keep the compiler from moving
+        // accesses across the two phases
+        typedef float v4f __attribute__((ext_vector_type(4)));
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const int oc_wave = oc_lane - 32 * (lane_id >> 5);          // first channel of the wave's 64
+        const int c = lane_id & 15;
+        const int64_t own = out_off[pass] - 32 * (lane_id >> 5);    // lanes 0 .. 31 hold rows 0 .. 31
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = 4 * i + (lane_id >> 4);
+            const v4f o = *(const __attribute__((address_space(3))) v4f*)(stage + row * 64 + ((c ^ (row & 15)) * 4));
+            const uint32_t lo = __shfl(static_cast<uint32_t>(own), row, 64);
+            const uint32_t hi = __shfl(static_cast<uint32_t>(static_cast<uint64_t>(own) >> 32), row, 64);
+            const int ok = __shfl(static_cast<int>(valid[pass]), row, 64);
+            const int64_t off = static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+            if (ok && oc_wave + 4 * c + 4 <= out_cs)
+                *reinterpret_cast<float4*>(static_cast<float*>(a.out) + off + 4 * c) = make_float4(o.x, o.y, o.z, o.w);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
     }
     if (fl & CF_OUT_FQ) {
         // stored byte = level + out_off (mod 256); -128 is a sign-bit flip, 0 nothing: one XOR mask
@@ -479,10 +522,11 @@ __device__ __forceinline__ void epilogue_addresses(const ConvArgs& a, int oc_lan
 template <uint32_t F>
 __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                              int m0, int m1, int batch, const v16f (&rres)[2][2],
-                                             lds_cfloat_ptr sp = nullptr, int sp_stride = 0, int oc0 = 0) {
+                                             lds_cfloat_ptr sp = nullptr, int sp_stride = 0, int oc0 = 0,
+                                             lds_float_ptr stage = nullptr) {
     EpiAddr e;
     epilogue_addresses(a, oc_lane, m0, m1, batch, e);
-    epilogue<F>(a, acc, oc_lane, e.valid, e.out_off, e.res_off, rres, sp, sp_stride, oc0);
+    epilogue<F>(a, acc, oc_lane, e.valid, e.out_off, e.res_off, rres, sp, sp_stride, oc0, nullptr, stage);
 }
 
 template <uint32_t F>
