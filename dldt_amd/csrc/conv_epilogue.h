@@ -293,6 +293,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
     // c ^ (r & 15): conflict-free for the writes (rows r .. r + 7, one chunk) and the reads (one row).
     constexpr bool kCanStage = F != kDyn && !(F & (CF_OUT_FQ | CF_OUT_I32)) && NOB == 2;
     const bool staged_out = kCanStage && stage != nullptr;
+    constexpr bool kCanStageBytes = F != kDyn && (F & CF_OUT_FQ) && NOB == 2;
     const int lane_id = static_cast<int>(threadIdx.x) & 63;
     auto tab = [&](int t, const float* g, int oc) {
         if (sp) {
@@ -489,6 +490,42 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
                 for (int q = 0; q < 4 * NOB; ++q) out_dw[pb][q] = add_bytes(out_dw[pb][q], off4);
         }
         const uint32_t xmask = flip ? 0x80808080u : 0u;
+        if (kCanStageBytes && stage != nullptr) {
+            // Bytes leave through the wave's LDS buffer as well: 64 rows (pixels) of the wave's 64
+            // channels, chunk c (16 bytes) of row r in slot c ^ ((r >> 2) & 3); four lanes then store
+            // the 64 contiguous bytes of one pixel instead of 16-byte pieces of 32 different pixels.
+            typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+            typedef __attribute__((address_space(3))) v4u* lds_v4u_ptr;
+            const lds_v4u_ptr st = (lds_v4u_ptr)stage;
+            const int h = lane_id >> 5;
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int row = 32 * pb + (lane_id & 31);
+                    v4u o;
+                    o.x = out_dw[pb][4 * j] ^ xmask; o.y = out_dw[pb][4 * j + 1] ^ xmask;
+                    o.z = out_dw[pb][4 * j + 2] ^ xmask; o.w = out_dw[pb][4 * j + 3] ^ xmask;
+                    st[row * 4 + ((2 * h + j) ^ ((row >> 2) & 3))] = o;
+                }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            const int oc_wave = oc_lane - 32 * h;
+            const int c = lane_id & 3;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = 16 * i + (lane_id >> 2), pb = i >> 1, src = row & 31;
+                const v4u o = st[row * 4 + (c ^ ((row >> 2) & 3))];
+                const int64_t own = out_off[pb] - 32 * h;
+                const uint32_t lo = __shfl(static_cast<uint32_t>(own), src, 64);
+                const uint32_t hi = __shfl(static_cast<uint32_t>(static_cast<uint64_t>(own) >> 32), src, 64);
+                const int ok = __shfl(static_cast<int>(valid[pb]), src, 64);
+                const int64_t off = static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+                if (ok && oc_wave + 16 * c < out_cs)
+                    *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + off + 16 * c) = make_uint4(o.x, o.y, o.z, o.w);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            return;
+        }
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb)
 #pragma unroll
