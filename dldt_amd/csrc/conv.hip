@@ -645,6 +645,7 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
     case E_F32: X(E_F32, __VA_ARGS__); break;                                                \
     case E_SCALE: X(E_SCALE, __VA_ARGS__); break;                                            \
     case E_SCALEFQ: X(E_SCALEFQ, __VA_ARGS__); break;                                        \
+    case E_DEQFQ: X(E_DEQFQ, __VA_ARGS__); break;                                            \
     case E_RESI8: X(E_RESI8, __VA_ARGS__); break;                                            \
     case E_F32RES: X(E_F32RES, __VA_ARGS__); break;                                          \
     case E_F32RELU: X(E_F32RELU, __VA_ARGS__); break;                                        \

@@ -117,6 +117,7 @@ constexpr uint32_t E_RESI8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_MUL | E_FQ;   
 constexpr uint32_t E_SCALEFQ = CF_BIAS | CF_SCALE | E_FQ;              // linear layer requantised to symmetric i8
 constexpr uint32_t E_F32RES = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32;   // linear layer + f32 residual, f32 out                      // MatMul' -> Multiply(s_a * s_b)
 constexpr uint32_t E_F32RELU = CF_BIAS | CF_SCALE | CF_RELU;
+constexpr uint32_t E_DEQFQ = CF_SCALE | E_FQ;                           // MatMul between activations, requantised (attention context)
 constexpr uint32_t E_CLAMPFQ = CF_BIAS | CF_SCALE | CF_CLAMP | E_FQ | CF_FQ_IL0;
 
 // Per-channel tables of the epilogue staged in LDS, one row of `stride` floats per table.  Every
@@ -294,6 +295,11 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
     constexpr bool kCanStage = F != kDyn && !(F & (CF_OUT_FQ | CF_OUT_I32)) && NOB == 2;
     const bool staged_out = kCanStage && stage != nullptr;
     constexpr bool kCanStageBytes = F != kDyn && (F & CF_OUT_FQ) && NOB == 2;
+    // an f32 residual that is the last operation in front of the store is added where the staged rows
+    // are read back: there a lane's residual piece is as contiguous as its store
+    constexpr bool kLateRes = kCanStage && (F & CF_RES) && (F & CF_RES_F32) &&
+                              !(F & (CF_RES_SUB | CF_RES_MUL | CF_POST_SCALE | CF_RELU | CF_CLAMP | CF_RES_GEMM));
+    const bool late_res = kLateRes && staged_out;
     const int lane_id = static_cast<int>(threadIdx.x) & 63;
     auto tab = [&](int t, const float* g, int oc) {
         if (sp) {
@@ -347,7 +353,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
                 p.d = tab(PT_D, a.fq_d, oc);
             }
         }
-        if ((fl & CF_RES) && (fl & CF_RES_F32)) {
+        if ((fl & CF_RES) && (fl & CF_RES_F32) && !late_res) {
 #pragma unroll
             for (int pb = 0; pb < 2; ++pb) {
                 if (staged_out && pb != pass_now) continue;
@@ -390,7 +396,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
         for (int pb = 0; pb < 2; ++pb) {
             if (staged_out && pb != pass) continue;   // staged: pixel block `pass` only
             float rv[4];
-            if (fl & CF_RES) {
+            if ((fl & CF_RES) && !late_res) {
                 if (fl & CF_RES_GEMM) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) rv[j] = rres[ob][pb][r0 + j];
@@ -406,7 +412,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
                 float x = static_cast<float>(acc[ob][pb][r0 + j]);
                 if (fl & CF_BIAS) x = x + bias_[j];
                 if (fl & CF_SCALE) x = x * scale_[j];
-                if (fl & CF_RES) {
+                if ((fl & CF_RES) && !late_res) {
                     float r = rv[j];
                     if (fl & CF_RES_SUB) r = r - rsub_[j];
                     if (fl & CF_RES_MUL) r = r * rmul_[j];
@@ -464,16 +470,34 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
         const int oc_wave = oc_lane - 32 * (lane_id >> 5);          // first channel of the wave's 64
         const int c = lane_id & 15;
         const int64_t own = out_off[pass] - 32 * (lane_id >> 5);    // lanes 0 .. 31 hold rows 0 .. 31
+        const int64_t own_res = res_off[pass] - 32 * (lane_id >> 5);
+        auto from_row = [&](int64_t v, int row) {
+            const uint32_t lo = __shfl(static_cast<uint32_t>(v), row, 64);
+            const uint32_t hi = __shfl(static_cast<uint32_t>(static_cast<uint64_t>(v) >> 32), row, 64);
+            return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+        };
+        float4 late[8];
+        bool ok[8];
+        int64_t off[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = 4 * i + (lane_id >> 4);
+            off[i] = from_row(own, row);
+            ok[i] = __shfl(static_cast<int>(valid[pass]), row, 64) != 0;
+            if (late_res) {   // all eight loads in flight together
+                late[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                const int64_t roff = from_row(own_res, row);
+                if (ok[i] && oc_wave + 4 * c + 4 <= a.res_sw) late[i] = ld4f(static_cast<const float*>(a.res) + roff + 4 * c);
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int row = 4 * i + (lane_id >> 4);
             const v4f o = *(const __attribute__((address_space(3))) v4f*)(stage + row * 64 + ((c ^ (row & 15)) * 4));
-            const uint32_t lo = __shfl(static_cast<uint32_t>(own), row, 64);
-            const uint32_t hi = __shfl(static_cast<uint32_t>(static_cast<uint64_t>(own) >> 32), row, 64);
-            const int ok = __shfl(static_cast<int>(valid[pass]), row, 64);
-            const int64_t off = static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
-            if (ok && oc_wave + 4 * c + 4 <= out_cs)
-                *reinterpret_cast<float4*>(static_cast<float*>(a.out) + off + 4 * c) = make_float4(o.x, o.y, o.z, o.w);
+            float4 r = make_float4(o.x, o.y, o.z, o.w);
+            if (late_res) { r.x = r.x + late[i].x; r.y = r.y + late[i].y; r.z = r.z + late[i].z; r.w = r.w + late[i].w; }
+            if (ok[i] && oc_wave + 4 * c + 4 <= out_cs)
+                *reinterpret_cast<float4*>(static_cast<float*>(a.out) + off[i] + 4 * c) = r;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
