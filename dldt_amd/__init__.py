@@ -5,5 +5,5 @@ Python binding used by the tests and the benchmark.  There is no CPU fallback: e
 object raises if the library is missing.
 """
 from ._lib import HipieError, lib  # noqa: F401
-from .ops import BatchedMatMul, Convolution, FakeQuantize, gelu, make_epilogue, mvn, softmax  # noqa: F401
+from .ops import BatchedMatMul, Convolution, FakeQuantize, attention, gelu, make_epilogue, mvn, softmax  # noqa: F401
 from .tensor import DeviceTensor  # noqa: F401

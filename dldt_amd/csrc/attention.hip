@@ -1,0 +1,225 @@
+// Self-attention core of a post-LPT encoder in one kernel:
+//     scores = MatMul'(q, k^T) * s1 -> Softmax -> FakeQuantize (i8) -> MatMul'(., v) * s2 [-> FakeQuantize]
+// (mat_mul.cpp:81-171 leaves the two TypeRelaxed MatMuls with their dequantization Multiply; softmax.hpp,
+// fake_quantize.hpp).  The f32 scores and probabilities of one encoder layer are 2 x 113 MB at
+// batch 16 x 12 heads x 384^2; here they never leave the registers.
+//
+// One workgroup (4 waves) takes 128 queries of one (sequence, head); a wave takes 32 of them against
+// all S keys.  Keys are the rows of the first MFMA operand and queries its columns, so a lane ends up
+// with S / 2 scores of ONE query (column l % 32; rows 8 (r / 4) + 4 (l / 32) + r % 4 of every 32-key
+// tile): the softmax reductions are a loop over the lane's registers plus one exchange with lane
+// l ^ 32.  The requantised probabilities of a tile, packed in register order, are already the second
+// MFMA's column operand for "32 keys in the order (r, l / 32)"; V is transposed into LDS in exactly
+// that key order, so the probabilities go from the accumulators of the first product into the
+// second without touching memory.  Integer sums are exact, every f32 step is one IEEE operation in
+// the graph's order; Softmax has tolerance parity like the stand-alone kernel.
+#include "conv_epilogue.h"
+#include "requant.h"
+
+namespace hipie {
+namespace {
+
+constexpr int kMaxSeq = 384;   // S / 2 accumulator registers per lane
+constexpr int kHeadDim = 64;
+
+struct AttentionArgs {
+    const int8_t *q, *k, *v;
+    int64_t ldq, sq, oq, ldk, sk, ok, ldv, sv, ov;   // row pitch, inner / outer batch stride (bytes)
+    void* out;
+    int64_t ldo, so, oo;                              // elements
+    float* scores;                                    // optional [batch][S][S] dumps (inspection), or null
+    float* probs;
+    int S, batch_inner;
+    float scale1, scale2;
+    Requant fq_p, fq_o;                               // fq_o.levels == 0: f32 output
+};
+
+template <int NT>   // NT = S / 32 key tiles
+__global__ __launch_bounds__(256) void attention_kernel(const AttentionArgs a) {
+    constexpr int S = NT * 32;
+    constexpr int VT_LD = S + 16;                     // odd number of 16-byte groups per row: conflict-free
+    __shared__ __attribute__((aligned(16))) int8_t sK[S * 64];       // [key][d], chunk c of row r in slot c ^ ((r >> 2) & 3)
+    __shared__ __attribute__((aligned(16))) int8_t sVT[64 * VT_LD];  // [d][tile][half][j]: key 32 t + 8 (j / 4) + 4 half + j % 4
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int b = blockIdx.y, bo = b / a.batch_inner, bi = b - bo * a.batch_inner;
+    const int8_t* qp = a.q + bo * a.oq + bi * a.sq;
+    const int8_t* kp = a.k + bo * a.ok + bi * a.sk;
+    const int8_t* vp = a.v + bo * a.ov + bi * a.sv;
+
+    // ---- K into LDS (rows of 64 bytes), V transposed into LDS ------------------------------------
+    for (int i = tid; i < S * 4; i += 256) {
+        const int r = i >> 2, c = i & 3;
+        const v4i x = *reinterpret_cast<const v4i*>(kp + r * a.ldk + c * 16);
+        *reinterpret_cast<v4i*>(&sK[r * 64 + ((c ^ ((r >> 2) & 3)) * 16)]) = x;
+    }
+    for (int i = tid; i < (S / 4) * 16; i += 256) {
+        const int d4 = i & 15, kq = i >> 4;            // 4 consecutive keys x 4 consecutive d
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = *reinterpret_cast<const uint32_t*>(vp + (4 * kq + j) * a.ldv + 4 * d4);
+        // 4 x 4 byte transpose: t[e] = bytes e of w[0..3]
+        const uint32_t lo01 = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u);   // w0.b0 w1.b0 w0.b1 w1.b1
+        const uint32_t hi01 = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);   // w0.b2 w1.b2 w0.b3 w1.b3
+        const uint32_t lo23 = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u);
+        const uint32_t hi23 = __builtin_amdgcn_perm(w[3], w[2], 0x07030602u);
+        const uint32_t t[4] = {__builtin_amdgcn_perm(lo23, lo01, 0x05040100u), __builtin_amdgcn_perm(lo23, lo01, 0x07060302u),
+                               __builtin_amdgcn_perm(hi23, hi01, 0x05040100u), __builtin_amdgcn_perm(hi23, hi01, 0x07060302u)};
+        const int key = 4 * kq, tile = key >> 5, in = key & 31;               // in = 8 a + 4 half
+        const int col = tile * 32 + ((in >> 2) & 1) * 16 + (in >> 3) * 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) *reinterpret_cast<uint32_t*>(&sVT[(4 * d4 + e) * VT_LD + col]) = t[e];
+    }
+
+    // ---- this wave's queries: the column operand of the first product, straight from memory ------
+    const int q_row = blockIdx.x * 128 + wave * 32 + l32;
+    const bool q_ok = q_row < a.S;
+    const int8_t* qrow = qp + static_cast<int64_t>(q_ok ? q_row : a.S - 1) * a.ldq;
+    const v4i qf[2] = {*reinterpret_cast<const v4i*>(qrow + 16 * h), *reinterpret_cast<const v4i*>(qrow + 32 + 16 * h)};
+    __syncthreads();
+
+    const int slot[2] = {((0 + h) ^ ((l32 >> 2) & 3)) * 16, ((2 + h) ^ ((l32 >> 2) & 3)) * 16};
+    float x[NT][16];
+    float m = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const v4i kf = *reinterpret_cast<const v4i*>(&sK[(32 * t + l32) * 64 + slot[ks]]);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[ks], acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            x[t][r] = static_cast<float>(acc[r]) * a.scale1;
+            m = fmaxf(m, x[t][r]);
+        }
+    }
+    const int64_t dump_row = (static_cast<int64_t>(b) * a.S + q_row) * a.S;   // [batch][query][key]
+    if (a.scores && q_ok) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) a.scores[dump_row + 32 * t + 8 * (r >> 2) + 4 * h + (r & 3)] = x[t][r];
+    }
+    // Softmax over the keys of this lane's query (softmax.hpp: subtract the maximum, exp, sum, divide)
+    m = fmaxf(m, __shfl_xor(m, 32, 64));
+    float s = 0.f;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            x[t][r] = expf(x[t][r] - m);
+            s += x[t][r];
+        }
+    s += __shfl_xor(s, 32, 64);
+
+    // probabilities -> i8 levels -> second product, one 32-key tile at a time
+    v16i ctx[2] = {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}};
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        v4i pf;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float4 p4 = make_float4(x[t][4 * g] / s, x[t][4 * g + 1] / s, x[t][4 * g + 2] / s, x[t][4 * g + 3] / s);
+            if (a.probs && q_ok)
+                *reinterpret_cast<float4*>(a.probs + dump_row + 32 * t + 8 * g + 4 * h) = p4;
+            pf[g] = static_cast<int>(requant4(a.fq_p, p4));
+        }
+#pragma unroll
+        for (int db = 0; db < 2; ++db) {
+            const v4i vf = *reinterpret_cast<const v4i*>(&sVT[(32 * db + l32) * VT_LD + 32 * t + 16 * h]);
+            ctx[db] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf, ctx[db], 0, 0, 0);
+        }
+    }
+
+    // ---- context of query q_row: d = 32 db + 8 (r / 4) + 4 h + r % 4 --------------------------------
+    if (!q_ok) return;
+    const int64_t orow = bo * a.oo + bi * a.so + static_cast<int64_t>(q_row) * a.ldo;
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int d = 32 * db + 8 * g + 4 * h;
+            const float4 o = make_float4(static_cast<float>(ctx[db][4 * g]) * a.scale2, static_cast<float>(ctx[db][4 * g + 1]) * a.scale2,
+                                         static_cast<float>(ctx[db][4 * g + 2]) * a.scale2, static_cast<float>(ctx[db][4 * g + 3]) * a.scale2);
+            if (a.fq_o.levels) *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(a.out) + orow + d) = requant4(a.fq_o, o);
+            else *reinterpret_cast<float4*>(static_cast<float*>(a.out) + orow + d) = o;
+        }
+}
+
+template <int NT>
+void launch(const AttentionArgs& a, int batches, hipStream_t s) {
+    hipLaunchKernelGGL(attention_kernel<NT>, dim3(static_cast<uint32_t>(ceil_div(a.S, 128)), static_cast<uint32_t>(batches)),
+                       dim3(256), 0, s, a);
+}
+
+}  // namespace
+}  // namespace hipie
+
+using namespace hipie;
+
+extern "C" {
+
+int hipie_attention_supported(int32_t seq, int32_t head_dim) {
+    return seq > 0 && seq % 32 == 0 && seq <= kMaxSeq && head_dim == kHeadDim;
+}
+
+int hipie_attention_run(const hipie_attention_desc* desc, const void* q, int64_t ldq, int64_t stride_q, int64_t outer_q,
+                        const void* k, int64_t ldk, int64_t stride_k, int64_t outer_k, const void* v, int64_t ldv,
+                        int64_t stride_v, int64_t outer_v, void* out, int64_t ldo, int64_t stride_o, int64_t outer_o,
+                        int32_t batch, int32_t batch_outer, float* scores, float* probs, void* stream) {
+    return guarded([&] {
+        HIPIE_REQUIRE(desc && q && k && v && out, HIPIE_PARAMETER_MISMATCH, "hipie_attention_run: null argument");
+        HIPIE_REQUIRE(hipie_attention_supported(desc->seq, desc->head_dim), HIPIE_NOT_IMPLEMENTED,
+                      "hipie_attention_run: sequence length %d (multiple of 32 up to %d) / head dimension %d (%d)", desc->seq,
+                      kMaxSeq, desc->head_dim, kHeadDim);
+        if (batch == 0 || batch_outer == 0) return;
+        HIPIE_REQUIRE(batch > 0 && batch_outer > 0 && static_cast<int64_t>(batch) * batch_outer < 65536, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_attention_run: batch %d x %d", batch, batch_outer);
+        const bool byte_out = desc->out_dtype == HIPIE_I8;
+        HIPIE_REQUIRE(byte_out || desc->out_dtype == HIPIE_F32, HIPIE_PARAMETER_MISMATCH, "hipie_attention_run: output type %d",
+                      desc->out_dtype);
+        auto aligned = [](const void* p, int64_t a, int64_t b, int64_t c, int64_t g) {
+            return reinterpret_cast<uintptr_t>(p) % g == 0 && a % g == 0 && b % g == 0 && c % g == 0;
+        };
+        HIPIE_REQUIRE(ldq >= kHeadDim && ldk >= kHeadDim && ldv >= kHeadDim && ldo >= kHeadDim && aligned(q, ldq, stride_q, outer_q, 16) &&
+                          aligned(k, ldk, stride_k, outer_k, 16) && aligned(v, ldv, stride_v, outer_v, 4) &&
+                          aligned(out, ldo, stride_o, outer_o, 4) && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                          reinterpret_cast<uintptr_t>(probs) % 16 == 0,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_attention_run: pitches and strides must keep 16-byte rows aligned");
+        AttentionArgs a{};
+        a.q = static_cast<const int8_t*>(q); a.k = static_cast<const int8_t*>(k); a.v = static_cast<const int8_t*>(v);
+        a.ldq = ldq; a.sq = stride_q; a.oq = outer_q;
+        a.ldk = ldk; a.sk = stride_k; a.ok = outer_k;
+        a.ldv = ldv; a.sv = stride_v; a.ov = outer_v;
+        a.out = out; a.ldo = ldo; a.so = stride_o; a.oo = outer_o;
+        a.scores = scores; a.probs = probs;
+        a.S = desc->seq;
+        a.batch_inner = batch;
+        a.scale1 = desc->score_scale;
+        a.scale2 = desc->context_scale;
+        a.fq_p = make_requant(&desc->prob_fq, "hipie_attention_run (probabilities)");
+        if (byte_out) a.fq_o = make_requant(&desc->out_fq, "hipie_attention_run (output)");
+        hipStream_t s = as_stream(stream);
+        const int batches = batch * batch_outer;
+        switch (desc->seq / 32) {
+        case 1: launch<1>(a, batches, s); break;
+        case 2: launch<2>(a, batches, s); break;
+        case 3: launch<3>(a, batches, s); break;
+        case 4: launch<4>(a, batches, s); break;
+        case 5: launch<5>(a, batches, s); break;
+        case 6: launch<6>(a, batches, s); break;
+        case 7: launch<7>(a, batches, s); break;
+        case 8: launch<8>(a, batches, s); break;
+        case 9: launch<9>(a, batches, s); break;
+        case 10: launch<10>(a, batches, s); break;
+        case 11: launch<11>(a, batches, s); break;
+        default: launch<12>(a, batches, s); break;
+        }
+        HIPIE_CHECK_HIP(hipGetLastError());
+    });
+}
+
+}  // extern "C"

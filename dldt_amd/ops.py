@@ -308,3 +308,38 @@ def gelu(x, requant=None, keep_f32=True):
         check(lib().hipie_gelu_q8(_dptr(x), _dptr(y) if y is not None else None, _dptr(q), ctypes.c_int64(x.numel()),
                                   ctypes.byref(r), _stream()))
     return _ret(y, q)
+
+
+class hipie_attention_desc(ctypes.Structure):
+    _fields_ = [("seq", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("score_scale", ctypes.c_float),
+                ("context_scale", ctypes.c_float), ("prob_fq", hipie_requant), ("out_dtype", ctypes.c_int32),
+                ("out_fq", hipie_requant)]
+
+
+def attention(q, k, v, score_scale, context_scale, prob_fq, out_fq=None, dump=False):
+    """Fused attention core over i8 tensors [B, NH, S, 64] (any strides with contiguous rows):
+    returns the context [B, NH, S, 64] (f32, or i8 when out_fq is given) and, with dump=True, also the
+    f32 scores and probabilities [B, NH, S, S].  prob_fq / out_fq = (in_low, in_high, out_low, levels)."""
+    import torch
+    B, NH, S, D = q.shape
+    assert k.shape == q.shape and v.shape == q.shape and q.dtype == torch.int8
+    for t in (q, k, v):
+        assert t.stride(3) == 1
+    d = hipie_attention_desc()
+    d.seq, d.head_dim = S, D
+    d.score_scale, d.context_scale = float(score_scale), float(context_scale)
+    d.prob_fq = hipie_requant(*[float(x) for x in prob_fq[:3]], int(prob_fq[3]))
+    d.out_dtype = I8 if out_fq is not None else F32
+    if out_fq is not None:
+        d.out_fq = hipie_requant(*[float(x) for x in out_fq[:3]], int(out_fq[3]))
+    out = torch.empty((B, NH, S, D), dtype=torch.int8 if out_fq is not None else torch.float32, device=q.device)
+    scores = torch.empty((B, NH, S, S), dtype=torch.float32, device=q.device) if dump else None
+    probs = torch.empty_like(scores) if dump else None
+    i64 = ctypes.c_int64
+    args = []
+    for t in (q, k, v):
+        args += [_dptr(t), i64(t.stride(2)), i64(t.stride(1)), i64(t.stride(0))]
+    check(lib().hipie_attention_run(ctypes.byref(d), *args, _dptr(out), i64(out.stride(2)), i64(out.stride(1)),
+                                    i64(out.stride(0)), ctypes.c_int32(NH), ctypes.c_int32(B),
+                                    _dptr(scores) if dump else None, _dptr(probs) if dump else None, _stream()))
+    return (out, scores, probs) if dump else out

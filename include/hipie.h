@@ -273,6 +273,30 @@ int hipie_softmax_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t 
 int hipie_mvn_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis, int normalize_variance, float eps,
                  int eps_inside_sqrt, const float* gamma, const float* beta, const hipie_requant* requant, void* stream);
 int hipie_gelu_q8(const float* x, float* y, int8_t* q, int64_t n, const hipie_requant* requant, void* stream);
+/* Self-attention core of a post-LPT encoder in one kernel, per (sequence, head):
+ *     MatMul'(q, k^T) * score_scale -> Softmax -> FakeQuantize(prob_fq) -> MatMul'(., v) * context_scale
+ *     [-> FakeQuantize(out_fq) when out_dtype is HIPIE_I8]
+ * i.e. the two TypeRelaxed MatMuls low_precision_transformations/src/mat_mul.cpp:81-171 leaves, with
+ * reference::softmax (softmax.hpp:20-50) and reference::fake_quantize between them.  q, k, v are i8
+ * [seq, head_dim] matrices addressed like the operands of hipie_matmul_run_nested (row pitch, inner and
+ * outer batch stride, in bytes); out is [seq, head_dim] f32 or i8 (pitch and strides in elements).
+ * The integer products are exact and every f32 step is one IEEE operation in that order; Softmax
+ * has tolerance parity.  scores / probs, when not NULL, receive the f32 values in front of and
+ * behind the Softmax as dense [batch_outer * batch][seq][seq] arrays (inspection; the kernel is
+ * otherwise the same).  Sequence lengths: multiples of 32 up to 384; head_dim 64
+ * (hipie_attention_supported). */
+typedef struct hipie_attention_desc {
+    int32_t seq, head_dim;
+    float score_scale, context_scale;
+    hipie_requant prob_fq;
+    int32_t out_dtype;          /* HIPIE_F32 or HIPIE_I8 */
+    hipie_requant out_fq;       /* used when out_dtype is HIPIE_I8 */
+} hipie_attention_desc;
+int hipie_attention_supported(int32_t seq, int32_t head_dim);
+int hipie_attention_run(const hipie_attention_desc* desc, const void* q, int64_t ldq, int64_t stride_q, int64_t outer_q,
+                        const void* k, int64_t ldk, int64_t stride_k, int64_t outer_k, const void* v, int64_t ldv,
+                        int64_t stride_v, int64_t outer_v, void* out, int64_t ldo, int64_t stride_o, int64_t outer_o,
+                        int32_t batch, int32_t batch_outer, float* scores, float* probs, void* stream);
 /* Transpose of the two inner dimensions of a byte tensor (opset1 Transpose on quantized activations,
  * e.g. V [S, d] -> [d, S] so that the context MatMul finds its reduction axis contiguous;
  * reference::transpose, .../reference/transpose.hpp:20-25): dst[b][c][r] = src[b][r][c], leading

@@ -131,3 +131,50 @@ def test_glue_requantisation_rejects_non_integer_levels():
         gelu(x, requant=(-1.0, 1.0, -0.5, 256))
     with pytest.raises(HipieError):
         gelu(x, requant=(1.0, -1.0, -128, 256))
+
+
+@pytest.mark.parametrize("B,NH,S", [(2, 3, 384), (1, 2, 96), (2, 1, 160), (1, 1, 32)])
+def test_fused_attention(orc, B, NH, S):
+    """scores bit-exact, Softmax within tolerance, and from the kernel's own probabilities the
+    requantisation, the context product and its dequantisation (and requantisation) bit-exact; the
+    kernel without the inspection outputs gives the same bytes.  q, k, v are head slices of one
+    [tokens, 3 * hidden] tensor, as a fused QKV projection leaves them."""
+    import torch
+    from dldt_amd import attention
+    rng = np.random.default_rng(S + NH)
+    H = NH * 64
+    qkv = rng.integers(-128, 128, (B, S, 3, NH, 64), dtype=np.int8)
+    qkv[:, :, 0] = np.clip(rng.normal(0, 20, (B, S, NH, 64)), -128, 127).astype(np.int8)
+    t = torch.from_numpy(qkv).cuda()
+    q, k, v = (t[:, :, i].permute(0, 2, 1, 3) for i in range(3))           # [B, NH, S, 64] views, row pitch 3 H
+    assert q.stride(2) == 3 * H
+    s1, s2 = np.float32(0.0007), np.float32(0.02 / 127)
+    il, ih = np.float32(-128.0 / 127), np.float32(1.0)
+    ctx, scores, probs = attention(q, k, v, s1, s2, (il, ih, -128, 256), dump=True)
+    qn, kn, vn = (np.ascontiguousarray(x.cpu().numpy()).astype(np.int32) for x in (q, k, v))
+    want_scores = orc.multiply(orc.matmul(qn, kn, False, True).astype(np.float32), s1)
+    np.testing.assert_array_equal(scores.cpu().numpy().view(np.uint32), want_scores.view(np.uint32))
+    p = probs.cpu().numpy()
+    np.testing.assert_allclose(p, orc.softmax(want_scores, -1), rtol=3e-6, atol=1e-8)
+    pq = orc.fake_quantize(p, il, ih, np.float32(-128), np.float32(127), 256).astype(np.int32)
+    assert len(np.unique(pq)) > 20
+    want_ctx = orc.multiply(orc.matmul(pq, vn).astype(np.float32), s2)
+    np.testing.assert_array_equal(ctx.cpu().numpy().view(np.uint32), want_ctx.view(np.uint32))
+    plain = attention(q, k, v, s1, s2, (il, ih, -128, 256))
+    assert torch.equal(plain, ctx)
+    # requantised output
+    ol, oh = np.float32(-128) * np.float32(0.004), np.float32(127) * np.float32(0.004)
+    cq = attention(q, k, v, s1, s2, (il, ih, -128, 256), out_fq=(ol, oh, -128, 256))
+    want_q = orc.fake_quantize(want_ctx, ol, oh, np.float32(-128), np.float32(127), 256).astype(np.int8)
+    np.testing.assert_array_equal(cq.cpu().numpy(), want_q)
+    assert len(np.unique(want_q)) > 40
+
+
+def test_fused_attention_rejects_unsupported_shapes():
+    import torch
+    from dldt_amd import HipieError, attention
+    for shape in [(1, 1, 48, 64), (1, 1, 416, 64), (1, 1, 64, 32)]:
+        x = torch.zeros(shape, dtype=torch.int8, device="cuda")
+        with pytest.raises(HipieError) as e:
+            attention(x, x, x, 1.0, 1.0, (-1.0, 1.0, -128, 256))
+        assert e.value.status == -2
