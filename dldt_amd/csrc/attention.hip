@@ -14,6 +14,7 @@
 // second without touching memory.  Integer sums are exact, every f32 step is one IEEE operation in
 // the graph's order; Softmax has tolerance parity like the stand-alone kernel.
 #include "conv_epilogue.h"
+#include "div2.h"
 #include "requant.h"
 
 namespace hipie {
@@ -32,10 +33,26 @@ struct AttentionArgs {
     int S, batch_inner;
     float scale1, scale2;
     Requant fq_p, fq_o;                               // fq_o.levels == 0: f32 output
+    float p_zh, p_zl;                                 // probabilities: two-operation division by fq_p.p.d
+    int p_div2;                                       // ... verified against IEEE division on the device
+    uint32_t p_xor, p_add;                            // stored byte = level + out_low (mod 256): XOR 0x80 per byte, or bytewise add
 };
 
-template <int NT>   // NT = S / 32 key tiles
-__global__ __launch_bounds__(256) void attention_kernel(const AttentionArgs a) {
+// level index k of four probabilities as four unsigned bytes (rounded to nearest-even and packed by
+// v_cvt_pk_u8_f32), then the output offset applied bytewise
+template <bool DIV2>
+__device__ __forceinline__ uint32_t prob_levels4(const AttentionArgs& a, float p0, float p1, float p2, float p3) {
+    const FqChannel& c = a.fq_p.p;
+    uint32_t w = 0;
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, false>(p0, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 0, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, false>(p1, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 1, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, false>(p2, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 2, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, false>(p3, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 3, w);
+    return a.p_add ? add_bytes(w, a.p_add) : (w ^ a.p_xor);
+}
+
+template <int NT, bool DIV2>   // NT = S / 32 key tiles
+__global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a) {
     constexpr int S = NT * 32;
     constexpr int VT_LD = S + 16;                     // odd number of 16-byte groups per row: conflict-free
     __shared__ __attribute__((aligned(16))) int8_t sK[S * 64];       // [key][d], chunk c of row r in slot c ^ ((r >> 2) & 3)
@@ -103,17 +120,22 @@ __global__ __launch_bounds__(256) void attention_kernel(const AttentionArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) a.scores[dump_row + 32 * t + 8 * (r >> 2) + 4 * h + (r & 3)] = x[t][r];
     }
-    // Softmax over the keys of this lane's query (softmax.hpp: subtract the maximum, exp, sum, divide)
+    // Softmax over the keys of this lane's query (softmax.hpp: subtract the maximum, exp, sum, divide).
+    // exp(x - m) as 2^((x - m) log2 e) on the hardware's exp2, the division as a multiplication by the
+    // reciprocal of the sum: within the tolerance the stand-alone kernel is held to.
     m = fmaxf(m, __shfl_xor(m, 32, 64));
+    constexpr float kLog2e = 1.4426950408889634f;
+    const float mL = -m * kLog2e;
     float s = 0.f;
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            x[t][r] = expf(x[t][r] - m);
+            x[t][r] = __builtin_amdgcn_exp2f(fmaf(x[t][r], kLog2e, mL));
             s += x[t][r];
         }
     s += __shfl_xor(s, 32, 64);
+    const float inv = 1.0f / s;
 
     // probabilities -> i8 levels -> second product, one 32-key tile at a time
     v16i ctx[2] = {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}};
@@ -122,10 +144,10 @@ __global__ __launch_bounds__(256) void attention_kernel(const AttentionArgs a) {
         v4i pf;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            float4 p4 = make_float4(x[t][4 * g] / s, x[t][4 * g + 1] / s, x[t][4 * g + 2] / s, x[t][4 * g + 3] / s);
+            const float4 p4 = make_float4(x[t][4 * g] * inv, x[t][4 * g + 1] * inv, x[t][4 * g + 2] * inv, x[t][4 * g + 3] * inv);
             if (a.probs && q_ok)
                 *reinterpret_cast<float4*>(a.probs + dump_row + 32 * t + 8 * g + 4 * h) = p4;
-            pf[g] = static_cast<int>(requant4(a.fq_p, p4));
+            pf[g] = static_cast<int>(prob_levels4<DIV2>(a, p4.x, p4.y, p4.z, p4.w));
         }
 #pragma unroll
         for (int db = 0; db < 2; ++db) {
@@ -151,8 +173,9 @@ __global__ __launch_bounds__(256) void attention_kernel(const AttentionArgs a) {
 
 template <int NT>
 void launch(const AttentionArgs& a, int batches, hipStream_t s) {
-    hipLaunchKernelGGL(attention_kernel<NT>, dim3(static_cast<uint32_t>(ceil_div(a.S, 128)), static_cast<uint32_t>(batches)),
-                       dim3(256), 0, s, a);
+    const dim3 grid(static_cast<uint32_t>(ceil_div(a.S, 128)), static_cast<uint32_t>(batches));
+    if (a.p_div2) hipLaunchKernelGGL((attention_kernel<NT, true>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((attention_kernel<NT, false>), grid, dim3(256), 0, s, a);
 }
 
 }  // namespace
@@ -160,27 +183,62 @@ void launch(const AttentionArgs& a, int batches, hipStream_t s) {
 
 using namespace hipie;
 
+struct hipie_attention {
+    int device = 0;
+    hipie_attention_desc d{};
+    AttentionArgs proto{};   // everything but the operands
+};
+
 extern "C" {
 
 int hipie_attention_supported(int32_t seq, int32_t head_dim) {
     return seq > 0 && seq % 32 == 0 && seq <= kMaxSeq && head_dim == kHeadDim;
 }
 
-int hipie_attention_run(const hipie_attention_desc* desc, const void* q, int64_t ldq, int64_t stride_q, int64_t outer_q,
+int hipie_attention_create(int device, const hipie_attention_desc* desc, hipie_attention** out) {
+    return guarded([&] {
+        HIPIE_REQUIRE(desc && out, HIPIE_PARAMETER_MISMATCH, "hipie_attention_create: null argument");
+        HIPIE_REQUIRE(hipie_attention_supported(desc->seq, desc->head_dim), HIPIE_NOT_IMPLEMENTED,
+                      "hipie_attention_create: sequence length %d (multiple of 32 up to %d) / head dimension %d (%d)", desc->seq,
+                      kMaxSeq, desc->head_dim, kHeadDim);
+        HIPIE_REQUIRE(desc->out_dtype == HIPIE_I8 || desc->out_dtype == HIPIE_F32, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_attention_create: output type %d", desc->out_dtype);
+        auto att = std::make_unique<hipie_attention>();
+        att->device = device;
+        att->d = *desc;
+        AttentionArgs& a = att->proto;
+        a.S = desc->seq;
+        a.scale1 = desc->score_scale;
+        a.scale2 = desc->context_scale;
+        a.fq_p = make_requant(&desc->prob_fq, "hipie_attention_create (probabilities)");
+        if (desc->out_dtype == HIPIE_I8) a.fq_o = make_requant(&desc->out_fq, "hipie_attention_create (output)");
+        // the probabilities' level index: two-operation division when the device confirms it against IEEE
+        // division for this divisor, else the reciprocal sequence when the host proved it on every level
+        // boundary; a divisor that has neither is left to the separate kernels
+        std::vector<float> zh, zl;
+        a.p_div2 = fq_div2_constants(device, std::vector<float>(1, a.fq_p.p.d), zh, zl) ? 1 : 0;
+        if (a.p_div2) { a.p_zh = zh[0]; a.p_zl = zl[0]; }
+        HIPIE_REQUIRE(a.p_div2 || a.fq_p.rcp || device < 0, HIPIE_NOT_IMPLEMENTED,
+                      "hipie_attention_create: no exact fast division for the probabilities' FakeQuantize range");
+        const int off = static_cast<int>(a.fq_p.p.ol) & 0xff;
+        a.p_xor = off == 0x80 ? 0x80808080u : 0u;
+        a.p_add = (off == 0x80 || off == 0) ? 0u : static_cast<uint32_t>(off) * 0x01010101u;
+        *out = att.release();
+    });
+}
+
+void hipie_attention_destroy(hipie_attention* att) { delete att; }
+
+int hipie_attention_run(const hipie_attention* att, const void* q, int64_t ldq, int64_t stride_q, int64_t outer_q,
                         const void* k, int64_t ldk, int64_t stride_k, int64_t outer_k, const void* v, int64_t ldv,
                         int64_t stride_v, int64_t outer_v, void* out, int64_t ldo, int64_t stride_o, int64_t outer_o,
                         int32_t batch, int32_t batch_outer, float* scores, float* probs, void* stream) {
     return guarded([&] {
-        HIPIE_REQUIRE(desc && q && k && v && out, HIPIE_PARAMETER_MISMATCH, "hipie_attention_run: null argument");
-        HIPIE_REQUIRE(hipie_attention_supported(desc->seq, desc->head_dim), HIPIE_NOT_IMPLEMENTED,
-                      "hipie_attention_run: sequence length %d (multiple of 32 up to %d) / head dimension %d (%d)", desc->seq,
-                      kMaxSeq, desc->head_dim, kHeadDim);
+        HIPIE_REQUIRE(att && q && k && v && out, HIPIE_PARAMETER_MISMATCH, "hipie_attention_run: null argument");
+        HIPIE_REQUIRE(att->device >= 0, HIPIE_NOT_ALLOCATED, "hipie_attention_run: host-only object");
         if (batch == 0 || batch_outer == 0) return;
         HIPIE_REQUIRE(batch > 0 && batch_outer > 0 && static_cast<int64_t>(batch) * batch_outer < 65536, HIPIE_PARAMETER_MISMATCH,
                       "hipie_attention_run: batch %d x %d", batch, batch_outer);
-        const bool byte_out = desc->out_dtype == HIPIE_I8;
-        HIPIE_REQUIRE(byte_out || desc->out_dtype == HIPIE_F32, HIPIE_PARAMETER_MISMATCH, "hipie_attention_run: output type %d",
-                      desc->out_dtype);
         auto aligned = [](const void* p, int64_t a, int64_t b, int64_t c, int64_t g) {
             return reinterpret_cast<uintptr_t>(p) % g == 0 && a % g == 0 && b % g == 0 && c % g == 0;
         };
@@ -189,22 +247,18 @@ int hipie_attention_run(const hipie_attention_desc* desc, const void* q, int64_t
                           aligned(out, ldo, stride_o, outer_o, 4) && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
                           reinterpret_cast<uintptr_t>(probs) % 16 == 0,
                       HIPIE_PARAMETER_MISMATCH, "hipie_attention_run: pitches and strides must keep 16-byte rows aligned");
-        AttentionArgs a{};
+        AttentionArgs a = att->proto;
         a.q = static_cast<const int8_t*>(q); a.k = static_cast<const int8_t*>(k); a.v = static_cast<const int8_t*>(v);
         a.ldq = ldq; a.sq = stride_q; a.oq = outer_q;
         a.ldk = ldk; a.sk = stride_k; a.ok = outer_k;
         a.ldv = ldv; a.sv = stride_v; a.ov = outer_v;
         a.out = out; a.ldo = ldo; a.so = stride_o; a.oo = outer_o;
         a.scores = scores; a.probs = probs;
-        a.S = desc->seq;
         a.batch_inner = batch;
-        a.scale1 = desc->score_scale;
-        a.scale2 = desc->context_scale;
-        a.fq_p = make_requant(&desc->prob_fq, "hipie_attention_run (probabilities)");
-        if (byte_out) a.fq_o = make_requant(&desc->out_fq, "hipie_attention_run (output)");
+        DeviceGuard dg(att->device);
         hipStream_t s = as_stream(stream);
         const int batches = batch * batch_outer;
-        switch (desc->seq / 32) {
+        switch (a.S / 32) {
         case 1: launch<1>(a, batches, s); break;
         case 2: launch<2>(a, batches, s); break;
         case 3: launch<3>(a, batches, s); break;

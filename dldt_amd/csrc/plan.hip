@@ -12,6 +12,7 @@
 #include <mutex>
 
 #include "graph.h"
+#include "requant.h"
 
 namespace hipie {
 namespace {
@@ -498,6 +499,30 @@ struct BatchMatMulStep : Step {
     }
 };
 
+// scores, Softmax, requantisation and context product of one attention block in one kernel
+struct AttentionStep : Step {
+    View q, k, v;
+    int64_t ld[3] = {0, 0, 0}, inner[3] = {0, 0, 0}, outer[3] = {0, 0, 0};
+    int out = -1, scores = -1, probs = -1;
+    int64_t ldo = 0, so = 0, oo = 0;
+    int32_t batch = 1, batch_outer = 1;
+    hipie_attention_desc desc{};
+    hipie_attention* att = nullptr;
+    ~AttentionStep() override { hipie_attention_destroy(att); }
+    void create(int device, const std::vector<TensorInfo>&) override {
+        check_status(hipie_attention_create(device, &desc, &att), name.c_str());
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
+             hipStream_t s) const override {
+        float* sc = scores >= 0 ? reinterpret_cast<float*>(arena + tensors[scores].offset) : nullptr;
+        float* pr = probs >= 0 ? reinterpret_cast<float*>(arena + tensors[probs].offset) : nullptr;
+        check_status(hipie_attention_run(att, q.ptr(arena, tensors, inputs), ld[0], inner[0], outer[0],
+                                         k.ptr(arena, tensors, inputs), ld[1], inner[1], outer[1],
+                                         v.ptr(arena, tensors, inputs), ld[2], inner[2], outer[2], arena + tensors[out].offset,
+                                         ldo, so, oo, batch, batch_outer, sc, pr, s), name.c_str());
+    }
+};
+
 // physical transpose of the two inner dimensions of a byte view (the right operand of a MatMul whose
 // reduction axis is not contiguous)
 struct MatTransposeStep : Step {
@@ -537,10 +562,14 @@ struct Planner {
     // HIPIE_KEEP_F32=1: store the f32 result of Softmax / MVN / Gelu even when only a fused
     // FakeQuantize reads it (inspection of the values behind the tolerance-only operations)
     bool keep_f32 = false;
+    // HIPIE_FUSE_ATTENTION=0: plan the attention core as separate MatMul / Softmax kernels
+    bool fuse_attention = true;
 
     explicit Planner(const hipie_graph& graph) : g(graph), values(graph.nodes.size()), visiting(graph.nodes.size(), 0) {
         const char* k = std::getenv("HIPIE_KEEP_F32");
         keep_f32 = k && k[0] == '1';
+        const char* f = std::getenv("HIPIE_FUSE_ATTENTION");
+        fuse_attention = !(f && f[0] == '0');
     }
 
     const GNode& N(int id) const { return g.nodes[id]; }
@@ -957,6 +986,141 @@ struct Planner {
         outer = r >= 4 ? v.stride[r - 4] : 0;
     }
 
+    // What follows a MatMul between activations: the dequantization Multiply(s_a * s_b), then optionally
+    // a Transpose that keeps the last axis last (the head merge of attention, written through the
+    // output strides), the head-merging Reshape and the next per-tensor FakeQuantize.  Returns the last
+    // absorbed node; oshape is the output tensor's (dense) shape, ostride the strides of the MatMul's
+    // own dimensions inside it.
+    int absorb_matmul_tail(int id, EpilogueSpec& e, std::vector<int64_t>& oshape, std::vector<int64_t>& ostride) {
+        const GNode& n = N(id);
+        const size_t r = n.shape.size();
+        e.out_dtype = HIPIE_F32;
+        int cur = id;
+        oshape = n.shape;
+        ostride = View::dense_strides(oshape);
+        hipie_requant rq{};
+        while (single_user(cur)) {
+            const int nx = N(cur).users[0];
+            const GNode& u = N(nx);
+            std::vector<float> c;
+            if (u.op == OP_MULTIPLY && e.scale.empty() && oshape == n.shape &&
+                last_axis_constant(u.in[0] == cur ? u.in[1] : u.in[0], -1, c)) {
+                e.scale = c;
+            } else if (u.op == OP_TRANSPOSE && u.axes.back() == static_cast<int64_t>(r) - 1 && oshape == n.shape) {
+                oshape = u.shape;
+                const auto ts = View::dense_strides(oshape);
+                for (size_t p = 0; p < r; ++p) ostride[u.axes[p]] = ts[p];
+            } else if (u.op == OP_RESHAPE && !keep_f32 && single_user(nx) && u.shape.back() % oshape.back() == 0 &&
+                       fusable_requant(N(nx).users[0], nx, rq)) {
+                // head merge in front of the FakeQuantize: the output tensor is dense, so the Reshape
+                // only renames its dimensions (the last one must stay a multiple of this MatMul's columns)
+                oshape = u.shape;
+            } else if (!keep_f32 && fusable_requant(nx, cur, rq)) {
+                e.levels = rq.levels;
+                e.fq_il.assign(1, rq.in_low);
+                e.fq_ih.assign(1, rq.in_high);
+                e.fq_ol = rq.out_low;
+                e.fq_oh = rq.out_low + static_cast<float>(rq.levels - 1);
+                e.out_dtype = HIPIE_I8;
+                oshape = u.shape;
+                cur = nx;
+                break;
+            } else {
+                break;
+            }
+            cur = nx;
+        }
+        return cur;
+    }
+
+    // MatMul'(q, k^T) -> Multiply -> Softmax -> FakeQuantize -> MatMul'(., v) -> Multiply [-> ...]: one kernel
+    // when the shapes fit it (hipie_attention_supported) and every link has a single user
+    bool try_plan_attention(int id, const View& qv, const View& kv /* as [.., S, D] */) {
+        const GNode& n = N(id);
+        const size_t r = qv.rank();
+        const int64_t S = qv.shape[r - 2], D = qv.shape[r - 1];
+        if (kv.shape[r - 2] != S || !hipie_attention_supported(static_cast<int32_t>(S), static_cast<int32_t>(D))) return false;
+        if (qv.stride[r - 1] != 1 || kv.stride[r - 1] != 1) return false;
+        if (!single_user(id)) return false;
+        const int mul = n.users[0];
+        std::vector<float> c1;
+        if (N(mul).op != OP_MULTIPLY || !last_axis_constant(N(mul).in[0] == id ? N(mul).in[1] : N(mul).in[0], -1, c1) ||
+            !single_user(mul))
+            return false;
+        const int sm = N(mul).users[0];
+        if (N(sm).op != OP_SOFTMAX || N(sm).axes[0] != static_cast<int64_t>(r) - 1 || !single_user(sm)) return false;
+        const int fq = N(sm).users[0];
+        hipie_requant rq{};
+        if (!fusable_requant(fq, sm, rq) || !single_user(fq)) return false;
+        Requant host_check{};
+        try {
+            host_check = make_requant(&rq, "attention");
+        } catch (...) {
+            return false;
+        }
+        if (!host_check.rcp) return false;   // an exact fast division is known without asking the device
+        const int mm2 = N(fq).users[0];
+        const GNode& m2 = N(mm2);
+        if (m2.op != OP_MATMUL || m2.in[0] != fq || m2.ta || m2.tb || N(m2.in[1]).op == OP_CONSTANT) return false;
+        if (!visit(m2.in[1])) return false;
+        const Value& vval = values[m2.in[1]];
+        if (vval.kind != VK_MAT || vval.view.dtype != HIPIE_I8 || vval.view.rank() != r) return false;
+        const View vv = vval.view;
+        if (vv.shape != qv.shape || vv.stride[r - 1] != 1) return false;
+
+        auto st = std::make_unique<AttentionStep>();
+        EpilogueSpec tail;
+        std::vector<int64_t> oshape, ostride;
+        const int cur = absorb_matmul_tail(mm2, tail, oshape, ostride);
+        if (tail.scale.empty()) return false;
+        st->q = qv; st->k = kv; st->v = vv;
+        st->ld[0] = qv.stride[r - 2]; st->ld[1] = kv.stride[r - 2]; st->ld[2] = vv.stride[r - 2];
+        batch_strides(qv, st->inner[0], st->outer[0]);
+        batch_strides(kv, st->inner[1], st->outer[1]);
+        batch_strides(vv, st->inner[2], st->outer[2]);
+        st->batch = static_cast<int32_t>(qv.shape[r - 3]);
+        st->batch_outer = r == 4 ? static_cast<int32_t>(qv.shape[0]) : 1;
+        hipie_attention_desc& d = st->desc;
+        d.seq = static_cast<int32_t>(S);
+        d.head_dim = static_cast<int32_t>(D);
+        d.score_scale = c1[0];
+        d.context_scale = tail.scale[0];
+        d.prob_fq = rq;
+        d.out_dtype = tail.out_dtype;
+        if (tail.out_dtype == HIPIE_I8) {
+            d.out_fq.in_low = tail.fq_il[0];
+            d.out_fq.in_high = tail.fq_ih[0];
+            d.out_fq.out_low = tail.fq_ol;
+            d.out_fq.levels = tail.levels;
+        }
+        // everything between the two products lives in registers; with HIPIE_KEEP_F32 the kernel also
+        // writes the values in front of and behind the Softmax
+        values[id].kind = VK_FUSED;
+        values[fq].kind = VK_FUSED;
+        if (keep_f32) {
+            st->scores = new_matrix(mul, HIPIE_F32, N(mul).shape);
+            set_matrix_value(mul, st->scores, HIPIE_F32);
+            st->probs = new_matrix(sm, HIPIE_F32, N(sm).shape);
+            set_matrix_value(sm, st->probs, HIPIE_F32);
+        } else {
+            values[mul].kind = VK_FUSED;
+            values[sm].kind = VK_FUSED;
+        }
+        mark_chain(mm2, cur);
+        st->out = new_matrix(cur, tail.out_dtype, oshape);
+        st->ldo = ostride[r - 2];
+        st->so = ostride[r - 3];
+        st->oo = r == 4 ? ostride[0] : 0;
+        st->name = N(cur).name;
+        st->type = "Attention";
+        st->macs = 2 * n.numel() * D;
+        st->bytes = qv.numel() + kv.numel() + vv.numel() + m2.numel() * (tail.out_dtype == HIPIE_F32 ? 4 : 1);
+        st->out_node = cur;
+        set_matrix_value(cur, st->out, tail.out_dtype);
+        steps.push_back(std::move(st));
+        return true;
+    }
+
     void plan_batch_matmul(int id, const View& av) {
         const GNode& n = N(id);
         const Value bval = value(n.in[1]);
@@ -975,6 +1139,7 @@ struct Planner {
             if (av.shape[i] != bv.shape[i]) unsupported(id, "broadcast batch dimensions");
         if (av.stride[r - 1] != 1) unsupported(id, "left operand with a strided reduction axis");
         if (K % 64 != 0) unsupported(id, "reduction length must be a multiple of 64");
+        if (fuse_attention && M == Nn && try_plan_attention(id, av, bv)) return;
         const int32_t inner = static_cast<int32_t>(av.shape[r - 3]), outer = r == 4 ? static_cast<int32_t>(av.shape[0]) : 1;
         if (bv.stride[r - 1] != 1) {
             // reduction axis not contiguous: transpose the operand's inner dimensions into a new tensor
@@ -1016,45 +1181,9 @@ struct Planner {
         batch_strides(av, st->sa, st->oa);
         st->ldb = bv.stride[r - 2];
         batch_strides(bv, st->sb, st->ob);
-        // epilogue: the dequantization Multiply(s_a * s_b), then optionally a Transpose that keeps the
-        // last axis last (the head merge of attention), written through the output strides
         EpilogueSpec& e = st->epi;
-        e.out_dtype = HIPIE_F32;
-        int cur = id;
-        std::vector<int64_t> oshape = n.shape;
-        std::vector<int64_t> ostride = View::dense_strides(oshape);   // of the MatMul's own dimensions
-        hipie_requant rq{};
-        while (single_user(cur)) {
-            const int nx = N(cur).users[0];
-            const GNode& u = N(nx);
-            std::vector<float> c;
-            if (u.op == OP_MULTIPLY && e.scale.empty() &&
-                last_axis_constant(u.in[0] == cur ? u.in[1] : u.in[0], -1, c)) {
-                e.scale = c;
-            } else if (u.op == OP_TRANSPOSE && u.axes.back() == static_cast<int64_t>(r) - 1 && oshape == n.shape) {
-                oshape = u.shape;
-                const auto ts = View::dense_strides(oshape);
-                for (size_t p = 0; p < r; ++p) ostride[u.axes[p]] = ts[p];
-            } else if (u.op == OP_RESHAPE && !keep_f32 && single_user(nx) && u.shape.back() % oshape.back() == 0 &&
-                       fusable_requant(N(nx).users[0], nx, rq)) {
-                // head merge in front of the FakeQuantize: the output tensor is dense, so the Reshape
-                // only renames its dimensions (the last one must stay a multiple of this MatMul's columns)
-                oshape = u.shape;
-            } else if (!keep_f32 && fusable_requant(nx, cur, rq)) {
-                e.levels = rq.levels;
-                e.fq_il.assign(1, rq.in_low);
-                e.fq_ih.assign(1, rq.in_high);
-                e.fq_ol = rq.out_low;
-                e.fq_oh = rq.out_low + static_cast<float>(rq.levels - 1);
-                e.out_dtype = HIPIE_I8;
-                oshape = u.shape;
-                cur = nx;
-                break;
-            } else {
-                break;
-            }
-            cur = nx;
-        }
+        std::vector<int64_t> oshape, ostride;
+        const int cur = absorb_matmul_tail(id, e, oshape, ostride);
         mark_chain(id, cur);
         st->out = new_matrix(cur, e.out_dtype, oshape);
         st->ldo = ostride[r - 2];

@@ -316,30 +316,50 @@ class hipie_attention_desc(ctypes.Structure):
                 ("out_fq", hipie_requant)]
 
 
+class Attention:
+    """Fused attention core (hipie_attention_*): MatMul'(q, k^T) * score_scale -> Softmax ->
+    FakeQuantize(prob_fq) -> MatMul'(., v) * context_scale [-> FakeQuantize(out_fq)].
+    prob_fq / out_fq = (in_low, in_high, out_low, levels)."""
+
+    def __init__(self, seq, head_dim, score_scale, context_scale, prob_fq, out_fq=None, device=0):
+        d = hipie_attention_desc()
+        d.seq, d.head_dim = seq, head_dim
+        d.score_scale, d.context_scale = float(score_scale), float(context_scale)
+        d.prob_fq = hipie_requant(*[float(x) for x in prob_fq[:3]], int(prob_fq[3]))
+        d.out_dtype = I8 if out_fq is not None else F32
+        if out_fq is not None:
+            d.out_fq = hipie_requant(*[float(x) for x in out_fq[:3]], int(out_fq[3]))
+        self.byte_out = out_fq is not None
+        self._h = ctypes.c_void_p()
+        check(lib().hipie_attention_create(ctypes.c_int(device), ctypes.byref(d), ctypes.byref(self._h)))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().hipie_attention_destroy(self._h)
+            self._h = None
+
+    def run(self, q, k, v, dump=False, out=None):
+        """q, k, v: i8 [B, NH, S, 64] (any strides with contiguous rows).  Returns the context
+        [B, NH, S, 64] and, with dump=True, also the f32 scores and probabilities [B, NH, S, S]."""
+        import torch
+        B, NH, S, D = q.shape
+        assert k.shape == q.shape and v.shape == q.shape and q.dtype == torch.int8
+        for t in (q, k, v):
+            assert t.stride(3) == 1
+        if out is None:
+            out = torch.empty((B, NH, S, D), dtype=torch.int8 if self.byte_out else torch.float32, device=q.device)
+        scores = torch.empty((B, NH, S, S), dtype=torch.float32, device=q.device) if dump else None
+        probs = torch.empty_like(scores) if dump else None
+        i64 = ctypes.c_int64
+        args = []
+        for t in (q, k, v, out):
+            args += [_dptr(t), i64(t.stride(2)), i64(t.stride(1)), i64(t.stride(0))]
+        check(lib().hipie_attention_run(self._h, *args, ctypes.c_int32(NH), ctypes.c_int32(B),
+                                        _dptr(scores) if dump else None, _dptr(probs) if dump else None, _stream()))
+        return (out, scores, probs) if dump else out
+
+
 def attention(q, k, v, score_scale, context_scale, prob_fq, out_fq=None, dump=False):
-    """Fused attention core over i8 tensors [B, NH, S, 64] (any strides with contiguous rows):
-    returns the context [B, NH, S, 64] (f32, or i8 when out_fq is given) and, with dump=True, also the
-    f32 scores and probabilities [B, NH, S, S].  prob_fq / out_fq = (in_low, in_high, out_low, levels)."""
-    import torch
-    B, NH, S, D = q.shape
-    assert k.shape == q.shape and v.shape == q.shape and q.dtype == torch.int8
-    for t in (q, k, v):
-        assert t.stride(3) == 1
-    d = hipie_attention_desc()
-    d.seq, d.head_dim = S, D
-    d.score_scale, d.context_scale = float(score_scale), float(context_scale)
-    d.prob_fq = hipie_requant(*[float(x) for x in prob_fq[:3]], int(prob_fq[3]))
-    d.out_dtype = I8 if out_fq is not None else F32
-    if out_fq is not None:
-        d.out_fq = hipie_requant(*[float(x) for x in out_fq[:3]], int(out_fq[3]))
-    out = torch.empty((B, NH, S, D), dtype=torch.int8 if out_fq is not None else torch.float32, device=q.device)
-    scores = torch.empty((B, NH, S, S), dtype=torch.float32, device=q.device) if dump else None
-    probs = torch.empty_like(scores) if dump else None
-    i64 = ctypes.c_int64
-    args = []
-    for t in (q, k, v):
-        args += [_dptr(t), i64(t.stride(2)), i64(t.stride(1)), i64(t.stride(0))]
-    check(lib().hipie_attention_run(ctypes.byref(d), *args, _dptr(out), i64(out.stride(2)), i64(out.stride(1)),
-                                    i64(out.stride(0)), ctypes.c_int32(NH), ctypes.c_int32(B),
-                                    _dptr(scores) if dump else None, _dptr(probs) if dump else None, _stream()))
-    return (out, scores, probs) if dump else out
+    """One-shot form of Attention (creates the load-time object for this call)."""
+    att = Attention(q.shape[2], q.shape[3], score_scale, context_scale, prob_fq, out_fq, q.device.index or 0)
+    return att.run(q, k, v, dump=dump)

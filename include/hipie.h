@@ -292,8 +292,12 @@ typedef struct hipie_attention_desc {
     int32_t out_dtype;          /* HIPIE_F32 or HIPIE_I8 */
     hipie_requant out_fq;       /* used when out_dtype is HIPIE_I8 */
 } hipie_attention_desc;
+typedef struct hipie_attention hipie_attention;
 int hipie_attention_supported(int32_t seq, int32_t head_dim);
-int hipie_attention_run(const hipie_attention_desc* desc, const void* q, int64_t ldq, int64_t stride_q, int64_t outer_q,
+/* device < 0 builds a host-only object (load-time checks without a GPU) */
+int hipie_attention_create(int device, const hipie_attention_desc* desc, hipie_attention** attention);
+void hipie_attention_destroy(hipie_attention* attention);
+int hipie_attention_run(const hipie_attention* attention, const void* q, int64_t ldq, int64_t stride_q, int64_t outer_q,
                         const void* k, int64_t ldk, int64_t stride_k, int64_t outer_k, const void* v, int64_t ldv,
                         int64_t stride_v, int64_t outer_v, void* out, int64_t ldo, int64_t stride_o, int64_t outer_o,
                         int32_t batch, int32_t batch_outer, float* scores, float* probs, void* stream);

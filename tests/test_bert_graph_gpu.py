@@ -18,8 +18,9 @@ GLUE_TOL = dict(p=dict(rtol=2e-6, atol=1e-8), h1=dict(rtol=1e-5, atol=4e-6), gel
                 y=dict(rtol=1e-5, atol=4e-6))
 
 
-def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq):
+def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq, fuse_attention=True):
     from dldt_amd import builders
+    monkeypatch.setenv("HIPIE_FUSE_ATTENTION", "1" if fuse_attention else "0")
     # first with every f32 value behind a tolerance-only op kept in the arena (segment-wise check) ...
     monkeypatch.setenv("HIPIE_KEEP_F32", "1")
     # ranges for the reduced width: about 30 levels per standard deviation, so the tails saturate
@@ -28,15 +29,21 @@ def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq):
     x = np.random.default_rng(70).normal(0, 1, (batch, seq, hidden)).astype(np.float32)
     plan = g.compile()
     types = [s["type"] for s in plan.steps]
-    assert types.count("MatMul") == 8 * layers and types.count("Transpose") == layers
-    assert types.count("Softmax+FakeQuantize") == layers and types.count("Gelu+FakeQuantize") == layers
+    if fuse_attention:      # the probabilities stay in registers between the two products
+        assert types.count("MatMul") == 6 * layers and types.count("Attention") == layers
+        assert "Transpose" not in types and "Softmax+FakeQuantize" not in types
+    else:
+        assert types.count("MatMul") == 8 * layers and types.count("Transpose") == layers
+        assert types.count("Softmax+FakeQuantize") == layers
+    assert types.count("Gelu+FakeQuantize") == layers
+    exact = [n for n in EXACT if not (fuse_attention and n == "pq")]
     req = plan.create_request()
     (y,) = req.infer(x)
     device = {n: req.matrix(n) for n in meta["glue"]}
     keep = [n for L in meta["layers"] for n in L.values()]
     want, kept = evaluate(orc, g.nodes, {"hidden_states": x}, keep=keep, override=device)
     for li, L in enumerate(meta["layers"]):
-        for name in EXACT:
+        for name in exact:
             w = kept[L[name]]
             have = req.matrix(L[name]).reshape(w.shape)
             if w.dtype == np.float32:
@@ -58,9 +65,10 @@ def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq):
     (y2,) = req2.infer(x)
     np.testing.assert_array_equal(y2.view(np.uint32), y.view(np.uint32))
     for li, L in enumerate(meta["layers"]):
-        for name in ("q", "k", "v", "scores", "pq", "ctxq", "attn", "h1q", "up", "gq", "down"):
+        stored = ("q", "k", "v", "ctxq", "attn", "h1q", "up", "gq", "down") + (() if fuse_attention else ("scores", "pq"))
+        for name in stored:
             np.testing.assert_array_equal(req2.matrix(L[name]), req.matrix(L[name]), err_msg="layer %d %s" % (li, name))
-        for name in ("p", "ctx", "gelu"):
+        for name in ("p", "ctx", "gelu") + (("scores", "pq") if fuse_attention else ()):
             with pytest.raises(Exception):
                 req2.matrix(L[name])
     return plan2, req2, x, y
@@ -79,6 +87,12 @@ def test_encoder_stack_matches_the_oracle(orc, monkeypatch):
 def test_encoder_stack_other_head_count_and_ragged_rows(orc, monkeypatch):
     """three heads, a sequence length that is not a multiple of the 128-row tiles"""
     _check_stack(orc, monkeypatch, layers=1, hidden=192, heads=3, ffn=320, batch=3, seq=64)
+
+
+def test_encoder_stack_with_separate_attention_kernels(orc, monkeypatch):
+    """the same graph with the attention core planned as MatMul, Softmax + FakeQuantize, Transpose, MatMul"""
+    _check_stack(orc, monkeypatch, layers=2, hidden=128, heads=2, ffn=256, batch=2, seq=128, fuse_attention=False)
+    _check_stack(orc, monkeypatch, layers=1, hidden=192, heads=3, ffn=320, batch=3, seq=64, fuse_attention=False)
 
 
 def test_unsupported_transformer_nodes_are_reported():

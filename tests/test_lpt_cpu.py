@@ -110,7 +110,7 @@ def test_full_size_mac_counts_match_the_published_architecture():
     assert 0.29e9 < builders.mobilenet_v2(batch=1, res=224)[1]["macs_per_image"] < 0.32e9
 
 
-def test_planner_encoder_stack_steps_and_views():
+def test_planner_encoder_stack_steps_and_views(monkeypatch):
     """BERT-style encoder: head split / merge are views (no step), the V operand gets one physical
     transpose, LayerNorm's Multiply and Add and the next FakeQuantize ride in the MVN step, and the published operation count of
     config 5 comes out: 565.3 GMAC for 12 layers at batch 16 x 384 tokens."""
@@ -119,11 +119,14 @@ def test_planner_encoder_stack_steps_and_views():
     g, meta = builders.bert_encoder(layers=2, hidden=128, heads=2, ffn=256, batch=2, seq=128, seed=7)
     plan = Plan(g, device=-1)
     types = [s["type"] for s in plan.steps]
-    attention = ["MatMul", "MatMul", "MatMul", "Softmax+FakeQuantize", "MatMul", "Transpose", "MatMul", "MatMul"]
+    attention = ["MatMul", "MatMul", "MatMul", "Attention", "MatMul"]
     ffn = ["MVN+FakeQuantize", "MatMul", "Gelu+FakeQuantize", "MatMul"]
     # every activation FakeQuantize but the first rides in the kernel that produces its input
     assert types == ["FakeQuantize"] + attention + ffn + ["MVN+FakeQuantize"] + attention + ffn + ["MVN", "Result"]
     assert sum(s["macs"] for s in plan.steps) == meta["macs"]
+    monkeypatch.setenv("HIPIE_FUSE_ATTENTION", "0")       # separate kernels: V gets one physical transpose
+    types = [s["type"] for s in Plan(g, device=-1).steps]
+    assert types[3:8] == ["MatMul", "Softmax+FakeQuantize", "MatMul", "Transpose", "MatMul"]
     T, H, FF = 16 * 384, 768, 3072
     assert 12 * (T * (4 * H * H + 2 * H * FF) + 2 * 16 * 12 * 384 * 384 * 64) == 565_325_070_336
 
