@@ -222,7 +222,16 @@ def config5():
     gamma, beta = torch.ones(H, device="cuda"), torch.zeros(H, device="cuda")
     glue("LayerNorm (MVN, gamma, beta)", lambda t: mvn(t, gamma=gamma, beta=beta), torch.randn((T, H), device="cuda"), 2)
     glue("GELU (erf)", gelu, torch.randn((T, FF), device="cuda"), 2)
-    r = _row("cfg5 one encoder layer, sum of the kernels above (LayerNorm twice)", layer_us,
+    # the attention core in one kernel: scores, softmax, requantisation, context (heads sliced out of [T, 3H])
+    from .ops import Attention
+    qkv = torch.randint(-128, 128, (B, S, 3, NH, 64), dtype=torch.int8, device="cuda")
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    att = Attention(S, 64, 0.0007, 0.02 / 127, (-128.0 / 127, 1.0, -128, 256), out_fq=(-0.5, 0.5 * 127 / 128, -128, 256))
+    ctx = torch.empty((B, NH, S, 64), dtype=torch.int8, device="cuda")
+    us = _time(lambda: att.run(q, k, v, out=ctx), reps=10, warm=3)
+    rows.append(_row("cfg5 fused attention %dx[%d,64]: scores, softmax, FakeQuantize, context -> i8" % (B * NH, S), us,
+                     macs=2 * B * NH * S * S * 64, bytes_=4 * B * NH * S * 64))
+    r = _row("cfg5 one encoder layer, sum of the separate kernels above (LayerNorm twice)", layer_us,
              macs=T * (4 * H * H + 2 * H * FF) + 2 * B * NH * S * S * 64, bound="mfma")
     r["sequences/s (12 layers, these kernels only)"] = B / (12 * layer_us) * 1e6
     rows.append(r)
