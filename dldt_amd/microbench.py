@@ -2,6 +2,7 @@
 """Kernel timings at the shapes of the five benchmark configurations, against each kernel's roofline.
 
     python -m dldt_amd.microbench            # all rows, markdown table on stdout
+    python -m dldt_amd.microbench encoder    # only the 12-layer encoder graph of config 5
 
 Rows: config 1 (one quantized 3x3 convolution block, batch 1), config 2 (per-channel FakeQuantize of
 [32,256,56,56]), config 3 (ResNet-50 v1.5 INT8, batch 1 and 64), config 4 (MobileNetV2 INT8, batch 64:
@@ -244,8 +245,14 @@ def config5():
     r["sequences/s (12 layers)"] = B / (12 * us) * 1e6
     rows.append(r)
     del layer
-    # the 12-layer encoder as a post-LPT graph through the planner (graph-level C ABI)
+    return rows + config5_graph()
+
+
+def config5_graph():
+    """the 12-layer encoder as a post-LPT graph through the planner (graph-level C ABI)"""
     from . import builders
+    B, S, H, NH, FF = 16, 384, 768, 12, 3072
+    rows = []
     g, meta = builders.bert_encoder(layers=12, hidden=H, heads=NH, ffn=FF, batch=B, seq=S)
     us, plan = _graph_time(g, reps=5, warm=2)
     r = _row("cfg5 BERT-base encoder, 12 layers, batch %d x %d tokens, one request (%d launches)" % (B, S, len(plan.steps)),
@@ -264,7 +271,7 @@ def main():
     import torch
     assert torch.cuda.is_available(), "microbench needs a GPU"
     which = sys.argv[1:] or ["1", "2", "3", "4", "5"]
-    table = {"1": config1, "2": config2, "3": config3, "4": config4, "5": config5}
+    table = {"1": config1, "2": config2, "3": config3, "4": config4, "5": config5, "encoder": config5_graph}
     print("| kernel / graph | us | TOP/s | GB/s | bound | fraction of peak | notes |")
     print("|---|---|---|---|---|---|---|")
     for k in which:
