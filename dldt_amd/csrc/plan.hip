@@ -564,12 +564,16 @@ struct Planner {
     bool keep_f32 = false;
     // HIPIE_FUSE_ATTENTION=0: plan the attention core as separate MatMul / Softmax kernels
     bool fuse_attention = true;
+    // HIPIE_MERGE_LINEAR=0: one GEMM per MatMul node even when several share their input
+    bool merge_linear = true;
 
     explicit Planner(const hipie_graph& graph) : g(graph), values(graph.nodes.size()), visiting(graph.nodes.size(), 0) {
         const char* k = std::getenv("HIPIE_KEEP_F32");
         keep_f32 = k && k[0] == '1';
         const char* f = std::getenv("HIPIE_FUSE_ATTENTION");
         fuse_attention = !(f && f[0] == '0');
+        const char* ml = std::getenv("HIPIE_MERGE_LINEAR");
+        merge_linear = !(ml && ml[0] == '0');
     }
 
     const GNode& N(int id) const { return g.nodes[id]; }
@@ -898,34 +902,16 @@ struct Planner {
     }
 
     // MatMul against constant i8 weights: a 1x1 convolution over [rows, K]
-    void plan_linear(int id, const View& av) {
-        const GNode& n = N(id);
-        const GNode& W = N(n.in[1]);
-        if (W.dtype != HIPIE_I8 || W.shape.size() != 2) unsupported(id, "weights must be a rank-2 i8 constant");
-        if (!av.dense() || av.tensor < 0 || av.offset != 0) unsupported(id, "left operand must be a whole dense tensor");
-        const int64_t IC = n.tb ? W.shape[1] : W.shape[0], OC = n.tb ? W.shape[0] : W.shape[1];
-        HIPIE_REQUIRE(av.shape.back() == IC, HIPIE_PARAMETER_MISMATCH, "node %d: inner dimensions %lld vs %lld", id,
-                      (long long)av.shape.back(), (long long)IC);
-        const int64_t T = av.numel() / IC;
-        auto st = std::make_unique<ConvStep>();
-        st->in = av.tensor;
-        if (tensors[av.tensor].w != T || tensors[av.tensor].c != IC) {   // same bytes, other row split
-            if (IC % 16 != 0) unsupported(id, "reduction length must be a multiple of 16");
-            st->in = new_tensor(tensors[av.tensor].producer, HIPIE_I8, 1, 1, static_cast<int>(T), static_cast<int>(IC),
-                                static_cast<int>(IC));
-            tensors[st->in].alias = av.tensor;
-        }
-        hipie_conv_desc& d = st->desc;
-        d.groups = 1;
-        d.kh = d.kw = d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1;
-        d.ic = static_cast<int>(IC);
-        d.oc = static_cast<int>(OC);
-        st->weights.resize(OC * IC);
-        const int8_t* w = reinterpret_cast<const int8_t*>(W.data.data());
-        for (int64_t o = 0; o < OC; ++o)
-            for (int64_t k = 0; k < IC; ++k) st->weights[o * IC + k] = n.tb ? w[o * IC + k] : w[k * OC + o];
+    // the elementwise chain behind a MatMul against constant weights
+    struct LinearChain {
+        EpilogueSpec e;
+        int cur = -1, res = -1, res_param = -1;
+        bool residual = false;
+    };
 
-        EpilogueSpec& e = st->epi;
+    LinearChain parse_linear_chain(int id, int64_t OC, int64_t T) {
+        LinearChain ch;
+        EpilogueSpec& e = ch.e;
         int cur = id, stage = 0;
         while (single_user(cur)) {
             const int nx = N(cur).users[0];
@@ -945,8 +931,9 @@ struct Planner {
                         break;
                     if (r.view.tensor >= 0 && (tensors[r.view.tensor].w != T || tensors[r.view.tensor].c != OC)) break;
                     e.residual_dtype = HIPIE_F32;
-                    st->res = r.view.tensor;
-                    st->res_param = r.view.param;
+                    ch.res = r.view.tensor;
+                    ch.res_param = r.view.param;
+                    ch.residual = true;
                     stage = 3;
                 } else {
                     break;
@@ -967,15 +954,123 @@ struct Planner {
             }
             cur = nx;
         }
-        mark_chain(id, cur);
-        st->out = new_matrix(cur, e.out_dtype, N(cur).shape);
-        st->name = N(cur).name;
+        ch.cur = cur;
+        return ch;
+    }
+
+    static void append_rows(std::vector<int8_t>& dst, const GNode& W, bool tb, int64_t OC, int64_t IC) {
+        const int8_t* w = reinterpret_cast<const int8_t*>(W.data.data());
+        const size_t base = dst.size();
+        dst.resize(base + static_cast<size_t>(OC * IC));
+        for (int64_t o = 0; o < OC; ++o)
+            for (int64_t k = 0; k < IC; ++k) dst[base + o * IC + k] = tb ? w[o * IC + k] : w[k * OC + o];
+    }
+
+    static void append_expanded(std::vector<float>& dst, const std::vector<float>& v, int64_t n) {
+        for (int64_t i = 0; i < n; ++i) dst.push_back(v[v.size() == 1 ? 0 : static_cast<size_t>(i)]);
+    }
+
+    // MatMul against constant i8 weights: a 1x1 convolution over [rows, K].  MatMuls that read the same
+    // activation and end in the same kind of requantisation (the Q, K, V projections of an attention
+    // block) become ONE GEMM over their concatenated output channels; each one's value is then a
+    // column slice of the shared output tensor.
+    void plan_linear(int id, const View& av) {
+        const GNode& n = N(id);
+        const GNode& W = N(n.in[1]);
+        if (W.dtype != HIPIE_I8 || W.shape.size() != 2) unsupported(id, "weights must be a rank-2 i8 constant");
+        if (!av.dense() || av.tensor < 0 || av.offset != 0) unsupported(id, "left operand must be a whole dense tensor");
+        const int64_t IC = n.tb ? W.shape[1] : W.shape[0], OC = n.tb ? W.shape[0] : W.shape[1];
+        HIPIE_REQUIRE(av.shape.back() == IC, HIPIE_PARAMETER_MISMATCH, "node %d: inner dimensions %lld vs %lld", id,
+                      (long long)av.shape.back(), (long long)IC);
+        const int64_t T = av.numel() / IC;
+        auto st = std::make_unique<ConvStep>();
+        st->in = av.tensor;
+        if (tensors[av.tensor].w != T || tensors[av.tensor].c != IC) {   // same bytes, other row split
+            if (IC % 16 != 0) unsupported(id, "reduction length must be a multiple of 16");
+            st->in = new_tensor(tensors[av.tensor].producer, HIPIE_I8, 1, 1, static_cast<int>(T), static_cast<int>(IC),
+                                static_cast<int>(IC));
+            tensors[st->in].alias = av.tensor;
+        }
+        LinearChain ch = parse_linear_chain(id, OC, T);
+
+        // siblings to merge with: unplanned MatMuls on the same activation whose chains look the same
+        std::vector<int> group(1, id);
+        std::vector<LinearChain> chains(1, ch);
+        std::vector<int64_t> ocs(1, OC);
+        auto mergeable = [](const LinearChain& c) {
+            return !c.residual && c.e.out_dtype == HIPIE_I8 && !c.e.bias.empty() && c.e.scale.empty();
+        };
+        if (merge_linear && mergeable(ch) && OC % 16 == 0) {
+            for (int u : N(n.in[0]).users) {
+                const GNode& m = N(u);
+                if (u == id || values[u].kind != VK_NONE || m.op != OP_MATMUL || m.in[0] != n.in[0] || m.ta || m.tb != n.tb) continue;
+                const GNode& W2 = N(m.in[1]);
+                if (W2.op != OP_CONSTANT || W2.dtype != HIPIE_I8 || W2.shape.size() != 2) continue;
+                const int64_t ic2 = m.tb ? W2.shape[1] : W2.shape[0], oc2 = m.tb ? W2.shape[0] : W2.shape[1];
+                if (ic2 != IC || oc2 % 16 != 0 || m.shape.size() != n.shape.size()) continue;
+                LinearChain c2 = parse_linear_chain(u, oc2, T);
+                if (!mergeable(c2) || c2.e.levels != ch.e.levels || c2.e.fq_ol != ch.e.fq_ol || c2.e.fq_oh != ch.e.fq_oh) continue;
+                group.push_back(u);
+                chains.push_back(std::move(c2));
+                ocs.push_back(oc2);
+            }
+        }
+        int64_t OCt = 0;
+        for (auto o : ocs) OCt += o;
+        hipie_conv_desc& d = st->desc;
+        d.groups = 1;
+        d.kh = d.kw = d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1;
+        d.ic = static_cast<int>(IC);
+        d.oc = static_cast<int>(OCt);
+        EpilogueSpec& e = st->epi;
+        if (group.size() == 1) {
+            e = ch.e;
+            append_rows(st->weights, W, n.tb, OC, IC);
+        } else {
+            e.out_dtype = HIPIE_I8;
+            e.levels = ch.e.levels;
+            e.fq_ol = ch.e.fq_ol;
+            e.fq_oh = ch.e.fq_oh;
+            for (size_t i = 0; i < group.size(); ++i) {
+                append_rows(st->weights, N(N(group[i]).in[1]), n.tb, ocs[i], IC);
+                append_expanded(e.bias, chains[i].e.bias, ocs[i]);
+                append_expanded(e.fq_il, chains[i].e.fq_il, ocs[i]);
+                append_expanded(e.fq_ih, chains[i].e.fq_ih, ocs[i]);
+            }
+        }
+        st->res = ch.res;
+        st->res_param = ch.res_param;
+        for (size_t i = 0; i < group.size(); ++i) mark_chain(group[i], chains[i].cur);
+        std::vector<int64_t> oshape = N(ch.cur).shape;
+        oshape.back() = OCt;
+        st->out = new_matrix(ch.cur, e.out_dtype, oshape);
+        st->name = N(ch.cur).name + (group.size() > 1 ? " (+" + std::to_string(group.size() - 1) + " sharing the input)" : "");
         st->type = "MatMul";
-        st->macs = T * OC * IC;
-        st->in_w_bytes = T * IC + OC * IC;
-        st->bytes = st->in_w_bytes + T * OC * (e.out_dtype == HIPIE_F32 ? 4 : 1) + (stage == 3 ? T * OC * 4 : 0);
-        st->out_node = cur;
-        set_matrix_value(cur, st->out, e.out_dtype);
+        st->macs = T * OCt * IC;
+        st->in_w_bytes = T * IC + OCt * IC;
+        st->bytes = st->in_w_bytes + T * OCt * (e.out_dtype == HIPIE_F32 ? 4 : 1) + (ch.residual ? T * OCt * 4 : 0);
+        st->out_node = ch.cur;
+        if (group.size() == 1) {
+            set_matrix_value(ch.cur, st->out, e.out_dtype);
+        } else {
+            int64_t col = 0;
+            for (size_t i = 0; i < group.size(); ++i) {   // column slice [.., ocs[i]] at `col` of [.., OCt]
+                View v;
+                v.tensor = st->out;
+                v.dtype = e.out_dtype;
+                v.shape = N(chains[i].cur).shape;
+                v.stride.assign(v.shape.size(), 1);
+                int64_t pitch = OCt;
+                for (size_t k = v.shape.size() - 1; k-- > 0;) {
+                    v.stride[k] = pitch;
+                    pitch *= v.shape[k];
+                }
+                v.offset = col;
+                col += ocs[i];
+                values[chains[i].cur].kind = VK_MAT;
+                values[chains[i].cur].view = v;
+            }
+        }
         steps.push_back(std::move(st));
     }
 
@@ -1529,6 +1624,8 @@ struct hipie_plan {
     std::vector<TensorInfo> tensors;
     std::vector<std::unique_ptr<Step>> steps;
     std::map<int, int> node_tensor;          // graph node -> tensor holding its value
+    struct Slice { int tensor; int64_t offset, rows, cols, pitch; };
+    std::map<int, Slice> node_slice;         // graph node -> rows x cols window of a tensor (row-major views)
     int64_t arena_bytes = 0;
     struct Io { std::string name; int dtype; std::vector<int64_t> shape; int64_t bytes; };
     std::vector<Io> inputs, outputs;
@@ -1597,11 +1694,15 @@ int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
         for (size_t i = 0; i < pl.values.size(); ++i)
             if (pl.values[i].kind == VK_TENSOR) {
                 plan->node_tensor[static_cast<int>(i)] = pl.values[i].tensor;
-            } else if (pl.values[i].kind == VK_MAT) {   // a dense view that is its whole tensor
+            } else if (pl.values[i].kind == VK_MAT) {   // a view that is [rows, cols] with one row pitch
                 const View& v = pl.values[i].view;
-                if (v.tensor >= 0 && v.offset == 0 && v.dense() &&
-                    v.numel() == static_cast<int64_t>(pl.tensors[v.tensor].w) * pl.tensors[v.tensor].c)
-                    plan->node_tensor[static_cast<int>(i)] = v.tensor;
+                const size_t r = v.rank();
+                bool ok = v.tensor >= 0 && r >= 1 && v.stride[r - 1] == 1;
+                for (size_t k = 0; ok && k + 2 < r; ++k) ok = v.stride[k] == v.stride[k + 1] * v.shape[k + 1];
+                if (ok) {
+                    const int64_t cols = v.shape[r - 1], rows = v.numel() / cols;
+                    plan->node_slice[static_cast<int>(i)] = {v.tensor, v.offset, rows, cols, r >= 2 ? v.stride[r - 2] : cols};
+                }
             }
         for (int p : g->params) {
             const GNode& n = g->nodes[p];
@@ -1826,6 +1927,20 @@ int hipie_request_perf(hipie_request* r, int step, float* ms) {
 int hipie_request_tensor(const hipie_request* r, int node_id, hipie_tensor* t) {
     return guarded([&] {
         HIPIE_REQUIRE(r && t, HIPIE_PARAMETER_MISMATCH, "hipie_request_tensor: null argument");
+        auto sl = r->plan->node_slice.find(node_id);
+        if (sl != r->plan->node_slice.end()) {   // row-major value: n = h = 1, w = rows, c = columns
+            const hipie_plan::Slice& v = sl->second;
+            const TensorInfo& ti = r->plan->tensors[v.tensor];
+            t->dtype = ti.dtype;
+            t->n = t->h = 1;
+            t->w = static_cast<int32_t>(v.rows);
+            t->c = static_cast<int32_t>(v.cols);
+            t->stride_w = v.pitch;
+            t->stride_h = t->stride_n = v.pitch * v.rows;
+            t->halo = 0;
+            t->data = r->arena.as<uint8_t>() + ti.offset + v.offset * ti.esize();
+            return;
+        }
         auto it = r->plan->node_tensor.find(node_id);
         HIPIE_REQUIRE(it != r->plan->node_tensor.end(), HIPIE_NOT_FOUND,
                       "hipie_request_tensor: node %d was fused away or is not a tensor", node_id);

@@ -18,9 +18,11 @@ GLUE_TOL = dict(p=dict(rtol=2e-6, atol=1e-8), h1=dict(rtol=1e-5, atol=4e-6), gel
                 y=dict(rtol=1e-5, atol=4e-6))
 
 
-def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq, fuse_attention=True):
+def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq, fuse_attention=True, merge_linear=True):
     from dldt_amd import builders
     monkeypatch.setenv("HIPIE_FUSE_ATTENTION", "1" if fuse_attention else "0")
+    monkeypatch.setenv("HIPIE_MERGE_LINEAR", "1" if merge_linear else "0")
+    gemms = 4 if merge_linear else 6                         # Q, K, V projections as one GEMM or three
     # first with every f32 value behind a tolerance-only op kept in the arena (segment-wise check) ...
     monkeypatch.setenv("HIPIE_KEEP_F32", "1")
     # ranges for the reduced width: about 30 levels per standard deviation, so the tails saturate
@@ -30,10 +32,10 @@ def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq, fuse_
     plan = g.compile()
     types = [s["type"] for s in plan.steps]
     if fuse_attention:      # the probabilities stay in registers between the two products
-        assert types.count("MatMul") == 6 * layers and types.count("Attention") == layers
+        assert types.count("MatMul") == gemms * layers and types.count("Attention") == layers
         assert "Transpose" not in types and "Softmax+FakeQuantize" not in types
     else:
-        assert types.count("MatMul") == 8 * layers and types.count("Transpose") == layers
+        assert types.count("MatMul") == (gemms + 2) * layers and types.count("Transpose") == layers
         assert types.count("Softmax+FakeQuantize") == layers
     assert types.count("Gelu+FakeQuantize") == layers
     exact = [n for n in EXACT if not (fuse_attention and n == "pq")]
@@ -92,7 +94,12 @@ def test_encoder_stack_other_head_count_and_ragged_rows(orc, monkeypatch):
 def test_encoder_stack_with_separate_attention_kernels(orc, monkeypatch):
     """the same graph with the attention core planned as MatMul, Softmax + FakeQuantize, Transpose, MatMul"""
     _check_stack(orc, monkeypatch, layers=2, hidden=128, heads=2, ffn=256, batch=2, seq=128, fuse_attention=False)
-    _check_stack(orc, monkeypatch, layers=1, hidden=192, heads=3, ffn=320, batch=3, seq=64, fuse_attention=False)
+    _check_stack(orc, monkeypatch, layers=1, hidden=192, heads=3, ffn=320, batch=3, seq=64, fuse_attention=False,
+                 merge_linear=False)
+
+
+def test_encoder_stack_with_one_gemm_per_matmul(orc, monkeypatch):
+    _check_stack(orc, monkeypatch, layers=1, hidden=128, heads=2, ffn=256, batch=2, seq=128, merge_linear=False)
 
 
 def test_unsupported_transformer_nodes_are_reported():

@@ -119,14 +119,17 @@ def test_planner_encoder_stack_steps_and_views(monkeypatch):
     g, meta = builders.bert_encoder(layers=2, hidden=128, heads=2, ffn=256, batch=2, seq=128, seed=7)
     plan = Plan(g, device=-1)
     types = [s["type"] for s in plan.steps]
-    attention = ["MatMul", "MatMul", "MatMul", "Attention", "MatMul"]
+    attention = ["MatMul", "Attention", "MatMul"]          # Q, K, V projections as one GEMM; the core; the output projection
     ffn = ["MVN+FakeQuantize", "MatMul", "Gelu+FakeQuantize", "MatMul"]
     # every activation FakeQuantize but the first rides in the kernel that produces its input
     assert types == ["FakeQuantize"] + attention + ffn + ["MVN+FakeQuantize"] + attention + ffn + ["MVN", "Result"]
     assert sum(s["macs"] for s in plan.steps) == meta["macs"]
     monkeypatch.setenv("HIPIE_FUSE_ATTENTION", "0")       # separate kernels: V gets one physical transpose
     types = [s["type"] for s in Plan(g, device=-1).steps]
-    assert types[3:8] == ["MatMul", "Softmax+FakeQuantize", "MatMul", "Transpose", "MatMul"]
+    assert types[1:6] == ["MatMul", "MatMul", "Softmax+FakeQuantize", "Transpose", "MatMul"]
+    monkeypatch.setenv("HIPIE_MERGE_LINEAR", "0")         # and one GEMM per MatMul node
+    types = [s["type"] for s in Plan(g, device=-1).steps]
+    assert types[1:8] == ["MatMul", "MatMul", "MatMul", "Softmax+FakeQuantize", "MatMul", "Transpose", "MatMul"]
     T, H, FF = 16 * 384, 768, 3072
     assert 12 * (T * (4 * H * H + 2 * H * FF) + 2 * 16 * 12 * 384 * 384 * 64) == 565_325_070_336
 
