@@ -404,7 +404,7 @@ def mobilenet_v2(batch=1, res=224, seed=20211, classes=1000, width=1.0, blocks=M
 BERT_RANGES = dict(x=4.0, q=1.2, k=3.0, v=3.0, p=1.0, ctx=1.0, h1=4.0, g=3.0)
 
 
-def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, seed=20211, ranges=None):
+def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, seed=20211, ranges=None, vocab=0):
     """BASELINE config 5: BERT-base style encoder stack in its post-LPT form.  Activations are
     per-tensor symmetric i8 (FakeQuantize ranges of signed_range), weights per-channel i8, Softmax /
     LayerNorm (MVN, Multiply, Add) / Gelu stay f32.
@@ -419,6 +419,10 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
     (MatMulTransformation, mat_mul.cpp:81-171; AddTransformation moves the bias in front of the
     Multiply, add.cpp:125-153; FakeQuantizeTransformation::fuseElementwise, fake_quantize.cpp:127-157.)
 
+    vocab > 0 puts the embedding front end in front (the graph input is then the i32 token ids
+    [batch, seq] instead of the f32 hidden states): Gather(word table [vocab, hidden], ids) +
+    position table [seq, hidden] + token-type row [hidden], LayerNorm.
+
     Returns (graph, meta); meta["layers"][l] maps tensor names to node ids, meta["glue"] lists the
     nodes that only have tolerance parity (Softmax, LayerNorm tails, Gelu)."""
     assert hidden % heads == 0
@@ -429,8 +433,15 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
     net = QuantizedNet()
     g = net.g
     nrm = lambda *shape: (rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02)).astype(np.float32)
-    x = g.parameter("hidden_states", (batch, seq, hidden))
     meta = dict(layers=[], glue=[], macs=0)
+    if vocab:
+        from .tensor import I32
+        ids = g.parameter("input_ids", (batch, seq), I32)
+        emb = g.gather(g.constant(nrm(vocab, hidden)), ids, 0)
+        emb = g.add(g.add(emb, g.constant(nrm(seq, hidden))), g.constant(nrm(hidden)))
+        meta["embeddings"] = emb
+    else:
+        x = g.parameter("hidden_states", (batch, seq, hidden))
 
     def fq(v, absmax):
         lo, hi = net.signed_range(absmax)
@@ -466,6 +477,9 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
     def split_heads(node):
         return g.transpose(g.reshape(node, (batch, seq, heads, D)), (0, 2, 1, 3))
 
+    if vocab:
+        x = layer_norm(emb)
+        meta["embedding_norm"] = x
     for _ in range(layers):
         L = {}
         wq_ = nrm(hidden, hidden) * np.float32(1.0 / np.sqrt(D))

@@ -286,6 +286,37 @@ void run_gelu(const float* x, float* y, int8_t* q, int64_t n, const hipie_requan
     HIPIE_CHECK_HIP(hipGetLastError());
 }
 
+// Embedding lookup: one wavefront per token copies its table row (float4 per lane and step) and adds
+// up to two addends in the graph's order.
+__global__ __launch_bounds__(kThreads) void embedding_rows(const float* __restrict__ table, int64_t vocab, int hidden,
+                                                           const int32_t* __restrict__ ids, int64_t tokens, int seq,
+                                                           const float* __restrict__ add0, int pos0,
+                                                           const float* __restrict__ add1, int pos1, float* __restrict__ out) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * (kThreads / 64) + (threadIdx.x >> 6);
+    if (t >= tokens) return;
+    const int lane = threadIdx.x & 63;
+    int64_t idx = ids[t];
+    if (idx < 0) idx += vocab;
+    idx = idx < 0 ? 0 : (idx >= vocab ? vocab - 1 : idx);
+    const int64_t p = t % seq;
+    const float* src = table + idx * hidden;
+    const float* a0 = add0 ? add0 + (pos0 ? p * hidden : 0) : nullptr;
+    const float* a1 = add1 ? add1 + (pos1 ? p * hidden : 0) : nullptr;
+    float* dst = out + t * hidden;
+    for (int i = 4 * lane; i < hidden; i += 256) {
+        float4 v = *reinterpret_cast<const float4*>(src + i);
+        if (a0) {
+            const float4 a = *reinterpret_cast<const float4*>(a0 + i);
+            v.x = v.x + a.x; v.y = v.y + a.y; v.z = v.z + a.z; v.w = v.w + a.w;
+        }
+        if (a1) {
+            const float4 a = *reinterpret_cast<const float4*>(a1 + i);
+            v.x = v.x + a.x; v.y = v.y + a.y; v.z = v.z + a.z; v.w = v.w + a.w;
+        }
+        *reinterpret_cast<float4*>(dst + i) = v;
+    }
+}
+
 // Batched 2-D transpose of bytes through a 64 x 64 LDS tile (row stride 65 words would not help
 // bytes: rows are read as 16-byte pieces and written back byte-wise from a 64 x 65 tile).
 // dst[b][c][r] = src[b][r][c]; the two inner dimensions of a Transpose node on an i8 tensor
@@ -349,6 +380,25 @@ int hipie_mvn_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis
 
 int hipie_gelu_q8(const float* x, float* y, int8_t* q, int64_t n, const hipie_requant* requant, void* stream) {
     return guarded([&] { run_gelu(x, y, q, n, requant, stream, "hipie_gelu_q8"); });
+}
+
+int hipie_embedding_f32(const float* table, int64_t vocabulary, int64_t hidden, const int32_t* ids, int64_t tokens,
+                        int64_t seq, const float* add0, int add0_per_position, const float* add1, int add1_per_position,
+                        float* out, void* stream) {
+    return guarded([&] {
+        if (tokens == 0) return;
+        HIPIE_REQUIRE(table && ids && out && vocabulary > 0 && tokens > 0 && seq > 0 && hidden > 0 && hidden % 4 == 0 &&
+                          hidden < (1ll << 31) && seq < (1ll << 31),
+                      HIPIE_PARAMETER_MISMATCH, "hipie_embedding_f32: bad argument (hidden must be a multiple of 4)");
+        for (const void* p : {static_cast<const void*>(table), static_cast<const void*>(add0), static_cast<const void*>(add1),
+                              static_cast<const void*>(out)})
+            HIPIE_REQUIRE(reinterpret_cast<uintptr_t>(p) % 16 == 0, HIPIE_PARAMETER_MISMATCH,
+                          "hipie_embedding_f32: buffers must be 16-byte aligned");
+        hipLaunchKernelGGL(embedding_rows, dim3(static_cast<uint32_t>(ceil_div(tokens, kThreads / 64))), dim3(kThreads), 0,
+                           as_stream(stream), table, vocabulary, static_cast<int>(hidden), ids, tokens, static_cast<int>(seq),
+                           add0, add0_per_position, add1, add1_per_position, out);
+        HIPIE_CHECK_HIP(hipGetLastError());
+    });
 }
 
 int hipie_transpose_bytes(const void* src, int64_t ld_src, int64_t batch_stride_src, void* dst, int64_t ld_dst,

@@ -9,8 +9,8 @@ const char* op_name(int op) {
     static const char* names[] = {"Parameter", "Constant", "FakeQuantize", "Convolution",
                                   "GroupConvolution", "MatMul", "Add", "Multiply", "Subtract", "Relu",
                                   "Clamp", "Convert", "MaxPool", "AvgPool", "Reshape", "Result", "Softmax", "MVN",
-                                  "Gelu", "Transpose"};
-    return op >= 0 && op <= OP_TRANSPOSE ? names[op] : "?";
+                                  "Gelu", "Transpose", "Gather"};
+    return op >= 0 && op <= OP_GATHER ? names[op] : "?";
 }
 
 namespace {
@@ -79,7 +79,7 @@ int hipie_graph_parameter(hipie_graph* g, const char* name, int dtype, const int
     return guarded([&] {
         HIPIE_REQUIRE(g && dims && id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_parameter: null argument");
         HIPIE_REQUIRE(rank >= 2 && rank <= 4, HIPIE_NOT_IMPLEMENTED, "hipie_graph_parameter: rank %d", rank);
-        HIPIE_REQUIRE(dtype == HIPIE_F32 || dtype == HIPIE_U8, HIPIE_NOT_IMPLEMENTED,
+        HIPIE_REQUIRE(dtype == HIPIE_F32 || dtype == HIPIE_U8 || dtype == HIPIE_I32, HIPIE_NOT_IMPLEMENTED,
                       "hipie_graph_parameter: element type %d", dtype);
         GNode n;
         n.op = OP_PARAMETER;
@@ -403,6 +403,29 @@ int hipie_graph_transpose(hipie_graph* g, int x, const int64_t* order, int rank,
             n.shape.push_back(X.shape[order[i]]);
         }
         n.dtype = X.dtype;
+        *id = add_node(g, std::move(n));
+    });
+}
+
+/* op::v1::Gather (ngraph/core/src/op/gather.cpp): out.shape = data.shape[:axis] + indices.shape + data.shape[axis+1:] */
+int hipie_graph_gather(hipie_graph* g, int data, int indices, int64_t axis, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_gather: null argument");
+        GNode& D = node(g, data, "hipie_graph_gather");
+        GNode& I = node(g, indices, "hipie_graph_gather");
+        const int64_t r = static_cast<int64_t>(D.shape.size());
+        HIPIE_REQUIRE(I.dtype == HIPIE_I32, HIPIE_PARAMETER_MISMATCH, "hipie_graph_gather: indices must be i32");
+        HIPIE_REQUIRE(axis >= -r && axis < r, HIPIE_PARAMETER_MISMATCH, "hipie_graph_gather: axis %lld of rank %lld",
+                      (long long)axis, (long long)r);
+        GNode n;
+        n.op = OP_GATHER;
+        n.in = {data, indices};
+        const int64_t ax = axis < 0 ? axis + r : axis;
+        n.axes = {ax};
+        n.dtype = D.dtype;
+        n.shape.assign(D.shape.begin(), D.shape.begin() + ax);
+        n.shape.insert(n.shape.end(), I.shape.begin(), I.shape.end());
+        n.shape.insert(n.shape.end(), D.shape.begin() + ax + 1, D.shape.end());
         *id = add_node(g, std::move(n));
     });
 }

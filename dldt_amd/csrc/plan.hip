@@ -523,6 +523,31 @@ struct AttentionStep : Step {
     }
 };
 
+// Gather of a constant f32 table by the i32 token ids of a request input, with the embedding Adds
+struct EmbeddingStep : Step {
+    int param = 0, out = -1;
+    int64_t vocab = 0, hidden = 0, tokens = 0, seq = 0;
+    std::vector<float> table, add[2];
+    bool per_position[2] = {false, false};
+    DeviceBuffer d_table, d_add[2];
+    void create(int device, const std::vector<TensorInfo>&) override {
+        if (device >= 0) {
+            d_table.upload(device, table.data(), table.size() * 4);
+            for (int i = 0; i < 2; ++i)
+                if (!add[i].empty()) d_add[i].upload(device, add[i].data(), add[i].size() * 4);
+        }
+        table.clear();
+        table.shrink_to_fit();
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
+             hipStream_t s) const override {
+        check_status(hipie_embedding_f32(d_table.as<float>(), vocab, hidden, static_cast<const int32_t*>(inputs[param]), tokens, seq,
+                                         add[0].empty() ? nullptr : d_add[0].as<float>(), per_position[0],
+                                         add[1].empty() ? nullptr : d_add[1].as<float>(), per_position[1],
+                                         reinterpret_cast<float*>(arena + tensors[out].offset), s), name.c_str());
+    }
+};
+
 // physical transpose of the two inner dimensions of a byte view (the right operand of a MatMul whose
 // reduction axis is not contiguous)
 struct MatTransposeStep : Step {
@@ -651,6 +676,7 @@ struct Planner {
         case OP_RESHAPE: mat ? plan_mat_reshape(id) : plan_reshape(id); break;
         case OP_TRANSPOSE: plan_mat_transpose(id); break;
         case OP_SOFTMAX: case OP_MVN: case OP_GELU: plan_glue(id); break;
+        case OP_GATHER: plan_gather(id); break;
         case OP_RESULT: mat ? plan_mat_result(id) : plan_result(id); values[id].kind = VK_FUSED; break;
         default: unsupported(id, "only planned as part of a fused convolution / pooling chain");
         }
@@ -675,6 +701,51 @@ struct Planner {
         v.stride = View::dense_strides(n.shape);
         values[id].kind = VK_MAT;
         values[id].view = v;
+    }
+
+    // Embedding front end: Gather(table f32 [V, H], ids i32 Parameter [B, S], axis 0) and the Adds of
+    // constants behind it (one row [H], or one row per position [S, H] / [1, S, H])
+    void plan_gather(int id) {
+        const GNode& n = N(id);
+        const GNode& T = N(n.in[0]);
+        const GNode& I = N(n.in[1]);
+        if (T.op != OP_CONSTANT || T.dtype != HIPIE_F32 || T.shape.size() != 2 || n.axes[0] != 0)
+            unsupported(id, "Gather is planned as a lookup in a constant f32 table [vocabulary, hidden] along axis 0");
+        if (I.op != OP_PARAMETER || I.dtype != HIPIE_I32 || I.shape.size() != 2)
+            unsupported(id, "Gather indices must be an i32 Parameter [batch, sequence]");
+        auto st = std::make_unique<EmbeddingStep>();
+        for (size_t i = 0; i < g.params.size(); ++i)
+            if (g.params[i] == n.in[1]) st->param = static_cast<int>(i);
+        st->vocab = T.shape[0];
+        st->hidden = T.shape[1];
+        st->seq = I.shape[1];
+        st->tokens = I.shape[0] * I.shape[1];
+        if (st->hidden % 4 != 0) unsupported(id, "hidden size must be a multiple of 4");
+        st->table.assign(T.f32(), T.f32() + T.numel());
+        int cur = id, k = 0;
+        while (k < 2 && single_user(cur)) {
+            const int nx = N(cur).users[0];
+            const GNode& u = N(nx);
+            if (u.op != OP_ADD) break;
+            const GNode& c = N(u.in[0] == cur ? u.in[1] : u.in[0]);
+            if (c.op != OP_CONSTANT || c.dtype != HIPIE_F32 || c.shape.empty() || c.shape.back() != st->hidden) break;
+            const int64_t ne = c.numel();
+            const bool row = ne == st->hidden;
+            const bool pos = ne == st->seq * st->hidden && c.shape.size() >= 2 && c.shape[c.shape.size() - 2] == st->seq;
+            if (!row && !pos) break;
+            st->add[k].assign(c.f32(), c.f32() + ne);
+            st->per_position[k] = !row;
+            ++k;
+            cur = nx;
+        }
+        mark_chain(id, cur);
+        st->out = new_matrix(cur, HIPIE_F32, n.shape);
+        st->name = N(cur).name;
+        st->type = "Gather";
+        st->bytes = n.numel() * 8;
+        st->out_node = cur;
+        set_matrix_value(cur, st->out, HIPIE_F32);
+        steps.push_back(std::move(st));
     }
 
     // constant broadcastable along the last axis: 1 or C numbers
@@ -1706,7 +1777,7 @@ int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
             }
         for (int p : g->params) {
             const GNode& n = g->nodes[p];
-            plan->inputs.push_back({n.name, n.dtype, n.shape, n.numel() * (n.dtype == HIPIE_F32 ? 4 : 1)});
+            plan->inputs.push_back({n.name, n.dtype, n.shape, n.numel() * (n.dtype == HIPIE_F32 || n.dtype == HIPIE_I32 ? 4 : 1)});
         }
         for (int r : g->results) {
             const GNode& n = g->nodes[r];

@@ -144,6 +144,11 @@ class Graph:
         check(lib().hipie_graph_transpose(self._h, x, _i64(order), len(order), ctypes.byref(i)))
         return self._rec(i.value, "Transpose", [x], self.nodes[x]["dtype"], order=tuple(order))
 
+    def gather(self, data, indices, axis=0):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_gather(self._h, data, indices, ctypes.c_int64(axis), ctypes.byref(i)))
+        return self._rec(i.value, "Gather", [data, indices], self.nodes[data]["dtype"], axis=axis)
+
     def result(self, x, name):
         check(lib().hipie_graph_result(self._h, x, name.encode()))
         self.results.append(len(self.nodes))
@@ -220,7 +225,7 @@ class Request:
     def device_buffers(self):
         """torch tensors shaped like the plan's inputs and outputs (for resident-in-HBM runs)."""
         import torch
-        tdt = {F32: torch.float32, U8: torch.uint8}
+        tdt = {F32: torch.float32, U8: torch.uint8, I32: torch.int32}
         dev = "cuda:%d" % self.plan.device
         ins = [torch.empty(d["shape"], dtype=tdt[d["dtype"]], device=dev) for d in self.plan.inputs]
         outs = [torch.empty(d["shape"], dtype=tdt[d["dtype"]], device=dev) for d in self.plan.outputs]

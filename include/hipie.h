@@ -273,6 +273,15 @@ int hipie_softmax_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t 
 int hipie_mvn_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis, int normalize_variance, float eps,
                  int eps_inside_sqrt, const float* gamma, const float* beta, const hipie_requant* requant, void* stream);
 int hipie_gelu_q8(const float* x, float* y, int8_t* q, int64_t n, const hipie_requant* requant, void* stream);
+/* Embedding front end of an encoder — reference::gather (.../reference/gather.hpp:18-66) of rows of a
+ * f32 table [vocabulary, hidden] by i32 token ids, followed by up to two reference::add steps in the
+ * graph's order: out[t] = (table[ids[t]] + add0) + add1, each addend (device pointer, or NULL) either
+ * one row [hidden] or one row per position [seq, hidden] (position embeddings; token t sits at
+ * position t % seq).  Negative ids count from the end like the reference; ids outside the table
+ * (undefined behaviour there) read its nearest row. */
+int hipie_embedding_f32(const float* table, int64_t vocabulary, int64_t hidden, const int32_t* ids, int64_t tokens,
+                        int64_t seq, const float* add0, int add0_per_position, const float* add1, int add1_per_position,
+                        float* out, void* stream);
 /* Self-attention core of a post-LPT encoder in one kernel, per (sequence, head):
  *     MatMul'(q, k^T) * score_scale -> Softmax -> FakeQuantize(prob_fq) -> MatMul'(., v) * context_scale
  *     [-> FakeQuantize(out_fq) when out_dtype is HIPIE_I8]
@@ -320,7 +329,8 @@ int hipie_transpose_bytes_nested(const void* src, int64_t ld_src, int64_t stride
  *    Supported nodes: Parameter(f32), Constant, FakeQuantize, Convolution, GroupConvolution,
  *    MatMul, Add, Multiply, Subtract, Relu, Clamp, Convert, MaxPool, AvgPool, Reshape, Result, and
  *    for transformer encoders (rank-3 Parameter [batch, sequence, hidden]): MatMul between two
- *    activations, Softmax, MVN, Gelu, Transpose.
+ *    activations, Softmax, MVN, Gelu, Transpose, and Gather of a constant table by an i32
+ *    Parameter [batch, sequence] (the embedding front end).
  * ==================================================================================== */
 typedef struct hipie_graph hipie_graph;
 typedef struct hipie_plan hipie_plan;
@@ -359,6 +369,9 @@ int hipie_graph_mvn(hipie_graph* g, int x, const int64_t* axes, int n_axes, int 
                     int eps_inside_sqrt, int* id);
 int hipie_graph_gelu(hipie_graph* g, int x, int* id);
 int hipie_graph_transpose(hipie_graph* g, int x, const int64_t* order, int rank, int* id);
+/* op::v1::Gather with the axis Constant's value; planned as an embedding lookup: f32 Constant table
+ * [vocabulary, hidden], i32 Parameter indices [batch, sequence], axis 0 */
+int hipie_graph_gather(hipie_graph* g, int data, int indices, int64_t axis, int* id);
 int hipie_graph_result(hipie_graph* g, int x, const char* name);
 int hipie_graph_set_name(hipie_graph* g, int id, const char* friendly_name);
 

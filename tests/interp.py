@@ -57,6 +57,9 @@ def evaluate(orc, nodes, feeds, keep=None, override=None):
                              not n["exclude_pad"], out_shape=oshape)
         elif op == "Reshape":
             v = x[0].reshape(n["shape"])
+        elif op == "Gather":
+            idx = np.where(x[1] < 0, x[1] + x[0].shape[n["axis"]], x[1])      # gather.hpp:58-59
+            v = np.ascontiguousarray(np.take(x[0], idx, axis=n["axis"]))
         elif op == "Transpose":
             v = np.ascontiguousarray(np.transpose(x[0], n["order"]))
         elif op == "Softmax":

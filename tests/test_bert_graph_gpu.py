@@ -111,3 +111,33 @@ def test_unsupported_transformer_nodes_are_reported():
     with pytest.raises(HipieError) as e:
         g.compile()
     assert e.value.status == -2 and "Softmax" in str(e.value)
+
+
+def test_encoder_with_embedding_front_end(orc, monkeypatch):
+    """token ids -> Gather(word table) + position table + token-type row -> LayerNorm -> one encoder layer;
+    ids include negative values (counted from the end of the table, gather.hpp:58-59)"""
+    from dldt_amd import builders
+    monkeypatch.setenv("HIPIE_KEEP_F32", "1")
+    B, S, H, V = 2, 64, 128, 500
+    g, meta = builders.bert_encoder(layers=1, hidden=H, heads=2, ffn=256, batch=B, seq=S, seed=9, vocab=V,
+                                    ranges=dict(q=0.12, k=0.9, v=0.9, ctx=0.6))
+    ids = np.random.default_rng(3).integers(-7, V, (B, S)).astype(np.int32)
+    assert (ids < 0).any()
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps[:2]] == ["Gather", "MVN+FakeQuantize"]
+    assert plan.inputs[0]["name"] == "input_ids" and plan.inputs[0]["shape"] == (B, S)
+    req = plan.create_request()
+    (y,) = req.infer(ids)
+    device = {n: req.matrix(n) for n in meta["glue"]}
+    L = meta["layers"][0]
+    keep = [meta["embeddings"]] + [L[k] for k in ("xq", "q", "ctx", "down")]
+    want, kept = evaluate(orc, g.nodes, {"input_ids": ids}, keep=keep, override=device)
+    emb = kept[meta["embeddings"]]
+    np.testing.assert_array_equal(req.matrix(meta["embeddings"]).reshape(emb.shape).view(np.uint32), emb.view(np.uint32))
+    w = kept[("oracle", meta["embedding_norm"])]
+    np.testing.assert_allclose(device[meta["embedding_norm"]].reshape(w.shape), w, rtol=1e-5, atol=4e-6)
+    for k in ("xq", "q"):
+        np.testing.assert_array_equal(req.matrix(L[k]).reshape(kept[L[k]].shape).view(np.int8), kept[L[k]].astype(np.int8))
+    for k in ("ctx", "down"):
+        np.testing.assert_array_equal(req.matrix(L[k]).reshape(kept[L[k]].shape).view(np.uint32), kept[L[k]].view(np.uint32))
+    np.testing.assert_array_equal(y.view(np.uint32), want["out"].view(np.uint32))

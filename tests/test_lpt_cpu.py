@@ -144,3 +144,13 @@ def test_planner_refuses_a_reshape_that_moves_bytes():
     with pytest.raises(HipieError) as e:
         g.compile(device=-1)
     assert e.value.status == -2 and "Reshape" in str(e.value)
+
+
+def test_planner_embedding_front_end():
+    from dldt_amd import builders
+    from dldt_amd.graph import Plan
+    g, meta = builders.bert_encoder(layers=1, hidden=128, heads=2, ffn=256, batch=2, seq=64, seed=9, vocab=300)
+    plan = Plan(g, device=-1)
+    types = [s["type"] for s in plan.steps]
+    assert types[:3] == ["Gather", "MVN+FakeQuantize", "MatMul"] and "FakeQuantize" not in types
+    assert plan.inputs[0]["dtype"] == 70 and plan.inputs[0]["shape"] == (2, 64)
