@@ -404,7 +404,8 @@ def mobilenet_v2(batch=1, res=224, seed=20211, classes=1000, width=1.0, blocks=M
 BERT_RANGES = dict(x=4.0, q=1.2, k=3.0, v=3.0, p=1.0, ctx=1.0, h1=4.0, g=3.0)
 
 
-def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, seed=20211, ranges=None, vocab=0):
+def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, seed=20211, ranges=None, vocab=0,
+                 mask=False):
     """BASELINE config 5: BERT-base style encoder stack in its post-LPT form.  Activations are
     per-tensor symmetric i8 (FakeQuantize ranges of signed_range), weights per-channel i8, Softmax /
     LayerNorm (MVN, Multiply, Add) / Gelu stay f32.
@@ -422,6 +423,9 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
     vocab > 0 puts the embedding front end in front (the graph input is then the i32 token ids
     [batch, seq] instead of the f32 hidden states): Gather(word table [vocab, hidden], ids) +
     position table [seq, hidden] + token-type row [hidden], LayerNorm.
+
+    mask=True adds a second graph input "attention_mask" f32 [batch, 1, 1, seq] that is added to the
+    scaled scores of every layer in front of the Softmax (0 for tokens to attend to, -10000 for padding).
 
     Returns (graph, meta); meta["layers"][l] maps tensor names to node ids, meta["glue"] lists the
     nodes that only have tolerance parity (Softmax, LayerNorm tails, Gelu)."""
@@ -480,6 +484,7 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
     if vocab:
         x = layer_norm(emb)
         meta["embedding_norm"] = x
+    mask_node = g.parameter("attention_mask", (batch, 1, 1, seq)) if mask else None
     for _ in range(layers):
         L = {}
         wq_ = nrm(hidden, hidden) * np.float32(1.0 / np.sqrt(D))
@@ -489,6 +494,8 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
         v = linear_fq(xq, nrm(hidden, hidden), nrm(hidden), r["v"])
         s = g.multiply(g.matmul(split_heads(q["node"]), split_heads(k["node"]), False, True),
                        g.constant(np.float32(q["scale"] * k["scale"]).reshape(())))
+        if mask_node is not None:
+            s = g.add(s, mask_node)
         p = g.softmax(s, -1)
         meta["glue"].append(p)
         pq = fq(p, r["p"])

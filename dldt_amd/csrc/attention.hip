@@ -1,5 +1,5 @@
 // Self-attention core of a post-LPT encoder in one kernel:
-//     scores = MatMul'(q, k^T) * s1 -> Softmax -> FakeQuantize (i8) -> MatMul'(., v) * s2 [-> FakeQuantize]
+//     scores = MatMul'(q, k^T) * s1 [+ mask] -> Softmax -> FakeQuantize (i8) -> MatMul'(., v) * s2 [-> FakeQuantize]
 // (mat_mul.cpp:81-171 leaves the two TypeRelaxed MatMuls with their dequantization Multiply; softmax.hpp,
 // fake_quantize.hpp).  The f32 scores and probabilities of one encoder layer are 2 x 113 MB at
 // batch 16 x 12 heads x 384^2; here they never leave the registers.
@@ -28,6 +28,8 @@ struct AttentionArgs {
     int64_t ldq, sq, oq, ldk, sk, ok, ldv, sv, ov;   // row pitch, inner / outer batch stride (bytes)
     void* out;
     int64_t ldo, so, oo;                              // elements
+    const float* mask;                                // optional additive mask row [S] per batch element, or null
+    int64_t mask_inner, mask_outer;                   // its batch strides (elements)
     float* scores;                                    // optional [batch][S][S] dumps (inspection), or null
     float* probs;
     int S, batch_inner;
@@ -97,6 +99,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
     __syncthreads();
 
     const int slot[2] = {((0 + h) ^ ((l32 >> 2) & 3)) * 16, ((2 + h) ^ ((l32 >> 2) & 3)) * 16};
+    const float* mrow = a.mask ? a.mask + bo * a.mask_outer + bi * a.mask_inner : nullptr;
     float x[NT][16];
     float m = -INFINITY;
 #pragma unroll
@@ -108,9 +111,17 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[ks], acc, 0, 0, 0);
         }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            x[t][r] = static_cast<float>(acc[r]) * a.scale1;
-            m = fmaxf(m, x[t][r]);
+        for (int g = 0; g < 4; ++g) {
+            float4 mk = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (mrow) mk = *reinterpret_cast<const float4*>(mrow + 32 * t + 8 * g + 4 * h);
+            const float mv[4] = {mk.x, mk.y, mk.z, mk.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float v = static_cast<float>(acc[4 * g + j]) * a.scale1;
+                if (mrow) v = v + mv[j];                 // the mask Add between the Multiply and the Softmax
+                x[t][4 * g + j] = v;
+                m = fmaxf(m, v);
+            }
         }
     }
     const int64_t dump_row = (static_cast<int64_t>(b) * a.S + q_row) * a.S;   // [batch][query][key]
@@ -232,9 +243,12 @@ void hipie_attention_destroy(hipie_attention* att) { delete att; }
 int hipie_attention_run(const hipie_attention* att, const void* q, int64_t ldq, int64_t stride_q, int64_t outer_q,
                         const void* k, int64_t ldk, int64_t stride_k, int64_t outer_k, const void* v, int64_t ldv,
                         int64_t stride_v, int64_t outer_v, void* out, int64_t ldo, int64_t stride_o, int64_t outer_o,
-                        int32_t batch, int32_t batch_outer, float* scores, float* probs, void* stream) {
+                        int32_t batch, int32_t batch_outer, const float* mask, int64_t mask_stride, int64_t mask_outer,
+                        float* scores, float* probs, void* stream) {
     return guarded([&] {
         HIPIE_REQUIRE(att && q && k && v && out, HIPIE_PARAMETER_MISMATCH, "hipie_attention_run: null argument");
+        HIPIE_REQUIRE(reinterpret_cast<uintptr_t>(mask) % 16 == 0 && mask_stride % 4 == 0 && mask_outer % 4 == 0,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_attention_run: mask rows must be 16-byte aligned");
         HIPIE_REQUIRE(att->device >= 0, HIPIE_NOT_ALLOCATED, "hipie_attention_run: host-only object");
         if (batch == 0 || batch_outer == 0) return;
         HIPIE_REQUIRE(batch > 0 && batch_outer > 0 && static_cast<int64_t>(batch) * batch_outer < 65536, HIPIE_PARAMETER_MISMATCH,
@@ -254,6 +268,7 @@ int hipie_attention_run(const hipie_attention* att, const void* q, int64_t ldq, 
         a.ldv = ldv; a.sv = stride_v; a.ov = outer_v;
         a.out = out; a.ldo = ldo; a.so = stride_o; a.oo = outer_o;
         a.scores = scores; a.probs = probs;
+        a.mask = mask; a.mask_inner = mask_stride; a.mask_outer = mask_outer;
         a.batch_inner = batch;
         DeviceGuard dg(att->device);
         hipStream_t s = as_stream(stream);

@@ -506,20 +506,27 @@ struct AttentionStep : Step {
     int out = -1, scores = -1, probs = -1;
     int64_t ldo = 0, so = 0, oo = 0;
     int32_t batch = 1, batch_outer = 1;
+    // additive mask [batch_outer, 1, 1, S]: a request input or a constant
+    bool masked = false;
+    int mask_param = -1;
+    std::vector<float> mask_const;
+    DeviceBuffer d_mask;
     hipie_attention_desc desc{};
     hipie_attention* att = nullptr;
     ~AttentionStep() override { hipie_attention_destroy(att); }
     void create(int device, const std::vector<TensorInfo>&) override {
         check_status(hipie_attention_create(device, &desc, &att), name.c_str());
+        if (device >= 0 && !mask_const.empty()) d_mask.upload(device, mask_const.data(), mask_const.size() * 4);
     }
     void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
              hipStream_t s) const override {
         float* sc = scores >= 0 ? reinterpret_cast<float*>(arena + tensors[scores].offset) : nullptr;
         float* pr = probs >= 0 ? reinterpret_cast<float*>(arena + tensors[probs].offset) : nullptr;
+        const float* mk = !masked ? nullptr : (mask_param >= 0 ? static_cast<const float*>(inputs[mask_param]) : d_mask.as<float>());
         check_status(hipie_attention_run(att, q.ptr(arena, tensors, inputs), ld[0], inner[0], outer[0],
                                          k.ptr(arena, tensors, inputs), ld[1], inner[1], outer[1],
                                          v.ptr(arena, tensors, inputs), ld[2], inner[2], outer[2], arena + tensors[out].offset,
-                                         ldo, so, oo, batch, batch_outer, sc, pr, s), name.c_str());
+                                         ldo, so, oo, batch, batch_outer, mk, 0, desc.seq, sc, pr, s), name.c_str());
     }
 };
 
@@ -1213,7 +1220,19 @@ struct Planner {
         if (N(mul).op != OP_MULTIPLY || !last_axis_constant(N(mul).in[0] == id ? N(mul).in[1] : N(mul).in[0], -1, c1) ||
             !single_user(mul))
             return false;
-        const int sm = N(mul).users[0];
+        // optional attention mask: Add of an f32 Parameter / Constant [batch, 1, 1, S] (rank-4 attention only)
+        int pre = mul, mask_node = -1;
+        if (N(N(mul).users[0]).op == OP_ADD && r == 4) {
+            const int add = N(mul).users[0];
+            const int other = N(add).in[0] == mul ? N(add).in[1] : N(add).in[0];
+            const GNode& mk = N(other);
+            const std::vector<int64_t> want = {qv.shape[0], 1, 1, S};
+            if ((mk.op != OP_PARAMETER && mk.op != OP_CONSTANT) || mk.dtype != HIPIE_F32 || mk.shape != want || !single_user(add))
+                return false;
+            pre = add;
+            mask_node = other;
+        }
+        const int sm = N(pre).users[0];
         if (N(sm).op != OP_SOFTMAX || N(sm).axes[0] != static_cast<int64_t>(r) - 1 || !single_user(sm)) return false;
         const int fq = N(sm).users[0];
         hipie_requant rq{};
@@ -1263,13 +1282,24 @@ struct Planner {
         // writes the values in front of and behind the Softmax
         values[id].kind = VK_FUSED;
         values[fq].kind = VK_FUSED;
-        if (keep_f32) {
-            st->scores = new_matrix(mul, HIPIE_F32, N(mul).shape);
-            set_matrix_value(mul, st->scores, HIPIE_F32);
+        if (mask_node >= 0) {
+            st->masked = true;
+            if (N(mask_node).op == OP_PARAMETER) {
+                (void)visit(mask_node);
+                for (size_t i = 0; i < g.params.size(); ++i)
+                    if (g.params[i] == mask_node) st->mask_param = static_cast<int>(i);
+            } else {
+                st->mask_const.assign(N(mask_node).f32(), N(mask_node).f32() + N(mask_node).numel());
+            }
+            values[mul].kind = VK_FUSED;
+        }
+        if (keep_f32) {   // the Softmax input and output
+            st->scores = new_matrix(pre, HIPIE_F32, N(pre).shape);
+            set_matrix_value(pre, st->scores, HIPIE_F32);
             st->probs = new_matrix(sm, HIPIE_F32, N(sm).shape);
             set_matrix_value(sm, st->probs, HIPIE_F32);
         } else {
-            values[mul].kind = VK_FUSED;
+            values[pre].kind = VK_FUSED;
             values[sm].kind = VK_FUSED;
         }
         mark_chain(mm2, cur);

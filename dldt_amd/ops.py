@@ -338,9 +338,10 @@ class Attention:
             lib().hipie_attention_destroy(self._h)
             self._h = None
 
-    def run(self, q, k, v, dump=False, out=None):
-        """q, k, v: i8 [B, NH, S, 64] (any strides with contiguous rows).  Returns the context
-        [B, NH, S, 64] and, with dump=True, also the f32 scores and probabilities [B, NH, S, S]."""
+    def run(self, q, k, v, dump=False, out=None, mask=None):
+        """q, k, v: i8 [B, NH, S, 64] (any strides with contiguous rows); mask: f32 [B, S] added to the
+        scaled scores of every head and query, or None.  Returns the context [B, NH, S, 64] and, with
+        dump=True, also the f32 Softmax inputs and probabilities [B, NH, S, S]."""
         import torch
         B, NH, S, D = q.shape
         assert k.shape == q.shape and v.shape == q.shape and q.dtype == torch.int8
@@ -354,12 +355,15 @@ class Attention:
         args = []
         for t in (q, k, v, out):
             args += [_dptr(t), i64(t.stride(2)), i64(t.stride(1)), i64(t.stride(0))]
+        if mask is not None:
+            assert mask.shape == (B, S) and mask.is_contiguous() and mask.dtype == torch.float32
         check(lib().hipie_attention_run(self._h, *args, ctypes.c_int32(NH), ctypes.c_int32(B),
+                                        _dptr(mask) if mask is not None else None, i64(0), i64(S),
                                         _dptr(scores) if dump else None, _dptr(probs) if dump else None, _stream()))
         return (out, scores, probs) if dump else out
 
 
-def attention(q, k, v, score_scale, context_scale, prob_fq, out_fq=None, dump=False):
+def attention(q, k, v, score_scale, context_scale, prob_fq, out_fq=None, dump=False, mask=None):
     """One-shot form of Attention (creates the load-time object for this call)."""
     att = Attention(q.shape[2], q.shape[3], score_scale, context_scale, prob_fq, out_fq, q.device.index or 0)
-    return att.run(q, k, v, dump=dump)
+    return att.run(q, k, v, dump=dump, mask=mask)

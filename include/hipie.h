@@ -283,14 +283,16 @@ int hipie_embedding_f32(const float* table, int64_t vocabulary, int64_t hidden, 
                         int64_t seq, const float* add0, int add0_per_position, const float* add1, int add1_per_position,
                         float* out, void* stream);
 /* Self-attention core of a post-LPT encoder in one kernel, per (sequence, head):
- *     MatMul'(q, k^T) * score_scale -> Softmax -> FakeQuantize(prob_fq) -> MatMul'(., v) * context_scale
+ *     MatMul'(q, k^T) * score_scale [+ mask] -> Softmax -> FakeQuantize(prob_fq) -> MatMul'(., v) * context_scale
  *     [-> FakeQuantize(out_fq) when out_dtype is HIPIE_I8]
  * i.e. the two TypeRelaxed MatMuls low_precision_transformations/src/mat_mul.cpp:81-171 leaves, with
  * reference::softmax (softmax.hpp:20-50) and reference::fake_quantize between them.  q, k, v are i8
  * [seq, head_dim] matrices addressed like the operands of hipie_matmul_run_nested (row pitch, inner and
  * outer batch stride, in bytes); out is [seq, head_dim] f32 or i8 (pitch and strides in elements).
  * The integer products are exact and every f32 step is one IEEE operation in that order; Softmax
- * has tolerance parity.  scores / probs, when not NULL, receive the f32 values in front of and
+ * has tolerance parity.  mask, when not NULL, is the additive attention mask: one f32 row [seq] per
+ * batch element (strides in elements; 0 shares a row between the heads of a sequence), added to the
+ * scaled scores of every query (reference::add with numpy broadcast).  scores / probs, when not NULL, receive the f32 values in front of and
  * behind the Softmax as dense [batch_outer * batch][seq][seq] arrays (inspection; the kernel is
  * otherwise the same).  Sequence lengths: multiples of 32 up to 384; head_dim 64
  * (hipie_attention_supported). */
@@ -309,7 +311,8 @@ void hipie_attention_destroy(hipie_attention* attention);
 int hipie_attention_run(const hipie_attention* attention, const void* q, int64_t ldq, int64_t stride_q, int64_t outer_q,
                         const void* k, int64_t ldk, int64_t stride_k, int64_t outer_k, const void* v, int64_t ldv,
                         int64_t stride_v, int64_t outer_v, void* out, int64_t ldo, int64_t stride_o, int64_t outer_o,
-                        int32_t batch, int32_t batch_outer, float* scores, float* probs, void* stream);
+                        int32_t batch, int32_t batch_outer, const float* mask, int64_t mask_stride, int64_t mask_outer,
+                        float* scores, float* probs, void* stream);
 /* Transpose of the two inner dimensions of a byte tensor (opset1 Transpose on quantized activations,
  * e.g. V [S, d] -> [d, S] so that the context MatMul finds its reduction axis contiguous;
  * reference::transpose, .../reference/transpose.hpp:20-25): dst[b][c][r] = src[b][r][c], leading

@@ -141,3 +141,33 @@ def test_encoder_with_embedding_front_end(orc, monkeypatch):
     for k in ("ctx", "down"):
         np.testing.assert_array_equal(req.matrix(L[k]).reshape(kept[L[k]].shape).view(np.uint32), kept[L[k]].view(np.uint32))
     np.testing.assert_array_equal(y.view(np.uint32), want["out"].view(np.uint32))
+
+
+def test_encoder_with_attention_mask(orc, monkeypatch):
+    """additive mask [batch, 1, 1, seq] between the score Multiply and the Softmax: padded keys get no weight"""
+    from dldt_amd import builders
+    monkeypatch.setenv("HIPIE_KEEP_F32", "1")
+    B, S, H = 2, 96, 128
+    g, meta = builders.bert_encoder(layers=2, hidden=H, heads=2, ffn=256, batch=B, seq=S, seed=11, mask=True,
+                                    ranges=dict(q=0.12, k=0.9, v=0.9, ctx=0.6))
+    rng = np.random.default_rng(12)
+    x = rng.normal(0, 1, (B, S, H)).astype(np.float32)
+    mask = np.zeros((B, 1, 1, S), np.float32)
+    mask[0, 0, 0, 70:] = -10000.0
+    mask[1, 0, 0, 33:] = -10000.0
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps].count("Attention") == 2 and len(plan.inputs) == 2
+    req = plan.create_request()
+    (y,) = req.infer(x, mask)
+    device = {n: req.matrix(n) for n in meta["glue"]}
+    keep = [n for L in meta["layers"] for n in L.values()]
+    want, kept = evaluate(orc, g.nodes, {"hidden_states": x, "attention_mask": mask}, keep=keep, override=device)
+    for li, L in enumerate(meta["layers"]):
+        p = device[L["p"]].reshape(B, 2, S, S)
+        assert p[0, :, :, 70:].max() == 0.0 and p[1, :, :, 33:].max() == 0.0
+        w = kept[("oracle", L["p"])]
+        np.testing.assert_allclose(p, w, rtol=3e-6, atol=1e-8, err_msg="layer %d" % li)
+        for name in ("ctx", "attn", "down"):
+            np.testing.assert_array_equal(req.matrix(L[name]).reshape(kept[L[name]].shape).view(np.uint32),
+                                          kept[L[name]].view(np.uint32), err_msg="layer %d %s" % (li, name))
+    np.testing.assert_array_equal(y.view(np.uint32), want["out"].view(np.uint32))
