@@ -30,9 +30,11 @@ class QuantizedNet:
         self.g = Graph()
 
     # -- graph input ---------------------------------------------------------------------------
-    def input(self, name, shape, in_high):
+    def input(self, name, shape, in_high, u8=False):
+        """f32 graph input, or (u8=True) a u8 one behind a Convert to f32: what a plugin sees when the user
+        sets input precision U8 (benchmark_app's default for images)."""
         g = self.g
-        x = g.parameter(name, shape)
+        x = g.convert(g.parameter(name, shape, U8), F32) if u8 else g.parameter(name, shape)
         d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(in_high))
         q = g.fake_quantize(x, np.float32(0), np.float32(in_high), d["new_low"], d["new_high"], 256, U8)
         return dict(node=q, scale=np.float32(d["scale"]))
@@ -126,14 +128,16 @@ def he_normal(rng, shape):
     return (rng.standard_normal(shape, dtype=np.float32) * np.float32(np.sqrt(2.0 / fan_in))).astype(np.float32)
 
 
-def conv_block(seed=20211, n=1, c=64, hw=56, oc=64):
-    """BASELINE config 1: FQ(u8) -> Conv 3x3 s1 p1 (per-channel i8 weights) -> bias -> ReLU, f32 out."""
+def conv_block(seed=20211, n=1, c=64, hw=56, oc=64, u8_input=False):
+    """BASELINE config 1: FQ(u8) -> Conv 3x3 s1 p1 (per-channel i8 weights) -> bias -> ReLU, f32 out.
+    u8_input: the graph input is a u8 tensor (values 0 .. 255) behind a Convert to f32."""
     rng = np.random.default_rng(seed)
-    x = rng.uniform(0, 2.55, (n, c, hw, hw)).astype(np.float32)
+    x = rng.integers(0, 256, (n, c, hw, hw)).astype(np.uint8) if u8_input else \
+        rng.uniform(0, 2.55, (n, c, hw, hw)).astype(np.float32)
     w = (rng.standard_normal((oc, c, 3, 3), dtype=np.float32) * np.float32(0.05)).astype(np.float32)
     b = (rng.standard_normal(oc, dtype=np.float32) * np.float32(0.1)).astype(np.float32)
     net = QuantizedNet()
-    a = net.input("data", x.shape, 2.55)
+    a = net.input("data", x.shape, 255.0, u8=True) if u8_input else net.input("data", x.shape, 2.55)
     y = net.conv_f32(a, w, b, pads=(1, 1), relu=True)
     net.g.result(y, "out")
     return net.g, dict(data=x), dict(w=w, b=b)

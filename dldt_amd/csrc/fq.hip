@@ -93,8 +93,8 @@ __global__ __launch_bounds__(kThreads) void fq_nchw_f32_vec4(const float4* __res
 // [N, C, HW] f32 -> [N, HW, c_stride] bytes.  A block transposes 64 pixels x 64 channels
 // through LDS so that both the f32 reads (256 B per channel row) and the byte writes (16 B per
 // thread, whole pixels contiguous) are coalesced.  grid = (N * ceil(HW/64), ceil(c_stride/64)).
-template <bool RCP>
-__global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc_q8(const float* __restrict__ x,
+template <bool RCP, typename TIn = float>
+__global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc_q8(const TIn* __restrict__ x,
                                                                 uint8_t* __restrict__ y,
                                                                 const FqChannel* __restrict__ tab,
                                                                 float lm1, float off, uint32_t hw,
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc_q8(const float* __re
             const uint32_t c = c0 + wave * 16 + cc + j;
             if (c < C && pix < hw) {
                 const FqChannel p = tab[c];
-                k[j] = fq_level_clamped<RCP>(p, lm1, x[(static_cast<int64_t>(n) * C + c) * hw + pix]);
+                k[j] = fq_level_clamped<RCP>(p, lm1, static_cast<float>(x[(static_cast<int64_t>(n) * C + c) * hw + pix]));
             } else {
                 k[j] = 0.0f;
             }
@@ -146,8 +146,15 @@ __global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc_q8(const float* __re
 
 // Image-like inputs (C <= 4) -> pixels of 4 bytes: a thread quantises 4 consecutive pixels of one
 // row from C coalesced float4 reads and writes 16 contiguous bytes.  W % 4 == 0.
-template <bool RCP>
-__global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc4_q8(const float* __restrict__ x,
+__device__ __forceinline__ float4 load4_as_float(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4_as_float(const uint8_t* p) {   // convert<uint8_t, float>: exact
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(p);
+    return make_float4(static_cast<float>(w & 0xffu), static_cast<float>((w >> 8) & 0xffu),
+                       static_cast<float>((w >> 16) & 0xffu), static_cast<float>(w >> 24));
+}
+
+template <bool RCP, typename TIn = float>
+__global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc4_q8(const TIn* __restrict__ x,
                                                                  uint8_t* __restrict__ y,
                                                                  const FqChannel* __restrict__ tab,
                                                                  float lm1, float off, uint32_t N, uint32_t C,
@@ -165,8 +172,7 @@ __global__ __launch_bounds__(kThreads) void fq_nchw_to_nhwc4_q8(const float* __r
         for (uint32_t c = 0; c < 4; ++c) {
             if (c < C) {
                 const FqChannel p = tab[c];
-                const float4 v = *reinterpret_cast<const float4*>(
-                    x + ((static_cast<int64_t>(n) * C + c) * H + h) * W + wq * 4);
+                const float4 v = load4_as_float(x + ((static_cast<int64_t>(n) * C + c) * H + h) * W + wq * 4);
                 k[0][c] = fq_level_clamped<RCP>(p, lm1, v.x);
                 k[1][c] = fq_level_clamped<RCP>(p, lm1, v.y);
                 k[2][c] = fq_level_clamped<RCP>(p, lm1, v.z);
@@ -260,6 +266,51 @@ struct hipie_fq {
     std::vector<FqChannel> host;
     DeviceBuffer table;
 };
+
+template <typename TIn>
+void run_q8_tensor(const hipie_fq* fq, const TIn* x, const hipie_tensor* out, void* stream) {
+    {
+        HIPIE_REQUIRE(fq && out, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: null argument");
+        HIPIE_REQUIRE(fq->table.ptr, HIPIE_NOT_ALLOCATED, "hipie_fq_run_q8_tensor: host-only object");
+        const int64_t hw = static_cast<int64_t>(out->h) * out->w;
+        if (out->n == 0 || hw == 0) return;
+        HIPIE_REQUIRE(x && out->data, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: null data");
+        HIPIE_REQUIRE(out->c == fq->C, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: %d channels, expected %lld",
+                      out->c, (long long)fq->C);
+        HIPIE_REQUIRE(fq->q8_ok && fq->clamp_ok, HIPIE_NOT_IMPLEMENTED,
+                      "hipie_fq_run_q8_tensor: needs input_low < input_high and consecutive integer output levels");
+        float off;
+        if (out->dtype == HIPIE_U8B) off = fq->q8_base - 128.0f;
+        else if (out->dtype == HIPIE_I8) off = fq->q8_base;
+        else fail(HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: output dtype %d", out->dtype);
+        HIPIE_REQUIRE(out->dtype == HIPIE_U8B ? fq->q8_base >= 0 : fq->q8_base + fq->lm1 <= 127.0f,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: levels do not fit the output type");
+        const int64_t cs = out->stride_w;
+        HIPIE_REQUIRE(cs >= fq->C && cs % 4 == 0 && reinterpret_cast<uintptr_t>(out->data) % 4 == 0 &&
+                          (cs % 16 != 0 || reinterpret_cast<uintptr_t>(out->data) % 16 == 0),
+                      HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: channel stride / alignment");
+        DeviceGuard g(fq->device);
+        if (fq->C <= 4 && cs == 4 && out->w % 4 == 0) {
+            auto k4 = fq->rcp ? fq_nchw_to_nhwc4_q8<true, TIn> : fq_nchw_to_nhwc4_q8<false, TIn>;
+            const int64_t work = static_cast<int64_t>(out->n) * out->h * (out->w / 4);
+            hipLaunchKernelGGL(k4, dim3(grid_for(work)), dim3(kThreads), 0, as_stream(stream), x,
+                               static_cast<uint8_t*>(out->data), fq->table.as<FqChannel>(), fq->lm1, off,
+                               static_cast<uint32_t>(out->n), static_cast<uint32_t>(fq->C),
+                               static_cast<uint32_t>(out->h), static_cast<uint32_t>(out->w), out->stride_n,
+                               out->stride_h);
+            HIPIE_CHECK_HIP(hipGetLastError());
+            return;
+        }
+        const uint32_t tiles = static_cast<uint32_t>(ceil_div(hw, 64));
+        auto k = fq->rcp ? fq_nchw_to_nhwc_q8<true, TIn> : fq_nchw_to_nhwc_q8<false, TIn>;
+        hipLaunchKernelGGL(k, dim3(static_cast<uint32_t>(out->n * tiles), static_cast<uint32_t>(ceil_div(cs, 64))),
+                           dim3(kThreads), 0, as_stream(stream), x, static_cast<uint8_t*>(out->data),
+                           fq->table.as<FqChannel>(), fq->lm1, off, static_cast<uint32_t>(hw),
+                           static_cast<uint32_t>(fq->C), static_cast<uint32_t>(cs), tiles,
+                           static_cast<uint32_t>(out->w), out->stride_n, out->stride_h);
+        HIPIE_CHECK_HIP(hipGetLastError());
+    }
+}
 
 extern "C" {
 
@@ -440,46 +491,13 @@ int hipie_fq_run_q8(const hipie_fq* fq, const float* x, void* y, int64_t n, int6
 }
 
 int hipie_fq_run_q8_tensor(const hipie_fq* fq, const float* x, const hipie_tensor* out, void* stream) {
+    return guarded([&] { run_q8_tensor(fq, x, out, stream); });
+}
+
+int hipie_fq_run_q8_tensor_u8(const hipie_fq* fq, const uint8_t* x, const hipie_tensor* out, void* stream) {
     return guarded([&] {
-        HIPIE_REQUIRE(fq && out, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: null argument");
-        HIPIE_REQUIRE(fq->table.ptr, HIPIE_NOT_ALLOCATED, "hipie_fq_run_q8_tensor: host-only object");
-        const int64_t hw = static_cast<int64_t>(out->h) * out->w;
-        if (out->n == 0 || hw == 0) return;
-        HIPIE_REQUIRE(x && out->data, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: null data");
-        HIPIE_REQUIRE(out->c == fq->C, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: %d channels, expected %lld",
-                      out->c, (long long)fq->C);
-        HIPIE_REQUIRE(fq->q8_ok && fq->clamp_ok, HIPIE_NOT_IMPLEMENTED,
-                      "hipie_fq_run_q8_tensor: needs input_low < input_high and consecutive integer output levels");
-        float off;
-        if (out->dtype == HIPIE_U8B) off = fq->q8_base - 128.0f;
-        else if (out->dtype == HIPIE_I8) off = fq->q8_base;
-        else fail(HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: output dtype %d", out->dtype);
-        HIPIE_REQUIRE(out->dtype == HIPIE_U8B ? fq->q8_base >= 0 : fq->q8_base + fq->lm1 <= 127.0f,
-                      HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: levels do not fit the output type");
-        const int64_t cs = out->stride_w;
-        HIPIE_REQUIRE(cs >= fq->C && cs % 4 == 0 && reinterpret_cast<uintptr_t>(out->data) % 4 == 0 &&
-                          (cs % 16 != 0 || reinterpret_cast<uintptr_t>(out->data) % 16 == 0),
-                      HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor: channel stride / alignment");
-        DeviceGuard g(fq->device);
-        if (fq->C <= 4 && cs == 4 && out->w % 4 == 0) {
-            auto k4 = fq->rcp ? fq_nchw_to_nhwc4_q8<true> : fq_nchw_to_nhwc4_q8<false>;
-            const int64_t work = static_cast<int64_t>(out->n) * out->h * (out->w / 4);
-            hipLaunchKernelGGL(k4, dim3(grid_for(work)), dim3(kThreads), 0, as_stream(stream), x,
-                               static_cast<uint8_t*>(out->data), fq->table.as<FqChannel>(), fq->lm1, off,
-                               static_cast<uint32_t>(out->n), static_cast<uint32_t>(fq->C),
-                               static_cast<uint32_t>(out->h), static_cast<uint32_t>(out->w), out->stride_n,
-                               out->stride_h);
-            HIPIE_CHECK_HIP(hipGetLastError());
-            return;
-        }
-        const uint32_t tiles = static_cast<uint32_t>(ceil_div(hw, 64));
-        auto k = fq->rcp ? fq_nchw_to_nhwc_q8<true> : fq_nchw_to_nhwc_q8<false>;
-        hipLaunchKernelGGL(k, dim3(static_cast<uint32_t>(out->n * tiles), static_cast<uint32_t>(ceil_div(cs, 64))),
-                           dim3(kThreads), 0, as_stream(stream), x, static_cast<uint8_t*>(out->data),
-                           fq->table.as<FqChannel>(), fq->lm1, off, static_cast<uint32_t>(hw),
-                           static_cast<uint32_t>(fq->C), static_cast<uint32_t>(cs), tiles,
-                           static_cast<uint32_t>(out->w), out->stride_n, out->stride_h);
-        HIPIE_CHECK_HIP(hipGetLastError());
+        HIPIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 4 == 0, HIPIE_PARAMETER_MISMATCH, "hipie_fq_run_q8_tensor_u8: unaligned input");
+        run_q8_tensor(fq, x, out, stream);
     });
 }
 

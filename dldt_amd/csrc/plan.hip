@@ -145,6 +145,7 @@ void check_status(int st, const char* what) {
 // FakeQuantize on a graph input: f32 NCHW in the request's input buffer -> byte NHWC tensor
 struct EntryStep : Step {
     int param_index = 0, out = -1;
+    bool u8_in = false;            // the request input holds u8 values (Parameter u8 -> Convert f32 -> FakeQuantize)
     int64_t channels = 0, levels = 0;
     std::vector<float> il, ih, ol, oh;
     hipie_fq* fq = nullptr;
@@ -156,7 +157,8 @@ struct EntryStep : Step {
     void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
              hipStream_t s) const override {
         const hipie_tensor d = tensors[out].desc(arena);
-        check_status(hipie_fq_run_q8_tensor(fq, static_cast<const float*>(inputs[param_index]), &d, s),
+        check_status(u8_in ? hipie_fq_run_q8_tensor_u8(fq, static_cast<const uint8_t*>(inputs[param_index]), &d, s)
+                           : hipie_fq_run_q8_tensor(fq, static_cast<const float*>(inputs[param_index]), &d, s),
                      name.c_str());
     }
 };
@@ -1399,9 +1401,12 @@ struct Planner {
         const Value& x = value(n.in[0]);
         if (x.kind != VK_PARAM) unsupported(id, "stand-alone FakeQuantize is only planned on graph inputs");
         if (n.dtype == HIPIE_F32) unsupported(id, "FakeQuantize with f32 output (graph was not run through LPT)");
-        const GNode& p = N(n.in[0]);
-        HIPIE_REQUIRE(p.dtype == HIPIE_F32, HIPIE_NOT_IMPLEMENTED, "u8 graph inputs are not planned yet");
+        const int param = N(n.in[0]).op == OP_CONVERT ? N(n.in[0]).in[0] : n.in[0];
+        const GNode& p = N(param);
+        HIPIE_REQUIRE(p.op == OP_PARAMETER && (p.dtype == HIPIE_F32 || (p.dtype == HIPIE_U8 && param != n.in[0])),
+                      HIPIE_NOT_IMPLEMENTED, "node %d: a u8 graph input needs a Convert to f32 in front of its FakeQuantize", id);
         auto st = std::make_unique<EntryStep>();
+        st->u8_in = p.dtype == HIPIE_U8;
         int nn, c, h, w;
         nhwc_dims(n.shape, nn, c, h, w);
         st->channels = c;
@@ -1411,15 +1416,16 @@ struct Planner {
             if (!channel_constant(n.in[1 + i], c, n.shape.size(), *dst[i]))
                 unsupported(id, "FakeQuantize bounds must be scalars or per-channel constants");
         for (size_t i = 0; i < g.params.size(); ++i)
-            if (g.params[i] == n.in[0]) st->param_index = static_cast<int>(i);
+            if (g.params[i] == param) st->param_index = static_cast<int>(i);
         // small-channel images keep a 4-byte pixel so the first convolution reads filter rows contiguously
         st->out = new_tensor(id, storage_type(n.dtype), nn, h, w, c, c <= 4 ? 4 : 0);
         st->name = n.name;
         st->type = "FakeQuantize";
-        st->bytes = n.numel() * 5;
+        st->bytes = n.numel() * (st->u8_in ? 2 : 5);
         st->out_node = id;
         values[id].kind = VK_TENSOR;
         values[id].tensor = st->out;
+        if (param != n.in[0]) values[n.in[0]].kind = VK_FUSED;
         steps.push_back(std::move(st));
     }
 
@@ -1427,6 +1433,10 @@ struct Planner {
         const GNode& n = N(id);
         const Value& x = value(n.in[0]);
         Value v;
+        if (n.op == OP_CONVERT && x.kind == VK_PARAM && N(n.in[0]).dtype == HIPIE_U8 && n.dtype == HIPIE_F32) {
+            values[id].kind = VK_PARAM;   // a u8 graph input seen as f32: read where the FakeQuantize behind it runs
+            return;
+        }
         if (n.op == OP_CONVERT) {
             if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1 || n.dtype != HIPIE_F32)
                 unsupported(id, "Convert is planned only as the start of a dequantization (u8/i8 -> f32)");

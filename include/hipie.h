@@ -120,6 +120,10 @@ int hipie_fq_run_q8(const hipie_fq* fq, const float* x, void* y, int64_t n, int6
 /* same as hipie_fq_run_q8 with NHWC output, but into an engine tensor (any strides / halo);
  * this is how a graph input enters the arena */
 int hipie_fq_run_q8_tensor(const hipie_fq* fq, const float* x, const hipie_tensor* out, void* stream);
+/* the same for an input blob of precision U8 (what benchmark_app feeds image inputs): the u8 -> f32
+ * Convert in front of the FakeQuantize (reference::convert<uint8_t, float>, as the template plugin's
+ * blobCopy does, docs/template_plugin/src/template_infer_request.cpp:115-129) happens in the kernel */
+int hipie_fq_run_q8_tensor_u8(const hipie_fq* fq, const uint8_t* x, const hipie_tensor* out, void* stream);
 
 /* host evaluation of exactly the arithmetic the device kernel uses (reciprocal multiply with
  * two FMA corrections); the planner checks it against IEEE division at every level boundary of
@@ -329,7 +333,7 @@ int hipie_transpose_bytes_nested(const void* src, int64_t ld_src, int64_t stride
  *    (ngraph/core/include/ngraph/function.hpp:126) of the post-LPT function and issues one call
  *    per node; value ids are returned in creation order.  Shapes are the reference's (NCHW,
  *    OIHW, [N, C]); element types are the node's output types (TypeRelaxed ops included).
- *    Supported nodes: Parameter(f32), Constant, FakeQuantize, Convolution, GroupConvolution,
+ *    Supported nodes: Parameter(f32; u8 behind a Convert to f32; i32 token ids), Constant, FakeQuantize, Convolution, GroupConvolution,
  *    MatMul, Add, Multiply, Subtract, Relu, Clamp, Convert, MaxPool, AvgPool, Reshape, Result, and
  *    for transformer encoders (rank-3 Parameter [batch, sequence, hidden]): MatMul between two
  *    activations, Softmax, MVN, Gelu, Transpose, and Gather of a constant table by an i32

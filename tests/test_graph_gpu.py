@@ -125,3 +125,20 @@ def test_requests_in_flight_do_not_disturb_each_other():
         torch.cuda.ExternalStream(r.stream).synchronize()
     for (_, outs), w in zip(bufs, want):
         np.testing.assert_array_equal(outs[0].cpu().numpy().view(np.uint32), w.view(np.uint32))
+
+
+@pytest.mark.parametrize("c,hw", [(64, 56), (3, 32), (20, 9)])
+def test_u8_graph_input(orc, c, hw):
+    """input precision U8: Parameter(u8) -> Convert(f32) -> FakeQuantize runs as one entry kernel that
+    reads the bytes (image-like 4-byte pixels, 64-channel tiles, ragged channels and widths)"""
+    from dldt_amd import builders
+    g, feeds, _ = builders.conv_block(seed=5, n=2, c=c, hw=hw, oc=32, u8_input=True)
+    want, _ = evaluate(orc, g.nodes, feeds)
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps] == ["FakeQuantize", "Convolution", "Result"]
+    assert plan.inputs[0]["dtype"] == 40
+    req = plan.create_request()
+    (got,) = req.infer(feeds["data"])
+    np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))
+    q_node = next(i for i, n in enumerate(g.nodes) if n["op"] == "FakeQuantize")
+    np.testing.assert_array_equal(req.tensor(q_node), feeds["data"])       # levels 0 .. 255 are the input bytes
