@@ -53,12 +53,13 @@ __device__ __forceinline__ uint32_t prob_levels4(const AttentionArgs& a, float p
     return a.p_add ? add_bytes(w, a.p_add) : (w ^ a.p_xor);
 }
 
-template <int NT, bool DIV2>   // NT = S / 32 key tiles
+template <int NT, bool DIV2, bool MASK>   // NT = S / 32 key tiles
 __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a) {
     constexpr int S = NT * 32;
     constexpr int VT_LD = S + 16;                     // odd number of 16-byte groups per row: conflict-free
     __shared__ __attribute__((aligned(16))) int8_t sK[S * 64];       // [key][d], chunk c of row r in slot c ^ ((r >> 2) & 3)
     __shared__ __attribute__((aligned(16))) int8_t sVT[64 * VT_LD];  // [d][tile][half][j]: key 32 t + 8 (j / 4) + 4 half + j % 4
+    __shared__ __attribute__((aligned(16))) float sMask[MASK ? S : 4];    // the sequence's mask row
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, h = lane >> 5;
@@ -91,6 +92,11 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
         for (int e = 0; e < 4; ++e) *reinterpret_cast<uint32_t*>(&sVT[(4 * d4 + e) * VT_LD + col]) = t[e];
     }
 
+    if constexpr (MASK) {
+        const float* mrow = a.mask + bo * a.mask_outer + bi * a.mask_inner;
+        for (int i = tid; i < S; i += 256) sMask[i] = mrow[i];
+    }
+
     // ---- this wave's queries: the column operand of the first product, straight from memory ------
     const int q_row = blockIdx.x * 128 + wave * 32 + l32;
     const bool q_ok = q_row < a.S;
@@ -99,7 +105,6 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
     __syncthreads();
 
     const int slot[2] = {((0 + h) ^ ((l32 >> 2) & 3)) * 16, ((2 + h) ^ ((l32 >> 2) & 3)) * 16};
-    const float* mrow = a.mask ? a.mask + bo * a.mask_outer + bi * a.mask_inner : nullptr;
     float x[NT][16];
     float m = -INFINITY;
 #pragma unroll
@@ -112,17 +117,20 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
         }
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            float4 mk = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (mrow) mk = *reinterpret_cast<const float4*>(mrow + 32 * t + 8 * g + 4 * h);
-            const float mv[4] = {mk.x, mk.y, mk.z, mk.w};
+            float mv[4] = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (MASK) {
+                const float4 mk = *reinterpret_cast<const float4*>(&sMask[32 * t + 8 * g + 4 * h]);
+                mv[0] = mk.x; mv[1] = mk.y; mv[2] = mk.z; mv[3] = mk.w;
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 float v = static_cast<float>(acc[4 * g + j]) * a.scale1;
-                if (mrow) v = v + mv[j];                 // the mask Add between the Multiply and the Softmax
+                if constexpr (MASK) v = v + mv[j];       // the mask Add between the Multiply and the Softmax
                 x[t][4 * g + j] = v;
                 m = fmaxf(m, v);
             }
         }
+        if constexpr (MASK) __builtin_amdgcn_sched_barrier(0);   // keep the mask reads next to their tile
     }
     const int64_t dump_row = (static_cast<int64_t>(b) * a.S + q_row) * a.S;   // [batch][query][key]
     if (a.scores && q_ok) {
@@ -185,8 +193,13 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
 template <int NT>
 void launch(const AttentionArgs& a, int batches, hipStream_t s) {
     const dim3 grid(static_cast<uint32_t>(ceil_div(a.S, 128)), static_cast<uint32_t>(batches));
-    if (a.p_div2) hipLaunchKernelGGL((attention_kernel<NT, true>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((attention_kernel<NT, false>), grid, dim3(256), 0, s, a);
+    if (a.mask) {
+        if (a.p_div2) hipLaunchKernelGGL((attention_kernel<NT, true, true>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((attention_kernel<NT, false, true>), grid, dim3(256), 0, s, a);
+    } else {
+        if (a.p_div2) hipLaunchKernelGGL((attention_kernel<NT, true, false>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((attention_kernel<NT, false, false>), grid, dim3(256), 0, s, a);
+    }
 }
 
 }  // namespace

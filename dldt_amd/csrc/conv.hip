@@ -14,8 +14,13 @@ constexpr int kRow = 64;  // LDS rows of the tiled kernels: 64 K-bytes, chunk c 
 
 // ------------------------------------------------------------------------------------------------
 // LDS-tiled kernel
-template <int WOC, int WPIX, uint32_t F>
-__global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && (F & CF_RES_GEMM))) ? (F == kDyn ? 3 : 4) : 2) void conv_tiled_kernel(const ConvArgs a) {
+// PAIR: the operands of two 64-byte K steps are requested together, eight lanes per row, so that a row's
+// 128-byte cache line crosses the L2 -> L1 path once instead of once per step (with four workgroups on a
+// compute unit the lines of one step, 128 KB, do not survive in the 32 KB L1 until the next step asks
+// for their other half: the operand loads alone run 1.4 times faster this way).  The two LDS buffers
+// then hold the two steps of a pair instead of alternating.
+template <int WOC, int WPIX, uint32_t F, bool PAIR = false>
+__global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && (F & CF_RES_GEMM))) ? ((F == kDyn || PAIR) ? 3 : 4) : 2) void conv_tiled_kernel(const ConvArgs a) {
     constexpr int NT = WOC * WPIX * 64;
     constexpr int BOC = WOC * 64, BPIX = WPIX * 64;
     constexpr int A_PIECES = BOC * 4 / NT, B_PIECES = BPIX * 4 / NT;
@@ -77,6 +82,89 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
             row = min(oc0 + row, wgt_rows - 1);
             a_ptr[i] = wgt_base + static_cast<int64_t>(row) * wgt_ld + chunk * 16;
         }
+        auto mfma_step = [&](int buf) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                v4i af[2], bf[2];
+#pragma unroll
+                for (int ob = 0; ob < 2; ++ob)
+                    af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][a_row[ob] * kRow + frag_slot[ks]]);
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+                    bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][b_row[pb] * kRow + frag_slot[ks]]);
+#pragma unroll
+                for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                    for (int pb = 0; pb < 2; ++pb)
+                        acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
+            }
+        };
+        if constexpr (PAIR) {
+            static_assert(NT == 256, "eight lanes per row, 32 rows per load instruction");
+            constexpr int RPI = NT / 8, A_P2 = BOC / RPI, B_P2 = BPIX / RPI;
+            const int sub = (tid >> 2) & 1, row0 = tid >> 3;          // chunk tid & 3 of step 2 j + sub, rows row0 + i RPI
+            const int slot2 = (chunk ^ ((tid >> 5) & 3)) * 16;        // RPI is a multiple of 16: one swizzle per thread
+            int32_t b_base2[B_P2];
+            const int8_t* a_ptr2[A_P2];
+#pragma unroll
+            for (int i = 0; i < B_P2; ++i) {
+                int m = pix0 + row0 + i * RPI;
+                m = m < a.M ? m : a.M - 1;
+                const PixelCoord p = decode_pixel(a, m);
+                b_base2[i] = p.n * in_sn + p.oh * csh * in_sh + p.ow * csw * in_sw + origin;
+            }
+#pragma unroll
+            for (int i = 0; i < A_P2; ++i) {
+                int row = row0 + i * RPI;
+                if (wgt_plain) {
+                    const int j = row & 31;
+                    row = (row & ~63) + 32 * ((j >> 2) & 1) + 16 * ((row >> 5) & 1) + 4 * (j >> 3) + (j & 3);
+                }
+                row = min(oc0 + row, wgt_rows - 1);
+                a_ptr2[i] = wgt_base + static_cast<int64_t>(row) * wgt_ld + chunk * 16;
+            }
+            v4i ga2[A_P2], gb2[B_P2];
+            auto load_pair = [&](int j) {
+                // an odd step count leaves the last pair half empty: its second half re-reads the last step
+                // (in bounds, never multiplied)
+                const int k0 = 2 * j, k1 = min(2 * j + 1, nk - 1);
+                const int4 ko0 = *reinterpret_cast<const int4*>(koff + 4 * k0);   // uniform: scalar loads
+                const int4 ko1 = *reinterpret_cast<const int4*>(koff + 4 * k1);
+                const int4 ko = sub ? ko1 : ko0;
+                const int32_t off = chunk == 0 ? ko.x : (chunk == 1 ? ko.y : (chunk == 2 ? ko.z : ko.w));
+                const int kk = sub ? k1 : k0;
+#pragma unroll
+                for (int i = 0; i < A_P2; ++i) ga2[i] = *reinterpret_cast<const v4i*>(a_ptr2[i] + kk * 64);
+#pragma unroll
+                for (int i = 0; i < B_P2; ++i) gb2[i] = *reinterpret_cast<const v4i*>(in_base + (b_base2[i] + off));
+            };
+            auto store_pair = [&]() {
+#pragma unroll
+                for (int i = 0; i < A_P2; ++i)
+                    *reinterpret_cast<v4i*>(&sA[sub][(row0 + i * RPI) * kRow + slot2]) = ga2[i];
+#pragma unroll
+                for (int i = 0; i < B_P2; ++i)
+                    *reinterpret_cast<v4i*>(&sB[sub][(row0 + i * RPI) * kRow + slot2]) = gb2[i];
+            };
+            const int npairs = (nk + 1) >> 1;
+            load_pair(0);
+            store_pair();
+            if (first) stage_params_store<F>(a, (lds_float_ptr)sP, BOC, tid, staged);
+            __syncthreads();
+            if (acc_from_lds) init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);
+            for (int j = 0; j < npairs; ++j) {
+                const bool more = j + 1 < npairs;
+                if (more) load_pair(j + 1);
+                mfma_step(0);
+                if (2 * j + 1 < nk) mfma_step(1);
+                __syncthreads();             // every wave has read this pair
+                if (more) {
+                    store_pair();
+                    __syncthreads();
+                }
+            }
+            return;
+        }
         v4i ga[A_PIECES], gb[B_PIECES];
         auto load_global = [&](int k) {
             const int4 ko = *reinterpret_cast<const int4*>(koff + 4 * k);   // uniform: scalar load
@@ -102,21 +190,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
         for (int k = 0; k < nk; ++k) {
             const int buf = k & 1;
             if (k + 1 < nk) load_global(k + 1);
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                v4i af[2], bf[2];
-#pragma unroll
-                for (int ob = 0; ob < 2; ++ob)
-                    af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][a_row[ob] * kRow + frag_slot[ks]]);
-#pragma unroll
-                for (int pb = 0; pb < 2; ++pb)
-                    bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][b_row[pb] * kRow + frag_slot[ks]]);
-#pragma unroll
-                for (int ob = 0; ob < 2; ++ob)
-#pragma unroll
-                    for (int pb = 0; pb < 2; ++pb)
-                        acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
-            }
+            mfma_step(buf);
             if (k + 1 < nk) store_lds(buf ^ 1);
             __syncthreads();
         }
@@ -125,6 +199,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     v16i acc[2][2];
     v16f rres[2][2];
     constexpr bool kFused = F != kDyn && (F & CF_RES_GEMM);
+    static_assert(!(kFused && PAIR), "the second GEMM keeps the single-step loop");
     if (kFused) {
         // shortcut convolution first: (float(acc2) + bias2[c]) * scale2[c] stays in registers
         ConvArgs a2 = a;
@@ -709,6 +784,20 @@ void launch_persist(const ConvArgs& a, hipStream_t s) {
     }
 }
 
+// the same tiles with the operands of two K steps requested together
+template <int WOC, int WPIX>
+void launch_tiled_pair(const ConvArgs& a, hipStream_t s, int batches = 1) {
+    const dim3 grid(a.p_per_xcd > 0 ? 8 * a.p_per_xcd * a.t_tiles : a.p_tiles * a.t_tiles, batches), block(WOC * WPIX * 64);
+    const uint32_t core = a.flags & ~CF_OUT_XOR;
+#define HIPIE_LAUNCH_PAIR(FLAGS, ...)                                                                  \
+    do {                                                                                               \
+        if constexpr ((FLAGS) != kDyn && ((FLAGS) & CF_RES_GEMM)) break;                                \
+        else hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, FLAGS, true>), grid, block, 0, s, a);    \
+    } while (0)
+    HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_PAIR, 0)
+#undef HIPIE_LAUNCH_PAIR
+}
+
 void launch_tiled_small(const ConvArgs& a, hipStream_t s) {   // 64 x 64 tile, one wave per workgroup
     const dim3 grid(a.p_per_xcd > 0 ? 8 * a.p_per_xcd * a.t_tiles : a.p_tiles * a.t_tiles), block(64);
     const uint32_t core = a.flags & ~CF_OUT_XOR;
@@ -1160,10 +1249,10 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 9, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 11, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
         if (c->depthwise) return;               // one kernel only
         if (c->fused && tile != 0 && tile != 4) return;   // the second GEMM exists in the 128 x 128 kernels
-        HIPIE_REQUIRE(tile < 8 || (!c->fused && persist_available(c->epi.flags)), HIPIE_PARAMETER_MISMATCH,
+        HIPIE_REQUIRE(tile < 8 || tile > 9 || (!c->fused && persist_available(c->epi.flags)), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the persistent kernels exist for byte outputs with a byte residual or none");
         HIPIE_REQUIRE(tile < 6 || tile > 7 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the split-K kernels need an even number of 64-byte K steps (K=%lld)", (long long)c->Kp);
@@ -1328,7 +1417,7 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
             return;
         }
         const int tile = c->tile;
-        const bool square = tile == 0 || tile == 4 || tile == 6 || tile == 8;
+        const bool square = tile == 0 || tile == 4 || tile == 6 || tile == 8 || tile == 10;
         const int boc = square ? 128 : 64;
         const int bpix = square ? 128 : (tile == 2 ? 64 : 256);
         a.p_tiles = static_cast<int32_t>(ceil_div(M, bpix));
@@ -1354,6 +1443,8 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         case 0: launch_tiled<2, 2>(a, s); break;
         case 1: launch_tiled<1, 4>(a, s); break;
         case 2: launch_tiled_small(a, s); break;
+        case 10: launch_tiled_pair<2, 2>(a, s); break;
+        case 11: launch_tiled_pair<1, 4>(a, s); break;
         default: {
             // persistent workgroups: as many as fit per CU by LDS (at most 4), spread over the
             // channel tiles; a multiple of 8 so that sibling channel tiles share an XCD
