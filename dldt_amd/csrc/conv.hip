@@ -721,6 +721,7 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
     case E_SCALE: X(E_SCALE, __VA_ARGS__); break;                                            \
     case E_SCALEFQ: X(E_SCALEFQ, __VA_ARGS__); break;                                        \
     case E_DEQFQ: X(E_DEQFQ, __VA_ARGS__); break;                                            \
+    case E_GELUFQ: X(E_GELUFQ, __VA_ARGS__); break;                                          \
     case E_RESI8: X(E_RESI8, __VA_ARGS__); break;                                            \
     case E_F32RES: X(E_F32RES, __VA_ARGS__); break;                                          \
     case E_F32RELU: X(E_F32RELU, __VA_ARGS__); break;                                        \
@@ -850,6 +851,7 @@ void Epilogue::build(int device_, const hipie_epilogue& e, int64_t oc, int64_t o
     if (e.post_scale) { vec(e.post_scale, e.n_post_scale, 1.f, "post_scale", h); up(post_scale, h); flags |= CF_POST_SCALE; }
     if (e.activation == 1) flags |= CF_RELU;
     else if (e.activation == 2) { flags |= CF_CLAMP; clamp_lo = e.clamp_lo; clamp_hi = e.clamp_hi; }
+    else if (e.activation == 3) flags |= CF_GELU;
     else HIPIE_REQUIRE(e.activation == 0, HIPIE_PARAMETER_MISMATCH, "epilogue: activation %d", e.activation);
     out_dtype = e.out_dtype;
     switch (e.out_dtype) {

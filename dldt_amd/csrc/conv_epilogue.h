@@ -4,6 +4,7 @@
 // oc_lane + 16*ob + r of pixel pb.
 #pragma once
 #include "conv_kernel.h"
+#include "gelu.h"
 #include "fq_math.h"
 
 namespace hipie {
@@ -117,6 +118,7 @@ constexpr uint32_t E_RESI8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_MUL | E_FQ;   
 constexpr uint32_t E_SCALEFQ = CF_BIAS | CF_SCALE | E_FQ;              // linear layer requantised to symmetric i8
 constexpr uint32_t E_F32RES = CF_BIAS | CF_SCALE | CF_RES | CF_RES_F32;   // linear layer + f32 residual, f32 out                      // MatMul' -> Multiply(s_a * s_b)
 constexpr uint32_t E_F32RELU = CF_BIAS | CF_SCALE | CF_RELU;
+constexpr uint32_t E_GELUFQ = CF_BIAS | CF_SCALE | CF_GELU | E_FQ;       // FFN up projection: Gelu and the next FakeQuantize in the GEMM
 constexpr uint32_t E_DEQFQ = CF_SCALE | E_FQ;                           // MatMul between activations, requantised (attention context)
 constexpr uint32_t E_CLAMPFQ = CF_BIAS | CF_SCALE | CF_CLAMP | E_FQ | CF_FQ_IL0;
 
@@ -298,7 +300,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
     // an f32 residual that is the last operation in front of the store is added where the staged rows
     // are read back: there a lane's residual piece is as contiguous as its store
     constexpr bool kLateRes = kCanStage && (F & CF_RES) && (F & CF_RES_F32) &&
-                              !(F & (CF_RES_SUB | CF_RES_MUL | CF_POST_SCALE | CF_RELU | CF_CLAMP | CF_RES_GEMM));
+                              !(F & (CF_RES_SUB | CF_RES_MUL | CF_POST_SCALE | CF_RELU | CF_CLAMP | CF_GELU | CF_RES_GEMM));
     const bool late_res = kLateRes && staged_out;
     const int lane_id = static_cast<int>(threadIdx.x) & 63;
     auto tab = [&](int t, const float* g, int oc) {
@@ -421,6 +423,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
                 if (fl & CF_POST_SCALE) x = x * post_[j];
                 if (fl & CF_RELU) x = x > 0.0f ? x : 0.0f;
                 if (fl & CF_CLAMP) x = x < a.clamp_lo ? a.clamp_lo : (x > a.clamp_hi ? a.clamp_hi : x);
+                if (fl & CF_GELU) x = gelu_one(x);
                 v[pb][j] = x;
             }
         }

@@ -45,6 +45,7 @@ enum ConvFlags : uint32_t {
     CF_FQ_IL0 = 1u << 13,     // every input_low is +0: x - il == x
     CF_OUT_XOR = 1u << 14,    // packed levels ^ 0x80808080 is the stored byte (offset -128)
     CF_FQ_DIV2 = 1u << 16,    // two-operation division by the channel constant: fma(n, fq_r, n * fq_r2), verified at load time
+    CF_GELU = 1u << 17,       // v = gelu(v), ERF mode (after scale / residual, in place of relu / clamp)
     CF_RES_GEMM = 1u << 15,   // residual = (float(acc2) + bias2[c]) * scale2[c] of a second GEMM run in the same kernel
 };
 

@@ -1018,6 +1018,10 @@ struct Planner {
                 } else {
                     break;
                 }
+            } else if (u.op == OP_GELU && stage < 5 && !keep_f32 && single_user(nx) && N(N(nx).users[0]).op == OP_FAKE_QUANTIZE &&
+                       N(N(nx).users[0]).dtype == HIPIE_I8) {
+                e.activation = 3;   // Gelu and the FakeQuantize behind it ride in the GEMM: its f32 result is never stored
+                stage = 5;
             } else if (u.op == OP_FAKE_QUANTIZE && u.in[0] == cur && u.dtype == HIPIE_I8) {
                 std::vector<float> ol, oh;
                 if (!last_axis_constant(u.in[1], OC, e.fq_il) || !last_axis_constant(u.in[2], OC, e.fq_ih) ||

@@ -146,7 +146,7 @@ int hipie_fq_div2_constants(int device, const float* d, int64_t n, float* zh, fl
  *        v = v * scale[c]                   dequantization Multiply (convolution.cpp:249-258)
  *        r = float(residual); r -= res_sub[c]; r *= res_mul[c]; v = v + r     (add.cpp:154-218)
  *        v = v * post_scale[c]
- *        relu | clamp(lo, hi)               relu.hpp, clamp.hpp
+ *        relu | clamp(lo, hi) | gelu        relu.hpp, clamp.hpp, gelu.hpp (same float as hipie_gelu_f32)
  *        FakeQuantize(in_low[c], in_high[c], out_low, out_high, levels) -> 8-bit     or f32 store
  *     Arrays are host pointers with 1 (broadcast) or OC values; NULL skips the step.
  * ==================================================================================== */
@@ -160,7 +160,7 @@ typedef struct hipie_epilogue {
     const float* res_sub;     int64_t n_res_sub;
     const float* res_mul;     int64_t n_res_mul;
     const float* post_scale;  int64_t n_post_scale;
-    int32_t activation;       /* 0 none, 1 relu, 2 clamp */
+    int32_t activation;       /* 0 none, 1 relu, 2 clamp, 3 gelu (ERF mode; tolerance parity like hipie_gelu_f32) */
     float clamp_lo, clamp_hi;
     int32_t out_dtype;        /* HIPIE_F32, HIPIE_U8B, HIPIE_I8, or HIPIE_I32 (raw accumulators) */
     int64_t fq_levels;

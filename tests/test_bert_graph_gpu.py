@@ -67,10 +67,10 @@ def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq, fuse_
     (y2,) = req2.infer(x)
     np.testing.assert_array_equal(y2.view(np.uint32), y.view(np.uint32))
     for li, L in enumerate(meta["layers"]):
-        stored = ("q", "k", "v", "ctxq", "attn", "h1q", "up", "gq", "down") + (() if fuse_attention else ("scores", "pq"))
+        stored = ("q", "k", "v", "ctxq", "attn", "h1q", "gq", "down") + (() if fuse_attention else ("scores", "pq"))
         for name in stored:
             np.testing.assert_array_equal(req2.matrix(L[name]), req.matrix(L[name]), err_msg="layer %d %s" % (li, name))
-        for name in ("p", "ctx", "gelu") + (("scores", "pq") if fuse_attention else ()):
+        for name in ("p", "ctx", "up", "gelu") + (("scores", "pq") if fuse_attention else ()):
             with pytest.raises(Exception):
                 req2.matrix(L[name])
     return plan2, req2, x, y

@@ -120,7 +120,7 @@ def test_planner_encoder_stack_steps_and_views(monkeypatch):
     plan = Plan(g, device=-1)
     types = [s["type"] for s in plan.steps]
     attention = ["MatMul", "Attention", "MatMul"]          # Q, K, V projections as one GEMM; the core; the output projection
-    ffn = ["MVN+FakeQuantize", "MatMul", "Gelu+FakeQuantize", "MatMul"]
+    ffn = ["MVN+FakeQuantize", "MatMul", "MatMul"]         # Gelu and its FakeQuantize ride in the up projection
     # every activation FakeQuantize but the first rides in the kernel that produces its input
     assert types == ["FakeQuantize"] + attention + ffn + ["MVN+FakeQuantize"] + attention + ffn + ["MVN", "Result"]
     assert sum(s["macs"] for s in plan.steps) == meta["macs"]
