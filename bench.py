@@ -64,8 +64,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU (requests are independent; see DESIGN.md for "
-                 "how the path shards); --gpus %d is not supported" % args.gpus)
+        sys.exit("bench.py: this build runs on one GPU (infer requests are independent, so more GPUs would each "
+                 "run their own plan and requests); --gpus %d is not supported" % args.gpus)
     import numpy as np
     import torch
     from dldt_amd import builders
