@@ -64,7 +64,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
                     const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk,
                     v16i (&acc)[2][2], bool first, bool acc_from_lds) {
         int32_t b_base[B_PIECES];
-        const int8_t* a_ptr[A_PIECES];
+        uint32_t a_off[A_PIECES];                          // unsigned: added to the uniform base by the load itself
 #pragma unroll
         for (int i = 0; i < B_PIECES; ++i) {
             int m = pix0 + ((tid + i * NT) >> 2);
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
                 row = (row & ~63) + 32 * ((j >> 2) & 1) + 16 * ((row >> 5) & 1) + 4 * (j >> 3) + (j & 3);
             }
             row = min(oc0 + row, wgt_rows - 1);
-            a_ptr[i] = wgt_base + static_cast<int64_t>(row) * wgt_ld + chunk * 16;
+            a_off[i] = static_cast<uint32_t>(row) * static_cast<uint32_t>(wgt_ld) + chunk * 16;
         }
         auto mfma_step = [&](int buf) {
 #pragma unroll
@@ -128,10 +128,15 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
                 // an odd step count leaves the last pair half empty: its second half re-reads the last step
                 // (in bounds, never multiplied)
                 const int k0 = 2 * j, k1 = min(2 * j + 1, nk - 1);
-                const int4 ko0 = *reinterpret_cast<const int4*>(koff + 4 * k0);   // uniform: scalar loads
-                const int4 ko1 = *reinterpret_cast<const int4*>(koff + 4 * k1);
-                const int4 ko = sub ? ko1 : ko0;
-                const int32_t off = chunk == 0 ? ko.x : (chunk == 1 ? ko.y : (chunk == 2 ? ko.z : ko.w));
+                int4 ko0 = *reinterpret_cast<const int4*>(koff + 4 * k0);   // uniform: scalar loads, taken as wave-uniform values
+                int4 ko1 = *reinterpret_cast<const int4*>(koff + 4 * k1);
+                ko0.x = __builtin_amdgcn_readfirstlane(ko0.x); ko0.y = __builtin_amdgcn_readfirstlane(ko0.y);
+                ko0.z = __builtin_amdgcn_readfirstlane(ko0.z); ko0.w = __builtin_amdgcn_readfirstlane(ko0.w);
+                ko1.x = __builtin_amdgcn_readfirstlane(ko1.x); ko1.y = __builtin_amdgcn_readfirstlane(ko1.y);
+                ko1.z = __builtin_amdgcn_readfirstlane(ko1.z); ko1.w = __builtin_amdgcn_readfirstlane(ko1.w);
+                const int32_t off0 = chunk == 0 ? ko0.x : (chunk == 1 ? ko0.y : (chunk == 2 ? ko0.z : ko0.w));
+                const int32_t off1 = chunk == 0 ? ko1.x : (chunk == 1 ? ko1.y : (chunk == 2 ? ko1.z : ko1.w));
+                const int32_t off = sub ? off1 : off0;
                 const int kk = sub ? k1 : k0;
 #pragma unroll
                 for (int i = 0; i < A_P2; ++i) ga2[i] = *reinterpret_cast<const v4i*>(a_ptr2[i] + kk * 64);
@@ -167,10 +172,15 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
         }
         v4i ga[A_PIECES], gb[B_PIECES];
         auto load_global = [&](int k) {
-            const int4 ko = *reinterpret_cast<const int4*>(koff + 4 * k);   // uniform: scalar load
+            int4 ko = *reinterpret_cast<const int4*>(koff + 4 * k);   // uniform: one scalar load of the step's four offsets
+            // taken as wave-uniform values: otherwise the select below becomes three divergent branches,
+            // each with its own scalar load and wait in front of the vector loads
+            ko.x = __builtin_amdgcn_readfirstlane(ko.x); ko.y = __builtin_amdgcn_readfirstlane(ko.y);
+            ko.z = __builtin_amdgcn_readfirstlane(ko.z); ko.w = __builtin_amdgcn_readfirstlane(ko.w);
             const int32_t off = chunk == 0 ? ko.x : (chunk == 1 ? ko.y : (chunk == 2 ? ko.z : ko.w));
+            const int8_t* wk = wgt_base + k * 64;                     // uniform part of the weight address
 #pragma unroll
-            for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(a_ptr[i] + k * 64);
+            for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(wk + a_off[i]);
 #pragma unroll
             for (int i = 0; i < B_PIECES; ++i) gb[i] = *reinterpret_cast<const v4i*>(in_base + (b_base[i] + off));
         };
