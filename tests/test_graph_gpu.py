@@ -142,3 +142,48 @@ def test_u8_graph_input(orc, c, hw):
     np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))
     q_node = next(i for i, n in enumerate(g.nodes) if n["op"] == "FakeQuantize")
     np.testing.assert_array_equal(req.tensor(q_node), feeds["data"])       # levels 0 .. 255 are the input bytes
+
+
+def test_compile_and_infer_from_many_threads(orc):
+    """LoadNetwork and Infer are called concurrently from many threads (behavior/core_threading_tests.hpp):
+    four host threads each compile their own plan of the same graph and run host-path inferences on their
+    own requests at the same time; a fifth provokes errors meanwhile (the error text is per thread).
+    Every result equals the single-threaded one."""
+    import threading
+    from dldt_amd import HipieError, builders
+    from dldt_amd.graph import Graph
+    g, _ = builders.resnet50(batch=2, res=64, width=16, classes=10, seed=7)
+    rng = np.random.default_rng(8)
+    xs = [rng.uniform(0, 1, (2, 3, 64, 64)).astype(np.float32) for _ in range(4)]
+    ref_req = g.compile().create_request()
+    want = [ref_req.infer(x)[0].copy() for x in xs]
+    got, errors = [None] * 4, []
+
+    def worker(i):
+        try:
+            req = g.compile().create_request()
+            for _ in range(6):
+                (y,) = req.infer(xs[i])
+            got[i] = y
+        except Exception as e:                                 # noqa: BLE001 - reported below
+            errors.append(repr(e))
+
+    def troublemaker():
+        for _ in range(20):
+            bad = Graph()
+            bad.result(bad.relu(bad.parameter("x", (1, 8, 4, 4))), "y")
+            try:
+                bad.compile()
+                errors.append("unsupported graph compiled")
+            except HipieError as e:
+                if "Relu" not in str(e):
+                    errors.append("error text of another thread: %s" % e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)] + [threading.Thread(target=troublemaker)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for y, w in zip(got, want):
+        np.testing.assert_array_equal(y.view(np.uint32), w.view(np.uint32))
