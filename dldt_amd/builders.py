@@ -43,8 +43,18 @@ class QuantizedNet:
         v = np.asarray(v, np.float32)
         return v.reshape((1, -1) + (1,) * (rank - 2))
 
+    def asymmetric(self, y, lo, hi):
+        """Activation FakeQuantize with an asymmetric range [lo, hi]: u8 levels 0 .. 255 with a zero point.
+        The activation carries the exact f32 shift (for f32 consumers) and the integer zero point that
+        ConvolutionTransformation leaves as Subtract in front of a convolution."""
+        d = lpt.decompose_fake_quantize(256, np.float32(lo), np.float32(hi), allow_zero_point=True)
+        assert d["has_zero_point"] and d["precision"] == U8
+        q = self.g.fake_quantize(y, np.float32(lo), np.float32(hi), d["new_low"], d["new_high"], 256, U8)
+        return dict(node=q, scale=np.float32(d["scale"]), shift=np.float32(d["shift"]),
+                    zero_point=np.float32(lpt.round_zero_point(d["shift"])))
+
     def _accumulate(self, act, w, bias, conv_attrs, matmul=False):
-        """Conv'/MatMul' -> Add(b / s): returns (node, s[c])."""
+        """[Subtract(zero point)] -> Conv'/MatMul' -> Add(b / s): returns (node, s[c])."""
         g = self.g
         wq, s_w = lpt.quantize_weights(w, 255)
         s = (np.float32(act["scale"]) * s_w).astype(np.float32)            # fold<Multiply>(s_a, s_w)
@@ -53,11 +63,14 @@ class QuantizedNet:
             # (the pattern LPT recognises, group_convolution.cpp:50-52); both fold into one constant
             wq = wq.reshape(wq.shape[0], 1, 1, wq.shape[2], wq.shape[3])
         wc = g.constant(wq, I8)
+        x = act["node"]
+        if act.get("zero_point", 0) != 0:      # TypeRelaxed Subtract(u8, u8) -> f32, written as Convert + Subtract
+            x = g.subtract(g.convert(x, F32), g.constant(np.float32(act["zero_point"]).reshape(())))
         if matmul:
-            y = g.matmul(act["node"], wc, False, True)
+            y = g.matmul(x, wc, False, True)
             rank = 2
         else:
-            y = g.convolution(act["node"], wc, **conv_attrs)
+            y = g.convolution(x, wc, **conv_attrs)
             rank = 4
         if bias is not None:
             b = np.asarray(bias, np.float32)
@@ -525,3 +538,28 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
     T = batch * seq
     meta["macs"] = layers * (T * (4 * hidden * hidden + 2 * hidden * ffn) + 2 * batch * heads * seq * seq * D)
     return g, meta
+
+
+def zero_point_net(seed=31, n=2, c=32, hw=20, oc=(48, 32)):
+    """Two quantized convolutions whose inputs have asymmetric ranges (u8 with zero points): a padded,
+    strided 3x3 and a 1x1; the second one's input FakeQuantize (asymmetric as well) rides in the first
+    one's epilogue.  Returns (graph, feeds, meta)."""
+    rng = np.random.default_rng(seed)
+    x = rng.normal(0.4, 1.0, (n, c, hw, hw)).astype(np.float32)
+    net = QuantizedNet()
+    g = net.g
+    a0 = net.asymmetric(g.parameter("data", x.shape), -1.7, 2.9)
+    w1 = (rng.standard_normal((oc[0], c, 3, 3), dtype=np.float32) * np.float32(0.06)).astype(np.float32)
+    b1 = (rng.standard_normal(oc[0], dtype=np.float32) * np.float32(0.2)).astype(np.float32)
+    y1, s1, rank = net._accumulate(a0, w1, b1, dict(strides=(2, 2), dilations=(1, 1), pads_begin=(1, 1), pads_end=(1, 1)))
+    lo, hi = np.float32(-2.2), np.float32(1.4)
+    d = lpt.decompose_fake_quantize(256, lo, hi, allow_zero_point=True)
+    q1 = g.fake_quantize(y1, net._channel((lo / s1).astype(np.float32), rank), net._channel((hi / s1).astype(np.float32), rank),
+                         d["new_low"], d["new_high"], 256, U8)
+    a1 = dict(node=q1, scale=np.float32(d["scale"]), shift=np.float32(d["shift"]),
+              zero_point=np.float32(lpt.round_zero_point(d["shift"])))
+    w2 = (rng.standard_normal((oc[1], oc[0], 1, 1), dtype=np.float32) * np.float32(0.1)).astype(np.float32)
+    b2 = (rng.standard_normal(oc[1], dtype=np.float32) * np.float32(0.2)).astype(np.float32)
+    y2 = net.conv_f32(a1, w2, b2)
+    g.result(y2, "out")
+    return g, dict(data=x), dict(acts=dict(a0=a0, a1=a1))

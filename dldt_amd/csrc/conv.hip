@@ -1020,7 +1020,8 @@ void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weight
                     w[packed_row(oc) * Kp + k] = v;
                     sum += v;
                 }
-        cr[oc] = d.in_dtype == HIPIE_U8B ? static_cast<int32_t>(128 * sum) : 0;
+        // stored byte = level - 128 (U8B) or level (I8); the product wanted is (level - zero point) * w
+        cr[oc] = static_cast<int32_t>(((d.in_dtype == HIPIE_U8B ? 128 : 0) - d.in_zero_point) * sum);
     });
     if (device >= 0) {
         wgt.upload(device, w.data(), w.size());
@@ -1037,6 +1038,9 @@ static void check_conv_desc(const hipie_conv_desc& d, const char* what) {
                   HIPIE_PARAMETER_MISMATCH, "%s: bad geometry", what);
     HIPIE_REQUIRE(d.in_c_stride >= d.ic && d.in_c_stride % 4 == 0, HIPIE_PARAMETER_MISMATCH,
                   "%s: in_c_stride=%d must be a multiple of 4 >= ic=%d", what, d.in_c_stride, d.ic);
+    const int lo = d.in_dtype == HIPIE_U8B ? 0 : -128;
+    HIPIE_REQUIRE(d.in_zero_point >= lo && d.in_zero_point <= lo + 255, HIPIE_PARAMETER_MISMATCH,
+                  "%s: zero point %d is not a level of the input type", what, d.in_zero_point);
 }
 
 static void conv_out_hw(const hipie_conv_desc& d, int h, int w, int& oh, int& ow) {
@@ -1184,7 +1188,7 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
                     w[static_cast<size_t>(t) * c->OCp + ch] = weights[ch * taps + t];
                     sum += weights[ch * taps + t];
                 }
-                corr[ch] = d.in_dtype == HIPIE_U8B ? 128 * sum : 0;
+                corr[ch] = ((d.in_dtype == HIPIE_U8B ? 128 : 0) - d.in_zero_point) * sum;
             }
             c->epi.build(device, *epilogue, d.oc, c->OCp);
             std::vector<uint32_t> rows;

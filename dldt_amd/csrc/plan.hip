@@ -23,6 +23,8 @@ struct TensorInfo {
     int64_t offset = 0, bytes = 0;
     int producer = -1;       // graph node whose value it holds
     int alias = -1;          // shares the bytes of this earlier tensor (same element count, other row split)
+    int fill_level = 0;      // level held by the halo and the channel padding (a consumer's zero point)
+    bool fill_fixed = false; // a consumer depends on fill_level
     int64_t esize() const { return dtype == HIPIE_F32 || dtype == HIPIE_I32 ? 4 : 1; }
     int wp() const { return w + 2 * halo; }
     int hp() const { return h + 2 * halo; }
@@ -1479,9 +1481,19 @@ struct Planner {
         const GNode& n = N(id);
         const bool is_mm = n.op == OP_MATMUL;
         const Value x = value(n.in[0]);
-        if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1)
-            unsupported(id, x.kind == VK_DEQ ? "activation zero points / unquantized inputs are not planned yet"
+        // Subtract(zero point) in front of the convolution: an integer per tensor (what optimizeSubtract
+        // leaves, network_helper.cpp:1479-1521) goes into the accumulators' initial value
+        int zero_point = 0;
+        if (x.kind == VK_DEQ && x.mul.empty() && !x.sub.empty() && tensors[x.tensor].esize() == 1) {
+            const float z = x.sub[0];
+            for (float v : x.sub)
+                if (v != z) unsupported(id, "per-channel activation zero points");
+            if (z != std::nearbyintf(z)) unsupported(id, "activation zero point that is not an integer level");
+            zero_point = static_cast<int>(z);
+        } else if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1) {
+            unsupported(id, x.kind == VK_DEQ ? "dequantized (f32) convolution inputs are not planned"
                                              : "input must be a quantized (u8/i8) tensor");
+        }
         const GNode& W = N(n.in[1]);
         if (W.op != OP_CONSTANT || W.dtype != HIPIE_I8) unsupported(id, "weights must be an i8 constant");
         auto st = std::make_unique<ConvStep>();
@@ -1523,6 +1535,14 @@ struct Planner {
         const int halo = std::max(std::max(d.pad_top, d.pad_bottom), std::max(d.pad_left, d.pad_right));
         tensors[x.tensor].halo = std::max(tensors[x.tensor].halo, halo);
         st->in = x.tensor;
+        d.in_zero_point = zero_point;
+        if (halo > 0) {   // padding is applied behind the Subtract: the halo must read as the zero point
+            TensorInfo& ti = tensors[x.tensor];
+            if (ti.fill_fixed && ti.fill_level != zero_point)
+                unsupported(id, "consumers of one tensor pad it with different levels");
+            ti.fill_level = zero_point;
+            ti.fill_fixed = true;
+        }
 
         // ---- absorb the elementwise chain behind the accumulator --------------------------------
         EpilogueSpec& e = st->epi;
@@ -1652,6 +1672,11 @@ struct Planner {
         a.include_pad = st->avg && !n.exclude_pad;
         const int halo = std::max(std::max(a.pt, a.pb), std::max(a.pl, a.pr));
         tensors[x.tensor].halo = std::max(tensors[x.tensor].halo, halo);
+        if (halo > 0) {   // pooling reads its padding as level 0
+            TensorInfo& ti = tensors[x.tensor];
+            if (ti.fill_fixed && ti.fill_level != 0) unsupported(id, "consumers of one tensor pad it with different levels");
+            ti.fill_fixed = true;
+        }
         st->in = x.tensor;
         int cur = id;
         int out_dtype = tensors[x.tensor].dtype;
@@ -1937,10 +1962,13 @@ int hipie_request_create(const hipie_plan* p, int perf_count, hipie_request** ou
         // level 0 everywhere: halos and channel padding are never written again
         uint8_t* a = r->arena.as<uint8_t>();
         HIPIE_CHECK_HIP(hipMemsetAsync(a, 0, static_cast<size_t>(p->arena_bytes), r->stream));
-        for (const auto& t : p->tensors)
-            if (t.dtype == HIPIE_U8B)
+        for (const auto& t : p->tensors) {
+            if (t.alias >= 0) continue;
+            const int byte = t.dtype == HIPIE_U8B ? t.fill_level - 128 : (t.dtype == HIPIE_I8 ? t.fill_level : 0);
+            if (byte != 0)
                 hipLaunchKernelGGL(fill_bytes, dim3(1024), dim3(256), 0, r->stream, a + t.offset, t.bytes,
-                                   static_cast<uint8_t>(0x80));
+                                   static_cast<uint8_t>(byte & 0xff));
+        }
         HIPIE_CHECK_HIP(hipGetLastError());
         for (const auto& io : p->inputs) {
             r->in_dev.emplace_back();

@@ -35,16 +35,25 @@ def data_precision_range(precision, levels):
     return mn.value, mx.value
 
 
-def decompose_fake_quantize(levels, out_low, out_high):
-    """NetworkHelper::decomposeFakeQuantize for an FQ whose precision getPrecisionDetails resolves.
+def decompose_fake_quantize(levels, out_low, out_high, allow_zero_point=False, precision=None):
+    """NetworkHelper::decomposeFakeQuantize for an FQ whose precision getPrecisionDetails resolves, or
+    (allow_zero_point) for an asymmetric range: the first supported activation precision, u8, with a
+    zero point (fake_quantize_decomposition.cpp:343-372).
+
+    precision forces the data precision (a layer that only takes u8 activations: the intervals'
+    own precision is then not among the supported ones and a zero point is used, :359-366).
 
     Returns dict(precision, new_low, new_high, scale, shift) with arrays shaped like out_low.
     """
     ol = np.ascontiguousarray(np.asarray(out_low, np.float32))
     oh = np.ascontiguousarray(np.asarray(out_high, np.float32))
     prec, _, zp = precision_details(levels, ol, oh)
+    if precision is not None and prec != precision:
+        prec, zp = precision, True
+    if prec is None and allow_zero_point:
+        prec, zp = U8, True
     if prec is None:
-        raise NotImplementedError("FakeQuantize needs a zero point (asymmetric range): next tier")
+        raise NotImplementedError("FakeQuantize needs a zero point (asymmetric range): pass allow_zero_point")
     mn, mx = data_precision_range(prec, levels)
     sc, sh, nl, nh = (np.empty(ol.size, np.float32) for _ in range(4))
     check(lib().hipie_lpt_decompose_fake_quantize(_p(ol.reshape(-1)), _p(oh.reshape(-1)), ctypes.c_int64(ol.size),
@@ -81,3 +90,10 @@ def quantize_weights(w, levels=255):
     q = fold_fake_quantize(w, -m, m, d["new_low"], d["new_high"], levels, round_values=True)
     assert np.abs(q).max() <= 127
     return q.astype(np.int8), d["scale"].astype(np.float32)
+
+
+def round_zero_point(shift):
+    """NetworkHelper::round(shift, u8) of optimizeSubtract (network_helper.cpp:485-494, 1500-1501):
+    Round-5 HALF_AWAY_FROM_ZERO, then Convert to the activation's integer type."""
+    s = np.asarray(shift, np.float32)
+    return (np.sign(s) * np.floor(np.abs(s) + np.float32(0.5))).astype(np.float32)

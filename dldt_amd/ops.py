@@ -107,7 +107,7 @@ class hipie_conv_desc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int32) for k in (
         "in_dtype", "ic", "oc", "kh", "kw", "stride_h", "stride_w", "dil_h", "dil_w",
         "pad_top", "pad_left", "pad_bottom", "pad_right", "groups", "in_c_stride",
-        "in_stride_h", "in_stride_w")]
+        "in_stride_h", "in_stride_w", "in_zero_point")]
 
 
 def make_epilogue(bias=None, scale=None, residual_dtype=0, res_sub=None, res_mul=None,
@@ -150,7 +150,7 @@ class Convolution:
     """
 
     def __init__(self, weights, in_tensor, strides=(1, 1), dilations=(1, 1), pads_begin=(0, 0),
-                 pads_end=(0, 0), epilogue=None, device=0):
+                 pads_end=(0, 0), epilogue=None, device=0, zero_point=0):
         w = np.ascontiguousarray(weights, np.int8)
         if w.ndim == 5:   # GroupConvolution filters [G, OC/G, IC/G, kh, kw]; depthwise only
             groups = w.shape[0]
@@ -162,7 +162,7 @@ class Convolution:
             self.oc, self.ic, self.kh, self.kw = w.shape
         d = hipie_conv_desc(in_tensor.dtype, self.ic, self.oc, self.kh, self.kw, strides[0], strides[1],
                             dilations[0], dilations[1], pads_begin[0], pads_begin[1], pads_end[0],
-                            pads_end[1], groups, in_tensor.cs, in_tensor.stride_h, in_tensor.stride_w)
+                            pads_end[1], groups, in_tensor.cs, in_tensor.stride_h, in_tensor.stride_w, int(zero_point))
         self.epilogue = epilogue or make_epilogue(out_dtype=I32)
         self._h = ctypes.c_void_p()
         check(lib().hipie_conv_create(ctypes.c_int(device), ctypes.byref(d),

@@ -22,7 +22,7 @@ _SLACK = 256  # bytes readable before and after the tensor (K-padding reads of t
 
 
 class DeviceTensor:
-    def __init__(self, n, h, w, c, dtype, halo=0, c_stride=None, device="cuda"):
+    def __init__(self, n, h, w, c, dtype, halo=0, c_stride=None, device="cuda", fill_level=0):
         import torch
         self.n, self.h, self.w, self.c, self.dtype, self.halo = n, h, w, c, dtype, halo
         gran = 16 if dtype in (U8B, I8, U8) else 4
@@ -32,7 +32,7 @@ class DeviceTensor:
         esz = torch.empty((), dtype=tdt).element_size()
         slack = _SLACK // esz
         self.numel = n * self.hp * self.wp * self.cs
-        fill = -128 if dtype == U8B else 0
+        fill = fill_level - 128 if dtype == U8B else fill_level      # halo and channel padding: this level
         self.buf = torch.full((self.numel + 2 * slack,), fill, dtype=tdt, device=device)
         self.view = self.buf[slack:slack + self.numel].view(n, self.hp, self.wp, self.cs)
         self.stride_w = self.cs
@@ -51,10 +51,10 @@ class DeviceTensor:
 
     # ---- host <-> device in the reference's layout (NCHW, plain values) ----------------------
     @classmethod
-    def from_nchw(cls, x, dtype, halo=0, c_stride=None, device="cuda"):
+    def from_nchw(cls, x, dtype, halo=0, c_stride=None, device="cuda", fill_level=0):
         import torch
         n, c, h, w = x.shape
-        t = cls(n, h, w, c, dtype, halo, c_stride, device)
+        t = cls(n, h, w, c, dtype, halo, c_stride, device, fill_level)
         a = np.ascontiguousarray(np.transpose(x, (0, 2, 3, 1)))
         if dtype == U8B:
             a = (a.astype(np.int16) - 128).astype(np.int8)

@@ -185,6 +185,12 @@ typedef struct hipie_conv_desc {
     int32_t groups;                       /* 1 */
     int32_t in_c_stride;                  /* channel stride of the input tensor (>= ic) */
     int32_t in_stride_h, in_stride_w;     /* element strides of the input tensor */
+    int32_t in_zero_point;                /* integer level subtracted from every input element: the
+                                             TypeRelaxed Subtract(u8 data, u8 shift) that
+                                             ConvolutionTransformation leaves in front of the convolution
+                                             (convolution.cpp:84-120, optimizeSubtract network_helper.cpp:1479-1521).
+                                             Padding is applied after the Subtract, so the halo of the
+                                             input tensor must hold this level (not level 0). */
 } hipie_conv_desc;
 
 typedef struct hipie_conv hipie_conv;

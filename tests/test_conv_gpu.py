@@ -315,3 +315,21 @@ def test_depthwise_conv_exact_and_relu6_requantize(orc, C, H, stride):
                 make_epilogue(bias=bias, scale=scale, activation="clamp", clamp=(0.0, 6.0), out_dtype=U8B,
                               fq=fq)).run(xin, out8)
     np.testing.assert_array_equal(out8.to_nchw(), want)
+
+
+@pytest.mark.parametrize("signed,zp", [(False, 0), (False, 37), (False, 255), (True, -128), (True, 5)])
+@pytest.mark.parametrize("depthwise", [False, True])
+def test_conv_input_zero_point(orc, signed, zp, depthwise):
+    """(x - zero point) * w summed exactly, with padding applied behind the subtraction: the input
+    tensor's halo holds the zero-point level"""
+    from dldt_amd import Convolution, DeviceTensor
+    rng = np.random.default_rng(zp + 1000 * signed + 7 * depthwise)
+    N, C, H, W, OC = 2, 32, 9, 11, 32 if depthwise else 40
+    x = rng.integers(-128 if signed else 0, 128 if signed else 256, (N, C, H, W)).astype(np.int32)
+    w = rng.integers(-127, 128, (C, 1, 1, 3, 3) if depthwise else (OC, C, 3, 3)).astype(np.int32)
+    want = orc.convolution(x - zp, w, (1, 1), (1, 1), (1, 1), (1, 1), grouped=depthwise)
+    xin = DeviceTensor.from_nchw(x, I8 if signed else U8B, halo=1, fill_level=zp)
+    conv = Convolution(w.astype(np.int8), xin, (1, 1), (1, 1), (1, 1), (1, 1), zero_point=zp)
+    out = DeviceTensor(N, H, W, OC, I32)
+    conv.run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw(), want)

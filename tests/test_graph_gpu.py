@@ -187,3 +187,19 @@ def test_compile_and_infer_from_many_threads(orc):
     assert not errors, errors
     for y, w in zip(got, want):
         np.testing.assert_array_equal(y.view(np.uint32), w.view(np.uint32))
+
+
+def test_activation_zero_points(orc):
+    """asymmetric activation ranges: u8 levels with an integer zero point subtracted in front of the
+    convolution (padding applies behind the Subtract: the padded taps contribute nothing)"""
+    from dldt_amd import builders
+    g, feeds, meta = builders.zero_point_net()
+    keep = [a["node"] for a in meta["acts"].values()]
+    want, kept = evaluate(orc, g.nodes, feeds, keep=keep)
+    plan = g.compile()
+    req = plan.create_request()
+    (got,) = req.infer(feeds["data"])
+    for name, a in meta["acts"].items():
+        np.testing.assert_array_equal(req.tensor(a["node"]), kept[a["node"]], err_msg=name)
+        assert kept[a["node"]].min() == 0 and kept[a["node"]].max() == 255      # both ends saturate
+    np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))

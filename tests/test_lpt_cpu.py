@@ -154,3 +154,34 @@ def test_planner_embedding_front_end():
     types = [s["type"] for s in plan.steps]
     assert types[:3] == ["Gather", "MVN+FakeQuantize", "MatMul"] and "FakeQuantize" not in types
     assert plan.inputs[0]["dtype"] == 70 and plan.inputs[0]["shape"] == (2, 64)
+
+
+def test_decompose_with_zero_point_golden():
+    """[-1.28, 1.27] on a layer that only takes u8: shift 128, scale 0.01
+    (lp_transformations/fake_quantize_transformation.cpp:153-183); optimizeSubtract rounds half away from zero."""
+    from dldt_amd import lpt
+    d = lpt.decompose_fake_quantize(256, np.float32(-1.28), np.float32(1.27), precision=40)
+    assert d["precision"] == 40 and d["has_zero_point"] and d["new_low"] == 0 and d["new_high"] == 255
+    np.testing.assert_allclose(d["scale"], 0.01, rtol=1e-6)
+    np.testing.assert_allclose(d["shift"], 128.0, rtol=1e-6)
+    np.testing.assert_array_equal(lpt.round_zero_point([94.239, 155.5, 0.49, 2.5, -0.5]), [94, 156, 0, 3, -1])
+    a = lpt.decompose_fake_quantize(256, np.float32(-0.5), np.float32(2.0), allow_zero_point=True)
+    assert a["precision"] == 40 and a["has_zero_point"]
+    np.testing.assert_allclose(a["shift"], 51.0, rtol=1e-6)          # (0 * 2 - 255 * -0.5) / 2.5
+
+
+def test_planner_takes_integer_zero_points():
+    from dldt_amd import HipieError, builders
+    from dldt_amd.graph import Graph, Plan
+    g, _, _ = builders.zero_point_net()
+    assert [s["type"] for s in Plan(g, device=-1).steps] == ["FakeQuantize", "Convolution", "Convolution", "Result"]
+    # a fractional zero point (Subtract not passed through optimizeSubtract) is refused by name
+    bad = Graph()
+    x = bad.parameter("x", (1, 16, 8, 8))
+    q = bad.fake_quantize(x, -1.0, 2.0, 0.0, 255.0, 256, 40)
+    s = bad.subtract(bad.convert(q, 10), bad.constant(np.float32(85.3).reshape(())))
+    y = bad.convolution(s, bad.constant(np.ones((16, 16, 1, 1), np.int8), 50))
+    bad.result(bad.multiply(y, bad.constant(np.float32(0.1).reshape(()))), "y")
+    with pytest.raises(HipieError) as e:
+        Plan(bad, device=-1)
+    assert e.value.status == -2 and "zero point" in str(e.value)
