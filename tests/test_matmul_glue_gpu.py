@@ -178,3 +178,31 @@ def test_fused_attention_rejects_unsupported_shapes():
         with pytest.raises(HipieError) as e:
             attention(x, x, x, 1.0, 1.0, (-1.0, 1.0, -128, 256))
         assert e.value.status == -2
+
+
+def test_fused_attention_with_mask(orc):
+    """additive mask row per sequence, shared by its heads: added to the scaled scores in front of the Softmax"""
+    import torch
+    from dldt_amd.ops import Attention
+    rng = np.random.default_rng(77)
+    B, NH, S = 3, 2, 160
+    t = torch.from_numpy(rng.integers(-60, 61, (B, S, 3, NH, 64), dtype=np.int8)).cuda()
+    q, k, v = (t[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    mask = np.zeros((B, S), np.float32)
+    mask[0, 100:] = -10000.0
+    mask[2, 7:] = -10000.0
+    mask[1] = rng.normal(0, 1, S).astype(np.float32)                       # any additive row, not only 0 / -10000
+    s1, s2 = np.float32(0.002), np.float32(0.01)
+    il, ih = np.float32(-128.0 / 127), np.float32(1.0)
+    att = Attention(S, 64, s1, s2, (il, ih, -128, 256))
+    ctx, scores, probs = att.run(q, k, v, dump=True, mask=torch.from_numpy(mask).cuda())
+    qn, kn, vn = (np.ascontiguousarray(x.cpu().numpy()).astype(np.int32) for x in (q, k, v))
+    want_scores = orc.add(orc.multiply(orc.matmul(qn, kn, False, True).astype(np.float32), s1), mask[:, None, None, :])
+    np.testing.assert_array_equal(scores.cpu().numpy().view(np.uint32), want_scores.view(np.uint32))
+    p = probs.cpu().numpy()
+    np.testing.assert_allclose(p, orc.softmax(want_scores, -1), rtol=3e-6, atol=1e-8)
+    assert p[0, :, :, 100:].max() == 0.0 and p[2, :, :, 7:].max() == 0.0
+    pq = orc.fake_quantize(p, il, ih, np.float32(-128), np.float32(127), 256).astype(np.int32)
+    want_ctx = orc.multiply(orc.matmul(pq, vn).astype(np.float32), s2)
+    np.testing.assert_array_equal(ctx.cpu().numpy().view(np.uint32), want_ctx.view(np.uint32))
+    assert torch.equal(att.run(q, k, v, mask=torch.from_numpy(mask).cuda()), ctx)
