@@ -15,6 +15,8 @@ const char* op_name(int op) {
 
 namespace {
 
+constexpr int64_t kMaxAttr = int64_t(1) << 20;   // strides, dilations, pads, windows: products with a dimension stay in int64
+
 size_t dtype_size(int dt) {
     switch (dt) {
     case HIPIE_F32: case HIPIE_I32: return 4;
@@ -33,6 +35,12 @@ GNode& node(hipie_graph* g, int id, const char* what) {
 
 int add_node(hipie_graph* g, GNode&& n) {
     const int id = static_cast<int>(g->nodes.size());
+    int64_t count = 1;
+    for (int64_t d : n.shape) {   // element counts stay far inside int64 for everything computed from them
+        HIPIE_REQUIRE(d >= 0 && (d == 0 || count <= (int64_t(1) << 40) / d), HIPIE_PARAMETER_MISMATCH,
+                      "%s: a value of more than 2^40 elements", op_name(n.op));
+        count *= d;
+    }
     if (n.name.empty()) n.name = std::string(op_name(n.op)) + "_" + std::to_string(id);
     for (int i : n.in) g->nodes[i].users.push_back(id);
     g->nodes.push_back(std::move(n));
@@ -81,6 +89,9 @@ int hipie_graph_parameter(hipie_graph* g, const char* name, int dtype, const int
         HIPIE_REQUIRE(rank >= 2 && rank <= 4, HIPIE_NOT_IMPLEMENTED, "hipie_graph_parameter: rank %d", rank);
         HIPIE_REQUIRE(dtype == HIPIE_F32 || dtype == HIPIE_U8 || dtype == HIPIE_I32, HIPIE_NOT_IMPLEMENTED,
                       "hipie_graph_parameter: element type %d", dtype);
+        for (int i = 0; i < rank; ++i)
+            HIPIE_REQUIRE(dims[i] > 0 && dims[i] < (int64_t(1) << 31), HIPIE_PARAMETER_MISMATCH,
+                          "hipie_graph_parameter: dimension %d is %lld", i, (long long)dims[i]);
         GNode n;
         n.op = OP_PARAMETER;
         n.name = name ? name : "";
@@ -95,6 +106,10 @@ int hipie_graph_constant(hipie_graph* g, int dtype, const int64_t* dims, int ran
     return guarded([&] {
         HIPIE_REQUIRE(g && id && data && (dims || rank == 0), HIPIE_PARAMETER_MISMATCH,
                       "hipie_graph_constant: null argument");
+        HIPIE_REQUIRE(rank >= 0 && rank <= 8, HIPIE_PARAMETER_MISMATCH, "hipie_graph_constant: rank %d", rank);
+        for (int i = 0; i < rank; ++i)
+            HIPIE_REQUIRE(dims[i] >= 0 && dims[i] < (int64_t(1) << 31), HIPIE_PARAMETER_MISMATCH,
+                          "hipie_graph_constant: dimension %d is %lld", i, (long long)dims[i]);
         GNode n;
         n.op = OP_CONSTANT;
         n.dtype = dtype;
@@ -156,7 +171,8 @@ static int add_conv(hipie_graph* g, int x, int w, const int64_t* strides, const 
         n.dtype = HIPIE_F32;  // TypeRelaxed<Convolution>: f32 holding the integer sum
         n.shape = {X.shape[0], W.shape[o] * G};
         for (int i = 0; i < 2; ++i) {
-            HIPIE_REQUIRE(n.strides[i] > 0 && n.dilations[i] > 0 && n.pads_begin[i] >= 0 && n.pads_end[i] >= 0,
+            HIPIE_REQUIRE(n.strides[i] > 0 && n.dilations[i] > 0 && n.pads_begin[i] >= 0 && n.pads_end[i] >= 0 &&
+                              std::max(std::max(n.strides[i], n.dilations[i]), std::max(n.pads_begin[i], n.pads_end[i])) < kMaxAttr,
                           HIPIE_PARAMETER_MISMATCH, "%s: attributes", what);
             const int64_t dk = n.dilations[i] * (W.shape[o + 2 + i] - 1) + 1;
             const int64_t span = X.shape[2 + i] + n.pads_begin[i] + n.pads_end[i] - dk;
@@ -287,7 +303,8 @@ static int add_pool(hipie_graph* g, int op, int x, const int64_t* kernel, const 
         n.dtype = out_dtype;
         n.shape = {X.shape[0], X.shape[1]};
         for (int i = 0; i < 2; ++i) {
-            HIPIE_REQUIRE(kernel[i] > 0 && strides[i] > 0 && pads_begin[i] >= 0 && pads_end[i] >= 0,
+            HIPIE_REQUIRE(kernel[i] > 0 && strides[i] > 0 && pads_begin[i] >= 0 && pads_end[i] >= 0 &&
+                              std::max(std::max(kernel[i], strides[i]), std::max(pads_begin[i], pads_end[i])) < kMaxAttr,
                           HIPIE_PARAMETER_MISMATCH, "%s: attributes", what);
             n.shape.push_back(pooled(X.shape[2 + i], pads_begin[i], pads_end[i], kernel[i], strides[i], n.ceil_mode));
         }
@@ -318,6 +335,10 @@ int hipie_graph_reshape(hipie_graph* g, int x, const int64_t* dims, int rank, in
         n.op = OP_RESHAPE;
         n.in = {x};
         n.dtype = X.dtype;
+        HIPIE_REQUIRE(rank >= 1 && rank <= 8, HIPIE_PARAMETER_MISMATCH, "hipie_graph_reshape: rank %d", rank);
+        for (int i = 0; i < rank; ++i)
+            HIPIE_REQUIRE(dims[i] > 0 && dims[i] < (int64_t(1) << 31), HIPIE_PARAMETER_MISMATCH,
+                          "hipie_graph_reshape: dimension %d is %lld", i, (long long)dims[i]);
         n.shape.assign(dims, dims + rank);
         HIPIE_REQUIRE(n.numel() == X.numel(), HIPIE_PARAMETER_MISMATCH,
                       "hipie_graph_reshape: element count changes");
@@ -451,3 +472,200 @@ int hipie_graph_set_name(hipie_graph* g, int id, const char* name) {
 }
 
 }  // extern "C"
+
+// ---------------------------------------------------------------------------------------------
+// Graph description as a byte stream (the model part of an exported plan).  Reading it REPLAYS the
+// description through the entry points above, one call per node, so a stream gets exactly the
+// validation and shape inference a freshly described graph gets; every length is checked against
+// the bytes that remain before it is used.
+namespace hipie {
+namespace {
+
+// writes into `dst` when there is one, counts the bytes either way
+struct Writer {
+    uint8_t* dst;
+    size_t n = 0;
+    void raw(const void* p, size_t len) {
+        if (dst && len) std::memcpy(dst + n, p, len);
+        n += len;
+    }
+    template <typename T> void pod(T v) { raw(&v, sizeof v); }
+    void str(const std::string& s) { pod<uint32_t>(static_cast<uint32_t>(s.size())); raw(s.data(), s.size()); }
+    void i64s(const std::vector<int64_t>& v) { pod<uint32_t>(static_cast<uint32_t>(v.size())); raw(v.data(), v.size() * 8); }
+    void ints(const std::vector<int>& v) { pod<uint32_t>(static_cast<uint32_t>(v.size())); raw(v.data(), v.size() * 4); }
+};
+
+struct Reader {
+    const uint8_t* p;
+    size_t left;
+    const uint8_t* take(size_t n) {
+        HIPIE_REQUIRE(n <= left, HIPIE_NETWORK_NOT_READ, "plan stream is truncated");
+        const uint8_t* q = p;
+        p += n;
+        left -= n;
+        return q;
+    }
+    template <typename T> T pod() { T v; std::memcpy(&v, take(sizeof v), sizeof v); return v; }
+    std::string str() {
+        const uint32_t n = pod<uint32_t>();
+        const uint8_t* q = take(n);
+        return std::string(reinterpret_cast<const char*>(q), n);
+    }
+    std::vector<int64_t> i64s(size_t max_len) {
+        const uint32_t n = pod<uint32_t>();
+        HIPIE_REQUIRE(n <= max_len, HIPIE_NETWORK_NOT_READ, "plan stream: attribute with %u entries", n);
+        std::vector<int64_t> v(n);
+        if (n) std::memcpy(v.data(), take(size_t(n) * 8), size_t(n) * 8);
+        return v;
+    }
+    std::vector<int> ints(size_t max_len) {
+        const uint32_t n = pod<uint32_t>();
+        HIPIE_REQUIRE(n <= max_len, HIPIE_NETWORK_NOT_READ, "plan stream: node with %u inputs", n);
+        std::vector<int> v(n);
+        if (n) std::memcpy(v.data(), take(size_t(n) * 4), size_t(n) * 4);
+        return v;
+    }
+};
+
+enum : uint8_t { F_TA = 1, F_TB = 2, F_EXCLUDE_PAD = 4, F_CEIL = 8, F_NORM_VAR = 16, F_EPS_INSIDE = 32 };
+
+}  // namespace
+
+size_t serialize_graph(const hipie_graph& g, uint8_t* dst) {
+    Writer w{dst};
+    w.pod<uint32_t>(static_cast<uint32_t>(g.nodes.size()));
+    for (const GNode& n : g.nodes) {
+        w.pod<int32_t>(n.op);
+        w.str(n.name);
+        w.ints(n.in);
+        w.pod<int32_t>(n.dtype);
+        w.i64s(n.shape);
+        w.i64s(n.strides);
+        w.i64s(n.dilations);
+        w.i64s(n.pads_begin);
+        w.i64s(n.pads_end);
+        w.i64s(n.kernel);
+        w.i64s(n.axes);
+        w.pod<int64_t>(n.levels);
+        w.pod<uint8_t>((n.ta ? F_TA : 0) | (n.tb ? F_TB : 0) | (n.exclude_pad ? F_EXCLUDE_PAD : 0) | (n.ceil_mode ? F_CEIL : 0) |
+                       (n.normalize_variance ? F_NORM_VAR : 0) | (n.eps_inside_sqrt ? F_EPS_INSIDE : 0));
+        w.pod<float>(n.lo);
+        w.pod<float>(n.hi);
+        w.pod<float>(n.eps);
+        w.pod<uint64_t>(n.data.size());
+        w.raw(n.data.data(), n.data.size());
+    }
+    return w.n;
+}
+
+hipie_graph* deserialize_graph(const uint8_t* bytes, size_t size) {
+    Reader r{bytes, size};
+    auto g = std::make_unique<hipie_graph>();
+    hipie_graph* G = g.get();
+    const uint32_t count = r.pod<uint32_t>();
+    HIPIE_REQUIRE(count <= size, HIPIE_NETWORK_NOT_READ, "plan stream: %u nodes in %zu bytes", count, size);
+    for (uint32_t i = 0; i < count; ++i) {
+        const int op = r.pod<int32_t>();
+        const std::string name = r.str();
+        const std::vector<int> in = r.ints(8);
+        const int dtype = r.pod<int32_t>();
+        const std::vector<int64_t> shape = r.i64s(8), strides = r.i64s(2), dilations = r.i64s(2), pads_begin = r.i64s(2),
+                                   pads_end = r.i64s(2), kernel = r.i64s(2), axes = r.i64s(8);
+        const int64_t levels = r.pod<int64_t>();
+        const uint8_t flags = r.pod<uint8_t>();
+        const float lo = r.pod<float>(), hi = r.pod<float>(), eps = r.pod<float>();
+        const uint64_t nbytes = r.pod<uint64_t>();
+        HIPIE_REQUIRE(nbytes <= r.left, HIPIE_NETWORK_NOT_READ, "plan stream is truncated");
+        const uint8_t* data = r.take(static_cast<size_t>(nbytes));
+        auto arity = [&](size_t n) {
+            HIPIE_REQUIRE(in.size() == n, HIPIE_NETWORK_NOT_READ, "plan stream: node %u (%s) has %zu inputs", i, op_name(op), in.size());
+        };
+        auto pair = [&](const std::vector<int64_t>& v) {
+            HIPIE_REQUIRE(v.size() == 2, HIPIE_NETWORK_NOT_READ, "plan stream: node %u (%s) lacks an attribute", i, op_name(op));
+            return v.data();
+        };
+        int id = static_cast<int>(i), st = HIPIE_OK;
+        switch (op) {
+        case OP_PARAMETER:
+            arity(0);
+            st = hipie_graph_parameter(G, name.c_str(), dtype, shape.data(), static_cast<int>(shape.size()), &id);
+            break;
+        case OP_CONSTANT: {
+            arity(0);
+            uint64_t want = dtype == HIPIE_F32 || dtype == HIPIE_I32 ? 4 : 1;
+            for (int64_t d : shape) {
+                HIPIE_REQUIRE(d >= 0 && (d == 0 || want <= nbytes / static_cast<uint64_t>(d)), HIPIE_NETWORK_NOT_READ,
+                              "plan stream: constant %u is larger than its payload", i);
+                want *= static_cast<uint64_t>(d);
+            }
+            HIPIE_REQUIRE(want == nbytes, HIPIE_NETWORK_NOT_READ, "plan stream: constant %u has %llu bytes for its shape, %llu stored", i,
+                          (unsigned long long)want, (unsigned long long)nbytes);
+            st = hipie_graph_constant(G, dtype, shape.data(), static_cast<int>(shape.size()), data, &id);
+            break;
+        }
+        case OP_FAKE_QUANTIZE:
+            arity(5);
+            st = hipie_graph_fake_quantize(G, in[0], in[1], in[2], in[3], in[4], levels, dtype, &id);
+            break;
+        case OP_CONVOLUTION:
+        case OP_GROUP_CONVOLUTION:
+            arity(2);
+            st = (op == OP_CONVOLUTION ? hipie_graph_convolution : hipie_graph_group_convolution)(
+                G, in[0], in[1], pair(strides), pair(dilations), pair(pads_begin), pair(pads_end), &id);
+            break;
+        case OP_MATMUL:
+            arity(2);
+            st = hipie_graph_matmul(G, in[0], in[1], flags & F_TA, flags & F_TB, &id);
+            break;
+        case OP_ADD: case OP_MULTIPLY: case OP_SUBTRACT:
+            arity(2);
+            st = hipie_graph_eltwise(G, op, in[0], in[1], &id);
+            break;
+        case OP_RELU: arity(1); st = hipie_graph_relu(G, in[0], &id); break;
+        case OP_CLAMP: arity(1); st = hipie_graph_clamp(G, in[0], lo, hi, &id); break;
+        case OP_CONVERT: arity(1); st = hipie_graph_convert(G, in[0], dtype, &id); break;
+        case OP_MAX_POOL:
+            arity(1);
+            st = hipie_graph_max_pool(G, in[0], pair(kernel), pair(strides), pair(pads_begin), pair(pads_end), flags & F_CEIL, &id);
+            break;
+        case OP_AVG_POOL:
+            arity(1);
+            st = hipie_graph_avg_pool(G, in[0], pair(kernel), pair(strides), pair(pads_begin), pair(pads_end), flags & F_EXCLUDE_PAD,
+                                      flags & F_CEIL, dtype, &id);
+            break;
+        case OP_RESHAPE: arity(1); st = hipie_graph_reshape(G, in[0], shape.data(), static_cast<int>(shape.size()), &id); break;
+        case OP_SOFTMAX:
+            arity(1);
+            HIPIE_REQUIRE(axes.size() == 1, HIPIE_NETWORK_NOT_READ, "plan stream: Softmax %u without an axis", i);
+            st = hipie_graph_softmax(G, in[0], axes[0], &id);
+            break;
+        case OP_MVN:
+            arity(1);
+            st = hipie_graph_mvn(G, in[0], axes.data(), static_cast<int>(axes.size()), flags & F_NORM_VAR, eps, flags & F_EPS_INSIDE, &id);
+            break;
+        case OP_GELU: arity(1); st = hipie_graph_gelu(G, in[0], &id); break;
+        case OP_TRANSPOSE: arity(1); st = hipie_graph_transpose(G, in[0], axes.data(), static_cast<int>(axes.size()), &id); break;
+        case OP_GATHER:
+            arity(2);
+            HIPIE_REQUIRE(axes.size() == 1, HIPIE_NETWORK_NOT_READ, "plan stream: Gather %u without an axis", i);
+            st = hipie_graph_gather(G, in[0], in[1], axes[0], &id);
+            break;
+        case OP_RESULT: arity(1); st = hipie_graph_result(G, in[0], name.c_str()); break;
+        default: fail(HIPIE_NETWORK_NOT_READ, "plan stream: node %u has unknown operation %d", i, op);
+        }
+        if (st != HIPIE_OK) {
+            const std::string why = hipie_last_error();
+            fail(HIPIE_NETWORK_NOT_READ, "plan stream: node %u (%s) is rejected: %s", i, op_name(op), why.c_str());
+        }
+        HIPIE_REQUIRE(G->nodes.size() == size_t(i) + 1 && id == static_cast<int>(i), HIPIE_UNEXPECTED, "plan stream: node numbering");
+        GNode& n = G->nodes[i];
+        HIPIE_REQUIRE(n.shape == shape && n.dtype == dtype, HIPIE_NETWORK_NOT_READ,
+                      "plan stream: node %u (%s): the stored shape or type is not the inferred one", i, op_name(op));
+        n.name = name;
+    }
+    HIPIE_REQUIRE(r.left == 0, HIPIE_NETWORK_NOT_READ, "plan stream: %zu bytes behind the last node", r.left);
+    return g.release();
+}
+
+}  // namespace hipie
+

@@ -47,3 +47,10 @@ struct hipie_graph {
     std::vector<hipie::GNode> nodes;
     std::vector<int> params, results;
 };
+
+namespace hipie {
+// the description as a byte stream (written to `dst` unless it is null; returns the byte count), and
+// back (through the validating entry points; throws HIPIE_NETWORK_NOT_READ on anything malformed)
+size_t serialize_graph(const hipie_graph& g, uint8_t* dst);
+hipie_graph* deserialize_graph(const uint8_t* bytes, size_t size);
+}  // namespace hipie

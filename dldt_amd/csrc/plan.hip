@@ -1762,7 +1762,7 @@ using namespace hipie;
 
 struct hipie_plan {
     int device = 0;
-    hipie_graph graph;                       // private copy (constants are dropped after packing)
+    hipie_graph graph;                       // the description the plan was compiled from (what an export writes)
     std::vector<TensorInfo> tensors;
     std::vector<std::unique_ptr<Step>> steps;
     std::map<int, int> node_tensor;          // graph node -> tensor holding its value
@@ -1805,6 +1805,131 @@ void enqueue(hipie_request* r, void* const* in, void* const* out) {
     if (r->perf) HIPIE_CHECK_HIP(hipEventRecord(r->events[p.steps.size()], r->stream));
 }
 
+// `preset`: kernel variants of an imported plan, one per step; used when they fit the steps planned
+// here (same count, variants exactly where steps have them), else the plan is tuned like a new one
+std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const std::vector<int>* preset) {
+    HIPIE_REQUIRE(!g->results.empty(), HIPIE_PARAMETER_MISMATCH, "hipie_compile: graph has no Result");
+    auto plan = std::make_unique<hipie_plan>();
+    plan->device = device;
+    plan->graph = *g;
+    Planner pl(*g);
+    for (int r : g->results) pl.visit(r);
+    // arena layout: one region per tensor, 256-byte aligned, with slack on both sides so that
+    // K-padding reads of a first-layer filter row stay inside the arena
+    int64_t off = 256;
+    for (auto& t : pl.tensors) {
+        t.bytes = static_cast<int64_t>(t.n) * t.hp() * t.wp() * t.cs * t.esize();
+        if (t.alias >= 0) {
+            t.offset = pl.tensors[t.alias].offset;
+            continue;
+        }
+        t.offset = off;
+        off = round_up(off + t.bytes + 256, 256);
+    }
+    plan->arena_bytes = off;
+    plan->tensors = pl.tensors;
+    for (auto& s : pl.steps) s->create(device, plan->tensors);
+    plan->steps = std::move(pl.steps);
+    for (size_t i = 0; i < pl.values.size(); ++i)
+        if (pl.values[i].kind == VK_TENSOR) {
+            plan->node_tensor[static_cast<int>(i)] = pl.values[i].tensor;
+        } else if (pl.values[i].kind == VK_MAT) {   // a view that is [rows, cols] with one row pitch
+            const View& v = pl.values[i].view;
+            const size_t r = v.rank();
+            bool ok = v.tensor >= 0 && r >= 1 && v.stride[r - 1] == 1;
+            for (size_t k = 0; ok && k + 2 < r; ++k) ok = v.stride[k] == v.stride[k + 1] * v.shape[k + 1];
+            if (ok) {
+                const int64_t cols = v.shape[r - 1], rows = v.numel() / cols;
+                plan->node_slice[static_cast<int>(i)] = {v.tensor, v.offset, rows, cols, r >= 2 ? v.stride[r - 2] : cols};
+            }
+        }
+    for (int p : g->params) {
+        const GNode& n = g->nodes[p];
+        plan->inputs.push_back({n.name, n.dtype, n.shape, n.numel() * (n.dtype == HIPIE_F32 || n.dtype == HIPIE_I32 ? 4 : 1)});
+    }
+    for (int r : g->results) {
+        const GNode& n = g->nodes[r];
+        const int dt = n.dtype == HIPIE_F32 ? HIPIE_F32 : HIPIE_U8;
+        plan->outputs.push_back({n.name, dt, n.shape, n.numel() * (dt == HIPIE_F32 ? 4 : 1)});
+    }
+    // Kernel selection by measurement on a scratch request (HIPIE_TUNE=0 keeps the shape-based
+    // defaults).  HIPIE_TUNE_FILE names a cache of the choices, one "step variant" pair a line:
+    // read when it matches this plan, written after tuning otherwise (the reference's GPU plugin
+    // keeps its tuning results in a file the same way, inference-engine/include/cldnn/cldnn_config.hpp:125 KEY_TUNING_FILE).
+    const char* tune_env = std::getenv("HIPIE_TUNE");
+    bool preset_used = false;
+    if (device >= 0 && preset && preset->size() == plan->steps.size()) {
+        bool match = true;
+        for (size_t i = 0; match && i < preset->size(); ++i) match = ((*preset)[i] < 0) == (plan->steps[i]->variant() < 0);
+        if (match) {
+            for (size_t i = 0; i < preset->size(); ++i) plan->steps[i]->set_variant((*preset)[i]);
+            preset_used = true;
+        }
+    }
+    if (device >= 0 && !preset_used && !(tune_env && tune_env[0] == '0')) {
+        const char* cache = std::getenv("HIPIE_TUNE_FILE");
+        bool loaded = false;
+        if (cache) {
+            if (FILE* f = std::fopen(cache, "r")) {
+                std::vector<int> v(plan->steps.size(), -2);
+                size_t n = 0;
+                int idx = 0, var = 0;
+                while (std::fscanf(f, "%d %d", &idx, &var) == 2)
+                    if (idx >= 0 && static_cast<size_t>(idx) < v.size() && v[idx] == -2) {
+                        v[idx] = var;
+                        ++n;
+                    }
+                std::fclose(f);
+                bool match = n == v.size();
+                for (size_t i = 0; match && i < v.size(); ++i)
+                    match = (v[i] < 0) == (plan->steps[i]->variant() < 0);
+                if (match) {
+                    for (size_t i = 0; i < v.size(); ++i) plan->steps[i]->set_variant(v[i]);
+                    loaded = true;
+                }
+            }
+        }
+        if (!loaded) {
+            // HIPIE_TUNE_STREAMS requests are assumed in flight together (default 3, the throughput
+            // mode of a plugin with three streams; 1 tunes for the latency of a lone request)
+            const char* ts = std::getenv("HIPIE_TUNE_STREAMS");
+            const int n_lanes = std::max(1, std::min(8, ts ? std::atoi(ts) : 3));
+            struct Scratch {
+                std::vector<hipie_request*> r;
+                ~Scratch() { for (auto* q : r) hipie_request_destroy(q); }
+            } scratch;
+            std::vector<TuneLane> lanes;
+            for (int l = 0; l < n_lanes; ++l) {
+                hipie_request* q = nullptr;
+                check_status(hipie_request_create(plan.get(), 0, &q), "hipie_compile: tuning request");
+                scratch.r.push_back(q);
+                TuneLane lane{q->arena.as<uint8_t>(), q->stream, {}};
+                for (auto& b : q->in_dev) lane.inputs.push_back(b.ptr);
+                lanes.push_back(std::move(lane));
+            }
+            DeviceGuard dg(device);
+            for (auto& s : plan->steps) s->tune(lanes, plan->tensors);
+            if (cache) {
+                if (FILE* f = std::fopen(cache, "w")) {
+                    for (size_t i = 0; i < plan->steps.size(); ++i)
+                        std::fprintf(f, "%zu %d\n", i, plan->steps[i]->variant());
+                    std::fclose(f);
+                }
+            }
+        }
+    }
+    return plan;
+}
+
+constexpr char kPlanMagic[8] = {'H', 'I', 'P', 'I', 'E', 'P', 'L', 'N'};
+constexpr uint32_t kPlanFormat = 1;
+
+uint64_t fnv1a(const uint8_t* p, size_t n) {
+    uint64_t h = 1469598103934665603ull;
+    for (size_t i = 0; i < n; ++i) h = (h ^ p[i]) * 1099511628211ull;
+    return h;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1812,107 +1937,64 @@ extern "C" {
 int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
     return guarded([&] {
         HIPIE_REQUIRE(g && out, HIPIE_PARAMETER_MISMATCH, "hipie_compile: null argument");
-        HIPIE_REQUIRE(!g->results.empty(), HIPIE_PARAMETER_MISMATCH, "hipie_compile: graph has no Result");
-        auto plan = std::make_unique<hipie_plan>();
-        plan->device = device;
-        Planner pl(*g);
-        for (int r : g->results) pl.visit(r);
-        // arena layout: one region per tensor, 256-byte aligned, with slack on both sides so that
-        // K-padding reads of a first-layer filter row stay inside the arena
-        int64_t off = 256;
-        for (auto& t : pl.tensors) {
-            t.bytes = static_cast<int64_t>(t.n) * t.hp() * t.wp() * t.cs * t.esize();
-            if (t.alias >= 0) {
-                t.offset = pl.tensors[t.alias].offset;
-                continue;
-            }
-            t.offset = off;
-            off = round_up(off + t.bytes + 256, 256);
+        *out = compile_plan(g, device, nullptr).release();
+    });
+}
+
+/* stream layout: magic[8], format u32, step count u32, one i32 kernel variant per step, graph bytes
+ * u64 + the graph description, FNV-1a of everything before it u64 */
+int hipie_plan_export(const hipie_plan* p, void* buffer, size_t capacity, size_t* size) {
+    return guarded([&] {
+        HIPIE_REQUIRE(p && size, HIPIE_PARAMETER_MISMATCH, "hipie_plan_export: null argument");
+        const size_t head = 16 + 4 * p->steps.size();
+        const size_t graph_bytes = serialize_graph(p->graph, nullptr);
+        *size = head + 8 + graph_bytes + 8;
+        if (!buffer) return;                              // size query
+        HIPIE_REQUIRE(capacity >= *size, HIPIE_OUT_OF_BOUNDS, "hipie_plan_export: %zu bytes needed, %zu given", *size, capacity);
+        uint8_t* b = static_cast<uint8_t*>(buffer);
+        std::memcpy(b, kPlanMagic, 8);
+        const uint32_t fmt = kPlanFormat, ns = static_cast<uint32_t>(p->steps.size());
+        std::memcpy(b + 8, &fmt, 4);
+        std::memcpy(b + 12, &ns, 4);
+        for (size_t i = 0; i < p->steps.size(); ++i) {
+            const int32_t v = p->steps[i]->variant();
+            std::memcpy(b + 16 + 4 * i, &v, 4);
         }
-        plan->arena_bytes = off;
-        plan->tensors = pl.tensors;
-        for (auto& s : pl.steps) s->create(device, plan->tensors);
-        plan->steps = std::move(pl.steps);
-        for (size_t i = 0; i < pl.values.size(); ++i)
-            if (pl.values[i].kind == VK_TENSOR) {
-                plan->node_tensor[static_cast<int>(i)] = pl.values[i].tensor;
-            } else if (pl.values[i].kind == VK_MAT) {   // a view that is [rows, cols] with one row pitch
-                const View& v = pl.values[i].view;
-                const size_t r = v.rank();
-                bool ok = v.tensor >= 0 && r >= 1 && v.stride[r - 1] == 1;
-                for (size_t k = 0; ok && k + 2 < r; ++k) ok = v.stride[k] == v.stride[k + 1] * v.shape[k + 1];
-                if (ok) {
-                    const int64_t cols = v.shape[r - 1], rows = v.numel() / cols;
-                    plan->node_slice[static_cast<int>(i)] = {v.tensor, v.offset, rows, cols, r >= 2 ? v.stride[r - 2] : cols};
-                }
-            }
-        for (int p : g->params) {
-            const GNode& n = g->nodes[p];
-            plan->inputs.push_back({n.name, n.dtype, n.shape, n.numel() * (n.dtype == HIPIE_F32 || n.dtype == HIPIE_I32 ? 4 : 1)});
+        const uint64_t gb = graph_bytes;
+        std::memcpy(b + head, &gb, 8);
+        serialize_graph(p->graph, b + head + 8);
+        const uint64_t h = fnv1a(b, *size - 8);
+        std::memcpy(b + *size - 8, &h, 8);
+    });
+}
+
+int hipie_plan_import(const void* blob, size_t size, int device, hipie_plan** out) {
+    return guarded([&] {
+        HIPIE_REQUIRE(blob && out, HIPIE_PARAMETER_MISMATCH, "hipie_plan_import: null argument");
+        const uint8_t* b = static_cast<const uint8_t*>(blob);
+        HIPIE_REQUIRE(size >= 8 + 4 + 4 + 8 + 8 && std::memcmp(b, kPlanMagic, 8) == 0, HIPIE_NETWORK_NOT_READ,
+                      "hipie_plan_import: not an exported plan");
+        uint32_t fmt, ns;
+        std::memcpy(&fmt, b + 8, 4);
+        std::memcpy(&ns, b + 12, 4);
+        HIPIE_REQUIRE(fmt == kPlanFormat, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: stream format %u, this library reads %u", fmt, kPlanFormat);
+        uint64_t stored;
+        std::memcpy(&stored, b + size - 8, 8);
+        HIPIE_REQUIRE(stored == fnv1a(b, size - 8), HIPIE_NETWORK_NOT_READ, "hipie_plan_import: checksum mismatch (damaged stream)");
+        HIPIE_REQUIRE(ns <= (size - 32) / 4, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: %u steps in %zu bytes", ns, size);
+        std::vector<int> variants(ns);
+        for (uint32_t i = 0; i < ns; ++i) {
+            int32_t v;
+            std::memcpy(&v, b + 16 + 4 * size_t(i), 4);
+            variants[i] = v;
         }
-        for (int r : g->results) {
-            const GNode& n = g->nodes[r];
-            const int dt = n.dtype == HIPIE_F32 ? HIPIE_F32 : HIPIE_U8;
-            plan->outputs.push_back({n.name, dt, n.shape, n.numel() * (dt == HIPIE_F32 ? 4 : 1)});
-        }
-        // Kernel selection by measurement on a scratch request (HIPIE_TUNE=0 keeps the shape-based
-        // defaults).  HIPIE_TUNE_FILE names a cache of the choices, one "step variant" pair a line:
-        // read when it matches this plan, written after tuning otherwise (the reference's GPU plugin
-        // keeps its tuning results in a file the same way, inference-engine/include/cldnn/cldnn_config.hpp:125 KEY_TUNING_FILE).
-        const char* tune_env = std::getenv("HIPIE_TUNE");
-        if (device >= 0 && !(tune_env && tune_env[0] == '0')) {
-            const char* cache = std::getenv("HIPIE_TUNE_FILE");
-            bool loaded = false;
-            if (cache) {
-                if (FILE* f = std::fopen(cache, "r")) {
-                    std::vector<int> v(plan->steps.size(), -2);
-                    size_t n = 0;
-                    int idx = 0, var = 0;
-                    while (std::fscanf(f, "%d %d", &idx, &var) == 2)
-                        if (idx >= 0 && static_cast<size_t>(idx) < v.size() && v[idx] == -2) {
-                            v[idx] = var;
-                            ++n;
-                        }
-                    std::fclose(f);
-                    bool match = n == v.size();
-                    for (size_t i = 0; match && i < v.size(); ++i)
-                        match = (v[i] < 0) == (plan->steps[i]->variant() < 0);
-                    if (match) {
-                        for (size_t i = 0; i < v.size(); ++i) plan->steps[i]->set_variant(v[i]);
-                        loaded = true;
-                    }
-                }
-            }
-            if (!loaded) {
-                // HIPIE_TUNE_STREAMS requests are assumed in flight together (default 3, the throughput
-                // mode of a plugin with three streams; 1 tunes for the latency of a lone request)
-                const char* ts = std::getenv("HIPIE_TUNE_STREAMS");
-                const int n_lanes = std::max(1, std::min(8, ts ? std::atoi(ts) : 3));
-                struct Scratch {
-                    std::vector<hipie_request*> r;
-                    ~Scratch() { for (auto* q : r) hipie_request_destroy(q); }
-                } scratch;
-                std::vector<TuneLane> lanes;
-                for (int l = 0; l < n_lanes; ++l) {
-                    hipie_request* q = nullptr;
-                    check_status(hipie_request_create(plan.get(), 0, &q), "hipie_compile: tuning request");
-                    scratch.r.push_back(q);
-                    TuneLane lane{q->arena.as<uint8_t>(), q->stream, {}};
-                    for (auto& b : q->in_dev) lane.inputs.push_back(b.ptr);
-                    lanes.push_back(std::move(lane));
-                }
-                DeviceGuard dg(device);
-                for (auto& s : plan->steps) s->tune(lanes, plan->tensors);
-                if (cache) {
-                    if (FILE* f = std::fopen(cache, "w")) {
-                        for (size_t i = 0; i < plan->steps.size(); ++i)
-                            std::fprintf(f, "%zu %d\n", i, plan->steps[i]->variant());
-                        std::fclose(f);
-                    }
-                }
-            }
-        }
-        *out = plan.release();
+        const size_t at = 16 + 4 * size_t(ns);
+        uint64_t gb;
+        std::memcpy(&gb, b + at, 8);
+        HIPIE_REQUIRE(gb == size - at - 16, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: graph description of %llu bytes in a stream of %zu",
+                      (unsigned long long)gb, size);
+        std::unique_ptr<hipie_graph> g(deserialize_graph(b + at + 8, static_cast<size_t>(gb)));
+        *out = compile_plan(g.get(), device, &variants).release();
     });
 }
 
@@ -1947,6 +2029,14 @@ int hipie_plan_step_info(const hipie_plan* p, int index, char* name, size_t name
         if (type && type_len) snprintf(type, type_len, "%s", s.type.c_str());
         if (macs) *macs = s.macs;
         if (bytes) *bytes = s.bytes;
+    });
+}
+
+int hipie_plan_step_variant(const hipie_plan* p, int index, int* variant) {
+    return guarded([&] {
+        HIPIE_REQUIRE(p && variant && index >= 0 && index < static_cast<int>(p->steps.size()), HIPIE_OUT_OF_BOUNDS,
+                      "hipie_plan_step_variant: index %d", index);
+        *variant = p->steps[index]->variant();
     });
 }
 

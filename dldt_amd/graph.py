@@ -165,9 +165,12 @@ class Graph:
 class Plan:
     """ExecutableNetwork analogue: fused steps + arena layout + uploaded constants."""
 
-    def __init__(self, graph, device=0):
+    def __init__(self, graph, device=0, _handle=None):
         self._h = ctypes.c_void_p()
-        check(lib().hipie_compile(graph._h, device, ctypes.byref(self._h)))
+        if _handle is not None:
+            self._h = _handle
+        else:
+            check(lib().hipie_compile(graph._h, device, ctypes.byref(self._h)))
         self.device = device
         L = lib()
         L.hipie_plan_arena_bytes.restype = ctypes.c_int64
@@ -179,15 +182,32 @@ class Plan:
             name, typ = ctypes.create_string_buffer(256), ctypes.create_string_buffer(64)
             macs, byts = ctypes.c_int64(), ctypes.c_int64()
             check(L.hipie_plan_step_info(self._h, i, name, 256, typ, 64, ctypes.byref(macs), ctypes.byref(byts)))
-            self.steps.append(dict(name=name.value.decode(), type=typ.value.decode(), macs=macs.value,
-                                   bytes=byts.value))
+            var = ctypes.c_int()
+            check(L.hipie_plan_step_variant(self._h, i, ctypes.byref(var)))
+            self.steps.append(dict(name=name.value.decode(errors="replace"), type=typ.value.decode(errors="replace"), macs=macs.value,
+                                   bytes=byts.value, variant=var.value))
+
+    def export(self):
+        """ExecutableNetwork::Export: the plan as bytes (graph description, constants, kernel choices)."""
+        size = ctypes.c_size_t()
+        check(lib().hipie_plan_export(self._h, None, ctypes.c_size_t(0), ctypes.byref(size)))
+        buf = ctypes.create_string_buffer(size.value)
+        check(lib().hipie_plan_export(self._h, buf, ctypes.c_size_t(size.value), ctypes.byref(size)))
+        return buf.raw[:size.value]
+
+    @classmethod
+    def load(cls, blob, device=0):
+        """Plugin::ImportNetwork: a plan from exported bytes; runs the kernels the exported plan ran."""
+        h = ctypes.c_void_p()
+        check(lib().hipie_plan_import(blob, ctypes.c_size_t(len(blob)), device, ctypes.byref(h)))
+        return cls(None, device, _handle=h)
 
     def _io(self, is_out, idx):
         name = ctypes.create_string_buffer(256)
         dt, rank = ctypes.c_int(), ctypes.c_int()
         dims = (ctypes.c_int64 * 4)()
         check(lib().hipie_plan_io_desc(self._h, is_out, idx, name, 256, ctypes.byref(dt), dims, ctypes.byref(rank)))
-        return dict(name=name.value.decode(), dtype=dt.value, shape=tuple(dims[:rank.value]))
+        return dict(name=name.value.decode(errors="replace"), dtype=dt.value, shape=tuple(dims[:rank.value]))
 
     def __del__(self):
         if getattr(self, "_h", None):

@@ -393,6 +393,18 @@ int hipie_graph_set_name(hipie_graph* g, int id, const char* friendly_name);
  * HBM arena, pack and upload constants.  The graph may be destroyed afterwards. */
 int hipie_compile(const hipie_graph* graph, int device, hipie_plan** plan);
 void hipie_plan_destroy(hipie_plan* plan);
+
+/* IExecutableNetworkInternal::Export(std::ostream&) (ie_iexecutable_network_internal.hpp:77-81) and
+ * IInferencePlugin::ImportNetwork(std::istream&, config) (ie_iplugin_internal.hpp:213-222), as the
+ * template plugin implements them (template_executable_network.cpp:179-201 writes the model,
+ * :43-75 reads it back and compiles it again).  The stream holds the graph description with its
+ * constants and the kernel variant chosen for every step, so an imported plan skips the timing runs
+ * of hipie_compile and runs the same kernels as the exported one; everything else (fusion, arena
+ * layout, constant packing) is redone, through the same validation as a newly described graph.
+ * hipie_plan_export with buffer == NULL only reports the size.  A stream that is truncated, damaged
+ * (checksum), of another format version or not a plan gives HIPIE_NETWORK_NOT_READ. */
+int hipie_plan_export(const hipie_plan* plan, void* buffer, size_t capacity, size_t* size);
+int hipie_plan_import(const void* stream, size_t size, int device, hipie_plan** plan);
 int hipie_plan_num_inputs(const hipie_plan* plan);
 int hipie_plan_num_outputs(const hipie_plan* plan);
 int hipie_plan_io_desc(const hipie_plan* plan, int is_output, int index, char* name, size_t name_len,
@@ -403,6 +415,9 @@ int64_t hipie_plan_arena_bytes(const hipie_plan* plan);
 int hipie_plan_num_steps(const hipie_plan* plan);
 int hipie_plan_step_info(const hipie_plan* plan, int index, char* name, size_t name_len, char* type,
                          size_t type_len, int64_t* macs, int64_t* bytes);
+/* the kernel variant a step runs (hipie_conv_set_tile numbering), -1 for a step without variants: part
+ * of what GetExecGraphInfo reports per executed node (exec_graph_info.hpp:34-76, implementation type) */
+int hipie_plan_step_variant(const hipie_plan* plan, int index, int* variant);
 
 /* IExecutableNetworkInternal::CreateInferRequestImpl: own stream + own activation arena; weights
  * stay shared in the plan.  perf_count mirrors the PERF_COUNT config key (ie_plugin_config.hpp:277). */

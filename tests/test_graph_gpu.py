@@ -203,3 +203,40 @@ def test_activation_zero_points(orc):
         np.testing.assert_array_equal(req.tensor(a["node"]), kept[a["node"]], err_msg=name)
         assert kept[a["node"]].min() == 0 and kept[a["node"]].max() == 255      # both ends saturate
     np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))
+
+
+@pytest.mark.parametrize("net", ["resnet", "encoder"])
+def test_exported_plan_runs_the_same_kernels(net, monkeypatch):
+    """ExecutableNetwork::Export -> Plugin::ImportNetwork: the imported plan takes its kernel variants from
+    the stream (no timing runs) and gives the exported plan's bytes"""
+    from dldt_amd import builders
+    from dldt_amd.graph import Plan
+    rng = np.random.default_rng(31)
+    if net == "resnet":
+        g, _ = builders.resnet50(batch=2, res=64, width=16, classes=10, seed=7)
+        feeds = [rng.uniform(0, 1, (2, 3, 64, 64)).astype(np.float32)]
+    else:
+        g, _ = builders.bert_encoder(layers=2, batch=2, seq=64, hidden=128, heads=2, ffn=256, seed=3)
+        feeds = [rng.normal(0, 1, (2, 64, 128)).astype(np.float32)]
+    monkeypatch.setenv("HIPIE_TUNE", "0")                # shape-based defaults in the exported plan ...
+    plan = g.compile()
+    want = plan.create_request().infer(*feeds)
+    blob = plan.export()
+    variants = [s["variant"] for s in plan.steps]
+    assert any(v >= 0 for v in variants)
+    monkeypatch.delenv("HIPIE_TUNE")                     # ... which a timing run at import would not keep everywhere
+    back = Plan.load(blob)
+    assert [s["variant"] for s in back.steps] == variants
+    assert [(s["name"], s["type"]) for s in back.steps] == [(s["name"], s["type"]) for s in plan.steps]
+    got = back.create_request().infer(*feeds)
+    for a, b in zip(got, want):
+        np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
+    tuned = g.compile()                                  # and the other way round: tuned choices survive HIPIE_TUNE=0
+    blob = tuned.export()
+    monkeypatch.setenv("HIPIE_TUNE", "0")
+    assert [s["variant"] for s in Plan.load(blob).steps] == [s["variant"] for s in tuned.steps]
+    monkeypatch.delenv("HIPIE_TUNE")
+    # a stream exported without a device (dry run) imports too: its steps carry no choices, the plan is tuned here
+    dry = Plan.load(g.compile(-1).export())
+    for a, b in zip(dry.create_request().infer(*feeds), want):
+        np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
