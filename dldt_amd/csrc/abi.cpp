@@ -38,4 +38,18 @@ int hipie_memcpy(void* dst, const void* src, size_t bytes, int to_device) {
     });
 }
 
+int hipie_host_alloc(size_t bytes, void** ptr) {
+    return guarded([&] {
+        HIPIE_REQUIRE(ptr, HIPIE_PARAMETER_MISMATCH, "hipie_host_alloc: null argument");
+        *ptr = nullptr;
+        HIPIE_CHECK_HIP(hipHostMalloc(ptr, bytes ? bytes : 1, hipHostMallocDefault));
+    });
+}
+
+int hipie_host_free(void* ptr) {
+    return guarded([&] {
+        if (ptr) HIPIE_CHECK_HIP(hipHostFree(ptr));
+    });
+}
+
 }  // extern "C"

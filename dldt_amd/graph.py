@@ -218,6 +218,23 @@ class Plan:
         return Request(self, perf_count)
 
 
+class PinnedArray:
+    """numpy array over page-locked host memory from hipie_host_alloc (`.array`); freed with the object"""
+
+    def __init__(self, shape, dtype):
+        self._p = ctypes.c_void_p()
+        n = int(np.prod(shape)) * np.dtype(dtype).itemsize
+        check(lib().hipie_host_alloc(ctypes.c_size_t(n), ctypes.byref(self._p)))
+        raw = (ctypes.c_uint8 * max(n, 1)).from_address(self._p.value)
+        self.array = np.frombuffer(raw, dtype=dtype, count=int(np.prod(shape))).reshape(shape)
+
+    def __del__(self):
+        if getattr(self, "_p", None):
+            self.array = None
+            lib().hipie_host_free(self._p)
+            self._p = None
+
+
 class Request:
     """InferRequest analogue: own stream and activation arena."""
 
@@ -241,6 +258,22 @@ class Request:
         op = (ctypes.c_void_p * len(outs))(*[a.ctypes.data for a in outs])
         check(lib().hipie_request_infer(self._h, ip, op, 0))
         return outs
+
+    def host_buffers(self):
+        """page-locked numpy arrays shaped like the plan's inputs and outputs (the request's blobs)"""
+        return ([PinnedArray(d["shape"], _NP[d["dtype"]]) for d in self.plan.inputs],
+                [PinnedArray(d["shape"], _NP[d["dtype"]]) for d in self.plan.outputs])
+
+    def start(self, ins, outs):
+        """StartAsync from host buffers (PinnedArray or numpy): copies and kernels are queued on the
+        request's stream; wait() returns when the outputs are complete."""
+        arr = lambda b: b.array if isinstance(b, PinnedArray) else b
+        ip = (ctypes.c_void_p * len(ins))(*[arr(b).ctypes.data for b in ins])
+        op = (ctypes.c_void_p * len(outs))(*[arr(b).ctypes.data for b in outs])
+        check(lib().hipie_request_start(self._h, ip, op, 0))
+
+    def wait(self):
+        check(lib().hipie_request_wait(self._h))
 
     def device_buffers(self):
         """torch tensors shaped like the plan's inputs and outputs (for resident-in-HBM runs)."""

@@ -72,6 +72,14 @@ int hipie_device_count(void);
 int hipie_device_name(int device, char* buf, size_t buf_len);
 /* synchronous copy between host and device memory (to_device = 1: host -> device) */
 int hipie_memcpy(void* dst, const void* src, size_t bytes, int to_device);
+/* Page-locked host memory for the blobs of an infer request (the allocator a plugin gives its
+ * input / output blobs in InferRequest::allocateBlobs, template_infer_request.cpp:63-101): from such
+ * buffers hipie_request_start returns as soon as the copies and kernels are queued, and the copies run
+ * at the link's rate (pageable buffers are copied through the runtime's own staging, about 40 % slower
+ * and synchronously).  Allocated fresh (never registered over existing memory); free with
+ * hipie_host_free before the process ends. */
+int hipie_host_alloc(size_t bytes, void** ptr);
+int hipie_host_free(void* ptr);
 
 /* ======================================================================================
  * Activation tensors handed to the engine's kernels: NHWC, channel stride 1, with a readable

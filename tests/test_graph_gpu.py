@@ -240,3 +240,39 @@ def test_exported_plan_runs_the_same_kernels(net, monkeypatch):
     dry = Plan.load(g.compile(-1).export())
     for a, b in zip(dry.create_request().infer(*feeds), want):
         np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_asynchronous_requests_from_page_locked_blobs():
+    """StartAsync / Wait over the request's own page-locked blobs, three requests in flight with different
+    images (benchmark_app's loop): results equal the synchronous host path; a started request is busy, and
+    waiting on an idle one is an error"""
+    from dldt_amd import HipieError, builders
+    g, _ = builders.resnet50(batch=4, res=96, width=32, classes=16, seed=5)
+    plan = g.compile()
+    rng = np.random.default_rng(12)
+    xs = [rng.uniform(0, 1, (4, 3, 96, 96)).astype(np.float32) for _ in range(7)]
+    sync = plan.create_request()
+    want = [sync.infer(x)[0].copy() for x in xs]
+    reqs = [plan.create_request() for _ in range(3)]
+    blobs = [r.host_buffers() for r in reqs]
+    got = [None] * len(xs)
+    running = {}
+    for i, x in enumerate(xs):
+        k = i % 3
+        if k in running:
+            reqs[k].wait()
+            got[running.pop(k)] = blobs[k][1][0].array.copy()
+        blobs[k][0][0].array[...] = x
+        reqs[k].start(*blobs[k])
+        running[k] = i
+    with pytest.raises(HipieError) as e:                 # REQUEST_BUSY: already started
+        reqs[0].start(*blobs[0])
+    assert e.value.status == -8
+    for k, i in running.items():
+        reqs[k].wait()
+        got[i] = blobs[k][1][0].array.copy()
+    with pytest.raises(HipieError) as e:                 # INFER_NOT_STARTED
+        reqs[0].wait()
+    assert e.value.status == -11
+    for a, b in zip(got, want):
+        np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
