@@ -333,3 +333,50 @@ def test_conv_input_zero_point(orc, signed, zp, depthwise):
     out = DeviceTensor(N, H, W, OC, I32)
     conv.run(xin, out)
     np.testing.assert_array_equal(out.to_nchw(), want)
+
+
+_WIDE_CASES = {}
+
+
+@pytest.mark.parametrize("tile", [0, 1, 4, 5, 6, 7, 10, 11])
+@pytest.mark.parametrize("kind", ["f32", "f32_res", "i8"])
+def test_conv_variants_on_ragged_channel_tiles(orc, kind, tile):
+    """320 output channels (two and a half 128-channel tiles, five of 64), 722 pixels (ragged
+    in every tile shape), f32 results with and without a late f32 residual and signed i8 levels: the
+    encoder GEMMs' epilogues, through every variant the tuner may pick for them."""
+    import torch
+    from dldt_amd import Convolution, DeviceTensor, make_epilogue
+    g = (2, 256, 19, 19, 320, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0))
+    if kind not in _WIDE_CASES:
+        rng = np.random.default_rng(zlib.crc32(kind.encode()) + 1)
+        x, w = _inputs(rng, g, signed=True)
+        acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+        OC = g[4]
+        amax = np.float32(np.abs(acc).max())
+        bias = rng.normal(0, amax / 20, OC).astype(np.float32)
+        scale = (rng.uniform(0.5, 2.0, OC) / amax).astype(np.float32)
+        res = None
+        if kind == "f32":
+            want, epi = _chain(orc, acc, bias=bias, scale=scale), dict(bias=bias, scale=scale, out_dtype=F32)
+        elif kind == "f32_res":
+            res = rng.normal(0, 1, acc.shape).astype(np.float32)
+            want = _chain(orc, acc, bias=bias, scale=scale, res=res)
+            epi = dict(bias=bias, scale=scale, residual_dtype=F32, out_dtype=F32)
+        else:
+            fq = (256, np.float32(-1.28), np.float32(1.27), -128.0, 127.0)
+            want = _chain(orc, acc, bias=bias, scale=scale, fq=fq).astype(np.int8)
+            epi = dict(bias=bias, scale=scale, out_dtype=I8, fq=fq)
+        _WIDE_CASES[kind] = (x, w, res, epi, want)
+    x, w, res, epi, want = _WIDE_CASES[kind]
+    xin = _device_in(x, g, signed=True)
+    conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10], make_epilogue(**epi))
+    conv.set_tile(tile)
+    out = DeviceTensor(2, 19, 19, 320, epi["out_dtype"])
+    rt = DeviceTensor.from_nchw(res, F32) if res is not None else None
+    conv.run(xin, out, rt)
+    torch.cuda.synchronize()
+    got = out.to_nchw()
+    if kind == "i8":
+        np.testing.assert_array_equal(got.view(np.int8) if got.dtype == np.uint8 else got.astype(np.int8), want)
+    else:
+        np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
