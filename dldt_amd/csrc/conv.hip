@@ -24,8 +24,12 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     constexpr int NT = WOC * WPIX * 64;
     constexpr int BOC = WOC * 64, BPIX = WPIX * 64;
     constexpr int A_PIECES = BOC * 4 / NT, B_PIECES = BPIX * 4 / NT;
-    __shared__ __attribute__((aligned(16))) int8_t sA[2][BOC * kRow];
-    __shared__ __attribute__((aligned(16))) int8_t sB[2][BPIX * kRow];
+    // PAIR: eight neighbouring lanes of a store instruction write one row of both buffers (the two steps
+    // of a pair).  The second buffer sits 128 bytes further and holds row r at position r ^ 1, so those
+    // two 64-byte pieces, and the four of sixteen lanes, fall on different LDS banks
+    constexpr int kBufPad = PAIR ? 128 : 0;
+    __shared__ __attribute__((aligned(256))) int8_t sA[2][BOC * kRow + kBufPad];
+    __shared__ __attribute__((aligned(256))) int8_t sB[2][BPIX * kRow + kBufPad];
     __shared__ __attribute__((aligned(16))) float sP[PT_ROWS * BOC];
 
     // block -> (pixel tile, channel tile): consecutive pixel tiles stay on one XCD
@@ -88,10 +92,10 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
                 v4i af[2], bf[2];
 #pragma unroll
                 for (int ob = 0; ob < 2; ++ob)
-                    af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][a_row[ob] * kRow + frag_slot[ks]]);
+                    af[ob] = *reinterpret_cast<const v4i*>(&sA[buf][(a_row[ob] ^ (PAIR ? buf : 0)) * kRow + frag_slot[ks]]);
 #pragma unroll
                 for (int pb = 0; pb < 2; ++pb)
-                    bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][b_row[pb] * kRow + frag_slot[ks]]);
+                    bf[pb] = *reinterpret_cast<const v4i*>(&sB[buf][(b_row[pb] ^ (PAIR ? buf : 0)) * kRow + frag_slot[ks]]);
 #pragma unroll
                 for (int ob = 0; ob < 2; ++ob)
 #pragma unroll
@@ -146,10 +150,10 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
             auto store_pair = [&]() {
 #pragma unroll
                 for (int i = 0; i < A_P2; ++i)
-                    *reinterpret_cast<v4i*>(&sA[sub][(row0 + i * RPI) * kRow + slot2]) = ga2[i];
+                    *reinterpret_cast<v4i*>(&sA[sub][((row0 + i * RPI) ^ sub) * kRow + slot2]) = ga2[i];
 #pragma unroll
                 for (int i = 0; i < B_P2; ++i)
-                    *reinterpret_cast<v4i*>(&sB[sub][(row0 + i * RPI) * kRow + slot2]) = gb2[i];
+                    *reinterpret_cast<v4i*>(&sB[sub][((row0 + i * RPI) ^ sub) * kRow + slot2]) = gb2[i];
             };
             const int npairs = (nk + 1) >> 1;
             load_pair(0);
