@@ -406,25 +406,11 @@ constexpr int waitcnt_vm(int n) {
     return 0x0F70 | (n & 15) | ((n >> 4) << 14);
 }
 
-// wait until at most LPS * younger of this wave's loads are outstanding (younger = 0..6 stages)
-template <int LPS>
-__device__ __forceinline__ void wait_vmcnt_stages(int younger) {
-    switch (younger) {
-    case 0: __builtin_amdgcn_s_waitcnt(waitcnt_vm(0)); break;
-    case 1: __builtin_amdgcn_s_waitcnt(waitcnt_vm(LPS)); break;
-    case 2: __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * LPS)); break;
-    case 3: __builtin_amdgcn_s_waitcnt(waitcnt_vm(3 * LPS)); break;
-    case 4: __builtin_amdgcn_s_waitcnt(waitcnt_vm(4 * LPS)); break;
-    case 5: __builtin_amdgcn_s_waitcnt(waitcnt_vm(5 * LPS)); break;
-    default: __builtin_amdgcn_s_waitcnt(waitcnt_vm(6 * LPS)); break;
-    }
-}
-
 // KS = 2: eight waves; wave group g (four waves, own ring) multiplies the K steps k = g mod 2 and
 // group 1 hands its partial sums to group 0 through LDS.  Twice the waves per compute unit keep
 // twice the loads in flight, which is what bounds the layers with fewer tiles than compute units.
 template <int WOC, int WPIX, uint32_t F, int KS>
-__global__ __launch_bounds__(WOC* WPIX * 64 * KS, KS == 2 ? 1 : ((F != kDyn && (F & CF_RES_GEMM)) ? 2 : 3))
+__global__ __launch_bounds__(WOC* WPIX * 64 * KS, KS == 2 ? 1 : 2)
 void conv_pipe_kernel(const ConvArgs a, const int stages) {
     constexpr int NT = WOC * WPIX * 64;          // threads of one wave group
     constexpr int NT_ALL = NT * KS;
@@ -448,7 +434,9 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
     const int pix0 = p_tile * BPIX, oc0 = t_tile * BOC;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    const int grp = KS == 1 ? 0 : (tid / NT), wave = (tid >> 6) % (NT / 64);
+    // wave-uniform by construction; said so, or the LDS base of every DMA load goes through a VGPR
+    const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = KS == 1 ? 0 : wave_all / (NT / 64), wave = wave_all % (NT / 64);
     const int woc = wave % WOC, wpix = wave / WOC;
     int8_t* const gring = ring + grp * stages * STAGE;
     const int l32 = lane & 31, h = lane >> 5;
@@ -491,13 +479,10 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
         int32_t* kt = reinterpret_cast<int32_t*>(ring + KS * stages * STAGE + PT_ROWS * BOC * 4);
         for (int i = tid; i < 4 * nk_all; i += NT_ALL) kt[i] = koff[i];
         __syncthreads();
-        int32_t off_next = kt[4 * grp + dma_chunk];
-        auto issue = [&](int stage, int j) {
+        auto issue = [&](int stage, int j, int32_t off) {
             int8_t* sa = gring + stage * STAGE;
             int8_t* sb = sa + BOC * 64;
             const int k = j * KS + grp;
-            const int32_t off = off_next;
-            off_next = kt[4 * (min(j + 1, nk - 1) * KS + grp) + dma_chunk];   // steps are issued in order
 #pragma unroll
             for (int i = 0; i < A_GROUPS; ++i)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(a_ptr[i] + k * 64),
@@ -509,18 +494,18 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
                                                  (__attribute__((address_space(3))) void*)(sb + (wave * B_GROUPS + i) * 1024),
                                                  16, 0, 0);
         };
-        // Software pipeline (stages >= 3).  Iteration k multiplies step k in two halves of 32 K
-        // bytes; the fragments of each half are read from LDS while the other half is in the matrix
+        // Software pipeline over a ring of 3 to 8 stages.  Iteration k multiplies step k in two halves of
+        // 32 K bytes; the fragments of each half are read from LDS while the other half is in the matrix
         // pipe, and the barrier sits between the halves:
         //   read (k, half 1) | mfma (k, half 0) | wait own loads of step k+1, barrier |
         //   refill the slot of step k-1 with step k+stages-1 | read (k+1, half 0) | mfma (k, half 1)
         // After barrier k every wave's part of step k+1 has landed and every wave has consumed
-        // step k-1, whose slot is the one refilled.
-        const int ahead = min(stages - 1, nk);
-        for (int s0 = 0; s0 < ahead; ++s0) issue(s0, s0);
-        wait_vmcnt_stages<LPS>(min(ahead - 1, 6));
-        __builtin_amdgcn_s_barrier();
-        int rd = 0, wr = ahead % stages;
+        // step k-1, whose slot is the one refilled.  A layer with no more workgroups than compute
+        // units has ONE wave per SIMD, and whatever that wave waits for between two matrix
+        // instructions is time the matrix pipe idles: the loop body is straight-line code (last
+        // iteration peeled, the K offset of the step to request read at the top, the ring depth a
+        // constant of the loop so that its wait is one instruction), and a deep ring keeps the
+        // slowest of a step's 256 cache lines (an L2 miss among them, most steps) off the critical path.
         v4i fa[2][2], fb[2][2];
         auto read_frags = [&](int slot, int ks, v4i (&af)[2], v4i (&bf)[2]) {
             const int8_t* sa = gring + slot * STAGE + (woc * 64) * 64;
@@ -537,23 +522,45 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
                 for (int pb = 0; pb < 2; ++pb)
                     acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
         };
-        read_frags(0, 0, fa[0], fb[0]);
-        for (int k = 0; k < nk; ++k) {
-            read_frags(rd, 1, fa[1], fb[1]);
-            mfma4(fa[0], fb[0]);
-            const int nrd = rd + 1 == stages ? 0 : rd + 1;
-            if (k + 1 < nk) {
-                // outstanding: steps k+1 .. min(k + stages - 2, nk - 1)
-                wait_vmcnt_stages<LPS>(min(min(stages - 3, nk - 2 - k), 6));
+        static_assert(5 * LPS < 64, "vmcnt is a 6-bit counter");
+        const int ahead = min(stages - 1, nk);
+        for (int s0 = 0; s0 < ahead; ++s0) issue(s0, s0, kt[4 * (s0 * KS + grp) + dma_chunk]);
+        // the loop for a ring of Y + 3 stages: in the steady state Y younger steps stay in flight behind
+        // step k+1; towards the end the wait is for everything (what is left in flight is due next anyway)
+        auto loop = [&](auto depth) {
+            constexpr int Y = decltype(depth)::value;
+            if (ahead - 1 >= Y + 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm((Y + 1) * LPS));   // step 0 of a full ring
+            else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+            __builtin_amdgcn_s_barrier();
+            int rd = 0, wr = ahead % stages;
+            read_frags(0, 0, fa[0], fb[0]);
+            for (int k = 0; k + 1 < nk; ++k) {
+                const int kn = k + Y + 2;                                        // the step requested in this iteration
+                const int32_t off_req = kt[4 * (min(kn, nk - 1) * KS + grp) + dma_chunk];
+                read_frags(rd, 1, fa[1], fb[1]);
+                mfma4(fa[0], fb[0]);
+                const int nrd = rd + 1 == Y + 3 ? 0 : rd + 1;
+                // outstanding: steps k+1 .. min(k + Y + 1, nk - 1)
+                if (k + Y + 1 < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm(Y * LPS));
+                else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
                 __builtin_amdgcn_s_barrier();
-                if (k + stages - 1 < nk) {
-                    issue(wr, k + stages - 1);
-                    wr = wr + 1 == stages ? 0 : wr + 1;
+                if (kn < nk) {
+                    issue(wr, kn, off_req);
+                    wr = wr + 1 == Y + 3 ? 0 : wr + 1;
                 }
                 read_frags(nrd, 0, fa[0], fb[0]);
+                mfma4(fa[1], fb[1]);
+                rd = nrd;
             }
+            read_frags(rd, 1, fa[1], fb[1]);                                     // last step: nothing left to request
+            mfma4(fa[0], fb[0]);
             mfma4(fa[1], fb[1]);
-            rd = nrd;
+        };
+        switch (stages) {                                                        // uniform
+        case 3: loop(std::integral_constant<int, 0>{}); break;
+        case 4: loop(std::integral_constant<int, 1>{}); break;
+        case 6: loop(std::integral_constant<int, 3>{}); break;
+        default: loop(std::integral_constant<int, 5>{}); break;                  // 8
         }
         __builtin_amdgcn_s_barrier();   // every wave is done reading before the ring is refilled
     };
@@ -765,13 +772,16 @@ void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) 
     const uint32_t core = a.flags & ~CF_OUT_XOR;
 #define HIPIE_LAUNCH_PIPE(FLAGS, ...)                                                                       \
     do {                                                                                                    \
-        static bool attr_set = false;                                                                       \
-        if (!attr_set) {                                                                                    \
-            HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_pipe_kernel<WOC, WPIX, FLAGS, KS>), \
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));   \
-            attr_set = true;                                                                                \
+        if constexpr ((FLAGS) != kDyn && ((FLAGS) & CF_RES_GEMM)) break;   /* the second GEMM exists in the tiled kernel only */ \
+        else {                                                                                              \
+            static bool attr_set = false;                                                                   \
+            if (!attr_set) {                                                                                \
+                HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_pipe_kernel<WOC, WPIX, FLAGS, KS>), \
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
+                attr_set = true;                                                                            \
+            }                                                                                               \
+            hipLaunchKernelGGL((conv_pipe_kernel<WOC, WPIX, FLAGS, KS>), grid, block, lds, s, a, stages);   \
         }                                                                                                   \
-        hipLaunchKernelGGL((conv_pipe_kernel<WOC, WPIX, FLAGS, KS>), grid, block, lds, s, a, stages);       \
     } while (0)
     HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_PIPE, 0)
 #undef HIPIE_LAUNCH_PIPE
@@ -1271,7 +1281,7 @@ int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
         HIPIE_REQUIRE(c && tile >= 0 && tile <= 11, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
         if (c->depthwise) return;               // one kernel only
-        if (c->fused && tile != 0 && tile != 4) return;   // the second GEMM exists in the 128 x 128 kernels
+        if (c->fused && tile != 0) return;      // the second GEMM exists in the 128 x 128 tiled kernel
         HIPIE_REQUIRE(tile < 8 || tile > 9 || (!c->fused && persist_available(c->epi.flags)), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the persistent kernels exist for byte outputs with a byte residual or none");
         HIPIE_REQUIRE(tile < 6 || tile > 7 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
@@ -1451,8 +1461,10 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         hipStream_t s = as_stream(stream);
         // ring depth: enough K steps in flight to cover the load latency, within 160 KB of LDS
         const int stage_bytes = (square ? 256 : 320) * 64 * (tile >= 6 ? 2 : 1);
-        const int max_stages = std::min(8, (144 * 1024) / stage_bytes);   // at most 6 younger stages + current + refill
-        const int stages = c->stages > 0 ? std::max(3, std::min(c->stages, max_stages)) : (tile == 4 ? 4 : 3);
+        // ring depth: 3, 4, 6 or 8 K steps (the depths the kernel has loops for), within 160 KB of LDS
+        const int max_stages = (144 * 1024) / stage_bytes;
+        int stages = c->stages > 0 ? c->stages : (tile == 4 ? 4 : 3);
+        stages = stages >= 8 && max_stages >= 8 ? 8 : (stages >= 6 && max_stages >= 6 ? 6 : (stages >= 4 && max_stages >= 4 ? 4 : 3));
         switch (tile) {
         case 4: launch_pipe<2, 2, 1>(a, stages, s); break;
         case 5: launch_pipe<1, 4, 1>(a, stages, s); break;

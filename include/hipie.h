@@ -233,7 +233,8 @@ int hipie_conv_get_tile(const hipie_conv* conv, int* tile);
 /* diagnostics: the epilogue's step flags (conv_kernel.h ConvFlags) and whether a kernel instance with
  * these steps compiled in exists (otherwise the generic, slower instance runs) */
 int hipie_conv_epilogue_flags(const hipie_conv* conv, uint32_t* flags, int* specialised);
-/* ring depth (2..8 K steps in LDS) of the pipelined variants; 0 = choose from K */
+/* ring depth of the pipelined variants: 3, 4, 6 or 8 K steps in LDS (other values round down, and to
+ * what fits 144 KB); 0 = the variant's default (4 for tile 4, else 3) */
 int hipie_conv_set_stages(hipie_conv* conv, int stages);
 int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,
                    const hipie_tensor* out, void* stream);
