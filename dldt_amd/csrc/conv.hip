@@ -628,6 +628,123 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// Row-tile kernel for 3 x 3, stride 1, pad 1 convolutions: the implicit GEMM above fetches every input
+// pixel once per filter tap (nine times), and the path from L2 into the compute unit is what bounds
+// these layers.  Here a workgroup takes whole output rows of one image (R rows, R * OW <= 256 pixels)
+// and 64 output channels; per 64 input channels it stages the input patch ((R + 2) x (OW + 2) pixels,
+// read from the tensor's own halo where the filter overhangs) and the nine 64-byte weight slices ONCE
+// in LDS, and the nine taps read their B fragments from the patch at shifted positions.  No barrier
+// inside the 72 matrix instructions of a chunk.  LDS rows are 64 bytes (patch pixels) and 576 bytes
+// (weights: 64 mod 256, so the same bank picture), chunk c of row r in slot c ^ ((r >> 2) & 3).
+constexpr int kPatchRows = 384;   // 24 KB: three waves' staging space later
+template <uint32_t F>
+__global__ __launch_bounds__(256, 2) void conv_rows_kernel(const ConvArgs a) {
+    __shared__ __attribute__((aligned(16))) int8_t sPatch[kPatchRows * 64];
+    __shared__ __attribute__((aligned(16))) int8_t sW[64 * 576];
+    __shared__ __attribute__((aligned(16))) float sP[PT_ROWS * 64];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, h = lane >> 5;
+    int p_tile, t_tile;
+    split_tile_index(a, blockIdx.x, p_tile, t_tile);
+    const int oc0 = t_tile * 64;
+    const int n = p_tile / a.tiles_per_image, ty = p_tile - n * a.tiles_per_image;
+    const int OH = a.OHOW / a.OW;
+    const int y0 = ty * a.rows_per_tile;                                  // first output row of the tile
+    const int rows = min(a.rows_per_tile, OH - y0);
+    const int count = rows * a.OW;                                        // pixels of this tile
+    const int pix0 = n * a.OHOW + y0 * a.OW;
+    const int PW = a.patch_w, patch_rows = (rows + 2) * PW;
+    const int oc_lane = oc0 + 32 * h;
+    stage_params<F>(a, oc0, (lds_float_ptr)sP, 64, tid, 256);
+
+    // patch position of the lane's two pixels at tap (0, 0)
+    int idx0[2];
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+        const int p = min(wave * 64 + pb * 32 + l32, count - 1);
+        int r, x;
+        fast_divmod(p, a.OW, a.inv_OW, r, x);
+        idx0[pb] = r * PW + x;
+    }
+    // input element (n, y0 - 1, -1, 0): the patch's first pixel (in the halo)
+    const int8_t* in0 = a.in + (static_cast<int64_t>(n) * a.in_sn + (y0 - 1) * a.in_sh - a.in_sw);
+    const int8_t* w0 = a.wgt + static_cast<int64_t>(oc0) * a.wgt_ld;
+
+    v16i acc[2][2];
+    v16f rres[2][2];
+    init_acc(a, oc_lane, acc);
+    const int chunks = a.Kp / 576;                                        // 64-channel slices of the input
+    for (int c = 0; c < chunks; ++c) {
+        if (c > 0) __syncthreads();                                       // everyone is done with the previous slice
+        // all requests of the slice go out before the first of them is awaited
+        constexpr int PP = kPatchRows * 4 / 256;                          // patch pieces per thread, at most
+        v4i pv[PP], wv[9];
+#pragma unroll
+        for (int j = 0; j < PP; ++j) {
+            const int i = min(tid + j * 256, patch_rows * 4 - 1);
+            const int row = i >> 2, ch = i & 3;
+            int py, px;
+            fast_divmod(row, PW, a.inv_patch_w, py, px);
+            pv[j] = *reinterpret_cast<const v4i*>(in0 + (py * a.in_sh + px * a.in_sw + c * 64 + ch * 16));
+        }
+#pragma unroll
+        for (int j = 0; j < 9; ++j) {                                     // 64 rows x 9 taps x 4 chunks = 9 x 256 pieces
+            const int i = tid + j * 256;
+            const int row = i / 36, rem = i - row * 36, tap = rem >> 2, ch = rem & 3;
+            const int wrow = min(oc0 + row, a.wgt_rows - 1) - oc0;
+            wv[j] = *reinterpret_cast<const v4i*>(w0 + (static_cast<int64_t>(wrow) * a.wgt_ld + tap * (chunks * 64) + c * 64 + ch * 16));
+        }
+#pragma unroll
+        for (int j = 0; j < PP; ++j) {
+            const int i = tid + j * 256;
+            const int row = i >> 2, ch = i & 3;
+            if (i < patch_rows * 4) *reinterpret_cast<v4i*>(&sPatch[row * 64 + ((ch ^ ((row >> 2) & 3)) << 4)]) = pv[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 9; ++j) {
+            const int i = tid + j * 256;
+            const int row = i / 36, rem = i - row * 36, tap = rem >> 2, ch = rem & 3;
+            *reinterpret_cast<v4i*>(&sW[row * 576 + tap * 64 + ((ch ^ ((row >> 2) & 3)) << 4)]) = wv[j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw) {
+                const int tap = kh * 3 + kw;
+                int idx[2];
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb) idx[pb] = idx0[pb] + kh * PW + kw;
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    v4i af[2], bf[2];
+#pragma unroll
+                    for (int ob = 0; ob < 2; ++ob) {
+                        const int row = ob * 32 + l32;
+                        af[ob] = *reinterpret_cast<const v4i*>(&sW[row * 576 + tap * 64 + (((2 * ks + h) ^ ((row >> 2) & 3)) << 4)]);
+                    }
+#pragma unroll
+                    for (int pb = 0; pb < 2; ++pb)
+                        bf[pb] = *reinterpret_cast<const v4i*>(&sPatch[idx[pb] * 64 + (((2 * ks + h) ^ ((idx[pb] >> 2) & 3)) << 4)]);
+#pragma unroll
+                    for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                        for (int pb = 0; pb < 2; ++pb)
+                            acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
+                }
+            }
+    }
+    __syncthreads();                                                      // the patch becomes the stores' staging space
+    ConvArgs e = a;
+    e.M = min(a.M, pix0 + count);                                         // pixels behind the tile's rows belong to the next tile
+    const int m0 = pix0 + wave * 64 + l32;
+    lds_float_ptr stage = wave < 3 ? (lds_float_ptr)&sPatch[0] + wave * 2048 : (lds_float_ptr)&sW[0];
+    run_epilogue<F>(e, acc, oc_lane, m0, m0 + 32, 0, rres, (lds_cfloat_ptr)sP, 64, oc0, stage);
+}
+
+// ------------------------------------------------------------------------------------------------
 // Streaming kernel: grid (x, channel tiles of 64); a workgroup of 4 waves walks pixel tiles of 256
 // (64 per wave) with stride gridDim.x.  Dynamic LDS: 64 rows of (Kp + 16) weight bytes.
 template <uint32_t F>
@@ -785,6 +902,29 @@ void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) 
     } while (0)
     HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_PIPE, 0)
 #undef HIPIE_LAUNCH_PIPE
+}
+
+bool rows_kernel_fits(const hipie_conv_desc& d) {
+    return d.groups == 1 && d.kh == 3 && d.kw == 3 && d.stride_h == 1 && d.stride_w == 1 && d.dil_h == 1 && d.dil_w == 1 &&
+           d.pad_top == 1 && d.pad_bottom == 1 && d.pad_left == 1 && d.pad_right == 1 && d.ic % 64 == 0;
+}
+
+// output rows per tile: at most 256 pixels, and a patch of (R + 2) x (OW + 2) pixels within the LDS buffer; 0: none fits
+int rows_per_tile(int oh, int ow) {
+    const int r = std::min(std::min(256 / ow, kPatchRows / (ow + 2) - 2), oh);
+    return r >= 1 ? r : 0;
+}
+
+void launch_rows(const ConvArgs& a, hipStream_t s) {
+    const dim3 grid(a.p_tiles * a.t_tiles), block(256);
+    const uint32_t core = a.flags & ~CF_OUT_XOR;
+#define HIPIE_LAUNCH_ROWS(FLAGS, ...)                                                    \
+    do {                                                                                 \
+        if constexpr ((FLAGS) != kDyn && ((FLAGS) & CF_RES_GEMM)) break;                  \
+        else hipLaunchKernelGGL((conv_rows_kernel<FLAGS>), grid, block, 0, s, a);        \
+    } while (0)
+    HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_ROWS, 0)
+#undef HIPIE_LAUNCH_ROWS
 }
 
 // the template instances of the persistent kernel: byte outputs and byte / no residual
@@ -1279,13 +1419,15 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 11, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 12, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
         if (c->depthwise) return;               // one kernel only
         if (c->fused && tile != 0) return;      // the second GEMM exists in the 128 x 128 tiled kernel
         HIPIE_REQUIRE(tile < 8 || tile > 9 || (!c->fused && persist_available(c->epi.flags)), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the persistent kernels exist for byte outputs with a byte residual or none");
         HIPIE_REQUIRE(tile < 6 || tile > 7 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the split-K kernels need an even number of 64-byte K steps (K=%lld)", (long long)c->Kp);
+        HIPIE_REQUIRE(tile != 12 || rows_kernel_fits(c->d), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_set_tile: the row-tile kernel takes 3 x 3, stride 1, pad 1, undilated convolutions over a multiple of 64 input channels");
         HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) + PT_ROWS * 64 * 4 <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: K=%lld does not fit the streaming kernel's LDS", (long long)c->Kp);
         c->tile = tile;
@@ -1446,7 +1588,25 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
             HIPIE_CHECK_HIP(hipGetLastError());
             return;
         }
-        const int tile = c->tile;
+        int tile = c->tile;
+        if (tile == 12) {
+            const int R = rows_per_tile(oh, ow);
+            if (R == 0 || in->halo < 1) {
+                tile = 0;                     // rows too wide for a patch: the general kernel
+            } else {
+                a.rows_per_tile = R;
+                a.tiles_per_image = static_cast<int32_t>(ceil_div(oh, R));
+                a.patch_w = ow + 2;
+                a.inv_patch_w = 1.0f / static_cast<float>(ow + 2);
+                a.p_tiles = in->n * a.tiles_per_image;
+                a.t_tiles = static_cast<int32_t>(ceil_div(d.oc, 64));
+                a.t_shift = (a.t_tiles & (a.t_tiles - 1)) == 0 ? __builtin_ctz(a.t_tiles) : -1;
+                DeviceGuard g(c->device);
+                launch_rows(a, as_stream(stream));
+                HIPIE_CHECK_HIP(hipGetLastError());
+                return;
+            }
+        }
         const bool square = tile == 0 || tile == 4 || tile == 6 || tile == 8 || tile == 10;
         const int boc = square ? 128 : 64;
         const int bpix = square ? 128 : (tile == 2 ? 64 : 256);

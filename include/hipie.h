@@ -225,7 +225,9 @@ int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* o
  * with fewer tiles than compute units; needs an even number of 64-byte K steps), 8 / 9 = 128 x 128 /
  * 64 x 256 persistent workgroups that prefetch the next pixel tile during the epilogue (small K; byte
  * outputs with a byte residual or none), 10 / 11 = 128 x 128 / 64 x 256 requesting the operands of two K
- * steps together (whole 128-byte lines per row).  A default is chosen
+ * steps together (whole 128-byte lines per row), 12 = whole output rows of one image x 64 channels per
+ * workgroup with the input patch and the nine weight slices staged once in LDS (3 x 3, stride 1, pad 1,
+ * undilated, input channels a multiple of 64; rows too wide for a patch run variant 0).  A default is chosen
  * from the shape; hipie_compile times the variants on the device and keeps the fastest.  Every
  * variant produces the same bits. */
 int hipie_conv_set_tile(hipie_conv* conv, int tile);

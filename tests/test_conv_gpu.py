@@ -380,3 +380,68 @@ def test_conv_variants_on_ragged_channel_tiles(orc, kind, tile):
         np.testing.assert_array_equal(got.view(np.int8) if got.dtype == np.uint8 else got.astype(np.int8), want)
     else:
         np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+
+_ROW_GEOMS = {
+    "c64_56x56": (2, 64, 56, 56, 64),
+    "c128_28x28_oc128": (3, 128, 28, 28, 128),
+    "ragged_13x19_oc96": (2, 64, 13, 19, 96),
+    "two_tiles_30x9_c192": (1, 192, 30, 9, 64),
+    "one_row_tiles_5x120": (2, 64, 5, 120, 64),
+    "too_wide_3x300": (1, 64, 3, 300, 64),          # no patch fits: the general kernel runs instead
+}
+
+
+@pytest.mark.parametrize("epi", ["i32", "fq", "res_u8"])
+@pytest.mark.parametrize("name", sorted(_ROW_GEOMS))
+def test_conv_row_tile_kernel(orc, name, epi):
+    """tile 12: whole output rows per workgroup, the input patch and the nine weight slices staged once in
+    LDS (3 x 3, stride 1, pad 1): ragged last tiles of an image, several channel tiles, several 64-channel
+    input slices, rows of up to 120 pixels"""
+    import torch
+    from dldt_amd import Convolution, DeviceTensor, HipieError, make_epilogue
+    N, C, H, W, OC = _ROW_GEOMS[name]
+    g = (N, C, H, W, OC, 3, 3, (1, 1), (1, 1), (1, 1), (1, 1))
+    rng = np.random.default_rng(zlib.crc32((name + epi).encode()))
+    x, w = _inputs(rng, g)
+    acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    xin = _device_in(x, g)
+    res = rt = None
+    if epi == "i32":
+        want, e, dt = acc, None, I32
+    else:
+        amax = np.float32(np.abs(acc).max())
+        bias = rng.normal(0, amax / 20, OC).astype(np.float32)
+        ih = rng.uniform(0.3, 1.0, OC).astype(np.float32) * amax
+        dt = U8B
+        if epi == "fq":
+            fq = (256, np.zeros(OC, np.float32), ih, 0.0, 255.0)
+            want = _chain(orc, acc, bias=bias, fq=fq).astype(np.uint8)
+            e = make_epilogue(bias=bias, out_dtype=U8B, fq=fq)
+        else:
+            scale = (rng.uniform(0.5, 2.0, OC) / amax).astype(np.float32)
+            res = rng.integers(0, 256, acc.shape).astype(np.int32)
+            s_x = rng.uniform(0.002, 0.004, OC).astype(np.float32)
+            fq = (256, 0.0, np.float32(1.7), 0.0, 255.0)
+            want = _chain(orc, acc, bias=bias, scale=scale, res=res, res_scale=s_x, fq=fq).astype(np.uint8)
+            e = make_epilogue(bias=bias, scale=scale, residual_dtype=U8B, res_mul=s_x, out_dtype=U8B, fq=fq)
+            rt = DeviceTensor.from_nchw(res, U8B)
+    conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10], e) if e is not None else \
+        Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10])
+    conv.set_tile(12)
+    out = DeviceTensor(N, H, W, OC, dt)
+    conv.run(xin, out, rt)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.to_nchw(), want)
+
+
+def test_row_tile_kernel_refuses_other_geometries():
+    from dldt_amd import Convolution, HipieError
+    for name in ("1x1_c64_oc256", "7x7_s2_p3_c3"):
+        g = GEOMS[name]
+        x, w = _inputs(np.random.default_rng(0), g)
+        conv = Convolution(w.astype(np.int8), _device_in(x, g), g[7], g[8], g[9], g[10])
+        with pytest.raises(HipieError) as e:
+            conv.set_tile(12)
+        assert e.value.status == -4
