@@ -445,3 +445,28 @@ def test_row_tile_kernel_refuses_other_geometries():
         with pytest.raises(HipieError) as e:
             conv.set_tile(12)
         assert e.value.status == -4
+
+
+@pytest.mark.parametrize("stages", [3, 4, 6, 8])
+@pytest.mark.parametrize("tile", [4, 5, 6, 7])
+@pytest.mark.parametrize("name", ["3x3_s1_p1_c64", "1x1_c64_oc256", "3x2_asym_c32_oc200", "3x3_s2_p1_c128"])
+def test_conv_pipelined_ring_depths(orc, name, tile, stages):
+    """every ring depth the pipelined kernels have a loop for (deeper ones than fit the LDS round down),
+    over K loops of 1 to 18 steps: fewer steps than stages, the peeled last step, the drained tail"""
+    import torch
+    from dldt_amd import Convolution, DeviceTensor, HipieError
+    g = GEOMS[name]
+    rng = np.random.default_rng(zlib.crc32(name.encode()) + 7)
+    x, w = _inputs(rng, g)
+    want = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    xin = _device_in(x, g)
+    conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10])
+    try:
+        conv.set_tile(tile, stages)
+    except HipieError as e:       # the split-K variants need an even number of K steps
+        assert 6 <= tile <= 7 and e.status == -4
+        pytest.skip(str(e))
+    out = DeviceTensor(want.shape[0], want.shape[2], want.shape[3], want.shape[1], I32)
+    conv.run(xin, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.to_nchw(), want)
