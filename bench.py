@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""ResNet-50 v1.5 INT8 inference throughput on one MI355X (BASELINE.json metric).
+"""ResNet-50 v1.5 INT8 inference throughput on one MI355X (the headline benchmark).
 
 One step = one batch-64 inference of the post-LPT graph (entry FakeQuantize, 53 fused int8 MFMA
 convolutions + FC, pools, exit), kernels only, inputs resident in HBM.  Like the reference's

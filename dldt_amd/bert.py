@@ -1,4 +1,4 @@
-"""One BERT-base style encoder layer in its post-LPT form (BASELINE config 5), composed on the host
+"""One BERT-base style encoder layer in its post-LPT form (benchmark configuration 5), composed on the host
 from the operator-level C ABI: per-tensor symmetric i8 activations, per-channel i8 weights, int8 MFMA
 GEMMs with fused dequantisation, fp32 softmax / LayerNorm / GELU.
 

@@ -142,7 +142,7 @@ def he_normal(rng, shape):
 
 
 def conv_block(seed=20211, n=1, c=64, hw=56, oc=64, u8_input=False):
-    """BASELINE config 1: FQ(u8) -> Conv 3x3 s1 p1 (per-channel i8 weights) -> bias -> ReLU, f32 out.
+    """benchmark configuration 1: FQ(u8) -> Conv 3x3 s1 p1 (per-channel i8 weights) -> bias -> ReLU, f32 out.
     u8_input: the graph input is a u8 tensor (values 0 .. 255) behind a Convert to f32."""
     rng = np.random.default_rng(seed)
     x = rng.integers(0, 256, (n, c, hw, hw)).astype(np.uint8) if u8_input else \
@@ -220,7 +220,7 @@ def resnet50_fp32(P, x, stages=RESNET50_STAGES, record=None):
 
 
 def resnet50(batch=1, res=224, seed=20211, classes=1000, width=64, stages=RESNET50_STAGES, calib_batch=2):
-    """BASELINE config 3 as a post-LPT graph.  Returns (graph, meta) where meta holds the
+    """benchmark configuration 3 as a post-LPT graph.  Returns (graph, meta) where meta holds the
     parameters, the calibrated ranges and the ids of every quantized activation."""
     P = resnet50_weights(seed, classes, width, stages)
     rng = np.random.default_rng(seed + 1)
@@ -364,7 +364,7 @@ def mobilenet_v2_fp32(P, x, width=1.0, blocks=MOBILENETV2_BLOCKS, last=1280, rec
 
 def mobilenet_v2(batch=1, res=224, seed=20211, classes=1000, width=1.0, blocks=MOBILENETV2_BLOCKS, last=1280,
                  calib_batch=2):
-    """BASELINE config 4 as a post-LPT graph: ReLU6 outputs are u8 [0, max], linear bottleneck
+    """benchmark configuration 4 as a post-LPT graph: ReLU6 outputs are u8 [0, max], linear bottleneck
     outputs symmetric i8; depthwise layers are GroupConvolutions with [G,1,1,3,3] i8 filters."""
     P = mobilenet_v2_weights(seed, classes, width, blocks, last)
     rng = np.random.default_rng(seed + 1)
@@ -423,7 +423,7 @@ BERT_RANGES = dict(x=4.0, q=1.2, k=3.0, v=3.0, p=1.0, ctx=1.0, h1=4.0, g=3.0)
 
 def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, seed=20211, ranges=None, vocab=0,
                  mask=False):
-    """BASELINE config 5: BERT-base style encoder stack in its post-LPT form.  Activations are
+    """benchmark configuration 5: BERT-base style encoder stack in its post-LPT form.  Activations are
     per-tensor symmetric i8 (FakeQuantize ranges of signed_range), weights per-channel i8, Softmax /
     LayerNorm (MVN, Multiply, Add) / Gelu stay f32.
 

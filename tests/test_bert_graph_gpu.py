@@ -1,4 +1,4 @@
-"""BERT-style encoder stack (BASELINE config 5 at reduced width) as a post-LPT graph through the
+"""BERT-style encoder stack (benchmark configuration 5 at reduced width) as a post-LPT graph through the
 planner: MatMul against constant weights and between activations, Reshape / Transpose as views,
 Softmax, LayerNorm, Gelu, per-tensor FakeQuantize.
 

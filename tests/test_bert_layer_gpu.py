@@ -1,4 +1,4 @@
-"""One BERT encoder layer (BASELINE config 5 at reduced width) composed from the C-ABI operators,
+"""One BERT encoder layer (benchmark configuration 5 at reduced width) composed from the C-ABI operators,
 checked segment by segment against the oracle.
 
 The fp32 glue (softmax, LayerNorm, GELU) has tolerance parity only, and a FakeQuantize behind it can

@@ -259,7 +259,7 @@ def test_conv_residual_add_relu_requantize(orc, res_kind):
 
 @pytest.mark.parametrize("act", [None, "relu", "clamp"])
 def test_conv_dequantised_f32_output(orc, act):
-    """Graph tail (BASELINE config 1): Conv' -> +b' -> *s[c] -> ReLU, f32 out; bit-exact floats."""
+    """Graph tail (benchmark configuration 1): Conv' -> +b' -> *s[c] -> ReLU, f32 out; bit-exact floats."""
     from dldt_amd import Convolution, DeviceTensor, make_epilogue
     g = GEOMS["3x3_s1_p1_c64"]
     rng = np.random.default_rng(10)

@@ -6,7 +6,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _per_channel_case(rng, N, C, H, W):
-    """BASELINE config 2 recipe: x ~ N(mu_c, 1), bounds = channel mean -+ 3 sigma."""
+    """benchmark configuration 2 recipe: x ~ N(mu_c, 1), bounds = channel mean -+ 3 sigma."""
     mu = rng.uniform(-0.5, 0.5, C).astype(np.float32)
     x = (rng.standard_normal((N, C, H, W), dtype=np.float32) + mu.reshape(1, C, 1, 1)).astype(np.float32)
     m = x.mean(axis=(0, 2, 3), dtype=np.float64)
@@ -89,7 +89,7 @@ def test_fq_empty_input():
 
 
 def test_fq_full_size_properties(orc):
-    """BASELINE config 2 at full size [32,256,56,56]: a seeded sample of planes is compared with
+    """benchmark configuration 2 at full size [32,256,56,56]: a seeded sample of planes is compared with
     the oracle; the whole tensor is checked through size-independent properties."""
     import torch
     from dldt_amd import FakeQuantize

@@ -8,7 +8,7 @@ pytestmark = pytest.mark.gpu
 
 
 def test_conv_block_config1(orc):
-    """BASELINE config 1: [1,64,56,56] -> FQ u8 -> 3x3 conv (i8 per-channel W) -> bias -> ReLU."""
+    """benchmark configuration 1: [1,64,56,56] -> FQ u8 -> 3x3 conv (i8 per-channel W) -> bias -> ReLU."""
     from dldt_amd import builders
     g, feeds, _ = builders.conv_block()
     want, _ = evaluate(orc, g.nodes, feeds)

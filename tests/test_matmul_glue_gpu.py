@@ -1,4 +1,4 @@
-"""MatMul on int8 MFMA (constant weights and activation x activation, BASELINE config 5 shapes) and
+"""MatMul on int8 MFMA (constant weights and activation x activation, benchmark configuration 5 shapes) and
 the fp32 glue (softmax, MVN/LayerNorm, GELU) through the C ABI vs the oracle."""
 import numpy as np
 import pytest
