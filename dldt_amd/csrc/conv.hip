@@ -66,15 +66,14 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     // one implicit GEMM over an operand set (activation tensor, packed weights, K-offset table)
     auto gemm = [&](const int8_t* in_base, int in_sn, int in_sh, int in_sw, int csh, int csw, int origin,
                     const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk,
-                    v16i (&acc)[2][2], bool first, bool acc_from_lds) {
+                    v16i (&acc)[2][2], bool first, bool acc_from_lds, bool flat) {
         int32_t b_base[B_PIECES];
         uint32_t a_off[A_PIECES];                          // unsigned: added to the uniform base by the load itself
 #pragma unroll
         for (int i = 0; i < B_PIECES; ++i) {
             int m = pix0 + ((tid + i * NT) >> 2);
             m = m < a.M ? m : a.M - 1;
-            const PixelCoord p = decode_pixel(a, m);
-            b_base[i] = p.n * in_sn + p.oh * csh * in_sh + p.ow * csw * in_sw + origin;
+            b_base[i] = window_offset(a, m, in_sn, in_sh, in_sw, csh, csw, flat) + origin;
         }
 #pragma unroll
         for (int i = 0; i < A_PIECES; ++i) {
@@ -114,8 +113,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
             for (int i = 0; i < B_P2; ++i) {
                 int m = pix0 + row0 + i * RPI;
                 m = m < a.M ? m : a.M - 1;
-                const PixelCoord p = decode_pixel(a, m);
-                b_base2[i] = p.n * in_sn + p.oh * csh * in_sh + p.ow * csw * in_sw + origin;
+                b_base2[i] = window_offset(a, m, in_sn, in_sh, in_sw, csh, csw, flat) + origin;
             }
 #pragma unroll
             for (int i = 0; i < A_P2; ++i) {
@@ -220,7 +218,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
         a2.corr = a.corr2;
         init_acc(a2, oc_lane, acc);
         gemm(a.in2, a.in2_sn, a.in2_sh, a.in2_sw, a.conv2_sh, a.conv2_sw, a.in2_origin, a.wgt2, a.Kp2, a.OCp, false,
-             a.koff2, a.nk2, acc, true, false);
+             a.koff2, a.nk2, acc, true, false, false);
 #pragma unroll
         for (int ob = 0; ob < 2; ++ob)
 #pragma unroll
@@ -239,7 +237,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     }
     if (kFused) init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);   // published by the shortcut GEMM's first barrier
     gemm(a.in + batch_offset(a, batch, a.batch_in, a.batch_in_o), a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
-         a.wgt + batch_offset(a, batch, a.batch_wgt, a.batch_wgt_o), a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused);
+         a.wgt + batch_offset(a, batch, a.batch_wgt, a.batch_wgt_o), a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused, a.flat_in != 0);
     const int m0 = pix0 + wpix * 64 + l32;
     // the K loop ends with a barrier, so the operand tiles are free: every wave takes 8 KB of them as
     // the staging buffer of its f32 stores (2 (BOC + BPIX) 64 bytes cover 8 KB per wave for all shapes)
@@ -304,8 +302,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const C
         for (int i = 0; i < B_PIECES; ++i) {
             int m = pix0 + ((tid + i * NT) >> 2);
             m = m < a.M ? m : a.M - 1;
-            const PixelCoord p = decode_pixel(a, m);
-            b_base[i] = p.n * a.in_sn + p.oh * a.conv_sh * a.in_sh + p.ow * a.conv_sw * a.in_sw + a.in_origin;
+            b_base[i] = window_offset(a, m, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.flat_in != 0) + a.in_origin;
         }
     };
     v4i ga[A_PIECES], gb[B_PIECES];
@@ -453,7 +450,7 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
 
     auto gemm = [&](const int8_t* in_base, int in_sn, int in_sh, int in_sw, int csh, int csw, int origin,
                     const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk_all,
-                    v16i (&acc)[2][2]) {
+                    v16i (&acc)[2][2], bool flat) {
         const int nk = nk_all / KS;   // steps of this wave group: local step j is global step j * KS + grp
         const int8_t* a_ptr[A_GROUPS];
         int32_t b_base[B_GROUPS];
@@ -471,8 +468,7 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
         for (int i = 0; i < B_GROUPS; ++i) {
             int m = pix0 + (wave * B_GROUPS + i) * 16 + dma_row;
             m = m < a.M ? m : a.M - 1;
-            const PixelCoord p = decode_pixel(a, m);
-            b_base[i] = p.n * in_sn + p.oh * csh * in_sh + p.ow * csw * in_sw + origin;
+            b_base[i] = window_offset(a, m, in_sn, in_sh, in_sw, csh, csw, flat) + origin;
         }
         // The K-offset table lives in LDS behind the ring: a vector-memory load of it would have to
         // be awaited with vmcnt(0), which drains every DMA load in flight and serialises the ring.
@@ -573,7 +569,7 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
         a2.corr = a.corr2;
         init_acc(a2, oc_lane, acc);
         gemm(a.in2, a.in2_sn, a.in2_sh, a.in2_sw, a.conv2_sh, a.conv2_sw, a.in2_origin, a.wgt2, a.Kp2, a.OCp, false,
-             a.koff2, a.nk2, acc);
+             a.koff2, a.nk2, acc, false);
 #pragma unroll
         for (int ob = 0; ob < 2; ++ob)
 #pragma unroll
@@ -601,7 +597,7 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
                 for (int r = 0; r < 16; ++r) acc[ob][pb][r] = 0;
     }
     gemm(a.in + batch * a.batch_in, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
-         a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc);
+         a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, a.flat_in != 0);
     if (KS == 2) {
         // partial sums of group 1 -> LDS (register r of thread t at dword r * NT + t), added by group 0
         int32_t* red = reinterpret_cast<int32_t*>(ring);
@@ -777,8 +773,7 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
         for (int pb = 0; pb < 2; ++pb) {
             int m = t * 256 + wave * 64 + pb * 32 + l32;
             m = m < a.M ? m : a.M - 1;
-            const PixelCoord p = decode_pixel(a, m);
-            b[pb] = p.n * a.in_sn + p.oh * a.conv_sh * a.in_sh + p.ow * a.conv_sw * a.in_sw + a.in_origin;
+            b[pb] = window_offset(a, m, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.flat_in != 0) + a.in_origin;
         }
     };
     auto load_b = [&](const int32_t (&b)[2], int k, v4i (&f)[2][2]) {
@@ -1573,6 +1568,12 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         a.out_sn = static_cast<int32_t>(out->stride_n);
         a.out_sh = static_cast<int32_t>(out->stride_h);
         a.out_sw = static_cast<int32_t>(out->stride_w);
+        // tensors that are dense in (n, h, w) for this convolution: pixel m sits at m * pixel stride
+        a.flat_in = static_cast<int64_t>(d.stride_h) * a.in_sh == static_cast<int64_t>(ow) * d.stride_w * a.in_sw &&
+                    a.in_sn == static_cast<int64_t>(oh) * ow * d.stride_w * a.in_sw;
+        a.flat_out = a.out_sh == static_cast<int64_t>(ow) * a.out_sw && a.out_sn == static_cast<int64_t>(oh) * ow * a.out_sw;
+        a.flat_res = a.res != nullptr && a.res_sh == static_cast<int64_t>(ow) * a.res_sw &&
+                     a.res_sn == static_cast<int64_t>(oh) * ow * a.res_sw;
         a.OC = d.oc;
         a.OCp = static_cast<int32_t>(c->OCp);
         a.Kp = static_cast<int32_t>(c->Kp);

@@ -51,6 +51,14 @@ __device__ __forceinline__ PixelCoord decode_pixel(const ConvArgs& a, int m) {
     return p;
 }
 
+// offset of output pixel m's window origin (padding not counted) in a tensor with strides sn, sh, sw under
+// convolution strides csh, csw; `flat`: the offset is linear in m (uniform flag computed on the host)
+__device__ __forceinline__ int window_offset(const ConvArgs& a, int m, int sn, int sh, int sw, int csh, int csw, bool flat) {
+    if (flat) return m * (csw * sw);
+    const PixelCoord p = decode_pixel(a, m);
+    return p.n * sn + p.oh * csh * sh + p.ow * csw * sw;
+}
+
 __device__ __forceinline__ float4 ld4f(const float* p) { return *reinterpret_cast<const float4*>(p); }
 
 // Accumulators start from the per-channel integer correction, so the epilogue begins with the
@@ -575,7 +583,13 @@ __device__ __forceinline__ void epilogue_addresses(const ConvArgs& a, int oc_lan
 #pragma unroll
     for (int pb = 0; pb < 2; ++pb) {
         e.valid[pb] = m[pb] < a.M;
-        const PixelCoord p = decode_pixel(a, e.valid[pb] ? m[pb] : a.M - 1);
+        const int mm = e.valid[pb] ? m[pb] : a.M - 1;
+        if (a.flat_out && (a.flat_res || !a.res)) {   // uniform: dense tensors, no decode
+            e.out_off[pb] = batch_offset(a, batch, a.batch_out, a.batch_out_o) + static_cast<int64_t>(mm) * a.out_sw + oc_lane;
+            e.res_off[pb] = batch * a.batch_res + static_cast<int64_t>(mm) * a.res_sw + oc_lane;
+            continue;
+        }
+        const PixelCoord p = decode_pixel(a, mm);
         e.out_off[pb] = batch_offset(a, batch, a.batch_out, a.batch_out_o) + static_cast<int64_t>(p.n) * a.out_sn + p.oh * a.out_sh +
                         p.ow * a.out_sw + oc_lane;
         e.res_off[pb] = batch * a.batch_res + static_cast<int64_t>(p.n) * a.res_sn + p.oh * a.res_sh +
