@@ -741,6 +741,105 @@ __global__ __launch_bounds__(256, 2) void conv_rows_kernel(const ConvArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// First-layer kernel: few input channels (pixel = 4 bytes), one 32-byte K slice per filter row (the
+// packing of such layers: kw * 4 <= 32 bytes of taps, zero-padded).  As an implicit GEMM the 7 x 7
+// stride-2 stem fetches every input byte about twelve times; here a workgroup takes R whole output rows
+// of one image x 64 channels, stages the input patch ((R - 1) stride + kh rows, 8 KB) and the weights
+// (64 x kh x 32 bytes) once, and a lane's B fragment of filter row kh is the 32 contiguous patch bytes
+// that start at its pixel's window (8-byte aligned: two ds_read_b64).  Bytes of the slice behind the
+// last tap meet zero weights.  Weight rows are 240 bytes apart in LDS (16 x 15: conflict-free b128 reads).
+constexpr int kStemPatch = 12288, kStemWRow = 240, kStemLds = 36864;
+template <uint32_t F>
+__global__ __launch_bounds__(256, 2) void conv_stem_kernel(const ConvArgs a) {
+    __shared__ __attribute__((aligned(16))) int8_t lds[kStemLds];          // patch | weights; later 4 x 8 KB of staging
+    __shared__ __attribute__((aligned(16))) float sP[PT_ROWS * 64];
+    int8_t* const sPatch = lds;
+    int8_t* const sW = lds + kStemPatch;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, h = lane >> 5;
+    int p_tile, t_tile;
+    split_tile_index(a, blockIdx.x, p_tile, t_tile);
+    const int oc0 = t_tile * 64;
+    const int n = p_tile / a.tiles_per_image, ty = p_tile - n * a.tiles_per_image;
+    const int R = a.rows_per_tile, y0 = ty * R;
+    const int count = R * a.OW, pix0 = n * a.OHOW + y0 * a.OW;
+    const int PWb = a.patch_w * 4;                                          // patch row in bytes
+    const int oc_lane = oc0 + 32 * h;
+    stage_params<F>(a, oc0, (lds_float_ptr)sP, 64, tid, 256);
+
+    // patch: input rows y0 * stride - pad_top .., columns -pad_left ..; dword by dword (rows start 4-byte aligned)
+    const int8_t* in0 = a.in + (static_cast<int64_t>(n) * a.in_sn + (y0 * a.conv_sh - a.stem_pad_top) * a.in_sh - a.stem_pad_left * 4);
+    const int row_dw = a.patch_w, total_dw = a.stem_patch_rows * row_dw;
+    constexpr int PD = kStemPatch / 4 / 256;                                // dwords per thread, at most
+    uint32_t pv[PD];
+#pragma unroll
+    for (int j = 0; j < PD; ++j) {
+        const int i = min(tid + j * 256, total_dw - 1);
+        int py, px;
+        fast_divmod(i, row_dw, a.inv_patch_w, py, px);
+        pv[j] = *reinterpret_cast<const uint32_t*>(in0 + (py * a.in_sh + px * 4));
+    }
+    // weights: the packed rows' kh * 32 bytes, 16 bytes at a time
+    const int w_pieces = 64 * a.stem_kh * 2;
+    const int8_t* w0 = a.wgt + static_cast<int64_t>(oc0) * a.wgt_ld;
+    v4i wv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int i = min(tid + j * 256, w_pieces - 1);
+        const int row = i / (a.stem_kh * 2), pc = i - row * (a.stem_kh * 2);
+        wv[j] = *reinterpret_cast<const v4i*>(w0 + (static_cast<int64_t>(row) * a.wgt_ld + pc * 16));
+    }
+#pragma unroll
+    for (int j = 0; j < PD; ++j) {
+        const int i = tid + j * 256;
+        if (i < total_dw) *reinterpret_cast<uint32_t*>(&sPatch[i * 4]) = pv[j];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int i = tid + j * 256;
+        const int row = i / (a.stem_kh * 2), pc = i - row * (a.stem_kh * 2);
+        if (i < w_pieces) *reinterpret_cast<v4i*>(&sW[row * kStemWRow + pc * 16]) = wv[j];
+    }
+    // window start of the lane's two pixels in the patch (bytes), filter row 0
+    int b0[2];
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+        const int p = min(wave * 64 + pb * 32 + l32, count - 1);
+        int r, x;
+        fast_divmod(p, a.OW, a.inv_OW, r, x);
+        b0[pb] = r * a.conv_sh * PWb + x * a.conv_sw * 4 + 16 * h;
+    }
+    v16i acc[2][2];
+    v16f rres[2][2];
+    init_acc(a, oc_lane, acc);
+    __syncthreads();
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    for (int kh = 0; kh < a.stem_kh; ++kh) {
+        v4i af[2], bf[2];
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob) af[ob] = *reinterpret_cast<const v4i*>(&sW[(ob * 32 + l32) * kStemWRow + kh * 32 + 16 * h]);
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb) {
+            const int8_t* q = &sPatch[b0[pb] + kh * PWb];
+            const v2i lo = *reinterpret_cast<const v2i*>(q), hi = *reinterpret_cast<const v2i*>(q + 8);
+            bf[pb].x = lo.x; bf[pb].y = lo.y; bf[pb].z = hi.x; bf[pb].w = hi.y;
+        }
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+                acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ob], bf[pb], acc[ob][pb], 0, 0, 0);
+    }
+    __syncthreads();                                                       // patch and weights become the stores' staging space
+    ConvArgs e = a;
+    e.M = min(a.M, pix0 + count);
+    const int m0 = pix0 + wave * 64 + l32;
+    run_epilogue<F>(e, acc, oc_lane, m0, m0 + 32, 0, rres, (lds_cfloat_ptr)sP, 64, oc0, (lds_float_ptr)lds + wave * 2048);
+}
+
+// ------------------------------------------------------------------------------------------------
 // Streaming kernel: grid (x, channel tiles of 64); a workgroup of 4 waves walks pixel tiles of 256
 // (64 per wave) with stride gridDim.x.  Dynamic LDS: 64 rows of (Kp + 16) weight bytes.
 template <uint32_t F>
@@ -908,6 +1007,24 @@ bool rows_kernel_fits(const hipie_conv_desc& d) {
 int rows_per_tile(int oh, int ow) {
     const int r = std::min(std::min(256 / ow, kPatchRows / (ow + 2) - 2), oh);
     return r >= 1 ? r : 0;
+}
+
+// the first-layer kernel's geometry: 4-byte pixels, one 32-byte slice per filter row, undilated
+bool stem_kernel_fits(const hipie_conv_desc& d) {
+    return d.groups == 1 && d.in_c_stride == 4 && d.in_stride_w == 4 && d.dil_h == 1 && d.dil_w == 1 && d.kw * 4 > 16 && d.kw * 4 <= 32 &&
+           d.kh <= 8 && (d.stride_w * 4) % 8 == 0;
+}
+
+void launch_stem(const ConvArgs& a, hipStream_t s) {
+    const dim3 grid(a.p_tiles * a.t_tiles), block(256);
+    const uint32_t core = a.flags & ~CF_OUT_XOR;
+#define HIPIE_LAUNCH_STEM(FLAGS, ...)                                                    \
+    do {                                                                                 \
+        if constexpr ((FLAGS) != kDyn && ((FLAGS) & CF_RES_GEMM)) break;                  \
+        else hipLaunchKernelGGL((conv_stem_kernel<FLAGS>), grid, block, 0, s, a);        \
+    } while (0)
+    HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_STEM, 0)
+#undef HIPIE_LAUNCH_STEM
 }
 
 void launch_rows(const ConvArgs& a, hipStream_t s) {
@@ -1414,13 +1531,15 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 12, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 13, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
         if (c->depthwise) return;               // one kernel only
         if (c->fused && tile != 0) return;      // the second GEMM exists in the 128 x 128 tiled kernel
         HIPIE_REQUIRE(tile < 8 || tile > 9 || (!c->fused && persist_available(c->epi.flags)), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the persistent kernels exist for byte outputs with a byte residual or none");
         HIPIE_REQUIRE(tile < 6 || tile > 7 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the split-K kernels need an even number of 64-byte K steps (K=%lld)", (long long)c->Kp);
+        HIPIE_REQUIRE(tile != 13 || stem_kernel_fits(c->d), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_set_tile: the first-layer kernel takes 4-byte pixels and filter rows of 5 to 8 taps, undilated");
         HIPIE_REQUIRE(tile != 12 || rows_kernel_fits(c->d), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the row-tile kernel takes 3 x 3, stride 1, pad 1, undilated convolutions over a multiple of 64 input channels");
         HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) + PT_ROWS * 64 * 4 <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
@@ -1590,6 +1709,36 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
             return;
         }
         int tile = c->tile;
+        if (tile == 13) {
+            // R whole output rows per tile (R divides OH): at most 256 pixels, the patch within its LDS buffer,
+            // and every byte the patch reads inside the tensor's halo
+            const int patch_w = (ow - 1) * d.stride_w + 8;
+            int R = 0;
+            for (int r = std::min(oh, 256 / std::max(ow, 1)); r >= 1 && R == 0; --r)
+                if (oh % r == 0 && ((r - 1) * d.stride_h + d.kh) * patch_w * 4 + 16 <= kStemPatch) R = r;
+            const bool inside = in->halo >= d.pad_top && in->halo >= d.pad_left &&
+                                (oh - 1) * d.stride_h - d.pad_top + d.kh - 1 <= in->h - 1 + in->halo &&
+                                (ow - 1) * d.stride_w - d.pad_left + 7 <= in->w - 1 + in->halo;
+            if (R == 0 || !inside || ow > 256) {
+                tile = 1;                     // the general kernel
+            } else {
+                a.rows_per_tile = R;
+                a.tiles_per_image = oh / R;
+                a.patch_w = patch_w;
+                a.inv_patch_w = 1.0f / static_cast<float>(patch_w);
+                a.stem_kh = d.kh;
+                a.stem_patch_rows = (R - 1) * d.stride_h + d.kh;
+                a.stem_pad_top = d.pad_top;
+                a.stem_pad_left = d.pad_left;
+                a.p_tiles = in->n * a.tiles_per_image;
+                a.t_tiles = static_cast<int32_t>(ceil_div(d.oc, 64));
+                a.t_shift = (a.t_tiles & (a.t_tiles - 1)) == 0 ? __builtin_ctz(a.t_tiles) : -1;
+                DeviceGuard g(c->device);
+                launch_stem(a, as_stream(stream));
+                HIPIE_CHECK_HIP(hipGetLastError());
+                return;
+            }
+        }
         if (tile == 12) {
             const int R = rows_per_tile(oh, ow);
             if (R == 0 || in->halo < 1) {

@@ -106,6 +106,8 @@ struct ConvArgs {
     // row-tile kernel (3 x 3, stride 1): output rows per tile, tiles per image, patch width OW + 2 and its reciprocal
     int32_t rows_per_tile, tiles_per_image, patch_w;
     float inv_patch_w;
+    // first-layer kernel (few channels, one 32-byte K slice per filter row): filter rows, patch rows, padding
+    int32_t stem_kh, stem_patch_rows, stem_pad_top, stem_pad_left;
 };
 
 }  // namespace hipie

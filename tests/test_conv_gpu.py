@@ -470,3 +470,45 @@ def test_conv_pipelined_ring_depths(orc, name, tile, stages):
     conv.run(xin, out)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(out.to_nchw(), want)
+
+
+_STEM_GEOMS = {
+    # (N, C, H, W, OC, KH, KW, strides, pads)
+    "resnet_stem_32": (2, 3, 32, 32, 64, 7, 7, (2, 2), (3, 3)),
+    "resnet_stem_rows_of_112": (1, 3, 20, 224, 64, 7, 7, (2, 2), (3, 3)),      # two output rows per tile
+    "odd_rows_oc96": (2, 3, 26, 38, 96, 7, 7, (2, 2), (3, 3)),                  # 13 output rows: one tile per image; 1.5 channel tiles
+    "6x6_s2_c4": (1, 4, 30, 22, 64, 6, 6, (2, 2), (2, 2)),
+    "5x8_s4x2_c2": (2, 2, 33, 40, 32, 5, 8, (4, 2), (2, 3)),
+}
+
+
+@pytest.mark.parametrize("extra_halo", [4, 0])
+@pytest.mark.parametrize("epi", ["i32", "fq"])
+@pytest.mark.parametrize("name", sorted(_STEM_GEOMS))
+def test_conv_first_layer_kernel(orc, name, epi, extra_halo):
+    """tile 13: 4-byte pixels, whole output rows per workgroup, patch and weights staged once, one 32-byte
+    K slice per filter row whose surplus bytes meet zero weights; with no more halo than the padding needs,
+    a patch that would overhang it makes the general kernel run instead"""
+    import torch
+    from dldt_amd import Convolution, DeviceTensor, make_epilogue
+    N, C, H, W, OC, KH, KW, st, pad = _STEM_GEOMS[name]
+    g = (N, C, H, W, OC, KH, KW, st, (1, 1), pad, pad)
+    rng = np.random.default_rng(zlib.crc32((name + epi).encode()))
+    x, w = _inputs(rng, g)
+    acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    from dldt_amd import DeviceTensor as DT
+    xin = DT.from_nchw(x, U8B, halo=max(pad) + extra_halo, c_stride=4)
+    if epi == "i32":
+        want, conv, dt = acc, Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10]), I32
+    else:
+        amax = np.float32(np.abs(acc).max())
+        bias = rng.normal(0, amax / 20, OC).astype(np.float32)
+        ih = rng.uniform(0.3, 1.0, OC).astype(np.float32) * amax
+        fq = (256, np.zeros(OC, np.float32), ih, 0.0, 255.0)
+        want = _chain(orc, acc, bias=bias, fq=fq).astype(np.uint8)
+        conv, dt = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10], make_epilogue(bias=bias, out_dtype=U8B, fq=fq)), U8B
+    conv.set_tile(13)
+    out = DeviceTensor(acc.shape[0], acc.shape[2], acc.shape[3], OC, dt)
+    conv.run(xin, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.to_nchw(), want)
