@@ -4,7 +4,9 @@
 #include "conv_epilogue.h"
 
 #include <cmath>
+#include <map>
 #include <memory>
+#include <mutex>
 
 namespace hipie {
 
@@ -586,7 +588,11 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
                     }
             }
     }
-    if (grp == 0) {
+    // K split over workgroups: part z of S multiplies the K steps [nk z / S, nk (z + 1) / S)
+    const int S = KS == 1 ? a.ksplit : 1, z = S > 1 ? static_cast<int>(blockIdx.z) : 0;
+    const int k_first = S > 1 ? (a.nk * z) / S : 0;
+    const int nk_part = S > 1 ? (a.nk * (z + 1)) / S - k_first : a.nk;
+    if (grp == 0 && z == 0) {
         init_acc(a, oc_lane, acc);
     } else {
 #pragma unroll
@@ -597,7 +603,48 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
                 for (int r = 0; r < 16; ++r) acc[ob][pb][r] = 0;
     }
     gemm(a.in + batch * a.batch_in, a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
-         a.wgt + batch * a.batch_wgt, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, a.flat_in != 0);
+         a.wgt + batch * a.batch_wgt + k_first * 64, a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff + 4 * k_first, nk_part, acc,
+         a.flat_in != 0);
+    if (KS == 1 && S > 1) {
+        // Every part stores its accumulators (register r of thread t at dword r * NT + t: whole cache lines per
+        // wave) and takes a ticket; the workgroup that draws the last ticket of its tile adds the other parts to
+        // its own registers and runs the epilogue, the others are done.  Integer sums do not depend on the order.
+        // No workgroup waits for another.  The partial sums cross between compute dies, whose L2 caches are not
+        // coherent with each other: they are written and read with device-scope accesses (which go through to
+        // memory) instead of fences, because a device-scope fence writes back or invalidates a die's whole L2
+        // and costs more than the split saves.
+        const int tile_id = t_tile * a.p_tiles + p_tile;
+        int32_t* const parts = a.ws_part + static_cast<int64_t>(tile_id) * S * (64 * NT);
+        int32_t* const mine = parts + z * (64 * NT) + tid;
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    __hip_atomic_store(&mine[((ob * 2 + pb) * 16 + r) * NT], acc[ob][pb][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));                            // the stores have reached device-wide memory
+        __syncthreads();
+        uint32_t* const ticket = reinterpret_cast<uint32_t*>(ring);          // the ring is no longer read
+        if (tid == 0) {
+            const uint32_t t = atomicAdd(a.ws_count + tile_id, 1u);
+            if (t == static_cast<uint32_t>(S - 1)) atomicExch(a.ws_count + tile_id, 0u);   // zero again for the next launch
+            *ticket = t;
+        }
+        __syncthreads();
+        if (*ticket != static_cast<uint32_t>(S - 1)) return;
+        for (int zz = 0; zz < S; ++zz) {
+            if (zz == z) continue;
+            const int32_t* const other = parts + zz * (64 * NT) + tid;
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[ob][pb][r] += __hip_atomic_load(&other[((ob * 2 + pb) * 16 + r) * NT], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
     if (KS == 2) {
         // partial sums of group 1 -> LDS (register r of thread t at dword r * NT + t), added by group 0
         int32_t* red = reinterpret_cast<int32_t*>(ring);
@@ -977,7 +1024,8 @@ void launch_tiled(const ConvArgs& a, hipStream_t s, int batches = 1) {
 
 template <int WOC, int WPIX, int KS>
 void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) {
-    const dim3 grid(a.p_per_xcd > 0 ? 8 * a.p_per_xcd * a.t_tiles : a.p_tiles * a.t_tiles, batches), block(WOC * WPIX * 64 * KS);
+    const dim3 grid(a.p_per_xcd > 0 ? 8 * a.p_per_xcd * a.t_tiles : a.p_tiles * a.t_tiles, batches, a.ksplit > 1 ? a.ksplit : 1),
+        block(WOC * WPIX * 64 * KS);
     const size_t lds = static_cast<size_t>(KS) * stages * (WOC + WPIX) * 64 * 64 + PT_ROWS * WOC * 64 * 4 +
                        16 * static_cast<size_t>(std::max(a.nk, a.nk2));
     const uint32_t core = a.flags & ~CF_OUT_XOR;
@@ -997,6 +1045,40 @@ void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) 
     HIPIE_FOR_EACH_EPILOGUE(HIPIE_LAUNCH_PIPE, 0)
 #undef HIPIE_LAUNCH_PIPE
 }
+
+// Workspace of the kernels that split K over workgroups: partial accumulators and arrival counters, one
+// per (device, stream).  Launches on one stream run one after another, so they can share it; launches on
+// different streams (several requests in flight) get their own.  It is created, or replaced by a larger
+// one after the stream has drained, on the first launch that needs it; the counters start at zero and every
+// launch leaves them at zero.  Kept until the process ends.
+struct SplitWorkspace {
+    DeviceBuffer part, count;
+    size_t tiles = 0;
+};
+SplitWorkspace& split_workspace(int device, hipStream_t s, size_t part_bytes, size_t tiles) {
+    static std::mutex mu;
+    static auto* pool = new std::map<std::pair<int, hipStream_t>, SplitWorkspace>();
+    std::lock_guard<std::mutex> lock(mu);
+    SplitWorkspace& w = (*pool)[std::make_pair(device, s)];
+    if (w.part.bytes < part_bytes || w.tiles < tiles) {
+        DeviceGuard g(device);
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        HIPIE_CHECK_HIP(hipStreamIsCapturing(s, &capturing));
+        HIPIE_REQUIRE(capturing == hipStreamCaptureStatusNone, HIPIE_NOT_ALLOCATED,
+                      "the split-K workspace of this stream is created by the first launch: run once before capturing");
+        HIPIE_CHECK_HIP(hipStreamSynchronize(s));
+        if (w.part.bytes < part_bytes) w.part.alloc(device, part_bytes);
+        if (w.tiles < tiles) {
+            w.count.alloc(device, tiles * sizeof(uint32_t));
+            HIPIE_CHECK_HIP(hipMemset(w.count.ptr, 0, tiles * sizeof(uint32_t)));
+            w.tiles = tiles;
+        }
+    }
+    return w;
+}
+
+// parts of the K split of variants 14 to 17: 2, 4, 8, 16
+int split_parts(int tile) { return 2 << (tile - 14); }
 
 bool rows_kernel_fits(const hipie_conv_desc& d) {
     return d.groups == 1 && d.kh == 3 && d.kw == 3 && d.stride_h == 1 && d.stride_w == 1 && d.dil_h == 1 && d.dil_w == 1 &&
@@ -1531,13 +1613,15 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 13, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 17, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
         if (c->depthwise) return;               // one kernel only
         if (c->fused && tile != 0) return;      // the second GEMM exists in the 128 x 128 tiled kernel
         HIPIE_REQUIRE(tile < 8 || tile > 9 || (!c->fused && persist_available(c->epi.flags)), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the persistent kernels exist for byte outputs with a byte residual or none");
         HIPIE_REQUIRE(tile < 6 || tile > 7 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the split-K kernels need an even number of 64-byte K steps (K=%lld)", (long long)c->Kp);
+        HIPIE_REQUIRE(tile < 14 || c->Kp / 64 >= 2 * split_parts(tile), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_set_tile: the K split over workgroups needs two 64-byte K steps per part (K=%lld)", (long long)c->Kp);
         HIPIE_REQUIRE(tile != 13 || stem_kernel_fits(c->d), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the first-layer kernel takes 4-byte pixels and filter rows of 5 to 8 taps, undilated");
         HIPIE_REQUIRE(tile != 12 || rows_kernel_fits(c->d), HIPIE_PARAMETER_MISMATCH,
@@ -1757,7 +1841,7 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
                 return;
             }
         }
-        const bool square = tile == 0 || tile == 4 || tile == 6 || tile == 8 || tile == 10;
+        const bool square = tile == 0 || tile == 4 || tile == 6 || tile == 8 || tile == 10 || tile >= 14;
         const int boc = square ? 128 : 64;
         const int bpix = square ? 128 : (tile == 2 ? 64 : 256);
         a.p_tiles = static_cast<int32_t>(ceil_div(M, bpix));
@@ -1770,12 +1854,26 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         DeviceGuard g(c->device);
         hipStream_t s = as_stream(stream);
         // ring depth: enough K steps in flight to cover the load latency, within 160 KB of LDS
-        const int stage_bytes = (square ? 256 : 320) * 64 * (tile >= 6 ? 2 : 1);
+        const int stage_bytes = (square ? 256 : 320) * 64 * (tile == 6 || tile == 7 ? 2 : 1);
         // ring depth: 3, 4, 6 or 8 K steps (the depths the kernel has loops for), within 160 KB of LDS
         const int max_stages = (144 * 1024) / stage_bytes;
-        int stages = c->stages > 0 ? c->stages : (tile == 4 ? 4 : 3);
+        int stages = c->stages > 0 ? c->stages : (tile == 4 || tile >= 14 ? 4 : 3);
         stages = stages >= 8 && max_stages >= 8 ? 8 : (stages >= 6 && max_stages >= 6 ? 6 : (stages >= 4 && max_stages >= 4 ? 4 : 3));
+        // the K split pays where a launch has fewer tiles than the device has compute units; with many tiles
+        // (more than 2048 workgroups, a 128 MB workspace) the plain pipelined kernel runs instead
+        if (tile >= 14 && static_cast<int64_t>(a.p_tiles) * a.t_tiles * split_parts(tile) > 2048) tile = 4;
+        if (tile >= 14) {
+            a.ksplit = split_parts(tile);
+            const size_t tiles = static_cast<size_t>(a.p_tiles) * a.t_tiles;
+            SplitWorkspace& w = split_workspace(c->device, s, tiles * a.ksplit * 64 * 256 * sizeof(int32_t), tiles);
+            a.ws_part = w.part.as<int32_t>();
+            a.ws_count = w.count.as<uint32_t>();
+        }
         switch (tile) {
+        case 14:
+        case 15:
+        case 16:
+        case 17:
         case 4: launch_pipe<2, 2, 1>(a, stages, s); break;
         case 5: launch_pipe<1, 4, 1>(a, stages, s); break;
         case 8: launch_persist<2, 2>(a, s); break;

@@ -108,6 +108,11 @@ struct ConvArgs {
     float inv_patch_w;
     // first-layer kernel (few channels, one 32-byte K slice per filter row): filter rows, patch rows, padding
     int32_t stem_kh, stem_patch_rows, stem_pad_top, stem_pad_left;
+    // K split over workgroups (pipelined kernel, grid.z = ksplit): partial accumulators of tile i, part z at
+    // ws_part + (i * ksplit + z) * 64 * threads dwords, arrival counter of tile i at ws_count[i] (zero between launches)
+    int32_t ksplit;
+    int32_t* ws_part;
+    uint32_t* ws_count;
 };
 
 }  // namespace hipie

@@ -273,7 +273,7 @@ struct ConvStep : Step {
         }
         int best = current;
         float best_ms = 0.f;
-        const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13};
+        const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17};
         for (size_t c = 0; c < sizeof(candidates) / sizeof(candidates[0]); ++c) {
             const int tile = candidates[c];
             if (c > 0 && tile == current) continue;

@@ -227,7 +227,13 @@ int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* o
  * outputs with a byte residual or none), 10 / 11 = 128 x 128 / 64 x 256 requesting the operands of two K
  * steps together (whole 128-byte lines per row), 12 = whole output rows of one image x 64 channels per
  * workgroup with the input patch and the nine weight slices staged once in LDS (3 x 3, stride 1, pad 1,
- * undilated, input channels a multiple of 64; rows too wide for a patch run variant 0).  A default is chosen
+ * undilated, input channels a multiple of 64; rows too wide for a patch run variant 0), 13 = the same idea for
+ * a first layer (4-byte pixels, filter rows of 5 to 8 taps, undilated: one 32-byte K slice per filter row; a
+ * patch that would overhang the tensor's halo runs variant 1), 14 to 17 = variant 4 with the K steps of a tile
+ * split over 2 / 4 / 8 / 16 workgroups (for launches with fewer tiles than compute units; at least two K steps per
+ * part; launches of more than 2048 workgroups run variant 4).  The partial sums of variants 14 to 17 pass through a
+ * workspace that the library keeps per (device, stream): it is allocated by the first such launch on a stream
+ * (which therefore must not be under graph capture) and kept until the process ends.  A default is chosen
  * from the shape; hipie_compile times the variants on the device and keeps the fastest.  Every
  * variant produces the same bits. */
 int hipie_conv_set_tile(hipie_conv* conv, int tile);

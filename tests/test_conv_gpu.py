@@ -512,3 +512,97 @@ def test_conv_first_layer_kernel(orc, name, epi, extra_halo):
     conv.run(xin, out)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(out.to_nchw(), want)
+
+
+_SPLIT_GEOMS = {
+    # (N, C, H, W, OC, KH, KW, strides, dilations, pads_begin, pads_end)
+    "3x3_c64_oc64": GEOMS["3x3_s1_p1_c64"],                                              # 9 K steps, 4 tiles
+    "3x3_s2_c128": GEOMS["3x3_s2_p1_c128"],                                              # 18 K steps, ragged pixel tile
+    "3x3_c96_oc200_7x7": (5, 96, 7, 7, 200, 3, 3, (1, 1), (1, 1), (1, 1), (1, 1)),       # 14 steps (13.5 padded), ragged both ways
+    "1x1_c704_oc136": (3, 704, 9, 9, 136, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0)),         # 11 steps: uneven parts
+    "1x1_c2304_oc72_one_tile": (1, 2304, 5, 5, 72, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0)),   # 36 steps, one tile, up to 16 parts
+    "3x3_c64_many_tiles": (20, 64, 28, 28, 320, 3, 3, (1, 1), (1, 1), (1, 1), (1, 1)),   # 123 x 3 tiles x 4 parts: more workgroups than fit at once
+}
+
+
+@pytest.mark.parametrize("tile", [14, 15, 16, 17])
+@pytest.mark.parametrize("epi", ["i32", "fq", "res_u8"])
+@pytest.mark.parametrize("name", sorted(_SPLIT_GEOMS))
+def test_conv_k_split_over_workgroups(orc, name, epi, tile):
+    """tiles 14 to 17: the K loop of a 128 x 128 tile split over 2 / 4 / 8 / 16 workgroups, partial accumulators through
+    a workspace, the last workgroup to arrive adds them and runs the epilogue.  Three launches in a row on
+    one stream with fresh inputs each time: the workspace and its counters are reused, stale partial sums
+    or a counter that is not back at zero would show."""
+    import torch
+    from dldt_amd import Convolution, DeviceTensor, HipieError, make_epilogue
+    g = _SPLIT_GEOMS[name]
+    N, C, H, W, OC = g[:5]
+    rng = np.random.default_rng(zlib.crc32((name + epi).encode()) + tile)
+    x, w = _inputs(rng, g)
+    acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    amax = np.float32(np.abs(acc).max())
+    bias = rng.normal(0, amax / 20, OC).astype(np.float32)
+    ih = rng.uniform(0.3, 1.0, OC).astype(np.float32) * amax
+    e, dt, res, res_kw = None, I32, None, {}
+    if epi == "fq":
+        fq = (256, np.zeros(OC, np.float32), ih, 0.0, 255.0)
+        chain = dict(bias=bias, fq=fq)
+        e, dt = make_epilogue(bias=bias, out_dtype=U8B, fq=fq), U8B
+    elif epi == "res_u8":
+        scale = (rng.uniform(0.5, 2.0, OC) / amax).astype(np.float32)
+        s_x = rng.uniform(0.002, 0.004, OC).astype(np.float32)
+        fq = (256, 0.0, np.float32(1.7), 0.0, 255.0)
+        chain = dict(bias=bias, scale=scale, res_scale=s_x, fq=fq)
+        e, dt = make_epilogue(bias=bias, scale=scale, residual_dtype=U8B, res_mul=s_x, out_dtype=U8B, fq=fq), U8B
+    xin = _device_in(x, g)
+    conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10], e) if e is not None else \
+        Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10])
+    try:
+        conv.set_tile(tile)
+    except HipieError as err:      # fewer than two K steps per part
+        assert err.status == -4 and (C * g[5] * g[6] + 63) // 64 < 2 * (2 << (tile - 14))
+        pytest.skip(str(err))
+    out = DeviceTensor(acc.shape[0], acc.shape[2], acc.shape[3], OC, dt)
+    for rep in range(3):
+        if rep:
+            x, _ = _inputs(rng, g)
+            acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+            xin = _device_in(x, g)
+        rt = None
+        if epi == "i32":
+            want = acc
+        else:
+            if epi == "res_u8":
+                res = rng.integers(0, 256, acc.shape).astype(np.int32)
+                rt = DeviceTensor.from_nchw(res, U8B)
+                want = _chain(orc, acc, res=res, **chain).astype(np.uint8)
+            else:
+                want = _chain(orc, acc, **chain).astype(np.uint8)
+        conv.run(xin, out, rt)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(out.to_nchw(), want, err_msg="launch %d" % rep)
+
+
+def test_conv_k_split_streams_have_own_workspace(orc):
+    """two streams run the same split-K convolution on different inputs at the same time, twenty launches
+    each: every stream has its own partial sums and counters"""
+    import torch
+    from dldt_amd import Convolution, DeviceTensor
+    g = _SPLIT_GEOMS["3x3_c96_oc200_7x7"]
+    rng = np.random.default_rng(99)
+    x0, w = _inputs(rng, g)
+    x1, _ = _inputs(rng, g)
+    wants = [orc.convolution(x, w, g[7], g[8], g[9], g[10]) for x in (x0, x1)]
+    xins = [_device_in(x, g) for x in (x0, x1)]
+    conv = Convolution(w.astype(np.int8), xins[0], g[7], g[8], g[9], g[10])
+    conv.set_tile(15)
+    outs = [DeviceTensor(wt.shape[0], wt.shape[2], wt.shape[3], wt.shape[1], I32) for wt in wants]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    for _ in range(20):
+        for i in range(2):
+            with torch.cuda.stream(streams[i]):
+                conv.run(xins[i], outs[i])
+    torch.cuda.synchronize()
+    for i in range(2):
+        np.testing.assert_array_equal(outs[i].to_nchw(), wants[i])
