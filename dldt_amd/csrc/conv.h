@@ -22,4 +22,8 @@ struct Epilogue {
 
 void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipStream_t s);
 
+// frees the split-K workspace kept for this stream, if any (for the owner of a stream, before it destroys
+// the stream and after the stream's work has finished)
+void release_split_workspace(int device, hipStream_t s);
+
 }  // namespace hipie

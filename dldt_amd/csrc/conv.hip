@@ -1055,11 +1055,18 @@ struct SplitWorkspace {
     DeviceBuffer part, count;
     size_t tiles = 0;
 };
+struct SplitPool {
+    std::mutex mu;
+    std::map<std::pair<int, hipStream_t>, SplitWorkspace> of_stream;
+};
+SplitPool& split_pool() {
+    static auto* pool = new SplitPool();   // never destroyed: the HIP runtime may be gone before static destructors run
+    return *pool;
+}
 SplitWorkspace& split_workspace(int device, hipStream_t s, size_t part_bytes, size_t tiles) {
-    static std::mutex mu;
-    static auto* pool = new std::map<std::pair<int, hipStream_t>, SplitWorkspace>();
-    std::lock_guard<std::mutex> lock(mu);
-    SplitWorkspace& w = (*pool)[std::make_pair(device, s)];
+    SplitPool& pool = split_pool();
+    std::lock_guard<std::mutex> lock(pool.mu);
+    SplitWorkspace& w = pool.of_stream[std::make_pair(device, s)];
     if (w.part.bytes < part_bytes || w.tiles < tiles) {
         DeviceGuard g(device);
         hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
@@ -1177,6 +1184,12 @@ void launch_stream(const ConvArgs& a, int grid_x, hipStream_t s) {
 }
 
 }  // namespace
+
+void release_split_workspace(int device, hipStream_t s) {
+    SplitPool& pool = split_pool();
+    std::lock_guard<std::mutex> lock(pool.mu);
+    pool.of_stream.erase(std::make_pair(device, s));
+}
 
 // ------------------------------------------------------------------------------------------------
 void Epilogue::build(int device_, const hipie_epilogue& e, int64_t oc, int64_t ocp) {

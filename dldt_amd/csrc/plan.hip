@@ -1784,7 +1784,11 @@ struct hipie_request {
     std::vector<void*> pending_out;          // host destinations of the running async infer
     ~hipie_request() {
         for (auto e : events) (void)hipEventDestroy(e);
-        if (stream) (void)hipStreamDestroy(stream);
+        if (stream) {
+            (void)hipStreamSynchronize(stream);
+            if (plan) release_split_workspace(plan->device, stream);
+            (void)hipStreamDestroy(stream);
+        }
     }
 };
 
