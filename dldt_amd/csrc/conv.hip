@@ -632,7 +632,9 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
             *ticket = t;
         }
         __syncthreads();
-        if (*ticket != static_cast<uint32_t>(S - 1)) return;
+        const uint32_t drawn = *ticket;
+        __syncthreads();                                                     // read by every wave before the epilogue stages its stores here
+        if (drawn != static_cast<uint32_t>(S - 1)) return;
         for (int zz = 0; zz < S; ++zz) {
             if (zz == z) continue;
             const int32_t* const other = parts + zz * (64 * NT) + tid;

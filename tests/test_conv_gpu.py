@@ -526,13 +526,14 @@ _SPLIT_GEOMS = {
 
 
 @pytest.mark.parametrize("tile", [14, 15, 16, 17])
-@pytest.mark.parametrize("epi", ["i32", "fq", "res_u8"])
+@pytest.mark.parametrize("epi", ["i32", "fq", "res_u8", "f32_res"])
 @pytest.mark.parametrize("name", sorted(_SPLIT_GEOMS))
 def test_conv_k_split_over_workgroups(orc, name, epi, tile):
     """tiles 14 to 17: the K loop of a 128 x 128 tile split over 2 / 4 / 8 / 16 workgroups, partial accumulators through
     a workspace, the last workgroup to arrive adds them and runs the epilogue.  Three launches in a row on
     one stream with fresh inputs each time: the workspace and its counters are reused, stale partial sums
-    or a counter that is not back at zero would show."""
+    or a counter that is not back at zero would show.  "f32_res" stores f32 through the LDS staging space that
+    also holds the drawn ticket."""
     import torch
     from dldt_amd import Convolution, DeviceTensor, HipieError, make_epilogue
     g = _SPLIT_GEOMS[name]
@@ -554,6 +555,10 @@ def test_conv_k_split_over_workgroups(orc, name, epi, tile):
         fq = (256, 0.0, np.float32(1.7), 0.0, 255.0)
         chain = dict(bias=bias, scale=scale, res_scale=s_x, fq=fq)
         e, dt = make_epilogue(bias=bias, scale=scale, residual_dtype=U8B, res_mul=s_x, out_dtype=U8B, fq=fq), U8B
+    elif epi == "f32_res":
+        scale = (rng.uniform(0.5, 2.0, OC) / amax).astype(np.float32)
+        chain = dict(bias=bias, scale=scale)
+        e, dt = make_epilogue(bias=bias, scale=scale, residual_dtype=F32, out_dtype=F32), F32
     xin = _device_in(x, g)
     conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10], e) if e is not None else \
         Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10])
@@ -571,6 +576,10 @@ def test_conv_k_split_over_workgroups(orc, name, epi, tile):
         rt = None
         if epi == "i32":
             want = acc
+        elif epi == "f32_res":
+            res = rng.normal(0, 1, acc.shape).astype(np.float32)
+            rt = DeviceTensor.from_nchw(res, F32)
+            want = _chain(orc, acc, res=res, **chain)
         else:
             if epi == "res_u8":
                 res = rng.integers(0, 256, acc.shape).astype(np.int32)
@@ -580,7 +589,10 @@ def test_conv_k_split_over_workgroups(orc, name, epi, tile):
                 want = _chain(orc, acc, **chain).astype(np.uint8)
         conv.run(xin, out, rt)
         torch.cuda.synchronize()
-        np.testing.assert_array_equal(out.to_nchw(), want, err_msg="launch %d" % rep)
+        got = out.to_nchw()
+        if dt == F32:
+            got, want = got.view(np.uint32), np.ascontiguousarray(want, np.float32).view(np.uint32)
+        np.testing.assert_array_equal(got, want, err_msg="launch %d" % rep)
 
 
 def test_conv_k_split_streams_have_own_workspace(orc):
