@@ -1079,7 +1079,8 @@ SplitWorkspace& split_workspace(int device, hipStream_t s, size_t part_bytes, si
         if (w.part.bytes < part_bytes) w.part.alloc(device, part_bytes);
         if (w.tiles < tiles) {
             w.count.alloc(device, tiles * sizeof(uint32_t));
-            HIPIE_CHECK_HIP(hipMemset(w.count.ptr, 0, tiles * sizeof(uint32_t)));
+            // on the launching stream: a memset on the null stream is not ordered before work on a non-blocking stream
+            HIPIE_CHECK_HIP(hipMemsetAsync(w.count.ptr, 0, tiles * sizeof(uint32_t), s));
             w.tiles = tiles;
         }
     }
