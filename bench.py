@@ -23,7 +23,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per convolution/FC launch at batch 64, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script (profiles/conv_kernels_resnet50_b64.md: 2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE, factors
 # calibrated on copies of known size in the same runs)
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH_B64 = 34.2e6
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH_B64 = 34.8e6
 
 
 def cpu_baseline(batch_images, budget_s=20.0):
