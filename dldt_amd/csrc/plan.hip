@@ -282,18 +282,24 @@ struct ConvStep : Step {
             check_status(hipie_conv_get_tile(conv, &applied), name.c_str());
             if (applied != tile) continue;   // not available for this layer (kept its previous variant)
             launch_all(2);
-            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipStreamSynchronize(lanes[l].stream));
-            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventRecord(e0[l], lanes[l].stream));
-            launch_all(5);
-            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventRecord(e1[l], lanes[l].stream));
-            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventSynchronize(e1[l]));
-            float ms = 0.f;   // earliest start to latest end
-            for (size_t a = 0; a < nl; ++a)
-                for (size_t b = 0; b < nl; ++b) {
-                    float t = 0.f;
-                    HIPIE_CHECK_HIP(hipEventElapsedTime(&t, e0[a], e1[b]));
-                    ms = std::max(ms, t);
-                }
+            // the fastest of three rounds of five launches: a round disturbed by something else on the
+            // device (another plan being compiled, a clock step) does not decide the choice
+            float ms = 0.f;
+            for (int round = 0; round < 3; ++round) {
+                for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipStreamSynchronize(lanes[l].stream));
+                for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventRecord(e0[l], lanes[l].stream));
+                launch_all(5);
+                for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventRecord(e1[l], lanes[l].stream));
+                for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventSynchronize(e1[l]));
+                float span = 0.f;   // earliest start to latest end
+                for (size_t a = 0; a < nl; ++a)
+                    for (size_t b = 0; b < nl; ++b) {
+                        float t = 0.f;
+                        HIPIE_CHECK_HIP(hipEventElapsedTime(&t, e0[a], e1[b]));
+                        span = std::max(span, t);
+                    }
+                ms = round == 0 ? span : std::min(ms, span);
+            }
             // a variant has to beat the best so far by more than the timing noise of seven launches,
             // otherwise the choice (and the run-to-run spread of a whole network) follows the noise
             if (c == 0 || ms < 0.97f * best_ms) {
