@@ -38,7 +38,7 @@ def cpu_baseline(batch_images, budget_s=20.0):
     g, _ = builders.resnet50(batch=1, res=224)
     x = np.random.default_rng(5).uniform(0, 1, (1, 3, 224, 224)).astype(np.float32)
     t0 = time.perf_counter()
-    evaluate(orc, g.nodes, {"data": x}, keep=[])
+    first, _ = evaluate(orc, g.nodes, {"data": x}, keep=[])
     one = time.perf_counter() - t0
     n = 1
     total = one
@@ -49,7 +49,24 @@ def cpu_baseline(batch_images, budget_s=20.0):
         n += 1
     return {"value": n / total, "unit": "images/sec", "cores": cores, "kind": "port",
             "sample": "%d image(s) of ResNet-50 v1.5 INT8 224x224 through oracle/ngraph_ops.c "
-                      "(scalar int32 reference loops, OpenMP over batch x output channels), %.1f s" % (n, total)}
+                      "(scalar int32 reference loops, OpenMP over batch x output channels), %.1f s" % (n, total)}, \
+        x, first["logits"]
+
+
+def parity_check(plan, batch, x, want):
+    """The oracle's image as image 0 of one inference of the benchmarked plan (the other images random):
+    its dequantised f32 logits against the oracle's, as the deviation relative to the output range and
+    as top-1 agreement.  Integer-exact kernels and the same f32 epilogue make them equal bit for bit."""
+    import numpy as np
+    xb = np.random.default_rng(11).uniform(0, 1, (batch,) + x.shape[1:]).astype(np.float32)
+    xb[0] = x[0]
+    (y,) = plan.create_request().infer(xb)
+    got, ref = y[0].astype(np.float64), want[0].astype(np.float64)
+    rng_out = float(ref.max() - ref.min()) or 1.0
+    return {"against": "oracle (reference ops on the post-LPT graph), image 0 of a batch-%d inference" % batch,
+            "bit_exact": bool(np.array_equal(y[0].view(np.uint32), want[0].view(np.uint32))),
+            "max_abs_over_output_range": float(np.abs(got - ref).max() / rng_out),
+            "top1_agreement": float(int(np.argmax(got)) == int(np.argmax(ref))), "images": 1}
 
 
 def main():
@@ -178,7 +195,10 @@ def main():
                                       for t in sorted({s["type"] for s in steps} - {"Convolution", "Convolution+Shortcut", "MatMul"})},
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.batch)
+        line["cpu_baseline"], x_one, want_one = cpu_baseline(args.batch)
+        line["parity"] = parity_check(plan, args.batch, x_one, want_one)
+        if not line["parity"]["bit_exact"]:
+            sys.stderr.write("bench.py: logits differ from the oracle's: %r\n" % (line["parity"],))
     print(json.dumps(line))
 
 

@@ -83,7 +83,7 @@ def test_small_mobilenet_v2_bit_exact(orc):
 
 @pytest.mark.parametrize("net", ["resnet50", "mobilenet_v2"])
 def test_full_size_batch_consistency(net):
-    """Full-size networks (224x224, width 1.0), where the oracle would take minutes: every image's
+    """Full-size networks (224x224, width 1.0) at a batch the oracle would take a while for: every image's
     logits in a batch-16 inference must equal, bit for bit, the logits of the same image inferred
     alone.  The two plans differ in tile counts, in the kernel variants the tuner picks and in which
     tiles are partial, so this pins the full-size indexing that the reduced networks cannot reach."""
@@ -99,6 +99,20 @@ def test_full_size_batch_consistency(net):
     for i in (0, 7, 15):
         (y1,) = req1.infer(x[i:i + 1])
         np.testing.assert_array_equal(y1.view(np.uint32), y16[i:i + 1].view(np.uint32), err_msg="image %d" % i)
+
+
+@pytest.mark.parametrize("net", ["resnet50", "mobilenet_v2"])
+def test_full_size_logits_match_oracle(orc, net):
+    """Full-size networks (224x224, width 1.0), two images: the dequantised f32 logits equal the oracle's bit
+    for bit, hence zero deviation relative to the output range and the same top-1 class for every image."""
+    from dldt_amd import builders
+    g, _ = getattr(builders, net)(batch=2, res=224)
+    x = np.random.default_rng(77).uniform(0, 1, (2, 3, 224, 224)).astype(np.float32)
+    (got,) = g.compile().create_request().infer(x)
+    want, _ = evaluate(orc, g.nodes, {"data": x}, keep=[])
+    np.testing.assert_array_equal(got.view(np.uint32), want["logits"].view(np.uint32))
+    assert (got.argmax(axis=1) == want["logits"].argmax(axis=1)).all()
+    assert np.ptp(want["logits"]) > 0
 
 
 def test_requests_in_flight_do_not_disturb_each_other():
