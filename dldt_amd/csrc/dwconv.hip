@@ -13,6 +13,17 @@
 namespace hipie {
 namespace {
 
+// Workgroups are handed to the eight XCDs in turn (blockIdx mod 8), and each XCD has its own L2.  Items run
+// along a row, then down the rows of an image: in launch order vertically adjacent output rows - which share
+// one (stride 2) or two (stride 1) of their three input rows - land on different XCDs, and every XCD fetches
+// the shared rows from memory for itself (FETCH_SIZE read 1.4 to 3.1 times the input).  With per_xcd > 0 the
+// grid has 8 * per_xcd workgroups and XCD x works through the contiguous range [x * per_xcd, (x + 1) * per_xcd)
+// of them, so neighbouring rows meet in one L2; indices past the last item fall out at the caller's bound check.
+__device__ __forceinline__ int64_t workgroup_index(int per_xcd) {
+    if (per_xcd <= 0) return blockIdx.x;
+    return static_cast<int64_t>(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+}
+
 __device__ __forceinline__ void mac_bytes(uint32_t x, uint32_t w, int& a0, int& a1, int& a2, int& a3) {
     a0 += static_cast<int>(static_cast<int8_t>(x)) * static_cast<int>(static_cast<int8_t>(w));
     a1 += static_cast<int>(static_cast<int8_t>(x >> 8)) * static_cast<int>(static_cast<int8_t>(w >> 8));
@@ -22,8 +33,8 @@ __device__ __forceinline__ void mac_bytes(uint32_t x, uint32_t w, int& a0, int& 
 
 template <uint32_t F>
 __global__ __launch_bounds__(256) void dwconv_kernel(const ConvArgs a, int KH, int KW, int dil_h, int dil_w,
-                                                     int cgroups, int64_t items) {
-    const int64_t item = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+                                                     int cgroups, int64_t items, int per_xcd) {
+    const int64_t item = workgroup_index(per_xcd) * 256 + threadIdx.x;
     if (item >= items) return;
     const int cgi = static_cast<int>(item % cgroups);
     const int m0 = static_cast<int>(item / cgroups) * 2;
@@ -66,8 +77,9 @@ __global__ __launch_bounds__(256) void dwconv_kernel(const ConvArgs a, int KH, i
 // cover are requested before the first multiply, so a wave waits for memory once instead of once
 // per tap, and the two windows share their overlapping input columns in registers.
 template <uint32_t F, int STRIDE>
-__global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cgroups, int pairs_per_row, int64_t items) {
-    const int64_t item = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+__global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cgroups, int pairs_per_row, int64_t items,
+                                                        int per_xcd) {
+    const int64_t item = workgroup_index(per_xcd) * 256 + threadIdx.x;
     if (item >= items) return;
     const int cgi = static_cast<int>(item % cgroups);
     const int pair = static_cast<int>(item / cgroups);
@@ -159,6 +171,17 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cg
 
 }  // namespace
 
+// grid of a launch of `workgroups` workgroups: XCD-contiguous order from 64 workgroups up (8 per XCD), the
+// plain order below that, where spreading the few workgroups matters more than sharing rows
+struct XcdGrid {
+    uint32_t blocks;
+    int per_xcd;
+    explicit XcdGrid(int64_t workgroups) {
+        per_xcd = workgroups >= 64 ? static_cast<int>(ceil_div(workgroups, 8)) : 0;
+        blocks = static_cast<uint32_t>(per_xcd > 0 ? 8 * static_cast<int64_t>(per_xcd) : workgroups);
+    }
+};
+
 void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipStream_t s) {
     const uint32_t core = a.flags & ~CF_OUT_XOR;
     const bool known = core == E_PLAIN0 || core == E_CLAMPFQ;
@@ -167,9 +190,11 @@ void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipS
         const int cgroups = std::min(a.OCp, a.in_sw) / 16;   // groups of 16 channels that exist in the tensors
         const int pairs_per_row = (a.OW + 1) / 2;
         const int64_t items = static_cast<int64_t>(a.M / a.OW) * pairs_per_row * cgroups;
-        const dim3 grid(static_cast<uint32_t>(ceil_div(items, 256))), block(256);
+        const XcdGrid xg(ceil_div(items, 256));
+        const dim3 grid(xg.blocks), block(256);
+        const int per_xcd = xg.per_xcd;
 #define HIPIE_LAUNCH_DW3(FLAGS, STRIDE) \
-    hipLaunchKernelGGL((dwconv3x3_kernel<FLAGS, STRIDE>), grid, block, 0, s, a, cgroups, pairs_per_row, items)
+    hipLaunchKernelGGL((dwconv3x3_kernel<FLAGS, STRIDE>), grid, block, 0, s, a, cgroups, pairs_per_row, items, per_xcd)
         if (core == E_PLAIN0) {
             if (a.conv_sh == 1) HIPIE_LAUNCH_DW3(E_PLAIN0, 1); else HIPIE_LAUNCH_DW3(E_PLAIN0, 2);
         } else {
@@ -180,11 +205,13 @@ void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipS
     }
     const int cgroups = a.OCp / 32;
     const int64_t items = ceil_div(a.M, 2) * cgroups;
-    const dim3 grid(static_cast<uint32_t>(ceil_div(items, 256))), block(256);
+    const XcdGrid xg(ceil_div(items, 256));
+    const dim3 grid(xg.blocks), block(256);
+    const int per_xcd = xg.per_xcd;
     switch (core) {
-    case E_PLAIN0: hipLaunchKernelGGL((dwconv_kernel<E_PLAIN0>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items); break;
-    case E_CLAMPFQ: hipLaunchKernelGGL((dwconv_kernel<E_CLAMPFQ>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items); break;
-    default: hipLaunchKernelGGL((dwconv_kernel<kDyn>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items); break;
+    case E_PLAIN0: hipLaunchKernelGGL((dwconv_kernel<E_PLAIN0>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
+    case E_CLAMPFQ: hipLaunchKernelGGL((dwconv_kernel<E_CLAMPFQ>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
+    default: hipLaunchKernelGGL((dwconv_kernel<kDyn>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
     }
 }
 
