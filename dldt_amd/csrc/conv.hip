@@ -1224,7 +1224,10 @@ void Epilogue::build(int device_, const hipie_epilogue& e, int64_t oc, int64_t o
     }
     if (e.post_scale) { vec(e.post_scale, e.n_post_scale, 1.f, "post_scale", h); up(post_scale, h); flags |= CF_POST_SCALE; }
     if (e.activation == 1) flags |= CF_RELU;
-    else if (e.activation == 2) { flags |= CF_CLAMP; clamp_lo = e.clamp_lo; clamp_hi = e.clamp_hi; }
+    else if (e.activation == 2) {
+        HIPIE_REQUIRE(e.clamp_lo <= e.clamp_hi, HIPIE_PARAMETER_MISMATCH, "epilogue: clamp range [%g, %g]", e.clamp_lo, e.clamp_hi);
+        flags |= CF_CLAMP; clamp_lo = e.clamp_lo; clamp_hi = e.clamp_hi;
+    }
     else if (e.activation == 3) flags |= CF_GELU;
     else HIPIE_REQUIRE(e.activation == 0, HIPIE_PARAMETER_MISMATCH, "epilogue: activation %d", e.activation);
     out_dtype = e.out_dtype;

@@ -430,7 +430,11 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
                 }
                 if (fl & CF_POST_SCALE) x = x * post_[j];
                 if (fl & CF_RELU) x = x > 0.0f ? x : 0.0f;
-                if (fl & CF_CLAMP) x = x < a.clamp_lo ? a.clamp_lo : (x > a.clamp_hi ? a.clamp_hi : x);
+                // clamp.hpp: x < lo ? lo : (x > hi ? hi : x).  In front of a FakeQuantize the median of three gives
+                // the same level in one instruction (x is finite; the two differ only in the sign of a zero,
+                // and both zeros are level 0 or the same distance from every level boundary)
+                if ((fl & CF_CLAMP) && (fl & CF_OUT_FQ)) x = __builtin_amdgcn_fmed3f(x, a.clamp_lo, a.clamp_hi);
+                else if (fl & CF_CLAMP) x = x < a.clamp_lo ? a.clamp_lo : (x > a.clamp_hi ? a.clamp_hi : x);
                 if (fl & CF_GELU) x = gelu_one(x);
                 v[pb][j] = x;
             }
