@@ -1065,9 +1065,12 @@ SplitPool& split_pool() {
     static auto* pool = new SplitPool();   // never destroyed: the HIP runtime may be gone before static destructors run
     return *pool;
 }
-SplitWorkspace& split_workspace(int device, hipStream_t s, size_t part_bytes, size_t tiles) {
+// The caller holds `lock` (on the pool's mutex) until its kernel is enqueued: another host thread that
+// launches on the same stream and needs a larger workspace waits, and its stream synchronisation then
+// covers that kernel before the old buffers are freed.
+SplitWorkspace& split_workspace(std::unique_lock<std::mutex>& lock, int device, hipStream_t s, size_t part_bytes, size_t tiles) {
     SplitPool& pool = split_pool();
-    std::lock_guard<std::mutex> lock(pool.mu);
+    lock = std::unique_lock<std::mutex>(pool.mu);
     SplitWorkspace& w = pool.of_stream[std::make_pair(device, s)];
     if (w.part.bytes < part_bytes || w.tiles < tiles) {
         DeviceGuard g(device);
@@ -1881,10 +1884,11 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         // the K split pays where a launch has fewer tiles than the device has compute units; with many tiles
         // (more than 2048 workgroups, a 128 MB workspace) the plain pipelined kernel runs instead
         if (tile >= 14 && static_cast<int64_t>(a.p_tiles) * a.t_tiles * split_parts(tile) > 2048) tile = 4;
+        std::unique_lock<std::mutex> workspace_lock;   // held across the launch below
         if (tile >= 14) {
             a.ksplit = split_parts(tile);
             const size_t tiles = static_cast<size_t>(a.p_tiles) * a.t_tiles;
-            SplitWorkspace& w = split_workspace(c->device, s, tiles * a.ksplit * 64 * 256 * sizeof(int32_t), tiles);
+            SplitWorkspace& w = split_workspace(workspace_lock, c->device, s, tiles * a.ksplit * 64 * 256 * sizeof(int32_t), tiles);
             a.ws_part = w.part.as<int32_t>();
             a.ws_count = w.count.as<uint32_t>();
         }
