@@ -62,3 +62,37 @@ def test_fq_host_only_object_cannot_run():
     st = dldt_amd.lib().hipie_fq_run_f32(fq._h, ctypes.c_void_p(16), ctypes.c_void_p(16),
                                          ctypes.c_int64(1), ctypes.c_int64(4), None)
     assert st == -10  # NOT_ALLOCATED
+
+
+def _host_conv(c, oc, k, epilogue=None):
+    """a convolution object without a device (weights packed on the host only)"""
+    import types
+    from dldt_amd import Convolution
+    t = types.SimpleNamespace(dtype=41, cs=-(-c // 16) * 16, stride_w=-(-c // 16) * 16, stride_h=20 * (-(-c // 16) * 16))
+    w = np.random.default_rng(1).integers(-127, 128, (oc, c, k, k)).astype(np.int8)
+    return Convolution(w, t, pads_begin=(k // 2, k // 2), pads_end=(k // 2, k // 2), epilogue=epilogue, device=-1)
+
+
+def test_conv_variant_numbers_are_checked_without_a_device():
+    """hipie_conv_set_tile: unknown numbers, the K split over workgroups on a K loop too short for its parts,
+    the first-layer and row-tile kernels on geometries they do not take"""
+    from dldt_amd import HipieError
+    long_k = _host_conv(256, 64, 3)            # 36 K steps of 64 bytes
+    for tile in (0, 4, 12, 14, 15, 16, 17):
+        long_k.set_tile(tile)
+    short_k = _host_conv(64, 64, 1)            # one K step
+    for tile in (18, -1, 12, 13, 14, 17):
+        with pytest.raises(HipieError) as e:
+            short_k.set_tile(tile)
+        assert e.value.status == -4, tile      # PARAMETER_MISMATCH
+    with pytest.raises(HipieError):
+        long_k.set_tile(13)                    # not a 4-byte-pixel first layer
+
+
+def test_epilogue_rejects_an_inverted_clamp_range():
+    from dldt_amd import HipieError, make_epilogue
+    fq = (256, 0.0, 6.0, 0.0, 255.0)
+    _host_conv(32, 32, 1, make_epilogue(activation="clamp", clamp=(0.0, 6.0), out_dtype=41, fq=fq))
+    with pytest.raises(HipieError) as e:
+        _host_conv(32, 32, 1, make_epilogue(activation="clamp", clamp=(6.0, 0.0), out_dtype=41, fq=fq))
+    assert e.value.status == -4
