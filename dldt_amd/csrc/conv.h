@@ -20,6 +20,11 @@ struct Epilogue {
     void fill(ConvArgs& a) const;
 };
 
+// cache-line kernels (conv_line.hip): shape 0 .. 4 = (wave groups, ring stages, K-step bytes) (1, 3, 128), (2, 3, 128),
+// (1, 4, 128), (2, 4, 128), (1, 4, 64)
+void launch_line(const ConvArgs& a, int shape, hipStream_t s);
+int line_row_bytes(int shape);
+
 void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipStream_t s);
 
 // frees the split-K workspace kept for this stream, if any (for the owner of a stream, before it destroys

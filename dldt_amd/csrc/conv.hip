@@ -2,6 +2,7 @@
 #include "conv.h"
 #include "div2.h"
 #include "conv_epilogue.h"
+#include "conv_dispatch.h"
 
 #include <cmath>
 #include <map>
@@ -990,30 +991,6 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
     }
 }
 
-// flag word -> kernel instance
-#define HIPIE_FOR_EACH_EPILOGUE(X, ...)                                                      \
-    switch (core) {                                                                          \
-    case E_PLAIN0: X(E_PLAIN0, __VA_ARGS__); break;                                          \
-    case E_PLAIN: X(E_PLAIN, __VA_ARGS__); break;                                            \
-    case E_RESU8: X(E_RESU8, __VA_ARGS__); break;                                            \
-    case E_RESF32: X(E_RESF32, __VA_ARGS__); break;                                          \
-    case E_RESGEMM: X(E_RESGEMM, __VA_ARGS__); break;                                        \
-    case E_F32: X(E_F32, __VA_ARGS__); break;                                                \
-    case E_SCALE: X(E_SCALE, __VA_ARGS__); break;                                            \
-    case E_SCALEFQ: X(E_SCALEFQ, __VA_ARGS__); break;                                        \
-    case E_DEQFQ: X(E_DEQFQ, __VA_ARGS__); break;                                            \
-    case E_GELUFQ: X(E_GELUFQ, __VA_ARGS__); break;                                          \
-    case E_RESI8: X(E_RESI8, __VA_ARGS__); break;                                            \
-    case E_F32RES: X(E_F32RES, __VA_ARGS__); break;                                          \
-    case E_F32RELU: X(E_F32RELU, __VA_ARGS__); break;                                        \
-    case E_CLAMPFQ: X(E_CLAMPFQ, __VA_ARGS__); break;                                        \
-    case E_PLAIN0 & ~CF_FQ_DIV2: X((E_PLAIN0 & ~CF_FQ_DIV2), __VA_ARGS__); break;            \
-    case E_RESU8 & ~CF_FQ_DIV2: X((E_RESU8 & ~CF_FQ_DIV2), __VA_ARGS__); break;              \
-    case E_RESGEMM & ~CF_FQ_DIV2: X((E_RESGEMM & ~CF_FQ_DIV2), __VA_ARGS__); break;          \
-    case E_CLAMPFQ & ~CF_FQ_DIV2: X((E_CLAMPFQ & ~CF_FQ_DIV2), __VA_ARGS__); break;          \
-    default: X(kDyn, __VA_ARGS__); break;                                                    \
-    }
-
 template <int WOC, int WPIX>
 void launch_tiled(const ConvArgs& a, hipStream_t s, int batches = 1) {
     const dim3 grid(a.p_per_xcd > 0 ? 8 * a.p_per_xcd * a.t_tiles : a.p_tiles * a.t_tiles, batches), block(WOC * WPIX * 64);
@@ -1104,6 +1081,11 @@ int rows_per_tile(int oh, int ow) {
     return r >= 1 ? r : 0;
 }
 
+// the cache-line kernels: a K step of `rb` bytes must stay inside one filter tap, and 32-bit buffer offsets
+bool line_kernel_fits(const hipie_conv_desc& d, int64_t Kp, int64_t OCp, int rb) {
+    return d.groups == 1 && d.in_c_stride % rb == 0 && Kp % rb == 0 && OCp * Kp < (int64_t(1) << 31);
+}
+
 // the first-layer kernel's geometry: 4-byte pixels, one 32-byte slice per filter row, undilated
 bool stem_kernel_fits(const hipie_conv_desc& d) {
     return d.groups == 1 && d.in_c_stride == 4 && d.in_stride_w == 4 && d.dil_h == 1 && d.dil_w == 1 && d.kw * 4 > 16 && d.kw * 4 <= 32 &&
@@ -1137,7 +1119,7 @@ void launch_rows(const ConvArgs& a, hipStream_t s) {
 // the template instances of the persistent kernel: byte outputs and byte / no residual
 bool persist_available(uint32_t flags) {
     switch (flags & ~CF_OUT_XOR) {
-    case E_PLAIN0: case E_PLAIN: case E_RESU8: case E_CLAMPFQ: return true;
+    case E_PLAIN0: case E_PLAIN: case E_RESU8: case E_CLAMPFQ: case E_SCALEFQ0: return true;
     default: return false;
     }
 }
@@ -1152,6 +1134,7 @@ void launch_persist(const ConvArgs& a, hipStream_t s) {
     case E_PLAIN: hipLaunchKernelGGL((conv_persist_kernel<WOC, WPIX, E_PLAIN>), grid, block, 0, s, a, n_per); break;
     case E_RESU8: hipLaunchKernelGGL((conv_persist_kernel<WOC, WPIX, E_RESU8>), grid, block, 0, s, a, n_per); break;
     case E_CLAMPFQ: hipLaunchKernelGGL((conv_persist_kernel<WOC, WPIX, E_CLAMPFQ>), grid, block, 0, s, a, n_per); break;
+    case E_SCALEFQ0: hipLaunchKernelGGL((conv_persist_kernel<WOC, WPIX, E_SCALEFQ0>), grid, block, 0, s, a, n_per); break;
     default: fail(HIPIE_GENERAL_ERROR, "persistent convolution kernel: no instance for epilogue %#x", a.flags);
     }
 }
@@ -1292,6 +1275,16 @@ void Epilogue::build(int device_, const hipie_epilogue& e, int64_t oc, int64_t o
         for (int64_t c = 0; c < ocp; ++c) il0 = il0 && il[c] == 0.0f && !std::signbit(il[c]);
         if (il0) flags |= CF_FQ_IL0;
         if (out_off == -128.0f) flags |= CF_OUT_XOR;
+        else if (out_off != 0.0f) flags |= CF_OUT_ADD;
+        if (lm1 == 255.0f) {
+            flags |= CF_FQ_SAT;
+            // a Clamp whose range holds every channel's FakeQuantize range changes no level: what it cuts off
+            // lies in the FakeQuantize's own saturating branches (clamp.hpp maps x to the bound, which the
+            // FakeQuantize maps to the same end level as any value beyond it)
+            bool covered = (flags & CF_CLAMP) != 0;
+            for (int64_t c = 0; covered && c < ocp; ++c) covered = clamp_lo <= il[c] && clamp_hi >= ih[c];
+            if (covered) flags &= ~CF_CLAMP;
+        }
         break;
     }
     default: fail(HIPIE_PARAMETER_MISMATCH, "epilogue: out dtype %d", e.out_dtype);
@@ -1635,14 +1628,17 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 17, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 22, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
         if (c->depthwise) return;               // one kernel only
         if (c->fused && tile != 0) return;      // the second GEMM exists in the 128 x 128 tiled kernel
         HIPIE_REQUIRE(tile < 8 || tile > 9 || (!c->fused && persist_available(c->epi.flags)), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the persistent kernels exist for byte outputs with a byte residual or none");
         HIPIE_REQUIRE(tile < 6 || tile > 7 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the split-K kernels need an even number of 64-byte K steps (K=%lld)", (long long)c->Kp);
-        HIPIE_REQUIRE(tile < 14 || c->Kp / 64 >= 2 * split_parts(tile), HIPIE_PARAMETER_MISMATCH,
+        HIPIE_REQUIRE(tile < 18 || line_kernel_fits(c->d, c->Kp, c->OCp, line_row_bytes(tile - 18)), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_set_tile: the cache-line kernels need a channel stride (%d) and K (%lld) that are multiples of their %d-byte K step",
+                      c->d.in_c_stride, (long long)c->Kp, line_row_bytes(tile - 18));
+        HIPIE_REQUIRE(tile < 14 || tile > 17 || c->Kp / 64 >= 2 * split_parts(tile), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the K split over workgroups needs two 64-byte K steps per part (K=%lld)", (long long)c->Kp);
         HIPIE_REQUIRE(tile != 13 || stem_kernel_fits(c->d), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the first-layer kernel takes 4-byte pixels and filter rows of 5 to 8 taps, undilated");
@@ -1883,9 +1879,9 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         stages = stages >= 8 && max_stages >= 8 ? 8 : (stages >= 6 && max_stages >= 6 ? 6 : (stages >= 4 && max_stages >= 4 ? 4 : 3));
         // the K split pays where a launch has fewer tiles than the device has compute units; with many tiles
         // (more than 2048 workgroups, a 128 MB workspace) the plain pipelined kernel runs instead
-        if (tile >= 14 && static_cast<int64_t>(a.p_tiles) * a.t_tiles * split_parts(tile) > 2048) tile = 4;
+        if (tile >= 14 && tile <= 17 && static_cast<int64_t>(a.p_tiles) * a.t_tiles * split_parts(tile) > 2048) tile = 4;
         std::unique_lock<std::mutex> workspace_lock;   // held across the launch below
-        if (tile >= 14) {
+        if (tile >= 14 && tile <= 17) {
             a.ksplit = split_parts(tile);
             const size_t tiles = static_cast<size_t>(a.p_tiles) * a.t_tiles;
             SplitWorkspace& w = split_workspace(workspace_lock, c->device, s, tiles * a.ksplit * 64 * 256 * sizeof(int32_t), tiles);
@@ -1893,6 +1889,7 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
             a.ws_count = w.count.as<uint32_t>();
         }
         switch (tile) {
+        case 18: case 19: case 20: case 21: case 22: launch_line(a, tile - 18, s); break;
         case 14:
         case 15:
         case 16:

@@ -81,9 +81,12 @@ __device__ __forceinline__ void init_acc(const ConvArgs& a, int oc_lane, v16i (&
 
 // level index of one value; the clamp folds both saturating branches of the reference
 // MODE 0: IEEE division, 1: reciprocal with two correction rounds, 2: fma(n, r, n * r2)
-template <int MODE, bool IL0>
+// SAT (256 levels only): no clamp.  x <= il gives n <= 0 and a product <= 0, x > ih gives n > d, a quotient
+// >= 1 (every form of the division is the correctly rounded one, which is monotone) and a product >= 255:
+// the packing conversion saturates both to the levels 0 and 255 the reference's branches name.
+template <int MODE, bool IL0, bool SAT = false>
 __device__ __forceinline__ float fq_level_fast(float x, float il, float ih, float d, float r, float r2, float lm1) {
-    const float xc = __builtin_amdgcn_fmed3f(x, il, ih);
+    const float xc = SAT ? x : __builtin_amdgcn_fmed3f(x, il, ih);
     const float n = IL0 ? xc : xc - il;
     float q;
     if (MODE == 2) {
@@ -114,7 +117,7 @@ __device__ __forceinline__ uint32_t add_bytes(uint32_t a, uint32_t b) {
 // with an empty asm: otherwise the compiler sinks the arithmetic into the store predicates and
 // hoists every table load of the epilogue to its top, which costs an occupancy step.
 constexpr uint32_t kDyn = 0xffffffffu;
-constexpr uint32_t E_FQ = CF_OUT_FQ | CF_FQ_RCP | CF_FQ_DIV2;   // the division every verified layer uses
+constexpr uint32_t E_FQ = CF_OUT_FQ | CF_FQ_RCP | CF_FQ_DIV2 | CF_FQ_SAT;   // 256 levels, the division every verified layer uses
 constexpr uint32_t E_PLAIN0 = CF_BIAS | E_FQ | CF_FQ_IL0;
 constexpr uint32_t E_PLAIN = CF_BIAS | E_FQ;
 constexpr uint32_t E_RESU8 = CF_BIAS | CF_SCALE | CF_RES | CF_RES_U8B | CF_RES_MUL | E_FQ | CF_FQ_IL0;
@@ -129,6 +132,7 @@ constexpr uint32_t E_F32RELU = CF_BIAS | CF_SCALE | CF_RELU;
 constexpr uint32_t E_GELUFQ = CF_BIAS | CF_SCALE | CF_GELU | E_FQ;       // FFN up projection: Gelu and the next FakeQuantize in the GEMM
 constexpr uint32_t E_DEQFQ = CF_SCALE | E_FQ;                           // MatMul between activations, requantised (attention context)
 constexpr uint32_t E_CLAMPFQ = CF_BIAS | CF_SCALE | CF_CLAMP | E_FQ | CF_FQ_IL0;
+constexpr uint32_t E_SCALEFQ0 = CF_BIAS | CF_SCALE | E_FQ | CF_FQ_IL0;   // the same behind a Clamp that holds the FakeQuantize's range (ReLU6 -> FQ(0, 6))
 
 // Per-channel tables of the epilogue staged in LDS, one row of `stride` floats per table.  Every
 // lane of a half-wave needs the same four channels at a time: read from global memory that is a
@@ -232,9 +236,11 @@ __device__ __forceinline__ void init_acc_lds(lds_cfloat_ptr sp, int stride, int 
     for (int ob = 0; ob < 2; ++ob)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const v4i c = *(const __attribute__((address_space(3))) v4i*)(corr + 16 * ob + 4 * q);
+            // one LDS read per accumulator tile (volatile: not merged into one read and four register copies per
+            // tile - the reads are broadcasts that cost no vector-ALU issue, the copies would)
 #pragma unroll
             for (int pb = 0; pb < 2; ++pb) {
+                const v4i c = *(const volatile __attribute__((address_space(3))) v4i*)(corr + 16 * ob + 4 * q);
                 acc[ob][pb][4 * q + 0] = c.x;
                 acc[ob][pb][4 * q + 1] = c.y;
                 acc[ob][pb][4 * q + 2] = c.z;
@@ -446,9 +452,15 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     float t;
-                    if (fl & CF_FQ_DIV2) {
+                    if ((fl & CF_FQ_DIV2) && (fl & CF_FQ_SAT)) {
+                        t = (fl & CF_FQ_IL0) ? fq_level_fast<2, true, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], r2_[j], a.lm1)
+                                             : fq_level_fast<2, false, true>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], r2_[j], a.lm1);
+                    } else if (fl & CF_FQ_DIV2) {
                         t = (fl & CF_FQ_IL0) ? fq_level_fast<2, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], r2_[j], a.lm1)
                                              : fq_level_fast<2, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], r2_[j], a.lm1);
+                    } else if ((fl & CF_FQ_RCP) && (fl & CF_FQ_SAT)) {
+                        t = (fl & CF_FQ_IL0) ? fq_level_fast<1, true, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], 0.f, a.lm1)
+                                             : fq_level_fast<1, false, true>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], 0.f, a.lm1);
                     } else if (fl & CF_FQ_RCP) {
                         t = (fl & CF_FQ_IL0) ? fq_level_fast<1, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], 0.f, a.lm1)
                                              : fq_level_fast<1, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], 0.f, a.lm1);
@@ -521,8 +533,8 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
         // stored byte = level + out_off (mod 256); -128 is a sign-bit flip, 0 nothing: one XOR mask
         // covers both, anything else goes through the bytewise add (one uniform branch for all stores)
         const bool flip = a.flags & CF_OUT_XOR;
-        const uint32_t off4 = (static_cast<uint32_t>(static_cast<int>(a.out_off)) & 0xffu) * 0x01010101u;
-        if (!flip && off4 != 0) {
+        if (fl & CF_OUT_ADD) {   // run-time flags only: no specialised instance carries this step
+            const uint32_t off4 = (static_cast<uint32_t>(static_cast<int>(a.out_off)) & 0xffu) * 0x01010101u;
 #pragma unroll
             for (int pb = 0; pb < 2; ++pb)
 #pragma unroll

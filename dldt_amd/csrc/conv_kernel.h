@@ -46,6 +46,8 @@ enum ConvFlags : uint32_t {
     CF_OUT_XOR = 1u << 14,    // packed levels ^ 0x80808080 is the stored byte (offset -128)
     CF_FQ_DIV2 = 1u << 16,    // two-operation division by the channel constant: fma(n, fq_r, n * fq_r2), verified at load time
     CF_GELU = 1u << 17,       // v = gelu(v), ERF mode (after scale / residual, in place of relu / clamp)
+    CF_FQ_SAT = 1u << 18,     // 256 levels: the packing conversion's own saturation to 0 .. 255 stands for both saturating branches
+    CF_OUT_ADD = 1u << 19,    // stored byte = level + out_off by a bytewise add (offsets other than 0 and -128)
     CF_RES_GEMM = 1u << 15,   // residual = (float(acc2) + bias2[c]) * scale2[c] of a second GEMM run in the same kernel
 };
 

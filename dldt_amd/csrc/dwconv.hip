@@ -184,7 +184,7 @@ struct XcdGrid {
 
 void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipStream_t s) {
     const uint32_t core = a.flags & ~CF_OUT_XOR;
-    const bool known = core == E_PLAIN0 || core == E_CLAMPFQ;
+    const bool known = core == E_PLAIN0 || core == E_CLAMPFQ || core == E_SCALEFQ0;
     if (KH == 3 && KW == 3 && dil_h == 1 && dil_w == 1 && a.conv_sh == a.conv_sw && (a.conv_sh == 1 || a.conv_sh == 2) &&
         known && !(a.flags & CF_RES)) {
         const int cgroups = std::min(a.OCp, a.in_sw) / 16;   // groups of 16 channels that exist in the tensors
@@ -197,6 +197,8 @@ void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipS
     hipLaunchKernelGGL((dwconv3x3_kernel<FLAGS, STRIDE>), grid, block, 0, s, a, cgroups, pairs_per_row, items, per_xcd)
         if (core == E_PLAIN0) {
             if (a.conv_sh == 1) HIPIE_LAUNCH_DW3(E_PLAIN0, 1); else HIPIE_LAUNCH_DW3(E_PLAIN0, 2);
+        } else if (core == E_SCALEFQ0) {
+            if (a.conv_sh == 1) HIPIE_LAUNCH_DW3(E_SCALEFQ0, 1); else HIPIE_LAUNCH_DW3(E_SCALEFQ0, 2);
         } else {
             if (a.conv_sh == 1) HIPIE_LAUNCH_DW3(E_CLAMPFQ, 1); else HIPIE_LAUNCH_DW3(E_CLAMPFQ, 2);
         }
@@ -211,6 +213,7 @@ void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipS
     switch (core) {
     case E_PLAIN0: hipLaunchKernelGGL((dwconv_kernel<E_PLAIN0>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
     case E_CLAMPFQ: hipLaunchKernelGGL((dwconv_kernel<E_CLAMPFQ>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
+    case E_SCALEFQ0: hipLaunchKernelGGL((dwconv_kernel<E_SCALEFQ0>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
     default: hipLaunchKernelGGL((dwconv_kernel<kDyn>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
     }
 }

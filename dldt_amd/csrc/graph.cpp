@@ -307,6 +307,11 @@ static int add_pool(hipie_graph* g, int op, int x, const int64_t* kernel, const 
                               std::max(std::max(kernel[i], strides[i]), std::max(pads_begin[i], pads_end[i])) < kMaxAttr,
                           HIPIE_PARAMETER_MISMATCH, "%s: attributes", what);
             n.shape.push_back(pooled(X.shape[2 + i], pads_begin[i], pads_end[i], kernel[i], strides[i], n.ceil_mode));
+            // every window must hold a cell of the tensor: one that lies in the padding alone has no maximum
+            // and no divisor in the reference (max_pool.hpp starts from lowest(), avg_pool.hpp divides by 0 cells)
+            const int64_t last_start = (n.shape.back() - 1) * strides[i] - pads_begin[i];
+            HIPIE_REQUIRE(pads_begin[i] < kernel[i] && last_start < X.shape[2 + i], HIPIE_PARAMETER_MISMATCH,
+                          "%s: a window along axis %d lies in the padding alone", what, 2 + i);
         }
         *id = add_node(g, std::move(n));
     });

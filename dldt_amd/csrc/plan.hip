@@ -273,7 +273,7 @@ struct ConvStep : Step {
         }
         int best = current;
         float best_ms = 0.f;
-        const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17};
+        const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22};
         for (size_t c = 0; c < sizeof(candidates) / sizeof(candidates[0]); ++c) {
             const int tile = candidates[c];
             if (c > 0 && tile == current) continue;
@@ -1678,13 +1678,8 @@ struct Planner {
         a.pt = static_cast<int>(n.pads_begin[0]); a.pl = static_cast<int>(n.pads_begin[1]);
         a.pb = static_cast<int>(n.pads_end[0]); a.pr = static_cast<int>(n.pads_end[1]);
         a.include_pad = st->avg && !n.exclude_pad;
-        const int halo = std::max(std::max(a.pt, a.pb), std::max(a.pl, a.pr));
-        tensors[x.tensor].halo = std::max(tensors[x.tensor].halo, halo);
-        if (halo > 0) {   // pooling reads its padding as level 0
-            TensorInfo& ti = tensors[x.tensor];
-            if (ti.fill_fixed && ti.fill_level != 0) unsupported(id, "consumers of one tensor pad it with different levels");
-            ti.fill_fixed = true;
-        }
+        // pooling reads no padding: both kernels keep their windows on the tensor's own cells (the reference
+        // skips padding cells), so the border may hold whatever the tensor's other consumers need
         st->in = x.tensor;
         int cur = id;
         int out_dtype = tensors[x.tensor].dtype;

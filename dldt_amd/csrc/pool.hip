@@ -23,50 +23,53 @@ struct ByteMax {
     __device__ __forceinline__ uint32_t stored() const { return (even | odd) ^ 0x80808080u; }
 };
 
-// One thread = 16 channels of one output pixel.  Padding cells hold the lowest value (level 0
-// for U8B, -128 for I8) in the tensor's halo, which is the identity of max; the window is
-// trimmed at the padded upper bound as in max_pool.hpp.  K3 = true: a 3 x 3 window that the upper
-// bounds do not trim, all nine loads requested up front.
-template <bool K3>
+// One thread = 16 channels of one output pixel.  The reference skips padding cells and starts from the
+// type's lowest value (max_pool.hpp); max is idempotent, so a window coordinate that falls into the
+// padding is moved onto the nearest cell of the tensor instead (every window holds at least one: the
+// graph refuses the others) and nothing is read from the tensor's border, whatever it holds.
+// K3 = true: a 3 x 3 window, all nine loads requested up front.  VEC = dwords per thread: 4 (16 channels), or 1
+// for tensors whose pixels hold four channels (image inputs).
+template <int VEC> struct PoolWord;
+template <> struct PoolWord<4> { typedef uint4 type; };
+template <> struct PoolWord<1> { typedef uint32_t type; };
+__device__ __forceinline__ void take_word(ByteMax (&r)[4], const uint4& v) { r[0].take(v.x); r[1].take(v.y); r[2].take(v.z); r[3].take(v.w); }
+__device__ __forceinline__ void take_word(ByteMax (&r)[1], const uint32_t& v) { r[0].take(v); }
+__device__ __forceinline__ uint4 stored_word(const ByteMax (&r)[4]) { return make_uint4(r[0].stored(), r[1].stored(), r[2].stored(), r[3].stored()); }
+__device__ __forceinline__ uint32_t stored_word(const ByteMax (&r)[1]) { return r[0].stored(); }
+
+template <bool K3, int VEC>
 __global__ __launch_bounds__(kThreads) void max_pool_nhwc_i8(PoolArgs a) {
+    typedef typename PoolWord<VEC>::type Word;
     const int64_t t = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-    const int cg = a.cs / 16;
+    const int cg = a.cs / (4 * VEC);
     if (t >= static_cast<int64_t>(a.M) * cg) return;
-    const int m = static_cast<int>(t / cg), c = static_cast<int>(t % cg) * 16;
+    const int m = static_cast<int>(t / cg), c = static_cast<int>(t % cg) * (4 * VEC);
     const int n = m / a.OHOW, rem = m - n * a.OHOW, oh = rem / a.OW, ow = rem - oh * a.OW;
     const int y0 = oh * a.sh - a.pt, x0 = ow * a.sw - a.pl;
     const int8_t* base = static_cast<const int8_t*>(a.in) + static_cast<int64_t>(n) * a.in_sn + c;
-    ByteMax r[4];
+    ByteMax r[VEC];
     if (K3) {
-        uint4 v[3][3];
-#pragma unroll
-        for (int y = 0; y < 3; ++y)
-#pragma unroll
-            for (int x = 0; x < 3; ++x)
-                v[y][x] = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(y0 + y) * a.in_sh + (x0 + x) * a.in_sw);
+        Word v[3][3];
 #pragma unroll
         for (int y = 0; y < 3; ++y)
 #pragma unroll
             for (int x = 0; x < 3; ++x) {
-                r[0].take(v[y][x].x);
-                r[1].take(v[y][x].y);
-                r[2].take(v[y][x].z);
-                r[3].take(v[y][x].w);
+                const int yy = min(max(y0 + y, 0), a.H - 1), xx = min(max(x0 + x, 0), a.W - 1);
+                v[y][x] = *reinterpret_cast<const Word*>(base + static_cast<int64_t>(yy) * a.in_sh + xx * a.in_sw);
             }
+#pragma unroll
+        for (int y = 0; y < 3; ++y)
+#pragma unroll
+            for (int x = 0; x < 3; ++x) take_word(r, v[y][x]);
     } else {
-        const int y1 = min(y0 + a.kh, a.H + a.pb), x1 = min(x0 + a.kw, a.W + a.pr);
-        for (int y = y0; y < y1; ++y)
-            for (int x = x0; x < x1; ++x) {
-                const uint4 v = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(y) * a.in_sh + x * a.in_sw);
-                r[0].take(v.x);
-                r[1].take(v.y);
-                r[2].take(v.z);
-                r[3].take(v.w);
-            }
+        const int ya = max(y0, 0), xa = max(x0, 0);
+        const int yb = min(min(y0 + a.kh, a.H + a.pb), a.H), xb = min(min(x0 + a.kw, a.W + a.pr), a.W);
+        for (int y = ya; y < yb; ++y)
+            for (int x = xa; x < xb; ++x)
+                take_word(r, *reinterpret_cast<const Word*>(base + static_cast<int64_t>(y) * a.in_sh + x * a.in_sw));
     }
-    *reinterpret_cast<uint4*>(static_cast<int8_t*>(a.out) + static_cast<int64_t>(n) * a.out_sn +
-                              oh * a.out_sh + ow * a.out_sw + c) =
-        make_uint4(r[0].stored(), r[1].stored(), r[2].stored(), r[3].stored());
+    *reinterpret_cast<Word*>(static_cast<int8_t*>(a.out) + static_cast<int64_t>(n) * a.out_sn +
+                             oh * a.out_sh + ow * a.out_sw + c) = stored_word(r);
 }
 
 // One thread = 4 channels of one output pixel.  Integer window sum (exact; equals the
@@ -167,14 +170,18 @@ __global__ __launch_bounds__(kThreads) void exit_nhwc_to_nchw(ExitArgs a) {
 }  // namespace
 
 void launch_max_pool(const PoolArgs& a, hipStream_t s) {
-    const int64_t threads = static_cast<int64_t>(a.M) * (a.cs / 16);
-    // every 3 x 3 window lies inside the padded tensor: the last one ends at (OH-1)*s - pad + 3 <= H + pad_end
+    const int vec = a.cs % 16 == 0 ? 4 : 1;
+    const int64_t threads = static_cast<int64_t>(a.M) * (a.cs / (4 * vec));
+    // no 3 x 3 window is trimmed at the padded upper bound: the last one ends at (OH-1)*s - pad + 3 <= H + pad_end
+    // (a trimmed cell inside the tensor would have to be left out; cells in the padding never count)
     const int OH = a.OHOW / a.OW;
     const bool k3 = a.kh == 3 && a.kw == 3 && (OH - 1) * a.sh - a.pt + 3 <= a.H + a.pb &&
                     (a.OW - 1) * a.sw - a.pl + 3 <= a.W + a.pr;
     const dim3 grid(static_cast<uint32_t>(ceil_div(threads, kThreads)));
-    if (k3) hipLaunchKernelGGL(max_pool_nhwc_i8<true>, grid, dim3(kThreads), 0, s, a);
-    else hipLaunchKernelGGL(max_pool_nhwc_i8<false>, grid, dim3(kThreads), 0, s, a);
+    if (k3 && vec == 4) hipLaunchKernelGGL((max_pool_nhwc_i8<true, 4>), grid, dim3(kThreads), 0, s, a);
+    else if (vec == 4) hipLaunchKernelGGL((max_pool_nhwc_i8<false, 4>), grid, dim3(kThreads), 0, s, a);
+    else if (k3) hipLaunchKernelGGL((max_pool_nhwc_i8<true, 1>), grid, dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL((max_pool_nhwc_i8<false, 1>), grid, dim3(kThreads), 0, s, a);
 }
 
 void launch_avg_pool(const PoolArgs& a, bool rcp, hipStream_t s) {

@@ -8,16 +8,38 @@ F32, U8, I8, I32 = 10, 40, 50, 70
 _NP = {F32: np.float32, U8: np.uint8, I8: np.int8, I32: np.int32}
 
 
-def evaluate(orc, nodes, feeds, keep=None, override=None):
+def needed_nodes(nodes, targets, stop=()):
+    """ids of the nodes that `targets` depend on, not looking behind the nodes in `stop` (whose values are given)"""
+    need, todo = set(), list(targets)
+    while todo:
+        i = todo.pop()
+        if i in need:
+            continue
+        need.add(i)
+        if i not in stop:
+            todo.extend(nodes[i]["inputs"])
+    return need
+
+
+def evaluate(orc, nodes, feeds, keep=None, override=None, targets=None):
     """feeds: {parameter name: array}.  Returns ({result name: array}, {node id: array} for `keep`).
     override: {node id: array} continues from these values behind the given nodes (a checker passes the
     device's own result of an op that only has tolerance parity); what the oracle computed for such a
-    node from the same inputs is returned in the second dict under ("oracle", node id)."""
+    node from the same inputs is returned in the second dict under ("oracle", node id).
+    targets: evaluate only what these nodes need, taking every overridden node as given (its own inputs are
+    not evaluated and it gets no ("oracle", id) entry): a slice of a deep graph at full size."""
     val = {}
     results = {}
     override = override or {}
     shadow = {}
+    need = needed_nodes(nodes, targets, stop=set(override)) if targets is not None else None
     for i, n in enumerate(nodes):
+        if need is not None:
+            if i not in need:
+                continue
+            if i in override:
+                val[i] = np.asarray(override[i])
+                continue
         op = n["op"]
         x = [val[j] for j in n["inputs"]]
         if op == "Parameter":

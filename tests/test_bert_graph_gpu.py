@@ -171,3 +171,51 @@ def test_encoder_with_attention_mask(orc, monkeypatch):
             np.testing.assert_array_equal(req.matrix(L[name]).reshape(kept[L[name]].shape).view(np.uint32),
                                           kept[L[name]].view(np.uint32), err_msg="layer %d %s" % (li, name))
     np.testing.assert_array_equal(y.view(np.uint32), want["out"].view(np.uint32))
+
+
+def test_encoder_full_size_first_and_last_layer(orc, monkeypatch):
+    """Benchmark configuration 5 at its stated size (12 layers x 768, 12 heads, FFN 3072, sequence 384, batch 16):
+    every integer segment of the first and the last layer (projections, attention, both FFN GEMMs with their
+    dequantisation, residual and requantisation) equals the oracle's, which continues from the device's own value
+    behind each tolerance-only op (Softmax, LayerNorm, Gelu) and, for the last layer, from the device's input of that
+    layer; the glue ops of both layers are compared with what the oracle makes of the device's inputs to them."""
+    from dldt_amd import builders
+    monkeypatch.setenv("HIPIE_KEEP_F32", "1")
+    B, S, H, NH, FF = 16, 384, 768, 12, 3072
+    g, meta = builders.bert_encoder(layers=12, hidden=H, heads=NH, ffn=FF, batch=B, seq=S)
+    x = np.random.default_rng(5).normal(0, 1, (B, S, H)).astype(np.float32)
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps].count("Attention") == 12
+    req = plan.create_request()
+    (y,) = req.infer(x)
+    assert np.isfinite(y).all()
+    shape = dict(p=(B, NH, S, S), h1=(B, S, H), gelu=(B, S, FF), y=(B, S, H), scores=(B, NH, S, S), attn=(B, S, H),
+                 up=(B, S, FF), down=(B, S, H))
+    glue_input = dict(p="scores", h1="attn", gelu="up", y="down")
+    for li in (0, 11):
+        L = meta["layers"][li]
+        mine = list(L.values())
+        given = {L[n]: req.matrix(L[n]).reshape(shape[n]) for n in GLUE_TOL}
+        if li > 0:
+            prev = meta["layers"][li - 1]["y"]
+            given[prev] = req.matrix(prev).reshape(B, S, H)
+        _, kept = evaluate(orc, g.nodes, {"hidden_states": x}, keep=mine, override=given, targets=mine)
+        for name in EXACT:
+            if name == "pq":
+                continue                                  # stays in registers inside the attention kernel
+            w = kept[L[name]]
+            have = req.matrix(L[name]).reshape(w.shape)
+            if w.dtype == np.float32:
+                np.testing.assert_array_equal(have.view(np.uint32), w.view(np.uint32), err_msg="layer %d %s" % (li, name))
+            else:
+                np.testing.assert_array_equal(have.view(np.int8), w.astype(np.int8), err_msg="layer %d %s" % (li, name))
+        assert len(np.unique(kept[L["q"]])) > 60
+        del kept
+        for name, tol in GLUE_TOL.items():               # each glue op from the device's own input to it
+            src = L[glue_input[name]]
+            _, one = evaluate(orc, g.nodes, {"hidden_states": x}, keep=[L[name]],
+                              override={src: req.matrix(src).reshape(shape[glue_input[name]])}, targets=[L[name]])
+            w = one[L[name]]
+            np.testing.assert_allclose(req.matrix(L[name]).reshape(w.shape), w, err_msg="layer %d %s" % (li, name), **tol)
+    np.testing.assert_array_equal(y.reshape(-1, H).view(np.uint32),
+                                  req.matrix(meta["layers"][11]["y"]).reshape(-1, H).view(np.uint32))

@@ -618,3 +618,93 @@ def test_conv_k_split_streams_have_own_workspace(orc):
     torch.cuda.synchronize()
     for i in range(2):
         np.testing.assert_array_equal(outs[i].to_nchw(), wants[i])
+
+
+# ---- cache-line kernels (tiles 18 - 22): 128-byte (64-byte) K steps through buffer loads that write LDS ----
+LINE_GEOMS = {
+    # name: geometry, what it covers
+    "1x1_c128_oc128_one_step": (2, 128, 9, 9, 128, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0)),          # one 128-byte step
+    "1x1_c256_oc200": (3, 256, 13, 13, 200, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0)),                  # two steps, ragged tiles
+    "1x1_s2_c384_oc72": (2, 384, 14, 14, 72, 1, 1, (2, 2), (1, 1), (0, 0), (0, 0)),                 # three steps: the ring exactly full
+    "3x3_s1_p1_c128": (2, 128, 12, 11, 256, 3, 3, (1, 1), (1, 1), (1, 1), (1, 1)),                  # nine steps, halo reads
+    "3x3_s2_p1_c256_oc320": (2, 256, 13, 13, 320, 3, 3, (2, 2), (1, 1), (1, 1), (1, 1)),            # 18 steps, two and a half channel tiles
+    "1x1_c1024_many_tiles": (20, 1024, 14, 14, 256, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0)),          # 31 pixel tiles: the XCD-aware order
+    "3x3_d2_p2_c128": (1, 128, 10, 9, 64, 3, 3, (1, 1), (2, 2), (2, 2), (2, 2)),                    # dilated taps
+    "1x1_c64_oc64": (3, 64, 17, 17, 64, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0)),                      # 64-byte steps only (tile 22)
+    "3x3_c64_oc96": (2, 64, 15, 14, 96, 3, 3, (1, 1), (1, 1), (1, 1), (1, 1)),                      # 64-byte steps only (tile 22)
+}
+
+
+@pytest.mark.parametrize("tile", [18, 19, 20, 21, 22])
+@pytest.mark.parametrize("name", sorted(LINE_GEOMS))
+def test_conv_line_kernels_exact(orc, name, tile):
+    """i32 accumulators and the fused bias + per-channel FakeQuantize bytes of every cache-line variant"""
+    import torch
+    from dldt_amd import Convolution, DeviceTensor, HipieError, make_epilogue
+    g = LINE_GEOMS[name]
+    rng = np.random.default_rng(zlib.crc32(name.encode()) + tile)
+    x, w = _inputs(rng, g)
+    want = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    xin = _device_in(x, g)
+    conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10])
+    step = 64 if tile == 22 else 128
+    if g[1] % step:
+        with pytest.raises(HipieError) as e:     # a K step must not straddle two filter taps
+            conv.set_tile(tile)
+        assert e.value.status == -4
+        return
+    conv.set_tile(tile)
+    out = DeviceTensor(want.shape[0], want.shape[2], want.shape[3], want.shape[1], I32)
+    conv.run(xin, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.to_nchw(), want)
+    OC = g[4]
+    amax = np.float32(np.abs(want).max())
+    bias = rng.normal(0, amax / 20, OC).astype(np.float32)
+    ih = rng.uniform(0.3, 1.0, OC).astype(np.float32) * amax
+    fq = (256, np.zeros(OC, np.float32), ih, 0.0, 255.0)
+    want8 = _chain(orc, want, bias=bias, fq=fq).astype(np.uint8)
+    conv8 = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10], make_epilogue(bias=bias, out_dtype=U8B, fq=fq))
+    conv8.set_tile(tile)
+    out8 = DeviceTensor(want.shape[0], want.shape[2], want.shape[3], OC, U8B)
+    conv8.run(xin, out8)
+    np.testing.assert_array_equal(out8.to_nchw(), want8)
+    assert np.all(out8.padded_channels() == 0)
+
+
+@pytest.mark.parametrize("tile", [18, 19, 22])
+@pytest.mark.parametrize("kind", ["res_u8", "f32", "i8_signed_in"])
+def test_conv_line_kernels_other_epilogues(orc, kind, tile):
+    """u8 residual + requantisation, dequantised f32 output (staged stores), signed i8 activations"""
+    from dldt_amd import Convolution, DeviceTensor, make_epilogue
+    g = (3, 128, 14, 13, 320, 1, 1, (1, 1), (1, 1), (0, 0), (0, 0))
+    rng = np.random.default_rng(zlib.crc32(kind.encode()) + tile)
+    signed = kind == "i8_signed_in"
+    x, w = _inputs(rng, g, signed=signed)
+    OC = g[4]
+    acc = orc.convolution(x, w, g[7], g[8], g[9], g[10])
+    amax = np.float32(np.abs(acc).max())
+    bias = rng.normal(0, amax / 20, OC).astype(np.float32)
+    xin = _device_in(x, g, signed=signed)
+    rt = None
+    if kind == "res_u8":
+        scale = (rng.uniform(0.5, 2.0, OC) / amax).astype(np.float32)
+        res = rng.integers(0, 256, acc.shape).astype(np.int32)
+        s_x = rng.uniform(0.002, 0.004, OC).astype(np.float32)
+        fq = (256, 0.0, np.float32(1.7), 0.0, 255.0)
+        want = _chain(orc, acc, bias=bias, scale=scale, res=res, res_scale=s_x, fq=fq).astype(np.uint8)
+        epi = make_epilogue(bias=bias, scale=scale, residual_dtype=U8B, res_mul=s_x, out_dtype=U8B, fq=fq)
+        rt = DeviceTensor.from_nchw(res, U8B)
+        out = DeviceTensor(acc.shape[0], acc.shape[2], acc.shape[3], OC, U8B)
+    else:
+        scale = (rng.uniform(0.5, 2.0, OC) * 1e-4).astype(np.float32)
+        want = _chain(orc, acc, bias=bias, scale=scale)
+        epi = make_epilogue(bias=bias, scale=scale, out_dtype=F32)
+        out = DeviceTensor(acc.shape[0], acc.shape[2], acc.shape[3], OC, F32)
+    conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10], epi)
+    conv.set_tile(tile)
+    conv.run(xin, out, rt)
+    if kind == "res_u8":
+        np.testing.assert_array_equal(out.to_nchw(), want)
+    else:
+        np.testing.assert_array_equal(out.to_nchw().view(np.uint32), want.view(np.uint32))

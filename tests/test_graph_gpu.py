@@ -290,3 +290,26 @@ def test_asynchronous_requests_from_page_locked_blobs():
     assert e.value.status == -11
     for a, b in zip(got, want):
         np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+@pytest.mark.parametrize("net", ["resnet50", "mobilenet_v2"])
+def test_full_size_batch_64(orc, net):
+    """The benchmarked configurations at their stated size (224x224, width 1.0, batch 64): the logits of four images
+    of a batch-64 inference equal, bit for bit, those of the same images inferred alone, and for two of them the
+    oracle's f32 logits (same top-1 class, zero deviation)."""
+    from dldt_amd import builders
+    build = getattr(builders, net)
+    rng = np.random.default_rng(64)
+    x = rng.uniform(0, 1, (64, 3, 224, 224)).astype(np.float32)
+    g64, _ = build(batch=64, res=224)
+    (y64,) = g64.compile().create_request().infer(x)
+    assert np.isfinite(y64).all() and len({y64[i].tobytes() for i in range(64)}) == 64   # 64 different images, 64 different results
+    g1, _ = build(batch=1, res=224)
+    req1 = g1.compile().create_request()
+    for i in (0, 21, 42, 63):
+        (y1,) = req1.infer(x[i:i + 1])
+        np.testing.assert_array_equal(y1.view(np.uint32), y64[i:i + 1].view(np.uint32), err_msg="image %d" % i)
+    for i in (0, 63):
+        want, _ = evaluate(orc, g1.nodes, {"data": x[i:i + 1]}, keep=[])
+        np.testing.assert_array_equal(y64[i:i + 1].view(np.uint32), want["logits"].view(np.uint32), err_msg="image %d" % i)
+        assert y64[i].argmax() == want["logits"][0].argmax()

@@ -1,0 +1,141 @@
+"""MaxPool / AvgPool on quantized NHWC tensors through the graph-level C ABI (hipie_graph_max_pool,
+hipie_graph_avg_pool) against the oracle: the reference's own hand vectors
+(ngraph/test/backend/max_pool.in.cpp, avg_pool.in.cpp, every 4-D case) and seeded u8 / i8 fuzz over
+ceil_mode, include-pad, asymmetric pads and windows whose in-bounds values are all negative."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _cases(stem):
+    with open(os.path.join(HERE, "golden", stem + ".json")) as f:
+        return {k: t for k, t in json.load(f)["tests"].items() if len(t["in_shape"]) == 4}
+
+
+def _pads(t):
+    """explicit pads of a golden (SAME_* resolved as the op's shape inference does)"""
+    pb, pe = list(t["pads_begin"]), list(t["pads_end"])
+    auto = t.get("auto_pad")
+    if auto:
+        for i in range(2):
+            total = max((t["out_shape"][2 + i] - 1) * t["strides"][i] + t["kernel"][i] - t["in_shape"][2 + i], 0)
+            lo, hi = total // 2, total - total // 2
+            pb[i], pe[i] = (lo, hi) if auto == "SAME_UPPER" else (hi, lo)
+    return pb, pe
+
+
+def _pool_graph(shape, signed, kind, kernel, strides, pb, pe, ceil, exclude_pad=True):
+    """Parameter f32 -> FakeQuantize to 8-bit levels (the identity on integer inputs) -> pool -> dequantization"""
+    from dldt_amd.graph import Graph
+    from dldt_amd.tensor import F32, I8, U8
+    g = Graph()
+    x = g.parameter("x", shape)
+    lo, hi = (-128.0, 127.0) if signed else (0.0, 255.0)
+    q = g.fake_quantize(x, lo, hi, lo, hi, 256, out_dtype=I8 if signed else U8)
+    if kind == "max":
+        p = g.max_pool(q, kernel, strides, pb, pe, ceil_mode=ceil)
+        y = g.multiply(g.convert(p, F32), g.constant(np.float32(0.5).reshape(1, 1, 1, 1)))
+    else:
+        # after LPT the AvgPool reads the levels themselves and declares an f32 result (avg_pool.cpp:36-45 moves the
+        # dequantization behind it)
+        p = g.avg_pool(q, kernel, strides, pb, pe, exclude_pad=exclude_pad, ceil_mode=ceil, out_dtype=F32)
+        y = p
+    g.result(y, "y")
+    return g, p
+
+
+def _run(orc, g, x):
+    from interp import evaluate
+    want, _ = evaluate(orc, g.nodes, {"x": x})
+    req = g.compile().create_request()
+    (got,) = req.infer(x)
+    return got, want["y"]
+
+
+@pytest.mark.parametrize("name", sorted(_cases("max_pool")))
+def test_max_pool_reference_vectors(orc, name):
+    t = _cases("max_pool")[name]
+    pb, pe = _pads(t)
+    x = np.asarray(t["a"], np.float32).reshape(t["in_shape"])
+    g, _ = _pool_graph(t["in_shape"], False, "max", t["kernel"], t["strides"], pb, pe, t.get("ceil", False))
+    got, want = _run(orc, g, x)
+    assert got.shape == tuple(t["out_shape"])
+    np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(got, 0.5 * np.asarray(t["result"], np.float32).reshape(t["out_shape"]))
+
+
+@pytest.mark.parametrize("name", sorted(_cases("avg_pool")))
+def test_avg_pool_reference_vectors(orc, name):
+    t = _cases("avg_pool")[name]
+    pb, pe = _pads(t)
+    x = np.asarray(t["a"], np.float32).reshape(t["in_shape"])
+    g, _ = _pool_graph(t["in_shape"], False, "avg", t["kernel"], t["strides"], pb, pe, t.get("ceil", False), t["exclude_pad"])
+    got, want = _run(orc, g, x)
+    assert got.shape == tuple(t["out_shape"])
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    np.testing.assert_array_equal(got, np.asarray(t["result"], np.float32).reshape(t["out_shape"]))
+
+
+GEOMETRIES = [
+    # kernel, strides, pads_begin, pads_end, ceil
+    ((3, 3), (2, 2), (1, 1), (1, 1), False),     # the ResNet stem pool
+    ((3, 3), (2, 2), (0, 0), (1, 1), True),
+    ((3, 3), (1, 1), (1, 1), (1, 1), False),
+    ((2, 2), (2, 2), (0, 0), (0, 0), True),
+    ((3, 2), (2, 1), (1, 0), (0, 1), False),     # asymmetric pads, rectangular window
+    ((5, 5), (3, 3), (2, 1), (1, 2), True),
+    ((2, 3), (1, 2), (1, 2), (0, 0), True),
+    ((7, 7), (1, 1), (0, 0), (0, 0), False),     # global pool of a 7 x 7 map
+]
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("geo", range(len(GEOMETRIES)))
+def test_max_pool_fuzz(orc, geo, signed):
+    kernel, strides, pb, pe, ceil = GEOMETRIES[geo]
+    rng = np.random.default_rng(100 + geo)
+    h, w = (7, 7) if kernel == (7, 7) else (13, 10)
+    shape = (3, 40, h, w)                         # 40 channels: padded to 48 in the arena
+    lo, hi = (-128, 128) if signed else (0, 256)
+    x = rng.integers(lo, hi, shape).astype(np.float32)
+    if signed:
+        x[1] = -np.abs(x[1]) - 1.0                # an image whose every value is negative: padding must never win
+        x[1] = np.maximum(x[1], -128.0)
+    g, p = _pool_graph(shape, signed, "max", kernel, strides, pb, pe, ceil)
+    got, want = _run(orc, g, x)
+    np.testing.assert_array_equal(got, want)
+    if signed:
+        assert got[1].max() < 0
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("exclude_pad", [True, False])
+@pytest.mark.parametrize("geo", range(len(GEOMETRIES)))
+def test_avg_pool_fuzz(orc, geo, exclude_pad, signed):
+    kernel, strides, pb, pe, ceil = GEOMETRIES[geo]
+    rng = np.random.default_rng(200 + geo)
+    h, w = (7, 7) if kernel == (7, 7) else (13, 10)
+    shape = (2, 24, h, w)
+    lo, hi = (-128, 128) if signed else (0, 256)
+    x = rng.integers(lo, hi, shape).astype(np.float32)
+    g, _ = _pool_graph(shape, signed, "avg", kernel, strides, pb, pe, ceil, exclude_pad)
+    got, want = _run(orc, g, x)
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_window_in_the_padding_alone_is_refused():
+    """ceil_mode can place the last window behind the tensor's last cell: the reference has no value for it"""
+    from dldt_amd import HipieError
+    from dldt_amd.graph import Graph
+    from dldt_amd.tensor import U8
+    g = Graph()
+    x = g.parameter("x", (1, 16, 4, 4))
+    q = g.fake_quantize(x, 0.0, 255.0, 0.0, 255.0, 256, out_dtype=U8)
+    with pytest.raises(HipieError):
+        g.max_pool(q, (2, 2), (3, 3), (0, 0), (2, 2), ceil_mode=True)   # windows start at 0, 3, 6: the third is padding only
