@@ -1067,6 +1067,40 @@ SplitWorkspace& split_workspace(std::unique_lock<std::mutex>& lock, int device, 
     return w;
 }
 
+// Scratch memory of the entry point that allocates nothing (hipie_conv_run_static): the partial sums and the
+// arrival counters of the K split in a device array of fixed size instead of an allocated workspace.  Every
+// device the library runs on holds its own copy until the process ends; all calls on a device share it.
+constexpr size_t kStaticParts = 256;                                          // 64 KB blocks of partial sums: 16 MB
+constexpr size_t kStaticPartBytes = kStaticParts * 64 * 256 * sizeof(int32_t);
+constexpr size_t kStaticTiles = 1024;                                         // arrival counters
+constexpr size_t kStaticScratchBytes = kStaticPartBytes + kStaticTiles * sizeof(uint32_t);
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+
+// The array's name is a host-side handle, not a device address: the address is asked for once per device, with
+// that device current, and only that pointer is ever passed to a kernel.
+struct StaticScratch {
+    std::mutex mu;
+    std::map<int, uint8_t*> of_device;
+};
+uint8_t* static_scratch(int device) {
+    static auto* table = new StaticScratch();   // never destroyed, like the workspace pool
+    std::lock_guard<std::mutex> lock(table->mu);
+    auto it = table->of_device.find(device);
+    if (it != table->of_device.end()) return it->second;
+    DeviceGuard g(device);
+    uint8_t* ptr = nullptr;
+    HIPIE_CHECK_HIP(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+    HIPIE_REQUIRE(ptr != nullptr, HIPIE_GENERAL_ERROR, "no device address for the static scratch array on device %d", device);
+    table->of_device[device] = ptr;
+    return ptr;
+}
+
+// arrival counters start at zero: a fill kernel (a memset node in a captured graph gave wrong replays here)
+__global__ void clear_counters_kernel(uint32_t* counters, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) counters[i] = 0u;
+}
+
 // parts of the K split of variants 14 to 17: 2, 4, 8, 16
 int split_parts(int tile) { return 2 << (tile - 14); }
 
@@ -1686,8 +1720,8 @@ int hipie_conv_out_dims(const hipie_conv* c, int32_t h, int32_t w, int32_t* oh, 
     });
 }
 
-int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tensor* residual,
-                   const hipie_tensor* out, void* stream) {
+static int conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tensor* residual,
+                    const hipie_tensor* out, void* stream, bool static_scratch_only) {
     return guarded([&] {
         HIPIE_REQUIRE(c && in && out, HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: null argument");
         HIPIE_REQUIRE(c->wgt.ptr, HIPIE_NOT_ALLOCATED, "hipie_conv_run: host-only object");
@@ -1884,9 +1918,23 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         if (tile >= 14 && tile <= 17) {
             a.ksplit = split_parts(tile);
             const size_t tiles = static_cast<size_t>(a.p_tiles) * a.t_tiles;
-            SplitWorkspace& w = split_workspace(workspace_lock, c->device, s, tiles * a.ksplit * 64 * 256 * sizeof(int32_t), tiles);
-            a.ws_part = w.part.as<int32_t>();
-            a.ws_count = w.count.as<uint32_t>();
+            if (static_scratch_only) {
+                // the device's fixed array instead of an allocated workspace: nothing is allocated, larger launches are refused
+                HIPIE_REQUIRE(tiles * a.ksplit <= kStaticParts && tiles <= kStaticTiles, HIPIE_OUT_OF_BOUNDS,
+                              "hipie_conv_run_static: %zu tiles x %d parts need %zu KB of partial sums, the static scratch holds %zu KB "
+                              "(use hipie_conv_run, which allocates its workspace)",
+                              tiles, a.ksplit, tiles * a.ksplit * 64, kStaticParts * 64);
+                uint8_t* const base = static_scratch(c->device);
+                a.ws_part = reinterpret_cast<int32_t*>(base);
+                a.ws_count = reinterpret_cast<uint32_t*>(base + kStaticPartBytes);
+                // the array keeps what the last call left (a launch that was cut short could have left counters behind)
+                hipLaunchKernelGGL(clear_counters_kernel, dim3(static_cast<uint32_t>(ceil_div(tiles, 256))), dim3(256), 0, s,
+                                   a.ws_count, static_cast<int>(tiles));
+            } else {
+                SplitWorkspace& w = split_workspace(workspace_lock, c->device, s, tiles * a.ksplit * 64 * 256 * sizeof(int32_t), tiles);
+                a.ws_part = w.part.as<int32_t>();
+                a.ws_count = w.count.as<uint32_t>();
+            }
         }
         switch (tile) {
         case 18: case 19: case 20: case 21: case 22: launch_line(a, tile - 18, s); break;
@@ -1918,6 +1966,16 @@ int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tens
         }
         HIPIE_CHECK_HIP(hipGetLastError());
     });
+}
+
+int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tensor* residual,
+                   const hipie_tensor* out, void* stream) {
+    return conv_run(c, in, residual, out, stream, false);
+}
+
+int hipie_conv_run_static(const hipie_conv* c, const hipie_tensor* in, const hipie_tensor* residual,
+                          const hipie_tensor* out, void* stream) {
+    return conv_run(c, in, residual, out, stream, true);
 }
 
 }  // extern "C"

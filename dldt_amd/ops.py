@@ -190,6 +190,14 @@ class Convolution:
                                    ctypes.byref(od), _stream()))
         return out
 
+    def run_static(self, x, out, residual=None):
+        """hipie_conv_run_static: the same launch with the K-split workspace in the library's fixed device array"""
+        xd, od = x.desc(), out.desc()
+        rd = residual.desc() if residual is not None else None
+        check(lib().hipie_conv_run_static(self._h, ctypes.byref(xd), ctypes.byref(rd) if rd else None,
+                                          ctypes.byref(od), _stream()))
+        return out
+
 
 class hipie_matmul_desc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int32) for k in ("a_dtype", "b_dtype", "k", "n")]

@@ -246,6 +246,16 @@ int hipie_conv_epilogue_flags(const hipie_conv* conv, uint32_t* flags, int* spec
 int hipie_conv_set_stages(hipie_conv* conv, int stages);
 int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,
                    const hipie_tensor* out, void* stream);
+/* hipie_conv_run for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same kernels,
+ * same bits; the one piece of device memory hipie_conv_run allocates - the workspace through which variants 14 to
+ * 17 pass their partial sums - is a fixed array inside the library instead (16 MB of partial sums = 256 blocks of
+ * 64 KB, one per tile and part, and 1024 arrival counters; each device the library runs on holds it until the
+ * process ends).  Launches that need more (tiles x parts > 256 or more than 1024 tiles) are refused with
+ * HIPIE_OUT_OF_BOUNDS; nothing is allocated or freed.  All calls on one device share the array: calls that overlap
+ * on one device (different streams or host threads) race on it and must be serialised by the caller. */
+int hipie_conv_run_static(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,
+                          const hipie_tensor* out, void* stream);
 
 /* ======================================================================================
  * 1d. MatMul between two activations (attention scores and context) — reference::matmul<int32_t>
