@@ -73,9 +73,7 @@ class QuantizedNet:
             y = g.convolution(x, wc, **conv_attrs)
             rank = 4
         if bias is not None:
-            b = np.asarray(bias, np.float32)
-            with np.errstate(divide="ignore", invalid="ignore"):
-                bdiv = np.where((b != 0) | (s != 0), b / s, np.float32(0)).astype(np.float32)  # bi / ai
+            bdiv = lpt.swap_multiply_and_add(bias, s)                          # bi / ai
             y = g.add(y, g.constant(self._channel(bdiv, rank)))
         return y, s, rank
 
@@ -94,8 +92,7 @@ class QuantizedNet:
         y, s, rank = self._accumulate(act, w, bias, attrs)
         lo, hi = self.signed_range(out_high) if signed else (np.float32(0), np.float32(out_high))
         d = lpt.decompose_fake_quantize(256, lo, hi)
-        il = (lo / s).astype(np.float32)                                     # fold<Divide>(il, s)
-        ih = (hi / s).astype(np.float32)
+        il, ih = lpt.fuse_elementwise(lpt.MULTIPLY, lo, hi, s)             # fold<Divide>(il, s), fold<Divide>(ih, s)
         q = g.fake_quantize(y, self._channel(il, rank), self._channel(ih, rank), d["new_low"], d["new_high"],
                             256, d["precision"])
         return dict(node=q, scale=np.float32(d["scale"]))
@@ -256,8 +253,8 @@ def resnet50(batch=1, res=224, seed=20211, classes=1000, width=64, stages=RESNET
     y = g.reshape(y, (batch, P["fc.w"].shape[1]))
     d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(R["pool"]))
     s_x = np.float32(a["scale"])
-    q = g.fake_quantize(y, (np.float32(0) / s_x).astype(np.float32), (np.float32(R["pool"]) / s_x).astype(np.float32),
-                        d["new_low"], d["new_high"], 256, U8)
+    il, ih = lpt.fuse_elementwise(lpt.MULTIPLY, np.float32(0), np.float32(R["pool"]), s_x)
+    q = g.fake_quantize(y, il.reshape(()), ih.reshape(()), d["new_low"], d["new_high"], 256, U8)
     pooled = dict(node=q, scale=np.float32(d["scale"]))
     acts["pool"] = pooled
     logits = net.conv_f32(pooled, P["fc.w"], P["fc.b"], matmul=True)
@@ -407,8 +404,8 @@ def mobilenet_v2(batch=1, res=224, seed=20211, classes=1000, width=1.0, blocks=M
     y = g.reshape(y, (batch, P["fc.w"].shape[1]))
     d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(R["pool"]))
     s_x = np.float32(a["scale"])
-    q = g.fake_quantize(y, (np.float32(0) / s_x).astype(np.float32), (np.float32(R["pool"]) / s_x).astype(np.float32),
-                        d["new_low"], d["new_high"], 256, U8)
+    il, ih = lpt.fuse_elementwise(lpt.MULTIPLY, np.float32(0), np.float32(R["pool"]), s_x)
+    q = g.fake_quantize(y, il.reshape(()), ih.reshape(()), d["new_low"], d["new_high"], 256, U8)
     pooled = dict(node=q, scale=np.float32(d["scale"]))
     acts["pool"] = pooled
     logits = net.conv_f32(pooled, P["fc.w"], P["fc.b"], matmul=True)
@@ -475,13 +472,14 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
         wq, s_w = lpt.quantize_weights(w, 255)
         s = (np.float32(act["scale"]) * s_w).astype(np.float32)
         y = g.matmul(act["node"], g.constant(wq, I8), False, True)
-        return g.add(y, g.constant((b / s).astype(np.float32))), s
+        return g.add(y, g.constant(lpt.swap_multiply_and_add(b, s))), s
 
     def linear_fq(act, w, b, absmax):
         y, s = linear(act, w, b)
         lo, hi = net.signed_range(absmax)
         d = lpt.decompose_fake_quantize(256, lo, hi)
-        q = g.fake_quantize(y, (lo / s).astype(np.float32), (hi / s).astype(np.float32), d["new_low"], d["new_high"],
+        il, ih = lpt.fuse_elementwise(lpt.MULTIPLY, lo, hi, s)
+        q = g.fake_quantize(y, il, ih, d["new_low"], d["new_high"],
                             256, I8)
         return dict(node=q, scale=np.float32(d["scale"]))
 

@@ -4,13 +4,36 @@
 // Reference: inference-engine/src/low_precision_transformations/src/
 //   layer_transformation.cpp:194-273 (getPrecisionDetails),
 //   include/low_precision/layer_transformation.hpp:63-107 (DataPrecision::getMin/MaxValue),
-//   network_helper.cpp:943-1087 (decomposeFakeQuantize), :700-827 (foldFakeQuantize).
+//   network_helper.cpp:943-1087 (decomposeFakeQuantize), :700-827 (foldFakeQuantize), :216-292 (swapMultiplyAndAdd),
+//   fake_quantize.cpp:127-183 (fuseElementwise), add.cpp:154-218 (AddTransformation), clamp.cpp:71-89.
+#include <algorithm>
 #include <cmath>
 #include <limits>
 
 #include "common.h"
 
 using namespace hipie;
+
+namespace {
+
+// What one output interval [lo, hi] of a FakeQuantize asks of the integer type that will hold its levels
+// (the per-interval decisions of getPrecisionDetails, layer_transformation.cpp:207-243).
+enum IntervalKind { kUnsigned, kUnsignedWithZeroPoint, kSigned, kSignedWithZeroPoint };
+
+IntervalKind classify_interval(float lo, float hi, int64_t levels) {
+    const bool crosses_zero = std::signbit(lo) != std::signbit(hi);
+    const bool lo_is_off_zero = std::fabs(lo) >= 1.e-6f;
+    if (!(crosses_zero && lo_is_off_zero)) return lo_is_off_zero ? kUnsignedWithZeroPoint : kUnsigned;
+    if (hi == 0.f) return kSignedWithZeroPoint;
+    // a signed interval needs no zero point when lo / hi is the ratio of the type's own ends (-128 / 127, or -1 for
+    // 255 levels) within 0.2 %
+    const float want = levels == 256 ? -128.f / 127.f : -1.f;
+    const float have = lo / hi;
+    const float off = std::fabs((have - want) / std::min(have, want));
+    return off > 0.002f ? kSignedWithZeroPoint : kSigned;
+}
+
+}  // namespace
 
 extern "C" {
 
@@ -20,36 +43,15 @@ int hipie_lpt_precision_details(int64_t levels, const float* out_low, const floa
     return guarded([&] {
         HIPIE_REQUIRE(out_low && out_high && precision && has_negative && has_zero_point && n > 0,
                       HIPIE_PARAMETER_MISMATCH, "hipie_lpt_precision_details: bad argument");
-        const float zeroThreshold = 1.e-6f;
-        const float asymmetryThreshold = 0.002f;
-        const float ratio256 = -128.f / 127.f;
-        bool hasNegative = false, signedPrecision = true, unsignedPrecision = true, hasZeroPoint = false;
-        for (int64_t i = 0; i < n; ++i) {
-            const bool signedInterval = std::signbit(out_low[i]) != std::signbit(out_high[i]);
-            const bool lowIsNotZero = std::fabs(out_low[i]) >= zeroThreshold;
-            if (signedInterval && lowIsNotZero) {
-                unsignedPrecision = false;
-                hasNegative = true;
-                if (out_high[i] != 0.f) {
-                    const float expectedRatio = levels == 256 ? ratio256 : -1.f;
-                    const float actualRatio = out_low[i] / out_high[i];
-                    const float actual = std::fabs((actualRatio - expectedRatio) / std::min(actualRatio, expectedRatio));
-                    if (actual > asymmetryThreshold) hasZeroPoint = true;
-                } else {
-                    hasZeroPoint = true;
-                }
-            } else {
-                signedPrecision = false;
-                if (lowIsNotZero) hasZeroPoint = lowIsNotZero;
-            }
-        }
-        *precision = 0;
-        if (!hasZeroPoint) {
-            if (signedPrecision && !unsignedPrecision) *precision = HIPIE_I8;
-            if (!signedPrecision && unsignedPrecision) *precision = HIPIE_U8;
-        }
-        *has_negative = hasNegative;
-        *has_zero_point = hasZeroPoint;
+        int seen[4] = {0, 0, 0, 0};
+        for (int64_t i = 0; i < n; ++i) ++seen[classify_interval(out_low[i], out_high[i], levels)];
+        const bool any_signed = seen[kSigned] + seen[kSignedWithZeroPoint] > 0;
+        const bool any_unsigned = seen[kUnsigned] + seen[kUnsignedWithZeroPoint] > 0;
+        const bool zero_point = seen[kUnsignedWithZeroPoint] + seen[kSignedWithZeroPoint] > 0;
+        // one integer type for all intervals, and only if none of them needs a zero point
+        *precision = zero_point || any_signed == any_unsigned ? 0 : (any_signed ? HIPIE_I8 : HIPIE_U8);
+        *has_negative = any_signed;
+        *has_zero_point = zero_point;
     });
 }
 
@@ -134,6 +136,84 @@ int hipie_lpt_fold_fake_quantize(const float* values, int64_t oc, int64_t inner,
                 out[c * inner + i] = q;
             }
         }
+    });
+}
+
+/* NetworkHelper::swapMultiplyAndAdd (network_helper.cpp:216-292): x * a + b  ==>  (x + b / a) * a.  out[i] = b[i] / a[i]
+ * with 1 or n values on either side, and 0 where both are 0 (the reference's guard against NaN). */
+int hipie_lpt_swap_multiply_and_add(const float* b, int64_t n_b, const float* a, int64_t n_a, float* out, int64_t n) {
+    return guarded([&] {
+        HIPIE_REQUIRE(b && a && out && n > 0 && (n_b == 1 || n_b == n) && (n_a == 1 || n_a == n), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_lpt_swap_multiply_and_add: %lld and %lld values for %lld", (long long)n_b, (long long)n_a, (long long)n);
+        for (int64_t i = 0; i < n; ++i) {
+            const float bi = b[n_b == 1 ? 0 : i], ai = a[n_a == 1 ? 0 : i];
+            out[i] = (bi != 0.f || ai != 0.f) ? bi / ai : 0.f;
+        }
+    });
+}
+
+/* FakeQuantizeTransformation::fuseElementwise (fake_quantize.cpp:127-183): the elementwise operation with a constant
+ * in front of a FakeQuantize moves into its input range.  kind: HIPIE_LPT_MULTIPLY (range / value; not fused -
+ * *fused = 0, range unchanged - when a value is <= 0 or a quotient is infinite), HIPIE_LPT_SUBTRACT (range + value),
+ * HIPIE_LPT_ADD (range - value).  1 or n values on either side. */
+int hipie_lpt_fuse_elementwise(int kind, const float* in_low, const float* in_high, int64_t n_range, const float* value,
+                               int64_t n_value, float* new_low, float* new_high, int64_t n, int* fused) {
+    return guarded([&] {
+        HIPIE_REQUIRE(in_low && in_high && value && new_low && new_high && fused && n > 0 && (n_range == 1 || n_range == n) &&
+                          (n_value == 1 || n_value == n),
+                      HIPIE_PARAMETER_MISMATCH, "hipie_lpt_fuse_elementwise: bad argument");
+        HIPIE_REQUIRE(kind >= HIPIE_LPT_MULTIPLY && kind <= HIPIE_LPT_ADD, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_lpt_fuse_elementwise: kind %d", kind);
+        *fused = 1;
+        for (int64_t i = 0; i < n; ++i) {
+            const float lo = in_low[n_range == 1 ? 0 : i], hi = in_high[n_range == 1 ? 0 : i], v = value[n_value == 1 ? 0 : i];
+            if (kind == HIPIE_LPT_MULTIPLY) {
+                new_low[i] = lo / v;
+                new_high[i] = hi / v;
+                if (v <= 0.f || std::isinf(new_low[i]) || std::isinf(new_high[i])) *fused = 0;
+            } else if (kind == HIPIE_LPT_SUBTRACT) {
+                new_low[i] = lo + v;
+                new_high[i] = hi + v;
+            } else {
+                new_low[i] = lo - v;
+                new_high[i] = hi - v;
+            }
+        }
+        if (!*fused)
+            for (int64_t i = 0; i < n; ++i) {
+                new_low[i] = in_low[n_range == 1 ? 0 : i];
+                new_high[i] = in_high[n_range == 1 ? 0 : i];
+            }
+    });
+}
+
+/* AddTransformation with dequantizations on both branches (add.cpp:154-218):
+ *   SC_full (X1 - SH_full) + SC_empty (X2 - SH_empty)  ==>  SC_empty ( SC' (X1 - SH') + X2 ),
+ *   SC' = SC_full / SC_empty,  SH' = SH_full + SC_empty SH_empty / SC_full  (the comment at :178-182);
+ * scale_after = SC_empty.  A missing Subtract is shift 0, a missing Multiply scale 1. */
+int hipie_lpt_add_both_branches(const float* shift_full, const float* scale_full, const float* shift_empty,
+                                const float* scale_empty, int64_t n, float* new_shift_full, float* new_scale_full,
+                                float* scale_after) {
+    return guarded([&] {
+        HIPIE_REQUIRE(shift_full && scale_full && shift_empty && scale_empty && new_shift_full && new_scale_full && scale_after && n > 0,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_lpt_add_both_branches: bad argument");
+        for (int64_t i = 0; i < n; ++i) {
+            new_shift_full[i] = shift_full[i] + (shift_empty[i] * scale_empty[i]) / scale_full[i];
+            new_scale_full[i] = scale_full[i] / scale_empty[i];
+            scale_after[i] = scale_empty[i];
+        }
+    });
+}
+
+/* ClampTransformation (clamp.cpp:71-89): the bounds of a Clamp that moves in front of a per-tensor dequantization
+ * (x - shift) * scale: divided by the scale (swapped first when it is negative), then the shift added; evaluated
+ * in double as the reference does. */
+int hipie_lpt_clamp_bounds(double min, double max, double scale, double shift, double* new_min, double* new_max) {
+    return guarded([&] {
+        HIPIE_REQUIRE(new_min && new_max && scale != 0.0, HIPIE_PARAMETER_MISMATCH, "hipie_lpt_clamp_bounds: bad argument");
+        if (scale < 0.0) std::swap(min, max);
+        *new_min = min / scale + shift;
+        *new_max = max / scale + shift;
     });
 }
 

@@ -597,6 +597,88 @@ struct MatExitStep : Step {
 };
 
 // ------------------------------------------------------------------------------------------------
+// Per-load configuration (what IInferencePlugin::LoadExeNetworkImpl receives as its config map,
+// template_config.cpp:16-57).  The environment variables of the same meaning are the process-wide defaults; a
+// key passed to hipie_compile_opts overrides them for that plan.
+struct PlanConfig {
+    bool perf_count = false;       // PERF_COUNT: requests created with perf_count < 0 time every step
+    int streams = 3;               // HIP_THROUGHPUT_STREAMS: requests assumed in flight (tuning lanes, OPTIMAL_NUMBER_OF_INFER_REQUESTS)
+    bool tune = true;              // HIP_TUNE: time the kernel variants at load
+    std::string tune_file;         // HIP_TUNE_FILE: cache of the choices
+    bool keep_f32 = false;         // HIP_KEEP_F32
+    bool fuse_attention = true;    // HIP_FUSE_ATTENTION
+    bool merge_linear = true;      // HIP_MERGE_LINEAR
+    int device_id = -1;            // DEVICE_ID (must agree with the device argument when given)
+    std::string network_name = "hipie_network";
+
+    static bool env_flag(const char* name, bool dflt) {
+        const char* v = std::getenv(name);
+        return v ? v[0] != '0' : dflt;
+    }
+    static PlanConfig from_environment() {
+        PlanConfig c;
+        c.tune = env_flag("HIPIE_TUNE", true);
+        if (const char* f = std::getenv("HIPIE_TUNE_FILE")) c.tune_file = f;
+        if (const char* ts = std::getenv("HIPIE_TUNE_STREAMS")) c.streams = std::max(1, std::min(8, std::atoi(ts)));
+        c.keep_f32 = env_flag("HIPIE_KEEP_F32", false);
+        c.fuse_attention = env_flag("HIPIE_FUSE_ATTENTION", true);
+        c.merge_linear = env_flag("HIPIE_MERGE_LINEAR", true);
+        return c;
+    }
+    static bool yes_no(const char* key, const char* v) {
+        if (!std::strcmp(v, "YES")) return true;
+        if (!std::strcmp(v, "NO")) return false;
+        fail(HIPIE_PARAMETER_MISMATCH, "config key %s takes YES or NO, not '%s'", key, v);
+    }
+    // unknown key: NOT_FOUND, as template_config.cpp:36-38 throws
+    void set(const char* key, const char* value) {
+        HIPIE_REQUIRE(key && value, HIPIE_PARAMETER_MISMATCH, "config: null key or value");
+        const std::string k = key;
+        if (k == "PERF_COUNT") perf_count = yes_no(key, value);
+        else if (k == "HIP_THROUGHPUT_STREAMS") {
+            if (!std::strcmp(value, "HIP_THROUGHPUT_AUTO")) streams = 3;
+            else {
+                char* end = nullptr;
+                const long n = std::strtol(value, &end, 10);
+                HIPIE_REQUIRE(end != value && *end == 0 && n >= 1 && n <= 8, HIPIE_PARAMETER_MISMATCH,
+                              "config key HIP_THROUGHPUT_STREAMS takes 1 .. 8 or HIP_THROUGHPUT_AUTO, not '%s'", value);
+                streams = static_cast<int>(n);
+            }
+        } else if (k == "DEVICE_ID") {
+            char* end = nullptr;
+            const long n = std::strtol(value, &end, 10);
+            HIPIE_REQUIRE(end != value && *end == 0 && n >= 0, HIPIE_PARAMETER_MISMATCH, "config key DEVICE_ID: '%s'", value);
+            device_id = static_cast<int>(n);
+        } else if (k == "HIP_TUNE") tune = yes_no(key, value);
+        else if (k == "HIP_TUNE_FILE") tune_file = value;
+        else if (k == "HIP_KEEP_F32") keep_f32 = yes_no(key, value);
+        else if (k == "HIP_FUSE_ATTENTION") fuse_attention = yes_no(key, value);
+        else if (k == "HIP_MERGE_LINEAR") merge_linear = yes_no(key, value);
+        else if (k == "NETWORK_NAME") network_name = value;
+        else fail(HIPIE_NOT_FOUND, "config key '%s' is not supported", key);
+    }
+    bool get(const std::string& k, std::string& v) const {
+        auto yn = [](bool b) { return std::string(b ? "YES" : "NO"); };
+        if (k == "PERF_COUNT") v = yn(perf_count);
+        else if (k == "HIP_THROUGHPUT_STREAMS") v = std::to_string(streams);
+        else if (k == "DEVICE_ID") v = std::to_string(device_id);
+        else if (k == "HIP_TUNE") v = yn(tune);
+        else if (k == "HIP_TUNE_FILE") v = tune_file;
+        else if (k == "HIP_KEEP_F32") v = yn(keep_f32);
+        else if (k == "HIP_FUSE_ATTENTION") v = yn(fuse_attention);
+        else if (k == "HIP_MERGE_LINEAR") v = yn(merge_linear);
+        else return false;
+        return true;
+    }
+};
+constexpr const char* kConfigKeys = "PERF_COUNT DEVICE_ID HIP_THROUGHPUT_STREAMS HIP_TUNE HIP_TUNE_FILE HIP_KEEP_F32 HIP_FUSE_ATTENTION HIP_MERGE_LINEAR";
+
+// thrown by the planner for a node it cannot take: the status and text of any Error, plus the node
+struct UnsupportedNode : Error {
+    int node;
+    UnsupportedNode(int n, const std::string& m) : Error(HIPIE_NOT_IMPLEMENTED, m), node(n) {}
+};
+
 struct Planner {
     const hipie_graph& g;
     std::vector<Value> values;
@@ -611,19 +693,16 @@ struct Planner {
     // HIPIE_MERGE_LINEAR=0: one GEMM per MatMul node even when several share their input
     bool merge_linear = true;
 
-    explicit Planner(const hipie_graph& graph) : g(graph), values(graph.nodes.size()), visiting(graph.nodes.size(), 0) {
-        const char* k = std::getenv("HIPIE_KEEP_F32");
-        keep_f32 = k && k[0] == '1';
-        const char* f = std::getenv("HIPIE_FUSE_ATTENTION");
-        fuse_attention = !(f && f[0] == '0');
-        const char* ml = std::getenv("HIPIE_MERGE_LINEAR");
-        merge_linear = !(ml && ml[0] == '0');
-    }
+    Planner(const hipie_graph& graph, const PlanConfig& cfg)
+        : g(graph), values(graph.nodes.size()), visiting(graph.nodes.size(), 0), keep_f32(cfg.keep_f32),
+          fuse_attention(cfg.fuse_attention), merge_linear(cfg.merge_linear) {}
 
     const GNode& N(int id) const { return g.nodes[id]; }
 
     [[noreturn]] void unsupported(int id, const char* why) const {
-        fail(HIPIE_NOT_IMPLEMENTED, "node %d '%s' (%s): %s", id, N(id).name.c_str(), op_name(N(id).op), why);
+        char buf[1024];
+        snprintf(buf, sizeof buf, "node %d '%s' (%s): %s", id, N(id).name.c_str(), op_name(N(id).op), why);
+        throw UnsupportedNode(id, buf);
     }
 
     // constant broadcastable along the channel axis of an [N, C, ...] value: 1 or C numbers
@@ -1772,6 +1851,7 @@ struct hipie_plan {
     int64_t arena_bytes = 0;
     struct Io { std::string name; int dtype; std::vector<int64_t> shape; int64_t bytes; };
     std::vector<Io> inputs, outputs;
+    PlanConfig config;
 };
 
 struct hipie_request {
@@ -1782,6 +1862,7 @@ struct hipie_request {
     bool perf = false;
     std::vector<hipEvent_t> events;
     bool started = false;
+    bool cancelled = false;                  // hipie_request_cancel was called on the running inference
     std::vector<void*> pending_out;          // host destinations of the running async infer
     ~hipie_request() {
         for (auto e : events) (void)hipEventDestroy(e);
@@ -1812,12 +1893,17 @@ void enqueue(hipie_request* r, void* const* in, void* const* out) {
 
 // `preset`: kernel variants of an imported plan, one per step; used when they fit the steps planned
 // here (same count, variants exactly where steps have them), else the plan is tuned like a new one
-std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const std::vector<int>* preset) {
+std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const std::vector<int>* preset,
+                                         const PlanConfig& cfg = PlanConfig::from_environment()) {
     HIPIE_REQUIRE(!g->results.empty(), HIPIE_PARAMETER_MISMATCH, "hipie_compile: graph has no Result");
+    HIPIE_REQUIRE(cfg.device_id < 0 || device < 0 || cfg.device_id == device, HIPIE_PARAMETER_MISMATCH,
+                  "hipie_compile: DEVICE_ID %d against device %d", cfg.device_id, device);
     auto plan = std::make_unique<hipie_plan>();
     plan->device = device;
     plan->graph = *g;
-    Planner pl(*g);
+    plan->config = cfg;
+    plan->config.device_id = device;
+    Planner pl(*g, cfg);
     for (int r : g->results) pl.visit(r);
     // arena layout: one region per tensor, 256-byte aligned, with slack on both sides so that
     // K-padding reads of a first-layer filter row stay inside the arena
@@ -1861,7 +1947,6 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
     // defaults).  HIPIE_TUNE_FILE names a cache of the choices, one "step variant" pair a line:
     // read when it matches this plan, written after tuning otherwise (the reference's GPU plugin
     // keeps its tuning results in a file the same way, inference-engine/include/cldnn/cldnn_config.hpp:125 KEY_TUNING_FILE).
-    const char* tune_env = std::getenv("HIPIE_TUNE");
     bool preset_used = false;
     if (device >= 0 && preset && preset->size() == plan->steps.size()) {
         bool match = true;
@@ -1871,8 +1956,8 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
             preset_used = true;
         }
     }
-    if (device >= 0 && !preset_used && !(tune_env && tune_env[0] == '0')) {
-        const char* cache = std::getenv("HIPIE_TUNE_FILE");
+    if (device >= 0 && !preset_used && cfg.tune) {
+        const char* cache = cfg.tune_file.empty() ? nullptr : cfg.tune_file.c_str();
         bool loaded = false;
         if (cache) {
             if (FILE* f = std::fopen(cache, "r")) {
@@ -1897,8 +1982,7 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
         if (!loaded) {
             // HIPIE_TUNE_STREAMS requests are assumed in flight together (default 3, the throughput
             // mode of a plugin with three streams; 1 tunes for the latency of a lone request)
-            const char* ts = std::getenv("HIPIE_TUNE_STREAMS");
-            const int n_lanes = std::max(1, std::min(8, ts ? std::atoi(ts) : 3));
+            const int n_lanes = std::max(1, std::min(8, cfg.streams));
             struct Scratch {
                 std::vector<hipie_request*> r;
                 ~Scratch() { for (auto* q : r) hipie_request_destroy(q); }
@@ -1943,6 +2027,130 @@ int hipie_compile(const hipie_graph* g, int device, hipie_plan** out) {
     return guarded([&] {
         HIPIE_REQUIRE(g && out, HIPIE_PARAMETER_MISMATCH, "hipie_compile: null argument");
         *out = compile_plan(g, device, nullptr).release();
+    });
+}
+
+int hipie_compile_opts(const hipie_graph* g, int device, const char* const* keys, const char* const* values, int n_opts,
+                       hipie_plan** out) {
+    return guarded([&] {
+        HIPIE_REQUIRE(g && out && n_opts >= 0 && (n_opts == 0 || (keys && values)), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_compile_opts: null argument");
+        PlanConfig cfg = PlanConfig::from_environment();
+        for (int i = 0; i < n_opts; ++i) cfg.set(keys[i], values[i]);
+        *out = compile_plan(g, device, nullptr, cfg).release();
+    });
+}
+
+/* IInferencePlugin::QueryNetwork (template_plugin.cpp:117-195): which nodes of the graph this engine can take.
+ * The planner is run without a device; a node it refuses is marked, turned into a boundary (its value becomes an
+ * input of the rest, its own inputs become results so that what feeds it is still planned) and the planner runs
+ * again, until a plan exists.  A node counts as supported when no run refused it. */
+int hipie_query(const hipie_graph* g, int* supported, int n_nodes, int* n_unsupported) {
+    return guarded([&] {
+        HIPIE_REQUIRE(g && supported && n_nodes == static_cast<int>(g->nodes.size()), HIPIE_PARAMETER_MISMATCH,
+                      "hipie_query: `supported` must hold one entry per node (%zu)", g ? g->nodes.size() : size_t(0));
+        hipie_graph work = *g;
+        for (int i = 0; i < n_nodes; ++i) supported[i] = 1;
+        int bad = 0;
+        const PlanConfig cfg = PlanConfig::from_environment();
+        for (int round = 0; round <= n_nodes; ++round) {
+            try {
+                if (work.results.empty()) break;
+                Planner pl(work, cfg);
+                for (int r : work.results) pl.visit(r);
+                break;
+            } catch (const UnsupportedNode& u) {
+                HIPIE_REQUIRE(u.node >= 0 && u.node < n_nodes && supported[u.node], HIPIE_UNEXPECTED,
+                              "hipie_query: the planner refused node %d twice", u.node);
+                supported[u.node] = 0;
+                ++bad;
+                GNode& x = work.nodes[u.node];
+                const std::vector<int> feeds = x.in;
+                if (x.op == OP_RESULT) {
+                    work.results.erase(std::remove(work.results.begin(), work.results.end(), u.node), work.results.end());
+                } else {
+                    for (int f : feeds) {                       // this node no longer uses its inputs
+                        auto& us = work.nodes[f].users;
+                        us.erase(std::remove(us.begin(), us.end(), u.node), us.end());
+                    }
+                    x.op = OP_PARAMETER;
+                    x.in.clear();
+                    x.data.clear();
+                    work.params.push_back(u.node);
+                }
+                for (int f : feeds) {                           // what fed it is still wanted: a result of the rest
+                    const GNode& fn = work.nodes[f];
+                    if (fn.op == OP_CONSTANT || fn.op == OP_PARAMETER) continue;
+                    GNode res;
+                    res.op = OP_RESULT;
+                    res.in = {f};
+                    res.dtype = fn.dtype;
+                    res.shape = fn.shape;
+                    res.name = "query_boundary_" + std::to_string(f);
+                    work.nodes[f].users.push_back(static_cast<int>(work.nodes.size()));
+                    work.results.push_back(static_cast<int>(work.nodes.size()));
+                    work.nodes.push_back(std::move(res));
+                }
+            }
+        }
+        if (n_unsupported) *n_unsupported = bad;
+    });
+}
+
+static int copy_text(const std::string& v, char* buf, size_t cap, const char* what) {
+    HIPIE_REQUIRE(buf && cap > v.size(), HIPIE_OUT_OF_BOUNDS, "%s: %zu bytes needed", what, v.size() + 1);
+    std::memcpy(buf, v.c_str(), v.size() + 1);
+    return HIPIE_OK;
+}
+
+/* IInferencePlugin::GetMetric (template_plugin.cpp:218-259): device-level metrics as text */
+int hipie_get_metric(int device, const char* name, char* buf, size_t cap) {
+    return guarded([&] {
+        HIPIE_REQUIRE(name, HIPIE_PARAMETER_MISMATCH, "hipie_get_metric: null name");
+        const std::string k = name;
+        std::string v;
+        if (k == "SUPPORTED_METRICS")
+            v = "AVAILABLE_DEVICES SUPPORTED_METRICS SUPPORTED_CONFIG_KEYS FULL_DEVICE_NAME IMPORT_EXPORT_SUPPORT DEVICE_ARCHITECTURE "
+                "OPTIMIZATION_CAPABILITIES RANGE_FOR_ASYNC_INFER_REQUESTS RANGE_FOR_STREAMS";
+        else if (k == "SUPPORTED_CONFIG_KEYS") v = kConfigKeys;
+        else if (k == "AVAILABLE_DEVICES") {
+            const int n = hipie_device_count();
+            for (int i = 0; i < n; ++i) v += (i ? " " : "") + std::to_string(i);
+        } else if (k == "FULL_DEVICE_NAME") {
+            char nm[256] = "";
+            check_status(hipie_device_name(device, nm, sizeof nm), "hipie_get_metric");
+            v = nm;
+        } else if (k == "IMPORT_EXPORT_SUPPORT") v = "YES";
+        else if (k == "DEVICE_ARCHITECTURE") v = "gfx950";
+        else if (k == "OPTIMIZATION_CAPABILITIES") v = "INT8 FP32";
+        else if (k == "RANGE_FOR_ASYNC_INFER_REQUESTS") v = "1 8 1";
+        else if (k == "RANGE_FOR_STREAMS") v = "1 8";
+        else fail(HIPIE_NOT_FOUND, "metric '%s' is not supported", name);
+        copy_text(v, buf, cap, "hipie_get_metric");
+    });
+}
+
+/* IExecutableNetworkInternal::GetMetric / GetConfig (template_executable_network.cpp:154-176) */
+int hipie_plan_get_metric(const hipie_plan* p, const char* name, char* buf, size_t cap) {
+    return guarded([&] {
+        HIPIE_REQUIRE(p && name, HIPIE_PARAMETER_MISMATCH, "hipie_plan_get_metric: null argument");
+        const std::string k = name;
+        std::string v;
+        if (k == "SUPPORTED_METRICS") v = "NETWORK_NAME SUPPORTED_METRICS SUPPORTED_CONFIG_KEYS OPTIMAL_NUMBER_OF_INFER_REQUESTS";
+        else if (k == "SUPPORTED_CONFIG_KEYS") v = kConfigKeys;
+        else if (k == "NETWORK_NAME") v = p->config.network_name;
+        else if (k == "OPTIMAL_NUMBER_OF_INFER_REQUESTS") v = std::to_string(p->config.streams);
+        else fail(HIPIE_NOT_FOUND, "metric '%s' is not supported", name);
+        copy_text(v, buf, cap, "hipie_plan_get_metric");
+    });
+}
+
+int hipie_plan_get_config(const hipie_plan* p, const char* key, char* buf, size_t cap) {
+    return guarded([&] {
+        HIPIE_REQUIRE(p && key, HIPIE_PARAMETER_MISMATCH, "hipie_plan_get_config: null argument");
+        std::string v;
+        HIPIE_REQUIRE(p->config.get(key, v), HIPIE_NOT_FOUND, "config key '%s' is not supported", key);
+        copy_text(v, buf, cap, "hipie_plan_get_config");
     });
 }
 
@@ -2020,6 +2228,7 @@ int hipie_plan_io_desc(const hipie_plan* p, int is_output, int index, char* name
         if (name && name_len) snprintf(name, name_len, "%s", v[index].name.c_str());
         *dtype = v[index].dtype;
         *rank = static_cast<int>(v[index].shape.size());
+        HIPIE_REQUIRE(*rank <= 8, HIPIE_UNEXPECTED, "hipie_plan_io_desc: rank %d", *rank);   // `dims` holds 8 entries
         for (int i = 0; i < *rank; ++i) dims[i] = v[index].shape[i];
     });
 }
@@ -2052,7 +2261,7 @@ int hipie_request_create(const hipie_plan* p, int perf_count, hipie_request** ou
                       "hipie_request_create: the plan was compiled without a device (dry run)");
         auto r = std::make_unique<hipie_request>();
         r->plan = p;
-        r->perf = perf_count != 0;
+        r->perf = perf_count < 0 ? p->config.perf_count : perf_count != 0;   // < 0: the plan's PERF_COUNT
         DeviceGuard g(p->device);
         HIPIE_CHECK_HIP(hipStreamCreateWithFlags(&r->stream, hipStreamNonBlocking));
         r->arena.alloc(p->device, static_cast<size_t>(p->arena_bytes));
@@ -2102,6 +2311,13 @@ int hipie_request_start(hipie_request* r, const void* const* inputs, void* const
         HIPIE_REQUIRE(!r->started, HIPIE_REQUEST_BUSY, "hipie_request_start: request is busy");
         const hipie_plan& p = *r->plan;
         DeviceGuard g(p.device);
+        // a failure half-way leaves copies or kernels queued that read the caller's buffers: the stream is drained
+        // before the error is reported, so that the caller may free or reuse them
+        struct Drain {
+            hipStream_t s;
+            bool armed = true;
+            ~Drain() { if (armed) (void)hipStreamSynchronize(s); }
+        } drain{r->stream};
         std::vector<void*> in(p.inputs.size()), out(p.outputs.size());
         for (size_t i = 0; i < in.size(); ++i) {
             HIPIE_REQUIRE(inputs[i], HIPIE_PARAMETER_MISMATCH, "hipie_request_start: input %zu is null", i);
@@ -2122,17 +2338,54 @@ int hipie_request_start(hipie_request* r, const void* const* inputs, void* const
             for (size_t i = 0; i < out.size(); ++i)
                 HIPIE_CHECK_HIP(hipMemcpyAsync(outputs[i], out[i], static_cast<size_t>(p.outputs[i].bytes),
                                                hipMemcpyDeviceToHost, r->stream));
+        drain.armed = false;
         r->started = true;
+        r->cancelled = false;
     });
 }
 
-int hipie_request_wait(hipie_request* r) {
+/* Wait(millis_timeout) of AsyncInferRequestThreadSafeDefault (ie_infer_async_request_thread_safe_default.hpp:167-204):
+ * -1 (RESULT_READY) blocks until the result is there, 0 (STATUS_ONLY) only asks, a positive value waits that many
+ * milliseconds at most; HIPIE_RESULT_NOT_READY leaves the request busy.  A request that was cancelled while it
+ * ran reports HIPIE_INFER_CANCELLED once its queued work has drained, and is idle afterwards. */
+int hipie_request_wait_for(hipie_request* r, int64_t timeout_ms) {
     return guarded([&] {
-        HIPIE_REQUIRE(r, HIPIE_PARAMETER_MISMATCH, "hipie_request_wait: null argument");
+        HIPIE_REQUIRE(r, HIPIE_PARAMETER_MISMATCH, "hipie_request_wait_for: null argument");
+        HIPIE_REQUIRE(timeout_ms >= -1, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_request_wait_for: timeout %lld (RESULT_READY = -1, STATUS_ONLY = 0, or milliseconds)", (long long)timeout_ms);
         HIPIE_REQUIRE(r->started, HIPIE_INFER_NOT_STARTED, "hipie_request_wait: nothing was started");
         DeviceGuard g(r->plan->device);
-        r->started = false;
-        HIPIE_CHECK_HIP(hipStreamSynchronize(r->stream));
+        if (timeout_ms < 0) {
+            r->started = false;
+            HIPIE_CHECK_HIP(hipStreamSynchronize(r->stream));
+        } else {
+            const auto deadline = std::chrono::steady_clock::now() + std::chrono::milliseconds(timeout_ms);
+            for (;;) {
+                const hipError_t q = hipStreamQuery(r->stream);
+                if (q == hipSuccess) break;
+                if (q != hipErrorNotReady) HIPIE_CHECK_HIP(q);
+                if (std::chrono::steady_clock::now() >= deadline) fail(HIPIE_RESULT_NOT_READY, "the inference is still running");
+                std::this_thread::sleep_for(std::chrono::microseconds(50));
+            }
+            r->started = false;
+        }
+        if (r->cancelled) {
+            r->cancelled = false;
+            fail(HIPIE_INFER_CANCELLED, "the inference was cancelled");
+        }
+    });
+}
+
+int hipie_request_wait(hipie_request* r) { return hipie_request_wait_for(r, -1); }
+
+/* Cancel (ie_infer_async_request_thread_safe_default.hpp:255-267).  The kernels and copies of a started inference are
+ * already queued on the request's stream and run to their end (nothing on the device can be revoked); the request is
+ * marked, its outputs are to be taken as undefined, and the next wait reports HIPIE_INFER_CANCELLED.  On an idle
+ * request it does nothing. */
+int hipie_request_cancel(hipie_request* r) {
+    return guarded([&] {
+        HIPIE_REQUIRE(r, HIPIE_PARAMETER_MISMATCH, "hipie_request_cancel: null argument");
+        if (r->started) r->cancelled = true;
     });
 }
 

@@ -158,19 +158,33 @@ class Graph:
         check(lib().hipie_graph_set_name(self._h, id_, name.encode()))
         self.nodes[id_]["name"] = name
 
-    def compile(self, device=0):
-        return Plan(self, device)
+    def compile(self, device=0, config=None):
+        """config: {key: value} as for Core::LoadNetwork (hipie_compile_opts); None = the process defaults"""
+        return Plan(self, device, config=config)
+
+    def query(self):
+        """QueryNetwork: list of booleans, one per node added so far (Result nodes included)"""
+        n = len(self.nodes)
+        flags = (ctypes.c_int * max(n, 1))()
+        bad = ctypes.c_int()
+        check(lib().hipie_query(self._h, flags, n, ctypes.byref(bad)))
+        return [bool(flags[i]) for i in range(n)]
 
 
 class Plan:
     """ExecutableNetwork analogue: fused steps + arena layout + uploaded constants."""
 
-    def __init__(self, graph, device=0, _handle=None):
+    def __init__(self, graph, device=0, _handle=None, config=None):
         self._h = ctypes.c_void_p()
         if _handle is not None:
             self._h = _handle
-        else:
+        elif config is None:
             check(lib().hipie_compile(graph._h, device, ctypes.byref(self._h)))
+        else:
+            items = [(str(k).encode(), str(v).encode()) for k, v in config.items()]
+            keys = (ctypes.c_char_p * max(len(items), 1))(*[k for k, _ in items])
+            vals = (ctypes.c_char_p * max(len(items), 1))(*[v for _, v in items])
+            check(lib().hipie_compile_opts(graph._h, device, keys, vals, len(items), ctypes.byref(self._h)))
         self.device = device
         L = lib()
         L.hipie_plan_arena_bytes.restype = ctypes.c_int64
@@ -202,10 +216,20 @@ class Plan:
         check(lib().hipie_plan_import(blob, ctypes.c_size_t(len(blob)), device, ctypes.byref(h)))
         return cls(None, device, _handle=h)
 
+    def metric(self, name):
+        buf = ctypes.create_string_buffer(1024)
+        check(lib().hipie_plan_get_metric(self._h, name.encode(), buf, ctypes.c_size_t(1024)))
+        return buf.value.decode()
+
+    def config(self, key):
+        buf = ctypes.create_string_buffer(1024)
+        check(lib().hipie_plan_get_config(self._h, key.encode(), buf, ctypes.c_size_t(1024)))
+        return buf.value.decode()
+
     def _io(self, is_out, idx):
         name = ctypes.create_string_buffer(256)
         dt, rank = ctypes.c_int(), ctypes.c_int()
-        dims = (ctypes.c_int64 * 4)()
+        dims = (ctypes.c_int64 * 8)()
         check(lib().hipie_plan_io_desc(self._h, is_out, idx, name, 256, ctypes.byref(dt), dims, ctypes.byref(rank)))
         return dict(name=name.value.decode(errors="replace"), dtype=dt.value, shape=tuple(dims[:rank.value]))
 
@@ -215,6 +239,7 @@ class Plan:
             self._h = None
 
     def create_request(self, perf_count=False):
+        """perf_count: True / False, or None for the plan's PERF_COUNT"""
         return Request(self, perf_count)
 
 
@@ -241,7 +266,7 @@ class Request:
     def __init__(self, plan, perf_count=False):
         self.plan = plan
         self._h = ctypes.c_void_p()
-        check(lib().hipie_request_create(plan._h, int(perf_count), ctypes.byref(self._h)))
+        check(lib().hipie_request_create(plan._h, -1 if perf_count is None else int(perf_count), ctypes.byref(self._h)))
 
     def __del__(self):
         if getattr(self, "_h", None):
@@ -274,6 +299,13 @@ class Request:
 
     def wait(self):
         check(lib().hipie_request_wait(self._h))
+
+    def wait_for(self, timeout_ms):
+        """Wait(ms): -1 blocks, 0 asks only; raises HipieError with status -9 (RESULT_NOT_READY) while it runs"""
+        check(lib().hipie_request_wait_for(self._h, ctypes.c_int64(timeout_ms)))
+
+    def cancel(self):
+        check(lib().hipie_request_cancel(self._h))
 
     def device_buffers(self):
         """torch tensors shaped like the plan's inputs and outputs (for resident-in-HBM runs)."""

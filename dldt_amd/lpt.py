@@ -97,3 +97,52 @@ def round_zero_point(shift):
     Round-5 HALF_AWAY_FROM_ZERO, then Convert to the activation's integer type."""
     s = np.asarray(shift, np.float32)
     return (np.sign(s) * np.floor(np.abs(s) + np.float32(0.5))).astype(np.float32)
+
+
+MULTIPLY, SUBTRACT, ADD = 1, 2, 3
+
+
+def _vec(a):
+    return np.ascontiguousarray(np.asarray(a, np.float32).reshape(-1))
+
+
+def swap_multiply_and_add(b, a):
+    """NetworkHelper::swapMultiplyAndAdd: the constant b / a of x * a + b ==> (x + b / a) * a (0 where both are 0)."""
+    bv, av = _vec(b), _vec(a)
+    n = max(bv.size, av.size)
+    out = np.empty(n, np.float32)
+    check(lib().hipie_lpt_swap_multiply_and_add(_p(bv), ctypes.c_int64(bv.size), _p(av), ctypes.c_int64(av.size), _p(out),
+                                                ctypes.c_int64(n)))
+    return out
+
+
+def fuse_elementwise(kind, in_low, in_high, value):
+    """FakeQuantizeTransformation::fuseElementwise: (new_low, new_high) of a FakeQuantize that absorbs the Multiply /
+    Subtract / Add by a constant in front of it, or None when the reference does not fuse (a non-positive factor)."""
+    lo, hi, v = _vec(in_low), _vec(in_high), _vec(value)
+    assert lo.size == hi.size
+    n = max(lo.size, v.size)
+    nl, nh = np.empty(n, np.float32), np.empty(n, np.float32)
+    fused = ctypes.c_int()
+    check(lib().hipie_lpt_fuse_elementwise(kind, _p(lo), _p(hi), ctypes.c_int64(lo.size), _p(v), ctypes.c_int64(v.size),
+                                           _p(nl), _p(nh), ctypes.c_int64(n), ctypes.byref(fused)))
+    return (nl, nh) if fused.value else None
+
+
+def add_both_branches(shift_full, scale_full, shift_empty, scale_empty):
+    """AddTransformation with dequantizations on both branches: (new shift, new scale) of the full path and the
+    scale of the Multiply behind the Add."""
+    a = [_vec(x) for x in (shift_full, scale_full, shift_empty, scale_empty)]
+    n = max(x.size for x in a)
+    a = [np.ascontiguousarray(np.broadcast_to(x, (n,))) for x in a]
+    out = [np.empty(n, np.float32) for _ in range(3)]
+    check(lib().hipie_lpt_add_both_branches(*[_p(x) for x in a], ctypes.c_int64(n), *[_p(x) for x in out]))
+    return tuple(out)
+
+
+def clamp_bounds(lo, hi, scale, shift=0.0):
+    """ClampTransformation: the bounds of a Clamp moved in front of the per-tensor dequantization (x - shift) * scale"""
+    a, b = ctypes.c_double(), ctypes.c_double()
+    check(lib().hipie_lpt_clamp_bounds(ctypes.c_double(lo), ctypes.c_double(hi), ctypes.c_double(scale), ctypes.c_double(shift),
+                                       ctypes.byref(a), ctypes.byref(b)))
+    return a.value, b.value

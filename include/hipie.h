@@ -419,7 +419,33 @@ int hipie_graph_set_name(hipie_graph* g, int id, const char* friendly_name);
 /* IInferencePlugin::LoadExeNetworkImpl (ie_iplugin_internal.hpp:270-271): fuse, lay out the static
  * HBM arena, pack and upload constants.  The graph may be destroyed afterwards. */
 int hipie_compile(const hipie_graph* graph, int device, hipie_plan** plan);
+/* The same with the config map LoadExeNetworkImpl receives (template_plugin.cpp:95-104, template_config.cpp:16-57) as
+ * n_opts key / value strings.  Keys: PERF_COUNT (YES | NO: default of hipie_request_create's perf_count = -1),
+ * DEVICE_ID (must name `device`), HIP_THROUGHPUT_STREAMS (1 .. 8 or HIP_THROUGHPUT_AUTO: the requests assumed in
+ * flight together; the kernel variants are timed that way and OPTIMAL_NUMBER_OF_INFER_REQUESTS reports it),
+ * HIP_TUNE (YES | NO: time the kernel variants at load, else shape-based defaults), HIP_TUNE_FILE (cache of the
+ * choices, like the reference GPU plugin's KEY_TUNING_FILE), HIP_FUSE_ATTENTION, HIP_MERGE_LINEAR, HIP_KEEP_F32
+ * (YES | NO), NETWORK_NAME.  An unknown key gives HIPIE_NOT_FOUND, a value the key does not take
+ * HIPIE_PARAMETER_MISMATCH.  The environment variables HIPIE_TUNE, HIPIE_TUNE_FILE, HIPIE_TUNE_STREAMS,
+ * HIPIE_FUSE_ATTENTION, HIPIE_MERGE_LINEAR, HIPIE_KEEP_F32 are the process-wide defaults of these keys. */
+int hipie_compile_opts(const hipie_graph* graph, int device, const char* const* keys, const char* const* values,
+                       int n_opts, hipie_plan** plan);
 void hipie_plan_destroy(hipie_plan* plan);
+/* IInferencePlugin::QueryNetwork (ie_iplugin_internal.hpp:255, template_plugin.cpp:117-195): supported[i] = 1 when
+ * the engine can take node i of the graph, 0 when it cannot (every such node, not only the first); n_nodes must be
+ * the graph's node count (ids are 0 .. n_nodes - 1 in the order the nodes were added); n_unsupported may be NULL.
+ * Needs no device. */
+int hipie_query(const hipie_graph* graph, int* supported, int n_nodes, int* n_unsupported);
+/* IInferencePlugin::GetMetric (ie_iplugin_internal.hpp:188, template_plugin.cpp:218-259) as text (lists are
+ * space-separated): SUPPORTED_METRICS, SUPPORTED_CONFIG_KEYS, AVAILABLE_DEVICES, FULL_DEVICE_NAME,
+ * IMPORT_EXPORT_SUPPORT, DEVICE_ARCHITECTURE, OPTIMIZATION_CAPABILITIES, RANGE_FOR_ASYNC_INFER_REQUESTS,
+ * RANGE_FOR_STREAMS; an unknown name gives HIPIE_NOT_FOUND, a buffer that is too small HIPIE_OUT_OF_BOUNDS. */
+int hipie_get_metric(int device, const char* name, char* buf, size_t buf_len);
+/* IExecutableNetworkInternal::GetMetric / GetConfig (template_executable_network.cpp:154-176): NETWORK_NAME,
+ * SUPPORTED_METRICS, SUPPORTED_CONFIG_KEYS, OPTIMAL_NUMBER_OF_INFER_REQUESTS (what benchmark_app asks for,
+ * samples/benchmark_app/main.cpp:456-472); the config keys of hipie_compile_opts with the values the plan was compiled with */
+int hipie_plan_get_metric(const hipie_plan* plan, const char* name, char* buf, size_t buf_len);
+int hipie_plan_get_config(const hipie_plan* plan, const char* key, char* buf, size_t buf_len);
 
 /* IExecutableNetworkInternal::Export(std::ostream&) (ie_iexecutable_network_internal.hpp:77-81) and
  * IInferencePlugin::ImportNetwork(std::istream&, config) (ie_iplugin_internal.hpp:213-222), as the
@@ -435,7 +461,7 @@ int hipie_plan_import(const void* stream, size_t size, int device, hipie_plan** 
 int hipie_plan_num_inputs(const hipie_plan* plan);
 int hipie_plan_num_outputs(const hipie_plan* plan);
 int hipie_plan_io_desc(const hipie_plan* plan, int is_output, int index, char* name, size_t name_len,
-                       int* dtype, int64_t* dims /* [4] */, int* rank);
+                       int* dtype, int64_t* dims /* [8]: ranks up to 8 */, int* rank);
 int64_t hipie_plan_arena_bytes(const hipie_plan* plan);
 /* executed (fused) steps, in order: the exec-graph / perf-counter view
  * (exec_graph_info.hpp:34-76, ie_common.h InferenceEngineProfileInfo) */
@@ -448,7 +474,7 @@ int hipie_plan_step_variant(const hipie_plan* plan, int index, int* variant);
 
 /* IExecutableNetworkInternal::CreateInferRequestImpl: own stream + own activation arena; weights
  * stay shared in the plan.  perf_count mirrors the PERF_COUNT config key (ie_plugin_config.hpp:277). */
-int hipie_request_create(const hipie_plan* plan, int perf_count, hipie_request** request);
+int hipie_request_create(const hipie_plan* plan, int perf_count /* 1, 0, or -1 = the plan's PERF_COUNT */, hipie_request** request);
 void hipie_request_destroy(hipie_request* request);
 /* IInferRequestInternal::InferImpl (ie_iinfer_request_internal.hpp:57).  inputs / outputs are dense
  * NCHW buffers in plan order: host memory (device_memory = 0: H2D, kernels, D2H on the request's
@@ -459,6 +485,15 @@ int hipie_request_infer(hipie_request* request, const void* const* inputs, void*
 int hipie_request_start(hipie_request* request, const void* const* inputs, void* const* outputs,
                         int device_memory);
 int hipie_request_wait(hipie_request* request);
+/* Wait(millis_timeout) (ie_infer_async_request_thread_safe_default.hpp:167-204): -1 = RESULT_READY (block; the same
+ * as hipie_request_wait), 0 = STATUS_ONLY (ask, do not wait), > 0 = wait at most that many milliseconds.
+ * HIPIE_RESULT_NOT_READY: still running, the request stays busy; HIPIE_INFER_NOT_STARTED: nothing was started;
+ * HIPIE_INFER_CANCELLED: the inference was cancelled (below), the request is idle again. */
+int hipie_request_wait_for(hipie_request* request, int64_t timeout_ms);
+/* Cancel (ie_infer_async_request_thread_safe_default.hpp:255-267).  Work that is queued on the request's stream runs
+ * to its end (nothing on the device is revoked); the outputs are undefined and the next wait gives
+ * HIPIE_INFER_CANCELLED.  On an idle request it does nothing. */
+int hipie_request_cancel(hipie_request* request);
 /* enqueue the kernels only, on the request's stream, without copies or synchronisation */
 int hipie_request_enqueue(hipie_request* request, const void* const* inputs, void* const* outputs);
 int hipie_request_stream(hipie_request* request, void** stream);
@@ -475,7 +510,12 @@ int hipie_request_tensor(const hipie_request* request, int node_id, hipie_tensor
  *      include/low_precision/layer_transformation.hpp:63-107   DataPrecision::getMin/MaxValue
  *      src/network_helper.cpp:943-1087               decomposeFakeQuantize (scale, shift, clamp)
  *      src/network_helper.cpp:700-827                foldFakeQuantize (i8 weights)
+ *      src/network_helper.cpp:216-292                swapMultiplyAndAdd (bias in front of the dequantization)
+ *      src/fake_quantize.cpp:127-183                 fuseElementwise (dequantization folded into the next range)
+ *      src/add.cpp:154-218                           AddTransformation, dequantizations on both branches
+ *      src/clamp.cpp:71-89                           Clamp bounds in front of a per-tensor dequantization
  * ==================================================================================== */
+enum { HIPIE_LPT_MULTIPLY = 1, HIPIE_LPT_SUBTRACT = 2, HIPIE_LPT_ADD = 3 };
 int hipie_lpt_precision_details(int64_t levels, const float* out_low, const float* out_high, int64_t n,
                                 int* precision, int* has_negative, int* has_zero_point);
 int hipie_lpt_data_precision_range(int precision, int64_t levels, float* min, float* max);
@@ -486,6 +526,14 @@ int hipie_lpt_fold_fake_quantize(const float* values, int64_t oc, int64_t inner,
                                  int64_t n_in_low, const float* in_high, int64_t n_in_high,
                                  const float* out_low, int64_t n_out_low, const float* out_high,
                                  int64_t n_out_high, int64_t levels, int round_values, float* out);
+
+int hipie_lpt_swap_multiply_and_add(const float* b, int64_t n_b, const float* a, int64_t n_a, float* b_over_a, int64_t n);
+int hipie_lpt_fuse_elementwise(int kind, const float* in_low, const float* in_high, int64_t n_range, const float* value,
+                               int64_t n_value, float* new_low, float* new_high, int64_t n, int* fused);
+int hipie_lpt_add_both_branches(const float* shift_full, const float* scale_full, const float* shift_empty,
+                                const float* scale_empty, int64_t n, float* new_shift_full, float* new_scale_full,
+                                float* scale_after);
+int hipie_lpt_clamp_bounds(double min, double max, double scale, double shift, double* new_min, double* new_max);
 
 #ifdef __cplusplus
 }

@@ -78,10 +78,11 @@ def test_conv_variant_numbers_are_checked_without_a_device():
     the first-layer and row-tile kernels on geometries they do not take"""
     from dldt_amd import HipieError
     long_k = _host_conv(256, 64, 3)            # 36 K steps of 64 bytes
-    for tile in (0, 4, 12, 14, 15, 16, 17):
+    for tile in (0, 4, 12, 14, 15, 16, 17, 18, 19, 20, 21, 22):
         long_k.set_tile(tile)
-    short_k = _host_conv(64, 64, 1)            # one K step
-    for tile in (18, -1, 12, 13, 14, 17):
+    short_k = _host_conv(64, 64, 1)            # one K step of 64 bytes: no 128-byte K steps either
+    short_k.set_tile(22)
+    for tile in (23, -1, 12, 13, 14, 17, 18, 21):
         with pytest.raises(HipieError) as e:
             short_k.set_tile(tile)
         assert e.value.status == -4, tile      # PARAMETER_MISMATCH
@@ -96,3 +97,104 @@ def test_epilogue_rejects_an_inverted_clamp_range():
     with pytest.raises(HipieError) as e:
         _host_conv(32, 32, 1, make_epilogue(activation="clamp", clamp=(6.0, 0.0), out_dtype=41, fq=fq))
     assert e.value.status == -4
+
+
+# ---- plugin-level surface: config map, metrics, QueryNetwork, request status paths (no device needed) ----
+def _tiny_graph(extra_relu=False):
+    """FakeQuantize -> 1x1 convolution -> bias -> FakeQuantize -> dequantization; optionally two stray Relu nodes"""
+    from dldt_amd.graph import Graph
+    from dldt_amd.tensor import F32, I8, U8
+    g = Graph()
+    x = g.parameter("x", (1, 16, 4, 4))
+    q = g.fake_quantize(x, 0.0, 2.55, 0.0, 255.0, 256, out_dtype=U8)
+    w = g.constant(np.ones((16, 16, 1, 1), np.int8), I8)
+    y = g.add(g.convolution(q, w), g.constant(np.zeros((1, 16, 1, 1), np.float32)))
+    q2 = g.fake_quantize(y, 0.0, 255.0, 0.0, 255.0, 256, out_dtype=U8)
+    out = g.multiply(g.convert(q2, F32), g.constant(np.float32(0.01).reshape(1, 1, 1, 1)))
+    ids = dict(x=x, q=q, conv=y, q2=q2, out=out)
+    if extra_relu:
+        ids["relu_a"] = g.relu(x)                       # a Relu no convolution absorbs: not planned
+        ids["relu_b"] = g.relu(g.multiply(x, g.constant(np.float32(2).reshape(1, 1, 1, 1))))
+        g.result(ids["relu_a"], "a")
+        g.result(ids["relu_b"], "b")
+    g.result(out, "y")
+    return g, ids
+
+
+def test_compile_options_and_their_status_codes():
+    g, _ = _tiny_graph()
+    plan = g.compile(-1, config={"PERF_COUNT": "YES", "HIP_THROUGHPUT_STREAMS": "5", "HIP_TUNE": "NO"})
+    assert plan.config("PERF_COUNT") == "YES" and plan.config("HIP_THROUGHPUT_STREAMS") == "5" and plan.config("HIP_TUNE") == "NO"
+    assert plan.metric("OPTIMAL_NUMBER_OF_INFER_REQUESTS") == "5"          # what benchmark_app asks the network for
+    assert "OPTIMAL_NUMBER_OF_INFER_REQUESTS" in plan.metric("SUPPORTED_METRICS").split()
+    assert "HIP_THROUGHPUT_STREAMS" in plan.metric("SUPPORTED_CONFIG_KEYS").split()
+    assert g.compile(-1, config={"HIP_THROUGHPUT_STREAMS": "HIP_THROUGHPUT_AUTO"}).metric("OPTIMAL_NUMBER_OF_INFER_REQUESTS") == "3"
+    assert g.compile(-1, config={}).config("PERF_COUNT") == "NO"
+    with pytest.raises(HipieError) as e:                                       # unknown key: NOT_FOUND
+        g.compile(-1, config={"CPU_THREADS_NUM": "4"})
+    assert e.value.status == -5 and "CPU_THREADS_NUM" in str(e.value)
+    for key, value in (("PERF_COUNT", "maybe"), ("HIP_THROUGHPUT_STREAMS", "0"), ("HIP_THROUGHPUT_STREAMS", "many"),
+                       ("DEVICE_ID", "x")):
+        with pytest.raises(HipieError) as e:                                   # a value the key does not take
+            g.compile(-1, config={key: value})
+        assert e.value.status == -4, (key, value)
+    with pytest.raises(HipieError) as e:
+        plan.metric("NO_SUCH_METRIC")
+    assert e.value.status == -5
+    with pytest.raises(HipieError) as e:
+        plan.config("NO_SUCH_KEY")
+    assert e.value.status == -5
+
+
+def test_environment_variables_are_only_defaults(monkeypatch):
+    g, _ = _tiny_graph()
+    monkeypatch.setenv("HIPIE_TUNE_STREAMS", "2")
+    monkeypatch.setenv("HIPIE_KEEP_F32", "1")
+    plan = g.compile(-1, config={})
+    assert plan.config("HIP_THROUGHPUT_STREAMS") == "2" and plan.config("HIP_KEEP_F32") == "YES"
+    plan = g.compile(-1, config={"HIP_THROUGHPUT_STREAMS": "4", "HIP_KEEP_F32": "NO"})
+    assert plan.config("HIP_THROUGHPUT_STREAMS") == "4" and plan.config("HIP_KEEP_F32") == "NO"
+
+
+def test_device_metrics():
+    import ctypes
+    lib = dldt_amd.lib()
+
+    def metric(name, cap=1024):
+        buf = ctypes.create_string_buffer(cap)
+        st = lib.hipie_get_metric(0, name.encode(), buf, ctypes.c_size_t(cap))
+        return st, buf.value.decode()
+
+    st, names = metric("SUPPORTED_METRICS")
+    assert st == 0
+    for name in ("AVAILABLE_DEVICES", "OPTIMIZATION_CAPABILITIES", "RANGE_FOR_ASYNC_INFER_REQUESTS", "IMPORT_EXPORT_SUPPORT",
+                 "DEVICE_ARCHITECTURE", "SUPPORTED_CONFIG_KEYS"):
+        assert name in names.split()
+    assert metric("OPTIMIZATION_CAPABILITIES") == (0, "INT8 FP32")
+    assert metric("IMPORT_EXPORT_SUPPORT") == (0, "YES")
+    assert metric("DEVICE_ARCHITECTURE") == (0, "gfx950")
+    assert metric("RANGE_FOR_ASYNC_INFER_REQUESTS")[1].split() == ["1", "8", "1"]
+    assert metric("NO_SUCH_METRIC")[0] == -5
+    assert metric("SUPPORTED_METRICS", cap=8)[0] == -6                          # buffer too small: OUT_OF_BOUNDS
+
+
+def test_query_reports_every_unsupported_node():
+    g, ids = _tiny_graph(extra_relu=True)
+    with pytest.raises(HipieError) as e:                                       # compiling stops at the first one ...
+        g.compile(-1)
+    assert e.value.status == -2
+    ok = g.query()                                                             # ... the query names them all
+    assert len(ok) == len(g.nodes)
+    assert not ok[ids["relu_a"]] and not ok[ids["relu_b"]]
+    for name in ("x", "q", "conv", "q2", "out"):
+        assert ok[ids[name]], name
+    g2, ids2 = _tiny_graph()
+    assert all(g2.query())
+
+
+def test_request_entry_points_reject_null_handles():
+    import ctypes
+    lib = dldt_amd.lib()
+    assert lib.hipie_request_wait_for(None, ctypes.c_int64(0)) == -4
+    assert lib.hipie_request_cancel(None) == -4
+    assert lib.hipie_request_wait(None) == -4

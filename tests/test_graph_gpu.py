@@ -313,3 +313,50 @@ def test_full_size_batch_64(orc, net):
         want, _ = evaluate(orc, g1.nodes, {"data": x[i:i + 1]}, keep=[])
         np.testing.assert_array_equal(y64[i:i + 1].view(np.uint32), want["logits"].view(np.uint32), err_msg="image %d" % i)
         assert y64[i].argmax() == want["logits"][0].argmax()
+
+
+def test_timed_wait_status_only_and_cancel():
+    """Wait(ms) and Cancel of the asynchronous request (ie_infer_async_request_thread_safe_default.hpp:167-204, 255-267):
+    STATUS_ONLY on a running inference says RESULT_NOT_READY and leaves it running, a timed wait returns the result, a
+    cancelled inference reports INFER_CANCELLED once and leaves the request idle and usable."""
+    from dldt_amd import HipieError, builders
+    g, _ = builders.resnet50(batch=64, res=224)
+    plan = g.compile(config={"HIP_TUNE": "NO", "PERF_COUNT": "YES"})
+    assert plan.config("PERF_COUNT") == "YES"
+    x = np.random.default_rng(21).uniform(0, 1, (64, 3, 224, 224)).astype(np.float32)
+    (want,) = plan.create_request().infer(x)
+    req = plan.create_request(perf_count=None)            # the plan's PERF_COUNT
+    ins, outs = req.host_buffers()
+    ins[0].array[...] = x
+    with pytest.raises(HipieError) as e:                  # idle: INFER_NOT_STARTED
+        req.wait_for(0)
+    assert e.value.status == -11
+    req.start(ins, outs)
+    not_ready = 0
+    while True:                                           # STATUS_ONLY until it is done
+        try:
+            req.wait_for(0)
+            break
+        except HipieError as err:
+            assert err.status == -9
+            not_ready += 1
+    assert not_ready > 0                                  # 38 MB over the host link and 54 kernels were not done at once
+    np.testing.assert_array_equal(outs[0].array.view(np.uint32), want.view(np.uint32))
+    assert sum(s["ms"] for s in req.perf()) > 0           # the per-step counters of PERF_COUNT = YES
+    outs[0].array[...] = 0
+    req.start(ins, outs)
+    req.wait_for(60000)
+    np.testing.assert_array_equal(outs[0].array.view(np.uint32), want.view(np.uint32))
+    req.start(ins, outs)
+    req.cancel()
+    with pytest.raises(HipieError) as e:
+        req.wait()
+    assert e.value.status == -13                          # INFER_CANCELLED, after the queued work has drained
+    with pytest.raises(HipieError) as e:                  # idle again
+        req.wait()
+    assert e.value.status == -11
+    req.cancel()                                          # nothing to cancel: no effect
+    outs[0].array[...] = 0
+    req.start(ins, outs)
+    req.wait()
+    np.testing.assert_array_equal(outs[0].array.view(np.uint32), want.view(np.uint32))

@@ -185,3 +185,58 @@ def test_planner_takes_integer_zero_points():
     with pytest.raises(HipieError) as e:
         Plan(bad, device=-1)
     assert e.value.status == -2 and "zero point" in str(e.value)
+
+
+@pytest.mark.parametrize("case", G["fuse_elementwise"]["cases"], ids=lambda c: c["name"].split(" (")[0])
+def test_fuse_elementwise_golden(case):
+    """FakeQuantizeTransformation::fuseElementwise against the ranges the reference's own test expects: the operations
+    are absorbed one at a time, the one next to the FakeQuantize first"""
+    kinds = {"multiply": lpt.MULTIPLY, "subtract": lpt.SUBTRACT, "add": lpt.ADD}
+    lo = np.float32(G["fuse_elementwise"]["in_low"])
+    hi = np.float32(G["fuse_elementwise"]["in_high"])
+    got = (np.atleast_1d(lo), np.atleast_1d(hi))
+    for kind, value in case["steps"]:
+        got = lpt.fuse_elementwise(kinds[kind], got[0], got[1], np.array(value, np.float32))
+        if got is None:
+            break
+    if case["new_low"] is None:
+        assert got is None
+    else:
+        np.testing.assert_allclose(got[0], case["new_low"], rtol=1e-6, atol=1e-5)
+        np.testing.assert_allclose(got[1], case["new_high"], rtol=1e-6, atol=1e-5)
+
+
+@pytest.mark.parametrize("case", G["add_both_branches"]["cases"], ids=lambda c: c["at"].split(" ")[0])
+def test_add_transformation_golden(case):
+    sh, sc, after = lpt.add_both_branches(case["full"][0], case["full"][1], case["empty"][0], case["empty"][1])
+    np.testing.assert_allclose([sh[0], sc[0]], case["new_full"], rtol=1e-6)
+    assert after[0] == np.float32(case["after"])
+
+
+def test_swap_multiply_and_add_guard_and_broadcast():
+    """bi / ai per element with either side broadcast, and 0 where both are 0 (network_helper.cpp:245-258); the
+    reference's tests hold no literal for this step: it is one IEEE division per element"""
+    b = np.array([1.0, 0.0, -3.0, 0.0], np.float32)
+    a = np.array([4.0, 0.0, 0.5, 2.0], np.float32)
+    got = lpt.swap_multiply_and_add(b, a)
+    np.testing.assert_array_equal(got, np.array([0.25, 0.0, -6.0, 0.0], np.float32))
+    np.testing.assert_array_equal(lpt.swap_multiply_and_add(np.float32(3), a[[0, 2, 3]]), np.float32(3) / a[[0, 2, 3]])
+    np.testing.assert_array_equal(lpt.swap_multiply_and_add(b, np.float32(0.1)), b / np.float32(0.1))
+
+
+def test_clamp_bounds_move_in_front_of_the_dequantization():
+    """clamp.cpp:71-89: bounds divided by the scale (swapped for a negative one), then shifted; ReLU6 behind a
+    per-tensor scale of 0.02 clamps the levels at 0 .. 300"""
+    assert lpt.clamp_bounds(0.0, 6.0, 0.02) == (0.0, 6.0 / 0.02)
+    assert lpt.clamp_bounds(0.0, 10.0, 3.0, 128.0) == (128.0, 10.0 / 3.0 + 128.0)
+    assert lpt.clamp_bounds(0.0, 10.0, -5.0, 128.0) == (10.0 / -5.0 + 128.0, 128.0)
+
+
+def test_builders_derive_their_constants_through_these_steps():
+    """the post-LPT graphs of the benchmark configurations take b / s and il / s, ih / s from the pinned entry points"""
+    import inspect
+    from dldt_amd import builders
+    src = inspect.getsource(builders)
+    assert "lpt.swap_multiply_and_add" in src and "lpt.fuse_elementwise" in src
+    code = "\n".join(l.split("#")[0] for l in src.splitlines() if '"""' not in l)
+    assert "b / s)" not in code and "/ s_x)" not in code and "/ s)" not in code
