@@ -25,7 +25,14 @@ struct Epilogue {
 void launch_line(const ConvArgs& a, int shape, hipStream_t s);
 int line_row_bytes(int shape);
 
-void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipStream_t s);
+// depthwise kernels (dwconv.hip).  variant 0: a lane computes its outputs from registers loaded straight from memory;
+// variant 1: 3 x 3 through an LDS patch with the window sliding in registers (dwconv_strip_fits says which layers)
+struct DwGeometry {
+    int in_h, in_w, halo;     // interior size of the input tensor and its readable border
+    int pad_top, pad_left;
+};
+bool dwconv_strip_fits(int KH, int KW, int dil_h, int dil_w, int stride_h, int stride_w, int in_c_stride, uint32_t flags);
+void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, int variant, const DwGeometry& g, hipStream_t s);
 
 // frees the split-K workspace kept for this stream, if any (for the owner of a stream, before it destroys
 // the stream and after the stream's work has finished)

@@ -1663,7 +1663,14 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
         HIPIE_REQUIRE(c && tile >= 0 && tile <= 22, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
-        if (c->depthwise) return;               // one kernel only
+        if (c->depthwise) {   // 0: registers only, 1: 3 x 3 through an LDS patch
+            HIPIE_REQUIRE(tile == 0 || (tile == 1 && !(c->epi.flags & CF_RES) &&
+                                        dwconv_strip_fits(c->d.kh, c->d.kw, c->d.dil_h, c->d.dil_w, c->d.stride_h, c->d.stride_w,
+                                                          c->d.in_c_stride, c->epi.flags)),
+                          HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: depthwise variant %d does not take this layer", tile);
+            c->tile = tile;
+            return;
+        }
         if (c->fused && tile != 0) return;      // the second GEMM exists in the 128 x 128 tiled kernel
         HIPIE_REQUIRE(tile < 8 || tile > 9 || (!c->fused && persist_available(c->epi.flags)), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the persistent kernels exist for byte outputs with a byte residual or none");
@@ -1687,7 +1694,7 @@ int hipie_conv_set_tile(hipie_conv* c, int tile) {
 int hipie_conv_get_tile(const hipie_conv* c, int* tile) {
     return guarded([&] {
         HIPIE_REQUIRE(c && tile, HIPIE_PARAMETER_MISMATCH, "hipie_conv_get_tile: null argument");
-        *tile = c->depthwise ? -1 : c->tile;
+        *tile = c->tile;
     });
 }
 
@@ -1840,7 +1847,8 @@ static int conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_ten
             HIPIE_REQUIRE(in->stride_w >= d.ic && in->stride_w % 16 == 0, HIPIE_PARAMETER_MISMATCH,
                           "hipie_conv_run: depthwise input channel stride");
             DeviceGuard g(c->device);
-            launch_dwconv(a, d.kh, d.kw, d.dil_h, d.dil_w, as_stream(stream));
+            const DwGeometry geo{in->h, in->w, in->halo, d.pad_top, d.pad_left};
+            launch_dwconv(a, d.kh, d.kw, d.dil_h, d.dil_w, c->tile, geo, as_stream(stream));
             HIPIE_CHECK_HIP(hipGetLastError());
             return;
         }

@@ -169,6 +169,173 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cg
     epilogue<F, 1>(a, acc, oc_lane, valid, out_off, res_off, none, nullptr, 0, 0);
 }
 
+
+// 3x3, dilation 1, stride 1 or 2, through LDS: a workgroup stages the input rows under R output rows of a strip of
+// columns (all channels, halo included) in LDS once, with 16-byte loads of whole pixels.  A lane owns FOUR channels
+// (one dword of a pixel) of four horizontally adjacent output pixels and walks down the R output rows: every input
+// row is read from LDS once per lane (6 dwords at stride 1, 9 at stride 2), transposed once (v_perm_b32) into one
+// dword per channel holding four consecutive pixels, and used for all three filter rows it belongs to, so the
+// 3 x 3 window slides in registers in both directions.  Per output: 4 VALU instructions of multiply work at stride 1
+// (7 at stride 2) plus the epilogue's 7 or 8; address arithmetic is per lane and per row, not per output.
+struct DwStrip {
+    int32_t cpb;              // dwords (groups of four channels) per pixel = in_sw / 4
+    float inv_cpb;
+    int32_t strips;           // strips of four output columns per workgroup
+    int32_t col_tiles, row_tiles;
+    int32_t cols_in;          // input columns staged per workgroup
+    int32_t pad_top, pad_left;
+    int32_t in_h_end, in_w_end;   // one past the last readable input row / column (interior + halo)
+    int32_t OH;
+    int32_t cgroups_out;      // groups of four channels that exist in the output tensor
+    int64_t tiles;
+    int32_t per_xcd;
+};
+
+constexpr int kDwRows = 7;    // output rows per workgroup: 7, 14, 28, 56, 112 are all multiples of it
+
+template <uint32_t F, int STRIDE>
+__global__ __launch_bounds__(256) void dwconv3x3_lds_kernel(const ConvArgs a, const DwStrip t) {
+    constexpr int R = kDwRows, ROWS_IN = (R - 1) * STRIDE + 3, NPX = 3 * STRIDE + 3;
+    extern __shared__ __attribute__((aligned(16))) int8_t patch[];
+    const int64_t wg = workgroup_index(t.per_xcd);
+    if (wg >= t.tiles) return;                        // whole workgroup, before the barrier
+    const int col_tile = static_cast<int>(wg % t.col_tiles);
+    const int64_t rest = wg / t.col_tiles;
+    const int row_tile = static_cast<int>(rest % t.row_tiles), n = static_cast<int>(rest / t.row_tiles);
+    const int oh0 = row_tile * R, ow0 = col_tile * 4 * t.strips;
+    const int ih0 = oh0 * STRIDE - t.pad_top, iw0 = ow0 * STRIDE - t.pad_left;
+    const int tid = threadIdx.x, nt = blockDim.x;
+
+    // ---- stage: rows_eff x cols_eff whole pixels, each row one contiguous run in memory and in LDS
+    // (holding the loads of the lower rows in registers until the first output rows are done was slower: the 32
+    // registers cost more occupancy than the overlap returned)
+    const int rows_eff = min(ROWS_IN, t.in_h_end - ih0), cols_eff = min(t.cols_in, t.in_w_end - iw0);
+    const int chunks_row = cols_eff * (a.in_sw >> 4), total = rows_eff * chunks_row;
+    const float inv_chunks_row = 1.0f / static_cast<float>(chunks_row);
+    const int8_t* const src = a.in + (static_cast<int64_t>(n) * a.in_sn + static_cast<int64_t>(ih0) * a.in_sh +
+                                      static_cast<int64_t>(iw0) * a.in_sw);
+    const int lds_row = t.cols_in * a.in_sw;
+    constexpr int NJ = 8;                             // loads in flight per thread and round
+    for (int base = 0; base < total; base += NJ * nt) {
+        uint4 v[NJ];
+        int dst[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int idx = base + j * nt + tid;
+            int row, ch;
+            fast_divmod(min(idx, total - 1), chunks_row, inv_chunks_row, row, ch);
+            dst[j] = idx < total ? row * lds_row + ch * 16 : -1;
+            v[j] = *reinterpret_cast<const uint4*>(src + static_cast<int64_t>(row) * a.in_sh + ch * 16);
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            if (dst[j] >= 0) *reinterpret_cast<uint4*>(patch + dst[j]) = v[j];
+    }
+
+    // ---- lane role
+    int strip, cg;
+    fast_divmod(tid, t.cpb, t.inv_cpb, strip, cg);
+    const bool lane_on = strip < t.strips;
+    if (!lane_on) { strip = 0; cg = 0; }
+    const int oc = 4 * cg;
+    uint32_t w[3][4], ws[3][4];                       // (w0, w1, w2, 0) of a filter row and the same one byte up
+#pragma unroll
+    for (int kh = 0; kh < 3; ++kh) {
+        const uint4 q = *reinterpret_cast<const uint4*>(a.wgt2 + (static_cast<int64_t>(kh) * a.OCp + oc) * 4);
+        w[kh][0] = q.x; w[kh][1] = q.y; w[kh][2] = q.z; w[kh][3] = q.w;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) ws[kh][c] = w[kh][c] << 8;
+    }
+    const int4 corr = *reinterpret_cast<const int4*>(a.corr + oc);
+    const int corr_[4] = {corr.x, corr.y, corr.z, corr.w};
+    float bias_[4], scale_[4], ih_[4], r_[4], r2_[4];
+    f4_to_array(ld4f(a.bias + oc), bias_);
+    if (F & CF_SCALE) f4_to_array(ld4f(a.scale + oc), scale_);
+    f4_to_array(ld4f(a.fq_ih + oc), ih_);
+    f4_to_array(ld4f(a.fq_r + oc), r_);
+    f4_to_array(ld4f(a.fq_r2 + oc), r2_);
+    const uint32_t xmask = (a.flags & CF_OUT_XOR) ? 0x80808080u : 0u;
+    const int ow_lane = ow0 + 4 * strip;
+    const bool store_on = lane_on && cg < t.cgroups_out;
+    int8_t* const out_lane = static_cast<int8_t*>(a.out) + (static_cast<int64_t>(n) * a.out_sn + static_cast<int64_t>(ow_lane) * a.out_sw + oc);
+
+    __syncthreads();
+
+    int acc[3][4][4];                                 // [output row mod 3][pixel][channel]
+#pragma unroll
+    for (int s = 0; s < 3; ++s)
+#pragma unroll
+        for (int px = 0; px < 4; ++px)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[s][px][c] = corr_[c];
+
+    auto transpose4 = [&](uint32_t p0, uint32_t p1, uint32_t p2, uint32_t p3, uint32_t (&o)[4]) {
+        const uint32_t lo01 = __builtin_amdgcn_perm(p1, p0, 0x05010400u), hi01 = __builtin_amdgcn_perm(p1, p0, 0x07030602u);
+        const uint32_t lo23 = __builtin_amdgcn_perm(p3, p2, 0x05010400u), hi23 = __builtin_amdgcn_perm(p3, p2, 0x07030602u);
+        o[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+        o[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+        o[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+        o[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+    };
+    const int8_t* lds_lane = patch + (4 * strip * STRIDE) * a.in_sw + oc;
+#pragma unroll
+    for (int i = 0; i < ROWS_IN; ++i) {
+        uint32_t p[NPX];
+#pragma unroll
+        for (int j = 0; j < NPX; ++j) p[j] = *reinterpret_cast<const uint32_t*>(lds_lane + i * lds_row + j * a.in_sw);
+        // T[g][c]: channel c of the four pixels under output pixel pair / pixel g
+        uint32_t T[STRIDE == 1 ? 2 : 4][4];
+        if (STRIDE == 1) {
+            transpose4(p[0], p[1], p[2], p[3], T[0]);
+            transpose4(p[2], p[3], p[4], p[5], T[1]);
+        } else {
+            transpose4(p[0], p[1], p[2], p[3], T[0]);
+            transpose4(p[2], p[3], p[4], p[5], T[1]);
+            transpose4(p[4], p[5], p[6], p[7], T[2]);
+            transpose4(p[6], p[7], p[8], p[8], T[3]);
+        }
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh) {
+            if ((i - kh) % STRIDE != 0 || i - kh < 0 || (i - kh) / STRIDE >= R) continue;
+            const int s = ((i - kh) / STRIDE) % 3;
+#pragma unroll
+            for (int px = 0; px < 4; ++px)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const uint32_t x = STRIDE == 1 ? T[px >> 1][c] : T[px][c];
+                    const uint32_t wv = (STRIDE == 1 && (px & 1)) ? ws[kh][c] : w[kh][c];
+                    acc[s][px][c] = __builtin_amdgcn_sdot4(static_cast<int>(x), static_cast<int>(wv), acc[s][px][c], false);
+                }
+        }
+        // output row r is complete behind input row r * STRIDE + 2
+        if (i >= 2 && (i - 2) % STRIDE == 0 && (i - 2) / STRIDE < R) {
+            const int r = (i - 2) / STRIDE, s = r % 3;
+            const int oh = oh0 + r;
+            uint32_t packed[4];
+#pragma unroll
+            for (int px = 0; px < 4; ++px) {
+                packed[px] = 0;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float x = static_cast<float>(acc[s][px][c]);
+                    x = x + bias_[c];
+                    if (F & CF_SCALE) x = x * scale_[c];
+                    if (F & CF_CLAMP) x = __builtin_amdgcn_fmed3f(x, a.clamp_lo, a.clamp_hi);
+                    const float lv = fq_level_fast<2, true, true>(x, 0.f, ih_[c], ih_[c], r_[c], r2_[c], a.lm1);
+                    packed[px] = __builtin_amdgcn_cvt_pk_u8_f32(lv, c, packed[px]);
+                    acc[s][px][c] = corr_[c];
+                }
+            }
+            if (store_on && oh < t.OH) {
+                int8_t* const o = out_lane + static_cast<int64_t>(oh) * a.out_sh;
+#pragma unroll
+                for (int px = 0; px < 4; ++px)
+                    if (ow_lane + px < a.OW) *reinterpret_cast<uint32_t*>(o + px * a.out_sw) = packed[px] ^ xmask;
+            }
+        }
+    }
+}
+
 }  // namespace
 
 // grid of a launch of `workgroups` workgroups: XCD-contiguous order from 64 workgroups up (8 per XCD), the
@@ -182,9 +349,75 @@ struct XcdGrid {
     }
 };
 
-void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, hipStream_t s) {
+// the LDS strip kernel takes 3 x 3, undilated, stride 1 or 2 (the same both ways) with one of the specialised epilogues,
+// pixels of at most 1024 bytes (a lane per four channels, at most 256 lanes) and no residual
+bool dwconv_strip_fits(int KH, int KW, int dil_h, int dil_w, int stride_h, int stride_w, int in_c_stride, uint32_t flags) {
+    const uint32_t core = flags & ~CF_OUT_XOR;
+    const bool known = core == E_PLAIN0 || core == E_CLAMPFQ || core == E_SCALEFQ0;
+    return KH == 3 && KW == 3 && dil_h == 1 && dil_w == 1 && stride_h == stride_w && (stride_h == 1 || stride_h == 2) && known &&
+           in_c_stride % 16 == 0 && in_c_stride <= 1024;
+}
+
+static void launch_dwconv_strip(const ConvArgs& a, const DwGeometry& g, hipStream_t s) {
+    const int stride = a.conv_sh;
+    DwStrip t;
+    t.cpb = a.in_sw / 4;
+    t.inv_cpb = 1.0f / static_cast<float>(t.cpb);
+    const int OH = a.OHOW / a.OW;
+    const int rows_in = (kDwRows - 1) * stride + 3;
+    // as many strips as fit 256 lanes, the row's width and 48 KB of LDS (three workgroups per compute unit)
+    int strips = std::max(1, 256 / t.cpb);
+    strips = std::min(strips, static_cast<int>(ceil_div(a.OW, 4)));
+    // (measured from 12 to 64 KB on the MobileNetV2 layers: smaller patches lose more to halo columns and idle lanes
+    // than the extra workgroups per compute unit return)
+    while (strips > 1 && static_cast<int64_t>(rows_in) * ((4 * strips - 1) * stride + 3) * a.in_sw > 48 * 1024) --strips;
+    t.strips = strips;
+    t.cols_in = (4 * strips - 1) * stride + 3;
+    t.col_tiles = static_cast<int>(ceil_div(a.OW, 4 * strips));
+    t.row_tiles = static_cast<int>(ceil_div(OH, kDwRows));
+    t.pad_top = g.pad_top;
+    t.pad_left = g.pad_left;
+    t.in_h_end = g.in_h + g.halo;
+    t.in_w_end = g.in_w + g.halo;
+    t.OH = OH;
+    t.cgroups_out = std::min(a.out_sw, a.in_sw) / 4;
+    t.tiles = static_cast<int64_t>(a.M / a.OHOW) * t.row_tiles * t.col_tiles;
+    const XcdGrid xg(t.tiles);
+    t.per_xcd = xg.per_xcd;
+    const size_t lds = static_cast<size_t>(rows_in) * t.cols_in * a.in_sw;
+    const int threads = static_cast<int>(round_up(strips * t.cpb, 64));
+    HIPIE_REQUIRE(lds <= 160 * 1024, HIPIE_GENERAL_ERROR, "depthwise strip kernel: %zu bytes of LDS", lds);
+    const dim3 grid(xg.blocks), block(static_cast<uint32_t>(threads));
+    const uint32_t core = a.flags & ~CF_OUT_XOR;
+#define HIPIE_LAUNCH_DWS(FLAGS, STRIDE)                                                                                     \
+    do {                                                                                                                    \
+        static bool attr_set = false;                                                                                       \
+        if (!attr_set) {                                                                                                    \
+            HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&dwconv3x3_lds_kernel<FLAGS, STRIDE>),         \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));                   \
+            attr_set = true;                                                                                                \
+        }                                                                                                                   \
+        hipLaunchKernelGGL((dwconv3x3_lds_kernel<FLAGS, STRIDE>), grid, block, lds, s, a, t);                               \
+    } while (0)
+    if (core == E_PLAIN0) {
+        if (stride == 1) HIPIE_LAUNCH_DWS(E_PLAIN0, 1); else HIPIE_LAUNCH_DWS(E_PLAIN0, 2);
+    } else if (core == E_SCALEFQ0) {
+        if (stride == 1) HIPIE_LAUNCH_DWS(E_SCALEFQ0, 1); else HIPIE_LAUNCH_DWS(E_SCALEFQ0, 2);
+    } else {
+        if (stride == 1) HIPIE_LAUNCH_DWS(E_CLAMPFQ, 1); else HIPIE_LAUNCH_DWS(E_CLAMPFQ, 2);
+    }
+#undef HIPIE_LAUNCH_DWS
+}
+
+void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, int variant, const DwGeometry& g, hipStream_t s) {
     const uint32_t core = a.flags & ~CF_OUT_XOR;
     const bool known = core == E_PLAIN0 || core == E_CLAMPFQ || core == E_SCALEFQ0;
+    if (variant == 1) {
+        HIPIE_REQUIRE(dwconv_strip_fits(KH, KW, dil_h, dil_w, a.conv_sh, a.conv_sw, a.in_sw, a.flags) && !(a.flags & CF_RES),
+                      HIPIE_GENERAL_ERROR, "depthwise strip kernel chosen for a layer it does not take");
+        launch_dwconv_strip(a, g, s);
+        return;
+    }
     if (KH == 3 && KW == 3 && dil_h == 1 && dil_w == 1 && a.conv_sh == a.conv_sw && (a.conv_sh == 1 || a.conv_sh == 2) &&
         known && !(a.flags & CF_RES)) {
         const int cgroups = std::min(a.OCp, a.in_sw) / 16;   // groups of 16 channels that exist in the tensors

@@ -250,7 +250,7 @@ struct ConvStep : Step {
         if (shortcut && !fused) shortcut->tune(lanes, tensors);
         int current = -1;
         check_status(hipie_conv_get_tile(conv, &current), name.c_str());
-        if (current < 0) return;   // depthwise: one kernel
+        if (current < 0) return;
         const size_t nl = lanes.size();
         std::vector<hipie_tensor> ti(nl), to(nl), tr(nl);
         for (size_t l = 0; l < nl; ++l) {

@@ -152,19 +152,25 @@ def config4():
     r["images/s"] = 64 / us3 * 1e6
     rows.append(r)
     rng = np.random.default_rng(4)
-    for c, hw, stride in ((96, 112, 2), (384, 14, 1), (960, 7, 1)):
+    # every distinct depthwise layer of MobileNetV2 with its own tail (bias, scale, ReLU6, FakeQuantize(0, 6)),
+    # both kernel variants: 0 = from registers, 1 = through an LDS patch with the window sliding in registers
+    for c, hw, stride in ((32, 112, 1), (96, 112, 2), (144, 56, 1), (144, 56, 2), (192, 28, 1), (192, 28, 2), (384, 14, 1),
+                          (576, 14, 1), (576, 14, 2), (960, 7, 1)):
         cs = -(-c // 16) * 16
         xin = DeviceTensor(64, hw, hw, c, U8B, halo=1)
         xin.interior().copy_(torch.randint(-128, 127, xin.interior().shape, dtype=torch.int8, device="cuda"))
         w = rng.integers(-127, 128, (c, 1, 1, 3, 3)).astype(np.int8)
-        fq = (256, 0.0, np.full(c, 3000.0, np.float32), 0.0, 255.0)
+        fq = (256, 0.0, np.float32(6.0), 0.0, 255.0)
         conv = Convolution(w, xin, (stride, stride), (1, 1), (1, 1), (1, 1),
-                           make_epilogue(bias=np.zeros(c, np.float32), out_dtype=U8B, fq=fq))
+                           make_epilogue(bias=np.zeros(c, np.float32), scale=np.full(c, 2e-4, np.float32), activation="clamp",
+                                         clamp=(0.0, 6.0), out_dtype=U8B, fq=fq))
         oh = (hw + 2 - 3) // stride + 1
         out = DeviceTensor(64, oh, oh, c, U8B)
-        rows.append(_row("cfg4 depthwise 3x3 s%d C=%d @%dx%d batch 64" % (stride, c, hw, hw),
-                         _time(lambda: conv.run(xin, out)), macs=64 * oh * oh * c * 9,
-                         bytes_=64 * (hw * hw + oh * oh) * cs + 9 * c, bound="hbm"))
+        for variant in (0, 1):
+            conv.set_tile(variant)
+            rows.append(_row("cfg4 depthwise 3x3 s%d C=%d @%dx%d batch 64, variant %d" % (stride, c, hw, hw, variant),
+                             _time(lambda: conv.run(xin, out)), macs=64 * oh * oh * c * 9,
+                             bytes_=64 * (hw * hw + oh * oh) * cs + 9 * c, bound="hbm"))
     return rows
 
 

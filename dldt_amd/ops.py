@@ -183,6 +183,11 @@ class Convolution:
         check(lib().hipie_conv_set_tile(self._h, tile))
         check(lib().hipie_conv_set_stages(self._h, stages))
 
+    def get_tile(self):
+        t = ctypes.c_int()
+        check(lib().hipie_conv_get_tile(self._h, ctypes.byref(t)))
+        return t.value
+
     def run(self, x, out, residual=None):
         xd, od = x.desc(), out.desc()
         rd = residual.desc() if residual is not None else None

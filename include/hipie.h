@@ -235,7 +235,11 @@ int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* o
  * workspace that the library keeps per (device, stream): it is allocated by the first such launch on a stream
  * (which therefore must not be under graph capture) and kept until the process ends.  A default is chosen
  * from the shape; hipie_compile times the variants on the device and keeps the fastest.  Every
- * variant produces the same bits. */
+ * variant produces the same bits.
+ * A depthwise convolution (group_convolution.hpp:78-144 with one filter per channel) has two variants of its own:
+ * 0 = every lane computes its outputs from registers loaded straight from memory, 1 = the input rows under seven
+ * output rows of a strip of columns are staged once in LDS and a lane slides the 3 x 3 window over them in registers
+ * (3 x 3, undilated, stride 1 or 2, pixels of at most 1024 bytes, FakeQuantize epilogue without residual). */
 int hipie_conv_set_tile(hipie_conv* conv, int tile);
 int hipie_conv_get_tile(const hipie_conv* conv, int* tile);
 /* diagnostics: the epilogue's step flags (conv_kernel.h ConvFlags) and whether a kernel instance with

@@ -317,6 +317,93 @@ def test_depthwise_conv_exact_and_relu6_requantize(orc, C, H, stride):
     np.testing.assert_array_equal(out8.to_nchw(), want)
 
 
+DW_STRIP_GEOMS = [
+    # N, C, H, W, stride, pads_begin, pads_end
+    (2, 144, 56, 56, 1, (1, 1), (1, 1)),      # MobileNetV2 stage shapes
+    (2, 144, 56, 56, 2, (1, 1), (1, 1)),
+    (1, 32, 112, 112, 1, (1, 1), (1, 1)),
+    (1, 96, 112, 112, 2, (1, 1), (1, 1)),
+    (2, 192, 28, 28, 1, (1, 1), (1, 1)),
+    (2, 384, 14, 14, 1, (1, 1), (1, 1)),
+    (2, 576, 14, 14, 2, (1, 1), (1, 1)),
+    (3, 960, 7, 7, 1, (1, 1), (1, 1)),
+    (2, 48, 15, 11, 1, (1, 1), (1, 1)),       # ragged: rows not a multiple of 7, columns not of 4, 3 pixels' worth of lanes idle
+    (2, 80, 9, 13, 2, (0, 0), (1, 1)),        # padding on the far sides only
+    (1, 16, 5, 3, 1, (1, 1), (1, 1)),         # one strip wider than the row
+    (1, 1008, 8, 6, 1, (1, 1), (1, 1)),       # 252 lanes of 256
+]
+
+
+@pytest.mark.parametrize("tail", ["clamp_fq", "scale_fq", "bias_fq"])
+@pytest.mark.parametrize("geo", range(len(DW_STRIP_GEOMS)))
+def test_depthwise_strip_variant_exact(orc, geo, tail):
+    """the depthwise variant that stages its input in LDS and slides the window in registers gives the reference's
+    levels bit for bit, for every FakeQuantize tail the depthwise kernels are specialised for"""
+    from dldt_amd import Convolution, DeviceTensor, make_epilogue
+    N, C, H, W, stride, pb, pe = DW_STRIP_GEOMS[geo]
+    rng = np.random.default_rng(900 + geo)
+    x = rng.integers(0, 256, (N, C, H, W)).astype(np.int32)
+    w = rng.integers(-127, 128, (C, 1, 1, 3, 3)).astype(np.int32)
+    st = (stride, stride)
+    acc = orc.convolution(x, w, st, (1, 1), pb, pe, grouped=True)
+    xin = DeviceTensor.from_nchw(x, U8B, halo=1)
+    _, _, OH, OW = acc.shape
+    bias = rng.normal(0, 3000, C).astype(np.float32)
+    if tail == "clamp_fq":      # the Clamp is narrower than the FakeQuantize's range: it stays in the kernel
+        scale = (rng.uniform(0.5, 2.0, C) * 2e-4).astype(np.float32)
+        fq = (256, 0.0, np.float32(8.0), 0.0, 255.0)
+        kw = dict(bias=bias, scale=scale, activation="clamp", clamp=(0.0, 6.0), fq=fq)
+        want = _chain(orc, acc, bias=bias, scale=scale, act="clamp", clamp=(0.0, 6.0), fq=fq)
+    elif tail == "scale_fq":    # ReLU6 in front of FQ(0, 6): the Clamp is implied by the FakeQuantize
+        scale = (rng.uniform(0.5, 2.0, C) * 2e-4).astype(np.float32)
+        fq = (256, 0.0, np.float32(6.0), 0.0, 255.0)
+        kw = dict(bias=bias, scale=scale, activation="clamp", clamp=(0.0, 6.0), fq=fq)
+        want = _chain(orc, acc, bias=bias, scale=scale, act="clamp", clamp=(0.0, 6.0), fq=fq)
+    else:
+        # per-channel divisors; a divisor without two-operation division constants sends the layer to the general
+        # kernel (no variant 1), so draw until every channel's divisor has them
+        from dldt_amd import HipieError
+        for attempt in range(8):
+            fq = (256, 0.0, rng.uniform(20000.0, 40000.0, C).astype(np.float32), 0.0, 255.0)
+            kw = dict(bias=bias, fq=fq)
+            probe = Convolution(w.astype(np.int8), xin, st, (1, 1), pb, pe, make_epilogue(out_dtype=U8B, **kw))
+            try:
+                probe.set_tile(1)
+                break
+            except HipieError:
+                continue
+        else:
+            pytest.fail("no draw of divisors was accepted")
+        want = _chain(orc, acc, bias=bias, fq=fq)
+    want = want.astype(np.uint8)
+    conv = Convolution(w.astype(np.int8), xin, st, (1, 1), pb, pe, make_epilogue(out_dtype=U8B, **kw))
+    got = {}
+    for variant in (0, 1):
+        conv.set_tile(variant)
+        assert conv.get_tile() == variant
+        out8 = DeviceTensor(N, OH, OW, C, U8B)
+        out8.interior().fill_(77)
+        conv.run(xin, out8)
+        got[variant] = out8.to_nchw()
+    np.testing.assert_array_equal(got[1], want)
+    np.testing.assert_array_equal(got[0], want)
+
+
+def test_depthwise_strip_variant_is_refused_where_it_does_not_apply():
+    from dldt_amd import Convolution, DeviceTensor, HipieError, make_epilogue
+    x = DeviceTensor(1, 9, 9, 32, U8B, halo=2)
+    w5 = np.ones((32, 1, 1, 5, 5), np.int8)
+    conv = Convolution(w5, x, (1, 1), (1, 1), (2, 2), (2, 2))      # raw sums, 5 x 5
+    with pytest.raises(HipieError):
+        conv.set_tile(1)
+    w3 = np.ones((32, 1, 1, 3, 3), np.int8)
+    conv = Convolution(w3, x, (1, 1), (2, 2), (2, 2), (2, 2),
+                       make_epilogue(bias=np.zeros(32, np.float32), out_dtype=U8B, fq=(256, 0.0, np.float32(6.0), 0.0, 255.0)))
+    with pytest.raises(HipieError):
+        conv.set_tile(1)                                            # dilated
+    conv.set_tile(0)
+
+
 @pytest.mark.parametrize("signed,zp", [(False, 0), (False, 37), (False, 255), (True, -128), (True, 5)])
 @pytest.mark.parametrize("depthwise", [False, True])
 def test_conv_input_zero_point(orc, signed, zp, depthwise):

@@ -14,7 +14,8 @@ def _per_channel_case(rng, N, C, H, W):
     return x, (m - 3 * s).astype(np.float32), (m + 3 * s).astype(np.float32)
 
 
-@pytest.mark.parametrize("shape", [(2, 16, 14, 14), (3, 5, 7, 9), (1, 64, 56, 56), (2, 256, 8, 8)])
+@pytest.mark.parametrize("shape", [(2, 16, 14, 14), (3, 5, 7, 9), (1, 64, 56, 56), (2, 256, 8, 8), (2, 100, 20, 13), (2, 130, 30, 30),
+                                   (1, 72, 4, 257)])
 def test_fq_levels_bit_exact(orc, shape):
     import torch
     from dldt_amd import FakeQuantize
