@@ -561,3 +561,31 @@ def zero_point_net(seed=31, n=2, c=32, hw=20, oc=(48, 32)):
     y2 = net.conv_f32(a1, w2, b2)
     g.result(y2, "out")
     return g, dict(data=x), dict(acts=dict(a0=a0, a1=a1))
+
+
+def concat_net(seed=41, n=2, c=32, hw=18, branches=(24, 40, 16), oc=48, signed=False):
+    """Branches of quantized convolutions joined by a Concat along the channels and consumed by another
+    convolution, in the form the low-precision transformations leave (concat.cpp:42-190): every branch's
+    FakeQuantize gets the same interval, the Concat takes the u8 (or i8) levels themselves and one per-tensor
+    dequantization follows it.  Channel counts that are no multiples of 4 or 16 exercise every copy width.
+    Returns (graph, feeds, meta)."""
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(0, 1, (n, c, hw, hw)).astype(np.float32)
+    net = QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    out_high = 3.0
+    acts = []
+    for i, oc_b in enumerate(branches):
+        k = 3 if i % 2 else 1
+        w = (rng.standard_normal((oc_b, c, k, k), dtype=np.float32) * np.float32(0.12 if k == 1 else 0.05)).astype(np.float32)
+        b = (rng.standard_normal(oc_b, dtype=np.float32) * np.float32(0.3)).astype(np.float32)
+        acts.append(net.conv(a0, w, b, out_high, pads=(k // 2, k // 2), signed=signed))
+    assert all(a["scale"] == acts[0]["scale"] for a in acts)
+    cat = dict(node=g.concat([a["node"] for a in acts], axis=1), scale=acts[0]["scale"])
+    g.result(net.dequantize(cat), "cat")
+    ct = sum(branches)
+    w = (rng.standard_normal((oc, ct, 3, 3), dtype=np.float32) * np.float32(0.04)).astype(np.float32)
+    b = (rng.standard_normal(oc, dtype=np.float32) * np.float32(0.2)).astype(np.float32)
+    g.result(net.conv_f32(cat, w, b, pads=(1, 1), relu=True), "out")
+    return g, dict(data=x), dict(concat=cat["node"], branches=[a["node"] for a in acts])

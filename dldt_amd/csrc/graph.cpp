@@ -9,8 +9,8 @@ const char* op_name(int op) {
     static const char* names[] = {"Parameter", "Constant", "FakeQuantize", "Convolution",
                                   "GroupConvolution", "MatMul", "Add", "Multiply", "Subtract", "Relu",
                                   "Clamp", "Convert", "MaxPool", "AvgPool", "Reshape", "Result", "Softmax", "MVN",
-                                  "Gelu", "Transpose", "Gather"};
-    return op >= 0 && op <= OP_GATHER ? names[op] : "?";
+                                  "Gelu", "Transpose", "Gather", "Concat"};
+    return op >= 0 && op <= OP_CONCAT ? names[op] : "?";
 }
 
 namespace {
@@ -456,6 +456,38 @@ int hipie_graph_gather(hipie_graph* g, int data, int indices, int64_t axis, int*
     });
 }
 
+/* op::v0::Concat (ngraph/core/src/op/concat.cpp validate_and_infer_types): same element type and rank, all
+ * dimensions but `axis` equal; the axis may be negative */
+int hipie_graph_concat(hipie_graph* g, const int* inputs, int n_inputs, int64_t axis, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id && inputs && n_inputs >= 1 && n_inputs <= 64, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_graph_concat: %d inputs (1 to 64)", n_inputs);
+        const GNode& X0 = node(g, inputs[0], "hipie_graph_concat");
+        const int64_t r = static_cast<int64_t>(X0.shape.size());
+        HIPIE_REQUIRE(axis >= -r && axis < r, HIPIE_PARAMETER_MISMATCH, "hipie_graph_concat: axis %lld of rank %lld",
+                      (long long)axis, (long long)r);
+        const int64_t ax = axis < 0 ? axis + r : axis;
+        GNode n;
+        n.op = OP_CONCAT;
+        n.axes = {ax};
+        n.dtype = X0.dtype;
+        n.shape = X0.shape;
+        n.shape[ax] = 0;
+        for (int i = 0; i < n_inputs; ++i) {
+            const GNode& X = node(g, inputs[i], "hipie_graph_concat");
+            HIPIE_REQUIRE(X.dtype == X0.dtype && X.shape.size() == X0.shape.size(), HIPIE_PARAMETER_MISMATCH,
+                          "hipie_graph_concat: input %d differs in type or rank", i);
+            for (int64_t k = 0; k < r; ++k)
+                HIPIE_REQUIRE(k == ax || X.shape[k] == X0.shape[k], HIPIE_PARAMETER_MISMATCH,
+                              "hipie_graph_concat: input %d differs in dimension %lld", i, (long long)k);
+            n.shape[ax] += X.shape[ax];
+            n.in.push_back(inputs[i]);
+        }
+        HIPIE_REQUIRE(n.shape[ax] < (int64_t(1) << 31), HIPIE_OUT_OF_BOUNDS, "hipie_graph_concat: concatenated dimension too large");
+        *id = add_node(g, std::move(n));
+    });
+}
+
 int hipie_graph_result(hipie_graph* g, int x, const char* name) {
     return guarded([&] {
         GNode& X = node(g, x, "hipie_graph_result");
@@ -572,7 +604,7 @@ hipie_graph* deserialize_graph(const uint8_t* bytes, size_t size) {
     for (uint32_t i = 0; i < count; ++i) {
         const int op = r.pod<int32_t>();
         const std::string name = r.str();
-        const std::vector<int> in = r.ints(8);
+        const std::vector<int> in = r.ints(64);
         const int dtype = r.pod<int32_t>();
         const std::vector<int64_t> shape = r.i64s(8), strides = r.i64s(2), dilations = r.i64s(2), pads_begin = r.i64s(2),
                                    pads_end = r.i64s(2), kernel = r.i64s(2), axes = r.i64s(8);
@@ -654,6 +686,10 @@ hipie_graph* deserialize_graph(const uint8_t* bytes, size_t size) {
             arity(2);
             HIPIE_REQUIRE(axes.size() == 1, HIPIE_NETWORK_NOT_READ, "plan stream: Gather %u without an axis", i);
             st = hipie_graph_gather(G, in[0], in[1], axes[0], &id);
+            break;
+        case OP_CONCAT:
+            HIPIE_REQUIRE(axes.size() == 1 && !in.empty(), HIPIE_NETWORK_NOT_READ, "plan stream: Concat %u without an axis or inputs", i);
+            st = hipie_graph_concat(G, in.data(), static_cast<int>(in.size()), axes[0], &id);
             break;
         case OP_RESULT: arity(1); st = hipie_graph_result(G, in[0], name.c_str()); break;
         default: fail(HIPIE_NETWORK_NOT_READ, "plan stream: node %u has unknown operation %d", i, op);

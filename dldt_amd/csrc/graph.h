@@ -14,7 +14,7 @@ namespace hipie {
 enum OpKind {
     OP_PARAMETER = 0, OP_CONSTANT, OP_FAKE_QUANTIZE, OP_CONVOLUTION, OP_GROUP_CONVOLUTION, OP_MATMUL,
     OP_ADD, OP_MULTIPLY, OP_SUBTRACT, OP_RELU, OP_CLAMP, OP_CONVERT, OP_MAX_POOL, OP_AVG_POOL,
-    OP_RESHAPE, OP_RESULT, OP_SOFTMAX, OP_MVN, OP_GELU, OP_TRANSPOSE, OP_GATHER
+    OP_RESHAPE, OP_RESULT, OP_SOFTMAX, OP_MVN, OP_GELU, OP_TRANSPOSE, OP_GATHER, OP_CONCAT
 };
 const char* op_name(int op);
 
@@ -28,7 +28,7 @@ struct GNode {
     int64_t levels = 0;
     bool ta = false, tb = false, exclude_pad = false, ceil_mode = false;
     float lo = 0, hi = 0;
-    std::vector<int64_t> axes;        // Softmax axis, MVN axes, Transpose order
+    std::vector<int64_t> axes;        // Softmax / Gather / Concat axis, MVN axes, Transpose order
     bool normalize_variance = true, eps_inside_sqrt = true;
     float eps = 0;
     std::vector<uint8_t> data;        // constant payload

@@ -127,6 +127,10 @@ struct Step {
     std::string name, type;
     int64_t macs = 0, bytes = 0;
     int out_node = -1;
+    // exec-graph attributes (exec_graph_info.hpp:34-76), filled once the plan is complete: the graph nodes this step
+    // stands for, the type it computes in (the CPU plugin reports its kernels' input type there: U8 / I8 for the
+    // integer kernels) and the type and layout of what it stores
+    std::string original_names, runtime_precision, output_precision, output_layout;
     virtual ~Step() = default;
     virtual void create(int device, const std::vector<TensorInfo>& tensors) = 0;
     virtual void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs,
@@ -397,6 +401,28 @@ struct PoolStep : Step {
 };
 
 // Result: engine tensor -> dense NCHW output buffer of the request (f32, or u8 levels)
+// Concat of byte tensors along the channel axis: one strided copy per input into its channel slice
+struct ConcatStep : Step {
+    std::vector<int> ins, c_off;
+    int out = -1;
+    void create(int, const std::vector<TensorInfo>&) override {}
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const*, void* const*, hipStream_t s) const override {
+        const hipie_tensor o = tensors[out].desc(arena);
+        for (size_t i = 0; i < ins.size(); ++i) {
+            const hipie_tensor x = tensors[ins[i]].desc(arena);
+            ConcatArgs a{};
+            a.in = static_cast<const int8_t*>(x.data);
+            a.out = static_cast<int8_t*>(o.data);
+            a.N = x.n; a.H = x.h; a.W = x.w; a.C = x.c;
+            a.in_sn = x.stride_n; a.in_sh = x.stride_h; a.in_sw = x.stride_w;
+            a.out_sn = o.stride_n; a.out_sh = o.stride_h; a.out_sw = o.stride_w;
+            a.c_off = c_off[i];
+            launch_concat_channels(a, s);
+        }
+        HIPIE_CHECK_HIP(hipGetLastError());
+    }
+};
+
 struct ExitStep : Step {
     int in = -1, result_index = 0, C = 0;
     bool out_u8 = false;
@@ -775,6 +801,7 @@ struct Planner {
         case OP_TRANSPOSE: plan_mat_transpose(id); break;
         case OP_SOFTMAX: case OP_MVN: case OP_GELU: plan_glue(id); break;
         case OP_GATHER: plan_gather(id); break;
+        case OP_CONCAT: plan_concat(id); break;
         case OP_RESULT: mat ? plan_mat_result(id) : plan_result(id); values[id].kind = VK_FUSED; break;
         default: unsupported(id, "only planned as part of a fused convolution / pooling chain");
         }
@@ -1815,6 +1842,37 @@ struct Planner {
         steps.push_back(std::move(st));
     }
 
+    // Concat of quantized branches (after LPT they share one interval, concat.cpp:42-190, and the dequantization sits
+    // behind the Concat): the levels are copied side by side
+    void plan_concat(int id) {
+        const GNode& n = N(id);
+        if (n.shape.size() != 4 || n.axes[0] != 1) unsupported(id, "Concat is planned along the channel axis of 4-D tensors");
+        auto st = std::make_unique<ConcatStep>();
+        int dtype = -1, off = 0;
+        int64_t bytes = 0;
+        for (int in : n.in) {
+            const Value x = value(in);
+            if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1)
+                unsupported(id, "Concat inputs must be quantized (u8/i8) tensors: dequantized branches are concatenated by LPT before it");
+            if (dtype >= 0 && tensors[x.tensor].dtype != dtype) unsupported(id, "Concat of u8 and i8 levels");
+            dtype = tensors[x.tensor].dtype;
+            st->ins.push_back(x.tensor);
+            st->c_off.push_back(off);
+            off += tensors[x.tensor].c;
+            bytes += N(in).numel();
+        }
+        int nn, c, h, w;
+        nhwc_dims(n.shape, nn, c, h, w);
+        st->out = new_tensor(id, dtype, nn, h, w, c);
+        st->name = n.name;
+        st->type = "Concat";
+        st->bytes = 2 * bytes;
+        st->out_node = id;
+        values[id].kind = VK_TENSOR;
+        values[id].tensor = st->out;
+        steps.push_back(std::move(st));
+    }
+
     void plan_result(int id) {
         const GNode& n = N(id);
         const Value x = value(n.in[0]);
@@ -1921,6 +1979,49 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
     plan->tensors = pl.tensors;
     for (auto& s : pl.steps) s->create(device, plan->tensors);
     plan->steps = std::move(pl.steps);
+    {
+        auto type_name = [](int dt) {
+            return dt == HIPIE_F32 ? "FP32" : (dt == HIPIE_I32 ? "I32" : (dt == HIPIE_I8 ? "I8" : "U8"));
+        };
+        std::vector<char> seen(g->nodes.size(), 0);
+        for (auto& s : plan->steps) {
+            if (s->out_node < 0) continue;
+            // the step's own node and every node behind it that was fused away (chains, merged siblings, shortcuts)
+            std::vector<int> stack(1, s->out_node), found;
+            while (!stack.empty()) {
+                const int v = stack.back();
+                stack.pop_back();
+                if (seen[v]) continue;
+                seen[v] = 1;
+                found.push_back(v);
+                for (int in : g->nodes[v].in)
+                    if (in >= 0 && pl.values[in].kind == VK_FUSED && g->nodes[in].op != OP_CONSTANT) stack.push_back(in);
+            }
+            std::sort(found.begin(), found.end());
+            for (int v : found) s->original_names += (s->original_names.empty() ? "" : ",") + g->nodes[v].name;
+            const GNode& on = g->nodes[s->out_node];
+            s->output_precision = type_name(on.dtype);
+            s->output_layout = on.shape.size() == 4 ? "NHWC" : (on.shape.size() == 2 ? "NC" : (on.shape.size() == 3 ? "CHW" : "ANY"));
+            // integer kernels compute in the type of the activations they read (through a symbolic dequantization
+            // in front of them); everything else in f32
+            int in_dt = HIPIE_F32;
+            const bool integer_kernel = s->type.find("Convolution") != std::string::npos || s->type.find("MatMul") != std::string::npos ||
+                                        s->type.find("Pool") != std::string::npos || s->type.find("Attention") != std::string::npos ||
+                                        s->type == "Transpose";
+            if (integer_kernel)
+                for (int v : found)
+                    for (int in : g->nodes[v].in) {
+                        if (in < 0 || g->nodes[in].op == OP_CONSTANT || std::binary_search(found.begin(), found.end(), in)) continue;
+                        const Value& iv = pl.values[in];
+                        int dt = HIPIE_F32;
+                        if ((iv.kind == VK_TENSOR || iv.kind == VK_DEQ) && iv.tensor >= 0) dt = pl.tensors[iv.tensor].dtype;
+                        else if (iv.kind == VK_MAT) dt = iv.view.dtype;
+                        if (dt == HIPIE_U8B || dt == HIPIE_U8) in_dt = HIPIE_U8;
+                        else if (dt == HIPIE_I8 && in_dt != HIPIE_U8) in_dt = HIPIE_I8;
+                    }
+            s->runtime_precision = type_name(in_dt);
+        }
+    }
     for (size_t i = 0; i < pl.values.size(); ++i)
         if (pl.values[i].kind == VK_TENSOR) {
             plan->node_tensor[static_cast<int>(i)] = pl.values[i].tensor;
@@ -2243,6 +2344,26 @@ int hipie_plan_step_info(const hipie_plan* p, int index, char* name, size_t name
         if (type && type_len) snprintf(type, type_len, "%s", s.type.c_str());
         if (macs) *macs = s.macs;
         if (bytes) *bytes = s.bytes;
+    });
+}
+
+/* the attributes GetExecGraphInfo attaches to an executed node (exec_graph_info.hpp:34-76), by their key there */
+int hipie_plan_step_rt_info(const hipie_plan* p, int index, const char* key, char* buf, size_t cap) {
+    return guarded([&] {
+        HIPIE_REQUIRE(p && key && index >= 0 && index < static_cast<int>(p->steps.size()), HIPIE_OUT_OF_BOUNDS,
+                      "hipie_plan_step_rt_info: index %d", index);
+        const Step& s = *p->steps[index];
+        const std::string k = key;
+        std::string v;
+        if (k == "originalLayersNames") v = s.original_names;
+        else if (k == "layerType") v = s.type;
+        else if (k == "runtimePrecision") v = s.runtime_precision;
+        else if (k == "outputPrecisions") v = s.output_precision;
+        else if (k == "outputLayouts") v = s.output_layout;
+        else if (k == "execOrder") v = std::to_string(index);
+        else if (k == "primitiveType") v = s.variant() >= 0 ? "hip_int8_v" + std::to_string(s.variant()) : "hip";
+        else fail(HIPIE_NOT_FOUND, "hipie_plan_step_rt_info: key '%s' (execTimeMcs is hipie_request_perf)", key);
+        copy_text(v, buf, cap, "hipie_plan_step_rt_info");
     });
 }
 

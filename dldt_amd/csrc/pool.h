@@ -36,7 +36,18 @@ struct ExitArgs {
     int32_t out_u8;
 };
 
+// Concat along the channel axis of byte NHWC tensors: one input's C channels copied to channels [c_off, c_off + C) of
+// the output (reference::concat, concat.hpp:17-57, is the same copy in NCHW order)
+struct ConcatArgs {
+    const int8_t* in;
+    int8_t* out;
+    int32_t N, H, W, C;
+    int64_t in_sn, in_sh, in_sw, out_sn, out_sh, out_sw;   // bytes
+    int32_t c_off;
+};
+
 void launch_max_pool(const PoolArgs& a, hipStream_t s);
+void launch_concat_channels(const ConcatArgs& a, hipStream_t s);
 void launch_avg_pool(const PoolArgs& a, bool rcp, hipStream_t s);
 void launch_exit(const ExitArgs& a, int in_dtype, hipStream_t s);
 

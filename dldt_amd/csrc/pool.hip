@@ -198,4 +198,53 @@ void launch_exit(const ExitArgs& a, int in_dtype, hipStream_t s) {
     else hipLaunchKernelGGL(exit_nhwc_to_nchw<int8_t>, grid, dim3(kThreads), 0, s, a);
 }
 
+namespace {
+
+// VEC bytes per thread and copy: 16 when the slice starts and ends on 16-byte boundaries of the output pixel, 4 on
+// 4-byte boundaries, else single bytes.  Consecutive threads take consecutive pieces of one pixel, then the next pixel.
+template <int VEC>
+__global__ __launch_bounds__(256) void concat_channels_kernel(const ConcatArgs a, int32_t pieces, float inv_pieces,
+                                                              float inv_W, float inv_HW, int64_t total) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total) return;
+    // idx -> (pixel, piece) -> (n, h, w): reciprocals with one correction step (the host keeps every quotient below 2^24)
+    auto divmod = [](int64_t v, int32_t d, float inv, int32_t& q, int32_t& r) {
+        q = static_cast<int32_t>(static_cast<float>(v) * inv);
+        int64_t rem = v - static_cast<int64_t>(q) * d;
+        if (rem < 0) { --q; rem += d; }
+        else if (rem >= d) { ++q; rem -= d; }
+        r = static_cast<int32_t>(rem);
+    };
+    int32_t pix, piece, n, hw, h, w;
+    divmod(idx, pieces, inv_pieces, pix, piece);
+    divmod(pix, a.H * a.W, inv_HW, n, hw);
+    divmod(hw, a.W, inv_W, h, w);
+    const int8_t* src = a.in + n * a.in_sn + h * a.in_sh + w * a.in_sw + piece * VEC;
+    int8_t* dst = a.out + n * a.out_sn + h * a.out_sh + w * a.out_sw + a.c_off + piece * VEC;
+    if (VEC == 16) *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
+    else if (VEC == 4) *reinterpret_cast<uint32_t*>(dst) = *reinterpret_cast<const uint32_t*>(src);
+    else *dst = *src;
+}
+
+}  // namespace
+
+void launch_concat_channels(const ConcatArgs& a, hipStream_t s) {
+    const int64_t pixels = static_cast<int64_t>(a.N) * a.H * a.W;
+    if (pixels == 0 || a.C == 0) return;
+    const bool al16 = a.C % 16 == 0 && a.c_off % 16 == 0 && a.out_sw % 16 == 0 && reinterpret_cast<uintptr_t>(a.out) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(a.in) % 16 == 0 && a.in_sw % 16 == 0;
+    const bool al4 = a.C % 4 == 0 && a.c_off % 4 == 0 && a.out_sw % 4 == 0 && reinterpret_cast<uintptr_t>(a.out) % 4 == 0 &&
+                     reinterpret_cast<uintptr_t>(a.in) % 4 == 0 && a.in_sw % 4 == 0;
+    const int vec = al16 ? 16 : (al4 ? 4 : 1);
+    const int32_t pieces = a.C / vec;
+    const int64_t total = pixels * pieces;
+    HIPIE_REQUIRE(pixels < (1 << 24) && total < (int64_t(1) << 31) * 256, HIPIE_OUT_OF_BOUNDS, "Concat: %lld pixels", (long long)pixels);
+    // the piece quotient must stay exact too: idx / pieces < 2^24 holds because it is the pixel index
+    const dim3 grid(static_cast<uint32_t>(ceil_div(total, 256))), block(256);
+    const float ip = 1.0f / static_cast<float>(pieces), iw = 1.0f / static_cast<float>(a.W), ihw = 1.0f / static_cast<float>(a.H * a.W);
+    if (vec == 16) hipLaunchKernelGGL(concat_channels_kernel<16>, grid, block, 0, s, a, pieces, ip, iw, ihw, total);
+    else if (vec == 4) hipLaunchKernelGGL(concat_channels_kernel<4>, grid, block, 0, s, a, pieces, ip, iw, ihw, total);
+    else hipLaunchKernelGGL(concat_channels_kernel<1>, grid, block, 0, s, a, pieces, ip, iw, ihw, total);
+}
+
 }  // namespace hipie

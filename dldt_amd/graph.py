@@ -149,6 +149,12 @@ class Graph:
         check(lib().hipie_graph_gather(self._h, data, indices, ctypes.c_int64(axis), ctypes.byref(i)))
         return self._rec(i.value, "Gather", [data, indices], self.nodes[data]["dtype"], axis=axis)
 
+    def concat(self, inputs, axis=1):
+        i = ctypes.c_int()
+        ids = (ctypes.c_int * len(inputs))(*inputs)
+        check(lib().hipie_graph_concat(self._h, ids, len(inputs), ctypes.c_int64(axis), ctypes.byref(i)))
+        return self._rec(i.value, "Concat", list(inputs), self.nodes[inputs[0]]["dtype"], axis=axis)
+
     def result(self, x, name):
         check(lib().hipie_graph_result(self._h, x, name.encode()))
         self.results.append(len(self.nodes))
@@ -200,6 +206,13 @@ class Plan:
             check(L.hipie_plan_step_variant(self._h, i, ctypes.byref(var)))
             self.steps.append(dict(name=name.value.decode(errors="replace"), type=typ.value.decode(errors="replace"), macs=macs.value,
                                    bytes=byts.value, variant=var.value))
+
+    def step_rt_info(self, index, key):
+        """an exec-graph attribute of one executed step (originalLayersNames, layerType, runtimePrecision,
+        outputPrecisions, outputLayouts, execOrder, primitiveType)"""
+        buf = ctypes.create_string_buffer(8192)
+        check(lib().hipie_plan_step_rt_info(self._h, index, key.encode(), buf, ctypes.c_size_t(len(buf))))
+        return buf.value.decode(errors="replace")
 
     def export(self):
         """ExecutableNetwork::Export: the plan as bytes (graph description, constants, kernel choices)."""

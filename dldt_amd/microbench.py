@@ -242,15 +242,6 @@ def config5():
              macs=T * (4 * H * H + 2 * H * FF) + 2 * B * NH * S * S * 64, bound="mfma")
     r["sequences/s (12 layers, these kernels only)"] = B / (12 * layer_us) * 1e6
     rows.append(r)
-    # the whole layer as composed by dldt_amd.bert (quantisation, transposes and per-sequence launches included)
-    from .bert import EncoderLayer
-    layer = EncoderLayer(hidden=H, heads=NH, ffn=FF, batch=B, seq=S)
-    x = torch.randn((B, S, H), device="cuda")
-    us = _time(lambda: layer.run(x), reps=5, warm=2)
-    r = _row("cfg5 one encoder layer end to end (dldt_amd.bert, %d launches)" % (15 + 3 * B), us, macs=layer.macs(), bound="mfma")
-    r["sequences/s (12 layers)"] = B / (12 * us) * 1e6
-    rows.append(r)
-    del layer
     return rows + config5_graph()
 
 

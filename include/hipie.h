@@ -417,6 +417,11 @@ int hipie_graph_transpose(hipie_graph* g, int x, const int64_t* order, int rank,
 /* op::v1::Gather with the axis Constant's value; planned as an embedding lookup: f32 Constant table
  * [vocabulary, hidden], i32 Parameter indices [batch, sequence], axis 0 */
 int hipie_graph_gather(hipie_graph* g, int data, int indices, int64_t axis, int* id);
+/* op::v0::Concat (ngraph/core/reference/include/ngraph/runtime/reference/concat.hpp:17-57: the inputs' elements copied
+ * side by side along `axis`).  After the low-precision transformations a Concat of quantized branches takes their u8 /
+ * i8 levels directly (low_precision_transformations/src/concat.cpp:42-190 gives every branch the same interval and
+ * moves the dequantization behind the Concat), which is the form the engine runs: byte tensors along the channel axis. */
+int hipie_graph_concat(hipie_graph* g, const int* inputs, int n_inputs, int64_t axis, int* id);
 int hipie_graph_result(hipie_graph* g, int x, const char* name);
 int hipie_graph_set_name(hipie_graph* g, int id, const char* friendly_name);
 
@@ -475,6 +480,12 @@ int hipie_plan_step_info(const hipie_plan* plan, int index, char* name, size_t n
 /* the kernel variant a step runs (hipie_conv_set_tile numbering), -1 for a step without variants: part
  * of what GetExecGraphInfo reports per executed node (exec_graph_info.hpp:34-76, implementation type) */
 int hipie_plan_step_variant(const hipie_plan* plan, int index, int* variant);
+/* the attributes GetExecGraphInfo attaches to every executed node (exec_graph_info.hpp:34-76), by their key there:
+ * originalLayersNames (comma-separated graph nodes the step stands for), layerType, runtimePrecision (U8 / I8 for the
+ * integer kernels: the type of the activations they multiply, as the CPU plugin reports it; FP32 otherwise),
+ * outputPrecisions, outputLayouts, execOrder, primitiveType ("hip_int8_v<variant>" | "hip"); execTimeMcs is
+ * hipie_request_perf.  HIPIE_NOT_FOUND for another key. */
+int hipie_plan_step_rt_info(const hipie_plan* plan, int index, const char* key, char* buf, size_t buf_len);
 
 /* IExecutableNetworkInternal::CreateInferRequestImpl: own stream + own activation arena; weights
  * stay shared in the plan.  perf_count mirrors the PERF_COUNT config key (ie_plugin_config.hpp:277). */

@@ -130,6 +130,10 @@ struct Translator {
         } else if (ngraph::is_type<ngraph::opset1::Gather>(node)) {
             const auto axis = constant_i64(n.input_value(2), n);
             check(hipie_graph_gather(g, in(n, 0), in(n, 1), axis.at(0), &id), "hipie_graph_gather");
+        } else if (const auto concat = ngraph::as_type_ptr<const ngraph::opset1::Concat>(node)) {
+            std::vector<int> inputs;
+            for (size_t i = 0; i < n.get_input_size(); ++i) inputs.push_back(in(n, i));
+            check(hipie_graph_concat(g, inputs.data(), static_cast<int>(inputs.size()), concat->get_axis(), &id), "hipie_graph_concat");
         } else if (ngraph::is_type<ngraph::opset1::Result>(node)) {
             // the request's output is named after the producer (template_executable_network.cpp:100-110)
             const auto producer = n.input_value(0);

@@ -186,9 +186,11 @@ std::map<std::string, InferenceEngine::InferenceEngineProfileInfo> InferRequest:
         info.status = InferenceEngine::InferenceEngineProfileInfo::EXECUTED;
         info.realTime_uSec = info.cpu_uSec = static_cast<long long>(ms * 1000.f);
         info.execution_index = static_cast<unsigned>(i);
-        int variant = -1;
-        hipie_plan_step_variant(plan, i, &variant);
-        std::snprintf(info.exec_type, sizeof info.exec_type, variant >= 0 ? "hip_i8_v%d" : "hip", variant);
+        // exec_type as the CPU plugin writes it: "<primitive>_<runtime precision>" (mkldnn_node.cpp getPrimitiveDescriptorType)
+        char primitive[64] = "", precision[16] = "";
+        check(hipie_plan_step_rt_info(plan, i, "primitiveType", primitive, sizeof primitive), "hipie_plan_step_rt_info");
+        check(hipie_plan_step_rt_info(plan, i, "runtimePrecision", precision, sizeof precision), "hipie_plan_step_rt_info");
+        std::snprintf(info.exec_type, sizeof info.exec_type, "%s_%s", primitive, precision);
         std::snprintf(info.layer_type, sizeof info.layer_type, "%s", type);
         perf[name] = info;
     }

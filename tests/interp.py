@@ -84,6 +84,8 @@ def evaluate(orc, nodes, feeds, keep=None, override=None, targets=None):
             v = np.ascontiguousarray(np.take(x[0], idx, axis=n["axis"]))
         elif op == "Transpose":
             v = np.ascontiguousarray(np.transpose(x[0], n["order"]))
+        elif op == "Concat":
+            v = np.concatenate(x, axis=n["axis"])             # concat.hpp:17-57: the inputs' elements side by side
         elif op == "Softmax":
             v = orc.softmax(x[0], n["axis"])
         elif op == "MVN":

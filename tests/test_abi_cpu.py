@@ -198,3 +198,59 @@ def test_request_entry_points_reject_null_handles():
     assert lib.hipie_request_wait_for(None, ctypes.c_int64(0)) == -4
     assert lib.hipie_request_cancel(None) == -4
     assert lib.hipie_request_wait(None) == -4
+
+
+def test_exec_graph_attributes_per_step():
+    """what GetExecGraphInfo attaches to an executed node (exec_graph_info.hpp:34-76): the fused original layers, the
+    type the kernel computes in (U8 for the integer convolutions, as the CPU plugin reports it), output type / layout"""
+    from dldt_amd import HipieError, builders
+    g, _ = builders.resnet50(batch=1, res=224)
+    plan = g.compile(-1)
+    info = [{k: plan.step_rt_info(i, k) for k in ("originalLayersNames", "layerType", "runtimePrecision", "outputPrecisions",
+                                                   "outputLayouts", "execOrder", "primitiveType")}
+            for i in range(len(plan.steps))]
+    assert info[0]["layerType"] == "FakeQuantize" and info[0]["runtimePrecision"] == "FP32" and info[0]["outputPrecisions"] == "U8"
+    convs = [r for r in info if r["layerType"].startswith("Convolution")]
+    assert len(convs) == 49 and all(r["runtimePrecision"] == "U8" and r["outputLayouts"] == "NHWC" for r in convs)
+    assert all(r["primitiveType"].startswith("hip_int8_v") for r in convs)
+    # a convolution stands for itself, its bias Add and the FakeQuantize behind it at least
+    assert all(len(r["originalLayersNames"].split(",")) >= 3 for r in convs)
+    fc = [r for r in info if r["layerType"] == "MatMul"]
+    assert len(fc) == 1 and fc[0]["outputPrecisions"] == "FP32" and fc[0]["runtimePrecision"] == "U8"
+    assert [int(r["execOrder"]) for r in info] == list(range(len(info)))
+    # every graph node that computes is named by exactly one step
+    named = [n for r in info for n in r["originalLayersNames"].split(",") if n]
+    assert len(named) == len(set(named))
+    with pytest.raises(HipieError) as e:
+        plan.step_rt_info(0, "execTimeMcs")
+    assert e.value.status == -5
+    with pytest.raises(HipieError) as e:
+        plan.step_rt_info(len(plan.steps), "layerType")
+    assert e.value.status == -6
+
+
+def test_concat_shape_inference_and_planner_limits():
+    """Concat infers its shape like op::v0::Concat (negative axis included), refuses mismatched inputs when the graph
+    is described, and the planner takes it along the channels of quantized 4-D tensors only"""
+    from dldt_amd import HipieError, builders
+    from dldt_amd.graph import Graph
+    from dldt_amd.tensor import U8
+    g = Graph()
+    a = g.parameter("a", (2, 3, 5, 5))
+    b = g.parameter("b", (2, 4, 5, 5))
+    c = g.concat([a, b], axis=-3)                   # the channel axis, counted from the end
+    with pytest.raises(HipieError) as e:
+        g.concat([a, b], axis=2)                    # dimension 1 differs
+    assert e.value.status == -4
+    with pytest.raises(HipieError):
+        g.concat([a, b], axis=4)
+    g.result(c, "c")
+    with pytest.raises(HipieError) as e:            # f32 branches: LPT would not have left the Concat there
+        g.compile(-1)
+    assert e.value.status == -2 and "Concat" in str(e.value)
+    g2, _, meta = builders.concat_net()
+    plan = g2.compile(-1)
+    assert [s["type"] for s in plan.steps].count("Concat") == 1
+    assert tuple(plan.outputs[0]["shape"]) == (2, 24 + 40 + 16, 18, 18)
+    sup = g2.query()
+    assert all(sup)

@@ -360,3 +360,24 @@ def test_timed_wait_status_only_and_cancel():
     req.start(ins, outs)
     req.wait()
     np.testing.assert_array_equal(outs[0].array.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("branches,signed", [((24, 40, 16), False), ((64, 64), False), ((7, 33, 5, 19), False), ((32, 16), True)])
+def test_concat_of_quantized_branches(orc, branches, signed):
+    """Concat of u8 / i8 branches with one shared interval (what ConcatTransformation leaves): the levels side by side,
+    bit-exact, whatever the slices' alignment; a padded convolution reads the concatenated tensor"""
+    from dldt_amd import builders
+    g, feeds, meta = builders.concat_net(branches=branches, signed=signed)
+    want, kept = evaluate(orc, g.nodes, feeds, keep=[meta["concat"]])
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps].count("Concat") == 1
+    req = plan.create_request()
+    got = dict(zip([o["name"] for o in plan.outputs], req.infer(feeds["data"])))
+    np.testing.assert_array_equal(req.tensor(meta["concat"]), kept[meta["concat"]])
+    for name in ("cat", "out"):
+        np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
+    # a second inference into the same arena: the slices are rewritten, nothing is left from the first
+    other = np.random.default_rng(5).uniform(0, 1, feeds["data"].shape).astype(np.float32)
+    want2, _ = evaluate(orc, g.nodes, dict(data=other))
+    got2 = dict(zip([o["name"] for o in plan.outputs], req.infer(other)))
+    np.testing.assert_array_equal(got2["out"].view(np.uint32), want2["out"].view(np.uint32))

@@ -206,3 +206,31 @@ def test_fused_attention_with_mask(orc):
     want_ctx = orc.multiply(orc.matmul(pq, vn).astype(np.float32), s2)
     np.testing.assert_array_equal(ctx.cpu().numpy().view(np.uint32), want_ctx.view(np.uint32))
     assert torch.equal(att.run(q, k, v, mask=torch.from_numpy(mask).cuda()), ctx)
+
+
+def test_nested_batches_inside_a_packed_tensor():
+    """hipie_matmul_run_nested / hipie_transpose_bytes_nested address (sequence, head) batches inside one
+    [tokens, 3 * hidden] tensor by pitch, inner and outer strides (the attention operands of an encoder without
+    copying the heads out): q k^T per head against numpy's integer product, and V transposed per head"""
+    import torch
+    from dldt_amd import BatchedMatMul, make_epilogue
+    from dldt_amd.ops import matmul_strided, transpose_bytes
+    from dldt_amd.tensor import I32
+    rng = np.random.default_rng(77)
+    B, S, NH, D = 2, 96, 3, 64
+    H = NH * D
+    qkv = rng.integers(-128, 128, (B * S, 3 * H)).astype(np.int8)
+    t = torch.from_numpy(qkv).cuda()
+    scores = torch.zeros((B, NH, S, S), dtype=torch.int32, device="cuda")
+    mm = BatchedMatMul(D, S, make_epilogue(out_dtype=I32))
+    base = t.data_ptr()
+    # head h of sequence b: rows b * S .., columns h * D .. (q) and H + h * D .. (k)
+    matmul_strided(mm, base, 3 * H, D, base + H, 3 * H, D, scores.data_ptr(), S, S * S, S, NH,
+                   batch_outer=B, outer_a=S * 3 * H, outer_b=S * 3 * H, outer_o=NH * S * S)
+    x = qkv.reshape(B, S, 3, NH, D).astype(np.int64)
+    want = np.einsum("bshd,bthd->bhst", x[:, :, 0], x[:, :, 1])
+    np.testing.assert_array_equal(scores.cpu().numpy(), want)
+    vt = torch.zeros((B, NH, D, S), dtype=torch.int8, device="cuda")
+    transpose_bytes(base + 2 * H, 3 * H, D, vt.data_ptr(), S, D * S, S, D, NH, batch_outer=B,
+                    outer_src=S * 3 * H, outer_dst=NH * D * S)
+    np.testing.assert_array_equal(vt.cpu().numpy(), qkv.reshape(B, S, 3, NH, D)[:, :, 2].transpose(0, 2, 3, 1))
