@@ -53,6 +53,18 @@ class QuantizedNet:
         return dict(node=q, scale=np.float32(d["scale"]), shift=np.float32(d["shift"]),
                     zero_point=np.float32(lpt.round_zero_point(d["shift"])))
 
+    def asymmetric_per_channel(self, y, lo, hi):
+        """The same with one interval per channel (allowed in front of a GroupConvolution, whose per-channel
+        dequantization folds into its per-channel weights scales): scales, shifts and zero points are vectors."""
+        d = [lpt.decompose_fake_quantize(256, np.float32(a), np.float32(b), allow_zero_point=True) for a, b in zip(lo, hi)]
+        assert all(k["precision"] == U8 for k in d) and len({(k["new_low"], k["new_high"]) for k in d}) == 1
+        rank = 4
+        q = self.g.fake_quantize(y, self._channel(np.asarray(lo, np.float32), rank), self._channel(np.asarray(hi, np.float32), rank),
+                                 d[0]["new_low"], d[0]["new_high"], 256, U8)
+        return dict(node=q, scale=np.array([k["scale"] for k in d], np.float32).reshape(-1),
+                    shift=np.array([k["shift"] for k in d], np.float32).reshape(-1),
+                    zero_point=np.array([lpt.round_zero_point(k["shift"]) for k in d], np.float32).reshape(-1))
+
     def _accumulate(self, act, w, bias, conv_attrs, matmul=False):
         """[Subtract(zero point)] -> Conv'/MatMul' -> Add(b / s): returns (node, s[c])."""
         g = self.g
@@ -64,8 +76,9 @@ class QuantizedNet:
             wq = wq.reshape(wq.shape[0], 1, 1, wq.shape[2], wq.shape[3])
         wc = g.constant(wq, I8)
         x = act["node"]
-        if act.get("zero_point", 0) != 0:      # TypeRelaxed Subtract(u8, u8) -> f32, written as Convert + Subtract
-            x = g.subtract(g.convert(x, F32), g.constant(np.float32(act["zero_point"]).reshape(())))
+        zp = np.asarray(act.get("zero_point", 0), np.float32)
+        if np.any(zp != 0):                    # TypeRelaxed Subtract(u8, u8) -> f32, written as Convert + Subtract
+            x = g.subtract(g.convert(x, F32), g.constant(zp.reshape(()) if zp.ndim == 0 else self._channel(zp, 4)))
         if matmul:
             y = g.matmul(x, wc, False, True)
             rank = 2
@@ -589,3 +602,26 @@ def concat_net(seed=41, n=2, c=32, hw=18, branches=(24, 40, 16), oc=48, signed=F
     b = (rng.standard_normal(oc, dtype=np.float32) * np.float32(0.2)).astype(np.float32)
     g.result(net.conv_f32(cat, w, b, pads=(1, 1), relu=True), "out")
     return g, dict(data=x), dict(concat=cat["node"], branches=[a["node"] for a in acts])
+
+
+def per_channel_zero_point_net(seed=47, n=2, c=48, hw=17, oc=40, stride=1):
+    """A depthwise convolution whose input is quantized per channel with asymmetric intervals: u8 levels with one
+    integer zero point per channel in front of the GroupConvolution (the only place the transformations leave
+    distinct per-channel zero points: convolution.cpp:97-120 broadcasts the Subtract constant over the channels,
+    and only a grouped convolution's input may be quantized per channel), padded, so the halo must hold every
+    channel's own level; then a dense 1 x 1 convolution to f32.  Returns (graph, feeds, meta)."""
+    rng = np.random.default_rng(seed)
+    x = rng.normal(0.3, 1.0, (n, c, hw, hw)).astype(np.float32)
+    net = QuantizedNet()
+    g = net.g
+    lo = rng.uniform(-2.5, -0.5, c).astype(np.float32)
+    hi = rng.uniform(0.8, 3.0, c).astype(np.float32)
+    a0 = net.asymmetric_per_channel(g.parameter("data", x.shape), lo, hi)
+    assert len(set(a0["zero_point"].tolist())) > 8
+    w1 = (rng.standard_normal((c, 1, 3, 3), dtype=np.float32) * np.float32(0.3)).astype(np.float32)
+    b1 = (rng.standard_normal(c, dtype=np.float32) * np.float32(0.2)).astype(np.float32)
+    a1 = net.conv(a0, w1, b1, 2.5, strides=(stride, stride), pads=(1, 1), grouped=True)
+    w2 = (rng.standard_normal((oc, c, 1, 1), dtype=np.float32) * np.float32(0.1)).astype(np.float32)
+    b2 = (rng.standard_normal(oc, dtype=np.float32) * np.float32(0.2)).astype(np.float32)
+    g.result(net.conv_f32(a1, w2, b2), "out")
+    return g, dict(data=x), dict(acts=dict(a0=a0, a1=a1))

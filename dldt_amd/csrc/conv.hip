@@ -1380,6 +1380,9 @@ struct hipie_matmul {
     Epilogue epi;
 };
 
+// the zero point of input channel ic
+static inline int zero_point_of(const hipie_conv_desc& d, int ic) { return d.in_zero_points ? d.in_zero_points[ic] : d.in_zero_point; }
+
 void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weights) {
     // K order (kh, kw, ic) over the padded channel stride.  A 16-byte piece must not straddle
     // two filter taps unless consecutive taps are contiguous in memory (in_stride_w == c stride).
@@ -1406,8 +1409,9 @@ void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weight
     }
     std::vector<int8_t> w(static_cast<size_t>(OCp) * Kp, 0);
     std::vector<int32_t> cr(OCp, 0);
+    const int stored_zero = d.in_dtype == HIPIE_U8B ? 128 : 0;
     parallel_for(d.oc, [&](int64_t oc) {
-        int64_t sum = 0;
+        int64_t corr = 0;
         for (int kh = 0; kh < d.kh; ++kh)
             for (int kw = 0; kw < d.kw; ++kw)
                 for (int ic = 0; ic < d.ic; ++ic) {
@@ -1415,10 +1419,10 @@ void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weight
                     const int64_t k = per_row ? kh * row_kp + kw * cs + ic
                                               : (static_cast<int64_t>(kh) * d.kw + kw) * cs + ic;
                     w[packed_row(oc) * Kp + k] = v;
-                    sum += v;
+                    // stored byte = level - 128 (U8B) or level (I8); the product wanted is (level - zero point) * w
+                    corr += static_cast<int64_t>(stored_zero - zero_point_of(d, ic)) * v;
                 }
-        // stored byte = level - 128 (U8B) or level (I8); the product wanted is (level - zero point) * w
-        cr[oc] = static_cast<int32_t>(((d.in_dtype == HIPIE_U8B ? 128 : 0) - d.in_zero_point) * sum);
+        cr[oc] = static_cast<int32_t>(corr);
     });
     if (device >= 0) {
         wgt.upload(device, w.data(), w.size());
@@ -1436,8 +1440,9 @@ static void check_conv_desc(const hipie_conv_desc& d, const char* what) {
     HIPIE_REQUIRE(d.in_c_stride >= d.ic && d.in_c_stride % 4 == 0, HIPIE_PARAMETER_MISMATCH,
                   "%s: in_c_stride=%d must be a multiple of 4 >= ic=%d", what, d.in_c_stride, d.ic);
     const int lo = d.in_dtype == HIPIE_U8B ? 0 : -128;
-    HIPIE_REQUIRE(d.in_zero_point >= lo && d.in_zero_point <= lo + 255, HIPIE_PARAMETER_MISMATCH,
-                  "%s: zero point %d is not a level of the input type", what, d.in_zero_point);
+    for (int ic = 0; ic < (d.in_zero_points ? d.ic : 1); ++ic)
+        HIPIE_REQUIRE(zero_point_of(d, ic) >= lo && zero_point_of(d, ic) <= lo + 255, HIPIE_PARAMETER_MISMATCH,
+                      "%s: zero point %d is not a level of the input type", what, zero_point_of(d, ic));
 }
 
 static void conv_out_hw(const hipie_conv_desc& d, int h, int w, int& oh, int& ow) {
@@ -1567,9 +1572,16 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
                       d.ic, d.oc);
         HIPIE_REQUIRE(d.in_c_stride >= d.ic && d.in_c_stride % 4 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_create: in_c_stride=%d must be a multiple of 4 >= ic=%d", d.in_c_stride, d.ic);
+        {
+            const int lo = d.in_dtype == HIPIE_U8B ? 0 : -128;
+            for (int ic = 0; ic < (d.in_zero_points ? d.ic : 1); ++ic)
+                HIPIE_REQUIRE(zero_point_of(d, ic) >= lo && zero_point_of(d, ic) <= lo + 255, HIPIE_PARAMETER_MISMATCH,
+                              "hipie_conv_create: zero point %d is not a level of the input type", zero_point_of(d, ic));
+        }
         auto c = std::make_unique<hipie_conv>();
         c->device = device;
         c->d = d;
+        c->d.in_zero_points = nullptr;   // the caller's array is read during this call only
         if (depthwise) {
             // weights [C][kh][kw] -> [kh*kw][OCp]; corr = 128 * sum of the channel's taps
             HIPIE_REQUIRE(d.in_c_stride % 16 == 0, HIPIE_NOT_IMPLEMENTED,
@@ -1585,7 +1597,7 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
                     w[static_cast<size_t>(t) * c->OCp + ch] = weights[ch * taps + t];
                     sum += weights[ch * taps + t];
                 }
-                corr[ch] = ((d.in_dtype == HIPIE_U8B ? 128 : 0) - d.in_zero_point) * sum;
+                corr[ch] = ((d.in_dtype == HIPIE_U8B ? 128 : 0) - zero_point_of(d, ch)) * sum;
             }
             c->epi.build(device, *epilogue, d.oc, c->OCp);
             std::vector<uint32_t> rows;
@@ -1643,6 +1655,7 @@ int hipie_conv_create_fused(int device, const hipie_conv_desc* desc, const int8_
                       "hipie_conv_create_fused: the fused form needs bias, scale, FakeQuantize with input_low 0");
         c->fused = true;
         c->sd = sd;
+        c->sd.in_zero_points = nullptr;
         c->sg.pack(device, sd, shortcut_weights);
         std::vector<float> b(c->OCp, 0.f), s(c->OCp, 1.f);
         for (int oc = 0; oc < sd.oc; ++oc) {

@@ -24,7 +24,8 @@ struct TensorInfo {
     int producer = -1;       // graph node whose value it holds
     int alias = -1;          // shares the bytes of this earlier tensor (same element count, other row split)
     int fill_level = 0;      // level held by the halo and the channel padding (a consumer's zero point)
-    bool fill_fixed = false; // a consumer depends on fill_level
+    std::vector<int> fill_levels;   // one level per channel instead (a consumer with per-channel zero points), or empty
+    bool fill_fixed = false; // a consumer depends on fill_level / fill_levels
     int64_t esize() const { return dtype == HIPIE_F32 || dtype == HIPIE_I32 ? 4 : 1; }
     int wp() const { return w + 2 * halo; }
     int hp() const { return h + 2 * halo; }
@@ -175,6 +176,7 @@ struct ConvStep : Step {
     hipie_conv_desc desc{};
     std::vector<int8_t> weights;   // OIHW
     EpilogueSpec epi;
+    std::vector<int32_t> zero_points;   // per input channel (a per-channel Subtract in front of the convolution), or empty
     hipie_conv* conv = nullptr;
     int64_t in_w_bytes = 0;        // input + weight bytes (what a fused consumer still has to read)
     // projection shortcut (Conv' -> Add -> Multiply, f32, used only by this step's residual Add):
@@ -188,6 +190,7 @@ struct ConvStep : Step {
         desc.in_c_stride = t.cs;
         desc.in_stride_w = t.cs;
         desc.in_stride_h = t.wp() * t.cs;
+        desc.in_zero_points = zero_points.empty() ? nullptr : zero_points.data();
     }
     void create(int device, const std::vector<TensorInfo>& tensors) override {
         fill_desc(tensors);
@@ -1598,12 +1601,20 @@ struct Planner {
         // Subtract(zero point) in front of the convolution: an integer per tensor (what optimizeSubtract
         // leaves, network_helper.cpp:1479-1521) goes into the accumulators' initial value
         int zero_point = 0;
+        std::vector<int32_t> zero_points;   // filled when the channels' zero points differ
         if (x.kind == VK_DEQ && x.mul.empty() && !x.sub.empty() && tensors[x.tensor].esize() == 1) {
             const float z = x.sub[0];
-            for (float v : x.sub)
-                if (v != z) unsupported(id, "per-channel activation zero points");
-            if (z != std::nearbyintf(z)) unsupported(id, "activation zero point that is not an integer level");
-            zero_point = static_cast<int>(z);
+            bool uniform = true;
+            for (float v : x.sub) {
+                if (v != std::nearbyintf(v)) unsupported(id, "activation zero point that is not an integer level");
+                uniform = uniform && v == z;
+            }
+            if (uniform) {
+                zero_point = static_cast<int>(z);
+            } else {
+                if (static_cast<int>(x.sub.size()) != tensors[x.tensor].c) unsupported(id, "zero points for other than every input channel");
+                for (float v : x.sub) zero_points.push_back(static_cast<int32_t>(v));
+            }
         } else if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1) {
             unsupported(id, x.kind == VK_DEQ ? "dequantized (f32) convolution inputs are not planned"
                                              : "input must be a quantized (u8/i8) tensor");
@@ -1650,11 +1661,14 @@ struct Planner {
         tensors[x.tensor].halo = std::max(tensors[x.tensor].halo, halo);
         st->in = x.tensor;
         d.in_zero_point = zero_point;
+        st->zero_points = zero_points;
         if (halo > 0) {   // padding is applied behind the Subtract: the halo must read as the zero point
             TensorInfo& ti = tensors[x.tensor];
-            if (ti.fill_fixed && ti.fill_level != zero_point)
+            const std::vector<int> levels(zero_points.begin(), zero_points.end());
+            if (ti.fill_fixed && (ti.fill_level != zero_point || ti.fill_levels != levels))
                 unsupported(id, "consumers of one tensor pad it with different levels");
             ti.fill_level = zero_point;
+            ti.fill_levels = levels;
             ti.fill_fixed = true;
         }
 
@@ -1910,6 +1924,7 @@ struct hipie_plan {
     struct Io { std::string name; int dtype; std::vector<int64_t> shape; int64_t bytes; };
     std::vector<Io> inputs, outputs;
     PlanConfig config;
+    std::map<int, DeviceBuffer> fill_patterns;   // tensor -> cs bytes: what a pixel of its halo holds, channel by channel
 };
 
 struct hipie_request {
@@ -1933,6 +1948,13 @@ struct hipie_request {
 };
 
 namespace {
+
+// every pixel of a tensor (halo included) gets the byte pattern[c] in channel c
+__global__ void fill_pixels(uint8_t* p, int64_t pixels, int cs, const uint8_t* pattern) {
+    const int64_t n = pixels * cs;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+        p[i] = pattern[i % cs];
+}
 
 __global__ void fill_bytes(uint8_t* p, int64_t n, uint8_t v) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
@@ -1977,6 +1999,14 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
     }
     plan->arena_bytes = off;
     plan->tensors = pl.tensors;
+    if (device >= 0)
+        for (size_t i = 0; i < plan->tensors.size(); ++i) {
+            const TensorInfo& t = plan->tensors[i];
+            if (t.fill_levels.empty() || t.alias >= 0) continue;
+            std::vector<uint8_t> pattern(t.cs, static_cast<uint8_t>(t.dtype == HIPIE_U8B ? 0x80 : 0));   // padding channels: level 0
+            for (int c = 0; c < t.c; ++c) pattern[c] = static_cast<uint8_t>((t.fill_levels[c] - (t.dtype == HIPIE_U8B ? 128 : 0)) & 0xff);
+            plan->fill_patterns[static_cast<int>(i)].upload(device, pattern.data(), pattern.size());
+        }
     for (auto& s : pl.steps) s->create(device, plan->tensors);
     plan->steps = std::move(pl.steps);
     {
@@ -2395,6 +2425,11 @@ int hipie_request_create(const hipie_plan* p, int perf_count, hipie_request** ou
             if (byte != 0)
                 hipLaunchKernelGGL(fill_bytes, dim3(1024), dim3(256), 0, r->stream, a + t.offset, t.bytes,
                                    static_cast<uint8_t>(byte & 0xff));
+        }
+        for (const auto& kv : p->fill_patterns) {
+            const TensorInfo& t = p->tensors[kv.first];
+            hipLaunchKernelGGL(fill_pixels, dim3(1024), dim3(256), 0, r->stream, a + t.offset,
+                               static_cast<int64_t>(t.n) * t.hp() * t.wp(), t.cs, kv.second.as<uint8_t>());
         }
         HIPIE_CHECK_HIP(hipGetLastError());
         for (const auto& io : p->inputs) {

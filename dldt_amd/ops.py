@@ -107,7 +107,7 @@ class hipie_conv_desc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int32) for k in (
         "in_dtype", "ic", "oc", "kh", "kw", "stride_h", "stride_w", "dil_h", "dil_w",
         "pad_top", "pad_left", "pad_bottom", "pad_right", "groups", "in_c_stride",
-        "in_stride_h", "in_stride_w", "in_zero_point")]
+        "in_stride_h", "in_stride_w", "in_zero_point")] + [("in_zero_points", ctypes.POINTER(ctypes.c_int32))]
 
 
 def make_epilogue(bias=None, scale=None, residual_dtype=0, res_sub=None, res_mul=None,
@@ -160,9 +160,14 @@ class Convolution:
         else:
             groups = 1
             self.oc, self.ic, self.kh, self.kw = w.shape
+        # zero_point: one integer level, or one per input channel
+        zps = None if np.ndim(zero_point) == 0 else np.ascontiguousarray(zero_point, np.int32)
         d = hipie_conv_desc(in_tensor.dtype, self.ic, self.oc, self.kh, self.kw, strides[0], strides[1],
                             dilations[0], dilations[1], pads_begin[0], pads_begin[1], pads_end[0],
-                            pads_end[1], groups, in_tensor.cs, in_tensor.stride_h, in_tensor.stride_w, int(zero_point))
+                            pads_end[1], groups, in_tensor.cs, in_tensor.stride_h, in_tensor.stride_w,
+                            0 if zps is not None else int(zero_point),
+                            zps.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)) if zps is not None else None)
+        assert zps is None or zps.shape == (self.ic,)
         self.epilogue = epilogue or make_epilogue(out_dtype=I32)
         self._h = ctypes.c_void_p()
         check(lib().hipie_conv_create(ctypes.c_int(device), ctypes.byref(d),

@@ -199,6 +199,11 @@ typedef struct hipie_conv_desc {
                                              (convolution.cpp:84-120, optimizeSubtract network_helper.cpp:1479-1521).
                                              Padding is applied after the Subtract, so the halo of the
                                              input tensor must hold this level (not level 0). */
+    const int32_t* in_zero_points;        /* NULL, or one level per input channel [ic] in place of in_zero_point
+                                             (a per-channel Subtract constant: what the transformation's explicit
+                                             broadcast, convolution.cpp:97-120, holds when the activations in front of a
+                                             grouped convolution are quantized per channel); the halo then holds
+                                             channel c's level in channel c.  Read during the create call only. */
 } hipie_conv_desc;
 
 typedef struct hipie_conv hipie_conv;

@@ -422,6 +422,34 @@ def test_conv_input_zero_point(orc, signed, zp, depthwise):
     np.testing.assert_array_equal(out.to_nchw(), want)
 
 
+@pytest.mark.parametrize("depthwise", [False, True])
+@pytest.mark.parametrize("signed", [False, True])
+def test_conv_per_channel_input_zero_points(orc, signed, depthwise):
+    """(x - zero point[c]) * w with one level per input channel; the halo holds channel c's level in channel c"""
+    from dldt_amd import Convolution, DeviceTensor
+    rng = np.random.default_rng(70 + signed + 2 * depthwise)
+    N, C, H, W, OC = 2, 32, 9, 11, 32 if depthwise else 40
+    lo, hi = (-128, 128) if signed else (0, 256)
+    x = rng.integers(lo, hi, (N, C, H, W)).astype(np.int32)
+    zp = rng.integers(lo, hi, C).astype(np.int32)
+    w = rng.integers(-127, 128, (C, 1, 1, 3, 3) if depthwise else (OC, C, 3, 3)).astype(np.int32)
+    want = orc.convolution(x - zp.reshape(1, C, 1, 1), w, (1, 1), (1, 1), (1, 1), (1, 1), grouped=depthwise)
+    xin = DeviceTensor.from_nchw(x, I8 if signed else U8B, halo=1, fill_level=0)
+    # the border: every pixel of the halo holds the channels' zero points
+    full = xin.view                                                # [N, H + 2, W + 2, cs] stored bytes
+    stored = (zp - (0 if signed else 128)).astype(np.int8)
+    import torch
+    pattern = torch.from_numpy(stored).to(full.device)
+    full[:, 0, :, :C] = pattern
+    full[:, -1, :, :C] = pattern
+    full[:, :, 0, :C] = pattern
+    full[:, :, -1, :C] = pattern
+    conv = Convolution(w.astype(np.int8), xin, (1, 1), (1, 1), (1, 1), (1, 1), zero_point=zp)
+    out = DeviceTensor(N, H, W, OC, I32)
+    conv.run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw(), want)
+
+
 _WIDE_CASES = {}
 
 

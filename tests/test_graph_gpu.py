@@ -381,3 +381,19 @@ def test_concat_of_quantized_branches(orc, branches, signed):
     want2, _ = evaluate(orc, g.nodes, dict(data=other))
     got2 = dict(zip([o["name"] for o in plan.outputs], req.infer(other)))
     np.testing.assert_array_equal(got2["out"].view(np.uint32), want2["out"].view(np.uint32))
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+def test_per_channel_activation_zero_points(orc, stride):
+    """one integer zero point per channel in front of a padded depthwise convolution: the halo holds every channel's
+    own level, the accumulators start from each channel's own correction"""
+    from dldt_amd import builders
+    g, feeds, meta = builders.per_channel_zero_point_net(stride=stride)
+    keep = [a["node"] for a in meta["acts"].values()]
+    want, kept = evaluate(orc, g.nodes, feeds, keep=keep)
+    plan = g.compile()
+    req = plan.create_request()
+    (got,) = req.infer(feeds["data"])
+    for name, a in meta["acts"].items():
+        np.testing.assert_array_equal(req.tensor(a["node"]), kept[a["node"]], err_msg=name)
+    np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))
