@@ -625,3 +625,43 @@ def per_channel_zero_point_net(seed=47, n=2, c=48, hw=17, oc=40, stride=1):
     b2 = (rng.standard_normal(oc, dtype=np.float32) * np.float32(0.2)).astype(np.float32)
     g.result(net.conv_f32(a1, w2, b2), "out")
     return g, dict(data=x), dict(acts=dict(a0=a0, a1=a1))
+
+
+def matmul_zero_point_net(seed=53, batch=2, seq=48, hidden=128, ffn=192):
+    """Row-major (transformer) path with asymmetric u8 activations: LayerNorm -> FakeQuantize(u8, zero point) ->
+    MatMul' -> Subtract(zero point x column sums of the weights) -> Add(b / s) -> FakeQuantize(u8, zero point; the
+    dequantization folded into its range) -> MatMul' -> Subtract -> Add -> Multiply(s) -> + residual, i.e. what
+    MatMulTransformation leaves when the activations in front of a MatMul have a zero point (mat_mul.cpp:95-121:
+    the Subtract moves BEHIND the MatMul as zero point x weights).  Returns (graph, meta)."""
+    rng = np.random.default_rng(seed)
+    net = QuantizedNet()
+    g = net.g
+    nrm = lambda *shape, s=0.05: (rng.standard_normal(shape, dtype=np.float32) * np.float32(s)).astype(np.float32)
+    x = g.parameter("hidden_states", (batch, seq, hidden))
+    n = g.mvn(x, (-1,), True, 1e-5, True)
+    h = g.add(g.multiply(n, g.constant(np.float32(1) + nrm(hidden))), g.constant(nrm(hidden) + np.float32(0.4)))
+
+    def fq_u8(v, lo, hi, fold=None):
+        d = lpt.decompose_fake_quantize(256, np.float32(lo), np.float32(hi), allow_zero_point=True)
+        assert d["has_zero_point"] and d["precision"] == U8
+        il, ih = (np.float32(lo), np.float32(hi)) if fold is None else lpt.fuse_elementwise(lpt.MULTIPLY, np.float32(lo), np.float32(hi), fold)
+        q = g.fake_quantize(v, il, ih, d["new_low"], d["new_high"], 256, U8)
+        return dict(node=q, scale=np.float32(d["scale"]).reshape(()), zero_point=np.float32(lpt.round_zero_point(d["shift"])).reshape(()))
+
+    def linear(act, w, b):
+        """MatMul' -> Subtract(zp * sum_k w) -> Add(b / s): returns (node, s[c])"""
+        wq, s_w = lpt.quantize_weights(w, 255)
+        s = (np.float32(act["scale"]) * s_w).astype(np.float32)
+        y = g.matmul(act["node"], g.constant(wq, I8), False, True)
+        # fold<MatMul>(broadcast(zero point) [1, K], weights): one f32 product per column, exact integers here
+        corr = (np.full((1, wq.shape[1]), act["zero_point"], np.float32) @ wq.astype(np.float32).T).reshape(-1).astype(np.float32)
+        y = g.subtract(y, g.constant(corr))
+        return g.add(y, g.constant(lpt.swap_multiply_and_add(b, s))), s
+
+    a0 = fq_u8(h, -1.6, 2.9)
+    y1, s1 = linear(a0, nrm(ffn, hidden), nrm(ffn, s=0.3))
+    a1 = fq_u8(y1, -0.7, 1.9, fold=s1)
+    y2, s2 = linear(a1, nrm(hidden, ffn), nrm(hidden, s=0.3))
+    out = g.add(g.multiply(y2, g.constant(s2)), h)
+    g.result(out, "out")
+    return g, dict(norm=h, a0=a0["node"], a1=a1["node"], zero_points=(float(a0["zero_point"]), float(a1["zero_point"])))

@@ -1422,7 +1422,7 @@ void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weight
                     // stored byte = level - 128 (U8B) or level (I8); the product wanted is (level - zero point) * w
                     corr += static_cast<int64_t>(stored_zero - zero_point_of(d, ic)) * v;
                 }
-        cr[oc] = static_cast<int32_t>(corr);
+        cr[oc] = static_cast<int32_t>(corr - (d.acc_sub ? d.acc_sub[oc] : 0));
     });
     if (device >= 0) {
         wgt.upload(device, w.data(), w.size());
@@ -1581,7 +1581,9 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
         auto c = std::make_unique<hipie_conv>();
         c->device = device;
         c->d = d;
-        c->d.in_zero_points = nullptr;   // the caller's array is read during this call only
+        c->d.in_zero_points = nullptr;   // the caller's arrays are read during this call only
+        c->d.acc_sub = nullptr;
+        HIPIE_REQUIRE(!(depthwise && d.acc_sub), HIPIE_NOT_IMPLEMENTED, "hipie_conv_create: acc_sub on a depthwise convolution");
         if (depthwise) {
             // weights [C][kh][kw] -> [kh*kw][OCp]; corr = 128 * sum of the channel's taps
             HIPIE_REQUIRE(d.in_c_stride % 16 == 0, HIPIE_NOT_IMPLEMENTED,
@@ -1656,6 +1658,7 @@ int hipie_conv_create_fused(int device, const hipie_conv_desc* desc, const int8_
         c->fused = true;
         c->sd = sd;
         c->sd.in_zero_points = nullptr;
+        c->sd.acc_sub = nullptr;
         c->sg.pack(device, sd, shortcut_weights);
         std::vector<float> b(c->OCp, 0.f), s(c->OCp, 1.f);
         for (int oc = 0; oc < sd.oc; ++oc) {

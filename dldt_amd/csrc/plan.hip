@@ -177,6 +177,7 @@ struct ConvStep : Step {
     std::vector<int8_t> weights;   // OIHW
     EpilogueSpec epi;
     std::vector<int32_t> zero_points;   // per input channel (a per-channel Subtract in front of the convolution), or empty
+    std::vector<int32_t> acc_sub;       // per output channel (the Subtract behind a MatMul with a zero point), or empty
     hipie_conv* conv = nullptr;
     int64_t in_w_bytes = 0;        // input + weight bytes (what a fused consumer still has to read)
     // projection shortcut (Conv' -> Add -> Multiply, f32, used only by this step's residual Add):
@@ -191,6 +192,7 @@ struct ConvStep : Step {
         desc.in_stride_w = t.cs;
         desc.in_stride_h = t.wp() * t.cs;
         desc.in_zero_points = zero_points.empty() ? nullptr : zero_points.data();
+        desc.acc_sub = acc_sub.empty() ? nullptr : acc_sub.data();
     }
     void create(int device, const std::vector<TensorInfo>& tensors) override {
         fill_desc(tensors);
@@ -468,6 +470,7 @@ struct MatFqStep : Step {
     int out = -1;
     int64_t n = 0, levels = 0;
     float il = 0, ih = 0, ol = 0, oh = 0;
+    int out_dtype = HIPIE_I8;      // HIPIE_U8B: u8 levels stored as level - 128
     hipie_fq* fq = nullptr;
     ~MatFqStep() override { hipie_fq_destroy(fq); }
     void create(int device, const std::vector<TensorInfo>&) override {
@@ -476,7 +479,7 @@ struct MatFqStep : Step {
     void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
              hipStream_t s) const override {
         check_status(hipie_fq_run_q8(fq, reinterpret_cast<const float*>(in.ptr(arena, tensors, inputs)),
-                                     arena + tensors[out].offset, 1, n, HIPIE_I8, HIPIE_NCHW, 0, s), name.c_str());
+                                     arena + tensors[out].offset, 1, n, static_cast<hipie_dtype>(out_dtype), HIPIE_NCHW, 0, s), name.c_str());
     }
 };
 
@@ -926,8 +929,9 @@ struct Planner {
     void plan_mat_fq(int id) {
         const GNode& n = N(id);
         const View x = dense_f32_input(id, "FakeQuantize input must be a dense f32 value");
-        if (n.dtype != HIPIE_I8) unsupported(id, "activations of the row-major path are symmetric i8");
+        if (n.dtype != HIPIE_I8 && n.dtype != HIPIE_U8) unsupported(id, "activations of the row-major path are i8 or u8 levels");
         auto st = std::make_unique<MatFqStep>();
+        st->out_dtype = storage_type(n.dtype);
         float* dst[4] = {&st->il, &st->ih, &st->ol, &st->oh};
         for (int i = 0; i < 4; ++i) {
             std::vector<float> c;
@@ -937,20 +941,25 @@ struct Planner {
         st->in = x;
         st->n = n.numel();
         st->levels = n.levels;
-        st->out = new_matrix(id, HIPIE_I8, n.shape);
+        st->out = new_matrix(id, st->out_dtype, n.shape);
         st->name = n.name;
         st->type = "FakeQuantize";
         st->bytes = n.numel() * 5;
         st->out_node = id;
-        set_matrix_value(id, st->out, HIPIE_I8);
+        set_matrix_value(id, st->out, st->out_dtype);
         steps.push_back(std::move(st));
     }
 
     // FakeQuantize node `u` on value `x` with per-tensor bounds whose outputs are the i8 integers
     // out_low + k: can be evaluated inside the kernel that produces x
-    bool fusable_requant(int u, int x, hipie_requant& rq) const {
+    // `storage`: where the caller can take u8 levels too, it receives the storage type (HIPIE_I8, or HIPIE_U8B: level - 128);
+    // without it only i8 is accepted
+    bool fusable_requant(int u, int x, hipie_requant& rq, int* storage = nullptr) const {
         const GNode& f = N(u);
-        if (f.op != OP_FAKE_QUANTIZE || f.in[0] != x || f.dtype != HIPIE_I8 || f.levels < 2 || f.levels > 256) return false;
+        if (f.op != OP_FAKE_QUANTIZE || f.in[0] != x || (f.dtype != HIPIE_I8 && !(f.dtype == HIPIE_U8 && storage)) || f.levels < 2 ||
+            f.levels > 256)
+            return false;
+        if (storage) *storage = f.dtype == HIPIE_U8 ? HIPIE_U8B : HIPIE_I8;
         float b[4];
         for (int i = 0; i < 4; ++i) {
             std::vector<float> c;
@@ -958,12 +967,13 @@ struct Planner {
             b[i] = c[0];
         }
         const float lm1 = static_cast<float>(f.levels - 1);
-        if (!(b[0] < b[1]) || b[2] != std::nearbyintf(b[2]) || b[2] < -128.f || b[3] != b[2] + lm1 || b[3] > 127.f) return false;
+        const float lo_level = f.dtype == HIPIE_U8 ? 0.f : -128.f;
+        if (!(b[0] < b[1]) || b[2] != std::nearbyintf(b[2]) || b[2] < lo_level || b[3] != b[2] + lm1 || b[3] > lo_level + 255.f) return false;
         for (int k = 0; k < f.levels; ++k)
             if (static_cast<float>(k) / lm1 * (b[3] - b[2]) + b[2] != b[2] + static_cast<float>(k)) return false;
         rq.in_low = b[0];
         rq.in_high = b[1];
-        rq.out_low = b[2];
+        rq.out_low = f.dtype == HIPIE_U8 ? b[2] - 128.f : b[2];   // u8 levels are stored as level - 128
         rq.levels = f.levels;
         return true;
     }
@@ -1002,9 +1012,9 @@ struct Planner {
         // A per-tensor FakeQuantize to i8 among the users rides in the same kernel; the f32 result is
         // then only stored when something else reads it too (rows the kernel cannot keep in registers
         // need it as well).
-        int fq_node = -1;
+        int fq_node = -1, fq_storage = HIPIE_I8;
         for (int u : N(cur).users)
-            if (fq_node < 0 && fusable_requant(u, cur, st->rq)) fq_node = u;
+            if (fq_node < 0 && fusable_requant(u, cur, st->rq, &fq_storage)) fq_node = u;
         const bool keep = fq_node < 0 || N(cur).users.size() > 1 || keep_f32 || C % 4 != 0 || C > 4096;
         if (keep) {
             st->out = new_matrix(cur, HIPIE_F32, n.shape);
@@ -1013,8 +1023,8 @@ struct Planner {
             values[cur].kind = VK_FUSED;
         }
         if (fq_node >= 0) {
-            st->outq = new_matrix(fq_node, HIPIE_I8, n.shape);
-            set_matrix_value(fq_node, st->outq, HIPIE_I8);
+            st->outq = new_matrix(fq_node, fq_storage, n.shape);
+            set_matrix_value(fq_node, st->outq, fq_storage);
         }
         st->name = N(fq_node >= 0 ? fq_node : cur).name;
         st->type = std::string(op_name(n.op)) + (fq_node >= 0 ? "+FakeQuantize" : "");
@@ -1094,9 +1104,11 @@ struct Planner {
     void plan_mat_matmul(int id) {
         const GNode& n = N(id);
         const Value a = value(n.in[0]);
-        if (a.view.dtype != HIPIE_I8) unsupported(id, "left operand must be quantized to i8");
+        const bool weights = N(n.in[1]).op == OP_CONSTANT;
+        if (a.view.dtype != HIPIE_I8 && !(weights && a.view.dtype == HIPIE_U8B))
+            unsupported(id, weights ? "left operand must be quantized (i8 or u8)" : "operands of a MatMul between activations must be i8");
         if (n.ta) unsupported(id, "transpose_a");
-        if (N(n.in[1]).op == OP_CONSTANT) plan_linear(id, a.view);
+        if (weights) plan_linear(id, a.view);
         else plan_batch_matmul(id, a.view);
     }
 
@@ -1104,6 +1116,7 @@ struct Planner {
     // the elementwise chain behind a MatMul against constant weights
     struct LinearChain {
         EpilogueSpec e;
+        std::vector<int32_t> acc_sub;   // the integer Subtract behind a MatMul whose activations have a zero point
         int cur = -1, res = -1, res_param = -1;
         bool residual = false;
     };
@@ -1115,7 +1128,16 @@ struct Planner {
         while (single_user(cur)) {
             const int nx = N(cur).users[0];
             const GNode& u = N(nx);
-            if (u.op == OP_ADD || u.op == OP_MULTIPLY) {
+            if (u.op == OP_SUBTRACT && cur == id && u.in[0] == cur) {
+                // DequantizationSubtract right behind the MatMul (mat_mul.cpp:95-121): zero point x column sums of the
+                // weights, integers that go into the accumulators' start
+                std::vector<float> c;
+                if (!last_axis_constant(u.in[1], OC, c)) break;
+                for (float v : c)
+                    if (v != std::nearbyintf(v) || std::fabs(v) >= 16777216.f) unsupported(nx, "MatMul zero-point correction that is not an integer");
+                if (c.size() == 1) c.assign(static_cast<size_t>(OC), c[0]);
+                for (float v : c) ch.acc_sub.push_back(static_cast<int32_t>(v));
+            } else if (u.op == OP_ADD || u.op == OP_MULTIPLY) {
                 const int other = u.in[0] == cur ? u.in[1] : u.in[0];
                 std::vector<float> c;
                 if (last_axis_constant(other, OC, c)) {
@@ -1138,10 +1160,10 @@ struct Planner {
                     break;
                 }
             } else if (u.op == OP_GELU && stage < 5 && !keep_f32 && single_user(nx) && N(N(nx).users[0]).op == OP_FAKE_QUANTIZE &&
-                       N(N(nx).users[0]).dtype == HIPIE_I8) {
+                       (N(N(nx).users[0]).dtype == HIPIE_I8 || N(N(nx).users[0]).dtype == HIPIE_U8)) {
                 e.activation = 3;   // Gelu and the FakeQuantize behind it ride in the GEMM: its f32 result is never stored
                 stage = 5;
-            } else if (u.op == OP_FAKE_QUANTIZE && u.in[0] == cur && u.dtype == HIPIE_I8) {
+            } else if (u.op == OP_FAKE_QUANTIZE && u.in[0] == cur && (u.dtype == HIPIE_I8 || u.dtype == HIPIE_U8)) {
                 std::vector<float> ol, oh;
                 if (!last_axis_constant(u.in[1], OC, e.fq_il) || !last_axis_constant(u.in[2], OC, e.fq_ih) ||
                     !last_axis_constant(u.in[3], -1, ol) || !last_axis_constant(u.in[4], -1, oh))
@@ -1149,7 +1171,7 @@ struct Planner {
                 e.fq_ol = ol[0];
                 e.fq_oh = oh[0];
                 e.levels = u.levels;
-                e.out_dtype = HIPIE_I8;
+                e.out_dtype = storage_type(u.dtype);
                 cur = nx;
                 break;
             } else {
@@ -1190,7 +1212,7 @@ struct Planner {
         st->in = av.tensor;
         if (tensors[av.tensor].w != T || tensors[av.tensor].c != IC) {   // same bytes, other row split
             if (IC % 16 != 0) unsupported(id, "reduction length must be a multiple of 16");
-            st->in = new_tensor(tensors[av.tensor].producer, HIPIE_I8, 1, 1, static_cast<int>(T), static_cast<int>(IC),
+            st->in = new_tensor(tensors[av.tensor].producer, tensors[av.tensor].dtype, 1, 1, static_cast<int>(T), static_cast<int>(IC),
                                 static_cast<int>(IC));
             tensors[st->in].alias = av.tensor;
         }
@@ -1201,7 +1223,7 @@ struct Planner {
         std::vector<LinearChain> chains(1, ch);
         std::vector<int64_t> ocs(1, OC);
         auto mergeable = [](const LinearChain& c) {
-            return !c.residual && c.e.out_dtype == HIPIE_I8 && !c.e.bias.empty() && c.e.scale.empty();
+            return !c.residual && c.acc_sub.empty() && c.e.out_dtype == HIPIE_I8 && !c.e.bias.empty() && c.e.scale.empty();
         };
         if (merge_linear && mergeable(ch) && OC % 16 == 0) {
             for (int u : N(n.in[0]).users) {
@@ -1243,6 +1265,18 @@ struct Planner {
         }
         st->res = ch.res;
         st->res_param = ch.res_param;
+        if (!ch.acc_sub.empty()) {
+            // The reference converts the raw u8 x i8 sum to f32 and subtracts there; starting the accumulator from
+            // -correction gives the same float exactly when neither the raw sum nor the difference can leave the 24 bits
+            // a float holds: 2 * 255 * sum_k |w[k][oc]| < 2^24 for every output channel.
+            for (int64_t o = 0; o < OC; ++o) {
+                int64_t mag = 0;
+                for (int64_t k = 0; k < IC; ++k) mag += std::abs(static_cast<int>(st->weights[o * IC + k]));
+                if (510 * mag >= (int64_t(1) << 24))
+                    unsupported(id, "MatMul with a zero point whose accumulators may exceed 2^24 (the f32 subtraction would round)");
+            }
+            st->acc_sub = ch.acc_sub;
+        }
         for (size_t i = 0; i < group.size(); ++i) mark_chain(group[i], chains[i].cur);
         std::vector<int64_t> oshape = N(ch.cur).shape;
         oshape.back() = OCt;

@@ -107,7 +107,8 @@ class hipie_conv_desc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int32) for k in (
         "in_dtype", "ic", "oc", "kh", "kw", "stride_h", "stride_w", "dil_h", "dil_w",
         "pad_top", "pad_left", "pad_bottom", "pad_right", "groups", "in_c_stride",
-        "in_stride_h", "in_stride_w", "in_zero_point")] + [("in_zero_points", ctypes.POINTER(ctypes.c_int32))]
+        "in_stride_h", "in_stride_w", "in_zero_point")] + [("in_zero_points", ctypes.POINTER(ctypes.c_int32)),
+                                                            ("acc_sub", ctypes.POINTER(ctypes.c_int32))]
 
 
 def make_epilogue(bias=None, scale=None, residual_dtype=0, res_sub=None, res_mul=None,
@@ -166,7 +167,7 @@ class Convolution:
                             dilations[0], dilations[1], pads_begin[0], pads_begin[1], pads_end[0],
                             pads_end[1], groups, in_tensor.cs, in_tensor.stride_h, in_tensor.stride_w,
                             0 if zps is not None else int(zero_point),
-                            zps.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)) if zps is not None else None)
+                            zps.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)) if zps is not None else None, None)
         assert zps is None or zps.shape == (self.ic,)
         self.epilogue = epilogue or make_epilogue(out_dtype=I32)
         self._h = ctypes.c_void_p()

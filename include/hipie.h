@@ -204,6 +204,11 @@ typedef struct hipie_conv_desc {
                                              broadcast, convolution.cpp:97-120, holds when the activations in front of a
                                              grouped convolution are quantized per channel); the halo then holds
                                              channel c's level in channel c.  Read during the create call only. */
+    const int32_t* acc_sub;               /* NULL, or one integer per output channel [oc] subtracted from the accumulator:
+                                             the DequantizationSubtract that MatMulTransformation puts BEHIND a MatMul whose
+                                             activations have a zero point (mat_mul.cpp:95-121: the zero point broadcast
+                                             along K and multiplied by the weights, i.e. zp * sum_k w[k][oc]).  Read during
+                                             the create call only. */
 } hipie_conv_desc;
 
 typedef struct hipie_conv hipie_conv;

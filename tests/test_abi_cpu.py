@@ -254,3 +254,33 @@ def test_concat_shape_inference_and_planner_limits():
     assert tuple(plan.outputs[0]["shape"]) == (2, 24 + 40 + 16, 18, 18)
     sup = g2.query()
     assert all(sup)
+
+
+def test_matmul_zero_point_correction_must_be_integers():
+    """the Subtract behind a MatMul with u8 activations goes into the integer accumulators: a constant that is not
+    integer-valued (it is zero point x column sums of i8 weights) is refused, and so is a u8 operand of a MatMul
+    between two activations"""
+    from dldt_amd import HipieError, builders
+    from dldt_amd.graph import Graph
+    from dldt_amd.tensor import I8, U8
+    plan = builders.matmul_zero_point_net()[0].compile(-1)
+    assert [s["type"] for s in plan.steps].count("MatMul") == 2
+
+    def net(corr, between_activations=False):
+        g = Graph()
+        x = g.parameter("x", (2, 16, 32))
+        q = g.fake_quantize(x, -1.0, 2.0, 0.0, 255.0, 256, U8)
+        if between_activations:
+            y = g.matmul(q, q, False, True)
+        else:
+            w = g.constant(np.ones((48, 32), np.int8), I8)
+            y = g.subtract(g.matmul(q, w, False, True), g.constant(np.full(48, corr, np.float32)))
+        g.result(g.multiply(y, g.constant(np.float32(0.01).reshape(()))), "y")
+        return g
+    net(32.0 * 85).compile(-1)
+    with pytest.raises(HipieError) as e:
+        net(2720.5).compile(-1)
+    assert e.value.status == -2 and "integer" in str(e.value)
+    with pytest.raises(HipieError) as e:
+        net(0.0, between_activations=True).compile(-1)
+    assert e.value.status == -2 and "i8" in str(e.value)

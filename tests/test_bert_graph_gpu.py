@@ -219,3 +219,32 @@ def test_encoder_full_size_first_and_last_layer(orc, monkeypatch):
             np.testing.assert_allclose(req.matrix(L[name]).reshape(w.shape), w, err_msg="layer %d %s" % (li, name), **tol)
     np.testing.assert_array_equal(y.reshape(-1, H).view(np.uint32),
                                   req.matrix(meta["layers"][11]["y"]).reshape(-1, H).view(np.uint32))
+
+
+def test_weight_matmuls_with_activation_zero_points(orc):
+    """u8 activations with zero points on the row-major path: the FakeQuantize behind a LayerNorm and the one in a
+    GEMM's epilogue write u8 levels, and the Subtract that MatMulTransformation leaves behind each MatMul (zero
+    point x column sums of the weights) starts the accumulators; everything behind the LayerNorm is bit-exact"""
+    from dldt_amd import builders
+    g, meta = builders.matmul_zero_point_net()
+    assert all(z not in (0.0, 128.0) for z in meta["zero_points"])
+    x = np.random.default_rng(8).normal(0, 1, (2, 48, 128)).astype(np.float32)
+    plan = g.compile(config={"HIP_KEEP_F32": "YES"})
+    types = [s["type"] for s in plan.steps]
+    assert types.count("MatMul") == 2 and "MVN+FakeQuantize" in types
+    req = plan.create_request()
+    (y,) = req.infer(x)
+    device = {meta["norm"]: req.matrix(meta["norm"])}
+    want, kept = evaluate(orc, g.nodes, {"hidden_states": x}, keep=[meta["a0"], meta["a1"]], override=device)
+    np.testing.assert_allclose(device[meta["norm"]].reshape(kept[("oracle", meta["norm"])].shape), kept[("oracle", meta["norm"])],
+                               rtol=1e-5, atol=4e-6)
+    for name in ("a0", "a1"):
+        w = kept[meta[name]]
+        assert w.dtype == np.uint8 and w.min() == 0 and w.max() == 255
+        have = req.matrix(meta[name]).reshape(w.shape)          # stored as level - 128, read back as levels
+        assert have.dtype == np.uint8
+        np.testing.assert_array_equal(have, w, err_msg=name)
+    np.testing.assert_array_equal(y.view(np.uint32), want["out"].view(np.uint32))
+    # without the kept f32 values: the same bits
+    (y2,) = g.compile().create_request().infer(x)
+    np.testing.assert_array_equal(y2.view(np.uint32), y.view(np.uint32))
