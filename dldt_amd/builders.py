@@ -629,7 +629,7 @@ def per_channel_zero_point_net(seed=47, n=2, c=48, hw=17, oc=40, stride=1):
 
 def matmul_zero_point_net(seed=53, batch=2, seq=48, hidden=128, ffn=192):
     """Row-major (transformer) path with asymmetric u8 activations: LayerNorm -> FakeQuantize(u8, zero point) ->
-    MatMul' -> Subtract(zero point x column sums of the weights) -> Add(b / s) -> FakeQuantize(u8, zero point; the
+    MatMul' -> Subtract(zero point x column sums of the weights) -> Add(bias over scale) -> FakeQuantize(u8, zero point; the
     dequantization folded into its range) -> MatMul' -> Subtract -> Add -> Multiply(s) -> + residual, i.e. what
     MatMulTransformation leaves when the activations in front of a MatMul have a zero point (mat_mul.cpp:95-121:
     the Subtract moves BEHIND the MatMul as zero point x weights).  Returns (graph, meta)."""
@@ -665,3 +665,31 @@ def matmul_zero_point_net(seed=53, batch=2, seq=48, hidden=128, ffn=192):
     out = g.add(g.multiply(y2, g.constant(s2)), h)
     g.result(out, "out")
     return g, dict(norm=h, a0=a0["node"], a1=a1["node"], zero_points=(float(a0["zero_point"]), float(a1["zero_point"])))
+
+
+def eltwise_net(seed=59, n=2, c=24, hw=14, oc=40):
+    """Elementwise nodes that no convolution absorbs: two pooled, dequantized u8 branches added, ReLU and a
+    FakeQuantize behind the Add (one kernel); the product of two f32 convolution results, clamped (one kernel, f32
+    result); a FakeQuantize of that f32 value on its own; a Subtract with a per-channel constant on the left.
+    Returns (graph, feeds, meta)."""
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(0, 1, (n, c, hw, hw)).astype(np.float32)
+    net = QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    w = lambda o, i, k, s: (rng.standard_normal((o, i, k, k), dtype=np.float32) * np.float32(s)).astype(np.float32)
+    b = lambda o: (rng.standard_normal(o, dtype=np.float32) * np.float32(0.2)).astype(np.float32)
+    a1 = net.conv(a0, w(oc, c, 3, 0.08), b(oc), 2.0, pads=(1, 1))
+    a2 = net.conv(a0, w(oc, c, 1, 0.15), b(oc), 3.0)
+    p1 = net.max_pool(a1, (3, 3), (1, 1), (1, 1))
+    p2 = net.max_pool(a2, (3, 3), (1, 1), (1, 1))
+    s = g.relu(g.add(net.dequantize(p1), net.dequantize(p2)))                 # Add of two dequantized byte tensors
+    a3 = net.requantize(s, 4.0)
+    f1 = net.conv_f32(a3, w(oc, oc, 1, 0.1), b(oc))
+    f2 = net.conv_f32(a1, w(oc, oc, 3, 0.04), b(oc), pads=(1, 1))
+    prod = g.clamp(g.multiply(f1, f2), -1.5, 2.5)                             # f32 x f32, Clamp behind it
+    g.result(prod, "prod")
+    a4 = net.requantize(prod, 2.5, signed=True)                               # FakeQuantize of a computed f32 value
+    left = g.subtract(g.constant(net._channel(np.linspace(-1, 1, oc).astype(np.float32), 4)), net.dequantize(a4))
+    g.result(left, "left")
+    return g, dict(data=x), dict(acts=dict(a3=a3, a4=a4))

@@ -15,4 +15,34 @@ bool fq_reciprocal_exact_on_boundaries(const FqChannel& p, float lm1);
 // r = correctly rounded 1/d
 float fq_rounded_reciprocal(float d);
 
+// Elementwise nodes that no convolution / pooling / MatMul chain absorbs, on NHWC operands:
+//     out = FakeQuantize?( act?( op(a, b) ) ),  op in {none (unary), Add, Subtract, Multiply}, a and b in graph order.
+// An operand is a per-channel constant, an f32 tensor, or a byte tensor behind its dequantization
+// (float(level) - sub[c]) * mul[c].  Reference: reference::add / subtract / multiply (autobroadcast_binop.hpp), relu.hpp,
+// clamp.hpp, fake_quantize.hpp:175-194, each step one f32 operation as in the graph.
+struct EltOperand {
+    const void* p = nullptr;          // tensor element (0, 0, 0, 0); null when the operand is `konst`
+    int32_t dtype = 0;                // HIPIE_F32, HIPIE_U8B or HIPIE_I8
+    int64_t sn = 0, sh = 0, sw = 0;   // element strides
+    const float* sub = nullptr;       // per channel, padded to a multiple of 4, or null
+    const float* mul = nullptr;
+    const float* konst = nullptr;     // per-channel constant operand, padded to a multiple of 4
+};
+struct EltArgs {
+    EltOperand a, b;
+    int32_t op = 0;                   // 0 none, 1 add, 2 subtract, 3 multiply
+    int32_t act = 0;                  // 0 none, 1 relu, 2 clamp(lo, hi)
+    float lo = 0, hi = 0;
+    void* out = nullptr;
+    int32_t out_dtype = HIPIE_F32;    // HIPIE_F32, or HIPIE_U8B / HIPIE_I8 behind a FakeQuantize
+    int64_t out_sn = 0, out_sh = 0, out_sw = 0;
+    int32_t N = 0, H = 0, W = 0, C = 0;
+};
+}  // namespace hipie
+struct hipie_fq;
+namespace hipie {
+// `fq` (null for an f32 result) must give integer levels (hipie_fq_create's q8 form); fq_gives_levels says whether it does
+bool fq_gives_levels(const hipie_fq* fq);
+void run_eltwise(const hipie_fq* fq, const EltArgs& a, hipStream_t s);
+
 }  // namespace hipie

@@ -432,6 +432,108 @@ void run_q8_tensor(const hipie_fq* fq, const TIn* x, const hipie_tensor* out, vo
     }
 }
 
+namespace {
+
+__device__ __forceinline__ void elt_load4(const EltOperand& o, int64_t pix_off, int c0, float (&v)[4]) {
+    if (o.konst) {
+        const float4 k = *reinterpret_cast<const float4*>(o.konst + c0);
+        v[0] = k.x; v[1] = k.y; v[2] = k.z; v[3] = k.w;
+        return;
+    }
+    if (o.dtype == HIPIE_F32) {
+        const float4 k = *reinterpret_cast<const float4*>(static_cast<const float*>(o.p) + pix_off + c0);
+        v[0] = k.x; v[1] = k.y; v[2] = k.z; v[3] = k.w;
+    } else {
+        const uint32_t w = *reinterpret_cast<const uint32_t*>(static_cast<const int8_t*>(o.p) + pix_off + c0);
+        const int bias = o.dtype == HIPIE_U8B ? 128 : 0;   // stored byte = level - 128
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = static_cast<float>(static_cast<int>(static_cast<int8_t>(w >> (8 * j))) + bias);   // Convert
+    }
+    if (o.sub) {
+        const float4 k = *reinterpret_cast<const float4*>(o.sub + c0);
+        v[0] = v[0] - k.x; v[1] = v[1] - k.y; v[2] = v[2] - k.z; v[3] = v[3] - k.w;
+    }
+    if (o.mul) {
+        const float4 k = *reinterpret_cast<const float4*>(o.mul + c0);
+        v[0] = v[0] * k.x; v[1] = v[1] * k.y; v[2] = v[2] * k.z; v[3] = v[3] * k.w;
+    }
+}
+
+// a thread computes four consecutive channels of one pixel
+template <bool RCP>
+__global__ __launch_bounds__(kThreads) void eltwise_nhwc_kernel(const EltArgs a, const FqChannel* __restrict__ tab, float lm1, float off,
+                                                                int32_t groups, float inv_groups, float inv_W, float inv_HW,
+                                                                int64_t total) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    auto divmod = [](int64_t v, int32_t d, float inv, int32_t& q, int32_t& r) {   // exact below 2^24 after one correction
+        q = static_cast<int32_t>(static_cast<float>(v) * inv);
+        int64_t rem = v - static_cast<int64_t>(q) * d;
+        if (rem < 0) { --q; rem += d; }
+        else if (rem >= d) { ++q; rem -= d; }
+        r = static_cast<int32_t>(rem);
+    };
+    int32_t pix, g, n, hw, h, w;
+    divmod(idx, groups, inv_groups, pix, g);
+    divmod(pix, a.H * a.W, inv_HW, n, hw);
+    divmod(hw, a.W, inv_W, h, w);
+    const int c0 = 4 * g;
+    float v[4], u[4];
+    elt_load4(a.a, n * a.a.sn + h * a.a.sh + w * a.a.sw, c0, v);
+    if (a.op != 0) {
+        elt_load4(a.b, n * a.b.sn + h * a.b.sh + w * a.b.sw, c0, u);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = a.op == 1 ? v[j] + u[j] : (a.op == 2 ? v[j] - u[j] : v[j] * u[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (a.act == 1) v[j] = v[j] > 0.0f ? v[j] : 0.0f;                                    // relu.hpp
+        else if (a.act == 2) v[j] = v[j] < a.lo ? a.lo : (v[j] > a.hi ? a.hi : v[j]);        // clamp.hpp
+    }
+    const int64_t o = n * a.out_sn + h * a.out_sh + w * a.out_sw + c0;
+    if (tab) {
+        float k[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) k[j] = c0 + j < a.C ? fq_level_clamped<RCP>(tab[c0 + j], lm1, v[j]) : 0.0f;
+        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(a.out) + o) = pack_levels(k[0], k[1], k[2], k[3], off);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = c0 + j < a.C ? v[j] : 0.0f;
+        *reinterpret_cast<float4*>(static_cast<float*>(a.out) + o) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+}
+
+}  // namespace
+
+bool hipie::fq_gives_levels(const hipie_fq* fq) { return fq && fq->q8_ok && fq->clamp_ok; }
+
+void hipie::run_eltwise(const hipie_fq* fq, const EltArgs& a, hipStream_t s) {
+    const int64_t pixels = static_cast<int64_t>(a.N) * a.H * a.W;
+    if (pixels == 0 || a.C == 0) return;
+    const int32_t groups = static_cast<int32_t>(ceil_div(a.C, 4));
+    HIPIE_REQUIRE(pixels < (1 << 24), HIPIE_OUT_OF_BOUNDS, "elementwise step: %lld pixels", (long long)pixels);
+    const int64_t total = pixels * groups;
+    float lm1 = 0.f, off = 0.f;
+    const FqChannel* tab = nullptr;
+    bool rcp = false;
+    if (a.out_dtype != HIPIE_F32) {
+        HIPIE_REQUIRE(fq_gives_levels(fq) && fq->table.ptr && fq->C == a.C, HIPIE_NOT_IMPLEMENTED,
+                      "elementwise step: the FakeQuantize behind it must give consecutive integer levels");
+        HIPIE_REQUIRE(a.out_dtype == HIPIE_U8B ? fq->q8_base >= 0 : fq->q8_base + fq->lm1 <= 127.0f, HIPIE_PARAMETER_MISMATCH,
+                      "elementwise step: levels do not fit the output type");
+        tab = fq->table.as<FqChannel>();
+        lm1 = fq->lm1;
+        off = a.out_dtype == HIPIE_U8B ? fq->q8_base - 128.0f : fq->q8_base;
+        rcp = fq->rcp;
+    }
+    DeviceGuard g(fq ? fq->device : 0);
+    const dim3 grid(static_cast<uint32_t>(ceil_div(total, kThreads))), block(kThreads);
+    const float ig = 1.0f / static_cast<float>(groups), iw = 1.0f / static_cast<float>(a.W), ihw = 1.0f / static_cast<float>(a.H * a.W);
+    if (rcp) hipLaunchKernelGGL(eltwise_nhwc_kernel<true>, grid, block, 0, s, a, tab, lm1, off, groups, ig, iw, ihw, total);
+    else hipLaunchKernelGGL(eltwise_nhwc_kernel<false>, grid, block, 0, s, a, tab, lm1, off, groups, ig, iw, ihw, total);
+    HIPIE_CHECK_HIP(hipGetLastError());
+}
+
 extern "C" {
 
 int hipie_fq_create(int device, int64_t channels, int64_t levels, const float* in_low,

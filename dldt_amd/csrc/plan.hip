@@ -11,6 +11,7 @@
 #include <condition_variable>
 #include <mutex>
 
+#include "fq.h"
 #include "graph.h"
 #include "requant.h"
 
@@ -428,6 +429,70 @@ struct ConcatStep : Step {
     }
 };
 
+// Elementwise nodes that no other step absorbs (run_eltwise in fq.hip): op(a, b) [-> Relu | Clamp] [-> FakeQuantize]
+struct EltwiseStep : Step {
+    struct Operand {
+        int tensor = -1;                 // arena tensor, or -1: per-channel constant
+        std::vector<float> sub, mul, konst;
+        DeviceBuffer d_sub, d_mul, d_konst;
+    };
+    Operand a, b;
+    int op = 0, act = 0;
+    float lo = 0, hi = 0;
+    int out = -1;
+    // FakeQuantize behind it
+    bool quantize = false;
+    int64_t levels = 0;
+    std::vector<float> il, ih;
+    float ol = 0, oh = 0;
+    hipie_fq* fq = nullptr;
+    ~EltwiseStep() override { hipie_fq_destroy(fq); }
+    void create(int device, const std::vector<TensorInfo>& tensors) override {
+        const int C = tensors[out].c;
+        if (quantize) {
+            check_status(hipie_fq_create(device, C, levels, il.data(), il.size(), ih.data(), ih.size(), &ol, 1, &oh, 1, &fq), name.c_str());
+            HIPIE_REQUIRE(fq_gives_levels(fq), HIPIE_NOT_IMPLEMENTED, "%s: FakeQuantize whose outputs are not consecutive integer levels",
+                          name.c_str());
+        }
+        if (device < 0) return;
+        const size_t padded = static_cast<size_t>(round_up(C, 4));
+        auto up = [&](const std::vector<float>& v, DeviceBuffer& d, float pad) {
+            if (v.empty()) return;
+            std::vector<float> o(padded, pad);
+            for (int c = 0; c < C; ++c) o[c] = v[v.size() == 1 ? 0 : c];
+            d.upload(device, o.data(), o.size() * 4);
+        };
+        for (Operand* o : {&a, &b}) {
+            up(o->sub, o->d_sub, 0.f);
+            up(o->mul, o->d_mul, 1.f);
+            up(o->konst, o->d_konst, 0.f);
+        }
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const*, void* const*, hipStream_t s) const override {
+        EltArgs e;
+        auto fill = [&](const Operand& o, EltOperand& d) {
+            if (o.tensor >= 0) {
+                const hipie_tensor t = tensors[o.tensor].desc(arena);
+                d.p = t.data;
+                d.dtype = t.dtype;
+                d.sn = t.stride_n; d.sh = t.stride_h; d.sw = t.stride_w;
+            }
+            d.sub = o.sub.empty() ? nullptr : o.d_sub.as<float>();
+            d.mul = o.mul.empty() ? nullptr : o.d_mul.as<float>();
+            d.konst = o.konst.empty() ? nullptr : o.d_konst.as<float>();
+        };
+        fill(a, e.a);
+        if (op != 0) fill(b, e.b);
+        e.op = op; e.act = act; e.lo = lo; e.hi = hi;
+        const hipie_tensor t = tensors[out].desc(arena);
+        e.out = t.data;
+        e.out_dtype = t.dtype;
+        e.out_sn = t.stride_n; e.out_sh = t.stride_h; e.out_sw = t.stride_w;
+        e.N = t.n; e.H = t.h; e.W = t.w; e.C = t.c;
+        run_eltwise(fq, e, s);
+    }
+};
+
 struct ExitStep : Step {
     int in = -1, result_index = 0, C = 0;
     bool out_u8 = false;
@@ -798,10 +863,23 @@ struct Planner {
         switch (n.op) {
         case OP_PARAMETER: plan_parameter(id); break;
         case OP_CONSTANT: values[id].kind = VK_CONST; break;
-        case OP_FAKE_QUANTIZE: mat ? plan_mat_fq(id) : plan_fake_quantize(id); break;
+        case OP_FAKE_QUANTIZE:
+            if (mat) plan_mat_fq(id);
+            else if (value(n.in[0]).kind == VK_PARAM) plan_fake_quantize(id);
+            else plan_eltwise(id);
+            break;
         case OP_MATMUL: mat ? plan_mat_matmul(id) : plan_conv(id); break;
         case OP_CONVOLUTION: case OP_GROUP_CONVOLUTION: plan_conv(id); break;
-        case OP_CONVERT: case OP_SUBTRACT: case OP_MULTIPLY: plan_dequant(id); break;
+        case OP_CONVERT: plan_dequant(id); break;
+        case OP_SUBTRACT: case OP_MULTIPLY:
+            // the dequantization of a byte tensor stays symbolic; anything else is an elementwise step of its own
+            if (value(n.in[0]).kind == VK_DEQ && N(n.in[1]).op == OP_CONSTANT && value(n.in[0]).mul.empty() &&
+                (n.op == OP_MULTIPLY || value(n.in[0]).sub.empty()))
+                plan_dequant(id);
+            else
+                plan_eltwise(id);
+            break;
+        case OP_ADD: case OP_RELU: case OP_CLAMP: plan_eltwise(id); break;
         case OP_MAX_POOL: case OP_AVG_POOL: plan_pool(id); break;
         case OP_RESHAPE: mat ? plan_mat_reshape(id) : plan_reshape(id); break;
         case OP_TRANSPOSE: plan_mat_transpose(id); break;
@@ -1918,6 +1996,83 @@ struct Planner {
         st->out_node = id;
         values[id].kind = VK_TENSOR;
         values[id].tensor = st->out;
+        steps.push_back(std::move(st));
+    }
+
+    // An elementwise node nothing absorbed: Add / Subtract / Multiply of two values (or a value and a per-channel
+    // constant in an order a dequantization does not have), Relu, Clamp, or a FakeQuantize of a computed value; with the
+    // Relu | Clamp and the FakeQuantize that follow it taken into the same kernel.
+    void plan_eltwise(int id) {
+        const GNode& n = N(id);
+        if (n.shape.size() != 4) unsupported(id, "stand-alone elementwise nodes are planned on 4-D (NHWC) values");
+        int nn, c, h, w;
+        nhwc_dims(n.shape, nn, c, h, w);
+        auto st = std::make_unique<EltwiseStep>();
+        auto operand = [&](int in, EltwiseStep::Operand& o) {
+            if (N(in).op == OP_CONSTANT) {
+                if (!channel_constant(in, c, n.shape.size(), o.konst)) unsupported(id, "elementwise constant must be scalar or per-channel");
+                return;
+            }
+            const Value x = value(in);
+            if (N(in).shape != n.shape) unsupported(id, "elementwise operands of different shapes (broadcast between tensors)");
+            if (x.kind == VK_DEQ) {
+                o.tensor = x.tensor;
+                o.sub = x.sub;
+                o.mul = x.mul;
+            } else if (x.kind == VK_TENSOR && tensors[x.tensor].dtype == HIPIE_F32) {
+                o.tensor = x.tensor;
+            } else {
+                unsupported(id, "elementwise operand must be an f32 tensor or a dequantized byte tensor");
+            }
+        };
+        const bool binary = n.op == OP_ADD || n.op == OP_SUBTRACT || n.op == OP_MULTIPLY;
+        operand(n.in[0], st->a);
+        if (binary) {
+            operand(n.in[1], st->b);
+            st->op = n.op == OP_ADD ? 1 : (n.op == OP_SUBTRACT ? 2 : 3);
+            if (st->a.tensor < 0 && st->b.tensor < 0) unsupported(id, "elementwise node on two constants (constant folding is the front end's)");
+        }
+        int cur = id;
+        auto take_activation = [&](const GNode& u) {
+            if (u.op == OP_RELU) st->act = 1;
+            else { st->act = 2; st->lo = u.lo; st->hi = u.hi; }
+        };
+        auto take_fq = [&](int node) {
+            const GNode& u = N(node);
+            std::vector<float> ol, oh;
+            if (u.dtype == HIPIE_F32 || !channel_constant(u.in[1], c, u.shape.size(), st->il) ||
+                !channel_constant(u.in[2], c, u.shape.size(), st->ih) || !channel_constant(u.in[3], c, u.shape.size(), ol) ||
+                !channel_constant(u.in[4], c, u.shape.size(), oh) || ol.size() != 1 || oh.size() != 1)
+                return false;
+            st->quantize = true;
+            st->levels = u.levels;
+            st->ol = ol[0];
+            st->oh = oh[0];
+            return true;
+        };
+        if (n.op == OP_RELU || n.op == OP_CLAMP) take_activation(n);
+        if (n.op == OP_FAKE_QUANTIZE) {
+            if (!take_fq(id)) unsupported(id, "FakeQuantize with f32 output or bounds that are not per-channel constants");
+        } else {
+            while (single_user(cur) && !st->quantize) {
+                const int nx = N(cur).users[0];
+                const GNode& u = N(nx);
+                if ((u.op == OP_RELU || u.op == OP_CLAMP) && st->act == 0) take_activation(u);
+                else if (u.op == OP_FAKE_QUANTIZE && u.in[0] == cur && take_fq(nx)) {}
+                else break;
+                cur = nx;
+            }
+            mark_chain(id, cur);
+        }
+        const int out_dtype = st->quantize ? storage_type(N(cur).dtype) : HIPIE_F32;
+        st->out = new_tensor(cur, out_dtype, nn, h, w, c);
+        st->name = N(cur).name;
+        st->type = std::string(n.op == OP_FAKE_QUANTIZE ? "FakeQuantize" : op_name(n.op)) + (st->quantize && n.op != OP_FAKE_QUANTIZE ? "+FakeQuantize" : "");
+        st->bytes = n.numel() * ((st->a.tensor >= 0 ? tensors[st->a.tensor].esize() : 0) + (st->b.tensor >= 0 ? tensors[st->b.tensor].esize() : 0) +
+                                 (out_dtype == HIPIE_F32 ? 4 : 1));
+        st->out_node = cur;
+        values[cur].kind = VK_TENSOR;
+        values[cur].tensor = st->out;
         steps.push_back(std::move(st));
     }
 

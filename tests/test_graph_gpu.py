@@ -397,3 +397,24 @@ def test_per_channel_activation_zero_points(orc, stride):
     for name, a in meta["acts"].items():
         np.testing.assert_array_equal(req.tensor(a["node"]), kept[a["node"]], err_msg=name)
     np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))
+
+
+def test_stand_alone_elementwise_nodes(orc):
+    """Add / Multiply / Subtract / Relu / Clamp / FakeQuantize that no convolution absorbs run as steps of their own,
+    with the activation and the FakeQuantize behind them in the same kernel; bit-exact"""
+    from dldt_amd import builders
+    g, feeds, meta = builders.eltwise_net()
+    keep = [a["node"] for a in meta["acts"].values()]
+    want, kept = evaluate(orc, g.nodes, feeds, keep=keep)
+    plan = g.compile()
+    types = [s["type"] for s in plan.steps]
+    assert "Add+FakeQuantize" in types and "Multiply" in types and "Subtract" in types and types.count("FakeQuantize") == 2
+    req = plan.create_request()
+    got = dict(zip([o["name"] for o in plan.outputs], req.infer(feeds["data"])))
+    for name, a in meta["acts"].items():
+        w = kept[a["node"]]
+        assert len(np.unique(w)) > 50
+        np.testing.assert_array_equal(req.tensor(a["node"]).astype(np.int16), w.astype(np.int16), err_msg=name)
+    for name in ("prod", "left"):
+        np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
+    assert all(g.query())
