@@ -70,7 +70,12 @@ class QuantizedNet:
         g = self.g
         wq, s_w = lpt.quantize_weights(w, 255)
         s = (np.float32(act["scale"]) * s_w).astype(np.float32)            # fold<Multiply>(s_a, s_w)
-        if conv_attrs.get("grouped"):
+        groups = conv_attrs.pop("groups", 0)
+        if groups:
+            # [OC, IC / G, kh, kw] -> [G, OC / G, IC / G, kh, kw]
+            wq = wq.reshape(groups, wq.shape[0] // groups, wq.shape[1], wq.shape[2], wq.shape[3])
+            conv_attrs["grouped"] = True
+        elif conv_attrs.get("grouped"):
             # GroupConvolution weights: FQ on [C, 1, kh, kw] then Reshape to [G, 1, 1, kh, kw]
             # (the pattern LPT recognises, group_convolution.cpp:50-52); both fold into one constant
             wq = wq.reshape(wq.shape[0], 1, 1, wq.shape[2], wq.shape[3])
@@ -97,11 +102,13 @@ class QuantizedNet:
         return np.float32(-hi * np.float32(128.0) / np.float32(127.0)), hi
 
     def conv(self, act, w, bias, out_high, strides=(1, 1), pads=(0, 0), dilations=(1, 1), signed=False,
-             grouped=False):
+             grouped=False, groups=0):
         """Quantized conv feeding the next activation FakeQuantize: [0, out_high] -> u8 (ReLU fused
         away) or, for linear outputs, the symmetric range of signed_range(out_high) -> i8."""
         g = self.g
         attrs = dict(strides=strides, dilations=dilations, pads_begin=pads, pads_end=pads, grouped=grouped)
+        if groups:
+            attrs["groups"] = groups
         y, s, rank = self._accumulate(act, w, bias, attrs)
         lo, hi = self.signed_range(out_high) if signed else (np.float32(0), np.float32(out_high))
         d = lpt.decompose_fake_quantize(256, lo, hi)

@@ -1566,10 +1566,25 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
                           d.dil_h > 0 && d.dil_w > 0 && d.pad_top >= 0 && d.pad_left >= 0 &&
                           d.pad_bottom >= 0 && d.pad_right >= 0,
                       HIPIE_PARAMETER_MISMATCH, "hipie_conv_create: bad geometry");
+        HIPIE_REQUIRE(d.groups >= 1 && d.ic % d.groups == 0 && d.oc % d.groups == 0, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_create: groups=%d does not divide ic=%d and oc=%d", d.groups, d.ic, d.oc);
+        if (d.groups > 1 && !(d.groups == d.ic && d.ic == d.oc)) {
+            // A grouped convolution that is not depthwise (weights [oc][ic / groups][kh][kw]) is the dense convolution
+            // with block-diagonal weights: reference::group_convolution (group_convolution.hpp:78-144) convolves every
+            // slice on its own, and the products added here are zeros.
+            const int64_t icg = d.ic / d.groups, ocg = d.oc / d.groups, taps = static_cast<int64_t>(d.kh) * d.kw;
+            std::vector<int8_t> dense(static_cast<size_t>(d.oc) * d.ic * taps, 0);
+            for (int64_t oc = 0; oc < d.oc; ++oc)
+                for (int64_t i = 0; i < icg; ++i)
+                    for (int64_t t = 0; t < taps; ++t)
+                        dense[static_cast<size_t>((oc * d.ic + (oc / ocg) * icg + i) * taps + t)] = weights[(oc * icg + i) * taps + t];
+            hipie_conv_desc dd = d;
+            dd.groups = 1;
+            const int st = hipie_conv_create(device, &dd, dense.data(), epilogue, out);
+            if (st != HIPIE_OK) fail(static_cast<hipie_status>(st), "%s", std::string(hipie_last_error()).c_str());
+            return;
+        }
         const bool depthwise = d.groups > 1;
-        HIPIE_REQUIRE(d.groups == 1 || (d.groups == d.ic && d.ic == d.oc), HIPIE_NOT_IMPLEMENTED,
-                      "hipie_conv_create: groups=%d with ic=%d oc=%d (only dense and depthwise are built)", d.groups,
-                      d.ic, d.oc);
         HIPIE_REQUIRE(d.in_c_stride >= d.ic && d.in_c_stride % 4 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_create: in_c_stride=%d must be a multiple of 4 >= ic=%d", d.in_c_stride, d.ic);
         {

@@ -1737,7 +1737,7 @@ struct Planner {
         const TensorInfo& tin = tensors[x.tensor];
         hipie_conv_desc& d = st->desc;
         d.groups = 1;
-        int64_t OC, IC;
+        int64_t OC, IC, grouped_macs_div = 1;
         if (is_mm) {
             if (n.ta || W.shape.size() != 2 || N(n.in[0]).shape.size() != 2)
                 unsupported(id, "MatMul is planned for [N,K] x constant [K,OC] / [OC,K]^T");
@@ -1750,20 +1750,34 @@ struct Planner {
                 for (int64_t k = 0; k < IC; ++k) st->weights[o * IC + k] = n.tb ? w[o * IC + k] : w[k * OC + o];
         } else {
             const bool grouped = n.op == OP_GROUP_CONVOLUTION;
-            if (grouped) {   // [G, OC/G, IC/G, kh, kw]: only depthwise (one filter per channel) is built
-                if (W.shape[1] != 1 || W.shape[2] != 1)
-                    unsupported(id, "grouped convolution other than depthwise");
-                d.groups = static_cast<int>(W.shape[0]);
-            }
-            OC = grouped ? W.shape[0] : W.shape[0];
-            IC = grouped ? W.shape[0] : W.shape[1];
+            // [G, OC/G, IC/G, kh, kw].  One filter per channel (depthwise) has kernels of its own; any other grouping runs
+            // as the dense convolution with block-diagonal weights it is equal to (reference::group_convolution,
+            // group_convolution.hpp:78-144, convolves each slice on its own: the products outside the blocks are the
+            // zeros added here, and integer sums do not change with them)
+            const bool depthwise = grouped && W.shape[1] == 1 && W.shape[2] == 1;
+            const int64_t G = grouped ? W.shape[0] : 1, ocg = grouped ? W.shape[1] : 0, icg = grouped ? W.shape[2] : 0;
+            if (depthwise) d.groups = static_cast<int>(G);
+            OC = grouped ? G * ocg : W.shape[0];
+            IC = grouped ? G * icg : W.shape[1];
+            grouped_macs_div = grouped && !depthwise ? G : 1;
             d.kh = static_cast<int>(W.shape[grouped ? 3 : 2]); d.kw = static_cast<int>(W.shape[grouped ? 4 : 3]);
             d.stride_h = static_cast<int>(n.strides[0]); d.stride_w = static_cast<int>(n.strides[1]);
             d.dil_h = static_cast<int>(n.dilations[0]); d.dil_w = static_cast<int>(n.dilations[1]);
             d.pad_top = static_cast<int>(n.pads_begin[0]); d.pad_left = static_cast<int>(n.pads_begin[1]);
             d.pad_bottom = static_cast<int>(n.pads_end[0]); d.pad_right = static_cast<int>(n.pads_end[1]);
-            st->weights.assign(reinterpret_cast<const int8_t*>(W.data.data()),
-                               reinterpret_cast<const int8_t*>(W.data.data()) + W.data.size());
+            const int8_t* wsrc = reinterpret_cast<const int8_t*>(W.data.data());
+            if (grouped && !depthwise) {
+                const int64_t taps = static_cast<int64_t>(d.kh) * d.kw;
+                st->weights.assign(static_cast<size_t>(OC * IC * taps), 0);
+                for (int64_t gi = 0; gi < G; ++gi)
+                    for (int64_t o = 0; o < ocg; ++o)
+                        for (int64_t i = 0; i < icg; ++i)
+                            for (int64_t t = 0; t < taps; ++t)
+                                st->weights[static_cast<size_t>(((gi * ocg + o) * IC + gi * icg + i) * taps + t)] =
+                                    wsrc[((gi * ocg + o) * icg + i) * taps + t];
+            } else {
+                st->weights.assign(wsrc, wsrc + W.data.size());
+            }
         }
         d.ic = static_cast<int>(IC);
         d.oc = static_cast<int>(OC);
@@ -1863,8 +1877,8 @@ struct Planner {
         nhwc_dims(N(cur).shape, nn, c, h, w);
         st->out = new_tensor(cur, e.out_dtype, nn, h, w, c);
         st->name = N(cur).name;
-        st->type = is_mm ? "MatMul" : (d.groups > 1 ? "GroupConvolution" : "Convolution");
-        st->macs = N(id).numel() * (d.groups > 1 ? 1 : IC) * d.kh * d.kw + (st->shortcut ? st->shortcut->macs : 0);
+        st->type = is_mm ? "MatMul" : (n.op == OP_GROUP_CONVOLUTION ? "GroupConvolution" : "Convolution");
+        st->macs = N(id).numel() * (d.groups > 1 ? 1 : IC / grouped_macs_div) * d.kh * d.kw + (st->shortcut ? st->shortcut->macs : 0);
         // algorithmic HBM bytes: every operand once (input, weights, output, residual); a fused
         // projection shortcut adds its input and weights and removes the f32 residual round trip
         auto elems = [&](int t) {

@@ -153,10 +153,9 @@ class Convolution:
     def __init__(self, weights, in_tensor, strides=(1, 1), dilations=(1, 1), pads_begin=(0, 0),
                  pads_end=(0, 0), epilogue=None, device=0, zero_point=0):
         w = np.ascontiguousarray(weights, np.int8)
-        if w.ndim == 5:   # GroupConvolution filters [G, OC/G, IC/G, kh, kw]; depthwise only
+        if w.ndim == 5:   # GroupConvolution filters [G, OC/G, IC/G, kh, kw] = [oc][ic / groups][kh][kw] in memory
             groups = w.shape[0]
-            assert w.shape[1] == 1 and w.shape[2] == 1, "only depthwise group convolution"
-            self.oc = self.ic = groups
+            self.oc, self.ic = groups * w.shape[1], groups * w.shape[2]
             self.kh, self.kw = w.shape[3:]
         else:
             groups = 1

@@ -190,7 +190,10 @@ typedef struct hipie_conv_desc {
     int32_t ic, oc, kh, kw;
     int32_t stride_h, stride_w, dil_h, dil_w;
     int32_t pad_top, pad_left, pad_bottom, pad_right;
-    int32_t groups;                       /* 1 */
+    int32_t groups;                       /* 1 = dense (weights [oc][ic][kh][kw]); > 1: weights [oc][ic / groups][kh][kw]
+                                             (group_convolution.hpp:78-144); groups == ic == oc (depthwise) has kernels of
+                                             its own, any other grouping runs as the dense convolution with
+                                             block-diagonal weights that it equals */
     int32_t in_c_stride;                  /* channel stride of the input tensor (>= ic) */
     int32_t in_stride_h, in_stride_w;     /* element strides of the input tensor */
     int32_t in_zero_point;                /* integer level subtracted from every input element: the

@@ -450,6 +450,25 @@ def test_conv_per_channel_input_zero_points(orc, signed, depthwise):
     np.testing.assert_array_equal(out.to_nchw(), want)
 
 
+@pytest.mark.parametrize("G,icg,ocg", [(2, 16, 24), (4, 8, 8), (32, 4, 4), (3, 5, 7)])
+def test_group_convolution_with_several_channels_per_group(orc, G, icg, ocg):
+    """GroupConvolution that is not depthwise (ResNeXt-style cardinality): every group convolved on its own
+    (group_convolution.hpp:78-144), i32 sums exact, with a zero point and padding"""
+    from dldt_amd import Convolution, DeviceTensor
+    rng = np.random.default_rng(G * 100 + icg)
+    N, H, W = 2, 9, 10
+    C, OC = G * icg, G * ocg
+    x = rng.integers(0, 256, (N, C, H, W)).astype(np.int32)
+    w = rng.integers(-127, 128, (G, ocg, icg, 3, 3)).astype(np.int32)
+    zp = 21
+    want = orc.convolution(x - zp, w, (2, 1), (1, 1), (1, 1), (1, 1), grouped=True)
+    xin = DeviceTensor.from_nchw(x, U8B, halo=1, fill_level=zp)
+    conv = Convolution(w.astype(np.int8), xin, (2, 1), (1, 1), (1, 1), (1, 1), zero_point=zp)
+    out = DeviceTensor(N, want.shape[2], want.shape[3], OC, I32)
+    conv.run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw(), want)
+
+
 _WIDE_CASES = {}
 
 

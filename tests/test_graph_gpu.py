@@ -418,3 +418,26 @@ def test_stand_alone_elementwise_nodes(orc):
     for name in ("prod", "left"):
         np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
     assert all(g.query())
+
+
+def test_grouped_convolution_in_a_graph(orc):
+    """a GroupConvolution with four channels per group between two dense convolutions, through the planner"""
+    from dldt_amd import builders
+    from dldt_amd.builders import QuantizedNet
+    rng = np.random.default_rng(61)
+    n, c, hw, groups = 2, 32, 12, 8
+    x = rng.uniform(0, 1, (n, c, hw, hw)).astype(np.float32)
+    net = QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    wn = lambda *s, k=0.1: (rng.standard_normal(s, dtype=np.float32) * np.float32(k)).astype(np.float32)
+    a1 = net.conv(a0, wn(64, c, 1, 1), wn(64, k=0.2), 2.0)
+    a2 = net.conv(a1, wn(64, 64 // groups, 3, 3, k=0.15), wn(64, k=0.2), 2.5, pads=(1, 1), groups=groups)
+    g.result(net.conv_f32(a2, wn(40, 64, 1, 1), wn(40, k=0.2)), "out")
+    want, kept = evaluate(orc, g.nodes, dict(data=x), keep=[a2["node"]])
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps].count("GroupConvolution") == 1
+    req = plan.create_request()
+    (got,) = req.infer(x)
+    np.testing.assert_array_equal(req.tensor(a2["node"]), kept[a2["node"]])
+    np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))
