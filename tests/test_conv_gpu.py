@@ -389,6 +389,49 @@ def test_depthwise_strip_variant_exact(orc, geo, tail):
     np.testing.assert_array_equal(got[0], want)
 
 
+@pytest.mark.parametrize("N,C,H,W,stride", [(2, 144, 9, 11, 1), (1, 16, 5, 3, 1), (3, 48, 13, 40, 2), (2, 96, 17, 17, 2),
+                                            (1, 1008, 6, 5, 1), (2, 32, 35, 70, 1), (1, 2048, 4, 4, 1)])
+def test_depthwise_variants_with_per_channel_zero_points(orc, N, C, H, W, stride):
+    """both depthwise variants (registers, LDS strip) on an input with one zero point per channel: the same levels as
+    the reference's chain, rows and columns that leave partial tiles"""
+    from dldt_amd import Convolution, DeviceTensor, HipieError, make_epilogue
+    rng = np.random.default_rng(C * 7 + H)
+    x = rng.integers(0, 256, (N, C, H, W)).astype(np.int32)
+    zp = rng.integers(0, 256, C).astype(np.int32)
+    w = rng.integers(-127, 128, (C, 1, 1, 3, 3)).astype(np.int32)
+    st = (stride, stride)
+    acc = orc.convolution(x - zp.reshape(1, C, 1, 1), w, st, (1, 1), (1, 1), (1, 1), grouped=True)
+    _, _, OH, OW = acc.shape
+    xin = DeviceTensor.from_nchw(x, U8B, halo=1, fill_level=0)
+    import torch
+    pattern = torch.from_numpy((zp - 128).astype(np.int8)).to(xin.view.device)
+    full = xin.view
+    full[:, 0, :, :C] = pattern
+    full[:, -1, :, :C] = pattern
+    full[:, :, 0, :C] = pattern
+    full[:, :, -1, :C] = pattern
+    bias = rng.normal(0, 3000, C).astype(np.float32)
+    scale = (rng.uniform(0.5, 2.0, C) * 2e-4).astype(np.float32)
+    fq = (256, 0.0, np.float32(6.0), 0.0, 255.0)
+    want = _chain(orc, acc, bias=bias, scale=scale, act="clamp", clamp=(0.0, 6.0), fq=fq).astype(np.uint8)
+    conv = Convolution(w.astype(np.int8), xin, st, (1, 1), (1, 1), (1, 1),
+                       make_epilogue(bias=bias, scale=scale, activation="clamp", clamp=(0.0, 6.0), out_dtype=U8B, fq=fq),
+                       zero_point=zp)
+    ran = []
+    for variant in (0, 1):
+        try:
+            conv.set_tile(variant)
+        except HipieError:
+            assert variant == 1 and C > 1024           # the strip kernel stops at pixels of 1024 bytes
+            continue
+        out8 = DeviceTensor(N, OH, OW, C, U8B)
+        out8.interior().fill_(77)
+        conv.run(xin, out8)
+        np.testing.assert_array_equal(out8.to_nchw(), want, err_msg="variant %d" % variant)
+        ran.append(variant)
+    assert 0 in ran and (1 in ran or C > 1024)
+
+
 def test_depthwise_strip_variant_is_refused_where_it_does_not_apply():
     from dldt_amd import Convolution, DeviceTensor, HipieError, make_epilogue
     x = DeviceTensor(1, 9, 9, 32, U8B, halo=2)
@@ -402,6 +445,9 @@ def test_depthwise_strip_variant_is_refused_where_it_does_not_apply():
     with pytest.raises(HipieError):
         conv.set_tile(1)                                            # dilated
     conv.set_tile(0)
+    conv = Convolution(w3, x, (1, 1), (1, 1), (1, 1), (1, 1))       # raw sums: the strip variant has no such tail
+    with pytest.raises(HipieError):
+        conv.set_tile(1)
 
 
 @pytest.mark.parametrize("signed,zp", [(False, 0), (False, 37), (False, 255), (True, -128), (True, 5)])
