@@ -439,7 +439,7 @@ BERT_RANGES = dict(x=4.0, q=1.2, k=3.0, v=3.0, p=1.0, ctx=1.0, h1=4.0, g=3.0)
 
 
 def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, seed=20211, ranges=None, vocab=0,
-                 mask=False):
+                 mask=False, unsigned_probs=False):
     """benchmark configuration 5: BERT-base style encoder stack in its post-LPT form.  Activations are
     per-tensor symmetric i8 (FakeQuantize ranges of signed_range), weights per-channel i8, Softmax /
     LayerNorm (MVN, Multiply, Add) / Gelu stay f32.
@@ -487,6 +487,14 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
         assert d["precision"] == I8
         return dict(node=g.fake_quantize(v, lo, hi, d["new_low"], d["new_high"], 256, I8), scale=np.float32(d["scale"]))
 
+    def fq_u8(v, high):
+        """FakeQuantize of a non-negative value (Softmax output) to u8 levels 0..255"""
+        from .tensor import U8
+        d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(high))
+        assert d["precision"] == U8 and d["shift"] == 0
+        return dict(node=g.fake_quantize(v, np.float32(0), np.float32(high), d["new_low"], d["new_high"], 256, U8),
+                    scale=np.float32(d["scale"]))
+
     def linear(act, w, b):
         """MatMul' -> Add(b / s): returns (node, s[c])"""
         wq, s_w = lpt.quantize_weights(w, 255)
@@ -533,7 +541,7 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
             s = g.add(s, mask_node)
         p = g.softmax(s, -1)
         meta["glue"].append(p)
-        pq = fq(p, r["p"])
+        pq = fq_u8(p, r["p"]) if unsigned_probs else fq(p, r["p"])
         c = g.multiply(g.matmul(pq["node"], split_heads(v["node"])),
                        g.constant(np.float32(pq["scale"] * v["scale"]).reshape(())))
         c_t = g.transpose(c, (0, 2, 1, 3))

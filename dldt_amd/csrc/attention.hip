@@ -38,6 +38,7 @@ struct AttentionArgs {
     float p_zh, p_zl;                                 // probabilities: two-operation division by fq_p.p.d
     int p_div2;                                       // ... verified against IEEE division on the device
     uint32_t p_xor, p_add;                            // stored byte = level + out_low (mod 256): XOR 0x80 per byte, or bytewise add
+    int p_bias;                                       // 128 when the probabilities are u8 levels (stored as level - 128), else 0
 };
 
 // level index k of four probabilities as four unsigned bytes (rounded to nearest-even and packed by
@@ -60,6 +61,9 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
     __shared__ __attribute__((aligned(16))) int8_t sK[S * 64];       // [key][d], chunk c of row r in slot c ^ ((r >> 2) & 3)
     __shared__ __attribute__((aligned(16))) int8_t sVT[64 * VT_LD];  // [d][tile][half][j]: key 32 t + 8 (j / 4) + 4 half + j % 4
     __shared__ __attribute__((aligned(16))) float sMask[MASK ? S : 4];    // the sequence's mask row
+    // u8 probabilities q are multiplied as q - 128: sum_k q_k v_k = sum_k (q_k - 128) v_k + 128 sum_k v_k, and the
+    // sums of V over the keys, one per d, start the accumulators of the second product
+    __shared__ __attribute__((aligned(16))) int32_t sVsum[64];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, h = lane >> 5;
@@ -74,6 +78,11 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
         const v4i x = *reinterpret_cast<const v4i*>(kp + r * a.ldk + c * 16);
         *reinterpret_cast<v4i*>(&sK[r * 64 + ((c ^ ((r >> 2) & 3)) * 16)]) = x;
     }
+    if (a.p_bias) {
+        if (tid < 64) sVsum[tid] = 0;
+        __syncthreads();
+    }
+    int32_t vsum[4] = {0, 0, 0, 0};                     // this thread's share of the sums (d4 = tid % 16 in every round)
     for (int i = tid; i < (S / 4) * 16; i += 256) {
         const int d4 = i & 15, kq = i >> 4;            // 4 consecutive keys x 4 consecutive d
         uint32_t w[4];
@@ -89,7 +98,14 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
         const int key = 4 * kq, tile = key >> 5, in = key & 31;               // in = 8 a + 4 half
         const int col = tile * 32 + ((in >> 2) & 1) * 16 + (in >> 3) * 4;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) *reinterpret_cast<uint32_t*>(&sVT[(4 * d4 + e) * VT_LD + col]) = t[e];
+        for (int e = 0; e < 4; ++e) {
+            *reinterpret_cast<uint32_t*>(&sVT[(4 * d4 + e) * VT_LD + col]) = t[e];
+            vsum[e] = __builtin_amdgcn_sdot4(static_cast<int>(t[e]), 0x01010101, vsum[e], false);
+        }
+    }
+    if (a.p_bias) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) atomicAdd(&sVsum[4 * (tid & 15) + e], vsum[e]);
     }
 
     if constexpr (MASK) {
@@ -158,6 +174,16 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
 
     // probabilities -> i8 levels -> second product, one 32-key tile at a time
     v16i ctx[2] = {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}};
+    if (a.p_bias) {     // register r of block db holds d = 32 db + 8 (r / 4) + 4 h + r % 4
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const v4i sv = *reinterpret_cast<const v4i*>(&sVsum[32 * db + 8 * g + 4 * h]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) ctx[db][4 * g + j] = sv[j] * a.p_bias;
+            }
+    }
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         v4i pf;
@@ -227,6 +253,8 @@ int hipie_attention_create(int device, const hipie_attention_desc* desc, hipie_a
                       kMaxSeq, desc->head_dim, kHeadDim);
         HIPIE_REQUIRE(desc->out_dtype == HIPIE_I8 || desc->out_dtype == HIPIE_F32, HIPIE_PARAMETER_MISMATCH,
                       "hipie_attention_create: output type %d", desc->out_dtype);
+        HIPIE_REQUIRE(desc->prob_dtype == 0 || desc->prob_dtype == HIPIE_I8 || desc->prob_dtype == HIPIE_U8B, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_attention_create: probabilities of type %d", desc->prob_dtype);
         auto att = std::make_unique<hipie_attention>();
         att->device = device;
         att->d = *desc;
@@ -244,6 +272,7 @@ int hipie_attention_create(int device, const hipie_attention_desc* desc, hipie_a
         if (a.p_div2) { a.p_zh = zh[0]; a.p_zl = zl[0]; }
         HIPIE_REQUIRE(a.p_div2 || a.fq_p.rcp || device < 0, HIPIE_NOT_IMPLEMENTED,
                       "hipie_attention_create: no exact fast division for the probabilities' FakeQuantize range");
+        a.p_bias = desc->prob_dtype == HIPIE_U8B ? 128 : 0;
         const int off = static_cast<int>(a.fq_p.p.ol) & 0xff;
         a.p_xor = off == 0x80 ? 0x80808080u : 0u;
         a.p_add = (off == 0x80 || off == 0) ? 0u : static_cast<uint32_t>(off) * 0x01010101u;

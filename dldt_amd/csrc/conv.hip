@@ -61,7 +61,8 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     const int batch = blockIdx.y;
     static_assert(BOC <= NT, "one table element per thread");
     StagedParams staged;
-    stage_params_load<F>(a, oc0, BOC, tid, staged);   // awaited only after the first K step has been requested
+    // (a batched MatMul with a u8 left operand has one row of accumulator corrections per batch element)
+    stage_params_load<F>(a, oc0, BOC, tid, staged, static_cast<int64_t>(batch) * a.batch_corr);   // awaited only after the first K step has been requested
     const int a_row[2] = {woc * 64 + l32, woc * 64 + 32 + l32};
     const int b_row[2] = {wpix * 64 + l32, wpix * 64 + 32 + l32};
     const int oc_lane = oc0 + woc * 64 + 32 * h;
@@ -1372,6 +1373,40 @@ struct hipie_conv {
     Epilogue epi;
 };
 
+// corr[b][n] = factor * sum_k Bt[b][n][k] for the rows n < N of every batch element b (0 for the padded rows up
+// to Np): a thread per row, 16 bytes a step, v_dot4_i32_i8 against four ones
+__global__ __launch_bounds__(256) void row_sums_kernel(const int8_t* bt, int64_t ldb, int64_t stride_b, int64_t outer_b,
+                                                       int32_t batch_inner, int32_t N, int32_t Np, int32_t K, int32_t factor,
+                                                       int32_t* corr, int64_t rows) {
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (row >= rows) return;
+    const int b = static_cast<int>(row / Np), n = static_cast<int>(row - static_cast<int64_t>(b) * Np);
+    int32_t sum = 0;
+    if (n < N) {
+        int64_t base = static_cast<int64_t>(b) * stride_b;
+        if (batch_inner > 0) {
+            const int o = b / batch_inner;
+            base = o * outer_b + static_cast<int64_t>(b - o * batch_inner) * stride_b;
+        }
+        const int8_t* p = bt + base + static_cast<int64_t>(n) * ldb;
+        for (int k = 0; k < K; k += 16) {
+            const uint4 v = *reinterpret_cast<const uint4*>(p + k);
+            sum = __builtin_amdgcn_sdot4(static_cast<int>(v.x), 0x01010101, sum, false);
+            sum = __builtin_amdgcn_sdot4(static_cast<int>(v.y), 0x01010101, sum, false);
+            sum = __builtin_amdgcn_sdot4(static_cast<int>(v.z), 0x01010101, sum, false);
+            sum = __builtin_amdgcn_sdot4(static_cast<int>(v.w), 0x01010101, sum, false);
+        }
+    }
+    corr[row] = sum * factor;
+}
+
+static void launch_row_sums(const int8_t* bt, int64_t ldb, int64_t stride_b, int64_t outer_b, int32_t batch_inner, int32_t N,
+                            int32_t Np, int32_t K, int32_t factor, int32_t* corr, int32_t batches, hipStream_t s) {
+    const int64_t rows = static_cast<int64_t>(batches) * Np;
+    hipLaunchKernelGGL(row_sums_kernel, dim3(static_cast<uint32_t>(ceil_div(rows, 256))), dim3(256), 0, s, bt, ldb, stride_b,
+                       outer_b, batch_inner, N, Np, K, factor, corr, rows);
+}
+
 struct hipie_matmul {
     int device = 0;
     hipie_matmul_desc d{};
@@ -1457,9 +1492,12 @@ int hipie_matmul_create(int device, const hipie_matmul_desc* desc, const hipie_e
     return guarded([&] {
         HIPIE_REQUIRE(desc && epilogue && out, HIPIE_PARAMETER_MISMATCH, "hipie_matmul_create: null argument");
         const hipie_matmul_desc& d = *desc;
-        HIPIE_REQUIRE(d.a_dtype == HIPIE_I8 && d.b_dtype == HIPIE_I8, HIPIE_NOT_IMPLEMENTED,
-                      "hipie_matmul_create: both operands must be i8 (a u8 left operand against a non-constant "
-                      "right operand would need its column sums at run time)");
+        HIPIE_REQUIRE((d.a_dtype == HIPIE_I8 || d.a_dtype == HIPIE_U8B) && d.b_dtype == HIPIE_I8, HIPIE_NOT_IMPLEMENTED,
+                      "hipie_matmul_create: the left operand must be i8 or u8, the right operand i8 (a u8 right operand "
+                      "would need one correction per output row)");
+        const int lo = d.a_dtype == HIPIE_U8B ? 0 : -128;
+        HIPIE_REQUIRE(d.a_zero_point >= lo && d.a_zero_point <= lo + 255 && (d.a_dtype == HIPIE_U8B || d.a_zero_point == 0),
+                      HIPIE_PARAMETER_MISMATCH, "hipie_matmul_create: zero point %d of the left operand", d.a_zero_point);
         HIPIE_REQUIRE(d.k > 0 && d.n > 0 && d.k % 64 == 0, HIPIE_NOT_IMPLEMENTED,
                       "hipie_matmul_create: K=%d must be a positive multiple of 64", d.k);
         auto m = std::make_unique<hipie_matmul>();
@@ -1490,6 +1528,21 @@ int hipie_matmul_run_nested(const hipie_matmul* mm, const void* a_ptr, int64_t l
                             const void* bt_ptr, int64_t ldb, int64_t stride_b, int64_t outer_b, void* out, int64_t ldo,
                             int64_t stride_o, int64_t outer_o, int32_t m, int32_t batch, int32_t batch_outer,
                             void* stream) {
+    return hipie_matmul_run_nested_ws(mm, a_ptr, lda, stride_a, outer_a, bt_ptr, ldb, stride_b, outer_b, out, ldo, stride_o,
+                                      outer_o, m, batch, batch_outer, nullptr, 0, stream);
+}
+
+int hipie_matmul_workspace_size(const hipie_matmul* mm, int32_t batch, int32_t batch_outer, size_t* bytes) {
+    return guarded([&] {
+        HIPIE_REQUIRE(mm && bytes && batch >= 0 && batch_outer >= 0, HIPIE_PARAMETER_MISMATCH, "hipie_matmul_workspace_size: argument");
+        *bytes = mm->d.a_dtype == HIPIE_U8B ? static_cast<size_t>(batch) * batch_outer * mm->Np * sizeof(int32_t) : 0;
+    });
+}
+
+int hipie_matmul_run_nested_ws(const hipie_matmul* mm, const void* a_ptr, int64_t lda, int64_t stride_a, int64_t outer_a,
+                               const void* bt_ptr, int64_t ldb, int64_t stride_b, int64_t outer_b, void* out, int64_t ldo,
+                               int64_t stride_o, int64_t outer_o, int32_t m, int32_t batch, int32_t batch_outer,
+                               void* workspace, size_t workspace_bytes, void* stream) {
     return guarded([&] {
         HIPIE_REQUIRE(mm, HIPIE_PARAMETER_MISMATCH, "hipie_matmul_run: null handle");
         HIPIE_REQUIRE(mm->koff.ptr, HIPIE_NOT_ALLOCATED, "hipie_matmul_run: host-only object");
@@ -1542,13 +1595,26 @@ int hipie_matmul_run_nested(const hipie_matmul* mm, const void* a_ptr, int64_t l
         a.batch_in_o = outer_a;
         a.batch_wgt_o = outer_b;
         a.batch_out_o = outer_o;
+        DeviceGuard g(mm->device);
+        if (d.a_dtype == HIPIE_U8B) {
+            // sum_k (q_k - z) b_k = sum_k (q_k - 128) b_k + (128 - z) sum_k b_k: the sums over K of the right operand's
+            // rows, one row of corrections per batch element, computed in front of the product on the same stream
+            const size_t need = static_cast<size_t>(batch) * batch_outer * mm->Np * sizeof(int32_t);
+            HIPIE_REQUIRE(workspace && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 16 == 0,
+                          HIPIE_PARAMETER_MISMATCH,
+                          "hipie_matmul_run: a u8 left operand needs a workspace of %zu bytes (hipie_matmul_workspace_size)", need);
+            launch_row_sums(static_cast<const int8_t*>(bt_ptr), ldb, stride_b, outer_b, batch_outer > 1 ? batch : 0, d.n,
+                            static_cast<int32_t>(mm->Np), d.k, 128 - d.a_zero_point, static_cast<int32_t*>(workspace),
+                            batch * batch_outer, as_stream(stream));
+            a.corr = static_cast<const int32_t*>(workspace);
+            a.batch_corr = static_cast<int32_t>(mm->Np);
+        }
         const bool wide = d.n > 64;
         const int boc = wide ? 128 : 64, bpix = wide ? 128 : 256;
         a.p_tiles = static_cast<int32_t>(ceil_div(m, bpix));
         a.t_tiles = static_cast<int32_t>(ceil_div(d.n, boc));
         a.t_shift = (a.t_tiles & (a.t_tiles - 1)) == 0 ? __builtin_ctz(a.t_tiles) : -1;
         a.p_per_xcd = 0;   // plain order: batches are spread over the XCDs by their launch order
-        DeviceGuard g(mm->device);
         if (wide) launch_tiled<2, 2>(a, as_stream(stream), batch * batch_outer);
         else launch_tiled<1, 4>(a, as_stream(stream), batch * batch_outer);
         HIPIE_CHECK_HIP(hipGetLastError());

@@ -152,11 +152,12 @@ struct StagedParams {
 };
 
 template <uint32_t F>
-__device__ __forceinline__ void stage_params_load(const ConvArgs& a, int oc0, int stride, int tid, StagedParams& r) {
+__device__ __forceinline__ void stage_params_load(const ConvArgs& a, int oc0, int stride, int tid, StagedParams& r,
+                                                  int64_t corr_shift = 0) {
     const uint32_t fl = F == kDyn ? a.flags : F;
     const int c = oc0 + (tid < stride ? tid : 0);
     auto get = [&](int t, const float* src) { r.v[t] = src[c]; };
-    r.corr = a.corr[c];
+    r.corr = a.corr[corr_shift + c];
     if (fl & CF_BIAS) get(PT_BIAS, a.bias);
     if (fl & CF_SCALE) get(PT_SCALE, a.scale);
     if (fl & CF_RES_SUB) get(PT_RSUB, a.res_sub);

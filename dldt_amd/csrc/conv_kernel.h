@@ -93,6 +93,7 @@ struct ConvArgs {
     // batch_inner = 0 means one level
     int32_t batch_inner;
     int64_t batch_in_o, batch_wgt_o, batch_out_o;
+    int32_t batch_corr;              // accumulator corrections per batch element: entries from one batch's row to the next (0: one row for all)
     int32_t wgt_ld, wgt_rows, wgt_plain;
     // fused shortcut convolution (CF_RES_GEMM): a second operand set accumulated first; its
     // dequantised result stays in registers as the residual of the main convolution

@@ -582,10 +582,11 @@ struct GlueStep : Step {
     }
 };
 
-// MatMul between two i8 activations, batched over one or two leading dimensions
+// MatMul between two activations (i8 or u8 on the left, i8 on the right), batched over one or two leading dimensions
 struct BatchMatMulStep : Step {
     View a, b;                     // b as [.., N, K] with K contiguous
     int out = -1;
+    int ws = -1;                   // row sums of the right operand, one row per batch element (u8 left operand only)
     int64_t lda = 0, sa = 0, oa = 0, ldb = 0, sb = 0, ob = 0, ldo = 0, so = 0, oo = 0;
     int32_t m = 0, k = 0, n = 0, batch = 1, outer = 1;
     EpilogueSpec epi;
@@ -602,8 +603,10 @@ struct BatchMatMulStep : Step {
     }
     void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*,
              hipStream_t s) const override {
-        check_status(hipie_matmul_run_nested(mm, a.ptr(arena, tensors, inputs), lda, sa, oa, b.ptr(arena, tensors, inputs), ldb,
-                                             sb, ob, arena + tensors[out].offset, ldo, so, oo, m, batch, outer, s),
+        check_status(hipie_matmul_run_nested_ws(mm, a.ptr(arena, tensors, inputs), lda, sa, oa, b.ptr(arena, tensors, inputs), ldb,
+                                                sb, ob, arena + tensors[out].offset, ldo, so, oo, m, batch, outer,
+                                                ws >= 0 ? arena + tensors[ws].offset : nullptr,
+                                                ws >= 0 ? static_cast<size_t>(tensors[ws].bytes) : 0, s),
                      name.c_str());
     }
 };
@@ -1183,8 +1186,7 @@ struct Planner {
         const GNode& n = N(id);
         const Value a = value(n.in[0]);
         const bool weights = N(n.in[1]).op == OP_CONSTANT;
-        if (a.view.dtype != HIPIE_I8 && !(weights && a.view.dtype == HIPIE_U8B))
-            unsupported(id, weights ? "left operand must be quantized (i8 or u8)" : "operands of a MatMul between activations must be i8");
+        if (a.view.dtype != HIPIE_I8 && a.view.dtype != HIPIE_U8B) unsupported(id, "left operand must be quantized (i8 or u8)");
         if (n.ta) unsupported(id, "transpose_a");
         if (weights) plan_linear(id, a.view);
         else plan_batch_matmul(id, a.view);
@@ -1473,7 +1475,8 @@ struct Planner {
         if (N(sm).op != OP_SOFTMAX || N(sm).axes[0] != static_cast<int64_t>(r) - 1 || !single_user(sm)) return false;
         const int fq = N(sm).users[0];
         hipie_requant rq{};
-        if (!fusable_requant(fq, sm, rq) || !single_user(fq)) return false;
+        int prob_storage = HIPIE_I8;
+        if (!fusable_requant(fq, sm, rq, &prob_storage) || !single_user(fq)) return false;
         Requant host_check{};
         try {
             host_check = make_requant(&rq, "attention");
@@ -1508,6 +1511,7 @@ struct Planner {
         d.score_scale = c1[0];
         d.context_scale = tail.scale[0];
         d.prob_fq = rq;
+        d.prob_dtype = prob_storage;
         d.out_dtype = tail.out_dtype;
         if (tail.out_dtype == HIPIE_I8) {
             d.out_fq.in_low = tail.fq_il[0];
@@ -1572,7 +1576,7 @@ struct Planner {
             if (av.shape[i] != bv.shape[i]) unsupported(id, "broadcast batch dimensions");
         if (av.stride[r - 1] != 1) unsupported(id, "left operand with a strided reduction axis");
         if (K % 64 != 0) unsupported(id, "reduction length must be a multiple of 64");
-        if (fuse_attention && M == Nn && try_plan_attention(id, av, bv)) return;
+        if (fuse_attention && M == Nn && av.dtype == HIPIE_I8 && try_plan_attention(id, av, bv)) return;   // (the scores' operands)
         const int32_t inner = static_cast<int32_t>(av.shape[r - 3]), outer = r == 4 ? static_cast<int32_t>(av.shape[0]) : 1;
         if (bv.stride[r - 1] != 1) {
             // reduction axis not contiguous: transpose the operand's inner dimensions into a new tensor
@@ -1619,6 +1623,8 @@ struct Planner {
         const int cur = absorb_matmul_tail(id, e, oshape, ostride);
         mark_chain(id, cur);
         st->out = new_matrix(cur, e.out_dtype, oshape);
+        if (av.dtype == HIPIE_U8B)   // level 0 stands for 0.0 here: a zero point would arrive as a Subtract, which is not taken
+            st->ws = new_tensor(id, HIPIE_I32, 1, 1, inner * outer, static_cast<int>(round_up(Nn, 128)));
         st->ldo = ostride[r - 2];
         st->so = ostride[r - 3];
         st->oo = r == 4 ? ostride[0] : 0;

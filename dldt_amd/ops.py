@@ -210,20 +210,21 @@ class Convolution:
 
 
 class hipie_matmul_desc(ctypes.Structure):
-    _fields_ = [(k, ctypes.c_int32) for k in ("a_dtype", "b_dtype", "k", "n")]
+    _fields_ = [(k, ctypes.c_int32) for k in ("a_dtype", "b_dtype", "k", "n", "a_zero_point")]
 
 
 class BatchedMatMul:
-    """i8 x i8 MatMul between two activation tensors: out[b] = A[b] @ Bt[b]^T (+ fused epilogue).
+    """i8 (or u8) x i8 MatMul between two activation tensors: out[b] = A[b] @ Bt[b]^T (+ fused epilogue).
 
-    ``a`` is a torch int8 tensor [batch, M, K], ``bt`` is [batch, N, K] (the transpose_b = true
-    form); the result is [batch, M, ldo] with ldo = N padded to the store granularity.
+    ``a`` is a torch int8 tensor [batch, M, K] (u8 levels stored as level - 128 with ``a_dtype=U8B``), ``bt`` is
+    [batch, N, K] (the transpose_b = true form); the result is [batch, M, ldo] with ldo = N padded to the store
+    granularity.
     """
 
-    def __init__(self, k, n, epilogue=None, device=0):
+    def __init__(self, k, n, epilogue=None, device=0, a_dtype=I8, a_zero_point=0):
         self.k, self.n = k, n
         self.epilogue = epilogue or make_epilogue(out_dtype=I32)
-        d = hipie_matmul_desc(I8, I8, k, n)
+        d = hipie_matmul_desc(a_dtype, I8, k, n, a_zero_point)
         self._h = ctypes.c_void_p()
         check(lib().hipie_matmul_create(ctypes.c_int(device), ctypes.byref(d), ctypes.byref(self.epilogue),
                                         ctypes.byref(self._h)))
@@ -245,9 +246,13 @@ class BatchedMatMul:
             out = torch.zeros((batch, m, ldo), dtype=tdt, device=a.device)
         assert out.shape == (batch, m, ldo) and out.dtype == tdt and out.is_contiguous()
         i64 = ctypes.c_int64
-        check(lib().hipie_matmul_run(self._h, _dptr(a), i64(k), i64(m * k), _dptr(bt), i64(k), i64(self.n * k),
-                                     _dptr(out), i64(ldo), i64(m * ldo), ctypes.c_int32(m), ctypes.c_int32(batch),
-                                     _stream()))
+        need = ctypes.c_size_t()
+        check(lib().hipie_matmul_workspace_size(self._h, ctypes.c_int32(batch), ctypes.c_int32(1), ctypes.byref(need)))
+        ws = torch.empty(max(need.value, 16), dtype=torch.int8, device=a.device)
+        check(lib().hipie_matmul_run_nested_ws(self._h, _dptr(a), i64(k), i64(m * k), i64(0), _dptr(bt), i64(k),
+                                               i64(self.n * k), i64(0), _dptr(out), i64(ldo), i64(m * ldo), i64(0),
+                                               ctypes.c_int32(m), ctypes.c_int32(batch), ctypes.c_int32(1),
+                                               _dptr(ws) if need.value else None, ctypes.c_size_t(need.value), _stream()))
         return out[..., :self.n]
 
 
@@ -331,7 +336,7 @@ def gelu(x, requant=None, keep_f32=True):
 class hipie_attention_desc(ctypes.Structure):
     _fields_ = [("seq", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("score_scale", ctypes.c_float),
                 ("context_scale", ctypes.c_float), ("prob_fq", hipie_requant), ("out_dtype", ctypes.c_int32),
-                ("out_fq", hipie_requant)]
+                ("out_fq", hipie_requant), ("prob_dtype", ctypes.c_int32)]
 
 
 class Attention:
@@ -339,8 +344,9 @@ class Attention:
     FakeQuantize(prob_fq) -> MatMul'(., v) * context_scale [-> FakeQuantize(out_fq)].
     prob_fq / out_fq = (in_low, in_high, out_low, levels)."""
 
-    def __init__(self, seq, head_dim, score_scale, context_scale, prob_fq, out_fq=None, device=0):
+    def __init__(self, seq, head_dim, score_scale, context_scale, prob_fq, out_fq=None, device=0, prob_dtype=I8):
         d = hipie_attention_desc()
+        d.prob_dtype = prob_dtype
         d.seq, d.head_dim = seq, head_dim
         d.score_scale, d.context_scale = float(score_scale), float(context_scale)
         d.prob_fq = hipie_requant(*[float(x) for x in prob_fq[:3]], int(prob_fq[3]))

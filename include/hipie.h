@@ -283,8 +283,9 @@ int hipie_conv_run_static(const hipie_conv* conv, const hipie_tensor* in, const 
  *     1x1 convolution (hipie_conv_*).  Leading dimensions and batch strides are in elements.
  * ==================================================================================== */
 typedef struct hipie_matmul_desc {
-    int32_t a_dtype, b_dtype;   /* HIPIE_I8 (symmetric activations on both sides) */
+    int32_t a_dtype, b_dtype;   /* left: HIPIE_I8 or HIPIE_U8B (u8 levels, e.g. quantized Softmax output); right: HIPIE_I8 */
     int32_t k, n;               /* reduction length (multiple of 64), output columns */
+    int32_t a_zero_point;       /* level of the u8 left operand that stands for 0.0 (0 for i8) */
 } hipie_matmul_desc;
 
 typedef struct hipie_matmul hipie_matmul;
@@ -301,6 +302,15 @@ int hipie_matmul_run_nested(const hipie_matmul* matmul, const void* a, int64_t l
                             const void* b_transposed, int64_t ldb, int64_t stride_b, int64_t outer_b, void* out,
                             int64_t ldo, int64_t stride_o, int64_t outer_o, int32_t m, int32_t batch,
                             int32_t batch_outer, void* stream);
+/* A u8 left operand is stored as level - 128: sum_k (q_k - z) b_k = sum_k (q_k - 128) b_k + (128 - z) sum_k b_k, and
+ * the sums over K of the right operand's rows (an activation here, not constant weights as in mat_mul.cpp:95-121) are
+ * computed on the stream in front of the product, into a workspace of hipie_matmul_workspace_size bytes that the
+ * caller owns (one per request in flight; 16-byte aligned; 0 bytes and not needed for an i8 left operand). */
+int hipie_matmul_workspace_size(const hipie_matmul* matmul, int32_t batch, int32_t batch_outer, size_t* bytes);
+int hipie_matmul_run_nested_ws(const hipie_matmul* matmul, const void* a, int64_t lda, int64_t stride_a, int64_t outer_a,
+                               const void* b_transposed, int64_t ldb, int64_t stride_b, int64_t outer_b, void* out,
+                               int64_t ldo, int64_t stride_o, int64_t outer_o, int32_t m, int32_t batch,
+                               int32_t batch_outer, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ======================================================================================
  * 1e. fp32 glue of the transformer path, over the last axis of a dense [rows, axis] f32 matrix
@@ -357,6 +367,8 @@ typedef struct hipie_attention_desc {
     hipie_requant prob_fq;
     int32_t out_dtype;          /* HIPIE_F32 or HIPIE_I8 */
     hipie_requant out_fq;       /* used when out_dtype is HIPIE_I8 */
+    int32_t prob_dtype;         /* HIPIE_I8 (also 0), or HIPIE_U8B: prob_fq gives u8 levels, out_low = first level - 128;
+                                 * the context product then starts from 128 x the sums of V over the keys */
 } hipie_attention_desc;
 typedef struct hipie_attention hipie_attention;
 int hipie_attention_supported(int32_t seq, int32_t head_dim);

@@ -18,7 +18,8 @@ GLUE_TOL = dict(p=dict(rtol=2e-6, atol=1e-8), h1=dict(rtol=1e-5, atol=4e-6), gel
                 y=dict(rtol=1e-5, atol=4e-6))
 
 
-def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq, fuse_attention=True, merge_linear=True):
+def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq, fuse_attention=True, merge_linear=True,
+                 unsigned_probs=False):
     from dldt_amd import builders
     monkeypatch.setenv("HIPIE_FUSE_ATTENTION", "1" if fuse_attention else "0")
     monkeypatch.setenv("HIPIE_MERGE_LINEAR", "1" if merge_linear else "0")
@@ -27,7 +28,7 @@ def _check_stack(orc, monkeypatch, layers, hidden, heads, ffn, batch, seq, fuse_
     monkeypatch.setenv("HIPIE_KEEP_F32", "1")
     # ranges for the reduced width: about 30 levels per standard deviation, so the tails saturate
     g, meta = builders.bert_encoder(layers=layers, hidden=hidden, heads=heads, ffn=ffn, batch=batch, seq=seq, seed=7,
-                                    ranges=dict(q=0.12, k=0.9, v=0.9, ctx=0.6))
+                                    ranges=dict(q=0.12, k=0.9, v=0.9, ctx=0.6), unsigned_probs=unsigned_probs)
     x = np.random.default_rng(70).normal(0, 1, (batch, seq, hidden)).astype(np.float32)
     plan = g.compile()
     types = [s["type"] for s in plan.steps]
@@ -96,6 +97,19 @@ def test_encoder_stack_with_separate_attention_kernels(orc, monkeypatch):
     _check_stack(orc, monkeypatch, layers=2, hidden=128, heads=2, ffn=256, batch=2, seq=128, fuse_attention=False)
     _check_stack(orc, monkeypatch, layers=1, hidden=192, heads=3, ffn=320, batch=3, seq=64, fuse_attention=False,
                  merge_linear=False)
+
+
+def test_encoder_stack_with_u8_probabilities(orc, monkeypatch):
+    """the Softmax output quantized to u8 levels 0..255 (what a calibration tool gives a non-negative tensor): the
+    context product takes a u8 left operand, with the sums over the keys of V's columns as accumulator corrections -
+    in the fused attention kernel and as separate steps"""
+    _check_stack(orc, monkeypatch, layers=2, hidden=128, heads=2, ffn=256, batch=2, seq=128, unsigned_probs=True)
+    _check_stack(orc, monkeypatch, layers=1, hidden=192, heads=3, ffn=320, batch=3, seq=64, unsigned_probs=True,
+                 merge_linear=False)
+    _check_stack(orc, monkeypatch, layers=1, hidden=128, heads=2, ffn=256, batch=2, seq=128, unsigned_probs=True,
+                 fuse_attention=False)
+    _check_stack(orc, monkeypatch, layers=1, hidden=192, heads=3, ffn=320, batch=3, seq=64, unsigned_probs=True,
+                 fuse_attention=False)
 
 
 def test_encoder_stack_with_one_gemm_per_matmul(orc, monkeypatch):

@@ -21,6 +21,49 @@ def test_batched_matmul_i8_exact(orc, batch, m, k, n):
     np.testing.assert_array_equal(got, want)
 
 
+@pytest.mark.parametrize("batch,m,k,n,zp", [(6, 384, 384, 64, 0), (3, 100, 128, 200, 0), (2, 7, 64, 40, 17), (5, 130, 192, 128, 255)])
+def test_batched_matmul_u8_left_operand(orc, batch, m, k, n, zp):
+    """u8 levels (a quantized Softmax output) times an i8 activation: exact i32 sums of (q - zero point) * b, the u8
+    operand stored as level - 128 and the row sums of the right operand folded into the accumulators' start; then the
+    dequantizing Multiply and the next FakeQuantize in the same kernel"""
+    import torch
+    from dldt_amd import BatchedMatMul, make_epilogue
+    rng = np.random.default_rng(m + n + zp)
+    a = rng.integers(0, 256, (batch, m, k)).astype(np.int32)
+    bt = rng.integers(-128, 128, (batch, n, k)).astype(np.int8)
+    want = orc.matmul(a - zp, bt.astype(np.int32), False, True)
+    ad = torch.from_numpy((a - 128).astype(np.int8)).cuda()
+    bd = torch.from_numpy(bt).cuda()
+    mm = BatchedMatMul(k, n, a_dtype=U8B, a_zero_point=zp)
+    np.testing.assert_array_equal(mm.run(ad, bd).cpu().numpy(), want)
+    np.testing.assert_array_equal(mm.run(ad, bd).cpu().numpy(), want)        # the workspace of a second call is its own
+    s = np.float32(1 / 255) * np.float32(0.03)
+    f = orc.multiply(want.astype(np.float32), s)
+    hi = np.float32(np.abs(f).max())
+    lo = np.float32(-hi * np.float32(128) / np.float32(127))
+    lv = orc.fake_quantize(f, lo, hi, np.float32(-128), np.float32(127), 256).astype(np.int8)
+    got8 = BatchedMatMul(k, n, make_epilogue(scale=[s], out_dtype=I8, fq=(256, lo, hi, -128.0, 127.0)), a_dtype=U8B,
+                         a_zero_point=zp).run(ad, bd)
+    np.testing.assert_array_equal(got8.cpu().numpy(), lv)
+
+
+def test_batched_matmul_u8_needs_its_workspace_and_a_level_as_zero_point():
+    import ctypes
+    import torch
+    from dldt_amd import BatchedMatMul, HipieError
+    from dldt_amd.ops import matmul_strided
+    with pytest.raises(HipieError):
+        BatchedMatMul(64, 64, a_dtype=U8B, a_zero_point=256)
+    with pytest.raises(HipieError):
+        BatchedMatMul(64, 64, a_zero_point=3)                      # an i8 operand has none
+    mm = BatchedMatMul(64, 64, a_dtype=U8B)
+    a = torch.zeros((1, 64, 64), dtype=torch.int8, device="cuda")
+    out = torch.zeros((1, 64, 64), dtype=torch.int32, device="cuda")
+    with pytest.raises(HipieError) as e:
+        matmul_strided(mm, a.data_ptr(), 64, 0, a.data_ptr(), 64, 0, out.data_ptr(), 64, 0, 64, 1)
+    assert "workspace" in str(e.value)
+
+
 def test_batched_matmul_scaled_and_requantized(orc):
     """MatMul' -> Multiply(s_a * s_b) -> f32, and -> FakeQuantize (symmetric i8) as the next MatMul wants it."""
     import torch
@@ -206,6 +249,39 @@ def test_fused_attention_with_mask(orc):
     want_ctx = orc.multiply(orc.matmul(pq, vn).astype(np.float32), s2)
     np.testing.assert_array_equal(ctx.cpu().numpy().view(np.uint32), want_ctx.view(np.uint32))
     assert torch.equal(att.run(q, k, v, mask=torch.from_numpy(mask).cuda()), ctx)
+
+
+@pytest.mark.parametrize("S,masked", [(128, False), (384, False), (160, True)])
+def test_fused_attention_with_u8_probabilities(orc, S, masked):
+    """the Softmax output quantized to u8 levels 0..255: stored as level - 128 for the signed matrix instruction, the
+    sums of V over the keys (times 128) start the accumulators of the context product"""
+    import torch
+    from dldt_amd.ops import Attention
+    rng = np.random.default_rng(S)
+    B, NH = 2, 3
+    t = torch.from_numpy(rng.integers(-70, 71, (B, S, 3, NH, 64), dtype=np.int8)).cuda()
+    q, k, v = (t[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    s1, s2 = np.float32(0.002), np.float32(0.01) / np.float32(255)
+    il, ih = np.float32(0.0), np.float32(1.0)
+    mask = None
+    if masked:
+        mask = np.zeros((B, S), np.float32)
+        mask[1, 90:] = -10000.0
+    att = Attention(S, 64, s1, s2, (il, ih, -128, 256), prob_dtype=U8B)
+    md = torch.from_numpy(mask).cuda() if masked else None
+    ctx, scores, probs = att.run(q, k, v, dump=True, mask=md)
+    qn, kn, vn = (np.ascontiguousarray(x.cpu().numpy()).astype(np.int32) for x in (q, k, v))
+    want_scores = orc.multiply(orc.matmul(qn, kn, False, True).astype(np.float32), s1)
+    if masked:
+        want_scores = orc.add(want_scores, mask[:, None, None, :])
+    np.testing.assert_array_equal(scores.cpu().numpy().view(np.uint32), want_scores.view(np.uint32))
+    p = probs.cpu().numpy()
+    np.testing.assert_allclose(p, orc.softmax(want_scores, -1), rtol=3e-6, atol=1e-8)
+    pq = orc.fake_quantize(p, il, ih, np.float32(0), np.float32(255), 256).astype(np.int32)    # from the device's f32 probabilities
+    assert pq.max() > 128 or S > 128
+    want_ctx = orc.multiply(orc.matmul(pq, vn).astype(np.float32), s2)
+    np.testing.assert_array_equal(ctx.cpu().numpy().view(np.uint32), want_ctx.view(np.uint32))
+    assert torch.equal(att.run(q, k, v, mask=md), ctx)
 
 
 def test_nested_batches_inside_a_packed_tensor():
