@@ -15,7 +15,7 @@ def _per_channel_case(rng, N, C, H, W):
 
 
 @pytest.mark.parametrize("shape", [(2, 16, 14, 14), (3, 5, 7, 9), (1, 64, 56, 56), (2, 256, 8, 8), (2, 100, 20, 13), (2, 130, 30, 30),
-                                   (1, 72, 4, 257)])
+                                   (1, 72, 4, 257), (1, 300, 6, 10), (2, 512, 12, 12), (1, 128, 1, 4)])
 def test_fq_levels_bit_exact(orc, shape):
     import torch
     from dldt_amd import FakeQuantize

@@ -141,10 +141,11 @@ def test_requests_in_flight_do_not_disturb_each_other():
         np.testing.assert_array_equal(outs[0].cpu().numpy().view(np.uint32), w.view(np.uint32))
 
 
-@pytest.mark.parametrize("c,hw", [(64, 56), (3, 32), (20, 9)])
+@pytest.mark.parametrize("c,hw", [(64, 56), (3, 32), (20, 9), (128, 28), (320, 6)])
 def test_u8_graph_input(orc, c, hw):
     """input precision U8: Parameter(u8) -> Convert(f32) -> FakeQuantize runs as one entry kernel that
-    reads the bytes (image-like 4-byte pixels, 64-channel tiles, ragged channels and widths)"""
+    reads the bytes (image-like 4-byte pixels, 64-channel tiles, whole-pixel tiles from 128 channels up, ragged
+    channels and widths)"""
     from dldt_amd import builders
     g, feeds, _ = builders.conv_block(seed=5, n=2, c=c, hw=hw, oc=32, u8_input=True)
     want, _ = evaluate(orc, g.nodes, feeds)
