@@ -69,8 +69,17 @@ class QuantizedNet:
         """[Subtract(zero point)] -> Conv'/MatMul' -> Add(b / s): returns (node, s[c])."""
         g = self.g
         wq, s_w = lpt.quantize_weights(w, 255)
-        s = (np.float32(act["scale"]) * s_w).astype(np.float32)            # fold<Multiply>(s_a, s_w)
         groups = conv_attrs.pop("groups", 0)
+        s_a = np.asarray(act["scale"], np.float32).reshape(-1)
+        if s_a.size > 1 and s_a.size != s_w.size:
+            # per-channel activation scales in front of a grouped convolution: one scale per group (the transformation
+            # takes the layer only if the scales are equal inside every group, group_convolution.cpp via
+            # WeightableLayerTransformation::canBeTransformed), repeated over the group's output channels
+            G = groups or s_a.size
+            per_group = s_a.reshape(G, -1)
+            assert np.all(per_group == per_group[:, :1])
+            s_a = np.repeat(per_group[:, 0], s_w.size // G)
+        s = (s_a * s_w).astype(np.float32)                                 # fold<Multiply>(s_a, s_w)
         if groups:
             # [OC, IC / G, kh, kw] -> [G, OC / G, IC / G, kh, kw]
             wq = wq.reshape(groups, wq.shape[0] // groups, wq.shape[1], wq.shape[2], wq.shape[3])
@@ -127,10 +136,14 @@ class QuantizedNet:
         y = g.clamp(g.multiply(y, g.constant(self._channel(s, rank))), 0.0, 6.0)
         return self.requantize(y, out_high)
 
-    def conv_f32(self, act, w, bias, strides=(1, 1), pads=(0, 0), relu=False, matmul=False):
+    def conv_f32(self, act, w, bias, strides=(1, 1), pads=(0, 0), relu=False, matmul=False, grouped=False, groups=0):
         """Quantized conv / FC whose result is consumed in f32: ... -> Multiply(s[c]) [-> ReLU]."""
         g = self.g
         attrs = dict(strides=strides, dilations=(1, 1), pads_begin=pads, pads_end=pads)
+        if grouped:
+            attrs["grouped"] = True
+        if groups:
+            attrs["groups"] = groups
         y, s, rank = self._accumulate(act, w, bias, attrs, matmul)
         y = g.multiply(y, g.constant(self._channel(s, rank)))
         return g.relu(y) if relu else y
@@ -268,7 +281,7 @@ def resnet50(batch=1, res=224, seed=20211, classes=1000, width=64, stages=RESNET
             # precision); the ReLU behind it was fused into the next FakeQuantize before LPT
             a = net.requantize(g.add(yc, sc), R[p + ".out"])
             acts[p + ".a"], acts[p + ".b"], acts[p + ".out"] = ya, yb, a
-    final_hw = res // 32
+    final_hw = res // (4 * int(np.prod([st[2] for st in stages])))     # stem and max-pool halve twice, then the stages' strides
     y = g.avg_pool(a["node"], (final_hw, final_hw), (1, 1), (0, 0), (0, 0), exclude_pad=True, out_dtype=F32)
     y = g.reshape(y, (batch, P["fc.w"].shape[1]))
     d = lpt.decompose_fake_quantize(256, np.float32(0), np.float32(R["pool"]))
@@ -471,7 +484,7 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
     net = QuantizedNet()
     g = net.g
     nrm = lambda *shape: (rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02)).astype(np.float32)
-    meta = dict(layers=[], glue=[], macs=0)
+    meta = dict(layers=[], glue=[], macs=0, linear=[], norm=[])   # linear / norm: the float parameters in the order of their use
     if vocab:
         from .tensor import I32
         ids = g.parameter("input_ids", (batch, seq), I32)
@@ -499,6 +512,7 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
         """MatMul' -> Add(b / s): returns (node, s[c])"""
         wq, s_w = lpt.quantize_weights(w, 255)
         s = (np.float32(act["scale"]) * s_w).astype(np.float32)
+        meta["linear"].append((w, b))
         y = g.matmul(act["node"], g.constant(wq, I8), False, True)
         return g.add(y, g.constant(lpt.swap_multiply_and_add(b, s))), s
 
@@ -517,7 +531,9 @@ def bert_encoder(layers=12, hidden=768, heads=12, ffn=3072, batch=16, seq=384, s
 
     def layer_norm(v):
         n = g.mvn(v, (-1,), True, 1e-5, True)
-        out = g.add(g.multiply(n, g.constant(np.float32(1) + nrm(hidden))), g.constant(nrm(hidden)))
+        gamma, beta = np.float32(1) + nrm(hidden), nrm(hidden)
+        meta["norm"].append((gamma, beta))
+        out = g.add(g.multiply(n, g.constant(gamma)), g.constant(beta))
         meta["glue"].append(out)
         return out
 

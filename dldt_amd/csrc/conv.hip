@@ -1634,10 +1634,12 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
                       HIPIE_PARAMETER_MISMATCH, "hipie_conv_create: bad geometry");
         HIPIE_REQUIRE(d.groups >= 1 && d.ic % d.groups == 0 && d.oc % d.groups == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_create: groups=%d does not divide ic=%d and oc=%d", d.groups, d.ic, d.oc);
-        if (d.groups > 1 && !(d.groups == d.ic && d.ic == d.oc)) {
+        if (d.groups > 1 && (!(d.groups == d.ic && d.ic == d.oc) || d.in_c_stride % 16 != 0)) {
             // A grouped convolution that is not depthwise (weights [oc][ic / groups][kh][kw]) is the dense convolution
             // with block-diagonal weights: reference::group_convolution (group_convolution.hpp:78-144) convolves every
-            // slice on its own, and the products added here are zeros.
+            // slice on its own, and the products added here are zeros.  So is a depthwise one over pixels that are
+            // not a multiple of 16 bytes (an image-like input of up to four channels), which the depthwise kernels,
+            // reading 16 channels per lane, do not take.
             const int64_t icg = d.ic / d.groups, ocg = d.oc / d.groups, taps = static_cast<int64_t>(d.kh) * d.kw;
             std::vector<int8_t> dense(static_cast<size_t>(d.oc) * d.ic * taps, 0);
             for (int64_t oc = 0; oc < d.oc; ++oc)
