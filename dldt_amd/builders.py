@@ -619,12 +619,13 @@ def concat_net(seed=41, n=2, c=32, hw=18, branches=(24, 40, 16), oc=48, signed=F
     g = net.g
     a0 = net.input("data", x.shape, 1.0)
     out_high = 3.0
-    acts = []
+    acts, params = [], []
     for i, oc_b in enumerate(branches):
         k = 3 if i % 2 else 1
         w = (rng.standard_normal((oc_b, c, k, k), dtype=np.float32) * np.float32(0.12 if k == 1 else 0.05)).astype(np.float32)
         b = (rng.standard_normal(oc_b, dtype=np.float32) * np.float32(0.3)).astype(np.float32)
         acts.append(net.conv(a0, w, b, out_high, pads=(k // 2, k // 2), signed=signed))
+        params.append((w, b))
     assert all(a["scale"] == acts[0]["scale"] for a in acts)
     cat = dict(node=g.concat([a["node"] for a in acts], axis=1), scale=acts[0]["scale"])
     g.result(net.dequantize(cat), "cat")
@@ -632,7 +633,8 @@ def concat_net(seed=41, n=2, c=32, hw=18, branches=(24, 40, 16), oc=48, signed=F
     w = (rng.standard_normal((oc, ct, 3, 3), dtype=np.float32) * np.float32(0.04)).astype(np.float32)
     b = (rng.standard_normal(oc, dtype=np.float32) * np.float32(0.2)).astype(np.float32)
     g.result(net.conv_f32(cat, w, b, pads=(1, 1), relu=True), "out")
-    return g, dict(data=x), dict(concat=cat["node"], branches=[a["node"] for a in acts])
+    params.append((w, b))
+    return g, dict(data=x), dict(concat=cat["node"], branches=[a["node"] for a in acts], params=params, out_high=out_high)
 
 
 def per_channel_zero_point_net(seed=47, n=2, c=48, hw=17, oc=40, stride=1):
@@ -658,7 +660,7 @@ def per_channel_zero_point_net(seed=47, n=2, c=48, hw=17, oc=40, stride=1):
     return g, dict(data=x), dict(acts=dict(a0=a0, a1=a1))
 
 
-def matmul_zero_point_net(seed=53, batch=2, seq=48, hidden=128, ffn=192):
+def matmul_zero_point_net(seed=53, batch=2, seq=48, hidden=128, ffn=192, r0=(-1.6, 2.9), r1=(-0.7, 1.9)):
     """Row-major (transformer) path with asymmetric u8 activations: LayerNorm -> FakeQuantize(u8, zero point) ->
     MatMul' -> Subtract(zero point x column sums of the weights) -> Add(bias over scale) -> FakeQuantize(u8, zero point; the
     dequantization folded into its range) -> MatMul' -> Subtract -> Add -> Multiply(s) -> + residual, i.e. what
@@ -683,19 +685,22 @@ def matmul_zero_point_net(seed=53, batch=2, seq=48, hidden=128, ffn=192):
         """MatMul' -> Subtract(zp * sum_k w) -> Add(b / s): returns (node, s[c])"""
         wq, s_w = lpt.quantize_weights(w, 255)
         s = (np.float32(act["scale"]) * s_w).astype(np.float32)
+        params.append((w, b))
         y = g.matmul(act["node"], g.constant(wq, I8), False, True)
         # fold<MatMul>(broadcast(zero point) [1, K], weights): one f32 product per column, exact integers here
         corr = (np.full((1, wq.shape[1]), act["zero_point"], np.float32) @ wq.astype(np.float32).T).reshape(-1).astype(np.float32)
         y = g.subtract(y, g.constant(corr))
         return g.add(y, g.constant(lpt.swap_multiply_and_add(b, s))), s
 
-    a0 = fq_u8(h, -1.6, 2.9)
+    params = []
+    a0 = fq_u8(h, r0[0], r0[1])
     y1, s1 = linear(a0, nrm(ffn, hidden), nrm(ffn, s=0.3))
-    a1 = fq_u8(y1, -0.7, 1.9, fold=s1)
+    a1 = fq_u8(y1, r1[0], r1[1], fold=s1)
     y2, s2 = linear(a1, nrm(hidden, ffn), nrm(hidden, s=0.3))
     out = g.add(g.multiply(y2, g.constant(s2)), h)
     g.result(out, "out")
-    return g, dict(norm=h, a0=a0["node"], a1=a1["node"], zero_points=(float(a0["zero_point"]), float(a1["zero_point"])))
+    return g, dict(norm=h, a0=a0["node"], a1=a1["node"], zero_points=(float(a0["zero_point"]), float(a1["zero_point"])),
+                   linear=params)
 
 
 def eltwise_net(seed=59, n=2, c=24, hw=14, oc=40):

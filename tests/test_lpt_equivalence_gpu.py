@@ -318,3 +318,74 @@ def test_encoder_layer_follows_its_float_graph(orc, monkeypatch, unsigned_probs)
     np.testing.assert_allclose(y, ref, rtol=0, atol=0.02 * np.abs(ref).max())
     assert np.abs(y - ref).mean() < 1e-3 * np.abs(ref).max()
     print(worst)
+
+
+def test_weight_matmuls_with_zero_points_equal_their_float_graph(orc):
+    """MatMuls against quantized weights whose activations are u8 levels with a zero point: the transformation moves the
+    zero point BEHIND the MatMul (zero point x column sums of the weights, mat_mul.cpp:95-121).  Intervals with exact
+    integer zero points (90 at scale 1/64, 45 at scale 1/128), so the transformed graph is the original one up to
+    f32 rounding.  The original starts from the device's LayerNorm output (an f32 approximation on the device)."""
+    from dldt_amd import builders, lpt
+    r0 = (-90 / 64, 165 / 64)
+    r1 = (-45 / 128, 210 / 128)
+    g, meta = builders.matmul_zero_point_net(r0=r0, r1=r1)
+    assert meta["zero_points"] == (90.0, 45.0)
+    x = np.random.default_rng(5).normal(0, 1, (2, 48, 128)).astype(np.float32)
+    req = g.compile().create_request()
+    (out,) = req.infer(x)
+    h = req.matrix(meta["norm"]).astype(np.float64).reshape(2, 48, 128)
+
+    def fq(v, r):
+        lo, hi = float(np.float32(r[0])), float(np.float32(r[1]))
+        lv = np.rint((np.clip(v, lo, hi) - lo) / (hi - lo) * 255.0)
+        return lv, lo + lv / 255.0 * (hi - lo)
+
+    def linear(i, v):
+        w, b = meta["linear"][i]
+        wq, s_w = lpt.quantize_weights(w, 255)
+        return v @ (wq.astype(np.float64) * s_w.astype(np.float64).reshape(-1, 1)).T + b.astype(np.float64)
+
+    lv0, a0 = fq(h, r0)
+    d = np.abs(req.matrix(meta["a0"]).astype(np.int64).reshape(lv0.shape) - lv0.astype(np.int64))
+    assert d.max() <= 1 and (d > 0).mean() < 0.002
+    lv1, a1 = fq(linear(0, a0), r1)
+    d = np.abs(req.matrix(meta["a1"]).astype(np.int64).reshape(lv1.shape) - lv1.astype(np.int64))
+    assert d.max() <= 1 and (d > 0).mean() < 0.002
+    assert lv0.min() == 0 and lv0.max() == 255 and len(np.unique(lv1)) > 200       # both intervals are used to their ends
+    ref = linear(1, a1) + h
+    np.testing.assert_allclose(out, ref, rtol=0, atol=0.01 * np.abs(ref).max())
+    assert np.abs(out - ref).mean() < 2e-4 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("signed", [False, True])
+def test_concat_of_quantized_branches_equals_its_float_graph(orc, signed):
+    """three convolution branches, each behind the same FakeQuantize interval, concatenated and convolved again:
+    the transformed graph concatenates the levels and dequantizes once (concat.cpp:42-190)"""
+    import torch
+    import torch.nn.functional as F
+    from dldt_amd import builders, lpt
+    g, feeds, meta = builders.concat_net(signed=signed)
+    req = g.compile().create_request()
+    cat_dev, out_dev = req.infer(feeds["data"])
+
+    def conv(i, v):
+        w, b = meta["params"][i]
+        wq, s_w = lpt.quantize_weights(w, 255)
+        return F.conv2d(v, torch.from_numpy(wq.astype(np.float64) * s_w.astype(np.float64).reshape(-1, 1, 1, 1)),
+                        torch.from_numpy(b.astype(np.float64)), padding=w.shape[-1] // 2)
+
+    _, x = _fq64(feeds["data"].astype(np.float64), 1.0)
+    x = torch.from_numpy(x)
+    hi = float(meta["out_high"])
+    lo = -hi * 128.0 / 127.0 if signed else 0.0
+    parts = []
+    for i in range(len(meta["branches"])):
+        v = conv(i, x).numpy()
+        lv = np.rint((np.clip(v, lo, hi) - lo) / (hi - lo) * 255.0)
+        parts.append(lo + lv / 255.0 * (hi - lo))
+    cat = np.concatenate(parts, axis=1)
+    np.testing.assert_allclose(cat_dev, cat, rtol=0, atol=1.01 * (hi - lo) / 255.0)       # at most one level anywhere
+    assert (np.abs(cat_dev - cat) > 1e-5).mean() < 0.002
+    ref = np.maximum(conv(len(parts), torch.from_numpy(cat)).numpy(), 0.0)
+    np.testing.assert_allclose(out_dev, ref, rtol=0, atol=0.01 * ref.max())
+    assert np.abs(out_dev - ref).mean() < 2e-4 * ref.max()
