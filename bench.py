@@ -257,6 +257,31 @@ def main():
                           "note": "wall clock over StartAsync/Wait from page-locked host blobs (f32 NCHW input): H2D + kernels + D2H; "
                                   "bound by the host link, never the headline value"}
         del hreqs, blobs
+        # the same with input precision U8 (benchmark_app's default for image inputs, main.cpp: "-ip" / U8 for images):
+        # a plan of the same network whose input is the u8 image behind a Convert, a quarter of the H2D bytes
+        g8, _ = builders.resnet50(batch=args.batch, res=224, u8_input=True)
+        plan8 = g8.compile(0)
+        hreqs = [plan8.create_request() for _ in range(nreq)]
+        blobs = [r.host_buffers() for r in hreqs]
+        for hin, _ in blobs:
+            hin[0].array[...] = rng.integers(0, 256, hin[0].array.shape).astype(hin[0].array.dtype)
+        for rounds in (nreq, n_host):
+            t0 = time.perf_counter()
+            busy = [False] * nreq
+            for i in range(rounds):
+                k = i % nreq
+                if busy[k]:
+                    hreqs[k].wait()
+                hreqs[k].start(*blobs[k])
+                busy[k] = True
+            for k in range(nreq):
+                if busy[k]:
+                    hreqs[k].wait()
+            host8_ms = (time.perf_counter() - t0) * 1e3 / rounds
+        host_inclusive["u8_input"] = {"images_per_sec": args.batch / (host8_ms * 1e-3), "ms_per_step": host8_ms,
+                                      "h2d_bytes_per_step": sum(b.array.nbytes for b in blobs[0][0]),
+                                      "input_dtype": str(blobs[0][0][0].array.dtype)}
+        del hreqs, blobs, plan8, g8
 
     # per-step HIP events on the same stream: time spent in the int8 MFMA kernel
     preq = plan.create_request(perf_count=True)

@@ -249,18 +249,25 @@ def resnet50_fp32(P, x, stages=RESNET50_STAGES, record=None):
     return v.numpy()
 
 
-def resnet50(batch=1, res=224, seed=20211, classes=1000, width=64, stages=RESNET50_STAGES, calib_batch=2):
+def resnet50(batch=1, res=224, seed=20211, classes=1000, width=64, stages=RESNET50_STAGES, calib_batch=2, u8_input=False):
     """benchmark configuration 3 as a post-LPT graph.  Returns (graph, meta) where meta holds the
-    parameters, the calibrated ranges and the ids of every quantized activation."""
+    parameters, the calibrated ranges and the ids of every quantized activation.
+    u8_input: the graph input is a u8 image (values 0 .. 255, input precision U8 as benchmark_app sets it for image
+    inputs) behind a Convert; the first layer's weights are those of a model fed 0 .. 255 instead of 0 .. 1."""
     P = resnet50_weights(seed, classes, width, stages)
     rng = np.random.default_rng(seed + 1)
     calib = rng.uniform(0, 1, (calib_batch, 3, res, res)).astype(np.float32)
+    if u8_input:
+        P["conv1.w"] = (P["conv1.w"] / np.float32(255)).astype(np.float32)
+        calib = np.floor(calib * np.float32(256)).clip(0, 255).astype(np.float32)
     R = {}
     resnet50_fp32(P, calib, stages, R)
+    if u8_input:
+        R["input"] = 255.0                      # every byte is its own level
     net = QuantizedNet()
     g = net.g
     acts = {}
-    a = net.input("data", (batch, 3, res, res), R["input"])
+    a = net.input("data", (batch, 3, res, res), R["input"], u8=u8_input)
     acts["input"] = a
     a = net.conv(a, P["conv1.w"], P["conv1.b"], R["conv1"], strides=(2, 2), pads=(3, 3))
     acts["conv1"] = a

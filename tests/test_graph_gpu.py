@@ -48,6 +48,26 @@ def test_small_resnet_bit_exact(orc, batch):
     np.testing.assert_array_equal(outs[0].cpu().numpy(), got)
 
 
+def test_small_resnet_with_u8_image_input(orc):
+    """the same topology with input precision U8 (the image bytes are the first FakeQuantize's levels): the plan the
+    host-inclusive measurement with u8 blobs runs"""
+    from dldt_amd import builders
+    g, meta = builders.resnet50(batch=2, res=64, width=16, classes=10, seed=7, u8_input=True)
+    x = np.random.default_rng(98).integers(0, 256, (2, 3, 64, 64)).astype(np.uint8)
+    keep = [a["node"] for a in meta["acts"].values()]
+    want, kept = evaluate(orc, g.nodes, {"data": x}, keep=keep)
+    plan = g.compile()
+    assert plan.inputs[0]["dtype"] == 40
+    req = plan.create_request()
+    (got,) = req.infer(x)
+    np.testing.assert_array_equal(req.tensor(meta["acts"]["input"]["node"]), x)
+    for name, a in meta["acts"].items():
+        w = kept[a["node"]]
+        np.testing.assert_array_equal(req.tensor(a["node"]).reshape(w.shape), w, err_msg=name)
+        assert len(np.unique(w)) > 50, name                 # the calibrated ranges are used, not saturated
+    np.testing.assert_array_equal(got.view(np.uint32), want["logits"].view(np.uint32))
+
+
 def test_planner_reports_unsupported_nodes():
     from dldt_amd import HipieError
     from dldt_amd.graph import Graph
