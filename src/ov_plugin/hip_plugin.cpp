@@ -144,7 +144,7 @@ InferenceEngine::QueryNetworkResult Plugin::QueryNetwork(const InferenceEngine::
     std::unordered_set<std::string> original;
     for (const auto& node : function->get_ops()) original.insert(node->get_friendly_name());
 
-    // the same transformations as at load, then the engine's own verdict per node of the transformed graph
+    // the same transformations as at load, then the engine's own answer per node of the transformed graph
     const auto transformed = transform_network(function);
     TranslatedGraph t = translate(transformed, true);
     std::vector<int> ok(t.node_names.size(), 0);
