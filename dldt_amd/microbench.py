@@ -79,6 +79,24 @@ def _throughput_time(plan, nreq=3, reps=60, warm=9):
     return (time.perf_counter() - t0) / reps * 1e6
 
 
+def _best_variant(conv, run, tiles=(0, 1, 4, 5, 10, 11, 12, 18, 19, 20, 21, 22)):
+    """(us, variant): the fastest of the kernel variants that take the layer, as the load-time tuner would choose"""
+    from . import HipieError
+    best = None
+    for tile in tiles:
+        try:
+            conv.set_tile(tile)
+        except HipieError:
+            continue
+        if conv.get_tile() != tile:
+            continue
+        us = _time(run)
+        if best is None or us < best[0]:
+            best = (us, tile)
+    conv.set_tile(best[1])
+    return best
+
+
 def _row(name, us, macs=0, bytes_=0, bound=None):
     tops = 2.0 * macs / us / 1e6 if macs else 0.0
     gbs = bytes_ / us / 1e3 if bytes_ else 0.0
@@ -195,9 +213,9 @@ def config5():
                                fq=(256, np.full(n, -128e3, np.float32), np.full(n, 127e3, np.float32), -128.0, 127.0))
         conv = Convolution(w, xin, epilogue=ep)
         out = DeviceTensor(1, 1, T, n, out_dtype)
-        us = _time(lambda: conv.run(xin, out))
+        us, variant = _best_variant(conv, lambda: conv.run(xin, out))
         layer_us += us * count
-        rows.append(_row("cfg5 %s [%d,%d]x[%d,%d] -> %s" % (name, T, k, k, n, "f32" if out_dtype == F32 else "i8"), us,
+        rows.append(_row("cfg5 %s [%d,%d]x[%d,%d] -> %s (variant %d)" % (name, T, k, k, n, "f32" if out_dtype == F32 else "i8", variant), us,
                          macs=T * k * n, bytes_=T * k + k * n + T * n * (4 if out_dtype == F32 else 1), bound="mfma"))
 
     linear("QKV projection", H, 3 * H, I8)
@@ -264,11 +282,52 @@ def config5_graph():
     return rows
 
 
+def vendor_gemm():
+    """The int8 GEMM of the vendor library (hipBLASLt behind torch._int_mm: plain [M, K] x [K, N] -> i32, no
+    epilogue, no convolution addressing) on the GEMM shapes of ResNet-50 batch-64 layers and of the encoder's FFN,
+    beside this library's convolution / MatMul kernels on the same layers with raw i32 output (the best of the kernel
+    variants that take the layer, as the load-time tuner would choose)."""
+    import numpy as np
+    import torch
+    from . import Convolution, DeviceTensor
+    from .tensor import I32, U8B
+    layers = [("ResNet stage-1 1x1 64->256 @56x56", 64, 64, 56, 256, 1),
+              ("ResNet stage-2 3x3 128->128 @28x28", 64, 128, 28, 128, 3),
+              ("ResNet stage-3 3x3 256->256 @14x14", 64, 256, 14, 256, 3),
+              ("ResNet stage-3 1x1 1024->256 @14x14", 64, 1024, 14, 256, 1),
+              ("ResNet stage-3 1x1 256->1024 @14x14", 64, 256, 14, 1024, 1),
+              ("ResNet stage-4 3x3 512->512 @7x7", 64, 512, 7, 512, 3),
+              ("encoder FFN up 768->3072, 6144 rows", 1, 768, 0, 3072, 1),
+              ("encoder FFN down 3072->768, 6144 rows", 1, 3072, 0, 768, 1)]
+    rows = []
+    rng = np.random.default_rng(1)
+    for name, n, c, hw, oc, k in layers:
+        h, w_ = (hw, hw) if hw else (1, 6144)
+        M, K = n * h * w_, c * k * k
+        a = torch.randint(-128, 127, (M, K), dtype=torch.int8, device="cuda")
+        b = torch.randint(-128, 127, (K, oc), dtype=torch.int8, device="cuda")
+        us_vendor = _time(lambda: torch._int_mm(a, b))
+        del a, b
+        x = DeviceTensor(n, h, w_, c, U8B, halo=k // 2)
+        wts = rng.integers(-127, 128, (oc, c, k, k)).astype(np.int8)
+        conv = Convolution(wts, x, (1, 1), (1, 1), (k // 2, k // 2), (k // 2, k // 2))
+        out = DeviceTensor(n, h, w_, oc, I32)
+        best = _best_variant(conv, lambda: conv.run(x, out))
+        rows.append(_row("%s: vendor GEMM [%d, %d] x [%d, %d] -> i32" % (name, M, K, K, oc), us_vendor, macs=M * K * oc, bound="mfma"))
+        rows.append(_row("%s: this library, i32 output (variant %d)" % (name, best[1]), best[0], macs=M * K * oc, bound="mfma"))
+    M = 8192
+    a = torch.randint(-128, 127, (M, M), dtype=torch.int8, device="cuda")
+    b = torch.randint(-128, 127, (M, M), dtype=torch.int8, device="cuda")
+    rows.append(_row("vendor GEMM [8192, 8192] x [8192, 8192] -> i32 (what a large square problem reaches)",
+                     _time(lambda: torch._int_mm(a, b), reps=10, warm=2), macs=M * M * M, bound="mfma"))
+    return rows
+
+
 def main():
     import torch
     assert torch.cuda.is_available(), "microbench needs a GPU"
     which = sys.argv[1:] or ["1", "2", "3", "4", "5"]
-    table = {"1": config1, "2": config2, "3": config3, "4": config4, "5": config5, "encoder": config5_graph}
+    table = {"1": config1, "2": config2, "3": config3, "4": config4, "5": config5, "encoder": config5_graph, "vendor": vendor_gemm}
     print("| kernel / graph | us | TOP/s | GB/s | bound | fraction of peak | notes |")
     print("|---|---|---|---|---|---|---|")
     for k in which:
