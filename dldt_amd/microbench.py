@@ -320,6 +320,13 @@ def vendor_gemm():
     b = torch.randint(-128, 127, (M, M), dtype=torch.int8, device="cuda")
     rows.append(_row("vendor GEMM [8192, 8192] x [8192, 8192] -> i32 (what a large square problem reaches)",
                      _time(lambda: torch._int_mm(a, b), reps=10, warm=2), macs=M * M * M, bound="mfma"))
+    del a, b
+    x = DeviceTensor(1, 1, M, M, U8B)
+    conv = Convolution(rng.integers(-127, 128, (M, M, 1, 1)).astype(np.int8), x)
+    out = DeviceTensor(1, 1, M, M, I32)
+    us, tile = _best_variant(conv, lambda: conv.run(x, out), tiles=(0, 4, 5, 10, 18, 19, 20, 21, 22))
+    rows.append(_row("this library on the same problem (1 x 1 convolution, 8192 channels, 8192 pixels, variant %d)" % tile, us,
+                     macs=M * M * M, bound="mfma"))
     return rows
 
 
