@@ -1,0 +1,69 @@
+// Diagnostics: what the device's matrix pipe delivers with nothing else in the way.  The published dense int8 peak
+// is a clock times a count of units; the rate a kernel can reach is what the device sustains with every SIMD issuing
+// matrix instructions back to back from registers - no memory, no LDS, no epilogue.  Roofline fractions read against
+// this number say how much of the gap to the published peak belongs to the kernels.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "hipie.h"
+
+namespace hipie {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// four independent accumulators per wave, so that consecutive matrix instructions never wait for each other
+__global__ __launch_bounds__(256) void mfma_rate_kernel(int iters, int* sink) {
+    const int lane = threadIdx.x & 63;
+    v4i a = {lane, lane + 1, lane + 2, lane + 3}, b = {lane ^ 5, lane ^ 9, lane ^ 17, lane ^ 33};
+    v16i acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[i], 0, 0, 0);
+    }
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s += acc[i][r];
+    if (s == 0x7fffffff) sink[0] = s;       // keeps the products alive; not taken for these operands
+}
+
+}  // namespace
+}  // namespace hipie
+
+using namespace hipie;
+
+extern "C" int hipie_probe_mfma_rate(int device, int iterations, int waves_per_simd, double* tops, double* milliseconds) {
+    return guarded([&] {
+        HIPIE_REQUIRE(tops && iterations > 0 && iterations <= (1 << 20) && waves_per_simd >= 1 && waves_per_simd <= 8,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_probe_mfma_rate: iterations %d, waves per SIMD %d", iterations, waves_per_simd);
+        DeviceGuard g(device);
+        hipDeviceProp_t prop;
+        HIPIE_CHECK_HIP(hipGetDeviceProperties(&prop, device));
+        int* sink = nullptr;
+        HIPIE_CHECK_HIP(hipMalloc(&sink, 16));
+        const int blocks = prop.multiProcessorCount * waves_per_simd;      // four waves each: one per SIMD
+        hipEvent_t e0, e1;
+        HIPIE_CHECK_HIP(hipEventCreate(&e0));
+        HIPIE_CHECK_HIP(hipEventCreate(&e1));
+        hipLaunchKernelGGL(mfma_rate_kernel, dim3(blocks), dim3(256), 0, nullptr, 16, sink);      // warm-up
+        HIPIE_CHECK_HIP(hipEventRecord(e0, nullptr));
+        hipLaunchKernelGGL(mfma_rate_kernel, dim3(blocks), dim3(256), 0, nullptr, iterations, sink);
+        HIPIE_CHECK_HIP(hipEventRecord(e1, nullptr));
+        HIPIE_CHECK_HIP(hipEventSynchronize(e1));
+        float ms = 0.f;
+        HIPIE_CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+        HIPIE_CHECK_HIP(hipEventDestroy(e0));
+        HIPIE_CHECK_HIP(hipEventDestroy(e1));
+        HIPIE_CHECK_HIP(hipFree(sink));
+        const double ops = 2.0 * 32 * 32 * 32 * 4.0 * iterations * 4.0 * blocks;     // per instruction x 4 per iteration x 4 waves
+        *tops = ops / (ms * 1e-3) / 1e12;
+        if (milliseconds) *milliseconds = ms;
+    });
+}

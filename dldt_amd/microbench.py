@@ -330,11 +330,26 @@ def vendor_gemm():
     return rows
 
 
+def mfma_rate():
+    """the matrix pipe alone: every SIMD issuing int8 matrix instructions from registers, 1 to 4 waves per SIMD"""
+    import ctypes
+    from ._lib import check, lib
+    rows = []
+    for waves in (1, 2, 4):
+        for iters in (20000, 200000):
+            tops, ms = ctypes.c_double(), ctypes.c_double()
+            check(lib().hipie_probe_mfma_rate(0, iters, waves, ctypes.byref(tops), ctypes.byref(ms)))
+            r = {"row": "int8 matrix instructions from registers, %d wave(s) per SIMD, %.1f ms" % (waves, ms.value),
+                 "us": ms.value * 1e3, "TOP/s": tops.value, "GB/s": 0.0, "bound": "mfma", "frac": tops.value / INT8_PEAK_TOPS}
+            rows.append(r)
+    return rows
+
+
 def main():
     import torch
     assert torch.cuda.is_available(), "microbench needs a GPU"
     which = sys.argv[1:] or ["1", "2", "3", "4", "5"]
-    table = {"1": config1, "2": config2, "3": config3, "4": config4, "5": config5, "encoder": config5_graph, "vendor": vendor_gemm}
+    table = {"1": config1, "2": config2, "3": config3, "4": config4, "5": config5, "encoder": config5_graph, "vendor": vendor_gemm, "mfma": mfma_rate}
     print("| kernel / graph | us | TOP/s | GB/s | bound | fraction of peak | notes |")
     print("|---|---|---|---|---|---|---|")
     for k in which:

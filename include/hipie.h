@@ -144,6 +144,10 @@ int hipie_fq_uses_reciprocal(const hipie_fq* fq);
  * over all 2^23 significands.  *verified = 1 when every divisor has a pair (otherwise the epilogue
  * keeps the reciprocal-with-corrections sequence and zh, zl are unspecified). */
 int hipie_fq_div2_constants(int device, const float* d, int64_t n, float* zh, float* zl, int* verified);
+/* Diagnostics, no counterpart in the reference: the int8 rate (TOP/s) the device sustains when every SIMD issues
+ * v_mfma_i32_32x32x32_i8 back to back from registers (waves_per_simd waves of 4 x iterations independent instructions,
+ * no memory traffic) - the ceiling a kernel's roofline fraction can be read against beside the published peak. */
+int hipie_probe_mfma_rate(int device, int iterations, int waves_per_simd, double* tops, double* milliseconds);
 
 /* ======================================================================================
  * 1b. Fused f32 epilogue applied to i32 accumulators, in this fixed order (each step one IEEE
