@@ -836,11 +836,16 @@ __global__ __launch_bounds__(256, 2) void conv_stem_kernel(const ConvArgs a) {
     const int w_pieces = 64 * a.stem_kh * 2;
     const int8_t* w0 = a.wgt + static_cast<int64_t>(oc0) * a.wgt_ld;
     v4i wv[4];
+    int w_at[4];                                                            // where the piece goes in LDS
+    const int ppr = a.stem_kh * 2;                                          // 16-byte pieces per weight row
+    const float inv_ppr = 1.0f / static_cast<float>(ppr);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int i = min(tid + j * 256, w_pieces - 1);
-        const int row = i / (a.stem_kh * 2), pc = i - row * (a.stem_kh * 2);
+        int row, pc;
+        fast_divmod(i, ppr, inv_ppr, row, pc);
         wv[j] = *reinterpret_cast<const v4i*>(w0 + (static_cast<int64_t>(row) * a.wgt_ld + pc * 16));
+        w_at[j] = row * kStemWRow + pc * 16;
     }
 #pragma unroll
     for (int j = 0; j < PD; ++j) {
@@ -848,11 +853,8 @@ __global__ __launch_bounds__(256, 2) void conv_stem_kernel(const ConvArgs a) {
         if (i < total_dw) *reinterpret_cast<uint32_t*>(&sPatch[i * 4]) = pv[j];
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int i = tid + j * 256;
-        const int row = i / (a.stem_kh * 2), pc = i - row * (a.stem_kh * 2);
-        if (i < w_pieces) *reinterpret_cast<v4i*>(&sW[row * kStemWRow + pc * 16]) = wv[j];
-    }
+    for (int j = 0; j < 4; ++j)
+        if (tid + j * 256 < w_pieces) *reinterpret_cast<v4i*>(&sW[w_at[j]]) = wv[j];
     // window start of the lane's two pixels in the patch (bytes), filter row 0
     int b0[2];
 #pragma unroll
