@@ -24,6 +24,11 @@ __device__ __forceinline__ int64_t workgroup_index(int per_xcd) {
     return static_cast<int64_t>(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
 }
 
+// reciprocals for the decode of a lane's item index; inv_cgroups = 0 says "too many items for them"
+struct ItemDecode {
+    float inv_cgroups, inv_pairs, inv_oh;
+};
+
 __device__ __forceinline__ void mac_bytes(uint32_t x, uint32_t w, int& a0, int& a1, int& a2, int& a3) {
     a0 += static_cast<int>(static_cast<int8_t>(x)) * static_cast<int>(static_cast<int8_t>(w));
     a1 += static_cast<int>(static_cast<int8_t>(x >> 8)) * static_cast<int>(static_cast<int8_t>(w >> 8));
@@ -33,11 +38,17 @@ __device__ __forceinline__ void mac_bytes(uint32_t x, uint32_t w, int& a0, int& 
 
 template <uint32_t F>
 __global__ __launch_bounds__(256) void dwconv_kernel(const ConvArgs a, int KH, int KW, int dil_h, int dil_w,
-                                                     int cgroups, int64_t items, int per_xcd) {
+                                                     int cgroups, int64_t items, int per_xcd, ItemDecode dec) {
     const int64_t item = workgroup_index(per_xcd) * 256 + threadIdx.x;
     if (item >= items) return;
-    const int cgi = static_cast<int>(item % cgroups);
-    const int m0 = static_cast<int>(item / cgroups) * 2;
+    int cgi, m_pair;
+    if (dec.inv_cgroups > 0.f) {
+        fast_divmod(static_cast<int>(item), cgroups, dec.inv_cgroups, m_pair, cgi);
+    } else {
+        cgi = static_cast<int>(item % cgroups);
+        m_pair = static_cast<int>(item / cgroups);
+    }
+    const int m0 = m_pair * 2;
     const int oc_lane = cgi * 32;
     int32_t base[2];
 #pragma unroll
@@ -78,16 +89,37 @@ __global__ __launch_bounds__(256) void dwconv_kernel(const ConvArgs a, int KH, i
 // per tap, and the two windows share their overlapping input columns in registers.
 template <uint32_t F, int STRIDE>
 __global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cgroups, int pairs_per_row, int64_t items,
-                                                        int per_xcd) {
+                                                        int per_xcd, ItemDecode dec) {
+    // The filter rows of all channels ([3][channels] dwords, three taps each) go through LDS: read from memory they
+    // are twelve more 16-byte vector loads per lane beside the fifteen of the input, and the kernel is bound by the
+    // rate at which the texture addresser takes those (its busy counter reads 80 % of the kernel's time).
+    extern __shared__ __attribute__((aligned(16))) uint32_t sFilt[];
+    const int cs = cgroups * 16;
+    for (int r = 0; r < 3; ++r)
+        for (int q = threadIdx.x; q < cs / 4; q += 256)
+            *reinterpret_cast<uint4*>(&sFilt[r * cs + 4 * q]) =
+                *reinterpret_cast<const uint4*>(a.wgt2 + (static_cast<int64_t>(r) * a.OCp + 4 * q) * 4);
+    __syncthreads();
     const int64_t item = workgroup_index(per_xcd) * 256 + threadIdx.x;
     if (item >= items) return;
-    const int cgi = static_cast<int>(item % cgroups);
-    const int pair = static_cast<int>(item / cgroups);
-    const int oc_lane = cgi * 16;
-    // pair -> (n, oh, ow0): pairs never straddle a row
+    // item -> (channel group, pair) -> (n, oh, ow0): pairs never straddle a row.  Below 2^24 items the quotients come
+    // from reciprocals (exact there); 64-bit and 32-bit integer divisions per lane cost more than the lane's multiplies.
     const int OH = a.OHOW / a.OW;
-    const int rowi = pair / pairs_per_row, ow0 = (pair - rowi * pairs_per_row) * 2;
-    const int n = rowi / OH, oh = rowi - n * OH;
+    int cgi, pair, rowi, ow0, n, oh;
+    if (dec.inv_cgroups > 0.f) {
+        fast_divmod(static_cast<int>(item), cgroups, dec.inv_cgroups, pair, cgi);
+        fast_divmod(pair, pairs_per_row, dec.inv_pairs, rowi, ow0);
+        fast_divmod(rowi, OH, dec.inv_oh, n, oh);
+        ow0 *= 2;
+    } else {
+        cgi = static_cast<int>(item % cgroups);
+        pair = static_cast<int>(item / cgroups);
+        rowi = pair / pairs_per_row;
+        ow0 = (pair - rowi * pairs_per_row) * 2;
+        n = rowi / OH;
+        oh = rowi - n * OH;
+    }
+    const int oc_lane = cgi * 16;
     constexpr int COLS = 3 + STRIDE;   // input columns under the two windows
     const int8_t* xp = a.in + (static_cast<int64_t>(n) * a.in_sn + oh * STRIDE * a.in_sh + ow0 * STRIDE * a.in_sw +
                                a.in_origin + oc_lane);
@@ -97,7 +129,7 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cg
     for (int r = 0; r < 3; ++r)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-            wr[r][q] = *reinterpret_cast<const uint4*>(a.wgt2 + (static_cast<int64_t>(r) * a.OCp + oc_lane + 4 * q) * 4);
+            wr[r][q] = *reinterpret_cast<const uint4*>(&sFilt[r * cs + oc_lane + 4 * q]);
     // the last pair of an odd row has one pixel: its second window's extra columns are clamped onto
     // existing ones (the results are discarded)
     const bool two = ow0 + 1 < a.OW;
@@ -419,15 +451,20 @@ void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, int 
         return;
     }
     if (KH == 3 && KW == 3 && dil_h == 1 && dil_w == 1 && a.conv_sh == a.conv_sw && (a.conv_sh == 1 || a.conv_sh == 2) &&
-        known && !(a.flags & CF_RES)) {
+        known && !(a.flags & CF_RES) && std::min(a.OCp, a.in_sw) * 12 <= 48 * 1024) {   // (the filter rows fit their LDS)
         const int cgroups = std::min(a.OCp, a.in_sw) / 16;   // groups of 16 channels that exist in the tensors
         const int pairs_per_row = (a.OW + 1) / 2;
         const int64_t items = static_cast<int64_t>(a.M / a.OW) * pairs_per_row * cgroups;
         const XcdGrid xg(ceil_div(items, 256));
         const dim3 grid(xg.blocks), block(256);
         const int per_xcd = xg.per_xcd;
+        const size_t filt_lds = static_cast<size_t>(cgroups) * 16 * 3 * 4;       // at most 48 KB at 4096 channels
+        ItemDecode dec{0.f, 0.f, 0.f};
+        if (items < (1 << 24))
+            dec = ItemDecode{1.0f / static_cast<float>(cgroups), 1.0f / static_cast<float>(pairs_per_row),
+                             1.0f / static_cast<float>(a.OHOW / a.OW)};
 #define HIPIE_LAUNCH_DW3(FLAGS, STRIDE) \
-    hipLaunchKernelGGL((dwconv3x3_kernel<FLAGS, STRIDE>), grid, block, 0, s, a, cgroups, pairs_per_row, items, per_xcd)
+    hipLaunchKernelGGL((dwconv3x3_kernel<FLAGS, STRIDE>), grid, block, filt_lds, s, a, cgroups, pairs_per_row, items, per_xcd, dec)
         if (core == E_PLAIN0) {
             if (a.conv_sh == 1) HIPIE_LAUNCH_DW3(E_PLAIN0, 1); else HIPIE_LAUNCH_DW3(E_PLAIN0, 2);
         } else if (core == E_SCALEFQ0) {
@@ -443,11 +480,13 @@ void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, int 
     const XcdGrid xg(ceil_div(items, 256));
     const dim3 grid(xg.blocks), block(256);
     const int per_xcd = xg.per_xcd;
+    ItemDecode dec{0.f, 0.f, 0.f};
+    if (items < (1 << 24)) dec.inv_cgroups = 1.0f / static_cast<float>(cgroups);
     switch (core) {
-    case E_PLAIN0: hipLaunchKernelGGL((dwconv_kernel<E_PLAIN0>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
-    case E_CLAMPFQ: hipLaunchKernelGGL((dwconv_kernel<E_CLAMPFQ>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
-    case E_SCALEFQ0: hipLaunchKernelGGL((dwconv_kernel<E_SCALEFQ0>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
-    default: hipLaunchKernelGGL((dwconv_kernel<kDyn>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd); break;
+    case E_PLAIN0: hipLaunchKernelGGL((dwconv_kernel<E_PLAIN0>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd, dec); break;
+    case E_CLAMPFQ: hipLaunchKernelGGL((dwconv_kernel<E_CLAMPFQ>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd, dec); break;
+    case E_SCALEFQ0: hipLaunchKernelGGL((dwconv_kernel<E_SCALEFQ0>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd, dec); break;
+    default: hipLaunchKernelGGL((dwconv_kernel<kDyn>), grid, block, 0, s, a, KH, KW, dil_h, dil_w, cgroups, items, per_xcd, dec); break;
     }
 }
 
