@@ -93,12 +93,15 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cg
     // The filter rows of all channels ([3][channels] dwords, three taps each) go through LDS: read from memory they
     // are twelve more 16-byte vector loads per lane beside the fifteen of the input, and the kernel is bound by the
     // rate at which the texture addresser takes those (its busy counter reads 80 % of the kernel's time).
+    // The epilogue's per-channel tables and the accumulator corrections take the same way (another twenty loads).
     extern __shared__ __attribute__((aligned(16))) uint32_t sFilt[];
     const int cs = cgroups * 16;
+    float* const sTab = reinterpret_cast<float*>(sFilt + 3 * cs);
     for (int r = 0; r < 3; ++r)
         for (int q = threadIdx.x; q < cs / 4; q += 256)
             *reinterpret_cast<uint4*>(&sFilt[r * cs + 4 * q]) =
                 *reinterpret_cast<const uint4*>(a.wgt2 + (static_cast<int64_t>(r) * a.OCp + 4 * q) * 4);
+    stage_params<F>(a, 0, (lds_float_ptr)sTab, cs, static_cast<int>(threadIdx.x), 256);
     __syncthreads();
     const int64_t item = workgroup_index(per_xcd) * 256 + threadIdx.x;
     if (item >= items) return;
@@ -142,8 +145,9 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cg
         }
     v16i acc[2][2];
     {
-        const int4 c0 = *reinterpret_cast<const int4*>(a.corr + oc_lane), c1 = *reinterpret_cast<const int4*>(a.corr + oc_lane + 4);
-        const int4 c2 = *reinterpret_cast<const int4*>(a.corr + oc_lane + 8), c3 = *reinterpret_cast<const int4*>(a.corr + oc_lane + 12);
+        const int32_t* const corr = reinterpret_cast<const int32_t*>(sTab) + PT_COUNT * cs + oc_lane;
+        const int4 c0 = *reinterpret_cast<const int4*>(corr), c1 = *reinterpret_cast<const int4*>(corr + 4);
+        const int4 c2 = *reinterpret_cast<const int4*>(corr + 8), c3 = *reinterpret_cast<const int4*>(corr + 12);
         const int cv[16] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w, c2.x, c2.y, c2.z, c2.w, c3.x, c3.y, c3.z, c3.w};
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb)
@@ -198,7 +202,7 @@ __global__ __launch_bounds__(256) void dwconv3x3_kernel(const ConvArgs a, int cg
         res_off[pb] = static_cast<int64_t>(n) * a.res_sn + oh * a.res_sh + ow * a.res_sw + oc_lane;
     }
     v16f none[2][2];
-    epilogue<F, 1>(a, acc, oc_lane, valid, out_off, res_off, none, nullptr, 0, 0);
+    epilogue<F, 1>(a, acc, oc_lane, valid, out_off, res_off, none, (lds_cfloat_ptr)sTab, cs, 0);
 }
 
 
@@ -451,20 +455,29 @@ void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, int 
         return;
     }
     if (KH == 3 && KW == 3 && dil_h == 1 && dil_w == 1 && a.conv_sh == a.conv_sw && (a.conv_sh == 1 || a.conv_sh == 2) &&
-        known && !(a.flags & CF_RES) && std::min(a.OCp, a.in_sw) * 12 <= 48 * 1024) {   // (the filter rows fit their LDS)
+        known && !(a.flags & CF_RES) && std::min(a.OCp, a.in_sw) * (3 + PT_ROWS) * 4 <= 60 * 1024) {   // (filter rows and tables fit their LDS)
         const int cgroups = std::min(a.OCp, a.in_sw) / 16;   // groups of 16 channels that exist in the tensors
         const int pairs_per_row = (a.OW + 1) / 2;
         const int64_t items = static_cast<int64_t>(a.M / a.OW) * pairs_per_row * cgroups;
         const XcdGrid xg(ceil_div(items, 256));
         const dim3 grid(xg.blocks), block(256);
         const int per_xcd = xg.per_xcd;
-        const size_t filt_lds = static_cast<size_t>(cgroups) * 16 * 3 * 4;       // at most 48 KB at 4096 channels
+        const size_t filt_lds = static_cast<size_t>(cgroups) * 16 * (3 + PT_ROWS) * 4;   // filter rows and tables: 60 bytes per channel
         ItemDecode dec{0.f, 0.f, 0.f};
         if (items < (1 << 24))
             dec = ItemDecode{1.0f / static_cast<float>(cgroups), 1.0f / static_cast<float>(pairs_per_row),
                              1.0f / static_cast<float>(a.OHOW / a.OW)};
-#define HIPIE_LAUNCH_DW3(FLAGS, STRIDE) \
-    hipLaunchKernelGGL((dwconv3x3_kernel<FLAGS, STRIDE>), grid, block, filt_lds, s, a, cgroups, pairs_per_row, items, per_xcd, dec)
+#define HIPIE_LAUNCH_DW3(FLAGS, STRIDE)                                                                                     \
+    do {                                                                                                                    \
+        static bool attr_set = false;                                                                                       \
+        if (!attr_set) {                                                                                                    \
+            HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&dwconv3x3_kernel<FLAGS, STRIDE>),            \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));                    \
+            attr_set = true;                                                                                                \
+        }                                                                                                                   \
+        hipLaunchKernelGGL((dwconv3x3_kernel<FLAGS, STRIDE>), grid, block, filt_lds, s, a, cgroups, pairs_per_row, items,   \
+                           per_xcd, dec);                                                                                   \
+    } while (0)
         if (core == E_PLAIN0) {
             if (a.conv_sh == 1) HIPIE_LAUNCH_DW3(E_PLAIN0, 1); else HIPIE_LAUNCH_DW3(E_PLAIN0, 2);
         } else if (core == E_SCALEFQ0) {
