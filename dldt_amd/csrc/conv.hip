@@ -243,6 +243,17 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     gemm(a.in + batch_offset(a, batch, a.batch_in, a.batch_in_o), a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
          a.wgt + batch_offset(a, batch, a.batch_wgt, a.batch_wgt_o), a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused, a.flat_in != 0);
     const int m0 = pix0 + wpix * 64 + l32;
+    if (a.pix_corr) {   // uniform: MatMul between activations whose right operand is stored as level - 128
+        const int32_t* pc = a.pix_corr + static_cast<int64_t>(batch) * a.batch_pix_corr;
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb) {
+            const int32_t v = pc[min(m0 + 32 * pb, a.M - 1)];
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[ob][pb][r] += v;
+        }
+    }
     // the K loop ends with a barrier, so the operand tiles are free: every wave takes 8 KB of them as
     // the staging buffer of its f32 stores (2 (BOC + BPIX) 64 bytes cover 8 KB per wave for all shapes)
     constexpr int kStageWavesA = 2 * BOC * kRow / 8192;
@@ -1375,11 +1386,11 @@ struct hipie_conv {
     Epilogue epi;
 };
 
-// corr[b][n] = factor * sum_k Bt[b][n][k] for the rows n < N of every batch element b (0 for the padded rows up
-// to Np): a thread per row, 16 bytes a step, v_dot4_i32_i8 against four ones
+// corr[b][n] = factor * sum_k Bt[b][n][k] + addend for the rows n < N of every batch element b (0 for the padded
+// rows up to Np): a thread per row, 16 bytes a step, v_dot4_i32_i8 against four ones
 __global__ __launch_bounds__(256) void row_sums_kernel(const int8_t* bt, int64_t ldb, int64_t stride_b, int64_t outer_b,
                                                        int32_t batch_inner, int32_t N, int32_t Np, int32_t K, int32_t factor,
-                                                       int32_t* corr, int64_t rows) {
+                                                       int32_t addend, int32_t* corr, int64_t rows) {
     const int64_t row = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (row >= rows) return;
     const int b = static_cast<int>(row / Np), n = static_cast<int>(row - static_cast<int64_t>(b) * Np);
@@ -1399,14 +1410,15 @@ __global__ __launch_bounds__(256) void row_sums_kernel(const int8_t* bt, int64_t
             sum = __builtin_amdgcn_sdot4(static_cast<int>(v.w), 0x01010101, sum, false);
         }
     }
-    corr[row] = sum * factor;
+    corr[row] = n < N ? sum * factor + addend : 0;
 }
 
 static void launch_row_sums(const int8_t* bt, int64_t ldb, int64_t stride_b, int64_t outer_b, int32_t batch_inner, int32_t N,
-                            int32_t Np, int32_t K, int32_t factor, int32_t* corr, int32_t batches, hipStream_t s) {
+                            int32_t Np, int32_t K, int32_t factor, int32_t addend, int32_t* corr, int32_t batches,
+                            hipStream_t s) {
     const int64_t rows = static_cast<int64_t>(batches) * Np;
     hipLaunchKernelGGL(row_sums_kernel, dim3(static_cast<uint32_t>(ceil_div(rows, 256))), dim3(256), 0, s, bt, ldb, stride_b,
-                       outer_b, batch_inner, N, Np, K, factor, corr, rows);
+                       outer_b, batch_inner, N, Np, K, factor, addend, corr, rows);
 }
 
 struct hipie_matmul {
@@ -1494,12 +1506,13 @@ int hipie_matmul_create(int device, const hipie_matmul_desc* desc, const hipie_e
     return guarded([&] {
         HIPIE_REQUIRE(desc && epilogue && out, HIPIE_PARAMETER_MISMATCH, "hipie_matmul_create: null argument");
         const hipie_matmul_desc& d = *desc;
-        HIPIE_REQUIRE((d.a_dtype == HIPIE_I8 || d.a_dtype == HIPIE_U8B) && d.b_dtype == HIPIE_I8, HIPIE_NOT_IMPLEMENTED,
-                      "hipie_matmul_create: the left operand must be i8 or u8, the right operand i8 (a u8 right operand "
-                      "would need one correction per output row)");
-        const int lo = d.a_dtype == HIPIE_U8B ? 0 : -128;
-        HIPIE_REQUIRE(d.a_zero_point >= lo && d.a_zero_point <= lo + 255 && (d.a_dtype == HIPIE_U8B || d.a_zero_point == 0),
+        HIPIE_REQUIRE((d.a_dtype == HIPIE_I8 || d.a_dtype == HIPIE_U8B) && (d.b_dtype == HIPIE_I8 || d.b_dtype == HIPIE_U8B),
+                      HIPIE_NOT_IMPLEMENTED, "hipie_matmul_create: operand dtypes %d, %d (i8 or u8 expected)", d.a_dtype,
+                      d.b_dtype);
+        HIPIE_REQUIRE(d.a_dtype == HIPIE_U8B ? (d.a_zero_point >= 0 && d.a_zero_point <= 255) : d.a_zero_point == 0,
                       HIPIE_PARAMETER_MISMATCH, "hipie_matmul_create: zero point %d of the left operand", d.a_zero_point);
+        HIPIE_REQUIRE(d.b_dtype == HIPIE_U8B ? (d.b_zero_point >= 0 && d.b_zero_point <= 255) : d.b_zero_point == 0,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_matmul_create: zero point %d of the right operand", d.b_zero_point);
         HIPIE_REQUIRE(d.k > 0 && d.n > 0 && d.k % 64 == 0, HIPIE_NOT_IMPLEMENTED,
                       "hipie_matmul_create: K=%d must be a positive multiple of 64", d.k);
         auto m = std::make_unique<hipie_matmul>();
@@ -1534,10 +1547,21 @@ int hipie_matmul_run_nested(const hipie_matmul* mm, const void* a_ptr, int64_t l
                                       outer_o, m, batch, batch_outer, nullptr, 0, stream);
 }
 
-int hipie_matmul_workspace_size(const hipie_matmul* mm, int32_t batch, int32_t batch_outer, size_t* bytes) {
+// workspace layout: [batches][Np] sums over the right operand's rows (u8 left operand), then [batches][round_up(m, 4)]
+// sums over the left operand's rows (u8 right operand)
+static size_t matmul_ws_left(const hipie_matmul* mm, int64_t batches) {
+    return mm->d.a_dtype == HIPIE_U8B ? static_cast<size_t>(batches * mm->Np) * sizeof(int32_t) : 0;
+}
+static size_t matmul_ws_right(const hipie_matmul* mm, int64_t m, int64_t batches) {
+    return mm->d.b_dtype == HIPIE_U8B ? static_cast<size_t>(batches * round_up(m, 4)) * sizeof(int32_t) : 0;
+}
+
+int hipie_matmul_workspace_size(const hipie_matmul* mm, int32_t m, int32_t batch, int32_t batch_outer, size_t* bytes) {
     return guarded([&] {
-        HIPIE_REQUIRE(mm && bytes && batch >= 0 && batch_outer >= 0, HIPIE_PARAMETER_MISMATCH, "hipie_matmul_workspace_size: argument");
-        *bytes = mm->d.a_dtype == HIPIE_U8B ? static_cast<size_t>(batch) * batch_outer * mm->Np * sizeof(int32_t) : 0;
+        HIPIE_REQUIRE(mm && bytes && m >= 0 && batch >= 0 && batch_outer >= 0, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_matmul_workspace_size: argument");
+        const int64_t batches = static_cast<int64_t>(batch) * batch_outer;
+        *bytes = matmul_ws_left(mm, batches) + matmul_ws_right(mm, m, batches);
     });
 }
 
@@ -1598,18 +1622,35 @@ int hipie_matmul_run_nested_ws(const hipie_matmul* mm, const void* a_ptr, int64_
         a.batch_wgt_o = outer_b;
         a.batch_out_o = outer_o;
         DeviceGuard g(mm->device);
-        if (d.a_dtype == HIPIE_U8B) {
-            // sum_k (q_k - z) b_k = sum_k (q_k - 128) b_k + (128 - z) sum_k b_k: the sums over K of the right operand's
-            // rows, one row of corrections per batch element, computed in front of the product on the same stream
-            const size_t need = static_cast<size_t>(batch) * batch_outer * mm->Np * sizeof(int32_t);
-            HIPIE_REQUIRE(workspace && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 16 == 0,
+        // Operands stored as level - 128 (u8): with a' = a - 128, b' = b - 128 the stored bytes and za, zb the levels that
+        // stand for 0.0,
+        //   sum_k (a_k - za)(b_k - zb) = sum_k a'_k b'_k + (128 - za) sum_k b'_k + (128 - zb) (sum_k a'_k + K (128 - za)).
+        // The second term is one number per output column and batch element (sums over the right operand's rows), the
+        // third one per output row (sums over the left operand's rows); both are computed on the same stream in front
+        // of the product.  An i8 operand is its own a' with "128 - z" = 0.
+        const int64_t batches = static_cast<int64_t>(batch) * batch_outer;
+        const size_t ws_left = matmul_ws_left(mm, batches), ws_right = matmul_ws_right(mm, m, batches);
+        if (ws_left + ws_right > 0)
+            HIPIE_REQUIRE(workspace && workspace_bytes >= ws_left + ws_right && reinterpret_cast<uintptr_t>(workspace) % 16 == 0,
                           HIPIE_PARAMETER_MISMATCH,
-                          "hipie_matmul_run: a u8 left operand needs a workspace of %zu bytes (hipie_matmul_workspace_size)", need);
+                          "hipie_matmul_run: a u8 operand needs a workspace of %zu bytes (hipie_matmul_workspace_size)",
+                          ws_left + ws_right);
+        const int32_t fa = d.a_dtype == HIPIE_U8B ? 128 - d.a_zero_point : 0;
+        const int32_t fb = d.b_dtype == HIPIE_U8B ? 128 - d.b_zero_point : 0;
+        if (d.a_dtype == HIPIE_U8B) {
             launch_row_sums(static_cast<const int8_t*>(bt_ptr), ldb, stride_b, outer_b, batch_outer > 1 ? batch : 0, d.n,
-                            static_cast<int32_t>(mm->Np), d.k, 128 - d.a_zero_point, static_cast<int32_t*>(workspace),
+                            static_cast<int32_t>(mm->Np), d.k, fa, 0, static_cast<int32_t*>(workspace),
                             batch * batch_outer, as_stream(stream));
             a.corr = static_cast<const int32_t*>(workspace);
             a.batch_corr = static_cast<int32_t>(mm->Np);
+        }
+        if (d.b_dtype == HIPIE_U8B) {
+            int32_t* rows = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + ws_left);
+            const int32_t mp = static_cast<int32_t>(round_up(m, 4));
+            launch_row_sums(static_cast<const int8_t*>(a_ptr), lda, stride_a, outer_a, batch_outer > 1 ? batch : 0, m, mp,
+                            d.k, fb, fb * fa * d.k, rows, batch * batch_outer, as_stream(stream));
+            a.pix_corr = rows;
+            a.batch_pix_corr = mp;
         }
         const bool wide = d.n > 64;
         const int boc = wide ? 128 : 64, bpix = wide ? 128 : 256;

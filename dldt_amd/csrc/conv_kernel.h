@@ -94,6 +94,10 @@ struct ConvArgs {
     int32_t batch_inner;
     int64_t batch_in_o, batch_wgt_o, batch_out_o;
     int32_t batch_corr;              // accumulator corrections per batch element: entries from one batch's row to the next (0: one row for all)
+    // batched MatMul with a u8 right operand: one integer per output ROW (pixel), added to every accumulator of the
+    // row in front of the epilogue; batch element b's rows start at pix_corr + b * batch_pix_corr.  nullptr: none
+    const int32_t* pix_corr;
+    int32_t batch_pix_corr;
     int32_t wgt_ld, wgt_rows, wgt_plain;
     // fused shortcut convolution (CF_RES_GEMM): a second operand set accumulated first; its
     // dequantised result stays in registers as the residual of the main convolution

@@ -582,11 +582,11 @@ struct GlueStep : Step {
     }
 };
 
-// MatMul between two activations (i8 or u8 on the left, i8 on the right), batched over one or two leading dimensions
+// MatMul between two activations (each i8 or u8), batched over one or two leading dimensions
 struct BatchMatMulStep : Step {
     View a, b;                     // b as [.., N, K] with K contiguous
     int out = -1;
-    int ws = -1;                   // row sums of the right operand, one row per batch element (u8 left operand only)
+    int ws = -1;                   // the sums over K that a u8 operand asks for (hipie_matmul_workspace_size bytes)
     int64_t lda = 0, sa = 0, oa = 0, ldb = 0, sb = 0, ob = 0, ldo = 0, so = 0, oo = 0;
     int32_t m = 0, k = 0, n = 0, batch = 1, outer = 1;
     EpilogueSpec epi;
@@ -1561,7 +1561,8 @@ struct Planner {
     void plan_batch_matmul(int id, const View& av) {
         const GNode& n = N(id);
         const Value bval = value(n.in[1]);
-        if (bval.kind != VK_MAT || bval.view.dtype != HIPIE_I8) unsupported(id, "right operand must be quantized to i8");
+        if (bval.kind != VK_MAT || (bval.view.dtype != HIPIE_I8 && bval.view.dtype != HIPIE_U8B))
+            unsupported(id, "right operand must be quantized (i8 or u8)");
         View bv = bval.view;
         const size_t r = av.rank();
         if (r < 3 || r > 4 || bv.rank() != r) unsupported(id, "MatMul between activations needs equal ranks of 3 or 4");
@@ -1576,7 +1577,8 @@ struct Planner {
             if (av.shape[i] != bv.shape[i]) unsupported(id, "broadcast batch dimensions");
         if (av.stride[r - 1] != 1) unsupported(id, "left operand with a strided reduction axis");
         if (K % 64 != 0) unsupported(id, "reduction length must be a multiple of 64");
-        if (fuse_attention && M == Nn && av.dtype == HIPIE_I8 && try_plan_attention(id, av, bv)) return;   // (the scores' operands)
+        if (fuse_attention && M == Nn && av.dtype == HIPIE_I8 && bv.dtype == HIPIE_I8 && try_plan_attention(id, av, bv))
+            return;   // (the scores' operands)
         const int32_t inner = static_cast<int32_t>(av.shape[r - 3]), outer = r == 4 ? static_cast<int32_t>(av.shape[0]) : 1;
         if (bv.stride[r - 1] != 1) {
             // reduction axis not contiguous: transpose the operand's inner dimensions into a new tensor
@@ -1588,7 +1590,7 @@ struct Planner {
             tp->ld_src = bv.stride[r - 1];
             batch_strides(bv, tp->s_src, tp->o_src);
             std::vector<int64_t> tshape(bv.shape);
-            tp->out = new_matrix(n.in[1], HIPIE_I8, tshape);
+            tp->out = new_matrix(n.in[1], bv.dtype, tshape);
             const auto ds = View::dense_strides(tshape);
             tp->ld_dst = K;
             tp->s_dst = ds[r - 3];
@@ -1600,7 +1602,7 @@ struct Planner {
             tp->bytes = 2 * bv.numel();
             View nb;
             nb.tensor = tp->out;
-            nb.dtype = HIPIE_I8;
+            nb.dtype = bv.dtype;
             nb.shape = tshape;
             nb.stride = ds;
             bv = nb;
@@ -1623,8 +1625,13 @@ struct Planner {
         const int cur = absorb_matmul_tail(id, e, oshape, ostride);
         mark_chain(id, cur);
         st->out = new_matrix(cur, e.out_dtype, oshape);
-        if (av.dtype == HIPIE_U8B)   // level 0 stands for 0.0 here: a zero point would arrive as a Subtract, which is not taken
-            st->ws = new_tensor(id, HIPIE_I32, 1, 1, inner * outer, static_cast<int>(round_up(Nn, 128)));
+        // level 0 of a u8 operand stands for 0.0 here: a zero point would arrive as a Subtract, which is not taken (nor
+        // does MatMulTransformation rewrite such a MatMul, mat_mul.cpp:231-236, :290-292).  One row of sums per batch
+        // element for either u8 operand: over the right operand's rows (u8 left), over the left operand's (u8 right)
+        {
+            const int64_t per_batch = (av.dtype == HIPIE_U8B ? round_up(Nn, 128) : 0) + (bv.dtype == HIPIE_U8B ? round_up(M, 4) : 0);
+            if (per_batch > 0) st->ws = new_tensor(id, HIPIE_I32, 1, 1, inner * outer, static_cast<int>(per_batch));
+        }
         st->ldo = ostride[r - 2];
         st->so = ostride[r - 3];
         st->oo = r == 4 ? ostride[0] : 0;

@@ -210,21 +210,21 @@ class Convolution:
 
 
 class hipie_matmul_desc(ctypes.Structure):
-    _fields_ = [(k, ctypes.c_int32) for k in ("a_dtype", "b_dtype", "k", "n", "a_zero_point")]
+    _fields_ = [(k, ctypes.c_int32) for k in ("a_dtype", "b_dtype", "k", "n", "a_zero_point", "b_zero_point")]
 
 
 class BatchedMatMul:
-    """i8 (or u8) x i8 MatMul between two activation tensors: out[b] = A[b] @ Bt[b]^T (+ fused epilogue).
+    """i8 / u8 x i8 / u8 MatMul between two activation tensors: out[b] = A[b] @ Bt[b]^T (+ fused epilogue).
 
     ``a`` is a torch int8 tensor [batch, M, K] (u8 levels stored as level - 128 with ``a_dtype=U8B``), ``bt`` is
-    [batch, N, K] (the transpose_b = true form); the result is [batch, M, ldo] with ldo = N padded to the store
-    granularity.
+    [batch, N, K] (the transpose_b = true form, ``b_dtype`` likewise); the result is [batch, M, ldo] with ldo = N
+    padded to the store granularity.
     """
 
-    def __init__(self, k, n, epilogue=None, device=0, a_dtype=I8, a_zero_point=0):
+    def __init__(self, k, n, epilogue=None, device=0, a_dtype=I8, a_zero_point=0, b_dtype=I8, b_zero_point=0):
         self.k, self.n = k, n
         self.epilogue = epilogue or make_epilogue(out_dtype=I32)
-        d = hipie_matmul_desc(a_dtype, I8, k, n, a_zero_point)
+        d = hipie_matmul_desc(a_dtype, b_dtype, k, n, a_zero_point, b_zero_point)
         self._h = ctypes.c_void_p()
         check(lib().hipie_matmul_create(ctypes.c_int(device), ctypes.byref(d), ctypes.byref(self.epilogue),
                                         ctypes.byref(self._h)))
@@ -247,7 +247,8 @@ class BatchedMatMul:
         assert out.shape == (batch, m, ldo) and out.dtype == tdt and out.is_contiguous()
         i64 = ctypes.c_int64
         need = ctypes.c_size_t()
-        check(lib().hipie_matmul_workspace_size(self._h, ctypes.c_int32(batch), ctypes.c_int32(1), ctypes.byref(need)))
+        check(lib().hipie_matmul_workspace_size(self._h, ctypes.c_int32(m), ctypes.c_int32(batch), ctypes.c_int32(1),
+                                                ctypes.byref(need)))
         ws = torch.empty(max(need.value, 16), dtype=torch.int8, device=a.device)
         check(lib().hipie_matmul_run_nested_ws(self._h, _dptr(a), i64(k), i64(m * k), i64(0), _dptr(bt), i64(k),
                                                i64(self.n * k), i64(0), _dptr(out), i64(ldo), i64(m * ldo), i64(0),

@@ -287,9 +287,12 @@ int hipie_conv_run_static(const hipie_conv* conv, const hipie_tensor* in, const 
  *     1x1 convolution (hipie_conv_*).  Leading dimensions and batch strides are in elements.
  * ==================================================================================== */
 typedef struct hipie_matmul_desc {
-    int32_t a_dtype, b_dtype;   /* left: HIPIE_I8 or HIPIE_U8B (u8 levels, e.g. quantized Softmax output); right: HIPIE_I8 */
+    int32_t a_dtype, b_dtype;   /* each HIPIE_I8 or HIPIE_U8B (u8 levels, e.g. a quantized Softmax or ReLU output) */
     int32_t k, n;               /* reduction length (multiple of 64), output columns */
-    int32_t a_zero_point;       /* level of the u8 left operand that stands for 0.0 (0 for i8) */
+    int32_t a_zero_point;       /* level of a u8 left operand that stands for 0.0 (0 for i8) */
+    int32_t b_zero_point;       /* the same for the right operand.  (MatMulTransformation itself only rewrites a MatMul
+                                 * between activations whose operands have no zero point, mat_mul.cpp:231-236, :265-267,
+                                 * :290-292: 0 is what a transformed graph carries.) */
 } hipie_matmul_desc;
 
 typedef struct hipie_matmul hipie_matmul;
@@ -306,11 +309,13 @@ int hipie_matmul_run_nested(const hipie_matmul* matmul, const void* a, int64_t l
                             const void* b_transposed, int64_t ldb, int64_t stride_b, int64_t outer_b, void* out,
                             int64_t ldo, int64_t stride_o, int64_t outer_o, int32_t m, int32_t batch,
                             int32_t batch_outer, void* stream);
-/* A u8 left operand is stored as level - 128: sum_k (q_k - z) b_k = sum_k (q_k - 128) b_k + (128 - z) sum_k b_k, and
- * the sums over K of the right operand's rows (an activation here, not constant weights as in mat_mul.cpp:95-121) are
- * computed on the stream in front of the product, into a workspace of hipie_matmul_workspace_size bytes that the
- * caller owns (one per request in flight; 16-byte aligned; 0 bytes and not needed for an i8 left operand). */
-int hipie_matmul_workspace_size(const hipie_matmul* matmul, int32_t batch, int32_t batch_outer, size_t* bytes);
+/* A u8 operand is stored as level - 128.  With a', b' the stored bytes and za, zb the zero points,
+ *   sum_k (a_k - za)(b_k - zb) = sum_k a'_k b'_k + (128 - za) sum_k b'_k + (128 - zb) (sum_k a'_k + K (128 - za)):
+ * the sums over K of the right operand's rows (u8 left operand; an activation here, not constant weights as in
+ * mat_mul.cpp:95-121) and of the left operand's rows (u8 right operand) are computed on the stream in front of the
+ * product, into a workspace of hipie_matmul_workspace_size(m, batch, batch_outer) bytes that the caller owns (one
+ * per request in flight; 16-byte aligned; 0 bytes and not needed when both operands are i8). */
+int hipie_matmul_workspace_size(const hipie_matmul* matmul, int32_t m, int32_t batch, int32_t batch_outer, size_t* bytes);
 int hipie_matmul_run_nested_ws(const hipie_matmul* matmul, const void* a, int64_t lda, int64_t stride_a, int64_t outer_a,
                                const void* b_transposed, int64_t ldb, int64_t stride_b, int64_t outer_b, void* out,
                                int64_t ldo, int64_t stride_o, int64_t outer_o, int32_t m, int32_t batch,

@@ -258,17 +258,17 @@ def test_concat_shape_inference_and_planner_limits():
 
 def test_matmul_zero_point_correction_must_be_integers():
     """the Subtract behind a MatMul with u8 activations goes into the integer accumulators: a constant that is not
-    integer-valued (it is zero point x column sums of i8 weights) is refused, and so is a u8 operand of a MatMul
-    between two activations"""
+    integer-valued (it is zero point x column sums of i8 weights) is refused.  A MatMul between two u8 activations is
+    planned (level 0 standing for 0.0 on both sides) when its reduction length is a multiple of 64"""
     from dldt_amd import HipieError, builders
     from dldt_amd.graph import Graph
     from dldt_amd.tensor import I8, U8
     plan = builders.matmul_zero_point_net()[0].compile(-1)
     assert [s["type"] for s in plan.steps].count("MatMul") == 2
 
-    def net(corr, between_activations=False):
+    def net(corr, between_activations=False, hidden=32):
         g = Graph()
-        x = g.parameter("x", (2, 16, 32))
+        x = g.parameter("x", (2, 16, hidden))
         q = g.fake_quantize(x, -1.0, 2.0, 0.0, 255.0, 256, U8)
         if between_activations:
             y = g.matmul(q, q, False, True)
@@ -283,4 +283,6 @@ def test_matmul_zero_point_correction_must_be_integers():
     assert e.value.status == -2 and "integer" in str(e.value)
     with pytest.raises(HipieError) as e:
         net(0.0, between_activations=True).compile(-1)
-    assert e.value.status == -2 and "i8" in str(e.value)
+    assert e.value.status == -2 and "multiple of 64" in str(e.value)
+    plan = net(0.0, between_activations=True, hidden=64).compile(-1)
+    assert [s["type"] for s in plan.steps].count("MatMul") == 1

@@ -76,16 +76,17 @@ def test_quantized_group_convolution_equals_its_float_graph(orc, c, oc, kernel, 
     assert np.abs(ref).max() > 0.5
 
 
-@pytest.mark.parametrize("left", ["u8", "i8"])
-def test_quantized_matmul_between_activations_equals_its_float_graph(orc, left):
-    """FakeQuantize(A) x FakeQuantize(B), both graph inputs: A to u8 levels of [0, 1] (or i8 symmetric), B to i8
-    symmetric; after the transformation an integer MatMul and one Multiply by both scales"""
+@pytest.mark.parametrize("left,right", [("u8", "i8"), ("i8", "i8"), ("i8", "u8"), ("u8", "u8")])
+def test_quantized_matmul_between_activations_equals_its_float_graph(orc, left, right):
+    """FakeQuantize(A) x FakeQuantize(B), both graph inputs, each to u8 levels of [0, hi] or to i8 symmetric (no zero
+    point either way: MatMulTransformation rewrites no other MatMul between activations, mat_mul.cpp:231-236,
+    :265-267, :290-292); after the transformation an integer MatMul and one Multiply by both scales"""
     from dldt_amd import lpt
     from dldt_amd.graph import Graph
     from dldt_amd.tensor import I8, U8
-    rng = np.random.default_rng(11 + (left == "u8"))
+    rng = np.random.default_rng(11 + (left == "u8") + 2 * (right == "u8"))
     A = (rng.uniform(0, 1, (4, 64, 128)) if left == "u8" else rng.normal(0, 0.4, (4, 64, 128))).astype(np.float32)
-    B = rng.normal(0, 0.5, (4, 128, 64)).astype(np.float32)
+    B = (rng.uniform(0, 1.5, (4, 128, 64)) if right == "u8" else rng.normal(0, 0.5, (4, 128, 64))).astype(np.float32)
     g = Graph()
     pa, pb = g.parameter("a", A.shape), g.parameter("b", B.shape)
     if left == "u8":
@@ -94,11 +95,12 @@ def test_quantized_matmul_between_activations_equals_its_float_graph(orc, left):
         hi_a = np.float32(1.0)
         lo_a = np.float32(-hi_a * np.float32(128) / np.float32(127))
     hi_b = np.float32(1.5)
-    lo_b = np.float32(-hi_b * np.float32(128) / np.float32(127))
+    lo_b = np.float32(0) if right == "u8" else np.float32(-hi_b * np.float32(128) / np.float32(127))
     da, db = lpt.decompose_fake_quantize(256, lo_a, hi_a), lpt.decompose_fake_quantize(256, lo_b, hi_b)
-    assert da["precision"] == (U8 if left == "u8" else I8) and db["precision"] == I8
+    assert da["precision"] == (U8 if left == "u8" else I8) and db["precision"] == (U8 if right == "u8" else I8)
+    assert not da.get("has_zero_point", False) and not db.get("has_zero_point", False)
     qa = g.fake_quantize(pa, lo_a, hi_a, da["new_low"], da["new_high"], 256, da["precision"])
-    qb = g.fake_quantize(pb, lo_b, hi_b, db["new_low"], db["new_high"], 256, I8)
+    qb = g.fake_quantize(pb, lo_b, hi_b, db["new_low"], db["new_high"], 256, db["precision"])
     s = np.float32(da["scale"]) * np.float32(db["scale"])
     g.result(g.multiply(g.matmul(qa, qb), g.constant(np.float32(s).reshape(()))), "out")
     want_graph, _ = evaluate(orc, g.nodes, {"a": A, "b": B})

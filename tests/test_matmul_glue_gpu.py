@@ -47,6 +47,42 @@ def test_batched_matmul_u8_left_operand(orc, batch, m, k, n, zp):
     np.testing.assert_array_equal(got8.cpu().numpy(), lv)
 
 
+@pytest.mark.parametrize("batch,m,k,n,za,zb", [(4, 384, 64, 384, None, 0), (3, 100, 128, 200, None, 0), (2, 7, 64, 40, None, 9),
+                                               (3, 130, 192, 128, 0, 0), (2, 257, 64, 72, 31, 200), (1, 64, 128, 64, 255, 255)])
+def test_batched_matmul_u8_right_operand(orc, batch, m, k, n, za, zb):
+    """A u8 right operand (an activation quantized behind a ReLU), against an i8 (za None) or a u8 left operand: exact
+    i32 sums of (a - za)(b - zb).  Stored as level - 128, the right operand asks for one correction per output row
+    (the sums over K of the left operand's rows), added to the accumulators in front of the epilogue."""
+    import torch
+    from dldt_amd import BatchedMatMul, make_epilogue
+    rng = np.random.default_rng(m + n + zb)
+    if za is None:
+        a = rng.integers(-128, 128, (batch, m, k)).astype(np.int32)
+        a_stored, kw = a.astype(np.int8), {}
+        a_real = a
+    else:
+        a = rng.integers(0, 256, (batch, m, k)).astype(np.int32)
+        a_stored, kw = (a - 128).astype(np.int8), dict(a_dtype=U8B, a_zero_point=za)
+        a_real = a - za
+    bt = rng.integers(0, 256, (batch, n, k)).astype(np.int32)
+    want = orc.matmul(a_real, bt - zb, False, True)
+    ad = torch.from_numpy(a_stored).cuda()
+    bd = torch.from_numpy((bt - 128).astype(np.int8)).cuda()
+    mm = BatchedMatMul(k, n, b_dtype=U8B, b_zero_point=zb, **kw)
+    np.testing.assert_array_equal(mm.run(ad, bd).cpu().numpy(), want)
+    np.testing.assert_array_equal(mm.run(ad, bd).cpu().numpy(), want)
+    s = np.float32(1 / 255) * np.float32(0.02)
+    f = orc.multiply(want.astype(np.float32), s)
+    hi = np.float32(np.abs(f).max())
+    lo = np.float32(-hi * np.float32(128) / np.float32(127))
+    lv = orc.fake_quantize(f, lo, hi, np.float32(-128), np.float32(127), 256).astype(np.int8)
+    got8 = BatchedMatMul(k, n, make_epilogue(scale=[s], out_dtype=I8, fq=(256, lo, hi, -128.0, 127.0)), b_dtype=U8B,
+                         b_zero_point=zb, **kw).run(ad, bd)
+    np.testing.assert_array_equal(got8.cpu().numpy(), lv)
+    gotf = BatchedMatMul(k, n, make_epilogue(scale=[s], out_dtype=F32), b_dtype=U8B, b_zero_point=zb, **kw).run(ad, bd)
+    np.testing.assert_array_equal(gotf.cpu().numpy().view(np.uint32), f.view(np.uint32))
+
+
 def test_batched_matmul_u8_needs_its_workspace_and_a_level_as_zero_point():
     import ctypes
     import torch
@@ -56,6 +92,15 @@ def test_batched_matmul_u8_needs_its_workspace_and_a_level_as_zero_point():
         BatchedMatMul(64, 64, a_dtype=U8B, a_zero_point=256)
     with pytest.raises(HipieError):
         BatchedMatMul(64, 64, a_zero_point=3)                      # an i8 operand has none
+    with pytest.raises(HipieError):
+        BatchedMatMul(64, 64, b_dtype=U8B, b_zero_point=-1)
+    with pytest.raises(HipieError):
+        BatchedMatMul(64, 64, b_zero_point=3)
+    a = torch.zeros((1, 64, 64), dtype=torch.int8, device="cuda")
+    out = torch.zeros((1, 64, 64), dtype=torch.int32, device="cuda")
+    with pytest.raises(HipieError) as e:
+        matmul_strided(BatchedMatMul(64, 64, b_dtype=U8B), a.data_ptr(), 64, 0, a.data_ptr(), 64, 0, out.data_ptr(), 64, 0, 64, 1)
+    assert "workspace" in str(e.value)
     mm = BatchedMatMul(64, 64, a_dtype=U8B)
     a = torch.zeros((1, 64, 64), dtype=torch.int8, device="cuda")
     out = torch.zeros((1, 64, 64), dtype=torch.int32, device="cuda")
