@@ -22,8 +22,11 @@ constexpr int kRow = 64;  // LDS rows of the tiled kernels: 64 K-bytes, chunk c 
 // compute unit the lines of one step, 128 KB, do not survive in the 32 KB L1 until the next step asks
 // for their other half: the operand loads alone run 1.4 times faster this way).  The two LDS buffers
 // then hold the two steps of a pair instead of alternating.
-template <int WOC, int WPIX, uint32_t F, bool PAIR = false>
-__global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && (F & CF_RES_GEMM))) ? ((F == kDyn || PAIR) ? 3 : 4) : 2) void conv_tiled_kernel(const ConvArgs a) {
+// PIXC: one integer per output row (ConvArgs::pix_corr) is added to the row's accumulators in front of the epilogue
+// (MatMul between activations with a u8 right operand).  A template constant: as a run-time branch its registers
+// pushed the 128-register instances of every convolution into spills.
+template <int WOC, int WPIX, uint32_t F, bool PAIR = false, bool PIXC = false>
+__global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && (F & CF_RES_GEMM))) ? ((F == kDyn || PAIR || PIXC) ? 3 : 4) : 2) void conv_tiled_kernel(const ConvArgs a) {
     constexpr int NT = WOC * WPIX * 64;
     constexpr int BOC = WOC * 64, BPIX = WPIX * 64;
     constexpr int A_PIECES = BOC * 4 / NT, B_PIECES = BPIX * 4 / NT;
@@ -243,7 +246,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     gemm(a.in + batch_offset(a, batch, a.batch_in, a.batch_in_o), a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
          a.wgt + batch_offset(a, batch, a.batch_wgt, a.batch_wgt_o), a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused, a.flat_in != 0);
     const int m0 = pix0 + wpix * 64 + l32;
-    if (a.pix_corr) {   // uniform: MatMul between activations whose right operand is stored as level - 128
+    if constexpr (PIXC) {   // MatMul between activations whose right operand is stored as level - 128
         const int32_t* pc = a.pix_corr + static_cast<int64_t>(batch) * a.batch_pix_corr;
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb) {
@@ -1015,6 +1018,18 @@ void launch_tiled(const ConvArgs& a, hipStream_t s, int batches = 1) {
 #undef HIPIE_LAUNCH_TILED
 }
 
+// the same tiles with one accumulator correction per output row (ConvArgs::pix_corr): the epilogues a MatMul between
+// activations ends in as template constants, any other through the instance that reads its flags at run time
+template <int WOC, int WPIX>
+void launch_tiled_pixc(const ConvArgs& a, hipStream_t s, int batches) {
+    const dim3 grid(a.p_tiles * a.t_tiles, batches), block(WOC * WPIX * 64);
+    switch (a.flags & ~CF_OUT_XOR) {
+    case E_SCALE: hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, E_SCALE, false, true>), grid, block, 0, s, a); break;
+    case E_DEQFQ: hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, E_DEQFQ, false, true>), grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL((conv_tiled_kernel<WOC, WPIX, kDyn, false, true>), grid, block, 0, s, a); break;
+    }
+}
+
 template <int WOC, int WPIX, int KS>
 void launch_pipe(const ConvArgs& a, int stages, hipStream_t s, int batches = 1) {
     const dim3 grid(a.p_per_xcd > 0 ? 8 * a.p_per_xcd * a.t_tiles : a.p_tiles * a.t_tiles, batches, a.ksplit > 1 ? a.ksplit : 1),
@@ -1658,8 +1673,14 @@ int hipie_matmul_run_nested_ws(const hipie_matmul* mm, const void* a_ptr, int64_
         a.t_tiles = static_cast<int32_t>(ceil_div(d.n, boc));
         a.t_shift = (a.t_tiles & (a.t_tiles - 1)) == 0 ? __builtin_ctz(a.t_tiles) : -1;
         a.p_per_xcd = 0;   // plain order: batches are spread over the XCDs by their launch order
-        if (wide) launch_tiled<2, 2>(a, as_stream(stream), batch * batch_outer);
-        else launch_tiled<1, 4>(a, as_stream(stream), batch * batch_outer);
+        if (a.pix_corr) {
+            if (wide) launch_tiled_pixc<2, 2>(a, as_stream(stream), batch * batch_outer);
+            else launch_tiled_pixc<1, 4>(a, as_stream(stream), batch * batch_outer);
+        } else if (wide) {
+            launch_tiled<2, 2>(a, as_stream(stream), batch * batch_outer);
+        } else {
+            launch_tiled<1, 4>(a, as_stream(stream), batch * batch_outer);
+        }
         HIPIE_CHECK_HIP(hipGetLastError());
     });
 }
