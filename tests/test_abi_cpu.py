@@ -286,3 +286,32 @@ def test_matmul_zero_point_correction_must_be_integers():
     assert e.value.status == -2 and "multiple of 64" in str(e.value)
     plan = net(0.0, between_activations=True, hidden=64).compile(-1)
     assert [s["type"] for s in plan.steps].count("MatMul") == 1
+
+
+def test_matmul_between_activations_descriptor_and_workspace():
+    """hipie_matmul_create on the host (device -1): operand types, zero points as levels of a u8 operand only, and the
+    workspace a u8 operand asks for - one i32 per padded output column (u8 left operand: sums over the right operand's
+    rows) plus one per output row rounded up to four (u8 right operand: sums over the left operand's rows), per batch
+    element"""
+    import ctypes
+    from dldt_amd import HipieError, lib
+    from dldt_amd.ops import BatchedMatMul
+    from dldt_amd.tensor import I8, U8B, F32
+
+    def size(mm, m, batch, outer):
+        need = ctypes.c_size_t(12345)
+        st = lib().hipie_matmul_workspace_size(mm._h, ctypes.c_int32(m), ctypes.c_int32(batch), ctypes.c_int32(outer),
+                                               ctypes.byref(need))
+        assert st == 0
+        return need.value
+
+    assert size(BatchedMatMul(64, 200, device=-1), 100, 3, 2) == 0
+    assert size(BatchedMatMul(64, 200, device=-1, a_dtype=U8B, a_zero_point=7), 100, 3, 2) == 6 * 256 * 4
+    assert size(BatchedMatMul(64, 200, device=-1, b_dtype=U8B), 101, 3, 2) == 6 * 104 * 4
+    assert size(BatchedMatMul(128, 64, device=-1, a_dtype=U8B, b_dtype=U8B, b_zero_point=255), 7, 5, 1) == 5 * (128 + 8) * 4
+    for bad in (dict(a_dtype=F32), dict(b_dtype=F32), dict(a_zero_point=1), dict(b_zero_point=1),
+                dict(a_dtype=U8B, a_zero_point=-1), dict(b_dtype=U8B, b_zero_point=256)):
+        with pytest.raises(HipieError):
+            BatchedMatMul(64, 64, device=-1, **bad)
+    with pytest.raises(HipieError):
+        BatchedMatMul(96, 64, device=-1)            # the reduction length is a multiple of 64
