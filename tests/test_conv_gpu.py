@@ -33,6 +33,17 @@ def _inputs(rng, g, signed=False):
     return x, w
 
 
+def _k_steps(g):
+    """64-byte steps of the K loop for geometry g: K runs over (kh, kw, padded channels), a 4-byte pixel (up to four
+    channels) has every filter row padded to 16 bytes instead"""
+    C, KH, KW = g[1], g[5], g[6]
+    if C <= 4:
+        k = KH * (-(-KW * 4 // 16) * 16)
+    else:
+        k = KH * KW * (-(-C // 16) * 16)
+    return -(-k // 64)
+
+
 def _device_in(x, g, signed=False):
     from dldt_amd import DeviceTensor
     pb, pe = g[9], g[10]
@@ -54,9 +65,10 @@ def test_conv_i32_accumulators_exact(orc, name, tile):
     conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10])
     try:
         conv.set_tile(tile)
-    except HipieError as e:       # the split-K variants need an even number of K steps
-        assert 6 <= tile <= 7 and e.status == -4
-        pytest.skip(str(e))
+    except HipieError as e:       # the variants that split K over two wave groups need an even number of K steps
+        assert 6 <= tile <= 7 and e.status == -4 and _k_steps(g) % 2 == 1
+        return                    # refused exactly where it should be: nothing to run
+    assert not (6 <= tile <= 7 and _k_steps(g) % 2 == 1)
     out = DeviceTensor(want.shape[0], want.shape[2], want.shape[3], want.shape[1], I32)
     conv.run(xin, out)
     torch.cuda.synchronize()
@@ -643,9 +655,10 @@ def test_conv_pipelined_ring_depths(orc, name, tile, stages):
     conv = Convolution(w.astype(np.int8), xin, g[7], g[8], g[9], g[10])
     try:
         conv.set_tile(tile, stages)
-    except HipieError as e:       # the split-K variants need an even number of K steps
-        assert 6 <= tile <= 7 and e.status == -4
-        pytest.skip(str(e))
+    except HipieError as e:       # the variants that split K over two wave groups need an even number of K steps
+        assert 6 <= tile <= 7 and e.status == -4 and _k_steps(g) % 2 == 1
+        return                    # refused exactly where it should be: nothing to run
+    assert not (6 <= tile <= 7 and _k_steps(g) % 2 == 1)
     out = DeviceTensor(want.shape[0], want.shape[2], want.shape[3], want.shape[1], I32)
     conv.run(xin, out)
     torch.cuda.synchronize()
@@ -745,8 +758,9 @@ def test_conv_k_split_over_workgroups(orc, name, epi, tile):
     try:
         conv.set_tile(tile)
     except HipieError as err:      # fewer than two K steps per part
-        assert err.status == -4 and (C * g[5] * g[6] + 63) // 64 < 2 * (2 << (tile - 14))
-        pytest.skip(str(err))
+        assert err.status == -4 and _k_steps(g) < 2 * (2 << (tile - 14))
+        return                     # refused exactly where it should be: nothing to run
+    assert _k_steps(g) >= 2 * (2 << (tile - 14))
     out = DeviceTensor(acc.shape[0], acc.shape[2], acc.shape[3], OC, dt)
     for rep in range(3):
         if rep:
