@@ -76,8 +76,9 @@ def test_quantized_group_convolution_equals_its_float_graph(orc, c, oc, kernel, 
     assert np.abs(ref).max() > 0.5
 
 
+@pytest.mark.parametrize("lead", [(4,), (2, 3)])
 @pytest.mark.parametrize("left,right", [("u8", "i8"), ("i8", "i8"), ("i8", "u8"), ("u8", "u8")])
-def test_quantized_matmul_between_activations_equals_its_float_graph(orc, left, right):
+def test_quantized_matmul_between_activations_equals_its_float_graph(orc, left, right, lead):
     """FakeQuantize(A) x FakeQuantize(B), both graph inputs, each to u8 levels of [0, hi] or to i8 symmetric (no zero
     point either way: MatMulTransformation rewrites no other MatMul between activations, mat_mul.cpp:231-236,
     :265-267, :290-292); after the transformation an integer MatMul and one Multiply by both scales"""
@@ -85,8 +86,12 @@ def test_quantized_matmul_between_activations_equals_its_float_graph(orc, left, 
     from dldt_amd.graph import Graph
     from dldt_amd.tensor import I8, U8
     rng = np.random.default_rng(11 + (left == "u8") + 2 * (right == "u8"))
-    A = (rng.uniform(0, 1, (4, 64, 128)) if left == "u8" else rng.normal(0, 0.4, (4, 64, 128))).astype(np.float32)
-    B = (rng.uniform(0, 1.5, (4, 128, 64)) if right == "u8" else rng.normal(0, 0.5, (4, 128, 64))).astype(np.float32)
+    # (one or two batch dimensions; the graph inputs are rank 3 either way, the second form reshapes the quantized
+    # tensors to rank 4 and walks the operands by an inner and an outer stride)
+    nb = int(np.prod(lead))
+    sa, sb = (nb, 64, 128), (nb, 128, 64)
+    A = (rng.uniform(0, 1, sa) if left == "u8" else rng.normal(0, 0.4, sa)).astype(np.float32)
+    B = (rng.uniform(0, 1.5, sb) if right == "u8" else rng.normal(0, 0.5, sb)).astype(np.float32)
     g = Graph()
     pa, pb = g.parameter("a", A.shape), g.parameter("b", B.shape)
     if left == "u8":
@@ -102,6 +107,8 @@ def test_quantized_matmul_between_activations_equals_its_float_graph(orc, left, 
     qa = g.fake_quantize(pa, lo_a, hi_a, da["new_low"], da["new_high"], 256, da["precision"])
     qb = g.fake_quantize(pb, lo_b, hi_b, db["new_low"], db["new_high"], 256, db["precision"])
     s = np.float32(da["scale"]) * np.float32(db["scale"])
+    if len(lead) == 2:
+        qa, qb = g.reshape(qa, lead + (64, 128)), g.reshape(qb, lead + (128, 64))
     g.result(g.multiply(g.matmul(qa, qb), g.constant(np.float32(s).reshape(()))), "out")
     want_graph, _ = evaluate(orc, g.nodes, {"a": A, "b": B})
     req = g.compile().create_request()
@@ -109,7 +116,7 @@ def test_quantized_matmul_between_activations_equals_its_float_graph(orc, left, 
     np.testing.assert_array_equal(got.view(np.uint32), want_graph["out"].view(np.uint32))
     a_fq = orc.fake_quantize(A, lo_a, hi_a, lo_a, hi_a, 256).astype(np.float64)
     b_fq = orc.fake_quantize(B, lo_b, hi_b, lo_b, hi_b, 256).astype(np.float64)
-    ref = a_fq @ b_fq
+    ref = (a_fq @ b_fq).reshape(got.shape)
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=2e-5 * np.abs(ref).max())
     assert np.abs(ref).max() > 1.0
 
