@@ -25,6 +25,11 @@ struct Epilogue {
 void launch_line(const ConvArgs& a, int shape, hipStream_t s);
 int line_row_bytes(int shape);
 
+// few pixels, many channels (conv_skinny.hip): 1 x 1 over a dense input, weights packed K-major ([Kp / 16][OCp] pieces of
+// 16 K bytes, passed as ConvArgs::wgt2), epilogues as skinny_epilogue_fits says
+bool skinny_epilogue_fits(uint32_t flags);
+void launch_skinny(const ConvArgs& a, hipStream_t s);
+
 // depthwise kernels (dwconv.hip).  variant 0: a lane computes its outputs from registers loaded straight from memory;
 // variant 1: 3 x 3 through an LDS patch with the window sliding in registers (dwconv_strip_fits says which layers)
 struct DwGeometry {

@@ -1398,6 +1398,7 @@ struct hipie_conv {
     int stages = 0;  // ring depth of the pipelined kernels (0 = choose from K)
     DeviceBuffer wgt, koff, corr;
     DeviceBuffer wgt_rows;   // depthwise 3 x 3: [kh][OCp] dwords, bytes (w[kh][0], w[kh][1], w[kh][2], 0) of a channel
+    DeviceBuffer wgt_k16;    // 1 x 1 with an epilogue the few-pixel kernel evaluates: [Kp / 16][OCp] pieces of 16 K bytes
     Epilogue epi;
 };
 
@@ -1773,6 +1774,16 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
         c->K = g.K; c->Kp = g.Kp; c->OCp = g.OCp;
         c->wgt = std::move(g.wgt); c->koff = std::move(g.koff); c->corr = std::move(g.corr);
         c->epi.build(device, *epilogue, d.oc, c->OCp);
+        if (device >= 0 && d.kh == 1 && d.kw == 1 && d.in_c_stride % 64 == 0 && c->Kp == d.in_c_stride && !d.acc_sub &&
+            skinny_epilogue_fits(c->epi.flags) && c->Kp * c->OCp <= (16 << 20) && c->Kp <= 7168) {   // (8 pixels x Kp bytes of LDS)
+            // the few-pixel kernel's packing (variant 23): piece k16 of channel oc at (k16 * OCp + oc) * 16
+            std::vector<int8_t> k16(static_cast<size_t>(c->Kp) * c->OCp, 0);
+            parallel_for(d.oc, [&](int64_t oc) {
+                for (int64_t k = 0; k < d.ic; ++k)
+                    k16[static_cast<size_t>(((k >> 4) * c->OCp + oc) * 16 + (k & 15))] = weights[oc * d.ic + k];
+            });
+            c->wgt_k16.upload(device, k16.data(), k16.size());
+        }
         // default: wide channel tiles when there are enough channels, else all waves on pixels
         // (the planner may override this after timing the candidates)
         c->tile = d.oc > 64 ? 0 : 1;
@@ -1825,7 +1836,7 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 22, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 23, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
         if (c->depthwise) {   // 0: registers only, 1: 3 x 3 through an LDS patch
             HIPIE_REQUIRE(tile == 0 || (tile == 1 && !(c->epi.flags & CF_RES) &&
                                         dwconv_strip_fits(c->d.kh, c->d.kw, c->d.dil_h, c->d.dil_w, c->d.stride_h, c->d.stride_w,
@@ -1839,7 +1850,7 @@ int hipie_conv_set_tile(hipie_conv* c, int tile) {
                       "hipie_conv_set_tile: the persistent kernels exist for byte outputs with a byte residual or none");
         HIPIE_REQUIRE(tile < 6 || tile > 7 || (c->Kp / 64) % 2 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the split-K kernels need an even number of 64-byte K steps (K=%lld)", (long long)c->Kp);
-        HIPIE_REQUIRE(tile < 18 || line_kernel_fits(c->d, c->Kp, c->OCp, line_row_bytes(tile - 18)), HIPIE_PARAMETER_MISMATCH,
+        HIPIE_REQUIRE(tile < 18 || tile > 22 || line_kernel_fits(c->d, c->Kp, c->OCp, line_row_bytes(tile - 18)), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the cache-line kernels need a channel stride (%d) and K (%lld) that are multiples of their %d-byte K step",
                       c->d.in_c_stride, (long long)c->Kp, line_row_bytes(tile - 18));
         HIPIE_REQUIRE(tile < 14 || tile > 17 || c->Kp / 64 >= 2 * split_parts(tile), HIPIE_PARAMETER_MISMATCH,
@@ -1848,6 +1859,11 @@ int hipie_conv_set_tile(hipie_conv* c, int tile) {
                       "hipie_conv_set_tile: the first-layer kernel takes 4-byte pixels and filter rows of 5 to 8 taps, undilated");
         HIPIE_REQUIRE(tile != 12 || rows_kernel_fits(c->d), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the row-tile kernel takes 3 x 3, stride 1, pad 1, undilated convolutions over a multiple of 64 input channels");
+        HIPIE_REQUIRE(tile != 23 || (c->wgt_k16.ptr && c->d.stride_h == 1 && c->d.stride_w == 1 && c->d.pad_top == 0 &&
+                                     c->d.pad_left == 0 && c->d.pad_bottom == 0 && c->d.pad_right == 0),
+                      HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_set_tile: the few-pixel kernel takes unpadded 1 x 1 convolutions over pixels of a multiple of 64 "
+                      "bytes with raw sums or a bias / scale / ReLU tail to f32");
         HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) + PT_ROWS * 64 * 4 <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: K=%lld does not fit the streaming kernel's LDS", (long long)c->Kp);
         c->tile = tile;
@@ -2108,6 +2124,10 @@ static int conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_ten
             }
         }
         switch (tile) {
+        case 23:
+            a.wgt2 = c->wgt_k16.as<int8_t>();
+            launch_skinny(a, s);
+            break;
         case 18: case 19: case 20: case 21: case 22: launch_line(a, tile - 18, s); break;
         case 14:
         case 15:

@@ -250,7 +250,10 @@ int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* o
  * split over 2 / 4 / 8 / 16 workgroups (for launches with fewer tiles than compute units; at least two K steps per
  * part; launches of more than 2048 workgroups run variant 4).  The partial sums of variants 14 to 17 pass through a
  * workspace that the library keeps per (device, stream): it is allocated by the first such launch on a stream
- * (which therefore must not be under graph capture) and kept until the process ends.  A default is chosen
+ * (which therefore must not be under graph capture) and kept until the process ends.  18 to 22 = 128 x 128 tiles
+ * whose K step is a whole cache line of every operand row, 23 = the few-pixel kernel (unpadded 1 x 1 over pixels of
+ * a multiple of 64 bytes, raw sums or a bias / scale / ReLU tail to f32: a lane per output channel on the vector
+ * pipe, K split over the waves of a workgroup; the FC layer of a classifier).  A default is chosen
  * from the shape; hipie_compile times the variants on the device and keeps the fastest.  Every
  * variant produces the same bits.
  * A depthwise convolution (group_convolution.hpp:78-144 with one filter per channel) has two variants of its own:

@@ -143,6 +143,47 @@ def test_fc_matmul_constant_weights(orc):
     np.testing.assert_array_equal(out.to_nchw()[:, :, 0, 0], want)
 
 
+@pytest.mark.parametrize("rows,k,n", [(64, 2048, 1000), (5, 2048, 1000), (70, 1280, 1000), (9, 64, 72), (3, 4096, 136), (1, 192, 64)])
+def test_few_pixel_kernel_on_fc_layers(orc, rows, k, n):
+    """the variant for 1 x 1 layers with few pixels and many channels (a lane per output channel, K split over the
+    four waves of a workgroup, weights packed K-major): raw i32 sums and the bias / scale [/ ReLU] tail to f32 bit for
+    bit, pixel counts that are not a multiple of 8, channel counts that are not a multiple of 64, K of one piece per wave
+    and of two rounds"""
+    from dldt_amd import Convolution, DeviceTensor, HipieError, make_epilogue
+    rng = np.random.default_rng(rows * 7 + n)
+    x = rng.integers(0, 256, (rows, k, 1, 1)).astype(np.int32)
+    w = rng.integers(-127, 128, (n, k, 1, 1)).astype(np.int32)
+    acc = orc.matmul(x[:, :, 0, 0], w[:, :, 0, 0], False, True)
+    xin = DeviceTensor.from_nchw(x, U8B)
+    conv = Convolution(w.astype(np.int8), xin)
+    conv.set_tile(23)
+    assert conv.get_tile() == 23
+    out = DeviceTensor(rows, 1, 1, n, I32)
+    conv.run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw()[:, :, 0, 0], acc)
+    bias = rng.normal(0, 500, n).astype(np.float32)
+    scale = rng.uniform(1e-4, 3e-4, n).astype(np.float32)
+    for relu in (False, True):
+        want = orc.multiply(orc.add(acc.astype(np.float32), bias), scale)
+        if relu:
+            want = orc.relu(want)
+        conv = Convolution(w.astype(np.int8), xin, epilogue=make_epilogue(bias=bias, scale=scale, activation="relu" if relu else None,
+                                                                         out_dtype=F32))
+        outs = {}
+        for tile in (0, 23):
+            conv.set_tile(tile)
+            o = DeviceTensor(rows, 1, 1, n, F32)
+            conv.run(xin, o)
+            outs[tile] = o.to_nchw()[:, :, 0, 0]
+        np.testing.assert_array_equal(outs[23].view(np.uint32), want.view(np.uint32))
+        np.testing.assert_array_equal(outs[0].view(np.uint32), want.view(np.uint32))
+    # a requantizing tail is not this kernel's: refused, the layer keeps its variant
+    fq = (256, 0.0, np.float32(4.0), 0.0, 255.0)
+    conv = Convolution(w.astype(np.int8), xin, epilogue=make_epilogue(bias=bias, scale=scale, out_dtype=U8B, fq=fq))
+    with pytest.raises(HipieError):
+        conv.set_tile(23)
+
+
 def test_softmax_mvn_gelu_tolerance(orc):
     import torch
     from dldt_amd import gelu, mvn, softmax
