@@ -1399,6 +1399,7 @@ struct hipie_conv {
     DeviceBuffer wgt, koff, corr;
     DeviceBuffer wgt_rows;   // depthwise 3 x 3: [kh][OCp] dwords, bytes (w[kh][0], w[kh][1], w[kh][2], 0) of a channel
     DeviceBuffer wgt_k16;    // 1 x 1 with an epilogue the few-pixel kernel evaluates: [Kp / 16][OCp] pieces of 16 K bytes
+    bool few_pixel_ok = false;   // the layer is one the few-pixel kernel takes (also known for a host-only object)
     Epilogue epi;
 };
 
@@ -1774,8 +1775,11 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
         c->K = g.K; c->Kp = g.Kp; c->OCp = g.OCp;
         c->wgt = std::move(g.wgt); c->koff = std::move(g.koff); c->corr = std::move(g.corr);
         c->epi.build(device, *epilogue, d.oc, c->OCp);
-        if (device >= 0 && d.kh == 1 && d.kw == 1 && d.in_c_stride % 64 == 0 && c->Kp == d.in_c_stride && !d.acc_sub &&
-            skinny_epilogue_fits(c->epi.flags) && c->Kp * c->OCp <= (16 << 20) && c->Kp <= 7168) {   // (8 pixels x Kp bytes of LDS)
+        c->few_pixel_ok = d.kh == 1 && d.kw == 1 && d.in_c_stride % 64 == 0 && c->Kp == d.in_c_stride && !d.acc_sub &&
+                          d.stride_h == 1 && d.stride_w == 1 && d.pad_top == 0 && d.pad_left == 0 && d.pad_bottom == 0 &&
+                          d.pad_right == 0 && skinny_epilogue_fits(c->epi.flags) && c->Kp * c->OCp <= (16 << 20) &&
+                          c->Kp <= 7168;   // (8 pixels x Kp bytes of LDS)
+        if (device >= 0 && c->few_pixel_ok) {
             // the few-pixel kernel's packing (variant 23): piece k16 of channel oc at (k16 * OCp + oc) * 16
             std::vector<int8_t> k16(static_cast<size_t>(c->Kp) * c->OCp, 0);
             parallel_for(d.oc, [&](int64_t oc) {
@@ -1859,9 +1863,7 @@ int hipie_conv_set_tile(hipie_conv* c, int tile) {
                       "hipie_conv_set_tile: the first-layer kernel takes 4-byte pixels and filter rows of 5 to 8 taps, undilated");
         HIPIE_REQUIRE(tile != 12 || rows_kernel_fits(c->d), HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the row-tile kernel takes 3 x 3, stride 1, pad 1, undilated convolutions over a multiple of 64 input channels");
-        HIPIE_REQUIRE(tile != 23 || (c->wgt_k16.ptr && c->d.stride_h == 1 && c->d.stride_w == 1 && c->d.pad_top == 0 &&
-                                     c->d.pad_left == 0 && c->d.pad_bottom == 0 && c->d.pad_right == 0),
-                      HIPIE_PARAMETER_MISMATCH,
+        HIPIE_REQUIRE(tile != 23 || c->few_pixel_ok, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the few-pixel kernel takes unpadded 1 x 1 convolutions over pixels of a multiple of 64 "
                       "bytes with raw sums or a bias / scale / ReLU tail to f32");
         HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) + PT_ROWS * 64 * 4 <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,

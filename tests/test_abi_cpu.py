@@ -82,12 +82,15 @@ def test_conv_variant_numbers_are_checked_without_a_device():
         long_k.set_tile(tile)
     short_k = _host_conv(64, 64, 1)            # one K step of 64 bytes: no 128-byte K steps either
     short_k.set_tile(22)
-    for tile in (23, -1, 12, 13, 14, 17, 18, 21):
+    short_k.set_tile(23)                       # an unpadded 1 x 1 with raw sums: the few-pixel kernel takes it
+    for tile in (24, -1, 12, 13, 14, 17, 18, 21):
         with pytest.raises(HipieError) as e:
             short_k.set_tile(tile)
         assert e.value.status == -4, tile      # PARAMETER_MISMATCH
     with pytest.raises(HipieError):
         long_k.set_tile(13)                    # not a 4-byte-pixel first layer
+    with pytest.raises(HipieError):
+        long_k.set_tile(23)                    # not a 1 x 1
 
 
 def test_epilogue_rejects_an_inverted_clamp_range():
