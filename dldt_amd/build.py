@@ -20,7 +20,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes", "-Wno-pass-failed",
     "-I", os.path.join(os.path.dirname(HERE), "include"),
-]
+] + os.environ.get("HIPIE_EXTRA_FLAGS", "").split()
 
 
 def _compile(src, force):

@@ -30,6 +30,19 @@ int line_row_bytes(int shape);
 bool skinny_epilogue_fits(uint32_t flags);
 void launch_skinny(const ConvArgs& a, hipStream_t s);
 
+// bottleneck-tail kernel (conv_block.hip): a 3 x 3 stride-1 pad-1 convolution over all of its 64, 128 or 256 output
+// channels per workgroup, input patch staged once in LDS; alone (b == nullptr) or with the 1 x 1 convolution behind it
+// run from the tile in LDS.  block_geometry: the tiling for an output of oh x ow pixels (ok = false: the kernel does
+// not take the layer); block_epilogues_fit: the epilogues the kernel is instantiated for
+struct BlockGeometry {
+    bool ok;
+    int nwc, rows, tiles_per_image, patch_w, csa, ppix;
+    size_t lds;
+};
+BlockGeometry block_geometry(int oc_a, int ic_a, int oh, int ow);
+bool block_epilogues_fit(uint32_t flags_a, bool fused, uint32_t flags_b);
+void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo, int images, hipStream_t s);
+
 // depthwise kernels (dwconv.hip).  variant 0: a lane computes its outputs from registers loaded straight from memory;
 // variant 1: 3 x 3 through an LDS patch with the window sliding in registers (dwconv_strip_fits says which layers)
 struct DwGeometry {

@@ -1144,6 +1144,21 @@ int rows_per_tile(int oh, int ow) {
     return r >= 1 ? r : 0;
 }
 
+// the bottleneck-tail kernel's first convolution: 3 x 3, stride 1, pad 1 over dense pixels of a multiple of 64 channels,
+// 64, 128 or 256 output channels, 32-bit buffer offsets
+bool block_first_fits(const hipie_conv_desc& d, int64_t Kp, int64_t OCp) {
+    return rows_kernel_fits(d) && d.in_c_stride == d.ic && d.in_stride_w == d.ic && Kp == 9 * static_cast<int64_t>(d.ic) &&
+           (d.oc == 64 || d.oc == 128 || d.oc == 256) && OCp * Kp < (int64_t(1) << 31);
+}
+
+// its second convolution: 1 x 1, stride 1, unpadded, over dense pixels of exactly 64, 128 or 256 channels, output
+// channels a multiple of that
+bool block_second_fits(const hipie_conv_desc& d, int64_t Kp, int64_t OCp) {
+    return d.groups == 1 && d.kh == 1 && d.kw == 1 && d.stride_h == 1 && d.stride_w == 1 && d.pad_top == 0 && d.pad_bottom == 0 &&
+           d.pad_left == 0 && d.pad_right == 0 && (d.ic == 64 || d.ic == 128 || d.ic == 256) && d.in_c_stride == d.ic &&
+           d.in_stride_w == d.ic && Kp == d.ic && d.oc % d.ic == 0 && OCp * Kp < (int64_t(1) << 31);
+}
+
 // the cache-line kernels: a K step of `rb` bytes must stay inside one filter tap, and 32-bit buffer offsets
 bool line_kernel_fits(const hipie_conv_desc& d, int64_t Kp, int64_t OCp, int rb) {
     return d.groups == 1 && d.in_c_stride % rb == 0 && Kp % rb == 0 && OCp * Kp < (int64_t(1) << 31);
@@ -1380,7 +1395,8 @@ static int64_t packed_row(int64_t oc) {
 struct PackedGemm {
     int64_t K = 0, Kp = 0, OCp = 0;
     DeviceBuffer wgt, koff, corr;
-    void pack(int device, const hipie_conv_desc& d, const int8_t* weights);
+    // `keep`: receives the packed matrix ([OCp][Kp], rows in MFMA order) for a second packing derived from it
+    void pack(int device, const hipie_conv_desc& d, const int8_t* weights, std::vector<int8_t>* keep = nullptr);
 };
 
 struct hipie_conv {
@@ -1399,6 +1415,8 @@ struct hipie_conv {
     DeviceBuffer wgt, koff, corr;
     DeviceBuffer wgt_rows;   // depthwise 3 x 3: [kh][OCp] dwords, bytes (w[kh][0], w[kh][1], w[kh][2], 0) of a channel
     DeviceBuffer wgt_k16;    // 1 x 1 with an epilogue the few-pixel kernel evaluates: [Kp / 16][OCp] pieces of 16 K bytes
+    DeviceBuffer wgt_steps;  // the bottleneck-tail kernel's packing (pack_fragments), where the layer can be one of its two
+    int steps_role = 0;      // 1: its 3 x 3 layer, 2: its 1 x 1 layer, 0: neither
     bool few_pixel_ok = false;   // the layer is one the few-pixel kernel takes (also known for a host-only object)
     Epilogue epi;
 };
@@ -1449,7 +1467,7 @@ struct hipie_matmul {
 // the zero point of input channel ic
 static inline int zero_point_of(const hipie_conv_desc& d, int ic) { return d.in_zero_points ? d.in_zero_points[ic] : d.in_zero_point; }
 
-void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weights) {
+void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weights, std::vector<int8_t>* keep) {
     // K order (kh, kw, ic) over the padded channel stride.  A 16-byte piece must not straddle
     // two filter taps unless consecutive taps are contiguous in memory (in_stride_w == c stride).
     const bool row_contig = d.in_stride_w == d.in_c_stride && d.dil_w == 1;
@@ -1495,6 +1513,40 @@ void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weight
         koff.upload(device, off.data(), off.size() * sizeof(int32_t));
         corr.upload(device, cr.data(), cr.size() * sizeof(int32_t));
     }
+    if (keep) *keep = std::move(w);
+}
+
+// The bottleneck-tail kernel's weight stream: the matrix in the order the kernel's waves use it, so that a wave's load
+// instruction is 1 KB of contiguous memory that lands in matrix operand registers as it is.  A step is 64 K bytes of `cm`
+// rows; inside a step come the row blocks of 64 (one per wave), inside a block the four fragments (ks, ob) - K bytes
+// [32 ks, 32 ks + 32) of rows [32 ob, 32 ob + 32) - and inside a fragment lane l's 16 bytes: row l % 32, K bytes
+// 16 (l / 32) onwards.  `first`: steps ordered (64-channel slab, filter tap) over all cm = OC rows of a 3 x 3 layer with
+// `ic` dense input channels; else (row block of cm = K rows, slab) of a 1 x 1 layer.
+static std::vector<int8_t> pack_fragments(const std::vector<int8_t>& w, int64_t Kp, bool first, int64_t cm, int64_t ic, int64_t oc) {
+    const int64_t step = cm * 64;
+    const int64_t slabs = first ? ic / 64 : cm / 64;
+    const int64_t n_steps = first ? 9 * slabs : (oc / cm) * slabs;
+    std::vector<int8_t> out(static_cast<size_t>(n_steps * step));
+    parallel_for(n_steps, [&](int64_t st) {
+        int64_t row0, k0;
+        if (first) {
+            const int64_t c = st / 9, tap = st % 9;
+            row0 = 0;
+            k0 = tap * ic + c * 64;
+        } else {
+            const int64_t pass = st / slabs, c = st % slabs;
+            row0 = pass * cm;
+            k0 = c * 64;
+        }
+        for (int64_t blk = 0; blk < cm / 64; ++blk)
+            for (int64_t f = 0; f < 4; ++f)
+                for (int64_t l = 0; l < 64; ++l) {
+                    const int64_t ks = f >> 1, ob = f & 1;
+                    std::memcpy(&out[static_cast<size_t>(st * step + ((blk * 4 + f) * 64 + l) * 16)],
+                                &w[static_cast<size_t>((row0 + blk * 64 + ob * 32 + (l & 31)) * Kp + k0 + ks * 32 + (l >> 5) * 16)], 16);
+                }
+    });
+    return out;
 }
 
 static void check_conv_desc(const hipie_conv_desc& d, const char* what) {
@@ -1771,10 +1823,19 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
             return;
         }
         PackedGemm g;
-        g.pack(device, d, weights);
+        std::vector<int8_t> packed;
+        g.pack(device, d, weights, &packed);
         c->K = g.K; c->Kp = g.Kp; c->OCp = g.OCp;
         c->wgt = std::move(g.wgt); c->koff = std::move(g.koff); c->corr = std::move(g.corr);
         c->epi.build(device, *epilogue, d.oc, c->OCp);
+        if (block_first_fits(d, c->Kp, c->OCp)) c->steps_role = 1;
+        else if (block_second_fits(d, c->Kp, c->OCp)) c->steps_role = 2;
+        if (device >= 0 && c->steps_role) {
+            const std::vector<int8_t> steps = pack_fragments(packed, c->Kp, c->steps_role == 1, c->steps_role == 1 ? d.oc : d.ic, d.ic, d.oc);
+            c->wgt_steps.upload(device, steps.data(), steps.size());
+        }
+        packed.clear();
+        packed.shrink_to_fit();
         c->few_pixel_ok = d.kh == 1 && d.kw == 1 && d.in_c_stride % 64 == 0 && c->Kp == d.in_c_stride && !d.acc_sub &&
                           d.stride_h == 1 && d.stride_w == 1 && d.pad_top == 0 && d.pad_left == 0 && d.pad_bottom == 0 &&
                           d.pad_right == 0 && skinny_epilogue_fits(c->epi.flags) && c->Kp * c->OCp <= (16 << 20) &&
@@ -1840,7 +1901,7 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && tile >= 0 && tile <= 23, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
+        HIPIE_REQUIRE(c && tile >= 0 && tile <= 24, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
         if (c->depthwise) {   // 0: registers only, 1: 3 x 3 through an LDS patch
             HIPIE_REQUIRE(tile == 0 || (tile == 1 && !(c->epi.flags & CF_RES) &&
                                         dwconv_strip_fits(c->d.kh, c->d.kw, c->d.dil_h, c->d.dil_w, c->d.stride_h, c->d.stride_w,
@@ -1866,6 +1927,10 @@ int hipie_conv_set_tile(hipie_conv* c, int tile) {
         HIPIE_REQUIRE(tile != 23 || c->few_pixel_ok, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: the few-pixel kernel takes unpadded 1 x 1 convolutions over pixels of a multiple of 64 "
                       "bytes with raw sums or a bias / scale / ReLU tail to f32");
+        HIPIE_REQUIRE(tile != 24 || (!c->fused && c->steps_role == 1 && block_epilogues_fit(c->epi.flags, false, 0)),
+                      HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_set_tile: the patch-staged kernel takes 3 x 3, stride 1, pad 1 convolutions over a multiple of 64 dense "
+                      "input channels with 64, 128 or 256 output channels, bias and a 256-level FakeQuantize from 0");
         HIPIE_REQUIRE(tile != 3 || 64 * (c->Kp + 16) + PT_ROWS * 64 * 4 <= 160 * 1024, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_set_tile: K=%lld does not fit the streaming kernel's LDS", (long long)c->Kp);
         c->tile = tile;
@@ -1908,122 +1973,133 @@ int hipie_conv_out_dims(const hipie_conv* c, int32_t h, int32_t w, int32_t* oh, 
     });
 }
 
+// Checks the tensors of one launch against the layer and fills the kernel arguments every variant shares; returns the
+// number of output pixels (0: nothing to do)
+static int64_t fill_conv_args(const hipie_conv* c, const hipie_tensor* in, const hipie_tensor* residual,
+                              const hipie_tensor* out, ConvArgs& a, int32_t& oh, int32_t& ow) {
+    HIPIE_REQUIRE(c && in && out, HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: null argument");
+    HIPIE_REQUIRE(c->wgt.ptr, HIPIE_NOT_ALLOCATED, "hipie_conv_run: host-only object");
+    const hipie_conv_desc& d = c->d;
+    HIPIE_REQUIRE(in->dtype == d.in_dtype && in->c == d.ic && in->stride_w == d.in_stride_w &&
+                      in->stride_h == d.in_stride_h,
+                  HIPIE_PARAMETER_MISMATCH,
+                  "hipie_conv_run: input (dtype %d, c %d, strides %lld/%lld) does not match the "
+                  "geometry the weights were packed for (dtype %d, c %d, strides %d/%d)",
+                  in->dtype, in->c, (long long)in->stride_h, (long long)in->stride_w, d.in_dtype, d.ic,
+                  d.in_stride_h, d.in_stride_w);
+    const int need_halo = std::max(std::max(d.pad_top, d.pad_bottom), std::max(d.pad_left, d.pad_right));
+    HIPIE_REQUIRE(in->halo >= need_halo, HIPIE_PARAMETER_MISMATCH,
+                  "hipie_conv_run: input halo %d < padding %d (the engine reads padding from the "
+                  "tensor's own border)", in->halo, need_halo);
+    oh = (in->h + d.pad_top + d.pad_bottom - (d.dil_h * (d.kh - 1) + 1)) / d.stride_h + 1;
+    ow = (in->w + d.pad_left + d.pad_right - (d.dil_w * (d.kw - 1) + 1)) / d.stride_w + 1;
+    HIPIE_REQUIRE(out->n == in->n && out->h == oh && out->w == ow && out->c == d.oc,
+                  HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: output is [%d,%d,%d,%d], expected [%d,%d,%d,%d]",
+                  out->n, out->h, out->w, out->c, in->n, oh, ow, d.oc);
+    HIPIE_REQUIRE(out->dtype == c->epi.out_dtype, HIPIE_PARAMETER_MISMATCH,
+                  "hipie_conv_run: output dtype %d, epilogue produces %d", out->dtype, c->epi.out_dtype);
+    const bool byte_out = out->dtype == HIPIE_U8B || out->dtype == HIPIE_I8;
+    HIPIE_REQUIRE(out->stride_w % (byte_out ? 16 : 4) == 0 && out->stride_w >= d.oc &&
+                      reinterpret_cast<uintptr_t>(out->data) % 16 == 0,
+                  HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: output channel stride/alignment");
+    HIPIE_REQUIRE(reinterpret_cast<uintptr_t>(in->data) % 4 == 0 &&
+                      (d.in_c_stride % 16 != 0 || reinterpret_cast<uintptr_t>(in->data) % 16 == 0),
+                  HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: input alignment");
+    const int64_t M = static_cast<int64_t>(in->n) * oh * ow;
+    if (M == 0) return 0;
+    const int64_t in_span = static_cast<int64_t>(in->n) * in->stride_n;
+    HIPIE_REQUIRE(in_span < (1ll << 31) && M < (1ll << 24), HIPIE_OUT_OF_BOUNDS,
+                  "hipie_conv_run: tensor too large (32-bit byte offsets, < 2^24 output pixels)");
+    a = ConvArgs{};
+    a.in = static_cast<const int8_t*>(in->data);
+    a.wgt = c->wgt.as<int8_t>();
+    a.wgt2 = c->wgt_rows.as<int8_t>();   // depthwise only; a fused shortcut overwrites it below
+    a.out = out->data;
+    a.koff = c->koff.as<int32_t>();
+    a.corr = c->corr.as<int32_t>();
+    c->epi.fill(a);
+    if (a.flags & CF_RES_GEMM) {
+        // `residual` is the INPUT of the fused shortcut convolution
+        HIPIE_REQUIRE(c->fused && residual && residual->data, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_run: shortcut input missing");
+        const hipie_conv_desc& sd = c->sd;
+        HIPIE_REQUIRE(residual->dtype == sd.in_dtype && residual->c == sd.ic && residual->n == in->n &&
+                          residual->stride_w == sd.in_stride_w && residual->stride_h == sd.in_stride_h,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: shortcut input does not match its packing");
+        int soh, sow;
+        conv_out_hw(sd, residual->h, residual->w, soh, sow);
+        HIPIE_REQUIRE(soh == oh && sow == ow, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_run: shortcut convolution yields %dx%d, main %dx%d", soh, sow, oh, ow);
+        HIPIE_REQUIRE(residual->halo >= std::max(std::max(sd.pad_top, sd.pad_bottom), std::max(sd.pad_left, sd.pad_right)),
+                      HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: shortcut input halo");
+        HIPIE_REQUIRE(static_cast<int64_t>(residual->n) * residual->stride_n < (1ll << 31), HIPIE_OUT_OF_BOUNDS,
+                      "hipie_conv_run: shortcut tensor too large");
+        a.in2 = static_cast<const int8_t*>(residual->data);
+        a.wgt2 = c->sg.wgt.as<int8_t>();
+        a.koff2 = c->sg.koff.as<int32_t>();
+        a.corr2 = c->sg.corr.as<int32_t>();
+        a.bias2 = c->s_bias.as<float>();
+        a.scale2 = c->s_scale.as<float>();
+        a.in2_sn = static_cast<int32_t>(residual->stride_n);
+        a.in2_sh = static_cast<int32_t>(residual->stride_h);
+        a.in2_sw = static_cast<int32_t>(residual->stride_w);
+        a.conv2_sh = sd.stride_h;
+        a.conv2_sw = sd.stride_w;
+        a.in2_origin = -(sd.pad_top * a.in2_sh + sd.pad_left * a.in2_sw);
+        a.Kp2 = static_cast<int32_t>(c->sg.Kp);
+        a.nk2 = static_cast<int32_t>(c->sg.Kp / 64);
+    } else if (a.flags & CF_RES) {
+        HIPIE_REQUIRE(residual && residual->data, HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: residual missing");
+        const int want = (a.flags & CF_RES_F32) ? HIPIE_F32 : ((a.flags & CF_RES_U8B) ? HIPIE_U8B : HIPIE_I8);
+        HIPIE_REQUIRE(residual->dtype == want && residual->n == out->n && residual->h == oh &&
+                          residual->w == ow && residual->c == d.oc,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: residual shape/dtype mismatch");
+        HIPIE_REQUIRE(residual->stride_w % ((a.flags & CF_RES_F32) ? 4 : 16) == 0 &&
+                          reinterpret_cast<uintptr_t>(residual->data) % 16 == 0,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: residual channel stride/alignment");
+        a.res = residual->data;
+        a.res_sn = static_cast<int32_t>(residual->stride_n);
+        a.res_sh = static_cast<int32_t>(residual->stride_h);
+        a.res_sw = static_cast<int32_t>(residual->stride_w);
+    }
+    a.M = static_cast<int32_t>(M);
+    a.OW = ow;
+    a.OHOW = oh * ow;
+    a.inv_OW = 1.0f / static_cast<float>(ow);
+    a.inv_OHOW = 1.0f / static_cast<float>(oh * ow);
+    a.in_sn = static_cast<int32_t>(in->stride_n);
+    a.in_sh = static_cast<int32_t>(in->stride_h);
+    a.in_sw = static_cast<int32_t>(in->stride_w);
+    a.conv_sh = d.stride_h;
+    a.conv_sw = d.stride_w;
+    a.in_origin = -(d.pad_top * a.in_sh + d.pad_left * a.in_sw);
+    a.out_sn = static_cast<int32_t>(out->stride_n);
+    a.out_sh = static_cast<int32_t>(out->stride_h);
+    a.out_sw = static_cast<int32_t>(out->stride_w);
+    // tensors that are dense in (n, h, w) for this convolution: pixel m sits at m * pixel stride
+    a.flat_in = static_cast<int64_t>(d.stride_h) * a.in_sh == static_cast<int64_t>(ow) * d.stride_w * a.in_sw &&
+                a.in_sn == static_cast<int64_t>(oh) * ow * d.stride_w * a.in_sw;
+    a.flat_out = a.out_sh == static_cast<int64_t>(ow) * a.out_sw && a.out_sn == static_cast<int64_t>(oh) * ow * a.out_sw;
+    a.flat_res = a.res != nullptr && a.res_sh == static_cast<int64_t>(ow) * a.res_sw &&
+                 a.res_sn == static_cast<int64_t>(oh) * ow * a.res_sw;
+    a.OC = d.oc;
+    a.OCp = static_cast<int32_t>(c->OCp);
+    a.Kp = static_cast<int32_t>(c->Kp);
+    a.nk = static_cast<int32_t>(c->Kp / 64);
+    a.wgt_ld = a.Kp;
+    a.wgt_rows = static_cast<int32_t>(c->OCp);
+    a.wgt_plain = 0;
+    return M;
+}
+
 static int conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tensor* residual,
                     const hipie_tensor* out, void* stream, bool static_scratch_only) {
     return guarded([&] {
-        HIPIE_REQUIRE(c && in && out, HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: null argument");
-        HIPIE_REQUIRE(c->wgt.ptr, HIPIE_NOT_ALLOCATED, "hipie_conv_run: host-only object");
-        const hipie_conv_desc& d = c->d;
-        HIPIE_REQUIRE(in->dtype == d.in_dtype && in->c == d.ic && in->stride_w == d.in_stride_w &&
-                          in->stride_h == d.in_stride_h,
-                      HIPIE_PARAMETER_MISMATCH,
-                      "hipie_conv_run: input (dtype %d, c %d, strides %lld/%lld) does not match the "
-                      "geometry the weights were packed for (dtype %d, c %d, strides %d/%d)",
-                      in->dtype, in->c, (long long)in->stride_h, (long long)in->stride_w, d.in_dtype, d.ic,
-                      d.in_stride_h, d.in_stride_w);
-        const int need_halo = std::max(std::max(d.pad_top, d.pad_bottom), std::max(d.pad_left, d.pad_right));
-        HIPIE_REQUIRE(in->halo >= need_halo, HIPIE_PARAMETER_MISMATCH,
-                      "hipie_conv_run: input halo %d < padding %d (the engine reads padding from the "
-                      "tensor's own border)", in->halo, need_halo);
+        ConvArgs a;
         int32_t oh, ow;
-        oh = (in->h + d.pad_top + d.pad_bottom - (d.dil_h * (d.kh - 1) + 1)) / d.stride_h + 1;
-        ow = (in->w + d.pad_left + d.pad_right - (d.dil_w * (d.kw - 1) + 1)) / d.stride_w + 1;
-        HIPIE_REQUIRE(out->n == in->n && out->h == oh && out->w == ow && out->c == d.oc,
-                      HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: output is [%d,%d,%d,%d], expected [%d,%d,%d,%d]",
-                      out->n, out->h, out->w, out->c, in->n, oh, ow, d.oc);
-        HIPIE_REQUIRE(out->dtype == c->epi.out_dtype, HIPIE_PARAMETER_MISMATCH,
-                      "hipie_conv_run: output dtype %d, epilogue produces %d", out->dtype, c->epi.out_dtype);
-        const bool byte_out = out->dtype == HIPIE_U8B || out->dtype == HIPIE_I8;
-        HIPIE_REQUIRE(out->stride_w % (byte_out ? 16 : 4) == 0 && out->stride_w >= d.oc &&
-                          reinterpret_cast<uintptr_t>(out->data) % 16 == 0,
-                      HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: output channel stride/alignment");
-        HIPIE_REQUIRE(reinterpret_cast<uintptr_t>(in->data) % 4 == 0 &&
-                          (d.in_c_stride % 16 != 0 || reinterpret_cast<uintptr_t>(in->data) % 16 == 0),
-                      HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: input alignment");
-        const int64_t M = static_cast<int64_t>(in->n) * oh * ow;
+        const int64_t M = fill_conv_args(c, in, residual, out, a, oh, ow);
         if (M == 0) return;
-        const int64_t in_span = static_cast<int64_t>(in->n) * in->stride_n;
-        HIPIE_REQUIRE(in_span < (1ll << 31) && M < (1ll << 24), HIPIE_OUT_OF_BOUNDS,
-                      "hipie_conv_run: tensor too large (32-bit byte offsets, < 2^24 output pixels)");
-        ConvArgs a{};
-        a.in = static_cast<const int8_t*>(in->data);
-        a.wgt = c->wgt.as<int8_t>();
-        a.wgt2 = c->wgt_rows.as<int8_t>();   // depthwise only; a fused shortcut overwrites it below
-        a.out = out->data;
-        a.koff = c->koff.as<int32_t>();
-        a.corr = c->corr.as<int32_t>();
-        c->epi.fill(a);
-        if (a.flags & CF_RES_GEMM) {
-            // `residual` is the INPUT of the fused shortcut convolution
-            HIPIE_REQUIRE(c->fused && residual && residual->data, HIPIE_PARAMETER_MISMATCH,
-                          "hipie_conv_run: shortcut input missing");
-            const hipie_conv_desc& sd = c->sd;
-            HIPIE_REQUIRE(residual->dtype == sd.in_dtype && residual->c == sd.ic && residual->n == in->n &&
-                              residual->stride_w == sd.in_stride_w && residual->stride_h == sd.in_stride_h,
-                          HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: shortcut input does not match its packing");
-            int soh, sow;
-            conv_out_hw(sd, residual->h, residual->w, soh, sow);
-            HIPIE_REQUIRE(soh == oh && sow == ow, HIPIE_PARAMETER_MISMATCH,
-                          "hipie_conv_run: shortcut convolution yields %dx%d, main %dx%d", soh, sow, oh, ow);
-            HIPIE_REQUIRE(residual->halo >= std::max(std::max(sd.pad_top, sd.pad_bottom), std::max(sd.pad_left, sd.pad_right)),
-                          HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: shortcut input halo");
-            HIPIE_REQUIRE(static_cast<int64_t>(residual->n) * residual->stride_n < (1ll << 31), HIPIE_OUT_OF_BOUNDS,
-                          "hipie_conv_run: shortcut tensor too large");
-            a.in2 = static_cast<const int8_t*>(residual->data);
-            a.wgt2 = c->sg.wgt.as<int8_t>();
-            a.koff2 = c->sg.koff.as<int32_t>();
-            a.corr2 = c->sg.corr.as<int32_t>();
-            a.bias2 = c->s_bias.as<float>();
-            a.scale2 = c->s_scale.as<float>();
-            a.in2_sn = static_cast<int32_t>(residual->stride_n);
-            a.in2_sh = static_cast<int32_t>(residual->stride_h);
-            a.in2_sw = static_cast<int32_t>(residual->stride_w);
-            a.conv2_sh = sd.stride_h;
-            a.conv2_sw = sd.stride_w;
-            a.in2_origin = -(sd.pad_top * a.in2_sh + sd.pad_left * a.in2_sw);
-            a.Kp2 = static_cast<int32_t>(c->sg.Kp);
-            a.nk2 = static_cast<int32_t>(c->sg.Kp / 64);
-        } else if (a.flags & CF_RES) {
-            HIPIE_REQUIRE(residual && residual->data, HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: residual missing");
-            const int want = (a.flags & CF_RES_F32) ? HIPIE_F32 : ((a.flags & CF_RES_U8B) ? HIPIE_U8B : HIPIE_I8);
-            HIPIE_REQUIRE(residual->dtype == want && residual->n == out->n && residual->h == oh &&
-                              residual->w == ow && residual->c == d.oc,
-                          HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: residual shape/dtype mismatch");
-            HIPIE_REQUIRE(residual->stride_w % ((a.flags & CF_RES_F32) ? 4 : 16) == 0 &&
-                              reinterpret_cast<uintptr_t>(residual->data) % 16 == 0,
-                          HIPIE_PARAMETER_MISMATCH, "hipie_conv_run: residual channel stride/alignment");
-            a.res = residual->data;
-            a.res_sn = static_cast<int32_t>(residual->stride_n);
-            a.res_sh = static_cast<int32_t>(residual->stride_h);
-            a.res_sw = static_cast<int32_t>(residual->stride_w);
-        }
-        a.M = static_cast<int32_t>(M);
-        a.OW = ow;
-        a.OHOW = oh * ow;
-        a.inv_OW = 1.0f / static_cast<float>(ow);
-        a.inv_OHOW = 1.0f / static_cast<float>(oh * ow);
-        a.in_sn = static_cast<int32_t>(in->stride_n);
-        a.in_sh = static_cast<int32_t>(in->stride_h);
-        a.in_sw = static_cast<int32_t>(in->stride_w);
-        a.conv_sh = d.stride_h;
-        a.conv_sw = d.stride_w;
-        a.in_origin = -(d.pad_top * a.in_sh + d.pad_left * a.in_sw);
-        a.out_sn = static_cast<int32_t>(out->stride_n);
-        a.out_sh = static_cast<int32_t>(out->stride_h);
-        a.out_sw = static_cast<int32_t>(out->stride_w);
-        // tensors that are dense in (n, h, w) for this convolution: pixel m sits at m * pixel stride
-        a.flat_in = static_cast<int64_t>(d.stride_h) * a.in_sh == static_cast<int64_t>(ow) * d.stride_w * a.in_sw &&
-                    a.in_sn == static_cast<int64_t>(oh) * ow * d.stride_w * a.in_sw;
-        a.flat_out = a.out_sh == static_cast<int64_t>(ow) * a.out_sw && a.out_sn == static_cast<int64_t>(oh) * ow * a.out_sw;
-        a.flat_res = a.res != nullptr && a.res_sh == static_cast<int64_t>(ow) * a.res_sw &&
-                     a.res_sn == static_cast<int64_t>(oh) * ow * a.res_sw;
-        a.OC = d.oc;
-        a.OCp = static_cast<int32_t>(c->OCp);
-        a.Kp = static_cast<int32_t>(c->Kp);
-        a.nk = static_cast<int32_t>(c->Kp / 64);
-        a.wgt_ld = a.Kp;
-        a.wgt_rows = static_cast<int32_t>(c->OCp);
-        a.wgt_plain = 0;
+        const hipie_conv_desc& d = c->d;
         if (c->depthwise) {
             HIPIE_REQUIRE(in->stride_w >= d.ic && in->stride_w % 16 == 0, HIPIE_PARAMETER_MISMATCH,
                           "hipie_conv_run: depthwise input channel stride");
@@ -2078,6 +2154,18 @@ static int conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_ten
                 a.t_shift = (a.t_tiles & (a.t_tiles - 1)) == 0 ? __builtin_ctz(a.t_tiles) : -1;
                 DeviceGuard g(c->device);
                 launch_rows(a, as_stream(stream));
+                HIPIE_CHECK_HIP(hipGetLastError());
+                return;
+            }
+        }
+        if (tile == 24) {
+            const BlockGeometry geo = block_geometry(d.oc, d.ic, oh, ow);
+            if (!geo.ok || in->halo < 1) {
+                tile = 0;                     // rows too wide for a tile: the general kernel
+            } else {
+                DeviceGuard g(c->device);
+                a.wgt = c->wgt_steps.as<int8_t>();
+                launch_block(a, nullptr, geo, in->n, as_stream(stream));
                 HIPIE_CHECK_HIP(hipGetLastError());
                 return;
             }
@@ -2164,6 +2252,56 @@ static int conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_ten
 int hipie_conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_tensor* residual,
                    const hipie_tensor* out, void* stream) {
     return conv_run(c, in, residual, out, stream, false);
+}
+
+int hipie_conv_pair_fits(const hipie_conv* first, const hipie_conv* second, int32_t h, int32_t w, int* fits) {
+    return guarded([&] {
+        HIPIE_REQUIRE(first && second && fits, HIPIE_PARAMETER_MISMATCH, "hipie_conv_pair_fits: null argument");
+        const hipie_conv_desc& da = first->d;
+        const hipie_conv_desc& db = second->d;
+        *fits = 0;
+        if (first->depthwise || second->depthwise || first->fused || second->fused) return;
+        if (first->steps_role != 1 || second->steps_role != 2 || db.ic != da.oc || db.in_dtype != first->epi.out_dtype) return;
+        if (!block_epilogues_fit(first->epi.flags, true, second->epi.flags)) return;
+        int oh, ow;
+        conv_out_hw(da, h, w, oh, ow);
+        *fits = block_geometry(da.oc, da.ic, oh, ow).ok ? 1 : 0;
+    });
+}
+
+int hipie_conv_run_pair(const hipie_conv* first, const hipie_conv* second, const hipie_tensor* in, const hipie_tensor* residual,
+                        const hipie_tensor* out, void* stream) {
+    return guarded([&] {
+        HIPIE_REQUIRE(first && second && in && out, HIPIE_PARAMETER_MISMATCH, "hipie_conv_run_pair: null argument");
+        int fits = 0;
+        const int st = hipie_conv_pair_fits(first, second, in->h, in->w, &fits);
+        if (st != HIPIE_OK) fail(static_cast<hipie_status>(st), "%s", std::string(hipie_last_error()).c_str());
+        HIPIE_REQUIRE(fits && in->halo >= 1, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_conv_run_pair: the fused kernel takes a 3 x 3, stride 1, pad 1 convolution (bias, FakeQuantize) over dense "
+                      "pixels with 64, 128 or 256 output channels followed by a 1 x 1 convolution over exactly those channels with a "
+                      "byte residual (ask hipie_conv_pair_fits first)");
+        HIPIE_REQUIRE(first->device == second->device, HIPIE_PARAMETER_MISMATCH, "hipie_conv_run_pair: layers of two devices");
+        // the intermediate tensor exists in LDS only: a descriptor of the shape the second layer was packed for,
+        // whose bytes nobody touches
+        hipie_tensor mid = *out;
+        mid.dtype = first->epi.out_dtype;
+        mid.c = first->d.oc;
+        mid.stride_w = second->d.in_stride_w;
+        mid.stride_h = second->d.in_stride_h;
+        mid.stride_n = static_cast<int64_t>(out->h) * mid.stride_h;
+        mid.halo = 0;
+        ConvArgs a, b;
+        int32_t oh, ow, oh2, ow2;
+        const int64_t M = fill_conv_args(first, in, nullptr, &mid, a, oh, ow);
+        if (M == 0) return;
+        (void)fill_conv_args(second, &mid, residual, out, b, oh2, ow2);
+        const BlockGeometry geo = block_geometry(first->d.oc, first->d.ic, oh, ow);
+        a.wgt = first->wgt_steps.as<int8_t>();
+        b.wgt = second->wgt_steps.as<int8_t>();
+        DeviceGuard g(first->device);
+        launch_block(a, &b, geo, in->n, as_stream(stream));
+        HIPIE_CHECK_HIP(hipGetLastError());
+    });
 }
 
 int hipie_conv_run_static(const hipie_conv* c, const hipie_tensor* in, const hipie_tensor* residual,

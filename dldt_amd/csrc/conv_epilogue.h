@@ -297,7 +297,10 @@ __device__ __forceinline__ void load_residual_bytes(const ConvArgs& a, int oc_la
 // sp: the tile's staged tables (stage_params) with local channel 0 = channel oc0, or nullptr to
 // read the tables from global memory
 // NOB = 2: a lane owns 32 channels (acc[0..1]); NOB = 1: 16 channels (acc[0] only)
-template <uint32_t F, int NOB = 2>
+// LDS_ONLY (byte outputs): the wave's 64 pixels x 64 channels stay in `stage` (row r = pixel, chunk c of 16 bytes in slot
+// c ^ ((r >> 2) & 3): the layout of an operand tile) and nothing is stored to memory - the tile is the next
+// convolution's operand
+template <uint32_t F, int NOB = 2, bool LDS_ONLY = false>
 __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                          const bool (&valid)[2], const int64_t (&out_off)[2],
                                          const int64_t (&res_off)[2], const v16f (&rres)[2][2],
@@ -561,6 +564,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
                     st[row * 4 + ((2 * h + j) ^ ((row >> 2) & 3))] = o;
                 }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (LDS_ONLY) return;
             const int oc_wave = oc_lane - 32 * h;
             const int c = lane_id & 3;
 #pragma unroll

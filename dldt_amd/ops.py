@@ -200,6 +200,20 @@ class Convolution:
                                    ctypes.byref(od), _stream()))
         return out
 
+    def pair_fits(self, second, h, w):
+        """hipie_conv_pair_fits: does the fused kernel take this layer followed by ``second`` on h x w inputs"""
+        fits = ctypes.c_int()
+        check(lib().hipie_conv_pair_fits(self._h, second._h, h, w, ctypes.byref(fits)))
+        return bool(fits.value)
+
+    def run_pair(self, second, x, out, residual=None):
+        """hipie_conv_run_pair: this layer and ``second`` in one kernel, the intermediate tensor kept in LDS"""
+        xd, od = x.desc(), out.desc()
+        rd = residual.desc() if residual is not None else None
+        check(lib().hipie_conv_run_pair(self._h, second._h, ctypes.byref(xd), ctypes.byref(rd) if rd else None,
+                                        ctypes.byref(od), _stream()))
+        return out
+
     def run_static(self, x, out, residual=None):
         """hipie_conv_run_static: the same launch with the K-split workspace in the library's fixed device array"""
         xd, od = x.desc(), out.desc()

@@ -253,7 +253,10 @@ int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* o
  * (which therefore must not be under graph capture) and kept until the process ends.  18 to 22 = 128 x 128 tiles
  * whose K step is a whole cache line of every operand row, 23 = the few-pixel kernel (unpadded 1 x 1 over pixels of
  * a multiple of 64 bytes, raw sums or a bias / scale / ReLU tail to f32: a lane per output channel on the vector
- * pipe, K split over the waves of a workgroup; the FC layer of a classifier).  A default is chosen
+ * pipe, K split over the waves of a workgroup; the FC layer of a classifier), 24 = whole output rows of one image x
+ * all 64, 128 or 256 output channels per workgroup, the input patch (every channel) staged once in LDS and the
+ * weights streamed through an LDS ring (3 x 3, stride 1, pad 1, undilated, dense pixels of a multiple of 64 channels,
+ * bias + 256-level FakeQuantize from 0; rows too wide for a tile run variant 0).  A default is chosen
  * from the shape; hipie_compile times the variants on the device and keeps the fastest.  Every
  * variant produces the same bits.
  * A depthwise convolution (group_convolution.hpp:78-144 with one filter per channel) has two variants of its own:
@@ -270,6 +273,18 @@ int hipie_conv_epilogue_flags(const hipie_conv* conv, uint32_t* flags, int* spec
 int hipie_conv_set_stages(hipie_conv* conv, int stages);
 int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,
                    const hipie_tensor* out, void* stream);
+/* Two consecutive convolutions in ONE kernel - the tail of a bottleneck block: `first` (3 x 3, stride 1, pad 1, bias,
+ * FakeQuantize to bytes) is computed for whole output rows of one image over all of its 64, 128 or 256 output
+ * channels, its level bytes stay in LDS in operand layout, and `second` (1 x 1 over exactly those channels, with its
+ * bias, scale, byte residual and FakeQuantize) runs from there: the intermediate tensor is neither written nor read,
+ * one launch instead of two.  Same arithmetic in the same order as hipie_conv_run on each layer, hence the same bits.
+ * The CPU plugin fuses consecutive convolutions into one primitive the same way
+ * (inference-engine/src/mkldnn_plugin/mkldnn_graph_optimizer.cpp:631-759 FuseConvolutionAndDWConvolution, and the
+ * sum post-op of :958-1130).  `in` is the first layer's input, `residual` and `out` the second layer's;
+ * hipie_conv_pair_fits says whether the kernel takes two layers on an input of h x w pixels. */
+int hipie_conv_pair_fits(const hipie_conv* first, const hipie_conv* second, int32_t h, int32_t w, int* fits);
+int hipie_conv_run_pair(const hipie_conv* first, const hipie_conv* second, const hipie_tensor* in,
+                        const hipie_tensor* residual, const hipie_tensor* out, void* stream);
 /* hipie_conv_run for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same kernels,
  * same bits; the one piece of device memory hipie_conv_run allocates - the workspace through which variants 14 to
