@@ -685,7 +685,7 @@ void conv_pipe_kernel(const ConvArgs a, const int stages) {
                 for (int r = 0; r < 16; ++r) acc[ob][pb][r] += red[((ob * 2 + pb) * 16 + r) * NT + t];
     }
     const int m0 = pix0 + wpix * 64 + l32;
-    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, batch, rres, (lds_cfloat_ptr)sP, BOC, oc0);
+    run_epilogue<F, true, false>(a, acc, oc_lane, m0, m0 + 32, batch, rres, (lds_cfloat_ptr)sP, BOC, oc0);   // tables in (dynamic) LDS, no staging
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -997,7 +997,7 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
         compute(cur, cur_k);
         if (cur_k + 1 == a.nk) {
             const int m0 = cur_tile * 256 + wave * 64 + l32;
-            run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, 0, (lds_cfloat_ptr)sP, 64, oc0);
+            run_epilogue<F, true>(a, acc, oc_lane, m0, m0 + 32, 0, (lds_cfloat_ptr)sP, 64, oc0);
             init_acc(a, oc_lane, acc);
         }
         return more;

@@ -66,14 +66,18 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 template <uint32_t FA, uint32_t FB, int NWC>
-__global__ __launch_bounds__(256, 2) void conv_block_kernel(const BlockArgs g) {
+__global__ __launch_bounds__(256, NWC == 4 ? 1 : 2) void conv_block_kernel(const BlockArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr bool kFused = FB != 0;
     constexpr int NW = 4, NWP = NW / NWC;
     constexpr int CM = NWC * 64, P = NWP * 64;
     constexpr int CSB = CM / 64;                // 64-byte slabs of the intermediate tile
     constexpr int WSTEP = NWC * 4096;           // weight bytes of one step: every wave row block's four fragments
-    constexpr int D = 3;                        // steps of weight fragments in flight (registers)
+    // steps of weight fragments in flight (registers; a divisor of nine, so that a tap always finds its step in the same
+    // registers).  With 256 channels a workgroup is alone on its compute unit and the stream is bound by latency:
+    // 36 KB per wave in flight run a step in 350 cycles where 12 KB take 490
+    constexpr int D = NWC == 4 ? 9 : 3;
+    constexpr int D0 = 3;                       // of them requested in front of the first barrier
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];
     // (not at LDS offset 0: the epilogue takes LDS pointers whose null value, zero, means "none")
     int8_t* const mid = lds + 256;                                         // [CSB][P][64 bytes]: 16 KB
@@ -140,7 +144,7 @@ __global__ __launch_bounds__(256, 2) void conv_block_kernel(const BlockArgs g) {
     };
     WFrag wreg[D];
 #pragma unroll
-    for (int s0 = 0; s0 < D; ++s0) load_wa(s0, wreg[s0]);                  // NA >= 9 > D
+    for (int s0 = 0; s0 < D0; ++s0) load_wa(s0, wreg[s0]);                 // NA >= 9 >= D
 
     stage_params_store<FA>(a, (lds_float_ptr)sPA, CM, tid, spa);
     if (kFused) stage_params_store<FB>(b, (lds_float_ptr)sPB0, CM, tid, spb);
@@ -194,6 +198,8 @@ __global__ __launch_bounds__(256, 2) void conv_block_kernel(const BlockArgs g) {
     // once anyway); the barrier makes every wave's part visible
     __builtin_amdgcn_s_waitcnt(block_waitcnt_vm_lds(0));
     __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int s0 = D0; s0 < D; ++s0) load_wa(s0, wreg[s0]);
     init_acc_lds((lds_cfloat_ptr)sPA, CM, woc * 64 + 32 * h, acc);
     HIPIE_STAMP(1);
 
@@ -223,8 +229,10 @@ __global__ __launch_bounds__(256, 2) void conv_block_kernel(const BlockArgs g) {
         __builtin_amdgcn_s_barrier();                                      // every wave is done with the patch: it becomes the stores' staging space
         ConvArgs e = a;
         e.M = min(a.M, pix0 + count);                                      // pixels behind the tile's rows belong to the next tile
-        run_epilogue<FA>(e, acc, woc * 64 + 32 * h, m0, m0 + 32, 0, rres, (lds_cfloat_ptr)sPA, CM, 0,
-                         (lds_float_ptr)patch + wave * 1024);
+        EpiAddr ea;
+        epilogue_addresses(e, woc * 64 + 32 * h, m0, m0 + 32, 0, ea);
+        epilogue<FA, 2, false, true>(e, acc, woc * 64 + 32 * h, ea.valid, ea.out_off, ea.res_off, rres, (lds_cfloat_ptr)sPA, CM, 0, nullptr,
+                                     (lds_float_ptr)patch + wave * 1024);
         HIPIE_STAMP(4);
         return;
     }
@@ -241,19 +249,52 @@ __global__ __launch_bounds__(256, 2) void conv_block_kernel(const BlockArgs g) {
         }
     };
     load_wb(0);
+    // where the lane's two pixels live in the output and residual tensors (channel 0 of the wave's part of pass 0), and
+    // the residual bytes of a pass: requested a pass ahead, like the weights
+    ConvArgs e = b;
+    e.M = min(b.M, pix0 + count);
+    EpiAddr ea;
+    epilogue_addresses(e, woc * 64 + 32 * h, m0, m0 + 32, 0, ea);
+    constexpr bool kByteRes = (FB & CF_RES) && !(FB & (CF_RES_F32 | CF_RES_GEMM));
+    // (requested as raw 16-byte pieces; the zeroing of pieces that do not exist waits until the pass consumes them - done
+    // at once it would wait for the loads the moment they are issued)
+    uint4 res_raw[2][2];
+    uint32_t res_cur[2][8];
+    auto res_exists = [&](int pass, int pb, int j) { return ea.valid[pb] && pass * CM + woc * 64 + 32 * h + 16 * j < e.res_sw; };
+    auto request_res = [&](int pass) {
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                // a lane without an element reads its (clamped, existing) pixel's first 16 bytes: no load hides in a branch
+                const int64_t off = res_exists(pass, pb, j) ? ea.res_off[pb] + pass * CM + 16 * j : ea.res_off[pb] - (woc * 64 + 32 * h);
+                res_raw[pb][j] = *reinterpret_cast<const uint4*>(static_cast<const int8_t*>(e.res) + off);
+            }
+    };
+    auto take_res = [&](int pass) {
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const bool ok = res_exists(pass, pb, j);
+                res_cur[pb][4 * j + 0] = ok ? res_raw[pb][j].x : 0u;
+                res_cur[pb][4 * j + 1] = ok ? res_raw[pb][j].y : 0u;
+                res_cur[pb][4 * j + 2] = ok ? res_raw[pb][j].z : 0u;
+                res_cur[pb][4 * j + 3] = ok ? res_raw[pb][j].w : 0u;
+            }
+    };
+    if (kByteRes) request_res(0);
 
     // ---- first epilogue: the tile's level bytes -> LDS, in the layout of an operand tile ------------------------------
     {
         const bool valid[2] = {true, true};
         const int64_t none[2] = {0, 0};
-        epilogue<FA, 2, true>(a, acc, woc * 64 + 32 * h, valid, none, none, rres, (lds_cfloat_ptr)sPA, CM, 0, nullptr,
+        epilogue<FA, 2, true, true>(a, acc, woc * 64 + 32 * h, valid, none, none, rres, (lds_cfloat_ptr)sPA, CM, 0, nullptr,
                               (lds_float_ptr)(mid + woc * (P * 64) + wpix * (64 * 64)));
     }
     HIPIE_STAMP(3);
 
     // ---- the 1 x 1 convolution: passes of CM output channels over the tile --------------------------------------------
-    ConvArgs e = b;
-    e.M = min(b.M, pix0 + count);
     for (int pass = 0; pass < g.passes; ++pass) {
         // pass 0: the tile is complete and the patch is free; later passes: everyone has left the previous epilogue
         // (whose tables the next store below overwrites)
@@ -269,13 +310,16 @@ __global__ __launch_bounds__(256, 2) void conv_block_kernel(const BlockArgs g) {
             if (C + 1 < CSB) read_b_mid(C + 1, bset[(C + 1) & 1]);
             mfma8(wb[C], bset[C & 1]);
         });
+        if (kByteRes) take_res(pass);
         if (more) {
             load_wb(pass + 1);
+            if (kByteRes) request_res(pass + 1);
             stage_params_store<FB>(b, tables_next, CM, tid, spb);
         }
         const int oc0 = pass * CM;
-        run_epilogue<FB>(e, acc, oc0 + woc * 64 + 32 * h, m0, m0 + 32, 0, rres, (lds_cfloat_ptr)tables, CM, oc0,
-                         (lds_float_ptr)patch + wave * 1024);
+        const int64_t oo[2] = {ea.out_off[0] + oc0, ea.out_off[1] + oc0}, ro[2] = {ea.res_off[0] + oc0, ea.res_off[1] + oc0};
+        epilogue<FB, 2, false, true>(e, acc, oc0 + woc * 64 + 32 * h, ea.valid, oo, ro, rres, (lds_cfloat_ptr)tables, CM, oc0,
+                     kByteRes ? res_cur : nullptr, (lds_float_ptr)patch + wave * 1024);
     }
     HIPIE_STAMP(4);
 #endif

@@ -300,7 +300,10 @@ __device__ __forceinline__ void load_residual_bytes(const ConvArgs& a, int oc_la
 // LDS_ONLY (byte outputs): the wave's 64 pixels x 64 channels stay in `stage` (row r = pixel, chunk c of 16 bytes in slot
 // c ^ ((r >> 2) & 3): the layout of an operand tile) and nothing is stored to memory - the tile is the next
 // convolution's operand
-template <uint32_t F, int NOB = 2, bool LDS_ONLY = false>
+// IN_LDS: the caller vouches that `sp` is set, STAGED that `stage` is (a pointer into dynamically sized LDS does not tell
+// the compiler, which then keeps both forms of every table read behind a run-time test and waits for all memory and
+// LDS operations in front of each group of channels)
+template <uint32_t F, int NOB = 2, bool LDS_ONLY = false, bool IN_LDS = false, bool STAGED = IN_LDS>
 __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                          const bool (&valid)[2], const int64_t (&out_off)[2],
                                          const int64_t (&res_off)[2], const v16f (&rres)[2][2],
@@ -313,7 +316,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
     // One pixel block (32 pixels) at a time, rows of 16 chunks with chunk c of row r kept in slot
     // c ^ (r & 15): conflict-free for the writes (rows r .. r + 7, one chunk) and the reads (one row).
     constexpr bool kCanStage = F != kDyn && !(F & (CF_OUT_FQ | CF_OUT_I32)) && NOB == 2;
-    const bool staged_out = kCanStage && stage != nullptr;
+    const bool staged_out = kCanStage && (STAGED || stage != nullptr);
     constexpr bool kCanStageBytes = F != kDyn && (F & CF_OUT_FQ) && NOB == 2;
     // an f32 residual that is the last operation in front of the store is added where the staged rows
     // are read back: there a lane's residual piece is as contiguous as its store
@@ -322,7 +325,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
     const bool late_res = kLateRes && staged_out;
     const int lane_id = static_cast<int>(threadIdx.x) & 63;
     auto tab = [&](int t, const float* g, int oc) {
-        if (sp) {
+        if (IN_LDS || sp) {
             typedef float v4f __attribute__((ext_vector_type(4)));
             const v4f v = *(const __attribute__((address_space(3))) v4f*)(sp + t * sp_stride + (oc - oc0));
             return make_float4(v.x, v.y, v.z, v.w);
@@ -545,7 +548,7 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
                 for (int q = 0; q < 4 * NOB; ++q) out_dw[pb][q] = add_bytes(out_dw[pb][q], off4);
         }
         const uint32_t xmask = flip ? 0x80808080u : 0u;
-        if (kCanStageBytes && stage != nullptr) {
+        if (kCanStageBytes && (STAGED || stage != nullptr)) {
             // Bytes leave through the wave's LDS buffer as well: 64 rows (pixels) of the wave's 64
             // channels, chunk c (16 bytes) of row r in slot c ^ ((r >> 2) & 3); four lanes then store
             // the 64 contiguous bytes of one pixel instead of 16-byte pieces of 32 different pixels.
@@ -618,22 +621,22 @@ __device__ __forceinline__ void epilogue_addresses(const ConvArgs& a, int oc_lan
     }
 }
 
-template <uint32_t F>
+template <uint32_t F, bool IN_LDS = false, bool STAGED = false>
 __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                              int m0, int m1, int batch, const v16f (&rres)[2][2],
                                              lds_cfloat_ptr sp = nullptr, int sp_stride = 0, int oc0 = 0,
                                              lds_float_ptr stage = nullptr) {
     EpiAddr e;
     epilogue_addresses(a, oc_lane, m0, m1, batch, e);
-    epilogue<F>(a, acc, oc_lane, e.valid, e.out_off, e.res_off, rres, sp, sp_stride, oc0, nullptr, stage);
+    epilogue<F, 2, false, IN_LDS, STAGED>(a, acc, oc_lane, e.valid, e.out_off, e.res_off, rres, sp, sp_stride, oc0, nullptr, stage);
 }
 
-template <uint32_t F>
+template <uint32_t F, bool IN_LDS = false>
 __device__ __forceinline__ void run_epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                              int m0, int m1, int batch = 0, lds_cfloat_ptr sp = nullptr,
                                              int sp_stride = 0, int oc0 = 0) {
     v16f none[2][2];
-    run_epilogue<F>(a, acc, oc_lane, m0, m1, batch, none, sp, sp_stride, oc0);
+    run_epilogue<F, IN_LDS, false>(a, acc, oc_lane, m0, m1, batch, none, sp, sp_stride, oc0);
 }
 
 }  // namespace hipie

@@ -212,7 +212,7 @@ __global__ __launch_bounds__(256 * KS, RB == 64 ? 2 : 1) void conv_line_kernel(c
     lds_float_ptr stage = (lds_float_ptr)(ring + (KS == 2 ? 65536 : 0)) + wave * 2048;
     v16f rres[2][2];
     const int m0 = pix0 + wpix * 64 + l32;
-    run_epilogue<F>(a, acc, oc_lane, m0, m0 + 32, 0, rres, (lds_cfloat_ptr)sP, BOC, oc0, stage);
+    run_epilogue<F, true, true>(a, acc, oc_lane, m0, m0 + 32, 0, rres, (lds_cfloat_ptr)sP, BOC, oc0, stage);   // both in (dynamic) LDS
 #endif
 }
 

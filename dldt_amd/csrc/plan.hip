@@ -144,6 +144,7 @@ struct Step {
     // the chosen variant as an integer (-1: the step has no variants), and its inverse
     virtual int variant() const { return -1; }
     virtual void set_variant(int) {}
+    virtual int launches() const { return 1; }   // kernels the step enqueues
 };
 
 void check_status(int st, const char* what) {
@@ -185,6 +186,7 @@ struct ConvStep : Step {
     // run inside this step's kernel when the fused form applies, else right before it
     std::unique_ptr<ConvStep> shortcut;
     bool fused = false;
+    float tuned_us = 0.f;          // per launch with every tuning lane busy, of the variant the tuner kept (0: not tuned)
     ~ConvStep() override { hipie_conv_destroy(conv); }
     void fill_desc(const std::vector<TensorInfo>& tensors) {
         const TensorInfo& t = tensors[in];
@@ -246,6 +248,7 @@ struct ConvStep : Step {
         r.halo = 0;
         return r;
     }
+    int launches() const override { return shortcut && !fused ? 2 : 1; }
     int variant() const override {
         int t = -1;
         if (conv) (void)hipie_conv_get_tile(conv, &t);
@@ -283,7 +286,7 @@ struct ConvStep : Step {
         }
         int best = current;
         float best_ms = 0.f, few_ms = -1.f;
-        const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22, 23};
+        const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22, 23, 24};
         for (size_t c = 0; c < sizeof(candidates) / sizeof(candidates[0]); ++c) {
             const int tile = candidates[c];
             if (c > 0 && tile == current) continue;
@@ -335,6 +338,7 @@ struct ConvStep : Step {
             (void)hipEventDestroy(e1[l]);
         }
         check_status(hipie_conv_set_tile(conv, best), name.c_str());
+        tuned_us = best_ms * 200.f / static_cast<float>(nl);
         if (std::getenv("HIPIE_TUNE_LOG")) {
             uint32_t fl = 0;
             int spec = 0;
@@ -342,6 +346,101 @@ struct ConvStep : Step {
             std::fprintf(stderr, "hipie tune: %-28s variant %d (%.1f us per launch with %zu in flight; default %d) epilogue %#x%s\n",
                          name.c_str(), best, best_ms * 200.f / static_cast<float>(nl), nl, current, fl, spec ? "" : " GENERIC");
         }
+    }
+};
+
+
+// A 3 x 3 convolution and the 1 x 1 convolution that is its only reader (the tail of a bottleneck block), planned as
+// two layers and run either one after the other or - where hipie_conv_pair_fits takes them and it is faster - as one
+// kernel that keeps the tensor between them in LDS (hipie_conv_run_pair).  Same bits either way.
+struct PairStep : Step {
+    std::unique_ptr<ConvStep> first, second;
+    int mode = 1;                  // PlanConfig::fuse_convs
+    bool fits = false, fused = false;
+    void create(int, const std::vector<TensorInfo>& tensors) override {   // (the layers exist already)
+        name = second->name;
+        macs = first->macs + second->macs;
+        out_node = second->out_node;
+        original_names = first->original_names + "," + second->original_names;
+        runtime_precision = first->runtime_precision;
+        output_precision = second->output_precision;
+        output_layout = second->output_layout;
+        const TensorInfo& ti = tensors[first->in];
+        int f = 0;
+        check_status(hipie_conv_pair_fits(first->conv, second->conv, ti.h, ti.w, &f), name.c_str());
+        fits = f != 0 && ti.halo >= 1 && second->res >= 0 && second->res_param < 0;
+        const TensorInfo& tm = tensors[first->out];
+        mid_bytes = static_cast<int64_t>(tm.n) * tm.h * tm.w * tm.c;
+        choose(fits && mode == 2);
+    }
+    int64_t mid_bytes = 0;         // the tensor between the layers: written and read when they run apart
+    void choose(bool one_kernel) {
+        fused = one_kernel;
+        type = fused ? "Convolution+Convolution" : "Convolution,Convolution";
+        bytes = first->bytes + second->bytes - (fused ? 2 * mid_bytes : 0);
+    }
+    int launches() const override { return fused ? 1 : first->launches() + second->launches(); }
+    void run_fused(uint8_t* arena, const std::vector<TensorInfo>& tensors, hipStream_t s) const {
+        const hipie_tensor i = tensors[first->in].desc(arena), o = tensors[second->out].desc(arena), r = tensors[second->res].desc(arena);
+        check_status(hipie_conv_run_pair(first->conv, second->conv, &i, &r, &o, s), name.c_str());
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const* outputs,
+             hipStream_t s) const override {
+        if (fused) {
+            run_fused(arena, tensors, s);
+        } else {
+            first->run(arena, tensors, inputs, outputs, s);
+            second->run(arena, tensors, inputs, outputs, s);
+        }
+    }
+    void tune(const std::vector<TuneLane>& lanes, const std::vector<TensorInfo>& tensors) override {
+        first->tune(lanes, tensors);
+        second->tune(lanes, tensors);
+        if (!fits || mode != 1) return;
+        const size_t nl = lanes.size();
+        std::vector<hipEvent_t> e0(nl), e1(nl);
+        for (size_t l = 0; l < nl; ++l) {
+            HIPIE_CHECK_HIP(hipEventCreate(&e0[l]));
+            HIPIE_CHECK_HIP(hipEventCreate(&e1[l]));
+        }
+        auto launch_all = [&](int times) {
+            for (int w = 0; w < times; ++w)
+                for (size_t l = 0; l < nl; ++l) run_fused(lanes[l].arena, tensors, lanes[l].stream);
+        };
+        launch_all(2);
+        float ms = 0.f;   // the same protocol as the layers' own variants: fastest of three rounds of five launches per lane
+        for (int round = 0; round < 3; ++round) {
+            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipStreamSynchronize(lanes[l].stream));
+            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventRecord(e0[l], lanes[l].stream));
+            launch_all(5);
+            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventRecord(e1[l], lanes[l].stream));
+            for (size_t l = 0; l < nl; ++l) HIPIE_CHECK_HIP(hipEventSynchronize(e1[l]));
+            float span = 0.f;
+            for (size_t a = 0; a < nl; ++a)
+                for (size_t b = 0; b < nl; ++b) {
+                    float t = 0.f;
+                    HIPIE_CHECK_HIP(hipEventElapsedTime(&t, e0[a], e1[b]));
+                    span = std::max(span, t);
+                }
+            ms = round == 0 ? span : std::min(ms, span);
+        }
+        for (size_t l = 0; l < nl; ++l) {
+            (void)hipEventDestroy(e0[l]);
+            (void)hipEventDestroy(e1[l]);
+        }
+        const float fused_us = ms * 200.f / static_cast<float>(nl), apart_us = first->tuned_us + second->tuned_us;
+        choose(apart_us > 0.f && fused_us < 0.97f * apart_us);
+        if (std::getenv("HIPIE_TUNE_LOG"))
+            std::fprintf(stderr, "hipie tune: %-28s one kernel %.1f us, two %.1f us per launch with %zu in flight: %s\n", name.c_str(),
+                         fused_us, apart_us, nl, fused ? "fused" : "apart");
+    }
+    // the layers' variants and the choice between one kernel and two, in one integer
+    int variant() const override { return first->variant() + 64 * second->variant() + (fused ? 4096 : 0); }
+    void set_variant(int v) override {
+        if (v < 0) return;
+        first->set_variant(v & 63);
+        second->set_variant((v >> 6) & 63);
+        choose(fits && (v & 4096) != 0 && mode != 0);
     }
 };
 
@@ -721,6 +820,8 @@ struct PlanConfig {
     bool keep_f32 = false;         // HIP_KEEP_F32
     bool fuse_attention = true;    // HIP_FUSE_ATTENTION
     bool merge_linear = true;      // HIP_MERGE_LINEAR
+    int fuse_convs = 1;            // HIP_FUSE_CONVOLUTIONS: a 3 x 3 convolution and the 1 x 1 behind it in one kernel - NO (0), AUTO
+                                   // (1: where the load-time measurement says it is faster), YES (2: wherever the kernel takes the pair)
     int device_id = -1;            // DEVICE_ID (must agree with the device argument when given)
     std::string network_name = "hipie_network";
 
@@ -736,6 +837,7 @@ struct PlanConfig {
         c.keep_f32 = env_flag("HIPIE_KEEP_F32", false);
         c.fuse_attention = env_flag("HIPIE_FUSE_ATTENTION", true);
         c.merge_linear = env_flag("HIPIE_MERGE_LINEAR", true);
+        if (const char* fc = std::getenv("HIPIE_FUSE_CONVS")) c.fuse_convs = std::max(0, std::min(2, std::atoi(fc)));
         return c;
     }
     static bool yes_no(const char* key, const char* v) {
@@ -767,6 +869,10 @@ struct PlanConfig {
         else if (k == "HIP_KEEP_F32") keep_f32 = yes_no(key, value);
         else if (k == "HIP_FUSE_ATTENTION") fuse_attention = yes_no(key, value);
         else if (k == "HIP_MERGE_LINEAR") merge_linear = yes_no(key, value);
+        else if (k == "HIP_FUSE_CONVOLUTIONS") {
+            if (!std::strcmp(value, "AUTO")) fuse_convs = 1;
+            else fuse_convs = yes_no(key, value) ? 2 : 0;
+        }
         else if (k == "NETWORK_NAME") network_name = value;
         else fail(HIPIE_NOT_FOUND, "config key '%s' is not supported", key);
     }
@@ -780,11 +886,12 @@ struct PlanConfig {
         else if (k == "HIP_KEEP_F32") v = yn(keep_f32);
         else if (k == "HIP_FUSE_ATTENTION") v = yn(fuse_attention);
         else if (k == "HIP_MERGE_LINEAR") v = yn(merge_linear);
+        else if (k == "HIP_FUSE_CONVOLUTIONS") v = fuse_convs == 1 ? "AUTO" : yn(fuse_convs == 2);
         else return false;
         return true;
     }
 };
-constexpr const char* kConfigKeys = "PERF_COUNT DEVICE_ID HIP_THROUGHPUT_STREAMS HIP_TUNE HIP_TUNE_FILE HIP_KEEP_F32 HIP_FUSE_ATTENTION HIP_MERGE_LINEAR";
+constexpr const char* kConfigKeys = "PERF_COUNT DEVICE_ID HIP_THROUGHPUT_STREAMS HIP_TUNE HIP_TUNE_FILE HIP_KEEP_F32 HIP_FUSE_ATTENTION HIP_MERGE_LINEAR HIP_FUSE_CONVOLUTIONS";
 
 // thrown by the planner for a node it cannot take: the status and text of any Error, plus the node
 struct UnsupportedNode : Error {
@@ -2281,6 +2388,33 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
             s->runtime_precision = type_name(in_dt);
         }
     }
+    // Bottleneck tails: a 3 x 3 convolution whose result only the next 1 x 1 convolution reads becomes one step with it
+    // (the pair stands where the 1 x 1 layer stood: everything it reads is computed by then)
+    if (cfg.fuse_convs != 0)
+        for (size_t i = 0; i < plan->steps.size(); ++i) {
+            auto* a = dynamic_cast<ConvStep*>(plan->steps[i].get());
+            if (!a || !a->conv || a->shortcut || a->res >= 0 || a->res_param >= 0 || a->out_node < 0 || a->desc.kh != 3 || a->desc.kw != 3) continue;
+            if (g->nodes[a->out_node].users.size() != 1) continue;
+            size_t j = i + 1;
+            ConvStep* b = nullptr;
+            for (; j < plan->steps.size() && !b; ++j) {
+                auto* c = dynamic_cast<ConvStep*>(plan->steps[j].get());
+                if (c && c->in == a->out) b = c;
+            }
+            if (!b || !b->conv || b->shortcut || b->res < 0) continue;
+            --j;
+            int fits = 0;
+            const TensorInfo& ti = plan->tensors[a->in];
+            if (hipie_conv_pair_fits(a->conv, b->conv, ti.h, ti.w, &fits) != HIPIE_OK || !fits) continue;
+            auto pair = std::make_unique<PairStep>();
+            pair->mode = cfg.fuse_convs;
+            pair->first.reset(static_cast<ConvStep*>(plan->steps[i].release()));
+            pair->second.reset(static_cast<ConvStep*>(plan->steps[j].release()));
+            pair->create(device, plan->tensors);
+            plan->steps[j] = std::move(pair);
+            plan->steps.erase(plan->steps.begin() + static_cast<std::ptrdiff_t>(i));
+            --i;
+        }
     for (size_t i = 0; i < pl.values.size(); ++i)
         if (pl.values[i].kind == VK_TENSOR) {
             plan->node_tensor[static_cast<int>(i)] = pl.values[i].tensor;
@@ -2621,6 +2755,7 @@ int hipie_plan_step_rt_info(const hipie_plan* p, int index, const char* key, cha
         else if (k == "outputLayouts") v = s.output_layout;
         else if (k == "execOrder") v = std::to_string(index);
         else if (k == "primitiveType") v = s.variant() >= 0 ? "hip_int8_v" + std::to_string(s.variant()) : "hip";
+        else if (k == "kernels") v = std::to_string(s.launches());
         else fail(HIPIE_NOT_FOUND, "hipie_plan_step_rt_info: key '%s' (execTimeMcs is hipie_request_perf)", key);
         copy_text(v, buf, cap, "hipie_plan_step_rt_info");
     });
@@ -2822,6 +2957,10 @@ int hipie_request_tensor(const hipie_request* r, int node_id, hipie_tensor* t) {
         auto it = r->plan->node_tensor.find(node_id);
         HIPIE_REQUIRE(it != r->plan->node_tensor.end(), HIPIE_NOT_FOUND,
                       "hipie_request_tensor: node %d was fused away or is not a tensor", node_id);
+        for (const auto& st : r->plan->steps)
+            if (auto* pair = dynamic_cast<const PairStep*>(st.get()))
+                HIPIE_REQUIRE(!(pair->fused && pair->first->out == it->second), HIPIE_NOT_FOUND,
+                              "hipie_request_tensor: node %d lives in LDS only (two convolutions run as one kernel)", node_id);
         *t = r->plan->tensors[it->second].desc(r->arena.as<uint8_t>());
     });
 }

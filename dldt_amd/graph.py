@@ -361,11 +361,16 @@ class Request:
         v = self.tensor(node_id)              # stored as n = h = 1, w = rows, c = columns
         return np.ascontiguousarray(v[0, :, 0, :].T)
 
-    def tensor(self, node_id):
-        """numpy NCHW copy of the arena tensor holding graph node `node_id` (u8 levels / f32)."""
+    def tensor(self, node_id, fused_ok=False):
+        """numpy NCHW copy of the arena tensor holding graph node `node_id` (u8 levels / f32).  fused_ok: None instead of
+        an error for a node whose value never reaches memory (fused away, or kept in LDS between two convolutions
+        that run as one kernel)."""
         import torch
         t = hipie_tensor()
-        check(lib().hipie_request_tensor(self._h, node_id, ctypes.byref(t)))
+        status = lib().hipie_request_tensor(self._h, node_id, ctypes.byref(t))
+        if status == -5 and fused_ok:
+            return None
+        check(status)
         esz = 4 if t.dtype in (F32, I32) else 1
         tdt = {F32: torch.float32, I32: torch.int32}.get(t.dtype, torch.int8)
         # view [n, h, w, c] through the strides

@@ -486,9 +486,13 @@ int hipie_compile(const hipie_graph* graph, int device, hipie_plan** plan);
  * flight together; the kernel variants are timed that way and OPTIMAL_NUMBER_OF_INFER_REQUESTS reports it),
  * HIP_TUNE (YES | NO: time the kernel variants at load, else shape-based defaults), HIP_TUNE_FILE (cache of the
  * choices, like the reference GPU plugin's KEY_TUNING_FILE), HIP_FUSE_ATTENTION, HIP_MERGE_LINEAR, HIP_KEEP_F32
- * (YES | NO), NETWORK_NAME.  An unknown key gives HIPIE_NOT_FOUND, a value the key does not take
+ * (YES | NO), HIP_FUSE_CONVOLUTIONS (a 3 x 3 convolution and the 1 x 1 convolution that alone reads its result as one
+ * kernel, hipie_conv_run_pair: AUTO = where the load-time measurement finds it faster, YES = wherever the kernel takes
+ * the pair, NO; the tensor between two layers run that way exists in LDS only and hipie_request_tensor gives
+ * HIPIE_NOT_FOUND for it), NETWORK_NAME.  An unknown key gives HIPIE_NOT_FOUND, a value the key does not take
  * HIPIE_PARAMETER_MISMATCH.  The environment variables HIPIE_TUNE, HIPIE_TUNE_FILE, HIPIE_TUNE_STREAMS,
- * HIPIE_FUSE_ATTENTION, HIPIE_MERGE_LINEAR, HIPIE_KEEP_F32 are the process-wide defaults of these keys. */
+ * HIPIE_FUSE_ATTENTION, HIPIE_MERGE_LINEAR, HIPIE_KEEP_F32, HIPIE_FUSE_CONVS (0 | 1 | 2 = NO | AUTO | YES) are the
+ * process-wide defaults of these keys. */
 int hipie_compile_opts(const hipie_graph* graph, int device, const char* const* keys, const char* const* values,
                        int n_opts, hipie_plan** plan);
 void hipie_plan_destroy(hipie_plan* plan);

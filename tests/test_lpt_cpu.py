@@ -83,10 +83,19 @@ def test_planner_fuses_resnet_block_chains():
     plan = Plan(g, device=-1)
     types = [s["type"] for s in plan.steps]
     # entry FQ, 53 convolutions (the 4 projection shortcuts run inside their residual convolution),
-    # max-pool, avg-pool(+FQ), FC, exit; every elementwise node is fused away
-    assert types.count("Convolution") == 45 and types.count("Convolution+Shortcut") == 4
+    # max-pool, avg-pool(+FQ), FC, exit; every elementwise node is fused away.  Seven bottleneck tails whose 3 x 3 layer
+    # has 64 or 128 channels (stages 3 and 4 of this narrow net, without the blocks with a convolution in the shortcut)
+    # are one step of two layers each
+    assert types.count("Convolution,Convolution") == 7 and "Convolution+Convolution" not in types   # (no measurement in a dry run)
+    assert types.count("Convolution") == 45 - 14 and types.count("Convolution+Shortcut") == 4
     assert types.count("MatMul") == 1 and types.count("MaxPool") == 1 and types.count("AvgPool") == 1
-    assert types[0] == "FakeQuantize" and types[-1] == "Result" and len(types) == 54
+    assert types[0] == "FakeQuantize" and types[-1] == "Result" and len(types) == 54 - 7
+    assert sum(int(plan.step_rt_info(i, "kernels")) for i in range(len(types))) == 54
+    always = Plan(g, device=-1, config={"HIP_FUSE_CONVOLUTIONS": "YES"})
+    assert [s["type"] for s in always.steps].count("Convolution+Convolution") == 7
+    assert sum(int(always.step_rt_info(i, "kernels")) for i in range(len(always.steps))) == 47
+    never = Plan(g, device=-1, config={"HIP_FUSE_CONVOLUTIONS": "NO"})
+    assert len(never.steps) == 54 and always.config("HIP_FUSE_CONVOLUTIONS") == "YES" and plan.config("HIP_FUSE_CONVOLUTIONS") == "AUTO"
     assert sum(s["macs"] for s in plan.steps) == meta["macs_per_image"]
     assert plan.arena_bytes > 0
     with pytest.raises(Exception) as e:

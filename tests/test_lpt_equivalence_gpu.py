@@ -153,7 +153,10 @@ def test_resnet_stack_follows_its_float_graph(orc):
     worst = {}
 
     def check(name, levels64):
-        dev = req.tensor(acts[name]["node"]).astype(np.int64)
+        dev = req.tensor(acts[name]["node"], fused_ok=True)
+        if dev is None:             # kept in LDS between two convolutions that run as one kernel: the next tensor tells
+            return
+        dev = dev.astype(np.int64)
         d = np.abs(dev - levels64.astype(np.int64))
         worst[name] = (float((d > 0).mean()), int(d.max()))
         assert d.max() <= 1 and (d > 0).mean() < 0.002, (name, worst[name])
@@ -217,7 +220,10 @@ def test_mobilenet_stack_follows_its_float_graph(orc):
     worst = {}
 
     def check(name, levels64):
-        dev = req.tensor(acts[name]["node"]).astype(np.int64)
+        dev = req.tensor(acts[name]["node"], fused_ok=True)
+        if dev is None:             # kept in LDS between two convolutions that run as one kernel: the next tensor tells
+            return
+        dev = dev.astype(np.int64)
         d = np.abs(dev - levels64.astype(np.int64))
         worst[name] = (float((d > 0).mean()), int(d.max()))
         assert d.max() <= 1 and (d > 0).mean() < 0.002, (name, worst[name])
