@@ -23,12 +23,17 @@ FLAGS = [
 ] + os.environ.get("HIPIE_EXTRA_FLAGS", "").split()
 
 
+# per-file additions: the bottleneck-tail kernel runs one or two waves per SIMD, where a wave's own instruction-level
+# parallelism is what hides latency - the scheduler is told to order for that instead of for registers
+EXTRA = {"conv_block.hip": os.environ.get("HIPIE_BLOCK_FLAGS", "").split()}
+
+
 def _compile(src, force):
     obj = os.path.join(CSRC, "build", os.path.basename(src) + ".o")
     deps = [src] + glob.glob(os.path.join(CSRC, "*.h")) + [os.path.join(os.path.dirname(HERE), "include", "hipie.h")]
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) > os.path.getmtime(d) for d in deps):
         return obj
-    cmd = [HIPCC] + FLAGS + (["-x", "hip"] if src.endswith(".hip") else []) + ["-c", src, "-o", obj]
+    cmd = [HIPCC] + FLAGS + EXTRA.get(os.path.basename(src), []) + (["-x", "hip"] if src.endswith(".hip") else []) + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

@@ -41,7 +41,8 @@ struct BlockGeometry {
 };
 BlockGeometry block_geometry(int oc_a, int ic_a, int oh, int ow);
 bool block_epilogues_fit(uint32_t flags_a, bool fused, uint32_t flags_b);
-void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo, int images, hipStream_t s);
+// deep: nine instead of three steps of weights in flight per wave, one workgroup per compute unit instead of two
+void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo, int images, bool deep, hipStream_t s);
 
 // depthwise kernels (dwconv.hip).  variant 0: a lane computes its outputs from registers loaded straight from memory;
 // variant 1: 3 x 3 through an LDS patch with the window sliding in registers (dwconv_strip_fits says which layers)

@@ -2165,7 +2165,7 @@ static int conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_ten
             } else {
                 DeviceGuard g(c->device);
                 a.wgt = c->wgt_steps.as<int8_t>();
-                launch_block(a, nullptr, geo, in->n, as_stream(stream));
+                launch_block(a, nullptr, geo, in->n, c->stages >= 6, as_stream(stream));
                 HIPIE_CHECK_HIP(hipGetLastError());
                 return;
             }
@@ -2299,7 +2299,7 @@ int hipie_conv_run_pair(const hipie_conv* first, const hipie_conv* second, const
         a.wgt = first->wgt_steps.as<int8_t>();
         b.wgt = second->wgt_steps.as<int8_t>();
         DeviceGuard g(first->device);
-        launch_block(a, &b, geo, in->n, as_stream(stream));
+        launch_block(a, &b, geo, in->n, first->stages >= 6, as_stream(stream));
         HIPIE_CHECK_HIP(hipGetLastError());
     });
 }

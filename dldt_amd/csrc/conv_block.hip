@@ -65,8 +65,8 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-template <uint32_t FA, uint32_t FB, int NWC>
-__global__ __launch_bounds__(256, NWC == 4 ? 1 : 2) void conv_block_kernel(const BlockArgs g) {
+template <uint32_t FA, uint32_t FB, int NWC, bool DEEP>
+__global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const BlockArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr bool kFused = FB != 0;
     constexpr int NW = 4, NWP = NW / NWC;
@@ -76,7 +76,9 @@ __global__ __launch_bounds__(256, NWC == 4 ? 1 : 2) void conv_block_kernel(const
     // steps of weight fragments in flight (registers; a divisor of nine, so that a tap always finds its step in the same
     // registers).  With 256 channels a workgroup is alone on its compute unit and the stream is bound by latency:
     // 36 KB per wave in flight run a step in 350 cycles where 12 KB take 490
-    constexpr int D = NWC == 4 ? 9 : 3;
+    // (DEEP: nine steps and one workgroup per compute unit, for a launch of no more workgroups than compute units; else
+    // three and two workgroups, which share the unit when several requests are in flight)
+    constexpr int D = DEEP ? 9 : 3;
     constexpr int D0 = 3;                       // of them requested in front of the first barrier
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];
     // (not at LDS offset 0: the epilogue takes LDS pointers whose null value, zero, means "none")
@@ -231,7 +233,7 @@ __global__ __launch_bounds__(256, NWC == 4 ? 1 : 2) void conv_block_kernel(const
         e.M = min(a.M, pix0 + count);                                      // pixels behind the tile's rows belong to the next tile
         EpiAddr ea;
         epilogue_addresses(e, woc * 64 + 32 * h, m0, m0 + 32, 0, ea);
-        epilogue<FA, 2, false, true>(e, acc, woc * 64 + 32 * h, ea.valid, ea.out_off, ea.res_off, rres, (lds_cfloat_ptr)sPA, CM, 0, nullptr,
+        epilogue<FA, 2, false, true, true, true>(e, acc, woc * 64 + 32 * h, ea.valid, ea.out_off, ea.res_off, rres, (lds_cfloat_ptr)sPA, CM, 0, nullptr,
                                      (lds_float_ptr)patch + wave * 1024);
         HIPIE_STAMP(4);
         return;
@@ -289,16 +291,25 @@ __global__ __launch_bounds__(256, NWC == 4 ? 1 : 2) void conv_block_kernel(const
     {
         const bool valid[2] = {true, true};
         const int64_t none[2] = {0, 0};
-        epilogue<FA, 2, true, true>(a, acc, woc * 64 + 32 * h, valid, none, none, rres, (lds_cfloat_ptr)sPA, CM, 0, nullptr,
+        epilogue<FA, 2, true, true, true, true>(a, acc, woc * 64 + 32 * h, valid, none, none, rres, (lds_cfloat_ptr)sPA, CM, 0, nullptr,
                               (lds_float_ptr)(mid + woc * (P * 64) + wpix * (64 * 64)));
     }
     HIPIE_STAMP(3);
 
     // ---- the 1 x 1 convolution: passes of CM output channels over the tile --------------------------------------------
+#ifdef HIPIE_BLOCK_STAMPS
+    long long t_bar = 0, t_mma = 0, t_epi = 0;
+#endif
     for (int pass = 0; pass < g.passes; ++pass) {
+#ifdef HIPIE_BLOCK_STAMPS
+        const long long q0 = clock64();
+#endif
         // pass 0: the tile is complete and the patch is free; later passes: everyone has left the previous epilogue
         // (whose tables the next store below overwrites)
         lds_barrier();
+#ifdef HIPIE_BLOCK_STAMPS
+        const long long q1 = clock64();
+#endif
         lds_float_ptr const tables = (lds_float_ptr)((pass & 1) ? sPA : sPB0);
         lds_float_ptr const tables_next = (lds_float_ptr)((pass & 1) ? sPB0 : sPA);
         const bool more = pass + 1 < g.passes;
@@ -310,6 +321,9 @@ __global__ __launch_bounds__(256, NWC == 4 ? 1 : 2) void conv_block_kernel(const
             if (C + 1 < CSB) read_b_mid(C + 1, bset[(C + 1) & 1]);
             mfma8(wb[C], bset[C & 1]);
         });
+#ifdef HIPIE_BLOCK_STAMPS
+        const long long q2 = clock64();
+#endif
         if (kByteRes) take_res(pass);
         if (more) {
             load_wb(pass + 1);
@@ -318,10 +332,22 @@ __global__ __launch_bounds__(256, NWC == 4 ? 1 : 2) void conv_block_kernel(const
         }
         const int oc0 = pass * CM;
         const int64_t oo[2] = {ea.out_off[0] + oc0, ea.out_off[1] + oc0}, ro[2] = {ea.res_off[0] + oc0, ea.res_off[1] + oc0};
-        epilogue<FB, 2, false, true>(e, acc, oc0 + woc * 64 + 32 * h, ea.valid, oo, ro, rres, (lds_cfloat_ptr)tables, CM, oc0,
+#ifdef HIPIE_BLOCK_NOSTORE
+        const bool vv[2] = {false, false};
+#else
+        const bool vv[2] = {ea.valid[0], ea.valid[1]};
+#endif
+        epilogue<FB, 2, false, true, true, true>(e, acc, oc0 + woc * 64 + 32 * h, vv, oo, ro, rres, (lds_cfloat_ptr)tables, CM, oc0,
                      kByteRes ? res_cur : nullptr, (lds_float_ptr)patch + wave * 1024);
+#ifdef HIPIE_BLOCK_STAMPS
+        const long long q3 = clock64();
+        t_bar += q1 - q0; t_mma += q2 - q1; t_epi += q3 - q2;
+#endif
     }
     HIPIE_STAMP(4);
+    HIPIE_STAMP_ADD(5, t_bar);
+    HIPIE_STAMP_ADD(6, t_mma);
+    HIPIE_STAMP_ADD(7, t_epi);
 #endif
 }
 
@@ -330,24 +356,26 @@ size_t block_lds_bytes(int nwc, int csa, int ppix) {
     return 256 + 16384 + 2 * PT_ROWS * cm * 4 + std::max<size_t>(static_cast<size_t>(csa) * ppix * 64, 16384);
 }
 
-template <uint32_t FA, uint32_t FB, int NWC>
+template <uint32_t FA, uint32_t FB, int NWC, bool DEEP>
 void launch_block_instance(const BlockArgs& g, size_t lds, hipStream_t s) {
     static bool attr_set = false;
     if (!attr_set) {
-        HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_block_kernel<FA, FB, NWC>),
+        HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_block_kernel<FA, FB, NWC, DEEP>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         attr_set = true;
     }
     const dim3 grid(g.p_per_xcd > 0 ? 8 * g.p_per_xcd : g.a.p_tiles), block(256);
-    hipLaunchKernelGGL((conv_block_kernel<FA, FB, NWC>), grid, block, lds, s, g);
+    hipLaunchKernelGGL((conv_block_kernel<FA, FB, NWC, DEEP>), grid, block, lds, s, g);
 }
 
 template <uint32_t FA, uint32_t FB>
-void launch_block_shape(const BlockArgs& g, int nwc, size_t lds, hipStream_t s) {
-    switch (nwc) {
-    case 1: launch_block_instance<FA, FB, 1>(g, lds, s); break;
-    case 2: launch_block_instance<FA, FB, 2>(g, lds, s); break;
-    case 4: launch_block_instance<FA, FB, 4>(g, lds, s); break;
+void launch_block_shape(const BlockArgs& g, int nwc, bool deep, size_t lds, hipStream_t s) {
+    switch (nwc * 2 + (deep ? 1 : 0)) {
+    case 2: case 3: launch_block_instance<FA, FB, 1, false>(g, lds, s); break;   // 64 channels: nine steps in all
+    case 4: launch_block_instance<FA, FB, 2, false>(g, lds, s); break;
+    case 5: launch_block_instance<FA, FB, 2, true>(g, lds, s); break;
+    case 8: launch_block_instance<FA, FB, 4, false>(g, lds, s); break;
+    case 9: launch_block_instance<FA, FB, 4, true>(g, lds, s); break;
     default: fail(HIPIE_GENERAL_ERROR, "block kernel: %d channel waves", nwc);
     }
 }
@@ -386,7 +414,7 @@ BlockGeometry block_geometry(int oc_a, int ic_a, int oh, int ow) {
     return r;
 }
 
-void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo, int images, hipStream_t s) {
+void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo, int images, bool deep, hipStream_t s) {
     BlockArgs g{};
     g.a = a;
     g.a.rows_per_tile = geo.rows;
@@ -409,7 +437,7 @@ void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo
     const int ia = block_index(kBlockFirst, a.flags), ib = b ? block_index(kBlockSecond, b->flags) : 3;
     HIPIE_REQUIRE(ia >= 0 && ib >= 0, HIPIE_GENERAL_ERROR, "block kernel: no instance for epilogues %#x / %#x", a.flags, b ? b->flags : 0u);
 #define HIPIE_BLOCK_CASE(IA, IB, FB) \
-    case (IA) * 4 + (IB): launch_block_shape<kBlockFirst[IA], FB>(g, geo.nwc, geo.lds, s); break;
+    case (IA) * 4 + (IB): launch_block_shape<kBlockFirst[IA], FB>(g, geo.nwc, deep, geo.lds, s); break;
     switch (ia * 4 + ib) {
         HIPIE_BLOCK_CASE(0, 0, kBlockSecond[0]) HIPIE_BLOCK_CASE(0, 1, kBlockSecond[1]) HIPIE_BLOCK_CASE(0, 2, kBlockSecond[2]) HIPIE_BLOCK_CASE(0, 3, 0u)
         HIPIE_BLOCK_CASE(1, 0, kBlockSecond[0]) HIPIE_BLOCK_CASE(1, 1, kBlockSecond[1]) HIPIE_BLOCK_CASE(1, 2, kBlockSecond[2]) HIPIE_BLOCK_CASE(1, 3, 0u)

@@ -303,7 +303,11 @@ __device__ __forceinline__ void load_residual_bytes(const ConvArgs& a, int oc_la
 // IN_LDS: the caller vouches that `sp` is set, STAGED that `stage` is (a pointer into dynamically sized LDS does not tell
 // the compiler, which then keeps both forms of every table read behind a run-time test and waits for all memory and
 // LDS operations in front of each group of channels)
-template <uint32_t F, int NOB = 2, bool LDS_ONLY = false, bool IN_LDS = false, bool STAGED = IN_LDS>
+// ILP: for a kernel whose waves run one or two to a SIMD - the eight values of a group of channels advance through the
+// FakeQuantize together, operation by operation (pinned, or the compiler folds them back into eight serial chains to
+// save registers), so that the wave's own independent instructions stand between an operation and its consumer
+#define HIPIE_PIN8(x) asm volatile("" : "+v"(x[0][0]), "+v"(x[0][1]), "+v"(x[0][2]), "+v"(x[0][3]), "+v"(x[1][0]), "+v"(x[1][1]), "+v"(x[1][2]), "+v"(x[1][3]))
+template <uint32_t F, int NOB = 2, bool LDS_ONLY = false, bool IN_LDS = false, bool STAGED = IN_LDS, bool ILP = false>
 __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2][2], int oc_lane,
                                          const bool (&valid)[2], const int64_t (&out_off)[2],
                                          const int64_t (&res_off)[2], const v16f (&rres)[2][2],
@@ -453,29 +457,56 @@ __device__ __forceinline__ void epilogue(const ConvArgs& a, const v16i (&acc)[2]
             }
         }
         if (fl & CF_OUT_FQ) {
+            // the eight values of a group advance together, operation by operation, and the two dwords are packed in
+            // turn: a wave that runs alone on its SIMD has nothing but its own independent instructions to put
+            // between an operation and the one that needs its result
             uint32_t packed[2] = {0, 0};
+            float t[2][4];
+            if (ILP && (fl & CF_FQ_DIV2) && (fl & CF_FQ_SAT)) {
+                float n[2][4], lo[2][4];
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        n[pb][j] = (fl & CF_FQ_IL0) ? v[pb][j] : v[pb][j] - il_[j];
+                        lo[pb][j] = n[pb][j] * r2_[j];
+                    }
+                HIPIE_PIN8(lo);
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) lo[pb][j] = fmaf(n[pb][j], rr_[j], lo[pb][j]);
+                HIPIE_PIN8(lo);
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) t[pb][j] = lo[pb][j] * a.lm1;
+                HIPIE_PIN8(t);
+            } else
 #pragma unroll
             for (int pb = 0; pb < 2; ++pb)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    float t;
                     if ((fl & CF_FQ_DIV2) && (fl & CF_FQ_SAT)) {
-                        t = (fl & CF_FQ_IL0) ? fq_level_fast<2, true, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], r2_[j], a.lm1)
-                                             : fq_level_fast<2, false, true>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], r2_[j], a.lm1);
+                        t[pb][j] = (fl & CF_FQ_IL0) ? fq_level_fast<2, true, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], r2_[j], a.lm1)
+                                                    : fq_level_fast<2, false, true>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], r2_[j], a.lm1);
                     } else if (fl & CF_FQ_DIV2) {
-                        t = (fl & CF_FQ_IL0) ? fq_level_fast<2, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], r2_[j], a.lm1)
-                                             : fq_level_fast<2, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], r2_[j], a.lm1);
+                        t[pb][j] = (fl & CF_FQ_IL0) ? fq_level_fast<2, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], r2_[j], a.lm1)
+                                                    : fq_level_fast<2, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], r2_[j], a.lm1);
                     } else if ((fl & CF_FQ_RCP) && (fl & CF_FQ_SAT)) {
-                        t = (fl & CF_FQ_IL0) ? fq_level_fast<1, true, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], 0.f, a.lm1)
-                                             : fq_level_fast<1, false, true>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], 0.f, a.lm1);
+                        t[pb][j] = (fl & CF_FQ_IL0) ? fq_level_fast<1, true, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], 0.f, a.lm1)
+                                                    : fq_level_fast<1, false, true>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], 0.f, a.lm1);
                     } else if (fl & CF_FQ_RCP) {
-                        t = (fl & CF_FQ_IL0) ? fq_level_fast<1, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], 0.f, a.lm1)
-                                             : fq_level_fast<1, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], 0.f, a.lm1);
+                        t[pb][j] = (fl & CF_FQ_IL0) ? fq_level_fast<1, true>(v[pb][j], 0.f, ih_[j], d_[j], rr_[j], 0.f, a.lm1)
+                                                    : fq_level_fast<1, false>(v[pb][j], il_[j], ih_[j], d_[j], rr_[j], 0.f, a.lm1);
                     } else {
-                        t = fq_level_fast<0, false>(v[pb][j], il_[j], ih_[j], d_[j], 0.f, 0.f, a.lm1);
+                        t[pb][j] = fq_level_fast<0, false>(v[pb][j], il_[j], ih_[j], d_[j], 0.f, 0.f, a.lm1);
                     }
-                    packed[pb] = __builtin_amdgcn_cvt_pk_u8_f32(t, j, packed[pb]);
                 }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb) packed[pb] = __builtin_amdgcn_cvt_pk_u8_f32(t[pb][j], j, packed[pb]);
             asm volatile("" : "+v"(packed[0]), "+v"(packed[1]) : : "memory");
             out_dw[0][e4] = packed[0];
             out_dw[1][e4] = packed[1];

@@ -249,13 +249,18 @@ struct ConvStep : Step {
         return r;
     }
     int launches() const override { return shortcut && !fused ? 2 : 1; }
+    bool deep = false;             // variant 24 with nine steps of weights in flight (hipie_conv_set_stages)
+    // kernel variant (hipie_conv_set_tile) + 32 for `deep`
     int variant() const override {
         int t = -1;
         if (conv) (void)hipie_conv_get_tile(conv, &t);
-        return t;
+        return t < 0 ? t : t + (deep ? 32 : 0);
     }
     void set_variant(int v) override {
-        if (conv && v >= 0) check_status(hipie_conv_set_tile(conv, v), name.c_str());
+        if (!conv || v < 0) return;
+        check_status(hipie_conv_set_tile(conv, v & 31), name.c_str());
+        deep = (v & 32) != 0;
+        check_status(hipie_conv_set_stages(conv, deep ? 8 : 0), name.c_str());
     }
     // Every variant computes the same integers, so the choice changes time only.  Variants a layer
     // cannot use are refused by hipie_conv_set_tile and skipped.
@@ -286,14 +291,15 @@ struct ConvStep : Step {
         }
         int best = current;
         float best_ms = 0.f, few_ms = -1.f;
-        const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22, 23, 24};
+        const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22, 23, 24, 24 + 32};
         for (size_t c = 0; c < sizeof(candidates) / sizeof(candidates[0]); ++c) {
-            const int tile = candidates[c];
-            if (c > 0 && tile == current) continue;
+            const int tile = candidates[c] & 31;
+            if (c > 0 && candidates[c] == current) continue;
             if (hipie_conv_set_tile(conv, tile) != HIPIE_OK) continue;
             int applied = -1;
             check_status(hipie_conv_get_tile(conv, &applied), name.c_str());
             if (applied != tile) continue;   // not available for this layer (kept its previous variant)
+            check_status(hipie_conv_set_stages(conv, (candidates[c] & 32) ? 8 : 0), name.c_str());
             launch_all(2);
             // the fastest of three rounds of five launches: a round disturbed by something else on the
             // device (another plan being compiled, a clock step) does not decide the choice
@@ -317,7 +323,7 @@ struct ConvStep : Step {
             // otherwise the choice (and the run-to-run spread of a whole network) follows the noise
             if (c == 0 || ms < 0.97f * best_ms) {
                 best_ms = ms;
-                best = tile;
+                best = candidates[c];
             }
             if (tile == 23) few_ms = ms;
         }
@@ -337,7 +343,7 @@ struct ConvStep : Step {
             (void)hipEventDestroy(e0[l]);
             (void)hipEventDestroy(e1[l]);
         }
-        check_status(hipie_conv_set_tile(conv, best), name.c_str());
+        set_variant(best);
         tuned_us = best_ms * 200.f / static_cast<float>(nl);
         if (std::getenv("HIPIE_TUNE_LOG")) {
             uint32_t fl = 0;
@@ -357,6 +363,7 @@ struct PairStep : Step {
     std::unique_ptr<ConvStep> first, second;
     int mode = 1;                  // PlanConfig::fuse_convs
     bool fits = false, fused = false;
+    bool deep = false;             // the fused kernel with nine steps of weights in flight (one workgroup per compute unit)
     void create(int, const std::vector<TensorInfo>& tensors) override {   // (the layers exist already)
         name = second->name;
         macs = first->macs + second->macs;
@@ -376,6 +383,8 @@ struct PairStep : Step {
     int64_t mid_bytes = 0;         // the tensor between the layers: written and read when they run apart
     void choose(bool one_kernel) {
         fused = one_kernel;
+        // the depth is a setting of the first layer's object: the pair's when they run as one kernel, else its own
+        if (first->conv) check_status(hipie_conv_set_stages(first->conv, (fused ? deep : first->deep) ? 8 : 0), name.c_str());
         type = fused ? "Convolution+Convolution" : "Convolution,Convolution";
         bytes = first->bytes + second->bytes - (fused ? 2 * mid_bytes : 0);
     }
@@ -396,7 +405,7 @@ struct PairStep : Step {
     void tune(const std::vector<TuneLane>& lanes, const std::vector<TensorInfo>& tensors) override {
         first->tune(lanes, tensors);
         second->tune(lanes, tensors);
-        if (!fits || mode != 1) return;
+        if (!fits || mode == 0) return;
         const size_t nl = lanes.size();
         std::vector<hipEvent_t> e0(nl), e1(nl);
         for (size_t l = 0; l < nl; ++l) {
@@ -407,6 +416,9 @@ struct PairStep : Step {
             for (int w = 0; w < times; ++w)
                 for (size_t l = 0; l < nl; ++l) run_fused(lanes[l].arena, tensors, lanes[l].stream);
         };
+        float best_fused = 0.f;
+        for (int d = 0; d < 2; ++d) {
+        check_status(hipie_conv_set_stages(first->conv, d ? 8 : 0), name.c_str());
         launch_all(2);
         float ms = 0.f;   // the same protocol as the layers' own variants: fastest of three rounds of five launches per lane
         for (int round = 0; round < 3; ++round) {
@@ -424,22 +436,28 @@ struct PairStep : Step {
                 }
             ms = round == 0 ? span : std::min(ms, span);
         }
+        if (d == 0 || ms < 0.97f * best_fused) {
+            best_fused = ms;
+            deep = d != 0;
+        }
+        }
         for (size_t l = 0; l < nl; ++l) {
             (void)hipEventDestroy(e0[l]);
             (void)hipEventDestroy(e1[l]);
         }
-        const float fused_us = ms * 200.f / static_cast<float>(nl), apart_us = first->tuned_us + second->tuned_us;
-        choose(apart_us > 0.f && fused_us < 0.97f * apart_us);
+        const float fused_us = best_fused * 200.f / static_cast<float>(nl), apart_us = first->tuned_us + second->tuned_us;
+        choose(mode == 2 || (apart_us > 0.f && fused_us < 0.97f * apart_us));
         if (std::getenv("HIPIE_TUNE_LOG"))
-            std::fprintf(stderr, "hipie tune: %-28s one kernel %.1f us, two %.1f us per launch with %zu in flight: %s\n", name.c_str(),
-                         fused_us, apart_us, nl, fused ? "fused" : "apart");
+            std::fprintf(stderr, "hipie tune: %-28s one kernel %.1f us (%s), two %.1f us per launch with %zu in flight: %s\n", name.c_str(),
+                         fused_us, deep ? "nine steps in flight" : "three steps in flight", apart_us, nl, fused ? "fused" : "apart");
     }
     // the layers' variants and the choice between one kernel and two, in one integer
-    int variant() const override { return first->variant() + 64 * second->variant() + (fused ? 4096 : 0); }
+    int variant() const override { return first->variant() + 64 * second->variant() + (fused ? 4096 : 0) + (deep ? 8192 : 0); }
     void set_variant(int v) override {
         if (v < 0) return;
         first->set_variant(v & 63);
         second->set_variant((v >> 6) & 63);
+        deep = (v & 8192) != 0;
         choose(fits && (v & 4096) != 0 && mode != 0);
     }
 };

@@ -269,7 +269,9 @@ int hipie_conv_get_tile(const hipie_conv* conv, int* tile);
  * these steps compiled in exists (otherwise the generic, slower instance runs) */
 int hipie_conv_epilogue_flags(const hipie_conv* conv, uint32_t* flags, int* specialised);
 /* ring depth of the pipelined variants: 3, 4, 6 or 8 K steps in LDS (other values round down, and to
- * what fits 144 KB); 0 = the variant's default (4 for tile 4, else 3) */
+ * what fits 144 KB); 0 = the variant's default (4 for tile 4, else 3).  Variant 24 and hipie_conv_run_pair (the
+ * setting of its first layer): 6 and more = nine steps of weights in flight in a wave's registers and one workgroup
+ * per compute unit (for a launch that runs alone), else three steps and two workgroups */
 int hipie_conv_set_stages(hipie_conv* conv, int stages);
 int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,
                    const hipie_tensor* out, void* stream);
