@@ -152,8 +152,11 @@ def main():
                     help="infer requests in flight, one stream each (HIP gives a process 4 hardware queues here and the "
                          "default stream holds one: 3 ran 15 % faster than 4)")
     ap.add_argument("--repeats", type=int, default=5, help="timed regions of --steps steps each; the median one is reported")
-    ap.add_argument("--tune-rounds", type=int, default=3,
-                    help="plans compiled (each tunes its kernels by timing them at load); the fastest over a short run is benchmarked")
+    ap.add_argument("--tune-rounds", type=int, default=1,
+                    help="plans compiled (each tunes its kernels by timing them at load); 1 = the one plan a user's LoadNetwork "
+                         "gets, more = the fastest of several over a short trial (every trial is reported)")
+    ap.add_argument("--settle-seconds", type=float, default=1.0,
+                    help="untimed inferences in front of the warm-up steps, so that the first timed region runs at the clocks the last one does")
     ap.add_argument("--no-host-inclusive", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -168,7 +171,7 @@ def main():
     g, meta = builders.resnet50(batch=args.batch, res=224)
     gen = torch.Generator(device="cuda").manual_seed(20211)
 
-    def run(plan, nreq, steps, warmup, repeats=1):
+    def run(plan, nreq, steps, warmup, repeats=1, settle=0.0):
         """`repeats` timed regions of `steps` inferences round-robin over nreq requests;
         ([ms per step by HIP events] per region, [wall ms per step] per region, device buffers)"""
         reqs = [plan.create_request(perf_count=False) for _ in range(nreq)]
@@ -177,6 +180,12 @@ def main():
             ins[0].copy_(torch.rand(ins[0].shape, generator=gen, device="cuda"))
         streams = [torch.cuda.ExternalStream(r.stream) for r in reqs]
         torch.cuda.synchronize()
+        t_settle = time.perf_counter()
+        while time.perf_counter() - t_settle < settle:       # the device reaches its steady clocks under this load
+            for i in range(3 * nreq):
+                reqs[i % nreq].enqueue(*bufs[i % nreq])
+            for st in streams:
+                st.synchronize()
         for i in range(warmup):
             reqs[i % nreq].enqueue(*bufs[i % nreq])
         for st in streams:
@@ -213,7 +222,7 @@ def main():
     trial_ms = [t[0] for t in plans]
     del plans
 
-    spans, walls, bufs = run(plan, args.requests, args.steps, args.warmup, repeats=max(1, args.repeats))
+    spans, walls, bufs = run(plan, args.requests, args.steps, args.warmup, repeats=max(1, args.repeats), settle=args.settle_seconds)
     order = sorted(range(len(spans)), key=lambda i: spans[i])
     mid = order[(len(order) - 1) // 2]          # the median region (the lower one of two)
     ms_per_step, wall_ms_step = spans[mid], walls[mid]

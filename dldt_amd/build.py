@@ -30,7 +30,7 @@ EXTRA = {"conv_block.hip": os.environ.get("HIPIE_BLOCK_FLAGS", "").split()}
 
 def _compile(src, force):
     obj = os.path.join(CSRC, "build", os.path.basename(src) + ".o")
-    deps = [src] + glob.glob(os.path.join(CSRC, "*.h")) + [os.path.join(os.path.dirname(HERE), "include", "hipie.h")]
+    deps = [src] + glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(os.path.join(os.path.dirname(HERE), "include", "*.h"))
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) > os.path.getmtime(d) for d in deps):
         return obj
     cmd = [HIPCC] + FLAGS + EXTRA.get(os.path.basename(src), []) + (["-x", "hip"] if src.endswith(".hip") else []) + ["-c", src, "-o", obj]

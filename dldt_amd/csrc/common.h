@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "../../include/hipie.h"
+#include "../../include/hipie_diag.h"
 
 namespace hipie {
 

@@ -50,7 +50,7 @@ struct DwGeometry {
     int in_h, in_w, halo;     // interior size of the input tensor and its readable border
     int pad_top, pad_left;
 };
-bool dwconv_strip_fits(int KH, int KW, int dil_h, int dil_w, int stride_h, int stride_w, int in_c_stride, uint32_t flags);
+bool dwconv_strip_fits(int KH, int KW, int dil_h, int dil_w, int stride_h, int stride_w, int in_c_stride, int ocp, uint32_t flags);
 void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, int variant, const DwGeometry& g, hipStream_t s);
 
 // frees the split-K workspace kept for this stream, if any (for the owner of a stream, before it destroys

@@ -1905,7 +1905,7 @@ int hipie_conv_set_tile(hipie_conv* c, int tile) {
         if (c->depthwise) {   // 0: registers only, 1: 3 x 3 through an LDS patch
             HIPIE_REQUIRE(tile == 0 || (tile == 1 && !(c->epi.flags & CF_RES) &&
                                         dwconv_strip_fits(c->d.kh, c->d.kw, c->d.dil_h, c->d.dil_w, c->d.stride_h, c->d.stride_w,
-                                                          c->d.in_c_stride, c->epi.flags)),
+                                                          c->d.in_c_stride, static_cast<int>(c->OCp), c->epi.flags)),
                           HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: depthwise variant %d does not take this layer", tile);
             c->tile = tile;
             return;

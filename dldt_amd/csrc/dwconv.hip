@@ -387,11 +387,12 @@ struct XcdGrid {
 
 // the LDS strip kernel takes 3 x 3, undilated, stride 1 or 2 (the same both ways) with one of the specialised epilogues,
 // pixels of at most 1024 bytes (a lane per four channels, at most 256 lanes) and no residual
-bool dwconv_strip_fits(int KH, int KW, int dil_h, int dil_w, int stride_h, int stride_w, int in_c_stride, uint32_t flags) {
+bool dwconv_strip_fits(int KH, int KW, int dil_h, int dil_w, int stride_h, int stride_w, int in_c_stride, int ocp, uint32_t flags) {
     const uint32_t core = flags & ~CF_OUT_XOR;
     const bool known = core == E_PLAIN0 || core == E_CLAMPFQ || core == E_SCALEFQ0;
+    // (a lane reads the weights and tables of the channels its pixel slice holds: the padded channel count must cover the stride)
     return KH == 3 && KW == 3 && dil_h == 1 && dil_w == 1 && stride_h == stride_w && (stride_h == 1 || stride_h == 2) && known &&
-           in_c_stride % 16 == 0 && in_c_stride <= 1024;
+           in_c_stride % 16 == 0 && in_c_stride <= 1024 && in_c_stride <= ocp;
 }
 
 static void launch_dwconv_strip(const ConvArgs& a, const DwGeometry& g, hipStream_t s) {
@@ -449,7 +450,7 @@ void launch_dwconv(const ConvArgs& a, int KH, int KW, int dil_h, int dil_w, int 
     const uint32_t core = a.flags & ~CF_OUT_XOR;
     const bool known = core == E_PLAIN0 || core == E_CLAMPFQ || core == E_SCALEFQ0;
     if (variant == 1) {
-        HIPIE_REQUIRE(dwconv_strip_fits(KH, KW, dil_h, dil_w, a.conv_sh, a.conv_sw, a.in_sw, a.flags) && !(a.flags & CF_RES),
+        HIPIE_REQUIRE(dwconv_strip_fits(KH, KW, dil_h, dil_w, a.conv_sh, a.conv_sw, a.in_sw, a.OCp, a.flags) && !(a.flags & CF_RES),
                       HIPIE_GENERAL_ERROR, "depthwise strip kernel chosen for a layer it does not take");
         launch_dwconv_strip(a, g, s);
         return;

@@ -37,6 +37,7 @@ struct EltArgs {
     int32_t out_dtype = HIPIE_F32;    // HIPIE_F32, or HIPIE_U8B / HIPIE_I8 behind a FakeQuantize
     int64_t out_sn = 0, out_sh = 0, out_sw = 0;
     int32_t N = 0, H = 0, W = 0, C = 0;
+    int32_t device = 0;               // where the tensors live (an f32 result has no FakeQuantize object to tell)
 };
 }  // namespace hipie
 struct hipie_fq;

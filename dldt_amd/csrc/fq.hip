@@ -563,11 +563,13 @@ __global__ __launch_bounds__(kThreads) void eltwise_nhwc_kernel(const EltArgs a,
                                                                 int64_t total) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
     if (idx >= total) return;
-    auto divmod = [](int64_t v, int32_t d, float inv, int32_t& q, int32_t& r) {   // exact below 2^24 after one correction
+    auto divmod = [](int64_t v, int32_t d, float inv, int32_t& q, int32_t& r) {   // estimate by reciprocal, exact by the remainder
         q = static_cast<int32_t>(static_cast<float>(v) * inv);
         int64_t rem = v - static_cast<int64_t>(q) * d;
-        if (rem < 0) { --q; rem += d; }
-        else if (rem >= d) { ++q; rem -= d; }
+        // the dividend may exceed 2^24 (only the quotient is below it): its conversion, the reciprocal and the product
+        // each round, so the estimate can be off by a few units - corrected until the remainder is in range
+        while (rem < 0) { --q; rem += d; }
+        while (rem >= d) { ++q; rem -= d; }
         r = static_cast<int32_t>(rem);
     };
     int32_t pix, g, n, hw, h, w;
@@ -623,7 +625,7 @@ void hipie::run_eltwise(const hipie_fq* fq, const EltArgs& a, hipStream_t s) {
         off = a.out_dtype == HIPIE_U8B ? fq->q8_base - 128.0f : fq->q8_base;
         rcp = fq->rcp;
     }
-    DeviceGuard g(fq ? fq->device : 0);
+    DeviceGuard g(fq ? fq->device : a.device);
     const dim3 grid(static_cast<uint32_t>(ceil_div(total, kThreads))), block(kThreads);
     const float ig = 1.0f / static_cast<float>(groups), iw = 1.0f / static_cast<float>(a.W), ihw = 1.0f / static_cast<float>(a.H * a.W);
     if (rcp) hipLaunchKernelGGL(eltwise_nhwc_kernel<true>, grid, block, 0, s, a, tab, lm1, off, groups, ig, iw, ihw, total);

@@ -7,6 +7,7 @@
 // them.  Every materialised tensor gets its own arena region (NHWC, padded channels, a halo as
 // wide as the largest padding among its consumers, pre-filled with level 0 once); nothing is
 // allocated or freed after compilation.
+#include <atomic>
 #include <chrono>
 #include <condition_variable>
 #include <mutex>
@@ -576,8 +577,10 @@ struct EltwiseStep : Step {
     std::vector<float> il, ih;
     float ol = 0, oh = 0;
     hipie_fq* fq = nullptr;
+    int device_ = 0;                     // the plan's device
     ~EltwiseStep() override { hipie_fq_destroy(fq); }
     void create(int device, const std::vector<TensorInfo>& tensors) override {
+        device_ = device;
         const int C = tensors[out].c;
         if (quantize) {
             check_status(hipie_fq_create(device, C, levels, il.data(), il.size(), ih.data(), ih.size(), &ol, 1, &oh, 1, &fq), name.c_str());
@@ -619,6 +622,7 @@ struct EltwiseStep : Step {
         e.out_dtype = t.dtype;
         e.out_sn = t.stride_n; e.out_sh = t.stride_h; e.out_sw = t.stride_w;
         e.N = t.n; e.H = t.h; e.W = t.w; e.C = t.c;
+        e.device = device_;
         run_eltwise(fq, e, s);
     }
 };
@@ -2288,8 +2292,9 @@ struct hipie_request {
     hipStream_t stream = nullptr;
     bool perf = false;
     std::vector<hipEvent_t> events;
-    bool started = false;
-    bool cancelled = false;                  // hipie_request_cancel was called on the running inference
+    // written by the thread that starts and waits, and by whichever thread calls hipie_request_cancel meanwhile
+    std::atomic<bool> started{false};
+    std::atomic<bool> cancelled{false};      // hipie_request_cancel was called on the running inference
     std::vector<void*> pending_out;          // host destinations of the running async infer
     ~hipie_request() {
         for (auto e : events) (void)hipEventDestroy(e);
@@ -2634,7 +2639,9 @@ int hipie_get_metric(int device, const char* name, char* buf, size_t cap) {
             v = nm;
         } else if (k == "IMPORT_EXPORT_SUPPORT") v = "YES";
         else if (k == "DEVICE_ARCHITECTURE") v = "gfx950";
-        else if (k == "OPTIMIZATION_CAPABILITIES") v = "INT8 FP32";
+        // INT8 only: convolutions and MatMuls are planned over quantized operands alone (an unquantized one is refused and
+        // reported unsupported by hipie_query); f32 is what the elementwise, Softmax, MVN and Gelu steps between them compute in
+        else if (k == "OPTIMIZATION_CAPABILITIES") v = "INT8";
         else if (k == "RANGE_FOR_ASYNC_INFER_REQUESTS") v = "1 8 1";
         else if (k == "RANGE_FOR_STREAMS") v = "1 8";
         else fail(HIPIE_NOT_FOUND, "metric '%s' is not supported", name);
@@ -2894,8 +2901,10 @@ int hipie_request_wait_for(hipie_request* r, int64_t timeout_ms) {
         HIPIE_REQUIRE(r->started, HIPIE_INFER_NOT_STARTED, "hipie_request_wait: nothing was started");
         DeviceGuard g(r->plan->device);
         if (timeout_ms < 0) {
+            // (the request stays busy while this blocks: a Cancel from another thread in the meantime is seen below)
+            const hipError_t e = hipStreamSynchronize(r->stream);
             r->started = false;
-            HIPIE_CHECK_HIP(hipStreamSynchronize(r->stream));
+            HIPIE_CHECK_HIP(e);
         } else {
             const auto deadline = std::chrono::steady_clock::now() + std::chrono::milliseconds(timeout_ms);
             for (;;) {
@@ -2907,10 +2916,7 @@ int hipie_request_wait_for(hipie_request* r, int64_t timeout_ms) {
             }
             r->started = false;
         }
-        if (r->cancelled) {
-            r->cancelled = false;
-            fail(HIPIE_INFER_CANCELLED, "the inference was cancelled");
-        }
+        if (r->cancelled.exchange(false)) fail(HIPIE_INFER_CANCELLED, "the inference was cancelled");
     });
 }
 

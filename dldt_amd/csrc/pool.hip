@@ -207,12 +207,15 @@ __global__ __launch_bounds__(256) void concat_channels_kernel(const ConcatArgs a
                                                               float inv_W, float inv_HW, int64_t total) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= total) return;
-    // idx -> (pixel, piece) -> (n, h, w): reciprocals with one correction step (the host keeps every quotient below 2^24)
+    // idx -> (pixel, piece) -> (n, h, w): float reciprocals give an estimate of each quotient (the host keeps every
+    // quotient below 2^24), the remainder corrects it exactly
     auto divmod = [](int64_t v, int32_t d, float inv, int32_t& q, int32_t& r) {
         q = static_cast<int32_t>(static_cast<float>(v) * inv);
         int64_t rem = v - static_cast<int64_t>(q) * d;
-        if (rem < 0) { --q; rem += d; }
-        else if (rem >= d) { ++q; rem -= d; }
+        // the dividend may exceed 2^24 (only the quotient is below it): its conversion, the reciprocal and the product
+        // each round, so the estimate can be off by a few units - corrected until the remainder is in range
+        while (rem < 0) { --q; rem += d; }
+        while (rem >= d) { ++q; rem -= d; }
         r = static_cast<int32_t>(rem);
     };
     int32_t pix, piece, n, hw, h, w;

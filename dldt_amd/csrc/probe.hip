@@ -5,7 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include "common.h"
-#include "hipie.h"
+#include "hipie_diag.h"
 
 namespace hipie {
 namespace {
@@ -34,10 +34,81 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(int iters, int* sink) {
     if (s == 0x7fffffff) sink[0] = s;       // keeps the products alive; not taken for these operands
 }
 
+// LDS read rate: every wave reads 1 KB per instruction (lane l the 16 bytes at 16 l of a 1 KB row: no bank conflict),
+// eight rows per iteration into eight register sets; with_mfma: four matrix instructions per four reads as well, the
+// mix of a 64 x 64 wave tile whose operands both come from LDS.  The first wave of the first workgroup reports the
+// core clocks its loop took.
+__global__ __launch_bounds__(256) void lds_rate_kernel(int iters, int with_mfma, long long* cycles, int* sink) {
+    __shared__ __attribute__((aligned(16))) int8_t buf[32768];
+    const int tid = threadIdx.x, lane = tid & 63;
+    for (int i = tid; i < 32768 / 16; i += 256) reinterpret_cast<v4i*>(buf)[i] = v4i{i, i + 1, i + 2, i + 3};
+    __syncthreads();
+    const int8_t* base = buf + (tid >> 6) * 8192 + lane * 16;
+    v4i r[8];
+    v16i acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[i][q] = 0;
+    int s = 0;
+    const long long t0 = clock64();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = *reinterpret_cast<const volatile v4i*>(base + i * 1024);
+        if (with_mfma) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i & 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(r[i], r[(i + 1) & 7], acc[i & 3], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s ^= r[i].x;
+        }
+    }
+    const long long t1 = clock64();
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) s += acc[i][q];
+    if (blockIdx.x == 0 && tid == 0) cycles[0] = t1 - t0;
+    if (s == 0x7fffffff) sink[0] = s;
+}
+
 }  // namespace
 }  // namespace hipie
 
 using namespace hipie;
+
+extern "C" int hipie_probe_lds_rate(int device, int iterations, int waves_per_simd, int with_mfma, double* bytes_per_clock_per_cu,
+                                    double* gigabytes_per_second) {
+    return guarded([&] {
+        HIPIE_REQUIRE(bytes_per_clock_per_cu && iterations > 0 && iterations <= (1 << 20) && waves_per_simd >= 1 && waves_per_simd <= 4,
+                      HIPIE_PARAMETER_MISMATCH, "hipie_probe_lds_rate: iterations %d, waves per SIMD %d", iterations, waves_per_simd);
+        DeviceGuard g(device);
+        hipDeviceProp_t prop;
+        HIPIE_CHECK_HIP(hipGetDeviceProperties(&prop, device));
+        long long* cycles = nullptr;
+        HIPIE_CHECK_HIP(hipMalloc(&cycles, 32));
+        int* sink = reinterpret_cast<int*>(cycles + 2);
+        const int blocks = prop.multiProcessorCount * waves_per_simd;      // four waves each: one per SIMD
+        hipEvent_t e0, e1;
+        HIPIE_CHECK_HIP(hipEventCreate(&e0));
+        HIPIE_CHECK_HIP(hipEventCreate(&e1));
+        hipLaunchKernelGGL(lds_rate_kernel, dim3(blocks), dim3(256), 0, nullptr, 16, with_mfma, cycles, sink);      // warm-up
+        HIPIE_CHECK_HIP(hipEventRecord(e0, nullptr));
+        hipLaunchKernelGGL(lds_rate_kernel, dim3(blocks), dim3(256), 0, nullptr, iterations, with_mfma, cycles, sink);
+        HIPIE_CHECK_HIP(hipEventRecord(e1, nullptr));
+        HIPIE_CHECK_HIP(hipEventSynchronize(e1));
+        float ms = 0.f;
+        HIPIE_CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+        long long host_cycles = 0;
+        HIPIE_CHECK_HIP(hipMemcpy(&host_cycles, cycles, sizeof host_cycles, hipMemcpyDeviceToHost));
+        HIPIE_CHECK_HIP(hipEventDestroy(e0));
+        HIPIE_CHECK_HIP(hipEventDestroy(e1));
+        HIPIE_CHECK_HIP(hipFree(cycles));
+        const double per_cu = 8.0 * 1024.0 * iterations * 4.0 * waves_per_simd;     // bytes read by the waves of one compute unit
+        *bytes_per_clock_per_cu = host_cycles > 0 ? per_cu / static_cast<double>(host_cycles) : 0.0;
+        if (gigabytes_per_second) *gigabytes_per_second = per_cu * prop.multiProcessorCount / (ms * 1e-3) / 1e9;
+    });
+}
 
 extern "C" int hipie_probe_mfma_rate(int device, int iterations, int waves_per_simd, double* tops, double* milliseconds) {
     return guarded([&] {

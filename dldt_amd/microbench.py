@@ -330,6 +330,22 @@ def vendor_gemm():
     return rows
 
 
+def lds_rate():
+    """LDS reads alone and mixed one to one with matrix instructions, 1 to 4 waves per SIMD (bytes per clock and compute
+    unit from a wave's own cycle counter; the GB/s column is the whole device by HIP events)"""
+    import ctypes
+    from ._lib import check, lib
+    rows = []
+    for with_mfma in (0, 1):
+        for waves in (1, 2, 4):
+            bpc, gbs = ctypes.c_double(), ctypes.c_double()
+            check(lib().hipie_probe_lds_rate(0, 20000, waves, with_mfma, ctypes.byref(bpc), ctypes.byref(gbs)))
+            what = "ds_read_b128 + one matrix instruction per read" if with_mfma else "ds_read_b128 alone"
+            rows.append({"row": "%s, %d wave(s) per SIMD: %.1f B/clk per compute unit" % (what, waves, bpc.value),
+                         "us": 0.0, "TOP/s": 0.0, "GB/s": gbs.value, "bound": "lds", "frac": bpc.value / 128.0})
+    return rows
+
+
 def mfma_rate():
     """the matrix pipe alone: every SIMD issuing int8 matrix instructions from registers, 1 to 4 waves per SIMD"""
     import ctypes
@@ -349,7 +365,7 @@ def main():
     import torch
     assert torch.cuda.is_available(), "microbench needs a GPU"
     which = sys.argv[1:] or ["1", "2", "3", "4", "5"]
-    table = {"1": config1, "2": config2, "3": config3, "4": config4, "5": config5, "encoder": config5_graph, "vendor": vendor_gemm, "mfma": mfma_rate}
+    table = {"1": config1, "2": config2, "3": config3, "4": config4, "5": config5, "encoder": config5_graph, "vendor": vendor_gemm, "mfma": mfma_rate, "lds": lds_rate}
     print("| kernel / graph | us | TOP/s | GB/s | bound | fraction of peak | notes |")
     print("|---|---|---|---|---|---|---|")
     for k in which:

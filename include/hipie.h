@@ -139,15 +139,6 @@ int hipie_fq_run_q8_tensor_u8(const hipie_fq* fq, const uint8_t* x, const hipie_
 float hipie_fq_host_eval(const hipie_fq* fq, int64_t channel, float x);
 /* 1 when the reciprocal path was proven equal to division on all boundaries of all channels */
 int hipie_fq_uses_reciprocal(const hipie_fq* fq);
-/* Constants of the convolution epilogue's two-operation division: for each divisor d[i] a pair with
- * fma(x, zh[i], x * zl[i]) == x / d[i] for every float x, checked on the device against IEEE division
- * over all 2^23 significands.  *verified = 1 when every divisor has a pair (otherwise the epilogue
- * keeps the reciprocal-with-corrections sequence and zh, zl are unspecified). */
-int hipie_fq_div2_constants(int device, const float* d, int64_t n, float* zh, float* zl, int* verified);
-/* Diagnostics, no counterpart in the reference: the int8 rate (TOP/s) the device sustains when every SIMD issues
- * v_mfma_i32_32x32x32_i8 back to back from registers (waves_per_simd waves of 4 x iterations independent instructions,
- * no memory traffic) - the ceiling a kernel's roofline fraction can be read against beside the published peak. */
-int hipie_probe_mfma_rate(int device, int iterations, int waves_per_simd, double* tops, double* milliseconds);
 
 /* ======================================================================================
  * 1b. Fused f32 epilogue applied to i32 accumulators, in this fixed order (each step one IEEE
@@ -236,43 +227,8 @@ int hipie_conv_create_fused(int device, const hipie_conv_desc* desc, const int8_
 void hipie_conv_destroy(hipie_conv* conv);
 /* output spatial dims for an input of h x w (convolution.hpp:168-183) */
 int hipie_conv_out_dims(const hipie_conv* conv, int32_t h, int32_t w, int32_t* oh, int32_t* ow);
-/* kernel variant: 0 = LDS-tiled 128 channels x 128 pixels, 1 = 64 x 256, 2 = 64 x 64, 3 = streaming
- * (weights resident in LDS), 4 / 5 = 128 x 128 / 64 x 256 with a multi-stage direct-to-LDS K pipeline,
- * 6 / 7 = the same two with eight waves that split the K steps between two wave groups (for layers
- * with fewer tiles than compute units; needs an even number of 64-byte K steps), 8 / 9 = 128 x 128 /
- * 64 x 256 persistent workgroups that prefetch the next pixel tile during the epilogue (small K; byte
- * outputs with a byte residual or none), 10 / 11 = 128 x 128 / 64 x 256 requesting the operands of two K
- * steps together (whole 128-byte lines per row), 12 = whole output rows of one image x 64 channels per
- * workgroup with the input patch and the nine weight slices staged once in LDS (3 x 3, stride 1, pad 1,
- * undilated, input channels a multiple of 64; rows too wide for a patch run variant 0), 13 = the same idea for
- * a first layer (4-byte pixels, filter rows of 5 to 8 taps, undilated: one 32-byte K slice per filter row; a
- * patch that would overhang the tensor's halo runs variant 1), 14 to 17 = variant 4 with the K steps of a tile
- * split over 2 / 4 / 8 / 16 workgroups (for launches with fewer tiles than compute units; at least two K steps per
- * part; launches of more than 2048 workgroups run variant 4).  The partial sums of variants 14 to 17 pass through a
- * workspace that the library keeps per (device, stream): it is allocated by the first such launch on a stream
- * (which therefore must not be under graph capture) and kept until the process ends.  18 to 22 = 128 x 128 tiles
- * whose K step is a whole cache line of every operand row, 23 = the few-pixel kernel (unpadded 1 x 1 over pixels of
- * a multiple of 64 bytes, raw sums or a bias / scale / ReLU tail to f32: a lane per output channel on the vector
- * pipe, K split over the waves of a workgroup; the FC layer of a classifier), 24 = whole output rows of one image x
- * all 64, 128 or 256 output channels per workgroup, the input patch (every channel) staged once in LDS and the
- * weights streamed through an LDS ring (3 x 3, stride 1, pad 1, undilated, dense pixels of a multiple of 64 channels,
- * bias + 256-level FakeQuantize from 0; rows too wide for a tile run variant 0).  A default is chosen
- * from the shape; hipie_compile times the variants on the device and keeps the fastest.  Every
- * variant produces the same bits.
- * A depthwise convolution (group_convolution.hpp:78-144 with one filter per channel) has two variants of its own:
- * 0 = every lane computes its outputs from registers loaded straight from memory, 1 = the input rows under seven
- * output rows of a strip of columns are staged once in LDS and a lane slides the 3 x 3 window over them in registers
- * (3 x 3, undilated, stride 1 or 2, pixels of at most 1024 bytes, FakeQuantize epilogue without residual). */
-int hipie_conv_set_tile(hipie_conv* conv, int tile);
-int hipie_conv_get_tile(const hipie_conv* conv, int* tile);
-/* diagnostics: the epilogue's step flags (conv_kernel.h ConvFlags) and whether a kernel instance with
- * these steps compiled in exists (otherwise the generic, slower instance runs) */
-int hipie_conv_epilogue_flags(const hipie_conv* conv, uint32_t* flags, int* specialised);
-/* ring depth of the pipelined variants: 3, 4, 6 or 8 K steps in LDS (other values round down, and to
- * what fits 144 KB); 0 = the variant's default (4 for tile 4, else 3).  Variant 24 and hipie_conv_run_pair (the
- * setting of its first layer): 6 and more = nine steps of weights in flight in a wave's registers and one workgroup
- * per compute unit (for a launch that runs alone), else three steps and two workgroups */
-int hipie_conv_set_stages(hipie_conv* conv, int stages);
+/* (the choice among the kernel variants that compute a layer - hipie_conv_set_tile and its companions - is in
+ * hipie_diag.h: hipie_compile makes it by measurement, a caller of the operator-level entry points may make it itself) */
 int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_tensor* residual,
                    const hipie_tensor* out, void* stream);
 /* Two consecutive convolutions in ONE kernel - the tail of a bottleneck block: `first` (3 x 3, stride 1, pad 1, bias,

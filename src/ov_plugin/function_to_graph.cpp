@@ -40,10 +40,29 @@ struct Translator {
     TranslatedGraph& out;
     std::unordered_map<const ngraph::Node*, int> id_of;
 
-    int in(const ngraph::Node& n, size_t i) const {
-        const auto it = id_of.find(n.get_input_node_ptr(i));
-        if (it == id_of.end()) IE_THROW(NotImplemented) << "HIP plugin: input " << i << " of " << n.get_friendly_name() << " was not translated";
-        return it->second;
+    // An i64 / u64 Constant is skipped when it is met (most are attributes their users read: axes, orders, target
+    // shapes).  One that a node takes as DATA - Gather indices, an integer table - is described here, on first use, as
+    // the i32 constant the engine's integer inputs are (values that do not fit are refused).
+    int in(const ngraph::Node& n, size_t i) {
+        const ngraph::Node* producer = n.get_input_node_ptr(i);
+        const auto it = id_of.find(producer);
+        if (it != id_of.end()) return it->second;
+        const auto c = ngraph::as_type_ptr<ngraph::opset1::Constant>(n.input_value(i).get_node_shared_ptr());
+        if (c && (c->get_element_type() == ngraph::element::i64 || c->get_element_type() == ngraph::element::u64)) {
+            const std::vector<int64_t> wide = c->cast_vector<int64_t>();
+            std::vector<int32_t> narrow(wide.size());
+            for (size_t k = 0; k < wide.size(); ++k) {
+                if (wide[k] < INT32_MIN || wide[k] > INT32_MAX)
+                    IE_THROW(NotImplemented) << "HIP plugin: 64-bit constant " << c->get_friendly_name() << " does not fit 32-bit integers";
+                narrow[k] = static_cast<int32_t>(wide[k]);
+            }
+            const auto d = as_i64(c->get_shape());
+            int id = -1;
+            check(hipie_graph_constant(g, HIPIE_I32, d.data(), static_cast<int>(d.size()), narrow.data(), &id), "hipie_graph_constant");
+            done(*c, id);
+            return id;
+        }
+        IE_THROW(NotImplemented) << "HIP plugin: input " << i << " of " << n.get_friendly_name() << " was not translated";
     }
     void done(const ngraph::Node& n, int id) {
         id_of[&n] = id;
@@ -166,7 +185,20 @@ TranslatedGraph translate(const std::shared_ptr<const ngraph::Function>& functio
                                     producer->get_output_element_type(0) == ngraph::element::u64);
             usable = attribute || t.id_of.count(producer) != 0;
         }
-        if (usable && t.node(node)) continue;
+        if (usable) {
+            // QueryNetwork (tolerate_unknown) wants a verdict per node, as the template plugin gives one
+            // (template_plugin.cpp:117-195): a node the helpers refuse - an element type, a dynamic shape, a 3-D
+            // convolution, an attribute that is not constant, a description hipie_graph_* rejects - is reported
+            // untranslated like a node of an unknown type, and so is everything that reads it
+            if (!tolerate_unknown) {
+                if (t.node(node)) continue;
+            } else {
+                try {
+                    if (t.node(node)) continue;
+                } catch (const InferenceEngine::Exception&) {
+                }
+            }
+        }
         if (!tolerate_unknown)
             IE_THROW(NotImplemented) << "HIP plugin: no kernel for node " << node->get_friendly_name() << " (" << node->get_type_name() << ")";
         out.untranslated.push_back(node->get_friendly_name());

@@ -173,7 +173,7 @@ def test_device_metrics():
     for name in ("AVAILABLE_DEVICES", "OPTIMIZATION_CAPABILITIES", "RANGE_FOR_ASYNC_INFER_REQUESTS", "IMPORT_EXPORT_SUPPORT",
                  "DEVICE_ARCHITECTURE", "SUPPORTED_CONFIG_KEYS"):
         assert name in names.split()
-    assert metric("OPTIMIZATION_CAPABILITIES") == (0, "INT8 FP32")
+    assert metric("OPTIMIZATION_CAPABILITIES") == (0, "INT8")       # no f32 convolution / MatMul path exists
     assert metric("IMPORT_EXPORT_SUPPORT") == (0, "YES")
     assert metric("DEVICE_ARCHITECTURE") == (0, "gfx950")
     assert metric("RANGE_FOR_ASYNC_INFER_REQUESTS")[1].split() == ["1", "8", "1"]
