@@ -2084,8 +2084,12 @@ struct Planner {
         st->in = x.tensor;
         int cur = id;
         int out_dtype = tensors[x.tensor].dtype;
-        if (st->avg) {
-            if (n.dtype != HIPIE_F32) unsupported(id, "AvgPool is planned with f32 output (not precision preserved)");
+        if (st->avg && n.dtype != HIPIE_F32) {
+            // precision preserved (LPT leaves the AvgPool on the quantized type when what reads it is quantized too,
+            // low_precision_transformations/src/avg_pool.cpp:36-45): the reference's integer instantiation
+            if (storage_type(n.dtype) != tensors[x.tensor].dtype) unsupported(id, "AvgPool whose result type is not its input's");
+            a.preserve = tensors[x.tensor].dtype == HIPIE_U8B ? 1 : 2;
+        } else if (st->avg) {
             out_dtype = HIPIE_F32;
             const int64_t C = n.shape[1];
             bool scaled = false;

@@ -16,6 +16,8 @@ struct PoolArgs {
     int32_t kh, kw, sh, sw, pt, pl, pb, pr;
     int32_t include_pad;
     int32_t in_bias;               // 128 for U8B storage, 0 for I8
+    int32_t preserve;              // AvgPool whose result has the input's type (precision preserved): 1 = u8 levels, 2 = i8;
+                                   // the window sum is kept modulo 256 as the reference's element-typed accumulator keeps it
     // AvgPool tail: optional Multiply and FakeQuantize tables, each [cs]
     const float* mul;
     const float* fq_il;

@@ -121,7 +121,19 @@ __global__ __launch_bounds__(kThreads) void avg_pool_nhwc_i8(PoolArgs a) {
         v[j] = x;
     }
     const int64_t o = static_cast<int64_t>(n) * a.out_sn + oh * a.out_sh + ow * a.out_sw + c;
-    if (a.fq_il) {
+    if (a.preserve) {
+        // avg_pool.hpp:236-262 for T = uint8_t / int8_t: T result (the sum wraps like the type), then
+        // static_cast<T>(nearbyint(float(result) / n)); stored as the tensor stores levels (u8: level - 128)
+        uint32_t packed = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int total = sum[j] + a.in_bias * cells;
+            const int r = a.preserve == 1 ? (total & 0xff) : static_cast<int>(static_cast<int8_t>(total & 0xff));
+            const int level = static_cast<int>(__builtin_rintf(static_cast<float>(r) / nf));
+            packed |= (static_cast<uint32_t>(level - (a.preserve == 1 ? 128 : 0)) & 0xffu) << (8 * j);
+        }
+        *reinterpret_cast<uint32_t*>(static_cast<int8_t*>(a.out) + o) = packed;
+    } else if (a.fq_il) {
         uint32_t packed = 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {

@@ -478,6 +478,38 @@ void orc_avg_pool_u8(const uint8_t* x, uint8_t* out, int64_t N, int64_t C, int64
     fesetround(old);
 }
 
+/* avg_pool.hpp:114-265, T = int8_t: as for uint8_t, the accumulator has the element type (the sum is kept modulo 256
+ * in two's complement), then static_cast<int8_t>(nearbyint(float(sum) / n)). */
+void orc_avg_pool_i8(const int8_t* x, int8_t* out, int64_t N, int64_t C, int64_t H, int64_t W,
+                     int64_t kh, int64_t kw, int64_t sh, int64_t sw, int64_t pbh, int64_t pbw,
+                     int64_t peh, int64_t pew, int64_t OH, int64_t OW, int include_pad) {
+    const int padding_present = pbh != 0 || pbw != 0 || peh != 0 || pew != 0;
+    int old = fegetround();
+    fesetround(FE_TONEAREST);
+    for (int64_t nc = 0; nc < N * C; ++nc)
+        for (int64_t oy = 0; oy < OH; ++oy)
+            for (int64_t ox = 0; ox < OW; ++ox) {
+                int64_t y0 = sh * oy, y1 = y0 + kh, x0 = sw * ox, x1 = x0 + kw;
+                if (y1 > H + pbh + peh) y1 = H + pbh + peh;
+                if (x1 > W + pbw + pew) x1 = W + pbw + pew;
+                int8_t r = 0;
+                size_t n = 0;
+                if (include_pad && padding_present) n = (size_t)(kh * kw);
+                for (int64_t y = y0; y < y1; ++y)
+                    for (int64_t xx = x0; xx < x1; ++xx) {
+                        int64_t iy = y - pbh, ix = xx - pbw;
+                        int in_bounds = !(iy < 0 || iy >= H || ix < 0 || ix >= W);
+                        if (in_bounds || include_pad) {
+                            int8_t v = in_bounds ? x[(nc * H + iy) * W + ix] : 0;
+                            r = (int8_t)(uint8_t)((uint8_t)r + (uint8_t)v);
+                            if (!padding_present || (in_bounds && !include_pad)) n++;
+                        }
+                    }
+                out[(nc * OH + oy) * OW + ox] = (int8_t)nearbyintf((float)r / n);
+            }
+    fesetround(old);
+}
+
 /* ---------------------------------------------------------------------------------------
  * fp32 glue: softmax.hpp (one axis: subtract max, exp, sum, divide), mvn.hpp (mvn_6:
  * mean, centre, mean of squares, sqrt(var + eps) or sqrt(var) + eps, divide), gelu.hpp

@@ -135,6 +135,7 @@ MAXPOOL_EXPORT(ref_max_pool_i32, int32_t)
     }
 AVGPOOL_EXPORT(ref_avg_pool_f32, float)
 AVGPOOL_EXPORT(ref_avg_pool_u8, uint8_t)
+AVGPOOL_EXPORT(ref_avg_pool_i8, int8_t)
 
 void ref_softmax_f32(const float* x, float* out, int64_t outer, int64_t axis, int64_t inner) {
     ref::softmax<float>(x, out, Shape{(size_t)outer, (size_t)axis, (size_t)inner}, AxisSet{1});

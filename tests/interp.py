@@ -75,7 +75,10 @@ def evaluate(orc, nodes, feeds, keep=None, override=None, targets=None):
         elif op == "AvgPool":
             oshape = orc.pool_out_shape(x[0].shape, n["kernel"], n["strides"], n["pads_begin"], n["pads_end"],
                                         n["ceil_mode"])
-            v = orc.avg_pool(x[0].astype(np.float32), n["kernel"], n["strides"], n["pads_begin"], n["pads_end"],
+            # f32 result: TypeRelaxed<AvgPool> over widened levels; u8 / i8 result (precision preserved): the reference's
+            # integer instantiation, whose accumulator has the element type (avg_pool.hpp:114-265)
+            src = x[0].astype(np.float32) if n["dtype"] == 10 else x[0]
+            v = orc.avg_pool(src, n["kernel"], n["strides"], n["pads_begin"], n["pads_end"],
                              not n["exclude_pad"], out_shape=oshape)
         elif op == "Reshape":
             v = x[0].reshape(n["shape"])

@@ -225,6 +225,9 @@ def test_avg_pool_vs_ref(orc, ref, include_pad):
         np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
         np.testing.assert_array_equal(orc.avg_pool(xu, k, s, pb, pe, include_pad),
                                       ref.avg_pool(xu, k, s, pb, pe, include_pad))
+        xi = (xu.astype(np.int16) - 128).astype(np.int8)      # (sums that leave the int8 range included: the reference keeps them modulo 256)
+        np.testing.assert_array_equal(orc.avg_pool(xi, k, s, pb, pe, include_pad),
+                                      ref.avg_pool(xi, k, s, pb, pe, include_pad))
 
 
 def test_fp32_glue_vs_ref(orc, ref):

@@ -30,7 +30,7 @@ def _pads(t):
     return pb, pe
 
 
-def _pool_graph(shape, signed, kind, kernel, strides, pb, pe, ceil, exclude_pad=True):
+def _pool_graph(shape, signed, kind, kernel, strides, pb, pe, ceil, exclude_pad=True, preserve=False):
     """Parameter f32 -> FakeQuantize to 8-bit levels (the identity on integer inputs) -> pool -> dequantization"""
     from dldt_amd.graph import Graph
     from dldt_amd.tensor import F32, I8, U8
@@ -44,8 +44,14 @@ def _pool_graph(shape, signed, kind, kernel, strides, pb, pe, ceil, exclude_pad=
     else:
         # after LPT the AvgPool reads the levels themselves and declares an f32 result (avg_pool.cpp:36-45 moves the
         # dequantization behind it)
-        p = g.avg_pool(q, kernel, strides, pb, pe, exclude_pad=exclude_pad, ceil_mode=ceil, out_dtype=F32)
-        y = p
+        if preserve:
+            # ... unless what reads the pool is quantized as well: then the AvgPool keeps the 8-bit type ("precision
+            # preserved") and the reference's integer instantiation rounds the mean to a level
+            p = g.avg_pool(q, kernel, strides, pb, pe, exclude_pad=exclude_pad, ceil_mode=ceil, out_dtype=I8 if signed else U8)
+            y = g.multiply(g.convert(p, F32), g.constant(np.float32(0.5).reshape(1, 1, 1, 1)))
+        else:
+            p = g.avg_pool(q, kernel, strides, pb, pe, exclude_pad=exclude_pad, ceil_mode=ceil, out_dtype=F32)
+            y = p
     g.result(y, "y")
     return g, p
 
@@ -131,6 +137,27 @@ def test_avg_pool_fuzz(orc, geo, exclude_pad, signed):
     g, _ = _pool_graph(shape, signed, "avg", kernel, strides, pb, pe, ceil, exclude_pad)
     got, want = _run(orc, g, x)
     np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("exclude_pad", [True, False])
+@pytest.mark.parametrize("geo", range(len(GEOMETRIES)))
+def test_precision_preserved_avg_pool(orc, geo, exclude_pad, signed):
+    """AvgPool with a u8 / i8 result (avg_pool.hpp for T = uint8_t / int8_t): nearbyint of the mean, ties to even, with
+    the window sum kept in the element type as the reference keeps it (small values in the first image: no sum wraps,
+    the result is the rounded mean; full-range values in the second: sums beyond the type wrap exactly alike)"""
+    kernel, strides, pb, pe, ceil = GEOMETRIES[geo]
+    rng = np.random.default_rng(300 + geo)
+    h, w = (7, 7) if kernel == (7, 7) else (13, 10)
+    shape = (2, 24, h, w)
+    lo, hi = (-128, 128) if signed else (0, 256)
+    x = rng.integers(lo, hi, shape).astype(np.float32)
+    small = 127 // (kernel[0] * kernel[1])
+    x[0] = rng.integers(-small if signed else 0, small + 1, shape[1:]).astype(np.float32)
+    g, p = _pool_graph(shape, signed, "avg", kernel, strides, pb, pe, ceil, exclude_pad, preserve=True)
+    got, want = _run(orc, g, x)
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert len(np.unique(got)) > 2
 
 
 def test_window_in_the_padding_alone_is_refused():
