@@ -10,6 +10,7 @@
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
+#include <map>
 #include <mutex>
 
 #include "fq.h"
@@ -133,7 +134,9 @@ struct Step {
     // exec-graph attributes (exec_graph_info.hpp:34-76), filled once the plan is complete: the graph nodes this step
     // stands for, the type it computes in (the CPU plugin reports its kernels' input type there: U8 / I8 for the
     // integer kernels) and the type and layout of what it stores
-    std::string original_names, runtime_precision, output_precision, output_layout;
+    std::string original_names, runtime_precision, output_precision, output_layout, output_dims;
+    std::vector<int> nodes;      // the graph nodes the step stands for (its own and every node fused into it)
+    std::vector<int> sources;    // where its operands come from: a step's index, or -(1 + k) for graph input k
     virtual ~Step() = default;
     virtual void create(int device, const std::vector<TensorInfo>& tensors) = 0;
     virtual void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs,
@@ -370,6 +373,9 @@ struct PairStep : Step {
         macs = first->macs + second->macs;
         out_node = second->out_node;
         original_names = first->original_names + "," + second->original_names;
+        nodes = first->nodes;
+        nodes.insert(nodes.end(), second->nodes.begin(), second->nodes.end());
+        output_dims = second->output_dims;
         runtime_precision = first->runtime_precision;
         output_precision = second->output_precision;
         output_layout = second->output_layout;
@@ -2392,7 +2398,9 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
             }
             std::sort(found.begin(), found.end());
             for (int v : found) s->original_names += (s->original_names.empty() ? "" : ",") + g->nodes[v].name;
+            s->nodes = found;
             const GNode& on = g->nodes[s->out_node];
+            for (size_t k = 0; k < on.shape.size(); ++k) s->output_dims += (k ? "," : "") + std::to_string(on.shape[k]);
             s->output_precision = type_name(on.dtype);
             s->output_layout = on.shape.size() == 4 ? "NHWC" : (on.shape.size() == 2 ? "NC" : (on.shape.size() == 3 ? "CHW" : "ANY"));
             // integer kernels compute in the type of the activations they read (through a symbolic dequantization
@@ -2442,6 +2450,38 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
             plan->steps.erase(plan->steps.begin() + static_cast<std::ptrdiff_t>(i));
             --i;
         }
+    {
+        // the edges of the executed graph (what GetExecGraphInfo draws): an operand of a step is a node outside its set -
+        // computed by another step, held by a tensor another step produced (a symbolic dequantization in between belongs
+        // to nobody), or a graph input
+        std::map<int, int> step_of_node, param_index;
+        for (size_t i = 0; i < plan->steps.size(); ++i)
+            for (int v : plan->steps[i]->nodes) step_of_node[v] = static_cast<int>(i);
+        for (size_t k = 0; k < g->params.size(); ++k) param_index[g->params[k]] = static_cast<int>(k);
+        for (size_t i = 0; i < plan->steps.size(); ++i) {
+            Step& st = *plan->steps[i];
+            std::vector<int> src;
+            for (int v : st.nodes) {
+                std::vector<int> pending(g->nodes[v].in.begin(), g->nodes[v].in.end());
+                while (!pending.empty()) {
+                    const int in = pending.back();
+                    pending.pop_back();
+                    if (in < 0 || g->nodes[in].op == OP_CONSTANT || std::binary_search(st.nodes.begin(), st.nodes.end(), in)) continue;
+                    int from = 0;
+                    bool known = true;
+                    const auto own = step_of_node.find(in);
+                    if (own != step_of_node.end() && own->second != static_cast<int>(i)) from = own->second;
+                    else if (param_index.count(in)) from = -(1 + param_index[in]);
+                    else if (own == step_of_node.end()) {   // a node no step owns (Convert / Subtract / Multiply over bytes, Reshape): look through it
+                        for (int up : g->nodes[in].in) pending.push_back(up);
+                        known = false;
+                    } else known = false;
+                    if (known && std::find(src.begin(), src.end(), from) == src.end()) src.push_back(from);
+                }
+            }
+            st.sources = src;
+        }
+    }
     for (size_t i = 0; i < pl.values.size(); ++i)
         if (pl.values[i].kind == VK_TENSOR) {
             plan->node_tensor[static_cast<int>(i)] = pl.values[i].tensor;
@@ -2785,8 +2825,20 @@ int hipie_plan_step_rt_info(const hipie_plan* p, int index, const char* key, cha
         else if (k == "execOrder") v = std::to_string(index);
         else if (k == "primitiveType") v = s.variant() >= 0 ? "hip_int8_v" + std::to_string(s.variant()) : "hip";
         else if (k == "kernels") v = std::to_string(s.launches());
+        else if (k == "outputDims") v = s.output_dims;
         else fail(HIPIE_NOT_FOUND, "hipie_plan_step_rt_info: key '%s' (execTimeMcs is hipie_request_perf)", key);
         copy_text(v, buf, cap, "hipie_plan_step_rt_info");
+    });
+}
+
+int hipie_plan_step_sources(const hipie_plan* p, int index, int* sources, int capacity, int* count) {
+    return guarded([&] {
+        HIPIE_REQUIRE(p && count && index >= 0 && index < static_cast<int>(p->steps.size()), HIPIE_OUT_OF_BOUNDS,
+                      "hipie_plan_step_sources: index %d", index);
+        const std::vector<int>& src = p->steps[index]->sources;
+        *count = static_cast<int>(src.size());
+        HIPIE_REQUIRE(sources || capacity == 0, HIPIE_PARAMETER_MISMATCH, "hipie_plan_step_sources: null array");
+        for (int i = 0; i < capacity && i < *count; ++i) sources[i] = src[static_cast<size_t>(i)];
     });
 }
 

@@ -207,6 +207,14 @@ class Plan:
             self.steps.append(dict(name=name.value.decode(errors="replace"), type=typ.value.decode(errors="replace"), macs=macs.value,
                                    bytes=byts.value, variant=var.value))
 
+    def step_sources(self, index):
+        """hipie_plan_step_sources: where the step's operands come from (step indices; -(1 + k) = graph input k)"""
+        n = ctypes.c_int()
+        check(lib().hipie_plan_step_sources(self._h, index, None, 0, ctypes.byref(n)))
+        buf = (ctypes.c_int * max(n.value, 1))()
+        check(lib().hipie_plan_step_sources(self._h, index, buf, n.value, ctypes.byref(n)))
+        return [buf[i] for i in range(n.value)]
+
     def step_rt_info(self, index, key):
         """an exec-graph attribute of one executed step (originalLayersNames, layerType, runtimePrecision,
         outputPrecisions, outputLayouts, execOrder, primitiveType)"""

@@ -498,8 +498,13 @@ int hipie_plan_step_variant(const hipie_plan* plan, int index, int* variant);
  * originalLayersNames (comma-separated graph nodes the step stands for), layerType, runtimePrecision (U8 / I8 for the
  * integer kernels: the type of the activations they multiply, as the CPU plugin reports it; FP32 otherwise),
  * outputPrecisions, outputLayouts, execOrder, primitiveType ("hip_int8_v<variant>" | "hip"); execTimeMcs is
- * hipie_request_perf.  HIPIE_NOT_FOUND for another key. */
+ * hipie_request_perf.  HIPIE_NOT_FOUND for another key.  Beside the reference's keys: "kernels" (launches the
+ * step enqueues) and "outputDims" (the shape of what it stores, comma separated, in the graph's dimension order). */
 int hipie_plan_step_rt_info(const hipie_plan* plan, int index, const char* key, char* buf, size_t buf_len);
+/* The edges of that graph: where the operands of step `index` come from - sources[i] >= 0 is the index of the step that
+ * produced one, sources[i] < 0 stands for graph input -(1 + sources[i]).  *count receives their number (at most
+ * `capacity` are written).  A step of layerType "Result" is what an output of the plan is read from. */
+int hipie_plan_step_sources(const hipie_plan* plan, int index, int* sources, int capacity, int* count);
 
 /* IExecutableNetworkInternal::CreateInferRequestImpl: own stream + own activation arena; weights
  * stay shared in the plan.  perf_count mirrors the PERF_COUNT config key (ie_plugin_config.hpp:277). */

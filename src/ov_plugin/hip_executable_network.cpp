@@ -1,8 +1,14 @@
 #include "hip_executable_network.hpp"
 
+#include <exec_graph_info.hpp>
 #include <ie_metric_helpers.hpp>
 #include <ie_plugin_config.hpp>
 #include <threading/ie_executor_manager.hpp>
+
+#include <ngraph/function.hpp>
+#include <ngraph/op/parameter.hpp>
+#include <ngraph/op/result.hpp>
+#include <ngraph/variant.hpp>
 
 #include <sstream>
 
@@ -135,6 +141,74 @@ InferenceEngine::Parameter ExecutableNetwork::GetMetric(const std::string& name)
 
 InferenceEngine::Parameter ExecutableNetwork::GetConfig(const std::string& name) const {
     return plan_text(false, name);
+}
+
+// The executed graph (ie_iexecutable_network_internal.hpp:87, exec_graph_info.hpp:34-76): one ExecutionNode per step of
+// the plan - a fused kernel - carrying the attributes of hipie_plan_step_rt_info under the reference's keys, wired by
+// hipie_plan_step_sources; graph inputs are Parameters, steps of layer type "Result" become Results.  The CPU plugin
+// builds its own the same way (mkldnn_plugin/mkldnn_graph_dumper.cpp:115-213).
+InferenceEngine::CNNNetwork ExecutableNetwork::GetExecGraphInfo() {
+    namespace info = ExecGraphInfoSerialization;
+    hipie_plan* plan = _plan.get();
+    auto text = [&](int step, const char* key) {
+        char buf[4096];
+        check(hipie_plan_step_rt_info(plan, step, key, buf, sizeof buf), key);
+        return std::string(buf);
+    };
+    auto precision_of = [](const std::string& p) {
+        if (p == "U8") return ngraph::element::u8;
+        if (p == "I8") return ngraph::element::i8;
+        if (p == "I32") return ngraph::element::i32;
+        return ngraph::element::f32;
+    };
+    auto dims_of = [](const std::string& csv) {
+        ngraph::Shape shape;
+        std::istringstream in(csv);
+        for (std::string d; std::getline(in, d, ',');) shape.push_back(static_cast<size_t>(std::stoull(d)));
+        return shape;
+    };
+    ngraph::ParameterVector params;
+    for (int i = 0; i < hipie_plan_num_inputs(plan); ++i) {
+        char name[256];
+        int dtype = 0, rank = 0;
+        int64_t dims[8];
+        check(hipie_plan_io_desc(plan, 0, i, name, sizeof name, &dtype, dims, &rank), "hipie_plan_io_desc");
+        const auto et = dtype == HIPIE_F32 ? ngraph::element::f32 : (dtype == HIPIE_I32 ? ngraph::element::i32 : ngraph::element::u8);
+        auto p = std::make_shared<ngraph::op::Parameter>(et, ngraph::Shape(dims, dims + rank));
+        p->set_friendly_name(name);
+        params.push_back(p);
+    }
+    ngraph::ResultVector results;
+    std::vector<std::shared_ptr<ngraph::Node>> nodes;
+    const int n_steps = hipie_plan_num_steps(plan);
+    for (int s = 0; s < n_steps; ++s) {
+        int count = 0;
+        check(hipie_plan_step_sources(plan, s, nullptr, 0, &count), "hipie_plan_step_sources");
+        std::vector<int> src(static_cast<size_t>(count));
+        if (count > 0) check(hipie_plan_step_sources(plan, s, src.data(), count, &count), "hipie_plan_step_sources");
+        ngraph::OutputVector inputs;
+        for (int from : src) inputs.push_back(from >= 0 ? nodes[static_cast<size_t>(from)]->output(0) : params[static_cast<size_t>(-1 - from)]->output(0));
+        char name[256], type[64];
+        int64_t macs = 0, bytes = 0;
+        check(hipie_plan_step_info(plan, s, name, sizeof name, type, sizeof type, &macs, &bytes), "hipie_plan_step_info");
+        std::shared_ptr<ngraph::Node> node;
+        if (std::string(type) == "Result" && !inputs.empty()) {
+            results.push_back(std::make_shared<ngraph::op::Result>(inputs.back()));
+            node = results.back();
+        } else {
+            node = std::make_shared<info::ExecutionNode>(inputs, 1);
+            node->set_output_type(0, precision_of(text(s, info::OUTPUT_PRECISIONS)), ngraph::PartialShape(dims_of(text(s, "outputDims"))));
+        }
+        for (const char* key : {info::ORIGINAL_NAMES, info::IMPL_TYPE, info::OUTPUT_PRECISIONS, info::OUTPUT_LAYOUTS, info::EXECUTION_ORDER,
+                                info::LAYER_TYPE, info::RUNTIME_PRECISION})
+            node->get_rt_info()[key] = std::make_shared<ngraph::VariantWrapper<std::string>>(text(s, key));
+        // (execTimeMcs belongs to a request's counters, GetPerformanceCounts; a plan that has not run reports none)
+        node->get_rt_info()[info::PERF_COUNTER] = std::make_shared<ngraph::VariantWrapper<std::string>>("not_executed");
+        node->set_friendly_name(name);
+        nodes.push_back(node);
+    }
+    if (results.empty()) IE_THROW() << "HIP plugin: the plan has no Result step";
+    return InferenceEngine::CNNNetwork(std::make_shared<ngraph::Function>(results, params, plan_text(true, EXEC_NETWORK_METRIC_KEY(NETWORK_NAME))));
 }
 
 void ExecutableNetwork::Export(std::ostream& model) {

@@ -20,6 +20,7 @@ public:
     InferenceEngine::Parameter GetMetric(const std::string& name) const override;
     InferenceEngine::Parameter GetConfig(const std::string& name) const override;
     void Export(std::ostream& model) override;
+    InferenceEngine::CNNNetwork GetExecGraphInfo() override;
 
     hipie_plan* plan() const { return _plan.get(); }
     int device() const { return _device; }

@@ -229,6 +229,13 @@ def test_exec_graph_attributes_per_step():
     # every graph node that computes is named by exactly one step
     named = [n for r in info for n in r["originalLayersNames"].split(",") if n]
     assert len(named) == len(set(named))
+    # the edges of the executed graph: the entry kernel reads graph input 0, everything else reads earlier steps; a
+    # bottleneck tail reads its 3 x 3 layer's input and the block input (the residual); every step but the Result is read
+    src = [plan.step_sources(i) for i in range(len(info))]
+    assert src[0] == [-1] and all(s and all(-1 <= v < i for v in s) for i, s in enumerate(src))
+    assert all(len(src[i]) == 2 for i, r in enumerate(info) if r["layerType"] == "Convolution,Convolution")
+    assert info[-1]["layerType"] == "Result" and set(range(len(info) - 1)) == {v for s in src for v in s if v >= 0}
+    assert plan.step_rt_info(1, "outputDims") == "1,64,112,112"
     with pytest.raises(HipieError) as e:
         plan.step_rt_info(0, "execTimeMcs")
     assert e.value.status == -5
