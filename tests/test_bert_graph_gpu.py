@@ -157,6 +157,35 @@ def test_encoder_with_embedding_front_end(orc, monkeypatch):
     np.testing.assert_array_equal(y.view(np.uint32), want["out"].view(np.uint32))
 
 
+def test_full_size_embedding_front_end_from_token_ids(orc, monkeypatch):
+    """Benchmark configuration 5 from its token ids: ids uniform in [0, 30522) for 16 sequences of 384 tokens, word table
+    [30522, 768] + position table + token-type row -> LayerNorm -> the first layer's quantized activations.  The lookup
+    and the sums are bit-exact, the normalisation within its tolerance, the i8 levels behind it equal to the reference
+    FakeQuantize of the device's own f32 values (one encoder layer: the other eleven repeat it and are covered by
+    test_encoder_full_size_first_and_last_layer)"""
+    from dldt_amd import builders
+    monkeypatch.setenv("HIPIE_KEEP_F32", "1")
+    B, S, H, V = 16, 384, 768, 30522
+    g, meta = builders.bert_encoder(layers=1, hidden=H, heads=12, ffn=3072, batch=B, seq=S, seed=21, vocab=V)
+    ids = np.random.default_rng(30522).integers(0, V, (B, S)).astype(np.int32)
+    assert ids.max() > V - 50 and ids.min() < 50
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps[:2]] == ["Gather", "MVN+FakeQuantize"]
+    assert plan.inputs[0]["name"] == "input_ids" and plan.inputs[0]["shape"] == (B, S)
+    req = plan.create_request()
+    req.infer(ids)
+    L = meta["layers"][0]
+    device = {n: req.matrix(n) for n in meta["glue"] if n == meta["embedding_norm"]}
+    _, kept = evaluate(orc, g.nodes, {"input_ids": ids}, keep=[meta["embeddings"], meta["embedding_norm"]],
+                       targets=[meta["embedding_norm"]])
+    emb = kept[meta["embeddings"]]
+    np.testing.assert_array_equal(req.matrix(meta["embeddings"]).reshape(emb.shape).view(np.uint32), emb.view(np.uint32))
+    w = kept[meta["embedding_norm"]]
+    np.testing.assert_allclose(device[meta["embedding_norm"]].reshape(w.shape), w, rtol=1e-5, atol=4e-6)
+    _, kept = evaluate(orc, g.nodes, {"input_ids": ids}, keep=[L["xq"]], override=device, targets=[L["xq"]])
+    np.testing.assert_array_equal(req.matrix(L["xq"]).reshape(kept[L["xq"]].shape).view(np.int8), kept[L["xq"]].astype(np.int8))
+
+
 def test_encoder_with_attention_mask(orc, monkeypatch):
     """additive mask [batch, 1, 1, seq] between the score Multiply and the Softmax: padded keys get no weight"""
     from dldt_amd import builders
