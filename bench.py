@@ -292,41 +292,11 @@ def main():
                                       "input_dtype": str(blobs[0][0][0].array.dtype)}
         del hreqs, blobs, plan8, g8
 
-    # per-step HIP events on the same stream: time spent in the int8 MFMA kernel
-    preq = plan.create_request(perf_count=True)
-    acc = {}
-    reps = max(3, min(10, args.steps))
-    for _ in range(2):
-        preq.infer_device(ins, outs)
-    for _ in range(reps):
-        preq.infer_device(ins, outs)
-        for i, st in enumerate(preq.perf()):
-            acc[i] = acc.get(i, 0.0) + st["ms"]
-    # An event between two kernels costs the stream about 2.7 us (the next dispatch waits for the event's
-    # signal): measured here with a small kernel launched back to back and then with an event in front of
-    # every launch, and taken off every step, so that a step's time is its kernel's duration (what a
-    # kernel trace of the same run shows).
-    pstream = torch.cuda.ExternalStream(preq.stream)
-    probe = torch.zeros(1 << 20, device="cuda")
-    with torch.cuda.stream(pstream):
-        n_probe = 50
-        for _ in range(5):
-            probe.add_(1)
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record(pstream)
-        for _ in range(n_probe):
-            probe.add_(1)
-        b.record(pstream)
-        evs = [torch.cuda.Event(enable_timing=True) for _ in range(n_probe + 1)]
-        for e in evs[:-1]:
-            e.record(pstream)
-            probe.add_(1)
-        evs[-1].record(pstream)
-        pstream.synchronize()
-        event_overhead_ms = max(0.0, (evs[0].elapsed_time(evs[-1]) - a.elapsed_time(b)) / n_probe)
-    # a step is one kernel, except a bottleneck tail that the load-time measurement left as two ("Convolution,Convolution")
-    steps = [dict(st, ms=max(acc[i] / reps - event_overhead_ms, 0.0), kernels=int(plan.step_rt_info(i, "kernels")))
-             for i, st in enumerate(plan.steps)]
+    # per-step HIP events on one request's stream, less the measured cost of an event between two kernels, so that a
+    # step's time is its kernels' duration (what a kernel trace of the same run shows).  A step is one kernel, except a
+    # bottleneck tail that the load-time measurement left as two ("Convolution,Convolution").
+    from dldt_amd.layers import attainable, step_times
+    steps, event_overhead_ms = step_times(plan, ins, outs, reps=max(3, min(10, args.steps)))
     MFMA_TYPES = ("Convolution", "Convolution+Shortcut", "Convolution+Convolution", "Convolution,Convolution", "MatMul")
     mfma = [s for s in steps if s["type"] in MFMA_TYPES]
     mfma_launches = sum(s["kernels"] for s in mfma)
@@ -355,13 +325,17 @@ def main():
         "frac_int8_peak_whole_net": total_ops / (ms_per_step * 1e-3) / 1e12 / INT8_PEAK_TOPS,
         "roofline": {"bound": "mfma", "achieved": achieved_tops, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s",
                      "frac": achieved_tops / INT8_PEAK_TOPS,
+                     "attainable_frac": attainable(mfma)["frac"], "attainable": attainable(mfma),
                      "traffic": profiled_traffic(args.batch)[0], "traffic_source": profiled_traffic(args.batch)[1],
                      "algorithmic_bytes_per_launch": sum(s["bytes"] for s in mfma) / mfma_launches,
                      "kernel": "conv_tiled_kernel / conv_pipe_kernel / conv_line_kernel / conv_block_kernel / conv_rows_kernel / conv_stem_kernel (all %d convolution/FC launches of one step)" % mfma_launches,
                      "ops_per_step": mfma_ops, "kernel_ms_per_step": mfma_ms,
                      "avg_launch_us": mfma_ms * 1e3 / mfma_launches, "event_overhead_us": event_overhead_ms * 1e3,
                      "note": "int8 TOP/s, dense peak 5.0 POP/s; launch durations by HIP events around every step on "
-                             "the request's stream, less the measured cost of an event between two kernels"},
+                             "the request's stream, less the measured cost of an event between two kernels.  attainable_frac: "
+                             "per step the largest of its matrix floor (ops / 5.0 POP/s), its vector floor (results x f32 "
+                             "instructions of the exact epilogue chain / 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz) and its memory "
+                             "floor (bytes / 8 TB/s), summed over the steps, over the summed measured durations"},
         "other_kernels_ms_per_step": {t: sum(s["ms"] for s in steps if s["type"] == t)
                                       for t in sorted({s["type"] for s in steps} - set(MFMA_TYPES))},
     }

@@ -8,6 +8,28 @@
 
 namespace hipie {
 
+// Packed convolution operands as the host produced them, in the order hipie_conv_create produced them.  A thread
+// that builds a plan installs a tape for a scope: recording keeps every packed matrix and correction vector; a tape
+// in playback hands them back to the same sequence of calls, which then upload instead of packing (a blob of another
+// size than the call expects means the tape belongs to other layers: HIPIE_NETWORK_NOT_READ).  Only values travel on
+// the tape, never offsets or sizes the kernels index with.
+struct PackTape {
+    std::vector<std::vector<uint8_t>> blobs;
+    size_t next = 0;
+    bool playing = false;
+    struct Scope {
+        explicit Scope(PackTape* t);
+        ~Scope();
+        Scope(const Scope&) = delete;
+        Scope& operator=(const Scope&) = delete;
+        PackTape* previous;
+    };
+    static PackTape* current();
+    bool take(void* dst, size_t bytes);          // playback: the next blob into dst; false when not playing
+    void give(const void* src, size_t bytes);    // recording: append; nothing while playing
+};
+
+
 // Per-channel epilogue tables on the device (padded to the packed channel count) + flags.
 struct Epilogue {
     int device = 0;

@@ -1325,19 +1325,18 @@ void Epilogue::build(int device_, const hipie_epilogue& e, int64_t oc, int64_t o
             out_off = ol;
         }
         std::vector<float> d(ocp), r(ocp);
-        std::atomic<bool> exact{true};
         for (int64_t c = 0; c < ocp; ++c) {
             HIPIE_REQUIRE(il[c] < ih[c], HIPIE_NOT_IMPLEMENTED,
                           "epilogue: FakeQuantize needs input_low < input_high (channel %lld)", (long long)c);
             d[c] = ih[c] - il[c];
         }
-        parallel_for(ocp, [&](int64_t c) {
-            FqChannel p{};
+        std::vector<FqChannel> ch(ocp);
+        for (int64_t c = 0; c < ocp; ++c) {
+            FqChannel& p = ch[c];
             p.il = il[c]; p.ih = ih[c]; p.lo = il[c]; p.hi = ih[c]; p.d = d[c];
-            p.r = fq_rounded_reciprocal(p.d);
-            r[c] = p.r;
-            if (!fq_reciprocal_exact_on_boundaries(p, lm1)) exact = false;
-        });
+            p.r = r[c] = fq_rounded_reciprocal(p.d);
+        }
+        const bool exact = fq_reciprocal_exact_on_all(ch.data(), ocp, lm1);
         up(fq_il, il); up(fq_ih, ih); up(fq_d, d); up(fq_r, r);
         flags |= CF_OUT_FQ;
         if (exact) flags |= CF_FQ_RCP;
@@ -1467,6 +1466,28 @@ struct hipie_matmul {
 // the zero point of input channel ic
 static inline int zero_point_of(const hipie_conv_desc& d, int ic) { return d.in_zero_points ? d.in_zero_points[ic] : d.in_zero_point; }
 
+namespace hipie {
+namespace {
+thread_local PackTape* t_tape = nullptr;
+}
+PackTape::Scope::Scope(PackTape* t) : previous(t_tape) { t_tape = t; }
+PackTape::Scope::~Scope() { t_tape = previous; }
+PackTape* PackTape::current() { return t_tape; }
+bool PackTape::take(void* dst, size_t bytes) {
+    if (!playing) return false;
+    HIPIE_REQUIRE(next < blobs.size() && blobs[next].size() == bytes, HIPIE_NETWORK_NOT_READ,
+                  "packed operands of the stream do not belong to this graph (blob %zu)", next);
+    std::memcpy(dst, blobs[next].data(), bytes);
+    ++next;
+    return true;
+}
+void PackTape::give(const void* src, size_t bytes) {
+    if (playing) return;
+    const uint8_t* b = static_cast<const uint8_t*>(src);
+    blobs.emplace_back(b, b + bytes);
+}
+}  // namespace hipie
+
 void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weights, std::vector<int8_t>* keep) {
     // K order (kh, kw, ic) over the padded channel stride.  A 16-byte piece must not straddle
     // two filter taps unless consecutive taps are contiguous in memory (in_stride_w == c stride).
@@ -1494,7 +1515,9 @@ void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weight
     std::vector<int8_t> w(static_cast<size_t>(OCp) * Kp, 0);
     std::vector<int32_t> cr(OCp, 0);
     const int stored_zero = d.in_dtype == HIPIE_U8B ? 128 : 0;
-    parallel_for(d.oc, [&](int64_t oc) {
+    PackTape* tape = PackTape::current();
+    const bool played = tape && tape->take(w.data(), w.size()) && tape->take(cr.data(), cr.size() * sizeof(int32_t));
+    if (!played) parallel_for(d.oc, [&](int64_t oc) {
         int64_t corr = 0;
         for (int kh = 0; kh < d.kh; ++kh)
             for (int kw = 0; kw < d.kw; ++kw)
@@ -1508,6 +1531,10 @@ void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weight
                 }
         cr[oc] = static_cast<int32_t>(corr - (d.acc_sub ? d.acc_sub[oc] : 0));
     });
+    if (tape && !played) {
+        tape->give(w.data(), w.size());
+        tape->give(cr.data(), cr.size() * sizeof(int32_t));
+    }
     if (device >= 0) {
         wgt.upload(device, w.data(), w.size());
         koff.upload(device, off.data(), off.size() * sizeof(int32_t));

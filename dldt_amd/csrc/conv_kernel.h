@@ -51,6 +51,37 @@ enum ConvFlags : uint32_t {
     CF_RES_GEMM = 1u << 15,   // residual = (float(acc2) + bias2[c]) * scale2[c] of a second GEMM run in the same kernel
 };
 
+// VALU instructions per output element of the epilogue's f32 chain (each of the graph's f32 operations is one
+// instruction here; a byte conversion or bytewise offset of a packed dword counts a quarter per element): what the
+// vector pipe has to issue for a layer's results whatever the kernel's shape.
+inline double epilogue_valu_ops(uint32_t f) {
+    if (f & CF_OUT_I32) return 0.0;
+    double n = 1.0;                                         // i32 -> f32 (the integer correction rides in the accumulator)
+    if (f & CF_BIAS) n += 1;
+    if (f & CF_SCALE) n += 1;
+    if (f & CF_RES) {
+        if (f & CF_RES_GEMM) n += 3;                        // the second accumulator: conversion, bias, scale
+        else if (!(f & CF_RES_F32)) n += (f & CF_RES_U8B) ? 1.25 : 1.0;
+        if (f & CF_RES_SUB) n += 1;
+        if (f & CF_RES_MUL) n += 1;
+        n += 1;                                             // the Add
+    }
+    if (f & CF_POST_SCALE) n += 1;
+    if (f & CF_RELU) n += 1;
+    if (f & CF_CLAMP) n += (f & CF_OUT_FQ) ? 1 : 2;
+    if (f & CF_GELU) n += 30;                               // erf by its polynomial
+    if (f & CF_OUT_FQ) {
+        if (!(f & CF_FQ_SAT)) n += 1;                       // median of three for the saturating branches
+        if (!(f & CF_FQ_IL0)) n += 1;                       // x - input_low
+        n += (f & CF_FQ_DIV2) ? 2 : ((f & CF_FQ_RCP) ? 5 : 10);
+        n += 2;                                             // * (levels - 1), rounding conversion into its byte
+        if (f & CF_OUT_XOR) n += 0.25;
+        if (f & CF_OUT_ADD) n += 1.25;
+    }
+    return n;
+}
+
+
 struct ConvArgs {
     const int8_t* in;     // element (n=0, h=0, w=0, c=0) of the input tensor
     const int8_t* wgt;    // packed [OCp][Kp]

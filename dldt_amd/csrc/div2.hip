@@ -10,6 +10,7 @@
 #include <map>
 
 #include "common.h"
+#include "fq.h"
 
 namespace hipie {
 namespace {
@@ -68,8 +69,27 @@ bool fq_div2_constants(int device, const std::vector<float>& d, std::vector<floa
         if (!std::isnormal(h) || !(l == 0.f || std::isnormal(l))) return false;   // l == 0: d is a power of two
     }
     DeviceGuard g(device);
-    std::vector<int> todo(n);
-    for (size_t i = 0; i < n; ++i) todo[i] = static_cast<int>(i);
+    // divisors the calling thread's table of earlier verdicts already answers need no run on the device
+    FqVerdicts* table = FqVerdicts::current();
+    auto bits_of = [](float v) {
+        uint32_t b;
+        std::memcpy(&b, &v, 4);
+        return b;
+    };
+    std::vector<int> todo;
+    for (size_t i = 0; i < n; ++i) {
+        if (table) {
+            const auto it = table->div2.find(bits_of(ud[i]));
+            if (it != table->div2.end()) {
+                if (!it->second.ok) return false;
+                uh[i] = it->second.zh;
+                ul[i] = it->second.zl;
+                continue;
+            }
+        }
+        todo.push_back(static_cast<int>(i));
+    }
+    const std::vector<int> asked = todo;
     // candidates: zh = RN(1/d) moved by hs units in the last place, zl = RN(1/d - zh) moved by ls
     static const int kShift[] = {0, 1, -1, 2, -2, 3, -3, 4, -4};
     DeviceBuffer bd, bh, bl, bf;
@@ -110,6 +130,10 @@ bool fq_div2_constants(int device, const std::vector<float>& d, std::vector<floa
             if (std::getenv("HIPIE_TUNE_LOG"))
                 std::fprintf(stderr, "hipie div2: %zu divisors, zh%+d zl%+d ulp: %zu unmatched\n", n, hs, ls, todo.size());
         }
+    }
+    if (table) {
+        for (int i : asked) table->div2[bits_of(ud[i])] = FqVerdicts::Div2{uh[i], ul[i], 1u};
+        for (int i : todo) table->div2[bits_of(ud[i])] = FqVerdicts::Div2{0.f, 0.f, 0u};
     }
     if (!todo.empty()) {
         if (std::getenv("HIPIE_TUNE_LOG"))

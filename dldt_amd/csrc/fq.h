@@ -1,6 +1,9 @@
 // FakeQuantize load-time checks shared with the convolution epilogue planner.
 #pragma once
+#include <array>
+#include <map>
 #include <memory>
+#include <vector>
 
 #include "common.h"
 #include "fq_math.h"
@@ -12,8 +15,31 @@ namespace hipie {
 // around every step of the reference means agreement everywhere between il and ih).
 bool fq_reciprocal_exact_on_boundaries(const FqChannel& p, float lm1);
 
+// The same for n channels at once: one check per distinct (il, ih, d, r), spread over the host's threads.
+// Returns true when every channel passes.
+bool fq_reciprocal_exact_on_all(const FqChannel* p, int64_t n, float lm1);
+
 // r = correctly rounded 1/d
 float fq_rounded_reciprocal(float d);
+
+// What the load-time checks found, keyed by the bits of their inputs: whether the reciprocal path gives the
+// reference's level on every boundary, and the two-operation division constants of a divisor (or that it has none).
+// Both are pure functions of their keys, so a table filled while one plan was built answers the same questions when
+// an exported plan is loaded again, without running the checks.  A thread that wants its checks recorded, or answered
+// from a table, installs one for a scope; the checks consult the calling thread's table only.
+struct FqVerdicts {
+    struct Div2 { float zh, zl; uint32_t ok; };
+    std::map<std::array<uint32_t, 5>, uint32_t> rcp;   // il, ih, d, r, levels - 1  ->  1 exact / 0 not
+    std::map<uint32_t, Div2> div2;                     // d  ->  verified pair, or ok = 0
+    struct Scope {
+        explicit Scope(FqVerdicts* v);
+        ~Scope();
+        Scope(const Scope&) = delete;
+        Scope& operator=(const Scope&) = delete;
+        FqVerdicts* previous;
+    };
+    static FqVerdicts* current();
+};
 
 // Elementwise nodes that no convolution / pooling / MatMul chain absorbs, on NHWC operands:
 //     out = FakeQuantize?( act?( op(a, b) ) ),  op in {none (unary), Add, Subtract, Multiply}, a and b in graph order.

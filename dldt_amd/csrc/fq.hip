@@ -418,7 +418,18 @@ float unordered(int32_t o) {
 
 }  // namespace
 
-bool fq_reciprocal_exact_on_boundaries(const FqChannel& p, float lm1) {
+namespace {
+
+thread_local FqVerdicts* t_verdicts = nullptr;
+
+std::array<uint32_t, 5> rcp_key(const FqChannel& p, float lm1) {
+    std::array<uint32_t, 5> k;
+    const float v[5] = {p.il, p.ih, p.d, p.r, lm1};
+    std::memcpy(k.data(), v, sizeof v);
+    return k;
+}
+
+bool check_boundaries(const FqChannel& p, float lm1) {
     if (!(p.il < p.ih)) return false;
     if (!(std::fabs(p.d) > 0x1p-60f && std::fabs(p.d) < 0x1p60f)) return false;
     uint32_t bits;
@@ -440,6 +451,42 @@ bool fq_reciprocal_exact_on_boundaries(const FqChannel& p, float lm1) {
         }
     }
     return true;
+}
+
+
+}  // namespace
+
+FqVerdicts::Scope::Scope(FqVerdicts* v) : previous(t_verdicts) { t_verdicts = v; }
+FqVerdicts::Scope::~Scope() { t_verdicts = previous; }
+FqVerdicts* FqVerdicts::current() { return t_verdicts; }
+
+bool fq_reciprocal_exact_on_boundaries(const FqChannel& p, float lm1) { return fq_reciprocal_exact_on_all(&p, 1, lm1); }
+
+bool fq_reciprocal_exact_on_all(const FqChannel* p, int64_t n, float lm1) {
+    FqVerdicts* table = t_verdicts;
+    std::map<std::array<uint32_t, 5>, uint32_t> local;
+    std::map<std::array<uint32_t, 5>, uint32_t>& known = table ? table->rcp : local;
+    std::vector<int64_t> open;                                  // first channel of every key not answered yet
+    {
+        std::map<std::array<uint32_t, 5>, int> asked;
+        for (int64_t c = 0; c < n; ++c) {
+            const auto key = rcp_key(p[c], lm1);
+            const auto it = known.find(key);
+            if (it != known.end()) {
+                if (!it->second) return false;
+            } else if (asked.emplace(key, 0).second) {
+                open.push_back(c);
+            }
+        }
+    }
+    std::vector<uint32_t> verdict(open.size());
+    parallel_for(static_cast<int64_t>(open.size()), [&](int64_t i) { verdict[i] = check_boundaries(p[open[i]], lm1) ? 1u : 0u; });
+    bool all = true;
+    for (size_t i = 0; i < open.size(); ++i) {
+        known[rcp_key(p[open[i]], lm1)] = verdict[i];
+        all = all && verdict[i];
+    }
+    return all;
 }
 
 }  // namespace hipie
@@ -669,11 +716,7 @@ int hipie_fq_create(int device, int64_t channels, int64_t levels, const float* i
             p.r = (p.d != 0.0f && std::isfinite(p.d)) ? fq_rounded_reciprocal(p.d) : 0.0f;
             if (!(p.il < p.ih)) fq->clamp_ok = false;
         }
-        std::atomic<bool> all_exact{true};
-        parallel_for(channels, [&](int64_t c) {
-            if (!fq_reciprocal_exact_on_boundaries(fq->host[c], fq->lm1)) all_exact = false;
-        });
-        fq->rcp = all_exact;
+        fq->rcp = fq_reciprocal_exact_on_all(fq->host.data(), channels, fq->lm1);
         // integer output forms: scalar out range whose op results are out_low + k exactly
         if (n_out_low == 1 && n_out_high == 1 && levels <= 256) {
             const float ol = out_low[0], oh = out_high[0];

@@ -149,6 +149,8 @@ struct Step {
     virtual int variant() const { return -1; }
     virtual void set_variant(int) {}
     virtual int launches() const { return 1; }   // kernels the step enqueues
+    // vector instructions x lanes the step's f32 chain needs per inference (results x epilogue_valu_ops); 0: not counted
+    virtual double valu_ops() const { return 0.0; }
 };
 
 void check_status(int st, const char* what) {
@@ -185,6 +187,7 @@ struct ConvStep : Step {
     std::vector<int32_t> zero_points;   // per input channel (a per-channel Subtract in front of the convolution), or empty
     std::vector<int32_t> acc_sub;       // per output channel (the Subtract behind a MatMul with a zero point), or empty
     hipie_conv* conv = nullptr;
+    int64_t results = 0;           // elements of the output tensor
     int64_t in_w_bytes = 0;        // input + weight bytes (what a fused consumer still has to read)
     // projection shortcut (Conv' -> Add -> Multiply, f32, used only by this step's residual Add):
     // run inside this step's kernel when the fused form applies, else right before it
@@ -253,6 +256,12 @@ struct ConvStep : Step {
         return r;
     }
     int launches() const override { return shortcut && !fused ? 2 : 1; }
+    double valu_ops() const override {
+        uint32_t flags = 0;
+        int specialised = 0;
+        if (!conv || hipie_conv_epilogue_flags(conv, &flags, &specialised) != HIPIE_OK) return 0.0;
+        return static_cast<double>(results) * epilogue_valu_ops(flags) + (shortcut && !fused ? shortcut->valu_ops() : 0.0);
+    }
     bool deep = false;             // variant 24 with nine steps of weights in flight (hipie_conv_set_stages)
     // kernel variant (hipie_conv_set_tile) + 32 for `deep`
     int variant() const override {
@@ -396,6 +405,7 @@ struct PairStep : Step {
         bytes = first->bytes + second->bytes - (fused ? 2 * mid_bytes : 0);
     }
     int launches() const override { return fused ? 1 : first->launches() + second->launches(); }
+    double valu_ops() const override { return first->valu_ops() + second->valu_ops(); }
     void run_fused(uint8_t* arena, const std::vector<TensorInfo>& tensors, hipStream_t s) const {
         const hipie_tensor i = tensors[first->in].desc(arena), o = tensors[second->out].desc(arena), r = tensors[second->res].desc(arena);
         check_status(hipie_conv_run_pair(first->conv, second->conv, &i, &r, &o, s), name.c_str());
@@ -501,16 +511,16 @@ struct PoolStep : Step {
             const auto il = expand(fq_il, 0.f), ih = expand(fq_ih, 1.f);
             std::vector<float> d(to.cs), r(to.cs);
             a.lm1 = static_cast<float>(static_cast<size_t>(levels - 1));
-            rcp = true;
+            std::vector<FqChannel> ch(to.cs);
             for (int c = 0; c < to.cs; ++c) {
                 HIPIE_REQUIRE(il[c] < ih[c], HIPIE_NOT_IMPLEMENTED, "%s: FakeQuantize needs low < high", name.c_str());
-                FqChannel p{};
+                FqChannel& p = ch[c];
                 p.il = il[c]; p.ih = ih[c]; p.lo = il[c]; p.hi = ih[c]; p.d = ih[c] - il[c];
                 p.r = fq_rounded_reciprocal(p.d);
                 d[c] = p.d;
                 r[c] = p.r;
-                if (!fq_reciprocal_exact_on_boundaries(p, a.lm1)) rcp = false;
             }
+            rcp = fq_reciprocal_exact_on_all(ch.data(), to.cs, a.lm1);
             HIPIE_REQUIRE(fq_ol == std::nearbyintf(fq_ol) && fq_oh == fq_ol + a.lm1, HIPIE_NOT_IMPLEMENTED,
                           "%s: output range is not consecutive integers", name.c_str());
             for (int k = 0; k < levels; ++k)
@@ -1512,6 +1522,7 @@ struct Planner {
         st->name = N(ch.cur).name + (group.size() > 1 ? " (+" + std::to_string(group.size() - 1) + " sharing the input)" : "");
         st->type = "MatMul";
         st->macs = T * OCt * IC;
+        st->results = T * OCt;
         st->in_w_bytes = T * IC + OCt * IC;
         st->bytes = st->in_w_bytes + T * OCt * (e.out_dtype == HIPIE_F32 ? 4 : 1) + (ch.residual ? T * OCt * 4 : 0);
         st->out_node = ch.cur;
@@ -2040,6 +2051,7 @@ struct Planner {
         st->name = N(cur).name;
         st->type = is_mm ? "MatMul" : (n.op == OP_GROUP_CONVOLUTION ? "GroupConvolution" : "Convolution");
         st->macs = N(id).numel() * (d.groups > 1 ? 1 : IC / grouped_macs_div) * d.kh * d.kw + (st->shortcut ? st->shortcut->macs : 0);
+        st->results = N(id).numel();
         // algorithmic HBM bytes: every operand once (input, weights, output, residual); a fused
         // projection shortcut adds its input and weights and removes the f32 residual round trip
         auto elems = [&](int t) {
@@ -2293,6 +2305,10 @@ struct hipie_plan {
     std::vector<Io> inputs, outputs;
     PlanConfig config;
     std::map<int, DeviceBuffer> fill_patterns;   // tensor -> cs bytes: what a pixel of its halo holds, channel by channel
+    // what building the steps computed on the host, kept for export: a plan loaded from a stream that holds them
+    // uploads the packed operands and takes the checks' verdicts instead of packing and checking again
+    FqVerdicts verdicts;
+    PackTape tape;
 };
 
 struct hipie_request {
@@ -2342,14 +2358,27 @@ void enqueue(hipie_request* r, void* const* in, void* const* out) {
 
 // `preset`: kernel variants of an imported plan, one per step; used when they fit the steps planned
 // here (same count, variants exactly where steps have them), else the plan is tuned like a new one
+struct PlanPrepared {       // the host work an exported plan carries (hipie_plan_import)
+    FqVerdicts verdicts;
+    PackTape tape;
+};
+
 std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const std::vector<int>* preset,
-                                         const PlanConfig& cfg = PlanConfig::from_environment()) {
+                                         const PlanConfig& cfg = PlanConfig::from_environment(), PlanPrepared* prepared = nullptr) {
     HIPIE_REQUIRE(!g->results.empty(), HIPIE_PARAMETER_MISMATCH, "hipie_compile: graph has no Result");
     HIPIE_REQUIRE(cfg.device_id < 0 || device < 0 || cfg.device_id == device, HIPIE_PARAMETER_MISMATCH,
                   "hipie_compile: DEVICE_ID %d against device %d", cfg.device_id, device);
     auto plan = std::make_unique<hipie_plan>();
     plan->device = device;
     plan->graph = *g;
+    if (prepared) {
+        plan->verdicts = std::move(prepared->verdicts);
+        plan->tape = std::move(prepared->tape);
+        plan->tape.playing = true;
+        plan->tape.next = 0;
+    }
+    FqVerdicts::Scope verdict_scope(&plan->verdicts);
+    PackTape::Scope tape_scope(&plan->tape);
     plan->config = cfg;
     plan->config.device_id = device;
     Planner pl(*g, cfg);
@@ -2377,6 +2406,8 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
             plan->fill_patterns[static_cast<int>(i)].upload(device, pattern.data(), pattern.size());
         }
     for (auto& s : pl.steps) s->create(device, plan->tensors);
+    HIPIE_REQUIRE(!plan->tape.playing || plan->tape.next == plan->tape.blobs.size(), HIPIE_NETWORK_NOT_READ,
+                  "hipie_plan_import: %zu packed operands in the stream, %zu used", plan->tape.blobs.size(), plan->tape.next);
     plan->steps = std::move(pl.steps);
     {
         auto type_name = [](int dt) {
@@ -2572,7 +2603,7 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
 }
 
 constexpr char kPlanMagic[8] = {'H', 'I', 'P', 'I', 'E', 'P', 'L', 'N'};
-constexpr uint32_t kPlanFormat = 1;
+constexpr uint32_t kPlanFormat = 2;
 
 uint64_t fnv1a(const uint8_t* p, size_t n) {
     uint64_t h = 1469598103934665603ull;
@@ -2717,14 +2748,18 @@ int hipie_plan_get_config(const hipie_plan* p, const char* key, char* buf, size_
     });
 }
 
-/* stream layout: magic[8], format u32, step count u32, one i32 kernel variant per step, graph bytes
- * u64 + the graph description, FNV-1a of everything before it u64 */
+/* stream layout: magic[8], format u32, step count u32, one i32 kernel variant per step, graph bytes u64 + the graph
+ * description, the load-time checks' verdicts (count u64 + 6 u32 each: il, ih, d, r, levels - 1, exact; count u64 +
+ * 4 u32 each: d, zh, zl, verified), the packed operands (count u64, then byte count u64 + bytes each), FNV-1a of
+ * everything before it u64 */
 int hipie_plan_export(const hipie_plan* p, void* buffer, size_t capacity, size_t* size) {
     return guarded([&] {
         HIPIE_REQUIRE(p && size, HIPIE_PARAMETER_MISMATCH, "hipie_plan_export: null argument");
         const size_t head = 16 + 4 * p->steps.size();
         const size_t graph_bytes = serialize_graph(p->graph, nullptr);
-        *size = head + 8 + graph_bytes + 8;
+        size_t prepared = 8 + 24 * p->verdicts.rcp.size() + 8 + 16 * p->verdicts.div2.size() + 8;
+        for (const auto& blob : p->tape.blobs) prepared += 8 + blob.size();
+        *size = head + 8 + graph_bytes + prepared + 8;
         if (!buffer) return;                              // size query
         HIPIE_REQUIRE(capacity >= *size, HIPIE_OUT_OF_BOUNDS, "hipie_plan_export: %zu bytes needed, %zu given", *size, capacity);
         uint8_t* b = static_cast<uint8_t*>(buffer);
@@ -2739,6 +2774,29 @@ int hipie_plan_export(const hipie_plan* p, void* buffer, size_t capacity, size_t
         const uint64_t gb = graph_bytes;
         std::memcpy(b + head, &gb, 8);
         serialize_graph(p->graph, b + head + 8);
+        uint8_t* w = b + head + 8 + graph_bytes;
+        auto put = [&](const void* src, size_t n) {
+            std::memcpy(w, src, n);
+            w += n;
+        };
+        auto put64 = [&](uint64_t v) { put(&v, 8); };
+        put64(p->verdicts.rcp.size());
+        for (const auto& kv : p->verdicts.rcp) {
+            put(kv.first.data(), 20);
+            put(&kv.second, 4);
+        }
+        put64(p->verdicts.div2.size());
+        for (const auto& kv : p->verdicts.div2) {
+            put(&kv.first, 4);
+            put(&kv.second.zh, 4);
+            put(&kv.second.zl, 4);
+            put(&kv.second.ok, 4);
+        }
+        put64(p->tape.blobs.size());
+        for (const auto& blob : p->tape.blobs) {
+            put64(blob.size());
+            put(blob.data(), blob.size());
+        }
         const uint64_t h = fnv1a(b, *size - 8);
         std::memcpy(b + *size - 8, &h, 8);
     });
@@ -2748,7 +2806,7 @@ int hipie_plan_import(const void* blob, size_t size, int device, hipie_plan** ou
     return guarded([&] {
         HIPIE_REQUIRE(blob && out, HIPIE_PARAMETER_MISMATCH, "hipie_plan_import: null argument");
         const uint8_t* b = static_cast<const uint8_t*>(blob);
-        HIPIE_REQUIRE(size >= 8 + 4 + 4 + 8 + 8 && std::memcmp(b, kPlanMagic, 8) == 0, HIPIE_NETWORK_NOT_READ,
+        HIPIE_REQUIRE(size >= 8 + 4 + 4 + 8 + 24 + 8 && std::memcmp(b, kPlanMagic, 8) == 0, HIPIE_NETWORK_NOT_READ,
                       "hipie_plan_import: not an exported plan");
         uint32_t fmt, ns;
         std::memcpy(&fmt, b + 8, 4);
@@ -2757,7 +2815,7 @@ int hipie_plan_import(const void* blob, size_t size, int device, hipie_plan** ou
         uint64_t stored;
         std::memcpy(&stored, b + size - 8, 8);
         HIPIE_REQUIRE(stored == fnv1a(b, size - 8), HIPIE_NETWORK_NOT_READ, "hipie_plan_import: checksum mismatch (damaged stream)");
-        HIPIE_REQUIRE(ns <= (size - 32) / 4, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: %u steps in %zu bytes", ns, size);
+        HIPIE_REQUIRE(ns <= (size - 56) / 4, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: %u steps in %zu bytes", ns, size);
         std::vector<int> variants(ns);
         for (uint32_t i = 0; i < ns; ++i) {
             int32_t v;
@@ -2765,12 +2823,59 @@ int hipie_plan_import(const void* blob, size_t size, int device, hipie_plan** ou
             variants[i] = v;
         }
         const size_t at = 16 + 4 * size_t(ns);
+        const uint8_t* const end = b + size - 8;            // the checksum follows
         uint64_t gb;
         std::memcpy(&gb, b + at, 8);
-        HIPIE_REQUIRE(gb == size - at - 16, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: graph description of %llu bytes in a stream of %zu",
+        HIPIE_REQUIRE(gb <= size - at - 8 - 24 - 8, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: graph description of %llu bytes in a stream of %zu",
                       (unsigned long long)gb, size);
         std::unique_ptr<hipie_graph> g(deserialize_graph(b + at + 8, static_cast<size_t>(gb)));
-        *out = compile_plan(g.get(), device, &variants).release();
+        const uint8_t* r = b + at + 8 + gb;
+        auto need = [&](uint64_t n, const char* what) {
+            HIPIE_REQUIRE(n <= static_cast<uint64_t>(end - r), HIPIE_NETWORK_NOT_READ, "hipie_plan_import: the stream ends inside its %s", what);
+        };
+        auto get64 = [&](const char* what) {
+            need(8, what);
+            uint64_t v;
+            std::memcpy(&v, r, 8);
+            r += 8;
+            return v;
+        };
+        PlanPrepared prepared;
+        const uint64_t n_rcp = get64("verdicts");
+        HIPIE_REQUIRE(n_rcp <= static_cast<uint64_t>(end - r) / 24, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: %llu verdicts", (unsigned long long)n_rcp);
+        for (uint64_t i = 0; i < n_rcp; ++i) {
+            std::array<uint32_t, 5> key;
+            uint32_t exact;
+            std::memcpy(key.data(), r, 20);
+            std::memcpy(&exact, r + 20, 4);
+            r += 24;
+            HIPIE_REQUIRE(exact <= 1, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: verdict %u", exact);
+            prepared.verdicts.rcp[key] = exact;
+        }
+        const uint64_t n_div2 = get64("division constants");
+        HIPIE_REQUIRE(n_div2 <= static_cast<uint64_t>(end - r) / 16, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: %llu divisors", (unsigned long long)n_div2);
+        for (uint64_t i = 0; i < n_div2; ++i) {
+            uint32_t key;
+            FqVerdicts::Div2 v;
+            std::memcpy(&key, r, 4);
+            std::memcpy(&v.zh, r + 4, 4);
+            std::memcpy(&v.zl, r + 8, 4);
+            std::memcpy(&v.ok, r + 12, 4);
+            r += 16;
+            HIPIE_REQUIRE(v.ok <= 1, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: verdict %u", v.ok);
+            prepared.verdicts.div2[key] = v;
+        }
+        const uint64_t n_blobs = get64("packed operands");
+        HIPIE_REQUIRE(n_blobs <= static_cast<uint64_t>(end - r) / 8, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: %llu packed operands", (unsigned long long)n_blobs);
+        prepared.tape.blobs.reserve(static_cast<size_t>(n_blobs));
+        for (uint64_t i = 0; i < n_blobs; ++i) {
+            const uint64_t n = get64("packed operands");
+            need(n, "packed operands");
+            prepared.tape.blobs.emplace_back(r, r + n);
+            r += n;
+        }
+        HIPIE_REQUIRE(r == end, HIPIE_NETWORK_NOT_READ, "hipie_plan_import: %zu bytes behind the packed operands", static_cast<size_t>(end - r));
+        *out = compile_plan(g.get(), device, &variants, PlanConfig::from_environment(), &prepared).release();
     });
 }
 
@@ -2825,6 +2930,7 @@ int hipie_plan_step_rt_info(const hipie_plan* p, int index, const char* key, cha
         else if (k == "execOrder") v = std::to_string(index);
         else if (k == "primitiveType") v = s.variant() >= 0 ? "hip_int8_v" + std::to_string(s.variant()) : "hip";
         else if (k == "kernels") v = std::to_string(s.launches());
+        else if (k == "valuOps") v = std::to_string(static_cast<long long>(s.valu_ops()));
         else if (k == "outputDims") v = s.output_dims;
         else fail(HIPIE_NOT_FOUND, "hipie_plan_step_rt_info: key '%s' (execTimeMcs is hipie_request_perf)", key);
         copy_text(v, buf, cap, "hipie_plan_step_rt_info");

@@ -331,8 +331,8 @@ def vendor_gemm():
 
 
 def lds_rate():
-    """LDS reads alone and mixed one to one with matrix instructions, 1 to 4 waves per SIMD (bytes per clock and compute
-    unit from a wave's own cycle counter; the GB/s column is the whole device by HIP events)"""
+    """LDS reads alone and mixed one to one with matrix instructions, 1 to 4 waves per SIMD (the GB/s column is the whole
+    device by HIP events; bytes per clock and compute unit divide it by the core clock a wave measured meanwhile)"""
     import ctypes
     from ._lib import check, lib
     rows = []
@@ -342,7 +342,8 @@ def lds_rate():
             check(lib().hipie_probe_lds_rate(0, 20000, waves, with_mfma, ctypes.byref(bpc), ctypes.byref(gbs)))
             what = "ds_read_b128 + one matrix instruction per read" if with_mfma else "ds_read_b128 alone"
             rows.append({"row": "%s, %d wave(s) per SIMD: %.1f B/clk per compute unit" % (what, waves, bpc.value),
-                         "us": 0.0, "TOP/s": 0.0, "GB/s": gbs.value, "bound": "lds", "frac": bpc.value / 128.0})
+                         "us": 0.0, "TOP/s": gbs.value * 64e-6 * 1e3 if with_mfma else 0.0, "GB/s": gbs.value, "bound": "lds",
+                         "frac": bpc.value / 128.0})
     return rows
 
 

@@ -62,9 +62,11 @@ int hipie_fq_div2_constants(int device, const float* d, int64_t n, float* zh, fl
  * no memory traffic) - the ceiling a kernel's roofline fraction can be read against beside the published peak. */
 int hipie_probe_mfma_rate(int device, int iterations, int waves_per_simd, double* tops, double* milliseconds);
 /* The LDS read rate the device sustains: waves_per_simd (1 .. 4) waves on every SIMD read 1 KB per ds_read_b128 from
- * conflict-free rows, eight reads per iteration; with_mfma = 1 adds one v_mfma_i32_32x32x32_i8 per read (the mix of a
- * 64 x 64 wave tile fed from LDS on both sides).  bytes_per_clock_per_cu is taken from a wave's own cycle counter,
- * gigabytes_per_second (may be NULL) from HIP events over the whole device. */
+ * conflict-free rows, eight reads per iteration (an even count), issued a step ahead of their use; with_mfma = 1 runs
+ * one v_mfma_i32_32x32x32_i8 per read meanwhile (the mix of a 64 x 64 wave tile fed from LDS on both sides).
+ * gigabytes_per_second (may be NULL) is the whole device by HIP events; bytes_per_clock_per_cu divides it by the
+ * compute units and by the core clock a wave measured during the launch (its cycle counter against the constant
+ * 100 MHz clock). */
 int hipie_probe_lds_rate(int device, int iterations, int waves_per_simd, int with_mfma, double* bytes_per_clock_per_cu,
                          double* gigabytes_per_second);
 

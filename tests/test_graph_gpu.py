@@ -249,6 +249,29 @@ def test_activation_zero_points(orc):
     np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))
 
 
+def test_imported_plan_uploads_the_packed_operands_of_the_stream(orc):
+    """Import does not pack weights again: it uploads what the stream holds.  Shown by a stream whose first packed
+    matrix was replaced by zeros (and sealed again): the graph description still holds the weights, the imported plan
+    computes with the zeros."""
+    from dldt_amd import builders
+    from dldt_amd.graph import Plan
+    from test_plan_stream_cpu import _reseal, sections
+    g = builders.conv_block(n=2, c=32, hw=12, oc=32)[0]
+    x = np.random.default_rng(5).uniform(0, 2.55, (2, 32, 12, 12)).astype(np.float32)
+    names = [n["name"] for n in g.nodes if n["op"] == "Parameter"]
+    ref, _ = evaluate(orc, g.nodes, {names[0]: x})
+    plan = g.compile()
+    blob = plan.export()
+    want = plan.create_request().infer(x)[0]
+    np.testing.assert_array_equal(want.view(np.uint32), ref[plan.outputs[0]["name"]].view(np.uint32))
+    np.testing.assert_array_equal(Plan.load(blob).create_request().infer(x)[0], want)
+    _, _, _, blobs = sections(blob)
+    off, n = max(blobs, key=lambda b: b[1])              # the packed weight matrix
+    zeroed = _reseal(blob[:off] + bytes(n) + blob[off + n:-8])
+    got = Plan.load(zeroed).create_request().infer(x)[0]
+    assert not np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("net", ["resnet", "encoder"])
 def test_exported_plan_runs_the_same_kernels(orc, net, monkeypatch):
     """ExecutableNetwork::Export -> Plugin::ImportNetwork: the imported plan takes its kernel variants from

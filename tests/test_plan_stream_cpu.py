@@ -21,6 +21,29 @@ def _reseal(body):
     return body + struct.pack("<Q", _fnv1a(body))
 
 
+def sections(blob):
+    """offsets inside an exported stream: (graph start, graph bytes, [(key offset of every reciprocal verdict)],
+    [(offset, size) of every packed operand])"""
+    n_steps = struct.unpack("<I", blob[12:16])[0]
+    at = 16 + 4 * n_steps
+    gb = struct.unpack("<Q", blob[at:at + 8])[0]
+    r = at + 8 + gb
+    n_rcp = struct.unpack("<Q", blob[r:r + 8])[0]
+    rcp = [r + 8 + 24 * i for i in range(n_rcp)]
+    r += 8 + 24 * n_rcp
+    n_div2 = struct.unpack("<Q", blob[r:r + 8])[0]
+    r += 8 + 16 * n_div2
+    n_blobs = struct.unpack("<Q", blob[r:r + 8])[0]
+    r += 8
+    blobs = []
+    for _ in range(n_blobs):
+        n = struct.unpack("<Q", blob[r:r + 8])[0]
+        blobs.append((r + 8, n))
+        r += 8 + n
+    assert r == len(blob) - 8
+    return at + 8, gb, rcp, blobs
+
+
 def _summary(plan):
     return [(s["name"], s["type"], s["macs"], s["bytes"]) for s in plan.steps], plan.inputs, plan.outputs, plan.arena_bytes
 
@@ -63,16 +86,40 @@ def test_refused_streams():
         assert e.value.status == -12, what
 
 
+def test_prepared_sections_are_validated():
+    """behind the graph: the load-time checks' verdicts and the packed operands.  What is not a verdict, ends early or
+    does not fit the layers of the graph is refused."""
+    blob = builders.conv_block()[0].compile(-1).export()
+    start, gb, rcp, blobs = sections(blob)
+    assert rcp and len(blobs) >= 2                       # a convolution: the packed matrix and its correction vector
+    off, n = blobs[0]
+    cases = {
+        "verdict that is no 0 / 1": blob[:rcp[0] + 20] + struct.pack("<I", 7) + blob[rcp[0] + 24:-8],
+        "operand of another size": blob[:off - 8] + struct.pack("<Q", n - 64) + blob[off:off + n - 64] + blob[off + n:-8],
+    }
+    count_at = blobs[0][0] - 16
+    cases["operand count beyond the stream"] = blob[:count_at] + struct.pack("<Q", 1 << 40) + blob[count_at + 8:-8]
+    # one operand fewer than the layers ask for
+    last_off, last_n = blobs[-1]
+    cases["operand missing"] = blob[:count_at] + struct.pack("<Q", len(blobs) - 1) + blob[count_at + 8:last_off - 8]
+    # one more than they use
+    cases["operand too many"] = blob[:count_at] + struct.pack("<Q", len(blobs) + 1) + blob[count_at + 8:-8] + struct.pack("<Q", 4) + b"abcd"
+    for what, body in cases.items():
+        with pytest.raises(HipieError) as e:
+            Plan.load(_reseal(body), -1)
+        assert e.value.status == -12, what
+
+
 def test_damaged_streams_with_a_valid_checksum_never_get_past_validation():
     """the checksum only catches accidents; behind it every field is checked again: random damage inside
     the graph description either still describes a valid graph or is refused with a status, never worse"""
     blob = builders.conv_block(n=1, c=16, hw=8, oc=16)[0].compile(-1).export()
     body = bytearray(blob[:-8])
-    n_steps = struct.unpack("<I", blob[12:16])[0]
-    start = 16 + 4 * n_steps + 8
+    start, gb, _, _ = sections(blob)
     rng = np.random.default_rng(1)
     # the structured part of the description (node headers) is where damage matters; constants are payload
-    offsets = [int(o) for o in rng.integers(start, len(body), 150)] + list(range(start, start + 120))
+    offsets = ([int(o) for o in rng.integers(start, start + gb, 150)] + list(range(start, start + 120)) +
+               [int(o) for o in rng.integers(start + gb, len(body), 80)])
     refused = loaded = 0
     for o in offsets:
         bad = bytearray(body)
