@@ -23,8 +23,8 @@ FLAGS = [
 ] + os.environ.get("HIPIE_EXTRA_FLAGS", "").split()
 
 
-# per-file additions: the bottleneck-tail kernel runs one or two waves per SIMD, where a wave's own instruction-level
-# parallelism is what hides latency - the scheduler is told to order for that instead of for registers
+# per-file additions from the environment (HIPIE_BLOCK_FLAGS="-DHIPIE_BLOCK_STAMPS" builds the bottleneck-tail kernel
+# with its cycle stamps; the library that ships is built without any)
 EXTRA = {"conv_block.hip": os.environ.get("HIPIE_BLOCK_FLAGS", "").split()}
 
 
