@@ -60,11 +60,15 @@ struct BlockGeometry {
     bool ok;
     int nwc, rows, tiles_per_image, patch_w, csa, ppix;
     size_t lds;
+    bool ok2;        // the fused form with two wave groups takes the layer too, with lds2 bytes of LDS
+    size_t lds2;
 };
 BlockGeometry block_geometry(int oc_a, int ic_a, int oh, int ow);
 bool block_epilogues_fit(uint32_t flags_a, bool fused, uint32_t flags_b);
-// deep: nine instead of three steps of weights in flight per wave, one workgroup per compute unit instead of two
-void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo, int images, bool deep, hipStream_t s);
+// form 0: three steps of weights in flight per wave, two workgroups per compute unit; 1: nine steps, one workgroup;
+// 2 (with b, where geo.ok2): eight waves in two groups that split the first layer's input slabs and take the second
+// layer's passes in turn
+void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo, int images, int form, hipStream_t s);
 
 // depthwise kernels (dwconv.hip).  variant 0: a lane computes its outputs from registers loaded straight from memory;
 // variant 1: 3 x 3 through an LDS patch with the window sliding in registers (dwconv_strip_fits says which layers)

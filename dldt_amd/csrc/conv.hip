@@ -2192,7 +2192,7 @@ static int conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_ten
             } else {
                 DeviceGuard g(c->device);
                 a.wgt = c->wgt_steps.as<int8_t>();
-                launch_block(a, nullptr, geo, in->n, c->stages >= 6, as_stream(stream));
+                launch_block(a, nullptr, geo, in->n, c->stages >= 6 ? 1 : 0, as_stream(stream));
                 HIPIE_CHECK_HIP(hipGetLastError());
                 return;
             }
@@ -2292,7 +2292,9 @@ int hipie_conv_pair_fits(const hipie_conv* first, const hipie_conv* second, int3
         if (!block_epilogues_fit(first->epi.flags, true, second->epi.flags)) return;
         int oh, ow;
         conv_out_hw(da, h, w, oh, ow);
-        *fits = block_geometry(da.oc, da.ic, oh, ow).ok ? 1 : 0;
+        const BlockGeometry geo = block_geometry(da.oc, da.ic, oh, ow);
+        // bit 0: the pair runs as one kernel; bit 1: also in the form with two wave groups (hipie_conv_set_stages 7)
+        *fits = geo.ok ? (1 | ((geo.ok2 && db.oc / da.oc >= 2) ? 2 : 0)) : 0;
     });
 }
 
@@ -2326,7 +2328,7 @@ int hipie_conv_run_pair(const hipie_conv* first, const hipie_conv* second, const
         a.wgt = first->wgt_steps.as<int8_t>();
         b.wgt = second->wgt_steps.as<int8_t>();
         DeviceGuard g(first->device);
-        launch_block(a, &b, geo, in->n, first->stages >= 6, as_stream(stream));
+        launch_block(a, &b, geo, in->n, first->stages == 7 ? 2 : (first->stages >= 6 ? 1 : 0), as_stream(stream));
         HIPIE_CHECK_HIP(hipGetLastError());
     });
 }

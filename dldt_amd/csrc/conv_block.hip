@@ -13,6 +13,10 @@
 //    tile; the second convolution runs passes of CM output channels over it, each ending in the ordinary epilogue
 //    (bias, scale, residual, FakeQuantize) and stores to memory.
 // FB == 0: the 3 x 3 convolution alone (its epilogue stores to memory).
+// NG == 2 (fused only): eight waves, two groups of four, for layers that give a compute unit one workgroup - a wave alone
+// on its SIMD runs the epilogues' dependent vector instructions at half the rate two waves reach together.  The groups
+// split the 3 x 3 convolution's input slabs (group 1 hands its partial sums to group 0 through LDS, group 0 requantises
+// the tile) and take the 1 x 1 convolution's passes in turn (group g: passes g, g + 2, ...).
 //
 // Reference semantics, as for every kernel here: reference::convolution<int32_t> on widened inputs
 // (ngraph/core/reference/include/ngraph/runtime/reference/convolution.hpp:63-146) for both convolutions, the elementwise
@@ -65,10 +69,11 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-template <uint32_t FA, uint32_t FB, int NWC, bool DEEP>
-__global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const BlockArgs g) {
+template <uint32_t FA, uint32_t FB, int NWC, bool DEEP, int NG = 1>
+__global__ __launch_bounds__(256 * NG, (DEEP || NG == 2) ? 1 : 2) void conv_block_kernel(const BlockArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr bool kFused = FB != 0;
+    static_assert(NG == 1 || (NG == 2 && kFused && !DEEP), "two wave groups: the fused form, three steps in flight");
     constexpr int NW = 4, NWP = NW / NWC;
     constexpr int CM = NWC * 64, P = NWP * 64;
     constexpr int CSB = CM / 64;                // 64-byte slabs of the intermediate tile
@@ -85,7 +90,10 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
     int8_t* const mid = lds + 256;                                         // [CSB][P][64 bytes]: 16 KB
     float* const sPB0 = reinterpret_cast<float*>(mid + P * CM);            // tables of the 1 x 1 convolution, even passes
     float* const sPA = sPB0 + PT_ROWS * CM;                                // tables of the 3 x 3 convolution; odd passes later
-    int8_t* const patch = reinterpret_cast<int8_t*>(sPA + PT_ROWS * CM);   // [csa][ppix][64]; later the stores' staging space
+    // (NG == 2: four table buffers - group 0 alternates between the first two, group 1 between the other two)
+    int8_t* const patch = reinterpret_cast<int8_t*>(sPA + (NG == 2 ? 3 : 1) * PT_ROWS * CM);   // [csa][ppix][64]; later the stores' staging space
+    // NG == 2: group 1's partial sums on their way to group 0, [register quad][wave][lane][16 bytes], behind the patch
+    int8_t* const xch = patch + max(g.csa * g.ppix * 64, NG * 16384);
 
     const ConvArgs& a = g.a;
     const ConvArgs& b = g.b;
@@ -97,7 +105,9 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
     }
     const int tid = threadIdx.x, lane = tid & 63;
     HIPIE_STAMP(0);
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = NG == 1 ? 0 : wave_all >> 2, wave = wave_all & 3;     // wave group, wave inside it
+    const int gtid = tid & 255;
     const int woc = wave % NWC, wpix = wave / NWC;
     const int l32 = lane & 31, h = lane >> 5;
 
@@ -108,20 +118,22 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
     const int count = rows * a.OW;                                         // pixels of this tile
     const int pix0 = n * a.OHOW + y0 * a.OW;
     const int PW = a.patch_w;
-    const int NA = 9 * g.csa;
+    // the slabs of the 3 x 3 convolution's input channels this wave group multiplies
+    const int c_begin = NG == 1 ? 0 : grp * (g.csa >> 1), c_end = NG == 1 ? g.csa : c_begin + (g.csa >> 1);
+    const int NA = 9 * c_end;                                              // one behind the group's last step
 
     // tables of both convolutions: requested first, stored to LDS behind the operand requests
     StagedParams spa, spb;
     stage_params_load<FA>(a, 0, CM, tid, spa);
-    if (kFused) stage_params_load<FB>(b, 0, CM, tid, spb);
+    if (kFused) stage_params_load<FB>(b, grp * CM, CM, gtid, spb);          // the group's first pass
 
     // ---- the patch: 1 KB loads of 16 pixels x 64 bytes, chunk c of pixel q in slot c ^ ((q >> 2) & 3) -------------
     {
         const int8_t* in0 = a.in + (static_cast<int64_t>(n) * a.in_sn + (y0 - 1) * a.in_sh - a.in_sw);   // patch pixel (0, 0), in the halo
         const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(in0), 0, 0x7fffffff, 0x00020000);
         const int npix = (a.rows_per_tile + 2) * PW, ngroups = g.ppix >> 4;
-        for (int grp = wave; grp < ngroups; grp += NW) {
-            const int q_lds = grp * 16 + (lane >> 2);
+        for (int grp16 = wave_all; grp16 < ngroups; grp16 += NW * NG) {
+            const int q_lds = grp16 * 16 + (lane >> 2);
             const int chunk = (lane & 3) ^ ((q_lds >> 2) & 3);
             const int q = min(q_lds, npix - 1);
             int py, px;
@@ -129,7 +141,7 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
             py = min(py, rows + 1);                                        // rows under a short last tile: never multiplied into a stored pixel
             const int32_t vo = py * a.in_sh + px * a.in_sw + chunk * 16;
             for (int c = 0; c < g.csa; ++c)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rp, HIPIE_LDS_PTR(patch + (c * g.ppix + grp * 16) * 64), 16, vo, c * 64, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rp, HIPIE_LDS_PTR(patch + (c * g.ppix + grp16 * 16) * 64), 16, vo, c * 64, 0, 0);
         }
     }
 
@@ -146,10 +158,10 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
     };
     WFrag wreg[D];
 #pragma unroll
-    for (int s0 = 0; s0 < D0; ++s0) load_wa(s0, wreg[s0]);                 // NA >= 9 >= D
+    for (int s0 = 0; s0 < D0; ++s0) load_wa(9 * c_begin + s0, wreg[s0]);   // a group has at least nine steps >= D
 
-    stage_params_store<FA>(a, (lds_float_ptr)sPA, CM, tid, spa);
-    if (kFused) stage_params_store<FB>(b, (lds_float_ptr)sPB0, CM, tid, spb);
+    stage_params_store<FA>(a, (lds_float_ptr)sPA, CM, tid, spa);           // (threads tid < CM: of group 0)
+    if (kFused) stage_params_store<FB>(b, (lds_float_ptr)(sPB0 + 2 * grp * PT_ROWS * CM), CM, gtid, spb);
 
     // ---- fragment addresses -----------------------------------------------------------------------------------------
     // pixel rows of 64 bytes, K chunk 2 ks + h in slot (2 ks + h) ^ ((row >> 2) & 3): ks = 1 flips bit 5
@@ -201,21 +213,30 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
     __builtin_amdgcn_s_waitcnt(block_waitcnt_vm_lds(0));
     __builtin_amdgcn_s_barrier();
 #pragma unroll
-    for (int s0 = D0; s0 < D; ++s0) load_wa(s0, wreg[s0]);
-    init_acc_lds((lds_cfloat_ptr)sPA, CM, woc * 64 + 32 * h, acc);
+    for (int s0 = D0; s0 < D; ++s0) load_wa(9 * c_begin + s0, wreg[s0]);
+    if (grp == 0) {
+        init_acc_lds((lds_cfloat_ptr)sPA, CM, woc * 64 + 32 * h, acc);
+    } else {
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[ob][pb][r] = 0;
+    }
     HIPIE_STAMP(1);
 
     // ---- the 3 x 3 convolution: no barrier, no LDS traffic but the patch reads ------------------------------------------
     BFrag bset[2];
-    read_b_patch(patch, poff[0], bset[0]);
-    for (int c = 0; c < g.csa; ++c) {
+    read_b_patch(patch + c_begin * (g.ppix * 64), poff[0], bset[0]);
+    for (int c = c_begin; c < c_end; ++c) {
         const int8_t* const slab = patch + c * (g.ppix * 64);
         const int step0 = c * 9;
         static_for<9>([&](auto tap_c) {
             constexpr int T = decltype(tap_c)::value;
             constexpr int cur = T & 1, nxt = cur ^ 1;
             if (T < 8) read_b_patch(slab, poff[(T + 1) % 9], bset[nxt]);
-            else if (c + 1 < g.csa) read_b_patch(slab + g.ppix * 64, poff[0], bset[nxt]);
+            else if (c + 1 < c_end) read_b_patch(slab + g.ppix * 64, poff[0], bset[nxt]);
             mfma8(wreg[T % D], bset[cur]);
             if (step0 + T + D < NA) load_wa(step0 + T + D, wreg[T % D]);
         });
@@ -238,6 +259,19 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
         HIPIE_STAMP(4);
         return;
     }
+    typedef __attribute__((address_space(3))) v4i* lds_v4i_ptr;
+    if (NG == 2 && grp == 1) {                                             // partial sums over this group's slabs: to group 0
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    v4i v;
+                    v.x = acc[ob][pb][4 * q]; v.y = acc[ob][pb][4 * q + 1]; v.z = acc[ob][pb][4 * q + 2]; v.w = acc[ob][pb][4 * q + 3];
+                    *(lds_v4i_ptr)(xch + ((((ob * 2 + pb) * 4 + q) * 4 + wave) * 64 + lane) * 16) = v;
+                }
+    }
 
     // ---- the 1 x 1 convolution's weights of a pass: requested while an epilogue runs ----------------------------------
     const int8_t* const wb_lane = b.wgt + (woc * 4096 + lane * 16);
@@ -250,7 +284,7 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
             for (int f = 0; f < 4; ++f) wb[c][f] = *reinterpret_cast<const v4i*>(p + f * 1024);
         }
     };
-    load_wb(0);
+    load_wb(grp);                                                          // (NG == 1: grp is 0)
     // where the lane's two pixels live in the output and residual tensors (channel 0 of the wave's part of pass 0), and
     // the residual bytes of a pass: requested a pass ahead, like the weights
     ConvArgs e = b;
@@ -285,10 +319,25 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
                 res_cur[pb][4 * j + 3] = ok ? res_raw[pb][j].w : 0u;
             }
     };
-    if (kByteRes) request_res(0);
+    if (kByteRes) request_res(grp);
+
+    if (NG == 2) {
+        lds_barrier();                                                     // group 1's sums are in LDS; everyone has left the patch
+        if (grp == 0) {
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const v4i v = *(lds_v4i_ptr)(xch + ((((ob * 2 + pb) * 4 + q) * 4 + wave) * 64 + lane) * 16);
+                        acc[ob][pb][4 * q] += v.x; acc[ob][pb][4 * q + 1] += v.y; acc[ob][pb][4 * q + 2] += v.z; acc[ob][pb][4 * q + 3] += v.w;
+                    }
+        }
+    }
 
     // ---- first epilogue: the tile's level bytes -> LDS, in the layout of an operand tile ------------------------------
-    {
+    if (grp == 0) {
         const bool valid[2] = {true, true};
         const int64_t none[2] = {0, 0};
         epilogue<FA, 2, true, true, true, true>(a, acc, woc * 64 + 32 * h, valid, none, none, rres, (lds_cfloat_ptr)sPA, CM, 0, nullptr,
@@ -300,20 +349,24 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
 #ifdef HIPIE_BLOCK_STAMPS
     long long t_bar = 0, t_mma = 0, t_epi = 0;
 #endif
-    for (int pass = 0; pass < g.passes; ++pass) {
+    for (int it = 0; it * NG < g.passes; ++it) {
+        const int pass = it * NG + grp;                                    // (NG == 2: the groups take the passes in turn)
 #ifdef HIPIE_BLOCK_STAMPS
         const long long q0 = clock64();
 #endif
-        // pass 0: the tile is complete and the patch is free; later passes: everyone has left the previous epilogue
+        // first pass: the tile is complete and the patch is free; later passes: everyone has left the previous epilogue
         // (whose tables the next store below overwrites)
         lds_barrier();
+        if (NG == 2 && pass >= g.passes) continue;                         // an odd number of passes: group 1 only meets the others
 #ifdef HIPIE_BLOCK_STAMPS
         const long long q1 = clock64();
 #endif
-        lds_float_ptr const tables = (lds_float_ptr)((pass & 1) ? sPA : sPB0);
-        lds_float_ptr const tables_next = (lds_float_ptr)((pass & 1) ? sPB0 : sPA);
-        const bool more = pass + 1 < g.passes;
-        if (more) stage_params_load<FB>(b, (pass + 1) * CM, CM, tid, spb);
+        float* const tab_a = NG == 1 ? sPB0 : sPB0 + 2 * grp * PT_ROWS * CM;
+        float* const tab_b = NG == 1 ? sPA : tab_a + PT_ROWS * CM;
+        lds_float_ptr const tables = (lds_float_ptr)((it & 1) ? tab_b : tab_a);
+        lds_float_ptr const tables_next = (lds_float_ptr)((it & 1) ? tab_a : tab_b);
+        const bool more = pass + NG < g.passes;
+        if (more) stage_params_load<FB>(b, (pass + NG) * CM, CM, gtid, spb);
         init_acc_lds((lds_cfloat_ptr)tables, CM, woc * 64 + 32 * h, acc);
         read_b_mid(0, bset[0]);
         static_for<CSB>([&](auto c_c) {
@@ -326,9 +379,9 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
 #endif
         if (kByteRes) take_res(pass);
         if (more) {
-            load_wb(pass + 1);
-            if (kByteRes) request_res(pass + 1);
-            stage_params_store<FB>(b, tables_next, CM, tid, spb);
+            load_wb(pass + NG);
+            if (kByteRes) request_res(pass + NG);
+            stage_params_store<FB>(b, tables_next, CM, gtid, spb);
         }
         const int oc0 = pass * CM;
         const int64_t oo[2] = {ea.out_off[0] + oc0, ea.out_off[1] + oc0}, ro[2] = {ea.res_off[0] + oc0, ea.res_off[1] + oc0};
@@ -338,7 +391,7 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
         const bool vv[2] = {ea.valid[0], ea.valid[1]};
 #endif
         epilogue<FB, 2, false, true, true, true>(e, acc, oc0 + woc * 64 + 32 * h, vv, oo, ro, rres, (lds_cfloat_ptr)tables, CM, oc0,
-                     kByteRes ? res_cur : nullptr, (lds_float_ptr)patch + wave * 1024);
+                     kByteRes ? res_cur : nullptr, (lds_float_ptr)patch + wave_all * 1024);
 #ifdef HIPIE_BLOCK_STAMPS
         const long long q3 = clock64();
         t_bar += q1 - q0; t_mma += q2 - q1; t_epi += q3 - q2;
@@ -351,26 +404,40 @@ __global__ __launch_bounds__(256, DEEP ? 1 : 2) void conv_block_kernel(const Blo
 #endif
 }
 
-size_t block_lds_bytes(int nwc, int csa, int ppix) {
+// ng = 2: the layout of the form with two wave groups (four table buffers, staging space for eight waves, 64 KB for
+// the partial sums that change groups)
+size_t block_lds_bytes(int nwc, int csa, int ppix, int ng) {
     const size_t cm = static_cast<size_t>(nwc) * 64;
-    return 256 + 16384 + 2 * PT_ROWS * cm * 4 + std::max<size_t>(static_cast<size_t>(csa) * ppix * 64, 16384);
+    return 256 + 16384 + 2 * ng * PT_ROWS * cm * 4 + std::max<size_t>(static_cast<size_t>(csa) * ppix * 64, ng * 16384) +
+           (ng == 2 ? 65536 : 0);
 }
 
-template <uint32_t FA, uint32_t FB, int NWC, bool DEEP>
+template <uint32_t FA, uint32_t FB, int NWC, bool DEEP, int NG = 1>
 void launch_block_instance(const BlockArgs& g, size_t lds, hipStream_t s) {
     static bool attr_set = false;
     if (!attr_set) {
-        HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_block_kernel<FA, FB, NWC, DEEP>),
+        HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_block_kernel<FA, FB, NWC, DEEP, NG>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         attr_set = true;
     }
-    const dim3 grid(g.p_per_xcd > 0 ? 8 * g.p_per_xcd : g.a.p_tiles), block(256);
-    hipLaunchKernelGGL((conv_block_kernel<FA, FB, NWC, DEEP>), grid, block, lds, s, g);
+    const dim3 grid(g.p_per_xcd > 0 ? 8 * g.p_per_xcd : g.a.p_tiles), block(256 * NG);
+    hipLaunchKernelGGL((conv_block_kernel<FA, FB, NWC, DEEP, NG>), grid, block, lds, s, g);
 }
 
+// form: 0 three steps of weights in flight and two workgroups per compute unit, 1 nine steps and one workgroup,
+// 2 (fused only) eight waves in two groups
 template <uint32_t FA, uint32_t FB>
-void launch_block_shape(const BlockArgs& g, int nwc, bool deep, size_t lds, hipStream_t s) {
-    switch (nwc * 2 + (deep ? 1 : 0)) {
+void launch_block_shape(const BlockArgs& g, int nwc, int form, size_t lds, hipStream_t s) {
+    if constexpr (FB != 0) {
+        if (form == 2) {
+            switch (nwc) {
+            case 2: launch_block_instance<FA, FB, 2, false, 2>(g, lds, s); return;
+            case 4: launch_block_instance<FA, FB, 4, false, 2>(g, lds, s); return;
+            default: fail(HIPIE_GENERAL_ERROR, "block kernel: two wave groups with %d channel waves", nwc);
+            }
+        }
+    }
+    switch (nwc * 2 + (form == 1 ? 1 : 0)) {
     case 2: case 3: launch_block_instance<FA, FB, 1, false>(g, lds, s); break;   // 64 channels: nine steps in all
     case 4: launch_block_instance<FA, FB, 2, false>(g, lds, s); break;
     case 5: launch_block_instance<FA, FB, 2, true>(g, lds, s); break;
@@ -409,12 +476,14 @@ BlockGeometry block_geometry(int oc_a, int ic_a, int oh, int ow) {
     r.patch_w = ow + 2;
     r.csa = ic_a / 64;
     r.ppix = static_cast<int>(round_up(static_cast<int64_t>(r.rows + 2) * r.patch_w, 16));
-    r.lds = block_lds_bytes(r.nwc, r.csa, r.ppix);
+    r.lds = block_lds_bytes(r.nwc, r.csa, r.ppix, 1);
     r.ok = r.lds <= 160 * 1024;
+    r.lds2 = block_lds_bytes(r.nwc, r.csa, r.ppix, 2);
+    r.ok2 = r.ok && r.nwc >= 2 && r.csa % 2 == 0 && r.lds2 <= 160 * 1024;   // (64 channels: the four waves already split the pixels)
     return r;
 }
 
-void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo, int images, bool deep, hipStream_t s) {
+void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo, int images, int form, hipStream_t s) {
     BlockArgs g{};
     g.a = a;
     g.a.rows_per_tile = geo.rows;
@@ -434,10 +503,14 @@ void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo
         g.passes = b->OC / cm;
         HIPIE_REQUIRE(b->OC % cm == 0 && 9 * geo.csa + g.passes * geo.nwc < (1 << 20), HIPIE_GENERAL_ERROR, "block kernel: channel counts");
     }
+    HIPIE_REQUIRE(form != 2 || (b && geo.ok2 && g.passes >= 2), HIPIE_NOT_IMPLEMENTED,
+                  "block kernel: the form with two wave groups takes a fused pair with an even number of input slabs, 128 or 256 "
+                  "channels between the layers and at least two passes");
+    const size_t lds = form == 2 ? geo.lds2 : geo.lds;
     const int ia = block_index(kBlockFirst, a.flags), ib = b ? block_index(kBlockSecond, b->flags) : 3;
     HIPIE_REQUIRE(ia >= 0 && ib >= 0, HIPIE_GENERAL_ERROR, "block kernel: no instance for epilogues %#x / %#x", a.flags, b ? b->flags : 0u);
 #define HIPIE_BLOCK_CASE(IA, IB, FB) \
-    case (IA) * 4 + (IB): launch_block_shape<kBlockFirst[IA], FB>(g, geo.nwc, deep, geo.lds, s); break;
+    case (IA) * 4 + (IB): launch_block_shape<kBlockFirst[IA], FB>(g, geo.nwc, form, lds, s); break;
     switch (ia * 4 + ib) {
         HIPIE_BLOCK_CASE(0, 0, kBlockSecond[0]) HIPIE_BLOCK_CASE(0, 1, kBlockSecond[1]) HIPIE_BLOCK_CASE(0, 2, kBlockSecond[2]) HIPIE_BLOCK_CASE(0, 3, 0u)
         HIPIE_BLOCK_CASE(1, 0, kBlockSecond[0]) HIPIE_BLOCK_CASE(1, 1, kBlockSecond[1]) HIPIE_BLOCK_CASE(1, 2, kBlockSecond[2]) HIPIE_BLOCK_CASE(1, 3, 0u)

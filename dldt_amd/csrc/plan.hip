@@ -375,8 +375,11 @@ struct ConvStep : Step {
 struct PairStep : Step {
     std::unique_ptr<ConvStep> first, second;
     int mode = 1;                  // PlanConfig::fuse_convs
-    bool fits = false, fused = false;
-    bool deep = false;             // the fused kernel with nine steps of weights in flight (one workgroup per compute unit)
+    bool fits = false, fused = false, fits_groups = false;
+    // form of the fused kernel: 0 three steps of weights in flight, 1 nine steps (one workgroup per compute unit),
+    // 2 eight waves in two groups (where fits_groups)
+    int form = 0;
+    static int stages_of(int form) { return form == 1 ? 8 : (form == 2 ? 7 : 0); }
     void create(int, const std::vector<TensorInfo>& tensors) override {   // (the layers exist already)
         name = second->name;
         macs = first->macs + second->macs;
@@ -392,6 +395,7 @@ struct PairStep : Step {
         int f = 0;
         check_status(hipie_conv_pair_fits(first->conv, second->conv, ti.h, ti.w, &f), name.c_str());
         fits = f != 0 && ti.halo >= 1 && second->res >= 0 && second->res_param < 0;
+        fits_groups = fits && (f & 2) != 0;
         const TensorInfo& tm = tensors[first->out];
         mid_bytes = static_cast<int64_t>(tm.n) * tm.h * tm.w * tm.c;
         choose(fits && mode == 2);
@@ -400,7 +404,7 @@ struct PairStep : Step {
     void choose(bool one_kernel) {
         fused = one_kernel;
         // the depth is a setting of the first layer's object: the pair's when they run as one kernel, else its own
-        if (first->conv) check_status(hipie_conv_set_stages(first->conv, (fused ? deep : first->deep) ? 8 : 0), name.c_str());
+        if (first->conv) check_status(hipie_conv_set_stages(first->conv, fused ? stages_of(form) : (first->deep ? 8 : 0)), name.c_str());
         type = fused ? "Convolution+Convolution" : "Convolution,Convolution";
         bytes = first->bytes + second->bytes - (fused ? 2 * mid_bytes : 0);
     }
@@ -434,8 +438,8 @@ struct PairStep : Step {
                 for (size_t l = 0; l < nl; ++l) run_fused(lanes[l].arena, tensors, lanes[l].stream);
         };
         float best_fused = 0.f;
-        for (int d = 0; d < 2; ++d) {
-        check_status(hipie_conv_set_stages(first->conv, d ? 8 : 0), name.c_str());
+        for (int d = 0; d < (fits_groups ? 3 : 2); ++d) {
+        check_status(hipie_conv_set_stages(first->conv, stages_of(d)), name.c_str());
         launch_all(2);
         float ms = 0.f;   // the same protocol as the layers' own variants: fastest of three rounds of five launches per lane
         for (int round = 0; round < 3; ++round) {
@@ -455,7 +459,7 @@ struct PairStep : Step {
         }
         if (d == 0 || ms < 0.97f * best_fused) {
             best_fused = ms;
-            deep = d != 0;
+            form = d;
         }
         }
         for (size_t l = 0; l < nl; ++l) {
@@ -466,15 +470,17 @@ struct PairStep : Step {
         choose(mode == 2 || (apart_us > 0.f && fused_us < 0.97f * apart_us));
         if (std::getenv("HIPIE_TUNE_LOG"))
             std::fprintf(stderr, "hipie tune: %-28s one kernel %.1f us (%s), two %.1f us per launch with %zu in flight: %s\n", name.c_str(),
-                         fused_us, deep ? "nine steps in flight" : "three steps in flight", apart_us, nl, fused ? "fused" : "apart");
+                         fused_us, form == 2 ? "two wave groups" : (form == 1 ? "nine steps in flight" : "three steps in flight"), apart_us, nl,
+                         fused ? "fused" : "apart");
     }
     // the layers' variants and the choice between one kernel and two, in one integer
-    int variant() const override { return first->variant() + 64 * second->variant() + (fused ? 4096 : 0) + (deep ? 8192 : 0); }
+    int variant() const override { return first->variant() + 64 * second->variant() + (fused ? 4096 : 0) + 8192 * form; }
     void set_variant(int v) override {
         if (v < 0) return;
         first->set_variant(v & 63);
         second->set_variant((v >> 6) & 63);
-        deep = (v & 8192) != 0;
+        form = (v >> 13) & 3;
+        if (form == 3 || (form == 2 && !fits_groups)) form = 0;
         choose(fits && (v & 4096) != 0 && mode != 0);
     }
 };

@@ -202,9 +202,16 @@ class Convolution:
 
     def pair_fits(self, second, h, w):
         """hipie_conv_pair_fits: does the fused kernel take this layer followed by ``second`` on h x w inputs"""
+        return bool(self.pair_forms(second, h, w))
+
+    def pair_forms(self, second, h, w):
+        """the raw answer of hipie_conv_pair_fits: 0, or bit 0 (fits) and bit 1 (also with two wave groups: stages 7)"""
         fits = ctypes.c_int()
         check(lib().hipie_conv_pair_fits(self._h, second._h, h, w, ctypes.byref(fits)))
-        return bool(fits.value)
+        return fits.value
+
+    def set_stages(self, stages):
+        check(lib().hipie_conv_set_stages(self._h, stages))
 
     def run_pair(self, second, x, out, residual=None):
         """hipie_conv_run_pair: this layer and ``second`` in one kernel, the intermediate tensor kept in LDS"""

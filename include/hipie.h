@@ -239,7 +239,8 @@ int hipie_conv_run(const hipie_conv* conv, const hipie_tensor* in, const hipie_t
  * The CPU plugin fuses consecutive convolutions into one primitive the same way
  * (inference-engine/src/mkldnn_plugin/mkldnn_graph_optimizer.cpp:631-759 FuseConvolutionAndDWConvolution, and the
  * sum post-op of :958-1130).  `in` is the first layer's input, `residual` and `out` the second layer's;
- * hipie_conv_pair_fits says whether the kernel takes two layers on an input of h x w pixels. */
+ * hipie_conv_pair_fits says whether the kernel takes two layers on an input of h x w pixels (*fits = 0: no; bit 0
+ * set: yes; bit 1: also in its form with eight waves per workgroup, see hipie_conv_set_stages in hipie_diag.h). */
 int hipie_conv_pair_fits(const hipie_conv* first, const hipie_conv* second, int32_t h, int32_t w, int* fits);
 int hipie_conv_run_pair(const hipie_conv* first, const hipie_conv* second, const hipie_tensor* in,
                         const hipie_tensor* residual, const hipie_tensor* out, void* stream);

@@ -48,7 +48,9 @@ int hipie_conv_epilogue_flags(const hipie_conv* conv, uint32_t* flags, int* spec
 /* ring depth of the pipelined variants: 3, 4, 6 or 8 K steps in LDS (other values round down, and to
  * what fits 144 KB); 0 = the variant's default (4 for tile 4, else 3).  Variant 24 and hipie_conv_run_pair (the
  * setting of its first layer): 6 and more = nine steps of weights in flight in a wave's registers and one workgroup
- * per compute unit (for a launch that runs alone), else three steps and two workgroups */
+ * per compute unit (for a launch that runs alone), else three steps and two workgroups; hipie_conv_run_pair only:
+ * 7 = eight waves in two groups that split the first layer's input channels and take the second layer's passes in
+ * turn (where hipie_conv_pair_fits reports bit 1; HIPIE_NOT_IMPLEMENTED elsewhere) */
 int hipie_conv_set_stages(hipie_conv* conv, int stages);
 
 /* Constants of the convolution epilogue's two-operation division: for each divisor d[i] a pair with

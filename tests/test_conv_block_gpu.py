@@ -20,7 +20,10 @@ CASES = {
     "c256_14x14": (2, 256, 14, 14, 256, 1024),        # stage 3: rows 4 + 4 + 4 + 2
     "c192_to_128_9x7": (1, 192, 9, 7, 128, 128),      # three input slabs, other channel count out, one pass
     "c64_to_256_5x5": (2, 64, 5, 5, 256, 256),        # a tile far smaller than its pixel slots
+    "c128_to_256_20x12": (2, 128, 20, 12, 256, 512),  # two input slabs, two passes, rows 5 + 5 + 5 + 5
 }
+# the cases the form with two wave groups takes (an even number of input slabs, 128 or 256 channels between the layers)
+TWO_GROUPS = ("c128_28x28", "c256_14x14", "c128_to_256_20x12")
 ST, DIL, PAD = (1, 1), (1, 1), (1, 1)
 
 
@@ -83,6 +86,18 @@ def test_fused_bottleneck_tail_gives_the_reference_bytes(orc, name):
     first.run_pair(second, xin, out, rt)
     np.testing.assert_array_equal(out.to_nchw(), want)
     assert np.all(out.padded_channels() == 0)
+    # the other forms of the kernel: nine steps of weights in flight, and eight waves in two groups where it applies
+    assert (first.pair_forms(second, H, W) & 2 != 0) == (name in TWO_GROUPS)
+    for stages in (8, 7) if name in TWO_GROUPS else (8,):
+        first.set_stages(stages)
+        again = DeviceTensor(N, H, W, OCB, U8B)
+        first.run_pair(second, xin, again, rt)
+        np.testing.assert_array_equal(again.to_nchw(), want, err_msg="stages %d" % stages)
+    if name not in TWO_GROUPS:
+        first.set_stages(7)
+        with pytest.raises(Exception):
+            first.run_pair(second, xin, DeviceTensor(N, H, W, OCB, U8B), rt)
+    first.set_stages(0)
     # the layers one after the other store the same bytes
     first.run(xin, tmid)
     np.testing.assert_array_equal(tmid.to_nchw(), mid)
