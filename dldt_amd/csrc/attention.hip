@@ -37,24 +37,27 @@ struct AttentionArgs {
     Requant fq_p, fq_o;                               // fq_o.levels == 0: f32 output
     float p_zh, p_zl;                                 // probabilities: two-operation division by fq_p.p.d
     int p_div2;                                       // ... verified against IEEE division on the device
+    int p_sat;                                        // input_low of the probabilities' FakeQuantize is +0 and it has 256 levels
     uint32_t p_xor, p_add;                            // stored byte = level + out_low (mod 256): XOR 0x80 per byte, or bytewise add
     int p_bias;                                       // 128 when the probabilities are u8 levels (stored as level - 128), else 0
 };
 
 // level index k of four probabilities as four unsigned bytes (rounded to nearest-even and packed by
 // v_cvt_pk_u8_f32), then the output offset applied bytewise
-template <bool DIV2>
+// PSAT: input_low is +0 and there are 256 levels - a probability is never below input_low, and the packing
+// conversion's saturation at 255 is the branch for values above input_high: no clamp, no subtraction
+template <bool DIV2, bool PSAT>
 __device__ __forceinline__ uint32_t prob_levels4(const AttentionArgs& a, float p0, float p1, float p2, float p3) {
     const FqChannel& c = a.fq_p.p;
     uint32_t w = 0;
-    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, false>(p0, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 0, w);
-    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, false>(p1, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 1, w);
-    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, false>(p2, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 2, w);
-    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, false>(p3, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 3, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, PSAT, PSAT>(p0, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 0, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, PSAT, PSAT>(p1, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 1, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, PSAT, PSAT>(p2, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 2, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, PSAT, PSAT>(p3, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 3, w);
     return a.p_add ? add_bytes(w, a.p_add) : (w ^ a.p_xor);
 }
 
-template <int NT, bool DIV2, bool MASK>   // NT = S / 32 key tiles
+template <int NT, bool DIV2, bool MASK, bool PSAT>   // NT = S / 32 key tiles
 __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a) {
     constexpr int S = NT * 32;
     constexpr int VT_LD = S + 16;                     // odd number of 16-byte groups per row: conflict-free
@@ -192,7 +195,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
             const float4 p4 = make_float4(x[t][4 * g] * inv, x[t][4 * g + 1] * inv, x[t][4 * g + 2] * inv, x[t][4 * g + 3] * inv);
             if (a.probs && q_ok)
                 *reinterpret_cast<float4*>(a.probs + dump_row + 32 * t + 8 * g + 4 * h) = p4;
-            pf[g] = static_cast<int>(prob_levels4<DIV2>(a, p4.x, p4.y, p4.z, p4.w));
+            pf[g] = static_cast<int>(prob_levels4<DIV2, PSAT>(a, p4.x, p4.y, p4.z, p4.w));
         }
 #pragma unroll
         for (int db = 0; db < 2; ++db) {
@@ -219,12 +222,15 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
 template <int NT>
 void launch(const AttentionArgs& a, int batches, hipStream_t s) {
     const dim3 grid(static_cast<uint32_t>(ceil_div(a.S, 128)), static_cast<uint32_t>(batches));
+    const bool sat = a.p_div2 && a.p_sat;             // (the form without clamp: compiled for the usual division only)
     if (a.mask) {
-        if (a.p_div2) hipLaunchKernelGGL((attention_kernel<NT, true, true>), grid, dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((attention_kernel<NT, false, true>), grid, dim3(256), 0, s, a);
+        if (sat) hipLaunchKernelGGL((attention_kernel<NT, true, true, true>), grid, dim3(256), 0, s, a);
+        else if (a.p_div2) hipLaunchKernelGGL((attention_kernel<NT, true, true, false>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((attention_kernel<NT, false, true, false>), grid, dim3(256), 0, s, a);
     } else {
-        if (a.p_div2) hipLaunchKernelGGL((attention_kernel<NT, true, false>), grid, dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((attention_kernel<NT, false, false>), grid, dim3(256), 0, s, a);
+        if (sat) hipLaunchKernelGGL((attention_kernel<NT, true, false, true>), grid, dim3(256), 0, s, a);
+        else if (a.p_div2) hipLaunchKernelGGL((attention_kernel<NT, true, false, false>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((attention_kernel<NT, false, false, false>), grid, dim3(256), 0, s, a);
     }
 }
 
@@ -262,6 +268,7 @@ int hipie_attention_create(int device, const hipie_attention_desc* desc, hipie_a
         a.S = desc->seq;
         a.scale1 = desc->score_scale;
         a.scale2 = desc->context_scale;
+
         a.fq_p = make_requant(&desc->prob_fq, "hipie_attention_create (probabilities)");
         if (desc->out_dtype == HIPIE_I8) a.fq_o = make_requant(&desc->out_fq, "hipie_attention_create (output)");
         // the probabilities' level index: two-operation division when the device confirms it against IEEE
@@ -272,6 +279,7 @@ int hipie_attention_create(int device, const hipie_attention_desc* desc, hipie_a
         if (a.p_div2) { a.p_zh = zh[0]; a.p_zl = zl[0]; }
         HIPIE_REQUIRE(a.p_div2 || a.fq_p.rcp || device < 0, HIPIE_NOT_IMPLEMENTED,
                       "hipie_attention_create: no exact fast division for the probabilities' FakeQuantize range");
+        a.p_sat = a.fq_p.p.il == 0.f && !std::signbit(a.fq_p.p.il) && a.fq_p.lm1 == 255.f;
         a.p_bias = desc->prob_dtype == HIPIE_U8B ? 128 : 0;
         const int off = static_cast<int>(a.fq_p.p.ol) & 0xff;
         a.p_xor = off == 0x80 ? 0x80808080u : 0u;
