@@ -69,6 +69,11 @@ bool block_epilogues_fit(uint32_t flags_a, bool fused, uint32_t flags_b);
 // 2 (with b, where geo.ok2): eight waves in two groups that split the first layer's input slabs and take the second
 // layer's passes in turn
 void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo, int images, int form, hipStream_t s);
+// the same kernel as a depthwise 3 x 3 convolution (stride 1 or 2, pad 1 on the top and left, a.wgt = [tap][OCp] bytes):
+// the taps' diagonal weight matrices on the matrix pipe, 256 pixels x one 64-channel slab per workgroup
+bool block_dw_epilogue_fits(uint32_t flags);
+BlockGeometry block_dw_geometry(int oh, int ow, int stride);
+void launch_block_dw(const ConvArgs& a, const BlockGeometry& geo, int images, hipStream_t s);
 
 // depthwise kernels (dwconv.hip).  variant 0: a lane computes its outputs from registers loaded straight from memory;
 // variant 1: 3 x 3 through an LDS patch with the window sliding in registers (dwconv_strip_fits says which layers)

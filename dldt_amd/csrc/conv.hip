@@ -1929,10 +1929,15 @@ void hipie_conv_destroy(hipie_conv* c) { delete c; }
 int hipie_conv_set_tile(hipie_conv* c, int tile) {
     return guarded([&] {
         HIPIE_REQUIRE(c && tile >= 0 && tile <= 24, HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: tile=%d", tile);
-        if (c->depthwise) {   // 0: registers only, 1: 3 x 3 through an LDS patch
+        if (c->depthwise) {   // 0: registers only, 1: 3 x 3 through an LDS patch, 2: 3 x 3 on the matrix pipe
+            const hipie_conv_desc& dd = c->d;
+            const bool matrix_ok = dd.kh == 3 && dd.kw == 3 && dd.dil_h == 1 && dd.dil_w == 1 && dd.stride_h == dd.stride_w &&
+                                   (dd.stride_h == 1 || dd.stride_h == 2) && dd.pad_top == 1 && dd.pad_left == 1 &&
+                                   block_dw_epilogue_fits(c->epi.flags);
             HIPIE_REQUIRE(tile == 0 || (tile == 1 && !(c->epi.flags & CF_RES) &&
                                         dwconv_strip_fits(c->d.kh, c->d.kw, c->d.dil_h, c->d.dil_w, c->d.stride_h, c->d.stride_w,
-                                                          c->d.in_c_stride, static_cast<int>(c->OCp), c->epi.flags)),
+                                                          c->d.in_c_stride, static_cast<int>(c->OCp), c->epi.flags)) ||
+                              (tile == 2 && matrix_ok),
                           HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: depthwise variant %d does not take this layer", tile);
             c->tile = tile;
             return;
@@ -2131,8 +2136,18 @@ static int conv_run(const hipie_conv* c, const hipie_tensor* in, const hipie_ten
             HIPIE_REQUIRE(in->stride_w >= d.ic && in->stride_w % 16 == 0, HIPIE_PARAMETER_MISMATCH,
                           "hipie_conv_run: depthwise input channel stride");
             DeviceGuard g(c->device);
+            if (c->tile == 2) {
+                // the matrix-pipe form reads a border of one pixel around the tensor; an output too wide for its tile, or a
+                // tensor without that border, runs the general kernel
+                const BlockGeometry bg = block_dw_geometry(oh, ow, d.stride_h);
+                if (bg.ok && in->halo >= 1 && (oh - 1) * d.stride_h + 1 <= in->h && (ow - 1) * d.stride_w + 1 <= in->w) {
+                    launch_block_dw(a, bg, in->n, as_stream(stream));
+                    HIPIE_CHECK_HIP(hipGetLastError());
+                    return;
+                }
+            }
             const DwGeometry geo{in->h, in->w, in->halo, d.pad_top, d.pad_left};
-            launch_dwconv(a, d.kh, d.kw, d.dil_h, d.dil_w, c->tile, geo, as_stream(stream));
+            launch_dwconv(a, d.kh, d.kw, d.dil_h, d.dil_w, c->tile == 2 ? 0 : c->tile, geo, as_stream(stream));
             HIPIE_CHECK_HIP(hipGetLastError());
             return;
         }

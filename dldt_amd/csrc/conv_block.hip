@@ -17,6 +17,12 @@
 // on its SIMD runs the epilogues' dependent vector instructions at half the rate two waves reach together.  The groups
 // split the 3 x 3 convolution's input slabs (group 1 hands its partial sums to group 0 through LDS, group 0 requantises
 // the tile) and take the 1 x 1 convolution's passes in turn (group g: passes g, g + 2, ...).
+// DW: a depthwise 3 x 3 convolution (stride 1 or 2) on the matrix pipe, which such a layer otherwise leaves idle: a
+// workgroup takes 256 pixels x the 64 channels of slab blockIdx.y; the weight operand of tap t is the 64 x 64 diagonal
+// matrix diag(w[t][c]), built in registers from the lane's two weight bytes per tap (a lane's 16-byte fragment holds
+// one diagonal element or none), and only the two diagonal 32 x 32 blocks are multiplied: 36 matrix instructions per
+// 64 x 64 outputs where the vector pipe needs 13 or more instructions per output
+// (reference::group_convolution, group_convolution.hpp:78-144, with one filter per channel).
 //
 // Reference semantics, as for every kernel here: reference::convolution<int32_t> on widened inputs
 // (ngraph/core/reference/include/ngraph/runtime/reference/convolution.hpp:63-146) for both convolutions, the elementwise
@@ -69,10 +75,11 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-template <uint32_t FA, uint32_t FB, int NWC, bool DEEP, int NG = 1>
+template <uint32_t FA, uint32_t FB, int NWC, bool DEEP, int NG = 1, bool DW = false>
 __global__ __launch_bounds__(256 * NG, (DEEP || NG == 2) ? 1 : 2) void conv_block_kernel(const BlockArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr bool kFused = FB != 0;
+    static_assert(!DW || (!kFused && NWC == 1 && NG == 1 && !DEEP), "depthwise: one 64-channel slab per workgroup, alone");
     static_assert(NG == 1 || (NG == 2 && kFused && !DEEP), "two wave groups: the fused form, three steps in flight");
     constexpr int NW = 4, NWP = NW / NWC;
     constexpr int CM = NWC * 64, P = NWP * 64;
@@ -118,28 +125,32 @@ __global__ __launch_bounds__(256 * NG, (DEEP || NG == 2) ? 1 : 2) void conv_bloc
     const int count = rows * a.OW;                                         // pixels of this tile
     const int pix0 = n * a.OHOW + y0 * a.OW;
     const int PW = a.patch_w;
+    const int cb = DW ? static_cast<int>(blockIdx.y) * 64 : 0;            // first channel of the workgroup (depthwise: its slab)
+    const int cs_ = DW ? a.conv_sh : 1;                                    // stride (the dense form is built for 1)
     // the slabs of the 3 x 3 convolution's input channels this wave group multiplies
     const int c_begin = NG == 1 ? 0 : grp * (g.csa >> 1), c_end = NG == 1 ? g.csa : c_begin + (g.csa >> 1);
     const int NA = 9 * c_end;                                              // one behind the group's last step
 
     // tables of both convolutions: requested first, stored to LDS behind the operand requests
     StagedParams spa, spb;
-    stage_params_load<FA>(a, 0, CM, tid, spa);
+    stage_params_load<FA>(a, cb, CM, tid, spa);
     if (kFused) stage_params_load<FB>(b, grp * CM, CM, gtid, spb);          // the group's first pass
 
     // ---- the patch: 1 KB loads of 16 pixels x 64 bytes, chunk c of pixel q in slot c ^ ((q >> 2) & 3) -------------
     {
-        const int8_t* in0 = a.in + (static_cast<int64_t>(n) * a.in_sn + (y0 - 1) * a.in_sh - a.in_sw);   // patch pixel (0, 0), in the halo
+        const int8_t* in0 = a.in + (static_cast<int64_t>(n) * a.in_sn + (y0 * cs_ - 1) * a.in_sh - a.in_sw + cb);   // patch pixel (0, 0), in the halo
         const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(in0), 0, 0x7fffffff, 0x00020000);
-        const int npix = (a.rows_per_tile + 2) * PW, ngroups = g.ppix >> 4;
+        const int npix = ((a.rows_per_tile - 1) * cs_ + 3) * PW, ngroups = g.ppix >> 4;
         for (int grp16 = wave_all; grp16 < ngroups; grp16 += NW * NG) {
             const int q_lds = grp16 * 16 + (lane >> 2);
             const int chunk = (lane & 3) ^ ((q_lds >> 2) & 3);
             const int q = min(q_lds, npix - 1);
             int py, px;
             fast_divmod(q, PW, a.inv_patch_w, py, px);
-            py = min(py, rows + 1);                                        // rows under a short last tile: never multiplied into a stored pixel
-            const int32_t vo = py * a.in_sh + px * a.in_sw + chunk * 16;
+            py = min(py, (rows - 1) * cs_ + 2);                            // rows under a short last tile: never multiplied into a stored pixel
+            // (depthwise: a slab that ends behind the pixel's channels re-reads the pixel's first bytes there instead of its
+            // neighbour's - those channels meet zero weights, and no byte behind the tensor is touched)
+            const int32_t vo = py * a.in_sh + px * a.in_sw + ((DW && cb + chunk * 16 >= a.in_sw) ? -cb : chunk * 16);
             for (int c = 0; c < g.csa; ++c)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rp, HIPIE_LDS_PTR(patch + (c * g.ppix + grp16 * 16) * 64), 16, vo, c * 64, 0, 0);
         }
@@ -157,8 +168,22 @@ __global__ __launch_bounds__(256 * NG, (DEEP || NG == 2) ? 1 : 2) void conv_bloc
         for (int f = 0; f < 4; ++f) r[f] = *reinterpret_cast<const v4i*>(p + f * 1024);
     };
     WFrag wreg[D];
+    if constexpr (!DW) {
 #pragma unroll
-    for (int s0 = 0; s0 < D0; ++s0) load_wa(9 * c_begin + s0, wreg[s0]);   // a group has at least nine steps >= D
+        for (int s0 = 0; s0 < D0; ++s0) load_wa(9 * c_begin + s0, wreg[s0]);   // a group has at least nine steps >= D
+    }
+    // depthwise: the lane's diagonal elements under every tap ([tap][OCp] bytes).  Row l32 of row block ob is channel
+    // 32 ((l32 >> 2) & 1) + 16 ob + 4 (l32 >> 3) + (l32 & 3) of the slab: the order in which the epilogue finds a lane's
+    // sixteen results of a block on consecutive channels (packed_row in conv.hip)
+    const int dw_c = 32 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3);
+    uint32_t wdiag[2][9];
+    if constexpr (DW) {
+#pragma unroll
+        for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+            for (int t = 0; t < 9; ++t)
+                wdiag[ob][t] = static_cast<uint8_t>(a.wgt[static_cast<int64_t>(t) * a.OCp + cb + 16 * ob + dw_c]);
+    }
 
     stage_params_store<FA>(a, (lds_float_ptr)sPA, CM, tid, spa);           // (threads tid < CM: of group 0)
     if (kFused) stage_params_store<FB>(b, (lds_float_ptr)(sPB0 + 2 * grp * PT_ROWS * CM), CM, gtid, spb);
@@ -172,13 +197,14 @@ __global__ __launch_bounds__(256 * NG, (DEEP || NG == 2) ? 1 : 2) void conv_bloc
         const int p = min(wpix * 64 + pb * 32 + l32, count - 1);
         int r, x;
         fast_divmod(p, a.OW, a.inv_OW, r, x);
-        const int idx0 = r * PW + x;
+        const int idx0 = r * cs_ * PW + x * cs_;
 #pragma unroll
         for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
             for (int kw = 0; kw < 3; ++kw) {
                 const int idx = idx0 + kh * PW + kw;
-                poff[kh * 3 + kw][pb] = idx * 64 + ((h ^ ((idx >> 2) & 3)) << 4);
+                // (depthwise: the half-waves read the chunks 2 h and 2 h + 1 - see the matrix instructions below)
+                poff[kh * 3 + kw][pb] = idx * 64 + (((DW ? 2 * h : h) ^ ((idx >> 2) & 3)) << 4);
             }
     }
     typedef v4i BFrag[4];                                                  // [ks * 2 + pb]
@@ -212,8 +238,10 @@ __global__ __launch_bounds__(256 * NG, (DEEP || NG == 2) ? 1 : 2) void conv_bloc
     // once anyway); the barrier makes every wave's part visible
     __builtin_amdgcn_s_waitcnt(block_waitcnt_vm_lds(0));
     __builtin_amdgcn_s_barrier();
+    if constexpr (!DW) {
 #pragma unroll
-    for (int s0 = D0; s0 < D; ++s0) load_wa(9 * c_begin + s0, wreg[s0]);
+        for (int s0 = D0; s0 < D; ++s0) load_wa(9 * c_begin + s0, wreg[s0]);
+    }
     if (grp == 0) {
         init_acc_lds((lds_cfloat_ptr)sPA, CM, woc * 64 + 32 * h, acc);
     } else {
@@ -228,6 +256,39 @@ __global__ __launch_bounds__(256 * NG, (DEEP || NG == 2) ? 1 : 2) void conv_bloc
 
     // ---- the 3 x 3 convolution: no barrier, no LDS traffic but the patch reads ------------------------------------------
     BFrag bset[2];
+    if constexpr (DW) {
+        // Row block ob holds the channels 16 ob .. 16 ob + 15 and 32 + 16 ob .. 47 + 16 ob, i.e. the 16-byte chunks ob and
+        // ob + 2 of a pixel: one matrix instruction per block multiplies exactly those 32 input channels when the lower
+        // half-wave reads chunk ob and the upper one chunk ob + 2.  A lane's A fragment then holds its row's diagonal
+        // element in byte 4 (l32 >> 3) + (l32 & 3) if its half is the one that carries the row's channel, zeros else.
+        const bool has = ((l32 >> 2) & 1) == h;
+        const int dsel = l32 >> 3, sh = (l32 & 3) * 8;
+        const uint32_t m0_ = has && dsel == 0 ? 0xffffffffu : 0u, m1_ = has && dsel == 1 ? 0xffffffffu : 0u,
+                       m2_ = has && dsel == 2 ? 0xffffffffu : 0u, m3_ = has && dsel == 3 ? 0xffffffffu : 0u;
+        auto read_b_dw = [&](const int (&po)[2], BFrag& bf) {                // [ob * 2 + pb]
+#pragma unroll
+            for (int ob = 0; ob < 2; ++ob)
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb) bf[ob * 2 + pb] = *reinterpret_cast<const v4i*>(patch + (ob ? (po[pb] ^ 16) : po[pb]));
+        };
+        if (wpix * 64 < count) {                                           // (a wave without pixels only meets the others)
+            read_b_dw(poff[0], bset[0]);
+            static_for<9>([&](auto tap_c) {
+                constexpr int T = decltype(tap_c)::value;
+                constexpr int cur = T & 1, nxt = cur ^ 1;
+                if (T < 8) read_b_dw(poff[T + 1 < 9 ? T + 1 : 0], bset[nxt]);
+#pragma unroll
+                for (int ob = 0; ob < 2; ++ob) {
+                    const uint32_t w = wdiag[ob][T] << sh;
+                    v4i af;
+                    af.x = static_cast<int>(w & m0_); af.y = static_cast<int>(w & m1_); af.z = static_cast<int>(w & m2_); af.w = static_cast<int>(w & m3_);
+#pragma unroll
+                    for (int pb = 0; pb < 2; ++pb)
+                        acc[ob][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bset[cur][ob * 2 + pb], acc[ob][pb], 0, 0, 0);
+                }
+            });
+        }
+    } else {
     read_b_patch(patch + c_begin * (g.ppix * 64), poff[0], bset[0]);
     for (int c = c_begin; c < c_end; ++c) {
         const int8_t* const slab = patch + c * (g.ppix * 64);
@@ -244,17 +305,19 @@ __global__ __launch_bounds__(256 * NG, (DEEP || NG == 2) ? 1 : 2) void conv_bloc
 #pragma unroll
         for (int f = 0; f < 4; ++f) bset[0][f] = bset[1][f];
     }
+    }
     HIPIE_STAMP(2);
 
     v16f rres[2][2];
     const int m0 = pix0 + wpix * 64 + l32;
     if (!kFused) {
         __builtin_amdgcn_s_barrier();                                      // every wave is done with the patch: it becomes the stores' staging space
+        if (DW && wpix * 64 >= count) return;
         ConvArgs e = a;
         e.M = min(a.M, pix0 + count);                                      // pixels behind the tile's rows belong to the next tile
         EpiAddr ea;
-        epilogue_addresses(e, woc * 64 + 32 * h, m0, m0 + 32, 0, ea);
-        epilogue<FA, 2, false, true, true, true>(e, acc, woc * 64 + 32 * h, ea.valid, ea.out_off, ea.res_off, rres, (lds_cfloat_ptr)sPA, CM, 0, nullptr,
+        epilogue_addresses(e, cb + woc * 64 + 32 * h, m0, m0 + 32, 0, ea);
+        epilogue<FA, 2, false, true, true, true>(e, acc, cb + woc * 64 + 32 * h, ea.valid, ea.out_off, ea.res_off, rres, (lds_cfloat_ptr)sPA, CM, cb, nullptr,
                                      (lds_float_ptr)patch + wave * 1024);
         HIPIE_STAMP(4);
         return;
@@ -517,6 +580,61 @@ void launch_block(const ConvArgs& a, const ConvArgs* b, const BlockGeometry& geo
         HIPIE_BLOCK_CASE(2, 0, kBlockSecond[0]) HIPIE_BLOCK_CASE(2, 1, kBlockSecond[1]) HIPIE_BLOCK_CASE(2, 2, kBlockSecond[2]) HIPIE_BLOCK_CASE(2, 3, 0u)
     }
 #undef HIPIE_BLOCK_CASE
+}
+
+// ---- depthwise 3 x 3 on the matrix pipe -------------------------------------------------------------------------------
+constexpr uint32_t kBlockDepthwise[3] = {E_PLAIN0, E_SCALEFQ0, E_CLAMPFQ};
+
+bool block_dw_epilogue_fits(uint32_t flags) { return block_index(kBlockDepthwise, flags) >= 0; }
+
+BlockGeometry block_dw_geometry(int oh, int ow, int stride) {
+    BlockGeometry r{};
+    if (ow < 1 || oh < 1 || ow > 256 || (stride != 1 && stride != 2)) return r;
+    r.nwc = 1;
+    r.rows = std::min(256 / ow, oh);
+    r.tiles_per_image = static_cast<int>(ceil_div(oh, r.rows));
+    r.patch_w = (ow - 1) * stride + 3;
+    r.csa = 1;
+    r.ppix = static_cast<int>(round_up(static_cast<int64_t>((r.rows - 1) * stride + 3) * r.patch_w, 16));
+    r.lds = block_lds_bytes(1, 1, r.ppix, 1);
+    r.ok = r.lds <= 160 * 1024;
+    return r;
+}
+
+template <uint32_t FA>
+static void launch_block_dw_instance(const BlockArgs& g, int slabs, size_t lds, hipStream_t s) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        HIPIE_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_block_kernel<FA, 0u, 1, false, 1, true>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_set = true;
+    }
+    const dim3 grid(g.p_per_xcd > 0 ? 8 * g.p_per_xcd : g.a.p_tiles, slabs), block(256);
+    hipLaunchKernelGGL((conv_block_kernel<FA, 0u, 1, false, 1, true>), grid, block, lds, s, g);
+}
+
+void launch_block_dw(const ConvArgs& a, const BlockGeometry& geo, int images, hipStream_t s) {
+    BlockArgs g{};
+    g.a = a;
+    g.a.rows_per_tile = geo.rows;
+    g.a.tiles_per_image = geo.tiles_per_image;
+    g.a.patch_w = geo.patch_w;
+    g.a.inv_patch_w = 1.0f / static_cast<float>(geo.patch_w);
+    g.a.p_tiles = images * geo.tiles_per_image;
+    g.csa = 1;
+    g.ppix = geo.ppix;
+    g.p_per_xcd = g.a.p_tiles >= 16 ? static_cast<int32_t>(ceil_div(g.a.p_tiles, 8)) : 0;
+#ifdef HIPIE_BLOCK_STAMPS
+    g.stamps = nullptr;
+#endif
+    const int slabs = static_cast<int>(ceil_div(a.OC, 64));
+    HIPIE_REQUIRE(slabs >= 1 && slabs <= 65535 && a.OCp >= slabs * 64, HIPIE_GENERAL_ERROR, "depthwise block kernel: %d channels", a.OC);
+    switch (block_index(kBlockDepthwise, a.flags)) {
+    case 0: launch_block_dw_instance<kBlockDepthwise[0]>(g, slabs, geo.lds, s); break;
+    case 1: launch_block_dw_instance<kBlockDepthwise[1]>(g, slabs, geo.lds, s); break;
+    case 2: launch_block_dw_instance<kBlockDepthwise[2]>(g, slabs, geo.lds, s); break;
+    default: fail(HIPIE_GENERAL_ERROR, "depthwise block kernel: no instance for epilogue %#x", a.flags);
+    }
 }
 
 #ifdef HIPIE_BLOCK_STAMPS

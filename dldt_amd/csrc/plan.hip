@@ -151,6 +151,7 @@ struct Step {
     virtual int launches() const { return 1; }   // kernels the step enqueues
     // vector instructions x lanes the step's f32 chain needs per inference (results x epilogue_valu_ops); 0: not counted
     virtual double valu_ops() const { return 0.0; }
+    virtual uint32_t epilogue_flags() const { return 0u; }   // the fused f32 chain of a convolution step as its flag word
 };
 
 void check_status(int st, const char* what) {
@@ -256,6 +257,11 @@ struct ConvStep : Step {
         return r;
     }
     int launches() const override { return shortcut && !fused ? 2 : 1; }
+    uint32_t epilogue_flags() const override {
+        uint32_t flags = 0;
+        int specialised = 0;
+        return conv && hipie_conv_epilogue_flags(conv, &flags, &specialised) == HIPIE_OK ? flags : 0u;
+    }
     double valu_ops() const override {
         uint32_t flags = 0;
         int specialised = 0;
@@ -306,8 +312,11 @@ struct ConvStep : Step {
         float best_ms = 0.f, few_ms = -1.f;
         const int candidates[] = {current, 0, 1, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20, 21, 22, 23, 24, 24 + 32};
         for (size_t c = 0; c < sizeof(candidates) / sizeof(candidates[0]); ++c) {
-            const int tile = candidates[c] & 31;
-            if (c > 0 && candidates[c] == current) continue;
+            // (1 stands for 2 as well on a depthwise layer, whose third variant is the matrix-pipe form; the dense variant 2
+            // is a tile shape that no layer of a batch wants)
+            for (int alt = 0; alt < (desc.groups > 1 && candidates[c] == 1 ? 2 : 1); ++alt) {
+            const int tile = alt ? 2 : (candidates[c] & 31);
+            if (c > 0 && candidates[c] == current && !alt) continue;
             if (hipie_conv_set_tile(conv, tile) != HIPIE_OK) continue;
             int applied = -1;
             check_status(hipie_conv_get_tile(conv, &applied), name.c_str());
@@ -334,11 +343,12 @@ struct ConvStep : Step {
             }
             // a variant has to beat the best so far by more than the timing noise of seven launches,
             // otherwise the choice (and the run-to-run spread of a whole network) follows the noise
-            if (c == 0 || ms < 0.97f * best_ms) {
+            if ((c == 0 && !alt) || ms < 0.97f * best_ms) {
                 best_ms = ms;
-                best = candidates[c];
+                best = alt ? 2 : candidates[c];
             }
             if (tile == 23) few_ms = ms;
+            }
         }
         // The candidates are timed back to back, their weights hot in the caches; in the network every other layer's
         // weights and tensors pass through between two uses.  A layer of a few pixels is little else than its weight
@@ -2937,6 +2947,7 @@ int hipie_plan_step_rt_info(const hipie_plan* p, int index, const char* key, cha
         else if (k == "primitiveType") v = s.variant() >= 0 ? "hip_int8_v" + std::to_string(s.variant()) : "hip";
         else if (k == "kernels") v = std::to_string(s.launches());
         else if (k == "valuOps") v = std::to_string(static_cast<long long>(s.valu_ops()));
+        else if (k == "epilogueFlags") v = std::to_string(s.epilogue_flags());
         else if (k == "outputDims") v = s.output_dims;
         else fail(HIPIE_NOT_FOUND, "hipie_plan_step_rt_info: key '%s' (execTimeMcs is hipie_request_perf)", key);
         copy_text(v, buf, cap, "hipie_plan_step_rt_info");

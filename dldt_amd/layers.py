@@ -2,6 +2,7 @@
 """Layer by layer: what each kernel of a plan could take at best, beside what it takes.
 
     python3 -m dldt_amd.layers                       # ResNet-50 INT8 batch 64: markdown table on stdout
+    python3 -m dldt_amd.layers --model mobilenet_v2  # MobileNetV2-1.0 INT8
     python3 -m dldt_amd.layers --steps-json s.json   # ... and the rows as JSON, followed by 20 inferences back to back on
                                                      #     one request, the last kernels the process launches
     python3 -m dldt_amd.layers --join trace.csv s.json   # the same table with the durations of a kernel trace of that run
@@ -139,6 +140,7 @@ def join(trace_csv, steps_json):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--model", choices=("resnet50", "mobilenet_v2"), default="resnet50")
     ap.add_argument("--steps-json")
     ap.add_argument("--join", nargs=2, metavar=("TRACE_CSV", "STEPS_JSON"))
     args = ap.parse_args()
@@ -152,7 +154,7 @@ def main():
     import torch
     from . import builders
     assert torch.cuda.is_available(), "needs a GPU"
-    g, _ = builders.resnet50(batch=args.batch, res=224)
+    g, _ = (builders.resnet50 if args.model == "resnet50" else builders.mobilenet_v2)(batch=args.batch, res=224)
     plan = g.compile(0)
     req = plan.create_request()
     ins, outs = req.device_buffers()

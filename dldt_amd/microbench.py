@@ -184,7 +184,7 @@ def config4():
                                          clamp=(0.0, 6.0), out_dtype=U8B, fq=fq))
         oh = (hw + 2 - 3) // stride + 1
         out = DeviceTensor(64, oh, oh, c, U8B)
-        for variant in (0, 1):
+        for variant in (0, 1, 2):
             conv.set_tile(variant)
             rows.append(_row("cfg4 depthwise 3x3 s%d C=%d @%dx%d batch 64, variant %d" % (stride, c, hw, hw, variant),
                              _time(lambda: conv.run(xin, out)), macs=64 * oh * oh * c * 9,

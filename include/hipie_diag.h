@@ -36,10 +36,13 @@ extern "C" {
  * bias + 256-level FakeQuantize from 0; rows too wide for a tile run variant 0).  A default is chosen
  * from the shape; hipie_compile times the variants on the device and keeps the fastest.  Every
  * variant produces the same bits.
- * A depthwise convolution (group_convolution.hpp:78-144 with one filter per channel) has two variants of its own:
+ * A depthwise convolution (group_convolution.hpp:78-144 with one filter per channel) has three variants of its own:
  * 0 = every lane computes its outputs from registers loaded straight from memory, 1 = the input rows under seven
  * output rows of a strip of columns are staged once in LDS and a lane slides the 3 x 3 window over them in registers
- * (3 x 3, undilated, stride 1 or 2, pixels of at most 1024 bytes, FakeQuantize epilogue without residual). */
+ * (3 x 3, undilated, stride 1 or 2, pixels of at most 1024 bytes, FakeQuantize epilogue without residual), 2 = the
+ * taps' diagonal weight matrices on the matrix pipe, 256 pixels x 64 channels per workgroup from an input patch staged
+ * once in LDS (3 x 3, undilated, stride 1 or 2, padding 1 on the top and left, input with a border of one pixel;
+ * an output row wider than 256 pixels runs variant 0). */
 int hipie_conv_set_tile(hipie_conv* conv, int tile);
 int hipie_conv_get_tile(const hipie_conv* conv, int* tile);
 /* diagnostics: the epilogue's step flags (conv_kernel.h ConvFlags) and whether a kernel instance with

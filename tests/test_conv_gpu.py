@@ -390,15 +390,20 @@ def test_depthwise_strip_variant_exact(orc, geo, tail):
     want = want.astype(np.uint8)
     conv = Convolution(w.astype(np.int8), xin, st, (1, 1), pb, pe, make_epilogue(out_dtype=U8B, **kw))
     got = {}
-    for variant in (0, 1):
+    for variant in (0, 1, 2):
+        if variant == 2 and pb != (1, 1):          # the matrix-pipe form is built for a padding of one on the top and left
+            with pytest.raises(Exception):
+                conv.set_tile(2)
+            continue
         conv.set_tile(variant)
         assert conv.get_tile() == variant
         out8 = DeviceTensor(N, OH, OW, C, U8B)
         out8.interior().fill_(77)
         conv.run(xin, out8)
         got[variant] = out8.to_nchw()
-    np.testing.assert_array_equal(got[1], want)
-    np.testing.assert_array_equal(got[0], want)
+        assert np.all(out8.padded_channels() == 0), "variant %d" % variant
+    for variant, levels in got.items():
+        np.testing.assert_array_equal(levels, want, err_msg="variant %d" % variant)
 
 
 @pytest.mark.parametrize("N,C,H,W,stride", [(2, 144, 9, 11, 1), (1, 16, 5, 3, 1), (3, 48, 13, 40, 2), (2, 96, 17, 17, 2),
@@ -430,7 +435,7 @@ def test_depthwise_variants_with_per_channel_zero_points(orc, N, C, H, W, stride
                        make_epilogue(bias=bias, scale=scale, activation="clamp", clamp=(0.0, 6.0), out_dtype=U8B, fq=fq),
                        zero_point=zp)
     ran = []
-    for variant in (0, 1):
+    for variant in (0, 1, 2):
         try:
             conv.set_tile(variant)
         except HipieError:
@@ -441,7 +446,7 @@ def test_depthwise_variants_with_per_channel_zero_points(orc, N, C, H, W, stride
         conv.run(xin, out8)
         np.testing.assert_array_equal(out8.to_nchw(), want, err_msg="variant %d" % variant)
         ran.append(variant)
-    assert 0 in ran and (1 in ran or C > 1024)
+    assert 0 in ran and 2 in ran and (1 in ran or C > 1024)
 
 
 def test_depthwise_strip_variant_is_refused_where_it_does_not_apply():
