@@ -141,6 +141,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--model", choices=("resnet50", "mobilenet_v2"), default="resnet50")
+    ap.add_argument("--tune-streams", type=int, default=0, help="requests the kernels are chosen for at load (0: the library's default)")
     ap.add_argument("--steps-json")
     ap.add_argument("--join", nargs=2, metavar=("TRACE_CSV", "STEPS_JSON"))
     args = ap.parse_args()
@@ -155,7 +156,7 @@ def main():
     from . import builders
     assert torch.cuda.is_available(), "needs a GPU"
     g, _ = (builders.resnet50 if args.model == "resnet50" else builders.mobilenet_v2)(batch=args.batch, res=224)
-    plan = g.compile(0)
+    plan = g.compile(0, config={"HIP_THROUGHPUT_STREAMS": str(args.tune_streams)} if args.tune_streams else None)
     req = plan.create_request()
     ins, outs = req.device_buffers()
     for t in ins:
