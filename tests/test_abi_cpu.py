@@ -236,6 +236,18 @@ def test_exec_graph_attributes_per_step():
     assert all(len(src[i]) == 2 for i, r in enumerate(info) if r["layerType"] == "Convolution,Convolution")
     assert info[-1]["layerType"] == "Result" and set(range(len(info) - 1)) == {v for s in src for v in s if v >= 0}
     assert plan.step_rt_info(1, "outputDims") == "1,64,112,112"
+    # the vector work of a step's f32 chain (results x instructions of its epilogue) and the chain's flag word: the stem
+    # is bias + FakeQuantize from 0 with the two-operation division, 6.25 instructions for each of 64 x 112 x 112 results
+    assert int(plan.step_rt_info(1, "epilogueFlags")) & ~(1 << 14) == 338433
+    assert int(plan.step_rt_info(1, "valuOps")) == int(6.25 * 64 * 112 * 112)
+    assert int(plan.step_rt_info(0, "valuOps")) == 0 and int(plan.step_rt_info(0, "epilogueFlags")) == 0
+    from dldt_amd.layers import attainable, floors
+    steps = [dict(s, valu_ops=int(plan.step_rt_info(i, "valuOps")), ms=1e-3) for i, s in enumerate(plan.steps)]
+    f = floors(steps[1])
+    assert f["mfma_us"] == pytest.approx(2 * steps[1]["macs"] / 5e15 * 1e6) and f["valu_us"] == pytest.approx(5017600 / 39.3216e12 * 1e6)
+    assert f["attainable_us"] == max(f["mfma_us"], f["valu_us"], f["hbm_us"]) and f["bound"] in ("mfma", "valu", "hbm")
+    a = attainable(steps)
+    assert a["measured_ms"] == pytest.approx(1e-3 * len(steps)) and 0 < a["frac"] and sum(a["bounds"].values()) == len(steps)
     with pytest.raises(HipieError) as e:
         plan.step_rt_info(0, "execTimeMcs")
     assert e.value.status == -5
