@@ -500,7 +500,9 @@ int hipie_plan_step_variant(const hipie_plan* plan, int index, int* variant);
  * integer kernels: the type of the activations they multiply, as the CPU plugin reports it; FP32 otherwise),
  * outputPrecisions, outputLayouts, execOrder, primitiveType ("hip_int8_v<variant>" | "hip"); execTimeMcs is
  * hipie_request_perf.  HIPIE_NOT_FOUND for another key.  Beside the reference's keys: "kernels" (launches the
- * step enqueues) and "outputDims" (the shape of what it stores, comma separated, in the graph's dimension order). */
+ * step enqueues), "outputDims" (the shape of what it stores, comma separated, in the graph's dimension order),
+ * "epilogueFlags" (the f32 chain fused behind a convolution as its flag word, 0 for other steps) and "valuOps" (results
+ * x vector instructions of that chain: what the step asks of the vector pipe whatever kernel runs it). */
 int hipie_plan_step_rt_info(const hipie_plan* plan, int index, const char* key, char* buf, size_t buf_len);
 /* The edges of that graph: where the operands of step `index` come from - sources[i] >= 0 is the index of the step that
  * produced one, sources[i] < 0 stands for graph input -(1 + sources[i]).  *count receives their number (at most
