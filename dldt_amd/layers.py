@@ -2,7 +2,7 @@
 """Layer by layer: what each kernel of a plan could take at best, beside what it takes.
 
     python3 -m dldt_amd.layers                       # ResNet-50 INT8 batch 64: markdown table on stdout
-    python3 -m dldt_amd.layers --model mobilenet_v2  # MobileNetV2-1.0 INT8
+    python3 -m dldt_amd.layers --model mobilenet_v2  # MobileNetV2-1.0 INT8 (bert_encoder: the 12-layer encoder, batch 16 x 384)
     python3 -m dldt_amd.layers --steps-json s.json   # ... and the rows as JSON, followed by 20 inferences back to back on
                                                      #     one request, the last kernels the process launches
     python3 -m dldt_amd.layers --join trace.csv s.json   # the same table with the durations of a kernel trace of that run
@@ -140,7 +140,7 @@ def join(trace_csv, steps_json):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--model", choices=("resnet50", "mobilenet_v2"), default="resnet50")
+    ap.add_argument("--model", choices=("resnet50", "mobilenet_v2", "bert_encoder"), default="resnet50")
     ap.add_argument("--tune-streams", type=int, default=0, help="requests the kernels are chosen for at load (0: the library's default)")
     ap.add_argument("--steps-json")
     ap.add_argument("--join", nargs=2, metavar=("TRACE_CSV", "STEPS_JSON"))
@@ -155,12 +155,15 @@ def main():
     import torch
     from . import builders
     assert torch.cuda.is_available(), "needs a GPU"
-    g, _ = (builders.resnet50 if args.model == "resnet50" else builders.mobilenet_v2)(batch=args.batch, res=224)
+    if args.model == "bert_encoder":     # 12 layers, hidden 768, sequence 384; --batch 64 stands for its own batch of 16
+        g, _ = builders.bert_encoder(batch=16 if args.batch == 64 else args.batch)
+    else:
+        g, _ = (builders.resnet50 if args.model == "resnet50" else builders.mobilenet_v2)(batch=args.batch, res=224)
     plan = g.compile(0, config={"HIP_THROUGHPUT_STREAMS": str(args.tune_streams)} if args.tune_streams else None)
     req = plan.create_request()
     ins, outs = req.device_buffers()
     for t in ins:
-        t.copy_(torch.rand(t.shape, device="cuda"))
+        t.copy_(torch.rand(t.shape, device="cuda") if t.dtype == torch.float32 else torch.zeros(t.shape, device="cuda").to(t.dtype))
     torch.cuda.synchronize()
     steps, over = step_times(plan, ins, outs)
     print(table(steps))
