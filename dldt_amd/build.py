@@ -23,9 +23,10 @@ FLAGS = [
 ] + os.environ.get("HIPIE_EXTRA_FLAGS", "").split()
 
 
-# per-file additions from the environment (HIPIE_BLOCK_FLAGS="-DHIPIE_BLOCK_STAMPS" builds the bottleneck-tail kernel
-# with its cycle stamps; the library that ships is built without any)
-EXTRA = {"conv_block.hip": os.environ.get("HIPIE_BLOCK_FLAGS", "").split()}
+# per-file additions from the environment (HIPIE_BLOCK_FLAGS="-DHIPIE_BLOCK_STAMPS" builds the bottleneck-tail kernel,
+# HIPIE_ATTENTION_FLAGS="-DHIPIE_ATT_STAMPS" the attention kernel, with cycle stamps; the library that ships is built without any)
+EXTRA = {"conv_block.hip": os.environ.get("HIPIE_BLOCK_FLAGS", "").split(),
+         "attention.hip": os.environ.get("HIPIE_ATTENTION_FLAGS", "").split()}
 
 
 def _compile(src, force):

@@ -38,6 +38,9 @@ struct AttentionArgs {
     float p_zh, p_zl;                                 // probabilities: two-operation division by fq_p.p.d
     int p_div2;                                       // ... verified against IEEE division on the device
     int p_sat;                                        // input_low of the probabilities' FakeQuantize is +0 and it has 256 levels
+#ifdef HIPIE_ATT_STAMPS
+    long long* stamps;                                // probe builds only: cycle stamps per workgroup
+#endif
     uint32_t p_xor, p_add;                            // stored byte = level + out_low (mod 256): XOR 0x80 per byte, or bytewise add
     int p_bias;                                       // 128 when the probabilities are u8 levels (stored as level - 128), else 0
 };
@@ -71,26 +74,63 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, h = lane >> 5;
     const int b = blockIdx.y, bo = b / a.batch_inner, bi = b - bo * a.batch_inner;
+#ifdef HIPIE_ATT_STAMPS
+#define ATT_STAMP(i) do { if (a.stamps && tid == 0) a.stamps[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = clock64(); } while (0)
+#else
+#define ATT_STAMP(i)
+#endif
+    ATT_STAMP(0);
     const int8_t* qp = a.q + bo * a.oq + bi * a.sq;
+#ifdef HIPIE_ATT_NOSTAGE   // timing probe: every workgroup stages the same K and V (wrong results, no memory traffic to speak of)
+    const int8_t* kp = a.k;
+    const int8_t* vp = a.v;
+#else
     const int8_t* kp = a.k + bo * a.ok + bi * a.sk;
     const int8_t* vp = a.v + bo * a.ov + bi * a.sv;
+#endif
 
     // ---- K into LDS (rows of 64 bytes), V transposed into LDS ------------------------------------
-    for (int i = tid; i < S * 4; i += 256) {
-        const int r = i >> 2, c = i & 3;
-        const v4i x = *reinterpret_cast<const v4i*>(kp + r * a.ldk + c * 16);
-        *reinterpret_cast<v4i*>(&sK[r * 64 + ((c ^ ((r >> 2) & 3)) * 16)]) = x;
+    // Every load of the staging is requested before the first is used: a round trip to memory in all, where a loop of
+    // load-and-store iterations pays one per iteration (a third of the kernel's time at S = 384).
+    constexpr int KI = (S * 4 + 255) / 256;           // 16-byte pieces of K per thread; and groups of 4 keys x 4 d of V
+    v4i kx[KI];
+    uint32_t vw[KI][4];
+#pragma unroll
+    for (int j = 0; j < KI; ++j) {
+        const int i = min(tid + j * 256, S * 4 - 1);
+        kx[j] = *reinterpret_cast<const v4i*>(kp + (i >> 2) * a.ldk + (i & 3) * 16);
     }
+#pragma unroll
+    for (int j = 0; j < KI; ++j) {
+        const int i = min(tid + j * 256, S * 4 - 1);
+        const int d4 = i & 15, kq = i >> 4;            // 4 consecutive keys x 4 consecutive d
+#pragma unroll
+        for (int q = 0; q < 4; ++q) vw[j][q] = *reinterpret_cast<const uint32_t*>(vp + (4 * kq + q) * a.ldv + 4 * d4);
+    }
+    // ---- this wave's queries: the column operand of the first product, straight from memory ------
+    const int q_row = blockIdx.x * 128 + wave * 32 + l32;
+    const bool q_ok = q_row < a.S;
+    const int8_t* qrow = qp + static_cast<int64_t>(q_ok ? q_row : a.S - 1) * a.ldq;
+    const v4i qf[2] = {*reinterpret_cast<const v4i*>(qrow + 16 * h), *reinterpret_cast<const v4i*>(qrow + 32 + 16 * h)};
     if (a.p_bias) {
         if (tid < 64) sVsum[tid] = 0;
         __syncthreads();
     }
-    int32_t vsum[4] = {0, 0, 0, 0};                     // this thread's share of the sums (d4 = tid % 16 in every round)
-    for (int i = tid; i < (S / 4) * 16; i += 256) {
-        const int d4 = i & 15, kq = i >> 4;            // 4 consecutive keys x 4 consecutive d
-        uint32_t w[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) w[j] = *reinterpret_cast<const uint32_t*>(vp + (4 * kq + j) * a.ldv + 4 * d4);
+    for (int j = 0; j < KI; ++j) {
+        const int i = tid + j * 256;
+        if (i < S * 4) {
+            const int r = i >> 2, c = i & 3;
+            *reinterpret_cast<v4i*>(&sK[r * 64 + ((c ^ ((r >> 2) & 3)) * 16)]) = kx[j];
+        }
+    }
+    int32_t vsum[4] = {0, 0, 0, 0};                     // this thread's share of the sums (d4 = tid % 16 in every round)
+#pragma unroll
+    for (int j = 0; j < KI; ++j) {
+        const int i = tid + j * 256;
+        if (i >= S * 4) continue;
+        const int d4 = i & 15, kq = i >> 4;
+        const uint32_t* w = vw[j];
         // 4 x 4 byte transpose: t[e] = bytes e of w[0..3]
         const uint32_t lo01 = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u);   // w0.b0 w1.b0 w0.b1 w1.b1
         const uint32_t hi01 = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);   // w0.b2 w1.b2 w0.b3 w1.b3
@@ -116,24 +156,37 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
         for (int i = tid; i < S; i += 256) sMask[i] = mrow[i];
     }
 
-    // ---- this wave's queries: the column operand of the first product, straight from memory ------
-    const int q_row = blockIdx.x * 128 + wave * 32 + l32;
-    const bool q_ok = q_row < a.S;
-    const int8_t* qrow = qp + static_cast<int64_t>(q_ok ? q_row : a.S - 1) * a.ldq;
-    const v4i qf[2] = {*reinterpret_cast<const v4i*>(qrow + 16 * h), *reinterpret_cast<const v4i*>(qrow + 32 + 16 * h)};
+    ATT_STAMP(1);
     __syncthreads();
+    ATT_STAMP(2);
 
     const int slot[2] = {((0 + h) ^ ((l32 >> 2) & 3)) * 16, ((2 + h) ^ ((l32 >> 2) & 3)) * 16};
-    float x[NT][16];
-    float m = -INFINITY;
+    v16i ctx[2] = {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}};
+    const int64_t dump_row = (static_cast<int64_t>(b) * a.S + q_row) * a.S;   // [batch][query][key]
+    constexpr float kLog2e = 1.4426950408889634f;
+    auto init_ctx = [&]() {
+        if (a.p_bias) {     // register r of block db holds d = 32 db + 8 (r / 4) + 4 h + r % 4
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
+            for (int db = 0; db < 2; ++db)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const v4i sv = *reinterpret_cast<const v4i*>(&sVsum[32 * db + 8 * g + 4 * h]);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) ctx[db][4 * g + j] = sv[j] * a.p_bias;
+                }
+        }
+    };
+    // the integer scores of key tile t, and from them the f32 scores (Multiply by the scale, then the mask's Add)
+    auto raw_scores = [&](int t) {
         v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             const v4i kf = *reinterpret_cast<const v4i*>(&sK[(32 * t + l32) * 64 + slot[ks]]);
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[ks], acc, 0, 0, 0);
         }
+        return acc;
+    };
+    auto f32_scores = [&](int t, const v16i& acc, float (&v)[16]) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             float mv[4] = {0.f, 0.f, 0.f, 0.f};
@@ -143,15 +196,37 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                float v = static_cast<float>(acc[4 * g + j]) * a.scale1;
-                if constexpr (MASK) v = v + mv[j];       // the mask Add between the Multiply and the Softmax
-                x[t][4 * g + j] = v;
-                m = fmaxf(m, v);
+                float x = static_cast<float>(acc[4 * g + j]) * a.scale1;
+                if constexpr (MASK) x = x + mv[j];       // the mask Add between the Multiply and the Softmax
+                v[4 * g + j] = x;
             }
         }
+    };
+    // probabilities of a tile -> levels -> second product
+    auto finish_tile = [&](int t, const float (&e)[16], float inv) {
+        v4i pf;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const float4 p4 = make_float4(e[4 * g] * inv, e[4 * g + 1] * inv, e[4 * g + 2] * inv, e[4 * g + 3] * inv);
+            if (a.probs && q_ok)
+                *reinterpret_cast<float4*>(a.probs + dump_row + 32 * t + 8 * g + 4 * h) = p4;
+            pf[g] = static_cast<int>(prob_levels4<DIV2, PSAT>(a, p4.x, p4.y, p4.z, p4.w));
+        }
+#pragma unroll
+        for (int db = 0; db < 2; ++db) {
+            const v4i vf = *reinterpret_cast<const v4i*>(&sVT[(32 * db + l32) * VT_LD + 32 * t + 16 * h]);
+            ctx[db] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf, ctx[db], 0, 0, 0);
+        }
+    };
+    float x[NT][16];
+    float m = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        f32_scores(t, raw_scores(t), x[t]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) m = fmaxf(m, x[t][r]);
         if constexpr (MASK) __builtin_amdgcn_sched_barrier(0);   // keep the mask reads next to their tile
     }
-    const int64_t dump_row = (static_cast<int64_t>(b) * a.S + q_row) * a.S;   // [batch][query][key]
     if (a.scores && q_ok) {
 #pragma unroll
         for (int t = 0; t < NT; ++t)
@@ -162,7 +237,6 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
     // exp(x - m) as 2^((x - m) log2 e) on the hardware's exp2, the division as a multiplication by the
     // reciprocal of the sum: within the tolerance the stand-alone kernel is held to.
     m = fmaxf(m, __shfl_xor(m, 32, 64));
-    constexpr float kLog2e = 1.4426950408889634f;
     const float mL = -m * kLog2e;
     float s = 0.f;
 #pragma unroll
@@ -174,36 +248,12 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
         }
     s += __shfl_xor(s, 32, 64);
     const float inv = 1.0f / s;
-
     // probabilities -> i8 levels -> second product, one 32-key tile at a time
-    v16i ctx[2] = {{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}};
-    if (a.p_bias) {     // register r of block db holds d = 32 db + 8 (r / 4) + 4 h + r % 4
+    init_ctx();
 #pragma unroll
-        for (int db = 0; db < 2; ++db)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const v4i sv = *reinterpret_cast<const v4i*>(&sVsum[32 * db + 8 * g + 4 * h]);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) ctx[db][4 * g + j] = sv[j] * a.p_bias;
-            }
-    }
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        v4i pf;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const float4 p4 = make_float4(x[t][4 * g] * inv, x[t][4 * g + 1] * inv, x[t][4 * g + 2] * inv, x[t][4 * g + 3] * inv);
-            if (a.probs && q_ok)
-                *reinterpret_cast<float4*>(a.probs + dump_row + 32 * t + 8 * g + 4 * h) = p4;
-            pf[g] = static_cast<int>(prob_levels4<DIV2, PSAT>(a, p4.x, p4.y, p4.z, p4.w));
-        }
-#pragma unroll
-        for (int db = 0; db < 2; ++db) {
-            const v4i vf = *reinterpret_cast<const v4i*>(&sVT[(32 * db + l32) * VT_LD + 32 * t + 16 * h]);
-            ctx[db] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf, ctx[db], 0, 0, 0);
-        }
-    }
+    for (int t = 0; t < NT; ++t) finish_tile(t, x[t], inv);
 
+    ATT_STAMP(5);
     // ---- context of query q_row: d = 32 db + 8 (r / 4) + 4 h + r % 4 --------------------------------
     if (!q_ok) return;
     const int64_t orow = bo * a.oo + bi * a.so + static_cast<int64_t>(q_row) * a.ldo;
@@ -223,21 +273,28 @@ template <int NT>
 void launch(const AttentionArgs& a, int batches, hipStream_t s) {
     const dim3 grid(static_cast<uint32_t>(ceil_div(a.S, 128)), static_cast<uint32_t>(batches));
     const bool sat = a.p_div2 && a.p_sat;             // (the form without clamp: compiled for the usual division only)
-    if (a.mask) {
-        if (sat) hipLaunchKernelGGL((attention_kernel<NT, true, true, true>), grid, dim3(256), 0, s, a);
-        else if (a.p_div2) hipLaunchKernelGGL((attention_kernel<NT, true, true, false>), grid, dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((attention_kernel<NT, false, true, false>), grid, dim3(256), 0, s, a);
-    } else {
-        if (sat) hipLaunchKernelGGL((attention_kernel<NT, true, false, true>), grid, dim3(256), 0, s, a);
-        else if (a.p_div2) hipLaunchKernelGGL((attention_kernel<NT, true, false, false>), grid, dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((attention_kernel<NT, false, false, false>), grid, dim3(256), 0, s, a);
+    const int form = (a.mask ? 4 : 0) + (sat ? 2 : (a.p_div2 ? 1 : 0));
+#define HIPIE_ATT_LAUNCH(D, M, P) hipLaunchKernelGGL((attention_kernel<NT, D, M, P>), grid, dim3(256), 0, s, a)
+    switch (form) {
+    case 0: HIPIE_ATT_LAUNCH(false, false, false); break;
+    case 1: HIPIE_ATT_LAUNCH(true, false, false); break;
+    case 2: HIPIE_ATT_LAUNCH(true, false, true); break;
+    case 4: HIPIE_ATT_LAUNCH(false, true, false); break;
+    case 5: HIPIE_ATT_LAUNCH(true, true, false); break;
+    default: HIPIE_ATT_LAUNCH(true, true, true); break;
     }
+#undef HIPIE_ATT_LAUNCH
 }
 
 }  // namespace
 }  // namespace hipie
 
 using namespace hipie;
+
+#ifdef HIPIE_ATT_STAMPS
+static long long* g_att_stamps = nullptr;
+extern "C" void hipie_debug_attention_stamps(long long* p) { g_att_stamps = p; }
+#endif
 
 struct hipie_attention {
     int device = 0;
@@ -320,6 +377,9 @@ int hipie_attention_run(const hipie_attention* att, const void* q, int64_t ldq, 
         a.scores = scores; a.probs = probs;
         a.mask = mask; a.mask_inner = mask_stride; a.mask_outer = mask_outer;
         a.batch_inner = batch;
+#ifdef HIPIE_ATT_STAMPS
+        a.stamps = g_att_stamps;
+#endif
         DeviceGuard dg(att->device);
         hipStream_t s = as_stream(stream);
         const int batches = batch * batch_outer;
