@@ -38,6 +38,8 @@ struct AttentionArgs {
     float p_zh, p_zl;                                 // probabilities: two-operation division by fq_p.p.d
     int p_div2;                                       // ... verified against IEEE division on the device
     int p_sat;                                        // input_low of the probabilities' FakeQuantize is +0 and it has 256 levels
+    int qblocks;                                      // blocks of 128 queries per batch element
+    int xcd_groups;                                   // 1: a one-dimensional grid that keeps the blocks of two neighbouring batch elements on one XCD
 #ifdef HIPIE_ATT_STAMPS
     long long* stamps;                                // probe builds only: cycle stamps per workgroup
 #endif
@@ -73,9 +75,18 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, h = lane >> 5;
-    const int b = blockIdx.y, bo = b / a.batch_inner, bi = b - bo * a.batch_inner;
+    // Which queries of which batch element: plain (x = query block, y = batch element), or - consecutive workgroups go
+    // to consecutive XCDs, each with its own L2 - the blocks of a pair of neighbouring heads on one XCD: they stage the
+    // same K and V rows, and two neighbouring heads' 64-byte rows share the 128-byte lines of a [tokens, 3 hidden] tensor
+    int qblk = blockIdx.x, b = blockIdx.y;
+    if (a.xcd_groups) {
+        const int id = blockIdx.x, per = 2 * a.qblocks, k = id >> 3, sub = k % per;
+        b = ((k / per) * 8 + (id & 7)) * 2 + sub / a.qblocks;
+        qblk = sub % a.qblocks;
+    }
+    const int bo = b / a.batch_inner, bi = b - bo * a.batch_inner;
 #ifdef HIPIE_ATT_STAMPS
-#define ATT_STAMP(i) do { if (a.stamps && tid == 0) a.stamps[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = clock64(); } while (0)
+#define ATT_STAMP(i) do { if (a.stamps && tid == 0) a.stamps[(b * a.qblocks + qblk) * 8 + (i)] = clock64(); } while (0)
 #else
 #define ATT_STAMP(i)
 #endif
@@ -108,7 +119,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
         for (int q = 0; q < 4; ++q) vw[j][q] = *reinterpret_cast<const uint32_t*>(vp + (4 * kq + q) * a.ldv + 4 * d4);
     }
     // ---- this wave's queries: the column operand of the first product, straight from memory ------
-    const int q_row = blockIdx.x * 128 + wave * 32 + l32;
+    const int q_row = qblk * 128 + wave * 32 + l32;
     const bool q_ok = q_row < a.S;
     const int8_t* qrow = qp + static_cast<int64_t>(q_ok ? q_row : a.S - 1) * a.ldq;
     const v4i qf[2] = {*reinterpret_cast<const v4i*>(qrow + 16 * h), *reinterpret_cast<const v4i*>(qrow + 32 + 16 * h)};
@@ -270,8 +281,11 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
 }
 
 template <int NT>
-void launch(const AttentionArgs& a, int batches, hipStream_t s) {
-    const dim3 grid(static_cast<uint32_t>(ceil_div(a.S, 128)), static_cast<uint32_t>(batches));
+void launch(const AttentionArgs& a_in, int batches, hipStream_t s) {
+    AttentionArgs a = a_in;
+    a.qblocks = static_cast<int>(ceil_div(a.S, 128));
+    a.xcd_groups = batches % 16 == 0 ? 1 : 0;         // pairs of batch elements, eight pairs at a time
+    const dim3 grid = a.xcd_groups ? dim3(static_cast<uint32_t>(a.qblocks) * batches) : dim3(a.qblocks, static_cast<uint32_t>(batches));
     const bool sat = a.p_div2 && a.p_sat;             // (the form without clamp: compiled for the usual division only)
     const int form = (a.mask ? 4 : 0) + (sat ? 2 : (a.p_div2 ? 1 : 0));
 #define HIPIE_ATT_LAUNCH(D, M, P) hipLaunchKernelGGL((attention_kernel<NT, D, M, P>), grid, dim3(256), 0, s, a)

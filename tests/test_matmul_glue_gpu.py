@@ -262,7 +262,8 @@ def test_glue_requantisation_rejects_non_integer_levels():
         gelu(x, requant=(1.0, -1.0, -128, 256))
 
 
-@pytest.mark.parametrize("B,NH,S", [(2, 3, 384), (1, 2, 96), (2, 1, 160), (1, 1, 32)])
+@pytest.mark.parametrize("B,NH,S", [(2, 3, 384), (1, 2, 96), (2, 1, 160), (1, 1, 32),
+                                    (4, 4, 160), (2, 8, 64)])      # 16 batch elements: the grid that groups neighbouring heads per XCD
 def test_fused_attention(orc, B, NH, S):
     """scores bit-exact, Softmax within tolerance, and from the kernel's own probabilities the
     requantisation, the context product and its dequantisation (and requantisation) bit-exact; the
