@@ -1,0 +1,98 @@
+// f32 Convolution / GroupConvolution / MatMul against constants and FakeQuantize with an f32 result: the layers of an
+// INT8 network that the low-precision transformations leave unquantized.  See convf.h.
+#include "convf.h"
+
+namespace hipie {
+namespace {
+
+__device__ __forceinline__ float source_value(const F32Source& s, int n, int c, int h, int w) {
+    const int64_t i = n * s.sn + c * s.sc + h * s.sh + w * s.sw;
+    if (s.dtype == HIPIE_F32) return static_cast<const float*>(s.p)[i];
+    const int level = static_cast<int>(static_cast<const int8_t*>(s.p)[i]) + (s.dtype == HIPIE_U8B ? 128 : 0);
+    float v = static_cast<float>(level);            // Convert
+    if (s.sub) v = v - s.sub[c];                    // Subtract
+    if (s.mul) v = v * s.mul[c];                    // Multiply
+    return v;
+}
+
+__global__ __launch_bounds__(256) void conv_f32_kernel(const ConvF32Args a) {
+    const int64_t total = static_cast<int64_t>(a.N) * a.OH * a.OW * a.OC;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int oc = static_cast<int>(i % a.OC);
+    int64_t p = i / a.OC;
+    const int ow = static_cast<int>(p % a.OW);
+    p /= a.OW;
+    const int oh = static_cast<int>(p % a.OH);
+    const int n = static_cast<int>(p / a.OH);
+    const int cg = a.C / a.groups, ocg = a.OC / a.groups;
+    const int c0 = (oc / ocg) * cg;
+    const int y0 = oh * a.stride_h - a.pad_top, x0 = ow * a.stride_w - a.pad_left;
+    const float* w = a.wgt + oc;
+    float sum = 0.f;
+    for (int c = 0; c < cg; ++c)
+        for (int kh = 0; kh < a.KH; ++kh) {
+            const int y = y0 + kh * a.dil_h;
+            for (int kw = 0; kw < a.KW; ++kw) {
+                const int x = x0 + kw * a.dil_w;
+                if (y < 0 || y >= a.H || x < 0 || x >= a.W) continue;       // padding cells are skipped, not added as zeros
+                const float prod = source_value(a.in, n, c0 + c, y, x) * w[static_cast<int64_t>((c * a.KH + kh) * a.KW + kw) * a.OC];
+                sum = sum + prod;
+            }
+        }
+    a.out[n * a.out_sn + oh * a.out_sh + ow * a.out_sw + oc] = sum;
+}
+
+template <bool QUANTIZE>
+__global__ __launch_bounds__(256) void fq_f32_kernel(const FqF32Args a) {
+    const int64_t total = static_cast<int64_t>(a.N) * a.H * a.W * a.C;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int c = static_cast<int>(i % a.C);
+    int64_t p = i / a.C;
+    const int w = static_cast<int>(p % a.W);
+    p /= a.W;
+    const int h = static_cast<int>(p % a.H);
+    const int n = static_cast<int>(p / a.H);
+    float v = source_value(a.in, n, c, h, w);
+    if constexpr (QUANTIZE) v = fq_value<false>(a.ch[a.per_channel ? c : 0], a.lm1, v);
+    a.out[n * a.out_sn + h * a.out_sh + w * a.out_sw + c] = v;
+}
+
+void check_source(const F32Source& s, const char* what) {
+    HIPIE_REQUIRE(s.p && (s.dtype == HIPIE_F32 || s.dtype == HIPIE_U8B || s.dtype == HIPIE_I8), HIPIE_PARAMETER_MISMATCH,
+                  "%s: input of type %d", what, s.dtype);
+    HIPIE_REQUIRE(s.dtype != HIPIE_F32 || (!s.sub && !s.mul), HIPIE_PARAMETER_MISMATCH, "%s: dequantization constants on an f32 input", what);
+}
+
+}  // namespace
+
+void launch_conv_f32(const ConvF32Args& a, hipStream_t s) {
+    check_source(a.in, "f32 convolution");
+    HIPIE_REQUIRE(a.wgt && a.out && a.N > 0 && a.C > 0 && a.H > 0 && a.W > 0 && a.OC > 0 && a.OH > 0 && a.OW > 0 && a.KH > 0 && a.KW > 0 &&
+                      a.stride_h > 0 && a.stride_w > 0 && a.dil_h > 0 && a.dil_w > 0 && a.groups > 0 && a.C % a.groups == 0 &&
+                      a.OC % a.groups == 0,
+                  HIPIE_PARAMETER_MISMATCH, "f32 convolution: shape");
+    const int64_t total = static_cast<int64_t>(a.N) * a.OH * a.OW * a.OC;
+    const int64_t blocks = ceil_div(total, 256);
+    HIPIE_REQUIRE(blocks < (int64_t{1} << 31), HIPIE_PARAMETER_MISMATCH, "f32 convolution: %lld outputs", (long long)total);
+    hipLaunchKernelGGL(conv_f32_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s, a);
+    HIPIE_CHECK_HIP(hipGetLastError());
+}
+
+static void launch_elementwise_f32(const FqF32Args& a, bool quantize, hipStream_t s) {
+    const char* what = quantize ? "f32 FakeQuantize" : "f32 copy";
+    check_source(a.in, what);
+    HIPIE_REQUIRE((a.ch || !quantize) && a.out && a.N > 0 && a.C > 0 && a.H > 0 && a.W > 0 && a.lm1 >= 1.f, HIPIE_PARAMETER_MISMATCH, "%s: shape", what);
+    const int64_t total = static_cast<int64_t>(a.N) * a.H * a.W * a.C;
+    const int64_t blocks = ceil_div(total, 256);
+    HIPIE_REQUIRE(blocks < (int64_t{1} << 31), HIPIE_PARAMETER_MISMATCH, "%s: %lld elements", what, (long long)total);
+    if (quantize) hipLaunchKernelGGL(fq_f32_kernel<true>, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(fq_f32_kernel<false>, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s, a);
+    HIPIE_CHECK_HIP(hipGetLastError());
+}
+
+void launch_fq_f32(const FqF32Args& a, hipStream_t s) { launch_elementwise_f32(a, true, s); }
+void launch_copy_f32(const FqF32Args& a, hipStream_t s) { launch_elementwise_f32(a, false, s); }
+
+}  // namespace hipie

@@ -13,6 +13,7 @@
 #include <map>
 #include <mutex>
 
+#include "convf.h"
 #include "fq.h"
 #include "graph.h"
 #include "requant.h"
@@ -137,6 +138,7 @@ struct Step {
     std::string original_names, runtime_precision, output_precision, output_layout, output_dims;
     std::vector<int> nodes;      // the graph nodes the step stands for (its own and every node fused into it)
     std::vector<int> sources;    // where its operands come from: a step's index, or -(1 + k) for graph input k
+    bool f32_kernel = false;     // computes in f32 whatever type its operand is stored in (an unquantized layer)
     virtual ~Step() = default;
     virtual void create(int device, const std::vector<TensorInfo>& tensors) = 0;
     virtual void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs,
@@ -693,6 +695,98 @@ struct ExitStep : Step {
     }
 };
 
+
+// ---- layers left in f32 (convf.hip) --------------------------------------------------------------------------------
+
+// Where such a layer reads its [N, C, H, W] operand: an f32 request input (NCHW), an f32 tensor of the arena (NHWC), or
+// the bytes of a quantized tensor behind their dequantization constants
+struct F32Input {
+    int tensor = -1, param = -1;
+    int n = 1, c = 1, h = 1, w = 1;
+    std::vector<float> sub, mul;
+    DeviceBuffer d_sub, d_mul;
+    void upload(int device) {
+        auto up = [&](const std::vector<float>& v, DeviceBuffer& d) {
+            if (v.empty() || device < 0) return;
+            std::vector<float> o(static_cast<size_t>(c));
+            for (int i = 0; i < c; ++i) o[i] = v[v.size() == 1 ? 0 : i];
+            d.upload(device, o.data(), o.size() * 4);
+        };
+        up(sub, d_sub);
+        up(mul, d_mul);
+    }
+    F32Source source(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs) const {
+        F32Source s;
+        if (tensor >= 0) {
+            const hipie_tensor t = tensors[tensor].desc(arena);
+            s.p = t.data;
+            s.dtype = t.dtype;
+            s.sn = t.stride_n; s.sc = 1; s.sh = t.stride_h; s.sw = t.stride_w;
+        } else {
+            s.p = inputs[param];
+            s.dtype = HIPIE_F32;
+            s.sn = static_cast<int64_t>(c) * h * w; s.sc = static_cast<int64_t>(h) * w; s.sh = w; s.sw = 1;
+        }
+        s.sub = sub.empty() ? nullptr : d_sub.as<float>();
+        s.mul = mul.empty() ? nullptr : d_mul.as<float>();
+        return s;
+    }
+    int64_t bytes(const std::vector<TensorInfo>& tensors) const {
+        return static_cast<int64_t>(n) * c * h * w * (tensor >= 0 ? tensors[tensor].esize() : 4);
+    }
+};
+
+// Convolution / GroupConvolution / MatMul of an f32 value with f32 constant weights
+struct ConvF32Step : Step {
+    F32Input src;
+    int out = -1;
+    std::vector<float> weights;        // [C / G][KH][KW][OC]
+    DeviceBuffer d_weights;
+    ConvF32Args geo{};                 // the shape part
+    void create(int device, const std::vector<TensorInfo>&) override {
+        if (device < 0) return;
+        d_weights.upload(device, weights.data(), weights.size() * 4);
+        src.upload(device);
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*, hipStream_t s) const override {
+        ConvF32Args a = geo;
+        a.in = src.source(arena, tensors, inputs);
+        a.wgt = d_weights.as<float>();
+        const hipie_tensor t = tensors[out].desc(arena);
+        a.out = static_cast<float*>(t.data);
+        a.out_sn = t.stride_n; a.out_sh = t.stride_h; a.out_sw = t.stride_w;
+        launch_conv_f32(a, s);
+    }
+};
+
+// FakeQuantize with an f32 result; without channels: the operand as an NHWC f32 tensor, nothing else (a graph input
+// in front of stand-alone elementwise nodes, which read NHWC)
+struct FqF32Step : Step {
+    F32Input src;
+    int out = -1;
+    std::vector<FqChannel> channels;   // one, or one per channel; none: copy
+    DeviceBuffer d_channels;
+    float lm1 = 255.f;
+    void create(int device, const std::vector<TensorInfo>&) override {
+        if (device < 0) return;
+        if (!channels.empty()) d_channels.upload(device, channels.data(), channels.size() * sizeof(FqChannel));
+        src.upload(device);
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*, hipStream_t s) const override {
+        FqF32Args a;
+        a.in = src.source(arena, tensors, inputs);
+        a.ch = d_channels.as<FqChannel>();
+        a.per_channel = channels.size() > 1 ? 1 : 0;
+        a.lm1 = lm1;
+        const hipie_tensor t = tensors[out].desc(arena);
+        a.out = static_cast<float*>(t.data);
+        a.out_sn = t.stride_n; a.out_sh = t.stride_h; a.out_sw = t.stride_w;
+        a.N = src.n; a.C = src.c; a.H = src.h; a.W = src.w;
+        if (channels.empty()) launch_copy_f32(a, s);
+        else launch_fq_f32(a, s);
+    }
+};
+
 // ---- steps over row-major views (transformer encoders) ------------------------------------------
 
 // FakeQuantize of a dense f32 value with per-tensor bounds -> i8 levels
@@ -1042,6 +1136,7 @@ struct Planner {
         case OP_CONSTANT: values[id].kind = VK_CONST; break;
         case OP_FAKE_QUANTIZE:
             if (mat) plan_mat_fq(id);
+            else if (n.dtype == HIPIE_F32) plan_fq_f32(id);
             else if (value(n.in[0]).kind == VK_PARAM) plan_fake_quantize(id);
             else plan_eltwise(id);
             break;
@@ -1894,8 +1989,145 @@ struct Planner {
         values[id] = x;
     }
 
+    // ---- layers the transformations left in f32 -------------------------------------------------------------
+    // the operand of such a layer: an f32 graph input, an f32 tensor, or a byte tensor behind its dequantization
+    bool f32_input(int node, F32Input& o) {
+        const Value x = value(node);
+        const GNode& src = N(node);
+        if (src.shape.size() != 4 && src.shape.size() != 2) return false;
+        nhwc_dims(src.shape, o.n, o.c, o.h, o.w);
+        if (x.kind == VK_PARAM && src.op == OP_PARAMETER && src.dtype == HIPIE_F32) {
+            for (size_t i = 0; i < g.params.size(); ++i)
+                if (g.params[i] == node) o.param = static_cast<int>(i);
+            return o.param >= 0;
+        }
+        if (x.kind == VK_TENSOR && tensors[x.tensor].dtype == HIPIE_F32) {
+            o.tensor = x.tensor;
+        } else if (x.kind == VK_DEQ && tensors[x.tensor].esize() == 1) {
+            o.tensor = x.tensor;
+            o.sub = x.sub;
+            o.mul = x.mul;
+        } else {
+            return false;
+        }
+        const TensorInfo& t = tensors[o.tensor];
+        return t.n == o.n && t.c == o.c && t.h == o.h && t.w == o.w;
+    }
+
+    // an f32 graph input ([N, C, H, W] or [N, C], NCHW in the request's buffer) as an NHWC tensor of the arena, for the
+    // elementwise nodes that read it directly (mean / scale preprocessing in front of the first FakeQuantize)
+    std::map<int, int> param_tensors;
+    int param_as_tensor(int node) {
+        const auto found = param_tensors.find(node);
+        if (found != param_tensors.end()) return found->second;
+        auto st = std::make_unique<FqF32Step>();
+        const bool ok = f32_input(node, st->src) && st->src.param >= 0;
+        HIPIE_REQUIRE(ok, HIPIE_GENERAL_ERROR, "node %d is not an f32 graph input of rank 2 or 4", node);
+        st->out = new_tensor(node, HIPIE_F32, st->src.n, st->src.h, st->src.w, st->src.c);
+        st->name = N(node).name;
+        st->type = "Reorder";
+        st->bytes = N(node).numel() * 8;
+        param_tensors[node] = st->out;
+        const int t = st->out;
+        steps.push_back(std::move(st));
+        return t;
+    }
+
+    // Convolution / GroupConvolution / MatMul whose weights are an f32 constant: no FakeQuantize stood in front of the
+    // layer, or the transformations did not take it (convolution.cpp:84-120, weightable_layer_transformation.cpp); the
+    // layer runs as the graph says, in f32, and the nodes behind it are planned on their own
+    void plan_conv_f32(int id) {
+        const GNode& n = N(id);
+        const GNode& W = N(n.in[1]);
+        const bool is_mm = n.op == OP_MATMUL, grouped = n.op == OP_GROUP_CONVOLUTION;
+        auto st = std::make_unique<ConvF32Step>();
+        if (!f32_input(n.in[0], st->src))
+            unsupported(id, "an f32 layer reads an f32 graph input, an f32 tensor or a dequantized byte tensor of rank 2 or 4");
+        ConvF32Args& a = st->geo;
+        const float* w = W.f32();
+        int64_t G = 1, ocg = 0, icg = 0, KH = 1, KW = 1;
+        if (is_mm) {
+            if (n.ta || W.shape.size() != 2 || N(n.in[0]).shape.size() != 2)
+                unsupported(id, "MatMul is planned for [N,K] x constant [K,OC] / [OC,K]^T");
+            icg = n.tb ? W.shape[1] : W.shape[0];
+            ocg = n.tb ? W.shape[0] : W.shape[1];
+            st->weights.resize(static_cast<size_t>(icg * ocg));
+            for (int64_t k = 0; k < icg; ++k)
+                for (int64_t o = 0; o < ocg; ++o) st->weights[static_cast<size_t>(k * ocg + o)] = n.tb ? w[o * icg + k] : w[k * ocg + o];
+        } else {
+            if (N(n.in[0]).shape.size() != 4 || W.shape.size() != (grouped ? 5u : 4u)) unsupported(id, "f32 convolutions are planned over two spatial dimensions");
+            const size_t b = grouped ? 1 : 0;
+            G = grouped ? W.shape[0] : 1;
+            ocg = W.shape[b]; icg = W.shape[b + 1]; KH = W.shape[b + 2]; KW = W.shape[b + 3];
+            const int64_t OCa = G * ocg;
+            st->weights.resize(static_cast<size_t>(OCa * icg * KH * KW));
+            for (int64_t oc = 0; oc < OCa; ++oc)
+                for (int64_t c = 0; c < icg; ++c)
+                    for (int64_t t = 0; t < KH * KW; ++t)
+                        st->weights[static_cast<size_t>((c * KH * KW + t) * OCa + oc)] = w[(oc * icg + c) * KH * KW + t];
+            a.stride_h = static_cast<int>(n.strides[0]); a.stride_w = static_cast<int>(n.strides[1]);
+            a.dil_h = static_cast<int>(n.dilations[0]); a.dil_w = static_cast<int>(n.dilations[1]);
+            a.pad_top = static_cast<int>(n.pads_begin[0]); a.pad_left = static_cast<int>(n.pads_begin[1]);
+        }
+        const int64_t OC = G * ocg, IC = G * icg;
+        HIPIE_REQUIRE(st->src.c == IC, HIPIE_PARAMETER_MISMATCH, "node %d: input has %d channels, weights %lld", id, st->src.c, (long long)IC);
+        int nn, c, h, ww;
+        nhwc_dims(n.shape, nn, c, h, ww);
+        HIPIE_REQUIRE(c == OC && nn == st->src.n, HIPIE_PARAMETER_MISMATCH, "node %d: output shape against the weights", id);
+        a.N = nn; a.C = static_cast<int>(IC); a.H = st->src.h; a.W = st->src.w; a.OC = c; a.OH = h; a.OW = ww;
+        a.KH = static_cast<int>(KH); a.KW = static_cast<int>(KW); a.groups = static_cast<int>(G);
+        st->out = new_tensor(id, HIPIE_F32, nn, h, ww, c);
+        st->name = n.name;
+        st->type = is_mm ? "MatMul" : (grouped ? "GroupConvolution" : "Convolution");
+        st->f32_kernel = true;
+        st->macs = n.numel() * icg * KH * KW;
+        st->bytes = st->src.bytes(tensors) + static_cast<int64_t>(st->weights.size()) * 4 + n.numel() * 4;
+        st->out_node = id;
+        values[id].kind = VK_TENSOR;
+        values[id].tensor = st->out;
+        steps.push_back(std::move(st));
+    }
+
+    // FakeQuantize whose result stays f32 (the layer behind it was not transformed): fake_quantize.hpp:175-194 as it stands
+    void plan_fq_f32(int id) {
+        const GNode& n = N(id);
+        auto st = std::make_unique<FqF32Step>();
+        if (!f32_input(n.in[0], st->src))
+            unsupported(id, "FakeQuantize with an f32 result reads an f32 graph input, an f32 tensor or a dequantized byte tensor of rank 2 or 4");
+        std::vector<float> b[4];
+        size_t count = 1;
+        for (int i = 0; i < 4; ++i) {
+            if (!channel_constant(n.in[1 + i], st->src.c, n.shape.size(), b[i]))
+                unsupported(id, "FakeQuantize bounds must be scalars or per-channel constants");
+            count = std::max(count, b[i].size());
+        }
+        HIPIE_REQUIRE(n.levels >= 2, HIPIE_PARAMETER_MISMATCH, "node %d: %lld levels", id, (long long)n.levels);
+        st->lm1 = static_cast<float>(n.levels - 1);
+        st->channels.resize(count);
+        for (size_t ch = 0; ch < count; ++ch) {
+            auto at = [&](int i) { return b[i][b[i].size() == 1 ? 0 : ch]; };
+            FqChannel& f = st->channels[ch];
+            f.il = at(0); f.ih = at(1); f.ol = at(2); f.oh = at(3);
+            f.lo = std::min(f.il, f.ih); f.hi = std::max(f.il, f.ih);
+            f.d = f.ih - f.il;
+            f.r = 0.f;
+        }
+        st->out = new_tensor(id, HIPIE_F32, st->src.n, st->src.h, st->src.w, st->src.c);
+        st->name = n.name;
+        st->type = "FakeQuantize";
+        st->bytes = st->src.bytes(tensors) + n.numel() * 4;
+        st->out_node = id;
+        values[id].kind = VK_TENSOR;
+        values[id].tensor = st->out;
+        steps.push_back(std::move(st));
+    }
+
     void plan_conv(int id) {
         const GNode& n = N(id);
+        if (N(n.in[1]).op == OP_CONSTANT && N(n.in[1]).dtype == HIPIE_F32) {
+            plan_conv_f32(id);
+            return;
+        }
         const bool is_mm = n.op == OP_MATMUL;
         const Value x = value(n.in[0]);
         // Subtract(zero point) in front of the convolution: an integer per tensor (what optimizeSubtract
@@ -2211,7 +2443,8 @@ struct Planner {
     // Relu | Clamp and the FakeQuantize that follow it taken into the same kernel.
     void plan_eltwise(int id) {
         const GNode& n = N(id);
-        if (n.shape.size() != 4) unsupported(id, "stand-alone elementwise nodes are planned on 4-D (NHWC) values");
+        // ([N, C, H, W], or [N, C] behind a flattening Reshape or an f32 MatMul: a tensor with one pixel per batch element)
+        if (n.shape.size() != 4 && n.shape.size() != 2) unsupported(id, "stand-alone elementwise nodes are planned on [N, C, H, W] and [N, C] values");
         int nn, c, h, w;
         nhwc_dims(n.shape, nn, c, h, w);
         auto st = std::make_unique<EltwiseStep>();
@@ -2228,8 +2461,10 @@ struct Planner {
                 o.mul = x.mul;
             } else if (x.kind == VK_TENSOR && tensors[x.tensor].dtype == HIPIE_F32) {
                 o.tensor = x.tensor;
+            } else if (x.kind == VK_PARAM && N(in).op == OP_PARAMETER && N(in).dtype == HIPIE_F32) {
+                o.tensor = param_as_tensor(in);
             } else {
-                unsupported(id, "elementwise operand must be an f32 tensor or a dequantized byte tensor");
+                unsupported(id, "elementwise operand must be an f32 graph input, an f32 tensor or a dequantized byte tensor");
             }
         };
         const bool binary = n.op == OP_ADD || n.op == OP_SUBTRACT || n.op == OP_MULTIPLY;
@@ -2456,7 +2691,7 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
             const bool integer_kernel = s->type.find("Convolution") != std::string::npos || s->type.find("MatMul") != std::string::npos ||
                                         s->type.find("Pool") != std::string::npos || s->type.find("Attention") != std::string::npos ||
                                         s->type == "Transpose";
-            if (integer_kernel)
+            if (integer_kernel && !s->f32_kernel)
                 for (int v : found)
                     for (int in : g->nodes[v].in) {
                         if (in < 0 || g->nodes[in].op == OP_CONSTANT || std::binary_search(found.begin(), found.end(), in)) continue;

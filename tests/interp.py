@@ -50,10 +50,16 @@ def evaluate(orc, nodes, feeds, keep=None, override=None, targets=None):
             v = orc.fake_quantize(x[0], x[1], x[2], x[3], x[4], n["levels"])
             if n["dtype"] != F32:
                 v = v.astype(_NP[n["dtype"]])            # TypeRelaxed output: Convert of the f32 result
+        elif op in ("Convolution", "GroupConvolution") and x[1].dtype == np.float32:
+            # a layer the transformations left alone: f32 weights, the reference's float instantiation
+            v = orc.convolution(x[0].astype(np.float32), x[1], n["strides"], n["dilations"], n["pads_begin"], n["pads_end"],
+                                grouped=op == "GroupConvolution")
         elif op in ("Convolution", "GroupConvolution"):
             v = orc.convolution(x[0].astype(np.int32), x[1].astype(np.int32), n["strides"], n["dilations"],
                                 n["pads_begin"], n["pads_end"], grouped=op == "GroupConvolution")
             v = v.astype(np.float32)                      # declared f32 holding the integer sum
+        elif op == "MatMul" and x[1].dtype == np.float32 and x[0].dtype == np.float32 and nodes[n["inputs"][1]]["op"] == "Constant":
+            v = orc.matmul(x[0], x[1], n["ta"], n["tb"])
         elif op == "MatMul":
             v = orc.matmul(x[0].astype(np.int32), x[1].astype(np.int32), n["ta"], n["tb"]).astype(np.float32)
         elif op == "Add":

@@ -104,7 +104,7 @@ def test_epilogue_rejects_an_inverted_clamp_range():
 
 # ---- plugin-level surface: config map, metrics, QueryNetwork, request status paths (no device needed) ----
 def _tiny_graph(extra_relu=False):
-    """FakeQuantize -> 1x1 convolution -> bias -> FakeQuantize -> dequantization; optionally two stray Relu nodes"""
+    """FakeQuantize -> 1x1 convolution -> bias -> FakeQuantize -> dequantization; optionally two stray f32 pooling nodes"""
     from dldt_amd.graph import Graph
     from dldt_amd.tensor import F32, I8, U8
     g = Graph()
@@ -116,8 +116,8 @@ def _tiny_graph(extra_relu=False):
     out = g.multiply(g.convert(q2, F32), g.constant(np.float32(0.01).reshape(1, 1, 1, 1)))
     ids = dict(x=x, q=q, conv=y, q2=q2, out=out)
     if extra_relu:
-        ids["relu_a"] = g.relu(x)                       # a Relu no convolution absorbs: not planned
-        ids["relu_b"] = g.relu(g.multiply(x, g.constant(np.float32(2).reshape(1, 1, 1, 1))))
+        ids["relu_a"] = g.max_pool(x, (2, 2), (2, 2))   # pooling of f32 values: not planned (pooling runs on quantized tensors)
+        ids["relu_b"] = g.max_pool(g.multiply(x, g.constant(np.float32(2).reshape(1, 1, 1, 1))), (2, 2), (2, 2))
         g.result(ids["relu_a"], "a")
         g.result(ids["relu_b"], "b")
     g.result(out, "y")
@@ -173,7 +173,8 @@ def test_device_metrics():
     for name in ("AVAILABLE_DEVICES", "OPTIMIZATION_CAPABILITIES", "RANGE_FOR_ASYNC_INFER_REQUESTS", "IMPORT_EXPORT_SUPPORT",
                  "DEVICE_ARCHITECTURE", "SUPPORTED_CONFIG_KEYS"):
         assert name in names.split()
-    assert metric("OPTIMIZATION_CAPABILITIES") == (0, "INT8")       # no f32 convolution / MatMul path exists
+    # (the unquantized layers of an INT8 network run in f32 kernels that are correct, not fast: not an FP32 device)
+    assert metric("OPTIMIZATION_CAPABILITIES") == (0, "INT8")
     assert metric("IMPORT_EXPORT_SUPPORT") == (0, "YES")
     assert metric("DEVICE_ARCHITECTURE") == (0, "gfx950")
     assert metric("RANGE_FOR_ASYNC_INFER_REQUESTS")[1].split() == ["1", "8", "1"]
@@ -342,3 +343,24 @@ def test_matmul_between_activations_descriptor_and_workspace():
             BatchedMatMul(64, 64, device=-1, **bad)
     with pytest.raises(HipieError):
         BatchedMatMul(96, 64, device=-1)            # the reduction length is a multiple of 64
+
+
+def test_unquantized_layers_are_planned_in_f32():
+    """a convolution with f32 weights (no FakeQuantize in front of it) and a FakeQuantize that keeps its f32 result are
+    planned as f32 steps, not refused: QueryNetwork takes every node, the exec graph reports FP32 for them and the
+    integer type for the quantized layer behind them"""
+    from dldt_amd.graph import Graph
+    from dldt_amd.tensor import I8, U8
+    g = Graph()
+    x = g.parameter("x", (1, 3, 8, 8))
+    y = g.relu(g.add(g.convolution(x, g.constant(np.ones((16, 3, 3, 3), np.float32)), pads_begin=(1, 1), pads_end=(1, 1)),
+                     g.constant(np.zeros((1, 16, 1, 1), np.float32))))
+    f = g.fake_quantize(y, -1.0, 1.0, -1.0, 1.0, 256)                        # f32 result
+    q = g.fake_quantize(f, 0.0, 2.55, 0.0, 255.0, 256, out_dtype=U8)
+    out = g.multiply(g.convolution(q, g.constant(np.ones((16, 16, 1, 1), np.int8), I8)), g.constant(np.float32(0.01).reshape(1, 1, 1, 1)))
+    g.result(out, "y")
+    assert all(g.query())
+    plan = g.compile(-1, config={"HIP_TUNE": "NO"})
+    rows = [(plan.steps[i]["type"], plan.step_rt_info(i, "runtimePrecision")) for i in range(len(plan.steps))]
+    assert rows[0] == ("Convolution", "FP32") and ("FakeQuantize", "FP32") in rows and ("Convolution", "U8") in rows, rows
+    assert plan.steps[0]["macs"] == 16 * 8 * 8 * 27
