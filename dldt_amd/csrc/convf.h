@@ -47,4 +47,19 @@ void launch_fq_f32(const FqF32Args& a, hipStream_t s);
 // the same walk without the FakeQuantize (ch unused): a graph input as the NHWC f32 tensor the elementwise kernels read
 void launch_copy_f32(const FqF32Args& a, hipStream_t s);
 
+
+// reference::max_pool<float> / avg_pool<float> (max_pool.hpp, avg_pool.hpp:114-265): the window runs over the padded
+// tensor and ends at its upper bound, padding cells are skipped (a maximum starts from lowest()); the mean adds the
+// window's cells row by row - zeros for padding cells when they count - and divides by the cell count of the
+// reference's rules (kernel area when padding counts and there is any, else the cells taken)
+struct PoolF32Args {
+    F32Source in;
+    float* out = nullptr;             // NHWC
+    int64_t out_sn = 0, out_sh = 0, out_sw = 0;
+    int32_t N = 0, C = 0, H = 0, W = 0, OH = 0, OW = 0;
+    int32_t kh = 1, kw = 1, sh = 1, sw = 1, pt = 0, pl = 0, pb = 0, pr = 0;
+    int32_t avg = 0, include_pad = 0;
+};
+void launch_pool_f32(const PoolF32Args& a, hipStream_t s);
+
 }  // namespace hipie

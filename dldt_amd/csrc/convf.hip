@@ -1,5 +1,5 @@
-// f32 Convolution / GroupConvolution / MatMul against constants and FakeQuantize with an f32 result: the layers of an
-// INT8 network that the low-precision transformations leave unquantized.  See convf.h.
+// f32 Convolution / GroupConvolution / MatMul against constants, FakeQuantize with an f32 result, MaxPool / AvgPool of f32
+// values: the layers of an INT8 network that the low-precision transformations leave unquantized.  See convf.h.
 #include "convf.h"
 
 namespace hipie {
@@ -59,6 +59,41 @@ __global__ __launch_bounds__(256) void fq_f32_kernel(const FqF32Args a) {
     a.out[n * a.out_sn + h * a.out_sh + w * a.out_sw + c] = v;
 }
 
+__global__ __launch_bounds__(256) void pool_f32_kernel(const PoolF32Args a) {
+    const int64_t total = static_cast<int64_t>(a.N) * a.OH * a.OW * a.C;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int c = static_cast<int>(i % a.C);
+    int64_t p = i / a.C;
+    const int ow = static_cast<int>(p % a.OW);
+    p /= a.OW;
+    const int oh = static_cast<int>(p % a.OH);
+    const int n = static_cast<int>(p / a.OH);
+    // window in the coordinates of the padded tensor, cut at its upper bound
+    const int y0 = a.sh * oh, x0 = a.sw * ow;
+    const int y1 = min(y0 + a.kh, a.H + a.pt + a.pb), x1 = min(x0 + a.kw, a.W + a.pl + a.pr);
+    const bool padding_present = a.pt != 0 || a.pl != 0 || a.pb != 0 || a.pr != 0;
+    float r = a.avg ? 0.f : -3.402823466e+38f;
+    int count = a.avg && a.include_pad && padding_present ? a.kh * a.kw : 0;
+    for (int y = y0; y < y1; ++y)
+        for (int x = x0; x < x1; ++x) {
+            const int iy = y - a.pt, ix = x - a.pl;
+            const bool inside = iy >= 0 && iy < a.H && ix >= 0 && ix < a.W;
+            if (!a.avg) {
+                if (inside) {
+                    const float v = source_value(a.in, n, c, iy, ix);
+                    r = v > r ? v : r;
+                }
+            } else if (inside || a.include_pad) {
+                const float v = inside ? source_value(a.in, n, c, iy, ix) : 0.0f;
+                r = r + v;
+                if (!padding_present || (inside && !a.include_pad)) ++count;
+            }
+        }
+    if (a.avg) r = r / static_cast<float>(count);
+    a.out[n * a.out_sn + oh * a.out_sh + ow * a.out_sw + c] = r;
+}
+
 void check_source(const F32Source& s, const char* what) {
     HIPIE_REQUIRE(s.p && (s.dtype == HIPIE_F32 || s.dtype == HIPIE_U8B || s.dtype == HIPIE_I8), HIPIE_PARAMETER_MISMATCH,
                   "%s: input of type %d", what, s.dtype);
@@ -89,6 +124,18 @@ static void launch_elementwise_f32(const FqF32Args& a, bool quantize, hipStream_
     HIPIE_REQUIRE(blocks < (int64_t{1} << 31), HIPIE_PARAMETER_MISMATCH, "%s: %lld elements", what, (long long)total);
     if (quantize) hipLaunchKernelGGL(fq_f32_kernel<true>, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s, a);
     else hipLaunchKernelGGL(fq_f32_kernel<false>, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s, a);
+    HIPIE_CHECK_HIP(hipGetLastError());
+}
+
+void launch_pool_f32(const PoolF32Args& a, hipStream_t s) {
+    check_source(a.in, "f32 pooling");
+    HIPIE_REQUIRE(a.out && a.N > 0 && a.C > 0 && a.H > 0 && a.W > 0 && a.OH > 0 && a.OW > 0 && a.kh > 0 && a.kw > 0 && a.sh > 0 && a.sw > 0 &&
+                      a.pt >= 0 && a.pl >= 0 && a.pb >= 0 && a.pr >= 0,
+                  HIPIE_PARAMETER_MISMATCH, "f32 pooling: shape");
+    const int64_t total = static_cast<int64_t>(a.N) * a.OH * a.OW * a.C;
+    const int64_t blocks = ceil_div(total, 256);
+    HIPIE_REQUIRE(blocks < (int64_t{1} << 31), HIPIE_PARAMETER_MISMATCH, "f32 pooling: %lld outputs", (long long)total);
+    hipLaunchKernelGGL(pool_f32_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s, a);
     HIPIE_CHECK_HIP(hipGetLastError());
 }
 

@@ -584,10 +584,11 @@ struct ConcatStep : Step {
             ConcatArgs a{};
             a.in = static_cast<const int8_t*>(x.data);
             a.out = static_cast<int8_t*>(o.data);
-            a.N = x.n; a.H = x.h; a.W = x.w; a.C = x.c;
-            a.in_sn = x.stride_n; a.in_sh = x.stride_h; a.in_sw = x.stride_w;
-            a.out_sn = o.stride_n; a.out_sh = o.stride_h; a.out_sw = o.stride_w;
-            a.c_off = c_off[i];
+            const int es = static_cast<int>(tensors[out].esize());   // (f32 branches: four bytes per element)
+            a.N = x.n; a.H = x.h; a.W = x.w; a.C = x.c * es;
+            a.in_sn = x.stride_n * es; a.in_sh = x.stride_h * es; a.in_sw = x.stride_w * es;
+            a.out_sn = o.stride_n * es; a.out_sh = o.stride_h * es; a.out_sw = o.stride_w * es;
+            a.c_off = c_off[i] * es;
             launch_concat_channels(a, s);
         }
         HIPIE_CHECK_HIP(hipGetLastError());
@@ -756,6 +757,22 @@ struct ConvF32Step : Step {
         a.out = static_cast<float*>(t.data);
         a.out_sn = t.stride_n; a.out_sh = t.stride_h; a.out_sw = t.stride_w;
         launch_conv_f32(a, s);
+    }
+};
+
+// MaxPool / AvgPool of an f32 value
+struct PoolF32Step : Step {
+    F32Input src;
+    int out = -1;
+    PoolF32Args geo{};
+    void create(int device, const std::vector<TensorInfo>&) override { src.upload(device); }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*, hipStream_t s) const override {
+        PoolF32Args a = geo;
+        a.in = src.source(arena, tensors, inputs);
+        const hipie_tensor t = tensors[out].desc(arena);
+        a.out = static_cast<float*>(t.data);
+        a.out_sn = t.stride_n; a.out_sh = t.stride_h; a.out_sw = t.stride_w;
+        launch_pool_f32(a, s);
     }
 };
 
@@ -2335,8 +2352,10 @@ struct Planner {
     void plan_pool(int id) {
         const GNode& n = N(id);
         const Value x = value(n.in[0]);
-        if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1)
-            unsupported(id, "pooling is planned on quantized (u8/i8) tensors");
+        if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1) {
+            plan_pool_f32(id);
+            return;
+        }
         auto st = std::make_unique<PoolStep>();
         st->avg = n.op == OP_AVG_POOL;
         PoolArgs& a = st->a;
@@ -2407,6 +2426,33 @@ struct Planner {
         steps.push_back(std::move(st));
     }
 
+    // pooling of an f32 value (a layer in front of the first FakeQuantize, or behind a layer left in f32)
+    void plan_pool_f32(int id) {
+        const GNode& n = N(id);
+        auto st = std::make_unique<PoolF32Step>();
+        if (n.shape.size() != 4 || n.dtype != HIPIE_F32 || !f32_input(n.in[0], st->src))
+            unsupported(id, "pooling is planned on quantized (u8/i8) tensors and on 4-D f32 values");
+        PoolF32Args& a = st->geo;
+        a.avg = n.op == OP_AVG_POOL;
+        a.kh = static_cast<int>(n.kernel[0]); a.kw = static_cast<int>(n.kernel[1]);
+        a.sh = static_cast<int>(n.strides[0]); a.sw = static_cast<int>(n.strides[1]);
+        a.pt = static_cast<int>(n.pads_begin[0]); a.pl = static_cast<int>(n.pads_begin[1]);
+        a.pb = static_cast<int>(n.pads_end[0]); a.pr = static_cast<int>(n.pads_end[1]);
+        a.include_pad = a.avg && !n.exclude_pad;
+        int nn, c, h, w;
+        nhwc_dims(n.shape, nn, c, h, w);
+        a.N = nn; a.C = c; a.H = st->src.h; a.W = st->src.w; a.OH = h; a.OW = w;
+        st->out = new_tensor(id, HIPIE_F32, nn, h, w, c);
+        st->name = n.name;
+        st->type = a.avg ? "AvgPool" : "MaxPool";
+        st->f32_kernel = true;
+        st->bytes = st->src.bytes(tensors) + n.numel() * 4;
+        st->out_node = id;
+        values[id].kind = VK_TENSOR;
+        values[id].tensor = st->out;
+        steps.push_back(std::move(st));
+    }
+
     // Concat of quantized branches (after LPT they share one interval, concat.cpp:42-190, and the dequantization sits
     // behind the Concat): the levels are copied side by side
     void plan_concat(int id) {
@@ -2417,14 +2463,15 @@ struct Planner {
         int64_t bytes = 0;
         for (int in : n.in) {
             const Value x = value(in);
-            if (x.kind != VK_TENSOR || tensors[x.tensor].esize() != 1)
-                unsupported(id, "Concat inputs must be quantized (u8/i8) tensors: dequantized branches are concatenated by LPT before it");
-            if (dtype >= 0 && tensors[x.tensor].dtype != dtype) unsupported(id, "Concat of u8 and i8 levels");
+            // quantized branches (their levels side by side), or f32 ones (branches no FakeQuantize follows)
+            if (x.kind != VK_TENSOR)
+                unsupported(id, "Concat inputs must be quantized (u8/i8) or f32 tensors: dequantized branches are concatenated by LPT before it");
+            if (dtype >= 0 && tensors[x.tensor].dtype != dtype) unsupported(id, "Concat of values of different types");
             dtype = tensors[x.tensor].dtype;
             st->ins.push_back(x.tensor);
             st->c_off.push_back(off);
             off += tensors[x.tensor].c;
-            bytes += N(in).numel();
+            bytes += N(in).numel() * tensors[x.tensor].esize();
         }
         int nn, c, h, w;
         nhwc_dims(n.shape, nn, c, h, w);

@@ -104,7 +104,7 @@ def test_epilogue_rejects_an_inverted_clamp_range():
 
 # ---- plugin-level surface: config map, metrics, QueryNetwork, request status paths (no device needed) ----
 def _tiny_graph(extra_relu=False):
-    """FakeQuantize -> 1x1 convolution -> bias -> FakeQuantize -> dequantization; optionally two stray f32 pooling nodes"""
+    """FakeQuantize -> 1x1 convolution -> bias -> FakeQuantize -> dequantization; optionally two stray Gelu nodes"""
     from dldt_amd.graph import Graph
     from dldt_amd.tensor import F32, I8, U8
     g = Graph()
@@ -116,8 +116,8 @@ def _tiny_graph(extra_relu=False):
     out = g.multiply(g.convert(q2, F32), g.constant(np.float32(0.01).reshape(1, 1, 1, 1)))
     ids = dict(x=x, q=q, conv=y, q2=q2, out=out)
     if extra_relu:
-        ids["relu_a"] = g.max_pool(x, (2, 2), (2, 2))   # pooling of f32 values: not planned (pooling runs on quantized tensors)
-        ids["relu_b"] = g.max_pool(g.multiply(x, g.constant(np.float32(2).reshape(1, 1, 1, 1))), (2, 2), (2, 2))
+        ids["relu_a"] = g.gelu(x)                       # Gelu of a 4-D value: not planned (it runs on the row-major path)
+        ids["relu_b"] = g.gelu(g.multiply(x, g.constant(np.float32(2).reshape(1, 1, 1, 1))))
         g.result(ids["relu_a"], "a")
         g.result(ids["relu_b"], "b")
     g.result(out, "y")

@@ -183,3 +183,31 @@ def test_mean_and_scale_in_front_of_the_first_fake_quantize(orc):
     np.testing.assert_array_equal(req.tensor(a["node"]), kept[a["node"]])
     np.testing.assert_array_equal(_bits(got), _bits(want["out"]))
     assert [plan.steps[i]["type"] for i in range(len(plan.steps))][0] == "Reorder"
+
+
+def test_f32_branches_pool_and_concat(orc):
+    """an unquantized stem with two branches: f32 convolution -> ReLU -> MaxPool (f32), a second f32 convolution of the
+    input with stride 2, Concat of both along the channels (f32), FakeQuantize to u8 levels, quantized convolution"""
+    from dldt_amd import builders
+    rng = np.random.default_rng(95)
+    x = rng.uniform(-1, 1, (2, 3, 18, 18)).astype(np.float32)
+    w0 = rng.normal(0, 0.3, (10, 3, 3, 3)).astype(np.float32)
+    w1 = rng.normal(0, 0.3, (6, 3, 1, 1)).astype(np.float32)
+    w2 = rng.normal(0, 0.1, (8, 16, 1, 1)).astype(np.float32)
+    b2 = rng.normal(0, 0.1, 8).astype(np.float32)
+    net = builders.QuantizedNet()
+    g = net.g
+    p = g.parameter("data", x.shape)
+    a = g.max_pool(g.relu(g.convolution(p, g.constant(w0), pads_begin=(1, 1), pads_end=(1, 1))), (3, 3), (2, 2), (1, 1), (1, 1))
+    b = g.convolution(p, g.constant(w1), strides=(2, 2))
+    cat = g.concat([a, b], axis=1)
+    q = net.requantize(g.relu(cat), 1.5)
+    g.result(net.conv_f32(q, w2, b2), "out")
+    want, kept = evaluate(orc, g.nodes, {"data": x}, keep=[cat, q["node"]])
+    plan = g.compile()
+    req = plan.create_request()
+    (got,) = req.infer(x)
+    np.testing.assert_array_equal(_bits(req.tensor(cat)), _bits(kept[cat]))
+    np.testing.assert_array_equal(req.tensor(q["node"]), kept[q["node"]])
+    np.testing.assert_array_equal(_bits(got), _bits(want["out"]))
+    assert all(g.query())

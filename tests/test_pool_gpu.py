@@ -170,3 +170,52 @@ def test_window_in_the_padding_alone_is_refused():
     q = g.fake_quantize(x, 0.0, 255.0, 0.0, 255.0, 256, out_dtype=U8)
     with pytest.raises(HipieError):
         g.max_pool(q, (2, 2), (3, 3), (0, 0), (2, 2), ceil_mode=True)   # windows start at 0, 3, 6: the third is padding only
+
+
+# ---- pooling of f32 values (a layer in front of the first FakeQuantize, or behind a layer left in f32) --------------------
+def _f32_pool(orc, x, kind, kernel, strides, pb, pe, ceil, exclude_pad=True):
+    from dldt_amd.graph import Graph
+    from interp import evaluate
+    g = Graph()
+    p = g.parameter("x", x.shape)
+    y = g.max_pool(p, kernel, strides, pb, pe, ceil_mode=ceil) if kind == "max" else \
+        g.avg_pool(p, kernel, strides, pb, pe, exclude_pad=exclude_pad, ceil_mode=ceil)
+    g.result(y, "y")
+    want, _ = evaluate(orc, g.nodes, {"x": x})
+    (got,) = g.compile().create_request().infer(x)
+    return got, want["y"]
+
+
+@pytest.mark.parametrize("name", sorted(_cases("max_pool")))
+def test_max_pool_reference_vectors_in_f32(orc, name):
+    """the reference's vectors as they stand: f32 in, f32 out, no quantization in between"""
+    t = _cases("max_pool")[name]
+    pb, pe = _pads(t)
+    x = np.asarray(t["a"], np.float32).reshape(t["in_shape"])
+    got, want = _f32_pool(orc, x, "max", t["kernel"], t["strides"], pb, pe, t.get("ceil", False))
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    np.testing.assert_array_equal(got, np.asarray(t["result"], np.float32).reshape(t["out_shape"]))
+
+
+@pytest.mark.parametrize("name", sorted(_cases("avg_pool")))
+def test_avg_pool_reference_vectors_in_f32(orc, name):
+    t = _cases("avg_pool")[name]
+    pb, pe = _pads(t)
+    x = np.asarray(t["a"], np.float32).reshape(t["in_shape"])
+    got, want = _f32_pool(orc, x, "avg", t["kernel"], t["strides"], pb, pe, t.get("ceil", False), t["exclude_pad"])
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    np.testing.assert_allclose(got, np.asarray(t["result"], np.float32).reshape(t["out_shape"]), rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("kind,exclude_pad", [("max", True), ("avg", True), ("avg", False)])
+@pytest.mark.parametrize("geo", range(len(GEOMETRIES)))
+def test_f32_pool_fuzz(orc, geo, kind, exclude_pad):
+    kernel, strides, pb, pe, ceil = GEOMETRIES[geo]
+    rng = np.random.default_rng(400 + geo)
+    h, w = (7, 7) if kernel == (7, 7) else (13, 10)
+    x = rng.normal(-0.5, 2.0, (2, 11, h, w)).astype(np.float32)
+    x[1] = -np.abs(x[1]) - np.float32(0.25)       # every value negative: padding must never win a maximum
+    got, want = _f32_pool(orc, x, kind, kernel, strides, pb, pe, ceil, exclude_pad)
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    if kind == "max":
+        assert got[1].max() < 0
