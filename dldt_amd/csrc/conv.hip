@@ -55,6 +55,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     const int woc = wave % WOC, wpix = wave / WOC;
     const int l32 = lane & 31, h = lane >> 5;
     const int chunk = tid & 3;
+    const PiecePick pick(chunk);
     // XOR swizzle instead of row padding: the thread that stages (row, chunk) and the lanes that read
     // fragments (rows l32 + 32 i, chunk 2 ks + h) agree on slot = chunk ^ ((row >> 2) & 3); rows that
     // differ by a multiple of 16 share the swizzle, so (tid + i NT) >> 2 and l32 + 32 i need one value each
@@ -137,14 +138,8 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
                 // an odd step count leaves the last pair half empty: its second half re-reads the last step
                 // (in bounds, never multiplied)
                 const int k0 = 2 * j, k1 = min(2 * j + 1, nk - 1);
-                int4 ko0 = *reinterpret_cast<const int4*>(koff + 4 * k0);   // uniform: scalar loads, taken as wave-uniform values
-                int4 ko1 = *reinterpret_cast<const int4*>(koff + 4 * k1);
-                ko0.x = __builtin_amdgcn_readfirstlane(ko0.x); ko0.y = __builtin_amdgcn_readfirstlane(ko0.y);
-                ko0.z = __builtin_amdgcn_readfirstlane(ko0.z); ko0.w = __builtin_amdgcn_readfirstlane(ko0.w);
-                ko1.x = __builtin_amdgcn_readfirstlane(ko1.x); ko1.y = __builtin_amdgcn_readfirstlane(ko1.y);
-                ko1.z = __builtin_amdgcn_readfirstlane(ko1.z); ko1.w = __builtin_amdgcn_readfirstlane(ko1.w);
-                const int32_t off0 = chunk == 0 ? ko0.x : (chunk == 1 ? ko0.y : (chunk == 2 ? ko0.z : ko0.w));
-                const int32_t off1 = chunk == 0 ? ko1.x : (chunk == 1 ? ko1.y : (chunk == 2 ? ko1.z : ko1.w));
+                const int4 ko0 = load_uniform_int4(koff + 4 * k0), ko1 = load_uniform_int4(koff + 4 * k1);
+                const int32_t off0 = pick(ko0), off1 = pick(ko1);
                 const int32_t off = sub ? off1 : off0;
                 const int kk = sub ? k1 : k0;
 #pragma unroll
@@ -181,12 +176,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
         }
         v4i ga[A_PIECES], gb[B_PIECES];
         auto load_global = [&](int k) {
-            int4 ko = *reinterpret_cast<const int4*>(koff + 4 * k);   // uniform: one scalar load of the step's four offsets
-            // taken as wave-uniform values: otherwise the select below becomes three divergent branches,
-            // each with its own scalar load and wait in front of the vector loads
-            ko.x = __builtin_amdgcn_readfirstlane(ko.x); ko.y = __builtin_amdgcn_readfirstlane(ko.y);
-            ko.z = __builtin_amdgcn_readfirstlane(ko.z); ko.w = __builtin_amdgcn_readfirstlane(ko.w);
-            const int32_t off = chunk == 0 ? ko.x : (chunk == 1 ? ko.y : (chunk == 2 ? ko.z : ko.w));
+            const int32_t off = pick(load_uniform_int4(koff + 4 * k));   // one scalar load of the step's four offsets
             const int8_t* wk = wgt_base + k * 64;                     // uniform part of the weight address
 #pragma unroll
             for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(wk + a_off[i]);
@@ -293,6 +283,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const C
     const int woc = wave % WOC, wpix = wave / WOC;
     const int l32 = lane & 31, h = lane >> 5;
     const int chunk = tid & 3;
+    const PiecePick pick(chunk);
     // XOR swizzle instead of row padding: the thread that stages (row, chunk) and the lanes that read
     // fragments (rows l32 + 32 i, chunk 2 ks + h) agree on slot = chunk ^ ((row >> 2) & 3); rows that
     // differ by a multiple of 16 share the swizzle, so (tid + i NT) >> 2 and l32 + 32 i need one value each
@@ -325,8 +316,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, 2) void conv_persist_kernel(const C
     };
     v4i ga[A_PIECES], gb[B_PIECES];
     auto load_global = [&](int k) {
-        const int4 ko = *reinterpret_cast<const int4*>(a.koff + 4 * k);
-        const int32_t off = chunk == 0 ? ko.x : (chunk == 1 ? ko.y : (chunk == 2 ? ko.z : ko.w));
+        const int32_t off = pick(load_uniform_int4(a.koff + 4 * k));
 #pragma unroll
         for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(a_ptr[i] + k * 64);
 #pragma unroll
@@ -943,7 +933,7 @@ __global__ __launch_bounds__(256, 2) void conv_stream_kernel(const ConvArgs a) {
         }
     };
     auto load_b = [&](const int32_t (&b)[2], int k, v4i (&f)[2][2]) {
-        const int4 ko = *reinterpret_cast<const int4*>(a.koff + 4 * k);   // uniform: scalar load
+        const int4 ko = load_uniform_int4(a.koff + 4 * k);
         const int32_t o0 = h ? ko.y : ko.x, o1 = h ? ko.w : ko.z;
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb) {

@@ -61,6 +61,30 @@ __device__ __forceinline__ int window_offset(const ConvArgs& a, int m, int sn, i
 
 __device__ __forceinline__ float4 ld4f(const float* p) { return *reinterpret_cast<const float4*>(p); }
 
+// Four consecutive dwords of a table no kernel writes, at an address every lane of the wave shares: read through the
+// constant address space, so that the load is a scalar one (one request per wave, waited for on the scalar / LDS counter).
+// As an ordinary global load behind a barrier the compiler issues it as a vector load - every lane asks - and waits for
+// it with vmcnt(0), i.e. for every vector load of the wave that is still on its way, in front of the loads that need it.
+__device__ __forceinline__ int4 load_uniform_int4(const int32_t* p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef int dwords4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(4))) const dwords4 constant_dwords4;
+    const dwords4 v = *reinterpret_cast<constant_dwords4*>(reinterpret_cast<uintptr_t>(p));
+    return make_int4(v.x, v.y, v.z, v.w);
+#else
+    return *reinterpret_cast<const int4*>(p);
+#endif
+}
+
+// A thread's piece (0 .. 3) of four such values, taken with masks: written as a chain of selects on scalar registers
+// it becomes divergent branches, each with a scalar load and a wait of its own.
+struct PiecePick {
+    int32_t m0, m1, m2, m3;
+    __device__ __forceinline__ explicit PiecePick(int piece)
+        : m0(piece == 0 ? -1 : 0), m1(piece == 1 ? -1 : 0), m2(piece == 2 ? -1 : 0), m3(piece == 3 ? -1 : 0) {}
+    __device__ __forceinline__ int32_t operator()(const int4& v) const { return (v.x & m0) | (v.y & m1) | (v.z & m2) | (v.w & m3); }
+};
+
 // Accumulators start from the per-channel integer correction, so the epilogue begins with the
 // exact u8 x i8 sum.  acc[ob][pb][r] = channel oc_lane + 16*ob + r of pixel pb.
 __device__ __forceinline__ void init_acc(const ConvArgs& a, int oc_lane, v16i (&acc)[2][2]) {
