@@ -439,14 +439,15 @@ bool check_boundaries(const FqChannel& p, float lm1) {
     const int32_t o_lo = ordered(p.il), o_hi = ordered(p.ih);
     for (int k = 1; k < levels; ++k) {
         // smallest x in (il, ih] whose reference level is >= k (the level is monotone in x)
-        int32_t a = o_lo, b = o_hi;  // level(a) < k <= level(b)
+        // (64-bit: the ordered images of il <= -2 and ih >= 2 are 2^31 or more apart)
+        int64_t a = o_lo, b = o_hi;  // level(a) < k <= level(b)
         if (fq_level_div(p, lm1, p.ih) < k) break;
         while (b - a > 1) {
-            const int32_t m = a + (b - a) / 2;
-            if (fq_level_div(p, lm1, unordered(m)) >= k) b = m; else a = m;
+            const int64_t m = a + (b - a) / 2;
+            if (fq_level_div(p, lm1, unordered(static_cast<int32_t>(m))) >= k) b = m; else a = m;
         }
-        for (int32_t o : {a, b, b + 1 <= o_hi ? b + 1 : b, a - 1 >= o_lo ? a - 1 : a}) {
-            const float x = unordered(o);
+        for (int64_t o : {a, b, b + 1 <= o_hi ? b + 1 : b, a - 1 >= o_lo ? a - 1 : a}) {
+            const float x = unordered(static_cast<int32_t>(o));
             if (fq_level_rcp(p, lm1, x) != fq_level_div(p, lm1, x)) return false;
         }
     }

@@ -46,7 +46,11 @@ def test_fq_host_arithmetic_matches_oracle(orc):
     fq = FakeQuantize(C, 256, il, ih, 0.0, 255.0, device=-1)
     assert fq.uses_reciprocal
     x = rng.normal(0, 2, 4000).astype(np.float32)
-    for c in (0, 17, 47):
+    # (a channel with il <= -2 and ih >= 2 among them: the load-time check bisects between the bounds' ordered integer
+    # images, which are 2^31 or more apart there)
+    wide = int(np.argmax((il <= -2) & (ih >= 2)))
+    assert il[wide] <= -2 and ih[wide] >= 2
+    for c in (0, 17, 47, wide):
         # tie-dense probe: level midpoints of this channel and their float neighbours
         k = np.arange(255, dtype=np.float32) + np.float32(0.5)
         mid = (il[c] + (ih[c] - il[c]) * (k / np.float32(255))).astype(np.float32)
