@@ -38,6 +38,7 @@ struct AttentionArgs {
     float p_zh, p_zl;                                 // probabilities: two-operation division by fq_p.p.d
     int p_div2;                                       // ... verified against IEEE division on the device
     int p_sat;                                        // input_low of the probabilities' FakeQuantize is +0 and it has 256 levels
+    int p_inside;                                     // ... or input_low <= 0 and input_high >= 1: a probability never leaves the interval
     int qblocks;                                      // blocks of 128 queries per batch element
     int xcd_groups;                                   // 1: a one-dimensional grid that keeps the blocks of two neighbouring batch elements on one XCD
 #ifdef HIPIE_ATT_STAMPS
@@ -49,20 +50,24 @@ struct AttentionArgs {
 
 // level index k of four probabilities as four unsigned bytes (rounded to nearest-even and packed by
 // v_cvt_pk_u8_f32), then the output offset applied bytewise
-// PSAT: input_low is +0 and there are 256 levels - a probability is never below input_low, and the packing
-// conversion's saturation at 255 is the branch for values above input_high: no clamp, no subtraction
-template <bool DIV2, bool PSAT>
+// PFORM 2: input_low is +0 and there are 256 levels - a probability is never below input_low, and the packing
+// conversion's saturation at 255 is the branch for values above input_high: no clamp, no subtraction.
+// PFORM 1: input_low <= 0 and input_high >= 1 - a probability (0 <= e / sum <= 1: the largest e is 2^0 and counted in
+// the sum) takes neither of the reference's saturating branches: no clamp.  PFORM 0: any interval.
+template <bool DIV2, int PFORM>
 __device__ __forceinline__ uint32_t prob_levels4(const AttentionArgs& a, float p0, float p1, float p2, float p3) {
     const FqChannel& c = a.fq_p.p;
+    constexpr int M = DIV2 ? 2 : 1;
+    constexpr bool IL0 = PFORM == 2, NOCLAMP = PFORM != 0;
     uint32_t w = 0;
-    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, PSAT, PSAT>(p0, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 0, w);
-    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, PSAT, PSAT>(p1, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 1, w);
-    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, PSAT, PSAT>(p2, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 2, w);
-    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<DIV2 ? 2 : 1, PSAT, PSAT>(p3, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 3, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<M, IL0, NOCLAMP>(p0, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 0, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<M, IL0, NOCLAMP>(p1, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 1, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<M, IL0, NOCLAMP>(p2, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 2, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(fq_level_fast<M, IL0, NOCLAMP>(p3, c.il, c.ih, c.d, DIV2 ? a.p_zh : c.r, a.p_zl, a.fq_p.lm1), 3, w);
     return a.p_add ? add_bytes(w, a.p_add) : (w ^ a.p_xor);
 }
 
-template <int NT, bool DIV2, bool MASK, bool PSAT>   // NT = S / 32 key tiles
+template <int NT, bool DIV2, bool MASK, int PFORM>   // NT = S / 32 key tiles
 __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a) {
     constexpr int S = NT * 32;
     constexpr int VT_LD = S + 16;                     // odd number of 16-byte groups per row: conflict-free
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(const AttentionArgs a
             const float4 p4 = make_float4(e[4 * g] * inv, e[4 * g + 1] * inv, e[4 * g + 2] * inv, e[4 * g + 3] * inv);
             if (a.probs && q_ok)
                 *reinterpret_cast<float4*>(a.probs + dump_row + 32 * t + 8 * g + 4 * h) = p4;
-            pf[g] = static_cast<int>(prob_levels4<DIV2, PSAT>(a, p4.x, p4.y, p4.z, p4.w));
+            pf[g] = static_cast<int>(prob_levels4<DIV2, PFORM>(a, p4.x, p4.y, p4.z, p4.w));
         }
 #pragma unroll
         for (int db = 0; db < 2; ++db) {
@@ -286,16 +291,19 @@ void launch(const AttentionArgs& a_in, int batches, hipStream_t s) {
     a.qblocks = static_cast<int>(ceil_div(a.S, 128));
     a.xcd_groups = batches % 16 == 0 ? 1 : 0;         // pairs of batch elements, eight pairs at a time
     const dim3 grid = a.xcd_groups ? dim3(static_cast<uint32_t>(a.qblocks) * batches) : dim3(a.qblocks, static_cast<uint32_t>(batches));
-    const bool sat = a.p_div2 && a.p_sat;             // (the form without clamp: compiled for the usual division only)
-    const int form = (a.mask ? 4 : 0) + (sat ? 2 : (a.p_div2 ? 1 : 0));
+    // (the forms without clamp: compiled for the usual division only)
+    const int pform = !a.p_div2 ? 0 : (a.p_sat ? 2 : (a.p_inside ? 1 : 0));
+    const int form = (a.mask ? 8 : 0) + (a.p_div2 ? 4 : 0) + pform;
 #define HIPIE_ATT_LAUNCH(D, M, P) hipLaunchKernelGGL((attention_kernel<NT, D, M, P>), grid, dim3(256), 0, s, a)
     switch (form) {
-    case 0: HIPIE_ATT_LAUNCH(false, false, false); break;
-    case 1: HIPIE_ATT_LAUNCH(true, false, false); break;
-    case 2: HIPIE_ATT_LAUNCH(true, false, true); break;
-    case 4: HIPIE_ATT_LAUNCH(false, true, false); break;
-    case 5: HIPIE_ATT_LAUNCH(true, true, false); break;
-    default: HIPIE_ATT_LAUNCH(true, true, true); break;
+    case 0: HIPIE_ATT_LAUNCH(false, false, 0); break;
+    case 4: HIPIE_ATT_LAUNCH(true, false, 0); break;
+    case 5: HIPIE_ATT_LAUNCH(true, false, 1); break;
+    case 6: HIPIE_ATT_LAUNCH(true, false, 2); break;
+    case 8: HIPIE_ATT_LAUNCH(false, true, 0); break;
+    case 12: HIPIE_ATT_LAUNCH(true, true, 0); break;
+    case 13: HIPIE_ATT_LAUNCH(true, true, 1); break;
+    default: HIPIE_ATT_LAUNCH(true, true, 2); break;
     }
 #undef HIPIE_ATT_LAUNCH
 }
@@ -351,6 +359,7 @@ int hipie_attention_create(int device, const hipie_attention_desc* desc, hipie_a
         HIPIE_REQUIRE(a.p_div2 || a.fq_p.rcp || device < 0, HIPIE_NOT_IMPLEMENTED,
                       "hipie_attention_create: no exact fast division for the probabilities' FakeQuantize range");
         a.p_sat = a.fq_p.p.il == 0.f && !std::signbit(a.fq_p.p.il) && a.fq_p.lm1 == 255.f;
+        a.p_inside = a.fq_p.p.il <= 0.f && a.fq_p.p.ih >= 1.f;
         a.p_bias = desc->prob_dtype == HIPIE_U8B ? 128 : 0;
         const int off = static_cast<int>(a.fq_p.p.ol) & 0xff;
         a.p_xor = off == 0x80 ? 0x80808080u : 0u;
