@@ -74,7 +74,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     // one implicit GEMM over an operand set (activation tensor, packed weights, K-offset table)
     auto gemm = [&](const int8_t* in_base, int in_sn, int in_sh, int in_sw, int csh, int csw, int origin,
                     const int8_t* wgt_base, int wgt_ld, int wgt_rows, bool wgt_plain, const int32_t* koff, int nk,
-                    v16i (&acc)[2][2], bool first, bool acc_from_lds, bool flat) {
+                    v16i (&acc)[2][2], bool first, bool acc_from_lds, bool flat, bool linear) {
         int32_t b_base[B_PIECES];
         uint32_t a_off[A_PIECES];                          // unsigned: added to the uniform base by the load itself
 #pragma unroll
@@ -175,14 +175,51 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
             return;
         }
         v4i ga[A_PIECES], gb[B_PIECES];
-        auto load_global = [&](int k) {
-            const int32_t off = pick(load_uniform_int4(koff + 4 * k));   // one scalar load of the step's four offsets
-            const int8_t* wk = wgt_base + k * 64;                     // uniform part of the weight address
+        if constexpr (F != kDyn && (F & CF_RES_GEMM)) {
+            // the kernel with two GEMMs keeps the shortcut's dequantised result in 64 registers next to the accumulators:
+            // plain loads through pointers here - the two buffer descriptors and the second copy of the loop below cost it
+            // registers it does not have (200 bytes of scratch per lane when tried)
+            auto load_global = [&](int k) {
+                const int32_t off = pick(load_uniform_int4(koff + 4 * k));   // one scalar load of the step's four offsets
+                const int8_t* wk = wgt_base + k * 64;                        // uniform part of the weight address
 #pragma unroll
-            for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(wk + a_off[i]);
+                for (int i = 0; i < A_PIECES; ++i) ga[i] = *reinterpret_cast<const v4i*>(wk + a_off[i]);
 #pragma unroll
-            for (int i = 0; i < B_PIECES; ++i) gb[i] = *reinterpret_cast<const v4i*>(in_base + (b_base[i] + off));
-        };
+                for (int i = 0; i < B_PIECES; ++i) gb[i] = *reinterpret_cast<const v4i*>(in_base + (b_base[i] + off));
+            };
+            auto store_lds = [&](int buf) {
+#pragma unroll
+                for (int i = 0; i < A_PIECES; ++i)
+                    *reinterpret_cast<v4i*>(&sA[buf][((tid + i * NT) >> 2) * kRow + lds_slot]) = ga[i];
+#pragma unroll
+                for (int i = 0; i < B_PIECES; ++i)
+                    *reinterpret_cast<v4i*>(&sB[buf][((tid + i * NT) >> 2) * kRow + lds_slot]) = gb[i];
+            };
+            load_global(0);
+            store_lds(0);
+            if (first) stage_params_store<F>(a, (lds_float_ptr)sP, BOC, tid, staged);
+            __syncthreads();
+            if (acc_from_lds) init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);
+            for (int k = 0; k < nk; ++k) {
+                const int buf = k & 1;
+                if (k + 1 < nk) load_global(k + 1);
+                mfma_step(buf);
+                if (k + 1 < nk) store_lds(buf ^ 1);
+                __syncthreads();
+            }
+            return;
+        }
+        // Both operands through buffer loads: a lane's offset in a register that does not change from step to step, the
+        // step's part in a scalar register - no 64-bit address arithmetic per load.  The activations' buffer starts at
+        // the window origin of pixel 0 (the tensor's element (0, 0, 0, 0) moved back by the padding), so that every
+        // offset is non-negative.  linear: the K pieces lie one behind the other in memory (a 1 x 1 convolution, a
+        // MatMul): step k is 64 k bytes behind step 0 and no table is read; else the lane adds its piece's entry of the
+        // step's four offsets.
+        const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(wgt_base), 0, 0x7fffffff, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(in_base + origin), 0, 0x7fffffff, 0x00020000);
+        int32_t b_vo[B_PIECES];
+#pragma unroll
+        for (int i = 0; i < B_PIECES; ++i) b_vo[i] = b_base[i] - origin + (linear ? chunk * 16 : 0);
         auto store_lds = [&](int buf) {
 #pragma unroll
             for (int i = 0; i < A_PIECES; ++i)
@@ -191,18 +228,36 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
             for (int i = 0; i < B_PIECES; ++i)
                 *reinterpret_cast<v4i*>(&sB[buf][((tid + i * NT) >> 2) * kRow + lds_slot]) = gb[i];
         };
-        load_global(0);
-        store_lds(0);
-        if (first) stage_params_store<F>(a, (lds_float_ptr)sP, BOC, tid, staged);
-        __syncthreads();
-        if (acc_from_lds) init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);
-        for (int k = 0; k < nk; ++k) {
-            const int buf = k & 1;
-            if (k + 1 < nk) load_global(k + 1);
-            mfma_step(buf);
-            if (k + 1 < nk) store_lds(buf ^ 1);
+        // (two copies of the loop behind a uniform branch: with the form as a run-time value inside one loop the
+        // compiler evaluates the table path for every step and selects)
+        auto k_loop = [&](auto linear_c) {
+            constexpr bool LINEAR = decltype(linear_c)::value;
+            auto load_global = [&](int k) {
+                const int32_t sk = k * 64;
+                // the step's four offsets: one scalar load, issued and awaited here, in front of the vector loads that
+                // need it (requested a step ahead it would be in flight during the LDS reads of the matrix
+                // instructions, whose partial waits then all become waits for everything)
+                const int32_t off = LINEAR ? 0 : pick(load_uniform_int4(koff + 4 * k));
+#pragma unroll
+                for (int i = 0; i < A_PIECES; ++i) ga[i] = __builtin_amdgcn_raw_buffer_load_b128(ra, static_cast<int32_t>(a_off[i]), sk, 0);
+#pragma unroll
+                for (int i = 0; i < B_PIECES; ++i) gb[i] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_vo[i] + off, LINEAR ? sk : 0, 0);
+            };
+            load_global(0);
+            store_lds(0);
+            if (first) stage_params_store<F>(a, (lds_float_ptr)sP, BOC, tid, staged);
             __syncthreads();
-        }
+            if (acc_from_lds) init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);
+            for (int k = 0; k < nk; ++k) {
+                const int buf = k & 1;
+                if (k + 1 < nk) load_global(k + 1);
+                mfma_step(buf);
+                if (k + 1 < nk) store_lds(buf ^ 1);
+                __syncthreads();
+            }
+        };
+        if (linear) k_loop(std::true_type{});
+        else k_loop(std::false_type{});
     };
 
     v16i acc[2][2];
@@ -215,7 +270,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
         a2.corr = a.corr2;
         init_acc(a2, oc_lane, acc);
         gemm(a.in2, a.in2_sn, a.in2_sh, a.in2_sw, a.conv2_sh, a.conv2_sw, a.in2_origin, a.wgt2, a.Kp2, a.OCp, false,
-             a.koff2, a.nk2, acc, true, false, false);
+             a.koff2, a.nk2, acc, true, false, false, a.k_linear2 != 0);
 #pragma unroll
         for (int ob = 0; ob < 2; ++ob)
 #pragma unroll
@@ -234,7 +289,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     }
     if (kFused) init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);   // published by the shortcut GEMM's first barrier
     gemm(a.in + batch_offset(a, batch, a.batch_in, a.batch_in_o), a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
-         a.wgt + batch_offset(a, batch, a.batch_wgt, a.batch_wgt_o), a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused, a.flat_in != 0);
+         a.wgt + batch_offset(a, batch, a.batch_wgt, a.batch_wgt_o), a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused, a.flat_in != 0, a.k_linear != 0);
     const int m0 = pix0 + wpix * 64 + l32;
     if constexpr (PIXC) {   // MatMul between activations whose right operand is stored as level - 128
         const int32_t* pc = a.pix_corr + static_cast<int64_t>(batch) * a.batch_pix_corr;
@@ -1383,6 +1438,7 @@ static int64_t packed_row(int64_t oc) {
 // order), byte offset of every 16-byte K piece, per-channel integer correction.
 struct PackedGemm {
     int64_t K = 0, Kp = 0, OCp = 0;
+    bool linear = false;           // koff[p] == 16 p for every piece: the K bytes of a pixel's window are contiguous
     DeviceBuffer wgt, koff, corr;
     // `keep`: receives the packed matrix ([OCp][Kp], rows in MFMA order) for a second packing derived from it
     void pack(int device, const hipie_conv_desc& d, const int8_t* weights, std::vector<int8_t>* keep = nullptr);
@@ -1392,6 +1448,7 @@ struct hipie_conv {
     int device = 0;
     hipie_conv_desc d{};
     int64_t K = 0, Kp = 0, OCp = 0;
+    bool k_linear = false;         // PackedGemm::linear of the main convolution
     // fused shortcut convolution (second operand set + its bias / scale tables)
     bool fused = false;
     hipie_conv_desc sd{};
@@ -1502,6 +1559,8 @@ void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weight
             off[p] = static_cast<int32_t>(kh * d.dil_h * d.in_stride_h + kw * d.dil_w * d.in_stride_w + ic0);
         }
     }
+    linear = true;
+    for (size_t p = 0; p < off.size(); ++p) linear = linear && off[p] == static_cast<int32_t>(16 * p);
     std::vector<int8_t> w(static_cast<size_t>(OCp) * Kp, 0);
     std::vector<int32_t> cr(OCp, 0);
     const int stored_zero = d.in_dtype == HIPIE_U8B ? 128 : 0;
@@ -1682,6 +1741,7 @@ int hipie_matmul_run_nested_ws(const hipie_matmul* mm, const void* a_ptr, int64_
         a.wgt = static_cast<const int8_t*>(bt_ptr);
         a.out = out;
         a.koff = mm->koff.as<int32_t>();
+        a.k_linear = 1;
         a.corr = mm->corr.as<int32_t>();
         mm->epi.fill(a);
         a.M = m;
@@ -1844,6 +1904,7 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
         g.pack(device, d, weights, &packed);
         c->K = g.K; c->Kp = g.Kp; c->OCp = g.OCp;
         c->wgt = std::move(g.wgt); c->koff = std::move(g.koff); c->corr = std::move(g.corr);
+        c->k_linear = g.linear;
         c->epi.build(device, *epilogue, d.oc, c->OCp);
         if (block_first_fits(d, c->Kp, c->OCp)) c->steps_role = 1;
         else if (block_second_fits(d, c->Kp, c->OCp)) c->steps_role = 2;
@@ -2038,6 +2099,7 @@ static int64_t fill_conv_args(const hipie_conv* c, const hipie_tensor* in, const
     a.wgt2 = c->wgt_rows.as<int8_t>();   // depthwise only; a fused shortcut overwrites it below
     a.out = out->data;
     a.koff = c->koff.as<int32_t>();
+    a.k_linear = c->k_linear ? 1 : 0;
     a.corr = c->corr.as<int32_t>();
     c->epi.fill(a);
     if (a.flags & CF_RES_GEMM) {
@@ -2059,6 +2121,7 @@ static int64_t fill_conv_args(const hipie_conv* c, const hipie_tensor* in, const
         a.in2 = static_cast<const int8_t*>(residual->data);
         a.wgt2 = c->sg.wgt.as<int8_t>();
         a.koff2 = c->sg.koff.as<int32_t>();
+        a.k_linear2 = c->sg.linear ? 1 : 0;
         a.corr2 = c->sg.corr.as<int32_t>();
         a.bias2 = c->s_bias.as<float>();
         a.scale2 = c->s_scale.as<float>();

@@ -141,6 +141,8 @@ struct ConvArgs {
     int32_t in2_sn, in2_sh, in2_sw, conv2_sh, conv2_sw, in2_origin, nk2, Kp2;
     // the input / output / residual tensor is dense in (n, h, w) for this convolution: no pixel decode
     int32_t flat_in, flat_out, flat_res;
+    // the K pieces of the convolution (of the fused shortcut) lie one behind the other in memory: koff[p] == 16 p
+    int32_t k_linear, k_linear2;
     // row-tile kernel (3 x 3, stride 1): output rows per tile, tiles per image, patch width OW + 2 and its reciprocal
     int32_t rows_per_tile, tiles_per_image, patch_w;
     float inv_patch_w;
