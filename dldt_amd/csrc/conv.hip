@@ -289,7 +289,7 @@ __global__ __launch_bounds__(WOC* WPIX * 64, (WOC * WPIX >= 4 && !(F != kDyn && 
     }
     if (kFused) init_acc_lds((lds_cfloat_ptr)sP, BOC, oc_lane - oc0, acc);   // published by the shortcut GEMM's first barrier
     gemm(a.in + batch_offset(a, batch, a.batch_in, a.batch_in_o), a.in_sn, a.in_sh, a.in_sw, a.conv_sh, a.conv_sw, a.in_origin,
-         a.wgt + batch_offset(a, batch, a.batch_wgt, a.batch_wgt_o), a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff, a.nk, acc, !kFused, !kFused, a.flat_in != 0, a.k_linear != 0);
+         a.wgt + batch_offset(a, batch, a.batch_wgt, a.batch_wgt_o), a.wgt_ld, a.wgt_rows, a.wgt_plain != 0, a.koff + t_tile * a.koff_tile, a.nk, acc, !kFused, !kFused, a.flat_in != 0, a.k_linear != 0);
     const int m0 = pix0 + wpix * 64 + l32;
     if constexpr (PIXC) {   // MatMul between activations whose right operand is stored as level - 128
         const int32_t* pc = a.pix_corr + static_cast<int64_t>(batch) * a.batch_pix_corr;
@@ -1442,6 +1442,12 @@ struct PackedGemm {
     DeviceBuffer wgt, koff, corr;
     // `keep`: receives the packed matrix ([OCp][Kp], rows in MFMA order) for a second packing derived from it
     void pack(int device, const hipie_conv_desc& d, const int8_t* weights, std::vector<int8_t>* keep = nullptr);
+    // A grouped convolution (weights [oc][ic / groups][kh][kw]) whose 64-channel output tiles each read one contiguous
+    // span of `span` input channels: K holds the span only (taps x span bytes), and every tile has a K-offset table of
+    // its own that starts at its span (koff_tile entries from one tile's table to the next)
+    static bool grouped_fits(const hipie_conv_desc& d, int64_t* span);
+    void pack_grouped(int device, const hipie_conv_desc& d, const int8_t* weights, int64_t span);
+    int64_t koff_tile = 0;
 };
 
 struct hipie_conv {
@@ -1449,6 +1455,7 @@ struct hipie_conv {
     hipie_conv_desc d{};
     int64_t K = 0, Kp = 0, OCp = 0;
     bool k_linear = false;         // PackedGemm::linear of the main convolution
+    int64_t koff_tile = 0;         // grouped convolution in its own form: entries from one 64-channel tile's K offsets to the next
     // fused shortcut convolution (second operand set + its bias / scale tables)
     bool fused = false;
     hipie_conv_desc sd{};
@@ -1534,6 +1541,63 @@ void PackTape::give(const void* src, size_t bytes) {
     blobs.emplace_back(b, b + bytes);
 }
 }  // namespace hipie
+
+bool PackedGemm::grouped_fits(const hipie_conv_desc& d, int64_t* span) {
+    if (d.groups <= 1 || d.ic % d.groups || d.oc % d.groups || d.oc % 64 || d.in_c_stride % 16) return false;
+    const int64_t icg = d.ic / d.groups, ocg = d.oc / d.groups;
+    int64_t s = 0;
+    if (64 % ocg == 0) s = (64 / ocg) * icg;          // a tile holds whole groups: their input channels, side by side
+    else if (ocg % 64 == 0) s = icg;                   // a tile lies inside one group
+    else return false;
+    // a tile's span starts at a multiple of 16 bytes and is whole 16-byte pieces; and it must be a real part of the
+    // input (a layer whose every tile reads every channel gains nothing over the dense form)
+    if (s % 16 != 0 || s >= d.ic) return false;
+    *span = s;
+    return true;
+}
+
+void PackedGemm::pack_grouped(int device, const hipie_conv_desc& d, const int8_t* weights, int64_t span) {
+    const int64_t icg = d.ic / d.groups, ocg = d.oc / d.groups, taps = static_cast<int64_t>(d.kh) * d.kw;
+    K = taps * span;
+    Kp = round_up(K, 64);
+    OCp = round_up(d.oc, 128);
+    linear = false;
+    const int64_t tiles = d.oc / 64;
+    koff_tile = Kp / 16;
+    auto span_start = [&](int64_t tile) { return ((tile * 64) / ocg) * icg; };   // first input channel a tile reads
+    std::vector<int32_t> off(static_cast<size_t>(round_up(d.oc, 128) / 64 * koff_tile), 0);   // (a padding tile reads its neighbour's span: zero weights)
+    for (int64_t t = 0; t < static_cast<int64_t>(off.size()) / koff_tile; ++t)
+        for (int64_t p = 0; p < K / 16; ++p) {
+            const int64_t k = p * 16, tap = k / span, ic0 = k % span, kh = tap / d.kw, kw = tap % d.kw;
+            off[static_cast<size_t>(t * koff_tile + p)] = static_cast<int32_t>(kh * d.dil_h * d.in_stride_h + kw * d.dil_w * d.in_stride_w +
+                                                                                  span_start(std::min(t, tiles - 1)) + ic0);
+        }
+    std::vector<int8_t> w(static_cast<size_t>(OCp) * Kp, 0);
+    std::vector<int32_t> cr(OCp, 0);
+    const int stored_zero = d.in_dtype == HIPIE_U8B ? 128 : 0;
+    PackTape* tape = PackTape::current();
+    const bool played = tape && tape->take(w.data(), w.size()) && tape->take(cr.data(), cr.size() * sizeof(int32_t));
+    if (!played) parallel_for(d.oc, [&](int64_t oc) {
+        const int64_t first = (oc / ocg) * icg, base = span_start(oc / 64);   // the group's channels inside the tile's span
+        int64_t corr = 0;
+        for (int64_t t = 0; t < taps; ++t)
+            for (int64_t i = 0; i < icg; ++i) {
+                const int8_t v = weights[(oc * icg + i) * taps + t];
+                w[static_cast<size_t>(packed_row(oc) * Kp + t * span + (first - base) + i)] = v;
+                corr += static_cast<int64_t>(stored_zero - zero_point_of(d, static_cast<int>(first + i))) * v;
+            }
+        cr[oc] = static_cast<int32_t>(corr - (d.acc_sub ? d.acc_sub[oc] : 0));
+    });
+    if (tape && !played) {
+        tape->give(w.data(), w.size());
+        tape->give(cr.data(), cr.size() * sizeof(int32_t));
+    }
+    if (device >= 0) {
+        wgt.upload(device, w.data(), w.size());
+        koff.upload(device, off.data(), off.size() * sizeof(int32_t));
+        corr.upload(device, cr.data(), cr.size() * sizeof(int32_t));
+    }
+}
 
 void PackedGemm::pack(int device, const hipie_conv_desc& d, const int8_t* weights, std::vector<int8_t>* keep) {
     // K order (kh, kw, ic) over the padded channel stride.  A 16-byte piece must not straddle
@@ -1829,7 +1893,9 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
                       HIPIE_PARAMETER_MISMATCH, "hipie_conv_create: bad geometry");
         HIPIE_REQUIRE(d.groups >= 1 && d.ic % d.groups == 0 && d.oc % d.groups == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_create: groups=%d does not divide ic=%d and oc=%d", d.groups, d.ic, d.oc);
-        if (d.groups > 1 && (!(d.groups == d.ic && d.ic == d.oc) || d.in_c_stride % 16 != 0)) {
+        int64_t group_span = 0;
+        const bool grouped_own = d.groups > 1 && !(d.groups == d.ic && d.ic == d.oc) && PackedGemm::grouped_fits(d, &group_span);
+        if (d.groups > 1 && !grouped_own && (!(d.groups == d.ic && d.ic == d.oc) || d.in_c_stride % 16 != 0)) {
             // A grouped convolution that is not depthwise (weights [oc][ic / groups][kh][kw]) is the dense convolution
             // with block-diagonal weights: reference::group_convolution (group_convolution.hpp:78-144) convolves every
             // slice on its own, and the products added here are zeros.  So is a depthwise one over pixels that are
@@ -1847,7 +1913,7 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
             if (st != HIPIE_OK) fail(static_cast<hipie_status>(st), "%s", std::string(hipie_last_error()).c_str());
             return;
         }
-        const bool depthwise = d.groups > 1;
+        const bool depthwise = d.groups > 1 && !grouped_own;
         HIPIE_REQUIRE(d.in_c_stride >= d.ic && d.in_c_stride % 4 == 0, HIPIE_PARAMETER_MISMATCH,
                       "hipie_conv_create: in_c_stride=%d must be a multiple of 4 >= ic=%d", d.in_c_stride, d.ic);
         {
@@ -1896,6 +1962,19 @@ int hipie_conv_create(int device, const hipie_conv_desc* desc, const int8_t* wei
                 c->corr.upload(device, corr.data(), corr.size() * sizeof(int32_t));
                 if (!rows.empty()) c->wgt_rows.upload(device, rows.data(), rows.size() * sizeof(uint32_t));
             }
+            *out = c.release();
+            return;
+        }
+        if (grouped_own) {
+            // the grouped form: tiles of 64 output channels over the K bytes of their own groups, in the tiled kernels
+            // whose channel tile is 64 wide (variants 1 and 2)
+            PackedGemm g;
+            g.pack_grouped(device, d, weights, group_span);
+            c->K = g.K; c->Kp = g.Kp; c->OCp = g.OCp;
+            c->wgt = std::move(g.wgt); c->koff = std::move(g.koff); c->corr = std::move(g.corr);
+            c->koff_tile = g.koff_tile;
+            c->epi.build(device, *epilogue, d.oc, c->OCp);
+            c->tile = 1;
             *out = c.release();
             return;
         }
@@ -1990,6 +2069,12 @@ int hipie_conv_set_tile(hipie_conv* c, int tile) {
                                                           c->d.in_c_stride, static_cast<int>(c->OCp), c->epi.flags)) ||
                               (tile == 2 && matrix_ok),
                           HIPIE_PARAMETER_MISMATCH, "hipie_conv_set_tile: depthwise variant %d does not take this layer", tile);
+            c->tile = tile;
+            return;
+        }
+        if (c->koff_tile) {   // a grouped convolution in its own form: the tiled kernels with 64-channel tiles
+            HIPIE_REQUIRE(tile == 1 || tile == 2, HIPIE_PARAMETER_MISMATCH,
+                          "hipie_conv_set_tile: a grouped convolution runs in the tiled kernels with 64-channel tiles (variants 1, 2)");
             c->tile = tile;
             return;
         }
@@ -2100,6 +2185,7 @@ static int64_t fill_conv_args(const hipie_conv* c, const hipie_tensor* in, const
     a.out = out->data;
     a.koff = c->koff.as<int32_t>();
     a.k_linear = c->k_linear ? 1 : 0;
+    a.koff_tile = static_cast<int32_t>(c->koff_tile);
     a.corr = c->corr.as<int32_t>();
     c->epi.fill(a);
     if (a.flags & CF_RES_GEMM) {

@@ -143,6 +143,8 @@ struct ConvArgs {
     int32_t flat_in, flat_out, flat_res;
     // the K pieces of the convolution (of the fused shortcut) lie one behind the other in memory: koff[p] == 16 p
     int32_t k_linear, k_linear2;
+    // grouped convolution in its own form: channel tile t (64 channels) reads its K offsets at koff + t * koff_tile
+    int32_t koff_tile;
     // row-tile kernel (3 x 3, stride 1): output rows per tile, tiles per image, patch width OW + 2 and its reciprocal
     int32_t rows_per_tile, tiles_per_image, patch_w;
     float inv_patch_w;

@@ -2193,9 +2193,13 @@ struct Planner {
             // zeros added here, and integer sums do not change with them)
             const bool depthwise = grouped && W.shape[1] == 1 && W.shape[2] == 1;
             const int64_t G = grouped ? W.shape[0] : 1, ocg = grouped ? W.shape[1] : 0, icg = grouped ? W.shape[2] : 0;
-            if (depthwise) d.groups = static_cast<int>(G);
             OC = grouped ? G * ocg : W.shape[0];
             IC = grouped ? G * icg : W.shape[1];
+            // groups of 16-byte-aligned channel spans under tiles of 64 output channels run in the grouped form of the
+            // tiled kernels (hipie_conv_create decides by the same rule); the weights go to it as they are
+            const bool own_form = grouped && !depthwise && G > 1 && OC % 64 == 0 &&
+                                  ((64 % ocg == 0 && ((64 / ocg) * icg) % 16 == 0 && (64 / ocg) * icg < IC) || (ocg % 64 == 0 && icg % 16 == 0));
+            if (depthwise || own_form) d.groups = static_cast<int>(G);
             grouped_macs_div = grouped && !depthwise ? G : 1;
             d.kh = static_cast<int>(W.shape[grouped ? 3 : 2]); d.kw = static_cast<int>(W.shape[grouped ? 4 : 3]);
             d.stride_h = static_cast<int>(n.strides[0]); d.stride_w = static_cast<int>(n.strides[1]);
@@ -2203,7 +2207,7 @@ struct Planner {
             d.pad_top = static_cast<int>(n.pads_begin[0]); d.pad_left = static_cast<int>(n.pads_begin[1]);
             d.pad_bottom = static_cast<int>(n.pads_end[0]); d.pad_right = static_cast<int>(n.pads_end[1]);
             const int8_t* wsrc = reinterpret_cast<const int8_t*>(W.data.data());
-            if (grouped && !depthwise) {
+            if (grouped && !depthwise && !own_form) {
                 const int64_t taps = static_cast<int64_t>(d.kh) * d.kw;
                 st->weights.assign(static_cast<size_t>(OC * IC * taps), 0);
                 for (int64_t gi = 0; gi < G; ++gi)
@@ -2315,7 +2319,7 @@ struct Planner {
         st->out = new_tensor(cur, e.out_dtype, nn, h, w, c);
         st->name = N(cur).name;
         st->type = is_mm ? "MatMul" : (n.op == OP_GROUP_CONVOLUTION ? "GroupConvolution" : "Convolution");
-        st->macs = N(id).numel() * (d.groups > 1 ? 1 : IC / grouped_macs_div) * d.kh * d.kw + (st->shortcut ? st->shortcut->macs : 0);
+        st->macs = N(id).numel() * (IC / std::max<int64_t>(d.groups, grouped_macs_div)) * d.kh * d.kw + (st->shortcut ? st->shortcut->macs : 0);
         st->results = N(id).numel();
         // algorithmic HBM bytes: every operand once (input, weights, output, residual); a fused
         // projection shortcut adds its input and weights and removes the f32 residual round trip
@@ -2323,7 +2327,7 @@ struct Planner {
             const TensorInfo& ti = tensors[t];
             return static_cast<int64_t>(ti.n) * ti.h * ti.w * ti.c * ti.esize();
         };
-        st->in_w_bytes = elems(st->in) + static_cast<int64_t>(OC) * (d.groups > 1 ? 1 : IC) * d.kh * d.kw;
+        st->in_w_bytes = elems(st->in) + static_cast<int64_t>(OC) * (IC / std::max<int64_t>(d.groups, 1)) * d.kh * d.kw;
         st->bytes = st->in_w_bytes + elems(st->out);
         if (st->shortcut) st->bytes += st->shortcut->in_w_bytes;
         else if (st->res >= 0) st->bytes += elems(st->res);

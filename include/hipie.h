@@ -187,8 +187,13 @@ typedef struct hipie_conv_desc {
     int32_t pad_top, pad_left, pad_bottom, pad_right;
     int32_t groups;                       /* 1 = dense (weights [oc][ic][kh][kw]); > 1: weights [oc][ic / groups][kh][kw]
                                              (group_convolution.hpp:78-144); groups == ic == oc (depthwise) has kernels of
-                                             its own, any other grouping runs as the dense convolution with
-                                             block-diagonal weights that it equals */
+                                             its own; groups whose input channels lie in 16-byte-aligned spans under tiles
+                                             of 64 output channels (oc a multiple of 64; 64 a multiple of oc / groups with
+                                             (64 / (oc / groups)) * (ic / groups) a multiple of 16 and less than ic, or
+                                             oc / groups a multiple of 64 with ic / groups a multiple of 16) multiply the
+                                             K bytes of their own groups only (variants 1 and 2 of hipie_conv_set_tile);
+                                             any other grouping runs as the dense convolution with block-diagonal
+                                             weights that it equals */
     int32_t in_c_stride;                  /* channel stride of the input tensor (>= ic) */
     int32_t in_stride_h, in_stride_w;     /* element strides of the input tensor */
     int32_t in_zero_point;                /* integer level subtracted from every input element: the

@@ -532,6 +532,42 @@ def test_group_convolution_with_several_channels_per_group(orc, G, icg, ocg):
     np.testing.assert_array_equal(out.to_nchw(), want)
 
 
+@pytest.mark.parametrize("tile", [1, 2])
+@pytest.mark.parametrize("G,icg,ocg,k", [(32, 4, 4, 3), (16, 8, 8, 3), (4, 64, 64, 3), (2, 128, 128, 1), (3, 16, 64, 3), (8, 32, 32, 1)])
+def test_group_convolution_in_its_own_form(orc, G, icg, ocg, k, tile):
+    """groups whose input channels lie in 16-byte-aligned spans under tiles of 64 output channels (ResNeXt cardinalities:
+    32 x 4, 16 x 8, 8 x 32; wide groups of 64 and 128 channels; 192 output channels, a ragged 128-channel tile): every
+    tile multiplies the K bytes of its own groups only, with a K-offset table of its own.  Both tiled kernels with
+    64-channel tiles, per-channel zero points, stride, padding; i32 sums exact against
+    reference::group_convolution on widened inputs"""
+    from dldt_amd import Convolution, DeviceTensor
+    rng = np.random.default_rng(G * 1000 + icg * 10 + k)
+    N, H, W = 2, 11, 9
+    C, OC = G * icg, G * ocg
+    x = rng.integers(0, 256, (N, C, H, W)).astype(np.int32)
+    w = rng.integers(-127, 128, (G, ocg, icg, k, k)).astype(np.int32)
+    zp = rng.integers(0, 256, C).astype(np.int32)
+    pad = k // 2
+    want = orc.convolution(x - zp.reshape(1, C, 1, 1), w, (1, 2), (1, 1), (pad, pad), (pad, pad), grouped=True)
+    xin = DeviceTensor.from_nchw(x, U8B, halo=pad, fill_level=0)
+    if pad:
+        import torch
+        full = xin.view
+        pattern = torch.from_numpy((zp - 128).astype(np.int8)).to(full.device)
+        full[:, 0, :, :C] = pattern
+        full[:, -1, :, :C] = pattern
+        full[:, :, 0, :C] = pattern
+        full[:, :, -1, :C] = pattern
+    conv = Convolution(w.astype(np.int8), xin, (1, 2), (1, 1), (pad, pad), (pad, pad), zero_point=zp)
+    conv.set_tile(tile)
+    assert conv.get_tile() == tile
+    with pytest.raises(Exception):
+        conv.set_tile(4)                  # the dense kernels do not know the per-tile tables
+    out = DeviceTensor(N, want.shape[2], want.shape[3], OC, I32)
+    conv.run(xin, out)
+    np.testing.assert_array_equal(out.to_nchw(), want)
+
+
 _WIDE_CASES = {}
 
 

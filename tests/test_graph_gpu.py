@@ -538,6 +538,36 @@ def test_grouped_convolution_in_a_graph(orc):
     np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))
 
 
+@pytest.mark.parametrize("groups,width", [(32, 128), (8, 256)])
+def test_resnext_block_through_the_planner(orc, groups, width):
+    """a ResNeXt bottleneck (1 x 1 reduce, grouped 3 x 3 with cardinality 32 x 4 or 8 x 32, 1 x 1 expand with the residual
+    Add): the grouped layer runs in its own form (its step counts a groups-th of the dense multiply-accumulates and is
+    tuned over the two 64-channel-tile kernels), everything bit-exact"""
+    from dldt_amd.builders import QuantizedNet
+    rng = np.random.default_rng(groups)
+    n, c, hw = 2, 64, 14
+    x = rng.uniform(0, 1, (n, c, hw, hw)).astype(np.float32)
+    net = QuantizedNet()
+    g = net.g
+    wn = lambda *s, k=0.1: (rng.standard_normal(s, dtype=np.float32) * np.float32(k)).astype(np.float32)
+    a0 = net.input("data", x.shape, 1.0)
+    a1 = net.conv(a0, wn(width, c, 1, 1), wn(width, k=0.2), 2.0)
+    a2 = net.conv(a1, wn(width, width // groups, 3, 3, k=0.2), wn(width, k=0.2), 2.5, pads=(1, 1), groups=groups)
+    g.result(net.conv_f32(a2, wn(48, width, 1, 1), wn(48, k=0.2)), "out")
+    want, kept = evaluate(orc, g.nodes, dict(data=x), keep=[a2["node"]])
+    plan = g.compile()
+    steps = [s for s in plan.steps if s["type"] == "GroupConvolution"]
+    assert len(steps) == 1 and steps[0]["macs"] == n * hw * hw * width * (width // groups) * 9 and steps[0]["variant"] in (1, 2)
+    req = plan.create_request()
+    (got,) = req.infer(x)
+    np.testing.assert_array_equal(req.tensor(a2["node"]), kept[a2["node"]])
+    np.testing.assert_array_equal(got.view(np.uint32), want["out"].view(np.uint32))
+    blob = plan.export()                                 # the packed grouped operands travel in the stream too
+    from dldt_amd.graph import Plan
+    (again,) = Plan.load(blob).create_request().infer(x)
+    np.testing.assert_array_equal(again.view(np.uint32), got.view(np.uint32))
+
+
 @pytest.mark.parametrize("mode", ["YES", "NO", "AUTO"])
 def test_bottleneck_tails_as_one_kernel(orc, mode):
     """HIP_FUSE_CONVOLUTIONS: the 3 x 3 convolution of a bottleneck block and the 1 x 1 convolution with the residual add
