@@ -574,8 +574,9 @@ struct PoolStep : Step {
 // Result: engine tensor -> dense NCHW output buffer of the request (f32, or u8 levels)
 // Concat of byte tensors along the channel axis: one strided copy per input into its channel slice
 struct ConcatStep : Step {
-    std::vector<int> ins, c_off;
+    std::vector<int> ins, c_off;      // c_off: where the input starts along `axis` of the output
     int out = -1;
+    int axis = 1;                     // of [N, C, H, W]
     void create(int, const std::vector<TensorInfo>&) override {}
     void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const*, void* const*, hipStream_t s) const override {
         const hipie_tensor o = tensors[out].desc(arena);
@@ -588,7 +589,11 @@ struct ConcatStep : Step {
             a.N = x.n; a.H = x.h; a.W = x.w; a.C = x.c * es;
             a.in_sn = x.stride_n * es; a.in_sh = x.stride_h * es; a.in_sw = x.stride_w * es;
             a.out_sn = o.stride_n * es; a.out_sh = o.stride_h * es; a.out_sw = o.stride_w * es;
-            a.c_off = c_off[i] * es;
+            // the input copied into its box of the output: first element moved along the axis, same walk
+            a.c_off = axis == 1 ? c_off[i] * es : 0;
+            if (axis == 0) a.out += c_off[i] * a.out_sn;
+            else if (axis == 2) a.out += c_off[i] * a.out_sh;
+            else if (axis == 3) a.out += c_off[i] * a.out_sw;
             launch_concat_channels(a, s);
         }
         HIPIE_CHECK_HIP(hipGetLastError());
@@ -599,6 +604,7 @@ struct ConcatStep : Step {
 struct EltwiseStep : Step {
     struct Operand {
         int tensor = -1;                 // arena tensor, or -1: per-channel constant
+        bool bn = false, bh = false, bw = false;   // the tensor has one element along N / H / W and is repeated along it
         std::vector<float> sub, mul, konst;
         DeviceBuffer d_sub, d_mul, d_konst;
     };
@@ -643,7 +649,7 @@ struct EltwiseStep : Step {
                 const hipie_tensor t = tensors[o.tensor].desc(arena);
                 d.p = t.data;
                 d.dtype = t.dtype;
-                d.sn = t.stride_n; d.sh = t.stride_h; d.sw = t.stride_w;
+                d.sn = o.bn ? 0 : t.stride_n; d.sh = o.bh ? 0 : t.stride_h; d.sw = o.bw ? 0 : t.stride_w;
             }
             d.sub = o.sub.empty() ? nullptr : o.d_sub.as<float>();
             d.mul = o.mul.empty() ? nullptr : o.d_mul.as<float>();
@@ -2461,8 +2467,10 @@ struct Planner {
     // behind the Concat): the levels are copied side by side
     void plan_concat(int id) {
         const GNode& n = N(id);
-        if (n.shape.size() != 4 || n.axes[0] != 1) unsupported(id, "Concat is planned along the channel axis of 4-D tensors");
+        if (n.shape.size() != 4) unsupported(id, "Concat is planned on 4-D tensors");
         auto st = std::make_unique<ConcatStep>();
+        st->axis = static_cast<int>(n.axes[0]);
+        const int ax = st->axis;
         int dtype = -1, off = 0;
         int64_t bytes = 0;
         for (int in : n.in) {
@@ -2474,7 +2482,7 @@ struct Planner {
             dtype = tensors[x.tensor].dtype;
             st->ins.push_back(x.tensor);
             st->c_off.push_back(off);
-            off += tensors[x.tensor].c;
+            off += static_cast<int>(N(in).shape[static_cast<size_t>(ax)]);
             bytes += N(in).numel() * tensors[x.tensor].esize();
         }
         int nn, c, h, w;
@@ -2505,7 +2513,16 @@ struct Planner {
                 return;
             }
             const Value x = value(in);
-            if (N(in).shape != n.shape) unsupported(id, "elementwise operands of different shapes (broadcast between tensors)");
+            // numpy broadcasting between two tensors along the batch and the spatial axes (a per-image, per-channel
+            // factor [N, C, 1, 1] on a feature map, a per-pixel map shared by the batch, ...); not along the channels
+            const std::vector<int64_t>& xs = N(in).shape;
+            if (xs.size() != n.shape.size() || (xs.size() > 1 && xs[1] != n.shape[1]))
+                unsupported(id, "elementwise operands that differ in rank or in their channels (broadcast along the channel axis)");
+            for (size_t k = 0; k < xs.size(); ++k) {
+                if (xs[k] == n.shape[k]) continue;
+                if (xs[k] != 1) unsupported(id, "elementwise operands whose shapes do not broadcast");
+                (k == 0 ? o.bn : (k == 2 ? o.bh : o.bw)) = true;
+            }
             if (x.kind == VK_DEQ) {
                 o.tensor = x.tensor;
                 o.sub = x.sub;

@@ -39,7 +39,8 @@ struct ExitArgs {
 };
 
 // Concat along the channel axis of byte NHWC tensors: one input's C channels copied to channels [c_off, c_off + C) of
-// the output (reference::concat, concat.hpp:17-57, is the same copy in NCHW order)
+// the output (reference::concat, concat.hpp:17-57, is the same copy in NCHW order).  Along N, H or W the caller moves
+// `out` to the first element of the input's box and passes c_off = 0.
 struct ConcatArgs {
     const int8_t* in;
     int8_t* out;

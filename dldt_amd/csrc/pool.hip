@@ -246,10 +246,11 @@ __global__ __launch_bounds__(256) void concat_channels_kernel(const ConcatArgs a
 void launch_concat_channels(const ConcatArgs& a, hipStream_t s) {
     const int64_t pixels = static_cast<int64_t>(a.N) * a.H * a.W;
     if (pixels == 0 || a.C == 0) return;
-    const bool al16 = a.C % 16 == 0 && a.c_off % 16 == 0 && a.out_sw % 16 == 0 && reinterpret_cast<uintptr_t>(a.out) % 16 == 0 &&
-                      reinterpret_cast<uintptr_t>(a.in) % 16 == 0 && a.in_sw % 16 == 0;
-    const bool al4 = a.C % 4 == 0 && a.c_off % 4 == 0 && a.out_sw % 4 == 0 && reinterpret_cast<uintptr_t>(a.out) % 4 == 0 &&
-                     reinterpret_cast<uintptr_t>(a.in) % 4 == 0 && a.in_sw % 4 == 0;
+    auto aligned = [&](int v) {
+        return a.C % v == 0 && a.c_off % v == 0 && reinterpret_cast<uintptr_t>(a.out) % v == 0 && reinterpret_cast<uintptr_t>(a.in) % v == 0 &&
+               a.out_sw % v == 0 && a.out_sh % v == 0 && a.out_sn % v == 0 && a.in_sw % v == 0 && a.in_sh % v == 0 && a.in_sn % v == 0;
+    };
+    const bool al16 = aligned(16), al4 = aligned(4);
     const int vec = al16 ? 16 : (al4 ? 4 : 1);
     const int32_t pieces = a.C / vec;
     const int64_t total = pixels * pieces;

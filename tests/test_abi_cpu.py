@@ -263,7 +263,7 @@ def test_exec_graph_attributes_per_step():
 
 def test_concat_shape_inference_and_planner_limits():
     """Concat infers its shape like op::v0::Concat (negative axis included), refuses mismatched inputs when the graph
-    is described, and the planner takes it along the channels of quantized 4-D tensors only"""
+    is described, and the planner takes it on 4-D tensors (bytes or f32), along any axis"""
     from dldt_amd import HipieError, builders
     from dldt_amd.graph import Graph
     from dldt_amd.tensor import U8
@@ -286,6 +286,13 @@ def test_concat_shape_inference_and_planner_limits():
     assert tuple(plan.outputs[0]["shape"]) == (2, 24 + 40 + 16, 18, 18)
     sup = g2.query()
     assert all(sup)
+    # along the rows: the output takes the sum of the inputs' heights
+    net = builders.QuantizedNet()
+    q = net.input("data", (2, 8, 5, 6), 1.0)
+    tall = net.g.concat([q["node"], q["node"], q["node"]], axis=2)
+    net.g.result(net.dequantize(dict(node=tall, scale=q["scale"])), "tall")
+    plan = net.g.compile(-1)
+    assert [s["type"] for s in plan.steps].count("Concat") == 1 and tuple(plan.outputs[0]["shape"]) == (2, 8, 15, 6)
 
 
 def test_matmul_zero_point_correction_must_be_integers():

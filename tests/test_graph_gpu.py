@@ -478,6 +478,91 @@ def test_concat_of_quantized_branches(orc, branches, signed):
     np.testing.assert_array_equal(got2["out"].view(np.uint32), want2["out"].view(np.uint32))
 
 
+@pytest.mark.parametrize("axis", [0, 2, 3, -1])
+@pytest.mark.parametrize("quantized", [True, False])
+def test_concat_along_the_batch_and_the_spatial_axes(orc, axis, quantized):
+    """Concat along N, H or W: every input lands in its box of the output (boxes of unequal extent along H and W);
+    u8 branches with one shared interval and f32 branches, and a padded convolution that reads across the seam"""
+    from dldt_amd import builders
+    rng = np.random.default_rng(300 + axis)
+    x = rng.uniform(0, 1, (2, 12, 11, 13)).astype(np.float32)
+    ax = axis % 4
+    kernels = [(1, 1), (3, 1) if ax == 2 else ((1, 3) if ax == 3 else (1, 1)), (1, 1)]
+    net = builders.QuantizedNet()
+    g = net.g
+    branches = []
+    if quantized:
+        a0 = net.input("data", x.shape, 1.0)
+        for k in kernels:
+            w = (rng.standard_normal((20, 12) + k, dtype=np.float32) * np.float32(0.15)).astype(np.float32)
+            b = (rng.standard_normal(20, dtype=np.float32) * np.float32(0.3)).astype(np.float32)
+            branches.append(net.conv(a0, w, b, 2.5))
+        cat = dict(node=g.concat([a["node"] for a in branches], axis=axis), scale=branches[0]["scale"])
+        node = cat["node"]
+        g.result(net.dequantize(cat), "cat")
+        w = (rng.standard_normal((24, 20, 3, 3), dtype=np.float32) * np.float32(0.05)).astype(np.float32)
+        g.result(net.conv_f32(cat, w, np.zeros(24, np.float32), pads=(1, 1)), "out")
+    else:
+        p = g.parameter("data", x.shape)
+        for k in kernels:
+            w = (rng.standard_normal((20, 12) + k, dtype=np.float32) * np.float32(0.15)).astype(np.float32)
+            branches.append(g.relu(g.convolution(p, g.constant(w))))
+        node = g.concat(branches, axis=axis)
+        g.result(node, "cat")
+        g.result(g.max_pool(node, (3, 3), (1, 1), (1, 1), (1, 1)), "out")
+    want, kept = evaluate(orc, g.nodes, {"data": x}, keep=[node])
+    assert want["cat"].shape[ax] == {0: 6, 2: 31, 3: 37}[ax]
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps].count("Concat") == 1
+    req = plan.create_request()
+    got = dict(zip([o["name"] for o in plan.outputs], req.infer(x)))
+    np.testing.assert_array_equal(req.tensor(node).view(np.uint8), kept[node].view(np.uint8))
+    for name in ("cat", "out"):
+        np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
+    assert all(g.query())
+
+
+def test_elementwise_broadcast_between_tensors(orc):
+    """Multiply / Add of a feature map with a value that has one element along the batch or the spatial axes: a
+    per-image, per-channel gate [N, C, 1, 1] (a squeeze-and-excitation block's), a map [1, C, H, W] shared by the batch
+    and a row [N, C, 1, W]; operands on either side, dequantized bytes and f32"""
+    from dldt_amd import builders
+    rng = np.random.default_rng(311)
+    x = rng.uniform(0, 1, (3, 16, 9, 10)).astype(np.float32)
+    shared = rng.uniform(-1, 1, (1, 16, 9, 10)).astype(np.float32)
+    row = rng.uniform(-1, 1, (3, 16, 1, 10)).astype(np.float32)
+    net = builders.QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    w = (rng.standard_normal((16, 16, 3, 3), dtype=np.float32) * np.float32(0.08)).astype(np.float32)
+    b = (rng.standard_normal(16, dtype=np.float32) * np.float32(0.2)).astype(np.float32)
+    fmap = net.conv(a0, w, b, 2.0, pads=(1, 1))                         # u8 feature map
+    # squeeze: global average of the dequantized map, a 1 x 1 convolution on it, its result [N, C, 1, 1] in f32
+    pooled = g.avg_pool(net.dequantize(fmap), (9, 10), (1, 1), (0, 0), (0, 0), exclude_pad=False)
+    wg = (rng.standard_normal((16, 16, 1, 1), dtype=np.float32) * np.float32(0.4)).astype(np.float32)
+    gate = g.relu(g.convolution(pooled, g.constant(wg)))
+    gated = g.multiply(net.dequantize(fmap), gate)                      # [N, C, H, W] * [N, C, 1, 1]
+    q = net.requantize(gated, 1.5)
+    g.result(net.dequantize(q), "gated")
+    ps = g.parameter("shared", shared.shape)
+    pr = g.parameter("row", row.shape)
+    g.result(g.add(ps, net.dequantize(fmap)), "plus_shared")            # the small operand first
+    g.result(g.subtract(net.dequantize(fmap), pr), "minus_row")
+    g.result(g.multiply(ps, pr), "outer")                               # both sides repeat: [1,C,H,W] * [N,C,1,W]
+    feeds = {"data": x, "shared": shared, "row": row}
+    want, kept = evaluate(orc, g.nodes, feeds, keep=[q["node"]])
+    plan = g.compile()
+    req = plan.create_request()
+    order = [feeds[i["name"]] for i in plan.inputs]
+    got = dict(zip([o["name"] for o in plan.outputs], req.infer(*order)))
+    assert len(np.unique(kept[q["node"]])) > 30
+    np.testing.assert_array_equal(req.tensor(q["node"]), kept[q["node"]])
+    for name in ("gated", "plus_shared", "minus_row", "outer"):
+        assert got[name].shape == want[name].shape == (3, 16, 9, 10)
+        np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
+    assert all(g.query())
+
+
 @pytest.mark.parametrize("stride", [1, 2])
 def test_per_channel_activation_zero_points(orc, stride):
     """one integer zero point per channel in front of a padded depthwise convolution: the halo holds every channel's
