@@ -80,25 +80,25 @@ class QuantizedNet:
             assert np.all(per_group == per_group[:, :1])
             s_a = np.repeat(per_group[:, 0], s_w.size // G)
         s = (s_a * s_w).astype(np.float32)                                 # fold<Multiply>(s_a, s_w)
+        out_rank = 2 if matmul else w.ndim          # [N, C, H, W], or [N, C, W] for filters over one spatial dimension
         if groups:
             # [OC, IC / G, kh, kw] -> [G, OC / G, IC / G, kh, kw]
-            wq = wq.reshape(groups, wq.shape[0] // groups, wq.shape[1], wq.shape[2], wq.shape[3])
+            wq = wq.reshape((groups, wq.shape[0] // groups) + wq.shape[1:])
             conv_attrs["grouped"] = True
         elif conv_attrs.get("grouped"):
             # GroupConvolution weights: FQ on [C, 1, kh, kw] then Reshape to [G, 1, 1, kh, kw]
             # (the pattern LPT recognises, group_convolution.cpp:50-52); both fold into one constant
-            wq = wq.reshape(wq.shape[0], 1, 1, wq.shape[2], wq.shape[3])
+            wq = wq.reshape((wq.shape[0], 1, 1) + wq.shape[2:])
         wc = g.constant(wq, I8)
         x = act["node"]
         zp = np.asarray(act.get("zero_point", 0), np.float32)
         if np.any(zp != 0):                    # TypeRelaxed Subtract(u8, u8) -> f32, written as Convert + Subtract
-            x = g.subtract(g.convert(x, F32), g.constant(zp.reshape(()) if zp.ndim == 0 else self._channel(zp, 4)))
+            x = g.subtract(g.convert(x, F32), g.constant(zp.reshape(()) if zp.ndim == 0 else self._channel(zp, out_rank)))
+        rank = out_rank
         if matmul:
             y = g.matmul(x, wc, False, True)
-            rank = 2
         else:
             y = g.convolution(x, wc, **conv_attrs)
-            rank = 4
         if bias is not None:
             bdiv = lpt.swap_multiply_and_add(bias, s)                          # bi / ai
             y = g.add(y, g.constant(self._channel(bdiv, rank)))
@@ -139,7 +139,7 @@ class QuantizedNet:
     def conv_f32(self, act, w, bias, strides=(1, 1), pads=(0, 0), relu=False, matmul=False, grouped=False, groups=0):
         """Quantized conv / FC whose result is consumed in f32: ... -> Multiply(s[c]) [-> ReLU]."""
         g = self.g
-        attrs = dict(strides=strides, dilations=(1, 1), pads_begin=pads, pads_end=pads)
+        attrs = dict(strides=strides, dilations=(1,) * len(strides), pads_begin=pads, pads_end=pads)
         if grouped:
             attrs["grouped"] = True
         if groups:

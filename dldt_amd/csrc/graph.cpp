@@ -154,8 +154,10 @@ static int add_conv(hipie_graph* g, int x, int w, const int64_t* strides, const 
                       "%s: null argument", what);
         GNode& X = node(g, x, what);
         GNode& W = node(g, w, what);
-        HIPIE_REQUIRE(X.shape.size() == 4, HIPIE_NOT_IMPLEMENTED, "%s: only 2-D spatial", what);
-        HIPIE_REQUIRE(W.shape.size() == (grouped ? 5u : 4u), HIPIE_PARAMETER_MISMATCH, "%s: filter rank", what);
+        // [N, C, H, W] or [N, C, W]: one attribute per spatial dimension (three spatial dimensions are not taken)
+        HIPIE_REQUIRE(X.shape.size() == 4 || X.shape.size() == 3, HIPIE_NOT_IMPLEMENTED, "%s: one or two spatial dimensions", what);
+        const int sp = static_cast<int>(X.shape.size()) - 2;
+        HIPIE_REQUIRE(W.shape.size() == X.shape.size() + (grouped ? 1u : 0u), HIPIE_PARAMETER_MISMATCH, "%s: filter rank", what);
         const int o = grouped ? 1 : 0;
         const int64_t G = grouped ? W.shape[0] : 1;
         HIPIE_REQUIRE(X.shape[1] == W.shape[o + 1] * G, HIPIE_PARAMETER_MISMATCH,
@@ -164,13 +166,13 @@ static int add_conv(hipie_graph* g, int x, int w, const int64_t* strides, const 
         GNode n;
         n.op = grouped ? OP_GROUP_CONVOLUTION : OP_CONVOLUTION;
         n.in = {x, w};
-        n.strides.assign(strides, strides + 2);
-        n.dilations.assign(dilations, dilations + 2);
-        n.pads_begin.assign(pads_begin, pads_begin + 2);
-        n.pads_end.assign(pads_end, pads_end + 2);
+        n.strides.assign(strides, strides + sp);
+        n.dilations.assign(dilations, dilations + sp);
+        n.pads_begin.assign(pads_begin, pads_begin + sp);
+        n.pads_end.assign(pads_end, pads_end + sp);
         n.dtype = HIPIE_F32;  // TypeRelaxed<Convolution>: f32 holding the integer sum
         n.shape = {X.shape[0], W.shape[o] * G};
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < sp; ++i) {
             HIPIE_REQUIRE(n.strides[i] > 0 && n.dilations[i] > 0 && n.pads_begin[i] >= 0 && n.pads_end[i] >= 0 &&
                               std::max(std::max(n.strides[i], n.dilations[i]), std::max(n.pads_begin[i], n.pads_end[i])) < kMaxAttr,
                           HIPIE_PARAMETER_MISMATCH, "%s: attributes", what);
@@ -290,19 +292,20 @@ static int add_pool(hipie_graph* g, int op, int x, const int64_t* kernel, const 
         HIPIE_REQUIRE(id && kernel && strides && pads_begin && pads_end, HIPIE_PARAMETER_MISMATCH,
                       "%s: null argument", what);
         GNode& X = node(g, x, what);
-        HIPIE_REQUIRE(X.shape.size() == 4, HIPIE_NOT_IMPLEMENTED, "%s: only 2-D spatial", what);
+        HIPIE_REQUIRE(X.shape.size() == 4 || X.shape.size() == 3, HIPIE_NOT_IMPLEMENTED, "%s: one or two spatial dimensions", what);
+        const int sp = static_cast<int>(X.shape.size()) - 2;
         GNode n;
         n.op = op;
         n.in = {x};
-        n.kernel.assign(kernel, kernel + 2);
-        n.strides.assign(strides, strides + 2);
-        n.pads_begin.assign(pads_begin, pads_begin + 2);
-        n.pads_end.assign(pads_end, pads_end + 2);
+        n.kernel.assign(kernel, kernel + sp);
+        n.strides.assign(strides, strides + sp);
+        n.pads_begin.assign(pads_begin, pads_begin + sp);
+        n.pads_end.assign(pads_end, pads_end + sp);
         n.exclude_pad = exclude_pad != 0;
         n.ceil_mode = ceil_mode != 0;
         n.dtype = out_dtype;
         n.shape = {X.shape[0], X.shape[1]};
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < sp; ++i) {
             HIPIE_REQUIRE(kernel[i] > 0 && strides[i] > 0 && pads_begin[i] >= 0 && pads_end[i] >= 0 &&
                               std::max(std::max(kernel[i], strides[i]), std::max(pads_begin[i], pads_end[i])) < kMaxAttr,
                           HIPIE_PARAMETER_MISMATCH, "%s: attributes", what);
@@ -617,8 +620,11 @@ hipie_graph* deserialize_graph(const uint8_t* bytes, size_t size) {
         auto arity = [&](size_t n) {
             HIPIE_REQUIRE(in.size() == n, HIPIE_NETWORK_NOT_READ, "plan stream: node %u (%s) has %zu inputs", i, op_name(op), in.size());
         };
-        auto pair = [&](const std::vector<int64_t>& v) {
-            HIPIE_REQUIRE(v.size() == 2, HIPIE_NETWORK_NOT_READ, "plan stream: node %u (%s) lacks an attribute", i, op_name(op));
+        auto pair = [&](const std::vector<int64_t>& v) {     // one entry per spatial dimension of the node's input
+            HIPIE_REQUIRE(!in.empty() && in[0] >= 0 && in[0] < static_cast<int>(G->nodes.size()), HIPIE_NETWORK_NOT_READ,
+                          "plan stream: node %u (%s) reads a value that is not there", i, op_name(op));
+            const size_t rank = G->nodes[static_cast<size_t>(in[0])].shape.size();
+            HIPIE_REQUIRE(rank >= 3 && v.size() == rank - 2, HIPIE_NETWORK_NOT_READ, "plan stream: node %u (%s) lacks an attribute", i, op_name(op));
             return v.data();
         };
         int id = static_cast<int>(i), st = HIPIE_OK;

@@ -2682,6 +2682,70 @@ struct PlanPrepared {       // the host work an exported plan carries (hipie_pla
     PackTape tape;
 };
 
+// Convolutions and pools over one spatial dimension ([N, C, W]) are planned over two with H = 1 - what
+// reference::convolution does with its own shapes (extend_to_3D, convolution.hpp:148-167: unit dimensions in front of
+// the spatial ones, stride and dilation 1 and no padding along them).  Every rank-3 value connected to such a node
+// through nodes that keep the layout (FakeQuantize, elementwise, Convert, Concat, pools, convolutions, inputs and
+// results) becomes [N, C, 1, W]; the constants they read get the unit axis in the same place.  Returns false when
+// the graph has no such node (`out` is then untouched).
+bool lift_one_spatial_dimension(const hipie_graph& g, hipie_graph& out) {
+    auto spatial_op = [](int op) { return op == OP_CONVOLUTION || op == OP_GROUP_CONVOLUTION || op == OP_MAX_POOL || op == OP_AVG_POOL; };
+    auto keeps_layout = [&](int op) {
+        return spatial_op(op) || op == OP_FAKE_QUANTIZE || op == OP_ADD || op == OP_SUBTRACT || op == OP_MULTIPLY || op == OP_RELU ||
+               op == OP_CLAMP || op == OP_CONVERT || op == OP_CONCAT || op == OP_PARAMETER || op == OP_RESULT;
+    };
+    const int n_nodes = static_cast<int>(g.nodes.size());
+    std::vector<char> lift(g.nodes.size(), 0);
+    std::vector<int> stack;
+    for (int i = 0; i < n_nodes; ++i) {
+        const GNode& n = g.nodes[static_cast<size_t>(i)];
+        if (spatial_op(n.op) && n.shape.size() == 3) { lift[static_cast<size_t>(i)] = 1; stack.push_back(i); }
+    }
+    if (stack.empty()) return false;
+    auto take = [&](int v) {
+        const GNode& n = g.nodes[static_cast<size_t>(v)];
+        if (lift[static_cast<size_t>(v)] || n.shape.size() != 3 || !keeps_layout(n.op)) return;
+        lift[static_cast<size_t>(v)] = 1;
+        stack.push_back(v);
+    };
+    while (!stack.empty()) {
+        const int v = stack.back();
+        stack.pop_back();
+        const GNode& n = g.nodes[static_cast<size_t>(v)];
+        // (a convolution's filter and a FakeQuantize's bounds are constants: handled below, never part of the walk)
+        for (int in : n.in)
+            if (in >= 0 && g.nodes[static_cast<size_t>(in)].op != OP_CONSTANT) take(in);
+        for (int u : n.users) take(u);
+    }
+    out = g;
+    auto unit_axis = [](std::vector<int64_t>& shape, size_t at) { shape.insert(shape.begin() + static_cast<std::ptrdiff_t>(at), 1); };
+    auto front = [](std::vector<int64_t>& v, int64_t unit) { v.insert(v.begin(), unit); };
+    for (int i = 0; i < n_nodes; ++i) {
+        if (!lift[static_cast<size_t>(i)]) continue;
+        GNode& n = out.nodes[static_cast<size_t>(i)];
+        unit_axis(n.shape, 2);
+        if (spatial_op(n.op)) {
+            front(n.strides, 1);
+            front(n.pads_begin, 0);
+            front(n.pads_end, 0);
+            if (n.op == OP_MAX_POOL || n.op == OP_AVG_POOL) front(n.kernel, 1);
+            else front(n.dilations, 1);
+        }
+        if (n.op == OP_CONCAT && !n.axes.empty() && n.axes[0] == 2) n.axes[0] = 3;
+        for (size_t k = 0; k < n.in.size(); ++k) {
+            if (n.in[k] < 0) continue;
+            GNode& c = out.nodes[static_cast<size_t>(n.in[k])];
+            if (c.op != OP_CONSTANT) continue;
+            const bool filter = (n.op == OP_CONVOLUTION || n.op == OP_GROUP_CONVOLUTION) && k == 1;
+            const size_t full = filter ? (n.op == OP_GROUP_CONVOLUTION ? 4u : 3u) : 3u;
+            // filters [OC, IC, KW] / [G, OC/G, IC/G, KW] and constants that name the width axis: the unit axis goes in
+            // front of the last one; lower ranks align from the right as before, except [C, 1], which names the channels
+            if (c.shape.size() == full || (!filter && c.shape.size() == 2)) unit_axis(c.shape, c.shape.size() - 1);
+        }
+    }
+    return true;
+}
+
 std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const std::vector<int>* preset,
                                          const PlanConfig& cfg = PlanConfig::from_environment(), PlanPrepared* prepared = nullptr) {
     HIPIE_REQUIRE(!g->results.empty(), HIPIE_PARAMETER_MISMATCH, "hipie_compile: graph has no Result");
@@ -2689,7 +2753,10 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
                   "hipie_compile: DEVICE_ID %d against device %d", cfg.device_id, device);
     auto plan = std::make_unique<hipie_plan>();
     plan->device = device;
-    plan->graph = *g;
+    plan->graph = *g;                       // the description as it was given: what an exported plan carries
+    const hipie_graph* const described = g;
+    hipie_graph lifted;
+    if (lift_one_spatial_dimension(*g, lifted)) g = &lifted;
     if (prepared) {
         plan->verdicts = std::move(prepared->verdicts);
         plan->tape = std::move(prepared->tape);
@@ -2845,12 +2912,13 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
                 plan->node_slice[static_cast<int>(i)] = {v.tensor, v.offset, rows, cols, r >= 2 ? v.stride[r - 2] : cols};
             }
         }
-    for (int p : g->params) {
-        const GNode& n = g->nodes[p];
+    // (inputs and outputs in the shapes of the description: [N, C, W] and [N, C, 1, W] are the same bytes)
+    for (int p : described->params) {
+        const GNode& n = described->nodes[p];
         plan->inputs.push_back({n.name, n.dtype, n.shape, n.numel() * (n.dtype == HIPIE_F32 || n.dtype == HIPIE_I32 ? 4 : 1)});
     }
-    for (int r : g->results) {
-        const GNode& n = g->nodes[r];
+    for (int r : described->results) {
+        const GNode& n = described->nodes[r];
         const int dt = n.dtype == HIPIE_F32 ? HIPIE_F32 : HIPIE_U8;
         plan->outputs.push_back({n.name, dt, n.shape, n.numel() * (dt == HIPIE_F32 ? 4 : 1)});
     }
@@ -2961,6 +3029,10 @@ int hipie_query(const hipie_graph* g, int* supported, int n_nodes, int* n_unsupp
         HIPIE_REQUIRE(g && supported && n_nodes == static_cast<int>(g->nodes.size()), HIPIE_PARAMETER_MISMATCH,
                       "hipie_query: `supported` must hold one entry per node (%zu)", g ? g->nodes.size() : size_t(0));
         hipie_graph work = *g;
+        {
+            hipie_graph lifted;
+            if (lift_one_spatial_dimension(work, lifted)) work = std::move(lifted);
+        }
         for (int i = 0; i < n_nodes; ++i) supported[i] = 1;
         int bad = 0;
         const PlanConfig cfg = PlanConfig::from_environment();

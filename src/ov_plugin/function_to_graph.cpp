@@ -92,12 +92,12 @@ struct Translator {
         } else if (const auto conv = ngraph::as_type_ptr<ngraph::opset1::Convolution>(node)) {
             const auto s = as_i64(conv->get_strides()), dl = as_i64(conv->get_dilations());
             const auto pb = as_i64(conv->get_pads_begin()), pe = as_i64(conv->get_pads_end());
-            if (s.size() != 2) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is not a 2-D convolution";
+            if (s.size() != 2 && s.size() != 1) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is a convolution over three spatial dimensions";
             check(hipie_graph_convolution(g, in(n, 0), in(n, 1), s.data(), dl.data(), pb.data(), pe.data(), &id), "hipie_graph_convolution");
         } else if (const auto gconv = ngraph::as_type_ptr<ngraph::opset1::GroupConvolution>(node)) {
             const auto s = as_i64(gconv->get_strides()), dl = as_i64(gconv->get_dilations());
             const auto pb = as_i64(gconv->get_pads_begin()), pe = as_i64(gconv->get_pads_end());
-            if (s.size() != 2) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is not a 2-D convolution";
+            if (s.size() != 2 && s.size() != 1) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is a convolution over three spatial dimensions";
             check(hipie_graph_group_convolution(g, in(n, 0), in(n, 1), s.data(), dl.data(), pb.data(), pe.data(), &id),
                   "hipie_graph_group_convolution");
         } else if (const auto mm = ngraph::as_type_ptr<ngraph::opset1::MatMul>(node)) {
@@ -117,13 +117,13 @@ struct Translator {
         } else if (const auto mp = ngraph::as_type_ptr<ngraph::opset1::MaxPool>(node)) {
             const auto k = as_i64(mp->get_kernel()), s = as_i64(mp->get_strides());
             const auto pb = as_i64(mp->get_pads_begin()), pe = as_i64(mp->get_pads_end());
-            if (k.size() != 2) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is not a 2-D pooling";
+            if (k.size() != 2 && k.size() != 1) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is a pooling over three spatial dimensions";
             check(hipie_graph_max_pool(g, in(n, 0), k.data(), s.data(), pb.data(), pe.data(),
                                        mp->get_rounding_type() == ngraph::op::RoundingType::CEIL, &id), "hipie_graph_max_pool");
         } else if (const auto ap = ngraph::as_type_ptr<ngraph::opset1::AvgPool>(node)) {
             const auto k = as_i64(ap->get_kernel()), s = as_i64(ap->get_strides());
             const auto pb = as_i64(ap->get_pads_begin()), pe = as_i64(ap->get_pads_end());
-            if (k.size() != 2) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is not a 2-D pooling";
+            if (k.size() != 2 && k.size() != 1) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is a pooling over three spatial dimensions";
             check(hipie_graph_avg_pool(g, in(n, 0), k.data(), s.data(), pb.data(), pe.data(), ap->get_exclude_pad(),
                                        ap->get_rounding_type() == ngraph::op::RoundingType::CEIL,
                                        element_type(n.get_output_element_type(0), n), &id), "hipie_graph_avg_pool");

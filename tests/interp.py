@@ -21,6 +21,16 @@ def needed_nodes(nodes, targets, stop=()):
     return need
 
 
+def _pool(orc, n, x):
+    oshape = orc.pool_out_shape(x.shape, n["kernel"], n["strides"], n["pads_begin"], n["pads_end"], n["ceil_mode"])
+    if n["op"] == "MaxPool":
+        return orc.max_pool(x, n["kernel"], n["strides"], n["pads_begin"], n["pads_end"], out_shape=oshape)
+    # f32 result: TypeRelaxed<AvgPool> over widened levels; u8 / i8 result (precision preserved): the reference's
+    # integer instantiation, whose accumulator has the element type (avg_pool.hpp:114-265)
+    src = x.astype(np.float32) if n["dtype"] == 10 else x
+    return orc.avg_pool(src, n["kernel"], n["strides"], n["pads_begin"], n["pads_end"], not n["exclude_pad"], out_shape=oshape)
+
+
 def evaluate(orc, nodes, feeds, keep=None, override=None, targets=None):
     """feeds: {parameter name: array}.  Returns ({result name: array}, {node id: array} for `keep`).
     override: {node id: array} continues from these values behind the given nodes (a checker passes the
@@ -74,18 +84,14 @@ def evaluate(orc, nodes, feeds, keep=None, override=None, targets=None):
             v = orc.clamp(x[0], n["lo"], n["hi"])
         elif op == "Convert":
             v = x[0].astype(_NP[n["dtype"]])
-        elif op == "MaxPool":
-            oshape = orc.pool_out_shape(x[0].shape, n["kernel"], n["strides"], n["pads_begin"], n["pads_end"],
-                                        n["ceil_mode"])
-            v = orc.max_pool(x[0], n["kernel"], n["strides"], n["pads_begin"], n["pads_end"], out_shape=oshape)
-        elif op == "AvgPool":
-            oshape = orc.pool_out_shape(x[0].shape, n["kernel"], n["strides"], n["pads_begin"], n["pads_end"],
-                                        n["ceil_mode"])
-            # f32 result: TypeRelaxed<AvgPool> over widened levels; u8 / i8 result (precision preserved): the reference's
-            # integer instantiation, whose accumulator has the element type (avg_pool.hpp:114-265)
-            src = x[0].astype(np.float32) if n["dtype"] == 10 else x[0]
-            v = orc.avg_pool(src, n["kernel"], n["strides"], n["pads_begin"], n["pads_end"],
-                             not n["exclude_pad"], out_shape=oshape)
+        elif op in ("MaxPool", "AvgPool") and x[0].ndim == 3:
+            # one spatial dimension: the same windows over [N, C, 1, W] (the reference's pools walk any number of
+            # spatial axes; a unit axis adds no cell to any window)
+            lifted = dict(n, kernel=(1, n["kernel"][0]), strides=(1, n["strides"][0]), pads_begin=(0, n["pads_begin"][0]),
+                          pads_end=(0, n["pads_end"][0]))
+            v = _pool(orc, lifted, x[0][:, :, None, :])[:, :, 0, :]
+        elif op in ("MaxPool", "AvgPool"):
+            v = _pool(orc, n, x[0])
         elif op == "Reshape":
             v = x[0].reshape(n["shape"])
         elif op == "Gather":

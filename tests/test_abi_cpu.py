@@ -295,6 +295,35 @@ def test_concat_shape_inference_and_planner_limits():
     assert [s["type"] for s in plan.steps].count("Concat") == 1 and tuple(plan.outputs[0]["shape"]) == (2, 8, 15, 6)
 
 
+def test_one_spatial_dimension_is_described_and_planned():
+    """[N, C, W] convolutions and pools: one attribute per spatial dimension, shapes inferred like the reference's
+    (infer_forward_conv_output_shape), planned as [N, C, 1, W] with the plan's inputs and outputs in the described rank;
+    a stream whose attribute count does not fit the input's rank is refused; three spatial dimensions are not taken"""
+    from dldt_amd import HipieError, builders
+    from dldt_amd.graph import Graph, Plan
+    net = builders.QuantizedNet()
+    g = net.g
+    rng = np.random.default_rng(3)
+    a0 = net.input("data", (2, 8, 40), 1.0)
+    w = rng.standard_normal((16, 8, 5), dtype=np.float32) * np.float32(0.1)
+    a1 = net.conv(a0, w, np.zeros(16, np.float32), 2.0, strides=(2,), pads=(1,), dilations=(2,))
+    assert g.nodes[a1["node"]]["op"] == "FakeQuantize"
+    a2 = net.max_pool(a1, (3,), (2,), (1,))
+    g.result(net.dequantize(a2), "out")
+    plan = g.compile(-1)
+    # (40 + 2 - (2 * 4 + 1)) / 2 + 1 = 17 columns, then (17 + 2 - 3) / 2 + 1 = 9
+    assert tuple(plan.outputs[0]["shape"]) == (2, 16, 9) and tuple(plan.inputs[0]["shape"]) == (2, 8, 40)
+    assert [s["type"] for s in plan.steps] == ["FakeQuantize", "Convolution", "MaxPool", "Result"]
+    assert plan.step_rt_info(1, "runtimePrecision") == "U8" and all(g.query())
+    blob = plan.export()
+    back = Plan.load(blob, -1)
+    assert tuple(back.outputs[0]["shape"]) == (2, 16, 9)
+    g5 = Graph()
+    with pytest.raises(HipieError) as e:            # [N, C, D, H, W]: refused where the value is described
+        g5.parameter("x", (1, 4, 6, 6, 6))
+    assert e.value.status == -2
+
+
 def test_matmul_zero_point_correction_must_be_integers():
     """the Subtract behind a MatMul with u8 activations goes into the integer accumulators: a constant that is not
     integer-valued (it is zero point x column sums of i8 weights) is refused.  A MatMul between two u8 activations is

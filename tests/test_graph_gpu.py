@@ -563,6 +563,48 @@ def test_elementwise_broadcast_between_tensors(orc):
     assert all(g.query())
 
 
+def test_convolutions_over_one_spatial_dimension(orc):
+    """[N, C, W] values: quantized Convolution (stride, dilation, padding), depthwise GroupConvolution, MaxPool and
+    AvgPool with filters and windows over the one axis, and an f32 convolution of the graph input - planned as the
+    same layers over [N, C, 1, W], bit-exact against the oracle's own one-dimensional loops; the plan's inputs and
+    outputs keep their rank, and an exported plan brings the description back as it was"""
+    from dldt_amd import builders
+    from dldt_amd.graph import Plan
+    rng = np.random.default_rng(71)
+    x = rng.uniform(0, 1, (3, 16, 50)).astype(np.float32)
+    net = builders.QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    rnd = lambda shape, s: (rng.standard_normal(shape, dtype=np.float32) * np.float32(s)).astype(np.float32)
+    a1 = net.conv(a0, rnd((32, 16, 5), 0.1), rnd(32, 0.2), 2.0, strides=(2,), pads=(2,), dilations=(1,))
+    a2 = net.conv(a1, rnd((32, 1, 3), 0.3), rnd(32, 0.2), 2.0, strides=(1,), pads=(2,), dilations=(2,), grouped=True)
+    a3 = net.max_pool(a2, (3,), (2,), (1,))
+    y = net.conv_f32(a3, rnd((24, 32, 3), 0.06), rnd(24, 0.1), strides=(1,), pads=(1,), relu=True)
+    g.result(y, "out")
+    g.result(g.avg_pool(net.dequantize(a3), (13,), (1,), (0,), (0,)), "mean")
+    p = g.nodes[g.nodes[a0["node"]]["inputs"][0]]
+    assert p["op"] == "Parameter"
+    f32 = g.relu(g.convolution(g.nodes[a0["node"]]["inputs"][0], g.constant(rnd((8, 16, 4), 0.2)), strides=(3,), dilations=(2,),
+                               pads_begin=(1,), pads_end=(2,)))
+    g.result(f32, "f32")
+    keep = [a1["node"], a2["node"], a3["node"]]
+    want, kept = evaluate(orc, g.nodes, {"data": x}, keep=keep)
+    assert want["out"].shape == (3, 24, 13) and want["mean"].shape == (3, 32, 1) and want["f32"].ndim == 3
+    plan = g.compile()
+    assert [tuple(i["shape"]) for i in plan.inputs] == [x.shape]
+    assert {o["name"]: tuple(o["shape"]) for o in plan.outputs} == {k: v.shape for k, v in want.items()}
+    again = Plan.load(plan.export())
+    for pl in (plan, again):
+        req = pl.create_request()
+        got = dict(zip([o["name"] for o in pl.outputs], req.infer(x)))
+        for node in keep:
+            assert len(np.unique(kept[node])) > 40
+            np.testing.assert_array_equal(req.tensor(node)[:, :, 0, :], kept[node])
+        for name in want:
+            np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
+    assert all(g.query())
+
+
 @pytest.mark.parametrize("stride", [1, 2])
 def test_per_channel_activation_zero_points(orc, stride):
     """one integer zero point per channel in front of a padded depthwise convolution: the halo holds every channel's
