@@ -182,6 +182,19 @@ __global__ __launch_bounds__(kThreads) void gelu_erf(const float* __restrict__ x
     }
 }
 
+// y = x + m over a dense value of up to four dimensions d[0..3]; m has stride ms[k] along dimension k (0 where it
+// has one element and is repeated).  One element per thread and step, the last dimension fastest.
+__global__ __launch_bounds__(kThreads) void add_broadcast(const float* __restrict__ x, const float* __restrict__ m,
+                                                          float* __restrict__ y, int64_t n, int32_t d1, int32_t d2, int32_t d3,
+                                                          int64_t ms0, int64_t ms1, int64_t ms2, int64_t ms3) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) {
+        const int64_t r2 = i / d3, r1 = r2 / d2, i0 = r1 / d1;
+        const int64_t i3 = i - r2 * d3, i2 = r2 - r1 * d2, i1 = r1 - i0 * d1;
+        y[i] = x[i] + m[i0 * ms0 + i1 * ms1 + i2 * ms2 + i3 * ms3];
+    }
+}
+
 // plain per-tensor requantisation of a dense f32 array (behind the long-row fallbacks)
 __global__ __launch_bounds__(kThreads) void requant_flat(const float* __restrict__ x, int8_t* __restrict__ q, int64_t n,
                                                          Requant fq) {
@@ -357,6 +370,33 @@ int hipie_mvn_f32(const float* x, float* y, int64_t rows, int64_t axis, int norm
 
 int hipie_gelu_f32(const float* x, float* y, int64_t n, void* stream) {
     return guarded([&] { run_gelu(x, y, nullptr, n, nullptr, stream, "hipie_gelu_f32"); });
+}
+
+int hipie_add_broadcast_f32(const float* x, const int64_t* dims, const float* addend, const int64_t* addend_dims, int rank,
+                            float* y, void* stream) {
+    return guarded([&] {
+        HIPIE_REQUIRE(x && dims && addend && addend_dims && y && rank >= 1 && rank <= 4, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_add_broadcast_f32: bad argument");
+        int64_t d[4] = {1, 1, 1, 1}, md[4] = {1, 1, 1, 1}, ms[4] = {0, 0, 0, 0};
+        for (int k = 0; k < rank; ++k) {
+            d[4 - rank + k] = dims[k];
+            md[4 - rank + k] = addend_dims[k];
+        }
+        int64_t n = 1, run = 1;
+        for (int k = 3; k >= 0; --k) {
+            HIPIE_REQUIRE(d[k] >= 0 && d[k] < (int64_t{1} << 31) && (md[k] == d[k] || md[k] == 1), HIPIE_PARAMETER_MISMATCH,
+                          "hipie_add_broadcast_f32: dimension %lld of the addend against %lld", (long long)md[k], (long long)d[k]);
+            ms[k] = md[k] == 1 ? 0 : run;
+            run *= md[k];
+            n *= d[k];
+            HIPIE_REQUIRE(n < (int64_t{1} << 40), HIPIE_PARAMETER_MISMATCH, "hipie_add_broadcast_f32: too many elements");
+        }
+        if (n == 0) return;
+        const int64_t blocks = std::min<int64_t>(ceil_div(n, kThreads), 256 * 32);
+        hipLaunchKernelGGL(add_broadcast, dim3(static_cast<uint32_t>(blocks)), dim3(kThreads), 0, as_stream(stream), x, addend, y, n,
+                           static_cast<int32_t>(d[1]), static_cast<int32_t>(d[2]), static_cast<int32_t>(d[3]), ms[0], ms[1], ms[2], ms[3]);
+        HIPIE_CHECK_HIP(hipGetLastError());
+    });
 }
 
 int hipie_softmax_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis, const hipie_requant* requant,

@@ -865,6 +865,26 @@ struct GlueStep : Step {
     }
 };
 
+// Add of a graph input or a constant to a dense f32 value of the row-major path, numpy broadcasting (an attention
+// mask on the scores where the attention core runs as separate kernels)
+struct MatAddStep : Step {
+    View in;
+    int out = -1;
+    int param = -1;                // the addend: a request input, or ...
+    std::vector<float> konst;      // ... a constant
+    DeviceBuffer d_konst;
+    std::vector<int64_t> dims, addend_dims;
+    void create(int device, const std::vector<TensorInfo>&) override {
+        if (device >= 0 && !konst.empty()) d_konst.upload(device, konst.data(), konst.size() * 4);
+    }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*, hipStream_t s) const override {
+        const float* m = param >= 0 ? static_cast<const float*>(inputs[param]) : d_konst.as<float>();
+        check_status(hipie_add_broadcast_f32(reinterpret_cast<const float*>(in.ptr(arena, tensors, inputs)), dims.data(), m, addend_dims.data(),
+                                             static_cast<int>(dims.size()), reinterpret_cast<float*>(arena + tensors[out].offset), s),
+                     name.c_str());
+    }
+};
+
 // MatMul between two activations (each i8 or u8), batched over one or two leading dimensions
 struct BatchMatMulStep : Step {
     View a, b;                     // b as [.., N, K] with K contiguous
@@ -1174,7 +1194,11 @@ struct Planner {
             else
                 plan_eltwise(id);
             break;
-        case OP_ADD: case OP_RELU: case OP_CLAMP: plan_eltwise(id); break;
+        case OP_ADD:
+            if (mat || (n.in.size() == 2 && N(n.in[1]).op != OP_CONSTANT && value(n.in[1]).kind == VK_MAT)) plan_mat_add(id);
+            else plan_eltwise(id);
+            break;
+        case OP_RELU: case OP_CLAMP: plan_eltwise(id); break;
         case OP_MAX_POOL: case OP_AVG_POOL: plan_pool(id); break;
         case OP_RESHAPE: mat ? plan_mat_reshape(id) : plan_reshape(id); break;
         case OP_TRANSPOSE: plan_mat_transpose(id); break;
@@ -1349,6 +1373,40 @@ struct Planner {
         rq.out_low = f.dtype == HIPIE_U8 ? b[2] - 128.f : b[2];   // u8 levels are stored as level - 128
         rq.levels = f.levels;
         return true;
+    }
+
+    // Add(value of the row-major path, f32 graph input | constant) with numpy broadcasting of the addend
+    void plan_mat_add(int id) {
+        const GNode& n = N(id);
+        const int xi = value(n.in[0]).kind == VK_MAT ? 0 : 1;
+        const Value& x = value(n.in[xi]);
+        const int other = n.in[1 - xi];
+        const GNode& m = N(other);
+        const size_t r = n.shape.size();
+        if (x.view.dtype != HIPIE_F32 || !x.view.dense() || x.view.shape != n.shape || r > 4)
+            unsupported(id, "Add on the row-major path takes a dense f32 value of up to four dimensions");
+        if ((m.op != OP_PARAMETER && m.op != OP_CONSTANT) || m.dtype != HIPIE_F32 || m.shape.size() != r)
+            unsupported(id, "Add on the row-major path takes an f32 graph input or constant of the value's rank as its addend");
+        for (size_t k = 0; k < r; ++k)
+            if (m.shape[k] != n.shape[k] && m.shape[k] != 1) unsupported(id, "addend that does not broadcast to the value");
+        auto st = std::make_unique<MatAddStep>();
+        st->in = x.view;
+        st->dims = n.shape;
+        st->addend_dims = m.shape;
+        if (m.op == OP_PARAMETER) {
+            (void)visit(other);
+            for (size_t i = 0; i < g.params.size(); ++i)
+                if (g.params[i] == other) st->param = static_cast<int>(i);
+        } else {
+            st->konst.assign(m.f32(), m.f32() + m.numel());
+        }
+        st->out = new_matrix(id, HIPIE_F32, n.shape);
+        set_matrix_value(id, st->out, HIPIE_F32);
+        st->name = n.name;
+        st->type = "Add";
+        st->bytes = n.numel() * 8 + m.numel() * 4;
+        st->out_node = id;
+        steps.push_back(std::move(st));
     }
 
     void plan_glue(int id) {

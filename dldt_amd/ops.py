@@ -355,6 +355,18 @@ def gelu(x, requant=None, keep_f32=True):
     return _ret(y, q)
 
 
+def add_broadcast(x, addend, out=None):
+    """x + addend for a contiguous f32 device tensor of up to four dimensions and an addend of the same rank whose
+    dimensions are x's or 1 (hipie_add_broadcast_f32); out may be x itself."""
+    import torch
+    assert x.is_contiguous() and addend.is_contiguous() and x.dtype == addend.dtype == torch.float32 and x.dim() == addend.dim()
+    y = torch.empty_like(x) if out is None else out
+    dims = (ctypes.c_int64 * x.dim())(*x.shape)
+    adims = (ctypes.c_int64 * x.dim())(*addend.shape)
+    check(lib().hipie_add_broadcast_f32(_dptr(x), dims, _dptr(addend), adims, x.dim(), _dptr(y), _stream()))
+    return y
+
+
 class hipie_attention_desc(ctypes.Structure):
     _fields_ = [("seq", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("score_scale", ctypes.c_float),
                 ("context_scale", ctypes.c_float), ("prob_fq", hipie_requant), ("out_dtype", ctypes.c_int32),

@@ -329,6 +329,12 @@ int hipie_softmax_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t 
 int hipie_mvn_q8(const float* x, float* y, int8_t* q, int64_t rows, int64_t axis, int normalize_variance, float eps,
                  int eps_inside_sqrt, const float* gamma, const float* beta, const hipie_requant* requant, void* stream);
 int hipie_gelu_q8(const float* x, float* y, int8_t* q, int64_t n, const hipie_requant* requant, void* stream);
+/* reference::add with numpy broadcasting (ngraph/core/reference/include/ngraph/runtime/reference/add.hpp over
+ * autobroadcast_binop.hpp) on the row-major path: y = x + addend for a dense f32 value of `rank` <= 4 dimensions
+ * `dims` and an addend of the same rank whose dimensions are the value's or 1 (an attention mask [batch, 1, 1, seq]
+ * on scores [batch, heads, seq, seq]).  One IEEE addition per element; x and y may be the same buffer. */
+int hipie_add_broadcast_f32(const float* x, const int64_t* dims, const float* addend, const int64_t* addend_dims, int rank,
+                            float* y, void* stream);
 /* Embedding front end of an encoder — reference::gather (.../reference/gather.hpp:18-66) of rows of a
  * f32 table [vocabulary, hidden] by i32 token ids, followed by up to two reference::add steps in the
  * graph's order: out[t] = (table[ids[t]] + add0) + add1, each addend (device pointer, or NULL) either

@@ -216,6 +216,45 @@ def test_encoder_with_attention_mask(orc, monkeypatch):
     np.testing.assert_array_equal(y.view(np.uint32), want["out"].view(np.uint32))
 
 
+@pytest.mark.parametrize("seq,fuse", [(128, False), (448, True)])
+def test_attention_mask_where_the_core_runs_as_separate_kernels(orc, monkeypatch, seq, fuse):
+    """the same mask where the attention core is not one kernel (switched off, or a sequence longer than the fused
+    kernel takes): MatMul -> Add(mask, numpy broadcasting over heads and queries) -> Softmax -> MatMul as steps of
+    their own; the Add is one f32 addition and compared bit for bit, the rest as in the fused form"""
+    from dldt_amd import builders
+    monkeypatch.setenv("HIPIE_KEEP_F32", "1")
+    monkeypatch.setenv("HIPIE_FUSE_ATTENTION", "1" if fuse else "0")
+    B, S, H = 2, seq, 128
+    g, meta = builders.bert_encoder(layers=1, hidden=H, heads=2, ffn=256, batch=B, seq=S, seed=13, mask=True,
+                                    ranges=dict(q=0.12, k=0.9, v=0.9, ctx=0.6))
+    rng = np.random.default_rng(14)
+    x = rng.normal(0, 1, (B, S, H)).astype(np.float32)
+    mask = np.zeros((B, 1, 1, S), np.float32)
+    mask[0, 0, 0, S - 30:] = -10000.0
+    mask[1, 0, 0, 33:] = -10000.0
+    plan = g.compile()
+    types = [s["type"] for s in plan.steps]
+    assert types.count("Attention") == 0 and types.count("Add") == 1 and len(plan.inputs) == 2
+    req = plan.create_request()
+    (y,) = req.infer(x, mask)
+    L = meta["layers"][0]
+    masked = next(i for i, n in enumerate(g.nodes) if n["op"] == "Add" and meta_mask(g) in n["inputs"])
+    device = {n: req.matrix(n) for n in meta["glue"]}
+    want, kept = evaluate(orc, g.nodes, {"hidden_states": x, "attention_mask": mask}, keep=list(L.values()) + [masked], override=device)
+    np.testing.assert_array_equal(req.matrix(masked).reshape(B, 2, S, S).view(np.uint32), kept[masked].view(np.uint32))
+    p = device[L["p"]].reshape(B, 2, S, S)
+    assert p[0, :, :, S - 30:].max() == 0.0 and p[1, :, :, 33:].max() == 0.0
+    np.testing.assert_allclose(p, kept[("oracle", L["p"])], rtol=3e-6, atol=1e-8)
+    for name in ("ctx", "attn", "down"):
+        np.testing.assert_array_equal(req.matrix(L[name]).reshape(kept[L[name]].shape).view(np.uint32), kept[L[name]].view(np.uint32), err_msg=name)
+    np.testing.assert_array_equal(y.view(np.uint32), want["out"].view(np.uint32))
+    assert all(g.query())
+
+
+def meta_mask(g):
+    return next(i for i, n in enumerate(g.nodes) if n["op"] == "Parameter" and n["name"] == "attention_mask")
+
+
 def test_encoder_full_size_first_and_last_layer(orc, monkeypatch):
     """Benchmark configuration 5 at its stated size (12 layers x 768, 12 heads, FFN 3072, sequence 384, batch 16):
     every integer segment of the first and the last layer (projections, attention, both FFN GEMMs with their

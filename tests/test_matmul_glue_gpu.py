@@ -205,6 +205,27 @@ def test_softmax_mvn_gelu_tolerance(orc):
     np.testing.assert_allclose(gelu(torch.from_numpy(f).cuda()).cpu().numpy(), orc.gelu_erf(f), rtol=1e-6, atol=1e-8)
 
 
+@pytest.mark.parametrize("shape,addend", [((2, 3, 40, 64), (2, 1, 1, 64)), ((2, 3, 40, 64), (1, 3, 40, 1)), ((2, 3, 40, 64), (2, 3, 40, 64)),
+                                          ((5, 33, 7), (1, 33, 1)), ((6, 10), (6, 1)), ((77,), (77,)), ((4, 2, 9, 5), (1, 1, 1, 1))])
+def test_add_with_a_broadcast_addend(orc, shape, addend):
+    """reference::add with numpy broadcasting: bit-exact, also in place; an addend that does not broadcast is refused"""
+    import torch
+    from dldt_amd import HipieError
+    from dldt_amd.ops import add_broadcast
+    rng = np.random.default_rng(len(shape) * 100 + sum(addend))
+    x = (rng.standard_normal(shape) * 5).astype(np.float32)
+    m = (rng.standard_normal(addend) * 5).astype(np.float32)
+    want = orc.add(x, m)
+    xd, md = torch.from_numpy(x).cuda(), torch.from_numpy(m).cuda()
+    np.testing.assert_array_equal(add_broadcast(xd, md).cpu().numpy().view(np.uint32), want.view(np.uint32))
+    add_broadcast(xd, md, out=xd)
+    np.testing.assert_array_equal(xd.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    if len(shape) > 1 and shape[-1] > 2:
+        with pytest.raises(HipieError) as e:
+            add_broadcast(xd, torch.zeros(shape[:-1] + (2,), device="cuda"))
+        assert e.value.status == -4
+
+
 @pytest.mark.parametrize("axis", [4, 64, 100, 252, 384, 390, 768, 1500, 3072, 4100])
 def test_glue_row_lengths(orc, axis):
     """rows held in registers (multiples of 4 up to 4096, partial last chunk) and the three-pass fallback"""
