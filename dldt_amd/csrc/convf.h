@@ -46,6 +46,10 @@ struct FqF32Args {
 void launch_fq_f32(const FqF32Args& a, hipStream_t s);
 // the same walk without the FakeQuantize (ch unused): a graph input as the NHWC f32 tensor the elementwise kernels read
 void launch_copy_f32(const FqF32Args& a, hipStream_t s);
+// reference::softmax (softmax.hpp:20-50) along the channel axis of the same walk (ch, lm1 unused): for every (n, h, w)
+// the maximum over the channels, exp(x - max), their sum, the quotients.  One wavefront per pixel; exp is the
+// device's, so the result agrees with the reference's to rounding, not bit for bit.
+void launch_softmax_channels_f32(const FqF32Args& a, hipStream_t s);
 
 
 // reference::max_pool<float> / avg_pool<float> (max_pool.hpp, avg_pool.hpp:114-265): the window runs over the padded

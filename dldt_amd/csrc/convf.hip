@@ -1,5 +1,6 @@
 // f32 Convolution / GroupConvolution / MatMul against constants, FakeQuantize with an f32 result, MaxPool / AvgPool of f32
-// values: the layers of an INT8 network that the low-precision transformations leave unquantized.  See convf.h.
+// values, Softmax over the channels: the layers of an INT8 network that the low-precision transformations leave
+// unquantized.  See convf.h.
 #include "convf.h"
 
 namespace hipie {
@@ -57,6 +58,33 @@ __global__ __launch_bounds__(256) void fq_f32_kernel(const FqF32Args a) {
     float v = source_value(a.in, n, c, h, w);
     if constexpr (QUANTIZE) v = fq_value<false>(a.ch[a.per_channel ? c : 0], a.lm1, v);
     a.out[n * a.out_sn + h * a.out_sh + w * a.out_sw + c] = v;
+}
+
+// one wavefront per pixel, its lanes striding over the channels: maximum, exp and sum (the exponentials parked in the
+// output), quotients
+__global__ __launch_bounds__(256) void softmax_channels_f32_kernel(const FqF32Args a) {
+    const int64_t pixels = static_cast<int64_t>(a.N) * a.H * a.W;
+    const int64_t pix = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (pix >= pixels) return;
+    const int lane = threadIdx.x & 63;
+    const int w = static_cast<int>(pix % a.W);
+    const int64_t p = pix / a.W;
+    const int h = static_cast<int>(p % a.H);
+    const int n = static_cast<int>(p / a.H);
+    float* out = a.out + n * a.out_sn + h * a.out_sh + w * a.out_sw;
+    float m = -INFINITY;
+    for (int c = lane; c < a.C; c += 64) m = fmaxf(m, source_value(a.in, n, c, h, w));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    float sum = 0.f;
+    for (int c = lane; c < a.C; c += 64) {
+        const float e = expf(source_value(a.in, n, c, h, w) - m);
+        out[c] = e;
+        sum += e;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    for (int c = lane; c < a.C; c += 64) out[c] = out[c] / sum;     // each lane reads back what it wrote itself
 }
 
 __global__ __launch_bounds__(256) void pool_f32_kernel(const PoolF32Args a) {
@@ -136,6 +164,16 @@ void launch_pool_f32(const PoolF32Args& a, hipStream_t s) {
     const int64_t blocks = ceil_div(total, 256);
     HIPIE_REQUIRE(blocks < (int64_t{1} << 31), HIPIE_PARAMETER_MISMATCH, "f32 pooling: %lld outputs", (long long)total);
     hipLaunchKernelGGL(pool_f32_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s, a);
+    HIPIE_CHECK_HIP(hipGetLastError());
+}
+
+void launch_softmax_channels_f32(const FqF32Args& a, hipStream_t s) {
+    check_source(a.in, "f32 Softmax");
+    HIPIE_REQUIRE(a.out && a.N > 0 && a.C > 0 && a.H > 0 && a.W > 0, HIPIE_PARAMETER_MISMATCH, "f32 Softmax: shape");
+    HIPIE_REQUIRE(static_cast<const void*>(a.out) != a.in.p, HIPIE_PARAMETER_MISMATCH, "f32 Softmax: in place");
+    const int64_t blocks = ceil_div(static_cast<int64_t>(a.N) * a.H * a.W, 4);
+    HIPIE_REQUIRE(blocks < (int64_t{1} << 31), HIPIE_PARAMETER_MISMATCH, "f32 Softmax: %lld pixels", (long long)(blocks * 4));
+    hipLaunchKernelGGL(softmax_channels_f32_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s, a);
     HIPIE_CHECK_HIP(hipGetLastError());
 }
 

@@ -810,6 +810,22 @@ struct FqF32Step : Step {
     }
 };
 
+// Softmax over the channel axis of an [N, C] or [N, C, H, W] value (the classifier's, a detection head's)
+struct SoftmaxF32Step : Step {
+    F32Input src;
+    int out = -1;
+    void create(int device, const std::vector<TensorInfo>&) override { src.upload(device); }
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*, hipStream_t s) const override {
+        FqF32Args a;
+        a.in = src.source(arena, tensors, inputs);
+        const hipie_tensor t = tensors[out].desc(arena);
+        a.out = static_cast<float*>(t.data);
+        a.out_sn = t.stride_n; a.out_sh = t.stride_h; a.out_sw = t.stride_w;
+        a.N = src.n; a.C = src.c; a.H = src.h; a.W = src.w;
+        launch_softmax_channels_f32(a, s);
+    }
+};
+
 // ---- steps over row-major views (transformer encoders) ------------------------------------------
 
 // FakeQuantize of a dense f32 value with per-tensor bounds -> i8 levels
@@ -1202,7 +1218,12 @@ struct Planner {
         case OP_MAX_POOL: case OP_AVG_POOL: plan_pool(id); break;
         case OP_RESHAPE: mat ? plan_mat_reshape(id) : plan_reshape(id); break;
         case OP_TRANSPOSE: plan_mat_transpose(id); break;
-        case OP_SOFTMAX: case OP_MVN: case OP_GELU: plan_glue(id); break;
+        case OP_SOFTMAX:
+            // over the channels of an [N, C] / [N, C, H, W] value: the f32 step; else the row-major path's kernel
+            if (!mat && (n.shape.size() == 2 || n.shape.size() == 4) && n.axes[0] == 1) plan_softmax_f32(id);
+            else plan_glue(id);
+            break;
+        case OP_MVN: case OP_GELU: plan_glue(id); break;
         case OP_GATHER: plan_gather(id); break;
         case OP_CONCAT: plan_concat(id); break;
         case OP_RESULT: mat ? plan_mat_result(id) : plan_result(id); values[id].kind = VK_FUSED; break;
@@ -2197,6 +2218,22 @@ struct Planner {
         st->name = n.name;
         st->type = "FakeQuantize";
         st->bytes = st->src.bytes(tensors) + n.numel() * 4;
+        st->out_node = id;
+        values[id].kind = VK_TENSOR;
+        values[id].tensor = st->out;
+        steps.push_back(std::move(st));
+    }
+
+    void plan_softmax_f32(int id) {
+        const GNode& n = N(id);
+        auto st = std::make_unique<SoftmaxF32Step>();
+        if (!f32_input(n.in[0], st->src))
+            unsupported(id, "Softmax over the channels reads an f32 graph input, an f32 tensor or a dequantized byte tensor of rank 2 or 4");
+        st->out = new_tensor(id, HIPIE_F32, st->src.n, st->src.h, st->src.w, st->src.c);
+        st->name = n.name;
+        st->type = "Softmax";
+        st->f32_kernel = true;
+        st->bytes = st->src.bytes(tensors) + n.numel() * 4 * 3;
         st->out_node = id;
         values[id].kind = VK_TENSOR;
         values[id].tensor = st->out;

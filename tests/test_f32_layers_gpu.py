@@ -211,3 +211,63 @@ def test_f32_branches_pool_and_concat(orc):
     np.testing.assert_array_equal(req.tensor(q["node"]), kept[q["node"]])
     np.testing.assert_array_equal(_bits(got), _bits(want["out"]))
     assert all(g.query())
+
+
+@pytest.mark.parametrize("classes", [1000, 1001, 10])
+def test_classifier_softmax(orc, classes):
+    """... -> global average pool -> FC -> Softmax over the classes ([N, C], axis 1 or -1): the tail public
+    classification models end with.  The logits in front of it bit for bit; the probabilities to rounding (exp is the
+    device's), every row summing to one"""
+    from dldt_amd import builders
+    rng = np.random.default_rng(classes)
+    x = rng.uniform(0, 1, (5, 16, 12, 12)).astype(np.float32)
+    net = builders.QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    a1 = net.conv(a0, (rng.standard_normal((64, 16, 3, 3)) * 0.08).astype(np.float32), np.zeros(64, np.float32), 2.0, pads=(1, 1))
+    pooled = g.avg_pool(net.dequantize(a1), (12, 12), (1, 1), (0, 0), (0, 0))
+    q = net.requantize(pooled, 1.0)
+    flat = dict(node=g.reshape(q["node"], (5, 64)), scale=q["scale"])
+    logits = net.conv_f32(flat, (rng.standard_normal((classes, 64)) * 0.5).astype(np.float32), (rng.standard_normal(classes)).astype(np.float32),
+                          matmul=True)
+    g.result(logits, "logits")
+    prob = g.softmax(logits, axis=-1 if classes == 10 else 1)
+    g.result(prob, "prob")
+    want, _ = evaluate(orc, g.nodes, {"data": x})
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps].count("Softmax") == 1
+    idx = [s["type"] for s in plan.steps].index("Softmax")
+    assert plan.step_rt_info(idx, "runtimePrecision") == "FP32"
+    req = plan.create_request()
+    got = dict(zip([o["name"] for o in plan.outputs], req.infer(x)))
+    np.testing.assert_array_equal(_bits(got["logits"]), _bits(want["logits"]))
+    assert got["prob"].shape == (5, classes) and np.ptp(want["logits"]) > 4
+    np.testing.assert_allclose(got["prob"], want["prob"], rtol=3e-6, atol=1e-9)
+    np.testing.assert_allclose(got["prob"].sum(1), 1.0, rtol=1e-6)
+    assert all(g.query())
+
+
+def test_softmax_over_the_channels_of_a_feature_map(orc):
+    """a segmentation or detection head: Softmax along axis 1 of [N, C, H, W] (21 classes per pixel), on an f32
+    convolution's result and on the dequantized levels of a quantized one"""
+    from dldt_amd import builders
+    rng = np.random.default_rng(2121)
+    x = rng.uniform(0, 1, (2, 8, 9, 11)).astype(np.float32)
+    net = builders.QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    head = net.conv_f32(a0, (rng.standard_normal((21, 8, 3, 3)) * 0.6).astype(np.float32), rng.standard_normal(21).astype(np.float32), pads=(1, 1))
+    g.result(g.softmax(head, axis=1), "per_pixel")
+    a1 = net.conv(a0, (rng.standard_normal((21, 8, 1, 1)) * 0.5).astype(np.float32), np.zeros(21, np.float32), 3.0, signed=True)
+    g.result(g.softmax(net.dequantize(a1), axis=-3), "of_levels")
+    want, _ = evaluate(orc, g.nodes, {"data": x})
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps].count("Softmax") == 2
+    req = plan.create_request()
+    got = dict(zip([o["name"] for o in plan.outputs], req.infer(x)))
+    for name in ("per_pixel", "of_levels"):
+        assert got[name].shape == (2, 21, 9, 11)
+        np.testing.assert_allclose(got[name], want[name], rtol=3e-6, atol=1e-9, err_msg=name)
+        np.testing.assert_allclose(got[name].sum(1), 1.0, rtol=1e-6)
+    assert want["per_pixel"].max() > 0.5
+    assert all(g.query())
