@@ -20,7 +20,8 @@ struct F32Source {
 };
 
 // reference::convolution<float> / reference::group_convolution<float> (convolution.hpp:63-146, group_convolution.hpp:78-144):
-// sum = 0; for every input channel of the group, filter row, filter column that is not padding: sum += x * w.
+// sum = 0; for every input channel of the group, filter plane, filter row, filter column that is not padding: sum += x * w
+// (convolve_3D_channels; one and two spatial dimensions are the same loops with unit extents in front).
 // MatMul against a constant (matmul.hpp:24-57, sum over k ascending from 0) is the 1 x 1 case.
 struct ConvF32Args {
     F32Source in;
@@ -30,6 +31,9 @@ struct ConvF32Args {
     int32_t N = 0, C = 0, H = 0, W = 0, OC = 0, OH = 0, OW = 0;
     int32_t KH = 1, KW = 1, stride_h = 1, stride_w = 1, dil_h = 1, dil_w = 1, pad_top = 0, pad_left = 0;
     int32_t groups = 1;
+    // three spatial dimensions: the values are [N, C, D * H, W] / [N, OC, OD * OH, OW] (depth and rows merged into the
+    // row axis), filters [C / G][KD][KH][KW][OC]; D = 1 otherwise
+    int32_t D = 1, OD = 1, KD = 1, stride_d = 1, dil_d = 1, pad_front = 0;
 };
 void launch_conv_f32(const ConvF32Args& a, hipStream_t s);
 
@@ -42,14 +46,16 @@ struct FqF32Args {
     float* out = nullptr;             // NHWC
     int64_t out_sn = 0, out_sh = 0, out_sw = 0;
     int32_t N = 0, C = 0, H = 0, W = 0;
+    int32_t axis = 1;                 // Softmax only: 0 .. 3 of [N, C, H, W]
 };
 void launch_fq_f32(const FqF32Args& a, hipStream_t s);
 // the same walk without the FakeQuantize (ch unused): a graph input as the NHWC f32 tensor the elementwise kernels read
 void launch_copy_f32(const FqF32Args& a, hipStream_t s);
-// reference::softmax (softmax.hpp:20-50) along the channel axis of the same walk (ch, lm1 unused): for every (n, h, w)
-// the maximum over the channels, exp(x - max), their sum, the quotients.  One wavefront per pixel; exp is the
-// device's, so the result agrees with the reference's to rounding, not bit for bit.
-void launch_softmax_channels_f32(const FqF32Args& a, hipStream_t s);
+// reference::softmax (softmax.hpp:20-50) along `axis` of the same walk (ch, lm1 unused): for every position of the other
+// three axes the maximum along the axis, exp(x - max), their sum, the quotients.  One wavefront per such row (over the
+// channels, the usual case, its lanes read consecutive elements); exp is the device's, so the result agrees with the
+// reference's to rounding, not bit for bit.
+void launch_softmax_f32(const FqF32Args& a, hipStream_t s);
 
 
 // reference::max_pool<float> / avg_pool<float> (max_pool.hpp, avg_pool.hpp:114-265): the window runs over the padded

@@ -86,7 +86,7 @@ void hipie_graph_destroy(hipie_graph* g) { delete g; }
 int hipie_graph_parameter(hipie_graph* g, const char* name, int dtype, const int64_t* dims, int rank, int* id) {
     return guarded([&] {
         HIPIE_REQUIRE(g && dims && id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_parameter: null argument");
-        HIPIE_REQUIRE(rank >= 2 && rank <= 4, HIPIE_NOT_IMPLEMENTED, "hipie_graph_parameter: rank %d", rank);
+        HIPIE_REQUIRE(rank >= 2 && rank <= 5, HIPIE_NOT_IMPLEMENTED, "hipie_graph_parameter: rank %d", rank);
         HIPIE_REQUIRE(dtype == HIPIE_F32 || dtype == HIPIE_U8 || dtype == HIPIE_I32, HIPIE_NOT_IMPLEMENTED,
                       "hipie_graph_parameter: element type %d", dtype);
         for (int i = 0; i < rank; ++i)
@@ -154,8 +154,8 @@ static int add_conv(hipie_graph* g, int x, int w, const int64_t* strides, const 
                       "%s: null argument", what);
         GNode& X = node(g, x, what);
         GNode& W = node(g, w, what);
-        // [N, C, H, W] or [N, C, W]: one attribute per spatial dimension (three spatial dimensions are not taken)
-        HIPIE_REQUIRE(X.shape.size() == 4 || X.shape.size() == 3, HIPIE_NOT_IMPLEMENTED, "%s: one or two spatial dimensions", what);
+        // [N, C, W], [N, C, H, W] or [N, C, D, H, W]: one attribute per spatial dimension
+        HIPIE_REQUIRE(X.shape.size() >= 3 && X.shape.size() <= 5, HIPIE_NOT_IMPLEMENTED, "%s: one to three spatial dimensions", what);
         const int sp = static_cast<int>(X.shape.size()) - 2;
         HIPIE_REQUIRE(W.shape.size() == X.shape.size() + (grouped ? 1u : 0u), HIPIE_PARAMETER_MISMATCH, "%s: filter rank", what);
         const int o = grouped ? 1 : 0;
@@ -609,8 +609,8 @@ hipie_graph* deserialize_graph(const uint8_t* bytes, size_t size) {
         const std::string name = r.str();
         const std::vector<int> in = r.ints(64);
         const int dtype = r.pod<int32_t>();
-        const std::vector<int64_t> shape = r.i64s(8), strides = r.i64s(2), dilations = r.i64s(2), pads_begin = r.i64s(2),
-                                   pads_end = r.i64s(2), kernel = r.i64s(2), axes = r.i64s(8);
+        const std::vector<int64_t> shape = r.i64s(8), strides = r.i64s(3), dilations = r.i64s(3), pads_begin = r.i64s(3),
+                                   pads_end = r.i64s(3), kernel = r.i64s(3), axes = r.i64s(8);
         const int64_t levels = r.pod<int64_t>();
         const uint8_t flags = r.pod<uint8_t>();
         const float lo = r.pod<float>(), hi = r.pod<float>(), eps = r.pod<float>();

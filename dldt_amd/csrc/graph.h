@@ -26,6 +26,8 @@ struct GNode {
     std::vector<int64_t> shape;       // NCHW / [N, C] as in the reference
     std::vector<int64_t> strides, dilations, pads_begin, pads_end, kernel;
     int64_t levels = 0;
+    int64_t depth = 0;                // planner only: depth D of the input of a convolution over three spatial dimensions
+                                      // whose values are held as [N, C, D * H, W] (never part of a description)
     bool ta = false, tb = false, exclude_pad = false, ceil_mode = false;
     float lo = 0, hi = 0;
     std::vector<int64_t> axes;        // Softmax / Gather / Concat axis, MVN axes, Transpose order

@@ -810,10 +810,11 @@ struct FqF32Step : Step {
     }
 };
 
-// Softmax over the channel axis of an [N, C] or [N, C, H, W] value (the classifier's, a detection head's)
+// Softmax along one axis of an [N, C] or [N, C, H, W] value (over the channels: the classifier's, a detection head's)
 struct SoftmaxF32Step : Step {
     F32Input src;
     int out = -1;
+    int axis = 1;
     void create(int device, const std::vector<TensorInfo>&) override { src.upload(device); }
     void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const*, hipStream_t s) const override {
         FqF32Args a;
@@ -822,7 +823,8 @@ struct SoftmaxF32Step : Step {
         a.out = static_cast<float*>(t.data);
         a.out_sn = t.stride_n; a.out_sh = t.stride_h; a.out_sw = t.stride_w;
         a.N = src.n; a.C = src.c; a.H = src.h; a.W = src.w;
-        launch_softmax_channels_f32(a, s);
+        a.axis = axis;
+        launch_softmax_f32(a, s);
     }
 };
 
@@ -1219,8 +1221,8 @@ struct Planner {
         case OP_RESHAPE: mat ? plan_mat_reshape(id) : plan_reshape(id); break;
         case OP_TRANSPOSE: plan_mat_transpose(id); break;
         case OP_SOFTMAX:
-            // over the channels of an [N, C] / [N, C, H, W] value: the f32 step; else the row-major path's kernel
-            if (!mat && (n.shape.size() == 2 || n.shape.size() == 4) && n.axes[0] == 1) plan_softmax_f32(id);
+            // an [N, C] / [N, C, H, W] value: the f32 step; else the row-major path's kernel
+            if (!mat && (n.shape.size() == 2 || n.shape.size() == 4)) plan_softmax_f32(id);
             else plan_glue(id);
             break;
         case OP_MVN: case OP_GELU: plan_glue(id); break;
@@ -2147,7 +2149,7 @@ struct Planner {
             unsupported(id, "an f32 layer reads an f32 graph input, an f32 tensor or a dequantized byte tensor of rank 2 or 4");
         ConvF32Args& a = st->geo;
         const float* w = W.f32();
-        int64_t G = 1, ocg = 0, icg = 0, KH = 1, KW = 1;
+        int64_t G = 1, ocg = 0, icg = 0, KD = 1, KH = 1, KW = 1;
         if (is_mm) {
             if (n.ta || W.shape.size() != 2 || N(n.in[0]).shape.size() != 2)
                 unsupported(id, "MatMul is planned for [N,K] x constant [K,OC] / [OC,K]^T");
@@ -2157,32 +2159,43 @@ struct Planner {
             for (int64_t k = 0; k < icg; ++k)
                 for (int64_t o = 0; o < ocg; ++o) st->weights[static_cast<size_t>(k * ocg + o)] = n.tb ? w[o * icg + k] : w[k * ocg + o];
         } else {
-            if (N(n.in[0]).shape.size() != 4 || W.shape.size() != (grouped ? 5u : 4u)) unsupported(id, "f32 convolutions are planned over two spatial dimensions");
-            const size_t b = grouped ? 1 : 0;
+            // two spatial dimensions, or three with the values held as [N, C, D * H, W] (GNode::depth)
+            const size_t sp = n.strides.size(), b = grouped ? 1 : 0;
+            if (N(n.in[0]).shape.size() != 4 || (sp != 2 && sp != 3) || (sp == 3) != (n.depth > 0) || W.shape.size() != sp + 2 + b)
+                unsupported(id, "f32 convolutions are planned over one to three spatial dimensions");
             G = grouped ? W.shape[0] : 1;
-            ocg = W.shape[b]; icg = W.shape[b + 1]; KH = W.shape[b + 2]; KW = W.shape[b + 3];
-            const int64_t OCa = G * ocg;
-            st->weights.resize(static_cast<size_t>(OCa * icg * KH * KW));
+            ocg = W.shape[b]; icg = W.shape[b + 1];
+            KD = sp == 3 ? W.shape[b + 2] : 1; KH = W.shape[b + sp]; KW = W.shape[b + sp + 1];
+            const int64_t OCa = G * ocg, taps = KD * KH * KW;
+            st->weights.resize(static_cast<size_t>(OCa * icg * taps));
             for (int64_t oc = 0; oc < OCa; ++oc)
                 for (int64_t c = 0; c < icg; ++c)
-                    for (int64_t t = 0; t < KH * KW; ++t)
-                        st->weights[static_cast<size_t>((c * KH * KW + t) * OCa + oc)] = w[(oc * icg + c) * KH * KW + t];
-            a.stride_h = static_cast<int>(n.strides[0]); a.stride_w = static_cast<int>(n.strides[1]);
-            a.dil_h = static_cast<int>(n.dilations[0]); a.dil_w = static_cast<int>(n.dilations[1]);
-            a.pad_top = static_cast<int>(n.pads_begin[0]); a.pad_left = static_cast<int>(n.pads_begin[1]);
+                    for (int64_t t = 0; t < taps; ++t)
+                        st->weights[static_cast<size_t>((c * taps + t) * OCa + oc)] = w[(oc * icg + c) * taps + t];
+            const size_t o = sp - 2;
+            a.stride_h = static_cast<int>(n.strides[o]); a.stride_w = static_cast<int>(n.strides[o + 1]);
+            a.dil_h = static_cast<int>(n.dilations[o]); a.dil_w = static_cast<int>(n.dilations[o + 1]);
+            a.pad_top = static_cast<int>(n.pads_begin[o]); a.pad_left = static_cast<int>(n.pads_begin[o + 1]);
+            if (sp == 3) {
+                a.D = static_cast<int>(n.depth);
+                a.KD = static_cast<int>(KD);
+                a.stride_d = static_cast<int>(n.strides[0]); a.dil_d = static_cast<int>(n.dilations[0]); a.pad_front = static_cast<int>(n.pads_begin[0]);
+                a.OD = static_cast<int>((n.depth + n.pads_begin[0] + n.pads_end[0] - (n.dilations[0] * (KD - 1) + 1)) / n.strides[0] + 1);
+            }
         }
         const int64_t OC = G * ocg, IC = G * icg;
         HIPIE_REQUIRE(st->src.c == IC, HIPIE_PARAMETER_MISMATCH, "node %d: input has %d channels, weights %lld", id, st->src.c, (long long)IC);
         int nn, c, h, ww;
         nhwc_dims(n.shape, nn, c, h, ww);
         HIPIE_REQUIRE(c == OC && nn == st->src.n, HIPIE_PARAMETER_MISMATCH, "node %d: output shape against the weights", id);
-        a.N = nn; a.C = static_cast<int>(IC); a.H = st->src.h; a.W = st->src.w; a.OC = c; a.OH = h; a.OW = ww;
+        HIPIE_REQUIRE(st->src.h % a.D == 0 && h % a.OD == 0, HIPIE_UNEXPECTED, "node %d: %d rows for a depth of %d, %d for %d", id, st->src.h, a.D, h, a.OD);
+        a.N = nn; a.C = static_cast<int>(IC); a.H = st->src.h / a.D; a.W = st->src.w; a.OC = c; a.OH = h / a.OD; a.OW = ww;
         a.KH = static_cast<int>(KH); a.KW = static_cast<int>(KW); a.groups = static_cast<int>(G);
         st->out = new_tensor(id, HIPIE_F32, nn, h, ww, c);
         st->name = n.name;
         st->type = is_mm ? "MatMul" : (grouped ? "GroupConvolution" : "Convolution");
         st->f32_kernel = true;
-        st->macs = n.numel() * icg * KH * KW;
+        st->macs = n.numel() * icg * KD * KH * KW;
         st->bytes = st->src.bytes(tensors) + static_cast<int64_t>(st->weights.size()) * 4 + n.numel() * 4;
         st->out_node = id;
         values[id].kind = VK_TENSOR;
@@ -2228,7 +2241,8 @@ struct Planner {
         const GNode& n = N(id);
         auto st = std::make_unique<SoftmaxF32Step>();
         if (!f32_input(n.in[0], st->src))
-            unsupported(id, "Softmax over the channels reads an f32 graph input, an f32 tensor or a dequantized byte tensor of rank 2 or 4");
+            unsupported(id, "Softmax reads an f32 graph input, an f32 tensor or a dequantized byte tensor of rank 2 or 4");
+        st->axis = static_cast<int>(n.axes[0]);
         st->out = new_tensor(id, HIPIE_F32, st->src.n, st->src.h, st->src.w, st->src.c);
         st->name = n.name;
         st->type = "Softmax";
@@ -2247,6 +2261,8 @@ struct Planner {
             return;
         }
         const bool is_mm = n.op == OP_MATMUL;
+        if (!is_mm && (n.strides.size() != 2 || n.depth > 0))
+            unsupported(id, "quantized convolutions are planned over one and two spatial dimensions (three: with f32 weights only)");
         const Value x = value(n.in[0]);
         // Subtract(zero point) in front of the convolution: an integer per tensor (what optimizeSubtract
         // leaves, network_helper.cpp:1479-1521) goes into the accumulators' initial value
@@ -2562,7 +2578,7 @@ struct Planner {
     // behind the Concat): the levels are copied side by side
     void plan_concat(int id) {
         const GNode& n = N(id);
-        if (n.shape.size() != 4) unsupported(id, "Concat is planned on 4-D tensors");
+        if (n.shape.size() != 4 || n.axes[0] < 0) unsupported(id, "Concat is planned on 4-D tensors");
         auto st = std::make_unique<ConcatStep>();
         st->axis = static_cast<int>(n.axes[0]);
         const int ax = st->axis;
@@ -2777,36 +2793,38 @@ struct PlanPrepared {       // the host work an exported plan carries (hipie_pla
     PackTape tape;
 };
 
-// Convolutions and pools over one spatial dimension ([N, C, W]) are planned over two with H = 1 - what
-// reference::convolution does with its own shapes (extend_to_3D, convolution.hpp:148-167: unit dimensions in front of
-// the spatial ones, stride and dilation 1 and no padding along them).  Every rank-3 value connected to such a node
-// through nodes that keep the layout (FakeQuantize, elementwise, Convert, Concat, pools, convolutions, inputs and
-// results) becomes [N, C, 1, W]; the constants they read get the unit axis in the same place.  Returns false when
-// the graph has no such node (`out` is then untouched).
-bool lift_one_spatial_dimension(const hipie_graph& g, hipie_graph& out) {
+// The planner's values have two spatial dimensions.  Convolutions and pools over ONE ([N, C, W]) are planned over two
+// with H = 1 - what reference::convolution does with its own shapes (extend_to_3D, convolution.hpp:148-167: unit
+// dimensions in front of the spatial ones, stride and dilation 1 and no padding along them).  Convolutions over THREE
+// ([N, C, D, H, W]) keep their attributes and filters, and their values are held as [N, C, D * H, W]: the same bytes
+// with depth and rows named by one index (GNode::depth keeps D for the kernel).  Every value of the same rank connected
+// to such a node through nodes that keep the layout (FakeQuantize, elementwise, Convert, Concat, pools, convolutions,
+// inputs and results) changes with it; the constants they read get or lose the unit axis in the same place.
+// Returns false when the graph has no such node (`out` is then untouched).
+bool to_two_spatial_dimensions(const hipie_graph& g, hipie_graph& out) {
     auto spatial_op = [](int op) { return op == OP_CONVOLUTION || op == OP_GROUP_CONVOLUTION || op == OP_MAX_POOL || op == OP_AVG_POOL; };
     auto keeps_layout = [&](int op) {
         return spatial_op(op) || op == OP_FAKE_QUANTIZE || op == OP_ADD || op == OP_SUBTRACT || op == OP_MULTIPLY || op == OP_RELU ||
                op == OP_CLAMP || op == OP_CONVERT || op == OP_CONCAT || op == OP_PARAMETER || op == OP_RESULT;
     };
     const int n_nodes = static_cast<int>(g.nodes.size());
-    std::vector<char> lift(g.nodes.size(), 0);
+    std::vector<char> change(g.nodes.size(), 0);
     std::vector<int> stack;
     for (int i = 0; i < n_nodes; ++i) {
         const GNode& n = g.nodes[static_cast<size_t>(i)];
-        if (spatial_op(n.op) && n.shape.size() == 3) { lift[static_cast<size_t>(i)] = 1; stack.push_back(i); }
+        if (spatial_op(n.op) && (n.shape.size() == 3 || n.shape.size() == 5)) { change[static_cast<size_t>(i)] = 1; stack.push_back(i); }
     }
     if (stack.empty()) return false;
-    auto take = [&](int v) {
-        const GNode& n = g.nodes[static_cast<size_t>(v)];
-        if (lift[static_cast<size_t>(v)] || n.shape.size() != 3 || !keeps_layout(n.op)) return;
-        lift[static_cast<size_t>(v)] = 1;
-        stack.push_back(v);
-    };
     while (!stack.empty()) {
         const int v = stack.back();
         stack.pop_back();
         const GNode& n = g.nodes[static_cast<size_t>(v)];
+        auto take = [&](int u) {
+            const GNode& m = g.nodes[static_cast<size_t>(u)];
+            if (change[static_cast<size_t>(u)] || m.shape.size() != n.shape.size() || !keeps_layout(m.op)) return;
+            change[static_cast<size_t>(u)] = 1;
+            stack.push_back(u);
+        };
         // (a convolution's filter and a FakeQuantize's bounds are constants: handled below, never part of the walk)
         for (int in : n.in)
             if (in >= 0 && g.nodes[static_cast<size_t>(in)].op != OP_CONSTANT) take(in);
@@ -2816,8 +2834,26 @@ bool lift_one_spatial_dimension(const hipie_graph& g, hipie_graph& out) {
     auto unit_axis = [](std::vector<int64_t>& shape, size_t at) { shape.insert(shape.begin() + static_cast<std::ptrdiff_t>(at), 1); };
     auto front = [](std::vector<int64_t>& v, int64_t unit) { v.insert(v.begin(), unit); };
     for (int i = 0; i < n_nodes; ++i) {
-        if (!lift[static_cast<size_t>(i)]) continue;
+        if (!change[static_cast<size_t>(i)]) continue;
         GNode& n = out.nodes[static_cast<size_t>(i)];
+        const bool filter_op = n.op == OP_CONVOLUTION || n.op == OP_GROUP_CONVOLUTION;
+        if (n.shape.size() == 5) {
+            // [N, C, D, H, W] -> [N, C, D * H, W]
+            if (filter_op) n.depth = g.nodes[static_cast<size_t>(n.in[0])].shape[2];
+            n.shape = {n.shape[0], n.shape[1], n.shape[2] * n.shape[3], n.shape[4]};
+            if (n.op == OP_CONCAT && !n.axes.empty()) {
+                // along the depth: whole blocks of rows side by side, the same bytes; along the rows: not these bytes
+                if (n.axes[0] == 3) n.axes[0] = -1;             // refused by the planner (no such axis)
+                else if (n.axes[0] == 4) n.axes[0] = 3;
+            }
+            for (size_t k = 0; k < n.in.size(); ++k) {
+                if (n.in[k] < 0 || (filter_op && k == 1)) continue;
+                GNode& c = out.nodes[static_cast<size_t>(n.in[k])];
+                // [1, C, 1, 1, 1] and the like lose a unit axis; anything that names a depth or a row stays and is refused
+                if (c.op == OP_CONSTANT && c.shape.size() == 5 && c.shape[2] == 1 && c.shape[3] == 1) c.shape.erase(c.shape.begin() + 2);
+            }
+            continue;
+        }
         unit_axis(n.shape, 2);
         if (spatial_op(n.op)) {
             front(n.strides, 1);
@@ -2831,7 +2867,7 @@ bool lift_one_spatial_dimension(const hipie_graph& g, hipie_graph& out) {
             if (n.in[k] < 0) continue;
             GNode& c = out.nodes[static_cast<size_t>(n.in[k])];
             if (c.op != OP_CONSTANT) continue;
-            const bool filter = (n.op == OP_CONVOLUTION || n.op == OP_GROUP_CONVOLUTION) && k == 1;
+            const bool filter = filter_op && k == 1;
             const size_t full = filter ? (n.op == OP_GROUP_CONVOLUTION ? 4u : 3u) : 3u;
             // filters [OC, IC, KW] / [G, OC/G, IC/G, KW] and constants that name the width axis: the unit axis goes in
             // front of the last one; lower ranks align from the right as before, except [C, 1], which names the channels
@@ -2851,7 +2887,7 @@ std::unique_ptr<hipie_plan> compile_plan(const hipie_graph* g, int device, const
     plan->graph = *g;                       // the description as it was given: what an exported plan carries
     const hipie_graph* const described = g;
     hipie_graph lifted;
-    if (lift_one_spatial_dimension(*g, lifted)) g = &lifted;
+    if (to_two_spatial_dimensions(*g, lifted)) g = &lifted;
     if (prepared) {
         plan->verdicts = std::move(prepared->verdicts);
         plan->tape = std::move(prepared->tape);
@@ -3126,7 +3162,7 @@ int hipie_query(const hipie_graph* g, int* supported, int n_nodes, int* n_unsupp
         hipie_graph work = *g;
         {
             hipie_graph lifted;
-            if (lift_one_spatial_dimension(work, lifted)) work = std::move(lifted);
+            if (to_two_spatial_dimensions(work, lifted)) work = std::move(lifted);
         }
         for (int i = 0; i < n_nodes; ++i) supported[i] = 1;
         int bad = 0;

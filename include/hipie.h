@@ -412,10 +412,12 @@ int hipie_graph_constant(hipie_graph* g, int dtype, const int64_t* dims, int ran
 /* op::v0::FakeQuantize (TypeRelaxed when out_dtype is HIPIE_U8 / HIPIE_I8) */
 int hipie_graph_fake_quantize(hipie_graph* g, int x, int in_low, int in_high, int out_low, int out_high,
                               int64_t levels, int out_dtype, int* id);
-/* op::v1::Convolution / GroupConvolution and the pools below: x is [N, C, H, W] or [N, C, W]; every attribute array
- * holds one entry per spatial dimension of x (2 or 1).  A value with one spatial dimension is planned as the same
- * value with H = 1, the way reference::convolution extends its shapes (convolution.hpp:148-167); three spatial
- * dimensions are refused (HIPIE_NOT_IMPLEMENTED). */
+/* op::v1::Convolution / GroupConvolution and the pools below: x is [N, C, H, W] or [N, C, W] (a convolution's also
+ * [N, C, D, H, W]); every attribute array holds one entry per spatial dimension of x.  A value with one spatial
+ * dimension is planned as the same value with H = 1, the way reference::convolution extends its shapes
+ * (convolution.hpp:148-167).  Over three spatial dimensions only convolutions with f32 weights are planned
+ * (reference::convolution<float>'s loops as they stand, convolution.hpp:63-146); quantized ones and pools are
+ * refused (HIPIE_NOT_IMPLEMENTED). */
 int hipie_graph_convolution(hipie_graph* g, int x, int weights, const int64_t* strides,
                             const int64_t* dilations, const int64_t* pads_begin, const int64_t* pads_end,
                             int* id);

@@ -92,12 +92,12 @@ struct Translator {
         } else if (const auto conv = ngraph::as_type_ptr<ngraph::opset1::Convolution>(node)) {
             const auto s = as_i64(conv->get_strides()), dl = as_i64(conv->get_dilations());
             const auto pb = as_i64(conv->get_pads_begin()), pe = as_i64(conv->get_pads_end());
-            if (s.size() != 2 && s.size() != 1) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is a convolution over three spatial dimensions";
+            if (s.size() < 1 || s.size() > 3) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is a convolution over " << s.size() << " spatial dimensions";
             check(hipie_graph_convolution(g, in(n, 0), in(n, 1), s.data(), dl.data(), pb.data(), pe.data(), &id), "hipie_graph_convolution");
         } else if (const auto gconv = ngraph::as_type_ptr<ngraph::opset1::GroupConvolution>(node)) {
             const auto s = as_i64(gconv->get_strides()), dl = as_i64(gconv->get_dilations());
             const auto pb = as_i64(gconv->get_pads_begin()), pe = as_i64(gconv->get_pads_end());
-            if (s.size() != 2 && s.size() != 1) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is a convolution over three spatial dimensions";
+            if (s.size() < 1 || s.size() > 3) IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << " is a convolution over " << s.size() << " spatial dimensions";
             check(hipie_graph_group_convolution(g, in(n, 0), in(n, 1), s.data(), dl.data(), pb.data(), pe.data(), &id),
                   "hipie_graph_group_convolution");
         } else if (const auto mm = ngraph::as_type_ptr<ngraph::opset1::MatMul>(node)) {

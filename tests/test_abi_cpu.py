@@ -298,7 +298,7 @@ def test_concat_shape_inference_and_planner_limits():
 def test_one_spatial_dimension_is_described_and_planned():
     """[N, C, W] convolutions and pools: one attribute per spatial dimension, shapes inferred like the reference's
     (infer_forward_conv_output_shape), planned as [N, C, 1, W] with the plan's inputs and outputs in the described rank;
-    a stream whose attribute count does not fit the input's rank is refused; three spatial dimensions are not taken"""
+    three spatial dimensions: f32 convolutions only"""
     from dldt_amd import HipieError, builders
     from dldt_amd.graph import Graph, Plan
     net = builders.QuantizedNet()
@@ -318,10 +318,26 @@ def test_one_spatial_dimension_is_described_and_planned():
     blob = plan.export()
     back = Plan.load(blob, -1)
     assert tuple(back.outputs[0]["shape"]) == (2, 16, 9)
+    # three spatial dimensions: convolutions with f32 weights are planned (values held as [N, C, D * H, W]), quantized
+    # ones are reported unsupported, pools are refused where they are described
     g5 = Graph()
-    with pytest.raises(HipieError) as e:            # [N, C, D, H, W]: refused where the value is described
-        g5.parameter("x", (1, 4, 6, 6, 6))
+    x5 = g5.parameter("x", (1, 4, 6, 5, 7))
+    y5 = g5.convolution(x5, g5.constant(np.ones((3, 4, 3, 1, 2), np.float32)), (2, 1, 1), (1, 1, 1), (1, 0, 0), (1, 0, 1))
+    g5.result(y5, "y")
+    plan = g5.compile(-1)
+    assert tuple(plan.outputs[0]["shape"]) == (1, 3, 3, 5, 7) and plan.steps[0]["type"] == "Convolution"
+    assert plan.steps[0]["macs"] == 3 * 3 * 5 * 7 * 4 * 3 * 1 * 2
+    with pytest.raises(HipieError) as e:
+        g5.max_pool(x5, (1, 1, 1), (1, 1, 1), (0, 0, 0), (0, 0, 0))
     assert e.value.status == -2
+    from dldt_amd.tensor import I8, U8
+    q5 = Graph()
+    xq = q5.fake_quantize(q5.parameter("x", (1, 4, 6, 5, 7)), np.float32(0), np.float32(2.55), np.float32(0), np.float32(255), 256, U8)
+    q5.result(q5.convolution(q5.convert(xq, 10), q5.constant(np.ones((3, 4, 1, 1, 1), np.int8), I8), (1, 1, 1), (1, 1, 1), (0, 0, 0), (0, 0, 0)), "y")
+    with pytest.raises(HipieError) as e:
+        q5.compile(-1)
+    assert e.value.status == -2 and "three" in str(e.value)
+    assert not all(q5.query())
 
 
 def test_matmul_zero_point_correction_must_be_integers():
