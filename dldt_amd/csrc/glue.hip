@@ -195,6 +195,18 @@ __global__ __launch_bounds__(kThreads) void add_broadcast(const float* __restric
     }
 }
 
+// dst (dense, dimensions d[0..4], the last fastest) = the elements of src at strides st[0..4]
+template <typename T>
+__global__ __launch_bounds__(kThreads) void copy_strided(const T* __restrict__ src, T* __restrict__ dst, int64_t n, int32_t d1, int32_t d2,
+                                                         int32_t d3, int32_t d4, int64_t s0, int64_t s1, int64_t s2, int64_t s3, int64_t s4) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < n; i += stride) {
+        const int64_t r3 = i / d4, r2 = r3 / d3, r1 = r2 / d2, i0 = r1 / d1;
+        const int64_t i4 = i - r3 * d4, i3 = r3 - r2 * d3, i2 = r2 - r1 * d2, i1 = r1 - i0 * d1;
+        dst[i] = src[i0 * s0 + i1 * s1 + i2 * s2 + i3 * s3 + i4 * s4];
+    }
+}
+
 // plain per-tensor requantisation of a dense f32 array (behind the long-row fallbacks)
 __global__ __launch_bounds__(kThreads) void requant_flat(const float* __restrict__ x, int8_t* __restrict__ q, int64_t n,
                                                          Requant fq) {
@@ -395,6 +407,34 @@ int hipie_add_broadcast_f32(const float* x, const int64_t* dims, const float* ad
         const int64_t blocks = std::min<int64_t>(ceil_div(n, kThreads), 256 * 32);
         hipLaunchKernelGGL(add_broadcast, dim3(static_cast<uint32_t>(blocks)), dim3(kThreads), 0, as_stream(stream), x, addend, y, n,
                            static_cast<int32_t>(d[1]), static_cast<int32_t>(d[2]), static_cast<int32_t>(d[3]), ms[0], ms[1], ms[2], ms[3]);
+        HIPIE_CHECK_HIP(hipGetLastError());
+    });
+}
+
+int hipie_copy_strided(const void* src, const int64_t* dims, const int64_t* strides, int rank, int element_bytes, void* dst,
+                       void* stream) {
+    return guarded([&] {
+        HIPIE_REQUIRE(src && dims && strides && dst && rank >= 1 && rank <= 5 && (element_bytes == 1 || element_bytes == 4),
+                      HIPIE_PARAMETER_MISMATCH, "hipie_copy_strided: bad argument");
+        int64_t d[5] = {1, 1, 1, 1, 1}, st[5] = {0, 0, 0, 0, 0}, n = 1;
+        for (int k = 0; k < rank; ++k) {
+            d[5 - rank + k] = dims[k];
+            st[5 - rank + k] = strides[k];
+            HIPIE_REQUIRE(dims[k] >= 0 && dims[k] < (int64_t{1} << 31) && strides[k] >= 0, HIPIE_PARAMETER_MISMATCH,
+                          "hipie_copy_strided: dimension %d", k);
+            n *= dims[k];
+            HIPIE_REQUIRE(n < (int64_t{1} << 40), HIPIE_PARAMETER_MISMATCH, "hipie_copy_strided: too many elements");
+        }
+        if (n == 0) return;
+        const dim3 grid(static_cast<uint32_t>(std::min<int64_t>(ceil_div(n, kThreads), 256 * 32))), block(kThreads);
+        hipStream_t s = as_stream(stream);
+        const int32_t d1 = static_cast<int32_t>(d[1]), d2 = static_cast<int32_t>(d[2]), d3 = static_cast<int32_t>(d[3]), d4 = static_cast<int32_t>(d[4]);
+        if (element_bytes == 4)
+            hipLaunchKernelGGL(copy_strided<uint32_t>, grid, block, 0, s, static_cast<const uint32_t*>(src), static_cast<uint32_t*>(dst), n, d1, d2,
+                               d3, d4, st[0], st[1], st[2], st[3], st[4]);
+        else
+            hipLaunchKernelGGL(copy_strided<uint8_t>, grid, block, 0, s, static_cast<const uint8_t*>(src), static_cast<uint8_t*>(dst), n, d1, d2, d3,
+                               d4, st[0], st[1], st[2], st[3], st[4]);
         HIPIE_CHECK_HIP(hipGetLastError());
     });
 }

@@ -9,8 +9,8 @@ const char* op_name(int op) {
     static const char* names[] = {"Parameter", "Constant", "FakeQuantize", "Convolution",
                                   "GroupConvolution", "MatMul", "Add", "Multiply", "Subtract", "Relu",
                                   "Clamp", "Convert", "MaxPool", "AvgPool", "Reshape", "Result", "Softmax", "MVN",
-                                  "Gelu", "Transpose", "Gather", "Concat"};
-    return op >= 0 && op <= OP_CONCAT ? names[op] : "?";
+                                  "Gelu", "Transpose", "Gather", "Concat", "Slice"};
+    return op >= 0 && op <= OP_SLICE ? names[op] : "?";
 }
 
 namespace {
@@ -491,6 +491,26 @@ int hipie_graph_concat(hipie_graph* g, const int* inputs, int n_inputs, int64_t 
     });
 }
 
+int hipie_graph_slice(hipie_graph* g, int x, int64_t axis, int64_t begin, int64_t end, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_slice: null argument");
+        const GNode& X = node(g, x, "hipie_graph_slice");
+        const int64_t r = static_cast<int64_t>(X.shape.size());
+        HIPIE_REQUIRE(axis >= -r && axis < r, HIPIE_PARAMETER_MISMATCH, "hipie_graph_slice: axis %lld of rank %lld", (long long)axis, (long long)r);
+        const int64_t ax = axis < 0 ? axis + r : axis;
+        HIPIE_REQUIRE(begin >= 0 && begin < end && end <= X.shape[static_cast<size_t>(ax)], HIPIE_PARAMETER_MISMATCH,
+                      "hipie_graph_slice: [%lld, %lld) of %lld elements", (long long)begin, (long long)end, (long long)X.shape[static_cast<size_t>(ax)]);
+        GNode n;
+        n.op = OP_SLICE;
+        n.in = {x};
+        n.axes = {ax, begin, end};
+        n.dtype = X.dtype;
+        n.shape = X.shape;
+        n.shape[static_cast<size_t>(ax)] = end - begin;
+        *id = add_node(g, std::move(n));
+    });
+}
+
 int hipie_graph_result(hipie_graph* g, int x, const char* name) {
     return guarded([&] {
         GNode& X = node(g, x, "hipie_graph_result");
@@ -696,6 +716,11 @@ hipie_graph* deserialize_graph(const uint8_t* bytes, size_t size) {
         case OP_CONCAT:
             HIPIE_REQUIRE(axes.size() == 1 && !in.empty(), HIPIE_NETWORK_NOT_READ, "plan stream: Concat %u without an axis or inputs", i);
             st = hipie_graph_concat(G, in.data(), static_cast<int>(in.size()), axes[0], &id);
+            break;
+        case OP_SLICE:
+            arity(1);
+            HIPIE_REQUIRE(axes.size() == 3, HIPIE_NETWORK_NOT_READ, "plan stream: Slice %u without its bounds", i);
+            st = hipie_graph_slice(G, in[0], axes[0], axes[1], axes[2], &id);
             break;
         case OP_RESULT: arity(1); st = hipie_graph_result(G, in[0], name.c_str()); break;
         default: fail(HIPIE_NETWORK_NOT_READ, "plan stream: node %u has unknown operation %d", i, op);

@@ -14,7 +14,7 @@ namespace hipie {
 enum OpKind {
     OP_PARAMETER = 0, OP_CONSTANT, OP_FAKE_QUANTIZE, OP_CONVOLUTION, OP_GROUP_CONVOLUTION, OP_MATMUL,
     OP_ADD, OP_MULTIPLY, OP_SUBTRACT, OP_RELU, OP_CLAMP, OP_CONVERT, OP_MAX_POOL, OP_AVG_POOL,
-    OP_RESHAPE, OP_RESULT, OP_SOFTMAX, OP_MVN, OP_GELU, OP_TRANSPOSE, OP_GATHER, OP_CONCAT
+    OP_RESHAPE, OP_RESULT, OP_SOFTMAX, OP_MVN, OP_GELU, OP_TRANSPOSE, OP_GATHER, OP_CONCAT, OP_SLICE
 };
 const char* op_name(int op);
 
@@ -30,7 +30,7 @@ struct GNode {
                                       // whose values are held as [N, C, D * H, W] (never part of a description)
     bool ta = false, tb = false, exclude_pad = false, ceil_mode = false;
     float lo = 0, hi = 0;
-    std::vector<int64_t> axes;        // Softmax / Gather / Concat axis, MVN axes, Transpose order
+    std::vector<int64_t> axes;        // Softmax / Gather / Concat axis, MVN axes, Transpose order, Slice {axis, begin, end}
     bool normalize_variance = true, eps_inside_sqrt = true;
     float eps = 0;
     std::vector<uint8_t> data;        // constant payload

@@ -1009,11 +1009,40 @@ struct MatExitStep : Step {
     View in;
     int result_index = 0;
     int64_t nbytes = 0;
+    bool strided = false;          // the view is a box inside a larger value (one output of a Split): gathered, not copied whole
     void create(int, const std::vector<TensorInfo>&) override {}
     void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const* inputs, void* const* outputs,
              hipStream_t s) const override {
-        HIPIE_CHECK_HIP(hipMemcpyAsync(outputs[result_index], in.ptr(arena, tensors, inputs), static_cast<size_t>(nbytes),
-                                       hipMemcpyDeviceToDevice, s));
+        if (strided)
+            check_status(hipie_copy_strided(in.ptr(arena, tensors, inputs), in.shape.data(), in.stride.data(), static_cast<int>(in.rank()),
+                                            static_cast<int>(in.esize()), outputs[result_index], s),
+                         name.c_str());
+        else
+            HIPIE_CHECK_HIP(hipMemcpyAsync(outputs[result_index], in.ptr(arena, tensors, inputs), static_cast<size_t>(nbytes),
+                                           hipMemcpyDeviceToDevice, s));
+    }
+};
+
+// One output of a Split on a value of the [N, C, H, W] path: its box copied into a tensor of its own (the byte copy of
+// ConcatStep, read side and write side exchanged)
+struct SliceStep : Step {
+    int in = -1, out = -1;
+    int axis = 1, begin = 0;       // of [N, C, H, W]
+    void create(int, const std::vector<TensorInfo>&) override {}
+    void run(uint8_t* arena, const std::vector<TensorInfo>& tensors, void* const*, void* const*, hipStream_t s) const override {
+        const hipie_tensor x = tensors[in].desc(arena);
+        const hipie_tensor o = tensors[out].desc(arena);
+        const int es = static_cast<int>(tensors[out].esize());
+        ConcatArgs a{};
+        a.in = static_cast<const int8_t*>(x.data);
+        a.out = static_cast<int8_t*>(o.data);
+        a.N = o.n; a.H = o.h; a.W = o.w; a.C = o.c * es;
+        a.in_sn = x.stride_n * es; a.in_sh = x.stride_h * es; a.in_sw = x.stride_w * es;
+        a.out_sn = o.stride_n * es; a.out_sh = o.stride_h * es; a.out_sw = o.stride_w * es;
+        a.c_off = 0;
+        a.in += begin * (axis == 0 ? a.in_sn : (axis == 1 ? es : (axis == 2 ? a.in_sh : a.in_sw)));
+        launch_concat_channels(a, s);
+        HIPIE_CHECK_HIP(hipGetLastError());
     }
 };
 
@@ -1228,6 +1257,7 @@ struct Planner {
         case OP_MVN: case OP_GELU: plan_glue(id); break;
         case OP_GATHER: plan_gather(id); break;
         case OP_CONCAT: plan_concat(id); break;
+        case OP_SLICE: plan_slice(id); break;
         case OP_RESULT: mat ? plan_mat_result(id) : plan_result(id); values[id].kind = VK_FUSED; break;
         default: unsupported(id, "only planned as part of a fused convolution / pooling chain");
         }
@@ -1542,8 +1572,14 @@ struct Planner {
     void plan_mat_result(int id) {
         const GNode& n = N(id);
         const Value& x = value(n.in[0]);
-        if (!x.view.dense()) unsupported(id, "Result of a transposed view");
         auto st = std::make_unique<MatExitStep>();
+        if (!x.view.dense()) {
+            // a box of a larger value (strides in the order of the dimensions) is gathered; a transposed view is not taken
+            bool ordered = x.view.rank() <= 5;
+            for (size_t k = 0; ordered && k + 1 < x.view.rank(); ++k) ordered = x.view.stride[k] >= x.view.stride[k + 1] * x.view.shape[k + 1];
+            if (!ordered || x.view.stride.back() != 1) unsupported(id, "Result of a transposed view");
+            st->strided = true;
+        }
         st->in = x.view;
         st->nbytes = x.view.numel() * x.view.esize();
         for (size_t i = 0; i < g.results.size(); ++i)
@@ -2081,10 +2117,71 @@ struct Planner {
         values[id] = v;
     }
 
+    // a graph input as a row-major view of the request's own buffer (its memory order is the graph's dimension order)
+    bool param_view(int node, View& v) {
+        const GNode& src = N(node);
+        if (src.op != OP_PARAMETER || (src.dtype != HIPIE_F32 && src.dtype != HIPIE_U8)) return false;
+        for (size_t i = 0; i < g.params.size(); ++i)
+            if (g.params[i] == node) v.param = static_cast<int>(i);
+        v.dtype = src.dtype;
+        v.shape = src.shape;
+        v.stride = View::dense_strides(src.shape);
+        return v.param >= 0;
+    }
+
+    // One output of a Split.  On the row-major path (and on a graph input) it is a view: offset and extent change, no
+    // byte moves.  On the [N, C, H, W] path the box is copied into a tensor of its own.
+    void plan_slice(int id) {
+        const GNode& n = N(id);
+        const Value& x = value(n.in[0]);
+        const size_t ax = static_cast<size_t>(n.axes[0]);
+        const int64_t begin = n.axes[1];
+        View v;
+        if (x.kind == VK_MAT || (x.kind == VK_PARAM && param_view(n.in[0], v))) {
+            if (x.kind == VK_MAT) v = x.view;
+            v.offset += begin * v.stride[ax];
+            v.shape[ax] = n.shape[ax];
+            values[id].kind = VK_MAT;
+            values[id].view = v;
+            return;
+        }
+        if ((x.kind != VK_TENSOR && x.kind != VK_DEQ) || (n.shape.size() != 4 && n.shape.size() != 2))
+            unsupported(id, "Split is planned on graph inputs, values of the row-major path and [N, C, H, W] / [N, C] tensors");
+        auto st = std::make_unique<SliceStep>();
+        st->in = x.tensor;
+        st->axis = static_cast<int>(ax);
+        st->begin = static_cast<int>(begin);
+        int nn, c, h, w;
+        nhwc_dims(n.shape, nn, c, h, w);
+        st->out = new_tensor(id, tensors[x.tensor].dtype, nn, h, w, c);
+        st->name = n.name;
+        st->type = "Split";
+        st->bytes = 2 * n.numel() * tensors[x.tensor].esize();
+        st->out_node = id;
+        values[id] = x;                       // a dequantization in front of the Split stays behind its outputs
+        values[id].tensor = st->out;
+        if (ax == 1) {
+            auto part = [&](std::vector<float>& k) {
+                if (k.size() > 1) k = std::vector<float>(k.begin() + begin, k.begin() + begin + c);
+            };
+            part(values[id].sub);
+            part(values[id].mul);
+        }
+        steps.push_back(std::move(st));
+    }
+
     void plan_reshape(int id) {
         const GNode& n = N(id);
         const Value& x = value(n.in[0]);
         const GNode& src = N(n.in[0]);
+        View pv;
+        if (x.kind == VK_PARAM && param_view(n.in[0], pv)) {      // the same bytes under other dimensions
+            pv.shape = n.shape;
+            pv.stride = View::dense_strides(n.shape);
+            values[id].kind = VK_MAT;
+            values[id].view = pv;
+            return;
+        }
         // [N, C, 1, 1] <-> [N, C]: same bytes in NHWC
         const bool flatten = src.shape.size() == 4 && n.shape.size() == 2 && src.shape[2] == 1 &&
                              src.shape[3] == 1 && n.shape[0] == src.shape[0] && n.shape[1] == src.shape[1];

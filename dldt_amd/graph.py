@@ -155,6 +155,17 @@ class Graph:
         check(lib().hipie_graph_concat(self._h, ids, len(inputs), ctypes.c_int64(axis), ctypes.byref(i)))
         return self._rec(i.value, "Concat", list(inputs), self.nodes[inputs[0]]["dtype"], axis=axis)
 
+    def slice(self, x, axis, begin, end):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_slice(self._h, x, ctypes.c_int64(axis), ctypes.c_int64(begin), ctypes.c_int64(end), ctypes.byref(i)))
+        return self._rec(i.value, "Slice", [x], self.nodes[x]["dtype"], axis=axis, begin=begin, end=end)
+
+    def split(self, x, axis, parts, length):
+        """op::v1::Split of an axis of `length` elements into `parts` equal outputs, one Slice each"""
+        assert length % parts == 0
+        step = length // parts
+        return [self.slice(x, axis, k * step, (k + 1) * step) for k in range(parts)]
+
     def result(self, x, name):
         check(lib().hipie_graph_result(self._h, x, name.encode()))
         self.results.append(len(self.nodes))

@@ -335,6 +335,11 @@ int hipie_gelu_q8(const float* x, float* y, int8_t* q, int64_t n, const hipie_re
  * on scores [batch, heads, seq, seq]).  One IEEE addition per element; x and y may be the same buffer. */
 int hipie_add_broadcast_f32(const float* x, const int64_t* dims, const float* addend, const int64_t* addend_dims, int rank,
                             float* y, void* stream);
+/* reference::slice with unit steps (ngraph/core/reference/include/ngraph/runtime/reference/slice.hpp; what
+ * reference::split takes each of its outputs with): dst, dense, receives the `rank` <= 5 dimensional box `dims` of
+ * src whose element (i0, .., i4) lies at sum(i_k * strides[k]) elements from src; elements of 1 or 4 bytes. */
+int hipie_copy_strided(const void* src, const int64_t* dims, const int64_t* strides, int rank, int element_bytes, void* dst,
+                       void* stream);
 /* Embedding front end of an encoder — reference::gather (.../reference/gather.hpp:18-66) of rows of a
  * f32 table [vocabulary, hidden] by i32 token ids, followed by up to two reference::add steps in the
  * graph's order: out[t] = (table[ids[t]] + add0) + add1, each addend (device pointer, or NULL) either
@@ -449,6 +454,9 @@ int hipie_graph_gather(hipie_graph* g, int data, int indices, int64_t axis, int*
  * i8 levels directly (low_precision_transformations/src/concat.cpp:42-190 gives every branch the same interval and
  * moves the dequantization behind the Concat), which is the form the engine runs: byte tensors along the channel axis. */
 int hipie_graph_concat(hipie_graph* g, const int* inputs, int n_inputs, int64_t axis, int* id);
+/* One output of op::v1::Split / op::v1::VariadicSplit: elements [begin, end) of x along `axis`, every other axis whole
+ * (ngraph/core/reference/src/runtime/reference/split.cpp:14-45 takes each output with reference::slice of that box). */
+int hipie_graph_slice(hipie_graph* g, int x, int64_t axis, int64_t begin, int64_t end, int* id);
 int hipie_graph_result(hipie_graph* g, int x, const char* name);
 int hipie_graph_set_name(hipie_graph* g, int id, const char* friendly_name);
 

@@ -1,5 +1,7 @@
 #include "function_to_graph.hpp"
 
+#include <map>
+
 #include <ngraph/opsets/opset1.hpp>
 #include <ngraph/opsets/opset2.hpp>
 #include <ngraph/opsets/opset6.hpp>
@@ -39,12 +41,19 @@ struct Translator {
     hipie_graph* g;
     TranslatedGraph& out;
     std::unordered_map<const ngraph::Node*, int> id_of;
+    // a node with several outputs (Split, VariadicSplit) is one Slice per output: (node, output index) -> id;
+    // id_of holds its first output's
+    std::map<std::pair<const ngraph::Node*, size_t>, int> output_id;
 
     // An i64 / u64 Constant is skipped when it is met (most are attributes their users read: axes, orders, target
     // shapes).  One that a node takes as DATA - Gather indices, an integer table - is described here, on first use, as
     // the i32 constant the engine's integer inputs are (values that do not fit are refused).
     int in(const ngraph::Node& n, size_t i) {
         const ngraph::Node* producer = n.get_input_node_ptr(i);
+        if (producer->get_output_size() > 1) {
+            const auto part = output_id.find({producer, n.input_value(i).get_index()});
+            if (part != output_id.end()) return part->second;
+        }
         const auto it = id_of.find(producer);
         if (it != id_of.end()) return it->second;
         const auto c = ngraph::as_type_ptr<ngraph::opset1::Constant>(n.input_value(i).get_node_shared_ptr());
@@ -149,6 +158,26 @@ struct Translator {
         } else if (ngraph::is_type<ngraph::opset1::Gather>(node)) {
             const auto axis = constant_i64(n.input_value(2), n);
             check(hipie_graph_gather(g, in(n, 0), in(n, 1), axis.at(0), &id), "hipie_graph_gather");
+        } else if (ngraph::is_type<ngraph::opset1::Split>(node) || ngraph::is_type<ngraph::opset1::VariadicSplit>(node)) {
+            // every output is the box reference::split takes for it: consecutive extents along the axis
+            const auto axis_c = constant_i64(n.input_value(1), n);
+            const int64_t rank = static_cast<int64_t>(n.get_input_shape(0).size());
+            const int64_t axis = axis_c.at(0) < 0 ? axis_c.at(0) + rank : axis_c.at(0);
+            const int x = in(n, 0);
+            int64_t begin = 0;
+            for (size_t k = 0; k < n.get_output_size(); ++k) {
+                const int64_t extent = static_cast<int64_t>(n.get_output_shape(k).at(static_cast<size_t>(axis)));
+                int part = -1;
+                check(hipie_graph_slice(g, x, axis, begin, begin + extent, &part), "hipie_graph_slice");
+                output_id[{&n, k}] = part;
+                const std::string name = n.get_friendly_name() + '.' + std::to_string(k);
+                check(hipie_graph_set_name(g, part, name.c_str()), "hipie_graph_set_name");
+                if (out.node_names.size() <= static_cast<size_t>(part)) out.node_names.resize(part + 1);
+                out.node_names[part] = n.get_friendly_name();
+                if (k == 0) id_of[&n] = part;
+                begin += extent;
+            }
+            return true;
         } else if (const auto concat = ngraph::as_type_ptr<const ngraph::opset1::Concat>(node)) {
             std::vector<int> inputs;
             for (size_t i = 0; i < n.get_input_size(); ++i) inputs.push_back(in(n, i));

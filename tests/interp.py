@@ -99,6 +99,11 @@ def evaluate(orc, nodes, feeds, keep=None, override=None, targets=None):
             v = np.ascontiguousarray(np.take(x[0], idx, axis=n["axis"]))
         elif op == "Transpose":
             v = np.ascontiguousarray(np.transpose(x[0], n["order"]))
+        elif op == "Slice":
+            # one output of reference::split: the box [begin, end) along the axis, every other axis whole
+            box = [slice(None)] * x[0].ndim
+            box[n["axis"]] = slice(n["begin"], n["end"])
+            v = np.ascontiguousarray(x[0][tuple(box)])
         elif op == "Concat":
             v = np.concatenate(x, axis=n["axis"])             # concat.hpp:17-57: the inputs' elements side by side
         elif op == "Softmax":

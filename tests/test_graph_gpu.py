@@ -605,6 +605,42 @@ def test_convolutions_over_one_spatial_dimension(orc):
     assert all(g.query())
 
 
+def test_split_of_quantized_and_f32_values(orc):
+    """a channel-split unit: the u8 levels of a convolution split along the channels, one half through another
+    quantized convolution, the halves concatenated again and convolved; an f32 feature map split along its rows; a
+    split of dequantized levels with per-channel scales (every part keeps its own channels' scales)"""
+    from dldt_amd import builders
+    rng = np.random.default_rng(404)
+    x = rng.uniform(0, 1, (2, 16, 12, 10)).astype(np.float32)
+    rnd = lambda shape, s: (rng.standard_normal(shape, dtype=np.float32) * np.float32(s)).astype(np.float32)
+    net = builders.QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    a1 = net.conv(a0, rnd((48, 16, 3, 3), 0.08), rnd(48, 0.2), 2.5, pads=(1, 1))
+    left, right = [dict(node=n, scale=a1["scale"]) for n in g.split(a1["node"], 1, 2, 48)]
+    worked = net.conv(right, rnd((24, 24, 3, 3), 0.07), rnd(24, 0.2), 2.5, pads=(1, 1))
+    assert worked["scale"] == a1["scale"]
+    cat = dict(node=g.concat([left["node"], worked["node"]], axis=1), scale=a1["scale"])
+    g.result(net.conv_f32(cat, rnd((20, 48, 1, 1), 0.1), rnd(20, 0.1)), "out")
+    f = net.conv_f32(a0, rnd((6, 16, 1, 1), 0.3), rnd(6, 0.1))
+    for k, piece in enumerate(g.split(f, 2, 3, 12)):
+        g.result(piece, "rows%d" % k)
+    deq = g.multiply(g.convert(a1["node"], 10), g.constant(rng.uniform(0.5, 2, (1, 48, 1, 1)).astype(np.float32)))
+    for k, piece in enumerate(g.split(deq, 1, 3, 48)):
+        g.result(piece, "scaled%d" % k)
+    keep = [left["node"], right["node"], worked["node"], cat["node"]]
+    want, kept = evaluate(orc, g.nodes, {"data": x}, keep=keep)
+    plan = g.compile()
+    assert [s["type"] for s in plan.steps].count("Split") == 2 + 3 + 3
+    req = plan.create_request()
+    got = dict(zip([o["name"] for o in plan.outputs], req.infer(x)))
+    for node in keep:
+        np.testing.assert_array_equal(req.tensor(node), kept[node])
+    for name in want:
+        np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
+    assert all(g.query())
+
+
 @pytest.mark.parametrize("stride", [1, 2])
 def test_per_channel_activation_zero_points(orc, stride):
     """one integer zero point per channel in front of a padded depthwise convolution: the halo holds every channel's

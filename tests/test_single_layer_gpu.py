@@ -90,3 +90,34 @@ def test_softmax(orc, shape):
         assert [s["type"] for s in plan.steps] == ["Softmax", "Result"]
         np.testing.assert_allclose(got["out"], want["out"], rtol=3e-6, atol=1e-9, err_msg="axis %d" % axis)
         np.testing.assert_allclose(got["out"].sum(axis), 1.0, rtol=1e-6)
+
+
+@pytest.mark.parametrize("shape,target", [((30, 30, 30, 30), (30, 30, 30, 30)), ((10, 10, 10, 10), (10, 10, 100))])
+def test_reshape(orc, shape, target):
+    """smoke_ReshapeCheckDynBatch, smoke_ReshapeCheck and smoke_ReshapeCheckNegative ({10, 0, 100} and {10, -1, 100}
+    both resolve to [10, 10, 100] before a plugin sees them): the same bytes under other dimensions"""
+    from dldt_amd.graph import Graph
+    g = Graph()
+    x = np.random.default_rng(len(target)).standard_normal(shape).astype(np.float32)
+    g.result(g.reshape(g.parameter("data", shape), target), "out")
+    want, _ = evaluate(orc, g.nodes, {"data": x})
+    plan, got = _run(g, {"data": x})
+    assert got["out"].shape == tuple(target)
+    np.testing.assert_array_equal(got["out"].view(np.uint32), want["out"].view(np.uint32))
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2, 3])
+def test_split(orc, axis):
+    """smoke_NumSplitsCheck: [30, 30, 30, 30] into 1, 2, 3, 5, 6, 10 and 30 equal parts along every axis, every part a
+    result"""
+    from dldt_amd.graph import Graph
+    x = np.random.default_rng(axis).standard_normal((30, 30, 30, 30)).astype(np.float32)
+    for parts in (1, 2, 3, 5, 6, 10, 30):
+        g = Graph()
+        p = g.parameter("data", x.shape)
+        for k, piece in enumerate(g.split(p, axis, parts, 30)):
+            g.result(piece, "out%d" % k)
+        plan, got = _run(g, {"data": x})
+        assert len(got) == parts
+        for k, piece in enumerate(np.split(x, parts, axis)):
+            np.testing.assert_array_equal(got["out%d" % k].view(np.uint32), piece.view(np.uint32), err_msg="%d parts, part %d" % (parts, k))
