@@ -42,9 +42,9 @@ struct FqVerdicts {
 };
 
 // Elementwise nodes that no convolution / pooling / MatMul chain absorbs, on NHWC operands:
-//     out = FakeQuantize?( act?( op(a, b) ) ),  op in {none (unary), Add, Subtract, Multiply}, a and b in graph order.
+//     out = FakeQuantize?( act?( op(a, b) ) ),  op in {none (unary), Add, Subtract, Multiply, PRelu}, a and b in graph order.
 // An operand is a per-channel constant, an f32 tensor, or a byte tensor behind its dequantization
-// (float(level) - sub[c]) * mul[c].  Reference: reference::add / subtract / multiply (autobroadcast_binop.hpp), relu.hpp,
+// (float(level) - sub[c]) * mul[c].  Reference: reference::add / subtract / multiply (autobroadcast_binop.hpp), prelu.hpp, relu.hpp,
 // clamp.hpp, fake_quantize.hpp:175-194, each step one f32 operation as in the graph.
 struct EltOperand {
     const void* p = nullptr;          // tensor element (0, 0, 0, 0); null when the operand is `konst`
@@ -56,7 +56,7 @@ struct EltOperand {
 };
 struct EltArgs {
     EltOperand a, b;
-    int32_t op = 0;                   // 0 none, 1 add, 2 subtract, 3 multiply
+    int32_t op = 0;                   // 0 none, 1 add, 2 subtract, 3 multiply, 4 prelu (a < 0 ? a * b : a)
     int32_t act = 0;                  // 0 none, 1 relu, 2 clamp(lo, hi)
     float lo = 0, hi = 0;
     void* out = nullptr;

@@ -630,7 +630,8 @@ __global__ __launch_bounds__(kThreads) void eltwise_nhwc_kernel(const EltArgs a,
     if (a.op != 0) {
         elt_load4(a.b, n * a.b.sn + h * a.b.sh + w * a.b.sw, c0, u);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = a.op == 1 ? v[j] + u[j] : (a.op == 2 ? v[j] - u[j] : v[j] * u[j]);
+        for (int j = 0; j < 4; ++j)
+            v[j] = a.op == 1 ? v[j] + u[j] : (a.op == 2 ? v[j] - u[j] : (a.op == 3 ? v[j] * u[j] : (v[j] < 0.0f ? v[j] * u[j] : v[j])));   // 4: prelu.hpp:43
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {

@@ -9,8 +9,8 @@ const char* op_name(int op) {
     static const char* names[] = {"Parameter", "Constant", "FakeQuantize", "Convolution",
                                   "GroupConvolution", "MatMul", "Add", "Multiply", "Subtract", "Relu",
                                   "Clamp", "Convert", "MaxPool", "AvgPool", "Reshape", "Result", "Softmax", "MVN",
-                                  "Gelu", "Transpose", "Gather", "Concat", "Slice"};
-    return op >= 0 && op <= OP_SLICE ? names[op] : "?";
+                                  "Gelu", "Transpose", "Gather", "Concat", "Slice", "PRelu"};
+    return op >= 0 && op <= OP_PRELU ? names[op] : "?";
 }
 
 namespace {
@@ -226,7 +226,7 @@ int hipie_graph_matmul(hipie_graph* g, int a, int b, int transpose_a, int transp
 int hipie_graph_eltwise(hipie_graph* g, int kind, int a, int b, int* id) {
     return guarded([&] {
         HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_eltwise: null argument");
-        HIPIE_REQUIRE(kind == OP_ADD || kind == OP_MULTIPLY || kind == OP_SUBTRACT, HIPIE_PARAMETER_MISMATCH,
+        HIPIE_REQUIRE(kind == OP_ADD || kind == OP_MULTIPLY || kind == OP_SUBTRACT || kind == OP_PRELU, HIPIE_PARAMETER_MISMATCH,
                       "hipie_graph_eltwise: kind %d", kind);
         GNode& A = node(g, a, "hipie_graph_eltwise");
         GNode& B = node(g, b, "hipie_graph_eltwise");
@@ -236,7 +236,17 @@ int hipie_graph_eltwise(hipie_graph* g, int kind, int a, int b, int* id) {
         n.op = kind;
         n.in = {a, b};
         n.dtype = HIPIE_F32;
-        n.shape = broadcast_shape(A.shape, B.shape, "hipie_graph_eltwise");
+        if (kind == OP_PRELU) {
+            // op::v0::PRelu: the result has the argument's shape; a one-dimensional slope with one element per channel
+            // is taken per channel (prelu.hpp:28-35), any other slope must broadcast onto the argument
+            const size_t channel_axis = A.shape.size() > 1 ? 1 : 0;
+            if (!(B.shape.size() == 1 && !A.shape.empty() && B.shape[0] == A.shape[channel_axis]))
+                HIPIE_REQUIRE(broadcast_shape(A.shape, B.shape, "hipie_graph_eltwise") == A.shape, HIPIE_PARAMETER_MISMATCH,
+                              "hipie_graph_eltwise: a PRelu slope larger than its argument");
+            n.shape = A.shape;
+        } else {
+            n.shape = broadcast_shape(A.shape, B.shape, "hipie_graph_eltwise");
+        }
         *id = add_node(g, std::move(n));
     });
 }
@@ -680,7 +690,7 @@ hipie_graph* deserialize_graph(const uint8_t* bytes, size_t size) {
             arity(2);
             st = hipie_graph_matmul(G, in[0], in[1], flags & F_TA, flags & F_TB, &id);
             break;
-        case OP_ADD: case OP_MULTIPLY: case OP_SUBTRACT:
+        case OP_ADD: case OP_MULTIPLY: case OP_SUBTRACT: case OP_PRELU:
             arity(2);
             st = hipie_graph_eltwise(G, op, in[0], in[1], &id);
             break;

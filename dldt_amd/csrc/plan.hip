@@ -1245,7 +1245,7 @@ struct Planner {
             if (mat || (n.in.size() == 2 && N(n.in[1]).op != OP_CONSTANT && value(n.in[1]).kind == VK_MAT)) plan_mat_add(id);
             else plan_eltwise(id);
             break;
-        case OP_RELU: case OP_CLAMP: plan_eltwise(id); break;
+        case OP_RELU: case OP_CLAMP: case OP_PRELU: plan_eltwise(id); break;
         case OP_MAX_POOL: case OP_AVG_POOL: plan_pool(id); break;
         case OP_RESHAPE: mat ? plan_mat_reshape(id) : plan_reshape(id); break;
         case OP_TRANSPOSE: plan_mat_transpose(id); break;
@@ -2717,7 +2717,11 @@ struct Planner {
         auto st = std::make_unique<EltwiseStep>();
         auto operand = [&](int in, EltwiseStep::Operand& o) {
             if (N(in).op == OP_CONSTANT) {
-                if (!channel_constant(in, c, n.shape.size(), o.konst)) unsupported(id, "elementwise constant must be scalar or per-channel");
+                // (a PRelu's one-dimensional slope with one element per channel names the channels, prelu.hpp:28-35)
+                const GNode& k = N(in);
+                if (n.op == OP_PRELU && k.dtype == HIPIE_F32 && k.shape.size() == 1 && k.shape[0] == c && n.shape.size() > 1)
+                    o.konst.assign(k.f32(), k.f32() + c);
+                else if (!channel_constant(in, c, n.shape.size(), o.konst)) unsupported(id, "elementwise constant must be scalar or per-channel");
                 return;
             }
             const Value x = value(in);
@@ -2743,11 +2747,11 @@ struct Planner {
                 unsupported(id, "elementwise operand must be an f32 graph input, an f32 tensor or a dequantized byte tensor");
             }
         };
-        const bool binary = n.op == OP_ADD || n.op == OP_SUBTRACT || n.op == OP_MULTIPLY;
+        const bool binary = n.op == OP_ADD || n.op == OP_SUBTRACT || n.op == OP_MULTIPLY || n.op == OP_PRELU;
         operand(n.in[0], st->a);
         if (binary) {
             operand(n.in[1], st->b);
-            st->op = n.op == OP_ADD ? 1 : (n.op == OP_SUBTRACT ? 2 : 3);
+            st->op = n.op == OP_ADD ? 1 : (n.op == OP_SUBTRACT ? 2 : (n.op == OP_MULTIPLY ? 3 : 4));
             if (st->a.tensor < 0 && st->b.tensor < 0) unsupported(id, "elementwise node on two constants (constant folding is the front end's)");
         }
         int cur = id;
@@ -2901,7 +2905,7 @@ struct PlanPrepared {       // the host work an exported plan carries (hipie_pla
 bool to_two_spatial_dimensions(const hipie_graph& g, hipie_graph& out) {
     auto spatial_op = [](int op) { return op == OP_CONVOLUTION || op == OP_GROUP_CONVOLUTION || op == OP_MAX_POOL || op == OP_AVG_POOL; };
     auto keeps_layout = [&](int op) {
-        return spatial_op(op) || op == OP_FAKE_QUANTIZE || op == OP_ADD || op == OP_SUBTRACT || op == OP_MULTIPLY || op == OP_RELU ||
+        return spatial_op(op) || op == OP_FAKE_QUANTIZE || op == OP_ADD || op == OP_SUBTRACT || op == OP_MULTIPLY || op == OP_RELU || op == OP_PRELU ||
                op == OP_CLAMP || op == OP_CONVERT || op == OP_CONCAT || op == OP_PARAMETER || op == OP_RESULT;
     };
     const int n_nodes = static_cast<int>(g.nodes.size());

@@ -11,7 +11,7 @@ import numpy as np
 from ._lib import check, lib
 from .tensor import F32, I8, I32, U8, U8B, hipie_tensor
 
-OP_ADD, OP_MULTIPLY, OP_SUBTRACT = 6, 7, 8
+OP_ADD, OP_MULTIPLY, OP_SUBTRACT, OP_PRELU = 6, 7, 8, 23
 _NP = {F32: np.float32, U8: np.uint8, I8: np.int8, I32: np.int32}
 
 
@@ -84,6 +84,9 @@ class Graph:
 
     def subtract(self, a, b):
         return self._eltwise(OP_SUBTRACT, "Subtract", a, b)
+
+    def prelu(self, x, slope):
+        return self._eltwise(OP_PRELU, "PRelu", x, slope)
 
     def relu(self, x):
         i = ctypes.c_int()

@@ -408,7 +408,9 @@ typedef struct hipie_graph hipie_graph;
 typedef struct hipie_plan hipie_plan;
 typedef struct hipie_request hipie_request;
 
-enum { HIPIE_OP_ADD = 6, HIPIE_OP_MULTIPLY = 7, HIPIE_OP_SUBTRACT = 8 }; /* hipie_graph_eltwise kinds */
+/* hipie_graph_eltwise kinds.  PRELU: op::v0::PRelu(a, slope) = a < 0 ? a * slope : a (reference prelu.hpp:22-47; a
+ * one-dimensional slope with one element per channel of `a` is taken per channel, any other broadcasts numpy-style) */
+enum { HIPIE_OP_ADD = 6, HIPIE_OP_MULTIPLY = 7, HIPIE_OP_SUBTRACT = 8, HIPIE_OP_PRELU = 23 };
 
 int hipie_graph_create(hipie_graph** graph);
 void hipie_graph_destroy(hipie_graph* graph);

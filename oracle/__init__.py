@@ -132,6 +132,13 @@ class _Ops:
     def divide(self, a, b):
         return self._binop("divide_f32", a, b)
 
+    def prelu(self, x, slope):
+        x = np.ascontiguousarray(x, np.float32)
+        slope = np.ascontiguousarray(slope, np.float32)
+        out = np.empty_like(x)
+        self._fn("prelu_f32")(_ptr(x), *_shape(x.shape), _ptr(slope), *_shape(slope.shape), _ptr(out))
+        return out
+
     def relu(self, x):
         x = np.ascontiguousarray(x, np.float32)
         out = np.empty_like(x)

@@ -15,6 +15,7 @@
  *   group_convolution  reference goldens group_convolution.in.cpp + _ref fuzz
  *   matmul             reference goldens matmul.in.cpp + numpy integer matmul + _ref fuzz
  *   add/mul/sub/relu/clamp/convert   numpy closed forms + _ref fuzz
+ *   prelu              36 reference goldens prelu.in.cpp (every literal vector there) + _ref fuzz
  *   max_pool/avg_pool  reference goldens + _ref fuzz
  *   softmax/mvn/gelu   _ref fuzz + scipy closed forms (tolerance only; libm-dependent)
  */
@@ -355,6 +356,22 @@ DEFINE_BINOP(orc_add_f32, x + y)
 DEFINE_BINOP(orc_subtract_f32, x - y)
 DEFINE_BINOP(orc_multiply_f32, x * y)
 DEFINE_BINOP(orc_divide_f32, x / y)
+
+/* prelu.hpp:22-47: a one-dimensional slope with as many elements as the argument has channels (axis 1, axis 0 for a
+ * one-dimensional argument) is taken per channel; any other slope broadcasts numpy-style; x < 0 ? x * slope : x */
+DEFINE_BINOP(orc_prelu_binop_f32, x < 0.0f ? x * y : x)
+void orc_prelu_f32(const float* a, const int64_t* a_shape, int ar, const float* slope, const int64_t* s_shape, int sr,
+                   float* out) {
+    int64_t channel_shape[ORC_MAX_RANK];
+    const int channel_axis = ar > 1 ? 1 : 0;
+    if (sr == 1 && a_shape[channel_axis] == s_shape[0]) {
+        for (int k = 0; k < ar; ++k) channel_shape[k] = 1;
+        channel_shape[channel_axis] = s_shape[0];
+        s_shape = channel_shape;
+        sr = ar;
+    }
+    orc_prelu_binop_f32(a, a_shape, ar, slope, s_shape, sr, a_shape, ar, out);
+}
 
 /* relu.hpp: arg > 0 ? arg : 0 */
 void orc_relu_f32(const float* x, float* out, int64_t n) {

@@ -18,6 +18,7 @@
 #include "ngraph/runtime/reference/max_pool.hpp"
 #include "ngraph/runtime/reference/multiply.hpp"
 #include "ngraph/runtime/reference/mvn.hpp"
+#include "ngraph/runtime/reference/prelu.hpp"
 #include "ngraph/runtime/reference/relu.hpp"
 #include "ngraph/runtime/reference/softmax.hpp"
 #include "ngraph/runtime/reference/subtract.hpp"
@@ -95,6 +96,10 @@ MATMUL_EXPORT(ref_matmul_i64, int64_t)
         ref::FN<float>(a, b, out, mk_shape(a_shape, ar), mk_shape(b_shape, br),                 \
                        op::AutoBroadcastSpec(op::AutoBroadcastType::NUMPY));                    \
     }
+void ref_prelu_f32(const float* a, const int64_t* a_shape, int ar, const float* slope, const int64_t* s_shape, int sr,
+                   float* out) {
+    ref::prelu<float>(a, slope, out, mk_shape(a_shape, ar), mk_shape(s_shape, sr));
+}
 BINOP_EXPORT(ref_add_f32, add)
 BINOP_EXPORT(ref_subtract_f32, subtract)
 BINOP_EXPORT(ref_multiply_f32, multiply)

@@ -117,6 +117,8 @@ struct Translator {
             check(hipie_graph_eltwise(g, HIPIE_OP_MULTIPLY, in(n, 0), in(n, 1), &id), "hipie_graph_eltwise");
         } else if (ngraph::is_type<ngraph::opset1::Subtract>(node)) {
             check(hipie_graph_eltwise(g, HIPIE_OP_SUBTRACT, in(n, 0), in(n, 1), &id), "hipie_graph_eltwise");
+        } else if (ngraph::is_type<ngraph::opset1::PRelu>(node)) {
+            check(hipie_graph_eltwise(g, HIPIE_OP_PRELU, in(n, 0), in(n, 1), &id), "hipie_graph_eltwise");
         } else if (ngraph::is_type<ngraph::opset1::Relu>(node)) {
             check(hipie_graph_relu(g, in(n, 0), &id), "hipie_graph_relu");
         } else if (const auto cl = ngraph::as_type_ptr<ngraph::opset1::Clamp>(node)) {

@@ -76,7 +76,7 @@ def extract(path):
 def main():
     ref = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
     backend = os.path.join(ref, "ngraph", "test", "backend")
-    for stem in ("fake_quantize", "convolution", "group_convolution", "max_pool", "avg_pool"):
+    for stem in ("fake_quantize", "convolution", "group_convolution", "max_pool", "avg_pool", "prelu"):
         rec = extract(os.path.join(backend, stem + ".in.cpp"))
         dst = os.path.join(HERE, stem + ".json")
         with open(dst, "w") as f:

@@ -78,6 +78,8 @@ def evaluate(orc, nodes, feeds, keep=None, override=None, targets=None):
             v = orc.multiply(x[0], x[1])
         elif op == "Subtract":
             v = orc.subtract(x[0], x[1])
+        elif op == "PRelu":
+            v = orc.prelu(x[0], x[1])
         elif op == "Relu":
             v = orc.relu(x[0])
         elif op == "Clamp":

@@ -641,6 +641,42 @@ def test_split_of_quantized_and_f32_values(orc):
     assert all(g.query())
 
 
+def test_prelu_between_a_quantized_convolution_and_its_fake_quantize(orc):
+    """what PReluTransformation leaves (prelu.cpp:39-47: the dequantization Multiply moves behind the PRelu and the
+    FakeQuantize that follows absorbs it): Conv' -> Add(b') -> PRelu(slope[C]) -> FakeQuantize with per-channel input
+    ranges -> i8 levels; a leaky ReLU (scalar slope) on dequantized levels; a [1, C, 1, 1] slope on an f32 value"""
+    from dldt_amd import builders, lpt
+    rng = np.random.default_rng(909)
+    x = rng.uniform(0, 1, (2, 16, 12, 10)).astype(np.float32)
+    rnd = lambda shape, s: (rng.standard_normal(shape, dtype=np.float32) * np.float32(s)).astype(np.float32)
+    net = builders.QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    y, s, rank = net._accumulate(a0, rnd((24, 16, 3, 3), 0.08), rnd(24, 0.3),
+                                 dict(strides=(1, 1), dilations=(1, 1), pads_begin=(1, 1), pads_end=(1, 1)))
+    y = g.prelu(y, g.constant(rng.uniform(0.05, 0.3, 24).astype(np.float32)))          # [C]: one slope per channel
+    lo, hi = net.signed_range(2.0)
+    d = lpt.decompose_fake_quantize(256, lo, hi)
+    il, ih = lpt.fuse_elementwise(lpt.MULTIPLY, lo, hi, s)
+    q = g.fake_quantize(y, net._channel(il, rank), net._channel(ih, rank), d["new_low"], d["new_high"], 256, d["precision"])
+    a1 = dict(node=q, scale=np.float32(d["scale"]))
+    g.result(net.conv_f32(a1, rnd((8, 24, 1, 1), 0.1), rnd(8, 0.1)), "out")
+    g.result(g.prelu(net.dequantize(a1), g.constant(np.float32(0.1))), "leaky")
+    f = net.conv_f32(a0, rnd((6, 16, 1, 1), 0.3), rnd(6, 0.2))
+    g.result(g.prelu(f, g.constant(rng.uniform(-0.5, 0.5, (1, 6, 1, 1)).astype(np.float32))), "per_channel")
+    want, kept = evaluate(orc, g.nodes, {"data": x}, keep=[q])
+    levels = kept[q].astype(np.int32)
+    assert len(np.unique(levels)) > 80 and 0.2 < (levels < 0).mean() < 0.8
+    plan = g.compile()
+    assert "PRelu+FakeQuantize" in [s["type"] for s in plan.steps]
+    req = plan.create_request()
+    got = dict(zip([o["name"] for o in plan.outputs], req.infer(x)))
+    np.testing.assert_array_equal(req.tensor(q), kept[q])
+    for name in want:
+        np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
+    assert all(g.query())
+
+
 @pytest.mark.parametrize("stride", [1, 2])
 def test_per_channel_activation_zero_points(orc, stride):
     """one integer zero point per channel in front of a padded depthwise convolution: the halo holds every channel's

@@ -28,6 +28,25 @@ def test_fake_quantize_golden(orc, name):
     np.testing.assert_allclose(got.ravel(), np.array(t["expected"], np.float32), rtol=1e-6)
 
 
+def _prelu_cases():
+    # (two of the 38 tests build their slope in a loop instead of writing it out: no literal vector to take)
+    return {k: v for k, v in load("prelu").items() if all(f in v for f in ("a", "slope", "out", "shape_a", "shape_slope"))}
+
+
+@pytest.mark.parametrize("name", sorted(_prelu_cases()))
+def test_prelu_golden(orc, name):
+    """ngraph/test/backend/prelu.in.cpp: scalar slopes, one per channel ([C], [C, 1, 1], [1, C, 1, W]), one per column,
+    whole tensors - the 1-D slope that names the channels against the 1-D slope that broadcasts along the last axis"""
+    t = _prelu_cases()[name]
+    a = np.array(t["a"], np.float32).reshape(t["shape_a"])
+    slope = np.array(t["slope"], np.float32).reshape(t["shape_slope"])
+    np.testing.assert_array_equal(orc.prelu(a, slope), np.array(t["out"], np.float32).reshape(t["shape_a"]))
+
+
+def test_prelu_golden_count():
+    assert len(_prelu_cases()) == 36
+
+
 def _conv_cases(stem):
     return {k: v for k, v in load(stem).items()
             if all(f in v for f in ("inputs", "filters", "outputs", "strides", "padding"))}
@@ -203,6 +222,10 @@ def test_elementwise_vs_ref(orc, ref):
             np.testing.assert_array_equal(x.view(np.uint32), y.view(np.uint32))
     np.testing.assert_array_equal(orc.relu(a), ref.relu(a))
     np.testing.assert_array_equal(orc.clamp(a, 0.0, 0.6), ref.clamp(a, 0.0, 0.6))
+    for sshape in ((1,), (5,), (3,), (1, 5, 1, 1), (5, 1, 1), (2, 5, 4, 3), (4, 1)):
+        slope = rng.normal(size=sshape).astype(np.float32)
+        x, y = orc.prelu(a, slope), ref.prelu(a, slope)
+        np.testing.assert_array_equal(x.view(np.uint32), y.view(np.uint32), err_msg=str(sshape))
 
 
 @pytest.mark.parametrize("dt", [np.uint8, np.int8, np.float32, np.int32])
