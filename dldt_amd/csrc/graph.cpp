@@ -5,6 +5,10 @@
 
 namespace hipie {
 
+// the kinds hipie_graph_eltwise takes are the planner's own operation numbers
+static_assert(HIPIE_OP_ADD == OP_ADD && HIPIE_OP_MULTIPLY == OP_MULTIPLY && HIPIE_OP_SUBTRACT == OP_SUBTRACT && HIPIE_OP_PRELU == OP_PRELU,
+              "include/hipie.h and graph.h number the elementwise operations differently");
+
 const char* op_name(int op) {
     static const char* names[] = {"Parameter", "Constant", "FakeQuantize", "Convolution",
                                   "GroupConvolution", "MatMul", "Add", "Multiply", "Subtract", "Relu",
