@@ -57,7 +57,7 @@ struct EltOperand {
 struct EltArgs {
     EltOperand a, b;
     int32_t op = 0;                   // 0 none, 1 add, 2 subtract, 3 multiply, 4 prelu (a < 0 ? a * b : a)
-    int32_t act = 0;                  // 0 none, 1 relu, 2 clamp(lo, hi)
+    int32_t act = 0;                  // 0 none, 1 relu, 2 clamp(lo, hi), 3 sigmoid, 4 hswish, 5 hsigmoid, 6 swish(beta = lo)
     float lo = 0, hi = 0;
     void* out = nullptr;
     int32_t out_dtype = HIPIE_F32;    // HIPIE_F32, or HIPIE_U8B / HIPIE_I8 behind a FakeQuantize

@@ -637,6 +637,10 @@ __global__ __launch_bounds__(kThreads) void eltwise_nhwc_kernel(const EltArgs a,
     for (int j = 0; j < 4; ++j) {
         if (a.act == 1) v[j] = v[j] > 0.0f ? v[j] : 0.0f;                                    // relu.hpp
         else if (a.act == 2) v[j] = v[j] < a.lo ? a.lo : (v[j] > a.hi ? a.hi : v[j]);        // clamp.hpp
+        else if (a.act == 3) v[j] = 1.0f / (1.0f + expf(-v[j]));                             // sigmoid.hpp
+        else if (a.act == 4) v[j] = v[j] * fminf(fmaxf(v[j] + 3.0f, 0.0f), 6.0f) / 6.0f;     // hswish.hpp: (x * clamped) / 6
+        else if (a.act == 5) v[j] = fminf(fmaxf(v[j] + 3.0f, 0.0f), 6.0f) / 6.0f;            // hsigmoid.hpp
+        else if (a.act == 6) v[j] = static_cast<float>(static_cast<double>(v[j]) / (1.0 + static_cast<double>(expf(-v[j] * a.lo))));   // swish.hpp: the sum and the quotient in double
     }
     const int64_t o = n * a.out_sn + h * a.out_sh + w * a.out_sw + c0;
     if (tab) {

@@ -6,15 +6,18 @@
 namespace hipie {
 
 // the kinds hipie_graph_eltwise takes are the planner's own operation numbers
-static_assert(HIPIE_OP_ADD == OP_ADD && HIPIE_OP_MULTIPLY == OP_MULTIPLY && HIPIE_OP_SUBTRACT == OP_SUBTRACT && HIPIE_OP_PRELU == OP_PRELU,
+static_assert(HIPIE_OP_ADD == OP_ADD && HIPIE_OP_MULTIPLY == OP_MULTIPLY && HIPIE_OP_SUBTRACT == OP_SUBTRACT && HIPIE_OP_PRELU == OP_PRELU &&
+                  HIPIE_OP_SIGMOID == OP_SIGMOID && HIPIE_OP_HSWISH == OP_HSWISH && HIPIE_OP_HSIGMOID == OP_HSIGMOID &&
+                  HIPIE_OP_SWISH == OP_SWISH,
               "include/hipie.h and graph.h number the elementwise operations differently");
 
 const char* op_name(int op) {
     static const char* names[] = {"Parameter", "Constant", "FakeQuantize", "Convolution",
                                   "GroupConvolution", "MatMul", "Add", "Multiply", "Subtract", "Relu",
                                   "Clamp", "Convert", "MaxPool", "AvgPool", "Reshape", "Result", "Softmax", "MVN",
-                                  "Gelu", "Transpose", "Gather", "Concat", "Slice", "PRelu"};
-    return op >= 0 && op <= OP_PRELU ? names[op] : "?";
+                                  "Gelu", "Transpose", "Gather", "Concat", "Slice", "PRelu",
+                                  "Sigmoid", "HSwish", "HSigmoid", "Swish"};
+    return op >= 0 && op <= OP_SWISH ? names[op] : "?";
 }
 
 namespace {
@@ -263,6 +266,23 @@ int hipie_graph_relu(hipie_graph* g, int x, int* id) {
         n.op = OP_RELU;
         n.in = {x};
         n.dtype = X.dtype;
+        n.shape = X.shape;
+        *id = add_node(g, std::move(n));
+    });
+}
+
+int hipie_graph_activation(hipie_graph* g, int kind, int x, float beta, int* id) {
+    return guarded([&] {
+        HIPIE_REQUIRE(id, HIPIE_PARAMETER_MISMATCH, "hipie_graph_activation: null argument");
+        HIPIE_REQUIRE(kind == OP_SIGMOID || kind == OP_HSWISH || kind == OP_HSIGMOID || kind == OP_SWISH, HIPIE_PARAMETER_MISMATCH,
+                      "hipie_graph_activation: kind %d", kind);
+        GNode& X = node(g, x, "hipie_graph_activation");
+        HIPIE_REQUIRE(X.dtype == HIPIE_F32, HIPIE_PARAMETER_MISMATCH, "hipie_graph_activation: data must be f32");
+        GNode n;
+        n.op = kind;
+        n.in = {x};
+        n.lo = kind == OP_SWISH ? beta : 0.f;
+        n.dtype = HIPIE_F32;
         n.shape = X.shape;
         *id = add_node(g, std::move(n));
     });
@@ -700,6 +720,7 @@ hipie_graph* deserialize_graph(const uint8_t* bytes, size_t size) {
             break;
         case OP_RELU: arity(1); st = hipie_graph_relu(G, in[0], &id); break;
         case OP_CLAMP: arity(1); st = hipie_graph_clamp(G, in[0], lo, hi, &id); break;
+        case OP_SIGMOID: case OP_HSWISH: case OP_HSIGMOID: case OP_SWISH: arity(1); st = hipie_graph_activation(G, op, in[0], lo, &id); break;
         case OP_CONVERT: arity(1); st = hipie_graph_convert(G, in[0], dtype, &id); break;
         case OP_MAX_POOL:
             arity(1);

@@ -14,7 +14,8 @@ namespace hipie {
 enum OpKind {
     OP_PARAMETER = 0, OP_CONSTANT, OP_FAKE_QUANTIZE, OP_CONVOLUTION, OP_GROUP_CONVOLUTION, OP_MATMUL,
     OP_ADD, OP_MULTIPLY, OP_SUBTRACT, OP_RELU, OP_CLAMP, OP_CONVERT, OP_MAX_POOL, OP_AVG_POOL,
-    OP_RESHAPE, OP_RESULT, OP_SOFTMAX, OP_MVN, OP_GELU, OP_TRANSPOSE, OP_GATHER, OP_CONCAT, OP_SLICE, OP_PRELU
+    OP_RESHAPE, OP_RESULT, OP_SOFTMAX, OP_MVN, OP_GELU, OP_TRANSPOSE, OP_GATHER, OP_CONCAT, OP_SLICE, OP_PRELU,
+    OP_SIGMOID, OP_HSWISH, OP_HSIGMOID, OP_SWISH          // (Swish: beta in GNode::lo)
 };
 const char* op_name(int op);
 

@@ -1245,7 +1245,9 @@ struct Planner {
             if (mat || (n.in.size() == 2 && N(n.in[1]).op != OP_CONSTANT && value(n.in[1]).kind == VK_MAT)) plan_mat_add(id);
             else plan_eltwise(id);
             break;
-        case OP_RELU: case OP_CLAMP: case OP_PRELU: plan_eltwise(id); break;
+        case OP_RELU: case OP_CLAMP: case OP_PRELU: case OP_SIGMOID: case OP_HSWISH: case OP_HSIGMOID: case OP_SWISH:
+            plan_eltwise(id);
+            break;
         case OP_MAX_POOL: case OP_AVG_POOL: plan_pool(id); break;
         case OP_RESHAPE: mat ? plan_mat_reshape(id) : plan_reshape(id); break;
         case OP_TRANSPOSE: plan_mat_transpose(id); break;
@@ -2755,9 +2757,16 @@ struct Planner {
             if (st->a.tensor < 0 && st->b.tensor < 0) unsupported(id, "elementwise node on two constants (constant folding is the front end's)");
         }
         int cur = id;
+        auto is_activation = [](int op) {
+            return op == OP_RELU || op == OP_CLAMP || op == OP_SIGMOID || op == OP_HSWISH || op == OP_HSIGMOID || op == OP_SWISH;
+        };
         auto take_activation = [&](const GNode& u) {
             if (u.op == OP_RELU) st->act = 1;
-            else { st->act = 2; st->lo = u.lo; st->hi = u.hi; }
+            else if (u.op == OP_CLAMP) { st->act = 2; st->lo = u.lo; st->hi = u.hi; }
+            else if (u.op == OP_SIGMOID) st->act = 3;
+            else if (u.op == OP_HSWISH) st->act = 4;
+            else if (u.op == OP_HSIGMOID) st->act = 5;
+            else { st->act = 6; st->lo = u.lo; }      // Swish: beta
         };
         auto take_fq = [&](int node) {
             const GNode& u = N(node);
@@ -2772,14 +2781,14 @@ struct Planner {
             st->oh = oh[0];
             return true;
         };
-        if (n.op == OP_RELU || n.op == OP_CLAMP) take_activation(n);
+        if (is_activation(n.op)) take_activation(n);
         if (n.op == OP_FAKE_QUANTIZE) {
             if (!take_fq(id)) unsupported(id, "FakeQuantize with f32 output or bounds that are not per-channel constants");
         } else {
             while (single_user(cur) && !st->quantize) {
                 const int nx = N(cur).users[0];
                 const GNode& u = N(nx);
-                if ((u.op == OP_RELU || u.op == OP_CLAMP) && st->act == 0) take_activation(u);
+                if (is_activation(u.op) && st->act == 0) take_activation(u);
                 else if (u.op == OP_FAKE_QUANTIZE && u.in[0] == cur && take_fq(nx)) {}
                 else break;
                 cur = nx;
@@ -2905,7 +2914,8 @@ struct PlanPrepared {       // the host work an exported plan carries (hipie_pla
 bool to_two_spatial_dimensions(const hipie_graph& g, hipie_graph& out) {
     auto spatial_op = [](int op) { return op == OP_CONVOLUTION || op == OP_GROUP_CONVOLUTION || op == OP_MAX_POOL || op == OP_AVG_POOL; };
     auto keeps_layout = [&](int op) {
-        return spatial_op(op) || op == OP_FAKE_QUANTIZE || op == OP_ADD || op == OP_SUBTRACT || op == OP_MULTIPLY || op == OP_RELU || op == OP_PRELU ||
+        return spatial_op(op) || op == OP_FAKE_QUANTIZE || op == OP_ADD || op == OP_SUBTRACT || op == OP_MULTIPLY || op == OP_RELU || op == OP_PRELU || op == OP_SIGMOID ||
+               op == OP_HSWISH || op == OP_HSIGMOID || op == OP_SWISH ||
                op == OP_CLAMP || op == OP_CONVERT || op == OP_CONCAT || op == OP_PARAMETER || op == OP_RESULT;
     };
     const int n_nodes = static_cast<int>(g.nodes.size());

@@ -12,6 +12,7 @@ from ._lib import check, lib
 from .tensor import F32, I8, I32, U8, U8B, hipie_tensor
 
 OP_ADD, OP_MULTIPLY, OP_SUBTRACT, OP_PRELU = 6, 7, 8, 23
+OP_SIGMOID, OP_HSWISH, OP_HSIGMOID, OP_SWISH = 24, 25, 26, 27
 _NP = {F32: np.float32, U8: np.uint8, I8: np.int8, I32: np.int32}
 
 
@@ -87,6 +88,23 @@ class Graph:
 
     def prelu(self, x, slope):
         return self._eltwise(OP_PRELU, "PRelu", x, slope)
+
+    def _activation(self, kind, name, x, beta=1.0):
+        i = ctypes.c_int()
+        check(lib().hipie_graph_activation(self._h, kind, x, ctypes.c_float(beta), ctypes.byref(i)))
+        return self._rec(i.value, name, [x], F32, beta=float(np.float32(beta)))
+
+    def sigmoid(self, x):
+        return self._activation(OP_SIGMOID, "Sigmoid", x)
+
+    def hswish(self, x):
+        return self._activation(OP_HSWISH, "HSwish", x)
+
+    def hsigmoid(self, x):
+        return self._activation(OP_HSIGMOID, "HSigmoid", x)
+
+    def swish(self, x, beta=1.0):
+        return self._activation(OP_SWISH, "Swish", x, beta)
 
     def relu(self, x):
         i = ctypes.c_int()

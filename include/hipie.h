@@ -411,6 +411,13 @@ typedef struct hipie_request hipie_request;
 /* hipie_graph_eltwise kinds.  PRELU: op::v0::PRelu(a, slope) = a < 0 ? a * slope : a (reference prelu.hpp:22-47; a
  * one-dimensional slope with one element per channel of `a` is taken per channel, any other broadcasts numpy-style) */
 enum { HIPIE_OP_ADD = 6, HIPIE_OP_MULTIPLY = 7, HIPIE_OP_SUBTRACT = 8, HIPIE_OP_PRELU = 23 };
+/* hipie_graph_activation kinds, f32 in and out (the low-precision transformations leave them in f32): Sigmoid
+ * 1 / (1 + exp(-x)) (reference sigmoid.hpp), op::v4::HSwish x * min(max(x + 3, 0), 6) / 6 (hswish.hpp), op::v5::HSigmoid
+ * min(max(x + 3, 0), 6) / 6 (hsigmoid.hpp), op::v4::Swish x / (1 + exp(-x * beta)) (swish.hpp; `beta` is read for
+ * Swish only).  HSwish and HSigmoid are the reference's f32 operations one by one; Sigmoid and Swish use the device's
+ * exp and agree to rounding. */
+enum { HIPIE_OP_SIGMOID = 24, HIPIE_OP_HSWISH = 25, HIPIE_OP_HSIGMOID = 26, HIPIE_OP_SWISH = 27 };
+int hipie_graph_activation(hipie_graph* g, int kind, int x, float beta, int* id);
 
 int hipie_graph_create(hipie_graph** graph);
 void hipie_graph_destroy(hipie_graph* graph);

@@ -139,6 +139,24 @@ class _Ops:
         self._fn("prelu_f32")(_ptr(x), *_shape(x.shape), _ptr(slope), *_shape(slope.shape), _ptr(out))
         return out
 
+    def _unary(self, name, x, *extra):
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.empty_like(x)
+        self._fn(name)(_ptr(x), *extra, _ptr(out), ctypes.c_int64(x.size))
+        return out
+
+    def sigmoid(self, x):
+        return self._unary("sigmoid_f32", x)
+
+    def hswish(self, x):
+        return self._unary("hswish_f32", x)
+
+    def hsigmoid(self, x):
+        return self._unary("hsigmoid_f32", x)
+
+    def swish(self, x, beta=1.0):
+        return self._unary("swish_f32", x, ctypes.c_float(beta))
+
     def relu(self, x):
         x = np.ascontiguousarray(x, np.float32)
         out = np.empty_like(x)

@@ -16,6 +16,9 @@
  *   matmul             reference goldens matmul.in.cpp + numpy integer matmul + _ref fuzz
  *   add/mul/sub/relu/clamp/convert   numpy closed forms + _ref fuzz
  *   prelu              36 reference goldens prelu.in.cpp (every literal vector there) + _ref fuzz
+ *   hswish/hsigmoid    _ref fuzz (bit-exact) + the points the definition fixes (0 below -3, x or 1 above 3, hswish(1) = 4/6)
+ *   sigmoid/swish      _ref fuzz + scipy closed forms (expit) on the inputs of sigmoid.in.cpp / swish.in.cpp, whose
+ *                      expected values are formulas, not vectors (tolerance only; libm-dependent)
  *   max_pool/avg_pool  reference goldens + _ref fuzz
  *   softmax/mvn/gelu   _ref fuzz + scipy closed forms (tolerance only; libm-dependent)
  */
@@ -371,6 +374,24 @@ void orc_prelu_f32(const float* a, const int64_t* a_shape, int ar, const float* 
         sr = ar;
     }
     orc_prelu_binop_f32(a, a_shape, ar, slope, s_shape, sr, a_shape, ar, out);
+}
+
+/* sigmoid.hpp: 1 / (1 + exp(-x)) in float; hswish.hpp: x * min(max(x + 3, 0), 6) / 6; hsigmoid.hpp: min(max(x + 3, 0), 6) / 6;
+ * swish.hpp: x / (1.0 + exp(-x * beta)) with the sum and the quotient in double (the literal 1.0) */
+void orc_sigmoid_f32(const float* x, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) {
+        const float e = expf(-x[i]);
+        out[i] = 1 / (1 + e);
+    }
+}
+void orc_hswish_f32(const float* x, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = x[i] * fminf(fmaxf(x[i] + 3.0f, 0.0f), 6.0f) / 6.0f;
+}
+void orc_hsigmoid_f32(const float* x, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = fminf(fmaxf(x[i] + 3.0f, 0.0f), 6.0f) / 6.0f;
+}
+void orc_swish_f32(const float* x, float beta, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = (float)(x[i] / (1.0 + expf(-x[i] * beta)));
 }
 
 /* relu.hpp: arg > 0 ? arg : 0 */

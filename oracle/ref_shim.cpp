@@ -18,7 +18,11 @@
 #include "ngraph/runtime/reference/max_pool.hpp"
 #include "ngraph/runtime/reference/multiply.hpp"
 #include "ngraph/runtime/reference/mvn.hpp"
+#include "ngraph/runtime/reference/hsigmoid.hpp"
+#include "ngraph/runtime/reference/hswish.hpp"
 #include "ngraph/runtime/reference/prelu.hpp"
+#include "ngraph/runtime/reference/sigmoid.hpp"
+#include "ngraph/runtime/reference/swish.hpp"
 #include "ngraph/runtime/reference/relu.hpp"
 #include "ngraph/runtime/reference/softmax.hpp"
 #include "ngraph/runtime/reference/subtract.hpp"
@@ -100,6 +104,10 @@ void ref_prelu_f32(const float* a, const int64_t* a_shape, int ar, const float* 
                    float* out) {
     ref::prelu<float>(a, slope, out, mk_shape(a_shape, ar), mk_shape(s_shape, sr));
 }
+void ref_sigmoid_f32(const float* x, float* out, int64_t n) { ref::sigmoid<float>(x, out, static_cast<size_t>(n)); }
+void ref_hswish_f32(const float* x, float* out, int64_t n) { ref::hswish<float>(x, out, static_cast<size_t>(n)); }
+void ref_hsigmoid_f32(const float* x, float* out, int64_t n) { ref::hsigmoid<float>(x, out, static_cast<size_t>(n)); }
+void ref_swish_f32(const float* x, float beta, float* out, int64_t n) { ref::swish<float>(x, &beta, out, static_cast<size_t>(n)); }
 BINOP_EXPORT(ref_add_f32, add)
 BINOP_EXPORT(ref_subtract_f32, subtract)
 BINOP_EXPORT(ref_multiply_f32, multiply)

@@ -117,6 +117,21 @@ struct Translator {
             check(hipie_graph_eltwise(g, HIPIE_OP_MULTIPLY, in(n, 0), in(n, 1), &id), "hipie_graph_eltwise");
         } else if (ngraph::is_type<ngraph::opset1::Subtract>(node)) {
             check(hipie_graph_eltwise(g, HIPIE_OP_SUBTRACT, in(n, 0), in(n, 1), &id), "hipie_graph_eltwise");
+        } else if (ngraph::is_type<ngraph::opset1::Sigmoid>(node)) {
+            check(hipie_graph_activation(g, HIPIE_OP_SIGMOID, in(n, 0), 1.0f, &id), "hipie_graph_activation");
+        } else if (ngraph::is_type<ngraph::opset7::HSwish>(node)) {
+            check(hipie_graph_activation(g, HIPIE_OP_HSWISH, in(n, 0), 1.0f, &id), "hipie_graph_activation");
+        } else if (ngraph::is_type<ngraph::opset7::HSigmoid>(node)) {
+            check(hipie_graph_activation(g, HIPIE_OP_HSIGMOID, in(n, 0), 1.0f, &id), "hipie_graph_activation");
+        } else if (ngraph::is_type<ngraph::opset7::Swish>(node)) {
+            float beta = 1.0f;
+            if (n.get_input_size() > 1) {
+                const auto b = ngraph::as_type_ptr<ngraph::opset1::Constant>(n.input_value(1).get_node_shared_ptr());
+                if (!b || ngraph::shape_size(b->get_shape()) != 1)
+                    IE_THROW(NotImplemented) << "HIP plugin: " << n.get_friendly_name() << ": Swish with a beta that is not a constant scalar";
+                beta = b->cast_vector<float>().at(0);
+            }
+            check(hipie_graph_activation(g, HIPIE_OP_SWISH, in(n, 0), beta, &id), "hipie_graph_activation");
         } else if (ngraph::is_type<ngraph::opset1::PRelu>(node)) {
             check(hipie_graph_eltwise(g, HIPIE_OP_PRELU, in(n, 0), in(n, 1), &id), "hipie_graph_eltwise");
         } else if (ngraph::is_type<ngraph::opset1::Relu>(node)) {

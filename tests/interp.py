@@ -80,6 +80,10 @@ def evaluate(orc, nodes, feeds, keep=None, override=None, targets=None):
             v = orc.subtract(x[0], x[1])
         elif op == "PRelu":
             v = orc.prelu(x[0], x[1])
+        elif op in ("Sigmoid", "HSwish", "HSigmoid"):
+            v = getattr(orc, op.lower())(x[0])
+        elif op == "Swish":
+            v = orc.swish(x[0], n["beta"])
         elif op == "Relu":
             v = orc.relu(x[0])
         elif op == "Clamp":

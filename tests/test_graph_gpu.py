@@ -677,6 +677,55 @@ def test_prelu_between_a_quantized_convolution_and_its_fake_quantize(orc):
     assert all(g.query())
 
 
+def test_hswish_sigmoid_swish_blocks(orc):
+    """the activations the low-precision transformations leave in f32 between a quantized convolution's dequantization
+    and the next FakeQuantize: Conv' -> Add -> Multiply -> HSwish -> FakeQuantize (bit-exact: every operation of
+    hswish.hpp is an IEEE f32 operation), an HSigmoid gate on a pooled value multiplied back onto the feature map (a
+    MobileNetV3 squeeze-and-excitation block), and Sigmoid / Swish, which use the device's exp: their f32 results to
+    rounding, and the quantized layers behind them bit-exact from the device's own values"""
+    from dldt_amd import builders
+    rng = np.random.default_rng(515)
+    x = rng.uniform(0, 1, (2, 16, 10, 12)).astype(np.float32)
+    rnd = lambda shape, s: (rng.standard_normal(shape, dtype=np.float32) * np.float32(s)).astype(np.float32)
+    net = builders.QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    hs = g.hswish(net.conv_f32(a0, rnd((24, 16, 3, 3), 0.12), rnd(24, 0.5), pads=(1, 1)))
+    a1 = net.requantize(hs, 3.0, signed=True)                     # i8: HSwish goes down to -0.375
+    g.result(net.dequantize(a1), "hswish_levels")
+    # squeeze-and-excitation with an HSigmoid gate
+    pooled = g.avg_pool(net.dequantize(a1), (10, 12), (1, 1), (0, 0), (0, 0))
+    gate = g.hsigmoid(g.convolution(pooled, g.constant(rnd((24, 24, 1, 1), 0.8))))
+    a2 = net.requantize(g.multiply(net.dequantize(a1), gate), 3.0, signed=True)
+    g.result(net.conv_f32(a2, rnd((8, 24, 1, 1), 0.1), rnd(8, 0.1)), "out")
+    f = net.conv_f32(a0, rnd((12, 16, 1, 1), 0.6), rnd(12, 0.5))
+    sg, sw = g.sigmoid(f), g.swish(f, 0.6)
+    g.result(sg, "sigmoid")
+    g.result(sw, "swish")
+    a3 = net.requantize(sw, 2.0, signed=True)
+    g.result(net.conv_f32(a3, rnd((6, 12, 1, 1), 0.2), rnd(6, 0.1)), "behind_swish")
+    keep = [hs, a1["node"], gate, a2["node"], a3["node"]]
+    plan = g.compile()
+    types = [s["type"] for s in plan.steps]
+    assert "HSwish+FakeQuantize" in types and "HSigmoid" in types and "Sigmoid" in types
+    req = plan.create_request()
+    got = dict(zip([o["name"] for o in plan.outputs], req.infer(x)))
+    want, kept = evaluate(orc, g.nodes, {"data": x}, keep=keep)
+    assert kept[hs].min() < -0.3 and len(np.unique(kept[a1["node"]])) > 80
+    for node in (a1["node"], a2["node"]):
+        np.testing.assert_array_equal(req.tensor(node), kept[node])
+    np.testing.assert_array_equal(req.tensor(gate).view(np.uint32), kept[gate].view(np.uint32))
+    for name in ("hswish_levels", "out"):
+        np.testing.assert_array_equal(got[name].view(np.uint32), want[name].view(np.uint32), err_msg=name)
+    np.testing.assert_allclose(got["sigmoid"], want["sigmoid"], rtol=3e-7, atol=0)
+    np.testing.assert_allclose(got["swish"], want["swish"], rtol=5e-7, atol=1e-9)
+    # what follows the Swish, from the device's own Swish
+    want2, kept2 = evaluate(orc, g.nodes, {"data": x}, keep=[a3["node"]], override={sw: got["swish"]})
+    np.testing.assert_array_equal(req.tensor(a3["node"]), kept2[a3["node"]])
+    np.testing.assert_array_equal(got["behind_swish"].view(np.uint32), want2["behind_swish"].view(np.uint32))
+    assert all(g.query())
+
+
 @pytest.mark.parametrize("stride", [1, 2])
 def test_per_channel_activation_zero_points(orc, stride):
     """one integer zero point per channel in front of a padded depthwise convolution: the halo holds every channel's

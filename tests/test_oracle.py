@@ -47,6 +47,24 @@ def test_prelu_golden_count():
     assert len(_prelu_cases()) == 36
 
 
+def test_activations_closed_forms(orc):
+    """Sigmoid and Swish on the inputs of the reference's sigmoid.in.cpp / swish.in.cpp (which compute their expected
+    values by formula) against scipy's expit in double, to rounding; HSwish and HSigmoid on the points their
+    definition fixes without arithmetic: 0 at and below -3, the identity (one) at and above 3, hswish(1) = 4 / 6"""
+    from scipy.special import expit
+    x = np.array([1, 8, -8, 17, -0.5, -1, 0.4, -5.7, -6, 3, -0.9, 23, 5, 3.3, 0.1, 0.6, 20, -7, -5.3, 3.5, -9, 11, 0], np.float32)
+    np.testing.assert_allclose(orc.sigmoid(x), expit(x.astype(np.float64)), rtol=2e-7, atol=0)
+    for beta in (1.0, 0.6, 0.33):
+        np.testing.assert_allclose(orc.swish(x, beta), x.astype(np.float64) * expit(x.astype(np.float64) * np.float64(np.float32(beta))), rtol=3e-7,
+                                   atol=1e-12)
+    pts = np.array([-1e30, -100, -3.0000002, -3, 3, 3.0000002, 100, 1e30], np.float32)
+    np.testing.assert_array_equal(orc.hsigmoid(pts), np.array([0, 0, 0, 0, 1, 1, 1, 1], np.float32))
+    np.testing.assert_array_equal(orc.hswish(pts)[:4], np.zeros(4, np.float32))
+    np.testing.assert_array_equal(orc.hswish(pts)[4:], pts[4:] * np.float32(6) / np.float32(6))
+    assert orc.hswish(np.float32([1]))[0] == np.float32(4) / np.float32(6)
+    assert orc.hsigmoid(np.float32([0]))[0] == np.float32(0.5) and orc.hswish(np.float32([-0.0]))[0] == 0
+
+
 def _conv_cases(stem):
     return {k: v for k, v in load(stem).items()
             if all(f in v for f in ("inputs", "filters", "outputs", "strides", "padding"))}
@@ -222,6 +240,12 @@ def test_elementwise_vs_ref(orc, ref):
             np.testing.assert_array_equal(x.view(np.uint32), y.view(np.uint32))
     np.testing.assert_array_equal(orc.relu(a), ref.relu(a))
     np.testing.assert_array_equal(orc.clamp(a, 0.0, 0.6), ref.clamp(a, 0.0, 0.6))
+    wide = (rng.normal(size=4096) * 4).astype(np.float32)
+    for op in ("hswish", "hsigmoid"):
+        np.testing.assert_array_equal(getattr(orc, op)(wide).view(np.uint32), getattr(ref, op)(wide).view(np.uint32), err_msg=op)
+    np.testing.assert_allclose(orc.sigmoid(wide), ref.sigmoid(wide), rtol=2e-7)
+    for beta in (1.0, 0.6):
+        np.testing.assert_allclose(orc.swish(wide, beta), ref.swish(wide, beta), rtol=3e-7, atol=1e-12)
     for sshape in ((1,), (5,), (3,), (1, 5, 1, 1), (5, 1, 1), (2, 5, 4, 3), (4, 1)):
         slope = rng.normal(size=sshape).astype(np.float32)
         x, y = orc.prelu(a, slope), ref.prelu(a, slope)
