@@ -91,6 +91,7 @@ struct Value {
     int tensor = -1;
     std::vector<float> sub, mul;   // VK_DEQ: (float(q) - sub) * mul, each empty / 1 / C values
     View view;                     // VK_MAT
+    bool flat = false;             // the [N, C, H, W] byte tensor stands for its Reshape to [N, C * H * W] (read by a MatMul)
 };
 
 struct EpilogueSpec {
@@ -1221,6 +1222,11 @@ struct Planner {
     void plan_node(int id) {
         const GNode& n = N(id);
         const bool mat = !n.in.empty() && n.op != OP_CONSTANT && value(n.in[0]).kind == VK_MAT;
+        // a flattened feature map keeps its NHWC bytes; only what reads it the way the reference reads [N, C * H * W]
+        // may follow: the zero point's Convert and Subtract, and the MatMul (a convolution with an H x W filter)
+        for (int in : n.in)
+            if (in >= 0 && N(in).op != OP_CONSTANT && values[in].flat && n.op != OP_MATMUL && n.op != OP_CONVERT && n.op != OP_SUBTRACT)
+                unsupported(id, "a flattened [N, C, H, W] value is read by a MatMul against constant weights");
         switch (n.op) {
         case OP_PARAMETER: plan_parameter(id); break;
         case OP_CONSTANT: values[id].kind = VK_CONST; break;
@@ -2102,11 +2108,13 @@ struct Planner {
                 unsupported(id, "Convert is planned only as the start of a dequantization (u8/i8 -> f32)");
             v.kind = VK_DEQ;
             v.tensor = x.tensor;
+            v.flat = x.flat;
         } else {
             if (x.kind != VK_DEQ) unsupported(id, "stand-alone elementwise op outside a fused chain");
             std::vector<float> c;
             if (!channel_constant(n.in[1], tensors[x.tensor].c, n.shape.size(), c))
                 unsupported(id, "dequantization constant must be scalar or per-channel");
+            if (x.flat && c.size() != 1) unsupported(id, "a flattened [N, C, H, W] value takes one zero point for all of it");
             v = x;
             if (n.op == OP_SUBTRACT) {
                 if (!v.mul.empty() || !v.sub.empty()) unsupported(id, "Subtract after Multiply in a dequantization");
@@ -2187,8 +2195,19 @@ struct Planner {
         // [N, C, 1, 1] <-> [N, C]: same bytes in NHWC
         const bool flatten = src.shape.size() == 4 && n.shape.size() == 2 && src.shape[2] == 1 &&
                              src.shape[3] == 1 && n.shape[0] == src.shape[0] && n.shape[1] == src.shape[1];
+        // [N, C, H, W] -> [N, C * H * W] of a byte tensor in front of a fully connected layer: the bytes stay NHWC and
+        // the MatMul runs as the convolution with an H x W filter it is equal to (its weights [OC, C * H * W] are that
+        // filter in the reference's own order)
+        const bool flatten_map = src.shape.size() == 4 && n.shape.size() == 2 && n.shape[0] == src.shape[0] &&
+                                 n.shape[1] == src.shape[1] * src.shape[2] * src.shape[3] && (x.kind == VK_TENSOR || x.kind == VK_DEQ) &&
+                                 tensors[x.tensor].esize() == 1 && x.mul.empty() && x.sub.size() <= 1;
+        if (!flatten && flatten_map) {
+            values[id] = x;
+            values[id].flat = true;
+            return;
+        }
         if (!flatten || (x.kind != VK_TENSOR && x.kind != VK_DEQ))
-            unsupported(id, "only [N,C,1,1] -> [N,C] reshapes are planned");
+            unsupported(id, "only [N,C,1,1] -> [N,C] reshapes (and [N,C,H,W] -> [N,C*H*W] of quantized values in front of a MatMul) are planned");
         values[id] = x;
     }
 
@@ -2401,6 +2420,13 @@ struct Planner {
             const int8_t* w = reinterpret_cast<const int8_t*>(W.data.data());
             for (int64_t o = 0; o < OC; ++o)
                 for (int64_t k = 0; k < IC; ++k) st->weights[o * IC + k] = n.tb ? w[o * IC + k] : w[k * OC + o];
+            if (x.flat) {
+                // rows of [C * H * W] weights are [C][H][W] filters: the layer is the convolution of the whole map
+                if (IC != static_cast<int64_t>(tin.c) * tin.h * tin.w) unsupported(id, "MatMul whose reduction length is not the flattened map's");
+                IC = tin.c;
+                d.kh = tin.h;
+                d.kw = tin.w;
+            }
         } else {
             const bool grouped = n.op == OP_GROUP_CONVOLUTION;
             // [G, OC/G, IC/G, kh, kw].  One filter per channel (depthwise) has kernels of its own; any other grouping runs

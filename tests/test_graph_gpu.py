@@ -478,6 +478,44 @@ def test_concat_of_quantized_branches(orc, branches, signed):
     np.testing.assert_array_equal(got2["out"].view(np.uint32), want2["out"].view(np.uint32))
 
 
+def _flattened_map_net(shape, oc, levels, seed=77):
+    from dldt_amd import builders
+    N, C, H, W = shape
+    rng = np.random.default_rng(seed + oc)
+    x = rng.uniform(0, 1, (N, 8, 2 * H - 1, 2 * W - 1)).astype(np.float32)
+    rnd = lambda s, scale: (rng.standard_normal(s, dtype=np.float32) * np.float32(scale)).astype(np.float32)
+    net = builders.QuantizedNet()
+    g = net.g
+    a0 = net.input("data", x.shape, 1.0)
+    w0, b0 = rnd((C, 8, 3, 3), 0.1), rnd(C, 0.2)
+    if levels == "zero point":
+        a1 = net.asymmetric(net.conv_f32(a0, w0, b0, strides=(2, 2), pads=(1, 1)), -0.7, 1.3)
+    else:
+        a1 = net.conv(a0, w0, b0, 2.0, strides=(2, 2), pads=(1, 1), signed=levels == "i8")
+    flat = dict(a1, node=g.reshape(a1["node"], (N, C * H * W)))
+    g.result(net.conv_f32(flat, rnd((oc, C * H * W), 0.05), rnd(oc, 0.2), matmul=True, relu=True), "fc")
+    return g, x, a1["node"]
+
+
+@pytest.mark.parametrize("shape,oc,levels", [((3, 32, 5, 6), 50, "u8"), ((2, 24, 7, 7), 130, "i8"), ((4, 16, 3, 4), 10, "zero point")])
+def test_fully_connected_layer_behind_a_flattened_feature_map(orc, shape, oc, levels):
+    """u8 / i8 feature map [N, C, H, W] -> Reshape [N, C * H * W] -> MatMul with i8 weights (a classifier without a global
+    pool in front, VGG / AlexNet style): the bytes stay where they are and the MatMul runs as the convolution with an
+    H x W filter that it is equal to; bit-exact, also where the activations carry a zero point"""
+    g, x, a1 = _flattened_map_net(shape, oc, levels)
+    N, C, H, W = shape
+    want, kept = evaluate(orc, g.nodes, {"data": x}, keep=[a1])
+    assert kept[a1].shape == shape
+    plan = g.compile()
+    types = [s["type"] for s in plan.steps]
+    assert types[-2:] == ["MatMul", "Result"] and plan.steps[-2]["macs"] == N * oc * C * H * W
+    req = plan.create_request()
+    (got,) = req.infer(x)
+    np.testing.assert_array_equal(req.tensor(a1), kept[a1])
+    assert got.shape == (N, oc)
+    np.testing.assert_array_equal(got.view(np.uint32), want["fc"].view(np.uint32))
+
+
 @pytest.mark.parametrize("axis", [0, 2, 3, -1])
 @pytest.mark.parametrize("quantized", [True, False])
 def test_concat_along_the_batch_and_the_spatial_axes(orc, axis, quantized):

@@ -155,6 +155,32 @@ def test_planner_refuses_a_reshape_that_moves_bytes():
     assert e.value.status == -2 and "Reshape" in str(e.value)
 
 
+def test_planner_flattened_feature_map_in_front_of_a_fully_connected_layer():
+    """[N, C, H, W] bytes -> Reshape [N, C * H * W] -> MatMul: planned as the convolution with an H x W filter; anything
+    else that would read the flattened value in the reference's [C][H][W] order is refused"""
+    from dldt_amd import HipieError, builders
+    rng = np.random.default_rng(3)
+    rnd = lambda s, k: (rng.standard_normal(s, dtype=np.float32) * np.float32(k)).astype(np.float32)
+    net = builders.QuantizedNet()
+    g = net.g
+    a0 = net.input("data", (2, 8, 9, 11), 1.0)
+    a1 = net.conv(a0, rnd((16, 8, 3, 3), 0.1), rnd(16, 0.2), 2.0, strides=(2, 2), pads=(1, 1))
+    flat = dict(a1, node=g.reshape(a1["node"], (2, 16 * 5 * 6)))
+    g.result(net.conv_f32(flat, rnd((10, 480), 0.05), rnd(10, 0.2), matmul=True), "fc")
+    plan = g.compile(device=-1)
+    assert [s["type"] for s in plan.steps] == ["FakeQuantize", "Convolution", "MatMul", "Result"]
+    assert plan.steps[2]["macs"] == 2 * 10 * 480 and plan.outputs[0]["shape"] == (2, 10)
+    # the flattened levels as a result of their own: their order in memory is not the reference's
+    net = builders.QuantizedNet()
+    g = net.g
+    a0 = net.input("data", (2, 8, 9, 11), 1.0)
+    a1 = net.conv(a0, rnd((16, 8, 3, 3), 0.1), rnd(16, 0.2), 2.0, strides=(2, 2), pads=(1, 1))
+    g.result(net.dequantize(dict(a1, node=g.reshape(a1["node"], (2, 480)))), "flat")
+    with pytest.raises(HipieError) as e:
+        g.compile(device=-1)
+    assert e.value.status == -2 and "flattened" in str(e.value)
+
+
 def test_planner_embedding_front_end():
     from dldt_amd import builders
     from dldt_amd.graph import Plan
