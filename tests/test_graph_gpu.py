@@ -497,7 +497,8 @@ def _flattened_map_net(shape, oc, levels, seed=77):
     return g, x, a1["node"]
 
 
-@pytest.mark.parametrize("shape,oc,levels", [((3, 32, 5, 6), 50, "u8"), ((2, 24, 7, 7), 130, "i8"), ((4, 16, 3, 4), 10, "zero point")])
+@pytest.mark.parametrize("shape,oc,levels", [((3, 32, 5, 6), 50, "u8"), ((2, 24, 7, 7), 130, "i8"), ((4, 16, 3, 4), 10, "zero point"),
+                                             ((64, 128, 7, 7), 1000, "u8")])
 def test_fully_connected_layer_behind_a_flattened_feature_map(orc, shape, oc, levels):
     """u8 / i8 feature map [N, C, H, W] -> Reshape [N, C * H * W] -> MatMul with i8 weights (a classifier without a global
     pool in front, VGG / AlexNet style): the bytes stay where they are and the MatMul runs as the convolution with an
